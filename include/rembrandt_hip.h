@@ -1,0 +1,203 @@
+/*
+ * rembrandt_hip.h -- C ABI of librembrandt_hip.so: the MI355X (gfx950) replacement for the native
+ * layer underneath rembrandt's single-GPU operator hot path.
+ *
+ * In the reference that native layer is three crates whose sources are not in its tree:
+ * `cuda_dnn::v4` (cuDNN), `array_cuda` (cuBLAS + device memory / streams) and
+ * `rembrandt_kernels::ffi` (hand-written kernels).  Each entry point below names the reference
+ * call site(s) it replaces (paths relative to the reference tree).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; device pointers unless a parameter is named `*_h` / `host`;
+ *   - every `rh_*` function returns 0 on success, a positive hipError_t value on a HIP failure,
+ *     or a negative RH_E_* code on a usage error.  The reference panics on every error
+ *     (`.unwrap()` / `panic!`, src/operator/mod.rs:1685-1696); a binding reproduces that by
+ *     unwrapping the return code.  The `rembrandt_kernel_*` symbols keep the reference's
+ *     `void` signatures; their launch status can be read with rh_last_error();
+ *   - nothing here allocates, frees or synchronises unless its name says so (`rh_malloc`,
+ *     `rh_free`, `*_sync`); all work is enqueued on the given stream;
+ *   - tensors are fp32, NCHW with W fastest (src/operator/mod.rs:1471-1474); filters
+ *     [K][C][R][S]; 2-D arrays are column-major with the first index fastest
+ *     (src/arch_new.rs:141-145), so an affine weight `(in, out)` is `[out][in]` in memory;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ */
+#ifndef REMBRANDT_HIP_H
+#define REMBRANDT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* rh_stream_t; /* hipStream_t */
+
+/* usage errors */
+#define RH_E_INVALID   (-1) /* bad argument (NULL pointer, non-positive dimension, unknown enum) */
+#define RH_E_WORKSPACE (-2) /* workspace missing or smaller than rh_conv2d_workspace_bytes()      */
+#define RH_E_UNSUPPORTED (-3)
+#define RH_E_LIMIT     (-4) /* size beyond a documented limit                                      */
+
+/* math / fusion flags of the conv and GEMM entry points */
+#define RH_MATH_FP32_MFMA          0x0  /* fp32 operands, v_mfma_f32_32x32x2_f32, fp32 accumulate (default) */
+#define RH_MATH_BF16_MFMA_FP32ACC  0x1  /* operands rounded to bf16 (RNE) on load, bf16 MFMA, fp32 accumulate */
+#define RH_FUSE_BIAS               0x10 /* conv fwd: add bias[k] in the epilogue (replaces the separate K2 pass) */
+#define RH_FUSE_RELU               0x20 /* conv fwd: max(.,0) in the epilogue (replaces the separate K3 pass)    */
+
+const char* rh_version(void);
+/* Status of the most recent launch made by a void `rembrandt_kernel_*` entry point on this thread. */
+int rh_last_error(void);
+const char* rh_error_string(int code);
+
+/* ---------------------------------------------------------------------------------------------
+ * Context + memory.  Replaces array_cuda::device::{context,memory}: DeviceContext::new(dev)
+ * (tools/train-mnist.rs:155-178), ctx.stream.ptr (src/operator/mod.rs:1112), ctx.sync()
+ * (src/operator/comm.rs:223), DeviceBuffer::zeros (mod.rs:940), send (mod.rs:1249-1267),
+ * sync_load / sync_store (src/operator/loss.rs:170-186, 212-213), set_constant (mod.rs:908-909),
+ * cast_bytes{,_normalized} (mod.rs:735-737).
+ * ------------------------------------------------------------------------------------------- */
+typedef struct rh_ctx rh_ctx;
+int rh_ctx_create(int device, rh_ctx** out);
+int rh_ctx_destroy(rh_ctx* ctx);
+rh_stream_t rh_ctx_stream(rh_ctx* ctx);
+int rh_ctx_sync(rh_ctx* ctx);
+int rh_malloc(rh_ctx* ctx, size_t bytes, void** dptr); /* zero-filled, like DeviceBuffer::zeros */
+int rh_free(rh_ctx* ctx, void* dptr);
+int rh_memset_f32(float* d, float value, size_t n, rh_stream_t stream);
+int rh_copy_d2d(void* dst, const void* src, size_t bytes, rh_stream_t stream);
+int rh_load_sync(rh_ctx* ctx, void* dst_d, const void* src_h, size_t bytes);
+int rh_store_sync(rh_ctx* ctx, void* dst_h, const void* src_d, size_t bytes);
+int rh_cast_u8_f32(const uint8_t* x, float* y, size_t n, float scale, rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Convolution.  Replaces cuda_dnn::v4 CudnnConvFwdOp::forward (src/operator/mod.rs:1684-1696,
+ * src/layer_new.rs:999-1011, src/layer.rs:1414-1420), CudnnConvBwdFilterOp::backward_filter
+ * (mod.rs:1765-1774, layer_new.rs:1092-1101), ::backward_bias (mod.rs:1775-1781) and
+ * CudnnConvBwdDataOp::backward_data (mod.rs:1783-1793).  Cross-correlation, symmetric padding,
+ * square stride; output extent max(0, in + 2*pad - size + stride) / stride (mod.rs:1393-1398).
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+  int32_t N, C, H, W; /* input  N x C x H x W */
+  int32_t K, R, S;    /* filter K x C x R x S */
+  int32_t stride, pad;
+} rh_conv_geom;
+
+enum { RH_CONV_FWD = 0, RH_CONV_BWD_FILTER = 1, RH_CONV_BWD_DATA = 2 };
+
+int32_t rh_conv2d_out_dim(int32_t in, int32_t size, int32_t stride, int32_t pad);
+/* Bytes of scratch the given pass needs (0 is possible). The scratch must be 256-byte aligned. */
+size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass);
+/* y = alpha * corr(x, w) + beta * y.  With RH_FUSE_BIAS, `bias` (length K) is added after the
+ * alpha/beta blend; with RH_FUSE_RELU the result is clamped at 0.  bias may be NULL otherwise. */
+int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x, const float* w, float beta,
+                  float* y, const float* bias, void* ws, size_t ws_bytes, int flags,
+                  rh_stream_t stream);
+/* dw = alpha * sum_{n,p,q} dy * x + beta * dw.  Deterministic two-pass split reduction. */
+int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const float* x, const float* dy,
+                         float beta, float* dw, void* ws, size_t ws_bytes, int flags,
+                         rh_stream_t stream);
+/* db[k] = alpha * sum_{n,p,q} dy[n,k,p,q] + beta * db[k];  plane = P*Q. */
+int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy,
+                       float beta, float* db, rh_stream_t stream);
+/* dx = alpha * corr^T(dy, w) + beta * dx. */
+int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const float* w, const float* dy,
+                       float beta, float* dx, void* ws, size_t ws_bytes, int flags,
+                       rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Bias add and ReLU.  rh_add_bias_nchw replaces CudnnAddOp::forward (mod.rs:1097-1103,
+ * 1697-1704): y[n,k,:] = alpha*bias[k] + beta*y[n,k,:].  The two rembrandt_kernel_* symbols keep
+ * the names and argument lists of rembrandt_kernels::ffi as seen at mod.rs:1108-1113,
+ * 1154-1160, 1709-1714, 1754-1760 (the stream argument is a hipStream_t).
+ * ------------------------------------------------------------------------------------------- */
+int rh_add_bias_nchw(const float* bias, float* y, int32_t plane, int32_t K, int32_t N, float alpha,
+                     float beta, rh_stream_t stream);
+void rembrandt_kernel_batch_map_rect_inplace(float* y, int32_t frame_len, int32_t batch,
+                                             rh_stream_t stream);
+void rembrandt_kernel_batch_map_rect_backprop_inplace(const float* y, int32_t frame_len,
+                                                      int32_t batch, float* dy, rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Column-major SGEMM and BLAS-1.  Replaces array_cuda's BlasMatrixExt::matrix_prod
+ * (mod.rs:1094, 1168, 1169, 1174), matrix_sum / row_vector_sum (mod.rs:1186-1189, 1203-1206,
+ * 1214-1217), matrix_scale / row_vector_scale (mod.rs:1199-1202, 1359-1362).
+ * C(m,n) = alpha * op(A) * op(B) + beta * C, all column-major; transX != 0 means transposed.
+ * ------------------------------------------------------------------------------------------- */
+/* Optional scratch (256-byte aligned): with it, GEMMs whose result has too few tiles to fill the
+ * GPU split the contraction across blocks and reduce in a fixed order; without it (ws == NULL)
+ * the same result is computed unsplit. */
+size_t rh_sgemm_workspace_bytes(int32_t m, int32_t n, int32_t k);
+int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k, float alpha, const float* A,
+             int32_t lda, const float* B, int32_t ldb, float beta, float* C, int32_t ldc, void* ws,
+             size_t ws_bytes, int flags, rh_stream_t stream);
+int rh_saxpy(int64_t n, float alpha, const float* x, float* y, rh_stream_t stream);
+int rh_sscal(int64_t n, float alpha, float* x, rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Pooling.  Replaces CudnnPoolingOp::forward / ::backward (mod.rs:2103-2107, 2115-2121; modes
+ * Max and AverageCountIncludingPadding, mod.rs:2061-2065; floor extent mod.rs:2022-2027) and the
+ * gen-1 kernels rembrandt_kernel_image_{max,average}_pool{,_backward} with their ceil extent and
+ * int32 arg-max mask (src/layer.rs:1741-1747, 1797-1813, 1824-1840).
+ * opt_argmax (may be NULL): per output element the h*W+w index inside its input plane of the
+ * selected tap (-1: window without in-range tap).  Backward overwrites dx; with opt_argmax
+ * given it does not read x or y.
+ * ------------------------------------------------------------------------------------------- */
+enum { RH_POOL_MAX = 0, RH_POOL_AVG_INCL_PAD = 1 };
+enum { RH_ROUND_FLOOR = 0, RH_ROUND_CEIL = 1 };
+typedef struct {
+  int32_t N, C, H, W;
+  int32_t size, stride, pad;
+  int32_t mode;  /* RH_POOL_* */
+  int32_t round; /* RH_ROUND_* */
+} rh_pool_geom;
+int32_t rh_pool2d_out_dim(int32_t in, int32_t size, int32_t stride, int32_t pad, int32_t round);
+int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, int32_t* opt_argmax,
+                  rh_stream_t stream);
+int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float* y, const float* dy, float* dx,
+                  const int32_t* opt_argmax, rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Softmax / KL loss / reductions.  rh_softmax_fwd replaces CudnnSoftmaxOp::forward
+ * (src/operator/loss.rs:121-126); the rembrandt_kernel_* symbols keep the rembrandt_kernels::ffi
+ * names and argument lists seen at loss.rs:132-140, 191-200, 203-210, 229-239.  The reference
+ * asserts len <= 1024 for the block reductions; these kernels have no such limit.
+ * ------------------------------------------------------------------------------------------- */
+int rh_softmax_fwd(const float* x, float* p, int32_t C, int32_t N, rh_stream_t stream);
+void rembrandt_kernel_batch_map_softmax_kl_backward(const float* p, int32_t C, int32_t N,
+                                                    const int32_t* labels, const float* weights,
+                                                    float* dx, rh_stream_t stream);
+void rembrandt_kernel_batch_map_softmax_kl_loss1(const float* p, int32_t C, int32_t N,
+                                                 const int32_t* labels, const float* weights,
+                                                 float beta, float* loss1, rh_stream_t stream);
+void rembrandt_kernel_batch_blockreduce_sum(const float* src, int32_t len, int32_t batch,
+                                            float* dst, float beta, rh_stream_t stream);
+void rembrandt_kernel_batch_blockreduce_argmax(const float* src, int32_t len, int32_t batch,
+                                               float* max_out, int32_t* idx_out,
+                                               rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * SGD.  rh_sgd_momentum_step is the fused form of the BLAS-1 sequence regularize ->
+ * accumulate_grads -> update_params -> reset (mod.rs:1178-1218, 1355-1363; driven by
+ * src/opt/sgd/new.rs:345-495):  g += l2*W (if l2 > 0); v = mu*v; v += scale*g; W += apply*v;
+ * g = 0 (if zero_grad).  rh_descend is the gen-1/gen-2 update g += l2*W; W -= s*g
+ * (src/layer_new.rs:596-617, src/layer.rs:1710-1715).
+ * ------------------------------------------------------------------------------------------- */
+int rh_sgd_momentum_step(int64_t n, float* W, float* g, float* v, float l2, float scale, float mu,
+                         float apply, int zero_grad, rh_stream_t stream);
+int rh_descend(int64_t n, float* W, float* g, float s, float l2, rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Host-side seeded generator for synthetic inputs and parameter initialisation (stands in for
+ * the rng crate's Xorshiftplus128Rng + rand 0.3 distributions of src/operator/mod.rs:964-1006,
+ * 1554-1592, whose bit streams cannot be reproduced).  Element i of stream (seed, stream_id) is
+ * a pure function of (seed, stream_id, i).  Host pointers.
+ * ------------------------------------------------------------------------------------------- */
+int rh_rng_fill_uniform(uint64_t seed, uint64_t stream_id, float* host, size_t n, float lo, float hi);
+int rh_rng_fill_normal(uint64_t seed, uint64_t stream_id, float* host, size_t n, float mean, float std);
+int rh_rng_fill_int(uint64_t seed, uint64_t stream_id, int32_t* host, size_t n, int32_t modulus);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* REMBRANDT_HIP_H */

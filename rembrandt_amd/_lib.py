@@ -1,0 +1,103 @@
+"""ctypes binding of librembrandt_hip.so (the C ABI declared in include/rembrandt_hip.h).
+
+The library is loaded from the package directory; there is no fallback implementation: if the
+shared object is missing, loading raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librembrandt_hip.so")
+
+RH_CONV_FWD, RH_CONV_BWD_FILTER, RH_CONV_BWD_DATA = 0, 1, 2
+RH_POOL_MAX, RH_POOL_AVG_INCL_PAD = 0, 1
+RH_ROUND_FLOOR, RH_ROUND_CEIL = 0, 1
+RH_FUSE_BIAS, RH_FUSE_RELU = 0x10, 0x20
+RH_MATH_BF16_MFMA_FP32ACC = 0x1
+RH_E_INVALID, RH_E_WORKSPACE, RH_E_UNSUPPORTED, RH_E_LIMIT = -1, -2, -3, -4
+
+
+class ConvGeom(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "K", "R", "S", "stride", "pad")]
+
+
+class PoolGeom(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "size", "stride", "pad", "mode", "round")]
+
+
+_vp, _f, _i32, _i64, _sz, _int = C.c_void_p, C.c_float, C.c_int32, C.c_int64, C.c_size_t, C.c_int
+
+# name -> (restype, argtypes).  Device pointers are passed as integers (c_void_p).
+PROTOTYPES = {
+    "rh_version": (C.c_char_p, []),
+    "rh_last_error": (_int, []),
+    "rh_error_string": (C.c_char_p, [_int]),
+    "rh_ctx_create": (_int, [_int, C.POINTER(_vp)]),
+    "rh_ctx_destroy": (_int, [_vp]),
+    "rh_ctx_stream": (_vp, [_vp]),
+    "rh_ctx_sync": (_int, [_vp]),
+    "rh_malloc": (_int, [_vp, _sz, C.POINTER(_vp)]),
+    "rh_free": (_int, [_vp, _vp]),
+    "rh_memset_f32": (_int, [_vp, _f, _sz, _vp]),
+    "rh_copy_d2d": (_int, [_vp, _vp, _sz, _vp]),
+    "rh_load_sync": (_int, [_vp, _vp, _vp, _sz]),
+    "rh_store_sync": (_int, [_vp, _vp, _vp, _sz]),
+    "rh_cast_u8_f32": (_int, [_vp, _vp, _sz, _f, _vp]),
+    "rh_conv2d_out_dim": (_i32, [_i32, _i32, _i32, _i32]),
+    "rh_conv2d_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _int]),
+    "rh_conv2d_fwd": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _vp, _sz, _int, _vp]),
+    "rh_conv2d_bwd_filter": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _sz, _int, _vp]),
+    "rh_conv2d_bwd_bias": (_int, [_i32, _i32, _i32, _f, _vp, _f, _vp, _vp]),
+    "rh_conv2d_bwd_data": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _sz, _int, _vp]),
+    "rh_add_bias_nchw": (_int, [_vp, _vp, _i32, _i32, _i32, _f, _f, _vp]),
+    "rembrandt_kernel_batch_map_rect_inplace": (None, [_vp, _i32, _i32, _vp]),
+    "rembrandt_kernel_batch_map_rect_backprop_inplace": (None, [_vp, _i32, _i32, _vp, _vp]),
+    "rh_sgemm_workspace_bytes": (_sz, [_i32, _i32, _i32]),
+    "rh_sgemm": (_int, [_int, _int, _i32, _i32, _i32, _f, _vp, _i32, _vp, _i32, _f, _vp, _i32, _vp, _sz, _int, _vp]),
+    "rh_saxpy": (_int, [_i64, _f, _vp, _vp, _vp]),
+    "rh_sscal": (_int, [_i64, _f, _vp, _vp]),
+    "rh_pool2d_out_dim": (_i32, [_i32, _i32, _i32, _i32, _i32]),
+    "rh_pool2d_fwd": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp]),
+    "rh_pool2d_bwd": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp, _vp, _vp]),
+    "rh_softmax_fwd": (_int, [_vp, _vp, _i32, _i32, _vp]),
+    "rembrandt_kernel_batch_map_softmax_kl_backward": (None, [_vp, _i32, _i32, _vp, _vp, _vp, _vp]),
+    "rembrandt_kernel_batch_map_softmax_kl_loss1": (None, [_vp, _i32, _i32, _vp, _vp, _f, _vp, _vp]),
+    "rembrandt_kernel_batch_blockreduce_sum": (None, [_vp, _i32, _i32, _vp, _f, _vp]),
+    "rembrandt_kernel_batch_blockreduce_argmax": (None, [_vp, _i32, _i32, _vp, _vp, _vp]),
+    "rh_sgd_momentum_step": (_int, [_i64, _vp, _vp, _vp, _f, _f, _f, _f, _int, _vp]),
+    "rh_descend": (_int, [_i64, _vp, _vp, _f, _f, _vp]),
+    "rh_rng_fill_uniform": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
+    "rh_rng_fill_normal": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
+    "rh_rng_fill_int": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _i32]),
+}
+
+_lib = None
+
+
+class RembrandtHipError(RuntimeError):
+    def __init__(self, code, where):
+        self.code = code
+        msg = lib().rh_error_string(code)
+        super().__init__("%s failed: %d (%s)" % (where, code, msg.decode() if msg else "?"))
+
+
+def lib():
+    """The loaded shared library, with prototypes set.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("%s is missing: build it with `python -m rembrandt_amd.build` "
+                              "(there is no CPU fallback)" % LIB_PATH)
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(code, where):
+    """Reproduces the reference's panic-on-error convention (src/operator/mod.rs:1685-1696)."""
+    if code != 0:
+        raise RembrandtHipError(code, where)

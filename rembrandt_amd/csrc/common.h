@@ -1,0 +1,36 @@
+// Shared helpers of the HIP translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/rembrandt_hip.h"
+
+namespace rh {
+
+inline hipStream_t to_stream(rh_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Status of the last launch made through a void rembrandt_kernel_* entry point (per thread).
+extern thread_local int g_last_error;
+
+inline int launch_status() { return static_cast<int>(hipGetLastError()); }
+
+template <class T>
+constexpr T cdiv(T a, T b) { return (a + b - 1) / b; }
+
+// Largest tensor the buffer-addressed kernels accept: byte offsets are 32-bit and the value
+// 0x80000000 is reserved as the "out of range, reads as zero" offset.
+constexpr size_t kMaxBufferBytes = size_t(1) << 31;
+
+constexpr int kWave = 64;
+
+// Grid size for a grid-stride elementwise kernel: enough blocks to keep 256 CUs busy with
+// several waves each, never more than the work needs.
+inline int stream_grid(size_t work_items, int block) {
+  size_t want = cdiv<size_t>(work_items, static_cast<size_t>(block));
+  const size_t cap = 256 * 16;
+  if (want > cap) want = cap;
+  if (want < 1) want = 1;
+  return static_cast<int>(want);
+}
+
+}  // namespace rh

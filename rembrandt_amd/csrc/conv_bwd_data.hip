@@ -1,0 +1,72 @@
+// Convolution backward-data (K7) as an implicit GEMM over the transposed filter:
+//   dx[n][c][h][w] = sum_{ko,r,s} w[ko][c][r][s] * dy[n][ko][(h+pad-r)/st][(w+pad-s)/st]
+// rows = input channels c (filter read through a k -> offset table), cols = input pixels
+// (dy gathered; a term exists only when both divisions are exact and land inside P x Q).
+#include "conv_common.h"
+
+namespace rh {
+
+__global__ void build_bwd_data_tab_kernel(int4* tab, int* atab, int n_entries, int KRS, int C, int R,
+                                          int S, int PQ, int Q, int st) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= n_entries) return;
+  if (k < KRS) {
+    const int ko = k / (R * S), rs = k - ko * (R * S), r = rs / S, s = rs - r * S;
+    const int rq = r / st, rr = r - rq * st, sq = s / st, sr = s - sq * st;
+    tab[k] = make_int4(ko * PQ - rq * Q - sq, -rq, -sq, rr * st + sr);
+    atab[k] = ko * C * R * S + r * S + s;
+  } else {
+    tab[k] = make_int4(0, -(1 << 28), 0, -1);
+    atab[k] = -1;
+  }
+}
+
+template <class T>
+static int run_bwd_data(int KRS, const DenseParams& ap, const GatherParams& bp, const EpiParams& ep,
+                        hipStream_t stream) {
+  typedef LoadDenseK<T::BM, T::BK, T::NT, true> AL;
+  typedef LoadGatherR<T::BN, T::BK, T::NT, true> BL;
+  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, KRS, 1, nullptr, stream);
+}
+
+}  // namespace rh
+
+using namespace rh;
+
+extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const float* w, const float* dy,
+                                  float beta, float* dx, void* ws, size_t ws_bytes, int flags,
+                                  rh_stream_t stream_) {
+  ConvDims d;
+  if (int e = conv_dims(g, &d)) return e;
+  if (!w || !dy || !dx) return RH_E_INVALID;
+  if (flags & RH_MATH_BF16_MFMA_FP32ACC) return RH_E_UNSUPPORTED;
+  const size_t need = rh_conv2d_workspace_bytes(g, RH_CONV_BWD_DATA);
+  if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return RH_E_WORKSPACE;
+  hipStream_t stream = to_stream(stream_);
+
+  const int KRS = d.K * d.R * d.S;
+  const int n_tab = round_up(KRS, kTabPad);
+  int4* tab = static_cast<int4*>(ws);
+  int* atab = reinterpret_cast<int*>(static_cast<char*>(ws) + align256(sizeof(int4) * (size_t)n_tab));
+  hipLaunchKernelGGL(build_bwd_data_tab_kernel, dim3(cdiv(n_tab, 256)), dim3(256), 0, stream, tab, atab,
+                     n_tab, KRS, d.C, d.R, d.S, d.P * d.Q, d.Q, d.st);
+  if (int e = launch_status()) return e;
+
+  DenseParams ap;
+  ap.ptr = w; ap.bytes = (uint32_t)(d.w_elems * 4); ap.rows = d.C; ap.K = KRS; ap.ld = d.R * d.S; ap.ktab = atab;
+  GatherParams bp;
+  bp.ptr = dy; bp.bytes = (uint32_t)(d.y_elems * 4);
+  bp.M = d.N * d.H * d.W; bp.inner = d.H * d.W; bp.innerW = d.W;
+  bp.img_stride = d.K * d.P * d.Q; bp.row_stride = d.Q; bp.st = d.st; bp.pad = d.pad;
+  bp.Hlim = d.P; bp.Wlim = d.Q; bp.ktab = tab;
+  EpiParams ep;
+  ep.out = dx; ep.bias = nullptr; ep.alpha = alpha; ep.beta = beta;
+  ep.rows = d.C; ep.cols = bp.M; ep.inner = d.H * d.W; ep.ld = 0; ep.relu = 0; ep.split_stride = 0;
+
+  switch (pick_bm(d.C)) {
+    case 128: return run_bwd_data<T128x128>(KRS, ap, bp, ep, stream);
+    case 96:  return run_bwd_data<T96x256>(KRS, ap, bp, ep, stream);
+    case 64:  return run_bwd_data<T64x256>(KRS, ap, bp, ep, stream);
+    default:  return run_bwd_data<T32x256>(KRS, ap, bp, ep, stream);
+  }
+}

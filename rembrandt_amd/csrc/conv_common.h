@@ -1,0 +1,83 @@
+// Host-side helpers shared by the three convolution passes.
+#pragma once
+#include "gemm_core.h"
+
+namespace rh {
+
+inline int conv_out_dim(int in, int size, int stride, int pad) {
+  int t = in + 2 * pad - size + stride;
+  if (t < 0) t = 0;
+  return t / stride;
+}
+
+inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+// Contraction tables are padded to a multiple of this many entries (>= every BK in use).
+constexpr int kTabPad = 64;
+
+struct ConvDims {
+  int N, C, H, W, K, R, S, st, pad, P, Q;
+  long long x_elems, w_elems, y_elems;
+};
+
+inline int conv_dims(const rh_conv_geom* g, ConvDims* d) {
+  if (!g) return RH_E_INVALID;
+  if (g->N <= 0 || g->C <= 0 || g->H <= 0 || g->W <= 0 || g->K <= 0 || g->R <= 0 || g->S <= 0 ||
+      g->stride <= 0 || g->pad < 0)
+    return RH_E_INVALID;
+  d->N = g->N; d->C = g->C; d->H = g->H; d->W = g->W; d->K = g->K; d->R = g->R; d->S = g->S;
+  d->st = g->stride; d->pad = g->pad;
+  d->P = conv_out_dim(g->H, g->R, g->stride, g->pad);
+  d->Q = conv_out_dim(g->W, g->S, g->stride, g->pad);
+  d->x_elems = (long long)g->N * g->C * g->H * g->W;
+  d->w_elems = (long long)g->K * g->C * g->R * g->S;
+  d->y_elems = (long long)g->N * g->K * d->P * d->Q;
+  if ((size_t)d->x_elems * 4 > kMaxBufferBytes || (size_t)d->y_elems * 4 > kMaxBufferBytes ||
+      (size_t)d->w_elems * 4 > kMaxBufferBytes)
+    return RH_E_LIMIT;
+  return 0;
+}
+
+// Row-tile height with the least zero padding for `rows` result rows; ties go to the taller tile.
+inline int pick_bm(int rows) {
+  const int cand[4] = {128, 96, 64, 32};
+  int best = 128;
+  long long best_pad = -1;
+  for (int i = 0; i < 4; ++i) {
+    const long long padded = (long long)round_up(rows, cand[i]);
+    if (best_pad < 0 || padded < best_pad) { best_pad = padded; best = cand[i]; }
+  }
+  return best;
+}
+
+template <class T, class AL, class BL, bool NCHW>
+inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Params& bp,
+                            const EpiParams& ep, int K, int splits, int* splits_used,
+                            hipStream_t stream) {
+  const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
+  const int k_chunks = cdiv(K, T::BK);
+  if (splits < 1) splits = 1;
+  const int cps = cdiv(k_chunks, splits) > 0 ? cdiv(k_chunks, splits) : 1;
+  const int used = cdiv(k_chunks, cps) > 0 ? cdiv(k_chunks, cps) : 1;
+  if (splits_used) *splits_used = used;
+  dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)used);
+  hipLaunchKernelGGL((mfma_gemm_kernel<T, AL, BL, NCHW>), grid, dim3(T::NT), 0, stream, ap, bp, ep,
+                     tiles_m, k_chunks, cps);
+  return launch_status();
+}
+
+// Tile shapes in use.  rows x cols x k, waves as WM x WN.
+typedef Tile<128, 128, 16, 2, 2> T128x128;
+typedef Tile<96, 256, 16, 1, 4> T96x256;
+typedef Tile<64, 256, 16, 1, 4> T64x256;
+typedef Tile<32, 256, 16, 1, 4> T32x256;
+
+// Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
+void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
+                         int ld, float alpha, float beta, hipStream_t stream);
+
+void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int HW, int W,
+                          hipStream_t stream);
+
+}  // namespace rh

@@ -1,0 +1,173 @@
+// Context, device memory, error strings and the host-side seeded generator.
+#include <math.h>
+#include <string.h>
+
+#include <algorithm>
+#include <thread>
+#include <vector>
+
+#include "common.h"
+
+struct rh_ctx {
+  int device;
+  hipStream_t stream;
+};
+
+using namespace rh;
+
+extern "C" const char* rh_version(void) { return "rembrandt-hip 0.1 (gfx950, fp32 MFMA)"; }
+
+extern "C" const char* rh_error_string(int code) {
+  switch (code) {
+    case 0: return "ok";
+    case RH_E_INVALID: return "invalid argument";
+    case RH_E_WORKSPACE: return "workspace missing, misaligned or too small";
+    case RH_E_UNSUPPORTED: return "unsupported option";
+    case RH_E_LIMIT: return "size beyond a documented limit";
+    default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown error";
+  }
+}
+
+extern "C" int rh_ctx_create(int device, rh_ctx** out) {
+  if (!out) return RH_E_INVALID;
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess) return (int)e;
+  if (device < 0 || device >= count) return RH_E_INVALID;
+  if ((e = hipSetDevice(device)) != hipSuccess) return (int)e;
+  rh_ctx* c = new rh_ctx;
+  c->device = device;
+  // default priority, non-blocking with respect to the legacy default stream
+  if ((e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking)) != hipSuccess) { delete c; return (int)e; }
+  *out = c;
+  return 0;
+}
+
+extern "C" int rh_ctx_destroy(rh_ctx* ctx) {
+  if (!ctx) return RH_E_INVALID;
+  hipError_t e = hipStreamSynchronize(ctx->stream);
+  hipError_t e2 = hipStreamDestroy(ctx->stream);
+  delete ctx;
+  return (int)(e != hipSuccess ? e : e2);
+}
+
+extern "C" rh_stream_t rh_ctx_stream(rh_ctx* ctx) { return ctx ? (rh_stream_t)ctx->stream : nullptr; }
+
+extern "C" int rh_ctx_sync(rh_ctx* ctx) {
+  if (!ctx) return RH_E_INVALID;
+  return (int)hipStreamSynchronize(ctx->stream);
+}
+
+extern "C" int rh_malloc(rh_ctx* ctx, size_t bytes, void** dptr) {
+  if (!ctx || !dptr) return RH_E_INVALID;
+  *dptr = nullptr;
+  if (bytes == 0) return 0;
+  hipError_t e = hipMalloc(dptr, bytes);
+  if (e != hipSuccess) return (int)e;
+  // zero with a fill kernel on the context's stream (buffers start as DeviceBuffer::zeros does)
+  const size_t words = bytes / 4;
+  if (words) {
+    if (int r = rh_memset_f32(static_cast<float*>(*dptr), 0.0f, words, (rh_stream_t)ctx->stream)) return r;
+  }
+  if (bytes % 4) {
+    e = hipMemsetAsync(static_cast<char*>(*dptr) + words * 4, 0, bytes % 4, ctx->stream);
+    if (e != hipSuccess) return (int)e;
+  }
+  return 0;
+}
+
+extern "C" int rh_free(rh_ctx* ctx, void* dptr) {
+  if (!ctx) return RH_E_INVALID;
+  if (!dptr) return 0;
+  hipError_t e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) return (int)e;
+  return (int)hipFree(dptr);
+}
+
+extern "C" int rh_copy_d2d(void* dst, const void* src, size_t bytes, rh_stream_t stream) {
+  if (bytes == 0) return 0;
+  if (!dst || !src) return RH_E_INVALID;
+  return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, to_stream(stream));
+}
+
+extern "C" int rh_load_sync(rh_ctx* ctx, void* dst_d, const void* src_h, size_t bytes) {
+  if (!ctx) return RH_E_INVALID;
+  if (bytes == 0) return 0;
+  if (!dst_d || !src_h) return RH_E_INVALID;
+  hipError_t e = hipMemcpyAsync(dst_d, src_h, bytes, hipMemcpyHostToDevice, ctx->stream);
+  if (e != hipSuccess) return (int)e;
+  return (int)hipStreamSynchronize(ctx->stream);
+}
+
+extern "C" int rh_store_sync(rh_ctx* ctx, void* dst_h, const void* src_d, size_t bytes) {
+  if (!ctx) return RH_E_INVALID;
+  if (bytes == 0) return 0;
+  if (!dst_h || !src_d) return RH_E_INVALID;
+  hipError_t e = hipMemcpyAsync(dst_h, src_d, bytes, hipMemcpyDeviceToHost, ctx->stream);
+  if (e != hipSuccess) return (int)e;
+  return (int)hipStreamSynchronize(ctx->stream);
+}
+
+// ---- seeded generator --------------------------------------------------------------------
+namespace {
+
+inline uint64_t mix64(uint64_t z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+inline uint64_t stream_key(uint64_t seed, uint64_t stream_id) {
+  return mix64(seed ^ mix64(stream_id + 0x9E3779B97F4A7C15ull));
+}
+inline uint64_t draw(uint64_t key, uint64_t i) { return mix64(key + (i + 1) * 0x9E3779B97F4A7C15ull); }
+
+template <class F>
+void parallel_for(size_t n, F f) {
+  unsigned hw = std::thread::hardware_concurrency();
+  size_t nt = std::min<size_t>(hw ? hw : 1, 16);
+  if (n < (size_t)1 << 16) nt = 1;
+  if (nt <= 1) { f(0, n); return; }
+  std::vector<std::thread> th;
+  const size_t chunk = (n + nt - 1) / nt;
+  for (size_t t = 0; t < nt; ++t) {
+    const size_t b = t * chunk, e = std::min(n, b + chunk);
+    if (b < e) th.emplace_back(f, b, e);
+  }
+  for (auto& t : th) t.join();
+}
+
+}  // namespace
+
+extern "C" int rh_rng_fill_uniform(uint64_t seed, uint64_t stream_id, float* host, size_t n, float lo, float hi) {
+  if (n && !host) return RH_E_INVALID;
+  const uint64_t key = stream_key(seed, stream_id);
+  parallel_for(n, [=](size_t b, size_t e) {
+    for (size_t i = b; i < e; ++i) {
+      const float u = (float)(draw(key, i) >> 40) * (1.0f / 16777216.0f);  // 24 bits: exact, in [0,1)
+      host[i] = lo + (hi - lo) * u;
+    }
+  });
+  return 0;
+}
+
+extern "C" int rh_rng_fill_normal(uint64_t seed, uint64_t stream_id, float* host, size_t n, float mean, float std) {
+  if (n && !host) return RH_E_INVALID;
+  const uint64_t key = stream_key(seed, stream_id);
+  parallel_for(n, [=](size_t b, size_t e) {
+    for (size_t i = b; i < e; ++i) {
+      // Box-Muller in double from two 53-bit uniforms; u1 in (0,1], u2 in [0,1)
+      const double u1 = (double)((draw(key, 2 * i) >> 11) + 1) * (1.0 / 9007199254740992.0);
+      const double u2 = (double)(draw(key, 2 * i + 1) >> 11) * (1.0 / 9007199254740992.0);
+      const double r = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
+      host[i] = (float)((double)mean + (double)std * r);
+    }
+  });
+  return 0;
+}
+
+extern "C" int rh_rng_fill_int(uint64_t seed, uint64_t stream_id, int32_t* host, size_t n, int32_t modulus) {
+  if ((n && !host) || modulus <= 0) return RH_E_INVALID;
+  const uint64_t key = stream_key(seed, stream_id);
+  for (size_t i = 0; i < n; ++i) host[i] = (int32_t)(draw(key, i) % (uint64_t)modulus);
+  return 0;
+}

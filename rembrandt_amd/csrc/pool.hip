@@ -1,0 +1,161 @@
+// Max / average pooling, forward and backward (K9 batch form, K9' arg-max mask + ceil extent).
+// Forward: one thread per output element scans its window (r outer, s inner; the first maximum
+// wins; padding never wins; the average divisor is always size*size).
+// Backward: one thread per *input* element gathers from every window that covers it, so
+// overlapping windows (3x3 stride 2) need no atomics and the sum order is fixed.
+#include "common.h"
+
+namespace rh {
+
+struct PoolDims { int N, C, H, W, k, st, pad, P, Q, mode; };
+
+inline int pool_out_dim(int in, int size, int stride, int pad, int round) {
+  if (round == RH_ROUND_CEIL) {
+    const int t = in + 2 * pad - size + stride - 1;
+    return t < 0 ? 0 : t / stride + 1;
+  }
+  int t = in + 2 * pad - size + stride;
+  if (t < 0) t = 0;
+  return t / stride;
+}
+
+__device__ __forceinline__ int window_argmax(const float* __restrict__ xp, int H, int W, int p, int q, int k, int st,
+                                             int pad, float* best_out) {
+  float best = 0.0f;
+  int bi = -1;
+  const int hs = p * st - pad, ws = q * st - pad;
+  for (int r = 0; r < k; ++r) {
+    const int h = hs + r;
+    if ((unsigned)h >= (unsigned)H) continue;
+    for (int s = 0; s < k; ++s) {
+      const int w = ws + s;
+      if ((unsigned)w >= (unsigned)W) continue;
+      const float v = xp[h * W + w];
+      if (bi < 0 || v > best) { best = v; bi = h * W + w; }
+    }
+  }
+  *best_out = best;
+  return bi;
+}
+
+__global__ void pool_fwd_kernel(PoolDims d, const float* __restrict__ x, float* __restrict__ y,
+                                int* __restrict__ argmax) {
+  const long long total = (long long)d.N * d.C * d.P * d.Q;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  const float inv = 1.0f / (float)(d.k * d.k);
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const int q = (int)(idx % d.Q);
+    const long long t = idx / d.Q;
+    const int p = (int)(t % d.P);
+    const long long nc = t / d.P;
+    const float* xp = x + nc * d.H * d.W;
+    if (d.mode == RH_POOL_MAX) {
+      float best;
+      const int bi = window_argmax(xp, d.H, d.W, p, q, d.k, d.st, d.pad, &best);
+      y[idx] = bi < 0 ? 0.0f : best;
+      if (argmax) argmax[idx] = bi;
+    } else {
+      float acc = 0.0f;
+      const int hs = p * d.st - d.pad, ws = q * d.st - d.pad;
+      for (int r = 0; r < d.k; ++r) {
+        const int h = hs + r;
+        if ((unsigned)h >= (unsigned)d.H) continue;
+        for (int s = 0; s < d.k; ++s) {
+          const int w = ws + s;
+          if ((unsigned)w < (unsigned)d.W) acc += xp[h * d.W + w];
+        }
+      }
+      y[idx] = acc * inv;
+    }
+  }
+}
+
+__global__ void pool_bwd_kernel(PoolDims d, const float* __restrict__ x, const float* __restrict__ dy,
+                                float* __restrict__ dx, const int* __restrict__ argmax) {
+  const long long total = (long long)d.N * d.C * d.H * d.W;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  const float inv = 1.0f / (float)(d.k * d.k);
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const int w = (int)(idx % d.W);
+    const long long t = idx / d.W;
+    const int h = (int)(t % d.H);
+    const long long nc = t / d.H;
+    // windows p with p*st - pad <= h <= p*st - pad + k - 1
+    const int th = h + d.pad - (d.k - 1), tw = w + d.pad - (d.k - 1);
+    const int p_lo = th > 0 ? (th + d.st - 1) / d.st : 0;
+    const int q_lo = tw > 0 ? (tw + d.st - 1) / d.st : 0;
+    int p_hi = (h + d.pad) / d.st, q_hi = (w + d.pad) / d.st;
+    if (p_hi > d.P - 1) p_hi = d.P - 1;
+    if (q_hi > d.Q - 1) q_hi = d.Q - 1;
+    const float* dyp = dy + nc * d.P * d.Q;
+    float acc = 0.0f;
+    if (d.mode == RH_POOL_MAX) {
+      const int me = h * d.W + w;
+      const float* xp = x ? x + nc * d.H * d.W : nullptr;
+      const int* ap = argmax ? argmax + nc * d.P * d.Q : nullptr;
+      for (int p = p_lo; p <= p_hi; ++p)
+        for (int q = q_lo; q <= q_hi; ++q) {
+          int bi;
+          if (ap) {
+            bi = ap[p * d.Q + q];
+          } else {
+            float best;
+            bi = window_argmax(xp, d.H, d.W, p, q, d.k, d.st, d.pad, &best);
+          }
+          if (bi == me) acc += dyp[p * d.Q + q];
+        }
+    } else {
+      for (int p = p_lo; p <= p_hi; ++p)
+        for (int q = q_lo; q <= q_hi; ++q) acc += dyp[p * d.Q + q] * inv;
+    }
+    dx[idx] = acc;
+  }
+}
+
+static int pool_dims(const rh_pool_geom* g, PoolDims* d) {
+  if (!g) return RH_E_INVALID;
+  if (g->N <= 0 || g->C <= 0 || g->H <= 0 || g->W <= 0 || g->size <= 0 || g->stride <= 0 || g->pad < 0)
+    return RH_E_INVALID;
+  if (g->mode != RH_POOL_MAX && g->mode != RH_POOL_AVG_INCL_PAD) return RH_E_INVALID;
+  if (g->round != RH_ROUND_FLOOR && g->round != RH_ROUND_CEIL) return RH_E_INVALID;
+  d->N = g->N; d->C = g->C; d->H = g->H; d->W = g->W; d->k = g->size; d->st = g->stride; d->pad = g->pad;
+  d->mode = g->mode;
+  d->P = pool_out_dim(g->H, g->size, g->stride, g->pad, g->round);
+  d->Q = pool_out_dim(g->W, g->size, g->stride, g->pad, g->round);
+  if ((long long)g->H * g->W >= (1ll << 31)) return RH_E_LIMIT;
+  return 0;
+}
+
+}  // namespace rh
+
+using namespace rh;
+
+extern "C" int32_t rh_pool2d_out_dim(int32_t in, int32_t size, int32_t stride, int32_t pad, int32_t round) {
+  if (stride <= 0) return 0;
+  return pool_out_dim(in, size, stride, pad, round);
+}
+
+extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, int32_t* opt_argmax,
+                             rh_stream_t stream) {
+  PoolDims d;
+  if (int e = pool_dims(g, &d)) return e;
+  if (!x || !y) return RH_E_INVALID;
+  const long long total = (long long)d.N * d.C * d.P * d.Q;
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(pool_fwd_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, to_stream(stream), d, x,
+                     y, opt_argmax);
+  return launch_status();
+}
+
+extern "C" int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float* y, const float* dy, float* dx,
+                             const int32_t* opt_argmax, rh_stream_t stream) {
+  (void)y;
+  PoolDims d;
+  if (int e = pool_dims(g, &d)) return e;
+  if (!dy || !dx) return RH_E_INVALID;
+  if (d.mode == RH_POOL_MAX && !opt_argmax && !x) return RH_E_INVALID;
+  const long long total = (long long)d.N * d.C * d.H * d.W;
+  hipLaunchKernelGGL(pool_bwd_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, to_stream(stream), d, x,
+                     dy, dx, opt_argmax);
+  return launch_status();
+}

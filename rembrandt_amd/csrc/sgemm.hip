@@ -1,0 +1,171 @@
+// Column-major SGEMM (K8) on the fp32 MFMA tile engine, plus the BLAS-1 calls (K14).
+//   C(m,n) = alpha * op(A)(m,k) * op(B)(k,n) + beta * C
+// The engine's lanes run along its column index, so C's contiguous index (its row im) is made the
+// engine column and C's column jn the engine row:  D[jn][im] = sum_l opB(l,jn) * opA(im,l).
+//   engine A operand (row jn): opB.  transB == 0: B[l + jn*ldb] (k contiguous); else B[jn + l*ldb].
+//   engine B operand (row im): opA.  transA == 0: A[im + l*lda] (rows contiguous); else A[l + im*lda].
+// When the result has too few tiles to fill the GPU (batch-sized GEMMs of the affine layers) and
+// scratch is given, the contraction is split across blocks and reduced in a fixed order.
+#include "conv_common.h"
+
+namespace rh {
+
+struct SgemmPlan { int bm, bn, splits; };
+
+static SgemmPlan plan_sgemm(int m, int n, int k) {
+  SgemmPlan p;
+  p.bm = pick_bm(n);
+  p.bn = p.bm == 128 ? 128 : 256;
+  const int tiles = cdiv(n, p.bm) * cdiv(m, p.bn);
+  const int k_chunks = cdiv(k, 16);
+  int want = 1;
+  if (tiles < 384) {
+    want = cdiv(768, tiles);
+    const int max_by_depth = k_chunks / 16 > 0 ? k_chunks / 16 : 1;
+    if (want > max_by_depth) want = max_by_depth;
+    if (want > 64) want = 64;
+  }
+  p.splits = want < 1 ? 1 : want;
+  return p;
+}
+
+template <class T, bool B_TRANS, bool A_TRANS>
+static int run_sgemm(const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k, int splits,
+                     int* used, hipStream_t stream) {
+  // engine A operand = opB: k contiguous unless transB; engine B operand = opA: rows contiguous unless transA
+  if constexpr (!B_TRANS && !A_TRANS)
+    return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseR<T::BN, T::BK, T::NT>, false>(
+        ap, bp, ep, k, splits, used, stream);
+  else if constexpr (!B_TRANS && A_TRANS)
+    return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseK<T::BN, T::BK, T::NT, false>, false>(
+        ap, bp, ep, k, splits, used, stream);
+  else if constexpr (B_TRANS && !A_TRANS)
+    return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseR<T::BN, T::BK, T::NT>, false>(
+        ap, bp, ep, k, splits, used, stream);
+  else
+    return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseK<T::BN, T::BK, T::NT, false>, false>(
+        ap, bp, ep, k, splits, used, stream);
+}
+
+template <bool B_TRANS, bool A_TRANS>
+static int dispatch_tile(int bm, const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k,
+                         int splits, int* used, hipStream_t stream) {
+  switch (bm) {
+    case 128: return run_sgemm<T128x128, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream);
+    case 64:  return run_sgemm<T64x256, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream);
+    default:  return run_sgemm<T32x256, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream);
+  }
+}
+
+// y[i] += alpha * x[i]
+__global__ void saxpy_kernel(long long n, float alpha, const float* __restrict__ x, float* __restrict__ y) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+  if (vec) {
+    const long long n4 = n >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    float4* y4 = reinterpret_cast<float4*>(y);
+    for (long long i = t; i < n4; i += stride) {
+      const float4 a = x4[i];
+      float4 b = y4[i];
+      b.x = fmaf(alpha, a.x, b.x); b.y = fmaf(alpha, a.y, b.y);
+      b.z = fmaf(alpha, a.z, b.z); b.w = fmaf(alpha, a.w, b.w);
+      y4[i] = b;
+    }
+    for (long long i = (n4 << 2) + t; i < n; i += stride) y[i] = fmaf(alpha, x[i], y[i]);
+  } else {
+    for (long long i = t; i < n; i += stride) y[i] = fmaf(alpha, x[i], y[i]);
+  }
+}
+
+// x[i] *= alpha
+__global__ void sscal_kernel(long long n, float alpha, float* __restrict__ x) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const long long n4 = n >> 2;
+    float4* x4 = reinterpret_cast<float4*>(x);
+    for (long long i = t; i < n4; i += stride) {
+      float4 a = x4[i];
+      a.x *= alpha; a.y *= alpha; a.z *= alpha; a.w *= alpha;
+      x4[i] = a;
+    }
+    for (long long i = (n4 << 2) + t; i < n; i += stride) x[i] *= alpha;
+  } else {
+    for (long long i = t; i < n; i += stride) x[i] *= alpha;
+  }
+}
+
+}  // namespace rh
+
+using namespace rh;
+
+extern "C" size_t rh_sgemm_workspace_bytes(int32_t m, int32_t n, int32_t k) {
+  if (m <= 0 || n <= 0 || k <= 0) return 0;
+  const SgemmPlan p = plan_sgemm(m, n, k);
+  if (p.splits <= 1) return 0;
+  return align256(sizeof(float) * (size_t)p.splits * m * n);
+}
+
+extern "C" int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k, float alpha, const float* A,
+                        int32_t lda, const float* B, int32_t ldb, float beta, float* C, int32_t ldc,
+                        void* ws, size_t ws_bytes, int flags, rh_stream_t stream_) {
+  if (m < 0 || n < 0 || k < 0 || !C) return RH_E_INVALID;
+  if (m == 0 || n == 0) return 0;
+  if (k > 0 && (!A || !B)) return RH_E_INVALID;
+  if (lda < (transA ? k : m) || ldb < (transB ? n : k) || ldc < m) return RH_E_INVALID;
+  if (flags & RH_MATH_BF16_MFMA_FP32ACC) return RH_E_UNSUPPORTED;
+  hipStream_t stream = to_stream(stream_);
+
+  const size_t a_elems = k > 0 ? (size_t)lda * ((transA ? m : k) - 1) + (transA ? k : m) : 0;
+  const size_t b_elems = k > 0 ? (size_t)ldb * ((transB ? k : n) - 1) + (transB ? n : k) : 0;
+  if (a_elems * 4 > kMaxBufferBytes || b_elems * 4 > kMaxBufferBytes ||
+      ((size_t)ldc * (n - 1) + m) * 4 > kMaxBufferBytes)
+    return RH_E_LIMIT;
+
+  DenseParams ap;  // engine A operand = opB, rows = n
+  ap.ptr = B; ap.bytes = (uint32_t)(b_elems * 4); ap.rows = n; ap.K = k; ap.ld = ldb; ap.ktab = nullptr;
+  DenseParams bp;  // engine B operand = opA, rows = m
+  bp.ptr = A; bp.bytes = (uint32_t)(a_elems * 4); bp.rows = m; bp.K = k; bp.ld = lda; bp.ktab = nullptr;
+
+  SgemmPlan plan = plan_sgemm(m, n, k);
+  const size_t need = plan.splits > 1 ? align256(sizeof(float) * (size_t)plan.splits * m * n) : 0;
+  if (plan.splits > 1 && (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255))) plan.splits = 1;
+
+  EpiParams ep;
+  ep.bias = nullptr; ep.alpha = alpha; ep.beta = beta; ep.rows = n; ep.cols = m; ep.inner = 0; ep.relu = 0;
+  if (plan.splits > 1) {
+    ep.out = static_cast<float*>(ws); ep.ld = m; ep.split_stride = (long long)m * n;
+  } else {
+    ep.out = C; ep.ld = ldc; ep.split_stride = 0;
+  }
+
+  int used = 1, e;
+  if (!transB && !transA)      e = dispatch_tile<false, false>(plan.bm, ap, bp, ep, k, plan.splits, &used, stream);
+  else if (!transB && transA)  e = dispatch_tile<false, true>(plan.bm, ap, bp, ep, k, plan.splits, &used, stream);
+  else if (transB && !transA)  e = dispatch_tile<true, false>(plan.bm, ap, bp, ep, k, plan.splits, &used, stream);
+  else                         e = dispatch_tile<true, true>(plan.bm, ap, bp, ep, k, plan.splits, &used, stream);
+  if (e) return e;
+  if (plan.splits > 1) {
+    launch_split_reduce(static_cast<const float*>(ws), used, (long long)m * n, C, n, m, ldc, alpha, beta, stream);
+    return launch_status();
+  }
+  return 0;
+}
+
+extern "C" int rh_saxpy(int64_t n, float alpha, const float* x, float* y, rh_stream_t stream) {
+  if (n < 0 || (n > 0 && (!x || !y))) return RH_E_INVALID;
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(saxpy_kernel, dim3(stream_grid((size_t)(n + 3) / 4, 256)), dim3(256), 0, to_stream(stream),
+                     (long long)n, alpha, x, y);
+  return launch_status();
+}
+
+extern "C" int rh_sscal(int64_t n, float alpha, float* x, rh_stream_t stream) {
+  if (n < 0 || (n > 0 && !x)) return RH_E_INVALID;
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(sscal_kernel, dim3(stream_grid((size_t)(n + 3) / 4, 256)), dim3(256), 0, to_stream(stream),
+                     (long long)n, alpha, x);
+  return launch_status();
+}

@@ -1,0 +1,225 @@
+"""Thin wrappers that call the C ABI on torch device tensors.
+
+torch provides device memory and the current HIP stream, nothing else: every function below
+passes raw `data_ptr()` values and sizes to librembrandt_hip.so.  Errors raise (the reference
+panics on every native error).
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import ConvGeom, PoolGeom, check, lib
+
+_ws_cache = {}
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    if t is None:
+        return C.c_void_p(0)
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensors only"
+    return C.c_void_p(t.data_ptr())
+
+
+def workspace(nbytes, device):
+    """A cached, 256-byte aligned scratch tensor of at least nbytes on `device`."""
+    key = str(device)
+    ws = _ws_cache.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        assert ws.data_ptr() % 256 == 0
+        _ws_cache[key] = ws
+    return ws
+
+
+def conv_geom(x_shape, w_shape, stride, pad):
+    N, Cc, H, W = x_shape
+    K, C2, R, S = w_shape
+    assert Cc == C2
+    return ConvGeom(N, Cc, H, W, K, R, S, stride, pad)
+
+
+def conv_out_shape(g):
+    out = lib().rh_conv2d_out_dim
+    return (g.N, g.K, out(g.H, g.R, g.stride, g.pad), out(g.W, g.S, g.stride, g.pad))
+
+
+def conv2d_fwd(x, w, stride, pad, bias=None, relu=False, alpha=1.0, beta=0.0, y=None):
+    g = conv_geom(x.shape, w.shape, stride, pad)
+    if y is None:
+        y = torch.empty(conv_out_shape(g), dtype=torch.float32, device=x.device)
+    need = lib().rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_FWD)
+    ws = workspace(need, x.device)
+    flags = (_lib.RH_FUSE_BIAS if bias is not None else 0) | (_lib.RH_FUSE_RELU if relu else 0)
+    check(lib().rh_conv2d_fwd(C.byref(g), alpha, _p(x), _p(w), beta, _p(y), _p(bias), _p(ws), ws.numel(), flags,
+                              _stream()), "rh_conv2d_fwd")
+    return y
+
+
+def conv2d_bwd_filter(x, dy, w_shape, stride, pad, alpha=1.0, beta=0.0, dw=None):
+    g = conv_geom(x.shape, w_shape, stride, pad)
+    if dw is None:
+        dw = torch.zeros(tuple(w_shape), dtype=torch.float32, device=x.device)
+    need = lib().rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_BWD_FILTER)
+    ws = workspace(need, x.device)
+    check(lib().rh_conv2d_bwd_filter(C.byref(g), alpha, _p(x), _p(dy), beta, _p(dw), _p(ws), ws.numel(), 0,
+                                     _stream()), "rh_conv2d_bwd_filter")
+    return dw
+
+
+def conv2d_bwd_bias(dy, alpha=1.0, beta=0.0, db=None):
+    N, K = dy.shape[0], dy.shape[1]
+    plane = dy.numel() // (N * K)
+    if db is None:
+        db = torch.zeros((K,), dtype=torch.float32, device=dy.device)
+    check(lib().rh_conv2d_bwd_bias(N, K, plane, alpha, _p(dy), beta, _p(db), _stream()), "rh_conv2d_bwd_bias")
+    return db
+
+
+def conv2d_bwd_data(w, dy, x_shape, stride, pad, alpha=1.0, beta=0.0, dx=None):
+    g = conv_geom(x_shape, w.shape, stride, pad)
+    if dx is None:
+        dx = torch.zeros(tuple(x_shape), dtype=torch.float32, device=w.device)
+    need = lib().rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_BWD_DATA)
+    ws = workspace(need, w.device)
+    check(lib().rh_conv2d_bwd_data(C.byref(g), alpha, _p(w), _p(dy), beta, _p(dx), _p(ws), ws.numel(), 0,
+                                   _stream()), "rh_conv2d_bwd_data")
+    return dx
+
+
+def add_bias_nchw(bias, y, alpha=1.0, beta=1.0):
+    N, K = y.shape[0], y.shape[1]
+    plane = y.numel() // (N * K)
+    check(lib().rh_add_bias_nchw(_p(bias), _p(y), plane, K, N, alpha, beta, _stream()), "rh_add_bias_nchw")
+    return y
+
+
+def _check_last(where):
+    check(lib().rh_last_error(), where)
+
+
+def rect_inplace(y):
+    lib().rembrandt_kernel_batch_map_rect_inplace(_p(y), y.numel() // y.shape[0], y.shape[0], _stream())
+    _check_last("rembrandt_kernel_batch_map_rect_inplace")
+    return y
+
+
+def rect_backprop_inplace(y, dy):
+    lib().rembrandt_kernel_batch_map_rect_backprop_inplace(_p(y), y.numel() // y.shape[0], y.shape[0], _p(dy),
+                                                           _stream())
+    _check_last("rembrandt_kernel_batch_map_rect_backprop_inplace")
+    return dy
+
+
+def sgemm(transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, use_workspace=True):
+    ws, nbytes = None, 0
+    if use_workspace:
+        nbytes = lib().rh_sgemm_workspace_bytes(m, n, k)
+        if nbytes:
+            ws = workspace(nbytes, Cm.device)
+            nbytes = ws.numel()
+    check(lib().rh_sgemm(int(transA), int(transB), m, n, k, alpha, _p(A), lda, _p(B), ldb, beta, _p(Cm), ldc,
+                         _p(ws), nbytes, 0, _stream()), "rh_sgemm")
+    return Cm
+
+
+def saxpy(alpha, x, y):
+    check(lib().rh_saxpy(x.numel(), alpha, _p(x), _p(y), _stream()), "rh_saxpy")
+    return y
+
+
+def sscal(alpha, x):
+    check(lib().rh_sscal(x.numel(), alpha, _p(x), _stream()), "rh_sscal")
+    return x
+
+
+def pool_geom(x_shape, size, stride, pad, mode, rounding=_lib.RH_ROUND_FLOOR):
+    N, Cc, H, W = x_shape
+    return PoolGeom(N, Cc, H, W, size, stride, pad, mode, rounding)
+
+
+def pool_out_shape(g):
+    out = lib().rh_pool2d_out_dim
+    return (g.N, g.C, out(g.H, g.size, g.stride, g.pad, g.round), out(g.W, g.size, g.stride, g.pad, g.round))
+
+
+def pool2d_fwd(x, size, stride, pad, mode, rounding=_lib.RH_ROUND_FLOOR, want_argmax=False):
+    g = pool_geom(x.shape, size, stride, pad, mode, rounding)
+    y = torch.empty(pool_out_shape(g), dtype=torch.float32, device=x.device)
+    am = torch.empty(y.shape, dtype=torch.int32, device=x.device) if want_argmax else None
+    check(lib().rh_pool2d_fwd(C.byref(g), _p(x), _p(y), _p(am), _stream()), "rh_pool2d_fwd")
+    return (y, am) if want_argmax else y
+
+
+def pool2d_bwd(x, y, dy, size, stride, pad, mode, rounding=_lib.RH_ROUND_FLOOR, argmax=None):
+    g = pool_geom(x.shape, size, stride, pad, mode, rounding)
+    dx = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)
+    check(lib().rh_pool2d_bwd(C.byref(g), _p(x), _p(y), _p(dy), _p(dx), _p(argmax), _stream()), "rh_pool2d_bwd")
+    return dx
+
+
+def softmax_fwd(x):
+    N, Cc = x.shape
+    p = torch.empty_like(x)
+    check(lib().rh_softmax_fwd(_p(x), _p(p), Cc, N, _stream()), "rh_softmax_fwd")
+    return p
+
+
+def softmax_kl_backward(p, labels, weights):
+    N, Cc = p.shape
+    dx = torch.empty_like(p)
+    lib().rembrandt_kernel_batch_map_softmax_kl_backward(_p(p), Cc, N, _p(labels), _p(weights), _p(dx), _stream())
+    _check_last("rembrandt_kernel_batch_map_softmax_kl_backward")
+    return dx
+
+
+def softmax_kl_loss1(p, labels, weights, beta=0.0, loss1=None):
+    N, Cc = p.shape
+    if loss1 is None:
+        loss1 = torch.zeros((N,), dtype=torch.float32, device=p.device)
+    lib().rembrandt_kernel_batch_map_softmax_kl_loss1(_p(p), Cc, N, _p(labels), _p(weights), beta, _p(loss1),
+                                                      _stream())
+    _check_last("rembrandt_kernel_batch_map_softmax_kl_loss1")
+    return loss1
+
+
+def blockreduce_sum(src, beta=0.0, dst=None):
+    batch, length = src.shape
+    if dst is None:
+        dst = torch.zeros((batch,), dtype=torch.float32, device=src.device)
+    lib().rembrandt_kernel_batch_blockreduce_sum(_p(src), length, batch, _p(dst), beta, _stream())
+    _check_last("rembrandt_kernel_batch_blockreduce_sum")
+    return dst
+
+
+def blockreduce_argmax(src):
+    batch, length = src.shape
+    mx = torch.empty((batch,), dtype=torch.float32, device=src.device)
+    idx = torch.empty((batch,), dtype=torch.int32, device=src.device)
+    lib().rembrandt_kernel_batch_blockreduce_argmax(_p(src), length, batch, _p(mx), _p(idx), _stream())
+    _check_last("rembrandt_kernel_batch_blockreduce_argmax")
+    return mx, idx
+
+
+def sgd_momentum_step(W, g, v, l2, scale, mu, apply, zero_grad=True):
+    check(lib().rh_sgd_momentum_step(W.numel(), _p(W), _p(g), _p(v), l2, scale, mu, apply, int(zero_grad),
+                                     _stream()), "rh_sgd_momentum_step")
+
+
+def descend(W, g, s, l2):
+    check(lib().rh_descend(W.numel(), _p(W), _p(g), s, l2, _stream()), "rh_descend")
+
+
+def cast_u8_f32(x, scale):
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    check(lib().rh_cast_u8_f32(_p(x), _p(y), x.numel(), scale, _stream()), "rh_cast_u8_f32")
+    return y
+
+
+def memset_f32(t, value):
+    check(lib().rh_memset_f32(_p(t), value, t.numel(), _stream()), "rh_memset_f32")
+    return t

@@ -1,0 +1,236 @@
+"""GPU parity: every C-ABI kernel against the CPU oracle on the same seeded inputs (small shapes)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from rembrandt_amd import _lib, ops, synth
+from conftest import assert_close, say
+
+pytestmark = pytest.mark.gpu
+
+
+def T(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def N(t):
+    return t.detach().cpu().numpy()
+
+
+CONV_CASES = [
+    # N, C, H, W, K, R, stride, pad
+    (2, 3, 9, 7, 4, 3, 1, 1),        # tiny, ragged everything
+    (3, 5, 13, 13, 20, 5, 1, 2),     # LeNet-like 5x5 pad 2, K=20
+    (2, 3, 35, 35, 96, 11, 4, 0),    # AlexNet conv1-like: 11x11 stride 4, K=96
+    (4, 16, 14, 14, 50, 5, 1, 2),    # K=50 -> 64-row tile
+    (2, 96, 13, 13, 256, 5, 1, 2),   # AlexNet conv2-like channels, 128-row tile, K_gemm 2400
+    (3, 40, 9, 9, 130, 3, 1, 1),     # K just above a tile boundary
+    (2, 24, 12, 12, 24, 1, 1, 0),    # 1x1
+    (2, 6, 15, 15, 10, 3, 2, 1),     # stride 2 with pad
+    (1, 4, 10, 10, 8, 3, 3, 0),      # stride 3
+    (70, 2, 6, 6, 5, 3, 1, 1),       # many images, pixel tiles straddle images
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=[str(c) for c in CONV_CASES])
+def test_conv2d_all_passes(dev, case):
+    Nn, C, H, W, K, R, st, pad = case
+    say("conv case", case)
+    x = synth.normal(11, 1, (Nn, C, H, W))
+    w = synth.normal(11, 2, (K, C, R, R))
+    b = synth.normal(11, 3, (K,))
+    y_ref = O.conv2d_fwd(x, w, st, pad)
+    dy = synth.normal(11, 4, y_ref.shape)
+    xd, wd, bd, dyd = T(x, dev), T(w, dev), T(b, dev), T(dy, dev)
+
+    y = ops.conv2d_fwd(xd, wd, st, pad)
+    assert_close(N(y), y_ref, "conv fwd")
+
+    # fused bias + relu epilogue == K1 -> K2 -> K3
+    yf = ops.conv2d_fwd(xd, wd, st, pad, bias=bd, relu=True)
+    ref_f = O.rect_inplace(O.add_bias_nchw(b, y_ref.copy()))
+    assert_close(N(yf), ref_f, "conv fwd fused bias+relu")
+
+    # alpha / beta blend
+    y0 = synth.normal(11, 5, y_ref.shape)
+    yb = ops.conv2d_fwd(xd, wd, st, pad, alpha=0.5, beta=2.0, y=T(y0, dev))
+    assert_close(N(yb), O.conv2d_fwd(x, w, st, pad, alpha=0.5, beta=2.0, y=y0.copy()), "conv fwd alpha/beta")
+
+    dw_ref = O.conv2d_bwd_filter(x, dy, w.shape, st, pad)
+    dw = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad)
+    assert_close(N(dw), dw_ref, "conv bwd filter")
+    dw0 = synth.normal(11, 6, w.shape)
+    dwa = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, alpha=1.0, beta=1.0, dw=T(dw0, dev))
+    assert_close(N(dwa), O.conv2d_bwd_filter(x, dy, w.shape, st, pad, 1.0, 1.0, dw0.copy()), "conv bwd filter beta=1")
+
+    db = ops.conv2d_bwd_bias(dyd)
+    assert_close(N(db), O.conv2d_bwd_bias(dy), "conv bwd bias")
+
+    dx_ref = O.conv2d_bwd_data(w, dy, x.shape, st, pad)
+    dx = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad)
+    assert_close(N(dx), dx_ref, "conv bwd data")
+    torch.cuda.synchronize()
+
+
+SGEMM_CASES = [
+    # transA, transB, m, n, k
+    (1, 0, 500, 64, 2450),   # affine forward  Y = W^T X
+    (0, 1, 300, 500, 64),    # affine bwd-W    dW += X dY^T
+    (0, 0, 300, 64, 500),    # affine bwd-X    dX = W dY
+    (1, 1, 37, 29, 53),
+    (0, 0, 1, 10, 64),
+    (0, 1, 1, 130, 70),      # the bias-gradient GEMV shape
+    (1, 0, 4096, 32, 1024),  # few tiles, deep contraction -> split path
+]
+
+
+@pytest.mark.parametrize("case", SGEMM_CASES, ids=[str(c) for c in SGEMM_CASES])
+@pytest.mark.parametrize("use_ws", [True, False])
+def test_sgemm(dev, case, use_ws):
+    tA, tB, m, n, k = case
+    say("sgemm case", case, "ws", use_ws)
+    a_shape = (m, k) if tA else (k, m)   # memory shape (row-major view of a column-major array)
+    b_shape = (k, n) if tB else (n, k)
+    lda, ldb, ldc = a_shape[1] + 3, b_shape[1] + 1, m + 2
+    A = synth.normal(12, 1, (a_shape[0], lda))
+    B = synth.normal(12, 2, (b_shape[0], ldb))
+    C0 = synth.normal(12, 3, (n, ldc))
+    for alpha, beta in ((1.0, 0.0), (0.5, 1.0)):
+        ref = O.sgemm(tA, tB, m, n, k, alpha, A, lda, B, ldb, beta, C0.copy(), ldc)
+        Cd = T(C0, dev)
+        ops.sgemm(tA, tB, m, n, k, alpha, T(A, dev), lda, T(B, dev), ldb, beta, Cd, ldc, use_workspace=use_ws)
+        got = N(Cd)
+        assert_close(got[:, :m], ref[:, :m], "sgemm alpha=%g beta=%g" % (alpha, beta))
+        assert np.array_equal(got[:, m:], C0[:, m:]), "sgemm wrote outside ldc padding"
+
+
+def test_bias_relu(dev):
+    for shape in [(3, 7, 5, 9), (2, 96, 27, 27), (64, 500), (5, 3, 16, 20)]:
+        say("bias/relu", shape)
+        y = synth.normal(13, 1, shape)
+        b = synth.normal(13, 2, (shape[1],))
+        yd = T(y, dev)
+        ops.add_bias_nchw(T(b, dev), yd)
+        ref = O.add_bias_nchw(b, y.copy())
+        assert_close(N(yd), ref, "add_bias")
+        ops.rect_inplace(yd)
+        ref = O.rect_inplace(ref)
+        assert np.array_equal(N(yd) > 0, ref > 0)
+        assert_close(N(yd), ref, "rect")
+        dy = synth.normal(13, 3, shape)
+        dyd = T(dy, dev)
+        ops.rect_backprop_inplace(yd, dyd)
+        assert np.array_equal(N(dyd), O.rect_backprop_inplace(ref, dy.copy())), "rect backprop is a pure mask"
+
+
+POOL_CASES = [
+    # N, C, H, size, stride, pad
+    (2, 3, 9, 3, 2, 0), (2, 3, 9, 3, 2, 1), (3, 4, 8, 2, 2, 0), (2, 2, 10, 3, 2, 0), (2, 5, 27, 3, 2, 0),
+    (1, 2, 6, 6, 1, 0), (2, 3, 7, 3, 1, 1), (2, 2, 13, 3, 3, 1),
+]
+
+
+@pytest.mark.parametrize("case", POOL_CASES, ids=[str(c) for c in POOL_CASES])
+@pytest.mark.parametrize("mode", [_lib.RH_POOL_MAX, _lib.RH_POOL_AVG_INCL_PAD])
+@pytest.mark.parametrize("rounding", [_lib.RH_ROUND_FLOOR, _lib.RH_ROUND_CEIL])
+def test_pool2d(dev, case, mode, rounding):
+    Nn, C, H, k, st, pad = case
+    say("pool case", case, mode, rounding)
+    x = synth.normal(14, 1, (Nn, C, H, H + 1))
+    # repeated values so that the first-maximum tie rule is exercised
+    x = np.round(x * 2) / 2
+    y_ref, am_ref = O.pool2d_fwd(x, k, st, pad, mode, rounding, want_argmax=True)
+    if y_ref.size == 0:
+        pytest.skip("empty output")
+    xd = T(x, dev)
+    y, am = ops.pool2d_fwd(xd, k, st, pad, mode, rounding, want_argmax=True)
+    assert_close(N(y), y_ref, "pool fwd")
+    if mode == _lib.RH_POOL_MAX:
+        assert np.array_equal(N(am), am_ref), "arg-max mask is bit-exact"
+    dy = synth.normal(14, 2, y_ref.shape)
+    dx_ref = O.pool2d_bwd(x, y_ref, dy, k, st, pad, mode, rounding)
+    dx = ops.pool2d_bwd(xd, y, T(dy, dev), k, st, pad, mode, rounding)
+    assert_close(N(dx), dx_ref, "pool bwd (recomputed arg-max)")
+    if mode == _lib.RH_POOL_MAX:
+        dx2 = ops.pool2d_bwd(xd, y, T(dy, dev), k, st, pad, mode, rounding, argmax=am)
+        assert np.array_equal(N(dx2), N(dx)), "mask-driven backward equals recomputed"
+
+
+@pytest.mark.parametrize("shape", [(64, 10), (256, 1000), (7, 1), (3, 5000)])
+def test_softmax_loss_argmax(dev, shape):
+    Nn, C = shape
+    say("softmax case", shape)
+    x = synth.normal(15, 1, shape, 0.0, 3.0)
+    labels = synth.integers(15, 2, (Nn,), C)
+    weights = synth.uniform(15, 3, (Nn,), 0.1, 1.0)
+    xd, ld, wd = T(x, dev), T(labels, dev), T(weights, dev)
+    p_ref = O.softmax_fwd(x)
+    p = ops.softmax_fwd(xd)
+    assert_close(N(p), p_ref, "softmax", atol=1e-7)
+    d = ops.softmax_kl_backward(p, ld, wd)
+    assert_close(N(d), O.softmax_kl_backward(N(p), labels, weights), "kl backward", atol=1e-7)
+    l1 = ops.softmax_kl_loss1(p, ld, wd)
+    l1_ref = O.softmax_kl_loss1(N(p), labels, weights)
+    assert_close(N(l1), l1_ref, "kl loss1")
+    l1b = ops.softmax_kl_loss1(p, ld, wd, beta=1.0, loss1=l1.clone())
+    assert_close(N(l1b), 2 * l1_ref, "kl loss1 accumulate")
+    tot = ops.blockreduce_sum(l1.reshape(1, Nn))
+    assert_close(N(tot), O.blockreduce_sum(N(l1).reshape(1, Nn)), "loss sum")
+    mx, idx = ops.blockreduce_argmax(p)
+    mx_ref, idx_ref = O.blockreduce_argmax(N(p))
+    assert np.array_equal(N(idx), idx_ref), "arg-max is bit-exact"
+    assert np.array_equal(N(mx), mx_ref)
+
+
+def test_argmax_ties(dev):
+    x = np.zeros((4, 700), np.float32)
+    x[0, [5, 300, 699]] = 2.0
+    x[1, :] = 1.0
+    x[2, 699] = 3.0
+    x[3, [64, 65]] = 7.0
+    mx, idx = ops.blockreduce_argmax(T(x, dev))
+    assert N(idx).tolist() == [5, 0, 699, 64]
+    assert N(mx).tolist() == [2.0, 1.0, 3.0, 7.0]
+
+
+@pytest.mark.parametrize("n", [1, 5, 1000, 1 << 20 | 3])
+def test_blas1_sgd(dev, n):
+    say("blas1/sgd n", n)
+    x = synth.normal(16, 1, (n,))
+    y = synth.normal(16, 2, (n,))
+    yd = T(y, dev)
+    ops.saxpy(0.25, T(x, dev), yd)
+    assert_close(N(yd), O.saxpy(0.25, x, y.copy()), "saxpy")
+    ops.sscal(-1.5, yd)
+    assert_close(N(yd), O.sscal(-1.5, O.saxpy(0.25, x, y.copy())), "sscal")
+    # unaligned views
+    if n > 8:
+        yd2 = T(y, dev)
+        ops.saxpy(2.0, T(x, dev)[1:], yd2[1:])
+        assert_close(N(yd2)[1:], O.saxpy(2.0, x[1:].copy(), y[1:].copy()), "saxpy unaligned")
+        assert N(yd2)[0] == y[0]
+    W, g, v = synth.normal(16, 3, (n,)), synth.normal(16, 4, (n,)), synth.normal(16, 5, (n,))
+    for (l2, scale, mu, apply, zg) in [(5e-4, -0.01, 0.9, 1.0, True), (0.0, 1.0, 0.9, -0.01, False)]:
+        Wd, gd, vd = T(W, dev), T(g, dev), T(v, dev)
+        ops.sgd_momentum_step(Wd, gd, vd, l2, scale, mu, apply, zg)
+        Wr, gr, vr = W.copy(), g.copy(), v.copy()
+        O.sgd_momentum_step(Wr, gr, vr, l2, scale, mu, apply, zg)
+        assert_close(N(Wd), Wr, "sgd W", atol=1e-7)
+        assert_close(N(vd), vr, "sgd v", atol=1e-7)
+        assert_close(N(gd), gr, "sgd g", atol=1e-7)
+    Wd, gd = T(W, dev), T(g, dev)
+    ops.descend(Wd, gd, 0.05, 1e-3)
+    Wr, gr = W.copy(), g.copy()
+    O.descend(Wr, gr, 0.05, 1e-3)
+    assert_close(N(Wd), Wr, "descend W", atol=1e-7)
+    assert_close(N(gd), gr, "descend g", atol=1e-7)
+
+
+def test_cast_and_fill(dev):
+    x = (synth.integers(17, 1, (1000003,), 256)).astype(np.uint8)
+    y = ops.cast_u8_f32(T(x, dev), 1.0 / 255.0)
+    assert np.array_equal(N(y), O.cast_u8_f32(x, 1.0 / 255.0))
+    t = torch.empty(1027, device=dev)
+    ops.memset_f32(t[1:], 1.0)
+    assert (N(t)[1:] == 1.0).all()
