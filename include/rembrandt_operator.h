@@ -1,0 +1,117 @@
+/*
+ * rembrandt_operator.h -- C ABI of the operator / graph / optimizer layer of librembrandt_hip.so.
+ *
+ * This is what a binding of the reference's *upper* boundary talks to: the Rust operator API
+ * (Operator / InputOperator / LossOperator traits, src/operator/mod.rs:61-109 and
+ * src/operator/loss.rs:20-39), the SequentialOperatorConfig builder and
+ * SequentialOperatorWorker (src/operator/worker.rs:133-477) and the SGD policy
+ * (src/opt/sgd/mod.rs:20-147, src/opt/sgd/new.rs:345-495).  Each function names the reference
+ * method it stands for.  Dimension triples are (width, height, channels) as in the reference.
+ *
+ * Every function returns 0 on success.  The reference panics on errors; here a failed
+ * precondition or native error returns RHO_E_PANIC and the text of the panic can be read with
+ * rho_last_message() (per thread).
+ */
+#ifndef REMBRANDT_OPERATOR_H
+#define REMBRANDT_OPERATOR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RHO_E_PANIC (-100)
+
+typedef struct rho_config rho_config; /* SequentialOperatorConfig */
+typedef struct rho_worker rho_worker; /* SequentialOperatorWorker + its DeviceContext */
+typedef struct rho_sgd rho_sgd;       /* SgdOpt (update block only) */
+
+const char* rho_last_message(void);
+
+/* enums: ActivationFunction (mod.rs:282-288), ParamsInit (mod.rs:290-297), PoolOperation (mod.rs:2005-2009),
+ * OpCapability (mod.rs:233-259), Momentum (opt/sgd/mod.rs:140-147), StepSizeSchedule (opt/sgd/mod.rs:44-80) */
+enum { RHO_ACT_IDENTITY = 0, RHO_ACT_RECT = 1, RHO_ACT_LOGISTIC = 2, RHO_ACT_TANH = 3 };
+enum { RHO_INIT_DISABLED = 0, RHO_INIT_UNIFORM = 1, RHO_INIT_NORMAL = 2, RHO_INIT_XAVIER = 3, RHO_INIT_KAIMING_FWD = 4 };
+enum { RHO_POOL_MAX = 0, RHO_POOL_AVERAGE = 1 };
+enum { RHO_CAP_FORWARD = 0, RHO_CAP_BACKWARD = 1 };
+enum { RHO_MOM_ZERO = 0, RHO_MOM_UPDATE = 1, RHO_MOM_UPDATE_NESTEROV = 2, RHO_MOM_GRADIENT = 3, RHO_MOM_GRADIENT_NESTEROV = 4 };
+enum { RHO_STEP_CONSTANT = 0, RHO_STEP_ANNEAL1 = 1, RHO_STEP_ANNEAL2 = 2, RHO_STEP_ANNEAL4 = 3, RHO_STEP_DECAY = 4, RHO_STEP_INVERSE = 5 };
+/* buffers of an operator, for rho_worker_buffer */
+enum { RHO_BUF_OUT_ACT = 0, RHO_BUF_OUT_DELTA = 1, RHO_BUF_WEIGHTS = 2, RHO_BUF_BIAS = 3, RHO_BUF_GRAD_WEIGHTS = 4,
+       RHO_BUF_GRAD_BIAS = 5, RHO_BUF_ACC_GRAD_WEIGHTS = 6, RHO_BUF_ACC_GRAD_BIAS = 7 };
+
+/* ---- SequentialOperatorConfig builder (worker.rs:133-228) ---- */
+int rho_config_new(rho_config** out);                                       /* ::new()            */
+int rho_config_free(rho_config* cfg);
+int rho_config_data3d(rho_config* cfg, int32_t w, int32_t h, int32_t c, int normalize);                /* .data3d()  */
+int rho_config_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t conv_size,
+                      int32_t conv_stride, int32_t conv_pad, int32_t out_channels, int act_func, int init_kind,
+                      float init_value);                                                              /* .conv2d()  */
+int rho_config_affine(rho_config* cfg, int32_t in_channels, int32_t out_channels, int act_func, int init_kind,
+                      float init_value);                                                              /* .affine()  */
+int rho_config_pool2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t pool_size,
+                      int32_t pool_stride, int32_t pool_pad, int pool_op, int ceil_mode);              /* .pool2d()  */
+int rho_config_softmax_kl_loss(rho_config* cfg, int32_t num_categories);                              /* .softmax_kl_loss() */
+int rho_config_params_len(const rho_config* cfg, int64_t* out);                                       /* .params_len() */
+/* Parses a `.model` file of the reference's grammar (src/config.rs:16-264) into a config.
+ * batch-independent; returns the input dims through the config's data3d entry. */
+int rho_config_from_model_file(const char* path, rho_config** out);
+
+/* ---- SequentialOperatorWorker (worker.rs:230-477) ---- */
+/* into_worker(): builds the chain on `device`.  fuse_epilogue != 0 folds bias+ReLU into the conv epilogue. */
+int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1,
+                   int device, int fuse_epilogue, rho_worker** out);
+int rho_worker_free(rho_worker* w);
+int rho_worker_hidden_count(rho_worker* w, int32_t* out);
+int rho_worker_op_kind(rho_worker* w, int32_t hidden_idx, const char** out);
+void* rho_worker_stream(rho_worker* w);                                      /* ctx.stream.ptr */
+int rho_worker_sync(rho_worker* w);                                          /* ctx.sync()     */
+int rho_worker_init_params(rho_worker* w, uint64_t seed0, uint64_t seed1);   /* Operator::init_params */
+/* InputOperator (mod.rs:101-109) */
+int rho_worker_expose_host_frame_buf(rho_worker* w, int32_t batch_idx, uint8_t** out);
+int rho_worker_load_frames(rho_worker* w, int32_t batch_size);
+int rho_worker_load_frames_f32(rho_worker* w, const float* host, int32_t batch_size);
+/* LossOperator (loss.rs:20-39) */
+int rho_worker_stage_label(rho_worker* w, int32_t batch_idx, int32_t category);
+int rho_worker_load_labels(rho_worker* w, int32_t batch_size);
+int rho_worker_stage_weight(rho_worker* w, int32_t batch_idx, float weight);
+int rho_worker_load_weights(rho_worker* w, int32_t batch_size);
+int rho_worker_store_loss(rho_worker* w, int32_t batch_size, float* out);
+int rho_worker_store_output_categories(rho_worker* w, int32_t batch_size);
+int rho_worker_get_output_categories(rho_worker* w, int32_t batch_size, int32_t* host_out);
+int rho_worker_accuracy_count(rho_worker* w, int32_t batch_size, int32_t* out);
+/* Operator (mod.rs:61-99), fanned out over the chain as in worker.rs:356-477 */
+int rho_worker_forward(rho_worker* w, int32_t batch_size, int training, int64_t t);
+int rho_worker_backward(rho_worker* w, int32_t batch_size);
+int rho_worker_regularize(rho_worker* w, float l2_reg_coef);
+int rho_worker_accumulate_grads(rho_worker* w, float scale, float momentum);
+int rho_worker_update_params(rho_worker* w, float scale);
+int rho_worker_update_params2(rho_worker* w, float grad_scale, float update_scale);
+int rho_worker_save_params(rho_worker* w);
+int rho_worker_restore_params(rho_worker* w);
+int rho_worker_reset(rho_worker* w);
+/* Device view of one buffer of hidden operator `hidden_idx` (-1: input operator's out_act,
+ * hidden_count: the loss operator's probabilities).  Returns RHO_E_PANIC if there is no such buffer. */
+int rho_worker_buffer(rho_worker* w, int32_t hidden_idx, int which, float** dptr, int64_t* len);
+/* Blocking copies between host memory and such a buffer (sync_store / sync_load). */
+int rho_worker_read_buffer(rho_worker* w, int32_t hidden_idx, int which, float* host, int64_t len);
+int rho_worker_write_buffer(rho_worker* w, int32_t hidden_idx, int which, const float* host, int64_t len);
+
+/* ---- SgdOpt update block (opt/sgd/new.rs:345-495, 623-633) ---- */
+int rho_sgd_new(int32_t minibatch_size, int step_kind, const float* steps, const int64_t* step_iters, int momentum_kind,
+                float mu, float l2_reg_coef, rho_sgd** out);
+int rho_sgd_free(rho_sgd* s);
+int rho_sgd_begin(rho_sgd* s, rho_worker* w);
+int rho_sgd_step(rho_sgd* s, rho_worker* w, int fused);
+int rho_sgd_iter_counter(rho_sgd* s, int64_t* out);
+int rho_sgd_step_size_at(rho_sgd* s, int64_t t, float* out);                 /* StepSizeSchedule::at_iter */
+/* One whole training step on a staged batch, in the order of SgdOpt::train (new.rs:325-343 + the
+ * update block): forward, store_output_categories, store_loss, backward, accuracy_count, step. */
+int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused, float* loss_out, int32_t* correct_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* REMBRANDT_OPERATOR_H */

@@ -1,0 +1,295 @@
+"""CPU restatement of the reference's sequential operator chain and SGD update block.
+
+TEST INFRASTRUCTURE ONLY (see oracle.c).  numpy arrays + the C oracle; one class per reference
+operator, same method names and the same order of operations as the Rust sources:
+
+  Conv2dOperator::forward/backward ........ src/operator/mod.rs:1663-1795
+  AffineOperator::forward/backward ........ src/operator/mod.rs:1075-1176
+  Pool2dOperator::forward/backward ........ src/operator/mod.rs:2103-2123
+  SoftmaxKLLossOperator ................... src/operator/loss.rs:118-261
+  regularize / accumulate_grads / update_params / update_params2 / reset
+                                            src/operator/mod.rs:1178-1236, 1355-1363
+  SequentialOperatorWorker fan-out ........ src/operator/worker.rs:356-477
+  SgdOpt update block ..................... src/opt/sgd/new.rs:345-495, 623-633
+
+`fast=True` switches the contractions to the fp32 im2col + SGEMM family (the timed CPU baseline);
+the default is the fp64-accumulating family (the parity checker).
+"""
+import numpy as np
+
+import oracle as O
+
+
+class _Params:
+    def __init__(self, w_shape, b_len):
+        self.weights = np.zeros(w_shape, np.float32)
+        self.bias = np.zeros((b_len,), np.float32)
+        self.grad_weights = np.zeros(w_shape, np.float32)
+        self.grad_bias = np.zeros((b_len,), np.float32)
+        self.acc_grad_weights = np.zeros(w_shape, np.float32)
+        self.acc_grad_bias = np.zeros((b_len,), np.float32)
+        self.save_weights = np.zeros(w_shape, np.float32)
+        self.save_bias = np.zeros((b_len,), np.float32)
+
+    def regularize(self, l2):
+        assert l2 >= 0.0
+        if l2 > 0.0:  # weights *and bias*: mod.rs:1186-1189
+            O.saxpy(l2, self.weights, self.grad_weights)
+            O.saxpy(l2, self.bias, self.grad_bias)
+
+    def accumulate_grads(self, scale, momentum):
+        O.sscal(momentum, self.acc_grad_weights)
+        O.sscal(momentum, self.acc_grad_bias)
+        O.saxpy(scale, self.grad_weights, self.acc_grad_weights)
+        O.saxpy(scale, self.grad_bias, self.acc_grad_bias)
+
+    def update_params(self, scale):
+        O.saxpy(scale, self.acc_grad_weights, self.weights)
+        O.saxpy(scale, self.acc_grad_bias, self.bias)
+
+    def update_params2(self, grad_scale, update_scale):
+        if grad_scale != 0.0:
+            O.saxpy(grad_scale, self.grad_weights, self.weights)
+            O.saxpy(grad_scale, self.grad_bias, self.bias)
+        if update_scale != 0.0:
+            O.saxpy(update_scale, self.acc_grad_weights, self.weights)
+            O.saxpy(update_scale, self.acc_grad_bias, self.bias)
+
+    def save_params(self):
+        self.save_weights[...] = self.weights
+        self.save_bias[...] = self.bias
+
+    def restore_params(self):
+        self.weights[...] = self.save_weights
+        self.bias[...] = self.save_bias
+
+    def reset(self):
+        O.sscal(0.0, self.grad_weights)
+        O.sscal(0.0, self.grad_bias)
+
+
+class Conv2dOperator:
+    kind = "Conv2dOperator"
+
+    def __init__(self, batch, in_dims, conv_size, conv_stride, conv_pad, out_channels, act_func, fast=False):
+        w, h, c = in_dims
+        self.x_shape = (batch, c, h, w)
+        self.stride, self.pad, self.act, self.fast = conv_stride, conv_pad, act_func, fast
+        self.p = _Params((out_channels, c, conv_size, conv_size), out_channels)
+        P = O.out_dim(h, conv_size, conv_stride, conv_pad)
+        Q = O.out_dim(w, conv_size, conv_stride, conv_pad)
+        self.out_dims = (Q, P, out_channels)
+        self.out_act = np.zeros((batch, out_channels, P, Q), np.float32)
+        self.out_delta = np.zeros_like(self.out_act)
+
+    def forward(self, in_act):
+        self.in_act = in_act
+        if self.fast:
+            self.out_act = O.fast_conv2d_fwd(in_act, self.p.weights, self.stride, self.pad)
+        else:
+            O.conv2d_fwd(in_act, self.p.weights, self.stride, self.pad, y=self.out_act)
+        O.add_bias_nchw(self.p.bias, self.out_act)
+        if self.act == "Rect":
+            O.rect_inplace(self.out_act)
+        return self.out_act
+
+    def backward(self, want_in_delta):
+        if self.act == "Rect":
+            O.rect_backprop_inplace(self.out_act, self.out_delta)
+        if self.fast:
+            O.fast_conv2d_bwd_filter(self.in_act, self.out_delta, self.p.grad_weights, self.stride, self.pad)
+        else:
+            O.conv2d_bwd_filter(self.in_act, self.out_delta, self.p.weights.shape, self.stride, self.pad, 1.0, 1.0,
+                                self.p.grad_weights)
+        O.conv2d_bwd_bias(self.out_delta, 1.0, 1.0, self.p.grad_bias)
+        if not want_in_delta:
+            return None
+        if self.fast:
+            return O.fast_conv2d_bwd_data(self.p.weights, self.out_delta, self.x_shape, self.stride, self.pad)
+        return O.conv2d_bwd_data(self.p.weights, self.out_delta, self.x_shape, self.stride, self.pad)
+
+
+class AffineOperator:
+    kind = "AffineOperator"
+
+    def __init__(self, batch, in_channels, out_channels, act_func, fast=False):
+        self.batch, self.i, self.o, self.act, self.fast = batch, in_channels, out_channels, act_func, fast
+        self.p = _Params((out_channels, in_channels), out_channels)  # (in, out) column-major = [out][in]
+        self.out_dims = (1, 1, out_channels)
+        self.out_act = np.zeros((batch, out_channels), np.float32)
+        self.out_delta = np.zeros_like(self.out_act)
+
+    def forward(self, in_act):
+        x = np.ascontiguousarray(in_act.reshape(self.batch, self.i))
+        self.in_act = x
+        if self.fast:
+            self.out_act = O.fast_gemm_rm(x, self.p.weights, transB=True)
+        else:  # out_act(out,B) = W(in,out)^T * X(in,B)
+            O.sgemm(1, 0, self.o, self.batch, self.i, 1.0, self.p.weights, self.i, x, self.i, 0.0, self.out_act, self.o)
+        O.add_bias_nchw(self.p.bias, self.out_act)
+        if self.act == "Rect":
+            O.rect_inplace(self.out_act)
+        return self.out_act
+
+    def backward(self, want_in_delta):
+        if self.act == "Rect":
+            O.rect_backprop_inplace(self.out_act, self.out_delta)
+        if self.fast:
+            O.fast_gemm_rm(self.out_delta, self.in_act, transA=True, out=self.p.grad_weights, accumulate=True)
+        else:  # dW(in,out) += X(in,B) * dY(out,B)^T
+            O.sgemm(0, 1, self.i, self.o, self.batch, 1.0, self.in_act, self.i, self.out_delta, self.o, 1.0,
+                    self.p.grad_weights, self.i)
+        O.conv2d_bwd_bias(self.out_delta, 1.0, 1.0, self.p.grad_bias)  # 1(1,B) * dY^T
+        if not want_in_delta:
+            return None
+        if self.fast:
+            return O.fast_gemm_rm(self.out_delta, self.p.weights)
+        dx = np.zeros((self.batch, self.i), np.float32)  # dX(in,B) = W(in,out) * dY(out,B)
+        O.sgemm(0, 0, self.i, self.batch, self.o, 1.0, self.p.weights, self.i, self.out_delta, self.o, 0.0, dx, self.i)
+        return dx
+
+
+class Pool2dOperator:
+    kind = "Pool2dOperator"
+    p = None
+
+    def __init__(self, batch, in_dims, pool_size, pool_stride, pool_pad, pool_op, ceil_mode=False):
+        w, h, c = in_dims
+        self.x_shape = (batch, c, h, w)
+        self.k, self.st, self.pad = pool_size, pool_stride, pool_pad
+        self.mode = O.POOL_MAX if pool_op == "Max" else O.POOL_AVG
+        self.rounding = O.ROUND_CEIL if ceil_mode else O.ROUND_FLOOR
+        g = O.pool_geom(self.x_shape, pool_size, pool_stride, pool_pad, self.mode, self.rounding)
+        shp = O.pool_out_shape(g)
+        self.out_dims = (shp[3], shp[2], c)
+        self.out_act = np.zeros(shp, np.float32)
+        self.out_delta = np.zeros(shp, np.float32)
+
+    def forward(self, in_act):
+        self.in_act = np.ascontiguousarray(in_act.reshape(self.x_shape))
+        self.out_act = O.pool2d_fwd(self.in_act, self.k, self.st, self.pad, self.mode, self.rounding)
+        return self.out_act
+
+    def backward(self, want_in_delta):
+        if not want_in_delta:
+            return None
+        return O.pool2d_bwd(self.in_act, self.out_act, self.out_delta, self.k, self.st, self.pad, self.mode, self.rounding)
+
+
+class SequentialOperatorWorker:
+    """layers: list of tuples mirroring the SequentialOperatorConfig builder calls, e.g.
+    ("conv2d", in_dims, size, stride, pad, out_channels, act), ("pool2d", in_dims, size, stride, pad, op, ceil),
+    ("affine", in, out, act); num_categories closes the chain with SoftmaxKLLoss."""
+
+    def __init__(self, layers, num_categories, batch, fast=False):
+        self.batch, self.C = batch, num_categories
+        self.hidden = []
+        for l in layers:
+            if l[0] == "conv2d":
+                self.hidden.append(Conv2dOperator(batch, *l[1:], fast=fast))
+            elif l[0] == "affine":
+                self.hidden.append(AffineOperator(batch, *l[1:], fast=fast))
+            elif l[0] == "pool2d":
+                self.hidden.append(Pool2dOperator(batch, *l[1:]))
+            else:
+                raise ValueError(l[0])
+        self.labels = np.zeros((batch,), np.int32)
+        self.weights = np.zeros((batch,), np.float32)
+        self.out_cats = np.zeros((batch,), np.int32)
+
+    def params_len(self):
+        return sum(op.p.weights.size + op.p.bias.size for op in self.hidden if op.p is not None)
+
+    def stage_batch(self, labels, weight):
+        self.labels[...] = labels
+        self.weights[...] = weight
+
+    def forward(self, frames):
+        act = frames
+        for op in self.hidden:
+            act = op.forward(act)
+        self.out_values = O.softmax_fwd(np.ascontiguousarray(act.reshape(self.batch, self.C)))
+
+    def store_output_categories(self):
+        _, self.out_cats = O.blockreduce_argmax(self.out_values)
+        return self.out_cats
+
+    def store_loss(self):
+        loss1 = O.softmax_kl_loss1(self.out_values, self.labels, self.weights)
+        return float(O.blockreduce_sum(loss1.reshape(1, -1))[0])
+
+    def accuracy_count(self):
+        return O.accuracy_count(self.labels, self.out_cats)
+
+    def backward(self):
+        delta = O.softmax_kl_backward(self.out_values, self.labels, self.weights)
+        for i in range(len(self.hidden) - 1, -1, -1):
+            op = self.hidden[i]
+            op.out_delta = np.ascontiguousarray(delta.reshape(op.out_act.shape))
+            delta = op.backward(want_in_delta=i > 0)  # the input operator exposes no deltas (mod.rs:632-634)
+
+    def _each(self, fn, *a):
+        for op in self.hidden:
+            if op.p is not None:
+                getattr(op.p, fn)(*a)
+
+    def regularize(self, l2): self._each("regularize", l2)
+    def accumulate_grads(self, scale, momentum): self._each("accumulate_grads", scale, momentum)
+    def update_params(self, scale): self._each("update_params", scale)
+    def update_params2(self, g, u): self._each("update_params2", g, u)
+    def save_params(self): self._each("save_params")
+    def restore_params(self): self._each("restore_params")
+    def reset(self): self._each("reset")
+
+
+def step_size_at(schedule, t):
+    """StepSizeSchedule::at_iter, src/opt/sgd/mod.rs:82-132."""
+    kind = schedule["kind"]
+    s, it = schedule.get("steps", []), schedule.get("iters", [])
+    if kind == "Constant":
+        return s[0]
+    if kind == "Anneal1":
+        return s[0] if t < it[1] else s[1]
+    if kind == "Anneal2":
+        return s[0] if t < it[1] else s[1] if t < it[2] else s[2]
+    if kind == "Anneal4":
+        return s[0] if t < it[1] else s[1] if t < it[2] else s[2] if t < it[3] else s[3] if t < it[4] else s[4]
+    if kind == "Inverse":
+        return np.float32(s[0]) / (np.float32(1.0) + np.float32(s[0]) * np.float32(s[1]) * np.float32(t))
+    raise NotImplementedError(kind)
+
+
+class SgdOpt:
+    def __init__(self, step_size=0.01, momentum=("Update", 0.9), l2_reg_coef=0.0):
+        self.step_size = np.float32(step_size)
+        self.kind, self.mu = (momentum, 0.0) if isinstance(momentum, str) else momentum
+        self.mu = np.float32(self.mu)
+        self.l2 = np.float32(l2_reg_coef)
+        self.iter_counter = 0
+
+    def begin(self, op):
+        if self.kind == "UpdateNesterov":
+            op.update_params(self.mu)
+        op.reset()
+
+    def step(self, op):
+        step, mu = float(self.step_size), float(self.mu)
+        op.regularize(float(self.l2))
+        if self.kind == "UpdateNesterov" and self.iter_counter > 0:
+            op.update_params(-mu)
+        self.iter_counter += 1
+        if self.kind == "Zero":
+            op.accumulate_grads(-step, 0.0)
+        elif self.kind in ("Update", "UpdateNesterov"):
+            op.accumulate_grads(-step, mu)
+        else:
+            op.accumulate_grads(1.0, mu)
+        if self.kind in ("Zero", "Update", "UpdateNesterov"):
+            op.update_params(1.0)
+        elif self.kind == "Gradient":
+            op.update_params(-step)
+        else:
+            op.update_params2(-step, float(np.float32(-step) * self.mu))
+        op.reset()
+        if self.kind == "UpdateNesterov":
+            op.update_params(mu)

@@ -55,10 +55,10 @@ int32_t orc_out_dim_floor(int32_t in, int32_t size, int32_t stride, int32_t pad)
   return t / stride;
 }
 
-/* Gen-1 pooling extent (ceil): (in + 2*pad - size + stride - 1)/stride + 1 (src/layer.rs:1741-1747). */
+/* Gen-1 pooling extent (ceil): max(0, in + 2*pad - size + stride - 1)/stride + 1 (src/layer.rs:1741-1747). */
 int32_t orc_out_dim_ceil(int32_t in, int32_t size, int32_t stride, int32_t pad) {
   int32_t t = in + 2 * pad - size + stride - 1;
-  if (t < 0) return 0;
+  if (t < 0) t = 0;
   return t / stride + 1;
 }
 

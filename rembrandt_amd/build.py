@@ -28,7 +28,7 @@ def sources():
 def _compile(src):
     rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
     obj = os.path.join(OBJ, rel + ".o")
-    cmd = [HIPCC] + FLAGS + (["-x", "hip"] if src.endswith(".cpp") else []) + ["-c", src, "-o", obj]
+    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     log = "\n".join(l for l in p.stdout.splitlines() if "packed-fp32-ops" not in l)
     if p.returncode != 0:

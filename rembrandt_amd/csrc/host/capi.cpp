@@ -1,0 +1,263 @@
+// C ABI of the operator / graph / optimizer layer (include/rembrandt_operator.h).
+#include <memory>
+#include <string>
+
+#include "../../../include/rembrandt_operator.h"
+#include "model_config.hpp"
+#include "operator.hpp"
+
+using namespace rembrandt;
+
+struct rho_config { SequentialOperatorConfig cfg; };
+struct rho_worker {
+  std::shared_ptr<DeviceContext> ctx;
+  std::unique_ptr<SequentialOperatorWorker> worker;
+};
+struct rho_sgd { std::unique_ptr<SgdOpt> opt; };
+
+static thread_local std::string g_message;
+
+#define RHO_TRY(...)                                    \
+  try { __VA_ARGS__; return 0; }                        \
+  catch (const std::exception& e) { g_message = e.what(); return RHO_E_PANIC; } \
+  catch (...) { g_message = "unknown exception"; return RHO_E_PANIC; }
+
+#define RHO_REQ(cond) do { if (!(cond)) panic(std::string("invalid argument: ") + #cond); } while (0)
+
+static ActivationFunction act_of(int a) {
+  switch (a) {
+    case RHO_ACT_IDENTITY: return ActivationFunction::Identity;
+    case RHO_ACT_RECT: return ActivationFunction::Rect;
+    case RHO_ACT_LOGISTIC: return ActivationFunction::Logistic;
+    case RHO_ACT_TANH: return ActivationFunction::Tanh;
+  }
+  panic("unknown activation function");
+}
+static ParamsInit init_of(int kind, float v) {
+  switch (kind) {
+    case RHO_INIT_DISABLED: return ParamsInit::MakeDisabled();
+    case RHO_INIT_UNIFORM: return ParamsInit::MakeUniform(v);
+    case RHO_INIT_NORMAL: return ParamsInit::MakeNormal(v);
+    case RHO_INIT_XAVIER: return ParamsInit::MakeXavier();
+    case RHO_INIT_KAIMING_FWD: return ParamsInit::MakeKaimingFwd();
+  }
+  panic("unknown params init");
+}
+
+static Operator* op_at(rho_worker* w, int32_t idx) {
+  RHO_REQ(w && w->worker);
+  const int32_t n = (int32_t)w->worker->hidden_count();
+  if (idx == -1) return w->worker->input_operator();
+  if (idx == n) return w->worker->loss_operator(0);
+  RHO_REQ(idx >= 0 && idx < n);
+  return w->worker->hidden_operator((size_t)idx);
+}
+
+extern "C" {
+
+const char* rho_last_message(void) { return g_message.c_str(); }
+
+int rho_config_new(rho_config** out) { RHO_TRY({ RHO_REQ(out); *out = new rho_config(); }) }
+int rho_config_free(rho_config* cfg) { RHO_TRY({ delete cfg; }) }
+
+int rho_config_data3d(rho_config* cfg, int32_t w, int32_t h, int32_t c, int normalize) {
+  RHO_TRY({
+    RHO_REQ(cfg && w > 0 && h > 0 && c > 0);
+    Data3dOperatorConfig d = {{(size_t)w, (size_t)h, (size_t)c}, normalize != 0};
+    cfg->cfg.data3d(d);
+  })
+}
+int rho_config_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t conv_size, int32_t conv_stride,
+                      int32_t conv_pad, int32_t out_channels, int act_func, int init_kind, float init_value) {
+  RHO_TRY({
+    RHO_REQ(cfg && in_w > 0 && in_h > 0 && in_c > 0 && conv_size > 0 && conv_stride > 0 && conv_pad >= 0 && out_channels > 0);
+    Conv2dOperatorConfig c = {{(size_t)in_w, (size_t)in_h, (size_t)in_c}, (size_t)conv_size, (size_t)conv_stride,
+                              (size_t)conv_pad, (size_t)out_channels, act_of(act_func), init_of(init_kind, init_value)};
+    cfg->cfg.conv2d(c);
+  })
+}
+int rho_config_affine(rho_config* cfg, int32_t in_channels, int32_t out_channels, int act_func, int init_kind, float init_value) {
+  RHO_TRY({
+    RHO_REQ(cfg && in_channels > 0 && out_channels > 0);
+    AffineOperatorConfig a = {(size_t)in_channels, (size_t)out_channels, act_of(act_func), init_of(init_kind, init_value)};
+    cfg->cfg.affine(a);
+  })
+}
+int rho_config_pool2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t pool_size, int32_t pool_stride,
+                      int32_t pool_pad, int pool_op, int ceil_mode) {
+  RHO_TRY({
+    RHO_REQ(cfg && in_w > 0 && in_h > 0 && in_c > 0 && pool_size > 0 && pool_stride > 0 && pool_pad >= 0);
+    RHO_REQ(pool_op == RHO_POOL_MAX || pool_op == RHO_POOL_AVERAGE);
+    Pool2dOperatorConfig p = {{(size_t)in_w, (size_t)in_h, (size_t)in_c}, (size_t)pool_size, (size_t)pool_stride,
+                              (size_t)pool_pad, pool_op == RHO_POOL_MAX ? PoolOperation::Max : PoolOperation::Average,
+                              ActivationFunction::Identity, ceil_mode != 0};
+    cfg->cfg.pool2d(p);
+  })
+}
+int rho_config_softmax_kl_loss(rho_config* cfg, int32_t num_categories) {
+  RHO_TRY({
+    RHO_REQ(cfg && num_categories > 0);
+    CategoricalLossConfig l = {(size_t)num_categories};
+    cfg->cfg.softmax_kl_loss(l);
+  })
+}
+int rho_config_params_len(const rho_config* cfg, int64_t* out) {
+  RHO_TRY({ RHO_REQ(cfg && out); *out = (int64_t)cfg->cfg.params_len(); })
+}
+int rho_config_from_model_file(const char* path, rho_config** out) {
+  RHO_TRY({
+    RHO_REQ(path && out);
+    std::unique_ptr<rho_config> c(new rho_config());
+    c->cfg = ModelConfigFile::open(path).to_sequential_config();
+    *out = c.release();
+  })
+}
+
+int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1, int device,
+                   int fuse_epilogue, rho_worker** out) {
+  RHO_TRY({
+    RHO_REQ(cfg && out && batch_size > 0);
+    std::unique_ptr<rho_worker> w(new rho_worker());
+    w->ctx = std::make_shared<DeviceContext>(device);
+    const uint64_t seed[2] = {seed0, seed1};
+    ExecOptions opts;
+    opts.fuse_epilogue = fuse_epilogue != 0;
+    w->worker.reset(new SequentialOperatorWorker(cfg->cfg, (size_t)batch_size,
+                                                 capability == RHO_CAP_FORWARD ? OpCapability::Forward : OpCapability::Backward,
+                                                 seed, w->ctx, opts));
+    *out = w.release();
+  })
+}
+int rho_worker_free(rho_worker* w) { RHO_TRY({ delete w; }) }
+int rho_worker_hidden_count(rho_worker* w, int32_t* out) { RHO_TRY({ RHO_REQ(w && out); *out = (int32_t)w->worker->hidden_count(); }) }
+int rho_worker_op_kind(rho_worker* w, int32_t hidden_idx, const char** out) { RHO_TRY({ RHO_REQ(out); *out = op_at(w, hidden_idx)->kind(); }) }
+void* rho_worker_stream(rho_worker* w) { return w ? w->ctx->stream() : nullptr; }
+int rho_worker_sync(rho_worker* w) { RHO_TRY({ RHO_REQ(w); w->ctx->sync(); }) }
+int rho_worker_init_params(rho_worker* w, uint64_t seed0, uint64_t seed1) {
+  RHO_TRY({ RHO_REQ(w); const uint64_t s[2] = {seed0, seed1}; w->worker->init_params(s); })
+}
+int rho_worker_expose_host_frame_buf(rho_worker* w, int32_t batch_idx, uint8_t** out) {
+  RHO_TRY({ RHO_REQ(w && out && batch_idx >= 0); *out = w->worker->input_operator()->expose_host_frame_buf((size_t)batch_idx); })
+}
+int rho_worker_load_frames(rho_worker* w, int32_t batch_size) {
+  RHO_TRY({ RHO_REQ(w && batch_size >= 0); w->worker->input_operator()->load_frames((size_t)batch_size); })
+}
+int rho_worker_load_frames_f32(rho_worker* w, const float* host, int32_t batch_size) {
+  RHO_TRY({ RHO_REQ(w && host && batch_size >= 0); w->worker->input_operator()->load_frames_f32(host, (size_t)batch_size); })
+}
+int rho_worker_stage_label(rho_worker* w, int32_t batch_idx, int32_t category) {
+  RHO_TRY({ RHO_REQ(w && batch_idx >= 0); w->worker->loss_operator(0)->stage_label((size_t)batch_idx, category); })
+}
+int rho_worker_load_labels(rho_worker* w, int32_t batch_size) {
+  RHO_TRY({ RHO_REQ(w && batch_size >= 0); w->worker->loss_operator(0)->load_labels((size_t)batch_size); })
+}
+int rho_worker_stage_weight(rho_worker* w, int32_t batch_idx, float weight) {
+  RHO_TRY({ RHO_REQ(w && batch_idx >= 0); w->worker->loss_operator(0)->stage_weight((size_t)batch_idx, weight); })
+}
+int rho_worker_load_weights(rho_worker* w, int32_t batch_size) {
+  RHO_TRY({ RHO_REQ(w && batch_size >= 0); w->worker->loss_operator(0)->load_weights((size_t)batch_size); })
+}
+int rho_worker_store_loss(rho_worker* w, int32_t batch_size, float* out) {
+  RHO_TRY({ RHO_REQ(w && out && batch_size >= 0); *out = w->worker->loss_operator(0)->store_loss((size_t)batch_size); })
+}
+int rho_worker_store_output_categories(rho_worker* w, int32_t batch_size) {
+  RHO_TRY({ RHO_REQ(w && batch_size >= 0); w->worker->loss_operator(0)->store_output_categories((size_t)batch_size); })
+}
+int rho_worker_get_output_categories(rho_worker* w, int32_t batch_size, int32_t* host_out) {
+  RHO_TRY({
+    RHO_REQ(w && host_out && batch_size >= 0 && (size_t)batch_size <= w->worker->batch_size());
+    const int32_t* c = w->worker->loss_operator(0)->get_output_categories((size_t)batch_size);
+    for (int32_t i = 0; i < batch_size; ++i) host_out[i] = c[i];
+  })
+}
+int rho_worker_accuracy_count(rho_worker* w, int32_t batch_size, int32_t* out) {
+  RHO_TRY({ RHO_REQ(w && out && batch_size >= 0); *out = (int32_t)w->worker->loss_operator(0)->accuracy_count((size_t)batch_size); })
+}
+int rho_worker_forward(rho_worker* w, int32_t batch_size, int training, int64_t t) {
+  RHO_TRY({
+    RHO_REQ(w && batch_size >= 0);
+    w->worker->forward((size_t)batch_size, training ? OpPhase::Training((size_t)t) : OpPhase::Inference());
+  })
+}
+int rho_worker_backward(rho_worker* w, int32_t batch_size) { RHO_TRY({ RHO_REQ(w && batch_size >= 0); w->worker->backward((size_t)batch_size); }) }
+int rho_worker_regularize(rho_worker* w, float l2) { RHO_TRY({ RHO_REQ(w); w->worker->regularize(Regularization::L2(l2)); }) }
+int rho_worker_accumulate_grads(rho_worker* w, float scale, float momentum) { RHO_TRY({ RHO_REQ(w); w->worker->accumulate_grads(scale, momentum); }) }
+int rho_worker_update_params(rho_worker* w, float scale) { RHO_TRY({ RHO_REQ(w); w->worker->update_params(scale); }) }
+int rho_worker_update_params2(rho_worker* w, float g, float u) { RHO_TRY({ RHO_REQ(w); w->worker->update_params2(g, u); }) }
+int rho_worker_save_params(rho_worker* w) { RHO_TRY({ RHO_REQ(w); w->worker->save_params(); }) }
+int rho_worker_restore_params(rho_worker* w) { RHO_TRY({ RHO_REQ(w); w->worker->restore_params(); }) }
+int rho_worker_reset(rho_worker* w) { RHO_TRY({ RHO_REQ(w); w->worker->reset(); }) }
+
+int rho_worker_buffer(rho_worker* w, int32_t hidden_idx, int which, float** dptr, int64_t* len) {
+  RHO_TRY({
+    RHO_REQ(dptr && len);
+    size_t n = 0;
+    if (!op_at(w, hidden_idx)->buffer(which, dptr, &n)) panic("operator has no such buffer");
+    *len = (int64_t)n;
+  })
+}
+int rho_worker_read_buffer(rho_worker* w, int32_t hidden_idx, int which, float* host, int64_t len) {
+  RHO_TRY({
+    RHO_REQ(host && len >= 0);
+    float* d = nullptr;
+    size_t n = 0;
+    if (!op_at(w, hidden_idx)->buffer(which, &d, &n)) panic("operator has no such buffer");
+    RHO_REQ((size_t)len <= n);
+    unwrap(rh_store_sync(w->ctx->raw(), host, d, (size_t)len * sizeof(float)), "sync_store");
+  })
+}
+int rho_worker_write_buffer(rho_worker* w, int32_t hidden_idx, int which, const float* host, int64_t len) {
+  RHO_TRY({
+    RHO_REQ(host && len >= 0);
+    float* d = nullptr;
+    size_t n = 0;
+    if (!op_at(w, hidden_idx)->buffer(which, &d, &n)) panic("operator has no such buffer");
+    RHO_REQ((size_t)len <= n);
+    unwrap(rh_load_sync(w->ctx->raw(), d, host, (size_t)len * sizeof(float)), "sync_load");
+  })
+}
+
+int rho_sgd_new(int32_t minibatch_size, int step_kind, const float* steps, const int64_t* step_iters, int momentum_kind,
+                float mu, float l2_reg_coef, rho_sgd** out) {
+  RHO_TRY({
+    RHO_REQ(out && steps && minibatch_size > 0 && step_kind >= 0 && step_kind <= RHO_STEP_INVERSE);
+    RHO_REQ(momentum_kind >= 0 && momentum_kind <= RHO_MOM_GRADIENT_NESTEROV);
+    SgdOptConfig c = SgdOptConfig();
+    c.minibatch_size = (size_t)minibatch_size;
+    c.step_size.kind = (StepSizeSchedule::Kind)step_kind;
+    for (int i = 0; i < 5; ++i) {
+      c.step_size.step[i] = steps[i];
+      c.step_size.iters[i] = step_iters ? (size_t)step_iters[i] : 0;
+    }
+    c.momentum.kind = (Momentum::Kind)momentum_kind;
+    c.momentum.mu = mu;
+    c.l2_reg_coef = l2_reg_coef;
+    std::unique_ptr<rho_sgd> s(new rho_sgd());
+    s->opt.reset(new SgdOpt(c));
+    *out = s.release();
+  })
+}
+int rho_sgd_free(rho_sgd* s) { RHO_TRY({ delete s; }) }
+int rho_sgd_begin(rho_sgd* s, rho_worker* w) { RHO_TRY({ RHO_REQ(s && w); s->opt->begin(w->worker.get()); }) }
+int rho_sgd_step(rho_sgd* s, rho_worker* w, int fused) { RHO_TRY({ RHO_REQ(s && w); s->opt->step(w->worker.get(), fused != 0); }) }
+int rho_sgd_iter_counter(rho_sgd* s, int64_t* out) { RHO_TRY({ RHO_REQ(s && out); *out = (int64_t)s->opt->iter_counter(); }) }
+int rho_sgd_step_size_at(rho_sgd* s, int64_t t, float* out) {
+  RHO_TRY({ RHO_REQ(s && out && t >= 0); *out = s->opt->config().step_size.at_iter((size_t)t); })
+}
+int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused, float* loss_out, int32_t* correct_out) {
+  RHO_TRY({
+    RHO_REQ(s && w && batch_size > 0);
+    SequentialOperatorWorker* op = w->worker.get();
+    const size_t b = (size_t)batch_size;
+    op->forward(b, OpPhase::Training(s->opt->iter_counter()));
+    op->loss_operator(0)->store_output_categories(b);
+    const float loss = op->loss_operator(0)->store_loss(b);
+    op->backward(b);
+    const size_t correct = op->loss_operator(0)->accuracy_count(b);
+    s->opt->step(op, fused != 0);
+    if (loss_out) *loss_out = loss;
+    if (correct_out) *correct_out = (int32_t)correct;
+  })
+}
+
+}  // extern "C"

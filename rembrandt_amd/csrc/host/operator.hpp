@@ -1,0 +1,307 @@
+// Host-side operator layer: a C++ mirror of the reference's Rust operator API for the
+// single-GPU hot path, written only against the C ABI of include/rembrandt_hip.h.
+//
+// Mirrors (paths relative to the reference tree):
+//   Operator / InputOperator traits ........ src/operator/mod.rs:61-109
+//   OpCapability, OpPhase, Regularization,
+//   ActivationFunction, ParamsInit ......... src/operator/mod.rs:233-297
+//   Data3dOperator (minimal) ............... src/operator/mod.rs:491-836
+//   AffineOperator ......................... src/operator/mod.rs:843-1364
+//   Conv2dOperator ......................... src/operator/mod.rs:1366-2003
+//   Pool2dOperator ......................... src/operator/mod.rs:2005-2132
+//   LossOperator, SoftmaxKLLossOperator .... src/operator/loss.rs:20-262
+//   SequentialOperatorConfig / Worker ...... src/operator/worker.rs:133-477
+//   SgdOptConfig, StepSizeSchedule,
+//   Momentum, the update block ............. src/opt/sgd/mod.rs:20-147, src/opt/sgd/new.rs:345-495
+//
+// Error behaviour: like the reference, which panics on every native error and on every violated
+// precondition, these classes throw std::runtime_error; nothing is recoverable.
+// Ownership: each operator owns its out_act / out_delta / parameter / gradient / momentum
+// buffers; neighbours share them by reference count (Rc<RefCell<DeviceBuffer>> in the reference).
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../../include/rembrandt_hip.h"
+
+namespace rembrandt {
+
+[[noreturn]] void panic(const std::string& msg);
+void unwrap(int code, const char* what);  // throws unless code == 0
+
+// ---- device runtime (stands in for array_cuda::device::{context,memory}) --------------------
+class DeviceContext {
+ public:
+  explicit DeviceContext(int device_idx);
+  ~DeviceContext();
+  DeviceContext(const DeviceContext&) = delete;
+  DeviceContext& operator=(const DeviceContext&) = delete;
+  rh_stream_t stream() const { return rh_ctx_stream(ctx_); }
+  rh_ctx* raw() const { return ctx_; }
+  void sync() const;
+
+ private:
+  rh_ctx* ctx_;
+};
+
+template <class T>
+class DeviceBuffer {
+ public:
+  // zero-filled, like DeviceBuffer::zeros(len, ctx)
+  DeviceBuffer(size_t len, std::shared_ptr<DeviceContext> ctx) : len_(len), ctx_(std::move(ctx)) {
+    void* p = nullptr;
+    unwrap(rh_malloc(ctx_->raw(), len * sizeof(T), &p), "rh_malloc");
+    ptr_ = static_cast<T*>(p);
+  }
+  ~DeviceBuffer() { rh_free(ctx_->raw(), ptr_); }
+  DeviceBuffer(const DeviceBuffer&) = delete;
+  DeviceBuffer& operator=(const DeviceBuffer&) = delete;
+  T* as_mut_ptr() { return ptr_; }
+  const T* as_ptr() const { return ptr_; }
+  size_t len() const { return len_; }
+  void sync_load(const T* host, size_t n) { unwrap(rh_load_sync(ctx_->raw(), ptr_, host, n * sizeof(T)), "sync_load"); }
+  void sync_store(T* host, size_t n) const { unwrap(rh_store_sync(ctx_->raw(), host, ptr_, n * sizeof(T)), "sync_store"); }
+
+ private:
+  T* ptr_ = nullptr;
+  size_t len_;
+  std::shared_ptr<DeviceContext> ctx_;
+};
+
+typedef std::shared_ptr<DeviceBuffer<float>> SharedDeviceBuf;
+
+// ---- small enums / value types ------------------------------------------------------------------
+enum class OpCapability { Forward, Backward };
+inline bool backward_enabled(OpCapability c) { return c != OpCapability::Forward; }
+
+struct OpPhase {
+  bool training;
+  size_t t;
+  static OpPhase Inference() { return {false, 0}; }
+  static OpPhase Training(size_t t) { return {true, t}; }
+};
+
+struct Regularization {  // only L2 exists (src/operator/mod.rs:267-270)
+  float l2_reg_coef;
+  static Regularization L2(float c) { return {c}; }
+};
+
+enum class ActivationFunction { Identity, Rect, Logistic, Tanh };  // only Identity and Rect are implemented
+
+struct ParamsInit {
+  enum Kind { Disabled, Uniform, Normal, Xavier, KaimingFwd } kind;
+  float value;  // half_range (Uniform) or std (Normal)
+  static ParamsInit MakeDisabled() { return {Disabled, 0.0f}; }
+  static ParamsInit MakeUniform(float half_range) { return {Uniform, half_range}; }
+  static ParamsInit MakeNormal(float std) { return {Normal, std}; }
+  static ParamsInit MakeXavier() { return {Xavier, 0.0f}; }
+  static ParamsInit MakeKaimingFwd() { return {KaimingFwd, 0.0f}; }
+};
+
+enum class PoolOperation { Max, Average };
+
+struct Dims3 {  // (width, height, channels), as in the reference
+  size_t w, h, c;
+  size_t len() const { return w * h * c; }
+};
+
+// ---- operator configs ---------------------------------------------------------------------------
+struct Data3dOperatorConfig {
+  Dims3 in_dims;
+  bool normalize;  // u8 frames are scaled by 1/255 when set (cast_bytes_normalized)
+};
+
+struct AffineOperatorConfig {
+  size_t in_channels, out_channels;
+  ActivationFunction act_func;
+  ParamsInit init_weights;
+  size_t params_len() const { return in_channels * out_channels + out_channels; }
+};
+
+struct Conv2dOperatorConfig {
+  Dims3 in_dims;
+  size_t conv_size, conv_stride, conv_pad, out_channels;
+  ActivationFunction act_func;
+  ParamsInit init_weights;
+  Dims3 get_out_dims() const;
+  size_t params_len() const { return conv_size * conv_size * in_dims.c * out_channels + out_channels; }
+};
+
+struct Pool2dOperatorConfig {
+  Dims3 in_dims;
+  size_t pool_size, pool_stride, pool_pad;
+  PoolOperation pool_op;
+  ActivationFunction act_func;  // present in the reference's struct, never read there either
+  bool ceil_mode;               // gen-1 extent (src/layer.rs:1741-1747); false = operator-style floor
+  Dims3 get_out_dims() const;
+};
+
+struct CategoricalLossConfig {
+  size_t num_categories;
+};
+
+struct OperatorConfig {
+  enum Kind { Data3d, Affine, Conv2d, Pool2d, SoftmaxKLLoss } kind;
+  Data3dOperatorConfig data3d;
+  AffineOperatorConfig affine;
+  Conv2dOperatorConfig conv2d;
+  Pool2dOperatorConfig pool2d;
+  CategoricalLossConfig loss;
+  size_t params_len() const;
+};
+
+// How kernels are scheduled inside the operators.  Both modes produce the same buffers at every
+// point where the reference's operators expose them.
+struct ExecOptions {
+  bool fuse_epilogue = true;  // conv bias + ReLU in the conv epilogue instead of K1 -> K2 -> K3
+};
+
+// ---- Operator trait -------------------------------------------------------------------------------
+class Operator {
+ public:
+  virtual ~Operator() {}
+  virtual size_t batch_size() const = 0;
+  virtual SharedDeviceBuf get_output_vars() const { return nullptr; }
+  virtual SharedDeviceBuf get_output_deltas() const { return nullptr; }
+  virtual void init_params(const uint64_t /*shared_seed*/[2]) {}
+  virtual void forward(size_t batch_size, OpPhase phase) = 0;
+  virtual void backward(size_t batch_size) = 0;
+  virtual void regularize(Regularization) {}
+  virtual void accumulate_grads(float /*scale*/, float /*momentum*/) {}
+  virtual void update_params(float /*scale*/) {}
+  virtual void update_params2(float /*grad_scale*/, float /*update_scale*/) {}
+  virtual void save_params() {}
+  virtual void restore_params() {}
+  virtual void reset() {}
+  // Fused regularize -> accumulate_grads(scale, momentum) -> update_params(apply) -> reset in
+  // one pass per tensor (same arithmetic, 24 instead of 52 bytes per parameter).
+  virtual void fused_sgd_step(float /*l2*/, float /*scale*/, float /*momentum*/, float /*apply*/) {}
+  // Device views for inspection: 0 out_act, 1 out_delta, 2 weights, 3 bias, 4 grad_weights,
+  // 5 grad_bias, 6 acc_grad_weights, 7 acc_grad_bias.  Returns false if the operator has no such buffer.
+  virtual bool buffer(int which, float** ptr, size_t* len) {
+    (void)which; (void)ptr; (void)len;
+    return false;
+  }
+  virtual const char* kind() const = 0;
+};
+
+class InputOperator : public Operator {
+ public:
+  virtual uint8_t* expose_host_frame_buf(size_t batch_idx) = 0;
+  virtual void load_frames(size_t batch_size) = 0;
+  // Synthetic fp32 frames (N(0,1) inputs of the benchmark configs): bypasses the u8 cast.
+  virtual void load_frames_f32(const float* host, size_t batch_size) = 0;
+};
+
+class LossOperator : public Operator {
+ public:
+  virtual void stage_label(size_t batch_idx, int32_t category) = 0;
+  virtual void load_labels(size_t batch_size) = 0;
+  virtual void stage_weight(size_t batch_idx, float weight) = 0;
+  virtual void load_weights(size_t batch_size) = 0;
+  virtual float store_loss(size_t batch_size) = 0;
+  virtual void store_output_categories(size_t batch_size) = 0;
+  virtual const int32_t* get_output_categories(size_t batch_size) const = 0;
+  virtual size_t accuracy_count(size_t batch_size) const = 0;
+};
+
+// ---- graph ----------------------------------------------------------------------------------------
+class SequentialOperatorConfig {
+ public:
+  OperatorConfig input_op;
+  bool has_input = false;
+  std::vector<OperatorConfig> hidden_ops;
+  OperatorConfig loss_op;
+  bool has_loss = false;
+
+  size_t params_len() const;
+  SequentialOperatorConfig& data3d(const Data3dOperatorConfig& cfg);
+  SequentialOperatorConfig& affine(const AffineOperatorConfig& cfg);
+  SequentialOperatorConfig& conv2d(const Conv2dOperatorConfig& cfg);
+  SequentialOperatorConfig& pool2d(const Pool2dOperatorConfig& cfg);
+  SequentialOperatorConfig& softmax_kl_loss(const CategoricalLossConfig& cfg);
+};
+
+class SequentialOperatorWorker : public Operator {
+ public:
+  SequentialOperatorWorker(const SequentialOperatorConfig& config, size_t batch_size, OpCapability capability,
+                           const uint64_t shared_seed[2], std::shared_ptr<DeviceContext> context,
+                           ExecOptions opts = ExecOptions());
+  // OperatorWorker (src/operator/worker.rs:52-76); a single worker: rank 0 of 1.
+  size_t num_workers() const { return 1; }
+  size_t worker_rank() const { return 0; }
+  const uint64_t* shared_seed() const { return shared_seed_; }
+  InputOperator* input_operator() { return input_op_.get(); }
+  size_t loss_count() const { return 1; }
+  LossOperator* loss_operator(size_t rank);
+  size_t hidden_count() const { return hidden_ops_.size(); }
+  Operator* hidden_operator(size_t i) { return hidden_ops_.at(i).get(); }
+  std::shared_ptr<DeviceContext> context() const { return context_; }
+
+  size_t batch_size() const override { return batch_size_; }
+  void init_params(const uint64_t shared_seed[2]) override;
+  void forward(size_t batch_size, OpPhase phase) override;
+  void backward(size_t batch_size) override;
+  void regularize(Regularization reg) override;
+  void accumulate_grads(float scale, float momentum) override;
+  void update_params(float scale) override;
+  void update_params2(float grad_scale, float update_scale) override;
+  void save_params() override;
+  void restore_params() override;
+  void reset() override;
+  void fused_sgd_step(float l2, float scale, float momentum, float apply) override;
+  const char* kind() const override { return "SequentialOperatorWorker"; }
+
+ private:
+  size_t batch_size_;
+  uint64_t shared_seed_[2];
+  std::shared_ptr<DeviceContext> context_;
+  std::unique_ptr<InputOperator> input_op_;
+  std::vector<std::unique_ptr<Operator>> hidden_ops_;
+  std::unique_ptr<LossOperator> loss_op_;
+};
+
+// ---- SGD policy (src/opt/sgd/mod.rs:20-147) ---------------------------------------------------------
+struct StepSizeSchedule {
+  enum Kind { Constant, Anneal1, Anneal2, Anneal4, Decay, Inverse } kind;
+  float step[5];     // step0..step4 (Constant: step[0]; Inverse: step[0] = init_step_size, step[1] = lambda)
+  size_t iters[5];   // iters[i] = step{i}_iters for i = 1..4
+  float at_iter(size_t t) const;
+  static StepSizeSchedule MakeConstant(float s);
+};
+
+struct Momentum {
+  enum Kind { Zero, Update, UpdateNesterov, Gradient, GradientNesterov } kind;
+  float mu;
+};
+
+struct SgdOptConfig {
+  size_t minibatch_size;
+  StepSizeSchedule step_size;
+  Momentum momentum;
+  float l2_reg_coef;
+};
+
+// The per-minibatch update block of SgdOpt::train (src/opt/sgd/new.rs:345-495, 623-633) for one
+// worker (no communication): regularize -> [Nesterov un-apply] -> iter_counter += 1 ->
+// accumulate_grads -> update_params -> reset -> [Nesterov re-apply].
+class SgdOpt {
+ public:
+  explicit SgdOpt(const SgdOptConfig& config) : config_(config) {}
+  // Called once before the first minibatch (src/opt/sgd/new.rs:257-271).
+  void begin(Operator* op);
+  // `fused`: use Operator::fused_sgd_step where the flavour allows it (Zero, Update, Gradient).
+  void step(Operator* op, bool fused);
+  size_t iter_counter() const { return iter_counter_; }
+  const SgdOptConfig& config() const { return config_; }
+
+ private:
+  SgdOptConfig config_;
+  size_t iter_counter_ = 0;
+};
+
+}  // namespace rembrandt

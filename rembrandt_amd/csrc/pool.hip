@@ -11,8 +11,10 @@ struct PoolDims { int N, C, H, W, k, st, pad, P, Q, mode; };
 
 inline int pool_out_dim(int in, int size, int stride, int pad, int round) {
   if (round == RH_ROUND_CEIL) {
-    const int t = in + 2 * pad - size + stride - 1;
-    return t < 0 ? 0 : t / stride + 1;
+    // max(0, in + 2*pad - size + stride - 1)/stride + 1 (src/layer.rs:1741-1747)
+    int t = in + 2 * pad - size + stride - 1;
+    if (t < 0) t = 0;
+    return t / stride + 1;
   }
   int t = in + 2 * pad - size + stride;
   if (t < 0) t = 0;

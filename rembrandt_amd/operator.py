@@ -1,0 +1,343 @@
+"""Python mirror of the operator / graph / optimizer layer (C ABI of include/rembrandt_operator.h).
+
+Class and method names follow the reference's Rust API (src/operator/mod.rs, src/operator/loss.rs,
+src/operator/worker.rs, src/opt/sgd/mod.rs); every method is one call into librembrandt_hip.so.
+Failures raise `Panic`, mirroring the reference's panic-on-error behaviour.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+ACT = {"Identity": 0, "Rect": 1, "Logistic": 2, "Tanh": 3}
+INIT = {"Disabled": 0, "Uniform": 1, "Normal": 2, "Xavier": 3, "KaimingFwd": 4}
+POOL = {"Max": 0, "Average": 1}
+MOMENTUM = {"Zero": 0, "Update": 1, "UpdateNesterov": 2, "Gradient": 3, "GradientNesterov": 4}
+STEP = {"Constant": 0, "Anneal1": 1, "Anneal2": 2, "Anneal4": 3, "Decay": 4, "Inverse": 5}
+BUF = {"out_act": 0, "out_delta": 1, "weights": 2, "bias": 3, "grad_weights": 4, "grad_bias": 5,
+       "acc_grad_weights": 6, "acc_grad_bias": 7}
+
+_vp, _i32, _i64, _f, _int, _u64 = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_int, C.c_uint64
+_P = C.POINTER
+
+PROTOTYPES = {
+    "rho_last_message": (C.c_char_p, []),
+    "rho_config_new": (_int, [_P(_vp)]),
+    "rho_config_free": (_int, [_vp]),
+    "rho_config_data3d": (_int, [_vp, _i32, _i32, _i32, _int]),
+    "rho_config_conv2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _int, _int, _f]),
+    "rho_config_affine": (_int, [_vp, _i32, _i32, _int, _int, _f]),
+    "rho_config_pool2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _int, _int]),
+    "rho_config_softmax_kl_loss": (_int, [_vp, _i32]),
+    "rho_config_params_len": (_int, [_vp, _P(_i64)]),
+    "rho_config_from_model_file": (_int, [C.c_char_p, _P(_vp)]),
+    "rho_worker_new": (_int, [_vp, _i32, _int, _u64, _u64, _int, _int, _P(_vp)]),
+    "rho_worker_free": (_int, [_vp]),
+    "rho_worker_hidden_count": (_int, [_vp, _P(_i32)]),
+    "rho_worker_op_kind": (_int, [_vp, _i32, _P(C.c_char_p)]),
+    "rho_worker_stream": (_vp, [_vp]),
+    "rho_worker_sync": (_int, [_vp]),
+    "rho_worker_init_params": (_int, [_vp, _u64, _u64]),
+    "rho_worker_expose_host_frame_buf": (_int, [_vp, _i32, _P(_vp)]),
+    "rho_worker_load_frames": (_int, [_vp, _i32]),
+    "rho_worker_load_frames_f32": (_int, [_vp, _vp, _i32]),
+    "rho_worker_stage_label": (_int, [_vp, _i32, _i32]),
+    "rho_worker_load_labels": (_int, [_vp, _i32]),
+    "rho_worker_stage_weight": (_int, [_vp, _i32, _f]),
+    "rho_worker_load_weights": (_int, [_vp, _i32]),
+    "rho_worker_store_loss": (_int, [_vp, _i32, _P(_f)]),
+    "rho_worker_store_output_categories": (_int, [_vp, _i32]),
+    "rho_worker_get_output_categories": (_int, [_vp, _i32, _vp]),
+    "rho_worker_accuracy_count": (_int, [_vp, _i32, _P(_i32)]),
+    "rho_worker_forward": (_int, [_vp, _i32, _int, _i64]),
+    "rho_worker_backward": (_int, [_vp, _i32]),
+    "rho_worker_regularize": (_int, [_vp, _f]),
+    "rho_worker_accumulate_grads": (_int, [_vp, _f, _f]),
+    "rho_worker_update_params": (_int, [_vp, _f]),
+    "rho_worker_update_params2": (_int, [_vp, _f, _f]),
+    "rho_worker_save_params": (_int, [_vp]),
+    "rho_worker_restore_params": (_int, [_vp]),
+    "rho_worker_reset": (_int, [_vp]),
+    "rho_worker_buffer": (_int, [_vp, _i32, _int, _P(_vp), _P(_i64)]),
+    "rho_worker_read_buffer": (_int, [_vp, _i32, _int, _vp, _i64]),
+    "rho_worker_write_buffer": (_int, [_vp, _i32, _int, _vp, _i64]),
+    "rho_sgd_new": (_int, [_i32, _int, _P(_f), _P(_i64), _int, _f, _f, _P(_vp)]),
+    "rho_sgd_free": (_int, [_vp]),
+    "rho_sgd_begin": (_int, [_vp, _vp]),
+    "rho_sgd_step": (_int, [_vp, _vp, _int]),
+    "rho_sgd_iter_counter": (_int, [_vp, _P(_i64)]),
+    "rho_sgd_step_size_at": (_int, [_vp, _i64, _P(_f)]),
+    "rho_sgd_train_batch": (_int, [_vp, _vp, _i32, _int, _P(_f), _P(_i32)]),
+}
+
+_bound = False
+
+
+class Panic(RuntimeError):
+    """The reference panics on every error of this layer; so does this mirror."""
+
+
+def lib():
+    global _bound
+    handle = _lib.lib()
+    if not _bound:
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _bound = True
+    return handle
+
+
+def _chk(code):
+    if code != 0:
+        msg = lib().rho_last_message()
+        raise Panic(msg.decode() if msg else "error %d" % code)
+
+
+def _init_args(init):
+    """('Normal', std) | ('Uniform', half_range) | 'Xavier' | 'KaimingFwd' | 'Disabled'"""
+    if isinstance(init, str):
+        return INIT[init], 0.0
+    return INIT[init[0]], float(init[1])
+
+
+class SequentialOperatorConfig:
+    """Fluent builder, src/operator/worker.rs:133-228.  Dimension triples are (width, height, channels)."""
+
+    def __init__(self, handle=None):
+        if handle is None:
+            h = _vp()
+            _chk(lib().rho_config_new(C.byref(h)))
+            handle = h
+        self._h = handle
+
+    @classmethod
+    def from_model_file(cls, path):
+        h = _vp()
+        _chk(lib().rho_config_from_model_file(str(path).encode(), C.byref(h)))
+        return cls(h)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().rho_config_free(self._h)
+            self._h = None
+
+    def data3d(self, in_dims, normalize=False):
+        _chk(lib().rho_config_data3d(self._h, in_dims[0], in_dims[1], in_dims[2], int(normalize)))
+        return self
+
+    def conv2d(self, in_dims, conv_size, conv_stride, conv_pad, out_channels, act_func="Rect", init_weights=("Normal", 0.01)):
+        k, v = _init_args(init_weights)
+        _chk(lib().rho_config_conv2d(self._h, in_dims[0], in_dims[1], in_dims[2], conv_size, conv_stride, conv_pad,
+                                     out_channels, ACT[act_func], k, v))
+        return self
+
+    def affine(self, in_channels, out_channels, act_func="Rect", init_weights=("Normal", 0.01)):
+        k, v = _init_args(init_weights)
+        _chk(lib().rho_config_affine(self._h, in_channels, out_channels, ACT[act_func], k, v))
+        return self
+
+    def pool2d(self, in_dims, pool_size, pool_stride, pool_pad, pool_op="Max", ceil_mode=False):
+        _chk(lib().rho_config_pool2d(self._h, in_dims[0], in_dims[1], in_dims[2], pool_size, pool_stride, pool_pad,
+                                     POOL[pool_op], int(ceil_mode)))
+        return self
+
+    def softmax_kl_loss(self, num_categories):
+        _chk(lib().rho_config_softmax_kl_loss(self._h, num_categories))
+        return self
+
+    def params_len(self):
+        out = _i64()
+        _chk(lib().rho_config_params_len(self._h, C.byref(out)))
+        return out.value
+
+
+class SequentialOperatorWorker:
+    """src/operator/worker.rs:230-477 plus the Input/Loss operator calls the optimizer makes on it."""
+
+    def __init__(self, config, batch_size, capability="Backward", shared_seed=(1, 2), device=0, fuse_epilogue=True):
+        h = _vp()
+        _chk(lib().rho_worker_new(config._h, batch_size, 0 if capability == "Forward" else 1, shared_seed[0],
+                                  shared_seed[1], device, int(fuse_epilogue), C.byref(h)))
+        self._h = h
+        self.batch_size = batch_size
+        self.shared_seed = tuple(shared_seed)
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().rho_worker_free(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def hidden_count(self):
+        out = _i32()
+        _chk(lib().rho_worker_hidden_count(self._h, C.byref(out)))
+        return out.value
+
+    def op_kind(self, idx):
+        out = C.c_char_p()
+        _chk(lib().rho_worker_op_kind(self._h, idx, C.byref(out)))
+        return out.value.decode()
+
+    def stream(self):
+        return lib().rho_worker_stream(self._h)
+
+    def sync(self):
+        _chk(lib().rho_worker_sync(self._h))
+
+    def init_params(self, shared_seed=None):
+        s = shared_seed or self.shared_seed
+        _chk(lib().rho_worker_init_params(self._h, s[0], s[1]))
+
+    # InputOperator
+    def load_frames_u8(self, frames):
+        """frames: uint8 array [batch][c][h][w]; staged through expose_host_frame_buf then load_frames."""
+        frames = np.ascontiguousarray(frames, np.uint8)
+        n = frames.shape[0]
+        flen = frames[0].size
+        for b in range(n):
+            p = _vp()
+            _chk(lib().rho_worker_expose_host_frame_buf(self._h, b, C.byref(p)))
+            C.memmove(p, frames[b].ctypes.data, flen)
+        _chk(lib().rho_worker_load_frames(self._h, n))
+
+    def load_frames_f32(self, frames):
+        frames = np.ascontiguousarray(frames, np.float32)
+        _chk(lib().rho_worker_load_frames_f32(self._h, frames.ctypes.data, frames.shape[0]))
+
+    # LossOperator
+    def stage_label(self, batch_idx, category):
+        _chk(lib().rho_worker_stage_label(self._h, batch_idx, int(category)))
+
+    def load_labels(self, batch_size):
+        _chk(lib().rho_worker_load_labels(self._h, batch_size))
+
+    def stage_weight(self, batch_idx, weight):
+        _chk(lib().rho_worker_stage_weight(self._h, batch_idx, float(weight)))
+
+    def load_weights(self, batch_size):
+        _chk(lib().rho_worker_load_weights(self._h, batch_size))
+
+    def stage_batch(self, labels, weight):
+        for b, l in enumerate(labels):
+            self.stage_label(b, int(l))
+            self.stage_weight(b, weight)
+        self.load_labels(len(labels))
+        self.load_weights(len(labels))
+
+    def store_loss(self, batch_size):
+        out = _f()
+        _chk(lib().rho_worker_store_loss(self._h, batch_size, C.byref(out)))
+        return out.value
+
+    def store_output_categories(self, batch_size):
+        _chk(lib().rho_worker_store_output_categories(self._h, batch_size))
+
+    def get_output_categories(self, batch_size):
+        out = np.zeros((batch_size,), np.int32)
+        _chk(lib().rho_worker_get_output_categories(self._h, batch_size, out.ctypes.data))
+        return out
+
+    def accuracy_count(self, batch_size):
+        out = _i32()
+        _chk(lib().rho_worker_accuracy_count(self._h, batch_size, C.byref(out)))
+        return out.value
+
+    # Operator
+    def forward(self, batch_size, training=True, t=0):
+        _chk(lib().rho_worker_forward(self._h, batch_size, int(training), t))
+
+    def backward(self, batch_size):
+        _chk(lib().rho_worker_backward(self._h, batch_size))
+
+    def regularize(self, l2_reg_coef):
+        _chk(lib().rho_worker_regularize(self._h, l2_reg_coef))
+
+    def accumulate_grads(self, scale, momentum):
+        _chk(lib().rho_worker_accumulate_grads(self._h, scale, momentum))
+
+    def update_params(self, scale):
+        _chk(lib().rho_worker_update_params(self._h, scale))
+
+    def update_params2(self, grad_scale, update_scale):
+        _chk(lib().rho_worker_update_params2(self._h, grad_scale, update_scale))
+
+    def save_params(self):
+        _chk(lib().rho_worker_save_params(self._h))
+
+    def restore_params(self):
+        _chk(lib().rho_worker_restore_params(self._h))
+
+    def reset(self):
+        _chk(lib().rho_worker_reset(self._h))
+
+    # inspection
+    def buffer_len(self, idx, which):
+        p, n = _vp(), _i64()
+        _chk(lib().rho_worker_buffer(self._h, idx, BUF[which], C.byref(p), C.byref(n)))
+        return n.value
+
+    def device_ptr(self, idx, which):
+        p, n = _vp(), _i64()
+        _chk(lib().rho_worker_buffer(self._h, idx, BUF[which], C.byref(p), C.byref(n)))
+        return p.value, n.value
+
+    def read(self, idx, which, count=None):
+        n = self.buffer_len(idx, which) if count is None else count
+        out = np.empty((n,), np.float32)
+        _chk(lib().rho_worker_read_buffer(self._h, idx, BUF[which], out.ctypes.data, n))
+        return out
+
+    def write(self, idx, which, values):
+        values = np.ascontiguousarray(values, np.float32).ravel()
+        _chk(lib().rho_worker_write_buffer(self._h, idx, BUF[which], values.ctypes.data, values.size))
+
+
+class SgdOpt:
+    """The update block of SgdOpt::train, src/opt/sgd/new.rs:345-495 (one worker, no communication)."""
+
+    def __init__(self, minibatch_size, step_size=0.01, momentum=("Update", 0.9), l2_reg_coef=0.0, schedule=None):
+        steps = (_f * 5)()
+        iters = (_i64 * 5)()
+        kind = STEP["Constant"]
+        if schedule is None:
+            steps[0] = step_size
+        else:
+            kind = STEP[schedule["kind"]]
+            for i, s in enumerate(schedule.get("steps", [])):
+                steps[i] = s
+            for i, it in enumerate(schedule.get("iters", [])):
+                iters[i] = it
+        mk, mu = (MOMENTUM[momentum], 0.0) if isinstance(momentum, str) else (MOMENTUM[momentum[0]], momentum[1])
+        h = _vp()
+        _chk(lib().rho_sgd_new(minibatch_size, kind, steps, iters, mk, mu, l2_reg_coef, C.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().rho_sgd_free(self._h)
+            self._h = None
+
+    def begin(self, worker):
+        _chk(lib().rho_sgd_begin(self._h, worker._h))
+
+    def step(self, worker, fused=True):
+        _chk(lib().rho_sgd_step(self._h, worker._h, int(fused)))
+
+    def iter_counter(self):
+        out = _i64()
+        _chk(lib().rho_sgd_iter_counter(self._h, C.byref(out)))
+        return out.value
+
+    def step_size_at(self, t):
+        out = _f()
+        _chk(lib().rho_sgd_step_size_at(self._h, t, C.byref(out)))
+        return out.value
+
+    def train_batch(self, worker, batch_size, fused=True):
+        loss, correct = _f(), _i32()
+        _chk(lib().rho_sgd_train_batch(self._h, worker._h, batch_size, int(fused), C.byref(loss), C.byref(correct)))
+        return loss.value, correct.value

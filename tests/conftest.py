@@ -28,6 +28,12 @@ def assert_close(got, ref, what, rtol=1e-4, atol=1e-5, scale_atol=True):
     if scale_atol and ref.size:
         a = atol * max(1.0, float(np.sqrt(np.mean(ref * ref))))
     err = np.abs(got - ref)
+    # tensors far below unit scale (gradients ~1e-4) would pass the absolute term vacuously:
+    # they must also agree to 1e-4 in relative L2 norm
+    ref_norm = float(np.sqrt(np.sum(ref * ref)))
+    if ref_norm > 0.0:
+        rel_l2 = float(np.sqrt(np.sum(err * err))) / ref_norm
+        assert rel_l2 <= 1e-4, "%s: relative L2 error %.3g > 1e-4" % (what, rel_l2)
     bound = a + rtol * np.abs(ref)
     bad = err > bound
     if bad.any():
