@@ -197,6 +197,17 @@ int rh_rng_fill_uniform(uint64_t seed, uint64_t stream_id, float* host, size_t n
 int rh_rng_fill_normal(uint64_t seed, uint64_t stream_id, float* host, size_t n, float mean, float std);
 int rh_rng_fill_int(uint64_t seed, uint64_t stream_id, int32_t* host, size_t n, int32_t modulus);
 
+/* ---------------------------------------------------------------------------------------------
+ * Per-launch timing (no counterpart in the reference, which only takes wall-clock laps around
+ * minibatches, src/opt/sgd/new.rs:273-274).  While enabled, every kernel launch of this library is
+ * bracketed by HIP events on its stream.  Record i = {kernel tag, algorithmic work (FLOPs for the
+ * MFMA contractions, bytes for the bandwidth-bound kernels), elapsed milliseconds}.
+ * ------------------------------------------------------------------------------------------- */
+int rh_profile_enable(int on);
+int rh_profile_count(void);
+int rh_profile_get(int i, const char** tag, double* work, float* ms);
+int rh_profile_reset(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -66,6 +66,10 @@ PROTOTYPES = {
     "rembrandt_kernel_batch_blockreduce_argmax": (None, [_vp, _i32, _i32, _vp, _vp, _vp]),
     "rh_sgd_momentum_step": (_int, [_i64, _vp, _vp, _vp, _f, _f, _f, _f, _int, _vp]),
     "rh_descend": (_int, [_i64, _vp, _vp, _f, _f, _vp]),
+    "rh_profile_enable": (_int, [_int]),
+    "rh_profile_count": (_int, []),
+    "rh_profile_get": (_int, [_int, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(_f)]),
+    "rh_profile_reset": (_int, []),
     "rh_rng_fill_uniform": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_normal": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_int": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _i32]),

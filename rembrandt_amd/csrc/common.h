@@ -33,4 +33,15 @@ inline int stream_grid(size_t work_items, int block) {
   return static_cast<int>(want);
 }
 
+// Optional per-launch timing with HIP events (off by default; rh_profile_enable).  A scope
+// records an event before and after the launches made inside it, on the stream they go to.
+// `work` is the algorithmic work of those launches: FLOPs for contractions, bytes otherwise.
+struct ProfScope {
+  ProfScope(const char* tag, double work, hipStream_t stream);
+  ~ProfScope();
+  void* slot;
+  hipStream_t stream;
+};
+extern bool g_profile_enabled;
+
 }  // namespace rh

@@ -23,10 +23,10 @@ __global__ void build_bwd_data_tab_kernel(int4* tab, int* atab, int n_entries, i
 
 template <class T>
 static int run_bwd_data(int KRS, const DenseParams& ap, const GatherParams& bp, const EpiParams& ep,
-                        hipStream_t stream) {
+                        hipStream_t stream, const char* tag) {
   typedef LoadDenseK<T::BM, T::BK, T::NT, true> AL;
   typedef LoadGatherR<T::BN, T::BK, T::NT, true> BL;
-  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, KRS, 1, nullptr, stream);
+  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, KRS, 1, nullptr, stream, tag);
 }
 
 }  // namespace rh
@@ -64,9 +64,9 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
   ep.rows = d.C; ep.cols = bp.M; ep.inner = d.H * d.W; ep.ld = 0; ep.relu = 0; ep.split_stride = 0;
 
   switch (pick_bm(d.C)) {
-    case 128: return run_bwd_data<T128x128>(KRS, ap, bp, ep, stream);
-    case 96:  return run_bwd_data<T96x256>(KRS, ap, bp, ep, stream);
-    case 64:  return run_bwd_data<T64x256>(KRS, ap, bp, ep, stream);
-    default:  return run_bwd_data<T32x256>(KRS, ap, bp, ep, stream);
+    case 128: return run_bwd_data<T128x128>(KRS, ap, bp, ep, stream, "conv_bwd_data_128x128");
+    case 96:  return run_bwd_data<T96x256>(KRS, ap, bp, ep, stream, "conv_bwd_data_96x256");
+    case 64:  return run_bwd_data<T64x256>(KRS, ap, bp, ep, stream, "conv_bwd_data_64x256");
+    default:  return run_bwd_data<T32x256>(KRS, ap, bp, ep, stream, "conv_bwd_data_32x256");
   }
 }

@@ -54,16 +54,17 @@ __global__ void split_reduce_kernel(const float* __restrict__ part, int splits, 
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
                          int ld, float alpha, float beta, hipStream_t stream) {
   const size_t total = (size_t)rows * cols;
+  ProfScope prof("split_reduce", 4.0 * (double)total * (splits + 1), stream);
   hipLaunchKernelGGL(split_reduce_kernel, dim3(stream_grid(total, 256)), dim3(256), 0, stream, part, splits,
                      split_stride, out, rows, cols, ld, alpha, beta);
 }
 
 template <class T>
 static int run_bwd_filter(const PixDyParams& ap, const PixXParams& bp, const EpiParams& ep, int M,
-                          int splits, int* used, hipStream_t stream) {
+                          int splits, int* used, hipStream_t stream, const char* tag) {
   typedef LoadPixDy<T::BM, T::BK, T::NT> AL;
   typedef LoadPixX<T::BN, T::BK, T::NT> BL;
-  return launch_mfma_gemm<T, AL, BL, false>(ap, bp, ep, M, splits, used, stream);
+  return launch_mfma_gemm<T, AL, BL, false>(ap, bp, ep, M, splits, used, stream, tag);
 }
 
 // db[k] = alpha * sum_{n, i<plane} dy[(n*K + k)*plane + i] + beta * db[k]; one block per k.
@@ -160,10 +161,10 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
     used = 0;
   } else {
     switch (plan.bm) {
-      case 128: e = run_bwd_filter<T128x128>(ap, bp, ep, M, plan.splits, &used, stream); break;
-      case 96:  e = run_bwd_filter<T96x256>(ap, bp, ep, M, plan.splits, &used, stream); break;
-      case 64:  e = run_bwd_filter<T64x256>(ap, bp, ep, M, plan.splits, &used, stream); break;
-      default:  e = run_bwd_filter<T32x256>(ap, bp, ep, M, plan.splits, &used, stream); break;
+      case 128: e = run_bwd_filter<T128x128>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_128x128"); break;
+      case 96:  e = run_bwd_filter<T96x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x256"); break;
+      case 64:  e = run_bwd_filter<T64x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_64x256"); break;
+      default:  e = run_bwd_filter<T32x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x256"); break;
     }
     if (e) return e;
   }
@@ -175,6 +176,7 @@ extern "C" int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alp
                                   float beta, float* db, rh_stream_t stream_) {
   if (N <= 0 || K <= 0 || plane <= 0 || !dy || !db) return RH_E_INVALID;
   hipStream_t stream = to_stream(stream_);
+  ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
   if (plane == 1) {
     hipLaunchKernelGGL(bwd_bias_rows_kernel, dim3(cdiv(K, 256)), dim3(256), 0, stream, dy, N, K, alpha, beta,
                        db);

@@ -54,7 +54,7 @@ inline int pick_bm(int rows) {
 template <class T, class AL, class BL, bool NCHW>
 inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Params& bp,
                             const EpiParams& ep, int K, int splits, int* splits_used,
-                            hipStream_t stream) {
+                            hipStream_t stream, const char* tag) {
   const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
   const int k_chunks = cdiv(K, T::BK);
   if (splits < 1) splits = 1;
@@ -62,6 +62,7 @@ inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Pa
   const int used = cdiv(k_chunks, cps) > 0 ? cdiv(k_chunks, cps) : 1;
   if (splits_used) *splits_used = used;
   dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)used);
+  ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)K, stream);
   hipLaunchKernelGGL((mfma_gemm_kernel<T, AL, BL, NCHW>), grid, dim3(T::NT), 0, stream, ap, bp, ep,
                      tiles_m, k_chunks, cps);
   return launch_status();

@@ -24,10 +24,10 @@ void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int H
 
 template <class T>
 static int run_fwd(const ConvDims& d, const DenseParams& ap, const GatherParams& bp,
-                   const EpiParams& ep, hipStream_t stream) {
+                   const EpiParams& ep, hipStream_t stream, const char* tag) {
   typedef LoadDenseK<T::BM, T::BK, T::NT, false> AL;
   typedef LoadGatherR<T::BN, T::BK, T::NT, false> BL;
-  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, d.C * d.R * d.S, 1, nullptr, stream);
+  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, d.C * d.R * d.S, 1, nullptr, stream, tag);
 }
 
 }  // namespace rh
@@ -71,9 +71,9 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
   ep.split_stride = 0;
 
   switch (pick_bm(d.K)) {
-    case 128: return run_fwd<T128x128>(d, ap, bp, ep, stream);
-    case 96:  return run_fwd<T96x256>(d, ap, bp, ep, stream);
-    case 64:  return run_fwd<T64x256>(d, ap, bp, ep, stream);
-    default:  return run_fwd<T32x256>(d, ap, bp, ep, stream);
+    case 128: return run_fwd<T128x128>(d, ap, bp, ep, stream, "conv_fwd_128x128");
+    case 96:  return run_fwd<T96x256>(d, ap, bp, ep, stream, "conv_fwd_96x256");
+    case 64:  return run_fwd<T64x256>(d, ap, bp, ep, stream, "conv_fwd_64x256");
+    default:  return run_fwd<T32x256>(d, ap, bp, ep, stream, "conv_fwd_32x256");
   }
 }

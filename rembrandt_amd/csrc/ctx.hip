@@ -3,6 +3,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
 #include <thread>
 #include <vector>
 
@@ -106,6 +107,69 @@ extern "C" int rh_store_sync(rh_ctx* ctx, void* dst_h, const void* src_d, size_t
   hipError_t e = hipMemcpyAsync(dst_h, src_d, bytes, hipMemcpyDeviceToHost, ctx->stream);
   if (e != hipSuccess) return (int)e;
   return (int)hipStreamSynchronize(ctx->stream);
+}
+
+// ---- per-launch timing -------------------------------------------------------------------
+namespace rh {
+
+bool g_profile_enabled = false;
+
+namespace {
+struct ProfRecord { const char* tag; double work; hipEvent_t e0, e1; };
+std::vector<ProfRecord*> g_records;
+std::mutex g_prof_mutex;
+}  // namespace
+
+ProfScope::ProfScope(const char* tag, double work, hipStream_t s) : slot(nullptr), stream(s) {
+  if (!g_profile_enabled) return;
+  ProfRecord* r = new ProfRecord{tag, work, nullptr, nullptr};
+  if (hipEventCreate(&r->e0) != hipSuccess || hipEventCreate(&r->e1) != hipSuccess) { delete r; return; }
+  (void)hipEventRecord(r->e0, s);
+  slot = r;
+}
+
+ProfScope::~ProfScope() {
+  if (!slot) return;
+  ProfRecord* r = static_cast<ProfRecord*>(slot);
+  (void)hipEventRecord(r->e1, stream);
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_records.push_back(r);
+}
+
+}  // namespace rh
+
+extern "C" int rh_profile_enable(int on) {
+  rh::g_profile_enabled = on != 0;
+  return 0;
+}
+
+extern "C" int rh_profile_count(void) {
+  std::lock_guard<std::mutex> lock(rh::g_prof_mutex);
+  return (int)rh::g_records.size();
+}
+
+// Record i: tag, algorithmic work, elapsed milliseconds (waits for the record's end event).
+extern "C" int rh_profile_get(int i, const char** tag, double* work, float* ms) {
+  std::lock_guard<std::mutex> lock(rh::g_prof_mutex);
+  if (i < 0 || i >= (int)rh::g_records.size() || !tag || !work || !ms) return RH_E_INVALID;
+  rh::ProfRecord* r = rh::g_records[(size_t)i];
+  hipError_t e = hipEventSynchronize(r->e1);
+  if (e != hipSuccess) return (int)e;
+  if ((e = hipEventElapsedTime(ms, r->e0, r->e1)) != hipSuccess) return (int)e;
+  *tag = r->tag;
+  *work = r->work;
+  return 0;
+}
+
+extern "C" int rh_profile_reset(void) {
+  std::lock_guard<std::mutex> lock(rh::g_prof_mutex);
+  for (rh::ProfRecord* r : rh::g_records) {
+    (void)hipEventDestroy(r->e0);
+    (void)hipEventDestroy(r->e1);
+    delete r;
+  }
+  rh::g_records.clear();
+  return 0;
 }
 
 // ---- seeded generator --------------------------------------------------------------------

@@ -116,6 +116,7 @@ extern "C" int rh_last_error(void) { return g_last_error; }
 extern "C" int rh_add_bias_nchw(const float* bias, float* y, int32_t plane, int32_t K, int32_t N, float alpha,
                                 float beta, rh_stream_t stream) {
   if (!bias || !y || plane <= 0 || K <= 0 || N <= 0) return RH_E_INVALID;
+  ProfScope prof("add_bias", 8.0 * (double)plane * K * N, to_stream(stream));
   if (plane >= 256 && (long long)N * K <= 65535) {
     dim3 grid((unsigned)cdiv(plane, 256 * 4), (unsigned)(N * K));
     hipLaunchKernelGGL(add_bias_plane_kernel, grid, dim3(256), 0, to_stream(stream), bias, y, plane, K, alpha, beta);
@@ -131,6 +132,7 @@ extern "C" void rembrandt_kernel_batch_map_rect_inplace(float* y, int32_t frame_
                                                         rh_stream_t stream) {
   const long long n = (long long)frame_len * batch;
   if (n <= 0 || !y) { g_last_error = n == 0 ? 0 : RH_E_INVALID; return; }
+  ProfScope prof("rect_fwd", 8.0 * (double)n, to_stream(stream));
   hipLaunchKernelGGL(rect_inplace_kernel, dim3(stream_grid((size_t)(n + 3) / 4, 256)), dim3(256), 0,
                      to_stream(stream), y, n);
   g_last_error = launch_status();
@@ -140,6 +142,7 @@ extern "C" void rembrandt_kernel_batch_map_rect_backprop_inplace(const float* y,
                                                                  float* dy, rh_stream_t stream) {
   const long long n = (long long)frame_len * batch;
   if (n <= 0 || !y || !dy) { g_last_error = n == 0 ? 0 : RH_E_INVALID; return; }
+  ProfScope prof("rect_bwd", 12.0 * (double)n, to_stream(stream));
   hipLaunchKernelGGL(rect_backprop_inplace_kernel, dim3(stream_grid((size_t)(n + 3) / 4, 256)), dim3(256), 0,
                      to_stream(stream), y, dy, n);
   g_last_error = launch_status();
@@ -148,6 +151,7 @@ extern "C" void rembrandt_kernel_batch_map_rect_backprop_inplace(const float* y,
 extern "C" int rh_memset_f32(float* d, float value, size_t n, rh_stream_t stream) {
   if (n == 0) return 0;
   if (!d) return RH_E_INVALID;
+  ProfScope prof("fill", 4.0 * (double)n, to_stream(stream));
   hipLaunchKernelGGL(fill_kernel, dim3(stream_grid((n + 3) / 4, 256)), dim3(256), 0, to_stream(stream), d, value,
                      (long long)n);
   return launch_status();
@@ -156,6 +160,7 @@ extern "C" int rh_memset_f32(float* d, float value, size_t n, rh_stream_t stream
 extern "C" int rh_cast_u8_f32(const uint8_t* x, float* y, size_t n, float scale, rh_stream_t stream) {
   if (n == 0) return 0;
   if (!x || !y) return RH_E_INVALID;
+  ProfScope prof("cast_u8_f32", 5.0 * (double)n, to_stream(stream));
   hipLaunchKernelGGL(cast_u8_f32_kernel, dim3(stream_grid((n + 3) / 4, 256)), dim3(256), 0, to_stream(stream), x,
                      y, (long long)n, scale);
   return launch_status();

@@ -144,6 +144,8 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
   if (!x || !y) return RH_E_INVALID;
   const long long total = (long long)d.N * d.C * d.P * d.Q;
   if (total == 0) return 0;
+  ProfScope prof(d.mode == RH_POOL_MAX ? "pool_max_fwd" : "pool_avg_fwd",
+                 4.0 * ((double)d.N * d.C * d.H * d.W + (double)total * (opt_argmax ? 2 : 1)), to_stream(stream));
   hipLaunchKernelGGL(pool_fwd_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, to_stream(stream), d, x,
                      y, opt_argmax);
   return launch_status();
@@ -157,6 +159,10 @@ extern "C" int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float*
   if (!dy || !dx) return RH_E_INVALID;
   if (d.mode == RH_POOL_MAX && !opt_argmax && !x) return RH_E_INVALID;
   const long long total = (long long)d.N * d.C * d.H * d.W;
+  const double out_elems = (double)d.N * d.C * d.P * d.Q;
+  // bytes: write dx, read dy, plus the arg-max mask or (max without mask) x itself
+  const double bwd_bytes = 4.0 * ((double)total + out_elems + (d.mode == RH_POOL_MAX ? (opt_argmax ? out_elems : (double)total) : 0.0));
+  ProfScope prof(d.mode == RH_POOL_MAX ? "pool_max_bwd" : "pool_avg_bwd", bwd_bytes, to_stream(stream));
   hipLaunchKernelGGL(pool_bwd_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, to_stream(stream), d, x,
                      dy, dx, opt_argmax);
   return launch_status();

@@ -64,6 +64,7 @@ extern "C" int rh_sgd_momentum_step(int64_t n, float* W, float* g, float* v, flo
                                     float apply, int zero_grad, rh_stream_t stream) {
   if (n < 0 || (n > 0 && (!W || !g || !v)) || l2 < 0.0f) return RH_E_INVALID;
   if (n == 0) return 0;
+  ProfScope prof("sgd_fused", 24.0 * (double)n, to_stream(stream));
   hipLaunchKernelGGL(sgd_momentum_kernel, dim3(stream_grid((size_t)(n + 3) / 4, 256)), dim3(256), 0,
                      to_stream(stream), (long long)n, W, g, v, l2, scale, mu, apply, zero_grad);
   return launch_status();
@@ -72,6 +73,7 @@ extern "C" int rh_sgd_momentum_step(int64_t n, float* W, float* g, float* v, flo
 extern "C" int rh_descend(int64_t n, float* W, float* g, float s, float l2, rh_stream_t stream) {
   if (n < 0 || (n > 0 && (!W || !g)) || l2 < 0.0f) return RH_E_INVALID;
   if (n == 0) return 0;
+  ProfScope prof("descend", 16.0 * (double)n, to_stream(stream));
   hipLaunchKernelGGL(descend_kernel, dim3(stream_grid((size_t)n, 256)), dim3(256), 0, to_stream(stream),
                      (long long)n, W, g, s, l2);
   return launch_status();

@@ -15,6 +15,7 @@ struct SgemmPlan { int bm, bn, splits; };
 static SgemmPlan plan_sgemm(int m, int n, int k) {
   SgemmPlan p;
   p.bm = pick_bm(n);
+  if (p.bm == 96) p.bm = round_up(n, 128) <= round_up(n, 64) ? 128 : 64;  // no 96-row tile for row-contiguous loads
   p.bn = p.bm == 128 ? 128 : 256;
   const int tiles = cdiv(n, p.bm) * cdiv(m, p.bn);
   const int k_chunks = cdiv(k, 16);
@@ -31,29 +32,29 @@ static SgemmPlan plan_sgemm(int m, int n, int k) {
 
 template <class T, bool B_TRANS, bool A_TRANS>
 static int run_sgemm(const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k, int splits,
-                     int* used, hipStream_t stream) {
+                     int* used, hipStream_t stream, const char* tag) {
   // engine A operand = opB: k contiguous unless transB; engine B operand = opA: rows contiguous unless transA
   if constexpr (!B_TRANS && !A_TRANS)
     return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseR<T::BN, T::BK, T::NT>, false>(
-        ap, bp, ep, k, splits, used, stream);
+        ap, bp, ep, k, splits, used, stream, tag);
   else if constexpr (!B_TRANS && A_TRANS)
     return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseK<T::BN, T::BK, T::NT, false>, false>(
-        ap, bp, ep, k, splits, used, stream);
+        ap, bp, ep, k, splits, used, stream, tag);
   else if constexpr (B_TRANS && !A_TRANS)
     return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseR<T::BN, T::BK, T::NT>, false>(
-        ap, bp, ep, k, splits, used, stream);
+        ap, bp, ep, k, splits, used, stream, tag);
   else
     return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseK<T::BN, T::BK, T::NT, false>, false>(
-        ap, bp, ep, k, splits, used, stream);
+        ap, bp, ep, k, splits, used, stream, tag);
 }
 
 template <bool B_TRANS, bool A_TRANS>
 static int dispatch_tile(int bm, const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k,
                          int splits, int* used, hipStream_t stream) {
   switch (bm) {
-    case 128: return run_sgemm<T128x128, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream);
-    case 64:  return run_sgemm<T64x256, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream);
-    default:  return run_sgemm<T32x256, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream);
+    case 128: return run_sgemm<T128x128, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream, "sgemm_128x128");
+    case 64:  return run_sgemm<T64x256, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream, "sgemm_64x256");
+    default:  return run_sgemm<T32x256, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream, "sgemm_32x256");
   }
 }
 
@@ -157,6 +158,7 @@ extern "C" int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k,
 extern "C" int rh_saxpy(int64_t n, float alpha, const float* x, float* y, rh_stream_t stream) {
   if (n < 0 || (n > 0 && (!x || !y))) return RH_E_INVALID;
   if (n == 0) return 0;
+  ProfScope prof("saxpy", 12.0 * (double)n, to_stream(stream));
   hipLaunchKernelGGL(saxpy_kernel, dim3(stream_grid((size_t)(n + 3) / 4, 256)), dim3(256), 0, to_stream(stream),
                      (long long)n, alpha, x, y);
   return launch_status();
@@ -165,6 +167,7 @@ extern "C" int rh_saxpy(int64_t n, float alpha, const float* x, float* y, rh_str
 extern "C" int rh_sscal(int64_t n, float alpha, float* x, rh_stream_t stream) {
   if (n < 0 || (n > 0 && !x)) return RH_E_INVALID;
   if (n == 0) return 0;
+  ProfScope prof("sscal", 8.0 * (double)n, to_stream(stream));
   hipLaunchKernelGGL(sscal_kernel, dim3(stream_grid((size_t)(n + 3) / 4, 256)), dim3(256), 0, to_stream(stream),
                      (long long)n, alpha, x);
   return launch_status();

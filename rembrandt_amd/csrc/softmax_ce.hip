@@ -116,6 +116,7 @@ using namespace rh;
 extern "C" int rh_softmax_fwd(const float* x, float* p, int32_t C, int32_t N, rh_stream_t stream) {
   if (!x || !p || C <= 0 || N < 0) return RH_E_INVALID;
   if (N == 0) return 0;
+  ProfScope prof("softmax_fwd", 8.0 * (double)C * N, to_stream(stream));
   hipLaunchKernelGGL(softmax_fwd_kernel, dim3(N), dim3(256), 0, to_stream(stream), x, p, C);
   return launch_status();
 }
@@ -126,6 +127,7 @@ extern "C" void rembrandt_kernel_batch_map_softmax_kl_backward(const float* p, i
   if (!p || !labels || !weights || !dx || C <= 0 || N < 0) { g_last_error = RH_E_INVALID; return; }
   if (N == 0) { g_last_error = 0; return; }
   const long long total = (long long)C * N;
+  ProfScope prof("softmax_kl_backward", 8.0 * (double)total, to_stream(stream));
   hipLaunchKernelGGL(softmax_kl_backward_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0,
                      to_stream(stream), p, C, total, labels, weights, dx);
   g_last_error = launch_status();
@@ -153,6 +155,7 @@ extern "C" void rembrandt_kernel_batch_blockreduce_argmax(const float* src, int3
                                                           float* max_out, int32_t* idx_out, rh_stream_t stream) {
   if (!src || !max_out || !idx_out || len <= 0 || batch < 0) { g_last_error = RH_E_INVALID; return; }
   if (batch == 0) { g_last_error = 0; return; }
+  ProfScope prof("argmax", 4.0 * (double)len * batch, to_stream(stream));
   hipLaunchKernelGGL(blockreduce_argmax_kernel, dim3(batch), dim3(256), 0, to_stream(stream), src, len, max_out,
                      idx_out);
   g_last_error = launch_status();

@@ -1,0 +1,161 @@
+"""CPU: host-side logic and the C-ABI surface (no kernel is launched here)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from rembrandt_amd import _lib, configs, operator, synth
+from rembrandt_amd.operator import Panic, SequentialOperatorConfig, SgdOpt
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+REF_EXAMPLES = "/root/reference/examples"
+
+
+def declared_symbols(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:rh|rho|rembrandt_kernel)_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    handle = C.CDLL(_lib.LIB_PATH)
+    names = declared_symbols("rembrandt_hip.h") + declared_symbols("rembrandt_operator.h")
+    assert len(names) > 80
+    missing = [n for n in names if not hasattr(handle, n)]
+    assert not missing, missing
+    # and the bindings cover the header
+    bound = set(_lib.PROTOTYPES) | set(operator.PROTOTYPES)
+    assert not [n for n in names if n not in bound], [n for n in names if n not in bound]
+    assert b"gfx950" in _lib.lib().rh_version()
+
+
+def test_error_codes_without_gpu():
+    lib = _lib.lib()
+    g = _lib.ConvGeom(0, 3, 8, 8, 4, 3, 3, 1, 1)
+    assert lib.rh_conv2d_fwd(C.byref(g), 1.0, 1, 1, 0.0, 1, None, None, 0, 0, None) == _lib.RH_E_INVALID
+    g = _lib.ConvGeom(2, 3, 8, 8, 4, 3, 3, 1, 1)
+    assert lib.rh_conv2d_fwd(C.byref(g), 1.0, None, None, 0.0, None, None, None, 0, 0, None) == _lib.RH_E_INVALID
+    assert lib.rh_conv2d_fwd(C.byref(g), 1.0, 256, 256, 0.0, 256, None, None, 0, 0, None) == _lib.RH_E_WORKSPACE
+    assert lib.rh_conv2d_fwd(C.byref(g), 1.0, 256, 256, 0.0, 256, None, 512, 1 << 20, _lib.RH_MATH_BF16_MFMA_FP32ACC, None) == _lib.RH_E_UNSUPPORTED
+    big = _lib.ConvGeom(4096, 512, 64, 64, 8, 3, 3, 1, 1)   # 32 GiB input: beyond the 2 GiB buffer-addressing limit
+    assert lib.rh_conv2d_fwd(C.byref(big), 1.0, 256, 256, 0.0, 256, None, 512, 1 << 20, 0, None) == _lib.RH_E_LIMIT
+    assert lib.rh_sgemm(0, 0, 4, 4, 4, 1.0, 256, 2, 256, 4, 0.0, 256, 4, None, 0, 0, None) == _lib.RH_E_INVALID  # lda < m
+    p = _lib.PoolGeom(1, 1, 4, 4, 2, 2, 0, 7, 0)
+    assert lib.rh_pool2d_fwd(C.byref(p), 256, 256, None, None) == _lib.RH_E_INVALID
+    assert lib.rh_sgd_momentum_step(4, 256, 256, 256, -1.0, 0.1, 0.9, 1.0, 1, None) == _lib.RH_E_INVALID  # l2 >= 0
+    assert lib.rh_error_string(_lib.RH_E_WORKSPACE) and lib.rh_error_string(0) == b"ok"
+
+
+def test_workspace_and_shape_helpers():
+    lib = _lib.lib()
+    assert [lib.rh_conv2d_out_dim(n, k, s, p) for (n, k, s, p) in [(227, 11, 4, 0), (27, 5, 1, 2), (13, 3, 1, 1), (2, 5, 1, 0)]] == [55, 27, 13, 0]
+    assert [lib.rh_pool2d_out_dim(n, 3, 2, 0, 0) for n in (55, 27, 13, 54)] == [27, 13, 6, 26]
+    assert [lib.rh_pool2d_out_dim(n, 3, 2, 0, 1) for n in (54, 27, 13)] == [27, 13, 6]
+    g = _lib.ConvGeom(256, 96, 27, 27, 256, 5, 5, 1, 2)
+    fwd = lib.rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_FWD)
+    bwf = lib.rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_BWD_FILTER)
+    bwd = lib.rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_BWD_DATA)
+    assert fwd % 256 == 0 and bwf % 256 == 0 and bwd % 256 == 0
+    assert fwd >= 2400 * 16 and bwd >= 6400 * 20 and bwf > fwd
+
+
+def test_rng_is_a_pure_function_of_seed_stream_index():
+    a = synth.normal(5, 7, (1000,))
+    assert np.array_equal(a, synth.normal(5, 7, (1000,)))
+    assert np.array_equal(a[:100], synth.normal(5, 7, (100,)))            # element i independent of n
+    assert not np.array_equal(a, synth.normal(5, 8, (1000,))) and not np.array_equal(a, synth.normal(6, 7, (1000,)))
+    big = synth.normal(1, 2, (1 << 20,))                                   # threaded fill == serial fill
+    assert np.array_equal(big[:1000], synth.normal(1, 2, (1000,)))
+    assert abs(float(big.mean())) < 5e-3 and abs(float(big.std()) - 1.0) < 5e-3
+    u = synth.uniform(3, 4, (1 << 18,), -2.0, 6.0)
+    assert u.min() >= -2.0 and u.max() < 6.0 and abs(float(u.mean()) - 2.0) < 3e-2
+    k = synth.integers(3, 5, (20000,), 10)
+    assert k.min() == 0 and k.max() == 9 and np.bincount(k).min() > 1700
+    # known answers of this generator (regression pin of the documented algorithm)
+    golden = np.load(os.path.join(ROOT, "tests", "golden", "rng_kat.npz"))
+    assert np.array_equal(synth.normal(0x5EED0004, 100, (16,)), golden["normal"])
+    assert np.array_equal(synth.uniform(0x5EED0001, 100, (16,)), golden["uniform"])
+    assert np.array_equal(synth.integers(0x5EED0004, 200, (16,), 1000), golden["integers"])
+
+
+def test_network_definitions_match_the_reference_geometry():
+    expect = {"lenet": (1256080, 64, 2.454272), "cifar10": (145578, 128, 8.858861568),
+              "alexnet": (62378344, 256, 1689.780781056), "nin": (7595176, 128, 818.931105792)}
+    for name, (params, batch, gflop) in expect.items():
+        net = configs.NETWORKS[name]()
+        assert configs.build_config(net).params_len() == params
+        assert abs(configs.train_flops(net, batch) / 1e9 - gflop) < 1e-6
+    dims, layers, ncat = configs.alexnet()
+    convs = [l for l in layers if l[0] == "conv2d"]
+    assert [l[1] for l in convs] == [(227, 227, 3), (27, 27, 96), (13, 13, 256), (13, 13, 384), (13, 13, 384)]
+    assert [l[1] for l in layers if l[0] == "affine"] == [9216, 4096, 4096]
+    assert [l[1][0] for l in configs.nin()[1] if l[0] == "pool2d"] == [54, 27, 13, 6]
+    assert [l[1] for l in configs.cifar10()[1] if l[0] == "affine"] == [1024, 64]
+
+
+def test_model_files_in_the_reference_grammar():
+    ex = os.path.join(ROOT, "examples")
+    assert SequentialOperatorConfig.from_model_file(os.path.join(ex, "lenet.model")).params_len() == 1256080
+    assert SequentialOperatorConfig.from_model_file(os.path.join(ex, "alexnet.model")).params_len() == 62378344
+    assert SequentialOperatorConfig.from_model_file(os.path.join(ex, "nin.model")).params_len() == 7595176
+    with pytest.raises(Panic):
+        SequentialOperatorConfig.from_model_file(os.path.join(ex, "does-not-exist.model"))
+
+
+def test_model_parser_errors(tmp_path):
+    def parse(text):
+        p = tmp_path / "m.model"
+        p.write_text(text)
+        return SequentialOperatorConfig.from_model_file(p)
+    data = '[[layer]]\nname = "data"\ntype = "data"\nraw_width = 8\nraw_height = 8\ncrop_width = 8\ncrop_height = 8\nchannels = 1\n'
+    fc = '[[layer]]\nname = "fc"\ntype = "fully_conn"\nout_channels = 3\nact_func = "identity"\ninit_weights = { kind = "normal", mean = 0.0, std = 0.1 }\n'
+    loss = '[[layer]]\nname = "loss"\ntype = "softmax_loss"\nnum_categories = 3\n'
+    assert parse(data + fc + loss).params_len() == 64 * 3 + 3
+    assert parse("# c\n" + data + "\n\n" + fc + "[opt]\nminibatch_size = 4 # ignored table\n" + loss).params_len() == 195
+    for bad in (data + fc,                                             # no loss layer
+                fc + loss,                                             # no input for the first layer
+                data + fc.replace('"identity"', '"relu"') + loss,      # act_func "relu" is not in the grammar (config.rs:123-129)
+                data + fc.replace('type = "fully_conn"\n', "") + loss,  # 'layer' missing 'type' field
+                data + fc + loss.replace("3", "4"),                    # input length != num_categories
+                data + fc.replace("std = 0.1", "std = 1") + loss,      # as_float() rejects an integer
+                data + fc.replace('kind = "normal"', 'kind = "xavier"') + loss,
+                data + '[[layer]]\nname = "n"\ntype = "local_res_norm"\ncross_size = 5\n' + fc + loss,
+                data + "garbage line\n" + fc + loss):
+        with pytest.raises(Panic):
+            parse(bad)
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_EXAMPLES), reason="reference tree not mounted")
+def test_reference_example_files():
+    assert SequentialOperatorConfig.from_model_file(os.path.join(REF_EXAMPLES, "imagenet_nin.model")).params_len() == 7595176
+    # 28 -> conv5 pad2 16ch -> pool2 -> 14x14x16 = 3136 -> fc100 -> fc10
+    assert SequentialOperatorConfig.from_model_file(os.path.join(REF_EXAMPLES, "mnist_lenet.model")).params_len() == \
+        (25 * 16 + 16) + (3136 * 100 + 100) + (100 * 10 + 10)
+    with pytest.raises(Panic):   # not parseable by the reference's own parser either (pool tables lack 'type', act_func "relu")
+        SequentialOperatorConfig.from_model_file(os.path.join(REF_EXAMPLES, "imagenet_alexnet.model"))
+
+
+def test_builder_preconditions():
+    with pytest.raises(Panic):
+        SequentialOperatorConfig().conv2d((8, 8, 1), 3, 0, 1, 4)       # stride 0
+    with pytest.raises(Panic):
+        SequentialOperatorConfig().affine(0, 4)
+    with pytest.raises(KeyError):
+        SequentialOperatorConfig().pool2d((8, 8, 1), 2, 2, 0, "Median")
+    cfg = SequentialOperatorConfig().data3d((8, 8, 1)).conv2d((8, 8, 1), 3, 1, 1, 4).pool2d((8, 8, 4), 2, 2, 0).affine(64, 3).softmax_kl_loss(3)
+    assert cfg.params_len() == (9 * 4 + 4) + (64 * 3 + 3)
+
+
+def test_step_size_schedules():
+    s = SgdOpt(64, schedule={"kind": "Anneal4", "steps": [1.0, 0.5, 0.25, 0.125, 0.0625], "iters": [0, 10, 20, 30, 40]})
+    assert [s.step_size_at(t) for t in (0, 9, 10, 19, 20, 29, 30, 39, 40, 10 ** 6)] == [1.0, 1.0, 0.5, 0.5, 0.25, 0.25, 0.125, 0.125, 0.0625, 0.0625]
+    s = SgdOpt(64, schedule={"kind": "Anneal1", "steps": [0.1, 0.01], "iters": [0, 5]})
+    assert [round(s.step_size_at(t), 6) for t in (4, 5)] == [0.1, 0.01]
+    s = SgdOpt(64, schedule={"kind": "Inverse", "steps": [0.1, 0.01]})
+    assert abs(s.step_size_at(100) - 0.1 / (1 + 0.1 * 0.01 * 100)) < 1e-7
+    assert SgdOpt(64, 0.25).step_size_at(12345) == 0.25
+    with pytest.raises(Panic):
+        SgdOpt(64, schedule={"kind": "Decay", "steps": [0.1]}).step_size_at(0)   # unimplemented!() in the reference too
+    assert SgdOpt(64, 0.1).iter_counter() == 0
