@@ -1,5 +1,7 @@
 // Host-side helpers shared by the three convolution passes.
 #pragma once
+#include <stdlib.h>
+
 #include "gemm_core.h"
 
 namespace rh {
@@ -62,8 +64,17 @@ inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Pa
   const int used = cdiv(k_chunks, cps) > 0 ? cdiv(k_chunks, cps) : 1;
   if (splits_used) *splits_used = used;
   dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)used);
+  constexpr size_t lds_bytes = sizeof(float) * 2 * T::BK * (AL::LD + BL::LD);
+  static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
+  if (lds_bytes > 48 * 1024) {
+    // opt in to more than the default dynamic LDS limit, once per kernel instantiation
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&mfma_gemm_kernel<T, AL, BL, NCHW>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (attr != hipSuccess) return (int)attr;
+  }
   ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)K, stream);
-  hipLaunchKernelGGL((mfma_gemm_kernel<T, AL, BL, NCHW>), grid, dim3(T::NT), 0, stream, ap, bp, ep,
+  hipLaunchKernelGGL((mfma_gemm_kernel<T, AL, BL, NCHW>), grid, dim3(T::NT), lds_bytes, stream, ap, bp, ep,
                      tiles_m, k_chunks, cps);
   return launch_status();
 }
@@ -73,6 +84,17 @@ typedef Tile<128, 128, 16, 2, 2> T128x128;
 typedef Tile<96, 256, 16, 1, 4> T96x256;
 typedef Tile<64, 256, 16, 1, 4> T64x256;
 typedef Tile<32, 256, 16, 1, 4> T32x256;
+// experimental shapes, selected with the RH_CONV_TILE environment variable
+typedef Tile<128, 256, 16, 2, 2> T128x256;
+typedef Tile<256, 128, 16, 2, 2> T256x128;
+typedef Tile<128, 128, 32, 2, 2> T128x128k32;
+typedef Tile<128, 256, 32, 2, 2> T128x256k32;
+typedef Tile<256, 256, 16, 2, 4> T256x256w8;
+
+inline int tile_override() {
+  static const int v = [] { const char* e = getenv("RH_CONV_TILE"); return e ? atoi(e) : 0; }();
+  return v;
+}
 
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,

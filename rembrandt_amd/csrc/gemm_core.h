@@ -14,6 +14,8 @@
 //   d[v] = D[8*(v/4) + 4*(lane/32) + v%4][lane % 32],  v = 0..15.
 // Lanes run along j, so j is always mapped to the memory-contiguous index of the output.
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace rh {
@@ -80,16 +82,16 @@ struct LoadDenseK {
       rowoff[i] = row < p.rows ? (uint32_t)row * (uint32_t)p.ld : kInvalidOff;
     }
   }
-  __device__ __forceinline__ void load(int k0, float (&v)[CNT]) {
+  uint32_t koff;
+  __device__ __forceinline__ void prep(int k0) {
     const int k = k0 + kk;
-    uint32_t koff = kInvalidOff;
+    koff = kInvalidOff;
     if (k < K) {
       if (HAS_TAB) { const int t = ktab[k]; koff = t >= 0 ? (uint32_t)t : kInvalidOff; }
       else koff = (uint32_t)k;
     }
-#pragma unroll
-    for (int i = 0; i < CNT; ++i) v[i] = buf_load_f32(rsrc, rowoff[i] + koff);
   }
+  __device__ __forceinline__ float load_one(int i) const { return buf_load_f32(rsrc, rowoff[i] + koff); }
   __device__ __forceinline__ void store(float* s, const float (&v)[CNT]) {
 #pragma unroll
     for (int i = 0; i < CNT; ++i) s[sbase + i * RSTEP] = v[i];
@@ -119,13 +121,12 @@ struct LoadDenseR {
     sbase = kk0 * LD + row;
     rowoff = (row0 + row) < p.rows ? (uint32_t)(row0 + row) : kInvalidOff;
   }
-  __device__ __forceinline__ void load(int k0, float (&v)[CNT]) {
-#pragma unroll
-    for (int i = 0; i < CNT; ++i) {
-      const int k = k0 + kk0 + i * KSTEP;
-      const uint32_t koff = k < K ? (uint32_t)k * (uint32_t)ld : kInvalidOff;
-      v[i] = buf_load_f32(rsrc, rowoff + koff);
-    }
+  int kcur;
+  __device__ __forceinline__ void prep(int k0) { kcur = k0 + kk0; }
+  __device__ __forceinline__ float load_one(int i) const {
+    const int k = kcur + i * KSTEP;
+    const uint32_t koff = k < K ? (uint32_t)k * (uint32_t)ld : kInvalidOff;
+    return buf_load_f32(rsrc, rowoff + koff);
   }
   __device__ __forceinline__ void store(float* s, const float (&v)[CNT]) {
 #pragma unroll
@@ -162,22 +163,25 @@ struct GatherParams {
 
 template <int ROWS, int BK, int NT, bool BWD>
 struct LoadGatherR {
-  static constexpr int CNT = ROWS * BK / NT, KSTEP = NT / ROWS;
+  // Thread (row, kk0) loads the CNT consecutive k values kk0*CNT .. kk0*CNT + CNT-1 of its row, so the
+  // table entries a wave needs in one K step are contiguous and wave-uniform: the compiler fetches
+  // them with a few wide scalar loads issued together, instead of one dependent load per element.
+  static constexpr int CNT = ROWS * BK / NT;
   static constexpr int LD = ROWS + lds_pad_kfast<BK>();
   static_assert(NT % ROWS == 0 && (ROWS * BK) % NT == 0 && ROWS % kWave == 0, "loader shape");
   typedef GatherParams Params;
   __amdgpu_buffer_rsrc_t rsrc;
   const int4* ktab;
-  int base, h0, w0, phase, Hlim, Wlim, kk0, sbase;
+  int base, h0, w0, phase, Hlim, Wlim, sbase;
 
   __device__ __forceinline__ void init(const Params& p, int row0, int tid) {
     rsrc = make_rsrc(p.ptr, p.bytes);
-    ktab = p.ktab;
     Hlim = p.Hlim;
     Wlim = p.Wlim;
     const int row = tid % ROWS;
-    kk0 = __builtin_amdgcn_readfirstlane(tid / ROWS);  // ROWS % 64 == 0: uniform per wave
-    sbase = kk0 * LD + row;
+    const int kk0 = __builtin_amdgcn_readfirstlane(tid / ROWS);  // ROWS % 64 == 0: uniform per wave
+    ktab = p.ktab + kk0 * CNT;
+    sbase = kk0 * CNT * LD + row;
     const int m = row0 + row;
     const bool valid = m < p.M;
     const int mm = valid ? m : 0;
@@ -198,18 +202,21 @@ struct LoadGatherR {
     base = n * p.img_stride + h0 * p.row_stride + w0;
     if (!valid) phase = -2;
   }
-  __device__ __forceinline__ void load(int k0, float (&v)[CNT]) {
+  int4 e[CNT];
+  __device__ __forceinline__ void prep(int k0) {
+    const int4* t = ktab + k0;
 #pragma unroll
-    for (int i = 0; i < CNT; ++i) {
-      const int4 e = ktab[k0 + kk0 + i * KSTEP];
-      const bool ok = (unsigned)(h0 + e.y) < (unsigned)Hlim && (unsigned)(w0 + e.z) < (unsigned)Wlim &&
-                      e.w == phase;
-      v[i] = buf_load_f32(rsrc, ok ? (uint32_t)(base + e.x) : kInvalidOff);
-    }
+    for (int i = 0; i < CNT; ++i) e[i] = t[i];
+  }
+  __device__ __forceinline__ float load_one(int i) const {
+    // bitwise, not short-circuit: no branches in the load path
+    const int ok = (int)((unsigned)(h0 + e[i].y) < (unsigned)Hlim) & (int)((unsigned)(w0 + e[i].z) < (unsigned)Wlim) &
+                   (int)(e[i].w == phase);
+    return buf_load_f32(rsrc, ok ? (uint32_t)(base + e[i].x) : kInvalidOff);
   }
   __device__ __forceinline__ void store(float* s, const float (&v)[CNT]) {
 #pragma unroll
-    for (int i = 0; i < CNT; ++i) s[sbase + i * KSTEP * LD] = v[i];
+    for (int i = 0; i < CNT; ++i) s[sbase + i * LD] = v[i];
   }
 };
 
@@ -252,16 +259,16 @@ struct LoadPixDy {
       rowoff[i] = row < p.rows ? (uint32_t)row * (uint32_t)p.PQ : kInvalidOff;
     }
   }
-  __device__ __forceinline__ void load(int k0, float (&v)[CNT]) {
+  uint32_t kbase;
+  __device__ __forceinline__ void prep(int k0) {
     const int pix = k0 + kk;
-    uint32_t kbase = kInvalidOff;
+    kbase = kInvalidOff;
     if (pix < M) {
       const int n = pix / PQ;
       kbase = (uint32_t)(n * img + (pix - n * PQ));
     }
-#pragma unroll
-    for (int i = 0; i < CNT; ++i) v[i] = buf_load_f32(rsrc, rowoff[i] + kbase);
   }
+  __device__ __forceinline__ float load_one(int i) const { return buf_load_f32(rsrc, rowoff[i] + kbase); }
   __device__ __forceinline__ void store(float* s, const float (&v)[CNT]) {
 #pragma unroll
     for (int i = 0; i < CNT; ++i) s[sbase + i * RSTEP] = v[i];
@@ -304,9 +311,10 @@ struct LoadPixX {
       }
     }
   }
-  __device__ __forceinline__ void load(int k0, float (&v)[CNT]) {
+  int h0, w0, base;
+  __device__ __forceinline__ void prep(int k0) {
     const int pix = k0 + kk;
-    int h0 = -(1 << 28), w0 = 0, base = 0;
+    h0 = -(1 << 28); w0 = 0; base = 0;
     if (pix < M) {
       const int n = pix / PQ;
       const int pq = pix - n * PQ;
@@ -316,11 +324,10 @@ struct LoadPixX {
       w0 = q * st - pad;
       base = n * img + h0 * W + w0;
     }
-#pragma unroll
-    for (int i = 0; i < CNT; ++i) {
-      const bool ok = (unsigned)(h0 + rr[i]) < (unsigned)H && (unsigned)(w0 + rs[i]) < (unsigned)W;
-      v[i] = buf_load_f32(rsrc, ok ? (uint32_t)(base + roff[i]) : kInvalidOff);
-    }
+  }
+  __device__ __forceinline__ float load_one(int i) const {
+    const int ok = (int)((unsigned)(h0 + rr[i]) < (unsigned)H) & (int)((unsigned)(w0 + rs[i]) < (unsigned)W);
+    return buf_load_f32(rsrc, ok ? (uint32_t)(base + roff[i]) : kInvalidOff);
   }
   __device__ __forceinline__ void store(float* s, const float (&v)[CNT]) {
 #pragma unroll
@@ -361,8 +368,10 @@ __global__ __launch_bounds__(T::NT) void mfma_gemm_kernel(typename AL::Params ap
                                                           int chunks_per_split) {
   constexpr int BM = T::BM, BN = T::BN, BK = T::BK, TM = T::TM, TN = T::TN;
   constexpr int LDA = AL::LD, LDB = BL::LD;
-  __shared__ float sA[2][BK * LDA];
-  __shared__ float sB[2][BK * LDB];
+  // dynamic LDS: [2][BK*LDA] for A, then [2][BK*LDB] for B
+  extern __shared__ float lds_dyn[];
+  float* const sA_base = lds_dyn;
+  float* const sB_base = lds_dyn + 2 * BK * LDA;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -393,44 +402,78 @@ __global__ __launch_bounds__(T::NT) void mfma_gemm_kernel(typename AL::Params ap
 
   float ra[AL::CNT], rb[BL::CNT];
   if (nk > 0) {
-    la.load(c_begin * BK, ra);
-    lb.load(c_begin * BK, rb);
-    la.store(sA[0], ra);
-    lb.store(sB[0], rb);
+    la.prep(c_begin * BK);
+    lb.prep(c_begin * BK);
+#pragma unroll
+    for (int i = 0; i < AL::CNT; ++i) ra[i] = la.load_one(i);
+#pragma unroll
+    for (int i = 0; i < BL::CNT; ++i) rb[i] = lb.load_one(i);
+    la.store(sA_base, ra);
+    lb.store(sB_base, rb);
   }
   __syncthreads();
 
   const int a_rd = (lane >> 5) * LDA + wm * (TM * 32) + (lane & 31);
   const int b_rd = (lane >> 5) * LDB + wn * (TN * 32) + (lane & 31);
 
-  for (int it = 0; it < nk; ++it) {
+  // One K step.  The instruction order is pinned with scheduling barriers into BK/2 groups of
+  //   [LDS operand reads of the next group] [address math + global loads of a slice of the next
+  //   K step's slabs] [TM*TN MFMAs of this group]
+  // so that a wave keeps the matrix pipe fed by itself: LDS latency hides behind the MFMAs of
+  // the group before, and the loader's VALU work issues in the shadow of running MFMAs.  The
+  // global loads sit in the first half of the step, giving them the second half (and the other
+  // waves' turns) to land before they are written to the other LDS buffer.
+  constexpr int STEPS = BK / 2;
+  constexpr int LSTEPS = STEPS / 2 > 0 ? STEPS / 2 : 1;
+  constexpr int A_PER = (AL::CNT + LSTEPS - 1) / LSTEPS, B_PER = (BL::CNT + LSTEPS - 1) / LSTEPS;
+  auto k_step = [&](int it, auto more_tag) {
+    constexpr bool MORE = decltype(more_tag)::value;
     const int cur = it & 1;
-    const bool more = it + 1 < nk;
-    if (more) {
-      la.load((c_begin + it + 1) * BK, ra);
-      lb.load((c_begin + it + 1) * BK, rb);
+    if (MORE) {
+      la.prep((c_begin + it + 1) * BK);
+      lb.prep((c_begin + it + 1) * BK);
     }
-    const float* pa = sA[cur] + a_rd;
-    const float* pb = sB[cur] + b_rd;
+    const float* pa = sA_base + cur * (BK * LDA) + a_rd;
+    const float* pb = sB_base + cur * (BK * LDB) + b_rd;
+    float a[2][TM], b[2][TN];
 #pragma unroll
-    for (int k2 = 0; k2 < BK; k2 += 2) {
-      float a[TM], b[TN];
+    for (int i = 0; i < TM; ++i) a[0][i] = pa[i * 32];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a[i] = pa[k2 * LDA + i * 32];
+    for (int j = 0; j < TN; ++j) b[0][j] = pb[j * 32];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) b[j] = pb[k2 * LDB + j * 32];
+    for (int g = 0; g < STEPS; ++g) {
+      const int c = g & 1, n = c ^ 1;
+      __builtin_amdgcn_sched_barrier(0);
+      if (g + 1 < STEPS) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[n][i] = pa[(2 * g + 2) * LDA + i * 32];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[n][j] = pb[(2 * g + 2) * LDB + j * 32];
+      }
+      if (MORE && g < LSTEPS) {
+#pragma unroll
+        for (int e = g * A_PER; e < (g + 1) * A_PER; ++e)
+          if (e < AL::CNT) ra[e] = la.load_one(e);
+#pragma unroll
+        for (int e = g * B_PER; e < (g + 1) * B_PER; ++e)
+          if (e < BL::CNT) rb[e] = lb.load_one(e);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c][i], b[c][j], acc[i][j], 0, 0, 0);
     }
-    if (more) {
-      la.store(sA[cur ^ 1], ra);
-      lb.store(sB[cur ^ 1], rb);
+    __builtin_amdgcn_sched_barrier(0);
+    if (MORE) {
+      la.store(sA_base + (cur ^ 1) * (BK * LDA), ra);
+      lb.store(sB_base + (cur ^ 1) * (BK * LDB), rb);
     }
     __syncthreads();
-  }
+  };
+  for (int it = 0; it + 1 < nk; ++it) k_step(it, std::true_type());
+  if (nk > 0) k_step(nk - 1, std::false_type());
 
   // ---- epilogue
   const bool split = ep.split_stride != 0;
