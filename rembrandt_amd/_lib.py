@@ -7,7 +7,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "librembrandt_hip.so")
+LIB_PATH = os.environ.get("RH_LIB") or os.path.join(_HERE, "librembrandt_hip.so")
 
 RH_CONV_FWD, RH_CONV_BWD_FILTER, RH_CONV_BWD_DATA = 0, 1, 2
 RH_POOL_MAX, RH_POOL_AVG_INCL_PAD = 0, 1
@@ -70,6 +70,8 @@ PROTOTYPES = {
     "rh_profile_count": (_int, []),
     "rh_profile_get": (_int, [_int, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(_f)]),
     "rh_profile_reset": (_int, []),
+    "rh_probe_mfma_loop": (_int, [_int, _int, _int, _vp, _vp]),
+    "rh_probe_copy": (_int, [_vp, _vp, _sz, _vp]),
     "rh_rng_fill_uniform": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_normal": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_int": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _i32]),

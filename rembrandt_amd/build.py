@@ -7,13 +7,13 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-OBJ = os.path.join(HERE, "build")
-LIB = os.path.join(HERE, "librembrandt_hip.so")
+OBJ = os.environ.get("RH_OBJ_DIR") or os.path.join(HERE, "build")
+LIB = os.environ.get("RH_LIB_OUT") or os.path.join(HERE, "librembrandt_hip.so")
 
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
          # packed fp32 instructions are not to be generated on this hardware pool
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + os.environ.get("RH_EXTRA_FLAGS", "").split()
 
 
 def sources():

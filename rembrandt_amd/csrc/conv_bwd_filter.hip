@@ -21,9 +21,12 @@ static BwdFilterPlan plan_bwd_filter(const ConvDims& d) {
   p.tiles = cdiv(d.K, p.bm) * cdiv(CRS, p.bn);
   const long long M = (long long)d.N * d.P * d.Q;
   const int k_chunks = (int)cdiv<long long>(M, 16);
-  // Aim at ~4 blocks per CU; every slice keeps at least 32 K steps so the prologue and the
-  // partial-sum traffic stay small next to the contraction.
-  int want = cdiv(1024, p.tiles);
+  // One full co-resident set of blocks (256 CUs x 3 blocks of this kernel per CU) and no partial
+  // second round: a block that runs alone on its CU uses the matrix pipe less well than three
+  // sharing it, so a ragged tail costs more than its share.  Every slice keeps at least 32 K
+  // steps so the prologue and the partial-sum traffic stay small next to the contraction.
+  const int slots = 256 * 3;
+  int want = slots / p.tiles;
   const int max_by_depth = k_chunks / 32 > 0 ? k_chunks / 32 : 1;
   if (want > max_by_depth) want = max_by_depth;
   if (want > 256) want = 256;

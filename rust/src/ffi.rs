@@ -1,0 +1,107 @@
+//! Raw bindings of include/rembrandt_hip.h: the replacement for `rembrandt_kernels::ffi`,
+//! `cuda_dnn::v4::ffi` and the cuBLAS/cudart calls of `array_cuda` on rembrandt's operator hot path.
+//! Written for the reference's toolchain (rustc 1.9 nightly, `libc` crate); not compiled in the image
+//! this library is built in (no Rust toolchain there).
+#![allow(non_camel_case_types)]
+
+use libc::{c_char, c_float, c_int, c_void, size_t};
+
+pub type rh_stream_t = *mut c_void; // hipStream_t
+pub enum rh_ctx {}
+
+#[repr(C)]
+#[derive(Clone, Copy, Debug)]
+pub struct rh_conv_geom {
+  pub n: i32, pub c: i32, pub h: i32, pub w: i32,
+  pub k: i32, pub r: i32, pub s: i32,
+  pub stride: i32, pub pad: i32,
+}
+
+#[repr(C)]
+#[derive(Clone, Copy, Debug)]
+pub struct rh_pool_geom {
+  pub n: i32, pub c: i32, pub h: i32, pub w: i32,
+  pub size: i32, pub stride: i32, pub pad: i32,
+  pub mode: i32,  // 0 max, 1 average (count includes padding)
+  pub round: i32, // 0 floor (operator), 1 ceil (gen-1 layer)
+}
+
+pub const RH_CONV_FWD: c_int = 0;
+pub const RH_CONV_BWD_FILTER: c_int = 1;
+pub const RH_CONV_BWD_DATA: c_int = 2;
+pub const RH_FUSE_BIAS: c_int = 0x10;
+pub const RH_FUSE_RELU: c_int = 0x20;
+
+#[link(name = "rembrandt_hip")]
+extern "C" {
+  pub fn rh_error_string(code: c_int) -> *const c_char;
+  pub fn rh_last_error() -> c_int;
+
+  pub fn rh_ctx_create(device: c_int, out: *mut *mut rh_ctx) -> c_int;
+  pub fn rh_ctx_destroy(ctx: *mut rh_ctx) -> c_int;
+  pub fn rh_ctx_stream(ctx: *mut rh_ctx) -> rh_stream_t;
+  pub fn rh_ctx_sync(ctx: *mut rh_ctx) -> c_int;
+  pub fn rh_malloc(ctx: *mut rh_ctx, bytes: size_t, dptr: *mut *mut c_void) -> c_int;
+  pub fn rh_free(ctx: *mut rh_ctx, dptr: *mut c_void) -> c_int;
+  pub fn rh_memset_f32(d: *mut f32, value: c_float, n: size_t, stream: rh_stream_t) -> c_int;
+  pub fn rh_copy_d2d(dst: *mut c_void, src: *const c_void, bytes: size_t, stream: rh_stream_t) -> c_int;
+  pub fn rh_load_sync(ctx: *mut rh_ctx, dst_d: *mut c_void, src_h: *const c_void, bytes: size_t) -> c_int;
+  pub fn rh_store_sync(ctx: *mut rh_ctx, dst_h: *mut c_void, src_d: *const c_void, bytes: size_t) -> c_int;
+  pub fn rh_cast_u8_f32(x: *const u8, y: *mut f32, n: size_t, scale: c_float, stream: rh_stream_t) -> c_int;
+
+  pub fn rh_conv2d_workspace_bytes(g: *const rh_conv_geom, pass: c_int) -> size_t;
+  pub fn rh_conv2d_fwd(g: *const rh_conv_geom, alpha: c_float, x: *const f32, w: *const f32, beta: c_float,
+                       y: *mut f32, bias: *const f32, ws: *mut c_void, ws_bytes: size_t, flags: c_int,
+                       stream: rh_stream_t) -> c_int;
+  pub fn rh_conv2d_bwd_filter(g: *const rh_conv_geom, alpha: c_float, x: *const f32, dy: *const f32,
+                              beta: c_float, dw: *mut f32, ws: *mut c_void, ws_bytes: size_t, flags: c_int,
+                              stream: rh_stream_t) -> c_int;
+  pub fn rh_conv2d_bwd_bias(n: i32, k: i32, plane: i32, alpha: c_float, dy: *const f32, beta: c_float,
+                            db: *mut f32, stream: rh_stream_t) -> c_int;
+  pub fn rh_conv2d_bwd_data(g: *const rh_conv_geom, alpha: c_float, w: *const f32, dy: *const f32,
+                            beta: c_float, dx: *mut f32, ws: *mut c_void, ws_bytes: size_t, flags: c_int,
+                            stream: rh_stream_t) -> c_int;
+
+  pub fn rh_add_bias_nchw(bias: *const f32, y: *mut f32, plane: i32, k: i32, n: i32, alpha: c_float,
+                          beta: c_float, stream: rh_stream_t) -> c_int;
+  // Same names and argument lists as rembrandt_kernels::ffi (src/operator/mod.rs:1108-1113, 1154-1160).
+  pub fn rembrandt_kernel_batch_map_rect_inplace(y: *mut f32, frame_len: i32, batch: i32, stream: rh_stream_t);
+  pub fn rembrandt_kernel_batch_map_rect_backprop_inplace(y: *const f32, frame_len: i32, batch: i32,
+                                                          dy: *mut f32, stream: rh_stream_t);
+
+  pub fn rh_sgemm_workspace_bytes(m: i32, n: i32, k: i32) -> size_t;
+  pub fn rh_sgemm(trans_a: c_int, trans_b: c_int, m: i32, n: i32, k: i32, alpha: c_float, a: *const f32,
+                  lda: i32, b: *const f32, ldb: i32, beta: c_float, c: *mut f32, ldc: i32, ws: *mut c_void,
+                  ws_bytes: size_t, flags: c_int, stream: rh_stream_t) -> c_int;
+  pub fn rh_saxpy(n: i64, alpha: c_float, x: *const f32, y: *mut f32, stream: rh_stream_t) -> c_int;
+  pub fn rh_sscal(n: i64, alpha: c_float, x: *mut f32, stream: rh_stream_t) -> c_int;
+
+  pub fn rh_pool2d_fwd(g: *const rh_pool_geom, x: *const f32, y: *mut f32, opt_argmax: *mut i32,
+                       stream: rh_stream_t) -> c_int;
+  pub fn rh_pool2d_bwd(g: *const rh_pool_geom, x: *const f32, y: *const f32, dy: *const f32, dx: *mut f32,
+                       opt_argmax: *const i32, stream: rh_stream_t) -> c_int;
+
+  pub fn rh_softmax_fwd(x: *const f32, p: *mut f32, c: i32, n: i32, stream: rh_stream_t) -> c_int;
+  // Same names and argument lists as rembrandt_kernels::ffi (src/operator/loss.rs:132-140, 191-210, 229-239).
+  pub fn rembrandt_kernel_batch_map_softmax_kl_backward(p: *const f32, c: i32, n: i32, labels: *const i32,
+                                                        weights: *const f32, dx: *mut f32, stream: rh_stream_t);
+  pub fn rembrandt_kernel_batch_map_softmax_kl_loss1(p: *const f32, c: i32, n: i32, labels: *const i32,
+                                                     weights: *const f32, beta: c_float, loss1: *mut f32,
+                                                     stream: rh_stream_t);
+  pub fn rembrandt_kernel_batch_blockreduce_sum(src: *const f32, len: i32, batch: i32, dst: *mut f32,
+                                                beta: c_float, stream: rh_stream_t);
+  pub fn rembrandt_kernel_batch_blockreduce_argmax(src: *const f32, len: i32, batch: i32, max_out: *mut f32,
+                                                   idx_out: *mut i32, stream: rh_stream_t);
+
+  pub fn rh_sgd_momentum_step(n: i64, w: *mut f32, g: *mut f32, v: *mut f32, l2: c_float, scale: c_float,
+                              mu: c_float, apply: c_float, zero_grad: c_int, stream: rh_stream_t) -> c_int;
+  pub fn rh_descend(n: i64, w: *mut f32, g: *mut f32, s: c_float, l2: c_float, stream: rh_stream_t) -> c_int;
+}
+
+/// The reference `unwrap()`s / `panic!`s on every native error (src/operator/mod.rs:1685-1696).
+pub fn unwrap(code: c_int, what: &str) {
+  if code != 0 {
+    let msg = unsafe { ::std::ffi::CStr::from_ptr(rh_error_string(code)) };
+    panic!("{} failed: {} ({:?})", what, code, msg);
+  }
+}
