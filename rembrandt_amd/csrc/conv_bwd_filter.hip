@@ -25,7 +25,7 @@ static BwdFilterPlan plan_bwd_filter(const ConvDims& d) {
   // second round: a block that runs alone on its CU uses the matrix pipe less well than three
   // sharing it, so a ragged tail costs more than its share.  Every slice keeps at least 32 K
   // steps so the prologue and the partial-sum traffic stay small next to the contraction.
-  const int slots = 256 * 3;
+  const int slots = 256 * (p.bm == 128 ? RH_OCC_128 : p.bm == 96 ? 2 : 3);
   int want = slots / p.tiles;
   const int max_by_depth = k_chunks / 32 > 0 ? k_chunks / 32 : 1;
   if (want > max_by_depth) want = max_by_depth;
@@ -60,6 +60,136 @@ void launch_split_reduce(const float* part, int splits, long long split_stride, 
   ProfScope prof("split_reduce", 4.0 * (double)total * (splits + 1), stream);
   hipLaunchKernelGGL(split_reduce_kernel, dim3(stream_grid(total, 256)), dim3(256), 0, stream, part, splits,
                      split_stride, out, rows, cols, ld, alpha, beta);
+}
+
+// ---- scalar-offset path ------------------------------------------------------------------------
+// Both operands are read with lanes along rows and a wave-uniform offset per contraction index
+// (an output pixel), from channel-last scratch copies:
+//   A = dyT[pix][ko]                      (rows ko;      k offset = pix*Kout*4)
+//   B = xT[n][hp][wp][c], zero padded     (rows (r,s,c); vbase = 4*((r*Wp+s)*C+c), k offset from a
+//                                          per-pixel table 4*C*((n*Hp + p*st)*Wp + q*st))
+// The result comes out as dw'[ko][(r,s,c)]; the reduction kernel puts it back in [ko][c][r][s] order.
+// The channel-last path pays two transposes; it wins when the contraction is deep relative to them.
+static bool use_soff_bwd_filter(const ConvDims& d) {
+  static const int force = [] { const char* e = getenv("RH_BWDF_SOFF"); return e ? atoi(e) : -1; }();
+  if (force >= 0) return force != 0;
+  // FLOPs of the contraction per byte the two transposes move (measured: conv1-like 119 and 1x1 24 lose,
+  // 3x3 / 5x5 layers at 690-875 win)
+  const double flops = 2.0 * d.K * d.C * d.R * d.S * (double)d.N * d.P * d.Q;
+  const double bytes = 8.0 * ((double)d.y_elems + (double)d.N * d.C * (d.H + 2 * d.pad) * (d.W + 2 * d.pad));
+  return flops / bytes >= 300.0;
+}
+
+struct BwdFilterSoffPlan {
+  int n_k, Hp, Wp, bm, bn, tiles, splits;
+  size_t tab_bytes, dyt_bytes, xt_bytes, part_bytes;
+  bool ok;
+  size_t total() const { return tab_bytes + dyt_bytes + xt_bytes + part_bytes; }
+};
+
+static BwdFilterSoffPlan plan_bwd_filter_soff(const ConvDims& d) {
+  BwdFilterSoffPlan p;
+  const int CRS = d.C * d.R * d.S;
+  const long long M = (long long)d.N * d.P * d.Q;
+  p.Hp = d.H + 2 * d.pad;
+  p.Wp = d.W + 2 * d.pad;
+  p.n_k = (int)((M + kTabPad - 1) / kTabPad * kTabPad);
+  p.bm = pick_bm(d.K);
+  p.bn = p.bm == 128 ? 128 : 256;
+  p.tiles = cdiv(d.K, p.bm) * cdiv(CRS, p.bn);
+  const int k_chunks = p.n_k / 16;
+  const int slots = 256 * (p.bm == 128 ? RH_OCC_128 : p.bm == 96 ? 2 : 3);
+  int want = slots / p.tiles;
+  const int max_by_depth = k_chunks / 32 > 0 ? k_chunks / 32 : 1;
+  if (want > max_by_depth) want = max_by_depth;
+  if (want > 256) want = 256;
+  if (want < 1) want = 1;
+  p.splits = want;
+  p.tab_bytes = align256(sizeof(int) * (size_t)p.n_k);
+  p.dyt_bytes = align256(sizeof(float) * (size_t)p.n_k * d.K);
+  p.xt_bytes = align256(sizeof(float) * (size_t)d.N * p.Hp * p.Wp * d.C);
+  p.part_bytes = align256(sizeof(float) * (size_t)p.splits * d.K * CRS);
+  p.ok = M > 0 && p.dyt_bytes <= kMaxBufferBytes && p.xt_bytes <= kMaxBufferBytes &&
+         (long long)d.S * d.C < (1 << 24);
+  return p;
+}
+
+// dst[n][pix][c] (pix over Hp x Wp, zero halo) = src[n][c][h][w]: 32 x 32 tiles through LDS so that both
+// the reads (along w) and the writes (along c) are contiguous.
+__global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                           int C, int H, int W, int Hp, int Wp, int halo) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int pix0 = blockIdx.x * 32, c0 = blockIdx.y * 32, n = blockIdx.z;
+  const int HpWp = Hp * Wp;
+  {
+    const int pix = pix0 + tx;
+    const int hp = pix / Wp, wp = pix - hp * Wp;
+    const int h = hp - halo, w = wp - halo;
+    const bool inside = pix < HpWp && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W;
+#pragma unroll
+    for (int j = 0; j < 32; j += 8) {
+      const int c = c0 + ty + j;
+      tile[ty + j][tx] = (inside && c < C) ? src[(((size_t)n * C + c) * H + h) * W + w] : 0.0f;
+    }
+  }
+  __syncthreads();
+  const int c = c0 + tx;
+#pragma unroll
+  for (int j = 0; j < 32; j += 8) {
+    const int pix = pix0 + ty + j;
+    if (pix < HpWp && c < C) dst[((size_t)n * HpWp + pix) * C + c] = tile[tx][ty + j];
+  }
+}
+
+static void launch_nchw_to_nhwc(const float* src, float* dst, int N, int C, int H, int W, int Hp, int Wp, int halo,
+                                hipStream_t stream) {
+  ProfScope prof("nchw_to_nhwc", 4.0 * ((double)N * C * H * W + (double)N * C * Hp * Wp), stream);
+  dim3 grid((unsigned)cdiv(Hp * Wp, 32), (unsigned)cdiv(C, 32), (unsigned)N);
+  hipLaunchKernelGGL(nchw_to_nhwc_kernel, grid, dim3(256), 0, stream, src, dst, C, H, W, Hp, Wp, halo);
+}
+
+// soff[pix] = 4*C*((n*Hp + p*st)*Wp + q*st) for pix = (n,p,q) < M, else 0; also zeroes the rows M..n_k of dyT.
+__global__ void prep_bwd_filter_soff_kernel(int* __restrict__ soff, float* __restrict__ dyT, int n_k, int M, int PQ,
+                                            int Q, int st, int Hp, int Wp, int C, int Kout) {
+  const int stride = gridDim.x * blockDim.x;
+  for (int pix = blockIdx.x * blockDim.x + threadIdx.x; pix < n_k; pix += stride) {
+    int off = 0;
+    if (pix < M) {
+      const int n = pix / PQ, pq = pix - n * PQ, p = pq / Q, q = pq - p * Q;
+      off = ((n * Hp + p * st) * Wp + q * st) * C * 4;
+    } else {
+      for (int k = 0; k < Kout; ++k) dyT[(size_t)pix * Kout + k] = 0.0f;
+    }
+    soff[pix] = off;
+  }
+}
+
+// dw[ko][c][r][s] = alpha * sum_s part[s][ko][(r,s,c)] + beta * dw
+__global__ void split_reduce_rsc_kernel(const float* __restrict__ part, int splits, long long split_stride,
+                                        float* __restrict__ dw, int K, int C, int R, int S, float alpha, float beta) {
+  const int CRS = C * R * S;
+  const long long total = (long long)K * CRS;
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long long)gridDim.x * blockDim.x) {
+    float acc = 0.0f;
+    for (int sp = 0; sp < splits; ++sp) acc += part[(long long)sp * split_stride + idx];
+    const int ko = (int)(idx / CRS), j = (int)(idx - (long long)ko * CRS);
+    const int r = j / (S * C), rem = j - r * (S * C), s2 = rem / C, c = rem - s2 * C;
+    float* dst = dw + (((size_t)ko * C + c) * R + r) * S + s2;
+    float val = alpha * acc;
+    if (beta != 0.0f) val += beta * *dst;
+    *dst = val;
+  }
+}
+
+template <class T>
+static int run_bwd_filter_soff(const RowSParams& ap, const RowSParams& bp, const EpiParams& ep, int n_k, int k_true,
+                               int splits, int* used, hipStream_t stream, const char* tag) {
+  constexpr int AROWS = T::BM % 64 == 0 ? T::BM : (T::BM + 63) / 64 * 64;
+  typedef LoadRowS<AROWS, T::BK, T::NT, true> AL;
+  typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
+  return launch_mfma_gemm<T, AL, BL, false>(ap, bp, ep, n_k, splits, used, stream, tag, k_true);
 }
 
 template <class T>
@@ -116,14 +246,22 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
   if (conv_dims(g, &d)) return 0;
   const int CRS = d.C * d.R * d.S, KRS = d.K * d.R * d.S;
   switch (pass) {
-    case RH_CONV_FWD:
-      return align256(sizeof(int4) * (size_t)round_up(CRS, kTabPad));
-    case RH_CONV_BWD_DATA:
-      return align256(sizeof(int4) * (size_t)round_up(KRS, kTabPad)) +
-             align256(sizeof(int) * (size_t)round_up(KRS, kTabPad));
+    case RH_CONV_FWD: {
+      const size_t legacy = align256(sizeof(int4) * (size_t)round_up(CRS, kTabPad));
+      const SoffPlan sp = plan_soff_fwd(d);
+      return sp.ok && sp.total() > legacy ? sp.total() : legacy;
+    }
+    case RH_CONV_BWD_DATA: {
+      const size_t legacy = align256(sizeof(int4) * (size_t)round_up(KRS, kTabPad)) +
+                            align256(sizeof(int) * (size_t)round_up(KRS, kTabPad));
+      const SoffPlan sp = plan_soff_bwd_data(d);
+      return sp.ok && sp.total() > legacy ? sp.total() : legacy;
+    }
     case RH_CONV_BWD_FILTER: {
       const BwdFilterPlan p = plan_bwd_filter(d);
-      return p.tab_bytes + p.part_bytes;
+      const BwdFilterSoffPlan sp = plan_bwd_filter_soff(d);
+      const size_t legacy = p.tab_bytes + p.part_bytes;
+      return sp.ok && sp.total() > legacy ? sp.total() : legacy;
     }
     default:
       return 0;
@@ -138,9 +276,51 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
   if (!x || !dy || !dw) return RH_E_INVALID;
   if (flags & RH_MATH_BF16_MFMA_FP32ACC) return RH_E_UNSUPPORTED;
   const BwdFilterPlan plan = plan_bwd_filter(d);
-  if (!ws || ws_bytes < plan.tab_bytes + plan.part_bytes || (reinterpret_cast<uintptr_t>(ws) & 255))
+  if (!ws || ws_bytes < rh_conv2d_workspace_bytes(g, RH_CONV_BWD_FILTER) || (reinterpret_cast<uintptr_t>(ws) & 255))
     return RH_E_WORKSPACE;
   hipStream_t stream = to_stream(stream_);
+
+  const BwdFilterSoffPlan sp = plan_bwd_filter_soff(d);
+  if (sp.ok && !legacy_gather() && use_soff_bwd_filter(d)) {
+    const int CRSs = d.C * d.R * d.S, Ms = d.N * d.P * d.Q;
+    char* base = static_cast<char*>(ws);
+    int* soff = reinterpret_cast<int*>(base);
+    float* dyT = reinterpret_cast<float*>(base + sp.tab_bytes);
+    float* xT = reinterpret_cast<float*>(base + sp.tab_bytes + sp.dyt_bytes);
+    float* parts = reinterpret_cast<float*>(base + sp.tab_bytes + sp.dyt_bytes + sp.xt_bytes);
+    hipLaunchKernelGGL(prep_bwd_filter_soff_kernel, dim3(cdiv(sp.n_k, 256)), dim3(256), 0, stream, soff, dyT, sp.n_k, Ms,
+                       d.P * d.Q, d.Q, d.st, sp.Hp, sp.Wp, d.C, d.K);
+    if (int e = launch_status()) return e;
+    launch_nchw_to_nhwc(dy, dyT, d.N, d.K, d.P, d.Q, d.P, d.Q, 0, stream);
+    if (int e = launch_status()) return e;
+    launch_nchw_to_nhwc(x, xT, d.N, d.C, d.H, d.W, sp.Hp, sp.Wp, d.pad, stream);
+    if (int e = launch_status()) return e;
+    RowSParams ap;  // dyT [pix][ko]
+    ap.ptr = dyT; ap.bytes = (uint32_t)(sizeof(float) * (size_t)sp.n_k * d.K);
+    ap.M = d.K; ap.inner = d.K; ap.innerW = d.K; ap.img_stride = 0; ap.a_stride = 0; ap.b_stride = 1;
+    ap.soff = nullptr; ap.ldk4 = d.K * 4;
+    RowSParams bp;  // xT [n][hp][wp][c]; rows j = (r, s, c)
+    bp.ptr = xT; bp.bytes = (uint32_t)(sizeof(float) * (size_t)d.N * sp.Hp * sp.Wp * d.C);
+    bp.M = CRSs; bp.inner = d.S * d.C; bp.innerW = d.S * d.C; bp.img_stride = sp.Wp * d.C; bp.a_stride = 0; bp.b_stride = 1;
+    bp.soff = soff; bp.ldk4 = 0;
+    EpiParams ep;
+    ep.out = parts; ep.bias = nullptr; ep.alpha = 1.0f; ep.beta = 0.0f;
+    ep.rows = d.K; ep.cols = CRSs; ep.inner = 0; ep.ld = CRSs; ep.relu = 0;
+    ep.split_stride = (long long)d.K * CRSs;
+    int used = 1, e = 0;
+    switch (sp.bm) {
+      case 128: e = run_bwd_filter_soff<T128x128>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_128x128"); break;
+      case 96:  e = run_bwd_filter_soff<T96x256>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_96x256"); break;
+      case 64:  e = run_bwd_filter_soff<T64x256>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_64x256"); break;
+      default:  e = run_bwd_filter_soff<T32x256>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_32x256"); break;
+    }
+    if (e) return e;
+    const long long total = (long long)d.K * CRSs;
+    ProfScope prof("split_reduce", 4.0 * (double)total * (used + 1), stream);
+    hipLaunchKernelGGL(split_reduce_rsc_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, parts, used,
+                       (long long)d.K * CRSs, dw, d.K, d.C, d.R, d.S, alpha, beta);
+    return launch_status();
+  }
 
   const int CRS = d.C * d.R * d.S;
   const int M = d.N * d.P * d.Q;

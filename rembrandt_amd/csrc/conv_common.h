@@ -56,7 +56,7 @@ inline int pick_bm(int rows) {
 template <class T, class AL, class BL, bool NCHW>
 inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Params& bp,
                             const EpiParams& ep, int K, int splits, int* splits_used,
-                            hipStream_t stream, const char* tag) {
+                            hipStream_t stream, const char* tag, int k_algorithmic = 0) {
   const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
   const int k_chunks = cdiv(K, T::BK);
   if (splits < 1) splits = 1;
@@ -73,14 +73,17 @@ inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Pa
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr != hipSuccess) return (int)attr;
   }
-  ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)K, stream);
+  ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)(k_algorithmic > 0 ? k_algorithmic : K), stream);
   hipLaunchKernelGGL((mfma_gemm_kernel<T, AL, BL, NCHW>), grid, dim3(T::NT), lds_bytes, stream, ap, bp, ep,
                      tiles_m, k_chunks, cps);
   return launch_status();
 }
 
+#ifndef RH_OCC_128
+#define RH_OCC_128 4
+#endif
 // Tile shapes in use.  rows x cols x k, waves as WM x WN.
-typedef Tile<128, 128, 16, 2, 2> T128x128;
+typedef Tile<128, 128, 16, 2, 2, RH_OCC_128> T128x128;
 typedef Tile<96, 256, 16, 1, 4> T96x256;
 typedef Tile<64, 256, 16, 1, 4> T64x256;
 typedef Tile<32, 256, 16, 1, 4> T32x256;
@@ -91,6 +94,12 @@ typedef Tile<128, 128, 32, 2, 2> T128x128k32;
 typedef Tile<128, 256, 32, 2, 2> T128x256k32;
 typedef Tile<256, 256, 16, 2, 4> T256x256w8;
 
+// RH_LEGACY_GATHER=1 forces the per-element gather loaders (kept for strided backward-data and as a cross-check).
+inline bool legacy_gather() {
+  static const bool v = [] { const char* e = getenv("RH_LEGACY_GATHER"); return e && atoi(e) != 0; }();
+  return v;
+}
+
 inline int tile_override() {
   static const int v = [] { const char* e = getenv("RH_CONV_TILE"); return e ? atoi(e) : 0; }();
   return v;
@@ -99,6 +108,51 @@ inline int tile_override() {
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
                          int ld, float alpha, float beta, hipStream_t stream);
+
+// Scratch layout of the scalar-offset forward / backward-data paths:
+//   [k -> byte offset table : n_k ints][transposed filter : n_k x rows floats][padded image copy]
+struct SoffPlan {
+  int n_k;         // contraction length rounded up to kTabPad
+  int Hp, Wp;      // padded image extent
+  int halo;        // zeros added on each side
+  size_t tab_bytes, wt_bytes, img_bytes;  // img_bytes == 0: the image is used in place
+  bool ok;         // false: fall back to the per-element gather path
+  size_t total() const { return tab_bytes + wt_bytes + img_bytes; }
+};
+
+inline SoffPlan plan_soff_fwd(const ConvDims& d) {
+  SoffPlan p;
+  p.n_k = round_up(d.C * d.R * d.S, kTabPad);
+  p.halo = d.pad;
+  p.Hp = d.H + 2 * d.pad;
+  p.Wp = d.W + 2 * d.pad;
+  p.tab_bytes = align256(sizeof(int) * (size_t)p.n_k);
+  p.wt_bytes = align256(sizeof(float) * (size_t)p.n_k * d.K);
+  const size_t img = sizeof(float) * (size_t)d.N * d.C * p.Hp * p.Wp;
+  p.img_bytes = d.pad > 0 ? align256(img) : 0;
+  p.ok = img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
+  return p;
+}
+
+// Backward-data with stride 1: dx[n,c,h,w] = sum dyp[n,ko,h+R-1-r,w+S-1-s] * w[ko,c,r,s] on dy padded
+// by R-1-pad zeros per side.
+inline SoffPlan plan_soff_bwd_data(const ConvDims& d) {
+  SoffPlan p;
+  p.n_k = round_up(d.K * d.R * d.S, kTabPad);
+  p.halo = d.R - 1 - d.pad;
+  p.Hp = d.P + 2 * p.halo;
+  p.Wp = d.Q + 2 * (d.S - 1 - d.pad);
+  p.tab_bytes = align256(sizeof(int) * (size_t)p.n_k);
+  p.wt_bytes = align256(sizeof(float) * (size_t)p.n_k * d.C);
+  const size_t img = p.halo >= 0 ? sizeof(float) * (size_t)d.N * d.K * p.Hp * p.Wp : 0;
+  p.img_bytes = p.halo > 0 ? align256(img) : 0;
+  p.ok = d.st == 1 && p.halo >= 0 && d.R == d.S && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
+  return p;
+}
+
+// dst[n][c][h+halo][w+halo] = src[n][c][h][w], zeros elsewhere; dst is planes x Hp x Wp.
+void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
+                      hipStream_t stream);
 
 void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int HW, int W,
                           hipStream_t stream);

@@ -22,6 +22,58 @@ void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int H
                      n_entries, CRS, R, S, HW, W);
 }
 
+// dst (planes x Hp x Wp) = src (planes x H x W) surrounded by `halo` zeros; one thread per 4 dst elements
+// of a row would need alignment care, so: one thread per dst element, rows contiguous across lanes.
+__global__ void pad_image_kernel(const float* __restrict__ src, float* __restrict__ dst, long long total, int H,
+                                 int W, int Hp, int Wp, int halo) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int wp = (int)(i % Wp);
+    const long long t = i / Wp;
+    const int hp = (int)(t % Hp);
+    const long long plane = t / Hp;
+    const int h = hp - halo, w = wp - halo;
+    dst[i] = ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) ? src[(plane * H + h) * W + w] : 0.0f;
+  }
+}
+
+void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
+                      hipStream_t stream) {
+  const long long total = planes * Hp * Wp;
+  ProfScope prof("pad_image", 4.0 * ((double)planes * H * W + (double)total), stream);
+  hipLaunchKernelGGL(pad_image_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, src, dst,
+                     total, H, W, Hp, Wp, halo);
+}
+
+// Forward scratch preparation: wT[k][ko] = w[ko][k] (zero rows for k >= CRS) and the k -> byte offset
+// table into the padded image, soff[k] = 4*(c*Hp*Wp + r*Wp + s) (0 past the end).
+__global__ void prep_fwd_soff_kernel(const float* __restrict__ w, float* __restrict__ wT, int* __restrict__ soff,
+                                     int n_k, int CRS, int K, int R, int S, int HpWp, int Wp) {
+  const long long total = (long long)n_k * K;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int k = (int)(i / K), ko = (int)(i - (long long)k * K);
+    wT[i] = k < CRS ? w[(size_t)ko * CRS + k] : 0.0f;
+    if (ko == 0) {
+      int off = 0;
+      if (k < CRS) {
+        const int c = k / (R * S), rs = k - c * (R * S), r = rs / S, s2 = rs - r * S;
+        off = (c * HpWp + r * Wp + s2) * 4;
+      }
+      soff[k] = off;
+    }
+  }
+}
+
+template <class T>
+static int run_fwd_soff(const RowSParams& ap, const RowSParams& bp, const EpiParams& ep, int n_k, int k_true,
+                        hipStream_t stream, const char* tag) {
+  constexpr int AROWS = T::BM % 64 == 0 ? T::BM : (T::BM + 63) / 64 * 64;  // loader rows: a multiple of the wave
+  typedef LoadRowS<AROWS, T::BK, T::NT, true> AL;
+  typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
+  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
+}
+
 template <class T>
 static int run_fwd(const ConvDims& d, const DenseParams& ap, const GatherParams& bp,
                    const EpiParams& ep, hipStream_t stream, const char* tag) {
@@ -53,6 +105,40 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
   hipStream_t stream = to_stream(stream_);
 
   const int CRS = d.C * d.R * d.S;
+  const SoffPlan sp = plan_soff_fwd(d);
+  if (sp.ok && !legacy_gather()) {
+    int* soff = static_cast<int*>(ws);
+    float* wT = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes);
+    const float* img = x;
+    if (sp.img_bytes) {
+      float* xp = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes);
+      launch_pad_image(x, xp, (long long)d.N * d.C, d.H, d.W, sp.Hp, sp.Wp, sp.halo, stream);
+      if (int e = launch_status()) return e;
+      img = xp;
+    }
+    hipLaunchKernelGGL(prep_fwd_soff_kernel, dim3(stream_grid((size_t)sp.n_k * d.K, 256)), dim3(256), 0, stream, w, wT,
+                       soff, sp.n_k, CRS, d.K, d.R, d.S, sp.Hp * sp.Wp, sp.Wp);
+    if (int e = launch_status()) return e;
+    RowSParams ap;  // transposed filter [k][ko]
+    ap.ptr = wT; ap.bytes = (uint32_t)(sizeof(float) * (size_t)sp.n_k * d.K);
+    ap.M = d.K; ap.inner = d.K; ap.innerW = d.K; ap.img_stride = 0; ap.a_stride = 0; ap.b_stride = 1;
+    ap.soff = nullptr; ap.ldk4 = d.K * 4;
+    RowSParams bp;  // padded image, rows = output pixels
+    bp.ptr = img; bp.bytes = (uint32_t)(sizeof(float) * (size_t)d.N * d.C * sp.Hp * sp.Wp);
+    bp.M = d.N * d.P * d.Q; bp.inner = d.P * d.Q; bp.innerW = d.Q;
+    bp.img_stride = d.C * sp.Hp * sp.Wp; bp.a_stride = d.st * sp.Wp; bp.b_stride = d.st;
+    bp.soff = soff; bp.ldk4 = 0;
+    EpiParams ep;
+    ep.out = y; ep.bias = (flags & RH_FUSE_BIAS) ? bias : nullptr; ep.alpha = alpha; ep.beta = beta;
+    ep.rows = d.K; ep.cols = bp.M; ep.inner = d.P * d.Q; ep.ld = 0; ep.relu = (flags & RH_FUSE_RELU) ? 1 : 0;
+    ep.split_stride = 0;
+    switch (pick_bm(d.K)) {
+      case 128: return run_fwd_soff<T128x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_128x128");
+      case 96:  return run_fwd_soff<T96x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_96x256");
+      case 64:  return run_fwd_soff<T64x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x256");
+      default:  return run_fwd_soff<T32x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_32x256");
+    }
+  }
   const int n_tab = round_up(CRS, kTabPad);
   int4* tab = static_cast<int4*>(ws);
   launch_build_fwd_tab(tab, n_tab, CRS, d.R, d.S, d.H * d.W, d.W, stream);

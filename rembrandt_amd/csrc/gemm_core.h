@@ -35,9 +35,10 @@ __device__ __forceinline__ float buf_load_f32(__amdgpu_buffer_rsrc_t r, uint32_t
   return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)(o << 2), 0, 0));
 }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_>
+// OCC = waves per SIMD the register allocation must leave room for (blocks per CU for 4-wave blocks).
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_ = 1>
 struct Tile {
-  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, OCC = OCC_;
   static constexpr int NT = WM * WN * kWave;
   static constexpr int TM = BM / (WM * 32), TN = BN / (WN * 32);
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile / wave mismatch");
@@ -221,6 +222,68 @@ struct LoadGatherR {
 };
 
 // ------------------------------------------------------------------------------------------
+// Scalar-offset operand: element (row, k) at  ptr + vbase(row) + soff(k)  (byte offsets), rows
+// along lanes.  vbase is fixed per lane for the whole K loop (VGPR), soff is wave-uniform (SGPR,
+// the soffset field of the buffer load), so loading an element costs no vector ALU work at all.
+// Used on operands prepared so that every (row, k) pair of a valid row is in range:
+//   * the filter transposed to [k][row] and zero padded to a multiple of the K step (LINEAR);
+//   * the gathered image, zero padded by the conv padding, with a k -> byte offset table
+//     (entries past the contraction length are 0: the filter rows there are zero).
+// A row past the end gets vbase = 0x80000000, which reads as 0.
+// Row decomposition: m -> (n, a, b) = (m / inner, (m % inner) / innerW, m % innerW);
+// vbase = 4 * (n*img_stride + a*a_stride + b*b_stride).
+// ------------------------------------------------------------------------------------------
+struct RowSParams {
+  const float* ptr; uint32_t bytes;
+  int M, inner, innerW;
+  int img_stride, a_stride, b_stride;
+  const int* soff;  // table of byte offsets (not LINEAR)
+  int ldk4;         // bytes between consecutive k (LINEAR)
+};
+
+template <int ROWS, int BK, int NT, bool LINEAR>
+struct LoadRowS {
+  static constexpr int CNT = ROWS * BK / NT;
+  static constexpr int LD = ROWS + lds_pad_kfast<BK>();
+  static_assert(NT % ROWS == 0 && (ROWS * BK) % NT == 0 && ROWS % kWave == 0, "loader shape");
+  typedef RowSParams Params;
+  __amdgpu_buffer_rsrc_t rsrc;
+  const int* tab;
+  uint32_t vbase;
+  int ldk4, kk0c, sbase;
+  int so[CNT];
+
+  __device__ __forceinline__ void init(const Params& p, int row0, int tid) {
+    rsrc = make_rsrc(p.ptr, p.bytes);
+    const int row = tid % ROWS;
+    const int kk0 = __builtin_amdgcn_readfirstlane(tid / ROWS);
+    kk0c = kk0 * CNT;
+    tab = p.soff;
+    ldk4 = p.ldk4;
+    sbase = kk0c * LD + row;
+    const int m = row0 + row;
+    const bool valid = m < p.M;
+    const int mm = valid ? m : 0;
+    const int n = mm / p.inner;
+    const int rem = mm - n * p.inner;
+    const int a = rem / p.innerW;
+    const int b = rem - a * p.innerW;
+    vbase = valid ? (uint32_t)(n * p.img_stride + a * p.a_stride + b * p.b_stride) << 2 : 0x80000000u;
+  }
+  __device__ __forceinline__ void prep(int k0) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) so[i] = LINEAR ? (k0 + kk0c + i) * ldk4 : tab[k0 + kk0c + i];
+  }
+  __device__ __forceinline__ float load_one(int i) const {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)vbase, so[i], 0));
+  }
+  __device__ __forceinline__ void store(float* s, const float (&v)[CNT]) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) s[sbase + i * LD] = v[i];
+  }
+};
+
+// ------------------------------------------------------------------------------------------
 // Backward-filter operands: the contraction index k is an output pixel (n,p,q); lanes run
 // along k because both dy and x are contiguous along q.
 //   A = dy:  element (ko, pix) = dy[(n*Kout + ko)*PQ + pq]
@@ -362,7 +425,7 @@ __device__ __forceinline__ int xcd_remap(int b, int nb) {
 }
 
 template <class T, class AL, class BL, bool NCHW>
-__global__ __launch_bounds__(T::NT) void mfma_gemm_kernel(typename AL::Params ap,
+__global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::Params ap,
                                                           typename BL::Params bp, EpiParams ep,
                                                           int tiles_m, int k_chunks,
                                                           int chunks_per_split) {
