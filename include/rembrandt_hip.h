@@ -100,6 +100,11 @@ int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const float* x, con
 /* db[k] = alpha * sum_{n,p,q} dy[n,k,p,q] + beta * db[k];  plane = P*Q. */
 int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy,
                        float beta, float* db, rh_stream_t stream);
+/* Same result through a two-stage reduction that fills the GPU when K is small (scratch from the caller;
+ * without scratch it falls back to the one-stage form). */
+size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane);
+int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
+                          float* db, void* ws, size_t ws_bytes, rh_stream_t stream);
 /* dx = alpha * corr^T(dy, w) + beta * dx. */
 int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const float* w, const float* dy,
                        float beta, float* dx, void* ws, size_t ws_bytes, int flags,

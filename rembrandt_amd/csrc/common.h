@@ -33,6 +33,33 @@ inline int stream_grid(size_t work_items, int block) {
   return static_cast<int>(want);
 }
 
+// Division of a non-negative 32-bit index (< 2^31) by a runtime constant as multiply-high + add + shift
+// (Granlund-Montgomery round-up method); the divisor's constants are computed once on the host.  The
+// bandwidth-bound kernels decompose a flat index per element: hardware integer division there costs
+// more instructions than everything else in the kernel.
+struct FastDiv {
+  uint32_t mul, shift, div;
+  FastDiv() : mul(1), shift(0), div(1) {}
+  explicit FastDiv(uint32_t d) : div(d) {
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    mul = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    shift = l;
+  }
+  __host__ __device__ __forceinline__ uint32_t quot(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (__umulhi(mul, n) + n) >> shift;
+#else
+    return (uint32_t)((((uint64_t)mul * n) >> 32) + n) >> shift;
+#endif
+  }
+  // n = q*div + r
+  __host__ __device__ __forceinline__ void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
+    q = quot(n);
+    r = n - q * div;
+  }
+};
+
 // Optional per-launch timing with HIP events (off by default; rh_profile_enable).  A scope
 // records an event before and after the launches made inside it, on the stream they go to.
 // `work` is the algorithmic work of those launches: FLOPs for contractions, bytes otherwise.

@@ -41,12 +41,11 @@ static BwdFilterPlan plan_bwd_filter(const ConvDims& d) {
 __global__ void split_reduce_kernel(const float* __restrict__ part, int splits, long long split_stride,
                                     float* __restrict__ out, int rows, int cols, int ld, float alpha,
                                     float beta) {
-  const long long total = (long long)rows * cols;
-  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (long long)gridDim.x * blockDim.x) {
+  const unsigned total = (unsigned)rows * (unsigned)cols;  // a filter gradient / GEMM result: far below 2^31
+  for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     float acc = 0.0f;
     for (int s = 0; s < splits; ++s) acc += part[(long long)s * split_stride + idx];
-    const int i = (int)(idx / cols), j = (int)(idx - (long long)i * cols);
+    const int i = (int)(idx / (unsigned)cols), j = (int)(idx - (unsigned)i * (unsigned)cols);
     float* dst = out + (size_t)i * ld + j;
     float val = alpha * acc;
     if (beta != 0.0f) val += beta * *dst;
@@ -169,12 +168,11 @@ __global__ void prep_bwd_filter_soff_kernel(int* __restrict__ soff, float* __res
 __global__ void split_reduce_rsc_kernel(const float* __restrict__ part, int splits, long long split_stride,
                                         float* __restrict__ dw, int K, int C, int R, int S, float alpha, float beta) {
   const int CRS = C * R * S;
-  const long long total = (long long)K * CRS;
-  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (long long)gridDim.x * blockDim.x) {
+  const unsigned total = (unsigned)K * (unsigned)CRS;
+  for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     float acc = 0.0f;
     for (int sp = 0; sp < splits; ++sp) acc += part[(long long)sp * split_stride + idx];
-    const int ko = (int)(idx / CRS), j = (int)(idx - (long long)ko * CRS);
+    const int ko = (int)(idx / (unsigned)CRS), j = (int)(idx - (unsigned)ko * (unsigned)CRS);
     const int r = j / (S * C), rem = j - r * (S * C), s2 = rem / C, c = rem - s2 * C;
     float* dst = dw + (((size_t)ko * C + c) * R + r) * S + s2;
     float val = alpha * acc;
@@ -200,29 +198,64 @@ static int run_bwd_filter(const PixDyParams& ap, const PixXParams& bp, const Epi
   return launch_mfma_gemm<T, AL, BL, false>(ap, bp, ep, M, splits, used, stream, tag);
 }
 
-// db[k] = alpha * sum_{n, i<plane} dy[(n*K + k)*plane + i] + beta * db[k]; one block per k.
+// db[k] = alpha * sum_{n, i<plane} dy[(n*K + k)*plane + i] + beta * db[k].  grid = (K, 1): the 16 waves of
+// a block each walk whole planes (one image at a time), lanes along the plane, no index divisions.
 __global__ __launch_bounds__(1024) void bwd_bias_kernel(const float* __restrict__ dy, int N, int K,
                                                         int plane, float alpha, float beta,
                                                         float* __restrict__ db) {
   const int k = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   float acc = 0.0f;
-  const long long total = (long long)N * plane;
-  for (long long t = threadIdx.x; t < total; t += blockDim.x) {
-    const int n = (int)(t / plane);
-    const int i = (int)(t - (long long)n * plane);
-    acc += dy[((size_t)n * K + k) * plane + i];
+  for (int n = wave; n < N; n += nwaves) {
+    const float* p = dy + ((size_t)n * K + k) * plane;
+    for (int i = lane; i < plane; i += 64) acc += p[i];
   }
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
   __shared__ float part[16];
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+  if (lane == 0) part[wave] = acc;
   __syncthreads();
   if (threadIdx.x == 0) {
     float s = 0.0f;
-    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) s += part[i];
+    for (int i = 0; i < nwaves; ++i) s += part[i];
     float v = alpha * s;
     if (beta != 0.0f) v += beta * db[k];
     db[k] = v;
   }
+}
+
+// Two-stage form for few channels and many images: block (k, g) sums the planes of images n = g, g+G, ...
+// into part[g*K + k]; bwd_bias_finish_kernel adds the G partial sums in a fixed order.
+__global__ __launch_bounds__(256) void bwd_bias_partial_kernel(const float* __restrict__ dy, int N, int K, int plane,
+                                                               float* __restrict__ part) {
+  const int k = blockIdx.x, g = blockIdx.y, G = gridDim.y;
+  float acc = 0.0f;
+  for (int n = g; n < N; n += G) {
+    const float* p = dy + ((size_t)n * K + k) * plane;
+    for (int i = threadIdx.x; i < plane; i += 256) acc += p[i];
+  }
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
+  __shared__ float sm[4];
+  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) part[(size_t)g * K + k] = sm[0] + sm[1] + sm[2] + sm[3];
+}
+
+__global__ void bwd_bias_finish_kernel(const float* __restrict__ part, int G, int K, float alpha, float beta,
+                                       float* __restrict__ db) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= K) return;
+  float s = 0.0f;
+  for (int g = 0; g < G; ++g) s += part[(size_t)g * K + k];
+  float v = alpha * s;
+  if (beta != 0.0f) v += beta * db[k];
+  db[k] = v;
+}
+
+static int bwd_bias_groups(int N, int K) {
+  int G = cdiv(2048, K);
+  if (G > N) G = N;
+  if (G > 64) G = 64;
+  return G < 1 ? 1 : G;
 }
 
 // plane == 1 (affine): dy is [N][K]; one thread per k walks the batch, coalesced across k.
@@ -352,6 +385,26 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
     if (e) return e;
   }
   launch_split_reduce(part, used, (long long)d.K * CRS, dw, d.K, CRS, CRS, alpha, beta, stream);
+  return launch_status();
+}
+
+extern "C" size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane) {
+  if (N <= 0 || K <= 0 || plane <= 1) return 0;
+  return align256(sizeof(float) * (size_t)bwd_bias_groups(N, K) * K);
+}
+
+extern "C" int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
+                                     float* db, void* ws, size_t ws_bytes, rh_stream_t stream_) {
+  if (N <= 0 || K <= 0 || plane <= 0 || !dy || !db) return RH_E_INVALID;
+  const size_t need = rh_conv2d_bwd_bias_workspace_bytes(N, K, plane);
+  if (plane == 1 || need == 0 || !ws || ws_bytes < need) return rh_conv2d_bwd_bias(N, K, plane, alpha, dy, beta, db, stream_);
+  hipStream_t stream = to_stream(stream_);
+  const int G = bwd_bias_groups(N, K);
+  float* part = static_cast<float*>(ws);
+  ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
+  hipLaunchKernelGGL(bwd_bias_partial_kernel, dim3(K, G), dim3(256), 0, stream, dy, N, K, plane, part);
+  if (int e = launch_status()) return e;
+  hipLaunchKernelGGL(bwd_bias_finish_kernel, dim3(cdiv(K, 256)), dim3(256), 0, stream, part, G, K, alpha, beta, db);
   return launch_status();
 }
 

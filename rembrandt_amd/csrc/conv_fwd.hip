@@ -24,25 +24,25 @@ void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int H
 
 // dst (planes x Hp x Wp) = src (planes x H x W) surrounded by `halo` zeros; one thread per 4 dst elements
 // of a row would need alignment care, so: one thread per dst element, rows contiguous across lanes.
-__global__ void pad_image_kernel(const float* __restrict__ src, float* __restrict__ dst, long long total, int H,
-                                 int W, int Hp, int Wp, int halo) {
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int wp = (int)(i % Wp);
-    const long long t = i / Wp;
-    const int hp = (int)(t % Hp);
-    const long long plane = t / Hp;
-    const int h = hp - halo, w = wp - halo;
-    dst[i] = ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) ? src[(plane * H + h) * W + w] : 0.0f;
+__global__ void pad_image_kernel(const float* __restrict__ src, float* __restrict__ dst, unsigned total, int H, int W,
+                                 FastDiv dHp, FastDiv dWp, int halo) {
+  const unsigned stride = gridDim.x * blockDim.x;
+  for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    uint32_t t, wp, plane, hp;
+    dWp.divmod(i, t, wp);
+    dHp.divmod(t, plane, hp);
+    const int h = (int)hp - halo, w = (int)wp - halo;
+    dst[i] = ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) ? src[((size_t)plane * H + h) * W + w] : 0.0f;
   }
 }
 
+// total elements of dst must be below 2^31 (a tensor is at most 2 GiB here)
 void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
                       hipStream_t stream) {
   const long long total = planes * Hp * Wp;
   ProfScope prof("pad_image", 4.0 * ((double)planes * H * W + (double)total), stream);
   hipLaunchKernelGGL(pad_image_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, src, dst,
-                     total, H, W, Hp, Wp, halo);
+                     (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo);
 }
 
 // Forward scratch preparation: wT[k][ko] = w[ko][k] (zero rows for k >= CRS) and the k -> byte offset

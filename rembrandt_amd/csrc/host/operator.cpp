@@ -395,6 +395,7 @@ class Conv2dOperator : public Operator {
     if (backward_enabled(capability)) {
       ws = std::max(ws, rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_FILTER));
       ws = std::max(ws, rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_DATA));
+      ws = std::max(ws, rh_conv2d_bwd_bias_workspace_bytes(g.N, g.K, (int)(out_dims_.w * out_dims_.h)));
     }
     workspace_.reset(new DeviceBuffer<uint8_t>(std::max<size_t>(ws, 256), context));
   }
@@ -431,8 +432,9 @@ class Conv2dOperator : public Operator {
     apply_rect_backprop(config_.act_func, out_act_->as_ptr(), out_dims_.len(), batch_size, out_delta_->as_mut_ptr(), s);
     unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in_act_->as_ptr(), out_delta_->as_ptr(), 1.0f, params_.grad_weights->as_mut_ptr(),
                                 workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward filter");
-    unwrap(rh_conv2d_bwd_bias((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), 1.0f,
-                              out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), s), "conv2d backward bias");
+    unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), 1.0f,
+                                 out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), workspace_->as_mut_ptr(),
+                                 workspace_->len(), s), "conv2d backward bias");
     if (in_delta_) {
       unwrap(rh_conv2d_bwd_data(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
                                 workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward data");

@@ -7,7 +7,7 @@
 
 namespace rh {
 
-struct PoolDims { int N, C, H, W, k, st, pad, P, Q, mode; };
+struct PoolDims { int N, C, H, W, k, st, pad, P, Q, mode; FastDiv dP, dQ, dH, dW, dSt; };
 
 inline int pool_out_dim(int in, int size, int stride, int pad, int round) {
   if (round == RH_ROUND_CEIL) {
@@ -40,17 +40,28 @@ __device__ __forceinline__ int window_argmax(const float* __restrict__ xp, int H
   return bi;
 }
 
+// I is the flat index type: 32-bit whenever the tensors allow it (64-bit divisions cost ~10x more).
+template <class I>
 __global__ void pool_fwd_kernel(PoolDims d, const float* __restrict__ x, float* __restrict__ y,
                                 int* __restrict__ argmax) {
-  const long long total = (long long)d.N * d.C * d.P * d.Q;
-  const long long stride = (long long)gridDim.x * blockDim.x;
+  const I total = (I)d.N * d.C * d.P * d.Q;
+  const I stride = (I)gridDim.x * blockDim.x;
   const float inv = 1.0f / (float)(d.k * d.k);
-  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-    const int q = (int)(idx % d.Q);
-    const long long t = idx / d.Q;
-    const int p = (int)(t % d.P);
-    const long long nc = t / d.P;
-    const float* xp = x + nc * d.H * d.W;
+  for (I idx = (I)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    I t, nc;
+    int q, p;
+    if (sizeof(I) == 4) {
+      uint32_t t32, q32, nc32, p32;
+      d.dQ.divmod((uint32_t)idx, t32, q32);
+      d.dP.divmod(t32, nc32, p32);
+      t = t32; nc = nc32; q = (int)q32; p = (int)p32;
+    } else {
+      t = idx / (I)d.Q;
+      q = (int)(idx - t * (I)d.Q);
+      nc = t / (I)d.P;
+      p = (int)(t - nc * (I)d.P);
+    }
+    const float* xp = x + (size_t)nc * d.H * d.W;
     if (d.mode == RH_POOL_MAX) {
       float best;
       const int bi = window_argmax(xp, d.H, d.W, p, q, d.k, d.st, d.pad, &best);
@@ -72,29 +83,39 @@ __global__ void pool_fwd_kernel(PoolDims d, const float* __restrict__ x, float* 
   }
 }
 
+template <class I>
 __global__ void pool_bwd_kernel(PoolDims d, const float* __restrict__ x, const float* __restrict__ dy,
                                 float* __restrict__ dx, const int* __restrict__ argmax) {
-  const long long total = (long long)d.N * d.C * d.H * d.W;
-  const long long stride = (long long)gridDim.x * blockDim.x;
+  const I total = (I)d.N * d.C * d.H * d.W;
+  const I stride = (I)gridDim.x * blockDim.x;
   const float inv = 1.0f / (float)(d.k * d.k);
-  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-    const int w = (int)(idx % d.W);
-    const long long t = idx / d.W;
-    const int h = (int)(t % d.H);
-    const long long nc = t / d.H;
+  for (I idx = (I)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    I t, nc;
+    int w, h;
+    if (sizeof(I) == 4) {
+      uint32_t t32, w32, nc32, h32;
+      d.dW.divmod((uint32_t)idx, t32, w32);
+      d.dH.divmod(t32, nc32, h32);
+      t = t32; nc = nc32; w = (int)w32; h = (int)h32;
+    } else {
+      t = idx / (I)d.W;
+      w = (int)(idx - t * (I)d.W);
+      nc = t / (I)d.H;
+      h = (int)(t - nc * (I)d.H);
+    }
     // windows p with p*st - pad <= h <= p*st - pad + k - 1
     const int th = h + d.pad - (d.k - 1), tw = w + d.pad - (d.k - 1);
-    const int p_lo = th > 0 ? (th + d.st - 1) / d.st : 0;
-    const int q_lo = tw > 0 ? (tw + d.st - 1) / d.st : 0;
-    int p_hi = (h + d.pad) / d.st, q_hi = (w + d.pad) / d.st;
+    const int p_lo = th > 0 ? (int)d.dSt.quot((uint32_t)(th + d.st - 1)) : 0;
+    const int q_lo = tw > 0 ? (int)d.dSt.quot((uint32_t)(tw + d.st - 1)) : 0;
+    int p_hi = (int)d.dSt.quot((uint32_t)(h + d.pad)), q_hi = (int)d.dSt.quot((uint32_t)(w + d.pad));
     if (p_hi > d.P - 1) p_hi = d.P - 1;
     if (q_hi > d.Q - 1) q_hi = d.Q - 1;
-    const float* dyp = dy + nc * d.P * d.Q;
+    const float* dyp = dy + (size_t)nc * d.P * d.Q;
     float acc = 0.0f;
     if (d.mode == RH_POOL_MAX) {
       const int me = h * d.W + w;
-      const float* xp = x ? x + nc * d.H * d.W : nullptr;
-      const int* ap = argmax ? argmax + nc * d.P * d.Q : nullptr;
+      const float* xp = x ? x + (size_t)nc * d.H * d.W : nullptr;
+      const int* ap = argmax ? argmax + (size_t)nc * d.P * d.Q : nullptr;
       for (int p = p_lo; p <= p_hi; ++p)
         for (int q = q_lo; q <= q_hi; ++q) {
           int bi;
@@ -114,6 +135,45 @@ __global__ void pool_bwd_kernel(PoolDims d, const float* __restrict__ x, const f
   }
 }
 
+// Max-pool backward driven by the arg-max mask, one block per group of PB consecutive planes: the
+// group's dy and mask (PB*P*Q values each) are staged in LDS with coalesced reads, then every input
+// element looks its covering windows up in LDS and dx is written coalesced.  No dependent global loads.
+__global__ __launch_bounds__(256) void pool_bwd_mask_lds_kernel(PoolDims d, FastDiv dHW, int PB, long long planes,
+                                                                const float* __restrict__ dy, const int* __restrict__ argmax,
+                                                                float* __restrict__ dx) {
+  extern __shared__ float lds_pool[];
+  const int PQ = d.P * d.Q, HW = d.H * d.W;
+  const long long plane0 = (long long)blockIdx.x * PB;
+  const int np = (int)(planes - plane0 < PB ? planes - plane0 : PB);
+  float* sdy = lds_pool;
+  int* smask = reinterpret_cast<int*>(lds_pool + PB * PQ);
+  const int n_out = np * PQ, n_in = np * HW;
+  const float* gdy = dy + plane0 * PQ;
+  const int* gm = argmax + plane0 * PQ;
+  for (int i = threadIdx.x; i < n_out; i += 256) { sdy[i] = gdy[i]; smask[i] = gm[i]; }
+  __syncthreads();
+  float* gdx = dx + plane0 * HW;
+  for (int e = threadIdx.x; e < n_in; e += 256) {
+    uint32_t pl, hw, h, w;
+    dHW.divmod((uint32_t)e, pl, hw);
+    d.dW.divmod(hw, h, w);
+    const int th = (int)h + d.pad - (d.k - 1), tw = (int)w + d.pad - (d.k - 1);
+    const int p_lo = th > 0 ? (int)d.dSt.quot((uint32_t)(th + d.st - 1)) : 0;
+    const int q_lo = tw > 0 ? (int)d.dSt.quot((uint32_t)(tw + d.st - 1)) : 0;
+    int p_hi = (int)d.dSt.quot(h + d.pad), q_hi = (int)d.dSt.quot(w + d.pad);
+    if (p_hi > d.P - 1) p_hi = d.P - 1;
+    if (q_hi > d.Q - 1) q_hi = d.Q - 1;
+    const int base = (int)pl * PQ;
+    float acc = 0.0f;
+    for (int p = p_lo; p <= p_hi; ++p)
+      for (int q = q_lo; q <= q_hi; ++q) {
+        const int o = base + p * d.Q + q;
+        if (smask[o] == (int)hw) acc += sdy[o];
+      }
+    gdx[e] = acc;
+  }
+}
+
 static int pool_dims(const rh_pool_geom* g, PoolDims* d) {
   if (!g) return RH_E_INVALID;
   if (g->N <= 0 || g->C <= 0 || g->H <= 0 || g->W <= 0 || g->size <= 0 || g->stride <= 0 || g->pad < 0)
@@ -125,6 +185,11 @@ static int pool_dims(const rh_pool_geom* g, PoolDims* d) {
   d->P = pool_out_dim(g->H, g->size, g->stride, g->pad, g->round);
   d->Q = pool_out_dim(g->W, g->size, g->stride, g->pad, g->round);
   if ((long long)g->H * g->W >= (1ll << 31)) return RH_E_LIMIT;
+  d->dP = FastDiv((uint32_t)(d->P > 0 ? d->P : 1));
+  d->dQ = FastDiv((uint32_t)(d->Q > 0 ? d->Q : 1));
+  d->dH = FastDiv((uint32_t)d->H);
+  d->dW = FastDiv((uint32_t)d->W);
+  d->dSt = FastDiv((uint32_t)d->st);
   return 0;
 }
 
@@ -146,8 +211,12 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
   if (total == 0) return 0;
   ProfScope prof(d.mode == RH_POOL_MAX ? "pool_max_fwd" : "pool_avg_fwd",
                  4.0 * ((double)d.N * d.C * d.H * d.W + (double)total * (opt_argmax ? 2 : 1)), to_stream(stream));
-  hipLaunchKernelGGL(pool_fwd_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, to_stream(stream), d, x,
-                     y, opt_argmax);
+  const long long in_total = (long long)d.N * d.C * d.H * d.W;
+  const dim3 grid((unsigned)cdiv<long long>(total, 256) > (1u << 20) ? (1u << 20) : (unsigned)cdiv<long long>(total, 256));
+  if (total < (1ll << 31) && in_total < (1ll << 31))
+    hipLaunchKernelGGL(pool_fwd_kernel<unsigned>, grid, dim3(256), 0, to_stream(stream), d, x, y, opt_argmax);
+  else
+    hipLaunchKernelGGL(pool_fwd_kernel<long long>, grid, dim3(256), 0, to_stream(stream), d, x, y, opt_argmax);
   return launch_status();
 }
 
@@ -163,7 +232,22 @@ extern "C" int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float*
   // bytes: write dx, read dy, plus the arg-max mask or (max without mask) x itself
   const double bwd_bytes = 4.0 * ((double)total + out_elems + (d.mode == RH_POOL_MAX ? (opt_argmax ? out_elems : (double)total) : 0.0));
   ProfScope prof(d.mode == RH_POOL_MAX ? "pool_max_bwd" : "pool_avg_bwd", bwd_bytes, to_stream(stream));
-  hipLaunchKernelGGL(pool_bwd_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, to_stream(stream), d, x,
-                     dy, dx, opt_argmax);
+  if (d.mode == RH_POOL_MAX && opt_argmax && d.P * d.Q <= 2048 && d.H * d.W <= (1 << 20)) {
+    const int PQ = d.P * d.Q;
+    int PB = 2048 / PQ;
+    if (PB > 64) PB = 64;
+    const long long planes = (long long)d.N * d.C;
+    const long long blocks = cdiv<long long>(planes, PB);
+    if (blocks < (1ll << 31)) {
+      hipLaunchKernelGGL(pool_bwd_mask_lds_kernel, dim3((unsigned)blocks), dim3(256), (size_t)PB * PQ * 8, to_stream(stream), d,
+                         FastDiv((uint32_t)(d.H * d.W)), PB, planes, dy, opt_argmax, dx);
+      return launch_status();
+    }
+  }
+  const dim3 grid((unsigned)cdiv<long long>(total, 256) > (1u << 20) ? (1u << 20) : (unsigned)cdiv<long long>(total, 256));
+  if (total < (1ll << 31))
+    hipLaunchKernelGGL(pool_bwd_kernel<unsigned>, grid, dim3(256), 0, to_stream(stream), d, x, dy, dx, opt_argmax);
+  else
+    hipLaunchKernelGGL(pool_bwd_kernel<long long>, grid, dim3(256), 0, to_stream(stream), d, x, dy, dx, opt_argmax);
   return launch_status();
 }

@@ -71,12 +71,17 @@ def conv2d_bwd_filter(x, dy, w_shape, stride, pad, alpha=1.0, beta=0.0, dw=None)
     return dw
 
 
-def conv2d_bwd_bias(dy, alpha=1.0, beta=0.0, db=None):
+def conv2d_bwd_bias(dy, alpha=1.0, beta=0.0, db=None, two_stage=False):
     N, K = dy.shape[0], dy.shape[1]
     plane = dy.numel() // (N * K)
     if db is None:
         db = torch.zeros((K,), dtype=torch.float32, device=dy.device)
-    check(lib().rh_conv2d_bwd_bias(N, K, plane, alpha, _p(dy), beta, _p(db), _stream()), "rh_conv2d_bwd_bias")
+    if two_stage:
+        ws = workspace(lib().rh_conv2d_bwd_bias_workspace_bytes(N, K, plane), dy.device)
+        check(lib().rh_conv2d_bwd_bias_ws(N, K, plane, alpha, _p(dy), beta, _p(db), _p(ws), ws.numel(), _stream()),
+              "rh_conv2d_bwd_bias_ws")
+    else:
+        check(lib().rh_conv2d_bwd_bias(N, K, plane, alpha, _p(dy), beta, _p(db), _stream()), "rh_conv2d_bwd_bias")
     return db
 
 

@@ -66,6 +66,9 @@ def test_conv2d_all_passes(dev, case):
 
     db = ops.conv2d_bwd_bias(dyd)
     assert_close(N(db), O.conv2d_bwd_bias(dy), "conv bwd bias")
+    db0 = synth.normal(11, 7, (K,))
+    db2 = ops.conv2d_bwd_bias(dyd, alpha=0.5, beta=1.0, db=T(db0, dev), two_stage=True)
+    assert_close(N(db2), O.conv2d_bwd_bias(dy, 0.5, 1.0, db0.copy()), "conv bwd bias (two-stage)")
 
     dx_ref = O.conv2d_bwd_data(w, dy, x.shape, st, pad)
     dx = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad)
