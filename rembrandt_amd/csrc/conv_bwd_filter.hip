@@ -223,51 +223,52 @@ __global__ __launch_bounds__(1024) void bwd_bias_kernel(const float* __restrict_
   }
 }
 
-// Two-stage form for few channels and many images: block (k, g) sums the planes of images n = g, g+G, ...
-// into part[g*K + k]; bwd_bias_finish_kernel adds the G partial sums in a fixed order.
-__global__ __launch_bounds__(256) void bwd_bias_partial_kernel(const float* __restrict__ dy, int N, int K, int plane,
-                                                               float* __restrict__ part) {
-  const int k = blockIdx.x, g = blockIdx.y, G = gridDim.y;
-  float acc = 0.0f;
-  for (int n = g; n < N; n += G) {
-    const float* p = dy + ((size_t)n * K + k) * plane;
-    for (int i = threadIdx.x; i < plane; i += 256) acc += p[i];
+// Two-stage form: stage 1 streams dy as an [N*K][plane] matrix, one wave per row, and writes the row sums
+// rowsum[n*K + k]; stage 2 (bwd_bias_rows_kernel) adds them over n in a fixed order.
+__global__ __launch_bounds__(256) void bwd_bias_rowsum_kernel(const float* __restrict__ dy, long long rows, int plane,
+                                                              float* __restrict__ rowsum) {
+  const int lane = threadIdx.x & 63;
+  const long long wave0 = (long long)blockIdx.x * 4 + (threadIdx.x >> 6), stride = (long long)gridDim.x * 4;
+  for (long long r = wave0; r < rows; r += stride) {
+    const float* p = dy + r * plane;
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+    int i = lane;
+    for (; i + 192 < plane; i += 256) {
+      a0 += p[i];
+      a1 += p[i + 64];
+      a2 += p[i + 128];
+      a3 += p[i + 192];
+    }
+    for (; i < plane; i += 64) a0 += p[i];
+    float acc = (a0 + a1) + (a2 + a3);
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
+    if (lane == 0) rowsum[r] = acc;
   }
-  for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
-  __shared__ float sm[4];
-  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = acc;
+}
+
+// Column sums of an [N][K] matrix (dy of an affine layer, or the row sums above): a block covers 64
+// columns; its 4 waves take every fourth row and are combined through LDS in a fixed order.
+__global__ __launch_bounds__(256) void bwd_bias_rows_kernel(const float* __restrict__ dy, int N, int K, float alpha,
+                                                            float beta, float* __restrict__ db) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int k = blockIdx.x * 64 + lane;
+  float a0 = 0.0f, a1 = 0.0f;
+  if (k < K) {
+    int n = wave;
+    for (; n + 4 < N; n += 8) {
+      a0 += dy[(size_t)n * K + k];
+      a1 += dy[(size_t)(n + 4) * K + k];
+    }
+    for (; n < N; n += 4) a0 += dy[(size_t)n * K + k];
+  }
+  __shared__ float sm[4][64];
+  sm[wave][lane] = a0 + a1;
   __syncthreads();
-  if (threadIdx.x == 0) part[(size_t)g * K + k] = sm[0] + sm[1] + sm[2] + sm[3];
-}
-
-__global__ void bwd_bias_finish_kernel(const float* __restrict__ part, int G, int K, float alpha, float beta,
-                                       float* __restrict__ db) {
-  const int k = blockIdx.x * blockDim.x + threadIdx.x;
-  if (k >= K) return;
-  float s = 0.0f;
-  for (int g = 0; g < G; ++g) s += part[(size_t)g * K + k];
-  float v = alpha * s;
-  if (beta != 0.0f) v += beta * db[k];
-  db[k] = v;
-}
-
-static int bwd_bias_groups(int N, int K) {
-  int G = cdiv(2048, K);
-  if (G > N) G = N;
-  if (G > 64) G = 64;
-  return G < 1 ? 1 : G;
-}
-
-// plane == 1 (affine): dy is [N][K]; one thread per k walks the batch, coalesced across k.
-__global__ void bwd_bias_rows_kernel(const float* __restrict__ dy, int N, int K, float alpha,
-                                     float beta, float* __restrict__ db) {
-  const int k = blockIdx.x * blockDim.x + threadIdx.x;
-  if (k >= K) return;
-  float acc = 0.0f;
-  for (int n = 0; n < N; ++n) acc += dy[(size_t)n * K + k];
-  float v = alpha * acc;
-  if (beta != 0.0f) v += beta * db[k];
-  db[k] = v;
+  if (wave == 0 && k < K) {
+    float v = alpha * ((sm[0][lane] + sm[1][lane]) + (sm[2][lane] + sm[3][lane]));
+    if (beta != 0.0f) v += beta * db[k];
+    db[k] = v;
+  }
 }
 
 }  // namespace rh
@@ -390,21 +391,23 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
 
 extern "C" size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane) {
   if (N <= 0 || K <= 0 || plane <= 1) return 0;
-  return align256(sizeof(float) * (size_t)bwd_bias_groups(N, K) * K);
+  return align256(sizeof(float) * (size_t)N * K);
 }
 
 extern "C" int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
-                                     float* db, void* ws, size_t ws_bytes, rh_stream_t stream_) {
+                                     float* db, void* ws, size_t ws_bytes, void* stream_) {
   if (N <= 0 || K <= 0 || plane <= 0 || !dy || !db) return RH_E_INVALID;
   const size_t need = rh_conv2d_bwd_bias_workspace_bytes(N, K, plane);
   if (plane == 1 || need == 0 || !ws || ws_bytes < need) return rh_conv2d_bwd_bias(N, K, plane, alpha, dy, beta, db, stream_);
   hipStream_t stream = to_stream(stream_);
-  const int G = bwd_bias_groups(N, K);
-  float* part = static_cast<float*>(ws);
+  float* rowsum = static_cast<float*>(ws);
+  const long long rows = (long long)N * K;
   ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
-  hipLaunchKernelGGL(bwd_bias_partial_kernel, dim3(K, G), dim3(256), 0, stream, dy, N, K, plane, part);
+  const long long blocks = cdiv<long long>(rows, 4);
+  hipLaunchKernelGGL(bwd_bias_rowsum_kernel, dim3((unsigned)(blocks > 65536 ? 65536 : blocks)), dim3(256), 0, stream, dy,
+                     rows, plane, rowsum);
   if (int e = launch_status()) return e;
-  hipLaunchKernelGGL(bwd_bias_finish_kernel, dim3(cdiv(K, 256)), dim3(256), 0, stream, part, G, K, alpha, beta, db);
+  hipLaunchKernelGGL(bwd_bias_rows_kernel, dim3(cdiv(K, 64)), dim3(256), 0, stream, rowsum, N, K, alpha, beta, db);
   return launch_status();
 }
 
@@ -414,7 +417,7 @@ extern "C" int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alp
   hipStream_t stream = to_stream(stream_);
   ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
   if (plane == 1) {
-    hipLaunchKernelGGL(bwd_bias_rows_kernel, dim3(cdiv(K, 256)), dim3(256), 0, stream, dy, N, K, alpha, beta,
+    hipLaunchKernelGGL(bwd_bias_rows_kernel, dim3(cdiv(K, 64)), dim3(256), 0, stream, dy, N, K, alpha, beta,
                        db);
   } else {
     hipLaunchKernelGGL(bwd_bias_kernel, dim3(K), dim3(1024), 0, stream, dy, N, K, plane, alpha, beta, db);
