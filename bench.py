@@ -18,6 +18,17 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
+# HBM-side bytes per launch (average over the launches of one step) of the MFMA kernels of the AlexNet
+# workload, from two hardware-counter runs of this script under `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE`; each counter scaled by what it reads for the library's plain 256 MiB copy kernel in
+# the same run (FETCH_SIZE reads 0.5 KiB per KiB copied -> x2.0, WRITE_SIZE 1.0 -> x1.0).  A counter run
+# cannot be nested inside this process, so the figures are carried here and named in `traffic_source`.
+MEASURED_TRAFFIC_BYTES = {
+    "alexnet": {"conv_bwd_filter_128x128": 1024 * (2.0 * 185562 + 66388),
+                "conv_fwd_128x128": 1024 * (2.0 * 72678 + 123152),
+                "conv_bwd_data_128x128": 1024 * (2.0 * 64209 + 70897)},
+}
+
 BATCH = {"alexnet": 256, "lenet": 64, "cifar10": 128, "nin": 128}
 NUM_CLASSES_SEED = 0x5EED0000
 
@@ -49,6 +60,32 @@ def collect_profile(lib, steps):
                     "ms_per_step": ms / steps, "avg_launch_ms": ms / count, "achieved": achieved, "peak": peak,
                     "unit": unit, "frac": achieved / peak})
     out.sort(key=lambda k: -k["ms_per_step"])
+    return out
+
+
+def calibrate(lib, torch):
+    """Sustained ceilings of this GPU, for auditing the roofline fractions: a register-only fp32 MFMA loop
+    (2 waves per SIMD) and a plain float4 copy of 1 GiB, both timed by the library's own HIP events."""
+    import ctypes as C
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sink = torch.zeros(4, dtype=torch.float32, device="cuda:0")
+    src = torch.ones(1 << 28, dtype=torch.float32, device="cuda:0")
+    dst = torch.empty_like(src)
+    out = {}
+    for rep in range(2):               # first round warms up, second is read
+        lib.rh_profile_reset()
+        lib.rh_profile_enable(1)
+        for _ in range(3):
+            lib.rh_probe_mfma_loop(512, 8, 10000, C.c_void_p(sink.data_ptr()), stream)
+            lib.rh_probe_copy(C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), src.numel(), stream)
+        torch.cuda.synchronize()
+        lib.rh_profile_enable(0)
+        recs = {k["kernel"]: k for k in collect_profile(lib, 1)}
+        out = {"mfma_fp32_loop_tflops": recs["probe_mfma_loop"]["achieved"] / 1e3,
+               "copy_1gib_gbs": recs["probe_copy"]["achieved"],
+               "device": torch.cuda.get_device_name(0),
+               "compute_units": torch.cuda.get_device_properties(0).multi_processor_count}
+    lib.rh_profile_reset()
     return out
 
 
@@ -85,8 +122,14 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="alexnet", choices=sorted(BATCH))
-    ap.add_argument("--cpu-sample", type=int, default=32, help="images in the CPU baseline step (0 = skip)")
+    ap.add_argument("--cpu-sample", type=int, default=512, help="images in the CPU baseline step (0 = skip; 512 is about 15 s on 16 cores)")
     ap.add_argument("--unfused", action="store_true", help="reference-style K1->K2->K3 and BLAS-1 SGD sequence")
+    ap.add_argument("--no-kernel-events", action="store_true",
+                    help="do not bracket each kernel with HIP events in the timed region (no per-kernel breakdown)")
+    ap.add_argument("--no-calibration", action="store_true", help="skip the MFMA-loop / copy ceiling probes")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="first launch the library's plain copy kernel 4 times over MIB MiB (a known-size "
+                         "reference for hardware byte counters collected around this command)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (pure data parallelism would all-reduce the flat gradient "
@@ -116,12 +159,45 @@ def main():
     sgd = SgdOpt(batch, 0.01, ("Update", 0.9), 0.0)
     sgd.begin(worker)
 
+    if args.calibrate_copy > 0:
+        import ctypes as C
+        n = args.calibrate_copy * (1 << 20) // 4
+        src = torch.ones(n, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            _lib.check(lib.rh_probe_copy(C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), n,
+                                         C.c_void_p(torch.cuda.current_stream().cuda_stream)), "rh_probe_copy")
+        torch.cuda.synchronize()
+        del src, dst
+
+    calibration = None if args.no_calibration else calibrate(lib, torch)
+
     for _ in range(args.warmup):
         sgd.train_batch(worker, batch, fused=not args.unfused)
     worker.sync()
     torch.cuda.synchronize()
-    lib.rh_profile_reset()
-    lib.rh_profile_enable(1)
+
+    # Untimed breakdown pass: every launch bracketed by HIP events (costs ~4 % of a step in event
+    # traffic, which is why it is kept out of the timed region).  It names the dominant kernel.
+    kernels, breakdown_steps = [], 0 if args.no_kernel_events else max(1, min(args.steps, 10))
+    if breakdown_steps:
+        lib.rh_profile_reset()
+        lib.rh_profile_filter(None)
+        lib.rh_profile_enable(1)
+        for _ in range(breakdown_steps):
+            sgd.train_batch(worker, batch, fused=not args.unfused)
+        worker.sync()
+        torch.cuda.synchronize()
+        lib.rh_profile_enable(0)
+        kernels = collect_profile(lib, breakdown_steps)
+        lib.rh_profile_reset()
+    mfma = [k for k in kernels if k["bound"] == "mfma"]
+    dom = mfma[0] if mfma else kernels[0] if kernels else None
+
+    # Timed region: exactly `steps` steps; only the dominant kernel's launches carry HIP events.
+    if dom is not None:
+        lib.rh_profile_filter(dom["kernel"].encode())
+        lib.rh_profile_enable(1)
     t0 = time.perf_counter()
     loss = 0.0
     for _ in range(args.steps):
@@ -130,11 +206,12 @@ def main():
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     lib.rh_profile_enable(0)
-    kernels = collect_profile(lib, args.steps)
+    if dom is not None:
+        live = [k for k in collect_profile(lib, args.steps) if k["kernel"] == dom["kernel"]]
+        dom = live[0] if live else dom
     lib.rh_profile_reset()
+    lib.rh_profile_filter(None)
 
-    mfma = [k for k in kernels if k["bound"] == "mfma"]
-    dom = mfma[0] if mfma else kernels[0]
     gemm_ms = sum(k["ms_per_step"] for k in mfma)
     gemm_flops = configs.train_flops(net, batch)
     result = {
@@ -154,10 +231,17 @@ def main():
                                "weights N(0,0.01), %s" % (args.workload, batch, dims[2], dims[1], dims[0],
                                                           "unfused reference sequence" if args.unfused else "fused epilogues"),
                    "global_batch": batch, "params": cfg.params_len(), "gemm_gflop_per_step": gemm_flops / 1e9},
-        "roofline": {"bound": dom["bound"], "kernel": dom["kernel"], "achieved": dom["achieved"], "peak": dom["peak"],
-                     "unit": dom["unit"], "frac": dom["frac"], "avg_launch_ms": dom["avg_launch_ms"], "traffic": None},
+        "roofline": None if dom is None else
+                    {"bound": dom["bound"], "kernel": dom["kernel"], "achieved": dom["achieved"], "peak": dom["peak"],
+                     "unit": dom["unit"], "frac": dom["frac"], "avg_launch_ms": dom["avg_launch_ms"],
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom["kernel"]),
+                     "traffic_unit": "bytes per launch (L2<->fabric, FETCH_SIZE + WRITE_SIZE counters)",
+                     "traffic_source": "rocprofv3 --pmc runs of this script; summary under profiles/"},
         "all_mfma": {"ms_per_step": gemm_ms, "achieved": gemm_flops / gemm_ms / 1e9 if gemm_ms else None,
                      "unit": "TFLOP/s", "frac": gemm_flops / gemm_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS if gemm_ms else None},
+        "calibration": calibration,
+        "kernels_note": "per-kernel table from an untimed pass of %d steps with HIP events on every launch; "
+                        "roofline.* is from events on the dominant kernel inside the timed region" % breakdown_steps,
         "kernels": kernels,
         "final_loss": loss,
     }

@@ -209,6 +209,8 @@ int rh_rng_fill_int(uint64_t seed, uint64_t stream_id, int32_t* host, size_t n, 
  * MFMA contractions, bytes for the bandwidth-bound kernels), elapsed milliseconds}.
  * ------------------------------------------------------------------------------------------- */
 int rh_profile_enable(int on);
+/* Record only launches whose tag starts with `prefix` (NULL or "" = all).  Set it while disabled. */
+int rh_profile_filter(const char* prefix);
 int rh_profile_count(void);
 int rh_profile_get(int i, const char** tag, double* work, float* ms);
 int rh_profile_reset(void);

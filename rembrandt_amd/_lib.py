@@ -69,6 +69,7 @@ PROTOTYPES = {
     "rh_sgd_momentum_step": (_int, [_i64, _vp, _vp, _vp, _f, _f, _f, _f, _int, _vp]),
     "rh_descend": (_int, [_i64, _vp, _vp, _f, _f, _vp]),
     "rh_profile_enable": (_int, [_int]),
+    "rh_profile_filter": (_int, [C.c_char_p]),
     "rh_profile_count": (_int, []),
     "rh_profile_get": (_int, [_int, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(_f)]),
     "rh_profile_reset": (_int, []),

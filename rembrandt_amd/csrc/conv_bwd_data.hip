@@ -47,7 +47,7 @@ static int run_bwd_data_soff(const RowSParams& ap, const RowSParams& bp, const E
   constexpr int AROWS = T::BM % 64 == 0 ? T::BM : (T::BM + 63) / 64 * 64;
   typedef LoadRowS<AROWS, T::BK, T::NT, true> AL;
   typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
-  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
+  return launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
 }
 
 template <class T>
@@ -55,7 +55,7 @@ static int run_bwd_data(int KRS, const DenseParams& ap, const GatherParams& bp, 
                         hipStream_t stream, const char* tag) {
   typedef LoadDenseK<T::BM, T::BK, T::NT, true> AL;
   typedef LoadGatherR<T::BN, T::BK, T::NT, true> BL;
-  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, KRS, 1, nullptr, stream, tag);
+  return launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, KRS, 1, nullptr, stream, tag);
 }
 
 }  // namespace rh

@@ -187,7 +187,7 @@ static int run_bwd_filter_soff(const RowSParams& ap, const RowSParams& bp, const
   constexpr int AROWS = T::BM % 64 == 0 ? T::BM : (T::BM + 63) / 64 * 64;
   typedef LoadRowS<AROWS, T::BK, T::NT, true> AL;
   typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
-  return launch_mfma_gemm<T, AL, BL, false>(ap, bp, ep, n_k, splits, used, stream, tag, k_true);
+  return launch_mfma_gemm<T, AL, BL, false, PassConvBwdFilter>(ap, bp, ep, n_k, splits, used, stream, tag, k_true);
 }
 
 template <class T>
@@ -195,7 +195,7 @@ static int run_bwd_filter(const PixDyParams& ap, const PixXParams& bp, const Epi
                           int splits, int* used, hipStream_t stream, const char* tag) {
   typedef LoadPixDy<T::BM, T::BK, T::NT> AL;
   typedef LoadPixX<T::BN, T::BK, T::NT> BL;
-  return launch_mfma_gemm<T, AL, BL, false>(ap, bp, ep, M, splits, used, stream, tag);
+  return launch_mfma_gemm<T, AL, BL, false, PassConvBwdFilter>(ap, bp, ep, M, splits, used, stream, tag);
 }
 
 // db[k] = alpha * sum_{n, i<plane} dy[(n*K + k)*plane + i] + beta * db[k].  grid = (K, 1): the 16 waves of

@@ -53,7 +53,7 @@ inline int pick_bm(int rows) {
   return best;
 }
 
-template <class T, class AL, class BL, bool NCHW>
+template <class T, class AL, class BL, bool NCHW, class PASS>
 inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Params& bp,
                             const EpiParams& ep, int K, int splits, int* splits_used,
                             hipStream_t stream, const char* tag, int k_algorithmic = 0) {
@@ -69,12 +69,12 @@ inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Pa
   if (lds_bytes > 48 * 1024) {
     // opt in to more than the default dynamic LDS limit, once per kernel instantiation
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&mfma_gemm_kernel<T, AL, BL, NCHW>),
+        reinterpret_cast<const void*>(&mfma_gemm_kernel<T, AL, BL, NCHW, PASS>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr != hipSuccess) return (int)attr;
   }
   ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)(k_algorithmic > 0 ? k_algorithmic : K), stream);
-  hipLaunchKernelGGL((mfma_gemm_kernel<T, AL, BL, NCHW>), grid, dim3(T::NT), lds_bytes, stream, ap, bp, ep,
+  hipLaunchKernelGGL((mfma_gemm_kernel<T, AL, BL, NCHW, PASS>), grid, dim3(T::NT), lds_bytes, stream, ap, bp, ep,
                      tiles_m, k_chunks, cps);
   return launch_status();
 }

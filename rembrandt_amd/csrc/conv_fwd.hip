@@ -71,7 +71,7 @@ static int run_fwd_soff(const RowSParams& ap, const RowSParams& bp, const EpiPar
   constexpr int AROWS = T::BM % 64 == 0 ? T::BM : (T::BM + 63) / 64 * 64;  // loader rows: a multiple of the wave
   typedef LoadRowS<AROWS, T::BK, T::NT, true> AL;
   typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
-  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
+  return launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
 }
 
 template <class T>
@@ -79,7 +79,7 @@ static int run_fwd(const ConvDims& d, const DenseParams& ap, const GatherParams&
                    const EpiParams& ep, hipStream_t stream, const char* tag) {
   typedef LoadDenseK<T::BM, T::BK, T::NT, false> AL;
   typedef LoadGatherR<T::BN, T::BK, T::NT, false> BL;
-  return launch_mfma_gemm<T, AL, BL, true>(ap, bp, ep, d.C * d.R * d.S, 1, nullptr, stream, tag);
+  return launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, d.C * d.R * d.S, 1, nullptr, stream, tag);
 }
 
 }  // namespace rh

@@ -5,6 +5,8 @@
 #include <algorithm>
 #include <mutex>
 #include <thread>
+#include <string>
+#include <cstring>
 #include <vector>
 
 #include "common.h"
@@ -118,10 +120,12 @@ namespace {
 struct ProfRecord { const char* tag; double work; hipEvent_t e0, e1; };
 std::vector<ProfRecord*> g_records;
 std::mutex g_prof_mutex;
+std::string g_prof_prefix;   // when non-empty only tags that start with it are recorded
 }  // namespace
 
 ProfScope::ProfScope(const char* tag, double work, hipStream_t s) : slot(nullptr), stream(s) {
   if (!g_profile_enabled) return;
+  if (!g_prof_prefix.empty() && std::strncmp(tag, g_prof_prefix.c_str(), g_prof_prefix.size()) != 0) return;
   ProfRecord* r = new ProfRecord{tag, work, nullptr, nullptr};
   if (hipEventCreate(&r->e0) != hipSuccess || hipEventCreate(&r->e1) != hipSuccess) { delete r; return; }
   (void)hipEventRecord(r->e0, s);
@@ -140,6 +144,12 @@ ProfScope::~ProfScope() {
 
 extern "C" int rh_profile_enable(int on) {
   rh::g_profile_enabled = on != 0;
+  return 0;
+}
+
+extern "C" int rh_profile_filter(const char* prefix) {
+  std::lock_guard<std::mutex> lock(rh::g_prof_mutex);
+  rh::g_prof_prefix = prefix ? prefix : "";
   return 0;
 }
 

@@ -403,7 +403,7 @@ struct LoadPixX {
 //   NCHW : out[((j / inner) * rows + i) * inner + j % inner]    (j = pixel, i = channel)
 //   dense: out[i * ld + j]
 // value = alpha*acc + beta*old (+ bias[i]) (clamped at 0 if relu).  With split_stride != 0 the
-// block writes its partial sum, unblended, to out + blockIdx.y * split_stride (dense).
+// block writes its partial sum, unblended, to out + split * split_stride (dense).
 // ------------------------------------------------------------------------------------------
 struct EpiParams {
   float* out;
@@ -424,7 +424,14 @@ __device__ __forceinline__ int xcd_remap(int b, int nb) {
   return start + idx;
 }
 
-template <class T, class AL, class BL, bool NCHW>
+// Pass tags: they only make the instantiations of one pass distinct kernels (and kernel names) from
+// those of another pass that uses the same tile and loaders.
+struct PassConvFwd {};
+struct PassConvBwdData {};
+struct PassConvBwdFilter {};
+struct PassSgemm {};
+
+template <class T, class AL, class BL, bool NCHW, class PASS>
 __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::Params ap,
                                                           typename BL::Params bp, EpiParams ep,
                                                           int tiles_m, int k_chunks,
@@ -441,11 +448,16 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % T::WM, wn = wave / T::WM;
 
-  const int logical = xcd_remap(blockIdx.x, gridDim.x);
+  // Blocks of the whole grid (tiles x splits, x fastest) are dealt to the 8 XCDs round-robin; remap so that
+  // each XCD's L2 sees a contiguous range of (split, tile): all tiles of a split read the same K range.
+  const int tiles = gridDim.x;
+  const int linear = xcd_remap(blockIdx.y * tiles + blockIdx.x, tiles * gridDim.y);
+  const int split_idx = __builtin_amdgcn_readfirstlane(linear / tiles);
+  const int logical = __builtin_amdgcn_readfirstlane(linear - split_idx * tiles);
   const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  const int c_begin = blockIdx.y * chunks_per_split;
+  const int c_begin = split_idx * chunks_per_split;
   int c_end = c_begin + chunks_per_split;
   if (c_end > k_chunks) c_end = k_chunks;
   const int nk = c_end - c_begin;
@@ -596,7 +608,7 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
   if (RH_EXP_NOSTORE == 2 && exp_sink == 123.25f) ep.out[0] = exp_sink;
   // ---- epilogue
   const bool split = ep.split_stride != 0;
-  float* out = ep.out + (split ? (long long)blockIdx.y * ep.split_stride : 0ll);
+  float* out = ep.out + (split ? (long long)split_idx * ep.split_stride : 0ll);
   const float alpha = split ? 1.0f : ep.alpha;
   const float beta = split ? 0.0f : ep.beta;
   const int row_stride = NCHW ? ep.inner : ep.ld;

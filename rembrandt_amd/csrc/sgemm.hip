@@ -35,16 +35,16 @@ static int run_sgemm(const DenseParams& ap, const DenseParams& bp, const EpiPara
                      int* used, hipStream_t stream, const char* tag) {
   // engine A operand = opB: k contiguous unless transB; engine B operand = opA: rows contiguous unless transA
   if constexpr (!B_TRANS && !A_TRANS)
-    return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseR<T::BN, T::BK, T::NT>, false>(
+    return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseR<T::BN, T::BK, T::NT>, false, PassSgemm>(
         ap, bp, ep, k, splits, used, stream, tag);
   else if constexpr (!B_TRANS && A_TRANS)
-    return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseK<T::BN, T::BK, T::NT, false>, false>(
+    return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseK<T::BN, T::BK, T::NT, false>, false, PassSgemm>(
         ap, bp, ep, k, splits, used, stream, tag);
   else if constexpr (B_TRANS && !A_TRANS)
-    return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseR<T::BN, T::BK, T::NT>, false>(
+    return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseR<T::BN, T::BK, T::NT>, false, PassSgemm>(
         ap, bp, ep, k, splits, used, stream, tag);
   else
-    return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseK<T::BN, T::BK, T::NT, false>, false>(
+    return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseK<T::BN, T::BK, T::NT, false>, false, PassSgemm>(
         ap, bp, ep, k, splits, used, stream, tag);
 }
 
