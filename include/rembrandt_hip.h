@@ -44,6 +44,10 @@ typedef void* rh_stream_t; /* hipStream_t */
 #define RH_MATH_BF16_MFMA_FP32ACC  0x1  /* operands rounded to bf16 (RNE) on load, bf16 MFMA, fp32 accumulate */
 #define RH_FUSE_BIAS               0x10 /* conv fwd: add bias[k] in the epilogue (replaces the separate K2 pass) */
 #define RH_FUSE_RELU               0x20 /* conv fwd: max(.,0) in the epilogue (replaces the separate K3 pass)    */
+/* loader family of the conv passes; neither bit = the library chooses (what the operators use) */
+#define RH_ALGO_GATHER             0x100 /* k -> {offset, dr, ds} table gather straight from the NCHW tensors      */
+#define RH_ALGO_SCALAR_OFFSET      0x200 /* scalar-offset loads on padded / transposed copies in the workspace,
+                                            wherever the geometry allows it (else the gather family)             */
 
 const char* rh_version(void);
 /* Status of the most recent launch made by a void `rembrandt_kernel_*` entry point on this thread. */

@@ -75,7 +75,7 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
 
   const int KRS = d.K * d.R * d.S;
   const SoffPlan sp = plan_soff_bwd_data(d);
-  if (sp.ok && !legacy_gather()) {
+  if (sp.ok && !(flags & RH_ALGO_GATHER)) {
     int* soff = static_cast<int*>(ws);
     float* wT = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes);
     const float* img = dy;

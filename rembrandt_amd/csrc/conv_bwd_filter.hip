@@ -70,8 +70,6 @@ void launch_split_reduce(const float* part, int splits, long long split_stride, 
 // The result comes out as dw'[ko][(r,s,c)]; the reduction kernel puts it back in [ko][c][r][s] order.
 // The channel-last path pays two transposes; it wins when the contraction is deep relative to them.
 static bool use_soff_bwd_filter(const ConvDims& d) {
-  static const int force = [] { const char* e = getenv("RH_BWDF_SOFF"); return e ? atoi(e) : -1; }();
-  if (force >= 0) return force != 0;
   // FLOPs of the contraction per byte the two transposes move (measured: conv1-like 119 and 1x1 24 lose,
   // 3x3 / 5x5 layers at 690-875 win)
   const double flops = 2.0 * d.K * d.C * d.R * d.S * (double)d.N * d.P * d.Q;
@@ -315,7 +313,7 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
   hipStream_t stream = to_stream(stream_);
 
   const BwdFilterSoffPlan sp = plan_bwd_filter_soff(d);
-  if (sp.ok && !legacy_gather() && use_soff_bwd_filter(d)) {
+  if (sp.ok && !(flags & RH_ALGO_GATHER) && ((flags & RH_ALGO_SCALAR_OFFSET) || use_soff_bwd_filter(d))) {
     const int CRSs = d.C * d.R * d.S, Ms = d.N * d.P * d.Q;
     char* base = static_cast<char*>(ws);
     int* soff = reinterpret_cast<int*>(base);

@@ -87,23 +87,6 @@ typedef Tile<128, 128, 16, 2, 2, RH_OCC_128> T128x128;
 typedef Tile<96, 256, 16, 1, 4> T96x256;
 typedef Tile<64, 256, 16, 1, 4> T64x256;
 typedef Tile<32, 256, 16, 1, 4> T32x256;
-// experimental shapes, selected with the RH_CONV_TILE environment variable
-typedef Tile<128, 256, 16, 2, 2> T128x256;
-typedef Tile<256, 128, 16, 2, 2> T256x128;
-typedef Tile<128, 128, 32, 2, 2> T128x128k32;
-typedef Tile<128, 256, 32, 2, 2> T128x256k32;
-typedef Tile<256, 256, 16, 2, 4> T256x256w8;
-
-// RH_LEGACY_GATHER=1 forces the per-element gather loaders (kept for strided backward-data and as a cross-check).
-inline bool legacy_gather() {
-  static const bool v = [] { const char* e = getenv("RH_LEGACY_GATHER"); return e && atoi(e) != 0; }();
-  return v;
-}
-
-inline int tile_override() {
-  static const int v = [] { const char* e = getenv("RH_CONV_TILE"); return e ? atoi(e) : 0; }();
-  return v;
-}
 
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,

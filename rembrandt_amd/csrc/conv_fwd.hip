@@ -106,7 +106,7 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
 
   const int CRS = d.C * d.R * d.S;
   const SoffPlan sp = plan_soff_fwd(d);
-  if (sp.ok && !legacy_gather()) {
+  if (sp.ok && !(flags & RH_ALGO_GATHER)) {
     int* soff = static_cast<int*>(ws);
     float* wT = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes);
     const float* img = x;
@@ -156,14 +156,6 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
   ep.rows = d.K; ep.cols = bp.M; ep.inner = d.P * d.Q; ep.ld = 0; ep.relu = (flags & RH_FUSE_RELU) ? 1 : 0;
   ep.split_stride = 0;
 
-  switch (tile_override()) {
-    case 1: return run_fwd<T128x256>(d, ap, bp, ep, stream, "conv_fwd_128x256");
-    case 2: return run_fwd<T256x128>(d, ap, bp, ep, stream, "conv_fwd_256x128");
-    case 3: return run_fwd<T128x128k32>(d, ap, bp, ep, stream, "conv_fwd_128x128k32");
-    case 4: return run_fwd<T128x256k32>(d, ap, bp, ep, stream, "conv_fwd_128x256k32");
-    case 5: return run_fwd<T256x256w8>(d, ap, bp, ep, stream, "conv_fwd_256x256w8");
-    default: break;
-  }
   switch (pick_bm(d.K)) {
     case 128: return run_fwd<T128x128>(d, ap, bp, ep, stream, "conv_fwd_128x128");
     case 96:  return run_fwd<T96x256>(d, ap, bp, ep, stream, "conv_fwd_96x256");

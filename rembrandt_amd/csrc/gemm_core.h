@@ -499,45 +499,15 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
   // global loads sit in the first half of the step, giving them the second half (and the other
   // waves' turns) to land before they are written to the other LDS buffer.
   constexpr int STEPS = BK / 2;
-#ifndef RH_LSTEPS_DIV
-#define RH_LSTEPS_DIV 2
-#endif
-  constexpr int LSTEPS = STEPS / RH_LSTEPS_DIV > 0 ? STEPS / RH_LSTEPS_DIV : 1;
+  constexpr int LSTEPS = STEPS / 2 > 0 ? STEPS / 2 : 1;  // groups that carry global loads
   constexpr int A_PER = (AL::CNT + LSTEPS - 1) / LSTEPS, B_PER = (BL::CNT + LSTEPS - 1) / LSTEPS;
-#ifndef RH_PREP_AHEAD
-#define RH_PREP_AHEAD 1
-#endif
-// timing experiments only (results are wrong when set)
-#ifndef RH_EXP_NOLOAD
-#define RH_EXP_NOLOAD 0
-#endif
-#ifndef RH_EXP_NOSTORE
-#define RH_EXP_NOSTORE 0
-#endif
-#ifndef RH_EXP_NOBARRIER
-#define RH_EXP_NOBARRIER 0
-#endif
-#ifndef RH_FINE_INTERLEAVE
-#define RH_FINE_INTERLEAVE 0
-#endif
-#ifndef RH_VALU_PER_MFMA
-#define RH_VALU_PER_MFMA 10
-#endif
-#ifndef RH_SETPRIO
-#define RH_SETPRIO 0
-#endif
-  if (RH_PREP_AHEAD && nk > 1) {
+  if (nk > 1) {
     la.prep((c_begin + 1) * BK);
     lb.prep((c_begin + 1) * BK);
   }
-  float exp_sink = 0.0f;
   auto k_step = [&](int it, auto more_tag) {
     constexpr bool MORE = decltype(more_tag)::value;
     const int cur = it & 1;
-    if (!RH_PREP_AHEAD && MORE) {
-      la.prep((c_begin + it + 1) * BK);
-      lb.prep((c_begin + it + 1) * BK);
-    }
     const float* pa = sA_base + cur * (BK * LDA) + a_rd;
     const float* pb = sB_base + cur * (BK * LDB) + b_rd;
     float a[2][TM], b[2][TN];
@@ -555,7 +525,7 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
 #pragma unroll
         for (int j = 0; j < TN; ++j) b[n][j] = pb[(2 * g + 2) * LDB + j * 32];
       }
-      if (MORE && g < LSTEPS && !RH_EXP_NOLOAD) {
+      if (MORE && g < LSTEPS) {
 #pragma unroll
         for (int e = g * A_PER; e < (g + 1) * A_PER; ++e)
           if (e < AL::CNT) ra[e] = la.load_one(e);
@@ -563,13 +533,13 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
         for (int e = g * B_PER; e < (g + 1) * B_PER; ++e)
           if (e < BL::CNT) rb[e] = lb.load_one(e);
       }
-      if (!RH_FINE_INTERLEAVE) __builtin_amdgcn_sched_barrier(0);  // loads and reads issue before this group's MFMAs
+      __builtin_amdgcn_sched_barrier(0);  // loads and reads issue before this group's MFMAs
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c][i], b[c][j], acc[i][j], 0, 0, 0);
-      if (RH_PREP_AHEAD && MORE && g == (LSTEPS < STEPS ? LSTEPS : STEPS - 1)) {
+      if (MORE && g == (LSTEPS < STEPS ? LSTEPS : STEPS - 1)) {
         // the table entries / pixel decomposition of the step after next: all loads of the next
         // step have been issued by now, and this leaves a whole half step for the scalar loads
         if (it + 2 < nk) {
@@ -577,35 +547,17 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
           lb.prep((c_begin + it + 2) * BK);
         }
       }
-      if (RH_FINE_INTERLEAVE) {
-        // Alternative issue order (measured slightly slower with three waves per SIMD): every MFMA
-        // followed by a share of the loader's address arithmetic and a global load.
-        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
-#pragma unroll
-        for (int m = 0; m < TM * TN; ++m) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, RH_VALU_PER_MFMA, 0);
-          __builtin_amdgcn_sched_group_barrier(0x020, (A_PER + B_PER + TM * TN - 1) / (TM * TN), 0);
-        }
-      }
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (MORE && !RH_EXP_NOSTORE) {
+    if (MORE) {
       la.store(sA_base + (cur ^ 1) * (BK * LDA), ra);
       lb.store(sB_base + (cur ^ 1) * (BK * LDB), rb);
     }
-    if (MORE && RH_EXP_NOSTORE == 2) {  // keep the loads alive without LDS traffic
-#pragma unroll
-      for (int i = 0; i < AL::CNT; ++i) exp_sink += ra[i];
-#pragma unroll
-      for (int i = 0; i < BL::CNT; ++i) exp_sink += rb[i];
-    }
-    if (!RH_EXP_NOBARRIER) __syncthreads();
+    __syncthreads();
   };
   for (int it = 0; it + 1 < nk; ++it) k_step(it, std::true_type());
   if (nk > 0) k_step(nk - 1, std::false_type());
 
-  if (RH_EXP_NOSTORE == 2 && exp_sink == 123.25f) ep.out[0] = exp_sink;
   // ---- epilogue
   const bool split = ep.split_stride != 0;
   float* out = ep.out + (split ? (long long)split_idx * ep.split_stride : 0ll);

@@ -48,25 +48,25 @@ def conv_out_shape(g):
     return (g.N, g.K, out(g.H, g.R, g.stride, g.pad), out(g.W, g.S, g.stride, g.pad))
 
 
-def conv2d_fwd(x, w, stride, pad, bias=None, relu=False, alpha=1.0, beta=0.0, y=None):
+def conv2d_fwd(x, w, stride, pad, bias=None, relu=False, alpha=1.0, beta=0.0, y=None, algo=0):
     g = conv_geom(x.shape, w.shape, stride, pad)
     if y is None:
         y = torch.empty(conv_out_shape(g), dtype=torch.float32, device=x.device)
     need = lib().rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_FWD)
     ws = workspace(need, x.device)
-    flags = (_lib.RH_FUSE_BIAS if bias is not None else 0) | (_lib.RH_FUSE_RELU if relu else 0)
+    flags = (_lib.RH_FUSE_BIAS if bias is not None else 0) | (_lib.RH_FUSE_RELU if relu else 0) | algo
     check(lib().rh_conv2d_fwd(C.byref(g), alpha, _p(x), _p(w), beta, _p(y), _p(bias), _p(ws), ws.numel(), flags,
                               _stream()), "rh_conv2d_fwd")
     return y
 
 
-def conv2d_bwd_filter(x, dy, w_shape, stride, pad, alpha=1.0, beta=0.0, dw=None):
+def conv2d_bwd_filter(x, dy, w_shape, stride, pad, alpha=1.0, beta=0.0, dw=None, algo=0):
     g = conv_geom(x.shape, w_shape, stride, pad)
     if dw is None:
         dw = torch.zeros(tuple(w_shape), dtype=torch.float32, device=x.device)
     need = lib().rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_BWD_FILTER)
     ws = workspace(need, x.device)
-    check(lib().rh_conv2d_bwd_filter(C.byref(g), alpha, _p(x), _p(dy), beta, _p(dw), _p(ws), ws.numel(), 0,
+    check(lib().rh_conv2d_bwd_filter(C.byref(g), alpha, _p(x), _p(dy), beta, _p(dw), _p(ws), ws.numel(), algo,
                                      _stream()), "rh_conv2d_bwd_filter")
     return dw
 
@@ -85,13 +85,13 @@ def conv2d_bwd_bias(dy, alpha=1.0, beta=0.0, db=None, two_stage=False):
     return db
 
 
-def conv2d_bwd_data(w, dy, x_shape, stride, pad, alpha=1.0, beta=0.0, dx=None):
+def conv2d_bwd_data(w, dy, x_shape, stride, pad, alpha=1.0, beta=0.0, dx=None, algo=0):
     g = conv_geom(x_shape, w.shape, stride, pad)
     if dx is None:
         dx = torch.zeros(tuple(x_shape), dtype=torch.float32, device=w.device)
     need = lib().rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_BWD_DATA)
     ws = workspace(need, w.device)
-    check(lib().rh_conv2d_bwd_data(C.byref(g), alpha, _p(w), _p(dy), beta, _p(dx), _p(ws), ws.numel(), 0,
+    check(lib().rh_conv2d_bwd_data(C.byref(g), alpha, _p(w), _p(dy), beta, _p(dx), _p(ws), ws.numel(), algo,
                                    _stream()), "rh_conv2d_bwd_data")
     return dx
 

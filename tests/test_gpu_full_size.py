@@ -1,0 +1,167 @@
+"""GPU parity at the full sizes of the benchmark configurations, where the CPU oracle cannot recompute
+whole tensors in seconds.  Each kernel is checked through the C ABI by
+  * the oracle on a random sample of output elements (plus the first and last element),
+  * size-independent properties: the adjoint identities <conv(x,w),dy> = <x,bwd_data(w,dy)> = <w,bwd_filter(x,dy)>,
+    exact linearity under a power-of-two scale, bit-identical results of repeated launches (the split
+    reductions add in a fixed order), sum(dx) = sum(dy) and arg-max-in-window for pooling,
+  * the oracle on whole slices where the operator is independent per plane (pooling) or cheap (SGD, affine).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from rembrandt_amd import _lib, ops, synth
+from conftest import assert_close, say
+
+pytestmark = pytest.mark.gpu
+
+
+def T(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def dot64(a, b):
+    return float((a.double() * b.double()).sum().item())
+
+
+def sample_idx(rng, total, n):
+    idx = rng.integers(0, total, n).astype(np.int64)
+    idx[0], idx[-1] = 0, total - 1
+    return idx
+
+
+FULL_CONV = {
+    # name: N, C, H, W, K, R, stride, pad
+    "sweep_a_alexnet_conv2": (256, 96, 27, 27, 256, 5, 1, 2),
+    "sweep_b_alexnet_conv3": (256, 256, 13, 13, 384, 3, 1, 1),
+    "sweep_c_1x1": (128, 96, 55, 55, 96, 1, 1, 0),
+    "alexnet_conv1": (256, 3, 227, 227, 96, 11, 4, 0),
+    "alexnet_conv5": (256, 384, 13, 13, 256, 3, 1, 1),
+}
+
+
+@pytest.mark.parametrize("name", sorted(FULL_CONV))
+def test_conv2d_full_size(dev, name):
+    Nn, C, H, W, K, R, st, pad = FULL_CONV[name]
+    say("full-size conv", name)
+    rng = np.random.default_rng(5)
+    x = synth.normal(21, 1, (Nn, C, H, W))
+    w = synth.normal(21, 2, (K, C, R, R))
+    xd, wd = T(x, dev), T(w, dev)
+    y = ops.conv2d_fwd(xd, wd, st, pad)
+    dy = synth.normal(21, 3, tuple(y.shape))
+    dyd = T(dy, dev)
+    dw = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad)
+    dx = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad)
+
+    # sampled oracle
+    i_y = sample_idx(rng, y.numel(), 4096)
+    assert_close(y.flatten()[T(i_y, dev)].cpu().numpy(), O.conv2d_fwd_at(x, w, st, pad, i_y), name + " fwd (sampled)")
+    i_w = sample_idx(rng, dw.numel(), 1024)
+    assert_close(dw.flatten()[T(i_w, dev)].cpu().numpy(), O.conv2d_bwd_filter_at(x, dy, w.shape, st, pad, i_w),
+                 name + " bwd filter (sampled)")
+    i_x = sample_idx(rng, dx.numel(), 4096)
+    assert_close(dx.flatten()[T(i_x, dev)].cpu().numpy(), O.conv2d_bwd_data_at(w, dy, x.shape, st, pad, i_x),
+                 name + " bwd data (sampled)")
+
+    # adjoint identities over the whole tensors (fp64 sums); scale = size of such a sum for unrelated vectors
+    a = dot64(y, dyd)
+    scale = float(y.double().norm().item() * dyd.double().norm().item()) / np.sqrt(y.numel())
+    assert abs(a - dot64(xd, dx)) <= 1e-4 * scale, (name, "bwd data adjoint", a, dot64(xd, dx), scale)
+    assert abs(a - dot64(wd, dw)) <= 1e-4 * scale, (name, "bwd filter adjoint", a, dot64(wd, dw), scale)
+
+    # exact linearity (scaling by 2 is exact in fp32) and run-to-run bit identity
+    assert torch.equal(ops.conv2d_fwd(xd, wd * 2.0, st, pad), y * 2.0), name + " fwd linearity"
+    assert torch.equal(ops.conv2d_bwd_filter(xd, dyd * 2.0, w.shape, st, pad), dw * 2.0), name + " bwd filter linearity"
+    assert torch.equal(ops.conv2d_bwd_data(wd * 2.0, dyd, x.shape, st, pad), dx * 2.0), name + " bwd data linearity"
+    assert torch.equal(ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad), dw), name + " bwd filter repeatable"
+
+    # fused epilogue and the bias gradient at this size
+    b = synth.normal(21, 4, (K,))
+    yf = ops.conv2d_fwd(xd, wd, st, pad, bias=T(b, dev), relu=True)
+    assert torch.equal(yf, torch.relu(y + T(b, dev).view(1, K, 1, 1))), name + " fused bias+relu"
+    db = ops.conv2d_bwd_bias(dyd, two_stage=True)
+    assert_close(db.cpu().numpy(), dy.sum(axis=(0, 2, 3), dtype=np.float64).astype(np.float32), name + " bias gradient")
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("shape", [(256, 96, 55, 55), (256, 256, 27, 27), (256, 256, 13, 13)],
+                         ids=["alexnet_pool1", "alexnet_pool2", "alexnet_pool5"])
+@pytest.mark.parametrize("mode", [_lib.RH_POOL_MAX, _lib.RH_POOL_AVG_INCL_PAD], ids=["max", "avg"])
+def test_pool2d_full_size(dev, shape, mode):
+    say("full-size pool", shape, mode)
+    Nn, C, H, W = shape
+    k, st, pad = 3, 2, 0
+    rng = np.random.default_rng(6)
+    x = synth.normal(22, 1, shape)
+    xd = T(x, dev)
+    if mode == _lib.RH_POOL_MAX:
+        y, am = ops.pool2d_fwd(xd, k, st, pad, mode, want_argmax=True)
+    else:
+        y, am = ops.pool2d_fwd(xd, k, st, pad, mode), None
+    dy = synth.normal(22, 2, tuple(y.shape))
+    dyd = T(dy, dev)
+    dx = ops.pool2d_bwd(xd, y, dyd, k, st, pad, mode, argmax=am)
+    dx_rescan = ops.pool2d_bwd(xd, y, dyd, k, st, pad, mode) if am is not None else dx
+    # whole planes against the oracle: pooling is independent per (n, c) plane
+    planes = sample_idx(rng, Nn * C, 48)
+    xs = x.reshape(Nn * C, 1, H, W)[planes]
+    ys, ams = O.pool2d_fwd(xs, k, st, pad, mode, want_argmax=True)
+    P, Q = y.shape[2], y.shape[3]
+    got_y = y.reshape(Nn * C, 1, P, Q)[T(planes, dev)].cpu().numpy()
+    if mode == _lib.RH_POOL_MAX:
+        assert np.array_equal(got_y, ys), "max pooling is exact"
+        assert np.array_equal(am.reshape(Nn * C, 1, P, Q)[T(planes, dev)].cpu().numpy(), ams)
+    else:
+        assert_close(got_y, ys, "avg pool fwd")
+    dys = dy.reshape(Nn * C, 1, P, Q)[planes]
+    dxs = O.pool2d_bwd(xs, ys, dys, k, st, pad, mode)
+    assert_close(dx.reshape(Nn * C, 1, H, W)[T(planes, dev)].cpu().numpy(), dxs, "pool bwd")
+    assert torch.equal(dx, dx_rescan), "mask-driven and window-rescan backward agree"
+    # conservation: every dy lands on exactly one x (max) / is spread with weights summing to 1 (avg, all windows inside)
+    tot_dy, tot_dx = float(dyd.double().sum().item()), float(dx.double().sum().item())
+    assert abs(tot_dy - tot_dx) <= 1e-5 * float(dyd.double().abs().sum().item())
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("case", [(1, 0, 4096, 256, 9216), (0, 1, 9216, 4096, 256), (0, 0, 9216, 256, 4096),
+                                  (1, 0, 1000, 256, 4096)],
+                         ids=["fc6_fwd", "fc6_bwd_w", "fc6_bwd_x", "fc8_fwd"])
+def test_sgemm_full_size(dev, case):
+    """The AlexNet affine GEMMs (column-major, as the operator issues them) against numpy fp64."""
+    ta, tb, m, n, k = case
+    say("full-size sgemm", case)
+    A = synth.normal(23, 1, (m, k) if ta else (k, m))      # column-major lda x cols stored as rows of a C array
+    B = synth.normal(23, 2, (k, n) if tb else (n, k))
+    C0 = synth.normal(23, 3, (n, m))
+    opA = A.astype(np.float64) if ta else A.astype(np.float64).T          # m x k
+    opB = B.astype(np.float64).T if tb else B.astype(np.float64)          # n x k (rows = columns of op(B))
+    ref = (opB @ opA.T) + C0.astype(np.float64)                           # stored [n][m] = column-major m x n
+    Cd = T(C0, dev)
+    ops.sgemm(ta, tb, m, n, k, 1.0, T(A, dev), A.shape[1], T(B, dev), B.shape[1], 1.0, Cd, m)
+    assert_close(Cd.cpu().numpy(), ref.astype(np.float32), "sgemm %s" % (case,))
+    torch.cuda.synchronize()
+
+
+def test_sgd_and_relu_full_size(dev):
+    """Fused SGD step on AlexNet's 62 378 344 parameters, ReLU forward/backward on conv1's 74 M activations."""
+    say("full-size sgd")
+    n = 62378344
+    W, g, v = synth.normal(24, 1, (n,)), synth.normal(24, 2, (n,)), synth.normal(24, 3, (n,))
+    Wd, gd, vd = T(W, dev), T(g, dev), T(v, dev)
+    ops.sgd_momentum_step(Wd, gd, vd, 5e-4, -0.01, 0.9, 1.0, zero_grad=True)
+    O.sgd_momentum_step(W, g, v, 5e-4, -0.01, 0.9, 1.0, True)
+    assert_close(Wd.cpu().numpy(), W, "sgd W")
+    assert_close(vd.cpu().numpy(), v, "sgd v")
+    assert not gd.any().item()
+    del Wd, gd, vd
+    say("full-size relu")
+    y = synth.normal(24, 4, (256, 96 * 55 * 55))
+    dy = synth.normal(24, 5, y.shape)
+    yd, dyd = T(y, dev), T(dy, dev)
+    ops.rect_inplace(yd)
+    assert torch.equal(yd, torch.relu(T(y, dev)))
+    ops.rect_backprop_inplace(yd, dyd)
+    assert torch.equal(dyd, T(dy, dev) * (yd > 0))
+    torch.cuda.synchronize()

@@ -127,6 +127,22 @@ def test_cifar_train_steps(dev):
     w.close()
 
 
+def test_alexnet_train_step(dev):
+    """BASELINE config 4 geometry (AlexNet-shaped: 11x11 stride-4 conv on 227x227, three 3x3/2 max-pools,
+    4096-wide affine layers, 1000 classes) at batch 4: one whole step, checkpoint by checkpoint."""
+    net, batch = configs.alexnet(), 4
+    w, ref = make_pair(net, batch, 0x5EED0004, True)
+    sgd = SgdOpt(batch, 0.01, ("Update", 0.9), 0.0)
+    rsgd = OG.SgdOpt(0.01, ("Update", 0.9), 0.0)
+    sgd.begin(w)
+    rsgd.begin(ref)
+    say("alexnet step")
+    x = synth.normal(0x5EED0004, 100, (batch, 3, 227, 227))
+    labels = synth.integers(0x5EED0004, 200, (batch,), 1000)
+    check_step(w, ref, sgd, rsgd, x, labels, batch, True, "alexnet step 0")
+    w.close()
+
+
 @pytest.mark.parametrize("flavour", ["Zero", "Update", "UpdateNesterov", "Gradient", "GradientNesterov"])
 def test_momentum_flavours(dev, flavour):
     """All five Momentum flavours on a small conv net (3 steps each, unfused BLAS-1 sequence and, where it

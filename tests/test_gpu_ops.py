@@ -33,10 +33,15 @@ CONV_CASES = [
 ]
 
 
+ALGOS = {"auto": 0, "gather": _lib.RH_ALGO_GATHER, "scalar_offset": _lib.RH_ALGO_SCALAR_OFFSET}
+
+
+@pytest.mark.parametrize("algo", sorted(ALGOS))
 @pytest.mark.parametrize("case", CONV_CASES, ids=[str(c) for c in CONV_CASES])
-def test_conv2d_all_passes(dev, case):
+def test_conv2d_all_passes(dev, case, algo):
     Nn, C, H, W, K, R, st, pad = case
-    say("conv case", case)
+    say("conv case", case, algo)
+    algo = ALGOS[algo]
     x = synth.normal(11, 1, (Nn, C, H, W))
     w = synth.normal(11, 2, (K, C, R, R))
     b = synth.normal(11, 3, (K,))
@@ -44,24 +49,24 @@ def test_conv2d_all_passes(dev, case):
     dy = synth.normal(11, 4, y_ref.shape)
     xd, wd, bd, dyd = T(x, dev), T(w, dev), T(b, dev), T(dy, dev)
 
-    y = ops.conv2d_fwd(xd, wd, st, pad)
+    y = ops.conv2d_fwd(xd, wd, st, pad, algo=algo)
     assert_close(N(y), y_ref, "conv fwd")
 
     # fused bias + relu epilogue == K1 -> K2 -> K3
-    yf = ops.conv2d_fwd(xd, wd, st, pad, bias=bd, relu=True)
+    yf = ops.conv2d_fwd(xd, wd, st, pad, bias=bd, relu=True, algo=algo)
     ref_f = O.rect_inplace(O.add_bias_nchw(b, y_ref.copy()))
     assert_close(N(yf), ref_f, "conv fwd fused bias+relu")
 
     # alpha / beta blend
     y0 = synth.normal(11, 5, y_ref.shape)
-    yb = ops.conv2d_fwd(xd, wd, st, pad, alpha=0.5, beta=2.0, y=T(y0, dev))
+    yb = ops.conv2d_fwd(xd, wd, st, pad, alpha=0.5, beta=2.0, y=T(y0, dev), algo=algo)
     assert_close(N(yb), O.conv2d_fwd(x, w, st, pad, alpha=0.5, beta=2.0, y=y0.copy()), "conv fwd alpha/beta")
 
     dw_ref = O.conv2d_bwd_filter(x, dy, w.shape, st, pad)
-    dw = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad)
+    dw = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, algo=algo)
     assert_close(N(dw), dw_ref, "conv bwd filter")
     dw0 = synth.normal(11, 6, w.shape)
-    dwa = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, alpha=1.0, beta=1.0, dw=T(dw0, dev))
+    dwa = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, alpha=1.0, beta=1.0, dw=T(dw0, dev), algo=algo)
     assert_close(N(dwa), O.conv2d_bwd_filter(x, dy, w.shape, st, pad, 1.0, 1.0, dw0.copy()), "conv bwd filter beta=1")
 
     db = ops.conv2d_bwd_bias(dyd)
@@ -71,7 +76,7 @@ def test_conv2d_all_passes(dev, case):
     assert_close(N(db2), O.conv2d_bwd_bias(dy, 0.5, 1.0, db0.copy()), "conv bwd bias (two-stage)")
 
     dx_ref = O.conv2d_bwd_data(w, dy, x.shape, st, pad)
-    dx = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad)
+    dx = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad, algo=algo)
     assert_close(N(dx), dx_ref, "conv bwd data")
     torch.cuda.synchronize()
 
