@@ -293,6 +293,13 @@ def descend(W, g, s, l2):
     lib().orc_descend(C.c_int64(W.size), _f(W), _f(g), C.c_float(s), C.c_float(l2))
 
 
+def round_bf16(x):
+    """fp32 values rounded to the nearest bf16 (ties to even), returned as fp32."""
+    y = np.ascontiguousarray(x, dtype=np.float32).copy()
+    lib().orc_round_bf16(_f(y), C.c_int64(y.size))
+    return y
+
+
 def cast_u8_f32(x, scale):
     assert x.dtype == np.uint8 and x.flags.c_contiguous
     y = np.zeros(x.shape, np.float32)

@@ -564,6 +564,23 @@ void orc_cast_u8_f32(const uint8_t* x, float* y, int64_t n, float scale) {
   for (int64_t i = 0; i < n; ++i) y[i] = scale * (float)x[i];
 }
 
+/* Operand rounding of the bf16 math mode (no counterpart in the reference, which is fp32 only; the mode is
+ * this build's RH_MATH_BF16_MFMA_FP32ACC): fp32 -> bf16 round-to-nearest-even -> back to fp32, in place.
+ * NaN stays NaN (quieted).  Pinned against torch's float32 -> bfloat16 -> float32 round trip. */
+void orc_round_bf16(float* x, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) {
+    uint32_t u;
+    memcpy(&u, &x[i], 4);
+    if ((u & 0x7f800000u) == 0x7f800000u && (u & 0x007fffffu)) {
+      u = (u | 0x00400000u) & 0xffff0000u;
+    } else {
+      u += 0x7fffu + ((u >> 16) & 1u);
+      u &= 0xffff0000u;
+    }
+    memcpy(&x[i], &u, 4);
+  }
+}
+
 /* ------------------------------------------------------------------------------------------
  * Fast family: fp32 im2col + blocked SGEMM with OpenMP.  The timed CPU baseline.
  * Row-major helper:  Cm[M][N] (+)= Am[M][K] * Bm[K][N]

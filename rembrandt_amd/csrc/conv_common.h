@@ -79,6 +79,26 @@ inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Pa
   return launch_status();
 }
 
+// Same grid and split logic for the bf16-operand kernel.  FLOPs are counted as for fp32.
+template <class T, class AL, class BL, bool NCHW, class PASS>
+inline int launch_mfma_gemm_bf16(const typename AL::Params& ap, const typename BL::Params& bp,
+                                 const EpiParams& ep, int K, int splits, int* splits_used,
+                                 hipStream_t stream, const char* tag, int k_algorithmic = 0) {
+  const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
+  const int k_chunks = cdiv(K, T::BK);
+  if (splits < 1) splits = 1;
+  const int cps = cdiv(k_chunks, splits) > 0 ? cdiv(k_chunks, splits) : 1;
+  const int used = cdiv(k_chunks, cps) > 0 ? cdiv(k_chunks, cps) : 1;
+  if (splits_used) *splits_used = used;
+  dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)used);
+  constexpr size_t lds_bytes = 16 * 2 * (T::BK / 8) * (T::BM + T::BN);
+  static_assert(lds_bytes <= 48 * 1024, "bf16 tile is expected to fit the default dynamic LDS limit");
+  ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)(k_algorithmic > 0 ? k_algorithmic : K), stream);
+  hipLaunchKernelGGL((mfma_gemm_bf16_kernel<T, AL, BL, NCHW, PASS>), grid, dim3(T::NT), lds_bytes, stream, ap, bp, ep,
+                     tiles_m, k_chunks, cps);
+  return launch_status();
+}
+
 #ifndef RH_OCC_128
 #define RH_OCC_128 4
 #endif

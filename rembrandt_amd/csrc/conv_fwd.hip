@@ -74,6 +74,16 @@ static int run_fwd_soff(const RowSParams& ap, const RowSParams& bp, const EpiPar
   return launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
 }
 
+// bf16-operand forward (128x128 tile only: the loader rows must equal the tile rows).
+static int run_fwd_soff_bf16(const RowSParams& ap, const RowSParams& bp, const EpiParams& ep, int n_k, int k_true,
+                             hipStream_t stream) {
+  typedef T128x128 T;
+  typedef LoadRowS<T::BM, T::BK, T::NT, true> AL;
+  typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
+  return launch_mfma_gemm_bf16<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, 1, nullptr, stream, "conv_fwd_bf16_128x128",
+                                                             k_true);
+}
+
 template <class T>
 static int run_fwd(const ConvDims& d, const DenseParams& ap, const GatherParams& bp,
                    const EpiParams& ep, hipStream_t stream, const char* tag) {
@@ -98,7 +108,6 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
   if (int e = conv_dims(g, &d)) return e;
   if (!x || !w || !y) return RH_E_INVALID;
   if ((flags & RH_FUSE_BIAS) && !bias) return RH_E_INVALID;
-  if (flags & RH_MATH_BF16_MFMA_FP32ACC) return RH_E_UNSUPPORTED;
   if (d.y_elems == 0) return 0;
   const size_t need = rh_conv2d_workspace_bytes(g, RH_CONV_FWD);
   if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return RH_E_WORKSPACE;
@@ -106,6 +115,7 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
 
   const int CRS = d.C * d.R * d.S;
   const SoffPlan sp = plan_soff_fwd(d);
+  if ((flags & RH_MATH_BF16_MFMA_FP32ACC) && (!sp.ok || (flags & RH_ALGO_GATHER))) return RH_E_UNSUPPORTED;
   if (sp.ok && !(flags & RH_ALGO_GATHER)) {
     int* soff = static_cast<int*>(ws);
     float* wT = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes);
@@ -132,6 +142,7 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
     ep.out = y; ep.bias = (flags & RH_FUSE_BIAS) ? bias : nullptr; ep.alpha = alpha; ep.beta = beta;
     ep.rows = d.K; ep.cols = bp.M; ep.inner = d.P * d.Q; ep.ld = 0; ep.relu = (flags & RH_FUSE_RELU) ? 1 : 0;
     ep.split_stride = 0;
+    if (flags & RH_MATH_BF16_MFMA_FP32ACC) return run_fwd_soff_bf16(ap, bp, ep, sp.n_k, CRS, stream);
     switch (pick_bm(d.K)) {
       case 128: return run_fwd_soff<T128x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_128x128");
       case 96:  return run_fwd_soff<T96x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_96x256");

@@ -233,6 +233,17 @@ struct LoadGatherR {
 // Row decomposition: m -> (n, a, b) = (m / inner, (m % inner) / innerW, m % innerW);
 // vbase = 4 * (n*img_stride + a*a_stride + b*b_stride).
 // ------------------------------------------------------------------------------------------
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+// {lo, hi} -> one dword of two bf16 (lo in bits 0-15), each rounded to nearest even (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  bf16x2_t p;
+  p[0] = (__bf16)lo;
+  p[1] = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, p);
+}
+
 struct RowSParams {
   const float* ptr; uint32_t bytes;
   int M, inner, innerW;
@@ -280,6 +291,22 @@ struct LoadRowS {
   __device__ __forceinline__ void store(float* s, const float (&v)[CNT]) {
 #pragma unroll
     for (int i = 0; i < CNT; ++i) s[sbase + i * LD] = v[i];
+  }
+  // bf16 form of store(): a thread's CNT values are consecutive k of one row.  They are rounded to bf16
+  // (round to nearest even) and written as 16-byte groups of 8 consecutive k: slab[kgroup][row] (uint4),
+  // which is exactly one lane's operand of v_mfma_f32_32x32x16_bf16.
+  __device__ __forceinline__ void store_bf16(uint4* s, const float (&v)[CNT]) {
+    static_assert(CNT % 8 == 0, "bf16 packing needs 8 consecutive k per thread");
+    const int row = sbase - kk0c * LD;
+#pragma unroll
+    for (int g = 0; g < CNT / 8; ++g) {
+      uint4 q;
+      q.x = pack_bf16(v[8 * g + 0], v[8 * g + 1]);
+      q.y = pack_bf16(v[8 * g + 2], v[8 * g + 3]);
+      q.z = pack_bf16(v[8 * g + 4], v[8 * g + 5]);
+      q.w = pack_bf16(v[8 * g + 6], v[8 * g + 7]);
+      s[(kk0c / 8 + g) * ROWS + row] = q;
+    }
   }
 };
 
@@ -424,6 +451,48 @@ __device__ __forceinline__ int xcd_remap(int b, int nb) {
   return start + idx;
 }
 
+// Epilogue shared by the fp32 and bf16 kernels: D (in the 32x32 MFMA accumulator layout: lane%32 = column,
+// rows 8*(v/4) + 4*(lane/32) + v%4) -> out, with the alpha/beta blend, optional bias and ReLU, or unblended
+// into this split's slab of the partial-sum buffer.
+template <class T, bool NCHW>
+__device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], const EpiParams& ep, int m0, int n0,
+                                           int wm, int wn, int lane, int split_idx) {
+  constexpr int TM = T::TM, TN = T::TN;
+  const bool split = ep.split_stride != 0;
+  float* out = ep.out + (split ? (long long)split_idx * ep.split_stride : 0ll);
+  const float alpha = split ? 1.0f : ep.alpha;
+  const float beta = split ? 0.0f : ep.beta;
+  const int row_stride = NCHW ? ep.inner : ep.ld;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+    if (col >= ep.cols) continue;
+    int coloff;
+    if (NCHW) {
+      const int img = col / ep.inner;
+      coloff = img * ep.rows * ep.inner + (col - img * ep.inner);
+    } else {
+      coloff = col;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int rbase = m0 + wm * (TM * 32) + i * 32 + (lane >> 5) * 4;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = rbase + (v >> 2) * 8 + (v & 3);
+        if (row < ep.rows) {
+          float* dst = out + (size_t)coloff + (size_t)row * row_stride;
+          float val = alpha * acc[i][j][v];
+          if (beta != 0.0f) val += beta * *dst;
+          if (!split && ep.bias) val += ep.bias[row];
+          if (!split && ep.relu) val = val > 0.0f ? val : 0.0f;
+          *dst = val;
+        }
+      }
+    }
+  }
+}
+
 // Pass tags: they only make the instantiations of one pass distinct kernels (and kernel names) from
 // those of another pass that uses the same tile and loaders.
 struct PassConvFwd {};
@@ -558,40 +627,115 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
   for (int it = 0; it + 1 < nk; ++it) k_step(it, std::true_type());
   if (nk > 0) k_step(nk - 1, std::false_type());
 
-  // ---- epilogue
-  const bool split = ep.split_stride != 0;
-  float* out = ep.out + (split ? (long long)split_idx * ep.split_stride : 0ll);
-  const float alpha = split ? 1.0f : ep.alpha;
-  const float beta = split ? 0.0f : ep.beta;
-  const int row_stride = NCHW ? ep.inner : ep.ld;
+  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, split_idx);
+}
+
+// ------------------------------------------------------------------------------------------
+// bf16-operand form of the same tile engine (RH_MATH_BF16_MFMA_FP32ACC): operands are read as fp32 by the
+// same loaders, rounded to bf16 when they are written to LDS, multiplied with v_mfma_f32_32x32x16_bf16
+// (8 k per lane per operand) and accumulated in fp32.  LDS slabs are [k/8][row] of 16-byte groups, double
+// buffered: a loader writes one ds_write_b128 per 8 values and an MFMA operand is one ds_read_b128.
+// ------------------------------------------------------------------------------------------
+template <class T, class AL, class BL, bool NCHW, class PASS>
+__global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_kernel(typename AL::Params ap,
+                                                                       typename BL::Params bp, EpiParams ep,
+                                                                       int tiles_m, int k_chunks,
+                                                                       int chunks_per_split) {
+  constexpr int BM = T::BM, BN = T::BN, BK = T::BK, TM = T::TM, TN = T::TN;
+  static_assert(BK % 16 == 0, "one bf16 MFMA contracts 16 k");
+  constexpr int KG = BK / 8;  // 16-byte groups per row and K step
+  extern __shared__ float lds_dyn[];
+  uint4* const sA_base = reinterpret_cast<uint4*>(lds_dyn);  // [2][KG][BM]
+  uint4* const sB_base = sA_base + 2 * KG * BM;              // [2][KG][BN]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % T::WM, wn = wave / T::WM;
+
+  const int tiles = gridDim.x;
+  const int linear = xcd_remap(blockIdx.y * tiles + blockIdx.x, tiles * gridDim.y);
+  const int split_idx = __builtin_amdgcn_readfirstlane(linear / tiles);
+  const int logical = __builtin_amdgcn_readfirstlane(linear - split_idx * tiles);
+  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int c_begin = split_idx * chunks_per_split;
+  int c_end = c_begin + chunks_per_split;
+  if (c_end > k_chunks) c_end = k_chunks;
+  const int nk = c_end - c_begin;
+
+  AL la;
+  BL lb;
+  la.init(ap, m0, tid);
+  lb.init(bp, n0, tid);
+
+  f32x16 acc[TM][TN];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
-    if (col >= ep.cols) continue;
-    int coloff;
-    if (NCHW) {
-      const int img = col / ep.inner;
-      coloff = img * ep.rows * ep.inner + (col - img * ep.inner);
-    } else {
-      coloff = col;
-    }
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int rbase = m0 + wm * (TM * 32) + i * 32 + (lane >> 5) * 4;
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = rbase + (v >> 2) * 8 + (v & 3);
-        if (row < ep.rows) {
-          float* dst = out + (size_t)coloff + (size_t)row * row_stride;
-          float val = alpha * acc[i][j][v];
-          if (beta != 0.0f) val += beta * *dst;
-          if (!split && ep.bias) val += ep.bias[row];
-          if (!split && ep.relu) val = val > 0.0f ? val : 0.0f;
-          *dst = val;
-        }
-      }
-    }
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  float ra[AL::CNT], rb[BL::CNT];
+  if (nk > 0) {
+    la.prep(c_begin * BK);
+    lb.prep(c_begin * BK);
+#pragma unroll
+    for (int i = 0; i < AL::CNT; ++i) ra[i] = la.load_one(i);
+#pragma unroll
+    for (int i = 0; i < BL::CNT; ++i) rb[i] = lb.load_one(i);
+    la.store_bf16(sA_base, ra);
+    lb.store_bf16(sB_base, rb);
   }
+  if (nk > 1) {
+    la.prep((c_begin + 1) * BK);
+    lb.prep((c_begin + 1) * BK);
+  }
+  __syncthreads();
+
+  const int a_rd = (lane >> 5) * BM + wm * (TM * 32) + (lane & 31);
+  const int b_rd = (lane >> 5) * BN + wn * (TN * 32) + (lane & 31);
+
+  auto k_step = [&](int it, auto more_tag) {
+    constexpr bool MORE = decltype(more_tag)::value;
+    const int cur = it & 1;
+    if (MORE) {
+#pragma unroll
+      for (int i = 0; i < AL::CNT; ++i) ra[i] = la.load_one(i);
+#pragma unroll
+      for (int i = 0; i < BL::CNT; ++i) rb[i] = lb.load_one(i);
+    }
+    const uint4* pa = sA_base + cur * (KG * BM) + a_rd;
+    const uint4* pb = sB_base + cur * (KG * BN) + b_rd;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8_t a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = __builtin_bit_cast(bf16x8_t, pa[(2 * ks) * BM + i * 32]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = __builtin_bit_cast(bf16x8_t, pb[(2 * ks) * BN + j * 32]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (MORE) {
+      if (it + 2 < nk) {  // all loads of the next step are issued: the offsets of the one after can be fetched
+        la.prep((c_begin + it + 2) * BK);
+        lb.prep((c_begin + it + 2) * BK);
+      }
+      la.store_bf16(sA_base + (cur ^ 1) * (KG * BM), ra);
+      lb.store_bf16(sB_base + (cur ^ 1) * (KG * BN), rb);
+    }
+    __syncthreads();
+  };
+  for (int it = 0; it + 1 < nk; ++it) k_step(it, std::true_type());
+  if (nk > 0) k_step(nk - 1, std::false_type());
+
+  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, split_idx);
 }
 
 }  // namespace rh

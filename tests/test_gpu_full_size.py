@@ -86,6 +86,26 @@ def test_conv2d_full_size(dev, name):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("name", sorted(FULL_CONV))
+def test_conv2d_fwd_bf16_full_size(dev, name):
+    Nn, C, H, W, K, R, st, pad = FULL_CONV[name]
+    say("full-size bf16 conv", name)
+    rng = np.random.default_rng(7)
+    x = synth.normal(25, 1, (Nn, C, H, W))
+    w = synth.normal(25, 2, (K, C, R, R))
+    y = ops.conv2d_fwd(T(x, dev), T(w, dev), st, pad, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)
+    i_y = sample_idx(rng, y.numel(), 4096)
+    ref = O.conv2d_fwd_at(O.round_bf16(x), O.round_bf16(w), st, pad, i_y)
+    assert_close(y.flatten()[T(i_y, dev)].cpu().numpy(), ref, name + " bf16 fwd (sampled)")
+    # exact linearity and agreement with the fp32 kernel on operands that are already bf16 values
+    xr, wr = T(O.round_bf16(x), dev), T(O.round_bf16(w), dev)
+    assert torch.equal(ops.conv2d_fwd(xr, wr * 2.0, st, pad, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC), y * 2.0)
+    y32 = ops.conv2d_fwd(xr, wr, st, pad)
+    err = float((y32 - y).double().norm().item() / y32.double().norm().item())
+    assert err <= 1e-5, (name, "bf16 vs fp32 kernel on bf16-exact operands", err)
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("shape", [(256, 96, 55, 55), (256, 256, 27, 27), (256, 256, 13, 13)],
                          ids=["alexnet_pool1", "alexnet_pool2", "alexnet_pool5"])
 @pytest.mark.parametrize("mode", [_lib.RH_POOL_MAX, _lib.RH_POOL_AVG_INCL_PAD], ids=["max", "avg"])

@@ -81,6 +81,28 @@ def test_conv2d_all_passes(dev, case, algo):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("case", CONV_CASES, ids=[str(c) for c in CONV_CASES])
+def test_conv2d_fwd_bf16_operands(dev, case):
+    """RH_MATH_BF16_MFMA_FP32ACC: operands rounded to bf16 (nearest even), products accumulated in fp32.
+    Reference = the fp64-accumulating oracle on operands rounded the same way."""
+    Nn, C, H, W, K, R, st, pad = case
+    say("bf16 conv case", case)
+    x = synth.normal(12, 1, (Nn, C, H, W))
+    w = synth.normal(12, 2, (K, C, R, R))
+    b = synth.normal(12, 3, (K,))
+    y_ref = O.conv2d_fwd(O.round_bf16(x), O.round_bf16(w), st, pad)
+    y = ops.conv2d_fwd(T(x, dev), T(w, dev), st, pad, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)
+    assert_close(N(y), y_ref, "bf16 conv fwd")
+    yf = ops.conv2d_fwd(T(x, dev), T(w, dev), st, pad, bias=T(b, dev), relu=True, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)
+    assert_close(N(yf), O.rect_inplace(O.add_bias_nchw(b, y_ref.copy())), "bf16 conv fwd fused bias+relu")
+    # operands that are already bf16 values give the fp32 path's result up to summation order
+    xr, wr = O.round_bf16(x), O.round_bf16(w)
+    y32 = ops.conv2d_fwd(T(xr, dev), T(wr, dev), st, pad)
+    y16 = ops.conv2d_fwd(T(xr, dev), T(wr, dev), st, pad, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)
+    assert_close(N(y16), N(y32), "bf16 path on bf16-exact operands == fp32 path")
+    torch.cuda.synchronize()
+
+
 SGEMM_CASES = [
     # transA, transB, m, n, k
     (1, 0, 500, 64, 2450),   # affine forward  Y = W^T X

@@ -38,7 +38,11 @@ def test_error_codes_without_gpu():
     g = _lib.ConvGeom(2, 3, 8, 8, 4, 3, 3, 1, 1)
     assert lib.rh_conv2d_fwd(C.byref(g), 1.0, None, None, 0.0, None, None, None, 0, 0, None) == _lib.RH_E_INVALID
     assert lib.rh_conv2d_fwd(C.byref(g), 1.0, 256, 256, 0.0, 256, None, None, 0, 0, None) == _lib.RH_E_WORKSPACE
-    assert lib.rh_conv2d_fwd(C.byref(g), 1.0, 256, 256, 0.0, 256, None, 512, 1 << 20, _lib.RH_MATH_BF16_MFMA_FP32ACC, None) == _lib.RH_E_UNSUPPORTED
+    # bf16 operands exist for the forward pass with scalar-offset loaders only
+    assert lib.rh_conv2d_fwd(C.byref(g), 1.0, 256, 256, 0.0, 256, None, 512, 1 << 20,
+                             _lib.RH_MATH_BF16_MFMA_FP32ACC | _lib.RH_ALGO_GATHER, None) == _lib.RH_E_UNSUPPORTED
+    assert lib.rh_conv2d_bwd_data(C.byref(g), 1.0, 256, 256, 0.0, 256, 512, 1 << 20, _lib.RH_MATH_BF16_MFMA_FP32ACC,
+                                  None) == _lib.RH_E_UNSUPPORTED
     big = _lib.ConvGeom(4096, 512, 64, 64, 8, 3, 3, 1, 1)   # 32 GiB input: beyond the 2 GiB buffer-addressing limit
     assert lib.rh_conv2d_fwd(C.byref(big), 1.0, 256, 256, 0.0, 256, None, 512, 1 << 20, 0, None) == _lib.RH_E_LIMIT
     assert lib.rh_sgemm(0, 0, 4, 4, 4, 1.0, 256, 2, 256, 4, 0.0, 256, 4, None, 0, 0, None) == _lib.RH_E_INVALID  # lda < m

@@ -346,3 +346,20 @@ def test_graph_gradients_by_finite_differences():
                 flat[i] = old
                 fd = (lp - lm) / (2 * eps)
                 assert abs(fd - gflat[i]) < 2e-3 * max(1.0, abs(fd)), (fd, gflat[i])
+
+
+def test_round_bf16_matches_torch_round_trip():
+    """orc_round_bf16 against torch's float32 -> bfloat16 -> float32 (round to nearest even), on random values,
+    exact ties, subnormals, infinities and the largest finite values (which round up to infinity)."""
+    rng = np.random.default_rng(9)
+    x = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-30, 30, 20000).astype(np.float32),
+        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 1.005859375, 3.3895314e38, 3.4028235e38, -3.4028235e38,
+                  np.inf, -np.inf, 1e-40, -1e-45, 65280.0, 65408.0], np.float32),
+        # every tie pattern: bf16 value + exactly half an ulp
+        (np.arange(0x3f800000, 0x3f800000 + (1 << 20), 1 << 15, dtype=np.uint32)).view(np.float32),
+    ])
+    want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    got = O.round_bf16(x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.isnan(O.round_bf16(np.array([np.nan], np.float32))[0])
