@@ -60,9 +60,14 @@ int rho_config_params_len(const rho_config* cfg, int64_t* out);                 
 int rho_config_from_model_file(const char* path, rho_config** out);
 
 /* ---- SequentialOperatorWorker (worker.rs:230-477) ---- */
-/* into_worker(): builds the chain on `device`.  fuse_epilogue != 0 folds bias+ReLU into the conv epilogue. */
+/* into_worker(): builds the chain on `device`.  exec_flags is a bit set (0 = the reference's kernel sequence in fp32):
+ *   RHO_EXEC_FUSE_EPILOGUE  fold bias+ReLU into the conv epilogue (same buffers at every point the operators expose);
+ *   RHO_EXEC_BF16_FORWARD   conv forward multiplies operands rounded to bf16 and accumulates in fp32
+ *                           (forward-only inference mode; backward passes stay fp32 and read the same buffers). */
+#define RHO_EXEC_FUSE_EPILOGUE 0x1
+#define RHO_EXEC_BF16_FORWARD  0x2
 int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1,
-                   int device, int fuse_epilogue, rho_worker** out);
+                   int device, int exec_flags, rho_worker** out);
 int rho_worker_free(rho_worker* w);
 int rho_worker_hidden_count(rho_worker* w, int32_t* out);
 int rho_worker_op_kind(rho_worker* w, int32_t hidden_idx, const char** out);

@@ -75,6 +75,7 @@ class Conv2dOperator:
         w, h, c = in_dims
         self.x_shape = (batch, c, h, w)
         self.stride, self.pad, self.act, self.fast = conv_stride, conv_pad, act_func, fast
+        self.bf16_forward = False   # forward multiplies operands rounded to bf16 (the build's inference math mode)
         self.p = _Params((out_channels, c, conv_size, conv_size), out_channels)
         P = O.out_dim(h, conv_size, conv_stride, conv_pad)
         Q = O.out_dim(w, conv_size, conv_stride, conv_pad)
@@ -84,7 +85,9 @@ class Conv2dOperator:
 
     def forward(self, in_act):
         self.in_act = in_act
-        if self.fast:
+        if self.bf16_forward:
+            O.conv2d_fwd(O.round_bf16(in_act), O.round_bf16(self.p.weights), self.stride, self.pad, y=self.out_act)
+        elif self.fast:
             self.out_act = O.fast_conv2d_fwd(in_act, self.p.weights, self.stride, self.pad)
         else:
             O.conv2d_fwd(in_act, self.p.weights, self.stride, self.pad, y=self.out_act)

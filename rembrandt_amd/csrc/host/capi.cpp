@@ -114,14 +114,15 @@ int rho_config_from_model_file(const char* path, rho_config** out) {
 }
 
 int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1, int device,
-                   int fuse_epilogue, rho_worker** out) {
+                   int exec_flags, rho_worker** out) {
   RHO_TRY({
     RHO_REQ(cfg && out && batch_size > 0);
     std::unique_ptr<rho_worker> w(new rho_worker());
     w->ctx = std::make_shared<DeviceContext>(device);
     const uint64_t seed[2] = {seed0, seed1};
     ExecOptions opts;
-    opts.fuse_epilogue = fuse_epilogue != 0;
+    opts.fuse_epilogue = (exec_flags & RHO_EXEC_FUSE_EPILOGUE) != 0;
+    opts.bf16_forward = (exec_flags & RHO_EXEC_BF16_FORWARD) != 0;
     w->worker.reset(new SequentialOperatorWorker(cfg->cfg, (size_t)batch_size,
                                                  capability == RHO_CAP_FORWARD ? OpCapability::Forward : OpCapability::Backward,
                                                  seed, w->ctx, opts));

@@ -412,13 +412,14 @@ class Conv2dOperator : public Operator {
     rh_stream_t s = context_->stream();
     const bool rect = config_.act_func == ActivationFunction::Rect;
     if (config_.act_func != ActivationFunction::Identity && !rect) panic("unimplemented activation function");
+    const int math = opts_.bf16_forward ? RH_MATH_BF16_MFMA_FP32ACC : 0;
     if (opts_.fuse_epilogue) {
-      const int flags = RH_FUSE_BIAS | (rect ? RH_FUSE_RELU : 0);
+      const int flags = RH_FUSE_BIAS | (rect ? RH_FUSE_RELU : 0) | math;
       unwrap(rh_conv2d_fwd(&g, 1.0f, in_act_->as_ptr(), params_.weights->as_ptr(), 0.0f, out_act_->as_mut_ptr(),
                            params_.bias->as_ptr(), workspace_->as_mut_ptr(), workspace_->len(), flags, s), "conv2d forward");
     } else {
       unwrap(rh_conv2d_fwd(&g, 1.0f, in_act_->as_ptr(), params_.weights->as_ptr(), 0.0f, out_act_->as_mut_ptr(), nullptr,
-                           workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d forward");
+                           workspace_->as_mut_ptr(), workspace_->len(), math, s), "conv2d forward");
       unwrap(rh_add_bias_nchw(params_.bias->as_ptr(), out_act_->as_mut_ptr(), (int)(out_dims_.w * out_dims_.h),
                               (int)out_dims_.c, (int)batch_size, 1.0f, 1.0f, s), "add_bias");
       apply_rect(config_.act_func, out_act_->as_mut_ptr(), out_dims_.len(), batch_size, s);

@@ -158,6 +158,7 @@ struct OperatorConfig {
 // point where the reference's operators expose them.
 struct ExecOptions {
   bool fuse_epilogue = true;  // conv bias + ReLU in the conv epilogue instead of K1 -> K2 -> K3
+  bool bf16_forward = false;  // conv forward on bf16-rounded operands with fp32 accumulation (inference mode)
 };
 
 // ---- Operator trait -------------------------------------------------------------------------------

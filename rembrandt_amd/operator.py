@@ -157,10 +157,11 @@ class SequentialOperatorConfig:
 class SequentialOperatorWorker:
     """src/operator/worker.rs:230-477 plus the Input/Loss operator calls the optimizer makes on it."""
 
-    def __init__(self, config, batch_size, capability="Backward", shared_seed=(1, 2), device=0, fuse_epilogue=True):
+    def __init__(self, config, batch_size, capability="Backward", shared_seed=(1, 2), device=0, fuse_epilogue=True,
+                 bf16_forward=False):
         h = _vp()
         _chk(lib().rho_worker_new(config._h, batch_size, 0 if capability == "Forward" else 1, shared_seed[0],
-                                  shared_seed[1], device, int(fuse_epilogue), C.byref(h)))
+                                  shared_seed[1], device, (1 if fuse_epilogue else 0) | (2 if bf16_forward else 0), C.byref(h)))
         self._h = h
         self.batch_size = batch_size
         self.shared_seed = tuple(shared_seed)

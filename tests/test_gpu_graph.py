@@ -143,6 +143,52 @@ def test_alexnet_train_step(dev):
     w.close()
 
 
+def test_nin_train_step(dev):
+    """BASELINE config 5 geometry (NIN-shaped: 1x1 "cccp" convolutions, ceil-mode max-pools, 6x6 average pool
+    into 1000 classes) at batch 2, fp32: one whole step, checkpoint by checkpoint."""
+    net, batch = configs.nin(), 2
+    w, ref = make_pair(net, batch, 0x5EED0005, True)
+    sgd = SgdOpt(batch, 0.01, ("Update", 0.9), 0.0)
+    rsgd = OG.SgdOpt(0.01, ("Update", 0.9), 0.0)
+    sgd.begin(w)
+    rsgd.begin(ref)
+    say("nin step")
+    x = synth.normal(0x5EED0005, 100, (batch, 3, 224, 224))
+    labels = synth.integers(0x5EED0005, 200, (batch,), 1000)
+    check_step(w, ref, sgd, rsgd, x, labels, batch, True, "nin step 0")
+    w.close()
+
+
+def test_nin_forward_bf16(dev):
+    """BASELINE config 5, forward only with bf16 operands and fp32 accumulation.  Each operator is compared
+    from the GPU's own input to it (a last-bit difference upstream may round to a different bf16 value)."""
+    net, batch = configs.nin(), 2
+    dims, layers, ncat = net
+    cfg = configs.build_config(net, init_std=0.05)
+    w = SequentialOperatorWorker(cfg, batch, "Forward", shared_seed=(0x5EED0005, 0x5EED0006), bf16_forward=True)
+    w.init_params()
+    ref = OG.SequentialOperatorWorker(layers, ncat, batch)
+    for i, op in enumerate(ref.hidden):
+        if op.p is not None:
+            op.p.weights[...] = w.read(i, "weights").reshape(op.p.weights.shape)
+            op.bf16_forward = True
+    say("nin bf16 forward")
+    x = synth.normal(0x5EED0005, 101, (batch, 3, 224, 224))
+    w.load_frames_f32(x)
+    w.forward(batch, training=False, t=0)
+    prev = x
+    for i, op in enumerate(ref.hidden):
+        want = op.forward(np.ascontiguousarray(prev.reshape(op.x_shape if hasattr(op, "x_shape") else prev.shape)))
+        got = w.read(i, "out_act")
+        assert np.abs(got).max() > 0, "layer %d is not all zero" % i
+        assert_close(got, want.ravel(), "nin bf16 out_act[%d] %s" % (i, op.kind))
+        prev = got.reshape(want.shape).copy()
+    n = len(ref.hidden)
+    assert_close(w.read(n, "out_act"), O.softmax_fwd(np.ascontiguousarray(prev.reshape(batch, ncat))).ravel(),
+                 "nin bf16 softmax", atol=1e-7)
+    w.close()
+
+
 @pytest.mark.parametrize("flavour", ["Zero", "Update", "UpdateNesterov", "Gradient", "GradientNesterov"])
 def test_momentum_flavours(dev, flavour):
     """All five Momentum flavours on a small conv net (3 steps each, unfused BLAS-1 sequence and, where it
