@@ -31,6 +31,9 @@ pub const RH_CONV_BWD_FILTER: c_int = 1;
 pub const RH_CONV_BWD_DATA: c_int = 2;
 pub const RH_FUSE_BIAS: c_int = 0x10;
 pub const RH_FUSE_RELU: c_int = 0x20;
+pub const RH_MATH_BF16_MFMA_FP32ACC: c_int = 0x1;
+pub const RH_ALGO_GATHER: c_int = 0x100;
+pub const RH_ALGO_SCALAR_OFFSET: c_int = 0x200;
 
 #[link(name = "rembrandt_hip")]
 extern "C" {
@@ -58,6 +61,9 @@ extern "C" {
                               stream: rh_stream_t) -> c_int;
   pub fn rh_conv2d_bwd_bias(n: i32, k: i32, plane: i32, alpha: c_float, dy: *const f32, beta: c_float,
                             db: *mut f32, stream: rh_stream_t) -> c_int;
+  pub fn rh_conv2d_bwd_bias_workspace_bytes(n: i32, k: i32, plane: i32) -> size_t;
+  pub fn rh_conv2d_bwd_bias_ws(n: i32, k: i32, plane: i32, alpha: c_float, dy: *const f32, beta: c_float,
+                               db: *mut f32, ws: *mut c_void, ws_bytes: size_t, stream: rh_stream_t) -> c_int;
   pub fn rh_conv2d_bwd_data(g: *const rh_conv_geom, alpha: c_float, w: *const f32, dy: *const f32,
                             beta: c_float, dx: *mut f32, ws: *mut c_void, ws_bytes: size_t, flags: c_int,
                             stream: rh_stream_t) -> c_int;
