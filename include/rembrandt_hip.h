@@ -197,6 +197,45 @@ int rh_sgd_momentum_step(int64_t n, float* W, float* g, float* v, float l2, floa
 int rh_descend(int64_t n, float* W, float* g, float s, float l2, rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Input preprocessing of Data3dOperator::forward (src/operator/mod.rs:640-790) and dropout
+ * (src/operator/mod.rs:2211-2248).  The three `rembrandt_kernel_*` symbols keep the names and argument
+ * lists of the reference's call sites; their bodies live in a crate outside its tree, so what they compute
+ * is this build's reading of those call sites:
+ *   rh_crop_nchw                 replaces CudnnTransformOp::transform on a strided 4-d view (mod.rs:666-691):
+ *                                dst[p][h][w] = src[p][off_h + h][off_w + w], p < planes = batch * channels.
+ *   ..._blockmap256_flip         dst[r][w] = src[r][width-1-w], r < rows (mod.rs:767-773); no width <= 256 limit.
+ *   ..._preproc_pca3_noise       dst[n][c][i] = src[n][c][i] + sum_j svecs[3j + c] * alphas[3n + j] * svals[j]
+ *                                (3 channels; mod.rs:716-725).
+ *   rembrandt_kernel_map_dropout mask[i] = rnd[i] > drop_ratio; out[i] = mask ? scale * in[i] : 0 (mod.rs:2221-2229).
+ *   ..._map_dropout_backprop     in_delta[i] = mask[i] ? scale * out_delta[i] : 0 (mod.rs:2239-2246).
+ * ------------------------------------------------------------------------------------------- */
+int rh_crop_nchw(const float* src, float* dst, int64_t planes, int32_t in_w, int32_t in_h, int32_t crop_w,
+                 int32_t crop_h, int32_t off_w, int32_t off_h, rh_stream_t stream);
+void rembrandt_kernel_batch_blockmap256_flip(const float* src, int32_t width, int32_t rows, float* dst,
+                                             rh_stream_t stream);
+void rembrandt_kernel_batch_map_preproc_pca3_noise(const float* src, int32_t spatial, int32_t batch,
+                                                   const float* alphas, const float* svals, const float* svecs,
+                                                   float* dst, rh_stream_t stream);
+void rembrandt_kernel_map_dropout(const float* in, int32_t n, float drop_ratio, float scale, const float* rnd,
+                                  float* out, int32_t* mask, rh_stream_t stream);
+void rembrandt_kernel_map_dropout_backprop(const float* out_delta, int32_t n, float drop_ratio, float scale,
+                                           const int32_t* mask, float* in_delta, rh_stream_t stream);
+
+/* Cross-channel local response normalisation (the `local_res_norm` layer type of the reference's `.model`
+ * grammar, examples/imagenet_alexnet.model:31-37; the reference's own layer is an empty stub,
+ * src/layer.rs:1846-1899, so the arithmetic is the published one those parameters name):
+ *   d[n,c,h,w] = min_div + scale * sum_{c' = c - size/2 .. c + (size-1)/2, clipped} x[n,c',h,w]^2
+ *   y = x * d^-power.   `denom` (same shape as x) receives d and is an input of the backward pass. */
+typedef struct rh_lrn_geom {
+  int32_t N, C, H, W;
+  int32_t size;
+  float scale, power, min_div;
+} rh_lrn_geom;
+int rh_lrn_fwd(const rh_lrn_geom* g, const float* x, float* y, float* denom, rh_stream_t stream);
+int rh_lrn_bwd(const rh_lrn_geom* g, const float* x, const float* y, const float* denom, const float* dy, float* dx,
+               rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Host-side seeded generator for synthetic inputs and parameter initialisation (stands in for
  * the rng crate's Xorshiftplus128Rng + rand 0.3 distributions of src/operator/mod.rs:964-1006,
  * 1554-1592, whose bit streams cannot be reproduced).  Element i of stream (seed, stream_id) is
@@ -205,6 +244,10 @@ int rh_descend(int64_t n, float* W, float* g, float s, float l2, rh_stream_t str
 int rh_rng_fill_uniform(uint64_t seed, uint64_t stream_id, float* host, size_t n, float lo, float hi);
 int rh_rng_fill_normal(uint64_t seed, uint64_t stream_id, float* host, size_t n, float mean, float std);
 int rh_rng_fill_int(uint64_t seed, uint64_t stream_id, int32_t* host, size_t n, int32_t modulus);
+/* Device form: dst[i] (device pointer) = element (first + i) of rh_rng_fill_uniform(seed, stream_id, ., ., 0, 1),
+ * bit for bit.  Stands in for DeviceBuffer::sample(&UniformDist) (mod.rs:2220). */
+int rh_rng_fill_uniform01_device(uint64_t seed, uint64_t stream_id, uint64_t first, float* dst, size_t n,
+                                 rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Per-launch timing (no counterpart in the reference, which only takes wall-clock laps around

@@ -305,3 +305,74 @@ def cast_u8_f32(x, scale):
     y = np.zeros(x.shape, np.float32)
     lib().orc_cast_u8_f32(x.ctypes.data_as(C.POINTER(C.c_uint8)), _f(y), C.c_int64(x.size), C.c_float(scale))
     return y
+
+
+# ---- Data3d preprocessing, dropout, local response normalisation (numpy restatements) ------------------------
+
+def crop_nchw(x, crop_w, crop_h, off_w, off_h):
+    """Strided 4-d copy of Data3dOperator's Crop (src/operator/mod.rs:666-691): one offset for the whole batch."""
+    return np.ascontiguousarray(x[:, :, off_h:off_h + crop_h, off_w:off_w + crop_w])
+
+
+def flip_x(x):
+    """FlipX (src/operator/mod.rs:751-777): every row of the batch reversed along the width."""
+    return np.ascontiguousarray(x[..., ::-1])
+
+
+def subtract_mean(x, mean, normalize):
+    """SubtractElemwiseMean (src/operator/mod.rs:732-749): x + alpha * mean, alpha = -1/255 if normalize else -1,
+    mean broadcast over the batch."""
+    alpha = np.float32(-1.0 / 255.0) if normalize else np.float32(-1.0)
+    return (x.astype(np.float64) + np.float64(alpha) * mean.astype(np.float64)[None]).astype(np.float32)
+
+
+def pca3_noise(x, alphas, svals, svecs):
+    """AddPixelwisePCALightingNoise in training (src/operator/mod.rs:709-727): channel c of image n is shifted by
+    sum_j svecs[j][c] * alphas[n][j] * svals[j] (svecs[j] = the j-th singular vector, as the operator flattens it,
+    mod.rs:523-533; which index the kernel treats as the channel is this build's choice)."""
+    shift = np.einsum("jc,nj,j->nc", svecs.reshape(3, 3).astype(np.float64), alphas.reshape(-1, 3).astype(np.float64),
+                      svals.astype(np.float64))
+    return (x.astype(np.float64) + shift[:, :, None, None]).astype(np.float32)
+
+
+def dropout(x, ratio, scale, rnd):
+    """rembrandt_kernel_map_dropout as called at src/operator/mod.rs:2221-2229: keep where rnd > ratio."""
+    mask = (rnd > np.float32(ratio)).astype(np.int32)
+    return (np.float32(scale) * x * mask).astype(np.float32), mask
+
+
+def dropout_backprop(dy, scale, mask):
+    """rembrandt_kernel_map_dropout_backprop as called at src/operator/mod.rs:2239-2246."""
+    return (np.float32(scale) * dy * mask).astype(np.float32)
+
+
+def lrn_fwd(x, size, scale, power, min_div):
+    """Cross-channel local response normalisation with the parameters of examples/imagenet_alexnet.model:31-37
+    (cross_size, scale, power, min_div): d = min_div + scale * sum over the clipped channel window of x^2,
+    y = x * d^-power.  fp64."""
+    N, Cc = x.shape[0], x.shape[1]
+    x64 = x.astype(np.float64)
+    d = np.empty_like(x64)
+    lo, hi = size // 2, (size - 1) // 2
+    for c in range(Cc):
+        c0, c1 = max(0, c - lo), min(Cc - 1, c + hi)
+        d[:, c] = min_div + scale * (x64[:, c0:c1 + 1] ** 2).sum(axis=1)
+    return (x64 * d ** (-power)).astype(np.float32), d.astype(np.float32)
+
+
+def lrn_bwd(x, dy, size, scale, power, min_div):
+    """Gradient of lrn_fwd w.r.t. x (fp64): dx[c] = dy[c] d[c]^-p - 2 scale p x[c] sum_{c': c in win(c')} dy[c'] y[c'] / d[c']."""
+    Cc = x.shape[1]
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    lo, hi = size // 2, (size - 1) // 2
+    d = np.empty_like(x64)
+    for c in range(Cc):
+        c0, c1 = max(0, c - lo), min(Cc - 1, c + hi)
+        d[:, c] = min_div + scale * (x64[:, c0:c1 + 1] ** 2).sum(axis=1)
+    y = x64 * d ** (-power)
+    t = dy64 * y / d
+    dx = dy64 * d ** (-power)
+    for c in range(Cc):
+        c0, c1 = max(0, c - hi), min(Cc - 1, c + lo)
+        dx[:, c] -= 2.0 * scale * power * x64[:, c] * t[:, c0:c1 + 1].sum(axis=1)
+    return dx.astype(np.float32)

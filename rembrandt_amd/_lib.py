@@ -22,6 +22,10 @@ class ConvGeom(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "K", "R", "S", "stride", "pad")]
 
 
+class LrnGeom(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "size")] + [(n, C.c_float) for n in ("scale", "power", "min_div")]
+
+
 class PoolGeom(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "size", "stride", "pad", "mode", "round")]
 
@@ -44,6 +48,14 @@ PROTOTYPES = {
     "rh_load_sync": (_int, [_vp, _vp, _vp, _sz]),
     "rh_store_sync": (_int, [_vp, _vp, _vp, _sz]),
     "rh_cast_u8_f32": (_int, [_vp, _vp, _sz, _f, _vp]),
+    "rh_crop_nchw": (_int, [_vp, _vp, C.c_int64, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "rembrandt_kernel_batch_blockmap256_flip": (None, [_vp, _i32, _i32, _vp, _vp]),
+    "rembrandt_kernel_batch_map_preproc_pca3_noise": (None, [_vp, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "rembrandt_kernel_map_dropout": (None, [_vp, _i32, _f, _f, _vp, _vp, _vp, _vp]),
+    "rembrandt_kernel_map_dropout_backprop": (None, [_vp, _i32, _f, _f, _vp, _vp, _vp]),
+    "rh_rng_fill_uniform01_device": (_int, [C.c_uint64, C.c_uint64, C.c_uint64, _vp, _sz, _vp]),
+    "rh_lrn_fwd": (_int, [C.POINTER(LrnGeom), _vp, _vp, _vp, _vp]),
+    "rh_lrn_bwd": (_int, [C.POINTER(LrnGeom), _vp, _vp, _vp, _vp, _vp, _vp]),
     "rh_conv2d_out_dim": (_i32, [_i32, _i32, _i32, _i32]),
     "rh_conv2d_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _int]),
     "rh_conv2d_fwd": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _vp, _sz, _int, _vp]),

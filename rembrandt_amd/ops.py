@@ -225,6 +225,69 @@ def cast_u8_f32(x, scale):
     return y
 
 
+def crop_nchw(x, crop_w, crop_h, off_w, off_h):
+    N, Cc, H, W = x.shape
+    y = torch.empty((N, Cc, crop_h, crop_w), dtype=torch.float32, device=x.device)
+    check(lib().rh_crop_nchw(_p(x), _p(y), N * Cc, W, H, crop_w, crop_h, off_w, off_h, _stream()), "rh_crop_nchw")
+    return y
+
+
+def flip_x(x):
+    y = torch.empty_like(x)
+    lib().rembrandt_kernel_batch_blockmap256_flip(_p(x), x.shape[-1], x.numel() // x.shape[-1], _p(y), _stream())
+    _check_last("rembrandt_kernel_batch_blockmap256_flip")
+    return y
+
+
+def pca3_noise(x, alphas, svals, svecs):
+    N, Cc, H, W = x.shape
+    assert Cc == 3
+    y = torch.empty_like(x)
+    lib().rembrandt_kernel_batch_map_preproc_pca3_noise(_p(x), H * W, N, _p(alphas), _p(svals), _p(svecs), _p(y), _stream())
+    _check_last("rembrandt_kernel_batch_map_preproc_pca3_noise")
+    return y
+
+
+def dropout(x, ratio, scale, rnd):
+    y = torch.empty_like(x)
+    mask = torch.empty(x.shape, dtype=torch.int32, device=x.device)
+    lib().rembrandt_kernel_map_dropout(_p(x), x.numel(), ratio, scale, _p(rnd), _p(y), _p(mask), _stream())
+    _check_last("rembrandt_kernel_map_dropout")
+    return y, mask
+
+
+def dropout_backprop(dy, ratio, scale, mask):
+    dx = torch.empty_like(dy)
+    lib().rembrandt_kernel_map_dropout_backprop(_p(dy), dy.numel(), ratio, scale, _p(mask), _p(dx), _stream())
+    _check_last("rembrandt_kernel_map_dropout_backprop")
+    return dx
+
+
+def rng_uniform01_device(seed, stream_id, first, n, device):
+    t = torch.empty((n,), dtype=torch.float32, device=device)
+    check(lib().rh_rng_fill_uniform01_device(seed, stream_id, first, _p(t), n, _stream()), "rh_rng_fill_uniform01_device")
+    return t
+
+
+def lrn_geom(x_shape, size, scale, power, min_div):
+    N, Cc, H, W = x_shape
+    return _lib.LrnGeom(N, Cc, H, W, size, scale, power, min_div)
+
+
+def lrn_fwd(x, size, scale, power, min_div):
+    g = lrn_geom(x.shape, size, scale, power, min_div)
+    y, d = torch.empty_like(x), torch.empty_like(x)
+    check(lib().rh_lrn_fwd(C.byref(g), _p(x), _p(y), _p(d), _stream()), "rh_lrn_fwd")
+    return y, d
+
+
+def lrn_bwd(x, y, d, dy, size, scale, power, min_div):
+    g = lrn_geom(x.shape, size, scale, power, min_div)
+    dx = torch.empty_like(x)
+    check(lib().rh_lrn_bwd(C.byref(g), _p(x), _p(y), _p(d), _p(dy), _p(dx), _stream()), "rh_lrn_bwd")
+    return dx
+
+
 def memset_f32(t, value):
     check(lib().rh_memset_f32(_p(t), value, t.numel(), _stream()), "rh_memset_f32")
     return t

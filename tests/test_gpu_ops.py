@@ -264,3 +264,55 @@ def test_cast_and_fill(dev):
     t = torch.empty(1027, device=dev)
     ops.memset_f32(t[1:], 1.0)
     assert (N(t)[1:] == 1.0).all()
+
+
+def test_preproc_kernels(dev):
+    say("preproc kernels")
+    x = synth.normal(13, 1, (5, 3, 37, 41))
+    xd = T(x, dev)
+    for (cw, ch, ow, oh) in ((41, 37, 0, 0), (32, 32, 9, 5), (1, 1, 40, 36), (17, 3, 0, 34)):
+        assert np.array_equal(N(ops.crop_nchw(xd, cw, ch, ow, oh)), O.crop_nchw(x, cw, ch, ow, oh))
+    assert np.array_equal(N(ops.flip_x(xd)), O.flip_x(x))
+    wide = synth.normal(13, 2, (2, 1, 3, 300))     # wider than the 256 the reference asserts
+    assert np.array_equal(N(ops.flip_x(T(wide, dev))), O.flip_x(wide))
+    alphas, svals, svecs = synth.normal(13, 3, (15,)), synth.uniform(13, 4, (3,)), synth.normal(13, 5, (9,))
+    assert_close(N(ops.pca3_noise(xd, T(alphas, dev), T(svals, dev), T(svecs, dev))), O.pca3_noise(x, alphas, svals, svecs),
+                 "pca3 noise")
+    # mean subtraction is the bias-add kernel with one "channel" per frame element
+    mean = synth.normal(13, 6, (3, 37, 41))
+    for normalize in (False, True):
+        y = T(x, dev).clone()
+        ops.add_bias_nchw(T(mean.ravel(), dev), y.view(5, -1, 1), alpha=(-1.0 / 255.0 if normalize else -1.0), beta=1.0)
+        assert_close(N(y), O.subtract_mean(x, mean, normalize), "subtract mean")
+    torch.cuda.synchronize()
+
+
+def test_dropout_and_device_rng(dev):
+    say("dropout / device rng")
+    n = (1 << 18) + 77
+    host = synth.uniform(31, 9, (n + 1000,))
+    got = ops.rng_uniform01_device(31, 9, 1000, n, dev)
+    assert np.array_equal(N(got), host[1000:]), "device generator == host generator, element by element"
+    x, dy = synth.normal(14, 1, (n,)), synth.normal(14, 2, (n,))
+    for ratio in (0.5, 0.1, 0.0, 1.0):
+        y, mask = ops.dropout(T(x, dev), ratio, 1.0, got)
+        y_ref, m_ref = O.dropout(x, ratio, 1.0, host[1000:])
+        assert np.array_equal(N(mask), m_ref) and np.array_equal(N(y), y_ref)
+        assert np.array_equal(N(ops.dropout_backprop(T(dy, dev), ratio, 1.0, mask)), O.dropout_backprop(dy, 1.0, m_ref))
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("case", [((2, 7, 5, 6), 5), ((3, 96, 27, 27), 5), ((1, 3, 4, 4), 5), ((2, 10, 3, 3), 4), ((2, 4, 3, 3), 1)])
+def test_lrn(dev, case):
+    shape, size = case
+    say("lrn", case)
+    scale, power, min_div = 1e-4, 0.75, 2.0
+    x = synth.normal(15, 1, shape) * np.float32(20.0)
+    dy = synth.normal(15, 2, shape)
+    y, d = ops.lrn_fwd(T(x, dev), size, scale, power, min_div)
+    y_ref, d_ref = O.lrn_fwd(x, size, scale, power, min_div)
+    assert_close(N(d), d_ref, "lrn denominators")
+    assert_close(N(y), y_ref, "lrn fwd")
+    dx = ops.lrn_bwd(T(x, dev), y, d, T(dy, dev), size, scale, power, min_div)
+    assert_close(N(dx), O.lrn_bwd(x, dy, size, scale, power, min_div), "lrn bwd")
+    torch.cuda.synchronize()

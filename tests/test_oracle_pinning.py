@@ -363,3 +363,46 @@ def test_round_bf16_matches_torch_round_trip():
     got = O.round_bf16(x)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     assert np.isnan(O.round_bf16(np.array([np.nan], np.float32))[0])
+
+
+def test_lrn_matches_torch_local_response_norm():
+    """lrn_fwd / lrn_bwd against torch's local_response_norm (fp64) and its autograd; torch divides alpha by the
+    window size, the `.model` parameter `scale` multiplies the plain sum."""
+    rng = np.random.default_rng(10)
+    for (shape, size) in (((2, 7, 3, 4), 5), ((1, 3, 2, 2), 5), ((2, 8, 3, 3), 4), ((2, 6, 2, 5), 1)):
+        x = rng.standard_normal(shape).astype(np.float32) * 3
+        dy = rng.standard_normal(shape).astype(np.float32)
+        scale, power, min_div = 1e-2, 0.75, 2.0
+        xt = torch.from_numpy(x).double().requires_grad_(True)
+        yt = F.local_response_norm(xt, size, alpha=scale * size, beta=power, k=min_div)
+        (gx,) = torch.autograd.grad(yt, xt, torch.from_numpy(dy).double())
+        y, d = O.lrn_fwd(x, size, scale, power, min_div)
+        np.testing.assert_allclose(y, yt.detach().numpy(), rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(O.lrn_bwd(x, dy, size, scale, power, min_div), gx.numpy(), rtol=1e-5, atol=1e-6)
+        assert (d >= min_div).all()
+
+
+def test_preproc_and_dropout_restatements():
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((3, 3, 9, 8)).astype(np.float32)
+    xt = torch.from_numpy(x)
+    assert np.array_equal(O.crop_nchw(x, 5, 4, 2, 3), xt[:, :, 3:7, 2:7].numpy())
+    assert np.array_equal(O.flip_x(x), torch.flip(xt, dims=[3]).numpy())
+    mean = rng.standard_normal((3, 9, 8)).astype(np.float32)
+    np.testing.assert_allclose(O.subtract_mean(x, mean, False), x - mean[None], rtol=0, atol=1e-7)
+    np.testing.assert_allclose(O.subtract_mean(x, mean, True), x - mean[None] / 255.0, rtol=0, atol=1e-6)
+    alphas, svals, svecs = (rng.standard_normal(9).astype(np.float32), rng.random(3).astype(np.float32),
+                            rng.standard_normal(9).astype(np.float32))
+    want = x.astype(np.float64).copy()
+    for n in range(3):
+        for c in range(3):
+            want[n, c] += sum(float(svecs[j * 3 + c]) * float(alphas[n * 3 + j]) * float(svals[j]) for j in range(3))
+    np.testing.assert_allclose(O.pca3_noise(x, alphas, svals, svecs), want, rtol=1e-6, atol=1e-6)
+    rnd = rng.random(x.shape).astype(np.float32)
+    y, mask = O.dropout(x, 0.5, 1.0, rnd)
+    assert mask.sum() == (rnd > 0.5).sum() and np.array_equal(y, np.where(rnd > 0.5, x, 0).astype(np.float32))
+    # backward is the adjoint of forward for a fixed mask
+    dy = rng.standard_normal(x.shape).astype(np.float32)
+    lhs = float((y.astype(np.float64) * dy).sum())
+    rhs = float((x.astype(np.float64) * O.dropout_backprop(dy, 1.0, mask)).sum())
+    assert abs(lhs - rhs) < 1e-9 * max(1.0, abs(lhs))
