@@ -53,7 +53,21 @@ int rho_config_affine(rho_config* cfg, int32_t in_channels, int32_t out_channels
                       float init_value);                                                              /* .affine()  */
 int rho_config_pool2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t pool_size,
                       int32_t pool_stride, int32_t pool_pad, int pool_op, int ceil_mode);              /* .pool2d()  */
-int rho_config_softmax_kl_loss(rho_config* cfg, int32_t num_categories);                              /* .softmax_kl_loss() */
+int rho_config_softmax_kl_loss(rho_config* cfg, int32_t num_categories);
+/* Data3dPreproc steps appended to the input operator's list, in call order (src/operator/mod.rs:395-423, 545-597).
+ * Crop and FlipX draw once per forward() for the whole batch in Training and are centre / off in Inference;
+ * SubtractElemwiseMean takes in_dims.len() values (W fastest) or an NdArray file; the mean is scaled by 1/255 when
+ * the input operator normalises.  PCA lighting noise: 3x3 singular vectors (row j = vector j), 3 singular values. */
+int rho_config_data3d_crop(rho_config* cfg, int32_t crop_width, int32_t crop_height);
+int rho_config_data3d_flip_x(rho_config* cfg);
+int rho_config_data3d_subtract_mean(rho_config* cfg, const float* mean, int64_t len);
+int rho_config_data3d_subtract_mean_file(rho_config* cfg, const char* mean_path);
+int rho_config_data3d_pca_lighting_noise(rho_config* cfg, const float* singular_vecs9, const float* singular_vals3,
+                                         float std_dev);
+int rho_config_dropout(rho_config* cfg, int32_t channels, float drop_ratio);                           /* .dropout() worker.rs:219 */
+/* `local_res_norm` layers of the .model grammar (cross-channel; the reference's layer is a stub, layer.rs:1846-1899). */
+int rho_config_local_res_norm(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t cross_size, float scale,
+                              float power, float min_div);                              /* .softmax_kl_loss() */
 int rho_config_params_len(const rho_config* cfg, int64_t* out);                                       /* .params_len() */
 /* Parses a `.model` file of the reference's grammar (src/config.rs:16-264) into a config.
  * batch-independent; returns the input dims through the config's data3d entry. */
@@ -69,6 +83,26 @@ int rho_config_from_model_file(const char* path, rho_config** out);
 int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1,
                    int device, int exec_flags, rho_worker** out);
 int rho_worker_free(rho_worker* w);
+/* Output frame shape of the input operator (after crops), and what its last forward() drew. */
+int rho_worker_input_out_dims(rho_worker* w, int32_t* out_w, int32_t* out_h, int32_t* out_c);
+int rho_worker_last_preproc_draws(rho_worker* w, int32_t* crop_off_w, int32_t* crop_off_h, int* flipped, float* alphas,
+                                  int64_t alphas_cap, int64_t* alphas_len);
+/* The uniform stream a DropoutOperator's last Training forward() consumed: rand[i] = element (first + i) of
+ * rh_rng_fill_uniform(seed, stream_id, ., ., 0, 1). */
+int rho_worker_dropout_stream(rho_worker* w, int32_t hidden_idx, uint64_t* seed, uint64_t* stream_id, uint64_t* first);
+/* encode/decode_params, encode/decode_state over all hidden operators (mod.rs:1008-1073, 1594-1661): a sequence of
+ * NdArray records ('N','D',0,1, u32 rank, u64 dims, fp32 LE data).  Call encode with buf == NULL to get the size. */
+int rho_worker_encode_params(rho_worker* w, uint8_t* buf, size_t cap, size_t* needed);
+int rho_worker_decode_params(rho_worker* w, const uint8_t* blob, size_t len, size_t* consumed);
+int rho_worker_encode_state(rho_worker* w, uint8_t* buf, size_t cap, size_t* needed);
+int rho_worker_decode_state(rho_worker* w, const uint8_t* blob, size_t len, size_t* consumed);
+/* Checkpoint files under `prefix` (worker/gossip_dist.rs:1230-1413): params.t_<t>.blob, params.latest.blob -> it,
+ * `checkpoint` (text: t), checkpoint.0 (previous), state.latest.blob.<rank>. */
+int rho_worker_checkpoint_params(rho_worker* w, int64_t t, const char* prefix);
+int rho_worker_checkpoint_state(rho_worker* w, const char* prefix);
+int rho_worker_can_rollback(rho_worker* w, const char* prefix, int64_t* t_or_minus1);
+int rho_worker_rollback_params(rho_worker* w, int64_t t_or_minus1 /* -1 = latest */, const char* prefix);
+int rho_worker_rollback_state(rho_worker* w, const char* prefix);
 int rho_worker_hidden_count(rho_worker* w, int32_t* out);
 int rho_worker_op_kind(rho_worker* w, int32_t hidden_idx, const char** out);
 void* rho_worker_stream(rho_worker* w);                                      /* ctx.stream.ptr */

@@ -179,6 +179,57 @@ class Pool2dOperator:
         return O.pool2d_bwd(self.in_act, self.out_act, self.out_delta, self.k, self.st, self.pad, self.mode, self.rounding)
 
 
+class DropoutOperator:
+    """src/operator/mod.rs:2134-2255.  `rnd` (the uniform samples of this forward) is set by the caller: the
+    reference draws them from a device generator whose stream cannot be reproduced."""
+    kind = "DropoutOperator"
+    p = None
+
+    def __init__(self, batch, channels, drop_ratio):
+        self.x_shape = (batch, channels)
+        self.ratio = drop_ratio
+        self.rnd = None
+        self.training = True
+        self.out_act = np.zeros(self.x_shape, np.float32)
+        self.out_delta = np.zeros(self.x_shape, np.float32)
+
+    def forward(self, in_act):
+        self.in_act = np.ascontiguousarray(in_act.reshape(self.x_shape))
+        if not self.training:
+            self.out_act = self.in_act.copy()
+            return self.out_act
+        self.out_act, self.mask = O.dropout(self.in_act, self.ratio, 1.0, self.rnd.reshape(self.x_shape))
+        return self.out_act
+
+    def backward(self, want_in_delta):
+        if not want_in_delta:
+            return None
+        return O.dropout_backprop(self.out_delta.reshape(self.x_shape), 1.0, self.mask)
+
+
+class LocalResNormOperator:
+    """Cross-channel local response normalisation (`local_res_norm` of the .model grammar)."""
+    kind = "LocalResNormOperator"
+    p = None
+
+    def __init__(self, batch, in_dims, cross_size, scale, power, min_div):
+        w, h, c = in_dims
+        self.x_shape = (batch, c, h, w)
+        self.args = (cross_size, scale, power, min_div)
+        self.out_act = np.zeros(self.x_shape, np.float32)
+        self.out_delta = np.zeros(self.x_shape, np.float32)
+
+    def forward(self, in_act):
+        self.in_act = np.ascontiguousarray(in_act.reshape(self.x_shape))
+        self.out_act, _ = O.lrn_fwd(self.in_act, *self.args)
+        return self.out_act
+
+    def backward(self, want_in_delta):
+        if not want_in_delta:
+            return None
+        return O.lrn_bwd(self.in_act, self.out_delta.reshape(self.x_shape), *self.args)
+
+
 class SequentialOperatorWorker:
     """layers: list of tuples mirroring the SequentialOperatorConfig builder calls, e.g.
     ("conv2d", in_dims, size, stride, pad, out_channels, act), ("pool2d", in_dims, size, stride, pad, op, ceil),
@@ -194,6 +245,10 @@ class SequentialOperatorWorker:
                 self.hidden.append(AffineOperator(batch, *l[1:], fast=fast))
             elif l[0] == "pool2d":
                 self.hidden.append(Pool2dOperator(batch, *l[1:]))
+            elif l[0] == "dropout":
+                self.hidden.append(DropoutOperator(batch, *l[1:]))
+            elif l[0] == "local_res_norm":
+                self.hidden.append(LocalResNormOperator(batch, *l[1:]))
             else:
                 raise ValueError(l[0])
         self.labels = np.zeros((batch,), np.int32)

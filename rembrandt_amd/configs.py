@@ -5,6 +5,8 @@ layer tuples repeat the arguments of the SequentialOperatorConfig builder calls:
     ("conv2d", in_dims, conv_size, conv_stride, conv_pad, out_channels, act_func)
     ("pool2d", in_dims, pool_size, pool_stride, pool_pad, pool_op, ceil_mode)
     ("affine", in_channels, out_channels, act_func)
+    ("dropout", channels, drop_ratio)
+    ("local_res_norm", in_dims, cross_size, scale, power, min_div)
 Geometry the benchmark text leaves open follows the reference's own tools:
 LeNet from tools/train-mnist.rs:79-133 (conv pad 2, conv activations Identity, FC1 in 2450),
 the CIFAR-10 net from tools/train-cifar10.rs:58-162 (3x3 stride-2 pools with pad 1),
@@ -14,7 +16,8 @@ from .operator import SequentialOperatorConfig
 
 
 def _chain(input_dims, spec):
-    """spec entries: ("conv", size, stride, pad, out, act) | ("pool", size, stride, pad, op[, ceil]) | ("fc", out, act)."""
+    """spec entries: ("conv", size, stride, pad, out, act) | ("pool", size, stride, pad, op[, ceil]) | ("fc", out, act)
+    | ("dropout", ratio) | ("lrn", cross_size, scale, power, min_div)."""
     w, h, c = input_dims
     layers = []
     for s in spec:
@@ -38,6 +41,10 @@ def _chain(input_dims, spec):
             _, out, act = s
             layers.append(("affine", w * h * c, out, act))
             w, h, c = 1, 1, out
+        elif s[0] == "dropout":
+            layers.append(("dropout", w * h * c, s[1]))
+        elif s[0] == "lrn":
+            layers.append(("local_res_norm", (w, h, c), s[1], s[2], s[3], s[4]))
         else:
             raise ValueError(s[0])
     return layers, w * h * c
@@ -95,6 +102,10 @@ def build_config(net, init_std=0.01):
             cfg.conv2d(l[1], l[2], l[3], l[4], l[5], l[6], ("Normal", init_std))
         elif l[0] == "pool2d":
             cfg.pool2d(l[1], l[2], l[3], l[4], l[5], l[6])
+        elif l[0] == "dropout":
+            cfg.dropout(l[1], l[2])
+        elif l[0] == "local_res_norm":
+            cfg.local_res_norm(l[1], l[2], l[3], l[4], l[5])
         else:
             cfg.affine(l[1], l[2], l[3], ("Normal", init_std))
     return cfg.softmax_kl_loss(num_categories)

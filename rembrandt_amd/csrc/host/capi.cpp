@@ -1,6 +1,8 @@
 // C ABI of the operator / graph / optimizer layer (include/rembrandt_operator.h).
 #include <memory>
 #include <string>
+#include <vector>
+#include <algorithm>
 
 #include "../../../include/rembrandt_operator.h"
 #include "model_config.hpp"
@@ -65,6 +67,74 @@ int rho_config_data3d(rho_config* cfg, int32_t w, int32_t h, int32_t c, int norm
     RHO_REQ(cfg && w > 0 && h > 0 && c > 0);
     Data3dOperatorConfig d = {{(size_t)w, (size_t)h, (size_t)c}, normalize != 0};
     cfg->cfg.data3d(d);
+  })
+}
+static Data3dOperatorConfig& input_cfg(rho_config* cfg) {
+  RHO_REQ(cfg && cfg->cfg.has_input);
+  return cfg->cfg.input_op.data3d;
+}
+int rho_config_data3d_crop(rho_config* cfg, int32_t crop_width, int32_t crop_height) {
+  RHO_TRY({
+    RHO_REQ(crop_width > 0 && crop_height > 0);
+    Data3dPreproc p;
+    p.kind = Data3dPreproc::Crop;
+    p.crop_width = (size_t)crop_width;
+    p.crop_height = (size_t)crop_height;
+    input_cfg(cfg).preprocs.push_back(p);
+    (void)input_cfg(cfg).get_out_dims();
+  })
+}
+int rho_config_data3d_flip_x(rho_config* cfg) {
+  RHO_TRY({
+    Data3dPreproc p;
+    p.kind = Data3dPreproc::FlipX;
+    input_cfg(cfg).preprocs.push_back(p);
+  })
+}
+int rho_config_data3d_subtract_mean(rho_config* cfg, const float* mean, int64_t len) {
+  RHO_TRY({
+    RHO_REQ(mean && len == (int64_t)input_cfg(cfg).in_dims.len());
+    Data3dPreproc p;
+    p.kind = Data3dPreproc::SubtractElemwiseMean;
+    p.mean_values.assign(mean, mean + len);
+    input_cfg(cfg).preprocs.push_back(p);
+  })
+}
+int rho_config_data3d_subtract_mean_file(rho_config* cfg, const char* mean_path) {
+  RHO_TRY({
+    RHO_REQ(mean_path && *mean_path);
+    Data3dPreproc p;
+    p.kind = Data3dPreproc::SubtractElemwiseMean;
+    p.mean_path = mean_path;
+    input_cfg(cfg).preprocs.push_back(p);
+  })
+}
+int rho_config_data3d_pca_lighting_noise(rho_config* cfg, const float* singular_vecs9, const float* singular_vals3, float std_dev) {
+  RHO_TRY({
+    RHO_REQ(singular_vecs9 && singular_vals3 && std_dev >= 0.0f);
+    Data3dPreproc p;
+    p.kind = Data3dPreproc::AddPixelwisePCALightingNoise;
+    for (int i = 0; i < 3; ++i) {
+      for (int j = 0; j < 3; ++j) p.singular_vecs[i][j] = singular_vecs9[i * 3 + j];
+      p.singular_vals[i] = singular_vals3[i];
+    }
+    p.std_dev = std_dev;
+    input_cfg(cfg).preprocs.push_back(p);
+  })
+}
+int rho_config_dropout(rho_config* cfg, int32_t channels, float drop_ratio) {
+  RHO_TRY({
+    RHO_REQ(cfg && channels > 0 && drop_ratio >= 0.0f && drop_ratio <= 1.0f);
+    DropoutOperatorConfig d = {(size_t)channels, drop_ratio};
+    cfg->cfg.dropout(d);
+  })
+}
+int rho_config_local_res_norm(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t cross_size, float scale,
+                              float power, float min_div) {
+  RHO_TRY({
+    RHO_REQ(cfg && in_w > 0 && in_h > 0 && in_c > 0 && cross_size > 0 && min_div > 0.0f);
+    LocalResNormOperatorConfig l = {{(size_t)in_w, (size_t)in_h, (size_t)in_c}, (size_t)cross_size, scale, power, min_div};
+    cfg->cfg.local_res_norm(l);
   })
 }
 int rho_config_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t conv_size, int32_t conv_stride,
@@ -145,6 +215,80 @@ int rho_worker_load_frames(rho_worker* w, int32_t batch_size) {
 }
 int rho_worker_load_frames_f32(rho_worker* w, const float* host, int32_t batch_size) {
   RHO_TRY({ RHO_REQ(w && host && batch_size >= 0); w->worker->input_operator()->load_frames_f32(host, (size_t)batch_size); })
+}
+int rho_worker_input_out_dims(rho_worker* w, int32_t* out_w, int32_t* out_h, int32_t* out_c) {
+  RHO_TRY({
+    RHO_REQ(w && out_w && out_h && out_c);
+    const Dims3 d = w->worker->input_operator()->out_dims();
+    *out_w = (int32_t)d.w; *out_h = (int32_t)d.h; *out_c = (int32_t)d.c;
+  })
+}
+int rho_worker_last_preproc_draws(rho_worker* w, int32_t* crop_off_w, int32_t* crop_off_h, int* flipped, float* alphas,
+                                  int64_t alphas_cap, int64_t* alphas_len) {
+  RHO_TRY({
+    RHO_REQ(w);
+    size_t ow = 0, oh = 0;
+    bool fl = false;
+    std::vector<float> a;
+    w->worker->input_operator()->last_preproc_draws(&ow, &oh, &fl, &a);
+    if (crop_off_w) *crop_off_w = (int32_t)ow;
+    if (crop_off_h) *crop_off_h = (int32_t)oh;
+    if (flipped) *flipped = fl ? 1 : 0;
+    if (alphas_len) *alphas_len = (int64_t)a.size();
+    if (alphas) {
+      RHO_REQ(alphas_cap >= (int64_t)a.size());
+      for (size_t i = 0; i < a.size(); ++i) alphas[i] = a[i];
+    }
+  })
+}
+int rho_worker_dropout_stream(rho_worker* w, int32_t hidden_idx, uint64_t* seed, uint64_t* stream_id, uint64_t* first) {
+  RHO_TRY({
+    RHO_REQ(w && seed && stream_id && first && hidden_idx >= 0 && (size_t)hidden_idx < w->worker->hidden_count());
+    if (!w->worker->dropout_stream((size_t)hidden_idx, seed, stream_id, first)) panic("not a DropoutOperator");
+  })
+}
+static int copy_blob(const std::vector<uint8_t>& blob, uint8_t* buf, size_t cap, size_t* needed) {
+  if (needed) *needed = blob.size();
+  if (buf) {
+    if (cap < blob.size()) panic("blob buffer too small");
+    std::copy(blob.begin(), blob.end(), buf);
+  }
+  return 0;
+}
+int rho_worker_encode_params(rho_worker* w, uint8_t* buf, size_t cap, size_t* needed) {
+  RHO_TRY({ RHO_REQ(w); std::vector<uint8_t> b; w->worker->encode_params(b); copy_blob(b, buf, cap, needed); })
+}
+int rho_worker_decode_params(rho_worker* w, const uint8_t* blob, size_t len, size_t* consumed) {
+  RHO_TRY({ RHO_REQ(w && blob); const size_t n = w->worker->decode_params(blob, len); if (consumed) *consumed = n; })
+}
+int rho_worker_encode_state(rho_worker* w, uint8_t* buf, size_t cap, size_t* needed) {
+  RHO_TRY({ RHO_REQ(w); std::vector<uint8_t> b; w->worker->encode_state(b); copy_blob(b, buf, cap, needed); })
+}
+int rho_worker_decode_state(rho_worker* w, const uint8_t* blob, size_t len, size_t* consumed) {
+  RHO_TRY({ RHO_REQ(w && blob); const size_t n = w->worker->decode_state(blob, len); if (consumed) *consumed = n; })
+}
+int rho_worker_checkpoint_params(rho_worker* w, int64_t t, const char* prefix) {
+  RHO_TRY({ RHO_REQ(w && prefix && t >= 0); w->worker->checkpoint_params((size_t)t, prefix); })
+}
+int rho_worker_checkpoint_state(rho_worker* w, const char* prefix) {
+  RHO_TRY({ RHO_REQ(w && prefix); w->worker->checkpoint_state(prefix); })
+}
+int rho_worker_can_rollback(rho_worker* w, const char* prefix, int64_t* t_or_minus1) {
+  RHO_TRY({
+    RHO_REQ(w && prefix && t_or_minus1);
+    size_t t = 0;
+    *t_or_minus1 = w->worker->can_rollback(prefix, &t) ? (int64_t)t : -1;
+  })
+}
+int rho_worker_rollback_params(rho_worker* w, int64_t t_or_minus1, const char* prefix) {
+  RHO_TRY({
+    RHO_REQ(w && prefix);
+    const size_t t = (size_t)t_or_minus1;
+    w->worker->rollback_params(t_or_minus1 >= 0 ? &t : nullptr, prefix);
+  })
+}
+int rho_worker_rollback_state(rho_worker* w, const char* prefix) {
+  RHO_TRY({ RHO_REQ(w && prefix); w->worker->rollback_state(prefix); })
 }
 int rho_worker_stage_label(rho_worker* w, int32_t batch_idx, int32_t category) {
   RHO_TRY({ RHO_REQ(w && batch_idx >= 0); w->worker->loss_operator(0)->stage_label((size_t)batch_idx, category); })

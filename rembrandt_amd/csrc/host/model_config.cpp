@@ -367,6 +367,14 @@ ModelConfigFile ModelConfigFile::parse(const std::string& text) {
       if (l.pool_stride == 0 || l.pool_size == 0) panic("pool needs positive pool_size and pool_stride");
     } else if (l.type == "local_res_norm") {
       l.cross_size = req_int(node, "cross_size");
+      auto opt_float = [&](const char* key, float dflt) {
+        const TomlValue* v = node.lookup(key);
+        if (!v) return dflt;
+        return v->kind == TomlValue::Integer ? (float)v->i : (float)v->as_float();  // `min_div = 2` in the examples
+      };
+      l.lrn_scale = opt_float("scale", 1.0e-4f);
+      l.lrn_power = opt_float("power", 0.75f);
+      l.lrn_min_div = opt_float("min_div", 2.0f);
     } else if (l.type == "dropout") {
       const TomlValue* r = node.lookup("drop_ratio");
       if (!r) panic("dropout layer is missing 'drop_ratio'");
@@ -397,7 +405,17 @@ SequentialOperatorConfig ModelConfigFile::to_sequential_config() const {
   SequentialOperatorConfig cfg;
   for (const LayerEntry& l : layers) {
     if (l.type == "data") {
-      cfg.data3d({{l.crop_width, l.crop_height, l.channels}, true});
+      // frames arrive at the raw size; a smaller crop becomes the input operator's Crop step
+      Data3dOperatorConfig d = {{l.raw_width, l.raw_height, l.channels}, true, {}};
+      if (l.crop_width > l.raw_width || l.crop_height > l.raw_height) panic("data layer: crop larger than the raw frame");
+      if (l.crop_width != l.raw_width || l.crop_height != l.raw_height) {
+        Data3dPreproc p;
+        p.kind = Data3dPreproc::Crop;
+        p.crop_width = l.crop_width;
+        p.crop_height = l.crop_height;
+        d.preprocs.push_back(p);
+      }
+      cfg.data3d(d);
     } else if (l.type == "conv2d") {
       cfg.conv2d({l.in_dims, l.conv_size, l.conv_stride, l.conv_pad, l.out_channels, l.act_func, l.init_weights});
     } else if (l.type == "pool") {
@@ -405,7 +423,9 @@ SequentialOperatorConfig ModelConfigFile::to_sequential_config() const {
     } else if (l.type == "fully_conn") {
       cfg.affine({l.in_dims.len(), l.out_channels, l.act_func, l.init_weights});
     } else if (l.type == "dropout") {
-      continue;  // identity at inference; the dropout operator is outside this build
+      cfg.dropout({l.in_dims.len(), l.drop_ratio});
+    } else if (l.type == "local_res_norm") {
+      cfg.local_res_norm({l.in_dims, l.cross_size, l.lrn_scale, l.lrn_power, l.lrn_min_div});
     } else if (l.type == "softmax_loss") {
       cfg.softmax_kl_loss({l.num_categories});
     } else {

@@ -44,6 +44,7 @@ struct LayerEntry {
   ActivationFunction act_func = ActivationFunction::Identity;
   ParamsInit init_weights = ParamsInit::MakeDisabled();
   float drop_ratio = 0.0f;
+  float lrn_scale = 0.0f, lrn_power = 0.0f, lrn_min_div = 0.0f;
 };
 
 class ModelConfigFile {
@@ -51,9 +52,9 @@ class ModelConfigFile {
   std::vector<LayerEntry> layers;
   static ModelConfigFile open(const std::string& path);
   static ModelConfigFile parse(const std::string& text);
-  // Chain models only (one name per layer).  Pool layers keep the gen-1 ceil extent; dropout
-  // layers are dropped from the chain (identity at inference); a fully_conn layer takes the
-  // flattened width*height*channels of its input.
+  // Chain models only (one name per layer).  Pool layers keep the gen-1 ceil extent; a data layer whose crop
+  // is smaller than its raw frame gets a Crop step; a fully_conn layer takes the flattened
+  // width*height*channels of its input.
   SequentialOperatorConfig to_sequential_config() const;
 };
 

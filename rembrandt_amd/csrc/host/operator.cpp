@@ -1,9 +1,14 @@
 // Host-side operator layer (see operator.hpp).  Uses only the C ABI of rembrandt_hip.h.
 #include "operator.hpp"
 
+#include <sys/stat.h>
+#include <unistd.h>
+
 #include <algorithm>
 #include <cmath>
+#include <cstdio>
 #include <cstring>
+#include <fstream>
 
 namespace rembrandt {
 
@@ -38,6 +43,53 @@ Dims3 Pool2dOperatorConfig::get_out_dims() const {
   const int r = ceil_mode ? RH_ROUND_CEIL : RH_ROUND_FLOOR;
   return {(size_t)rh_pool2d_out_dim((int)in_dims.w, (int)pool_size, (int)pool_stride, (int)pool_pad, r),
           (size_t)rh_pool2d_out_dim((int)in_dims.h, (int)pool_size, (int)pool_stride, (int)pool_pad, r), in_dims.c};
+}
+
+Dims3 Data3dOperatorConfig::get_out_dims() const {
+  Dims3 out = in_dims;
+  for (const auto& p : preprocs) {
+    if (p.kind == Data3dPreproc::Crop) {
+      if (p.crop_width > out.w || p.crop_height > out.h) panic("assertion failed: crop fits the frame");
+      out = {p.crop_width, p.crop_height, out.c};
+    }
+  }
+  return out;
+}
+
+// ---- NdArray blobs ----------------------------------------------------------------------------------
+void ndarray_serialize(std::vector<uint8_t>& out, const float* data, const size_t* dims, size_t ndim) {
+  const uint8_t magic[4] = {'N', 'D', 0, 1};
+  out.insert(out.end(), magic, magic + 4);
+  const uint32_t nd = (uint32_t)ndim;
+  for (int b = 0; b < 4; ++b) out.push_back((uint8_t)(nd >> (8 * b)));
+  size_t count = 1;
+  for (size_t i = 0; i < ndim; ++i) {
+    const uint64_t d = dims[i];
+    for (int b = 0; b < 8; ++b) out.push_back((uint8_t)(d >> (8 * b)));
+    count *= dims[i];
+  }
+  const uint8_t* bytes = reinterpret_cast<const uint8_t*>(data);  // little-endian host
+  out.insert(out.end(), bytes, bytes + count * sizeof(float));
+}
+
+size_t ndarray_deserialize(const uint8_t* blob, size_t len, std::vector<size_t>* dims, std::vector<float>* data) {
+  if (len < 8 || blob[0] != 'N' || blob[1] != 'D' || blob[2] != 0 || blob[3] != 1) panic("NdArray: bad magic");
+  uint32_t nd = 0;
+  for (int b = 0; b < 4; ++b) nd |= (uint32_t)blob[4 + b] << (8 * b);
+  if (nd == 0 || nd > 8 || len < 8 + 8 * (size_t)nd) panic("NdArray: bad rank or truncated header");
+  dims->clear();
+  size_t count = 1, off = 8;
+  for (uint32_t i = 0; i < nd; ++i, off += 8) {
+    uint64_t d = 0;
+    for (int b = 0; b < 8; ++b) d |= (uint64_t)blob[off + b] << (8 * b);
+    if (d != 0 && count > (size_t)1 << 40) panic("NdArray: dimensions overflow");
+    dims->push_back((size_t)d);
+    count *= (size_t)d;
+  }
+  if (len - off < count * sizeof(float)) panic("NdArray: truncated data");
+  data->resize(count);
+  if (count) std::memcpy(data->data(), blob + off, count * sizeof(float));
+  return off + count * sizeof(float);
 }
 
 size_t OperatorConfig::params_len() const {
@@ -81,6 +133,20 @@ SequentialOperatorConfig& SequentialOperatorConfig::pool2d(const Pool2dOperatorC
   hidden_ops.push_back(c);
   return *this;
 }
+SequentialOperatorConfig& SequentialOperatorConfig::dropout(const DropoutOperatorConfig& cfg) {
+  OperatorConfig c = OperatorConfig();
+  c.kind = OperatorConfig::Dropout;
+  c.dropout = cfg;
+  hidden_ops.push_back(c);
+  return *this;
+}
+SequentialOperatorConfig& SequentialOperatorConfig::local_res_norm(const LocalResNormOperatorConfig& cfg) {
+  OperatorConfig c = OperatorConfig();
+  c.kind = OperatorConfig::LocalResNorm;
+  c.lrn = cfg;
+  hidden_ops.push_back(c);
+  return *this;
+}
 SequentialOperatorConfig& SequentialOperatorConfig::softmax_kl_loss(const CategoricalLossConfig& cfg) {
   loss_op = OperatorConfig();
   loss_op.kind = OperatorConfig::SoftmaxKLLoss;
@@ -99,10 +165,12 @@ struct ParamTensors {
   // backward-capable operators only
   std::unique_ptr<DeviceBuffer<float>> grad_weights, grad_bias, acc_grad_weights, acc_grad_bias, save_weights, save_bias;
   size_t wlen = 0, blen = 0;
+  size_t wrows = 0, wcols = 0;  // bound of the weights as the reference's Array2d: (in or R*S*C, out), first index fastest
   Ctx ctx;
 
   void alloc(size_t wl, size_t bl, bool backward, Ctx c) {
     wlen = wl; blen = bl; ctx = c;
+    wcols = bl; wrows = bl ? wl / bl : 0;
     weights.reset(new DeviceBuffer<float>(wl, c));
     bias.reset(new DeviceBuffer<float>(bl, c));
     if (backward) {
@@ -202,6 +270,36 @@ struct ParamTensors {
     weights->sync_load(w.data(), wlen);
     bias->sync_load(b.data(), blen);
   }
+  void encode_pair(std::vector<uint8_t>& blob, const DeviceBuffer<float>& w, const DeviceBuffer<float>& b) const {
+    ctx->sync();
+    std::vector<float> hw(wlen), hb(blen);
+    w.sync_store(hw.data(), wlen);
+    b.sync_store(hb.data(), blen);
+    const size_t wd[2] = {wrows, wcols}, bd[2] = {1, blen};
+    ndarray_serialize(blob, hw.data(), wd, 2);
+    ndarray_serialize(blob, hb.data(), bd, 2);
+  }
+  size_t decode_pair(const uint8_t* blob, size_t len, DeviceBuffer<float>& w, DeviceBuffer<float>& b, const char* who) {
+    std::vector<size_t> dims;
+    std::vector<float> data;
+    size_t off = ndarray_deserialize(blob, len, &dims, &data);
+    if (dims.size() != 2 || dims[0] != wrows || dims[1] != wcols) panic(std::string(who) + ": weights blob has the wrong bound");
+    w.sync_load(data.data(), wlen);
+    off += ndarray_deserialize(blob + off, len - off, &dims, &data);
+    if (dims.size() != 2 || dims[0] != 1 || dims[1] != blen) panic(std::string(who) + ": bias blob has the wrong bound");
+    b.sync_load(data.data(), blen);
+    return off;
+  }
+  void encode_params(std::vector<uint8_t>& blob) const { encode_pair(blob, *weights, *bias); }
+  size_t decode_params(const uint8_t* blob, size_t len, const char* who) { return decode_pair(blob, len, *weights, *bias, who); }
+  void encode_state(std::vector<uint8_t>& blob) const {
+    RB_ASSERT(has_backward());
+    encode_pair(blob, *acc_grad_weights, *acc_grad_bias);
+  }
+  size_t decode_state(const uint8_t* blob, size_t len, const char* who) {
+    RB_ASSERT(has_backward());
+    return decode_pair(blob, len, *acc_grad_weights, *acc_grad_bias, who);
+  }
   bool buffer(int which, float** ptr, size_t* len) {
     DeviceBuffer<float>* b = nullptr;
     switch (which) {
@@ -242,17 +340,69 @@ void apply_rect_backprop(ActivationFunction f, const float* y, size_t frame_len,
   }
 }
 
-// ---- Data3dOperator (minimal: u8 staging + cast, or fp32 frames) ------------------------------------------
+// xorshift128+ for per-operator seed derivation (Xorshiftplus128Rng in src/operator/worker.rs:361-367) and the
+// input operator's crop / flip draws (src/operator/mod.rs:503,619); the reference's bit streams are not reproducible here.
+struct Xorshiftplus128 {
+  uint64_t s0, s1;
+  explicit Xorshiftplus128(const uint64_t seed[2]) : s0(seed[0]), s1(seed[1]) {
+    if (s0 == 0 && s1 == 0) s1 = 0x9E3779B97F4A7C15ull;
+  }
+  uint64_t next_u64() {
+    uint64_t x = s0;
+    const uint64_t y = s1;
+    s0 = y;
+    x ^= x << 23;
+    s1 = x ^ y ^ (x >> 17) ^ (y >> 26);
+    return s1 + y;
+  }
+};
+
+
+// ---- Data3dOperator ---------------------------------------------------------------------------------------
+// u8 staging -> H2D -> cast (optionally /255) -> preprocessing steps ping-ponging between tmp_buf and out_buf so
+// that the last one lands in out_buf (src/operator/mod.rs:640-790).  Crop offsets and the flip coin are drawn
+// once per forward() for the whole batch, as in the reference; Inference uses the centre crop and no flip/noise.
 class Data3dOperator : public InputOperator {
  public:
-  Data3dOperator(size_t batch_size, const Data3dOperatorConfig& config, Ctx context)
+  Data3dOperator(size_t batch_size, const Data3dOperatorConfig& config, Ctx context, const uint64_t seed[2])
       : batch_cap_(batch_size), config_(config), context_(context),
         in_buf_h_(batch_size * config.in_dims.len(), 0),
         in_buf_(new DeviceBuffer<uint8_t>(batch_size * config.in_dims.len(), context)),
-        out_buf_(new DeviceBuffer<float>(batch_size * config.in_dims.len(), context)) {}
+        out_buf_(new DeviceBuffer<float>(batch_size * config.in_dims.len(), context)),
+        rng_(seed), noise_seed_(seed[0] ^ 0x5043414Eull) {
+    (void)config_.get_out_dims();  // asserts that every crop fits
+    if (!config.preprocs.empty()) tmp_buf_.reset(new DeviceBuffer<float>(batch_size * config.in_dims.len(), context));
+    for (const auto& p : config.preprocs) {
+      PreprocState st;
+      if (p.kind == Data3dPreproc::SubtractElemwiseMean) {
+        std::vector<float> mean = p.mean_values;
+        if (!p.mean_path.empty()) {
+          std::ifstream f(p.mean_path, std::ios::binary);
+          if (!f) panic("failed to open mean path: " + p.mean_path);
+          std::vector<uint8_t> blob((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+          std::vector<size_t> dims;
+          ndarray_deserialize(blob.data(), blob.size(), &dims, &mean);
+        }
+        if (mean.size() != config.in_dims.len()) panic("failed to deserialize mean array: wrong length");
+        st.dev.reset(new DeviceBuffer<float>(mean.size(), context));
+        st.dev->sync_load(mean.data(), mean.size());
+      } else if (p.kind == Data3dPreproc::AddPixelwisePCALightingNoise) {
+        RB_ASSERT(config.in_dims.c == 3);
+        // [svecs: 9][svals: 3][alphas: 3*batch]
+        st.dev.reset(new DeviceBuffer<float>(12 + 3 * batch_size, context));
+        float h[12];
+        for (int i = 0; i < 3; ++i)
+          for (int j = 0; j < 3; ++j) h[i * 3 + j] = p.singular_vecs[i][j];
+        for (int j = 0; j < 3; ++j) h[9 + j] = p.singular_vals[j];
+        st.dev->sync_load(h, 12);
+      }
+      states_.push_back(std::move(st));
+    }
+  }
   size_t batch_size() const override { return batch_cap_; }
   SharedDeviceBuf get_output_vars() const override { return out_buf_; }
   SharedDeviceBuf get_output_deltas() const override { return nullptr; }  // src/operator/mod.rs:632-634
+  Dims3 out_dims() const override { return config_.get_out_dims(); }
   uint8_t* expose_host_frame_buf(size_t batch_idx) override {
     RB_ASSERT(batch_idx < batch_cap_);
     return in_buf_h_.data() + batch_idx * config_.in_dims.len();
@@ -260,20 +410,101 @@ class Data3dOperator : public InputOperator {
   void load_frames(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
     in_buf_->sync_load(in_buf_h_.data(), in_buf_h_.size());
+    f32_loaded_ = false;
   }
   void load_frames_f32(const float* host, size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
-    out_buf_->sync_load(host, batch_size * config_.in_dims.len());
+    const size_t n = batch_size * config_.in_dims.len();
+    if (config_.preprocs.empty()) {
+      out_buf_->sync_load(host, n);  // frames are placed where the cast would put them
+    } else {
+      if (!f32_frames_) f32_frames_.reset(new DeviceBuffer<float>(batch_cap_ * config_.in_dims.len(), context_));
+      f32_frames_->sync_load(host, n);
+    }
     f32_loaded_ = true;
   }
-  void forward(size_t batch_size, OpPhase) override {
+  void forward(size_t batch_size, OpPhase phase) override {
     RB_ASSERT(batch_size <= batch_cap_);
-    if (f32_loaded_) return;  // frames were placed in out_buf directly
-    const size_t n = batch_size * config_.in_dims.len();
-    unwrap(rh_cast_u8_f32(in_buf_->as_ptr(), out_buf_->as_mut_ptr(), n, config_.normalize ? 1.0f / 255.0f : 1.0f,
-                          context_->stream()), "cast_bytes");
+    rh_stream_t s = context_->stream();
+    const size_t num_preprocs = config_.preprocs.size();
+    const size_t in_len = batch_size * config_.in_dims.len();
+    float* const out = out_buf_->as_mut_ptr();
+    float* const tmp = tmp_buf_ ? tmp_buf_->as_mut_ptr() : nullptr;
+    float* cur = num_preprocs % 2 == 0 ? out : tmp;
+    if (f32_loaded_) {
+      if (num_preprocs) unwrap(rh_copy_d2d(cur, f32_frames_->as_ptr(), in_len * sizeof(float), s), "send");
+    } else {
+      unwrap(rh_cast_u8_f32(in_buf_->as_ptr(), cur, in_len, config_.normalize ? 1.0f / 255.0f : 1.0f, s), "cast_bytes");
+    }
+    Dims3 dims = config_.in_dims;
+    last_alphas_.clear();
+    last_flip_ = false;
+    for (size_t r = 0; r < num_preprocs; ++r) {
+      const Data3dPreproc& p = config_.preprocs[r];
+      float* const dst = cur == out ? tmp : out;
+      const size_t len = batch_size * dims.len();
+      switch (p.kind) {
+        case Data3dPreproc::Crop: {
+          size_t off_w, off_h;
+          if (phase.training) {  // uniform over [0, max_offset] (src/operator/mod.rs:553-569, 681-685)
+            off_w = (size_t)(rng_.next_u64() % (uint64_t)(dims.w - p.crop_width + 1));
+            off_h = (size_t)(rng_.next_u64() % (uint64_t)(dims.h - p.crop_height + 1));
+          } else {
+            off_w = (dims.w - p.crop_width) / 2;
+            off_h = (dims.h - p.crop_height) / 2;
+          }
+          last_off_w_ = off_w;
+          last_off_h_ = off_h;
+          unwrap(rh_crop_nchw(cur, dst, (int64_t)(batch_size * dims.c), (int)dims.w, (int)dims.h, (int)p.crop_width,
+                              (int)p.crop_height, (int)off_w, (int)off_h, s), "crop transform");
+          dims = {p.crop_width, p.crop_height, dims.c};
+          break;
+        }
+        case Data3dPreproc::FlipX: {
+          const bool flip = phase.training && (rng_.next_u64() & 1);
+          last_flip_ = flip;
+          if (flip) {
+            rembrandt_kernel_batch_blockmap256_flip(cur, (int32_t)dims.w, (int32_t)(dims.h * dims.c * batch_size), dst, s);
+            unwrap_last("rembrandt_kernel_batch_blockmap256_flip");
+          } else {
+            unwrap(rh_copy_d2d(dst, cur, len * sizeof(float), s), "send");
+          }
+          break;
+        }
+        case Data3dPreproc::SubtractElemwiseMean: {
+          RB_ASSERT(dims.len() == config_.in_dims.len());  // the mean has the input frame's shape
+          const float alpha = config_.normalize ? -1.0f / 255.0f : -1.0f;
+          unwrap(rh_copy_d2d(dst, cur, len * sizeof(float), s), "send");
+          unwrap(rh_add_bias_nchw(states_[r].dev->as_ptr(), dst, 1, (int32_t)dims.len(), (int32_t)batch_size, alpha, 1.0f, s),
+                 "subtract mean");
+          break;
+        }
+        case Data3dPreproc::AddPixelwisePCALightingNoise: {
+          if (phase.training) {
+            last_alphas_.resize(3 * batch_size);
+            unwrap(rh_rng_fill_normal(noise_seed_, noise_draws_++, last_alphas_.data(), last_alphas_.size(), 0.0f, p.std_dev),
+                   "sample alphas");
+            float* base = states_[r].dev->as_mut_ptr();
+            unwrap(rh_load_sync(context_->raw(), base + 12, last_alphas_.data(), last_alphas_.size() * sizeof(float)), "sync_load");
+            rembrandt_kernel_batch_map_preproc_pca3_noise(cur, (int32_t)(dims.w * dims.h), (int32_t)batch_size, base + 12,
+                                                          base + 9, base, dst, s);
+            unwrap_last("rembrandt_kernel_batch_map_preproc_pca3_noise");
+          } else {
+            unwrap(rh_copy_d2d(dst, cur, len * sizeof(float), s), "send");
+          }
+          break;
+        }
+      }
+      cur = dst;
+    }
   }
   void backward(size_t) override {}
+  void last_preproc_draws(size_t* crop_off_w, size_t* crop_off_h, bool* flipped, std::vector<float>* alphas) const override {
+    if (crop_off_w) *crop_off_w = last_off_w_;
+    if (crop_off_h) *crop_off_h = last_off_h_;
+    if (flipped) *flipped = last_flip_;
+    if (alphas) *alphas = last_alphas_;
+  }
   bool buffer(int which, float** ptr, size_t* len) override {
     if (which != 0) return false;
     *ptr = out_buf_->as_mut_ptr();
@@ -283,12 +514,22 @@ class Data3dOperator : public InputOperator {
   const char* kind() const override { return "Data3dOperator"; }
 
  private:
+  struct PreprocState {
+    std::unique_ptr<DeviceBuffer<float>> dev;
+  };
   size_t batch_cap_;
   Data3dOperatorConfig config_;
   Ctx context_;
   std::vector<uint8_t> in_buf_h_;
   std::unique_ptr<DeviceBuffer<uint8_t>> in_buf_;
+  std::unique_ptr<DeviceBuffer<float>> tmp_buf_, f32_frames_;
   SharedDeviceBuf out_buf_;
+  std::vector<PreprocState> states_;
+  Xorshiftplus128 rng_;
+  uint64_t noise_seed_, noise_draws_ = 0;
+  size_t last_off_w_ = 0, last_off_h_ = 0;
+  bool last_flip_ = false;
+  std::vector<float> last_alphas_;
   bool f32_loaded_ = false;
 };
 
@@ -354,6 +595,10 @@ class AffineOperator : public Operator {
   void save_params() override { params_.save_params(); }
   void restore_params() override { params_.restore_params(); }
   void reset() override { params_.reset(); }
+  void encode_params(std::vector<uint8_t>& blob) override { params_.encode_params(blob); }
+  size_t decode_params(const uint8_t* blob, size_t len) override { return params_.decode_params(blob, len, kind()); }
+  void encode_state(std::vector<uint8_t>& blob) override { params_.encode_state(blob); }
+  size_t decode_state(const uint8_t* blob, size_t len) override { return params_.decode_state(blob, len, kind()); }
   void fused_sgd_step(float l2, float scale, float mu, float apply) override { params_.fused_sgd_step(l2, scale, mu, apply); }
   bool buffer(int which, float** ptr, size_t* len) override {
     if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
@@ -448,6 +693,10 @@ class Conv2dOperator : public Operator {
   void save_params() override { params_.save_params(); }
   void restore_params() override { params_.restore_params(); }
   void reset() override { params_.reset(); }
+  void encode_params(std::vector<uint8_t>& blob) override { params_.encode_params(blob); }
+  size_t decode_params(const uint8_t* blob, size_t len) override { return params_.decode_params(blob, len, kind()); }
+  void encode_state(std::vector<uint8_t>& blob) override { params_.encode_state(blob); }
+  size_t decode_state(const uint8_t* blob, size_t len) override { return params_.decode_state(blob, len, kind()); }
   void fused_sgd_step(float l2, float scale, float mu, float apply) override { params_.fused_sgd_step(l2, scale, mu, apply); }
   bool buffer(int which, float** ptr, size_t* len) override {
     if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
@@ -529,6 +778,118 @@ class Pool2dOperator : public Operator {
   Dims3 out_dims_;
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   std::unique_ptr<DeviceBuffer<int32_t>> argmax_;
+};
+
+// ---- DropoutOperator (src/operator/mod.rs:2134-2255) -------------------------------------------------------
+// Training: rand_samples <- uniform [0,1) from the device generator, mask = rand > drop_ratio, out = in * mask
+// (scale argument 1.0: no rescaling, as the reference passes it); Inference: a copy.
+class DropoutOperator : public Operator {
+ public:
+  DropoutOperator(size_t batch_size, const DropoutOperatorConfig& config, const Operator* prev_op, Ctx context,
+                  uint64_t seed, uint64_t stream_id)
+      : batch_cap_(batch_size), config_(config), context_(context), seed_(seed), stream_id_(stream_id),
+        rand_samples_(config.channels * batch_size, context), drop_mask_(config.channels * batch_size, context) {
+    RB_ASSERT(prev_op != nullptr);
+    in_act_ = prev_op->get_output_vars();
+    if (!in_act_) panic("DropoutOperator missing required prev operator output vars");
+    in_delta_ = prev_op->get_output_deltas();
+    RB_ASSERT(in_act_->len() >= config.channels * batch_size);
+    out_act_.reset(new DeviceBuffer<float>(config.channels * batch_size, context));
+    out_delta_.reset(new DeviceBuffer<float>(config.channels * batch_size, context));
+  }
+  size_t batch_size() const override { return batch_cap_; }
+  SharedDeviceBuf get_output_vars() const override { return out_act_; }
+  SharedDeviceBuf get_output_deltas() const override { return out_delta_; }
+  void forward(size_t batch_size, OpPhase phase) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    rh_stream_t s = context_->stream();
+    const size_t n = config_.channels * batch_size;
+    if (!phase.training) {
+      unwrap(rh_copy_d2d(out_act_->as_mut_ptr(), in_act_->as_ptr(), n * sizeof(float), s), "send");
+      return;
+    }
+    last_first_ = next_first_;
+    unwrap(rh_rng_fill_uniform01_device(seed_, stream_id_, next_first_, rand_samples_.as_mut_ptr(), n, s), "sample");
+    next_first_ += n;
+    rembrandt_kernel_map_dropout(in_act_->as_ptr(), (int32_t)n, config_.drop_ratio, 1.0f, rand_samples_.as_ptr(),
+                                 out_act_->as_mut_ptr(), drop_mask_.as_mut_ptr(), s);
+    unwrap_last("rembrandt_kernel_map_dropout");
+  }
+  void backward(size_t batch_size) override {
+    if (!in_delta_) return;
+    RB_ASSERT(batch_size <= batch_cap_);
+    rembrandt_kernel_map_dropout_backprop(out_delta_->as_ptr(), (int32_t)(config_.channels * batch_size), config_.drop_ratio,
+                                          1.0f, drop_mask_.as_ptr(), in_delta_->as_mut_ptr(), context_->stream());
+    unwrap_last("rembrandt_kernel_map_dropout_backprop");
+  }
+  bool buffer(int which, float** ptr, size_t* len) override {
+    if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
+    if (which == 1) { *ptr = out_delta_->as_mut_ptr(); *len = out_delta_->len(); return true; }
+    return false;
+  }
+  void stream(uint64_t* seed, uint64_t* stream_id, uint64_t* first) const {
+    *seed = seed_; *stream_id = stream_id_; *first = last_first_;
+  }
+  const char* kind() const override { return "DropoutOperator"; }
+
+ private:
+  size_t batch_cap_;
+  DropoutOperatorConfig config_;
+  Ctx context_;
+  uint64_t seed_, stream_id_, next_first_ = 0, last_first_ = 0;
+  SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
+  DeviceBuffer<float> rand_samples_;
+  DeviceBuffer<int32_t> drop_mask_;
+};
+
+// ---- LocalResNormOperator: cross-channel response normalisation (no counterpart operator in the reference) ----
+class LocalResNormOperator : public Operator {
+ public:
+  LocalResNormOperator(size_t batch_size, const LocalResNormOperatorConfig& config, const Operator* prev_op, Ctx context)
+      : batch_cap_(batch_size), config_(config), context_(context), denom_(config.in_dims.len() * batch_size, context) {
+    RB_ASSERT(prev_op != nullptr);
+    in_act_ = prev_op->get_output_vars();
+    if (!in_act_) panic("LocalResNormOperator missing required prev operator output vars");
+    in_delta_ = prev_op->get_output_deltas();
+    RB_ASSERT(in_act_->len() >= config.in_dims.len() * batch_size);
+    RB_ASSERT(config.cross_size > 0 && config.min_div > 0.0f);
+    out_act_.reset(new DeviceBuffer<float>(config.in_dims.len() * batch_size, context));
+    out_delta_.reset(new DeviceBuffer<float>(config.in_dims.len() * batch_size, context));
+  }
+  size_t batch_size() const override { return batch_cap_; }
+  SharedDeviceBuf get_output_vars() const override { return out_act_; }
+  SharedDeviceBuf get_output_deltas() const override { return out_delta_; }
+  void forward(size_t batch_size, OpPhase) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    const rh_lrn_geom g = geom(batch_size);
+    unwrap(rh_lrn_fwd(&g, in_act_->as_ptr(), out_act_->as_mut_ptr(), denom_.as_mut_ptr(), context_->stream()), "lrn forward");
+  }
+  void backward(size_t batch_size) override {
+    if (!in_delta_) return;
+    RB_ASSERT(batch_size <= batch_cap_);
+    const rh_lrn_geom g = geom(batch_size);
+    unwrap(rh_lrn_bwd(&g, in_act_->as_ptr(), out_act_->as_ptr(), denom_.as_ptr(), out_delta_->as_ptr(),
+                      in_delta_->as_mut_ptr(), context_->stream()), "lrn backward");
+  }
+  bool buffer(int which, float** ptr, size_t* len) override {
+    if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
+    if (which == 1) { *ptr = out_delta_->as_mut_ptr(); *len = out_delta_->len(); return true; }
+    return false;
+  }
+  const char* kind() const override { return "LocalResNormOperator"; }
+
+ private:
+  rh_lrn_geom geom(size_t batch) const {
+    rh_lrn_geom g;
+    g.N = (int)batch; g.C = (int)config_.in_dims.c; g.H = (int)config_.in_dims.h; g.W = (int)config_.in_dims.w;
+    g.size = (int)config_.cross_size; g.scale = config_.scale; g.power = config_.power; g.min_div = config_.min_div;
+    return g;
+  }
+  size_t batch_cap_;
+  LocalResNormOperatorConfig config_;
+  Ctx context_;
+  SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
+  DeviceBuffer<float> denom_;
 };
 
 // ---- SoftmaxKLLossOperator ------------------------------------------------------------------------------
@@ -626,23 +987,6 @@ class SoftmaxKLLossOperator : public LossOperator {
   DeviceBuffer<float> out_loss1_, out_loss_;
 };
 
-// xorshift128+ used only to derive per-operator seeds from the shared seed
-// (Xorshiftplus128Rng in src/operator/worker.rs:361-367; its bit stream is not reproducible here).
-struct Xorshiftplus128 {
-  uint64_t s0, s1;
-  explicit Xorshiftplus128(const uint64_t seed[2]) : s0(seed[0]), s1(seed[1]) {
-    if (s0 == 0 && s1 == 0) s1 = 0x9E3779B97F4A7C15ull;
-  }
-  uint64_t next_u64() {
-    uint64_t x = s0;
-    const uint64_t y = s1;
-    s0 = y;
-    x ^= x << 23;
-    s1 = x ^ y ^ (x >> 17) ^ (y >> 26);
-    return s1 + y;
-  }
-};
-
 }  // namespace
 
 // ---- SequentialOperatorWorker ---------------------------------------------------------------------------
@@ -655,7 +999,8 @@ SequentialOperatorWorker::SequentialOperatorWorker(const SequentialOperatorConfi
   RB_ASSERT(batch_size > 0);
   if (!config.has_input || config.input_op.kind != OperatorConfig::Data3d) panic("SequentialOperatorWorker: missing input operator");
   if (!config.has_loss) panic("SequentialOperatorWorker: missing loss operator");
-  input_op_.reset(new Data3dOperator(batch_size, config.input_op.data3d, context));
+  const uint64_t input_seed[2] = {shared_seed[0] ^ 0x44617461336421ull, shared_seed[1] + 0x9E3779B97F4A7C15ull};
+  input_op_.reset(new Data3dOperator(batch_size, config.input_op.data3d, context, input_seed));
   const Operator* prev = input_op_.get();
   size_t params_off = 0;
   for (const auto& c : config.hidden_ops) {
@@ -664,6 +1009,11 @@ SequentialOperatorWorker::SequentialOperatorWorker(const SequentialOperatorConfi
       case OperatorConfig::Affine: op.reset(new AffineOperator(batch_size, capability, c.affine, prev, context)); break;
       case OperatorConfig::Conv2d: op.reset(new Conv2dOperator(batch_size, capability, c.conv2d, prev, context, opts)); break;
       case OperatorConfig::Pool2d: op.reset(new Pool2dOperator(batch_size, c.pool2d, prev, context)); break;
+      case OperatorConfig::Dropout:
+        op.reset(new DropoutOperator(batch_size, c.dropout, prev, context, shared_seed[0] ^ (shared_seed[1] << 32 | shared_seed[1] >> 32),
+                                     0xD0000000ull + hidden_ops_.size()));
+        break;
+      case OperatorConfig::LocalResNorm: op.reset(new LocalResNormOperator(batch_size, c.lrn, prev, context)); break;
       default: panic("SequentialOperatorWorker: not a hidden operator");
     }
     params_off += c.params_len();
@@ -705,6 +1055,117 @@ void SequentialOperatorWorker::restore_params() { for (auto& op : hidden_ops_) o
 void SequentialOperatorWorker::reset() { for (auto& op : hidden_ops_) op->reset(); }
 void SequentialOperatorWorker::fused_sgd_step(float l2, float scale, float mu, float apply) {
   for (auto& op : hidden_ops_) op->fused_sgd_step(l2, scale, mu, apply);
+}
+
+void SequentialOperatorWorker::encode_params(std::vector<uint8_t>& blob) { for (auto& op : hidden_ops_) op->encode_params(blob); }
+size_t SequentialOperatorWorker::decode_params(const uint8_t* blob, size_t len) {
+  size_t off = 0;
+  for (auto& op : hidden_ops_) off += op->decode_params(blob + off, len - off);
+  return off;
+}
+void SequentialOperatorWorker::encode_state(std::vector<uint8_t>& blob) {
+  for (auto& op : hidden_ops_) {  // params then momentum, operator by operator (gossip_dist.rs:1287-1291)
+    op->encode_params(blob);
+    op->encode_state(blob);
+  }
+}
+size_t SequentialOperatorWorker::decode_state(const uint8_t* blob, size_t len) {
+  size_t off = 0;
+  for (auto& op : hidden_ops_) {
+    off += op->decode_params(blob + off, len - off);
+    off += op->decode_state(blob + off, len - off);
+  }
+  return off;
+}
+
+namespace {
+void make_dirs(const std::string& path) {  // create_dir_all; errors ignored as in the reference
+  std::string cur;
+  for (size_t i = 0; i <= path.size(); ++i) {
+    if (i == path.size() || path[i] == '/') {
+      if (!cur.empty()) ::mkdir(cur.c_str(), 0777);
+    }
+    if (i < path.size()) cur.push_back(path[i]);
+  }
+}
+void write_file(const std::string& path, const std::vector<uint8_t>& blob, const char* who) {
+  std::ofstream f(path, std::ios::binary | std::ios::trunc);
+  if (!f) panic(std::string(who) + ": failed to open blob file: " + path);
+  f.write(reinterpret_cast<const char*>(blob.data()), (std::streamsize)blob.size());
+  if (!f) panic(std::string(who) + ": failed to write to blob file: " + path);
+}
+std::vector<uint8_t> read_file(const std::string& path, const char* who) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) panic(std::string(who) + ": failed to open blob file: " + path);
+  return std::vector<uint8_t>((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+}
+}  // namespace
+
+void SequentialOperatorWorker::checkpoint_params(size_t t, const std::string& prefix) {
+  make_dirs(prefix);
+  std::vector<uint8_t> blob;
+  encode_params(blob);
+  const std::string name = "params.t_" + std::to_string(t) + ".blob";
+  write_file(prefix + "/" + name, blob, "checkpoint_params");
+  const std::string latest = prefix + "/params.latest.blob";
+  ::unlink(latest.c_str());
+  if (::symlink(name.c_str(), latest.c_str()) != 0) panic("checkpoint_params: failed to symlink latest blob");
+  const std::string ck = prefix + "/checkpoint";
+  {
+    std::ifstream old(ck, std::ios::binary);
+    if (old) {
+      std::ofstream bak(prefix + "/checkpoint.0", std::ios::binary | std::ios::trunc);
+      bak << old.rdbuf();
+    }
+  }
+  std::ofstream f(ck, std::ios::trunc);
+  if (!f) panic("checkpoint_params: failed to open checkpoint file");
+  f << t << "\n";
+}
+
+void SequentialOperatorWorker::checkpoint_state(const std::string& prefix) {
+  make_dirs(prefix);
+  std::vector<uint8_t> blob;
+  encode_state(blob);
+  write_file(prefix + "/state.latest.blob." + std::to_string(worker_rank()), blob, "checkpoint_state");
+}
+
+bool SequentialOperatorWorker::can_rollback(const std::string& prefix, size_t* t) const {
+  std::ifstream f(prefix + "/checkpoint");
+  if (!f) return false;
+  std::string line;
+  if (!std::getline(f, line)) return false;
+  char* end = nullptr;
+  const unsigned long long v = std::strtoull(line.c_str(), &end, 10);
+  if (end == line.c_str()) return false;
+  if (t) *t = (size_t)v;
+  return true;
+}
+
+void SequentialOperatorWorker::rollback_params(const size_t* t, const std::string& prefix) {
+  std::string path;
+  if (t) {
+    size_t latest = 0;
+    if (!can_rollback(prefix, &latest)) panic("rollback_params: checkpoint file is missing or empty, but requested iter " + std::to_string(*t));
+    RB_ASSERT(*t <= latest);
+    path = prefix + "/params.t_" + std::to_string(*t) + ".blob";
+  } else {
+    path = prefix + "/params.latest.blob";
+  }
+  const std::vector<uint8_t> blob = read_file(path, "rollback_params");
+  decode_params(blob.data(), blob.size());
+}
+
+void SequentialOperatorWorker::rollback_state(const std::string& prefix) {
+  const std::vector<uint8_t> blob = read_file(prefix + "/state.latest.blob." + std::to_string(worker_rank()), "rollback_state");
+  decode_state(blob.data(), blob.size());
+}
+
+bool SequentialOperatorWorker::dropout_stream(size_t hidden_idx, uint64_t* seed, uint64_t* stream_id, uint64_t* first) const {
+  const DropoutOperator* d = dynamic_cast<const DropoutOperator*>(hidden_ops_.at(hidden_idx).get());
+  if (!d) return false;
+  d->stream(seed, stream_id, first);
+  return true;
 }
 
 // ---- SGD policy -----------------------------------------------------------------------------------------

@@ -5,7 +5,10 @@
 //   Operator / InputOperator traits ........ src/operator/mod.rs:61-109
 //   OpCapability, OpPhase, Regularization,
 //   ActivationFunction, ParamsInit ......... src/operator/mod.rs:233-297
-//   Data3dOperator (minimal) ............... src/operator/mod.rs:491-836
+//   Data3dOperator + preprocessing ......... src/operator/mod.rs:395-836
+//   DropoutOperator ........................ src/operator/mod.rs:2134-2255
+//   encode/decode_params/state ............. src/operator/mod.rs:1008-1073, 1594-1661
+//   checkpoint / rollback files ............ src/worker/gossip_dist.rs:1230-1413
 //   AffineOperator ......................... src/operator/mod.rs:843-1364
 //   Conv2dOperator ......................... src/operator/mod.rs:1366-2003
 //   Pool2dOperator ......................... src/operator/mod.rs:2005-2132
@@ -110,9 +113,23 @@ struct Dims3 {  // (width, height, channels), as in the reference
 };
 
 // ---- operator configs ---------------------------------------------------------------------------
+// Data3dPreproc (src/operator/mod.rs:395-423).  AddPixelwiseColorNoise and NormalizePixelwise are
+// `unimplemented!()` in the reference and are not offered here.
+struct Data3dPreproc {
+  enum Kind { Crop, FlipX, SubtractElemwiseMean, AddPixelwisePCALightingNoise } kind;
+  size_t crop_width = 0, crop_height = 0;      // Crop
+  std::string mean_path;                       // SubtractElemwiseMean: an NdArray file of in_dims ...
+  std::vector<float> mean_values;              // ... or the values themselves (in_dims.len() floats, W fastest)
+  float singular_vecs[3][3] = {{0}};           // AddPixelwisePCALightingNoise
+  float singular_vals[3] = {0};
+  float std_dev = 0.0f;
+};
+
 struct Data3dOperatorConfig {
   Dims3 in_dims;
   bool normalize;  // u8 frames are scaled by 1/255 when set (cast_bytes_normalized)
+  std::vector<Data3dPreproc> preprocs;
+  Dims3 get_out_dims() const;  // src/operator/mod.rs:432-462
 };
 
 struct AffineOperatorConfig {
@@ -140,17 +157,32 @@ struct Pool2dOperatorConfig {
   Dims3 get_out_dims() const;
 };
 
+struct DropoutOperatorConfig {  // src/operator/mod.rs:2134-2138
+  size_t channels;
+  float drop_ratio;
+};
+
+// The `local_res_norm` layer type of the `.model` grammar (examples/imagenet_alexnet.model:31-37); the
+// reference's own layer for it is an empty stub (src/layer.rs:1846-1899).
+struct LocalResNormOperatorConfig {
+  Dims3 in_dims;
+  size_t cross_size;
+  float scale, power, min_div;
+};
+
 struct CategoricalLossConfig {
   size_t num_categories;
 };
 
 struct OperatorConfig {
-  enum Kind { Data3d, Affine, Conv2d, Pool2d, SoftmaxKLLoss } kind;
+  enum Kind { Data3d, Affine, Conv2d, Pool2d, SoftmaxKLLoss, Dropout, LocalResNorm } kind;
   Data3dOperatorConfig data3d;
   AffineOperatorConfig affine;
   Conv2dOperatorConfig conv2d;
   Pool2dOperatorConfig pool2d;
   CategoricalLossConfig loss;
+  DropoutOperatorConfig dropout;
+  LocalResNormOperatorConfig lrn;
   size_t params_len() const;
 };
 
@@ -181,6 +213,12 @@ class Operator {
   // Fused regularize -> accumulate_grads(scale, momentum) -> update_params(apply) -> reset in
   // one pass per tensor (same arithmetic, 24 instead of 52 bytes per parameter).
   virtual void fused_sgd_step(float /*l2*/, float /*scale*/, float /*momentum*/, float /*apply*/) {}
+  // Parameter / optimizer-state blobs: a sequence of serialised NdArrays (weights then bias; for the state the
+  // momentum buffers).  decode_* return the number of bytes consumed (src/operator/mod.rs:1008-1073).
+  virtual void encode_params(std::vector<uint8_t>& /*blob*/) {}
+  virtual size_t decode_params(const uint8_t* /*blob*/, size_t /*len*/) { return 0; }
+  virtual void encode_state(std::vector<uint8_t>& /*blob*/) {}
+  virtual size_t decode_state(const uint8_t* /*blob*/, size_t /*len*/) { return 0; }
   // Device views for inspection: 0 out_act, 1 out_delta, 2 weights, 3 bias, 4 grad_weights,
   // 5 grad_bias, 6 acc_grad_weights, 7 acc_grad_bias.  Returns false if the operator has no such buffer.
   virtual bool buffer(int which, float** ptr, size_t* len) {
@@ -196,6 +234,10 @@ class InputOperator : public Operator {
   virtual void load_frames(size_t batch_size) = 0;
   // Synthetic fp32 frames (N(0,1) inputs of the benchmark configs): bypasses the u8 cast.
   virtual void load_frames_f32(const float* host, size_t batch_size) = 0;
+  // What the last forward() drew for its random preprocessing steps: crop offsets (of the last Crop), whether
+  // the batch was flipped, and the 3*batch PCA lighting coefficients (empty if that step is absent or idle).
+  virtual void last_preproc_draws(size_t* crop_off_w, size_t* crop_off_h, bool* flipped, std::vector<float>* alphas) const = 0;
+  virtual Dims3 out_dims() const = 0;
 };
 
 class LossOperator : public Operator {
@@ -224,6 +266,8 @@ class SequentialOperatorConfig {
   SequentialOperatorConfig& affine(const AffineOperatorConfig& cfg);
   SequentialOperatorConfig& conv2d(const Conv2dOperatorConfig& cfg);
   SequentialOperatorConfig& pool2d(const Pool2dOperatorConfig& cfg);
+  SequentialOperatorConfig& dropout(const DropoutOperatorConfig& cfg);              // src/operator/worker.rs:219-222
+  SequentialOperatorConfig& local_res_norm(const LocalResNormOperatorConfig& cfg);
   SequentialOperatorConfig& softmax_kl_loss(const CategoricalLossConfig& cfg);
 };
 
@@ -256,6 +300,20 @@ class SequentialOperatorWorker : public Operator {
   void reset() override;
   void fused_sgd_step(float l2, float scale, float momentum, float apply) override;
   const char* kind() const override { return "SequentialOperatorWorker"; }
+  void encode_params(std::vector<uint8_t>& blob) override;
+  size_t decode_params(const uint8_t* blob, size_t len) override;
+  void encode_state(std::vector<uint8_t>& blob) override;
+  size_t decode_state(const uint8_t* blob, size_t len) override;
+  // Checkpoint files under `prefix` (src/worker/gossip_dist.rs:1230-1413): params.t_<t>.blob, the symlink
+  // params.latest.blob, the text file `checkpoint` holding t (previous one kept as checkpoint.0), and
+  // state.latest.blob.<rank> (params + momentum per operator).
+  void checkpoint_params(size_t t, const std::string& prefix);
+  void checkpoint_state(const std::string& prefix);
+  bool can_rollback(const std::string& prefix, size_t* t) const;
+  void rollback_params(const size_t* t /* nullptr = latest */, const std::string& prefix);
+  void rollback_state(const std::string& prefix);
+  // Uniform stream a DropoutOperator's last forward() consumed: (seed, stream id, first element).
+  bool dropout_stream(size_t hidden_idx, uint64_t* seed, uint64_t* stream_id, uint64_t* first) const;
 
  private:
   size_t batch_size_;
@@ -304,5 +362,11 @@ class SgdOpt {
   SgdOptConfig config_;
   size_t iter_counter_ = 0;
 };
+
+// ---- NdArray (de)serialisation (header of tools/dump-array3d-header.rs:8-15) ------------------------------
+// 'N' 'D' 0x00 0x01, u32 LE ndim, u64 LE dims[ndim], then the fp32 LE values in memory order (first index fastest).
+void ndarray_serialize(std::vector<uint8_t>& out, const float* data, const size_t* dims, size_t ndim);
+// Returns the bytes consumed; panics on a malformed header or a short blob.
+size_t ndarray_deserialize(const uint8_t* blob, size_t len, std::vector<size_t>* dims, std::vector<float>* data);
 
 }  // namespace rembrandt

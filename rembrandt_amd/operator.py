@@ -30,10 +30,29 @@ PROTOTYPES = {
     "rho_config_affine": (_int, [_vp, _i32, _i32, _int, _int, _f]),
     "rho_config_pool2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _int, _int]),
     "rho_config_softmax_kl_loss": (_int, [_vp, _i32]),
+    "rho_config_data3d_crop": (_int, [_vp, _i32, _i32]),
+    "rho_config_data3d_flip_x": (_int, [_vp]),
+    "rho_config_data3d_subtract_mean": (_int, [_vp, _vp, _i64]),
+    "rho_config_data3d_subtract_mean_file": (_int, [_vp, C.c_char_p]),
+    "rho_config_data3d_pca_lighting_noise": (_int, [_vp, _vp, _vp, _f]),
+    "rho_config_dropout": (_int, [_vp, _i32, _f]),
+    "rho_config_local_res_norm": (_int, [_vp, _i32, _i32, _i32, _i32, _f, _f, _f]),
     "rho_config_params_len": (_int, [_vp, _P(_i64)]),
     "rho_config_from_model_file": (_int, [C.c_char_p, _P(_vp)]),
     "rho_worker_new": (_int, [_vp, _i32, _int, _u64, _u64, _int, _int, _P(_vp)]),
     "rho_worker_free": (_int, [_vp]),
+    "rho_worker_input_out_dims": (_int, [_vp, _P(_i32), _P(_i32), _P(_i32)]),
+    "rho_worker_last_preproc_draws": (_int, [_vp, _P(_i32), _P(_i32), _P(_int), _vp, _i64, _P(_i64)]),
+    "rho_worker_dropout_stream": (_int, [_vp, _i32, _P(_u64), _P(_u64), _P(_u64)]),
+    "rho_worker_encode_params": (_int, [_vp, _vp, C.c_size_t, _P(C.c_size_t)]),
+    "rho_worker_decode_params": (_int, [_vp, _vp, C.c_size_t, _P(C.c_size_t)]),
+    "rho_worker_encode_state": (_int, [_vp, _vp, C.c_size_t, _P(C.c_size_t)]),
+    "rho_worker_decode_state": (_int, [_vp, _vp, C.c_size_t, _P(C.c_size_t)]),
+    "rho_worker_checkpoint_params": (_int, [_vp, _i64, C.c_char_p]),
+    "rho_worker_checkpoint_state": (_int, [_vp, C.c_char_p]),
+    "rho_worker_can_rollback": (_int, [_vp, C.c_char_p, _P(_i64)]),
+    "rho_worker_rollback_params": (_int, [_vp, _i64, C.c_char_p]),
+    "rho_worker_rollback_state": (_int, [_vp, C.c_char_p]),
     "rho_worker_hidden_count": (_int, [_vp, _P(_i32)]),
     "rho_worker_op_kind": (_int, [_vp, _i32, _P(C.c_char_p)]),
     "rho_worker_stream": (_vp, [_vp]),
@@ -144,6 +163,37 @@ class SequentialOperatorConfig:
                                      POOL[pool_op], int(ceil_mode)))
         return self
 
+    # Data3dPreproc steps (src/operator/mod.rs:395-423), appended in call order
+    def crop(self, crop_width, crop_height):
+        _chk(lib().rho_config_data3d_crop(self._h, crop_width, crop_height))
+        return self
+
+    def flip_x(self):
+        _chk(lib().rho_config_data3d_flip_x(self._h))
+        return self
+
+    def subtract_elemwise_mean(self, mean=None, mean_path=None):
+        if mean_path is not None:
+            _chk(lib().rho_config_data3d_subtract_mean_file(self._h, str(mean_path).encode()))
+        else:
+            mean = np.ascontiguousarray(mean, np.float32)
+            _chk(lib().rho_config_data3d_subtract_mean(self._h, mean.ctypes.data, mean.size))
+        return self
+
+    def pca_lighting_noise(self, singular_vecs, singular_vals, std_dev):
+        v = np.ascontiguousarray(singular_vecs, np.float32).reshape(9)
+        l = np.ascontiguousarray(singular_vals, np.float32).reshape(3)
+        _chk(lib().rho_config_data3d_pca_lighting_noise(self._h, v.ctypes.data, l.ctypes.data, std_dev))
+        return self
+
+    def dropout(self, channels, drop_ratio):
+        _chk(lib().rho_config_dropout(self._h, channels, drop_ratio))
+        return self
+
+    def local_res_norm(self, in_dims, cross_size, scale, power, min_div):
+        _chk(lib().rho_config_local_res_norm(self._h, in_dims[0], in_dims[1], in_dims[2], cross_size, scale, power, min_div))
+        return self
+
     def softmax_kl_loss(self, num_categories):
         _chk(lib().rho_config_softmax_kl_loss(self._h, num_categories))
         return self
@@ -208,6 +258,66 @@ class SequentialOperatorWorker:
     def load_frames_f32(self, frames):
         frames = np.ascontiguousarray(frames, np.float32)
         _chk(lib().rho_worker_load_frames_f32(self._h, frames.ctypes.data, frames.shape[0]))
+
+    def input_out_dims(self):
+        w, h, c = _i32(), _i32(), _i32()
+        _chk(lib().rho_worker_input_out_dims(self._h, C.byref(w), C.byref(h), C.byref(c)))
+        return w.value, h.value, c.value
+
+    def last_preproc_draws(self):
+        """(crop_off_w, crop_off_h, flipped, alphas) of the input operator's last forward()."""
+        ow, oh, fl, n = _i32(), _i32(), _int(), _i64()
+        _chk(lib().rho_worker_last_preproc_draws(self._h, C.byref(ow), C.byref(oh), C.byref(fl), None, 0, C.byref(n)))
+        alphas = np.zeros((n.value,), np.float32)
+        if n.value:
+            _chk(lib().rho_worker_last_preproc_draws(self._h, None, None, None, alphas.ctypes.data, n.value, None))
+        return ow.value, oh.value, bool(fl.value), alphas
+
+    def dropout_stream(self, idx):
+        a, b, c = _u64(), _u64(), _u64()
+        _chk(lib().rho_worker_dropout_stream(self._h, idx, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
+    # parameter / state blobs and checkpoints
+    def _encode(self, fn):
+        n = C.c_size_t()
+        _chk(fn(self._h, None, 0, C.byref(n)))
+        buf = (C.c_uint8 * n.value)()
+        _chk(fn(self._h, buf, n.value, None))
+        return bytes(buf)
+
+    def encode_params(self):
+        return self._encode(lib().rho_worker_encode_params)
+
+    def encode_state(self):
+        return self._encode(lib().rho_worker_encode_state)
+
+    def decode_params(self, blob):
+        n = C.c_size_t()
+        _chk(lib().rho_worker_decode_params(self._h, C.c_char_p(blob), len(blob), C.byref(n)))
+        return n.value
+
+    def decode_state(self, blob):
+        n = C.c_size_t()
+        _chk(lib().rho_worker_decode_state(self._h, C.c_char_p(blob), len(blob), C.byref(n)))
+        return n.value
+
+    def checkpoint_params(self, t, prefix):
+        _chk(lib().rho_worker_checkpoint_params(self._h, t, str(prefix).encode()))
+
+    def checkpoint_state(self, prefix):
+        _chk(lib().rho_worker_checkpoint_state(self._h, str(prefix).encode()))
+
+    def can_rollback(self, prefix):
+        t = _i64()
+        _chk(lib().rho_worker_can_rollback(self._h, str(prefix).encode(), C.byref(t)))
+        return None if t.value < 0 else t.value
+
+    def rollback_params(self, prefix, t=None):
+        _chk(lib().rho_worker_rollback_params(self._h, -1 if t is None else t, str(prefix).encode()))
+
+    def rollback_state(self, prefix):
+        _chk(lib().rho_worker_rollback_state(self._h, str(prefix).encode()))
 
     # LossOperator
     def stage_label(self, batch_idx, category):

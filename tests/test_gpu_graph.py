@@ -3,13 +3,15 @@ CPU restatement of the reference's operator chain, checkpoint by checkpoint, on 
 inputs.  Order of checks: input -> each out_act -> probabilities -> loss, categories (exact),
 accuracy count (exact) -> for each operator in reverse its out_delta (after the in-place ReLU mask),
 grad_weights, grad_bias -> after the update: acc_grad_*, weights, bias -> grads == 0 exactly."""
+import os
+
 import numpy as np
 import pytest
 
 import oracle as O
 from oracle import graph as OG
 from rembrandt_amd import configs, synth
-from rembrandt_amd.operator import SequentialOperatorWorker, SgdOpt
+from rembrandt_amd.operator import SequentialOperatorConfig, SequentialOperatorWorker, SgdOpt
 from conftest import assert_close, say
 
 pytestmark = pytest.mark.gpu
@@ -39,6 +41,11 @@ def check_step(w, ref, sgd, rsgd, x, labels, minibatch, fused_sgd, tag):
     w.stage_batch(labels, 1.0 / minibatch)
     ref.stage_batch(labels, 1.0 / minibatch)
     w.forward(batch, training=True, t=sgd.iter_counter())
+    for i, op in enumerate(ref.hidden):
+        if op.kind == "DropoutOperator":   # the uniform samples this forward consumed, regenerated on the host
+            seed, stream_id, first = w.dropout_stream(i)
+            n = int(np.prod(op.x_shape))
+            op.rnd = synth.uniform(seed, stream_id, (first + n,))[first:]
     ref.forward(x)
     assert_close(w.read(-1, "out_act"), x.ravel(), tag + " input")
     n = len(ref.hidden)
@@ -140,6 +147,34 @@ def test_alexnet_train_step(dev):
     x = synth.normal(0x5EED0004, 100, (batch, 3, 227, 227))
     labels = synth.integers(0x5EED0004, 200, (batch,), 1000)
     check_step(w, ref, sgd, rsgd, x, labels, batch, True, "alexnet step 0")
+    w.close()
+
+
+def test_dropout_lrn_train_steps(dev):
+    """A chain with a local response normalisation and two dropout operators (the layer types the example
+    `.model` files add around the benchmark operators): 3 steps, each with fresh dropout masks."""
+    dims = (14, 14, 3)
+    net = (dims, *configs._chain(dims, [("conv", 3, 1, 1, 8, "Rect"), ("lrn", 5, 1e-2, 0.75, 2.0), ("pool", 2, 2, 0, "Max"),
+                                        ("dropout", 0.3), ("fc", 32, "Rect"), ("dropout", 0.5), ("fc", 6, "Identity")]))
+    batch = 16
+    w, ref = make_pair(net, batch, 91, True)
+    assert [w.op_kind(i) for i in (1, 3, 5)] == ["LocalResNormOperator", "DropoutOperator", "DropoutOperator"]
+    sgd = SgdOpt(batch, 0.05, ("Update", 0.9), 1e-4)
+    rsgd = OG.SgdOpt(0.05, ("Update", 0.9), 1e-4)
+    sgd.begin(w)
+    rsgd.begin(ref)
+    masks = []
+    for step in range(3):
+        say("dropout/lrn step", step)
+        x = synth.normal(91, 100 + step, (batch, 3, 14, 14))
+        labels = synth.integers(91, 200 + step, (batch,), 6)
+        check_step(w, ref, sgd, rsgd, x, labels, batch, True, "dropout/lrn step %d" % step)
+        masks.append(ref.hidden[5].mask.copy())
+        assert 0.3 < masks[-1].mean() < 0.7
+    assert not np.array_equal(masks[0], masks[1]) and not np.array_equal(masks[1], masks[2])
+    # Inference: dropout is the identity
+    w.forward(batch, training=False, t=0)
+    assert np.array_equal(w.read(3, "out_act"), w.read(2, "out_act"))
     w.close()
 
 
@@ -281,3 +316,125 @@ def test_panics(dev):
     with pytest.raises(Panic):
         fwd_only.backward(4)  # assert!(self.backward.is_some())
     w.close(); w2.close(); fwd_only.close()
+
+
+def _tiny_head(cfg, dims, ncat=4):
+    return cfg.affine(dims[0] * dims[1] * dims[2], ncat, "Identity", ("Normal", 0.05)).softmax_kl_loss(ncat)
+
+
+@pytest.mark.parametrize("normalize", [False, True])
+def test_data3d_preprocessing(dev, normalize, tmp_path):
+    """Data3dOperator: u8 frames -> cast (/255 when normalising) -> SubtractElemwiseMean -> FlipX -> Crop, the order
+    the reference's tools use (tools/train-imagenet.rs:63-70), then PCA lighting noise.  The output is compared with
+    the numpy restatement for the offsets / coin / coefficients the operator reports having drawn."""
+    say("data3d preprocessing", normalize)
+    in_dims, crop, batch = (23, 19, 3), (16, 12), 6
+    rng = np.random.default_rng(17)
+    frames = rng.integers(0, 256, (batch, 3, 19, 23), dtype=np.uint8)
+    mean = synth.uniform(18, 1, (3, 19, 23), 0.0, 255.0)
+    svecs, svals = synth.normal(18, 2, (3, 3)), synth.uniform(18, 3, (3,))
+    # the mean comes from an NdArray file, as in the reference (dims (w, h, c), values W fastest)
+    mean_path = tmp_path / "mean.ndarray"
+    import struct
+    mean_path.write_bytes(b"ND\x00\x01" + struct.pack("<I3Q", 3, 23, 19, 3) + mean.tobytes())
+    cfg = (SequentialOperatorConfig().data3d(in_dims, normalize=normalize).subtract_elemwise_mean(mean_path=mean_path)
+           .flip_x().crop(*crop).pca_lighting_noise(svecs, svals, 0.1))
+    w = SequentialOperatorWorker(_tiny_head(cfg, (crop[0], crop[1], 3)), batch, "Forward", shared_seed=(5, 6))
+    assert w.input_out_dims() == (16, 12, 3)
+    w.init_params()
+    w.load_frames_u8(frames)
+    base = frames.astype(np.float32) * (np.float32(1.0 / 255.0) if normalize else np.float32(1.0))
+    seen_flip, seen_off = set(), set()
+    for t in range(12):
+        w.forward(batch, training=True, t=t)
+        off_w, off_h, flipped, alphas = w.last_preproc_draws()
+        assert 0 <= off_w <= 23 - 16 and 0 <= off_h <= 19 - 12 and alphas.shape == (3 * batch,)
+        seen_flip.add(flipped)
+        seen_off.add((off_w, off_h))
+        want = O.subtract_mean(base, mean, normalize)
+        if flipped:
+            want = O.flip_x(want)
+        want = O.pca3_noise(O.crop_nchw(want, crop[0], crop[1], off_w, off_h), alphas, svals, svecs.ravel())
+        got = w.read(-1, "out_act", batch * 3 * 12 * 16)
+        assert_close(got, want.ravel(), "data3d training output (draw %d)" % t)
+    assert seen_flip == {False, True} and len(seen_off) > 3, "both coin faces and several offsets occur in 12 draws"
+    # Inference: centre crop, no flip, no noise
+    w.forward(batch, training=False, t=0)
+    off_w, off_h, flipped, alphas = w.last_preproc_draws()
+    assert (off_w, off_h, flipped, alphas.size) == ((23 - 16) // 2, (19 - 12) // 2, False, 0)
+    want = O.crop_nchw(O.subtract_mean(base, mean, normalize), crop[0], crop[1], off_w, off_h)
+    assert_close(w.read(-1, "out_act", want.size), want.ravel(), "data3d inference output")
+    # fp32 frames take the same path minus the cast, and survive repeated forwards
+    w.load_frames_f32(base)
+    for _ in range(2):
+        w.forward(batch, training=False, t=0)
+        assert_close(w.read(-1, "out_act", want.size), want.ravel(), "data3d inference output from fp32 frames")
+    w.close()
+
+
+def test_param_blobs_and_checkpoints(dev, tmp_path):
+    """encode/decode_params/state and the checkpoint files: bytes are NdArray records of the documented layout,
+    a round trip through another worker reproduces parameters and momentum exactly, rollback picks the iteration."""
+    import struct
+    net, batch = configs.lenet(), 8
+    w, ref = make_pair(net, batch, 123, True)
+    sgd = SgdOpt(batch, 0.01, ("Update", 0.9), 5e-4)
+    sgd.begin(w)
+    x = synth.uniform(123, 1, (batch, 1, 28, 28))
+    labels = synth.integers(123, 2, (batch,), 10)
+    w.load_frames_f32(x)
+    w.stage_batch(labels, 1.0 / batch)
+    sgd.train_batch(w, batch)
+    blob = w.encode_params()
+    # walk the records: conv1 (25, 20), (1, 20), conv2 (500, 50), (1, 50), fc1 (2450, 500), (1, 500), fc2 (500, 10), (1, 10)
+    off, bounds = 0, []
+    params = {0: "weights", 1: "bias"}
+    expect_ops = [i for i in range(w.hidden_count()) if w.op_kind(i) != "Pool2dOperator"]
+    k = 0
+    while off < len(blob):
+        assert blob[off:off + 4] == b"ND\x00\x01"
+        (rank,) = struct.unpack_from("<I", blob, off + 4)
+        dims = struct.unpack_from("<%dQ" % rank, blob, off + 8)
+        n = int(np.prod(dims))
+        data = np.frombuffer(blob, np.float32, n, off + 8 + 8 * rank)
+        assert np.array_equal(data, w.read(expect_ops[k // 2], params[k % 2])), "record %d holds the device buffer" % k
+        bounds.append(dims)
+        off += 8 + 8 * rank + 4 * n
+        k += 1
+    assert bounds == [(25, 20), (1, 20), (500, 50), (1, 50), (2450, 500), (1, 500), (500, 10), (1, 10)]
+    state = w.encode_state()
+    assert len(state) == 2 * len(blob)
+
+    prefix = tmp_path / "ckpt"
+    w.checkpoint_params(1, prefix)
+    w.checkpoint_state(prefix)
+    sgd.train_batch(w, batch)
+    w.checkpoint_params(2, prefix)
+    assert sorted(os.listdir(prefix)) == ["checkpoint", "checkpoint.0", "params.latest.blob", "params.t_1.blob",
+                                          "params.t_2.blob", "state.latest.blob.0"]
+    assert (prefix / "checkpoint").read_text() == "2\n" and (prefix / "checkpoint.0").read_text() == "1\n"
+    assert os.readlink(prefix / "params.latest.blob") == "params.t_2.blob"
+    assert (prefix / "params.t_1.blob").read_bytes() == blob
+
+    cfg = configs.build_config(net)
+    w2 = SequentialOperatorWorker(cfg, batch, "Backward", shared_seed=(9, 9))
+    w2.init_params()
+    assert w2.can_rollback(tmp_path / "nowhere") is None and w2.can_rollback(prefix) == 2
+    w2.rollback_params(prefix)            # latest = t_2
+    for i in expect_ops:
+        assert np.array_equal(w2.read(i, "weights"), w.read(i, "weights"))
+    w2.rollback_params(prefix, t=1)
+    assert w2.encode_params() == blob
+    w2.rollback_state(prefix)             # params of t=1 plus the momentum buffers
+    assert w2.encode_state() == state
+    with pytest.raises(Exception):
+        w2.rollback_params(prefix, t=3)   # beyond the latest checkpoint
+    with pytest.raises(Exception):
+        w2.decode_params(blob[:-4])       # truncated
+    # a blob of another architecture is refused
+    other = SequentialOperatorWorker(configs.build_config(configs.cifar10()), 4, "Forward", shared_seed=(1, 1))
+    with pytest.raises(Exception):
+        other.decode_params(blob)
+    other.close()
+    w2.close()
+    w.close()

@@ -118,6 +118,9 @@ def test_model_parser_errors(tmp_path):
     loss = '[[layer]]\nname = "loss"\ntype = "softmax_loss"\nnum_categories = 3\n'
     assert parse(data + fc + loss).params_len() == 64 * 3 + 3
     assert parse("# c\n" + data + "\n\n" + fc + "[opt]\nminibatch_size = 4 # ignored table\n" + loss).params_len() == 195
+    lrn = '[[layer]]\nname = "n"\ntype = "local_res_norm"\ncross_size = 5\nscale = 0.0001\npower = 0.75\nmin_div = 2\n'
+    drop = '[[layer]]\nname = "d"\ntype = "dropout"\ndrop_ratio = 0.5\n'
+    assert parse(data + lrn + drop + fc + loss).params_len() == 195
     for bad in (data + fc,                                             # no loss layer
                 fc + loss,                                             # no input for the first layer
                 data + fc.replace('"identity"', '"relu"') + loss,      # act_func "relu" is not in the grammar (config.rs:123-129)
@@ -125,7 +128,8 @@ def test_model_parser_errors(tmp_path):
                 data + fc + loss.replace("3", "4"),                    # input length != num_categories
                 data + fc.replace("std = 0.1", "std = 1") + loss,      # as_float() rejects an integer
                 data + fc.replace('kind = "normal"', 'kind = "xavier"') + loss,
-                data + '[[layer]]\nname = "n"\ntype = "local_res_norm"\ncross_size = 5\n' + fc + loss,
+                data + '[[layer]]\nname = "n"\ntype = "local_res_norm"\n' + fc + loss,   # missing cross_size
+                data + '[[layer]]\nname = "d"\ntype = "dropout"\n' + fc + loss,          # missing drop_ratio
                 data + "garbage line\n" + fc + loss):
         with pytest.raises(Panic):
             parse(bad)
