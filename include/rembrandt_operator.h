@@ -145,10 +145,52 @@ int rho_sgd_free(rho_sgd* s);
 int rho_sgd_begin(rho_sgd* s, rho_worker* w);
 int rho_sgd_step(rho_sgd* s, rho_worker* w, int fused);
 int rho_sgd_iter_counter(rho_sgd* s, int64_t* out);
+int rho_sgd_set_iter_counter(rho_sgd* s, int64_t t);   /* resuming: init_t of new.rs:231-252 */
 int rho_sgd_step_size_at(rho_sgd* s, int64_t t, float* out);                 /* StepSizeSchedule::at_iter */
 /* One whole training step on a staged batch, in the order of SgdOpt::train (new.rs:325-343 + the
  * update block): forward, store_output_categories, store_loss, backward, accuracy_count, step. */
 int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused, float* loss_out, int32_t* correct_out);
+
+/* ---- data sources (src/data_new.rs:282-357, 648-883) ----
+ * source: "mnist" (idx3-ubyte frames + idx1-ubyte labels) or "cifar10" (3073-byte records: label, 3 planes of 32x32).
+ * rho_dataset_open_from_file reads a `.data` file ([dataset.<key>] source / data_path / labels_path). */
+typedef struct rho_dataset rho_dataset;
+int rho_dataset_open(const char* source, const char* data_path, const char* labels_path, rho_dataset** out);
+int rho_dataset_open_from_file(const char* data_file_path, const char* key, rho_dataset** out);
+int rho_dataset_free(rho_dataset* d);
+int rho_dataset_num_samples(const rho_dataset* d, int64_t* out);
+int rho_dataset_frame_dims(const rho_dataset* d, int32_t* w, int32_t* h, int32_t* c);
+int rho_dataset_get_sample(const rho_dataset* d, int64_t idx, uint8_t* frame_out /* may be NULL */, int32_t* category);
+
+/* ---- SgdOpt::train / validate for one worker (src/opt/sgd/new.rs:209-766) ----
+ * Samples are staged through expose_host_frame_buf / stage_label / stage_weight(1/minibatch); every full batch runs
+ * forward(Training{t}) -> arg-max, loss read-backs -> backward; every minibatch_size samples the update block runs
+ * (gradients of the batches in between accumulate).  At every checkpoint_iters-th iteration: save_params (Discard),
+ * checkpoint_state + checkpoint_params every save_iters, validation (Inference phase, weights 1/num_samples) every
+ * valid_iters, restore_params (Discard).  The trace `t,event,loss,error,elapsed` goes to
+ * <checkpoint_dir>/trace_sgd.log[.N].  init: resume_from < 0 = InitOrResume (rollback_state if a `checkpoint` file
+ * exists, else init_params(shared_seed)), otherwise ResumeFrom{t}.  The reference loops for ever; max_iters ends it. */
+#define RHO_ORDER_SEQUENTIAL     0  /* SampleIterator          */
+#define RHO_ORDER_RANDOM_EPISODE 1  /* RandomEpisodeIterator: uniform with replacement */
+#define RHO_ORDER_CYCLIC_EPISODE 2  /* CyclicEpisodeIterator   */
+typedef struct rho_train_config {
+  const char* checkpoint_dir;  /* NULL or "": no log, no checkpoints */
+  int64_t resume_from;
+  int64_t display_iters, checkpoint_iters, save_iters, valid_iters;
+  int checkpoint_discard;
+  int64_t max_iters;
+  int fused;
+} rho_train_config;
+typedef struct rho_train_stats {
+  int64_t iters, epochs;
+  float last_loss, last_error;
+  int64_t valid_runs;
+  float valid_loss, valid_error;
+  char log_path[512];
+} rho_train_stats;
+int rho_sgd_train(rho_sgd* s, rho_worker* w, const rho_dataset* train, int train_order, uint64_t order_seed,
+                  const rho_dataset* valid /* may be NULL */, const rho_train_config* cfg, rho_train_stats* stats_out);
+int rho_sgd_validate(rho_worker* w, const rho_dataset* valid, float* loss, float* accuracy);
 
 #ifdef __cplusplus
 }

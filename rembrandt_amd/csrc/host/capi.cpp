@@ -1,10 +1,12 @@
 // C ABI of the operator / graph / optimizer layer (include/rembrandt_operator.h).
+#include <cstdio>
 #include <memory>
 #include <string>
 #include <vector>
 #include <algorithm>
 
 #include "../../../include/rembrandt_operator.h"
+#include "data_source.hpp"
 #include "model_config.hpp"
 #include "operator.hpp"
 
@@ -16,6 +18,7 @@ struct rho_worker {
   std::unique_ptr<SequentialOperatorWorker> worker;
 };
 struct rho_sgd { std::unique_ptr<SgdOpt> opt; };
+struct rho_dataset { std::unique_ptr<DataSource> src; };
 
 static thread_local std::string g_message;
 
@@ -385,6 +388,7 @@ int rho_sgd_new(int32_t minibatch_size, int step_kind, const float* steps, const
 int rho_sgd_free(rho_sgd* s) { RHO_TRY({ delete s; }) }
 int rho_sgd_begin(rho_sgd* s, rho_worker* w) { RHO_TRY({ RHO_REQ(s && w); s->opt->begin(w->worker.get()); }) }
 int rho_sgd_step(rho_sgd* s, rho_worker* w, int fused) { RHO_TRY({ RHO_REQ(s && w); s->opt->step(w->worker.get(), fused != 0); }) }
+int rho_sgd_set_iter_counter(rho_sgd* s, int64_t t) { RHO_TRY({ RHO_REQ(s && t >= 0); s->opt->set_iter_counter((size_t)t); }) }
 int rho_sgd_iter_counter(rho_sgd* s, int64_t* out) { RHO_TRY({ RHO_REQ(s && out); *out = (int64_t)s->opt->iter_counter(); }) }
 int rho_sgd_step_size_at(rho_sgd* s, int64_t t, float* out) {
   RHO_TRY({ RHO_REQ(s && out && t >= 0); *out = s->opt->config().step_size.at_iter((size_t)t); })
@@ -405,4 +409,84 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
   })
 }
 
+
+int rho_dataset_open(const char* source, const char* data_path, const char* labels_path, rho_dataset** out) {
+  RHO_TRY({
+    RHO_REQ(source && data_path && out);
+    DataSourceConfig c;
+    c.source = source;
+    c.data_path = data_path;
+    if (labels_path && *labels_path) { c.labels_path = labels_path; c.has_labels = true; }
+    std::unique_ptr<rho_dataset> d(new rho_dataset());
+    d->src = build_data_source(c);
+    *out = d.release();
+  })
+}
+int rho_dataset_open_from_file(const char* data_file_path, const char* key, rho_dataset** out) {
+  RHO_TRY({
+    RHO_REQ(data_file_path && key && out);
+    std::unique_ptr<rho_dataset> d(new rho_dataset());
+    d->src = build_data_source(DatasetConfig::open(data_file_path), key);
+    *out = d.release();
+  })
+}
+int rho_dataset_free(rho_dataset* d) { RHO_TRY({ delete d; }) }
+int rho_dataset_num_samples(const rho_dataset* d, int64_t* out) { RHO_TRY({ RHO_REQ(d && out); *out = (int64_t)d->src->num_samples(); }) }
+int rho_dataset_frame_dims(const rho_dataset* d, int32_t* w, int32_t* h, int32_t* c) {
+  RHO_TRY({
+    RHO_REQ(d && w && h && c);
+    const Dims3 dims = d->src->frame_dims();
+    *w = (int32_t)dims.w; *h = (int32_t)dims.h; *c = (int32_t)dims.c;
+  })
+}
+int rho_dataset_get_sample(const rho_dataset* d, int64_t idx, uint8_t* frame_out, int32_t* category) {
+  RHO_TRY({
+    RHO_REQ(d && idx >= 0 && category);
+    const uint8_t* f = nullptr;
+    if (!d->src->get_sample((size_t)idx, &f, category)) panic("sample index out of range");
+    if (frame_out) std::copy(f, f + d->src->frame_dims().len(), frame_out);
+  })
+}
+
+int rho_sgd_train(rho_sgd* s, rho_worker* w, const rho_dataset* train, int train_order, uint64_t order_seed,
+                  const rho_dataset* valid, const rho_train_config* cfg, rho_train_stats* stats_out) {
+  RHO_TRY({
+    RHO_REQ(s && w && train && cfg);
+    RHO_REQ(train_order >= RHO_ORDER_SEQUENTIAL && train_order <= RHO_ORDER_CYCLIC_EPISODE);
+    SgdTrainConfig c;
+    c.init = cfg->resume_from >= 0 ? SgdTrainConfig::ResumeFrom : SgdTrainConfig::InitOrResume;
+    c.resume_t = cfg->resume_from >= 0 ? (size_t)cfg->resume_from : 0;
+    c.checkpoint_dir = cfg->checkpoint_dir ? cfg->checkpoint_dir : "";
+    c.display_iters = (size_t)cfg->display_iters;
+    c.checkpoint_iters = (size_t)cfg->checkpoint_iters;
+    c.save_iters = (size_t)cfg->save_iters;
+    c.valid_iters = (size_t)cfg->valid_iters;
+    c.checkpoint_discard = cfg->checkpoint_discard != 0;
+    c.max_iters = (size_t)cfg->max_iters;
+    c.fused = cfg->fused != 0;
+    const uint64_t seed[2] = {order_seed, order_seed ^ 0x9E3779B97F4A7C15ull};
+    DataIter train_iter(train->src.get(), (DataIter::Kind)train_order, seed);
+    std::unique_ptr<DataIter> valid_iter;
+    if (valid) valid_iter.reset(new DataIter(valid->src.get(), DataIter::Sequential, seed));
+    const SgdTrainStats st = sgd_train(*s->opt, *w->worker, train_iter, valid_iter.get(), c);
+    if (stats_out) {
+      stats_out->iters = (int64_t)st.iters;
+      stats_out->epochs = (int64_t)st.epochs;
+      stats_out->last_loss = st.last_loss;
+      stats_out->last_error = st.last_error;
+      stats_out->valid_runs = (int64_t)st.valid_runs;
+      stats_out->valid_loss = st.valid_loss;
+      stats_out->valid_error = st.valid_error;
+      std::snprintf(stats_out->log_path, sizeof(stats_out->log_path), "%s", st.log_path.c_str());
+    }
+  })
+}
+int rho_sgd_validate(rho_worker* w, const rho_dataset* valid, float* loss, float* accuracy) {
+  RHO_TRY({
+    RHO_REQ(w && valid);
+    const uint64_t seed[2] = {1, 2};
+    DataIter it(valid->src.get(), DataIter::Sequential, seed);
+    sgd_validate(*w->worker, it, loss, accuracy);
+  })
+}
 }  // extern "C"

@@ -403,6 +403,7 @@ class Data3dOperator : public InputOperator {
   SharedDeviceBuf get_output_vars() const override { return out_buf_; }
   SharedDeviceBuf get_output_deltas() const override { return nullptr; }  // src/operator/mod.rs:632-634
   Dims3 out_dims() const override { return config_.get_out_dims(); }
+  size_t in_frame_len() const override { return config_.in_dims.len(); }
   uint8_t* expose_host_frame_buf(size_t batch_idx) override {
     RB_ASSERT(batch_idx < batch_cap_);
     return in_buf_h_.data() + batch_idx * config_.in_dims.len();
@@ -1194,7 +1195,7 @@ void SgdOpt::begin(Operator* op) {
   op->reset();
 }
 
-void SgdOpt::step(Operator* op, bool fused) {
+void SgdOpt::step(Operator* op, bool fused, bool defer_reapply) {
   const float l2 = config_.l2_reg_coef;
   const float step_size = config_.step_size.at_iter(iter_counter_);  // before the increment (StepSizeReference::Local)
   const float mu = config_.momentum.mu;
@@ -1224,7 +1225,11 @@ void SgdOpt::step(Operator* op, bool fused) {
     case Momentum::GradientNesterov: op->update_params2(-step_size, -step_size * mu); break;
   }
   op->reset();
-  if (k == Momentum::UpdateNesterov) op->update_params(mu);
+  if (k == Momentum::UpdateNesterov && !defer_reapply) op->update_params(mu);
+}
+
+void SgdOpt::reapply(Operator* op) {
+  if (config_.momentum.kind == Momentum::UpdateNesterov) op->update_params(config_.momentum.mu);
 }
 
 }  // namespace rembrandt

@@ -234,6 +234,7 @@ class InputOperator : public Operator {
   virtual void load_frames(size_t batch_size) = 0;
   // Synthetic fp32 frames (N(0,1) inputs of the benchmark configs): bypasses the u8 cast.
   virtual void load_frames_f32(const float* host, size_t batch_size) = 0;
+  virtual size_t in_frame_len() const = 0;  // bytes per staged frame
   // What the last forward() drew for its random preprocessing steps: crop offsets (of the last Crop), whether
   // the batch was flipped, and the 3*batch PCA lighting coefficients (empty if that step is absent or idle).
   virtual void last_preproc_draws(size_t* crop_off_w, size_t* crop_off_h, bool* flipped, std::vector<float>* alphas) const = 0;
@@ -354,8 +355,12 @@ class SgdOpt {
   // Called once before the first minibatch (src/opt/sgd/new.rs:257-271).
   void begin(Operator* op);
   // `fused`: use Operator::fused_sgd_step where the flavour allows it (Zero, Update, Gradient).
-  void step(Operator* op, bool fused);
+  // `defer_reapply`: leave out the look-ahead `W += mu*v` that ends an UpdateNesterov step; the caller runs
+  // reapply() after whatever must see the plain parameters (checkpoints, validation: new.rs:623-633).
+  void step(Operator* op, bool fused, bool defer_reapply = false);
+  void reapply(Operator* op);
   size_t iter_counter() const { return iter_counter_; }
+  void set_iter_counter(size_t t) { iter_counter_ = t; }  // resuming from a checkpoint
   const SgdOptConfig& config() const { return config_; }
 
  private:

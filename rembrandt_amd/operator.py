@@ -86,9 +86,31 @@ PROTOTYPES = {
     "rho_sgd_begin": (_int, [_vp, _vp]),
     "rho_sgd_step": (_int, [_vp, _vp, _int]),
     "rho_sgd_iter_counter": (_int, [_vp, _P(_i64)]),
+    "rho_sgd_set_iter_counter": (_int, [_vp, _i64]),
     "rho_sgd_step_size_at": (_int, [_vp, _i64, _P(_f)]),
     "rho_sgd_train_batch": (_int, [_vp, _vp, _i32, _int, _P(_f), _P(_i32)]),
+    "rho_dataset_open": (_int, [C.c_char_p, C.c_char_p, C.c_char_p, _P(_vp)]),
+    "rho_dataset_open_from_file": (_int, [C.c_char_p, C.c_char_p, _P(_vp)]),
+    "rho_dataset_free": (_int, [_vp]),
+    "rho_dataset_num_samples": (_int, [_vp, _P(_i64)]),
+    "rho_dataset_frame_dims": (_int, [_vp, _P(_i32), _P(_i32), _P(_i32)]),
+    "rho_dataset_get_sample": (_int, [_vp, _i64, _vp, _P(_i32)]),
+    "rho_sgd_train": (_int, [_vp, _vp, _vp, _int, _u64, _vp, _vp, _vp]),
+    "rho_sgd_validate": (_int, [_vp, _vp, _P(_f), _P(_f)]),
 }
+
+
+class TrainConfig(C.Structure):
+    _fields_ = [("checkpoint_dir", C.c_char_p), ("resume_from", _i64), ("display_iters", _i64), ("checkpoint_iters", _i64),
+                ("save_iters", _i64), ("valid_iters", _i64), ("checkpoint_discard", _int), ("max_iters", _i64), ("fused", _int)]
+
+
+class TrainStats(C.Structure):
+    _fields_ = [("iters", _i64), ("epochs", _i64), ("last_loss", _f), ("last_error", _f), ("valid_runs", _i64),
+                ("valid_loss", _f), ("valid_error", _f), ("log_path", C.c_char * 512)]
+
+
+ORDER = {"Sequential": 0, "RandomEpisode": 1, "CyclicEpisode": 2}
 
 _bound = False
 
@@ -407,6 +429,41 @@ class SequentialOperatorWorker:
         _chk(lib().rho_worker_write_buffer(self._h, idx, BUF[which], values.ctypes.data, values.size))
 
 
+class DataSource:
+    """MnistDataSource / Cifar10DataSource (src/data_new.rs:648-883), or an entry of a `.data` file."""
+
+    def __init__(self, source=None, data_path=None, labels_path=None, data_file=None, key=None):
+        h = _vp()
+        if data_file is not None:
+            _chk(lib().rho_dataset_open_from_file(str(data_file).encode(), key.encode(), C.byref(h)))
+        else:
+            _chk(lib().rho_dataset_open(source.encode(), str(data_path).encode(),
+                                        str(labels_path).encode() if labels_path else None, C.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().rho_dataset_free(self._h)
+            self._h = None
+
+    def num_samples(self):
+        n = _i64()
+        _chk(lib().rho_dataset_num_samples(self._h, C.byref(n)))
+        return n.value
+
+    def frame_dims(self):
+        w, h, c = _i32(), _i32(), _i32()
+        _chk(lib().rho_dataset_frame_dims(self._h, C.byref(w), C.byref(h), C.byref(c)))
+        return w.value, h.value, c.value
+
+    def get_sample(self, idx):
+        w, h, c = self.frame_dims()
+        frame = np.empty((c, h, w), np.uint8)
+        cat = _i32()
+        _chk(lib().rho_dataset_get_sample(self._h, idx, frame.ctypes.data, C.byref(cat)))
+        return frame, cat.value
+
+
 class SgdOpt:
     """The update block of SgdOpt::train, src/opt/sgd/new.rs:345-495 (one worker, no communication)."""
 
@@ -434,6 +491,28 @@ class SgdOpt:
 
     def begin(self, worker):
         _chk(lib().rho_sgd_begin(self._h, worker._h))
+
+    def set_iter_counter(self, t):
+        _chk(lib().rho_sgd_set_iter_counter(self._h, t))
+
+    def train(self, worker, train_data, max_iters, valid_data=None, order="Sequential", order_seed=1, checkpoint_dir=None,
+              resume_from=None, display_iters=0, checkpoint_iters=0, save_iters=0, valid_iters=0, checkpoint_discard=False,
+              fused=True):
+        """SgdOpt::train (src/opt/sgd/new.rs:209-639) for one worker, ended after max_iters minibatches."""
+        cfg = TrainConfig(str(checkpoint_dir).encode() if checkpoint_dir else None, -1 if resume_from is None else resume_from,
+                          display_iters, checkpoint_iters, save_iters, valid_iters, int(checkpoint_discard), max_iters, int(fused))
+        st = TrainStats()
+        _chk(lib().rho_sgd_train(self._h, worker._h, train_data._h, ORDER[order], order_seed,
+                                 valid_data._h if valid_data is not None else None, C.byref(cfg), C.byref(st)))
+        return {"iters": st.iters, "epochs": st.epochs, "last_loss": st.last_loss, "last_error": st.last_error,
+                "valid_runs": st.valid_runs, "valid_loss": st.valid_loss, "valid_error": st.valid_error,
+                "log_path": st.log_path.decode()}
+
+    @staticmethod
+    def validate(worker, valid_data):
+        loss, acc = _f(), _f()
+        _chk(lib().rho_sgd_validate(worker._h, valid_data._h, C.byref(loss), C.byref(acc)))
+        return loss.value, acc.value
 
     def step(self, worker, fused=True):
         _chk(lib().rho_sgd_step(self._h, worker._h, int(fused)))

@@ -167,3 +167,57 @@ def test_step_size_schedules():
     with pytest.raises(Panic):
         SgdOpt(64, schedule={"kind": "Decay", "steps": [0.1]}).step_size_at(0)   # unimplemented!() in the reference too
     assert SgdOpt(64, 0.1).iter_counter() == 0
+
+
+def _write_idx(path, arr):
+    import struct
+    arr = np.ascontiguousarray(arr, np.uint8)
+    with open(path, "wb") as f:
+        f.write(struct.pack(">I", 0x0800 | arr.ndim))
+        for d in arr.shape:
+            f.write(struct.pack(">I", d))
+        f.write(arr.tobytes())
+
+
+def test_mnist_and_cifar_sources(tmp_path):
+    """idx / CIFAR-binary readers (src/data_new.rs:648-883): header parsing, frame dims, sample access, the
+    `.data` file route, and the malformed-file panics."""
+    from rembrandt_amd.operator import DataSource
+    rng = np.random.default_rng(3)
+    imgs = rng.integers(0, 256, (11, 6, 9), dtype=np.uint8)       # 11 frames of 6 rows x 9 columns
+    labels = rng.integers(0, 10, (11,), dtype=np.uint8)
+    _write_idx(tmp_path / "img.idx", imgs)
+    _write_idx(tmp_path / "lab.idx", labels)
+    ds = DataSource("mnist", tmp_path / "img.idx", tmp_path / "lab.idx")
+    assert ds.num_samples() == 11 and ds.frame_dims() == (9, 6, 1)
+    for i in (0, 5, 10):
+        frame, cat = ds.get_sample(i)
+        assert np.array_equal(frame[0], imgs[i]) and cat == labels[i]
+    with pytest.raises(Panic):
+        ds.get_sample(11)
+    recs = np.zeros((7, 3073), np.uint8)
+    recs[:, 0] = np.arange(7)
+    recs[:, 1:] = rng.integers(0, 256, (7, 3072), dtype=np.uint8)
+    (tmp_path / "c.bin").write_bytes(recs.tobytes())
+    cs = DataSource("cifar10", tmp_path / "c.bin")
+    assert cs.num_samples() == 7 and cs.frame_dims() == (32, 32, 3)
+    frame, cat = cs.get_sample(4)
+    assert cat == 4 and np.array_equal(frame.ravel(), recs[4, 1:])
+    (tmp_path / "d.data").write_text('[dataset.train]\nsource = "mnist"\ndata_path = "%s"\nlabels_path = "%s"\n'
+                                     '[dataset.valid]\nsource = "cifar10"\ndata_path = "%s"\n'
+                                     % (tmp_path / "img.idx", tmp_path / "lab.idx", tmp_path / "c.bin"))
+    assert DataSource(data_file=tmp_path / "d.data", key="train").num_samples() == 11
+    assert DataSource(data_file=tmp_path / "d.data", key="valid").frame_dims() == (32, 32, 3)
+    # malformed inputs
+    (tmp_path / "short.bin").write_bytes(b"\0" * 3000)
+    _write_idx(tmp_path / "lab_short.idx", labels[:5])
+    (tmp_path / "badmagic.idx").write_bytes(b"\0\0\x0d\x03" + b"\0" * 12)
+    (tmp_path / "trunc.idx").write_bytes((tmp_path / "img.idx").read_bytes()[:-3])
+    for args in (("cifar10", tmp_path / "short.bin", None), ("mnist", tmp_path / "img.idx", None),
+                 ("mnist", tmp_path / "img.idx", tmp_path / "lab_short.idx"), ("mnist", tmp_path / "badmagic.idx", tmp_path / "lab.idx"),
+                 ("mnist", tmp_path / "trunc.idx", tmp_path / "lab.idx"), ("mnist", tmp_path / "nope.idx", tmp_path / "lab.idx"),
+                 ("episodb", tmp_path / "img.idx", None)):
+        with pytest.raises(Panic):
+            DataSource(*args)
+    with pytest.raises(Panic):
+        DataSource(data_file=tmp_path / "d.data", key="test")
