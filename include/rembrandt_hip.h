@@ -266,6 +266,8 @@ int rh_profile_reset(void);
  * fp32 MFMA loop (blocks x 4 waves, each issuing iters * nacc MFMAs, nacc in {4, 8}; FLOPs =
  * blocks * 4 * iters * nacc * 4096) and a float4 copy of n floats (bytes = 8 * n). */
 int rh_probe_mfma_loop(int blocks, int nacc, int iters, float* sink, rh_stream_t stream);
+/* The same loop on operands that differ per lane and per instruction (realistic data toggling and power draw). */
+int rh_probe_mfma_loop_varied(int blocks, int iters, float* sink, rh_stream_t stream);
 int rh_probe_copy(const float* src, float* dst, size_t n, rh_stream_t stream);
 
 #ifdef __cplusplus

@@ -87,6 +87,7 @@ PROTOTYPES = {
     "rh_profile_get": (_int, [_int, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(_f)]),
     "rh_profile_reset": (_int, []),
     "rh_probe_mfma_loop": (_int, [_int, _int, _int, _vp, _vp]),
+    "rh_probe_mfma_loop_varied": (_int, [_int, _int, _vp, _vp]),
     "rh_probe_copy": (_int, [_vp, _vp, _sz, _vp]),
     "rh_rng_fill_uniform": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_normal": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),

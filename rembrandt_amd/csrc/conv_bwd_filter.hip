@@ -8,6 +8,18 @@
 
 namespace rh {
 
+// Column tile (filter taps) for a row tile: 128-row tiles pair with 128 columns; narrower row tiles take 256
+// columns unless 128 pads the tap count less (AlexNet conv1: 363 taps = 3 x 128 - 21 instead of 2 x 256 - 149).
+static int pick_bn(int bm, int cols) {
+  if (bm == 128) return 128;
+  if (bm == 96 && round_up(cols, 128) < round_up(cols, 256)) return 128;
+  return 256;
+}
+// Blocks of a tile shape that one CU holds at a time (registers and LDS), times 256 CUs.
+static int resident_slots(int bm, int bn) {
+  return 256 * (bm == 128 ? RH_OCC_128 : bm == 96 ? (bn == 128 ? 4 : 2) : 3);
+}
+
 struct BwdFilterPlan {
   int bm, bn, tiles, splits;
   size_t tab_bytes, part_bytes;
@@ -17,7 +29,7 @@ static BwdFilterPlan plan_bwd_filter(const ConvDims& d) {
   BwdFilterPlan p;
   const int CRS = d.C * d.R * d.S;
   p.bm = pick_bm(d.K);
-  p.bn = p.bm == 128 ? 128 : 256;
+  p.bn = pick_bn(p.bm, CRS);
   p.tiles = cdiv(d.K, p.bm) * cdiv(CRS, p.bn);
   const long long M = (long long)d.N * d.P * d.Q;
   const int k_chunks = (int)cdiv<long long>(M, 16);
@@ -25,11 +37,11 @@ static BwdFilterPlan plan_bwd_filter(const ConvDims& d) {
   // second round: a block that runs alone on its CU uses the matrix pipe less well than three
   // sharing it, so a ragged tail costs more than its share.  Every slice keeps at least 32 K
   // steps so the prologue and the partial-sum traffic stay small next to the contraction.
-  const int slots = 256 * (p.bm == 128 ? RH_OCC_128 : p.bm == 96 ? 2 : 3);
+  const int slots = resident_slots(p.bm, p.bn);
   int want = slots / p.tiles;
   const int max_by_depth = k_chunks / 32 > 0 ? k_chunks / 32 : 1;
   if (want > max_by_depth) want = max_by_depth;
-  if (want > 256) want = 256;
+  if (want > 512) want = 512;
   if (want < 1) want = 1;
   p.splits = want;
   p.tab_bytes = align256(sizeof(int4) * (size_t)round_up(CRS, kTabPad));
@@ -70,11 +82,11 @@ void launch_split_reduce(const float* part, int splits, long long split_stride, 
 // The result comes out as dw'[ko][(r,s,c)]; the reduction kernel puts it back in [ko][c][r][s] order.
 // The channel-last path pays two transposes; it wins when the contraction is deep relative to them.
 static bool use_soff_bwd_filter(const ConvDims& d) {
-  // FLOPs of the contraction per byte the two transposes move (measured: conv1-like 119 and 1x1 24 lose,
-  // 3x3 / 5x5 layers at 690-875 win)
+  // FLOPs of the contraction per byte the two transposes move (measured: 11x11 stride-4 first layers at 59,
+  // small 5x5 layers at 75-78 and 1x1 at 12 lose or tie; 3x3 / 5x5 layers at 288-402 win by 25 %)
   const double flops = 2.0 * d.K * d.C * d.R * d.S * (double)d.N * d.P * d.Q;
   const double bytes = 8.0 * ((double)d.y_elems + (double)d.N * d.C * (d.H + 2 * d.pad) * (d.W + 2 * d.pad));
-  return flops / bytes >= 300.0;
+  return flops / bytes >= 150.0;
 }
 
 struct BwdFilterSoffPlan {
@@ -92,10 +104,10 @@ static BwdFilterSoffPlan plan_bwd_filter_soff(const ConvDims& d) {
   p.Wp = d.W + 2 * d.pad;
   p.n_k = (int)((M + kTabPad - 1) / kTabPad * kTabPad);
   p.bm = pick_bm(d.K);
-  p.bn = p.bm == 128 ? 128 : 256;
+  p.bn = pick_bn(p.bm, CRS);
   p.tiles = cdiv(d.K, p.bm) * cdiv(CRS, p.bn);
   const int k_chunks = p.n_k / 16;
-  const int slots = 256 * (p.bm == 128 ? RH_OCC_128 : p.bm == 96 ? 2 : 3);
+  const int slots = resident_slots(p.bm, p.bn);
   int want = slots / p.tiles;
   const int max_by_depth = k_chunks / 32 > 0 ? k_chunks / 32 : 1;
   if (want > max_by_depth) want = max_by_depth;
@@ -342,7 +354,10 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
     int used = 1, e = 0;
     switch (sp.bm) {
       case 128: e = run_bwd_filter_soff<T128x128>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_128x128"); break;
-      case 96:  e = run_bwd_filter_soff<T96x256>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_96x256"); break;
+      case 96:
+        e = sp.bn == 128 ? run_bwd_filter_soff<T96x128>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_96x128")
+                         : run_bwd_filter_soff<T96x256>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_96x256");
+        break;
       case 64:  e = run_bwd_filter_soff<T64x256>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_64x256"); break;
       default:  e = run_bwd_filter_soff<T32x256>(ap, bp, ep, sp.n_k, Ms, sp.splits, &used, stream, "conv_bwd_filter_32x256"); break;
     }
@@ -377,7 +392,10 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
   } else {
     switch (plan.bm) {
       case 128: e = run_bwd_filter<T128x128>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_128x128"); break;
-      case 96:  e = run_bwd_filter<T96x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x256"); break;
+      case 96:
+        e = plan.bn == 128 ? run_bwd_filter<T96x128>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x128")
+                           : run_bwd_filter<T96x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x256");
+        break;
       case 64:  e = run_bwd_filter<T64x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_64x256"); break;
       default:  e = run_bwd_filter<T32x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x256"); break;
     }

@@ -105,6 +105,7 @@ inline int launch_mfma_gemm_bf16(const typename AL::Params& ap, const typename B
 // Tile shapes in use.  rows x cols x k, waves as WM x WN.
 typedef Tile<128, 128, 16, 2, 2, RH_OCC_128> T128x128;
 typedef Tile<96, 256, 16, 1, 4> T96x256;
+typedef Tile<96, 128, 16, 1, 4, 4> T96x128;
 typedef Tile<64, 256, 16, 1, 4> T64x256;
 typedef Tile<32, 256, 16, 1, 4> T32x256;
 

@@ -25,6 +25,36 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, float* sink) 
   if (s == 123.456f) sink[0] = s;  // keeps the loop alive; never true in practice
 }
 
+// Same loop with operands that differ per lane and per instruction (8 A and 8 B registers of pseudo-random
+// values in [-2, 2), rotated through): the data toggling of a real contraction, hence its power draw, which the
+// constant-operand loop above does not have.
+__global__ __launch_bounds__(256) void mfma_loop_varied_kernel(int iters, float* sink) {
+  f32x16 acc[8];
+  float a[8], b[8];
+  uint32_t h = (threadIdx.x + 1u) * 2654435761u ^ (blockIdx.x + 1u) * 40503u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    h = h * 1664525u + 1013904223u;
+    a[i] = (float)(int)(h >> 8) * (1.0f / 4194304.0f) - 2.0f;
+    h = h * 1664525u + 1013904223u;
+    b[i] = (float)(int)(h >> 8) * (1.0f / 4194304.0f) - 2.0f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][v] = a[i] * (float)v;
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[(i * 3 + 1) & 7], acc[i], 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[(i + 5) & 7], b[i], acc[i], 0, 0, 0);
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s += acc[i][v];
+  if (s == 123.456f) sink[0] = s;
+}
+
 __global__ void copy_kernel(const float4* __restrict__ src, float4* __restrict__ dst, long long n4) {
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
@@ -42,6 +72,14 @@ extern "C" int rh_probe_mfma_loop(int blocks, int nacc, int iters, float* sink, 
   if (nacc == 4) hipLaunchKernelGGL(mfma_loop_kernel<4>, dim3(blocks), dim3(256), 0, to_stream(stream), iters, sink);
   else if (nacc == 8) hipLaunchKernelGGL(mfma_loop_kernel<8>, dim3(blocks), dim3(256), 0, to_stream(stream), iters, sink);
   else return RH_E_INVALID;
+  return launch_status();
+}
+
+// Launches blocks x 256 threads; every wave issues iters * 16 MFMAs on varied operands.
+extern "C" int rh_probe_mfma_loop_varied(int blocks, int iters, float* sink, rh_stream_t stream) {
+  if (blocks <= 0 || iters <= 0 || !sink) return RH_E_INVALID;
+  ProfScope prof("probe_mfma_varied", (double)blocks * 4.0 * iters * 16 * 4096.0, to_stream(stream));
+  hipLaunchKernelGGL(mfma_loop_varied_kernel, dim3(blocks), dim3(256), 0, to_stream(stream), iters, sink);
   return launch_status();
 }
 
