@@ -102,7 +102,7 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
     ep.rows = d.C; ep.cols = bp.M; ep.inner = d.H * d.W; ep.ld = 0; ep.relu = 0; ep.split_stride = 0;
     switch (pick_bm(d.C)) {
       case 128: return run_bwd_data_soff<T128x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_128x128");
-      case 96:  return run_bwd_data_soff<T96x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_96x256");
+      case 96:  return run_bwd_data_soff<T96x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_96x128");
       case 64:  return run_bwd_data_soff<T64x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_64x256");
       default:  return run_bwd_data_soff<T32x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_32x256");
     }

@@ -49,14 +49,29 @@ static BwdFilterPlan plan_bwd_filter(const ConvDims& d) {
   return p;
 }
 
+// Sum of part[s*stride + idx] over s < splits in a fixed order: four interleaved partial sums (so that four
+// loads are in flight per thread), combined as (a0 + a1) + (a2 + a3).
+__device__ __forceinline__ float sum_splits(const float* __restrict__ part, int splits, long long stride, unsigned idx) {
+  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+  const float* p = part + idx;
+  int s = 0;
+  for (; s + 3 < splits; s += 4) {
+    a0 += p[(long long)s * stride];
+    a1 += p[(long long)(s + 1) * stride];
+    a2 += p[(long long)(s + 2) * stride];
+    a3 += p[(long long)(s + 3) * stride];
+  }
+  for (; s < splits; ++s) a0 += p[(long long)s * stride];
+  return (a0 + a1) + (a2 + a3);
+}
+
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
 __global__ void split_reduce_kernel(const float* __restrict__ part, int splits, long long split_stride,
                                     float* __restrict__ out, int rows, int cols, int ld, float alpha,
                                     float beta) {
   const unsigned total = (unsigned)rows * (unsigned)cols;  // a filter gradient / GEMM result: far below 2^31
   for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
-    float acc = 0.0f;
-    for (int s = 0; s < splits; ++s) acc += part[(long long)s * split_stride + idx];
+    const float acc = sum_splits(part, splits, split_stride, idx);
     const int i = (int)(idx / (unsigned)cols), j = (int)(idx - (unsigned)i * (unsigned)cols);
     float* dst = out + (size_t)i * ld + j;
     float val = alpha * acc;
@@ -180,8 +195,7 @@ __global__ void split_reduce_rsc_kernel(const float* __restrict__ part, int spli
   const int CRS = C * R * S;
   const unsigned total = (unsigned)K * (unsigned)CRS;
   for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
-    float acc = 0.0f;
-    for (int sp = 0; sp < splits; ++sp) acc += part[(long long)sp * split_stride + idx];
+    const float acc = sum_splits(part, splits, split_stride, idx);
     const int ko = (int)(idx / (unsigned)CRS), j = (int)(idx - (unsigned)ko * (unsigned)CRS);
     const int r = j / (S * C), rem = j - r * (S * C), s2 = rem / C, c = rem - s2 * C;
     float* dst = dw + (((size_t)ko * C + c) * R + r) * S + s2;
@@ -255,6 +269,51 @@ __global__ __launch_bounds__(256) void bwd_bias_rowsum_kernel(const float* __res
     if (lane == 0) rowsum[r] = acc;
   }
 }
+
+// Small planes (13x13, 27x27): dy viewed as an [N][K*plane] matrix; block column (j, g) adds images n = g, g+G, ...
+// for 256 consecutive j, fully coalesced: part[g][j].  bwd_bias_planes_finish_kernel then adds, per channel, the G
+// partial planes in a fixed order.
+__global__ __launch_bounds__(256) void bwd_bias_colsum_kernel(const float* __restrict__ dy, int N, int KP,
+                                                              float* __restrict__ part) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  const int g = blockIdx.y, G = gridDim.y;
+  if (j >= KP) return;
+  float a0 = 0.0f, a1 = 0.0f;
+  int n = g;
+  for (; n + G < N; n += 2 * G) {
+    a0 += dy[(size_t)n * KP + j];
+    a1 += dy[(size_t)(n + G) * KP + j];
+  }
+  if (n < N) a0 += dy[(size_t)n * KP + j];
+  part[(size_t)g * KP + j] = a0 + a1;
+}
+
+__global__ __launch_bounds__(256) void bwd_bias_planes_finish_kernel(const float* __restrict__ part, int G, int KP, int plane,
+                                                                     float alpha, float beta, float* __restrict__ db) {
+  const int k = blockIdx.x;
+  float acc = 0.0f;
+  for (int g = 0; g < G; ++g) {
+    const float* p = part + (size_t)g * KP + (size_t)k * plane;
+    for (int i = threadIdx.x; i < plane; i += 256) acc += p[i];
+  }
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
+  __shared__ float sm[4];
+  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float v = alpha * ((sm[0] + sm[1]) + (sm[2] + sm[3]));
+    if (beta != 0.0f) v += beta * db[k];
+    db[k] = v;
+  }
+}
+
+static int bwd_bias_col_groups(int N, long long KP) {
+  long long G = cdiv<long long>(1 << 20, KP);
+  if (G > 16) G = 16;
+  if (G > N) G = N;
+  return G < 1 ? 1 : (int)G;
+}
+constexpr int kBiasSmallPlane = 1024;  // below: column form; from here on: one wave per (n, k) row
 
 // Column sums of an [N][K] matrix (dy of an affine layer, or the row sums above): a block covers 64
 // columns; its 4 waves take every fourth row and are combined through LDS in a fixed order.
@@ -407,6 +466,7 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
 
 extern "C" size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane) {
   if (N <= 0 || K <= 0 || plane <= 1) return 0;
+  if (plane < kBiasSmallPlane) return align256(sizeof(float) * (size_t)bwd_bias_col_groups(N, (long long)K * plane) * K * plane);
   return align256(sizeof(float) * (size_t)N * K);
 }
 
@@ -419,6 +479,13 @@ extern "C" int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float 
   float* rowsum = static_cast<float*>(ws);
   const long long rows = (long long)N * K;
   ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
+  if (plane < kBiasSmallPlane && (long long)K * plane < (1ll << 31)) {
+    const int KP = K * plane, G = bwd_bias_col_groups(N, KP);
+    hipLaunchKernelGGL(bwd_bias_colsum_kernel, dim3(cdiv(KP, 256), G), dim3(256), 0, stream, dy, N, KP, rowsum);
+    if (int e = launch_status()) return e;
+    hipLaunchKernelGGL(bwd_bias_planes_finish_kernel, dim3(K), dim3(256), 0, stream, rowsum, G, KP, plane, alpha, beta, db);
+    return launch_status();
+  }
   const long long blocks = cdiv<long long>(rows, 4);
   hipLaunchKernelGGL(bwd_bias_rowsum_kernel, dim3((unsigned)(blocks > 65536 ? 65536 : blocks)), dim3(256), 0, stream, dy,
                      rows, plane, rowsum);

@@ -145,7 +145,7 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
     if (flags & RH_MATH_BF16_MFMA_FP32ACC) return run_fwd_soff_bf16(ap, bp, ep, sp.n_k, CRS, stream);
     switch (pick_bm(d.K)) {
       case 128: return run_fwd_soff<T128x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_128x128");
-      case 96:  return run_fwd_soff<T96x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_96x256");
+      case 96:  return run_fwd_soff<T96x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_96x128");
       case 64:  return run_fwd_soff<T64x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x256");
       default:  return run_fwd_soff<T32x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_32x256");
     }

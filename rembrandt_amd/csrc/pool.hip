@@ -83,6 +83,62 @@ __global__ void pool_fwd_kernel(PoolDims d, const float* __restrict__ x, float* 
   }
 }
 
+// Forward with the input planes of a block staged in LDS: PB consecutive (n, c) planes are read with coalesced
+// loads, windows are scanned in LDS (overlapping windows re-read LDS, not L1), and y / arg-max are written
+// coalesced.  Same arithmetic and tie rule as pool_fwd_kernel.
+__global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv dPQ, int PB, long long planes,
+                                                           const float* __restrict__ x, float* __restrict__ y,
+                                                           int* __restrict__ argmax) {
+  extern __shared__ float lds_pool[];
+  const int HW = d.H * d.W, PQ = d.P * d.Q;
+  const long long plane0 = (long long)blockIdx.x * PB;
+  const int np = (int)(planes - plane0 < PB ? planes - plane0 : PB);
+  const float* gx = x + plane0 * HW;
+  const int n_in = np * HW, n_out = np * PQ;
+  // The staged copy keeps the global address's position inside a 16-byte group, so that the body of the copy
+  // is float4 on both sides whatever the plane size (55*55 floats is not a multiple of four).
+  const int phase = (int)((reinterpret_cast<uintptr_t>(gx) >> 2) & 3);
+  float* const sx = lds_pool + phase;
+  const int head = (4 - phase) & 3;
+  {
+    const int h = head < n_in ? head : n_in;
+    if ((int)threadIdx.x < h) sx[threadIdx.x] = gx[threadIdx.x];
+    const int n4 = (n_in - h) >> 2;
+    const float4* g4 = reinterpret_cast<const float4*>(gx + h);
+    float4* s4 = reinterpret_cast<float4*>(sx + h);
+    for (int i = threadIdx.x; i < n4; i += 256) s4[i] = g4[i];
+    for (int i = h + (n4 << 2) + threadIdx.x; i < n_in; i += 256) sx[i] = gx[i];
+  }
+  __syncthreads();
+  float* gy = y + plane0 * PQ;
+  int* gm = argmax ? argmax + plane0 * PQ : nullptr;
+  const float inv = 1.0f / (float)(d.k * d.k);
+  for (int o = threadIdx.x; o < n_out; o += 256) {
+    uint32_t pl, pq, p, q;
+    dPQ.divmod((uint32_t)o, pl, pq);
+    d.dQ.divmod(pq, p, q);
+    const float* xp = sx + pl * HW;
+    if (d.mode == RH_POOL_MAX) {
+      float best;
+      const int bi = window_argmax(xp, d.H, d.W, (int)p, (int)q, d.k, d.st, d.pad, &best);
+      gy[o] = bi < 0 ? 0.0f : best;
+      if (gm) gm[o] = bi;
+    } else {
+      float acc = 0.0f;
+      const int hs = (int)p * d.st - d.pad, ws = (int)q * d.st - d.pad;
+      for (int r = 0; r < d.k; ++r) {
+        const int h = hs + r;
+        if ((unsigned)h >= (unsigned)d.H) continue;
+        for (int s2 = 0; s2 < d.k; ++s2) {
+          const int w = ws + s2;
+          if ((unsigned)w < (unsigned)d.W) acc += xp[h * d.W + w];
+        }
+      }
+      gy[o] = acc * inv;
+    }
+  }
+}
+
 template <class I>
 __global__ void pool_bwd_kernel(PoolDims d, const float* __restrict__ x, const float* __restrict__ dy,
                                 float* __restrict__ dx, const int* __restrict__ argmax) {
@@ -153,7 +209,7 @@ __global__ __launch_bounds__(256) void pool_bwd_mask_lds_kernel(PoolDims d, Fast
   for (int i = threadIdx.x; i < n_out; i += 256) { sdy[i] = gdy[i]; smask[i] = gm[i]; }
   __syncthreads();
   float* gdx = dx + plane0 * HW;
-  for (int e = threadIdx.x; e < n_in; e += 256) {
+  auto value = [&](int e) -> float {
     uint32_t pl, hw, h, w;
     dHW.divmod((uint32_t)e, pl, hw);
     d.dW.divmod(hw, h, w);
@@ -170,8 +226,24 @@ __global__ __launch_bounds__(256) void pool_bwd_mask_lds_kernel(PoolDims d, Fast
         const int o = base + p * d.Q + q;
         if (smask[o] == (int)hw) acc += sdy[o];
       }
-    gdx[e] = acc;
+    return acc;
+  };
+  // four consecutive elements per thread and one 16-byte store, after a scalar head up to the first aligned address
+  const int phase = (int)((reinterpret_cast<uintptr_t>(gdx) >> 2) & 3);
+  const int head = ((4 - phase) & 3) < n_in ? ((4 - phase) & 3) : n_in;
+  if ((int)threadIdx.x < head) gdx[threadIdx.x] = value((int)threadIdx.x);
+  const int n4 = (n_in - head) >> 2;
+  float4* g4 = reinterpret_cast<float4*>(gdx + head);
+  for (int g = threadIdx.x; g < n4; g += 256) {
+    const int e = head + 4 * g;
+    float4 v;
+    v.x = value(e);
+    v.y = value(e + 1);
+    v.z = value(e + 2);
+    v.w = value(e + 3);
+    g4[g] = v;
   }
+  for (int e = head + (n4 << 2) + threadIdx.x; e < n_in; e += 256) gdx[e] = value(e);
 }
 
 static int pool_dims(const rh_pool_geom* g, PoolDims* d) {
@@ -212,6 +284,21 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
   ProfScope prof(d.mode == RH_POOL_MAX ? "pool_max_fwd" : "pool_avg_fwd",
                  4.0 * ((double)d.N * d.C * d.H * d.W + (double)total * (opt_argmax ? 2 : 1)), to_stream(stream));
   const long long in_total = (long long)d.N * d.C * d.H * d.W;
+  // about 16 KB of input planes per block (measured best: more LDS per block leaves too few blocks per CU to
+  // overlap one block's loads with another's window scans); a single larger plane still goes through LDS
+  constexpr int kLdsFloats = 4096;
+  if (d.H * d.W <= 12288 && d.P * d.Q > 0) {
+    int PB = kLdsFloats / (d.H * d.W);
+    if (PB < 1) PB = 1;
+    if (PB > 64) PB = 64;
+    const long long planes = (long long)d.N * d.C;
+    const long long blocks = cdiv<long long>(planes, PB);
+    if (blocks < (1ll << 31) && (long long)PB * d.P * d.Q < (1ll << 31)) {
+      hipLaunchKernelGGL(pool_fwd_lds_kernel, dim3((unsigned)blocks), dim3(256), ((size_t)PB * d.H * d.W + 4) * sizeof(float),
+                         to_stream(stream), d, FastDiv((uint32_t)(d.P * d.Q)), PB, planes, x, y, opt_argmax);
+      return launch_status();
+    }
+  }
   const dim3 grid((unsigned)cdiv<long long>(total, 256) > (1u << 20) ? (1u << 20) : (unsigned)cdiv<long long>(total, 256));
   if (total < (1ll << 31) && in_total < (1ll << 31))
     hipLaunchKernelGGL(pool_fwd_kernel<unsigned>, grid, dim3(256), 0, to_stream(stream), d, x, y, opt_argmax);
