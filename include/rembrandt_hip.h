@@ -165,6 +165,14 @@ int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, int32_t* opt_
                   rh_stream_t stream);
 int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float* y, const float* dy, float* dx,
                   const int32_t* opt_argmax, rh_stream_t stream);
+/* Max-pool backward with the backward mask of the ReLU that produced x folded in (the pair K9' + K4 of
+ * Pool2dOperator::backward followed by the producer's rect_backprop, src/operator/mod.rs:2113-2121, 1731-1738):
+ * dx = [x > 0] * pool_bwd(dy).  x is not read: an arg-max element carries x = y, so windows with y <= 0 route
+ * nothing.  Needs the arg-max mask of the forward pass; rh_pool2d_bwd_relu_supported says whether the geometry is
+ * covered (else use rh_pool2d_bwd and the separate ReLU kernel). */
+int rh_pool2d_bwd_relu_supported(const rh_pool_geom* g);
+int rh_pool2d_bwd_relu(const rh_pool_geom* g, const float* y, const float* dy, float* dx, const int32_t* argmax,
+                       rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Softmax / KL loss / reductions.  rh_softmax_fwd replaces CudnnSoftmaxOp::forward

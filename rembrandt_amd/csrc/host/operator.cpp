@@ -676,7 +676,8 @@ class Conv2dOperator : public Operator {
     RB_ASSERT(batch_size <= batch_cap_);
     const rh_conv_geom g = geom(batch_size);
     rh_stream_t s = context_->stream();
-    apply_rect_backprop(config_.act_func, out_act_->as_ptr(), out_dims_.len(), batch_size, out_delta_->as_mut_ptr(), s);
+    if (!act_bwd_folded_)
+      apply_rect_backprop(config_.act_func, out_act_->as_ptr(), out_dims_.len(), batch_size, out_delta_->as_mut_ptr(), s);
     unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in_act_->as_ptr(), out_delta_->as_ptr(), 1.0f, params_.grad_weights->as_mut_ptr(),
                                 workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward filter");
     unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), 1.0f,
@@ -705,8 +706,14 @@ class Conv2dOperator : public Operator {
     return params_.buffer(which, ptr, len);
   }
   const char* kind() const override { return "Conv2dOperator"; }
+  bool fold_activation_backward() override {
+    if (config_.act_func != ActivationFunction::Rect) return false;
+    act_bwd_folded_ = true;
+    return true;
+  }
 
  private:
+  bool act_bwd_folded_ = false;
   rh_conv_geom geom(size_t batch) const {
     rh_conv_geom g;
     g.N = (int)batch; g.C = (int)config_.in_dims.c; g.H = (int)config_.in_dims.h; g.W = (int)config_.in_dims.w;
@@ -727,7 +734,7 @@ class Conv2dOperator : public Operator {
 // ---- Pool2dOperator -------------------------------------------------------------------------------------
 class Pool2dOperator : public Operator {
  public:
-  Pool2dOperator(size_t batch_size, const Pool2dOperatorConfig& config, const Operator* prev_op, Ctx context)
+  Pool2dOperator(size_t batch_size, const Pool2dOperatorConfig& config, Operator* prev_op, Ctx context, const ExecOptions& opts)
       : batch_cap_(batch_size), config_(config), context_(context) {
     RB_ASSERT(prev_op != nullptr);
     in_act_ = prev_op->get_output_vars();
@@ -738,8 +745,11 @@ class Pool2dOperator : public Operator {
     out_act_.reset(new DeviceBuffer<float>(out_dims_.len() * batch_size, context));
     out_delta_.reset(new DeviceBuffer<float>(out_dims_.len() * batch_size, context));
     // private arg-max mask: lets backward route deltas without re-scanning the windows
-    if (config.pool_op == PoolOperation::Max && in_delta_)
+    if (config.pool_op == PoolOperation::Max && in_delta_) {
       argmax_.reset(new DeviceBuffer<int32_t>(out_dims_.len() * batch_size, context));
+      const rh_pool_geom g = geom(batch_size);
+      if (opts.fuse_epilogue && rh_pool2d_bwd_relu_supported(&g)) fold_relu_ = prev_op->fold_activation_backward();
+    }
   }
   size_t batch_size() const override { return batch_cap_; }
   SharedDeviceBuf get_output_vars() const override { return out_act_; }
@@ -754,6 +764,11 @@ class Pool2dOperator : public Operator {
     if (!in_delta_) return;
     RB_ASSERT(batch_size <= batch_cap_);
     const rh_pool_geom g = geom(batch_size);
+    if (fold_relu_) {
+      unwrap(rh_pool2d_bwd_relu(&g, out_act_->as_ptr(), out_delta_->as_ptr(), in_delta_->as_mut_ptr(), argmax_->as_ptr(),
+                                context_->stream()), "pooling backward");
+      return;
+    }
     unwrap(rh_pool2d_bwd(&g, in_act_->as_ptr(), out_act_->as_ptr(), out_delta_->as_ptr(), in_delta_->as_mut_ptr(),
                          argmax_ ? argmax_->as_ptr() : nullptr, context_->stream()), "pooling backward");
   }
@@ -779,6 +794,7 @@ class Pool2dOperator : public Operator {
   Dims3 out_dims_;
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   std::unique_ptr<DeviceBuffer<int32_t>> argmax_;
+  bool fold_relu_ = false;  // backward also applies the producer's ReLU mask
 };
 
 // ---- DropoutOperator (src/operator/mod.rs:2134-2255) -------------------------------------------------------
@@ -1002,14 +1018,14 @@ SequentialOperatorWorker::SequentialOperatorWorker(const SequentialOperatorConfi
   if (!config.has_loss) panic("SequentialOperatorWorker: missing loss operator");
   const uint64_t input_seed[2] = {shared_seed[0] ^ 0x44617461336421ull, shared_seed[1] + 0x9E3779B97F4A7C15ull};
   input_op_.reset(new Data3dOperator(batch_size, config.input_op.data3d, context, input_seed));
-  const Operator* prev = input_op_.get();
+  Operator* prev = input_op_.get();
   size_t params_off = 0;
   for (const auto& c : config.hidden_ops) {
     std::unique_ptr<Operator> op;
     switch (c.kind) {
       case OperatorConfig::Affine: op.reset(new AffineOperator(batch_size, capability, c.affine, prev, context)); break;
       case OperatorConfig::Conv2d: op.reset(new Conv2dOperator(batch_size, capability, c.conv2d, prev, context, opts)); break;
-      case OperatorConfig::Pool2d: op.reset(new Pool2dOperator(batch_size, c.pool2d, prev, context)); break;
+      case OperatorConfig::Pool2d: op.reset(new Pool2dOperator(batch_size, c.pool2d, prev, context, opts)); break;
       case OperatorConfig::Dropout:
         op.reset(new DropoutOperator(batch_size, c.dropout, prev, context, shared_seed[0] ^ (shared_seed[1] << 32 | shared_seed[1] >> 32),
                                      0xD0000000ull + hidden_ops_.size()));

@@ -213,6 +213,10 @@ class Operator {
   // Fused regularize -> accumulate_grads(scale, momentum) -> update_params(apply) -> reset in
   // one pass per tensor (same arithmetic, 24 instead of 52 bytes per parameter).
   virtual void fused_sgd_step(float /*l2*/, float /*scale*/, float /*momentum*/, float /*apply*/) {}
+  // A consumer that can apply this operator's activation backward mask itself (max-pool backward folds the ReLU
+  // mask) asks for it at construction; an operator that agrees skips its own mask pass in backward().  The
+  // out_delta buffer holds the same values after the chain's backward either way.
+  virtual bool fold_activation_backward() { return false; }
   // Parameter / optimizer-state blobs: a sequence of serialised NdArrays (weights then bias; for the state the
   // momentum buffers).  decode_* return the number of bytes consumed (src/operator/mod.rs:1008-1073).
   virtual void encode_params(std::vector<uint8_t>& /*blob*/) {}

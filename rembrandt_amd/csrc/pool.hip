@@ -194,9 +194,11 @@ __global__ void pool_bwd_kernel(PoolDims d, const float* __restrict__ x, const f
 // Max-pool backward driven by the arg-max mask, one block per group of PB consecutive planes: the
 // group's dy and mask (PB*P*Q values each) are staged in LDS with coalesced reads, then every input
 // element looks its covering windows up in LDS and dx is written coalesced.  No dependent global loads.
+// With `y` (the pooled outputs) the backward mask of a ReLU that produced x is folded in: an arg-max element
+// carries x = y, so "dx = 0 where x <= 0" is "skip windows whose maximum y is <= 0".
 __global__ __launch_bounds__(256) void pool_bwd_mask_lds_kernel(PoolDims d, FastDiv dHW, int PB, long long planes,
                                                                 const float* __restrict__ dy, const int* __restrict__ argmax,
-                                                                float* __restrict__ dx) {
+                                                                const float* __restrict__ y, float* __restrict__ dx) {
   extern __shared__ float lds_pool[];
   const int PQ = d.P * d.Q, HW = d.H * d.W;
   const long long plane0 = (long long)blockIdx.x * PB;
@@ -206,7 +208,12 @@ __global__ __launch_bounds__(256) void pool_bwd_mask_lds_kernel(PoolDims d, Fast
   const int n_out = np * PQ, n_in = np * HW;
   const float* gdy = dy + plane0 * PQ;
   const int* gm = argmax + plane0 * PQ;
-  for (int i = threadIdx.x; i < n_out; i += 256) { sdy[i] = gdy[i]; smask[i] = gm[i]; }
+  if (y) {  // a window whose maximum is not positive routes nothing: give it an index no element has
+    const float* gy = y + plane0 * PQ;
+    for (int i = threadIdx.x; i < n_out; i += 256) { sdy[i] = gdy[i]; smask[i] = gy[i] > 0.0f ? gm[i] : -1; }
+  } else {
+    for (int i = threadIdx.x; i < n_out; i += 256) { sdy[i] = gdy[i]; smask[i] = gm[i]; }
+  }
   __syncthreads();
   float* gdx = dx + plane0 * HW;
   auto value = [&](int e) -> float {
@@ -307,6 +314,39 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
   return launch_status();
 }
 
+static bool lds_bwd_ok(const PoolDims& d) { return d.P * d.Q <= 2048 && d.H * d.W <= (1 << 20); }
+
+static int launch_pool_bwd_lds(const PoolDims& d, const float* dy, const int32_t* argmax, const float* relu_y, float* dx,
+                               rh_stream_t stream) {
+  const int PQ = d.P * d.Q;
+  int PB = 2048 / PQ;
+  if (PB > 64) PB = 64;
+  const long long planes = (long long)d.N * d.C;
+  const long long blocks = cdiv<long long>(planes, PB);
+  if (blocks >= (1ll << 31)) return RH_E_LIMIT;
+  hipLaunchKernelGGL(pool_bwd_mask_lds_kernel, dim3((unsigned)blocks), dim3(256), (size_t)PB * PQ * 8, to_stream(stream), d,
+                     FastDiv((uint32_t)(d.H * d.W)), PB, planes, dy, argmax, relu_y, dx);
+  return launch_status();
+}
+
+extern "C" int rh_pool2d_bwd_relu_supported(const rh_pool_geom* g) {
+  PoolDims d;
+  if (pool_dims(g, &d)) return 0;
+  return d.mode == RH_POOL_MAX && lds_bwd_ok(d) && (long long)d.N * d.C < (1ll << 31) ? 1 : 0;
+}
+
+extern "C" int rh_pool2d_bwd_relu(const rh_pool_geom* g, const float* y, const float* dy, float* dx, const int32_t* argmax,
+                                  rh_stream_t stream) {
+  PoolDims d;
+  if (int e = pool_dims(g, &d)) return e;
+  if (!y || !dy || !dx || !argmax) return RH_E_INVALID;
+  if (!rh_pool2d_bwd_relu_supported(g)) return RH_E_UNSUPPORTED;
+  const double in_elems = (double)d.N * d.C * d.H * d.W, out_elems = (double)d.N * d.C * d.P * d.Q;
+  if (in_elems == 0) return 0;
+  ProfScope prof("pool_max_bwd_relu", 4.0 * (in_elems + 3.0 * out_elems), to_stream(stream));
+  return launch_pool_bwd_lds(d, dy, argmax, y, dx, stream);
+}
+
 extern "C" int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float* y, const float* dy, float* dx,
                              const int32_t* opt_argmax, rh_stream_t stream) {
   (void)y;
@@ -319,18 +359,8 @@ extern "C" int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float*
   // bytes: write dx, read dy, plus the arg-max mask or (max without mask) x itself
   const double bwd_bytes = 4.0 * ((double)total + out_elems + (d.mode == RH_POOL_MAX ? (opt_argmax ? out_elems : (double)total) : 0.0));
   ProfScope prof(d.mode == RH_POOL_MAX ? "pool_max_bwd" : "pool_avg_bwd", bwd_bytes, to_stream(stream));
-  if (d.mode == RH_POOL_MAX && opt_argmax && d.P * d.Q <= 2048 && d.H * d.W <= (1 << 20)) {
-    const int PQ = d.P * d.Q;
-    int PB = 2048 / PQ;
-    if (PB > 64) PB = 64;
-    const long long planes = (long long)d.N * d.C;
-    const long long blocks = cdiv<long long>(planes, PB);
-    if (blocks < (1ll << 31)) {
-      hipLaunchKernelGGL(pool_bwd_mask_lds_kernel, dim3((unsigned)blocks), dim3(256), (size_t)PB * PQ * 8, to_stream(stream), d,
-                         FastDiv((uint32_t)(d.H * d.W)), PB, planes, dy, opt_argmax, dx);
-      return launch_status();
-    }
-  }
+  if (d.mode == RH_POOL_MAX && opt_argmax && lds_bwd_ok(d) && (long long)d.N * d.C < (1ll << 31))
+    return launch_pool_bwd_lds(d, dy, opt_argmax, nullptr, dx, stream);
   const dim3 grid((unsigned)cdiv<long long>(total, 256) > (1u << 20) ? (1u << 20) : (unsigned)cdiv<long long>(total, 256));
   if (total < (1ll << 31))
     hipLaunchKernelGGL(pool_bwd_kernel<unsigned>, grid, dim3(256), 0, to_stream(stream), d, x, dy, dx, opt_argmax);

@@ -167,6 +167,14 @@ def pool2d_bwd(x, y, dy, size, stride, pad, mode, rounding=_lib.RH_ROUND_FLOOR, 
     return dx
 
 
+def pool2d_bwd_relu(x_shape, y, dy, size, stride, pad, argmax, rounding=_lib.RH_ROUND_FLOOR):
+    """Max-pool backward with the producer's ReLU backward mask folded in."""
+    g = pool_geom(x_shape, size, stride, pad, _lib.RH_POOL_MAX, rounding)
+    dx = torch.empty(tuple(x_shape), dtype=torch.float32, device=dy.device)
+    check(lib().rh_pool2d_bwd_relu(C.byref(g), _p(y), _p(dy), _p(dx), _p(argmax), _stream()), "rh_pool2d_bwd_relu")
+    return dx
+
+
 def softmax_fwd(x):
     N, Cc = x.shape
     p = torch.empty_like(x)

@@ -316,3 +316,27 @@ def test_lrn(dev, case):
     dx = ops.lrn_bwd(T(x, dev), y, d, T(dy, dev), size, scale, power, min_div)
     assert_close(N(dx), O.lrn_bwd(x, dy, size, scale, power, min_div), "lrn bwd")
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("case", [(2, 3, 9, 3, 2, 0), (2, 3, 9, 3, 2, 1), (3, 4, 8, 2, 2, 0), (2, 5, 27, 3, 2, 0), (2, 2, 13, 3, 3, 1)])
+@pytest.mark.parametrize("rounding", [_lib.RH_ROUND_FLOOR, _lib.RH_ROUND_CEIL])
+def test_pool2d_bwd_with_folded_relu_mask(dev, case, rounding):
+    """rh_pool2d_bwd_relu == max-pool backward followed by the ReLU backward mask of the pool's input
+    (Pool2dOperator::backward then the producer's rect_backprop), on inputs with whole windows of zeros."""
+    Nn, C, H, k, st, pad = case
+    say("pool bwd + relu case", case, rounding)
+    x = O.rect_inplace(synth.normal(16, 1, (Nn, C, H, H)) - np.float32(0.8))     # ~80 % zeros: some windows are all zero
+    xd = T(x, dev)
+    y, am = ops.pool2d_fwd(xd, k, st, pad, _lib.RH_POOL_MAX, rounding, want_argmax=True)
+    assert (N(y) == 0).any() and (N(y) > 0).any()
+    dy = synth.normal(16, 2, tuple(y.shape))
+    want = O.pool2d_bwd(x, N(y), dy, k, st, pad, O.POOL_MAX, rounding)
+    O.rect_backprop_inplace(x, want)
+    got = N(ops.pool2d_bwd_relu(x.shape, y, T(dy, dev), k, st, pad, am, rounding))
+    assert np.array_equal(got == 0, want == 0), "same elements are masked"
+    assert_close(got, want, "pool bwd with folded relu mask")    # elements fed by several windows add in another order
+    # and it is bit-identical to the two GPU kernels it replaces
+    two = ops.pool2d_bwd(xd, y, T(dy, dev), k, st, pad, _lib.RH_POOL_MAX, rounding, argmax=am)
+    ops.rect_backprop_inplace(xd, two)
+    assert np.array_equal(got, N(two))
+    torch.cuda.synchronize()
