@@ -20,8 +20,9 @@ static SgemmPlan plan_sgemm(int m, int n, int k) {
   const int tiles = cdiv(n, p.bm) * cdiv(m, p.bn);
   const int k_chunks = cdiv(k, 16);
   int want = 1;
-  if (tiles < 384) {
-    want = cdiv(768, tiles);
+  const int slots = 256 * (p.bm == 128 ? RH_OCC_128 : 3);  // blocks of this tile the GPU holds at a time
+  if (tiles <= slots / 2) {
+    want = slots / tiles;
     const int max_by_depth = k_chunks / 16 > 0 ? k_chunks / 16 : 1;
     if (want > max_by_depth) want = max_by_depth;
     if (want > 64) want = 64;
@@ -30,31 +31,61 @@ static SgemmPlan plan_sgemm(int m, int n, int k) {
   return p;
 }
 
-template <class T, bool B_TRANS, bool A_TRANS>
+// A rows-contiguous dense operand seen by the scalar-offset loader: lane offset = row, wave-uniform offset = k*ld.
+// Used only when k is a multiple of the K step: the scalar offset takes no part in the buffer range check, so a
+// K tail must not be read this way.
+static RowSParams rows_params(const DenseParams& d) {
+  RowSParams r;
+  r.ptr = d.ptr; r.bytes = d.bytes;
+  r.M = d.rows; r.inner = d.rows > 0 ? d.rows : 1; r.innerW = r.inner;
+  r.img_stride = 0; r.a_stride = 0; r.b_stride = 1;
+  r.soff = nullptr; r.ldk4 = d.ld * 4;
+  return r;
+}
+
+template <class T, bool B_TRANS, bool A_TRANS, bool RS>
 static int run_sgemm(const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k, int splits,
                      int* used, hipStream_t stream, const char* tag) {
   // engine A operand = opB: k contiguous unless transB; engine B operand = opA: rows contiguous unless transA
-  if constexpr (!B_TRANS && !A_TRANS)
-    return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseR<T::BN, T::BK, T::NT>, false, PassSgemm>(
-        ap, bp, ep, k, splits, used, stream, tag);
-  else if constexpr (!B_TRANS && A_TRANS)
-    return launch_mfma_gemm<T, LoadDenseK<T::BM, T::BK, T::NT, false>, LoadDenseK<T::BN, T::BK, T::NT, false>, false, PassSgemm>(
-        ap, bp, ep, k, splits, used, stream, tag);
-  else if constexpr (B_TRANS && !A_TRANS)
-    return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseR<T::BN, T::BK, T::NT>, false, PassSgemm>(
-        ap, bp, ep, k, splits, used, stream, tag);
-  else
-    return launch_mfma_gemm<T, LoadDenseR<T::BM, T::BK, T::NT>, LoadDenseK<T::BN, T::BK, T::NT, false>, false, PassSgemm>(
-        ap, bp, ep, k, splits, used, stream, tag);
+  typedef LoadDenseK<T::BM, T::BK, T::NT, false> AK;
+  typedef LoadDenseK<T::BN, T::BK, T::NT, false> BK_;
+  if constexpr (RS) {
+    typedef LoadRowS<T::BM, T::BK, T::NT, true> AR;
+    typedef LoadRowS<T::BN, T::BK, T::NT, true> BR;
+    if constexpr (!B_TRANS && !A_TRANS)
+      return launch_mfma_gemm<T, AK, BR, false, PassSgemm>(ap, rows_params(bp), ep, k, splits, used, stream, tag);
+    else if constexpr (!B_TRANS && A_TRANS)
+      return launch_mfma_gemm<T, AK, BK_, false, PassSgemm>(ap, bp, ep, k, splits, used, stream, tag);
+    else if constexpr (B_TRANS && !A_TRANS)
+      return launch_mfma_gemm<T, AR, BR, false, PassSgemm>(rows_params(ap), rows_params(bp), ep, k, splits, used, stream, tag);
+    else
+      return launch_mfma_gemm<T, AR, BK_, false, PassSgemm>(rows_params(ap), bp, ep, k, splits, used, stream, tag);
+  } else {
+    typedef LoadDenseR<T::BM, T::BK, T::NT> AR;
+    typedef LoadDenseR<T::BN, T::BK, T::NT> BR;
+    if constexpr (!B_TRANS && !A_TRANS)
+      return launch_mfma_gemm<T, AK, BR, false, PassSgemm>(ap, bp, ep, k, splits, used, stream, tag);
+    else if constexpr (!B_TRANS && A_TRANS)
+      return launch_mfma_gemm<T, AK, BK_, false, PassSgemm>(ap, bp, ep, k, splits, used, stream, tag);
+    else if constexpr (B_TRANS && !A_TRANS)
+      return launch_mfma_gemm<T, AR, BR, false, PassSgemm>(ap, bp, ep, k, splits, used, stream, tag);
+    else
+      return launch_mfma_gemm<T, AR, BK_, false, PassSgemm>(ap, bp, ep, k, splits, used, stream, tag);
+  }
 }
 
 template <bool B_TRANS, bool A_TRANS>
 static int dispatch_tile(int bm, const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k,
                          int splits, int* used, hipStream_t stream) {
+  const bool rs = k % 16 == 0 && (B_TRANS || !A_TRANS);
   switch (bm) {
-    case 128: return run_sgemm<T128x128, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream, "sgemm_128x128");
-    case 64:  return run_sgemm<T64x256, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream, "sgemm_64x256");
-    default:  return run_sgemm<T32x256, B_TRANS, A_TRANS>(ap, bp, ep, k, splits, used, stream, "sgemm_32x256");
+    case 128:
+      return rs ? run_sgemm<T128x128, B_TRANS, A_TRANS, true>(ap, bp, ep, k, splits, used, stream, "sgemm_128x128")
+                : run_sgemm<T128x128, B_TRANS, A_TRANS, false>(ap, bp, ep, k, splits, used, stream, "sgemm_128x128");
+    case 64:
+      return rs ? run_sgemm<T64x256, B_TRANS, A_TRANS, true>(ap, bp, ep, k, splits, used, stream, "sgemm_64x256")
+                : run_sgemm<T64x256, B_TRANS, A_TRANS, false>(ap, bp, ep, k, splits, used, stream, "sgemm_64x256");
+    default:  return run_sgemm<T32x256, B_TRANS, A_TRANS, false>(ap, bp, ep, k, splits, used, stream, "sgemm_32x256");
   }
 }
 
