@@ -77,12 +77,18 @@ int rho_config_from_model_file(const char* path, rho_config** out);
 /* into_worker(): builds the chain on `device`.  exec_flags is a bit set (0 = the reference's kernel sequence in fp32):
  *   RHO_EXEC_FUSE_EPILOGUE  fold bias+ReLU into the conv epilogue (same buffers at every point the operators expose);
  *   RHO_EXEC_BF16_FORWARD   conv forward multiplies operands rounded to bf16 and accumulates in fp32
- *                           (forward-only inference mode; backward passes stay fp32 and read the same buffers). */
+ *                           (forward-only inference mode; backward passes stay fp32 and read the same buffers);
+ *   RHO_EXEC_OVERLAP_BACKWARD  conv filter / bias gradients run on a second stream beside the data gradient; the
+ *                           streams are joined at the end of backward (same results: no kernel changes). */
 #define RHO_EXEC_FUSE_EPILOGUE 0x1
 #define RHO_EXEC_BF16_FORWARD  0x2
+#define RHO_EXEC_OVERLAP_BACKWARD 0x4
 int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1,
                    int device, int exec_flags, rho_worker** out);
 int rho_worker_free(rho_worker* w);
+/* Run-time switch of RHO_EXEC_OVERLAP_BACKWARD for a worker built with it (per-kernel timings are only meaningful
+ * with it off: kernels that share the GPU stretch each other's durations). */
+int rho_worker_set_overlap_backward(rho_worker* w, int on);
 /* Output frame shape of the input operator (after crops), and what its last forward() drew. */
 int rho_worker_input_out_dims(rho_worker* w, int32_t* out_w, int32_t* out_h, int32_t* out_c);
 int rho_worker_last_preproc_draws(rho_worker* w, int32_t* crop_off_w, int32_t* crop_off_h, int* flipped, float* alphas,

@@ -41,6 +41,9 @@ PROTOTYPES = {
     "rh_ctx_destroy": (_int, [_vp]),
     "rh_ctx_stream": (_vp, [_vp]),
     "rh_ctx_sync": (_int, [_vp]),
+    "rh_ctx_aux_stream": (_vp, [_vp]),
+    "rh_ctx_fork": (_int, [_vp]),
+    "rh_ctx_join": (_int, [_vp]),
     "rh_malloc": (_int, [_vp, _sz, C.POINTER(_vp)]),
     "rh_free": (_int, [_vp, _vp]),
     "rh_memset_f32": (_int, [_vp, _f, _sz, _vp]),

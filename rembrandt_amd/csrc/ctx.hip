@@ -14,6 +14,10 @@
 struct rh_ctx {
   int device;
   hipStream_t stream;
+  // second stream for work that may overlap the main stream's (created on first use), and the two events
+  // that order the streams against each other
+  hipStream_t aux = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
 };
 
 using namespace rh;
@@ -48,6 +52,12 @@ extern "C" int rh_ctx_create(int device, rh_ctx** out) {
 
 extern "C" int rh_ctx_destroy(rh_ctx* ctx) {
   if (!ctx) return RH_E_INVALID;
+  if (ctx->aux) {
+    (void)hipStreamSynchronize(ctx->aux);
+    (void)hipStreamDestroy(ctx->aux);
+    (void)hipEventDestroy(ctx->ev_fork);
+    (void)hipEventDestroy(ctx->ev_join);
+  }
   hipError_t e = hipStreamSynchronize(ctx->stream);
   hipError_t e2 = hipStreamDestroy(ctx->stream);
   delete ctx;
@@ -58,7 +68,46 @@ extern "C" rh_stream_t rh_ctx_stream(rh_ctx* ctx) { return ctx ? (rh_stream_t)ct
 
 extern "C" int rh_ctx_sync(rh_ctx* ctx) {
   if (!ctx) return RH_E_INVALID;
+  if (ctx->aux) {
+    hipError_t e = hipStreamSynchronize(ctx->aux);
+    if (e != hipSuccess) return (int)e;
+  }
   return (int)hipStreamSynchronize(ctx->stream);
+}
+
+extern "C" rh_stream_t rh_ctx_aux_stream(rh_ctx* ctx) {
+  if (!ctx) return nullptr;
+  if (!ctx->aux) {
+    if (hipSetDevice(ctx->device) != hipSuccess) return nullptr;
+    hipStream_t s = nullptr;
+    hipEvent_t a = nullptr, b = nullptr;
+    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) return nullptr;  // default priority
+    if (hipEventCreateWithFlags(&a, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&b, hipEventDisableTiming) != hipSuccess) {
+      (void)hipStreamDestroy(s);
+      if (a) (void)hipEventDestroy(a);
+      return nullptr;
+    }
+    ctx->aux = s; ctx->ev_fork = a; ctx->ev_join = b;
+  }
+  return (rh_stream_t)ctx->aux;
+}
+
+// Work enqueued on the second stream after this call runs after everything the main stream holds now.
+extern "C" int rh_ctx_fork(rh_ctx* ctx) {
+  if (!ctx || !rh_ctx_aux_stream(ctx)) return RH_E_INVALID;
+  hipError_t e = hipEventRecord(ctx->ev_fork, ctx->stream);
+  if (e != hipSuccess) return (int)e;
+  return (int)hipStreamWaitEvent(ctx->aux, ctx->ev_fork, 0);
+}
+
+// Work enqueued on the main stream after this call runs after everything the second stream holds now.
+extern "C" int rh_ctx_join(rh_ctx* ctx) {
+  if (!ctx) return RH_E_INVALID;
+  if (!ctx->aux) return 0;
+  hipError_t e = hipEventRecord(ctx->ev_join, ctx->aux);
+  if (e != hipSuccess) return (int)e;
+  return (int)hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0);
 }
 
 extern "C" int rh_malloc(rh_ctx* ctx, size_t bytes, void** dptr) {

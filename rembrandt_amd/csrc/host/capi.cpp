@@ -196,6 +196,7 @@ int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, ui
     ExecOptions opts;
     opts.fuse_epilogue = (exec_flags & RHO_EXEC_FUSE_EPILOGUE) != 0;
     opts.bf16_forward = (exec_flags & RHO_EXEC_BF16_FORWARD) != 0;
+    opts.overlap_backward = (exec_flags & RHO_EXEC_OVERLAP_BACKWARD) != 0;
     w->worker.reset(new SequentialOperatorWorker(cfg->cfg, (size_t)batch_size,
                                                  capability == RHO_CAP_FORWARD ? OpCapability::Forward : OpCapability::Backward,
                                                  seed, w->ctx, opts));
@@ -203,6 +204,7 @@ int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, ui
   })
 }
 int rho_worker_free(rho_worker* w) { RHO_TRY({ delete w; }) }
+int rho_worker_set_overlap_backward(rho_worker* w, int on) { RHO_TRY({ RHO_REQ(w); w->worker->set_overlap_backward(on != 0); }) }
 int rho_worker_hidden_count(rho_worker* w, int32_t* out) { RHO_TRY({ RHO_REQ(w && out); *out = (int32_t)w->worker->hidden_count(); }) }
 int rho_worker_op_kind(rho_worker* w, int32_t hidden_idx, const char** out) { RHO_TRY({ RHO_REQ(out); *out = op_at(w, hidden_idx)->kind(); }) }
 void* rho_worker_stream(rho_worker* w) { return w ? w->ctx->stream() : nullptr; }

@@ -26,6 +26,13 @@ static void unwrap_last(const char* what) { unwrap(rh_last_error(), what); }
 DeviceContext::DeviceContext(int device_idx) : ctx_(nullptr) { unwrap(rh_ctx_create(device_idx, &ctx_), "rh_ctx_create"); }
 DeviceContext::~DeviceContext() { rh_ctx_destroy(ctx_); }
 void DeviceContext::sync() const { unwrap(rh_ctx_sync(ctx_), "rh_ctx_sync"); }
+rh_stream_t DeviceContext::aux_stream() const {
+  rh_stream_t s = rh_ctx_aux_stream(ctx_);
+  if (!s) panic("rh_ctx_aux_stream failed");
+  return s;
+}
+void DeviceContext::fork() const { unwrap(rh_ctx_fork(ctx_), "rh_ctx_fork"); }
+void DeviceContext::join() const { unwrap(rh_ctx_join(ctx_), "rh_ctx_join"); }
 
 // ---- configs ----------------------------------------------------------------------------------------
 static size_t out_dim_floor(size_t in, size_t size, size_t stride, size_t pad) {
@@ -644,6 +651,12 @@ class Conv2dOperator : public Operator {
       ws = std::max(ws, rh_conv2d_bwd_bias_workspace_bytes(g.N, g.K, (int)(out_dims_.w * out_dims_.h)));
     }
     workspace_.reset(new DeviceBuffer<uint8_t>(std::max<size_t>(ws, 256), context));
+    if (backward_enabled(capability) && opts.overlap_backward) {
+      // the filter / bias gradients run on the second stream with scratch of their own
+      size_t wa = rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_FILTER);
+      wa = std::max(wa, rh_conv2d_bwd_bias_workspace_bytes(g.N, g.K, (int)(out_dims_.w * out_dims_.h)));
+      workspace_aux_.reset(new DeviceBuffer<uint8_t>(std::max<size_t>(wa, 256), context));
+    }
   }
   size_t batch_size() const override { return batch_cap_; }
   SharedDeviceBuf get_output_vars() const override { return out_act_; }
@@ -678,11 +691,18 @@ class Conv2dOperator : public Operator {
     rh_stream_t s = context_->stream();
     if (!act_bwd_folded_)
       apply_rect_backprop(config_.act_func, out_act_->as_ptr(), out_dims_.len(), batch_size, out_delta_->as_mut_ptr(), s);
+    rh_stream_t sg = s;                        // stream and scratch of the two gradient kernels
+    DeviceBuffer<uint8_t>* wg = workspace_.get();
+    if (workspace_aux_ && overlap_on_) {
+      context_->fork();                        // the second stream sees the masked out_delta
+      sg = context_->aux_stream();
+      wg = workspace_aux_.get();
+    }
     unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in_act_->as_ptr(), out_delta_->as_ptr(), 1.0f, params_.grad_weights->as_mut_ptr(),
-                                workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward filter");
+                                wg->as_mut_ptr(), wg->len(), 0, sg), "conv2d backward filter");
     unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), 1.0f,
-                                 out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), workspace_->as_mut_ptr(),
-                                 workspace_->len(), s), "conv2d backward bias");
+                                 out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), wg->as_mut_ptr(),
+                                 wg->len(), sg), "conv2d backward bias");
     if (in_delta_) {
       unwrap(rh_conv2d_bwd_data(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
                                 workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward data");
@@ -711,6 +731,7 @@ class Conv2dOperator : public Operator {
     act_bwd_folded_ = true;
     return true;
   }
+  void set_overlap_backward(bool on) override { overlap_on_ = on; }
 
  private:
   bool act_bwd_folded_ = false;
@@ -728,7 +749,8 @@ class Conv2dOperator : public Operator {
   Dims3 out_dims_;
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   ParamTensors params_;
-  std::unique_ptr<DeviceBuffer<uint8_t>> workspace_;
+  std::unique_ptr<DeviceBuffer<uint8_t>> workspace_, workspace_aux_;
+  bool overlap_on_ = true;
 };
 
 // ---- Pool2dOperator -------------------------------------------------------------------------------------
@@ -1062,6 +1084,7 @@ void SequentialOperatorWorker::forward(size_t batch_size, OpPhase phase) {
 void SequentialOperatorWorker::backward(size_t batch_size) {
   loss_op_->backward(batch_size);
   for (auto it = hidden_ops_.rbegin(); it != hidden_ops_.rend(); ++it) (*it)->backward(batch_size);
+  context_->join();  // gradients computed on the second stream are complete for whatever the main stream does next
 }
 void SequentialOperatorWorker::regularize(Regularization reg) { for (auto& op : hidden_ops_) op->regularize(reg); }
 void SequentialOperatorWorker::accumulate_grads(float scale, float momentum) { for (auto& op : hidden_ops_) op->accumulate_grads(scale, momentum); }
@@ -1070,6 +1093,10 @@ void SequentialOperatorWorker::update_params2(float g, float u) { for (auto& op 
 void SequentialOperatorWorker::save_params() { for (auto& op : hidden_ops_) op->save_params(); }
 void SequentialOperatorWorker::restore_params() { for (auto& op : hidden_ops_) op->restore_params(); }
 void SequentialOperatorWorker::reset() { for (auto& op : hidden_ops_) op->reset(); }
+void SequentialOperatorWorker::set_overlap_backward(bool on) {
+  context_->join();
+  for (auto& op : hidden_ops_) op->set_overlap_backward(on);
+}
 void SequentialOperatorWorker::fused_sgd_step(float l2, float scale, float mu, float apply) {
   for (auto& op : hidden_ops_) op->fused_sgd_step(l2, scale, mu, apply);
 }

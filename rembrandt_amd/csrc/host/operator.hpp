@@ -44,6 +44,9 @@ class DeviceContext {
   DeviceContext(const DeviceContext&) = delete;
   DeviceContext& operator=(const DeviceContext&) = delete;
   rh_stream_t stream() const { return rh_ctx_stream(ctx_); }
+  rh_stream_t aux_stream() const;  // second stream for launches that may overlap the main one
+  void fork() const;               // aux waits for main
+  void join() const;               // main waits for aux
   rh_ctx* raw() const { return ctx_; }
   void sync() const;
 
@@ -191,6 +194,10 @@ struct OperatorConfig {
 struct ExecOptions {
   bool fuse_epilogue = true;  // conv bias + ReLU in the conv epilogue instead of K1 -> K2 -> K3
   bool bf16_forward = false;  // conv forward on bf16-rounded operands with fp32 accumulation (inference mode)
+  // Conv backward: filter and bias gradients on the context's second stream beside the data gradient on the
+  // main one (the bandwidth-bound operand copies of one hide behind the other's contraction); joined at the end
+  // of SequentialOperatorWorker::backward.
+  bool overlap_backward = true;
 };
 
 // ---- Operator trait -------------------------------------------------------------------------------
@@ -217,6 +224,9 @@ class Operator {
   // mask) asks for it at construction; an operator that agrees skips its own mask pass in backward().  The
   // out_delta buffer holds the same values after the chain's backward either way.
   virtual bool fold_activation_backward() { return false; }
+  // Switches the second-stream placement of gradient kernels on or off at run time (no effect on results, nor on
+  // operators built without it).
+  virtual void set_overlap_backward(bool /*on*/) {}
   // Parameter / optimizer-state blobs: a sequence of serialised NdArrays (weights then bias; for the state the
   // momentum buffers).  decode_* return the number of bytes consumed (src/operator/mod.rs:1008-1073).
   virtual void encode_params(std::vector<uint8_t>& /*blob*/) {}
@@ -304,6 +314,7 @@ class SequentialOperatorWorker : public Operator {
   void restore_params() override;
   void reset() override;
   void fused_sgd_step(float l2, float scale, float momentum, float apply) override;
+  void set_overlap_backward(bool on) override;
   const char* kind() const override { return "SequentialOperatorWorker"; }
   void encode_params(std::vector<uint8_t>& blob) override;
   size_t decode_params(const uint8_t* blob, size_t len) override;

@@ -41,6 +41,7 @@ PROTOTYPES = {
     "rho_config_from_model_file": (_int, [C.c_char_p, _P(_vp)]),
     "rho_worker_new": (_int, [_vp, _i32, _int, _u64, _u64, _int, _int, _P(_vp)]),
     "rho_worker_free": (_int, [_vp]),
+    "rho_worker_set_overlap_backward": (_int, [_vp, _int]),
     "rho_worker_input_out_dims": (_int, [_vp, _P(_i32), _P(_i32), _P(_i32)]),
     "rho_worker_last_preproc_draws": (_int, [_vp, _P(_i32), _P(_i32), _P(_int), _vp, _i64, _P(_i64)]),
     "rho_worker_dropout_stream": (_int, [_vp, _i32, _P(_u64), _P(_u64), _P(_u64)]),
@@ -230,10 +231,11 @@ class SequentialOperatorWorker:
     """src/operator/worker.rs:230-477 plus the Input/Loss operator calls the optimizer makes on it."""
 
     def __init__(self, config, batch_size, capability="Backward", shared_seed=(1, 2), device=0, fuse_epilogue=True,
-                 bf16_forward=False):
+                 bf16_forward=False, overlap_backward=True):
         h = _vp()
         _chk(lib().rho_worker_new(config._h, batch_size, 0 if capability == "Forward" else 1, shared_seed[0],
-                                  shared_seed[1], device, (1 if fuse_epilogue else 0) | (2 if bf16_forward else 0), C.byref(h)))
+                                  shared_seed[1], device, (1 if fuse_epilogue else 0) | (2 if bf16_forward else 0) | (4 if overlap_backward else 0),
+                                  C.byref(h)))
         self._h = h
         self.batch_size = batch_size
         self.shared_seed = tuple(shared_seed)
@@ -244,6 +246,9 @@ class SequentialOperatorWorker:
             self._h = None
 
     __del__ = close
+
+    def set_overlap_backward(self, on):
+        _chk(lib().rho_worker_set_overlap_backward(self._h, int(on)))
 
     def hidden_count(self):
         out = _i32()
