@@ -342,13 +342,16 @@ int rho_worker_buffer(rho_worker* w, int32_t hidden_idx, int which, float** dptr
   RHO_TRY({
     RHO_REQ(dptr && len);
     size_t n = 0;
+    RHO_REQ(w);
+    w->worker->settle();
     if (!op_at(w, hidden_idx)->buffer(which, dptr, &n)) panic("operator has no such buffer");
     *len = (int64_t)n;
   })
 }
 int rho_worker_read_buffer(rho_worker* w, int32_t hidden_idx, int which, float* host, int64_t len) {
   RHO_TRY({
-    RHO_REQ(host && len >= 0);
+    RHO_REQ(w && host && len >= 0);
+    w->worker->settle();
     float* d = nullptr;
     size_t n = 0;
     if (!op_at(w, hidden_idx)->buffer(which, &d, &n)) panic("operator has no such buffer");
@@ -358,7 +361,8 @@ int rho_worker_read_buffer(rho_worker* w, int32_t hidden_idx, int which, float* 
 }
 int rho_worker_write_buffer(rho_worker* w, int32_t hidden_idx, int which, const float* host, int64_t len) {
   RHO_TRY({
-    RHO_REQ(host && len >= 0);
+    RHO_REQ(w && host && len >= 0);
+    w->worker->settle();
     float* d = nullptr;
     size_t n = 0;
     if (!op_at(w, hidden_idx)->buffer(which, &d, &n)) panic("operator has no such buffer");

@@ -243,12 +243,13 @@ struct ParamTensors {
     unwrap(rh_sscal((int64_t)wlen, 0.0f, grad_weights->as_mut_ptr(), s()), "matrix_scale");
     unwrap(rh_sscal((int64_t)blen, 0.0f, grad_bias->as_mut_ptr(), s()), "row_vector_scale");
   }
-  void fused_sgd_step(float l2, float scale, float momentum, float apply) {
+  void fused_sgd_step(float l2, float scale, float momentum, float apply, rh_stream_t st = nullptr) {
     RB_ASSERT(has_backward());
+    if (!st) st = s();
     unwrap(rh_sgd_momentum_step((int64_t)wlen, weights->as_mut_ptr(), grad_weights->as_mut_ptr(),
-                                acc_grad_weights->as_mut_ptr(), l2, scale, momentum, apply, 1, s()), "rh_sgd_momentum_step");
+                                acc_grad_weights->as_mut_ptr(), l2, scale, momentum, apply, 1, st), "rh_sgd_momentum_step");
     unwrap(rh_sgd_momentum_step((int64_t)blen, bias->as_mut_ptr(), grad_bias->as_mut_ptr(),
-                                acc_grad_bias->as_mut_ptr(), l2, scale, momentum, apply, 1, s()), "rh_sgd_momentum_step");
+                                acc_grad_bias->as_mut_ptr(), l2, scale, momentum, apply, 1, st), "rh_sgd_momentum_step");
   }
   // Host-side sampling in memory order, then a blocking H2D copy (src/operator/mod.rs:964-1006, 1554-1592).
   void init(const ParamsInit& init, const uint64_t seed[2], size_t fan_in, size_t fan_out, bool xavier_ok, const char* who) {
@@ -545,8 +546,9 @@ class Data3dOperator : public InputOperator {
 class AffineOperator : public Operator {
  public:
   AffineOperator(size_t batch_size, OpCapability capability, const AffineOperatorConfig& config, const Operator* prev_op,
-                 Ctx context)
-      : batch_cap_(batch_size), config_(config), context_(context) {
+                 Ctx context, const ExecOptions& opts)
+      : batch_cap_(batch_size), config_(config), context_(context),
+        overlap_built_(opts.overlap_backward && backward_enabled(capability)), overlap_on_(overlap_built_) {
     RB_ASSERT(prev_op != nullptr);
     in_act_ = prev_op->get_output_vars();
     if (!in_act_) panic("AffineOperator missing required prev operator output vars");
@@ -607,7 +609,11 @@ class AffineOperator : public Operator {
   size_t decode_params(const uint8_t* blob, size_t len) override { return params_.decode_params(blob, len, kind()); }
   void encode_state(std::vector<uint8_t>& blob) override { params_.encode_state(blob); }
   size_t decode_state(const uint8_t* blob, size_t len) override { return params_.decode_state(blob, len, kind()); }
-  void fused_sgd_step(float l2, float scale, float mu, float apply) override { params_.fused_sgd_step(l2, scale, mu, apply); }
+  void fused_sgd_step(float l2, float scale, float mu, float apply) override {
+    params_.fused_sgd_step(l2, scale, mu, apply, overlap_on_ ? context_->aux_stream() : nullptr);
+  }
+  bool updates_on_second_stream() const override { return overlap_on_; }
+  void set_overlap_backward(bool on) override { overlap_on_ = on && overlap_built_; }
   bool buffer(int which, float** ptr, size_t* len) override {
     if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
     if (which == 1) { *ptr = out_delta_->as_mut_ptr(); *len = out_delta_->len(); return true; }
@@ -624,6 +630,7 @@ class AffineOperator : public Operator {
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   ParamTensors params_;
   std::unique_ptr<DeviceBuffer<uint8_t>> workspace_;
+  bool overlap_built_, overlap_on_;  // fused SGD step of this (large) parameter block on the second stream
 };
 
 // ---- Conv2dOperator -------------------------------------------------------------------------------------
@@ -1045,7 +1052,7 @@ SequentialOperatorWorker::SequentialOperatorWorker(const SequentialOperatorConfi
   for (const auto& c : config.hidden_ops) {
     std::unique_ptr<Operator> op;
     switch (c.kind) {
-      case OperatorConfig::Affine: op.reset(new AffineOperator(batch_size, capability, c.affine, prev, context)); break;
+      case OperatorConfig::Affine: op.reset(new AffineOperator(batch_size, capability, c.affine, prev, context, opts)); break;
       case OperatorConfig::Conv2d: op.reset(new Conv2dOperator(batch_size, capability, c.conv2d, prev, context, opts)); break;
       case OperatorConfig::Pool2d: op.reset(new Pool2dOperator(batch_size, c.pool2d, prev, context, opts)); break;
       case OperatorConfig::Dropout:
@@ -1069,7 +1076,15 @@ LossOperator* SequentialOperatorWorker::loss_operator(size_t rank) {
   return loss_op_.get();
 }
 
+void SequentialOperatorWorker::settle() {
+  if (aux_pending_) {
+    context_->join();
+    aux_pending_ = false;
+  }
+}
+
 void SequentialOperatorWorker::init_params(const uint64_t shared_seed[2]) {
+  settle();
   Xorshiftplus128 rng(shared_seed);
   for (auto& op : hidden_ops_) {
     const uint64_t op_seed[2] = {rng.next_u64(), rng.next_u64()};
@@ -1078,42 +1093,59 @@ void SequentialOperatorWorker::init_params(const uint64_t shared_seed[2]) {
 }
 void SequentialOperatorWorker::forward(size_t batch_size, OpPhase phase) {
   input_op_->forward(batch_size, phase);
-  for (auto& op : hidden_ops_) op->forward(batch_size, phase);
+  for (auto& op : hidden_ops_) {
+    if (aux_pending_ && op->updates_on_second_stream()) settle();  // its parameters were updated on the second stream
+    op->forward(batch_size, phase);
+  }
   loss_op_->forward(batch_size, phase);
 }
 void SequentialOperatorWorker::backward(size_t batch_size) {
+  settle();
   loss_op_->backward(batch_size);
   for (auto it = hidden_ops_.rbegin(); it != hidden_ops_.rend(); ++it) (*it)->backward(batch_size);
   context_->join();  // gradients computed on the second stream are complete for whatever the main stream does next
 }
-void SequentialOperatorWorker::regularize(Regularization reg) { for (auto& op : hidden_ops_) op->regularize(reg); }
-void SequentialOperatorWorker::accumulate_grads(float scale, float momentum) { for (auto& op : hidden_ops_) op->accumulate_grads(scale, momentum); }
-void SequentialOperatorWorker::update_params(float scale) { for (auto& op : hidden_ops_) op->update_params(scale); }
-void SequentialOperatorWorker::update_params2(float g, float u) { for (auto& op : hidden_ops_) op->update_params2(g, u); }
-void SequentialOperatorWorker::save_params() { for (auto& op : hidden_ops_) op->save_params(); }
-void SequentialOperatorWorker::restore_params() { for (auto& op : hidden_ops_) op->restore_params(); }
-void SequentialOperatorWorker::reset() { for (auto& op : hidden_ops_) op->reset(); }
+void SequentialOperatorWorker::regularize(Regularization reg) { settle(); for (auto& op : hidden_ops_) op->regularize(reg); }
+void SequentialOperatorWorker::accumulate_grads(float scale, float momentum) { settle(); for (auto& op : hidden_ops_) op->accumulate_grads(scale, momentum); }
+void SequentialOperatorWorker::update_params(float scale) { settle(); for (auto& op : hidden_ops_) op->update_params(scale); }
+void SequentialOperatorWorker::update_params2(float g, float u) { settle(); for (auto& op : hidden_ops_) op->update_params2(g, u); }
+void SequentialOperatorWorker::save_params() { settle(); for (auto& op : hidden_ops_) op->save_params(); }
+void SequentialOperatorWorker::restore_params() { settle(); for (auto& op : hidden_ops_) op->restore_params(); }
+void SequentialOperatorWorker::reset() { settle(); for (auto& op : hidden_ops_) op->reset(); }
 void SequentialOperatorWorker::set_overlap_backward(bool on) {
+  settle();
   context_->join();
   for (auto& op : hidden_ops_) op->set_overlap_backward(on);
 }
 void SequentialOperatorWorker::fused_sgd_step(float l2, float scale, float mu, float apply) {
-  for (auto& op : hidden_ops_) op->fused_sgd_step(l2, scale, mu, apply);
+  settle();
+  // Operators that say so take their step on the second stream (forked here: it sees the finished gradients); the
+  // next forward pass joins in front of the first of them, so these updates hide behind the layers before it.
+  for (auto& op : hidden_ops_) {
+    if (op->updates_on_second_stream() && !aux_pending_) {
+      context_->fork();
+      aux_pending_ = true;
+    }
+    op->fused_sgd_step(l2, scale, mu, apply);
+  }
 }
 
-void SequentialOperatorWorker::encode_params(std::vector<uint8_t>& blob) { for (auto& op : hidden_ops_) op->encode_params(blob); }
+void SequentialOperatorWorker::encode_params(std::vector<uint8_t>& blob) { settle(); for (auto& op : hidden_ops_) op->encode_params(blob); }
 size_t SequentialOperatorWorker::decode_params(const uint8_t* blob, size_t len) {
+  settle();
   size_t off = 0;
   for (auto& op : hidden_ops_) off += op->decode_params(blob + off, len - off);
   return off;
 }
 void SequentialOperatorWorker::encode_state(std::vector<uint8_t>& blob) {
+  settle();
   for (auto& op : hidden_ops_) {  // params then momentum, operator by operator (gossip_dist.rs:1287-1291)
     op->encode_params(blob);
     op->encode_state(blob);
   }
 }
 size_t SequentialOperatorWorker::decode_state(const uint8_t* blob, size_t len) {
+  settle();
   size_t off = 0;
   for (auto& op : hidden_ops_) {
     off += op->decode_params(blob + off, len - off);

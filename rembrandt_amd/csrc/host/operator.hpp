@@ -227,6 +227,10 @@ class Operator {
   // Switches the second-stream placement of gradient kernels on or off at run time (no effect on results, nor on
   // operators built without it).
   virtual void set_overlap_backward(bool /*on*/) {}
+  // An operator whose fused SGD step may run on the context's second stream (large parameter blocks that the
+  // next forward pass needs late: the affine layers) says so; the worker then joins the streams before that
+  // operator's next forward and before anything else touches parameters.
+  virtual bool updates_on_second_stream() const { return false; }
   // Parameter / optimizer-state blobs: a sequence of serialised NdArrays (weights then bias; for the state the
   // momentum buffers).  decode_* return the number of bytes consumed (src/operator/mod.rs:1008-1073).
   virtual void encode_params(std::vector<uint8_t>& /*blob*/) {}
@@ -315,6 +319,9 @@ class SequentialOperatorWorker : public Operator {
   void reset() override;
   void fused_sgd_step(float l2, float scale, float momentum, float apply) override;
   void set_overlap_backward(bool on) override;
+  // Joins the second stream if parameter updates are still in flight on it (called by every method but forward,
+  // which joins lazily in front of the first operator concerned).
+  void settle();
   const char* kind() const override { return "SequentialOperatorWorker"; }
   void encode_params(std::vector<uint8_t>& blob) override;
   size_t decode_params(const uint8_t* blob, size_t len) override;
@@ -338,6 +345,7 @@ class SequentialOperatorWorker : public Operator {
   std::unique_ptr<InputOperator> input_op_;
   std::vector<std::unique_ptr<Operator>> hidden_ops_;
   std::unique_ptr<LossOperator> loss_op_;
+  bool aux_pending_ = false;
 };
 
 // ---- SGD policy (src/opt/sgd/mod.rs:20-147) ---------------------------------------------------------
