@@ -404,12 +404,17 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
     RHO_REQ(s && w && batch_size > 0);
     SequentialOperatorWorker* op = w->worker.get();
     const size_t b = (size_t)batch_size;
+    // forward -> arg-max and loss kernels -> backward -> update are all enqueued before the two read-backs, so
+    // the GPU works through the step without waiting for the host (same results as the reference's order:
+    // store_output_categories, store_loss, backward; nothing in between writes what they read)
     op->forward(b, OpPhase::Training(s->opt->iter_counter()));
-    op->loss_operator(0)->store_output_categories(b);
-    const float loss = op->loss_operator(0)->store_loss(b);
+    op->loss_operator(0)->enqueue_output_categories(b);
+    op->loss_operator(0)->enqueue_loss(b);
     op->backward(b);
-    const size_t correct = op->loss_operator(0)->accuracy_count(b);
     s->opt->step(op, fused != 0);
+    op->loss_operator(0)->fetch_output_categories(b);
+    const float loss = op->loss_operator(0)->fetch_loss();
+    const size_t correct = op->loss_operator(0)->accuracy_count(b);
     if (loss_out) *loss_out = loss;
     if (correct_out) *correct_out = (int32_t)correct;
   })

@@ -985,6 +985,10 @@ class SoftmaxKLLossOperator : public LossOperator {
     weights_.sync_load(weights_h_.data(), batch_cap_);
   }
   float store_loss(size_t batch_size) override {
+    enqueue_loss(batch_size);
+    return fetch_loss();
+  }
+  void enqueue_loss(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
     rh_stream_t s = context_->stream();
     rembrandt_kernel_batch_map_softmax_kl_loss1(out_values_.as_ptr(), (int)loss_config_.num_categories, (int)batch_size,
@@ -992,15 +996,24 @@ class SoftmaxKLLossOperator : public LossOperator {
     unwrap_last("rembrandt_kernel_batch_map_softmax_kl_loss1");
     rembrandt_kernel_batch_blockreduce_sum(out_loss1_.as_ptr(), (int)batch_size, 1, out_loss_.as_mut_ptr(), 0.0f, s);
     unwrap_last("rembrandt_kernel_batch_blockreduce_sum");
+  }
+  float fetch_loss() override {
     float h = 0.0f;
     out_loss_.sync_store(&h, 1);
     return h;
   }
   void store_output_categories(size_t batch_size) override {
+    enqueue_output_categories(batch_size);
+    fetch_output_categories(batch_size);
+  }
+  void enqueue_output_categories(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
     rembrandt_kernel_batch_blockreduce_argmax(out_values_.as_ptr(), (int)loss_config_.num_categories, (int)batch_size,
                                               max_value_.as_mut_ptr(), out_cats_.as_mut_ptr(), context_->stream());
     unwrap_last("rembrandt_kernel_batch_blockreduce_argmax");
+  }
+  void fetch_output_categories(size_t batch_size) override {
+    RB_ASSERT(batch_size <= batch_cap_);
     out_cats_.sync_store(out_cats_h_.data(), batch_cap_);
   }
   const int32_t* get_output_categories(size_t) const override { return out_cats_h_.data(); }

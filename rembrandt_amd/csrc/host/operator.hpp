@@ -267,6 +267,13 @@ class LossOperator : public Operator {
   virtual void load_weights(size_t batch_size) = 0;
   virtual float store_loss(size_t batch_size) = 0;
   virtual void store_output_categories(size_t batch_size) = 0;
+  // The two halves of store_loss / store_output_categories: enqueue_* launches the kernels that leave the result in
+  // device buffers nothing else writes, fetch_* copies it to the host (blocking).  A caller may enqueue more work
+  // (the backward pass) in between, so the GPU does not idle during the read-backs.
+  virtual void enqueue_loss(size_t batch_size) = 0;
+  virtual float fetch_loss() = 0;
+  virtual void enqueue_output_categories(size_t batch_size) = 0;
+  virtual void fetch_output_categories(size_t batch_size) = 0;
   virtual const int32_t* get_output_categories(size_t batch_size) const = 0;
   virtual size_t accuracy_count(size_t batch_size) const = 0;
 };
