@@ -81,7 +81,7 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
     const float* img = dy;
     if (sp.img_bytes) {
       float* dyp = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes);
-      launch_pad_image(dy, dyp, (long long)d.N * d.K, d.P, d.Q, sp.Hp, sp.Wp, sp.halo, stream);
+      launch_pad_image(dy, dyp, (long long)d.N * d.K, d.P, d.Q, sp.Hp, sp.Wp, sp.halo, stream, d.st);
       if (int e = launch_status()) return e;
       img = dyp;
     }

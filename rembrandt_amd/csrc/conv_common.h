@@ -140,23 +140,26 @@ inline SoffPlan plan_soff_fwd(const ConvDims& d) {
 
 // Backward-data with stride 1: dx[n,c,h,w] = sum dyp[n,ko,h+R-1-r,w+S-1-s] * w[ko,c,r,s] on dy padded
 // by R-1-pad zeros per side.
+// Backward-data as a stride-1 correlation of the flipped filter with dy.  For stride > 1 the padded copy of dy is
+// also dilated (dy[p][q] lands on [halo + st*p][halo + st*q], zeros between): the contraction then multiplies
+// (st^2 - 1)/st^2 zeros, but runs on the scalar-offset loaders; the copy is (H + R - 1) x (W + S - 1) per plane.
 inline SoffPlan plan_soff_bwd_data(const ConvDims& d) {
   SoffPlan p;
   p.n_k = round_up(d.K * d.R * d.S, kTabPad);
   p.halo = d.R - 1 - d.pad;
-  p.Hp = d.P + 2 * p.halo;
-  p.Wp = d.Q + 2 * (d.S - 1 - d.pad);
+  p.Hp = d.H + d.R - 1;   // = P + 2*halo when the stride is 1
+  p.Wp = d.W + d.S - 1;
   p.tab_bytes = align256(sizeof(int) * (size_t)p.n_k);
   p.wt_bytes = align256(sizeof(float) * (size_t)p.n_k * d.C);
   const size_t img = p.halo >= 0 ? sizeof(float) * (size_t)d.N * d.K * p.Hp * p.Wp : 0;
-  p.img_bytes = p.halo > 0 ? align256(img) : 0;
-  p.ok = d.st == 1 && p.halo >= 0 && d.R == d.S && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
+  p.img_bytes = (p.halo > 0 || d.st > 1 || p.Hp != d.P || p.Wp != d.Q) ? align256(img) : 0;
+  p.ok = p.halo >= 0 && d.R == d.S && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
   return p;
 }
 
-// dst[n][c][h+halo][w+halo] = src[n][c][h][w], zeros elsewhere; dst is planes x Hp x Wp.
+// dst[n][c][halo + dil*h][halo + dil*w] = src[n][c][h][w], zeros elsewhere; dst is planes x Hp x Wp.
 void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
-                      hipStream_t stream);
+                      hipStream_t stream, int dil = 1);
 
 void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int HW, int W,
                           hipStream_t stream);

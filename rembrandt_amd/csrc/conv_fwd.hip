@@ -36,11 +36,36 @@ __global__ void pad_image_kernel(const float* __restrict__ src, float* __restric
   }
 }
 
+// The same with the source dilated: src[h][w] lands on [halo + dil*h][halo + dil*w].
+__global__ void pad_dilate_image_kernel(const float* __restrict__ src, float* __restrict__ dst, unsigned total, int H, int W,
+                                        FastDiv dHp, FastDiv dWp, int halo, FastDiv dDil) {
+  const unsigned stride = gridDim.x * blockDim.x;
+  for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    uint32_t t, wp, plane, hp;
+    dWp.divmod(i, t, wp);
+    dHp.divmod(t, plane, hp);
+    const int hd = (int)hp - halo, wd = (int)wp - halo;
+    float v = 0.0f;
+    if (hd >= 0 && wd >= 0) {
+      uint32_t h, hr, w, wr;
+      dDil.divmod((uint32_t)hd, h, hr);
+      dDil.divmod((uint32_t)wd, w, wr);
+      if (hr == 0 && wr == 0 && h < (uint32_t)H && w < (uint32_t)W) v = src[((size_t)plane * H + h) * W + w];
+    }
+    dst[i] = v;
+  }
+}
+
 // total elements of dst must be below 2^31 (a tensor is at most 2 GiB here)
 void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
-                      hipStream_t stream) {
+                      hipStream_t stream, int dil) {
   const long long total = planes * Hp * Wp;
   ProfScope prof("pad_image", 4.0 * ((double)planes * H * W + (double)total), stream);
+  if (dil > 1) {
+    hipLaunchKernelGGL(pad_dilate_image_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, src, dst,
+                       (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, FastDiv((uint32_t)dil));
+    return;
+  }
   hipLaunchKernelGGL(pad_image_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, src, dst,
                      (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo);
 }

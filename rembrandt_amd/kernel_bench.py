@@ -23,6 +23,7 @@ CONV_LAYERS = {
     "alexnet_conv1": (256, 3, 227, 227, 96, 11, 4, 0),
     "alexnet_conv4": (256, 384, 13, 13, 384, 3, 1, 1),
     "alexnet_conv5": (256, 384, 13, 13, 256, 3, 1, 1),
+    "stride2_3x3": (64, 64, 56, 56, 128, 3, 2, 1),   # a strided layer in mid-network (its backward-data is needed)
 }
 FC_LAYERS = {"alexnet_fc6": (256, 9216, 4096), "alexnet_fc7": (256, 4096, 4096), "alexnet_fc8": (256, 4096, 1000)}
 
