@@ -106,6 +106,14 @@ inline int launch_mfma_gemm_bf16(const typename AL::Params& ap, const typename B
 typedef Tile<128, 128, 16, 2, 2, RH_OCC_128> T128x128;
 typedef Tile<96, 256, 16, 1, 4> T96x256;
 typedef Tile<96, 128, 16, 1, 4, 4> T96x128;
+#ifndef RH_BF16_BK
+#define RH_BF16_BK 32
+#endif
+#ifndef RH_BF16_OCC
+#define RH_BF16_OCC 3
+#endif
+// bf16-operand kernel: a deeper K step keeps more operand loads in flight per wave (its MFMAs are 16x shorter)
+typedef Tile<128, 128, RH_BF16_BK, 2, 2, RH_BF16_OCC> T128x128bf;
 typedef Tile<64, 256, 16, 1, 4> T64x256;
 typedef Tile<32, 256, 16, 1, 4> T32x256;
 

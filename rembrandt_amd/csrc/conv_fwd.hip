@@ -102,7 +102,7 @@ static int run_fwd_soff(const RowSParams& ap, const RowSParams& bp, const EpiPar
 // bf16-operand forward (128x128 tile only: the loader rows must equal the tile rows).
 static int run_fwd_soff_bf16(const RowSParams& ap, const RowSParams& bp, const EpiParams& ep, int n_k, int k_true,
                              hipStream_t stream) {
-  typedef T128x128 T;
+  typedef T128x128bf T;
   typedef LoadRowS<T::BM, T::BK, T::NT, true> AL;
   typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
   return launch_mfma_gemm_bf16<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, 1, nullptr, stream, "conv_fwd_bf16_128x128",
