@@ -250,6 +250,34 @@ int rh_lrn_bwd(const rh_lrn_geom* g, const float* x, const float* y, const float
                rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Spatial batch normalisation, NCHW fp32, `plane` = H*W.  Replaces CudnnBatchNormOp in
+ * cudnnBatchNormMode_t::Spatial (constructed at src/operator/conv.rs:225-232; forward_inference :493-506,
+ * forward_training :520-535, backward :594-607).  With m = N*plane values per channel:
+ *   mean_c = sum(x)/m,  ivar_c = 1/sqrt(sum((x-mean_c)^2)/m + epsilon)
+ *   forward_training:  y = alpha*(scale_c*(x-mean_c)*ivar_c + bias_c) + beta*y
+ *                      cached_mean = mean, cached_ivar = ivar,
+ *                      running_mean = (1-ema_factor)*running_mean + ema_factor*mean
+ *                      running_ivar = (1-ema_factor)*running_ivar + ema_factor*ivar
+ *   forward_inference: the same map with (running_mean, running_ivar) in place of the batch statistics
+ *   backward:          dscale_c = beta_param*dscale_c + alpha_param*sum(dy*xhat),  xhat = (x-cached_mean)*cached_ivar
+ *                      dbias_c  = beta_param*dbias_c  + alpha_param*sum(dy)
+ *                      dx = alpha_data*scale_c*cached_ivar*(dy - sum(dy)/m - xhat*sum(dy*xhat)/m) + beta_data*dx
+ * The moving "ivar" is an average of inverse standard deviations, as the reference's buffer names
+ * (bn_running_ivar, initialised to 1) say; what cuDNN v4 kept in that buffer cannot be checked here.
+ * RH_FUSE_RELU (forward only) clamps the blended result at 0: the in-place ReLU that follows the call in the
+ * reference (src/operator/conv.rs:538-551).  `ws` needs rh_bnorm_workspace_bytes(N, C, plane) bytes. */
+size_t rh_bnorm_workspace_bytes(int N, int C, int plane);
+int rh_bnorm_fwd_train(int N, int C, int plane, float alpha, const float* x, float beta, float* y, double ema_factor,
+                       double epsilon, const float* scale, const float* bias, float* running_mean, float* running_ivar,
+                       float* cached_mean, float* cached_ivar, void* ws, size_t ws_bytes, int flags, rh_stream_t stream);
+int rh_bnorm_fwd_infer(int N, int C, int plane, float alpha, const float* x, float beta, float* y, double epsilon,
+                       const float* scale, const float* bias, const float* running_mean, const float* running_ivar,
+                       void* ws, size_t ws_bytes, int flags, rh_stream_t stream);
+int rh_bnorm_bwd(int N, int C, int plane, float alpha_data, float beta_data, const float* x, const float* dy, float* dx,
+                 float alpha_param, float beta_param, double epsilon, const float* scale, float* dscale, float* dbias,
+                 const float* cached_mean, const float* cached_ivar, void* ws, size_t ws_bytes, rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Host-side seeded generator for synthetic inputs and parameter initialisation (stands in for
  * the rng crate's Xorshiftplus128Rng + rand 0.3 distributions of src/operator/mod.rs:964-1006,
  * 1554-1592, whose bit streams cannot be reproduced).  Element i of stream (seed, stream_id) is

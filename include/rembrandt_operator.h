@@ -40,7 +40,12 @@ enum { RHO_MOM_ZERO = 0, RHO_MOM_UPDATE = 1, RHO_MOM_UPDATE_NESTEROV = 2, RHO_MO
 enum { RHO_STEP_CONSTANT = 0, RHO_STEP_ANNEAL1 = 1, RHO_STEP_ANNEAL2 = 2, RHO_STEP_ANNEAL4 = 3, RHO_STEP_DECAY = 4, RHO_STEP_INVERSE = 5 };
 /* buffers of an operator, for rho_worker_buffer */
 enum { RHO_BUF_OUT_ACT = 0, RHO_BUF_OUT_DELTA = 1, RHO_BUF_WEIGHTS = 2, RHO_BUF_BIAS = 3, RHO_BUF_GRAD_WEIGHTS = 4,
-       RHO_BUF_GRAD_BIAS = 5, RHO_BUF_ACC_GRAD_WEIGHTS = 6, RHO_BUF_ACC_GRAD_BIAS = 7 };
+       RHO_BUF_GRAD_BIAS = 5, RHO_BUF_ACC_GRAD_WEIGHTS = 6, RHO_BUF_ACC_GRAD_BIAS = 7,
+       /* batch-normalised operators: RHO_BUF_UNIT*u + id addresses conv + batch-norm unit u = 0, 1, 2 (ids 2, 4, 6 as above) */
+       RHO_BUF_BN_SCALE = 8, RHO_BUF_BN_BIAS = 9, RHO_BUF_BN_SCALE_GRAD = 10, RHO_BUF_BN_BIAS_GRAD = 11,
+       RHO_BUF_BN_RUNNING_MEAN = 12, RHO_BUF_BN_RUNNING_IVAR = 13, RHO_BUF_BN_CACHED_MEAN = 14, RHO_BUF_BN_CACHED_IVAR = 15,
+       RHO_BUF_ACC_BN_SCALE_GRAD = 16, RHO_BUF_ACC_BN_BIAS_GRAD = 17, RHO_BUF_PRE_ACT = 18, RHO_BUF_PRE_DELTA = 19,
+       RHO_BUF_MID_ACT = 30, RHO_BUF_MID_DELTA = 31, RHO_BUF_UNIT = 100 };
 
 /* ---- SequentialOperatorConfig builder (worker.rs:133-228) ---- */
 int rho_config_new(rho_config** out);                                       /* ::new()            */
@@ -49,6 +54,19 @@ int rho_config_data3d(rho_config* cfg, int32_t w, int32_t h, int32_t c, int norm
 int rho_config_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t conv_size,
                       int32_t conv_stride, int32_t conv_pad, int32_t out_channels, int act_func, int init_kind,
                       float init_value);                                                              /* .conv2d()  */
+/* The batch-normalised operators of src/operator/conv.rs.  `mov_avg_kind`: RHO_BNORM_CUMULATIVE (newest batch weighs
+ * 1/(1+t)) or RHO_BNORM_EXPONENTIAL (1 at t = 0, `ema_factor` afterwards), BNormMovingAverage::at_iter (:58-72). */
+enum { RHO_BNORM_CUMULATIVE = 0, RHO_BNORM_EXPONENTIAL = 1 };
+int rho_config_bnorm_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t conv_size,
+                            int32_t conv_stride, int32_t conv_pad, int32_t out_channels, int mov_avg_kind,
+                            double ema_factor, double epsilon, int act_func, int init_kind,
+                            float init_value);                                            /* .bnorm_conv2d() (worker.rs:189)          */
+int rho_config_stack_res_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int mov_avg_kind,
+                                double ema_factor, double epsilon, int act_func, int init_kind,
+                                float init_value);                                        /* .stack_res_conv2d() (worker.rs:194)      */
+int rho_config_proj_stack_res_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t out_w,
+                                     int32_t out_h, int32_t out_c, int mov_avg_kind, double ema_factor, double epsilon,
+                                     int act_func, int init_kind, float init_value);      /* .proj_stack_res_conv2d() (worker.rs:199) */
 int rho_config_affine(rho_config* cfg, int32_t in_channels, int32_t out_channels, int act_func, int init_kind,
                       float init_value);                                                              /* .affine()  */
 int rho_config_pool2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t pool_size,

@@ -376,3 +376,54 @@ def lrn_bwd(x, dy, size, scale, power, min_div):
         c0, c1 = max(0, c - hi), min(Cc - 1, c + lo)
         dx[:, c] -= 2.0 * scale * power * x64[:, c] * t[:, c0:c1 + 1].sum(axis=1)
     return dx.astype(np.float32)
+
+
+# ---- spatial batch normalisation (numpy restatement of the cuDNN Spatial mode the reference calls, ------------
+# ---- src/operator/conv.rs:493-535, 594-607; fp64 arithmetic on the fp32 inputs) ---------------------------------
+def bnorm_mov_avg_at_iter(kind, ema_factor, t):
+    """BNormMovingAverage::at_iter (src/operator/conv.rs:58-72)."""
+    if kind == "Cumulative":
+        return 1.0 / (1.0 + t)
+    assert kind == "Exponential"
+    return 1.0 if t == 0 else float(ema_factor)
+
+
+def bnorm_fwd_train(x, scale, bias, running_mean, running_ivar, ema_factor, epsilon, alpha=1.0, beta=0.0, y=None):
+    """Returns (y, cached_mean, cached_ivar, new_running_mean, new_running_ivar).  Statistics are per channel over
+    (n, h, w), variance biased (divided by m); the moving pair averages mean and inverse standard deviation
+    ("parity unpinned" for the second: what cuDNN v4 kept in resultRunningInvVariance is not checkable here)."""
+    x64 = x.astype(np.float64)
+    mean = x64.mean(axis=(0, 2, 3))
+    var = ((x64 - mean[None, :, None, None]) ** 2).mean(axis=(0, 2, 3))
+    ivar = 1.0 / np.sqrt(var + epsilon)
+    out = scale.astype(np.float64)[None, :, None, None] * (x64 - mean[None, :, None, None]) * ivar[None, :, None, None] \
+        + bias.astype(np.float64)[None, :, None, None]
+    out = alpha * out
+    if beta != 0.0:
+        out = out + beta * y.astype(np.float64)
+    new_rm = (1.0 - ema_factor) * running_mean.astype(np.float64) + ema_factor * mean
+    new_ri = (1.0 - ema_factor) * running_ivar.astype(np.float64) + ema_factor * ivar
+    f = np.float32
+    return out.astype(f), mean.astype(f), ivar.astype(f), new_rm.astype(f), new_ri.astype(f)
+
+
+def bnorm_fwd_infer(x, scale, bias, running_mean, running_ivar, alpha=1.0, beta=0.0, y=None):
+    b = lambda v: v.astype(np.float64)[None, :, None, None]
+    out = alpha * (b(scale) * (x.astype(np.float64) - b(running_mean)) * b(running_ivar) + b(bias))
+    if beta != 0.0:
+        out = out + beta * y.astype(np.float64)
+    return out.astype(np.float32)
+
+
+def bnorm_bwd(x, dy, scale, cached_mean, cached_ivar):
+    """Returns (dx, dscale, dbias) of y = scale*xhat + bias with xhat = (x - mean(x))*ivar(x), the batch statistics
+    being functions of x: dx = scale*ivar*(dy - mean(dy) - xhat*mean(dy*xhat))."""
+    b = lambda v: v.astype(np.float64)[None, :, None, None]
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    xhat = (x64 - b(cached_mean)) * b(cached_ivar)
+    dbias = dy64.sum(axis=(0, 2, 3))
+    dscale = (dy64 * xhat).sum(axis=(0, 2, 3))
+    m = x.shape[0] * x.shape[2] * x.shape[3]
+    dx = b(scale) * b(cached_ivar) * (dy64 - (dbias / m)[None, :, None, None] - xhat * (dscale / m)[None, :, None, None])
+    f = np.float32
+    return dx.astype(f), dscale.astype(f), dbias.astype(f)

@@ -11,6 +11,8 @@ operator, same method names and the same order of operations as the Rust sources
                                             src/operator/mod.rs:1178-1236, 1355-1363
   SequentialOperatorWorker fan-out ........ src/operator/worker.rs:356-477
   SgdOpt update block ..................... src/opt/sgd/new.rs:345-495, 623-633
+  BNormConv2d / StackResConv2d / ProjStackResConv2d operators
+                                            src/operator/conv.rs:461-912, 1497-2182, 2935-3560
 
 `fast=True` switches the contractions to the fp32 im2col + SGEMM family (the timed CPU baseline);
 the default is the fp64-accumulating family (the parity checker).
@@ -230,14 +232,236 @@ class LocalResNormOperator:
         return O.lrn_bwd(self.in_act, self.out_delta.reshape(self.x_shape), *self.args)
 
 
+class _BNormUnit:
+    """conv (no bias) + spatial batch norm with the reference's buffers and update rules per unit
+    (src/operator/conv.rs:133-160 buffers; :640-911 regularize the filter only, accumulate / update / save / restore /
+    reset the filter, scale and bias; the moving statistics travel with save / restore)."""
+
+    def __init__(self, batch, in_dims, size, stride, pad, out_channels):
+        w, h, c = in_dims
+        self.x_shape = (batch, c, h, w)
+        self.stride, self.pad = stride, pad
+        f = np.float32
+        self.weights = np.zeros((out_channels, c, size, size), f)
+        self.grad_weights, self.acc_grad_weights, self.save_weights = (np.zeros_like(self.weights) for _ in range(3))
+        K = out_channels
+        self.scale, self.bias = np.ones(K, f), np.zeros(K, f)
+        self.running_mean, self.running_ivar = np.zeros(K, f), np.ones(K, f)
+        self.scale_grad, self.bias_grad, self.acc_scale_grad, self.acc_bias_grad = (np.zeros(K, f) for _ in range(4))
+        self.save_scale, self.save_bias, self.save_running_mean, self.save_running_ivar = (np.zeros(K, f) for _ in range(4))
+        self.cached_mean, self.cached_ivar = np.zeros(K, f), np.zeros(K, f)
+        P, Q = O.out_dim(h, size, stride, pad), O.out_dim(w, size, stride, pad)
+        self.out_dims = (Q, P, K)
+        self.pre_act = np.zeros((batch, K, P, Q), f)
+        self.bf16_forward = False
+
+    def forward(self, in_act, out, beta_out, training, t, mov_avg, epsilon):
+        """Returns beta_out*out + BN(conv(in_act)) (forward_training / forward_inference, conv.rs:493-535)."""
+        in_act = np.ascontiguousarray(in_act.reshape(self.x_shape))
+        self.in_act = in_act
+        if self.bf16_forward:
+            O.conv2d_fwd(O.round_bf16(in_act), O.round_bf16(self.weights), self.stride, self.pad, y=self.pre_act)
+        else:
+            O.conv2d_fwd(in_act, self.weights, self.stride, self.pad, y=self.pre_act)
+        if training:
+            ema = O.bnorm_mov_avg_at_iter(mov_avg[0], mov_avg[1], t)
+            y, self.cached_mean, self.cached_ivar, self.running_mean, self.running_ivar = O.bnorm_fwd_train(
+                self.pre_act, self.scale, self.bias, self.running_mean, self.running_ivar, ema, epsilon, 1.0, beta_out, out)
+            return y
+        return O.bnorm_fwd_infer(self.pre_act, self.scale, self.bias, self.running_mean, self.running_ivar, 1.0, beta_out, out)
+
+    def backward_params(self, out_delta):
+        """pre_delta = dBN(out_delta), scale / bias gradients accumulated (beta 1); grad_weights += dconv (conv.rs:594-618)."""
+        self.pre_delta, ds, db = O.bnorm_bwd(self.pre_act, out_delta, self.scale, self.cached_mean, self.cached_ivar)
+        self.scale_grad = (self.scale_grad + ds).astype(np.float32)
+        self.bias_grad = (self.bias_grad + db).astype(np.float32)
+        O.conv2d_bwd_filter(self.in_act, self.pre_delta, self.weights.shape, self.stride, self.pad, 1.0, 1.0, self.grad_weights)
+
+    def backward_data(self, beta=0.0, dx=None):
+        return O.conv2d_bwd_data(self.weights, self.pre_delta, self.x_shape, self.stride, self.pad, 1.0, beta, dx)
+
+    def _triples(self):
+        return ((self.weights, self.grad_weights, self.acc_grad_weights), (self.scale, self.scale_grad, self.acc_scale_grad),
+                (self.bias, self.bias_grad, self.acc_bias_grad))
+
+    def regularize(self, l2):
+        assert l2 >= 0.0
+        if l2 > 0.0:
+            O.saxpy(l2, self.weights, self.grad_weights)
+
+    def accumulate_grads(self, scale, momentum):
+        for _, g, v in self._triples():
+            O.sscal(momentum, v)
+            O.saxpy(scale, g, v)
+
+    def update_params(self, scale):
+        for w, _, v in self._triples():
+            O.saxpy(scale, v, w)
+
+    def update_params2(self, grad_scale, update_scale):
+        if grad_scale != 0.0:
+            for w, g, _ in self._triples():
+                O.saxpy(grad_scale, g, w)
+        if update_scale != 0.0:
+            for w, _, v in self._triples():
+                O.saxpy(update_scale, v, w)
+
+    def save_params(self):
+        self.save_weights[...] = self.weights
+        self.save_scale[...], self.save_bias[...] = self.scale, self.bias
+        self.save_running_mean[...], self.save_running_ivar[...] = self.running_mean, self.running_ivar
+
+    def restore_params(self):
+        self.weights[...] = self.save_weights
+        self.scale[...], self.bias[...] = self.save_scale, self.save_bias
+        self.running_mean, self.running_ivar = self.save_running_mean.copy(), self.save_running_ivar.copy()
+
+    def reset(self):
+        for _, g, _ in self._triples():
+            O.sscal(0.0, g)
+
+    def params_len(self):
+        return self.weights.size + 4 * self.scale.size
+
+
+class _UnitsParams:
+    """What SequentialOperatorWorker fans the SGD methods out to, for an operator made of several units."""
+
+    def __init__(self, units):
+        self.units = units
+
+    def params_len(self):
+        return sum(u.params_len() for u in self.units)
+
+    def __getattr__(self, name):
+        if name in ("regularize", "accumulate_grads", "update_params", "update_params2", "save_params", "restore_params", "reset"):
+            return lambda *a: [getattr(u, name)(*a) for u in self.units]
+        raise AttributeError(name)
+
+
+class BNormConv2dOperator:
+    """out = act(BN(conv(in))) (src/operator/conv.rs:461-640)."""
+    kind = "BNormConv2dOperator"
+    wants_phase = True
+
+    def __init__(self, batch, in_dims, conv_size, conv_stride, conv_pad, out_channels, act_func, mov_avg=("Exponential", 0.1),
+                 epsilon=1e-5):
+        self.units = [_BNormUnit(batch, in_dims, conv_size, conv_stride, conv_pad, out_channels)]
+        self.p = _UnitsParams(self.units)
+        self.act, self.mov_avg, self.epsilon = act_func, mov_avg, epsilon
+        self.out_dims = self.units[0].out_dims
+        self.out_act = np.zeros_like(self.units[0].pre_act)
+        self.out_delta = np.zeros_like(self.out_act)
+
+    def forward(self, in_act, training=True, t=0):
+        self.out_act = self.units[0].forward(in_act, None, 0.0, training, t, self.mov_avg, self.epsilon)
+        if self.act == "Rect":
+            O.rect_inplace(self.out_act)
+        return self.out_act
+
+    def backward(self, want_in_delta):
+        if self.act == "Rect":
+            O.rect_backprop_inplace(self.out_act, self.out_delta)
+        self.units[0].backward_params(self.out_delta)
+        return self.units[0].backward_data() if want_in_delta else None
+
+
+class StackResConv2dOperator:
+    """out = act(in + BN2(conv2(act(BN1(conv1(in)))))), 3x3 / stride 1 / pad 1 (src/operator/conv.rs:1497-1830)."""
+    kind = "StackResConv2dOperator"
+    wants_phase = True
+
+    def __init__(self, batch, in_dims, act_func, mov_avg=("Exponential", 0.1), epsilon=1e-5):
+        c = in_dims[2]
+        self.units = [_BNormUnit(batch, in_dims, 3, 1, 1, c), _BNormUnit(batch, in_dims, 3, 1, 1, c)]
+        self.p = _UnitsParams(self.units)
+        self.act, self.mov_avg, self.epsilon = act_func, mov_avg, epsilon
+        self.out_dims = in_dims
+        self.out_act = np.zeros_like(self.units[0].pre_act)
+        self.out_delta = np.zeros_like(self.out_act)
+
+    def forward(self, in_act, training=True, t=0):
+        u1, u2 = self.units
+        self.mid_act = u1.forward(in_act, None, 0.0, training, t, self.mov_avg, self.epsilon)
+        if self.act == "Rect":
+            O.rect_inplace(self.mid_act)
+        self.out_act = u2.forward(self.mid_act, in_act.reshape(self.out_act.shape), 1.0, training, t, self.mov_avg, self.epsilon)
+        if self.act == "Rect":
+            O.rect_inplace(self.out_act)
+        return self.out_act
+
+    def backward(self, want_in_delta):
+        u1, u2 = self.units
+        if self.act == "Rect":
+            O.rect_backprop_inplace(self.out_act, self.out_delta)
+        u2.backward_params(self.out_delta)
+        self.mid_delta = u2.backward_data()
+        if self.act == "Rect":
+            O.rect_backprop_inplace(self.mid_act, self.mid_delta)
+        u1.backward_params(self.mid_delta)
+        if not want_in_delta:
+            return None
+        return u1.backward_data(1.0, self.out_delta.reshape(u1.x_shape).copy())
+
+
+class ProjStackResConv2dOperator:
+    """out = act(BN2(conv2(act(BN1(conv1(in))))) + BN3(conv3(in))): conv1 3x3 / stride s / pad 1, conv2 3x3 / 1 / 1,
+    conv3 1x1 / stride s / pad 0, s = 1 or 2 from the two extents (src/operator/conv.rs:2331-2338, 2935-3385)."""
+    kind = "ProjStackResConv2dOperator"
+    wants_phase = True
+
+    def __init__(self, batch, in_dims, out_dims, act_func, mov_avg=("Exponential", 0.1), epsilon=1e-5):
+        if in_dims[:2] == out_dims[:2]:
+            s = 1
+        else:
+            assert in_dims[0] == 2 * out_dims[0] and in_dims[1] == 2 * out_dims[1]
+            s = 2
+        oc = out_dims[2]
+        self.units = [_BNormUnit(batch, in_dims, 3, s, 1, oc), _BNormUnit(batch, out_dims, 3, 1, 1, oc),
+                      _BNormUnit(batch, in_dims, 1, s, 0, oc)]
+        self.p = _UnitsParams(self.units)
+        self.act, self.mov_avg, self.epsilon = act_func, mov_avg, epsilon
+        self.out_dims = out_dims
+        self.out_act = np.zeros_like(self.units[1].pre_act)
+        self.out_delta = np.zeros_like(self.out_act)
+
+    def forward(self, in_act, training=True, t=0):
+        u1, u2, u3 = self.units
+        self.mid_act = u1.forward(in_act, None, 0.0, training, t, self.mov_avg, self.epsilon)
+        if self.act == "Rect":
+            O.rect_inplace(self.mid_act)
+        out = u2.forward(self.mid_act, None, 0.0, training, t, self.mov_avg, self.epsilon)
+        self.out_act = u3.forward(in_act, out, 1.0, training, t, self.mov_avg, self.epsilon)
+        if self.act == "Rect":
+            O.rect_inplace(self.out_act)
+        return self.out_act
+
+    def backward(self, want_in_delta):
+        u1, u2, u3 = self.units
+        if self.act == "Rect":
+            O.rect_backprop_inplace(self.out_act, self.out_delta)
+        u2.backward_params(self.out_delta)
+        self.mid_delta = u2.backward_data()
+        if self.act == "Rect":
+            O.rect_backprop_inplace(self.mid_act, self.mid_delta)
+        u1.backward_params(self.mid_delta)
+        u3.backward_params(self.out_delta)
+        if not want_in_delta:
+            return None
+        return u3.backward_data(1.0, u1.backward_data())
+
+
 class SequentialOperatorWorker:
     """layers: list of tuples mirroring the SequentialOperatorConfig builder calls, e.g.
     ("conv2d", in_dims, size, stride, pad, out_channels, act), ("pool2d", in_dims, size, stride, pad, op, ceil),
     ("affine", in, out, act); num_categories closes the chain with SoftmaxKLLoss."""
 
-    def __init__(self, layers, num_categories, batch, fast=False):
+    def __init__(self, layers, num_categories, batch, fast=False, bnorm_mov_avg=("Exponential", 0.1), bnorm_epsilon=1e-5):
         self.batch, self.C = batch, num_categories
         self.hidden = []
+        if isinstance(bnorm_mov_avg, str):
+            bnorm_mov_avg = (bnorm_mov_avg, 0.0)
+        bnorm = {"mov_avg": bnorm_mov_avg, "epsilon": bnorm_epsilon}
         for l in layers:
             if l[0] == "conv2d":
                 self.hidden.append(Conv2dOperator(batch, *l[1:], fast=fast))
@@ -249,6 +473,12 @@ class SequentialOperatorWorker:
                 self.hidden.append(DropoutOperator(batch, *l[1:]))
             elif l[0] == "local_res_norm":
                 self.hidden.append(LocalResNormOperator(batch, *l[1:]))
+            elif l[0] == "bnorm_conv2d":
+                self.hidden.append(BNormConv2dOperator(batch, *l[1:], **bnorm))
+            elif l[0] == "stack_res_conv2d":
+                self.hidden.append(StackResConv2dOperator(batch, *l[1:], **bnorm))
+            elif l[0] == "proj_stack_res_conv2d":
+                self.hidden.append(ProjStackResConv2dOperator(batch, *l[1:], **bnorm))
             else:
                 raise ValueError(l[0])
         self.labels = np.zeros((batch,), np.int32)
@@ -256,16 +486,18 @@ class SequentialOperatorWorker:
         self.out_cats = np.zeros((batch,), np.int32)
 
     def params_len(self):
-        return sum(op.p.weights.size + op.p.bias.size for op in self.hidden if op.p is not None)
+        return sum(op.p.params_len() if hasattr(op.p, "params_len") else op.p.weights.size + op.p.bias.size
+                   for op in self.hidden if op.p is not None)
 
     def stage_batch(self, labels, weight):
         self.labels[...] = labels
         self.weights[...] = weight
 
-    def forward(self, frames):
+    def forward(self, frames, training=True, t=0):
+        """`training`, `t`: the OpPhase the batch-normalised operators read (Training{t} or Inference)."""
         act = frames
         for op in self.hidden:
-            act = op.forward(act)
+            act = op.forward(act, training, t) if getattr(op, "wants_phase", False) else op.forward(act)
         self.out_values = O.softmax_fwd(np.ascontiguousarray(act.reshape(self.batch, self.C)))
 
     def store_output_categories(self):

@@ -59,6 +59,12 @@ PROTOTYPES = {
     "rh_rng_fill_uniform01_device": (_int, [C.c_uint64, C.c_uint64, C.c_uint64, _vp, _sz, _vp]),
     "rh_lrn_fwd": (_int, [C.POINTER(LrnGeom), _vp, _vp, _vp, _vp]),
     "rh_lrn_bwd": (_int, [C.POINTER(LrnGeom), _vp, _vp, _vp, _vp, _vp, _vp]),
+    "rh_bnorm_workspace_bytes": (_sz, [_int, _int, _int]),
+    "rh_bnorm_fwd_train": (_int, [_int, _int, _int, _f, _vp, _f, _vp, C.c_double, C.c_double, _vp, _vp, _vp, _vp, _vp, _vp,
+                                  _vp, _sz, _int, _vp]),
+    "rh_bnorm_fwd_infer": (_int, [_int, _int, _int, _f, _vp, _f, _vp, C.c_double, _vp, _vp, _vp, _vp, _vp, _sz, _int, _vp]),
+    "rh_bnorm_bwd": (_int, [_int, _int, _int, _f, _f, _vp, _vp, _vp, _f, _f, C.c_double, _vp, _vp, _vp, _vp, _vp, _vp, _sz,
+                            _vp]),
     "rh_conv2d_out_dim": (_i32, [_i32, _i32, _i32, _i32]),
     "rh_conv2d_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _int]),
     "rh_conv2d_fwd": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _vp, _sz, _int, _vp]),

@@ -149,6 +149,44 @@ int rho_config_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c,
     cfg->cfg.conv2d(c);
   })
 }
+static BNormMovingAverage mov_avg_of(int kind, double ema_factor) {
+  if (kind == RHO_BNORM_CUMULATIVE) return BNormMovingAverage::MakeCumulative();
+  if (kind != RHO_BNORM_EXPONENTIAL || !(ema_factor >= 0.0 && ema_factor <= 1.0)) panic("unknown batch norm moving average");
+  return BNormMovingAverage::MakeExponential(ema_factor);
+}
+int rho_config_bnorm_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t conv_size, int32_t conv_stride,
+                            int32_t conv_pad, int32_t out_channels, int mov_avg_kind, double ema_factor, double epsilon,
+                            int act_func, int init_kind, float init_value) {
+  RHO_TRY({
+    RHO_REQ(cfg && in_w > 0 && in_h > 0 && in_c > 0 && conv_size > 0 && conv_stride > 0 && conv_pad >= 0 && out_channels > 0);
+    RHO_REQ(epsilon > 0.0);
+    BNormConv2dOperatorConfig c = {{(size_t)in_w, (size_t)in_h, (size_t)in_c}, (size_t)conv_size, (size_t)conv_stride,
+                                   (size_t)conv_pad, (size_t)out_channels, mov_avg_of(mov_avg_kind, ema_factor), epsilon,
+                                   act_of(act_func), init_of(init_kind, init_value)};
+    cfg->cfg.bnorm_conv2d(c);
+  })
+}
+int rho_config_stack_res_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int mov_avg_kind, double ema_factor,
+                                double epsilon, int act_func, int init_kind, float init_value) {
+  RHO_TRY({
+    RHO_REQ(cfg && in_w > 0 && in_h > 0 && in_c > 0 && epsilon > 0.0);
+    StackResConv2dOperatorConfig c = {{(size_t)in_w, (size_t)in_h, (size_t)in_c}, mov_avg_of(mov_avg_kind, ema_factor), epsilon,
+                                      act_of(act_func), init_of(init_kind, init_value)};
+    cfg->cfg.stack_res_conv2d(c);
+  })
+}
+int rho_config_proj_stack_res_conv2d(rho_config* cfg, int32_t in_w, int32_t in_h, int32_t in_c, int32_t out_w, int32_t out_h,
+                                     int32_t out_c, int mov_avg_kind, double ema_factor, double epsilon, int act_func,
+                                     int init_kind, float init_value) {
+  RHO_TRY({
+    RHO_REQ(cfg && in_w > 0 && in_h > 0 && in_c > 0 && out_w > 0 && out_h > 0 && out_c > 0 && epsilon > 0.0);
+    RHO_REQ((in_w == out_w && in_h == out_h) || (in_w == 2 * out_w && in_h == 2 * out_h));
+    ProjStackResConv2dOperatorConfig c = {{(size_t)in_w, (size_t)in_h, (size_t)in_c}, {(size_t)out_w, (size_t)out_h, (size_t)out_c},
+                                          mov_avg_of(mov_avg_kind, ema_factor), epsilon, act_of(act_func),
+                                          init_of(init_kind, init_value)};
+    cfg->cfg.proj_stack_res_conv2d(c);
+  })
+}
 int rho_config_affine(rho_config* cfg, int32_t in_channels, int32_t out_channels, int act_func, int init_kind, float init_value) {
   RHO_TRY({
     RHO_REQ(cfg && in_channels > 0 && out_channels > 0);

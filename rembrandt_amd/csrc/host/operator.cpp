@@ -46,6 +46,11 @@ Dims3 Conv2dOperatorConfig::get_out_dims() const {
           out_dim_floor(in_dims.h, conv_size, conv_stride, conv_pad), out_channels};
 }
 
+Dims3 BNormConv2dOperatorConfig::get_out_dims() const {
+  return {out_dim_floor(in_dims.w, conv_size, conv_stride, conv_pad),
+          out_dim_floor(in_dims.h, conv_size, conv_stride, conv_pad), out_channels};
+}
+
 Dims3 Pool2dOperatorConfig::get_out_dims() const {
   const int r = ceil_mode ? RH_ROUND_CEIL : RH_ROUND_FLOOR;
   return {(size_t)rh_pool2d_out_dim((int)in_dims.w, (int)pool_size, (int)pool_stride, (int)pool_pad, r),
@@ -103,6 +108,9 @@ size_t OperatorConfig::params_len() const {
   switch (kind) {
     case Affine: return affine.params_len();
     case Conv2d: return conv2d.params_len();
+    case BNormConv2d: return bnorm_conv2d.params_len();
+    case StackResConv2d: return stack_res_conv2d.params_len();
+    case ProjStackResConv2d: return proj_stack_res_conv2d.params_len();
     default: return 0;
   }
 }
@@ -151,6 +159,27 @@ SequentialOperatorConfig& SequentialOperatorConfig::local_res_norm(const LocalRe
   OperatorConfig c = OperatorConfig();
   c.kind = OperatorConfig::LocalResNorm;
   c.lrn = cfg;
+  hidden_ops.push_back(c);
+  return *this;
+}
+SequentialOperatorConfig& SequentialOperatorConfig::bnorm_conv2d(const BNormConv2dOperatorConfig& cfg) {
+  OperatorConfig c{};
+  c.kind = OperatorConfig::BNormConv2d;
+  c.bnorm_conv2d = cfg;
+  hidden_ops.push_back(c);
+  return *this;
+}
+SequentialOperatorConfig& SequentialOperatorConfig::stack_res_conv2d(const StackResConv2dOperatorConfig& cfg) {
+  OperatorConfig c{};
+  c.kind = OperatorConfig::StackResConv2d;
+  c.stack_res_conv2d = cfg;
+  hidden_ops.push_back(c);
+  return *this;
+}
+SequentialOperatorConfig& SequentialOperatorConfig::proj_stack_res_conv2d(const ProjStackResConv2dOperatorConfig& cfg) {
+  OperatorConfig c{};
+  c.kind = OperatorConfig::ProjStackResConv2d;
+  c.proj_stack_res_conv2d = cfg;
   hidden_ops.push_back(c);
   return *this;
 }
@@ -938,6 +967,454 @@ class LocalResNormOperator : public Operator {
   DeviceBuffer<float> denom_;
 };
 
+// ---- conv (no bias) + spatial batch norm: the unit the three batch-normalised operators are made of ------------
+// Buffers and update rules per unit as in src/operator/conv.rs:133-160 (buffers), :640-911 (regularize on the
+// filter only; accumulate / update / save / restore / reset on filter, scale and bias; the moving statistics are
+// saved and restored with the parameters).
+struct BNormConvUnit {
+  typedef std::unique_ptr<DeviceBuffer<float>> Buf;
+  Dims3 in_dims, out_dims;
+  size_t conv_size = 0, conv_stride = 1, conv_pad = 0, wlen = 0, chans = 0, batch_cap = 0;
+  Ctx ctx;
+  Buf weights, grad_weights, acc_grad_weights, save_weights;
+  Buf scale, bias, scale_grad, bias_grad, acc_scale_grad, acc_bias_grad, save_scale, save_bias;
+  Buf running_mean, running_ivar, save_running_mean, save_running_ivar, cached_mean, cached_ivar;
+  Buf pre_act, pre_delta;  // the conv output the batch norm reads, and the gradient w.r.t. it
+  bool backward = false;
+
+  void alloc(size_t batch, Dims3 in, size_t size, size_t stride, size_t pad, size_t out_channels, bool bwd, Ctx c) {
+    in_dims = in; conv_size = size; conv_stride = stride; conv_pad = pad; chans = out_channels; ctx = c; backward = bwd;
+    batch_cap = batch;
+    out_dims = {out_dim_floor(in.w, size, stride, pad), out_dim_floor(in.h, size, stride, pad), out_channels};
+    wlen = size * size * in.c * out_channels;
+    auto mk = [&](size_t n) { return Buf(new DeviceBuffer<float>(n, c)); };
+    weights = mk(wlen);
+    scale = mk(chans); bias = mk(chans); running_mean = mk(chans); running_ivar = mk(chans);
+    cached_mean = mk(chans); cached_ivar = mk(chans);
+    scale_grad = mk(chans); bias_grad = mk(chans); acc_scale_grad = mk(chans); acc_bias_grad = mk(chans);
+    save_scale = mk(chans); save_bias = mk(chans); save_running_mean = mk(chans); save_running_ivar = mk(chans);
+    pre_act = mk(out_dims.len() * batch);
+    if (bwd) {
+      grad_weights = mk(wlen); acc_grad_weights = mk(wlen); save_weights = mk(wlen);
+      pre_delta = mk(out_dims.len() * batch);
+    }
+  }
+  rh_conv_geom geom(size_t batch) const {
+    rh_conv_geom g;
+    g.N = (int)batch; g.C = (int)in_dims.c; g.H = (int)in_dims.h; g.W = (int)in_dims.w;
+    g.K = (int)chans; g.R = g.S = (int)conv_size; g.stride = (int)conv_stride; g.pad = (int)conv_pad;
+    return g;
+  }
+  int plane() const { return (int)(out_dims.w * out_dims.h); }
+  size_t workspace_bytes() const {
+    const rh_conv_geom g = geom(batch_cap);
+    size_t ws = std::max(rh_conv2d_workspace_bytes(&g, RH_CONV_FWD), rh_bnorm_workspace_bytes(g.N, g.K, plane()));
+    if (backward) {
+      ws = std::max(ws, rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_FILTER));
+      ws = std::max(ws, rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_DATA));
+    }
+    return ws;
+  }
+  rh_stream_t s() const { return ctx->stream(); }
+  void fill(DeviceBuffer<float>& b, float v) { unwrap(rh_memset_f32(b.as_mut_ptr(), v, b.len(), s()), "set_constant"); }
+
+  // Filter from the seeded generator (fan-in = size*size*in channels); scale 1, bias 0, moving mean 0, moving
+  // inverse deviation 1 (src/operator/conv.rs:292-345).
+  void init(const ParamsInit& init, uint64_t seed, uint64_t stream_id, const char* who) {
+    std::vector<float> w(wlen);
+    const size_t fan_in = conv_size * conv_size * in_dims.c;
+    switch (init.kind) {
+      case ParamsInit::Disabled: panic(std::string(who) + ": params init explicitly disabled");
+      case ParamsInit::Uniform:
+        unwrap(rh_rng_fill_uniform(seed, stream_id, w.data(), wlen, -init.value, init.value), "rh_rng_fill_uniform");
+        break;
+      case ParamsInit::Normal:
+        unwrap(rh_rng_fill_normal(seed, stream_id, w.data(), wlen, 0.0f, init.value), "rh_rng_fill_normal");
+        break;
+      case ParamsInit::Xavier: panic(std::string(who) + ": Xavier init is unimplemented for this operator");
+      case ParamsInit::KaimingFwd:
+        unwrap(rh_rng_fill_normal(seed, stream_id, w.data(), wlen, 0.0f, (float)std::sqrt(2.0 / (double)fan_in)),
+               "rh_rng_fill_normal");
+        break;
+    }
+    weights->sync_load(w.data(), wlen);
+    fill(*scale, 1.0f); fill(*bias, 0.0f); fill(*running_mean, 0.0f); fill(*running_ivar, 1.0f);
+  }
+
+  // out = beta_out*out + BN(conv(in)); `relu` clamps the blended result (the in-place rect that follows in the reference).
+  void forward(size_t batch, const float* in, float* out, float beta_out, OpPhase phase, const BNormMovingAverage& avg,
+               double epsilon, bool relu, DeviceBuffer<uint8_t>& ws, bool bf16) {
+    const rh_conv_geom g = geom(batch);
+    unwrap(rh_conv2d_fwd(&g, 1.0f, in, weights->as_ptr(), 0.0f, pre_act->as_mut_ptr(), nullptr, ws.as_mut_ptr(), ws.len(),
+                         bf16 ? RH_MATH_BF16_MFMA_FP32ACC : 0, s()), "conv2d forward");
+    const int flags = relu ? RH_FUSE_RELU : 0;
+    if (phase.training) {
+      if (!backward) panic("batch norm training missing backward operator");
+      unwrap(rh_bnorm_fwd_train(g.N, g.K, plane(), 1.0f, pre_act->as_ptr(), beta_out, out, avg.at_iter(phase.t), epsilon,
+                                scale->as_ptr(), bias->as_ptr(), running_mean->as_mut_ptr(), running_ivar->as_mut_ptr(),
+                                cached_mean->as_mut_ptr(), cached_ivar->as_mut_ptr(), ws.as_mut_ptr(), ws.len(), flags, s()),
+             "batch norm forward training");
+    } else {
+      unwrap(rh_bnorm_fwd_infer(g.N, g.K, plane(), 1.0f, pre_act->as_ptr(), beta_out, out, epsilon, scale->as_ptr(),
+                                bias->as_ptr(), running_mean->as_ptr(), running_ivar->as_ptr(), ws.as_mut_ptr(), ws.len(),
+                                flags, s()), "batch norm forward inference");
+    }
+  }
+  // pre_delta = dBN(out_delta) with the scale / bias gradients accumulated, then grad_weights += dconv(in, pre_delta).
+  void backward_params(size_t batch, const float* in, const float* out_delta, double epsilon, DeviceBuffer<uint8_t>& ws) {
+    RB_ASSERT(backward);
+    const rh_conv_geom g = geom(batch);
+    unwrap(rh_bnorm_bwd(g.N, g.K, plane(), 1.0f, 0.0f, pre_act->as_ptr(), out_delta, pre_delta->as_mut_ptr(), 1.0f, 1.0f,
+                        epsilon, scale->as_ptr(), scale_grad->as_mut_ptr(), bias_grad->as_mut_ptr(), cached_mean->as_ptr(),
+                        cached_ivar->as_ptr(), ws.as_mut_ptr(), ws.len(), s()), "batch norm backward");
+    unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in, pre_delta->as_ptr(), 1.0f, grad_weights->as_mut_ptr(), ws.as_mut_ptr(),
+                                ws.len(), 0, s()), "conv2d backward filter");
+  }
+  // in_delta = beta*in_delta + dconv^T(weights, pre_delta)
+  void backward_data(size_t batch, float* in_delta, float beta, DeviceBuffer<uint8_t>& ws) {
+    const rh_conv_geom g = geom(batch);
+    unwrap(rh_conv2d_bwd_data(&g, 1.0f, weights->as_ptr(), pre_delta->as_ptr(), beta, in_delta, ws.as_mut_ptr(), ws.len(), 0,
+                              s()), "conv2d backward data");
+  }
+
+  void axpy(float a, const DeviceBuffer<float>& x, DeviceBuffer<float>& y) {
+    unwrap(rh_saxpy((int64_t)x.len(), a, x.as_ptr(), y.as_mut_ptr(), s()), "sum");
+  }
+  void scal(float a, DeviceBuffer<float>& x) { unwrap(rh_sscal((int64_t)x.len(), a, x.as_mut_ptr(), s()), "scale"); }
+  void copy(DeviceBuffer<float>& dst, const DeviceBuffer<float>& src) {
+    unwrap(rh_copy_d2d(dst.as_mut_ptr(), src.as_ptr(), src.len() * 4, s()), "send");
+  }
+  void regularize(Regularization reg) {
+    RB_ASSERT(backward);
+    RB_ASSERT(reg.l2_reg_coef >= 0.0f);
+    if (reg.l2_reg_coef > 0.0f) axpy(reg.l2_reg_coef, *weights, *grad_weights);
+  }
+  void accumulate_grads(float sc, float momentum) {
+    RB_ASSERT(backward);
+    scal(momentum, *acc_grad_weights); axpy(sc, *grad_weights, *acc_grad_weights);
+    scal(momentum, *acc_scale_grad); axpy(sc, *scale_grad, *acc_scale_grad);
+    scal(momentum, *acc_bias_grad); axpy(sc, *bias_grad, *acc_bias_grad);
+  }
+  void update_params(float sc) {
+    RB_ASSERT(backward);
+    axpy(sc, *acc_grad_weights, *weights); axpy(sc, *acc_scale_grad, *scale); axpy(sc, *acc_bias_grad, *bias);
+  }
+  void update_params2(float grad_scale, float update_scale) {
+    RB_ASSERT(backward);
+    if (grad_scale != 0.0f) { axpy(grad_scale, *grad_weights, *weights); axpy(grad_scale, *scale_grad, *scale); axpy(grad_scale, *bias_grad, *bias); }
+    if (update_scale != 0.0f) { axpy(update_scale, *acc_grad_weights, *weights); axpy(update_scale, *acc_scale_grad, *scale); axpy(update_scale, *acc_bias_grad, *bias); }
+  }
+  void save_params() {
+    RB_ASSERT(backward);
+    copy(*save_weights, *weights); copy(*save_scale, *scale); copy(*save_bias, *bias);
+    copy(*save_running_mean, *running_mean); copy(*save_running_ivar, *running_ivar);
+  }
+  void restore_params() {
+    RB_ASSERT(backward);
+    copy(*weights, *save_weights); copy(*scale, *save_scale); copy(*bias, *save_bias);
+    copy(*running_mean, *save_running_mean); copy(*running_ivar, *save_running_ivar);
+  }
+  void reset() {
+    if (!backward) return;
+    scal(0.0f, *grad_weights); scal(0.0f, *scale_grad); scal(0.0f, *bias_grad);
+  }
+  void fused_sgd_step(float l2, float sc, float momentum, float apply) {
+    RB_ASSERT(backward);
+    unwrap(rh_sgd_momentum_step((int64_t)wlen, weights->as_mut_ptr(), grad_weights->as_mut_ptr(), acc_grad_weights->as_mut_ptr(),
+                                l2, sc, momentum, apply, 1, s()), "rh_sgd_momentum_step");
+    unwrap(rh_sgd_momentum_step((int64_t)chans, scale->as_mut_ptr(), scale_grad->as_mut_ptr(), acc_scale_grad->as_mut_ptr(),
+                                0.0f, sc, momentum, apply, 1, s()), "rh_sgd_momentum_step");
+    unwrap(rh_sgd_momentum_step((int64_t)chans, bias->as_mut_ptr(), bias_grad->as_mut_ptr(), acc_bias_grad->as_mut_ptr(),
+                                0.0f, sc, momentum, apply, 1, s()), "rh_sgd_momentum_step");
+  }
+  // Blobs: filter as (size*size*in channels, out channels), then four (1, out channels) rows
+  // (src/operator/conv.rs:361-406 params: scale, bias, moving mean, moving inverse deviation;
+  //  :408-459 state: momentum of filter, scale, bias, then the cached batch mean and inverse deviation).
+  void encode(std::vector<uint8_t>& blob, const DeviceBuffer<float>& w, const DeviceBuffer<float>* const rows[4]) const {
+    ctx->sync();
+    std::vector<float> h(wlen);
+    w.sync_store(h.data(), wlen);
+    const size_t wd[2] = {wlen / chans, chans}, rd[2] = {1, chans};
+    ndarray_serialize(blob, h.data(), wd, 2);
+    for (int i = 0; i < 4; ++i) {
+      std::vector<float> r(chans);
+      rows[i]->sync_store(r.data(), chans);
+      ndarray_serialize(blob, r.data(), rd, 2);
+    }
+  }
+  size_t decode(const uint8_t* blob, size_t len, DeviceBuffer<float>& w, DeviceBuffer<float>* const rows[4], const char* who) {
+    std::vector<size_t> dims;
+    std::vector<float> data;
+    size_t off = ndarray_deserialize(blob, len, &dims, &data);
+    if (dims.size() != 2 || dims[0] != wlen / chans || dims[1] != chans) panic(std::string(who) + ": weights blob has the wrong bound");
+    w.sync_load(data.data(), wlen);
+    for (int i = 0; i < 4; ++i) {
+      off += ndarray_deserialize(blob + off, len - off, &dims, &data);
+      if (dims.size() != 2 || dims[0] != 1 || dims[1] != chans) panic(std::string(who) + ": batch norm blob has the wrong bound");
+      rows[i]->sync_load(data.data(), chans);
+    }
+    return off;
+  }
+  void encode_params(std::vector<uint8_t>& blob) const {
+    const DeviceBuffer<float>* const rows[4] = {scale.get(), bias.get(), running_mean.get(), running_ivar.get()};
+    encode(blob, *weights, rows);
+  }
+  size_t decode_params(const uint8_t* blob, size_t len, const char* who) {
+    DeviceBuffer<float>* const rows[4] = {scale.get(), bias.get(), running_mean.get(), running_ivar.get()};
+    return decode(blob, len, *weights, rows, who);
+  }
+  void encode_state(std::vector<uint8_t>& blob) const {
+    RB_ASSERT(backward);
+    const DeviceBuffer<float>* const rows[4] = {acc_scale_grad.get(), acc_bias_grad.get(), cached_mean.get(), cached_ivar.get()};
+    encode(blob, *acc_grad_weights, rows);
+  }
+  size_t decode_state(const uint8_t* blob, size_t len, const char* who) {
+    RB_ASSERT(backward);
+    DeviceBuffer<float>* const rows[4] = {acc_scale_grad.get(), acc_bias_grad.get(), cached_mean.get(), cached_ivar.get()};
+    return decode(blob, len, *acc_grad_weights, rows, who);
+  }
+  bool buffer(int id, float** ptr, size_t* len) {
+    DeviceBuffer<float>* b = nullptr;
+    switch (id) {
+      case 2: b = weights.get(); break;
+      case 4: b = grad_weights.get(); break;
+      case 6: b = acc_grad_weights.get(); break;
+      case 8: b = scale.get(); break;
+      case 9: b = bias.get(); break;
+      case 10: b = scale_grad.get(); break;
+      case 11: b = bias_grad.get(); break;
+      case 12: b = running_mean.get(); break;
+      case 13: b = running_ivar.get(); break;
+      case 14: b = cached_mean.get(); break;
+      case 15: b = cached_ivar.get(); break;
+      case 16: b = acc_scale_grad.get(); break;
+      case 17: b = acc_bias_grad.get(); break;
+      case 18: b = pre_act.get(); break;
+      case 19: b = pre_delta.get(); break;
+      default: return false;
+    }
+    if (!b) return false;
+    *ptr = b->as_mut_ptr();
+    *len = b->len();
+    return true;
+  }
+};
+
+// Common part of the three batch-normalised operators: the units' parameter plumbing.
+class BNormUnitsOperator : public Operator {
+ public:
+  BNormUnitsOperator(size_t batch_size, size_t n_units, const Operator* prev_op, Ctx context, ExecOptions opts, const char* who)
+      : batch_cap_(batch_size), units_(n_units), context_(context), opts_(opts) {
+    RB_ASSERT(prev_op != nullptr);
+    in_act_ = prev_op->get_output_vars();
+    if (!in_act_) panic(std::string(who) + " missing required prev operator output vars");
+    in_delta_ = prev_op->get_output_deltas();
+  }
+  size_t batch_size() const override { return batch_cap_; }
+  SharedDeviceBuf get_output_vars() const override { return out_act_; }
+  SharedDeviceBuf get_output_deltas() const override { return out_delta_; }
+  void regularize(Regularization reg) override { for (auto& u : units_) u.regularize(reg); }
+  void accumulate_grads(float scale, float momentum) override { for (auto& u : units_) u.accumulate_grads(scale, momentum); }
+  void update_params(float scale) override { for (auto& u : units_) u.update_params(scale); }
+  void update_params2(float g, float v) override { for (auto& u : units_) u.update_params2(g, v); }
+  void save_params() override { for (auto& u : units_) u.save_params(); }
+  void restore_params() override { for (auto& u : units_) u.restore_params(); }
+  void reset() override { for (auto& u : units_) u.reset(); }
+  void fused_sgd_step(float l2, float scale, float mu, float apply) override { for (auto& u : units_) u.fused_sgd_step(l2, scale, mu, apply); }
+  void encode_params(std::vector<uint8_t>& blob) override { for (auto& u : units_) u.encode_params(blob); }
+  size_t decode_params(const uint8_t* blob, size_t len) override {
+    size_t off = 0;
+    for (auto& u : units_) off += u.decode_params(blob + off, len - off, kind());
+    return off;
+  }
+  void encode_state(std::vector<uint8_t>& blob) override { for (auto& u : units_) u.encode_state(blob); }
+  size_t decode_state(const uint8_t* blob, size_t len) override {
+    size_t off = 0;
+    for (auto& u : units_) off += u.decode_state(blob + off, len - off, kind());
+    return off;
+  }
+  void init_params(const uint64_t seed[2]) override {
+    for (size_t u = 0; u < units_.size(); ++u) units_[u].init(init_weights_, seed[0], seed[1] + 0x9E3779B97F4A7C15ull * u, kind());
+  }
+  bool buffer(int which, float** ptr, size_t* len) override {
+    if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
+    if (which == 1) { *ptr = out_delta_->as_mut_ptr(); *len = out_delta_->len(); return true; }
+    if (which == 30 && mid_act_) { *ptr = mid_act_->as_mut_ptr(); *len = mid_act_->len(); return true; }
+    if (which == 31 && mid_delta_) { *ptr = mid_delta_->as_mut_ptr(); *len = mid_delta_->len(); return true; }
+    const int u = which / 100;
+    if (u < 0 || (size_t)u >= units_.size()) return false;
+    return units_[(size_t)u].buffer(which % 100, ptr, len);
+  }
+
+ protected:
+  void alloc_common(Dims3 out_dims, bool bwd) {
+    out_act_.reset(new DeviceBuffer<float>(out_dims.len() * batch_cap_, context_));
+    out_delta_.reset(new DeviceBuffer<float>(out_dims.len() * batch_cap_, context_));
+    size_t ws = 256;
+    for (auto& u : units_) ws = std::max(ws, u.workspace_bytes());
+    workspace_.reset(new DeviceBuffer<uint8_t>(ws, context_));
+    (void)bwd;
+  }
+  // ReLU after a batch norm: inside its apply kernel, or as the separate in-place pass of the reference.
+  bool fuse_relu(ActivationFunction f) const {
+    if (f != ActivationFunction::Identity && f != ActivationFunction::Rect) panic("unimplemented activation function");
+    return f == ActivationFunction::Rect && opts_.fuse_epilogue;
+  }
+  void rect_after(ActivationFunction f, DeviceBuffer<float>& act, size_t frame_len, size_t batch) {
+    if (!opts_.fuse_epilogue) apply_rect(f, act.as_mut_ptr(), frame_len, batch, context_->stream());
+  }
+  size_t batch_cap_;
+  std::vector<BNormConvUnit> units_;
+  Ctx context_;
+  ExecOptions opts_;
+  ParamsInit init_weights_ = ParamsInit::MakeDisabled();
+  SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
+  std::unique_ptr<DeviceBuffer<float>> mid_act_, mid_delta_;
+  std::unique_ptr<DeviceBuffer<uint8_t>> workspace_;
+};
+
+// ---- BNormConv2dOperator (src/operator/conv.rs:106-912) ---------------------------------------------------
+class BNormConv2dOperator : public BNormUnitsOperator {
+ public:
+  BNormConv2dOperator(size_t batch_size, OpCapability capability, const BNormConv2dOperatorConfig& config, const Operator* prev_op,
+                      Ctx context, ExecOptions opts)
+      : BNormUnitsOperator(batch_size, 1, prev_op, context, opts, "BNormConv2dOperator"), config_(config) {
+    RB_ASSERT(in_act_->len() >= config.in_dims.len() * batch_size);
+    init_weights_ = config.init_weights;
+    units_[0].alloc(batch_size, config.in_dims, config.conv_size, config.conv_stride, config.conv_pad, config.out_channels,
+                    backward_enabled(capability), context);
+    alloc_common(units_[0].out_dims, backward_enabled(capability));
+  }
+  void forward(size_t batch_size, OpPhase phase) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    BNormConvUnit& u = units_[0];
+    u.forward(batch_size, in_act_->as_ptr(), out_act_->as_mut_ptr(), 0.0f, phase, config_.bnorm_mov_avg, config_.bnorm_epsilon,
+              fuse_relu(config_.act_func), *workspace_, opts_.bf16_forward);
+    rect_after(config_.act_func, *out_act_, u.out_dims.len(), batch_size);
+  }
+  void backward(size_t batch_size) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    BNormConvUnit& u = units_[0];
+    apply_rect_backprop(config_.act_func, out_act_->as_ptr(), u.out_dims.len(), batch_size, out_delta_->as_mut_ptr(), context_->stream());
+    u.backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    if (in_delta_) u.backward_data(batch_size, in_delta_->as_mut_ptr(), 0.0f, *workspace_);
+  }
+  const char* kind() const override { return "BNormConv2dOperator"; }
+
+ private:
+  BNormConv2dOperatorConfig config_;
+};
+
+// ---- StackResConv2dOperator (src/operator/conv.rs:937-2182) -----------------------------------------------
+// forward (:1497-1672): out <- in; mid = act(BN1(conv1(in))); out += BN2(conv2(mid)); out = act(out).
+// backward (:1674-1830): mask out_delta; unit 2 gradients, mid_delta = conv2^T; mask mid_delta; unit 1 gradients;
+// in_delta <- out_delta; in_delta += conv1^T.
+class StackResConv2dOperator : public BNormUnitsOperator {
+ public:
+  StackResConv2dOperator(size_t batch_size, OpCapability capability, const StackResConv2dOperatorConfig& config,
+                         const Operator* prev_op, Ctx context, ExecOptions opts)
+      : BNormUnitsOperator(batch_size, 2, prev_op, context, opts, "StackResConv2dOperator"), config_(config) {
+    RB_ASSERT(in_act_->len() >= config.in_dims.len() * batch_size);
+    init_weights_ = config.init_weights;
+    const bool bwd = backward_enabled(capability);
+    for (auto& u : units_) u.alloc(batch_size, config.in_dims, 3, 1, 1, config.in_dims.c, bwd, context);
+    alloc_common(config.in_dims, bwd);
+    mid_act_.reset(new DeviceBuffer<float>(config.in_dims.len() * batch_size, context));
+    if (bwd) mid_delta_.reset(new DeviceBuffer<float>(config.in_dims.len() * batch_size, context));
+  }
+  void forward(size_t batch_size, OpPhase phase) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    const size_t len = config_.in_dims.len();
+    const bool fuse = fuse_relu(config_.act_func);
+    units_[0].forward(batch_size, in_act_->as_ptr(), mid_act_->as_mut_ptr(), 0.0f, phase, config_.bnorm_mov_avg,
+                      config_.bnorm_epsilon, fuse, *workspace_, opts_.bf16_forward);
+    rect_after(config_.act_func, *mid_act_, len, batch_size);
+    unwrap(rh_copy_d2d(out_act_->as_mut_ptr(), in_act_->as_ptr(), len * batch_size * 4, context_->stream()), "send");
+    units_[1].forward(batch_size, mid_act_->as_ptr(), out_act_->as_mut_ptr(), 1.0f, phase, config_.bnorm_mov_avg,
+                      config_.bnorm_epsilon, fuse, *workspace_, opts_.bf16_forward);
+    rect_after(config_.act_func, *out_act_, len, batch_size);
+  }
+  void backward(size_t batch_size) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    RB_ASSERT((bool)mid_delta_);
+    const size_t len = config_.in_dims.len();
+    rh_stream_t s = context_->stream();
+    apply_rect_backprop(config_.act_func, out_act_->as_ptr(), len, batch_size, out_delta_->as_mut_ptr(), s);
+    units_[1].backward_params(batch_size, mid_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    units_[1].backward_data(batch_size, mid_delta_->as_mut_ptr(), 0.0f, *workspace_);
+    apply_rect_backprop(config_.act_func, mid_act_->as_ptr(), len, batch_size, mid_delta_->as_mut_ptr(), s);
+    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    if (in_delta_) {
+      unwrap(rh_copy_d2d(in_delta_->as_mut_ptr(), out_delta_->as_ptr(), len * batch_size * 4, s), "send");
+      units_[0].backward_data(batch_size, in_delta_->as_mut_ptr(), 1.0f, *workspace_);
+    }
+  }
+  const char* kind() const override { return "StackResConv2dOperator"; }
+
+ private:
+  StackResConv2dOperatorConfig config_;
+};
+
+// ---- ProjStackResConv2dOperator (src/operator/conv.rs:2210-3560) ------------------------------------------
+// forward (:2935-3172): mid = act(BN1(conv1(in))); out = BN2(conv2(mid)); out += BN3(conv3(in)); out = act(out).
+// backward (:3174-3385): mask out_delta; unit 2 gradients, mid_delta = conv2^T; mask mid_delta; unit 1 gradients;
+// unit 3 gradients from out_delta; in_delta = conv1^T; in_delta += conv3^T.
+class ProjStackResConv2dOperator : public BNormUnitsOperator {
+ public:
+  ProjStackResConv2dOperator(size_t batch_size, OpCapability capability, const ProjStackResConv2dOperatorConfig& config,
+                             const Operator* prev_op, Ctx context, ExecOptions opts)
+      : BNormUnitsOperator(batch_size, 3, prev_op, context, opts, "ProjStackResConv2dOperator"), config_(config) {
+    RB_ASSERT(in_act_->len() >= config.in_dims.len() * batch_size);
+    init_weights_ = config.init_weights;
+    const Dims3 in = config.in_dims, out = config.out_dims;
+    size_t stride;
+    if (in.w == out.w && in.h == out.h) stride = 1;
+    else if (in.w == 2 * out.w && in.h == 2 * out.h) stride = 2;
+    else panic("ProjStackResConv2dOperator: the output extent must equal or halve the input extent");
+    const bool bwd = backward_enabled(capability);
+    units_[0].alloc(batch_size, in, 3, stride, 1, out.c, bwd, context);
+    units_[1].alloc(batch_size, out, 3, 1, 1, out.c, bwd, context);
+    units_[2].alloc(batch_size, in, 1, stride, 0, out.c, bwd, context);
+    for (auto& u : units_) RB_ASSERT(u.out_dims.w == out.w && u.out_dims.h == out.h);
+    alloc_common(out, bwd);
+    mid_act_.reset(new DeviceBuffer<float>(out.len() * batch_size, context));
+    if (bwd) mid_delta_.reset(new DeviceBuffer<float>(out.len() * batch_size, context));
+  }
+  void forward(size_t batch_size, OpPhase phase) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    const size_t len = config_.out_dims.len();
+    const bool fuse = fuse_relu(config_.act_func);
+    units_[0].forward(batch_size, in_act_->as_ptr(), mid_act_->as_mut_ptr(), 0.0f, phase, config_.bnorm_mov_avg,
+                      config_.bnorm_epsilon, fuse, *workspace_, opts_.bf16_forward);
+    rect_after(config_.act_func, *mid_act_, len, batch_size);
+    units_[1].forward(batch_size, mid_act_->as_ptr(), out_act_->as_mut_ptr(), 0.0f, phase, config_.bnorm_mov_avg,
+                      config_.bnorm_epsilon, false, *workspace_, opts_.bf16_forward);
+    units_[2].forward(batch_size, in_act_->as_ptr(), out_act_->as_mut_ptr(), 1.0f, phase, config_.bnorm_mov_avg,
+                      config_.bnorm_epsilon, fuse, *workspace_, opts_.bf16_forward);
+    rect_after(config_.act_func, *out_act_, len, batch_size);
+  }
+  void backward(size_t batch_size) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    RB_ASSERT((bool)mid_delta_);
+    const size_t len = config_.out_dims.len();
+    rh_stream_t s = context_->stream();
+    apply_rect_backprop(config_.act_func, out_act_->as_ptr(), len, batch_size, out_delta_->as_mut_ptr(), s);
+    units_[1].backward_params(batch_size, mid_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    units_[1].backward_data(batch_size, mid_delta_->as_mut_ptr(), 0.0f, *workspace_);
+    apply_rect_backprop(config_.act_func, mid_act_->as_ptr(), len, batch_size, mid_delta_->as_mut_ptr(), s);
+    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    units_[2].backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    if (in_delta_) {
+      units_[0].backward_data(batch_size, in_delta_->as_mut_ptr(), 0.0f, *workspace_);
+      units_[2].backward_data(batch_size, in_delta_->as_mut_ptr(), 1.0f, *workspace_);
+    }
+  }
+  const char* kind() const override { return "ProjStackResConv2dOperator"; }
+
+ private:
+  ProjStackResConv2dOperatorConfig config_;
+};
+
 // ---- SoftmaxKLLossOperator ------------------------------------------------------------------------------
 class SoftmaxKLLossOperator : public LossOperator {
  public:
@@ -1073,6 +1550,15 @@ SequentialOperatorWorker::SequentialOperatorWorker(const SequentialOperatorConfi
                                      0xD0000000ull + hidden_ops_.size()));
         break;
       case OperatorConfig::LocalResNorm: op.reset(new LocalResNormOperator(batch_size, c.lrn, prev, context)); break;
+      case OperatorConfig::BNormConv2d:
+        op.reset(new BNormConv2dOperator(batch_size, capability, c.bnorm_conv2d, prev, context, opts));
+        break;
+      case OperatorConfig::StackResConv2d:
+        op.reset(new StackResConv2dOperator(batch_size, capability, c.stack_res_conv2d, prev, context, opts));
+        break;
+      case OperatorConfig::ProjStackResConv2d:
+        op.reset(new ProjStackResConv2dOperator(batch_size, capability, c.proj_stack_res_conv2d, prev, context, opts));
+        break;
       default: panic("SequentialOperatorWorker: not a hidden operator");
     }
     params_off += c.params_len();

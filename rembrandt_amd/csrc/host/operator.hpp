@@ -173,12 +173,65 @@ struct LocalResNormOperatorConfig {
   float scale, power, min_div;
 };
 
+// How the moving batch-norm statistics weigh the newest batch at iteration t (src/operator/conv.rs:52-73).
+struct BNormMovingAverage {
+  enum Kind { Cumulative, Exponential } kind;
+  double ema_factor;
+  static BNormMovingAverage MakeCumulative() { return {Cumulative, 0.0}; }
+  static BNormMovingAverage MakeExponential(double f) { return {Exponential, f}; }
+  double at_iter(size_t t) const {
+    if (kind == Cumulative) return 1.0 / (1.0 + (double)t);
+    return t == 0 ? 1.0 : ema_factor;
+  }
+};
+
+// conv (no bias) -> spatial batch norm -> activation (src/operator/conv.rs:75-104)
+struct BNormConv2dOperatorConfig {
+  Dims3 in_dims;
+  size_t conv_size, conv_stride, conv_pad, out_channels;
+  BNormMovingAverage bnorm_mov_avg;
+  double bnorm_epsilon;
+  ActivationFunction act_func;
+  ParamsInit init_weights;
+  Dims3 get_out_dims() const;
+  size_t params_len() const { return conv_size * conv_size * in_dims.c * out_channels + 4 * out_channels; }
+};
+
+// y = act(x + BN2(conv3x3(act(BN1(conv3x3(x)))))), channels and extent unchanged (src/operator/conv.rs:914-935)
+struct StackResConv2dOperatorConfig {
+  Dims3 in_dims;
+  BNormMovingAverage bnorm_mov_avg;
+  double bnorm_epsilon;
+  ActivationFunction act_func;
+  ParamsInit init_weights;
+  Dims3 get_out_dims() const { return in_dims; }
+  size_t params_len() const { return 2 * (3 * 3 * in_dims.c * in_dims.c + 4 * in_dims.c); }
+};
+
+// y = act(BN3(conv1x1/s(x)) + BN2(conv3x3(act(BN1(conv3x3/s(x)))))); s = 1 when the extent is kept, 2 when it halves
+// (src/operator/conv.rs:2184-2208, 2331-2338)
+struct ProjStackResConv2dOperatorConfig {
+  Dims3 in_dims, out_dims;
+  BNormMovingAverage bnorm_mov_avg;
+  double bnorm_epsilon;
+  ActivationFunction act_func;
+  ParamsInit init_weights;
+  Dims3 get_out_dims() const { return out_dims; }
+  size_t params_len() const {
+    return 3 * 3 * in_dims.c * out_dims.c + 3 * 3 * out_dims.c * out_dims.c + in_dims.c * out_dims.c + 12 * out_dims.c;
+  }
+};
+
 struct CategoricalLossConfig {
   size_t num_categories;
 };
 
 struct OperatorConfig {
-  enum Kind { Data3d, Affine, Conv2d, Pool2d, SoftmaxKLLoss, Dropout, LocalResNorm } kind;
+  enum Kind { Data3d, Affine, Conv2d, Pool2d, SoftmaxKLLoss, Dropout, LocalResNorm, BNormConv2d, StackResConv2d,
+              ProjStackResConv2d } kind;
+  BNormConv2dOperatorConfig bnorm_conv2d;
+  StackResConv2dOperatorConfig stack_res_conv2d;
+  ProjStackResConv2dOperatorConfig proj_stack_res_conv2d;
   Data3dOperatorConfig data3d;
   AffineOperatorConfig affine;
   Conv2dOperatorConfig conv2d;
@@ -239,6 +292,11 @@ class Operator {
   virtual size_t decode_state(const uint8_t* /*blob*/, size_t /*len*/) { return 0; }
   // Device views for inspection: 0 out_act, 1 out_delta, 2 weights, 3 bias, 4 grad_weights,
   // 5 grad_bias, 6 acc_grad_weights, 7 acc_grad_bias.  Returns false if the operator has no such buffer.
+  // The batch-normalised operators number their conv + batch-norm units u = 0, 1, 2 and answer 100*u + id with
+  // id = 2 weights, 4 grad_weights, 6 acc_grad_weights, 8 bn_scale, 9 bn_bias, 10 bn_scale_grad, 11 bn_bias_grad,
+  // 12 bn_running_mean, 13 bn_running_ivar, 14 bn_cached_mean, 15 bn_cached_ivar, 16 acc_bn_scale_grad,
+  // 17 acc_bn_bias_grad, 18 the unit's conv output (before the batch norm), 19 the gradient w.r.t. it; 30 / 31 are
+  // the activation between the two stacked units and its gradient.
   virtual bool buffer(int which, float** ptr, size_t* len) {
     (void)which; (void)ptr; (void)len;
     return false;
@@ -294,6 +352,9 @@ class SequentialOperatorConfig {
   SequentialOperatorConfig& pool2d(const Pool2dOperatorConfig& cfg);
   SequentialOperatorConfig& dropout(const DropoutOperatorConfig& cfg);              // src/operator/worker.rs:219-222
   SequentialOperatorConfig& local_res_norm(const LocalResNormOperatorConfig& cfg);
+  SequentialOperatorConfig& bnorm_conv2d(const BNormConv2dOperatorConfig& cfg);                    // worker.rs:189-192
+  SequentialOperatorConfig& stack_res_conv2d(const StackResConv2dOperatorConfig& cfg);            // worker.rs:194-197
+  SequentialOperatorConfig& proj_stack_res_conv2d(const ProjStackResConv2dOperatorConfig& cfg);   // worker.rs:199-202
   SequentialOperatorConfig& softmax_kl_loss(const CategoricalLossConfig& cfg);
 };
 

@@ -16,7 +16,29 @@ POOL = {"Max": 0, "Average": 1}
 MOMENTUM = {"Zero": 0, "Update": 1, "UpdateNesterov": 2, "Gradient": 3, "GradientNesterov": 4}
 STEP = {"Constant": 0, "Anneal1": 1, "Anneal2": 2, "Anneal4": 3, "Decay": 4, "Inverse": 5}
 BUF = {"out_act": 0, "out_delta": 1, "weights": 2, "bias": 3, "grad_weights": 4, "grad_bias": 5,
-       "acc_grad_weights": 6, "acc_grad_bias": 7}
+       "acc_grad_weights": 6, "acc_grad_bias": 7,
+       # batch-normalised operators; "u<k>.<name>" addresses conv + batch-norm unit k (100*k + id)
+       "bn_scale": 8, "bn_bias": 9, "bn_scale_grad": 10, "bn_bias_grad": 11, "bn_running_mean": 12, "bn_running_ivar": 13,
+       "bn_cached_mean": 14, "bn_cached_ivar": 15, "acc_bn_scale_grad": 16, "acc_bn_bias_grad": 17, "pre_act": 18,
+       "pre_delta": 19, "mid_act": 30, "mid_delta": 31}
+BNORM_AVG = {"Cumulative": 0, "Exponential": 1}
+
+
+def buf_id(which):
+    """'weights' -> 2; 'u1.bn_scale' -> 108; integers pass through."""
+    if isinstance(which, int):
+        return which
+    if which[0] == "u" and "." in which:
+        unit, name = which.split(".", 1)
+        return 100 * int(unit[1:]) + BUF[name]
+    return BUF[which]
+
+
+def _avg_args(mov_avg):
+    """'Cumulative' | ('Exponential', ema_factor) -> (kind, ema_factor)"""
+    if isinstance(mov_avg, str):
+        return BNORM_AVG[mov_avg], 0.0
+    return BNORM_AVG[mov_avg[0]], float(mov_avg[1])
 
 _vp, _i32, _i64, _f, _int, _u64 = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_int, C.c_uint64
 _P = C.POINTER
@@ -27,6 +49,10 @@ PROTOTYPES = {
     "rho_config_free": (_int, [_vp]),
     "rho_config_data3d": (_int, [_vp, _i32, _i32, _i32, _int]),
     "rho_config_conv2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _int, _int, _f]),
+    "rho_config_bnorm_conv2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _int, C.c_double, C.c_double, _int, _int, _f]),
+    "rho_config_stack_res_conv2d": (_int, [_vp, _i32, _i32, _i32, _int, C.c_double, C.c_double, _int, _int, _f]),
+    "rho_config_proj_stack_res_conv2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _int, C.c_double, C.c_double, _int, _int,
+                                                _f]),
     "rho_config_affine": (_int, [_vp, _i32, _i32, _int, _int, _f]),
     "rho_config_pool2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _int, _int]),
     "rho_config_softmax_kl_loss": (_int, [_vp, _i32]),
@@ -174,6 +200,30 @@ class SequentialOperatorConfig:
         k, v = _init_args(init_weights)
         _chk(lib().rho_config_conv2d(self._h, in_dims[0], in_dims[1], in_dims[2], conv_size, conv_stride, conv_pad,
                                      out_channels, ACT[act_func], k, v))
+        return self
+
+    def bnorm_conv2d(self, in_dims, conv_size, conv_stride, conv_pad, out_channels, bnorm_mov_avg=("Exponential", 0.1),
+                     bnorm_epsilon=1e-5, act_func="Rect", init_weights="KaimingFwd"):
+        k, v = _init_args(init_weights)
+        a, f = _avg_args(bnorm_mov_avg)
+        _chk(lib().rho_config_bnorm_conv2d(self._h, in_dims[0], in_dims[1], in_dims[2], conv_size, conv_stride, conv_pad,
+                                           out_channels, a, f, bnorm_epsilon, ACT[act_func], k, v))
+        return self
+
+    def stack_res_conv2d(self, in_dims, bnorm_mov_avg=("Exponential", 0.1), bnorm_epsilon=1e-5, act_func="Rect",
+                         init_weights="KaimingFwd"):
+        k, v = _init_args(init_weights)
+        a, f = _avg_args(bnorm_mov_avg)
+        _chk(lib().rho_config_stack_res_conv2d(self._h, in_dims[0], in_dims[1], in_dims[2], a, f, bnorm_epsilon, ACT[act_func],
+                                               k, v))
+        return self
+
+    def proj_stack_res_conv2d(self, in_dims, out_dims, bnorm_mov_avg=("Exponential", 0.1), bnorm_epsilon=1e-5, act_func="Rect",
+                              init_weights="KaimingFwd"):
+        k, v = _init_args(init_weights)
+        a, f = _avg_args(bnorm_mov_avg)
+        _chk(lib().rho_config_proj_stack_res_conv2d(self._h, in_dims[0], in_dims[1], in_dims[2], out_dims[0], out_dims[1],
+                                                    out_dims[2], a, f, bnorm_epsilon, ACT[act_func], k, v))
         return self
 
     def affine(self, in_channels, out_channels, act_func="Rect", init_weights=("Normal", 0.01)):
@@ -415,23 +465,23 @@ class SequentialOperatorWorker:
     # inspection
     def buffer_len(self, idx, which):
         p, n = _vp(), _i64()
-        _chk(lib().rho_worker_buffer(self._h, idx, BUF[which], C.byref(p), C.byref(n)))
+        _chk(lib().rho_worker_buffer(self._h, idx, buf_id(which), C.byref(p), C.byref(n)))
         return n.value
 
     def device_ptr(self, idx, which):
         p, n = _vp(), _i64()
-        _chk(lib().rho_worker_buffer(self._h, idx, BUF[which], C.byref(p), C.byref(n)))
+        _chk(lib().rho_worker_buffer(self._h, idx, buf_id(which), C.byref(p), C.byref(n)))
         return p.value, n.value
 
     def read(self, idx, which, count=None):
         n = self.buffer_len(idx, which) if count is None else count
         out = np.empty((n,), np.float32)
-        _chk(lib().rho_worker_read_buffer(self._h, idx, BUF[which], out.ctypes.data, n))
+        _chk(lib().rho_worker_read_buffer(self._h, idx, buf_id(which), out.ctypes.data, n))
         return out
 
     def write(self, idx, which, values):
         values = np.ascontiguousarray(values, np.float32).ravel()
-        _chk(lib().rho_worker_write_buffer(self._h, idx, BUF[which], values.ctypes.data, values.size))
+        _chk(lib().rho_worker_write_buffer(self._h, idx, buf_id(which), values.ctypes.data, values.size))
 
 
 class DataSource:

@@ -296,6 +296,55 @@ def lrn_bwd(x, y, d, dy, size, scale, power, min_div):
     return dx
 
 
+def _bnorm_ws(x):
+    N, Cc, H, W = x.shape
+    nbytes = lib().rh_bnorm_workspace_bytes(N, Cc, H * W)
+    return torch.empty(nbytes, dtype=torch.uint8, device=x.device), nbytes
+
+
+def bnorm_fwd_train(x, scale, bias, running_mean, running_ivar, ema_factor, epsilon, alpha=1.0, beta=0.0, y=None, relu=False):
+    """Spatial batch-norm, training mode: returns (y, cached_mean, cached_ivar); the running pair is updated in place."""
+    N, Cc, H, W = x.shape
+    if y is None:
+        assert beta == 0.0
+        y = torch.empty_like(x)
+    cm, ci = torch.empty_like(scale), torch.empty_like(scale)
+    ws, nbytes = _bnorm_ws(x)
+    check(lib().rh_bnorm_fwd_train(N, Cc, H * W, alpha, _p(x), beta, _p(y), ema_factor, epsilon, _p(scale), _p(bias),
+                                   _p(running_mean), _p(running_ivar), _p(cm), _p(ci), _p(ws), nbytes,
+                                   _lib.RH_FUSE_RELU if relu else 0, _stream()), "rh_bnorm_fwd_train")
+    return y, cm, ci
+
+
+def bnorm_fwd_infer(x, scale, bias, running_mean, running_ivar, epsilon, alpha=1.0, beta=0.0, y=None, relu=False):
+    N, Cc, H, W = x.shape
+    if y is None:
+        assert beta == 0.0
+        y = torch.empty_like(x)
+    ws, nbytes = _bnorm_ws(x)
+    check(lib().rh_bnorm_fwd_infer(N, Cc, H * W, alpha, _p(x), beta, _p(y), epsilon, _p(scale), _p(bias), _p(running_mean),
+                                   _p(running_ivar), _p(ws), nbytes, _lib.RH_FUSE_RELU if relu else 0, _stream()),
+          "rh_bnorm_fwd_infer")
+    return y
+
+
+def bnorm_bwd(x, dy, scale, cached_mean, cached_ivar, epsilon, dscale=None, dbias=None, alpha_data=1.0, beta_data=0.0,
+              dx=None, alpha_param=1.0, beta_param=0.0):
+    """Returns (dx, dscale, dbias); with beta_param = 1 the parameter gradients accumulate as in the reference."""
+    N, Cc, H, W = x.shape
+    if dx is None:
+        assert beta_data == 0.0
+        dx = torch.empty_like(x)
+    if dscale is None:
+        assert beta_param == 0.0
+        dscale, dbias = torch.empty_like(scale), torch.empty_like(scale)
+    ws, nbytes = _bnorm_ws(x)
+    check(lib().rh_bnorm_bwd(N, Cc, H * W, alpha_data, beta_data, _p(x), _p(dy), _p(dx), alpha_param, beta_param, epsilon,
+                             _p(scale), _p(dscale), _p(dbias), _p(cached_mean), _p(cached_ivar), _p(ws), nbytes, _stream()),
+          "rh_bnorm_bwd")
+    return dx, dscale, dbias
+
+
 def memset_f32(t, value):
     check(lib().rh_memset_f32(_p(t), value, t.numel(), _stream()), "rh_memset_f32")
     return t

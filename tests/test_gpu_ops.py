@@ -318,6 +318,56 @@ def test_lrn(dev, case):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("shape", [(4, 3, 5, 6), (6, 5, 1, 1), (3, 2, 7, 7), (1, 4, 3, 3), (8, 64, 56, 56), (16, 512, 7, 7),
+                                   (2, 3, 112, 112), (5, 7, 13, 9)])
+def test_bnorm(dev, shape):
+    """Spatial batch normalisation: training forward (batch statistics, moving averages, blend, fused ReLU),
+    inference forward and backward against the fp64 restatement; one channel carries a mean 25x its deviation.
+    (Two values per channel are left out: there dx cancels to ~epsilon analytically and has no stable digits.)"""
+    say("bnorm", shape)
+    C = shape[1]
+    x = synth.normal(17, 1, shape) * np.float32(2.0) + np.linspace(-1, 50, C, dtype=np.float32)[None, :, None, None]
+    dy = synth.normal(17, 2, shape)
+    y0 = synth.normal(17, 3, shape)
+    scale, bias = synth.normal(17, 4, (C,)) + np.float32(1.0), synth.normal(17, 5, (C,))
+    rm, ri = synth.normal(17, 6, (C,)), np.abs(synth.normal(17, 7, (C,))) + np.float32(0.5)
+    eps, ema = 1e-5, 0.1
+    y_ref, cm_ref, ci_ref, rm_ref, ri_ref = O.bnorm_fwd_train(x, scale, bias, rm, ri, ema, eps)
+    xd, sd, bd = T(x, dev), T(scale, dev), T(bias, dev)
+    rmd, rid = T(rm, dev), T(ri, dev)
+    y, cm, ci = ops.bnorm_fwd_train(xd, sd, bd, rmd, rid, ema, eps)
+    assert_close(N(cm), cm_ref, "batch mean")
+    assert_close(N(ci), ci_ref, "batch inverse deviation")
+    assert_close(N(rmd), rm_ref, "running mean")
+    assert_close(N(rid), ri_ref, "running inverse deviation")
+    # normalised values of a channel with |mean| >> deviation lose |mean|/deviation ulps of x itself (fp32 inputs)
+    assert_close(N(y), y_ref, "bnorm fwd", atol=2e-5)
+    # blend into an existing tensor with the ReLU fused (the residual add of the stacked operators)
+    yb = T(y0, dev)
+    rm2, ri2 = T(rm, dev), T(ri, dev)
+    ops.bnorm_fwd_train(xd, sd, bd, rm2, ri2, ema, eps, alpha=1.0, beta=1.0, y=yb, relu=True)
+    want = O.bnorm_fwd_train(x, scale, bias, rm, ri, ema, eps, alpha=1.0, beta=1.0, y=y0)[0]
+    got = N(yb)
+    unsure = np.abs(want) < 1e-4 * max(1.0, float(np.sqrt((want ** 2).mean())))
+    assert np.array_equal((got > 0)[~unsure], (want > 0)[~unsure])
+    assert_close(got, np.maximum(want, 0), "bnorm fwd blend + relu", atol=2e-5)
+    assert np.array_equal(N(rm2), N(rmd)) and np.array_equal(N(ri2), N(rid)), "statistics do not depend on the blend"
+    yi = ops.bnorm_fwd_infer(xd, sd, bd, T(rm, dev), T(ri, dev), eps)
+    assert_close(N(yi), O.bnorm_fwd_infer(x, scale, bias, rm, ri), "bnorm inference", atol=2e-5)
+    # backward on the statistics the device cached; parameter gradients accumulate with beta_param = 1
+    dx_ref, ds_ref, db_ref = O.bnorm_bwd(x, dy, scale, N(cm), N(ci))
+    ds0, db0 = synth.normal(17, 8, (C,)), synth.normal(17, 9, (C,))
+    dsd, dbd = T(ds0, dev), T(db0, dev)
+    dx, _, _ = ops.bnorm_bwd(xd, T(dy, dev), sd, cm, ci, eps, dscale=dsd, dbias=dbd, beta_param=1.0)
+    assert_close(N(dx), dx_ref, "bnorm bwd dx", atol=2e-5)
+    assert_close(N(dsd), ds_ref.astype(np.float64) + ds0, "bnorm dscale", atol=2e-5)
+    assert_close(N(dbd), db_ref.astype(np.float64) + db0, "bnorm dbias", atol=2e-5)
+    dx2 = T(y0, dev)
+    ops.bnorm_bwd(xd, T(dy, dev), sd, cm, ci, eps, alpha_data=1.0, beta_data=1.0, dx=dx2)
+    assert_close(N(dx2), dx_ref.astype(np.float64) + y0, "bnorm bwd dx blended", atol=2e-5)
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("case", [(2, 3, 9, 3, 2, 0), (2, 3, 9, 3, 2, 1), (3, 4, 8, 2, 2, 0), (2, 5, 27, 3, 2, 0), (2, 2, 13, 3, 3, 1)])
 @pytest.mark.parametrize("rounding", [_lib.RH_ROUND_FLOOR, _lib.RH_ROUND_CEIL])
 def test_pool2d_bwd_with_folded_relu_mask(dev, case, rounding):

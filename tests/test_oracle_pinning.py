@@ -382,6 +382,116 @@ def test_lrn_matches_torch_local_response_norm():
         assert (d >= min_div).all()
 
 
+def test_bnorm_matches_torch_batch_norm():
+    """bnorm_fwd_train / bnorm_fwd_infer / bnorm_bwd against torch.nn.functional.batch_norm (fp64) and its autograd,
+    on a channel with a large mean as well.  torch keeps a running *variance* (unbiased); the reference's buffer is
+    named running_ivar, so only the running mean and the cached batch statistics are compared, and the moving
+    inverse standard deviation is checked against its own definition (parity unpinned for that buffer)."""
+    rng = np.random.default_rng(12)
+    for shape in ((4, 3, 5, 6), (2, 5, 1, 1), (3, 2, 7, 7), (1, 4, 3, 3)):
+        C = shape[1]
+        x = rng.standard_normal(shape).astype(np.float32) * 2 + np.linspace(-1, 50, C, dtype=np.float32)[None, :, None, None]
+        dy = rng.standard_normal(shape).astype(np.float32)
+        scale, bias = (rng.standard_normal(C).astype(np.float32) + 1, rng.standard_normal(C).astype(np.float32))
+        rm, ri = rng.standard_normal(C).astype(np.float32), rng.random(C).astype(np.float32) + 0.5
+        eps, ema = 1e-5, 0.1
+        xt = torch.from_numpy(x).double().requires_grad_(True)
+        st, bt = torch.from_numpy(scale).double().requires_grad_(True), torch.from_numpy(bias).double().requires_grad_(True)
+        trm, trv = torch.from_numpy(rm).double().clone(), torch.ones(C, dtype=torch.float64)
+        yt = F.batch_norm(xt, trm, trv, st, bt, training=True, momentum=ema, eps=eps)
+        gx, gs, gb = torch.autograd.grad(yt, (xt, st, bt), torch.from_numpy(dy).double())
+        y, cm, ci, nrm, nri = O.bnorm_fwd_train(x, scale, bias, rm, ri, ema, eps)
+        np.testing.assert_allclose(y, yt.detach().numpy(), rtol=1e-6, atol=1e-6)
+        np.testing.assert_allclose(nrm, trm.numpy(), rtol=1e-6, atol=1e-6)
+        x64 = x.astype(np.float64)
+        np.testing.assert_allclose(cm, x64.mean(axis=(0, 2, 3)), rtol=1e-6)
+        np.testing.assert_allclose(ci, 1.0 / np.sqrt(x64.var(axis=(0, 2, 3)) + eps), rtol=1e-6)
+        np.testing.assert_allclose(nri, 0.9 * ri + 0.1 * ci, rtol=1e-6)
+        dx, ds, db = O.bnorm_bwd(x, dy, scale, cm, ci)
+        np.testing.assert_allclose(dx, gx.numpy(), rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(ds, gs.numpy(), rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(db, gb.numpy(), rtol=1e-5, atol=1e-5)
+        # blend and inference: y = alpha*bn(x) + beta*y0; inference with torch's (mean, var) <-> (mean, 1/sqrt(var+eps))
+        y0 = rng.standard_normal(shape).astype(np.float32)
+        yb = O.bnorm_fwd_train(x, scale, bias, rm, ri, ema, eps, alpha=0.5, beta=2.0, y=y0)[0]
+        np.testing.assert_allclose(yb, 0.5 * yt.detach().numpy() + 2.0 * y0, rtol=1e-6, atol=1e-5)
+        var = rng.random(C) + 0.3
+        yi = F.batch_norm(torch.from_numpy(x).double(), torch.from_numpy(rm).double(), torch.from_numpy(var),
+                          torch.from_numpy(scale).double(), torch.from_numpy(bias).double(), training=False, eps=eps)
+        got = O.bnorm_fwd_infer(x, scale, bias, rm, (1.0 / np.sqrt(var + eps)).astype(np.float32))
+        np.testing.assert_allclose(got, yi.numpy(), rtol=1e-5, atol=1e-5)
+    assert O.bnorm_mov_avg_at_iter("Cumulative", 0.1, 0) == 1.0 and O.bnorm_mov_avg_at_iter("Cumulative", 0.1, 3) == 0.25
+    assert O.bnorm_mov_avg_at_iter("Exponential", 0.1, 0) == 1.0 and O.bnorm_mov_avg_at_iter("Exponential", 0.1, 7) == 0.1
+
+
+def _torch_unit(x, u, eps):
+    """conv (no bias) + training-mode batch norm of one unit, on torch fp64 leaves."""
+    z = F.conv2d(x, u["w"], None, u["stride"], u["pad"])
+    return F.batch_norm(z, None, None, u["scale"], u["bias"], training=True, eps=eps)
+
+
+@pytest.mark.parametrize("kind", ["bnorm_conv2d", "stack_res_conv2d", "proj_stack_res_conv2d_s2", "proj_stack_res_conv2d_s1"])
+def test_bnorm_operators_match_torch_autograd(kind):
+    """The wiring of the batch-normalised operators (residual add, where the ReLU masks act, which deltas add up)
+    against torch autograd of the same composite in fp64: out_act, in_delta and every parameter gradient."""
+    from oracle import graph as OG
+    rng = np.random.default_rng(13)
+    batch, eps = 3, 1e-5
+    if kind == "bnorm_conv2d":
+        in_dims = (9, 8, 3)
+        op = OG.BNormConv2dOperator(batch, in_dims, 3, 2, 1, 5, "Rect", epsilon=eps)
+    elif kind == "stack_res_conv2d":
+        in_dims = (6, 5, 4)
+        op = OG.StackResConv2dOperator(batch, in_dims, "Rect", epsilon=eps)
+    elif kind == "proj_stack_res_conv2d_s2":
+        in_dims = (8, 6, 3)
+        op = OG.ProjStackResConv2dOperator(batch, in_dims, (4, 3, 5), "Rect", epsilon=eps)
+    else:
+        in_dims = (5, 4, 3)
+        op = OG.ProjStackResConv2dOperator(batch, in_dims, (5, 4, 6), "Rect", epsilon=eps)
+    tu = []
+    for u in op.units:
+        u.weights[...] = rng.standard_normal(u.weights.shape) * 0.4
+        u.scale[...] = 1 + 0.3 * rng.standard_normal(u.scale.shape)
+        u.bias[...] = 0.3 * rng.standard_normal(u.bias.shape)
+        tu.append({"w": torch.from_numpy(u.weights).double().requires_grad_(True),
+                   "scale": torch.from_numpy(u.scale).double().requires_grad_(True),
+                   "bias": torch.from_numpy(u.bias).double().requires_grad_(True), "stride": u.stride, "pad": u.pad})
+    x = rng.standard_normal((batch, in_dims[2], in_dims[1], in_dims[0])).astype(np.float32)
+    xt = torch.from_numpy(x).double().requires_grad_(True)
+    if kind == "bnorm_conv2d":
+        yt = torch.relu(_torch_unit(xt, tu[0], eps))
+    elif kind == "stack_res_conv2d":
+        yt = torch.relu(xt + _torch_unit(torch.relu(_torch_unit(xt, tu[0], eps)), tu[1], eps))
+    else:
+        yt = torch.relu(_torch_unit(torch.relu(_torch_unit(xt, tu[0], eps)), tu[1], eps) + _torch_unit(xt, tu[2], eps))
+    y = op.forward(x, True, 0)
+    np.testing.assert_allclose(y, yt.detach().numpy(), rtol=1e-5, atol=1e-5)
+    assert tuple(yt.shape[1:]) == (op.out_dims[2], op.out_dims[1], op.out_dims[0])
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    leaves = [xt] + [t[k] for t in tu for k in ("w", "scale", "bias")]
+    grads = torch.autograd.grad(yt, leaves, torch.from_numpy(dy).double())
+    op.out_delta = dy.copy()
+    dx = op.backward(True)
+    np.testing.assert_allclose(dx, grads[0].numpy(), rtol=1e-4, atol=2e-5)
+    for k, u in enumerate(op.units):
+        gw, gs, gb = grads[1 + 3 * k: 4 + 3 * k]
+        np.testing.assert_allclose(u.grad_weights, gw.numpy(), rtol=1e-4, atol=2e-5)
+        np.testing.assert_allclose(u.scale_grad, gs.numpy(), rtol=1e-4, atol=2e-5)
+        np.testing.assert_allclose(u.bias_grad, gb.numpy(), rtol=1e-4, atol=2e-5)
+    # a second backward accumulates the parameter gradients (beta = 1) until reset()
+    g1 = op.units[0].grad_weights.copy()
+    op.out_delta = dy.copy()
+    op.backward(True)
+    np.testing.assert_allclose(op.units[0].grad_weights, 2 * g1, rtol=1e-5, atol=1e-6)
+    op.p.reset()
+    assert not op.units[0].grad_weights.any() and not op.units[0].scale_grad.any()
+    # weight decay reaches the filters only
+    op.p.regularize(0.5)
+    np.testing.assert_allclose(op.units[0].grad_weights, 0.5 * op.units[0].weights, rtol=1e-6)
+    assert not op.units[0].scale_grad.any() and not op.units[0].bias_grad.any()
+
+
 def test_preproc_and_dropout_restatements():
     rng = np.random.default_rng(11)
     x = rng.standard_normal((3, 3, 9, 8)).astype(np.float32)
