@@ -29,7 +29,7 @@ MEASURED_TRAFFIC_BYTES = {
                 "conv_bwd_data_128x128": 1024 * (2.0 * 63944 + 70941)},
 }
 
-BATCH = {"alexnet": 256, "lenet": 64, "cifar10": 128, "nin": 128}
+BATCH = {"alexnet": 256, "lenet": 64, "cifar10": 128, "nin": 128, "resnet18": 64}
 NUM_CLASSES_SEED = 0x5EED0000
 
 
@@ -98,7 +98,10 @@ def cpu_baseline(net, sample_images):
     ref = OG.SequentialOperatorWorker(layers, ncat, sample_images, fast=True)
     rng = np.random.default_rng(0)
     for op in ref.hidden:
-        if op.p is not None:
+        if hasattr(op, "units"):
+            for u in op.units:
+                u.weights[...] = rng.standard_normal(u.weights.shape, dtype=np.float32) * np.float32(np.sqrt(2.0 / u.weights[0].size))
+        elif op.p is not None:
             op.p.weights[...] = rng.standard_normal(op.p.weights.shape, dtype=np.float32) * np.float32(0.01)
     x = rng.standard_normal((sample_images, dims[2], dims[1], dims[0]), dtype=np.float32)
     labels = rng.integers(0, ncat, (sample_images,)).astype(np.int32)
@@ -113,7 +116,7 @@ def cpu_baseline(net, sample_images):
     sgd.step(ref)
     dt = time.perf_counter() - t0
     return {"value": sample_images / dt, "unit": "images/sec", "cores": oracle.num_threads(), "kind": "port",
-            "sample": "one fwd+bwd+SGD step of the same AlexNet-shaped graph on %d images (%.1f s)" % (sample_images, dt)}
+            "sample": "one fwd+bwd+SGD step of the same operator graph on %d images (%.1f s)" % (sample_images, dt)}
 
 
 def main():
@@ -222,7 +225,8 @@ def main():
     gemm_ms = sum(k["ms_per_step"] for k in mfma)
     gemm_flops = configs.train_flops(net, batch)
     result = {
-        "metric": "train images/sec (fwd+bwd+SGD) AlexNet b256 fp32; conv/FC % MFMA peak",
+        "metric": "train images/sec (fwd+bwd+SGD) AlexNet b256 fp32; conv/FC % MFMA peak" if args.workload == "alexnet" else
+                  "train images/sec (fwd+bwd+SGD) %s b%d fp32" % (args.workload, batch),
         "value": batch * args.steps / dt,
         "unit": "images/sec",
         "n_gpus": 1,

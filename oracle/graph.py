@@ -237,10 +237,10 @@ class _BNormUnit:
     (src/operator/conv.rs:133-160 buffers; :640-911 regularize the filter only, accumulate / update / save / restore /
     reset the filter, scale and bias; the moving statistics travel with save / restore)."""
 
-    def __init__(self, batch, in_dims, size, stride, pad, out_channels):
+    def __init__(self, batch, in_dims, size, stride, pad, out_channels, fast=False):
         w, h, c = in_dims
         self.x_shape = (batch, c, h, w)
-        self.stride, self.pad = stride, pad
+        self.stride, self.pad, self.fast = stride, pad, fast
         f = np.float32
         self.weights = np.zeros((out_channels, c, size, size), f)
         self.grad_weights, self.acc_grad_weights, self.save_weights = (np.zeros_like(self.weights) for _ in range(3))
@@ -261,6 +261,8 @@ class _BNormUnit:
         self.in_act = in_act
         if self.bf16_forward:
             O.conv2d_fwd(O.round_bf16(in_act), O.round_bf16(self.weights), self.stride, self.pad, y=self.pre_act)
+        elif self.fast:
+            self.pre_act = O.fast_conv2d_fwd(in_act, self.weights, self.stride, self.pad)
         else:
             O.conv2d_fwd(in_act, self.weights, self.stride, self.pad, y=self.pre_act)
         if training:
@@ -275,9 +277,16 @@ class _BNormUnit:
         self.pre_delta, ds, db = O.bnorm_bwd(self.pre_act, out_delta, self.scale, self.cached_mean, self.cached_ivar)
         self.scale_grad = (self.scale_grad + ds).astype(np.float32)
         self.bias_grad = (self.bias_grad + db).astype(np.float32)
-        O.conv2d_bwd_filter(self.in_act, self.pre_delta, self.weights.shape, self.stride, self.pad, 1.0, 1.0, self.grad_weights)
+        if self.fast:
+            O.fast_conv2d_bwd_filter(self.in_act, self.pre_delta, self.grad_weights, self.stride, self.pad)
+        else:
+            O.conv2d_bwd_filter(self.in_act, self.pre_delta, self.weights.shape, self.stride, self.pad, 1.0, 1.0,
+                                self.grad_weights)
 
     def backward_data(self, beta=0.0, dx=None):
+        if self.fast:
+            d = O.fast_conv2d_bwd_data(self.weights, self.pre_delta, self.x_shape, self.stride, self.pad)
+            return d if beta == 0.0 else (d + np.float32(beta) * dx).astype(np.float32)
         return O.conv2d_bwd_data(self.weights, self.pre_delta, self.x_shape, self.stride, self.pad, 1.0, beta, dx)
 
     def _triples(self):
@@ -345,8 +354,8 @@ class BNormConv2dOperator:
     wants_phase = True
 
     def __init__(self, batch, in_dims, conv_size, conv_stride, conv_pad, out_channels, act_func, mov_avg=("Exponential", 0.1),
-                 epsilon=1e-5):
-        self.units = [_BNormUnit(batch, in_dims, conv_size, conv_stride, conv_pad, out_channels)]
+                 epsilon=1e-5, fast=False):
+        self.units = [_BNormUnit(batch, in_dims, conv_size, conv_stride, conv_pad, out_channels, fast)]
         self.p = _UnitsParams(self.units)
         self.act, self.mov_avg, self.epsilon = act_func, mov_avg, epsilon
         self.out_dims = self.units[0].out_dims
@@ -371,9 +380,9 @@ class StackResConv2dOperator:
     kind = "StackResConv2dOperator"
     wants_phase = True
 
-    def __init__(self, batch, in_dims, act_func, mov_avg=("Exponential", 0.1), epsilon=1e-5):
+    def __init__(self, batch, in_dims, act_func, mov_avg=("Exponential", 0.1), epsilon=1e-5, fast=False):
         c = in_dims[2]
-        self.units = [_BNormUnit(batch, in_dims, 3, 1, 1, c), _BNormUnit(batch, in_dims, 3, 1, 1, c)]
+        self.units = [_BNormUnit(batch, in_dims, 3, 1, 1, c, fast), _BNormUnit(batch, in_dims, 3, 1, 1, c, fast)]
         self.p = _UnitsParams(self.units)
         self.act, self.mov_avg, self.epsilon = act_func, mov_avg, epsilon
         self.out_dims = in_dims
@@ -410,15 +419,15 @@ class ProjStackResConv2dOperator:
     kind = "ProjStackResConv2dOperator"
     wants_phase = True
 
-    def __init__(self, batch, in_dims, out_dims, act_func, mov_avg=("Exponential", 0.1), epsilon=1e-5):
+    def __init__(self, batch, in_dims, out_dims, act_func, mov_avg=("Exponential", 0.1), epsilon=1e-5, fast=False):
         if in_dims[:2] == out_dims[:2]:
             s = 1
         else:
             assert in_dims[0] == 2 * out_dims[0] and in_dims[1] == 2 * out_dims[1]
             s = 2
         oc = out_dims[2]
-        self.units = [_BNormUnit(batch, in_dims, 3, s, 1, oc), _BNormUnit(batch, out_dims, 3, 1, 1, oc),
-                      _BNormUnit(batch, in_dims, 1, s, 0, oc)]
+        self.units = [_BNormUnit(batch, in_dims, 3, s, 1, oc, fast), _BNormUnit(batch, out_dims, 3, 1, 1, oc, fast),
+                      _BNormUnit(batch, in_dims, 1, s, 0, oc, fast)]
         self.p = _UnitsParams(self.units)
         self.act, self.mov_avg, self.epsilon = act_func, mov_avg, epsilon
         self.out_dims = out_dims
@@ -461,7 +470,7 @@ class SequentialOperatorWorker:
         self.hidden = []
         if isinstance(bnorm_mov_avg, str):
             bnorm_mov_avg = (bnorm_mov_avg, 0.0)
-        bnorm = {"mov_avg": bnorm_mov_avg, "epsilon": bnorm_epsilon}
+        bnorm = {"mov_avg": bnorm_mov_avg, "epsilon": bnorm_epsilon, "fast": fast}
         for l in layers:
             if l[0] == "conv2d":
                 self.hidden.append(Conv2dOperator(batch, *l[1:], fast=fast))

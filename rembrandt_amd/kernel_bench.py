@@ -24,6 +24,16 @@ CONV_LAYERS = {
     "alexnet_conv4": (256, 384, 13, 13, 384, 3, 1, 1),
     "alexnet_conv5": (256, 384, 13, 13, 256, 3, 1, 1),
     "stride2_3x3": (64, 64, 56, 56, 128, 3, 2, 1),   # a strided layer in mid-network (its backward-data is needed)
+    # the distinct convolutions of the ResNet-18 template at batch 64
+    "resnet_conv1": (64, 3, 224, 224, 64, 7, 2, 3),
+    "resnet_56_64": (64, 64, 56, 56, 64, 3, 1, 1),
+    "resnet_28_128": (64, 128, 28, 28, 128, 3, 1, 1),
+    "resnet_14_256": (64, 256, 14, 14, 256, 3, 1, 1),
+    "resnet_7_512": (64, 512, 7, 7, 512, 3, 1, 1),
+    "resnet_down_256": (64, 128, 28, 28, 256, 3, 2, 1),
+    "resnet_down_512": (64, 256, 14, 14, 512, 3, 2, 1),
+    "resnet_proj_128": (64, 64, 56, 56, 128, 1, 2, 0),
+    "resnet_proj_512": (64, 256, 14, 14, 512, 1, 2, 0),
 }
 FC_LAYERS = {"alexnet_fc6": (256, 9216, 4096), "alexnet_fc7": (256, 4096, 4096), "alexnet_fc8": (256, 4096, 1000)}
 
@@ -31,7 +41,7 @@ FC_LAYERS = {"alexnet_fc6": (256, 9216, 4096), "alexnet_fc7": (256, 4096, 4096),
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("what", nargs="*", default=["conv", "fc", "mem"], help="conv | fc | mem")
-    ap.add_argument("--layer", default=None, help="one of %s" % ", ".join(list(CONV_LAYERS) + list(FC_LAYERS)))
+    ap.add_argument("--layer", default=None, help="a prefix of: %s" % ", ".join(list(CONV_LAYERS) + list(FC_LAYERS)))
     ap.add_argument("--passes", default="fwd,bwd_filter,bwd_data,fwd_bf16")
     ap.add_argument("--iters", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
@@ -66,7 +76,7 @@ def main(argv=None):
 
     if "conv" in args.what:
         for name, (N, C, H, W, K, R, st, pad) in CONV_LAYERS.items():
-            if args.layer and args.layer != name:
+            if args.layer and not name.startswith(args.layer):
                 continue
             x = torch.randn(N, C, H, W, device=dev)
             if args.relu_data:
@@ -89,7 +99,7 @@ def main(argv=None):
             del x, w, y, dy
     if "fc" in args.what:
         for name, (B, i, o) in FC_LAYERS.items():
-            if args.layer and args.layer != name:
+            if args.layer and not name.startswith(args.layer):
                 continue
             X, Wt, dY = torch.randn(B, i, device=dev), torch.randn(o, i, device=dev), torch.randn(B, o, device=dev)
             Y, dW, dX = torch.empty(B, o, device=dev), torch.zeros(o, i, device=dev), torch.empty(B, i, device=dev)
@@ -117,6 +127,21 @@ def main(argv=None):
         W_, g, v = torch.randn(P, device=dev), torch.randn(P, device=dev), torch.zeros(P, device=dev)
         report("sgd_momentum_step", "alexnet_params", timeit(lambda: ops.sgd_momentum_step(W_, g, v, 0.0, -0.01, 0.9, 1.0, True)),
                24.0 * P, "hbm")
+        for shp in ((256, 64, 56, 56), (256, 512, 7, 7)):
+            xb, dyb = torch.randn(*shp, device=dev), torch.randn(*shp, device=dev)
+            Cb, nb = shp[1], xb.numel()
+            sc, bi = torch.ones(Cb, device=dev), torch.zeros(Cb, device=dev)
+            rm, ri = torch.zeros(Cb, device=dev), torch.ones(Cb, device=dev)
+            yb = torch.empty_like(xb)
+            _, cm, ci = ops.bnorm_fwd_train(xb, sc, bi, rm, ri, 0.1, 1e-5, y=yb)
+            name = "bnorm_%dx%dx%dx%d" % shp
+            report("bnorm_fwd_train", name, timeit(lambda: ops.bnorm_fwd_train(xb, sc, bi, rm, ri, 0.1, 1e-5, y=yb, relu=True)),
+                   12.0 * nb, "hbm")
+            report("bnorm_fwd_infer", name, timeit(lambda: ops.bnorm_fwd_infer(xb, sc, bi, rm, ri, 1e-5, y=yb)), 8.0 * nb, "hbm")
+            dxb, ds, db = torch.empty_like(xb), torch.zeros(Cb, device=dev), torch.zeros(Cb, device=dev)
+            report("bnorm_bwd", name, timeit(lambda: ops.bnorm_bwd(xb, dyb, sc, cm, ci, 1e-5, dscale=ds, dbias=db, dx=dxb,
+                                                                   beta_param=1.0)), 20.0 * nb, "hbm")
+            del xb, dyb, yb, dxb
         logits = torch.randn(256, 1000, device=dev)
         report("softmax_fwd", "alexnet_logits", timeit(lambda: ops.softmax_fwd(logits)), 8.0 * logits.numel(), "hbm")
     return 0

@@ -26,6 +26,14 @@ pub struct rh_pool_geom {
   pub round: i32, // 0 floor (operator), 1 ceil (gen-1 layer)
 }
 
+#[repr(C)]
+#[derive(Clone, Copy, Debug)]
+pub struct rh_lrn_geom {
+  pub n: i32, pub c: i32, pub h: i32, pub w: i32,
+  pub size: i32,
+  pub scale: c_float, pub power: c_float, pub min_div: c_float,
+}
+
 pub const RH_CONV_FWD: c_int = 0;
 pub const RH_CONV_BWD_FILTER: c_int = 1;
 pub const RH_CONV_BWD_DATA: c_int = 2;
@@ -102,6 +110,50 @@ extern "C" {
   pub fn rh_sgd_momentum_step(n: i64, w: *mut f32, g: *mut f32, v: *mut f32, l2: c_float, scale: c_float,
                               mu: c_float, apply: c_float, zero_grad: c_int, stream: rh_stream_t) -> c_int;
   pub fn rh_descend(n: i64, w: *mut f32, g: *mut f32, s: c_float, l2: c_float, stream: rh_stream_t) -> c_int;
+
+  // Second stream of the context (no counterpart in the reference, which issues everything on ctx.stream).
+  pub fn rh_ctx_aux_stream(ctx: *mut rh_ctx) -> rh_stream_t;
+  pub fn rh_ctx_fork(ctx: *mut rh_ctx) -> c_int;
+  pub fn rh_ctx_join(ctx: *mut rh_ctx) -> c_int;
+
+  // Max-pool backward that also applies the ReLU backward mask of the operator below (one pass instead of two).
+  pub fn rh_pool2d_bwd_relu_supported(g: *const rh_pool_geom) -> c_int;
+  pub fn rh_pool2d_bwd_relu(g: *const rh_pool_geom, y: *const f32, dy: *const f32, dx: *mut f32,
+                            argmax: *const i32, stream: rh_stream_t) -> c_int;
+
+  // Data3dOperator preprocessing (src/operator/mod.rs:666-691, 716-725, 767-773) and dropout (mod.rs:2220-2246).
+  pub fn rh_crop_nchw(src: *const f32, dst: *mut f32, planes: i64, in_w: i32, in_h: i32, crop_w: i32, crop_h: i32,
+                      off_w: i32, off_h: i32, stream: rh_stream_t) -> c_int;
+  pub fn rembrandt_kernel_batch_blockmap256_flip(src: *const f32, width: i32, rows: i32, dst: *mut f32,
+                                                 stream: rh_stream_t);
+  pub fn rembrandt_kernel_batch_map_preproc_pca3_noise(src: *const f32, spatial: i32, batch: i32,
+                                                       alphas: *const f32, svals: *const f32, svecs: *const f32,
+                                                       dst: *mut f32, stream: rh_stream_t);
+  pub fn rembrandt_kernel_map_dropout(input: *const f32, n: i32, drop_ratio: c_float, scale: c_float,
+                                      rnd: *const f32, out: *mut f32, mask: *mut i32, stream: rh_stream_t);
+  pub fn rembrandt_kernel_map_dropout_backprop(out_delta: *const f32, n: i32, drop_ratio: c_float, scale: c_float,
+                                               mask: *const i32, in_delta: *mut f32, stream: rh_stream_t);
+  pub fn rh_rng_fill_uniform01_device(seed: u64, stream_id: u64, first: u64, dst: *mut f32, n: size_t,
+                                      stream: rh_stream_t) -> c_int;
+  pub fn rh_lrn_fwd(g: *const rh_lrn_geom, x: *const f32, y: *mut f32, denom: *mut f32, stream: rh_stream_t) -> c_int;
+  pub fn rh_lrn_bwd(g: *const rh_lrn_geom, x: *const f32, y: *const f32, denom: *const f32, dy: *const f32,
+                    dx: *mut f32, stream: rh_stream_t) -> c_int;
+
+  // CudnnBatchNormOp in Spatial mode (src/operator/conv.rs:493-535, 594-607): same alpha/beta pairs and buffer order.
+  pub fn rh_bnorm_workspace_bytes(n: c_int, c: c_int, plane: c_int) -> size_t;
+  pub fn rh_bnorm_fwd_train(n: c_int, c: c_int, plane: c_int, alpha: c_float, x: *const f32, beta: c_float,
+                            y: *mut f32, ema_factor: f64, epsilon: f64, scale: *const f32, bias: *const f32,
+                            running_mean: *mut f32, running_ivar: *mut f32, cached_mean: *mut f32,
+                            cached_ivar: *mut f32, ws: *mut c_void, ws_bytes: size_t, flags: c_int,
+                            stream: rh_stream_t) -> c_int;
+  pub fn rh_bnorm_fwd_infer(n: c_int, c: c_int, plane: c_int, alpha: c_float, x: *const f32, beta: c_float,
+                            y: *mut f32, epsilon: f64, scale: *const f32, bias: *const f32,
+                            running_mean: *const f32, running_ivar: *const f32, ws: *mut c_void, ws_bytes: size_t,
+                            flags: c_int, stream: rh_stream_t) -> c_int;
+  pub fn rh_bnorm_bwd(n: c_int, c: c_int, plane: c_int, alpha_data: c_float, beta_data: c_float, x: *const f32,
+                      dy: *const f32, dx: *mut f32, alpha_param: c_float, beta_param: c_float, epsilon: f64,
+                      scale: *const f32, dscale: *mut f32, dbias: *mut f32, cached_mean: *const f32,
+                      cached_ivar: *const f32, ws: *mut c_void, ws_bytes: size_t, stream: rh_stream_t) -> c_int;
 }
 
 /// The reference `unwrap()`s / `panic!`s on every native error (src/operator/mod.rs:1685-1696).
