@@ -29,7 +29,7 @@ MEASURED_TRAFFIC_BYTES = {
                 "conv_bwd_data_128x128": 1024 * (2.0 * 63944 + 70941)},
 }
 
-BATCH = {"alexnet": 256, "lenet": 64, "cifar10": 128, "nin": 128, "resnet18": 64}
+BATCH = {"alexnet": 256, "lenet": 64, "cifar10": 128, "nin": 128, "resnet18": 256}
 NUM_CLASSES_SEED = 0x5EED0000
 
 

@@ -114,8 +114,15 @@ typedef Tile<96, 128, 16, 1, 4, 4> T96x128;
 #endif
 // bf16-operand kernel: a deeper K step keeps more operand loads in flight per wave (its MFMAs are 16x shorter)
 typedef Tile<128, 128, RH_BF16_BK, 2, 2, RH_BF16_OCC> T128x128bf;
-typedef Tile<64, 256, 16, 1, 4> T64x256;
-typedef Tile<32, 256, 16, 1, 4> T32x256;
+typedef Tile<64, 256, 16, 1, 4, 3> T64x256;
+typedef Tile<32, 256, 16, 1, 4, 3> T32x256;
+// Half the K step: 20 KB of LDS, so a CU holds 4 blocks instead of 3.  For grids that need a second round of
+// blocks at 3 per CU but fit in one at 4 (e.g. 64 output channels over 64 x 56 x 56 pixels: 784 tiles).
+typedef Tile<64, 256, 8, 1, 4, 4> T64x256k8;
+inline bool prefer_k8_64(long long cols) {
+  const long long tiles = cdiv<long long>(cols, 256);
+  return cdiv<long long>(tiles, 1024) < cdiv<long long>(tiles, 768);
+}
 
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
@@ -128,9 +135,32 @@ struct SoffPlan {
   int Hp, Wp;      // padded image extent
   int halo;        // zeros added on each side
   size_t tab_bytes, wt_bytes, img_bytes;  // img_bytes == 0: the image is used in place
+  int splits;      // > 1: the contraction is cut into this many slices, partial results in part_bytes of scratch
+  size_t part_bytes;
   bool ok;         // false: fall back to the per-element gather path
-  size_t total() const { return tab_bytes + wt_bytes + img_bytes; }
+  size_t total() const { return tab_bytes + wt_bytes + img_bytes + part_bytes; }
 };
+
+// A forward / backward-data launch whose tiles would occupy under half of the block slots the GPU holds at a time
+// (small images late in a network, small batches) cuts the contraction into slices so that the slots fill; every
+// slice keeps at least 16 K steps.  Partial results go to scratch slabs shaped like the output and are added in a
+// fixed order by split_reduce_nchw.  Returns the slice count (1: no split).
+inline int plan_k_split(int rows, long long cols, int n_k) {
+  const int bm = pick_bm(rows), bn = bm >= 96 ? 128 : 256;
+  const long long slots = 256 * (bm >= 96 ? 4 : 3);
+  const long long tiles = (long long)cdiv(rows, bm) * cdiv<long long>(cols, bn);
+  if (tiles * 2 > slots) return 1;
+  long long want = slots / tiles;
+  const long long by_depth = (n_k / 16) / 16;
+  if (want > by_depth) want = by_depth;
+  if (want > 16) want = 16;
+  return want < 3 ? 1 : (int)want;   // two slices only trade one round of blocks for the partial-sum traffic
+}
+
+// out[i] = alpha * sum_s part[s*stride + i] + beta*out[i] (+ bias[channel], ReLU) over an NCHW tensor of `total`
+// elements, channel = (i / inner) % rows.
+void launch_split_reduce_nchw(const float* part, int splits, long long stride, float* out, long long total, int inner,
+                              int rows, float alpha, float beta, const float* bias, int relu, hipStream_t stream);
 
 inline SoffPlan plan_soff_fwd(const ConvDims& d) {
   SoffPlan p;
@@ -143,6 +173,8 @@ inline SoffPlan plan_soff_fwd(const ConvDims& d) {
   const size_t img = sizeof(float) * (size_t)d.N * d.C * p.Hp * p.Wp;
   p.img_bytes = d.pad > 0 ? align256(img) : 0;
   p.ok = img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
+  p.splits = plan_k_split(d.K, (long long)d.N * d.P * d.Q, p.n_k);
+  p.part_bytes = p.splits > 1 ? align256(sizeof(float) * (size_t)p.splits * (size_t)d.y_elems) : 0;
   return p;
 }
 
@@ -162,6 +194,8 @@ inline SoffPlan plan_soff_bwd_data(const ConvDims& d) {
   const size_t img = p.halo >= 0 ? sizeof(float) * (size_t)d.N * d.K * p.Hp * p.Wp : 0;
   p.img_bytes = (p.halo > 0 || d.st > 1 || p.Hp != d.P || p.Wp != d.Q) ? align256(img) : 0;
   p.ok = p.halo >= 0 && d.R == d.S && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
+  p.splits = plan_k_split(d.C, (long long)d.N * d.H * d.W, p.n_k);
+  p.part_bytes = p.splits > 1 ? align256(sizeof(float) * (size_t)p.splits * (size_t)d.x_elems) : 0;
   return p;
 }
 

@@ -38,6 +38,13 @@ FULL_CONV = {
     "sweep_c_1x1": (128, 96, 55, 55, 96, 1, 1, 0),
     "alexnet_conv1": (256, 3, 227, 227, 96, 11, 4, 0),
     "alexnet_conv5": (256, 384, 13, 13, 256, 3, 1, 1),
+    # ResNet-18 template at batch 64: 64-row tiles with the halved K step (784 tiles), contraction cut into slices
+    # (7x7 and 14x14 extents), a strided 3x3 layer and a strided 1x1 projection
+    "resnet_56_64": (64, 64, 56, 56, 64, 3, 1, 1),
+    "resnet_14_256": (64, 256, 14, 14, 256, 3, 1, 1),
+    "resnet_7_512": (64, 512, 7, 7, 512, 3, 1, 1),
+    "resnet_down_512": (64, 256, 14, 14, 512, 3, 2, 1),
+    "resnet_proj_128": (64, 64, 56, 56, 128, 1, 2, 0),
 }
 
 
