@@ -1061,14 +1061,28 @@ struct BNormConvUnit {
     }
   }
   // pre_delta = dBN(out_delta) with the scale / bias gradients accumulated, then grad_weights += dconv(in, pre_delta).
-  void backward_params(size_t batch, const float* in, const float* out_delta, double epsilon, DeviceBuffer<uint8_t>& ws) {
+  // With `ws_aux` the filter gradient goes to the context's second stream (scratch of its own) and overlaps whatever
+  // the main stream does next with pre_delta (the data gradient); the worker joins at the end of backward.
+  void backward_params(size_t batch, const float* in, const float* out_delta, double epsilon, DeviceBuffer<uint8_t>& ws,
+                       DeviceBuffer<uint8_t>* ws_aux) {
     RB_ASSERT(backward);
     const rh_conv_geom g = geom(batch);
     unwrap(rh_bnorm_bwd(g.N, g.K, plane(), 1.0f, 0.0f, pre_act->as_ptr(), out_delta, pre_delta->as_mut_ptr(), 1.0f, 1.0f,
                         epsilon, scale->as_ptr(), scale_grad->as_mut_ptr(), bias_grad->as_mut_ptr(), cached_mean->as_ptr(),
                         cached_ivar->as_ptr(), ws.as_mut_ptr(), ws.len(), s()), "batch norm backward");
-    unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in, pre_delta->as_ptr(), 1.0f, grad_weights->as_mut_ptr(), ws.as_mut_ptr(),
-                                ws.len(), 0, s()), "conv2d backward filter");
+    rh_stream_t sg = s();
+    DeviceBuffer<uint8_t>* wg = &ws;
+    if (ws_aux) {
+      ctx->fork();
+      sg = ctx->aux_stream();
+      wg = ws_aux;
+    }
+    unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in, pre_delta->as_ptr(), 1.0f, grad_weights->as_mut_ptr(), wg->as_mut_ptr(),
+                                wg->len(), 0, sg), "conv2d backward filter");
+  }
+  size_t aux_workspace_bytes() const {
+    const rh_conv_geom g = geom(batch_cap);
+    return rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_FILTER);
   }
   // in_delta = beta*in_delta + dconv^T(weights, pre_delta)
   void backward_data(size_t batch, float* in_delta, float beta, DeviceBuffer<uint8_t>& ws) {
@@ -1253,8 +1267,14 @@ class BNormUnitsOperator : public Operator {
     size_t ws = 256;
     for (auto& u : units_) ws = std::max(ws, u.workspace_bytes());
     workspace_.reset(new DeviceBuffer<uint8_t>(ws, context_));
-    (void)bwd;
+    if (bwd && opts_.overlap_backward) {
+      size_t wa = 256;
+      for (auto& u : units_) wa = std::max(wa, u.aux_workspace_bytes());
+      workspace_aux_.reset(new DeviceBuffer<uint8_t>(wa, context_));
+    }
   }
+  // scratch of the filter gradients when they run on the second stream, else null
+  DeviceBuffer<uint8_t>* aux_ws() { return workspace_aux_ && overlap_on_ ? workspace_aux_.get() : nullptr; }
   // ReLU after a batch norm: inside its apply kernel, or as the separate in-place pass of the reference.
   bool fuse_relu(ActivationFunction f) const {
     if (f != ActivationFunction::Identity && f != ActivationFunction::Rect) panic("unimplemented activation function");
@@ -1270,7 +1290,11 @@ class BNormUnitsOperator : public Operator {
   ParamsInit init_weights_ = ParamsInit::MakeDisabled();
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   std::unique_ptr<DeviceBuffer<float>> mid_act_, mid_delta_;
-  std::unique_ptr<DeviceBuffer<uint8_t>> workspace_;
+  std::unique_ptr<DeviceBuffer<uint8_t>> workspace_, workspace_aux_;
+  bool overlap_on_ = true;
+
+ public:
+  void set_overlap_backward(bool on) override { overlap_on_ = on; }
 };
 
 // ---- BNormConv2dOperator (src/operator/conv.rs:106-912) ---------------------------------------------------
@@ -1295,13 +1319,20 @@ class BNormConv2dOperator : public BNormUnitsOperator {
   void backward(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
     BNormConvUnit& u = units_[0];
-    apply_rect_backprop(config_.act_func, out_act_->as_ptr(), u.out_dims.len(), batch_size, out_delta_->as_mut_ptr(), context_->stream());
-    u.backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    if (!act_bwd_folded_)
+      apply_rect_backprop(config_.act_func, out_act_->as_ptr(), u.out_dims.len(), batch_size, out_delta_->as_mut_ptr(), context_->stream());
+    u.backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
     if (in_delta_) u.backward_data(batch_size, in_delta_->as_mut_ptr(), 0.0f, *workspace_);
   }
   const char* kind() const override { return "BNormConv2dOperator"; }
+  bool fold_activation_backward() override {
+    if (config_.act_func != ActivationFunction::Rect) return false;
+    act_bwd_folded_ = true;
+    return true;
+  }
 
  private:
+  bool act_bwd_folded_ = false;
   BNormConv2dOperatorConfig config_;
 };
 
@@ -1340,10 +1371,10 @@ class StackResConv2dOperator : public BNormUnitsOperator {
     const size_t len = config_.in_dims.len();
     rh_stream_t s = context_->stream();
     apply_rect_backprop(config_.act_func, out_act_->as_ptr(), len, batch_size, out_delta_->as_mut_ptr(), s);
-    units_[1].backward_params(batch_size, mid_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    units_[1].backward_params(batch_size, mid_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
     units_[1].backward_data(batch_size, mid_delta_->as_mut_ptr(), 0.0f, *workspace_);
     apply_rect_backprop(config_.act_func, mid_act_->as_ptr(), len, batch_size, mid_delta_->as_mut_ptr(), s);
-    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
     if (in_delta_) {
       unwrap(rh_copy_d2d(in_delta_->as_mut_ptr(), out_delta_->as_ptr(), len * batch_size * 4, s), "send");
       units_[0].backward_data(batch_size, in_delta_->as_mut_ptr(), 1.0f, *workspace_);
@@ -1399,11 +1430,11 @@ class ProjStackResConv2dOperator : public BNormUnitsOperator {
     const size_t len = config_.out_dims.len();
     rh_stream_t s = context_->stream();
     apply_rect_backprop(config_.act_func, out_act_->as_ptr(), len, batch_size, out_delta_->as_mut_ptr(), s);
-    units_[1].backward_params(batch_size, mid_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    units_[1].backward_params(batch_size, mid_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
     units_[1].backward_data(batch_size, mid_delta_->as_mut_ptr(), 0.0f, *workspace_);
     apply_rect_backprop(config_.act_func, mid_act_->as_ptr(), len, batch_size, mid_delta_->as_mut_ptr(), s);
-    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
-    units_[2].backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_);
+    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
+    units_[2].backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
     if (in_delta_) {
       units_[0].backward_data(batch_size, in_delta_->as_mut_ptr(), 0.0f, *workspace_);
       units_[2].backward_data(batch_size, in_delta_->as_mut_ptr(), 1.0f, *workspace_);

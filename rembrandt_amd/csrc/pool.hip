@@ -314,13 +314,15 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
   return launch_status();
 }
 
-static bool lds_bwd_ok(const PoolDims& d) { return d.P * d.Q <= 2048 && d.H * d.W <= (1 << 20); }
+// The dy and mask of at least one whole plane must fit the block's LDS (8 bytes per pooled element, 32 KB at most).
+static bool lds_bwd_ok(const PoolDims& d) { return d.P * d.Q <= 4096 && d.H * d.W <= (1 << 20); }
 
 static int launch_pool_bwd_lds(const PoolDims& d, const float* dy, const int32_t* argmax, const float* relu_y, float* dx,
                                rh_stream_t stream) {
   const int PQ = d.P * d.Q;
   int PB = 2048 / PQ;
   if (PB > 64) PB = 64;
+  if (PB < 1) PB = 1;
   const long long planes = (long long)d.N * d.C;
   const long long blocks = cdiv<long long>(planes, PB);
   if (blocks >= (1ll << 31)) return RH_E_LIMIT;
