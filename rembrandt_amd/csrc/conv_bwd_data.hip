@@ -41,6 +41,66 @@ __global__ void prep_bwd_data_soff_kernel(const float* __restrict__ w, float* __
   }
 }
 
+// One residue class of the strided form: wT[k][c] = w[ko][c][a + st*i][b + st*j] for k = (ko, i, j) (zero rows past
+// the end) and soff[k] = 4*(ko*Hp*Wp + (Ra-1-i)*Wp + (Sb-1-j)) into the padded dy.
+__global__ void prep_bwd_data_phase_kernel(const float* __restrict__ w, float* __restrict__ wT, int* __restrict__ soff,
+                                           int n_k, int k_true, int C, int R, int S, int st, int a, int b, int Ra, int Sb,
+                                           int HpWp, int Wp) {
+  const long long total = (long long)n_k * C;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const int k = (int)(idx / C), c = (int)(idx - (long long)k * C);
+    float v = 0.0f;
+    int off = 0;
+    if (k < k_true) {
+      const int ko = k / (Ra * Sb), ij = k - ko * (Ra * Sb), i = ij / Sb, j = ij - i * Sb;
+      v = w[(((size_t)ko * C + c) * R + (a + st * i)) * S + (b + st * j)];
+      off = (ko * HpWp + (Ra - 1 - i) * Wp + (Sb - 1 - j)) * 4;
+    }
+    wT[idx] = v;
+    if (c == 0) soff[k] = off;
+  }
+}
+
+// dx[n][c][h][w] = alpha * (result of the class of (h + pad, w + pad) at its (u, v)) + beta * dx; classes without
+// filter taps contribute 0.
+struct PhaseTable {
+  int u0[kMaxPhaseStride * kMaxPhaseStride], U[kMaxPhaseStride * kMaxPhaseStride];
+  int v0[kMaxPhaseStride * kMaxPhaseStride], V[kMaxPhaseStride * kMaxPhaseStride];
+  long long off[kMaxPhaseStride * kMaxPhaseStride];  // < 0: no taps
+};
+__global__ __launch_bounds__(256) void phase_interleave_kernel(const float* __restrict__ sub, float* __restrict__ dx,
+                                                               unsigned total, FastDiv dW, FastDiv dH, FastDiv dSt, int st,
+                                                               int pad, PhaseTable t, float alpha, float beta) {
+  // per class: {offset of its result minus the offset of its first pixel, row length V, plane size U*V}; the table is
+  // indexed per element, so it lives in LDS rather than in the kernel arguments
+  __shared__ long long s_base[kMaxPhaseStride * kMaxPhaseStride];
+  __shared__ int s_V[kMaxPhaseStride * kMaxPhaseStride], s_UV[kMaxPhaseStride * kMaxPhaseStride];
+  if (threadIdx.x < kMaxPhaseStride * kMaxPhaseStride) {
+    const int i = threadIdx.x;
+    const bool live = i < st * st && t.off[i] >= 0;
+    s_base[i] = live ? t.off[i] - ((long long)t.u0[i] * t.V[i] + t.v0[i]) : -1;
+    s_V[i] = live ? t.V[i] : 0;
+    s_UV[i] = live ? t.U[i] * t.V[i] : 0;
+  }
+  __syncthreads();
+  const unsigned step = gridDim.x * blockDim.x;
+  for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += step) {
+    uint32_t rest, w, plane, h, u, a, v, b;
+    dW.divmod(idx, rest, w);
+    dH.divmod(rest, plane, h);
+    dSt.divmod(h + (uint32_t)pad, u, a);
+    dSt.divmod(w + (uint32_t)pad, v, b);
+    const int ph = (int)(a * st + b);
+    const int V = s_V[ph];
+    float val = 0.0f;
+    if (V > 0) val = sub[s_base[ph] + (long long)plane * s_UV[ph] + (long long)u * V + v];
+    val *= alpha;
+    if (beta != 0.0f) val = fmaf(beta, dx[idx], val);
+    dx[idx] = val;
+  }
+}
+
 template <class T>
 static int run_bwd_data_soff(const RowSParams& ap, const RowSParams& bp, EpiParams ep, int n_k, int k_true,
                              hipStream_t stream, const char* tag, int splits, float* part) {
@@ -82,6 +142,63 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
   hipStream_t stream = to_stream(stream_);
 
   const int KRS = d.K * d.R * d.S;
+  const PhasePlan pp = plan_phase_bwd_data(d);
+  if (pp.ok && !(flags & RH_ALGO_GATHER)) {
+    if (d.x_elems == 0) return 0;
+    char* base = static_cast<char*>(ws);
+    int* soff = reinterpret_cast<int*>(base);
+    float* wT = reinterpret_cast<float*>(base + pp.tab_bytes);
+    float* sub = reinterpret_cast<float*>(base + pp.tab_bytes + pp.wt_bytes + pp.img_bytes);
+    float* part = reinterpret_cast<float*>(base + pp.tab_bytes + pp.wt_bytes + pp.img_bytes + pp.sub_bytes);
+    const float* img = dy;
+    if (pp.img_bytes) {
+      float* dyp = reinterpret_cast<float*>(base + pp.tab_bytes + pp.wt_bytes);
+      launch_pad_image(dy, dyp, (long long)d.N * d.K, d.P, d.Q, pp.Hp, pp.Wp, pp.L, stream);
+      if (int e = launch_status()) return e;
+      img = dyp;
+    }
+    const size_t img_floats = (size_t)d.N * d.K * pp.Hp * pp.Wp;
+    PhaseTable tab;
+    for (int a = 0; a < d.st; ++a)
+      for (int b = 0; b < d.st; ++b) {
+        const int i = a * d.st + b;
+        const PhaseGeom& g = pp.ph[i];
+        const bool live = g.Ra > 0 && g.Sb > 0 && g.U > 0 && g.V > 0;
+        tab.u0[i] = g.u0; tab.U[i] = g.U; tab.v0[i] = g.v0; tab.V[i] = g.V; tab.off[i] = live ? g.sub_off : -1;
+        if (!live) continue;
+        const int k_true = d.K * g.Ra * g.Sb, n_k = round_up(k_true, kTabPad);
+        hipLaunchKernelGGL(prep_bwd_data_phase_kernel, dim3(stream_grid((size_t)n_k * d.C, 256)), dim3(256), 0, stream, w, wT,
+                           soff, n_k, k_true, d.C, d.R, d.S, d.st, a, b, g.Ra, g.Sb, pp.Hp * pp.Wp, pp.Wp);
+        if (int e = launch_status()) return e;
+        RowSParams ap;  // transposed sub-filter [k][c]
+        ap.ptr = wT; ap.bytes = (uint32_t)(sizeof(float) * (size_t)n_k * d.C);
+        ap.M = d.C; ap.inner = d.C; ap.innerW = d.C; ap.img_stride = 0; ap.a_stride = 0; ap.b_stride = 1;
+        ap.soff = nullptr; ap.ldk4 = d.C * 4;
+        // padded dy seen from the class's first pixel and first tap: rows = (n, u - u0, v - v0)
+        const size_t first = (size_t)(g.u0 + pp.L - (g.Ra - 1)) * pp.Wp + (size_t)(g.v0 + pp.L - (g.Sb - 1));
+        RowSParams bp;
+        bp.ptr = img + first; bp.bytes = (uint32_t)(sizeof(float) * (img_floats - first));
+        bp.M = d.N * g.U * g.V; bp.inner = g.U * g.V; bp.innerW = g.V;
+        bp.img_stride = d.K * pp.Hp * pp.Wp; bp.a_stride = pp.Wp; bp.b_stride = 1;
+        bp.soff = soff; bp.ldk4 = 0;
+        EpiParams ep;
+        ep.out = sub + g.sub_off; ep.bias = nullptr; ep.alpha = 1.0f; ep.beta = 0.0f;
+        ep.rows = d.C; ep.cols = bp.M; ep.inner = g.U * g.V; ep.ld = 0; ep.relu = 0; ep.split_stride = 0;
+        int e;
+        switch (pick_bm(d.C)) {
+          case 128: e = run_bwd_data_soff<T128x128>(ap, bp, ep, n_k, k_true, stream, "conv_bwd_data_128x128", g.splits, part); break;
+          case 96:  e = run_bwd_data_soff<T96x128>(ap, bp, ep, n_k, k_true, stream, "conv_bwd_data_96x128", g.splits, part); break;
+          case 64:  e = run_bwd_data_soff<T64x256>(ap, bp, ep, n_k, k_true, stream, "conv_bwd_data_64x256", g.splits, part); break;
+          default:  e = run_bwd_data_soff<T32x256>(ap, bp, ep, n_k, k_true, stream, "conv_bwd_data_32x256", g.splits, part); break;
+        }
+        if (e) return e;
+      }
+    ProfScope prof("phase_interleave", 8.0 * (double)d.x_elems, stream);
+    hipLaunchKernelGGL(phase_interleave_kernel, dim3(stream_grid((size_t)d.x_elems, 256)), dim3(256), 0, stream, sub, dx,
+                       (unsigned)d.x_elems, FastDiv((uint32_t)d.W), FastDiv((uint32_t)d.H), FastDiv((uint32_t)d.st), d.st, d.pad,
+                       tab, alpha, beta);
+    return launch_status();
+  }
   const SoffPlan sp = plan_soff_bwd_data(d);
   if (sp.ok && !(flags & RH_ALGO_GATHER)) {
     int* soff = static_cast<int*>(ws);

@@ -101,7 +101,13 @@ static bool use_soff_bwd_filter(const ConvDims& d) {
   // small 5x5 layers at 75-78 and 1x1 at 12 lose or tie; 3x3 / 5x5 layers at 288-402 win by 25 %)
   const double flops = 2.0 * d.K * d.C * d.R * d.S * (double)d.N * d.P * d.Q;
   const double bytes = 8.0 * ((double)d.y_elems + (double)d.N * d.C * (d.H + 2 * d.pad) * (d.W + 2 * d.pad));
-  return flops / bytes >= 150.0;
+  // The contraction itself runs at about 100 (64-row tiles) / 125 (128-row) TFLOP/s on this path against 65 / 90 with
+  // the gather loaders, and the transposes move their bytes at about 3.8 TB/s: break-even near 50 / 85 FLOPs per byte
+  // (measured: 64 -> 64 channels 3x3 on 56x56 at 70 wins by 13 %, 128 -> 128 on 28x28 at 134 by 11 %, a stride-2
+  // 64 -> 128 layer at 46 loses by 6 %).
+  // 32-row tiles (half of the loader rows idle) tie at 75-78.
+  const int bm = pick_bm(d.K);
+  return flops / bytes >= (bm == 64 ? 60.0 : bm == 32 ? 150.0 : 100.0);
 }
 
 struct BwdFilterSoffPlan {
@@ -357,6 +363,8 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
     case RH_CONV_BWD_DATA: {
       const size_t legacy = align256(sizeof(int4) * (size_t)round_up(KRS, kTabPad)) +
                             align256(sizeof(int) * (size_t)round_up(KRS, kTabPad));
+      const PhasePlan pp = plan_phase_bwd_data(d);
+      if (pp.ok) return pp.total() > legacy ? pp.total() : legacy;
       const SoffPlan sp = plan_soff_bwd_data(d);
       return sp.ok && sp.total() > legacy ? sp.total() : legacy;
     }

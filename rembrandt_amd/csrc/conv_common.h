@@ -199,6 +199,76 @@ inline SoffPlan plan_soff_bwd_data(const ConvDims& d) {
   return p;
 }
 
+// Backward-data with stride st > 1, decomposed by the residue (a, b) of (h + pad, w + pad) modulo st: an input pixel
+// with h + pad = st*u + a only meets the filter rows r = a + st*i, and then through dy row p = u - i.  Each of the
+// st*st classes is therefore a stride-1 correlation of dy with the sub-filter w[ko][c][a + st*i][b + st*j] over the
+// sub-grid (u, v) of that class, with no wasted products.  Scratch: one padded copy of dy shared by all classes
+// (halo L = ceil(R/st) - 1 on top / left, zeros below / right up to the largest u any class reaches), the transposed
+// sub-filter and offset table of the class at hand, and the dense per-class results, which one pass interleaves into dx.
+constexpr int kMaxPhaseStride = 4;
+struct PhaseGeom {
+  int Ra, Sb;          // filter rows / columns of the class (0: the class receives nothing)
+  int u0, U, v0, V;    // first u, v of the class inside the image and how many
+  long long sub_off;   // where the class's dense [n][c][U][V] result starts in the scratch, in floats
+  int splits;          // slices of the class's contraction (plan_k_split)
+};
+struct PhasePlan {
+  bool ok;
+  int L, Hp, Wp, n_k;  // n_k: the largest padded contraction length among the classes
+  size_t tab_bytes, wt_bytes, img_bytes, sub_bytes, part_bytes;
+  PhaseGeom ph[kMaxPhaseStride * kMaxPhaseStride];
+  size_t total() const { return tab_bytes + wt_bytes + img_bytes + sub_bytes + part_bytes; }
+};
+
+inline void phase_axis(int a, int st, int pad, int extent, int taps, int* n_taps, int* first, int* count) {
+  *n_taps = a < taps ? (taps - a + st - 1) / st : 0;
+  const int lo = pad > a ? (pad - a + st - 1) / st : 0;
+  const int top = extent - 1 + pad - a;
+  const int hi = top >= 0 ? top / st + 1 : 0;
+  *first = lo;
+  *count = hi > lo ? hi - lo : 0;
+}
+
+inline PhasePlan plan_phase_bwd_data(const ConvDims& d) {
+  PhasePlan p;
+  p.ok = false;
+  p.L = p.Hp = p.Wp = p.n_k = 0;
+  p.tab_bytes = p.wt_bytes = p.img_bytes = p.sub_bytes = p.part_bytes = 0;
+  if (d.st < 2 || d.st > kMaxPhaseStride || d.P <= 0 || d.Q <= 0) return p;
+  const int st = d.st;
+  p.L = (d.R > d.S ? d.R : d.S);
+  p.L = (p.L + st - 1) / st - 1;
+  const int umax = (d.H - 1 + d.pad) / st + 1, vmax = (d.W - 1 + d.pad) / st + 1;
+  p.Hp = p.L + (d.P > umax ? d.P : umax);
+  p.Wp = p.L + (d.Q > vmax ? d.Q : vmax);
+  long long off = 0;
+  int max_taps = 0;
+  for (int a = 0; a < st; ++a)
+    for (int b = 0; b < st; ++b) {
+      PhaseGeom& g = p.ph[a * st + b];
+      phase_axis(a, st, d.pad, d.H, d.R, &g.Ra, &g.u0, &g.U);
+      phase_axis(b, st, d.pad, d.W, d.S, &g.Sb, &g.v0, &g.V);
+      g.sub_off = off;
+      const long long elems = (long long)d.N * d.C * g.U * g.V;
+      off += elems;
+      if (g.Ra * g.Sb > max_taps) max_taps = g.Ra * g.Sb;
+      g.splits = 1;
+      if (g.Ra * g.Sb > 0 && elems > 0) {
+        g.splits = plan_k_split(d.C, (long long)d.N * g.U * g.V, round_up(d.K * g.Ra * g.Sb, kTabPad));
+        const size_t part = g.splits > 1 ? align256(sizeof(float) * (size_t)g.splits * (size_t)elems) : 0;
+        if (part > p.part_bytes) p.part_bytes = part;
+      }
+    }
+  p.n_k = round_up(d.K * (max_taps > 0 ? max_taps : 1), kTabPad);
+  p.tab_bytes = align256(sizeof(int) * (size_t)p.n_k);
+  p.wt_bytes = align256(sizeof(float) * (size_t)p.n_k * d.C);
+  const size_t img = sizeof(float) * (size_t)d.N * d.K * p.Hp * p.Wp;
+  p.img_bytes = (p.L > 0 || p.Hp != d.P || p.Wp != d.Q) ? align256(img) : 0;
+  p.sub_bytes = align256(sizeof(float) * (size_t)off);
+  p.ok = img <= kMaxBufferBytes && (size_t)off * 4 <= kMaxBufferBytes;
+  return p;
+}
+
 // dst[n][c][halo + dil*h][halo + dil*w] = src[n][c][h][w], zeros elsewhere; dst is planes x Hp x Wp.
 void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
                       hipStream_t stream, int dil = 1);

@@ -30,6 +30,15 @@ CONV_CASES = [
     (2, 6, 15, 15, 10, 3, 2, 1),     # stride 2 with pad
     (1, 4, 10, 10, 8, 3, 3, 0),      # stride 3
     (70, 2, 6, 6, 5, 3, 1, 1),       # many images, pixel tiles straddle images
+    # strided backward-data by residue classes: classes without filter taps (1x1), odd extents whose last rows no
+    # window covers, 7x7 stride 2 pad 3, stride 4 with padding, a contraction deep enough to be cut into slices,
+    # and a stride beyond the class form (zero-dilated copy)
+    (2, 8, 12, 12, 16, 1, 2, 0),
+    (2, 5, 14, 11, 6, 3, 2, 0),
+    (2, 3, 30, 30, 16, 7, 2, 3),
+    (2, 4, 21, 21, 6, 5, 4, 2),
+    (2, 8, 14, 14, 256, 3, 2, 1),
+    (1, 3, 16, 16, 4, 5, 5, 0),
 ]
 
 
