@@ -103,10 +103,22 @@ __global__ __launch_bounds__(256) void phase_interleave_kernel(const float* __re
 
 template <class T>
 static int run_bwd_data_soff(const RowSParams& ap, const RowSParams& bp, EpiParams ep, int n_k, int k_true,
-                             hipStream_t stream, const char* tag, int splits, float* part) {
+                             hipStream_t stream, const char* tag, int splits, float* part,
+                             const TailSplit* tail = nullptr) {
   constexpr int AROWS = T::BM % 64 == 0 ? T::BM : (T::BM + 63) / 64 * 64;
   typedef LoadRowS<AROWS, T::BK, T::NT, true> AL;
   typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
+  if (splits <= 1 && tail && tail->splits > 1) {
+    // whole tiles blend into dx as usual; the sliced tail goes through `part` and one reduction over its columns
+    const EpiParams fin = ep;
+    const long long total = (long long)ep.rows * ep.cols;
+    ep.part = part; ep.split_stride = total;
+    ep.full_tiles = tail->full_tiles; ep.tail_tiles = tail->tail_tiles; ep.tail_splits = tail->splits;
+    if (int e = launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true)) return e;
+    launch_split_reduce_nchw(part, tail->splits, total, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta, nullptr, 0,
+                             stream, tail->col0);
+    return launch_status();
+  }
   if (splits <= 1) return launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
   // slices of the contraction write unblended partial results; one reduction applies the alpha / beta blend
   const EpiParams fin = ep;
@@ -227,13 +239,13 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
     ep.rows = d.C; ep.cols = bp.M; ep.inner = d.H * d.W; ep.ld = 0; ep.relu = 0; ep.split_stride = 0;
     float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes + sp.img_bytes);
     switch (pick_bm(d.C)) {
-      case 128: return run_bwd_data_soff<T128x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_128x128", sp.splits, part);
-      case 96:  return run_bwd_data_soff<T96x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_96x128", sp.splits, part);
+      case 128: return run_bwd_data_soff<T128x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_128x128", sp.splits, part, &sp.tail);
+      case 96:  return run_bwd_data_soff<T96x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_96x128", sp.splits, part, &sp.tail);
       case 64:
         if (cdiv(d.C, 64) == 1 && prefer_k8_64(ep.cols))
-          return run_bwd_data_soff<T64x256k8>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_64x256k8", sp.splits, part);
-        return run_bwd_data_soff<T64x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_64x256", sp.splits, part);
-      default:  return run_bwd_data_soff<T32x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_32x256", sp.splits, part);
+          return run_bwd_data_soff<T64x256k8>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_64x256k8", sp.splits, part, &sp.tail);
+        return run_bwd_data_soff<T64x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_64x256", sp.splits, part, &sp.tail);
+      default:  return run_bwd_data_soff<T32x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_32x256", sp.splits, part, &sp.tail);
     }
   }
   const int n_tab = round_up(KRS, kTabPad);

@@ -59,11 +59,16 @@ inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Pa
                             hipStream_t stream, const char* tag, int k_algorithmic = 0) {
   const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
   const int k_chunks = cdiv(K, T::BK);
+  if (ep.tail_tiles > 0) splits = ep.tail_splits;  // tail form: the slices apply to the last tail_tiles tiles only
   if (splits < 1) splits = 1;
   const int cps = cdiv(k_chunks, splits) > 0 ? cdiv(k_chunks, splits) : 1;
   const int used = cdiv(k_chunks, cps) > 0 ? cdiv(k_chunks, cps) : 1;
   if (splits_used) *splits_used = used;
   dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)used);
+  if (ep.tail_tiles > 0) {
+    if (used != ep.tail_splits || ep.full_tiles + ep.tail_tiles != tiles_m * tiles_n) return RH_E_INVALID;
+    grid = dim3((unsigned)(ep.full_tiles + ep.tail_tiles * ep.tail_splits), 1u);
+  }
   constexpr size_t lds_bytes = sizeof(float) * 2 * T::BK * (AL::LD + BL::LD);
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
   if (lds_bytes > 48 * 1024) {
@@ -128,6 +133,39 @@ inline bool prefer_k8_64(long long cols) {
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
                          int ld, float alpha, float beta, hipStream_t stream);
 
+// Tail form of a forward / backward-data launch (see EpiParams): when all tiles are resident at once and their count
+// is not close to a multiple of the 256 CUs, the column tiles beyond the last multiple are cut into `splits` slices
+// so that every CU ends up with nearly the same work.  splits == 1: not worth it.
+struct TailSplit {
+  int full_tiles, tail_tiles, splits;
+  long long col0;  // first column of the tail
+};
+inline TailSplit plan_tail_split(int rows, long long cols, int n_k) {
+  TailSplit t = {0, 0, 1, 0};
+  const int bm = pick_bm(rows), bn = bm >= 96 ? 128 : 256;
+  const int tiles_m = cdiv(rows, bm);
+  const long long tiles_n = cdiv<long long>(cols, bn), T = tiles_m * tiles_n;
+  const bool k8 = bm == 64 && tiles_m == 1 && prefer_k8_64(cols);  // the 64x256 tile with the halved K step: 4 per CU
+  const long long slots = 256 * (bm >= 96 || k8 ? 4 : 3);
+  if (T > slots || T * 3 <= slots) return t;  // several rounds of blocks, or the whole-result split applies
+  const long long full_cols = (T / 256 * 256) / tiles_m, full = full_cols * tiles_m, tail = T - full;
+  if (tail == 0 || full == 0) return t;
+  // Busiest CU in units of one tile's time: whole tiles + its pieces + the partial-sum traffic of those pieces
+  // (a tile alone on a CU at ~0.47 TFLOP/s; a piece's slab written and read at a CU's share of ~4 TB/s).
+  const double tile_us = 2.0 * bm * bn * (double)n_k / 0.47e6, piece_us = 8.0 * bm * bn / 15.6e3;
+  const int k_chunks = n_k / 16;
+  double best = (double)cdiv<long long>(T, 256);
+  const double need = 0.93 * best;
+  for (int S = 2; S <= 16 && S * 8 <= k_chunks; ++S) {
+    if (k_chunks % S != 0) continue;  // equal slices, for the 16- and the 8-deep K step alike
+    const long long pieces = cdiv<long long>(tail * S, 256);
+    const double cost = (double)cdiv<long long>(full, 256) + (double)pieces / S + pieces * piece_us / tile_us;
+    if (cost < best && cost <= need) { best = cost; t.splits = S; }
+  }
+  if (t.splits > 1) { t.full_tiles = (int)full; t.tail_tiles = (int)tail; t.col0 = full_cols * bn; }
+  return t;
+}
+
 // Scratch layout of the scalar-offset forward / backward-data paths:
 //   [k -> byte offset table : n_k ints][transposed filter : n_k x rows floats][padded image copy]
 struct SoffPlan {
@@ -136,6 +174,7 @@ struct SoffPlan {
   int halo;        // zeros added on each side
   size_t tab_bytes, wt_bytes, img_bytes;  // img_bytes == 0: the image is used in place
   int splits;      // > 1: the contraction is cut into this many slices, partial results in part_bytes of scratch
+  TailSplit tail;  // tail.splits > 1: only the last tiles are cut (splits == 1 then)
   size_t part_bytes;
   bool ok;         // false: fall back to the per-element gather path
   size_t total() const { return tab_bytes + wt_bytes + img_bytes + part_bytes; }
@@ -158,9 +197,11 @@ inline int plan_k_split(int rows, long long cols, int n_k) {
 }
 
 // out[i] = alpha * sum_s part[s*stride + i] + beta*out[i] (+ bias[channel], ReLU) over an NCHW tensor of `total`
-// elements, channel = (i / inner) % rows.
+// elements, channel = (i / inner) % rows; only elements whose column (image * inner + pixel) is >= col0.
 void launch_split_reduce_nchw(const float* part, int splits, long long stride, float* out, long long total, int inner,
-                              int rows, float alpha, float beta, const float* bias, int relu, hipStream_t stream);
+                              int rows, float alpha, float beta, const float* bias, int relu, hipStream_t stream,
+                              long long col0 = 0);
+
 
 inline SoffPlan plan_soff_fwd(const ConvDims& d) {
   SoffPlan p;
@@ -174,7 +215,9 @@ inline SoffPlan plan_soff_fwd(const ConvDims& d) {
   p.img_bytes = d.pad > 0 ? align256(img) : 0;
   p.ok = img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
   p.splits = plan_k_split(d.K, (long long)d.N * d.P * d.Q, p.n_k);
-  p.part_bytes = p.splits > 1 ? align256(sizeof(float) * (size_t)p.splits * (size_t)d.y_elems) : 0;
+  p.tail = plan_tail_split(d.K, (long long)d.N * d.P * d.Q, p.n_k);
+  const int slabs_f = p.splits > 1 ? p.splits : p.tail.splits;
+  p.part_bytes = slabs_f > 1 ? align256(sizeof(float) * (size_t)slabs_f * (size_t)d.y_elems) : 0;
   return p;
 }
 
@@ -195,7 +238,10 @@ inline SoffPlan plan_soff_bwd_data(const ConvDims& d) {
   p.img_bytes = (p.halo > 0 || d.st > 1 || p.Hp != d.P || p.Wp != d.Q) ? align256(img) : 0;
   p.ok = p.halo >= 0 && d.R == d.S && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
   p.splits = plan_k_split(d.C, (long long)d.N * d.H * d.W, p.n_k);
-  p.part_bytes = p.splits > 1 ? align256(sizeof(float) * (size_t)p.splits * (size_t)d.x_elems) : 0;
+  p.tail = plan_tail_split(d.C, (long long)d.N * d.H * d.W, p.n_k);
+  if (d.st > 1) p.tail.splits = 1;  // the zero-dilated form is a fallback only
+  const int slabs_b = p.splits > 1 ? p.splits : p.tail.splits;
+  p.part_bytes = slabs_b > 1 ? align256(sizeof(float) * (size_t)slabs_b * (size_t)d.x_elems) : 0;
   return p;
 }
 

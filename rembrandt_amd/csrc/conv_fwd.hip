@@ -91,11 +91,16 @@ __global__ void prep_fwd_soff_kernel(const float* __restrict__ w, float* __restr
 }
 
 __global__ __launch_bounds__(256) void split_reduce_nchw_kernel(const float* __restrict__ part, int splits, long long stride,
-                                                                float* __restrict__ out, unsigned total, FastDiv inner,
-                                                                FastDiv rows, float alpha, float beta,
-                                                                const float* __restrict__ bias, int relu) {
+                                                                float* __restrict__ out, unsigned first, unsigned total,
+                                                                FastDiv inner, FastDiv rows, float alpha, float beta,
+                                                                const float* __restrict__ bias, int relu,
+                                                                unsigned col0) {
   const unsigned step = gridDim.x * blockDim.x;
-  for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
+  for (unsigned i = first + blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
+    if (col0 > 0) {  // column = image * inner + pixel
+      const uint32_t plane = inner.quot(i), img = rows.quot(plane);
+      if (img * inner.div + (i - plane * inner.div) < col0) continue;
+    }
     float a0 = 0.0f, a1 = 0.0f;
     int s = 0;
     for (; s + 1 < splits; s += 2) {
@@ -115,23 +120,38 @@ __global__ __launch_bounds__(256) void split_reduce_nchw_kernel(const float* __r
 }
 
 void launch_split_reduce_nchw(const float* part, int splits, long long stride, float* out, long long total, int inner,
-                              int rows, float alpha, float beta, const float* bias, int relu, hipStream_t stream) {
-  ProfScope prof("split_reduce", 4.0 * (double)total * (splits + 1), stream);
-  hipLaunchKernelGGL(split_reduce_nchw_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, part, splits,
-                     stride, out, (unsigned)total, FastDiv((uint32_t)inner), FastDiv((uint32_t)rows), alpha, beta, bias, relu);
+                              int rows, float alpha, float beta, const float* bias, int relu, hipStream_t stream,
+                              long long col0) {
+  // elements before the image that holds column col0 are not part of the reduction
+  const long long first = col0 > 0 ? (col0 / inner) * (long long)rows * inner : 0;
+  ProfScope prof("split_reduce", 4.0 * (double)(total - first) * (splits + 1), stream);
+  hipLaunchKernelGGL(split_reduce_nchw_kernel, dim3(stream_grid((size_t)(total - first), 256)), dim3(256), 0, stream, part,
+                     splits, stride, out, (unsigned)first, (unsigned)total, FastDiv((uint32_t)inner), FastDiv((uint32_t)rows),
+                     alpha, beta, bias, relu, (unsigned)col0);
 }
 
 // `splits` > 1: slices of the contraction write unblended partial results to `part`, then one reduction applies the
 // alpha / beta blend, bias and ReLU.
 template <class T>
 static int run_fwd_soff(const RowSParams& ap, const RowSParams& bp, EpiParams ep, int n_k, int k_true,
-                        hipStream_t stream, const char* tag, int splits = 1, float* part = nullptr) {
+                        hipStream_t stream, const char* tag, int splits = 1, float* part = nullptr,
+                        const TailSplit* tail = nullptr) {
   constexpr int AROWS = T::BM % 64 == 0 ? T::BM : (T::BM + 63) / 64 * 64;  // loader rows: a multiple of the wave
   typedef LoadRowS<AROWS, T::BK, T::NT, true> AL;
   typedef LoadRowS<T::BN, T::BK, T::NT, false> BL;
+  const long long total = (long long)ep.rows * ep.cols;
+  if (splits <= 1 && tail && tail->splits > 1) {
+    // whole tiles blend into y as usual; the sliced tail goes through `part` and one reduction over its columns
+    const EpiParams fin = ep;
+    ep.part = part; ep.split_stride = total;
+    ep.full_tiles = tail->full_tiles; ep.tail_tiles = tail->tail_tiles; ep.tail_splits = tail->splits;
+    if (int e = launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true)) return e;
+    launch_split_reduce_nchw(part, tail->splits, total, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta, fin.bias,
+                             fin.relu, stream, tail->col0);
+    return launch_status();
+  }
   if (splits <= 1) return launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
   const EpiParams fin = ep;
-  const long long total = (long long)ep.rows * ep.cols;
   ep.out = part; ep.split_stride = total;
   int used = 1;
   if (int e = launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, splits, &used, stream, tag, k_true)) return e;
@@ -211,13 +231,13 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
     if (flags & RH_MATH_BF16_MFMA_FP32ACC) return run_fwd_soff_bf16(ap, bp, ep, sp.n_k, CRS, stream);
     float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes + sp.img_bytes);
     switch (pick_bm(d.K)) {
-      case 128: return run_fwd_soff<T128x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_128x128", sp.splits, part);
-      case 96:  return run_fwd_soff<T96x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_96x128", sp.splits, part);
+      case 128: return run_fwd_soff<T128x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_128x128", sp.splits, part, &sp.tail);
+      case 96:  return run_fwd_soff<T96x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_96x128", sp.splits, part, &sp.tail);
       case 64:
         if (cdiv(d.K, 64) == 1 && prefer_k8_64(ep.cols))
-          return run_fwd_soff<T64x256k8>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x256k8", sp.splits, part);
-        return run_fwd_soff<T64x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x256", sp.splits, part);
-      default:  return run_fwd_soff<T32x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_32x256", sp.splits, part);
+          return run_fwd_soff<T64x256k8>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x256k8", sp.splits, part, &sp.tail);
+        return run_fwd_soff<T64x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x256", sp.splits, part, &sp.tail);
+      default:  return run_fwd_soff<T32x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_32x256", sp.splits, part, &sp.tail);
     }
   }
   const int n_tab = round_up(CRS, kTabPad);

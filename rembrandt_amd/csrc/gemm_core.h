@@ -431,6 +431,12 @@ struct LoadPixX {
 //   dense: out[i * ld + j]
 // value = alpha*acc + beta*old (+ bias[i]) (clamped at 0 if relu).  With split_stride != 0 the
 // block writes its partial sum, unblended, to out + split * split_stride (dense).
+//
+// Tail form (tail_tiles > 0, 1-D grid): the first full_tiles tiles of the logical order are computed whole and
+// blended into `out`; each of the last tail_tiles tiles is computed by tail_splits blocks over slices of the
+// contraction, which write unblended partial sums to part + slice * split_stride.  It evens out a grid whose tile
+// count is a little over a multiple of the CU count (676 tiles on 256 CUs: a quarter of the CUs would carry three
+// tiles, the rest two) without paying partial-sum traffic for the whole result.
 // ------------------------------------------------------------------------------------------
 struct EpiParams {
   float* out;
@@ -439,6 +445,8 @@ struct EpiParams {
   int rows, cols, inner, ld;
   int relu;
   long long split_stride;
+  float* part = nullptr;
+  int full_tiles = 0, tail_tiles = 0, tail_splits = 0;
 };
 
 // Blocks are handed to the 8 XCDs round-robin by the hardware.  Renumber them so that every
@@ -458,8 +466,8 @@ template <class T, bool NCHW>
 __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], const EpiParams& ep, int m0, int n0,
                                            int wm, int wn, int lane, int split_idx) {
   constexpr int TM = T::TM, TN = T::TN;
-  const bool split = ep.split_stride != 0;
-  float* out = ep.out + (split ? (long long)split_idx * ep.split_stride : 0ll);
+  const bool split = split_idx >= 0;  // < 0: blend into the result
+  float* out = split ? (ep.tail_tiles > 0 ? ep.part : ep.out) + (long long)split_idx * ep.split_stride : ep.out;
   const float alpha = split ? 1.0f : ep.alpha;
   const float beta = split ? 0.0f : ep.beta;
   const int row_stride = NCHW ? ep.inner : ep.ld;
@@ -519,15 +527,36 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
 
   // Blocks of the whole grid (tiles x splits, x fastest) are dealt to the 8 XCDs round-robin; remap so that
   // each XCD's L2 sees a contiguous range of (split, tile): all tiles of a split read the same K range.
-  const int tiles = gridDim.x;
-  const int linear = xcd_remap(blockIdx.y * tiles + blockIdx.x, tiles * gridDim.y);
-  const int split_idx = __builtin_amdgcn_readfirstlane(linear / tiles);
-  const int logical = __builtin_amdgcn_readfirstlane(linear - split_idx * tiles);
+  int slice, logical, dst_split;  // slice of the contraction, tile, and where the result goes (< 0: blended into out)
+  if (ep.tail_tiles > 0) {
+    const int b = blockIdx.x;
+    if (b < ep.full_tiles) {
+      logical = xcd_remap(b, ep.full_tiles);
+      slice = 0;
+      dst_split = -1;
+    } else {
+      const int r = xcd_remap(b - ep.full_tiles, ep.tail_tiles * ep.tail_splits);
+      slice = r / ep.tail_tiles;
+      logical = ep.full_tiles + (r - slice * ep.tail_tiles);
+      dst_split = slice;
+    }
+  } else {
+    const int tiles = gridDim.x;
+    const int linear = xcd_remap(blockIdx.y * tiles + blockIdx.x, tiles * gridDim.y);
+    slice = linear / tiles;
+    logical = linear - slice * tiles;
+    dst_split = ep.split_stride != 0 ? slice : -1;
+  }
+  slice = __builtin_amdgcn_readfirstlane(slice);
+  logical = __builtin_amdgcn_readfirstlane(logical);
+  dst_split = __builtin_amdgcn_readfirstlane(dst_split);
   const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  const int c_begin = split_idx * chunks_per_split;
-  int c_end = c_begin + chunks_per_split;
+  // whole tiles of the tail form cover the full contraction; every other block covers its slice
+  const bool whole = ep.tail_tiles > 0 && dst_split < 0;
+  const int c_begin = whole ? 0 : slice * chunks_per_split;
+  int c_end = whole ? k_chunks : c_begin + chunks_per_split;
   if (c_end > k_chunks) c_end = k_chunks;
   const int nk = c_end - c_begin;
 
@@ -627,7 +656,7 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
   for (int it = 0; it + 1 < nk; ++it) k_step(it, std::true_type());
   if (nk > 0) k_step(nk - 1, std::false_type());
 
-  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, split_idx);
+  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, dst_split);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -735,7 +764,7 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_kernel(typename 
   for (int it = 0; it + 1 < nk; ++it) k_step(it, std::true_type());
   if (nk > 0) k_step(nk - 1, std::false_type());
 
-  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, split_idx);
+  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, ep.split_stride != 0 ? split_idx : -1);
 }
 
 }  // namespace rh

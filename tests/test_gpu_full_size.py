@@ -45,6 +45,8 @@ FULL_CONV = {
     "resnet_7_512": (64, 512, 7, 7, 512, 3, 1, 1),
     "resnet_down_512": (64, 256, 14, 14, 512, 3, 2, 1),
     "resnet_proj_128": (64, 64, 56, 56, 128, 1, 2, 0),
+    # 784 tiles on 256 CUs: the last 16 tiles are cut into slices (as are the last 164 of alexnet_conv5's 676)
+    "resnet_14_256_b256": (256, 256, 14, 14, 256, 3, 1, 1),
 }
 
 
