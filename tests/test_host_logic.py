@@ -145,6 +145,31 @@ def test_reference_example_files():
         SequentialOperatorConfig.from_model_file(os.path.join(REF_EXAMPLES, "imagenet_alexnet.model"))
 
 
+def test_resnet18_template_and_bnorm_builders():
+    """The ResNet-18 template (src/templates/resnet.rs:367-520): operator sequence, extents, and the parameter count
+    the reference's params_len formulas give (filter + 4 per batch-norm channel; conv.rs:97-103, 926-934, 2197-2207)."""
+    dims, layers, ncat = configs.resnet18()
+    assert dims == (224, 224, 3) and ncat == 1000
+    assert [l[0] for l in layers] == ["bnorm_conv2d", "pool2d"] + ["stack_res_conv2d"] * 2 + \
+        ["proj_stack_res_conv2d", "stack_res_conv2d"] * 3 + ["pool2d", "affine"]
+    assert [l[2] for l in layers if l[0] == "proj_stack_res_conv2d"] == [(28, 28, 128), (14, 14, 256), (7, 7, 512)]
+    assert layers[1][1] == (112, 112, 64) and layers[2][1] == (56, 56, 64) and layers[-1][1] == 512
+    want = (7 * 7 * 3 * 64 + 4 * 64) + 512 * 1000 + 1000
+    for c in (64, 128, 256, 512):
+        want += (2 if c == 64 else 1) * 2 * (9 * c * c + 4 * c)                  # plain residual units
+        if c > 64:
+            want += 9 * (c // 2) * c + 9 * c * c + (c // 2) * c + 12 * c        # the projecting unit in front of them
+    assert configs.build_config(configs.resnet18()).params_len() == want == 11699112
+    with pytest.raises(Panic):   # the output extent must equal or halve the input extent
+        SequentialOperatorConfig().proj_stack_res_conv2d((28, 28, 64), (9, 9, 128))
+    with pytest.raises(Panic):
+        SequentialOperatorConfig().bnorm_conv2d((8, 8, 3), 3, 1, 1, 4, bnorm_epsilon=0.0)
+    with pytest.raises(KeyError):
+        SequentialOperatorConfig().stack_res_conv2d((8, 8, 4), bnorm_mov_avg="Median")
+    cfg = SequentialOperatorConfig().data3d((8, 8, 3)).bnorm_conv2d((8, 8, 3), 3, 2, 1, 4, "Cumulative").stack_res_conv2d((4, 4, 4))
+    assert cfg.params_len() == (27 * 4 + 16) + 2 * (9 * 16 + 16)
+
+
 def test_builder_preconditions():
     with pytest.raises(Panic):
         SequentialOperatorConfig().conv2d((8, 8, 1), 3, 0, 1, 4)       # stride 0
