@@ -4,6 +4,12 @@ TEST INFRASTRUCTURE ONLY: imported by the tests, by the smoke check and by the b
 baseline leg; the shipped package never imports it.  All arrays are C-contiguous numpy arrays
 in the layouts of the reference (NCHW activations, [K][C][R][S] filters, [out][in] affine
 weights, [batch][chan] affine activations).
+
+The numpy restatements further down (Data3d preprocessing, dropout, local response normalisation, spatial batch
+normalisation) are pinned by the CPU test-suite against torch CPU fp64 routines and their autograd.  Parity unpinned
+against the reference itself, whose kernels for these live outside its tree: the dropout comparison (`>` taken,
+not `>=`), the LRN arithmetic (the reference's layer is a stub; the published formula its parameters name), and what
+the batch-norm buffer `bn_running_ivar` accumulates (taken: the moving average of 1/sqrt(var + epsilon)).
 """
 import ctypes as C
 import os
