@@ -127,6 +127,8 @@ def main():
     ap.add_argument("--workload", default="alexnet", choices=sorted(BATCH))
     ap.add_argument("--cpu-sample", type=int, default=512, help="images in the CPU baseline step (0 = skip; 512 is about 15 s on 16 cores)")
     ap.add_argument("--unfused", action="store_true", help="reference-style K1->K2->K3 and BLAS-1 SGD sequence")
+    ap.add_argument("--graph", action="store_true",
+                    help="record each train step into a HIP graph and replay it (for the launch-bound small networks)")
     ap.add_argument("--no-overlap", action="store_true",
                     help="conv filter / bias gradients on the main stream instead of the second stream")
     ap.add_argument("--no-kernel-events", action="store_true",
@@ -155,7 +157,8 @@ def main():
     seed = NUM_CLASSES_SEED + 4
     cfg = configs.build_config(net)
     worker = SequentialOperatorWorker(cfg, batch, "Backward", shared_seed=(seed, seed + 1), device=0,
-                                      fuse_epilogue=not args.unfused, overlap_backward=not args.no_overlap)
+                                      fuse_epilogue=not args.unfused, overlap_backward=not args.no_overlap,
+                                      graph_steps=args.graph)
     worker.init_params()
     x = synth.normal(seed, 100, (batch, dims[2], dims[1], dims[0]))
     labels = synth.integers(seed, 200, (batch,), ncat)
@@ -241,7 +244,8 @@ def main():
         "config": {"workload": "%s-shaped train step (fwd+bwd+SGD momentum 0.9), batch %d, fp32, input %dx%dx%d N(0,1), "
                                "weights N(0,0.01), %s%s" % (args.workload, batch, dims[2], dims[1], dims[0],
                                                             "unfused reference sequence" if args.unfused else "fused epilogues",
-                                                            "" if args.no_overlap else ", two-stream backward"),
+                                                            ("" if args.no_overlap else ", two-stream backward") +
+                                                            (", steps replayed as a HIP graph" if args.graph else "")),
                    "global_batch": batch, "params": cfg.params_len(), "gemm_gflop_per_step": gemm_flops / 1e9},
         "roofline": None if dom is None else
                     {"bound": dom["bound"], "kernel": dom["kernel"], "achieved": dom["achieved"], "peak": dom["peak"],

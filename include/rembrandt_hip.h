@@ -72,6 +72,17 @@ int rh_ctx_sync(rh_ctx* ctx);                       /* both streams */
 rh_stream_t rh_ctx_aux_stream(rh_ctx* ctx);
 int rh_ctx_fork(rh_ctx* ctx);
 int rh_ctx_join(rh_ctx* ctx);
+/* Stream capture (no counterpart in the reference, which launches every kernel of every step from the host): between
+ * rh_ctx_begin_capture and rh_ctx_end_capture the launches made on the context's streams are recorded into a HIP graph
+ * instead of executed; rh_graph_launch replays the recording on the main stream.  For launch-bound sequences (a whole
+ * train step of a LeNet-sized network is ~60 launches of a few microseconds).  Only kernel launches and
+ * device-to-device copies may be recorded: calls that copy to or from the host, synchronise, allocate or memset return
+ * an error or break the recording.  rh_ctx_end_capture(ctx, NULL) discards a recording. */
+typedef struct rh_graph rh_graph;
+int rh_ctx_begin_capture(rh_ctx* ctx);
+int rh_ctx_end_capture(rh_ctx* ctx, rh_graph** out);
+int rh_graph_launch(rh_graph* g, rh_ctx* ctx);
+int rh_graph_destroy(rh_graph* g);
 int rh_malloc(rh_ctx* ctx, size_t bytes, void** dptr); /* zero-filled, like DeviceBuffer::zeros */
 int rh_free(rh_ctx* ctx, void* dptr);
 int rh_memset_f32(float* d, float value, size_t n, rh_stream_t stream);
@@ -298,6 +309,7 @@ int rh_rng_fill_uniform01_device(uint64_t seed, uint64_t stream_id, uint64_t fir
  * MFMA contractions, bytes for the bandwidth-bound kernels), elapsed milliseconds}.
  * ------------------------------------------------------------------------------------------- */
 int rh_profile_enable(int on);
+int rh_profile_enabled(void);
 /* Record only launches whose tag starts with `prefix` (NULL or "" = all).  Set it while disabled. */
 int rh_profile_filter(const char* prefix);
 int rh_profile_count(void);

@@ -101,9 +101,18 @@ int rho_config_from_model_file(const char* path, rho_config** out);
 #define RHO_EXEC_FUSE_EPILOGUE 0x1
 #define RHO_EXEC_BF16_FORWARD  0x2
 #define RHO_EXEC_OVERLAP_BACKWARD 0x4
+/*   RHO_EXEC_GRAPH_STEPS    rho_sgd_train_batch records a whole step (forward, loss kernels, backward, update) into a HIP
+ *                           graph the second time it sees a (batch size, optimizer scalars) combination and replays it
+ *                           from then on: one launch per step instead of ~60 for a LeNet-sized network.  Steps whose
+ *                           launch arguments change every step (random input preprocessing, dropout, a cumulative
+ *                           batch-norm average, a step-size schedule at a boundary) run launch by launch as usual;
+ *                           results are bit-identical either way. */
+#define RHO_EXEC_GRAPH_STEPS 0x8
 int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1,
                    int device, int exec_flags, rho_worker** out);
 int rho_worker_free(rho_worker* w);
+/* Number of rho_sgd_train_batch calls on this worker that ran as one graph launch (RHO_EXEC_GRAPH_STEPS). */
+int rho_worker_graph_launches(rho_worker* w, int64_t* out);
 /* Run-time switch of RHO_EXEC_OVERLAP_BACKWARD for a worker built with it (per-kernel timings are only meaningful
  * with it off: kernels that share the GPU stretch each other's durations). */
 int rho_worker_set_overlap_backward(rho_worker* w, int on);

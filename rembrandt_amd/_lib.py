@@ -59,6 +59,11 @@ PROTOTYPES = {
     "rh_rng_fill_uniform01_device": (_int, [C.c_uint64, C.c_uint64, C.c_uint64, _vp, _sz, _vp]),
     "rh_lrn_fwd": (_int, [C.POINTER(LrnGeom), _vp, _vp, _vp, _vp]),
     "rh_lrn_bwd": (_int, [C.POINTER(LrnGeom), _vp, _vp, _vp, _vp, _vp, _vp]),
+    "rh_ctx_begin_capture": (_int, [_vp]),
+    "rh_ctx_end_capture": (_int, [_vp, C.POINTER(_vp)]),
+    "rh_graph_launch": (_int, [_vp, _vp]),
+    "rh_graph_destroy": (_int, [_vp]),
+    "rh_profile_enabled": (_int, []),
     "rh_bnorm_workspace_bytes": (_sz, [_int, _int, _int]),
     "rh_bnorm_fwd_train": (_int, [_int, _int, _int, _f, _vp, _f, _vp, C.c_double, C.c_double, _vp, _vp, _vp, _vp, _vp, _vp,
                                   _vp, _sz, _int, _vp]),

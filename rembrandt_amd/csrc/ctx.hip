@@ -18,6 +18,14 @@ struct rh_ctx {
   // that order the streams against each other
   hipStream_t aux = nullptr;
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  bool aux_dirty = false;   // the second stream was given work (fork) that the main stream has not waited for yet
+  bool capturing = false;   // between rh_ctx_begin_capture and rh_ctx_end_capture
+};
+
+// A captured and instantiated sequence of launches of one context (both streams).
+struct rh_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
 };
 
 using namespace rh;
@@ -90,6 +98,7 @@ extern "C" rh_stream_t rh_ctx_aux_stream(rh_ctx* ctx) {
     }
     ctx->aux = s; ctx->ev_fork = a; ctx->ev_join = b;
   }
+  ctx->aux_dirty = true;  // whoever asked for the stream may put work on it
   return (rh_stream_t)ctx->aux;
 }
 
@@ -98,16 +107,76 @@ extern "C" int rh_ctx_fork(rh_ctx* ctx) {
   if (!ctx || !rh_ctx_aux_stream(ctx)) return RH_E_INVALID;
   hipError_t e = hipEventRecord(ctx->ev_fork, ctx->stream);
   if (e != hipSuccess) return (int)e;
+  ctx->aux_dirty = true;
   return (int)hipStreamWaitEvent(ctx->aux, ctx->ev_fork, 0);
 }
 
 // Work enqueued on the main stream after this call runs after everything the second stream holds now.
 extern "C" int rh_ctx_join(rh_ctx* ctx) {
   if (!ctx) return RH_E_INVALID;
-  if (!ctx->aux) return 0;
+  if (!ctx->aux || !ctx->aux_dirty) return 0;  // nothing was forked since the last join
   hipError_t e = hipEventRecord(ctx->ev_join, ctx->aux);
   if (e != hipSuccess) return (int)e;
+  ctx->aux_dirty = false;
   return (int)hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0);
+}
+
+// ---- stream capture: a launch-bound sequence (a whole train step of a small network) recorded once and replayed ----
+// Between begin and end every launch on the context's streams is recorded instead of executed; the second stream
+// joins the recording through rh_ctx_fork and must have been joined again (rh_ctx_join) before the end.  Only kernel
+// launches and device-to-device copies may be recorded: no host copies, synchronisation, allocation or memset calls.
+extern "C" int rh_ctx_begin_capture(rh_ctx* ctx) {
+  if (!ctx || ctx->capturing) return RH_E_INVALID;
+  if (ctx->aux_dirty) {  // work forked before the recording must not leak into it
+    if (int e = rh_ctx_join(ctx)) return e;
+  }
+  hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
+  if (e != hipSuccess) return (int)e;
+  ctx->capturing = true;
+  return 0;
+}
+
+// Ends the recording; with `out` the graph is instantiated and returned, without it the recording is discarded
+// (the way out of a sequence that failed half-way).
+extern "C" int rh_ctx_end_capture(rh_ctx* ctx, rh_graph** out) {
+  if (!ctx || !ctx->capturing) return RH_E_INVALID;
+  ctx->capturing = false;
+  if (out) *out = nullptr;
+  hipGraph_t g = nullptr;
+  hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+  ctx->aux_dirty = false;
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return (int)e;
+  }
+  if (!out) {
+    if (g) (void)hipGraphDestroy(g);
+    return 0;
+  }
+  hipGraphExec_t x = nullptr;
+  e = hipGraphInstantiate(&x, g, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(g);
+    return (int)e;
+  }
+  rh_graph* r = new rh_graph;
+  r->graph = g;
+  r->exec = x;
+  *out = r;
+  return 0;
+}
+
+extern "C" int rh_graph_launch(rh_graph* g, rh_ctx* ctx) {
+  if (!g || !ctx || ctx->capturing) return RH_E_INVALID;
+  return (int)hipGraphLaunch(g->exec, ctx->stream);
+}
+
+extern "C" int rh_graph_destroy(rh_graph* g) {
+  if (!g) return RH_E_INVALID;
+  hipError_t e = hipGraphExecDestroy(g->exec);
+  hipError_t e2 = hipGraphDestroy(g->graph);
+  delete g;
+  return (int)(e != hipSuccess ? e : e2);
 }
 
 extern "C" int rh_malloc(rh_ctx* ctx, size_t bytes, void** dptr) {
@@ -190,6 +259,8 @@ ProfScope::~ProfScope() {
 }
 
 }  // namespace rh
+
+extern "C" int rh_profile_enabled(void) { return rh::g_profile_enabled ? 1 : 0; }
 
 extern "C" int rh_profile_enable(int on) {
   rh::g_profile_enabled = on != 0;

@@ -1,7 +1,11 @@
 // C ABI of the operator / graph / optimizer layer (include/rembrandt_operator.h).
 #include <cstdio>
 #include <memory>
+#include <cstring>
+#include <map>
+#include <set>
 #include <string>
+#include <tuple>
 #include <vector>
 #include <algorithm>
 
@@ -13,9 +17,34 @@
 using namespace rembrandt;
 
 struct rho_config { SequentialOperatorConfig cfg; };
+// What makes two train steps the same sequence of launches with the same arguments.
+struct StepKey {
+  size_t batch;
+  int fused, momentum_kind;
+  uint32_t step_size_bits, l2_bits, mu_bits;
+  bool first_iter;  // the Nesterov un-apply is skipped at iteration 0
+  bool operator<(const StepKey& o) const {
+    return std::tie(batch, fused, momentum_kind, step_size_bits, l2_bits, mu_bits, first_iter) <
+           std::tie(o.batch, o.fused, o.momentum_kind, o.step_size_bits, o.l2_bits, o.mu_bits, o.first_iter);
+  }
+};
+
 struct rho_worker {
   std::shared_ptr<DeviceContext> ctx;
   std::unique_ptr<SequentialOperatorWorker> worker;
+  bool graph_steps = false;
+  int64_t graph_launches = 0;                // steps that ran as a graph launch
+  std::map<StepKey, rh_graph*> step_graphs;  // recorded steps
+  std::set<StepKey> seen_steps;              // combinations that ran once launch by launch
+  void drop_graphs() {
+    for (auto& kv : step_graphs) (void)rh_graph_destroy(kv.second);
+    step_graphs.clear();
+    seen_steps.clear();
+  }
+  ~rho_worker() {
+    if (ctx) (void)rh_ctx_sync(ctx->raw());
+    drop_graphs();
+  }
 };
 struct rho_sgd { std::unique_ptr<SgdOpt> opt; };
 struct rho_dataset { std::unique_ptr<DataSource> src; };
@@ -235,6 +264,8 @@ int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, ui
     opts.fuse_epilogue = (exec_flags & RHO_EXEC_FUSE_EPILOGUE) != 0;
     opts.bf16_forward = (exec_flags & RHO_EXEC_BF16_FORWARD) != 0;
     opts.overlap_backward = (exec_flags & RHO_EXEC_OVERLAP_BACKWARD) != 0;
+    opts.graph_steps = (exec_flags & RHO_EXEC_GRAPH_STEPS) != 0;
+    w->graph_steps = opts.graph_steps;
     w->worker.reset(new SequentialOperatorWorker(cfg->cfg, (size_t)batch_size,
                                                  capability == RHO_CAP_FORWARD ? OpCapability::Forward : OpCapability::Backward,
                                                  seed, w->ctx, opts));
@@ -242,7 +273,15 @@ int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, ui
   })
 }
 int rho_worker_free(rho_worker* w) { RHO_TRY({ delete w; }) }
-int rho_worker_set_overlap_backward(rho_worker* w, int on) { RHO_TRY({ RHO_REQ(w); w->worker->set_overlap_backward(on != 0); }) }
+int rho_worker_set_overlap_backward(rho_worker* w, int on) {
+  RHO_TRY({
+    RHO_REQ(w);
+    w->ctx->sync();
+    w->drop_graphs();  // recorded steps carry the old placement
+    w->worker->set_overlap_backward(on != 0);
+  })
+}
+int rho_worker_graph_launches(rho_worker* w, int64_t* out) { RHO_TRY({ RHO_REQ(w && out); *out = w->graph_launches; }) }
 int rho_worker_hidden_count(rho_worker* w, int32_t* out) { RHO_TRY({ RHO_REQ(w && out); *out = (int32_t)w->worker->hidden_count(); }) }
 int rho_worker_op_kind(rho_worker* w, int32_t hidden_idx, const char** out) { RHO_TRY({ RHO_REQ(out); *out = op_at(w, hidden_idx)->kind(); }) }
 void* rho_worker_stream(rho_worker* w) { return w ? w->ctx->stream() : nullptr; }
@@ -437,19 +476,63 @@ int rho_sgd_iter_counter(rho_sgd* s, int64_t* out) { RHO_TRY({ RHO_REQ(s && out)
 int rho_sgd_step_size_at(rho_sgd* s, int64_t t, float* out) {
   RHO_TRY({ RHO_REQ(s && out && t >= 0); *out = s->opt->config().step_size.at_iter((size_t)t); })
 }
+static uint32_t float_bits(float v) {
+  uint32_t u;
+  std::memcpy(&u, &v, sizeof u);
+  return u;
+}
+
 int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused, float* loss_out, int32_t* correct_out) {
   RHO_TRY({
     RHO_REQ(s && w && batch_size > 0);
     SequentialOperatorWorker* op = w->worker.get();
     const size_t b = (size_t)batch_size;
+    const size_t t = s->opt->iter_counter();
+    const OpPhase phase = OpPhase::Training(t);
     // forward -> arg-max and loss kernels -> backward -> update are all enqueued before the two read-backs, so
     // the GPU works through the step without waiting for the host (same results as the reference's order:
     // store_output_categories, store_loss, backward; nothing in between writes what they read)
-    op->forward(b, OpPhase::Training(s->opt->iter_counter()));
-    op->loss_operator(0)->enqueue_output_categories(b);
-    op->loss_operator(0)->enqueue_loss(b);
-    op->backward(b);
-    s->opt->step(op, fused != 0);
+    auto enqueue_step = [&]() {
+      op->forward(b, phase);
+      op->loss_operator(0)->enqueue_output_categories(b);
+      op->loss_operator(0)->enqueue_loss(b);
+      op->backward(b);
+      s->opt->step(op, fused != 0);
+    };
+    bool done = false;
+    if (w->graph_steps && !rh_profile_enabled() && op->graph_safe(phase)) {
+      const SgdOptConfig& c = s->opt->config();
+      const StepKey key = {b, fused != 0 ? 1 : 0, (int)c.momentum.kind, float_bits(c.step_size.at_iter(t)),
+                           float_bits(c.l2_reg_coef), float_bits(c.momentum.mu), t == 0};
+      auto it = w->step_graphs.find(key);
+      if (it != w->step_graphs.end()) {
+        w->ctx->launch(it->second);
+        s->opt->set_iter_counter(t + 1);  // what step() does on the host
+        w->graph_launches += 1;
+        done = true;
+      } else if (w->seen_steps.count(key)) {
+        // second time: record.  (The first time ran launch by launch, which also created everything that is made on
+        // first use: the second stream, kernel attributes.)
+        op->settle();
+        w->ctx->begin_capture();
+        try {
+          enqueue_step();
+          op->settle();  // updates issued on the second stream rejoin the recording
+        } catch (...) {
+          w->ctx->abort_capture();
+          s->opt->set_iter_counter(t);
+          throw;
+        }
+        rh_graph* g = w->ctx->end_capture();
+        w->step_graphs[key] = g;
+        w->ctx->launch(g);  // nothing ran while recording; step() already advanced the iteration counter
+        w->graph_launches += 1;
+        done = true;
+      } else {
+        w->seen_steps.insert(key);
+      }
+    }
+    if (!done) enqueue_step();
     op->loss_operator(0)->fetch_output_categories(b);
     const float loss = op->loss_operator(0)->fetch_loss();
     const size_t correct = op->loss_operator(0)->accuracy_count(b);

@@ -33,6 +33,14 @@ rh_stream_t DeviceContext::aux_stream() const {
 }
 void DeviceContext::fork() const { unwrap(rh_ctx_fork(ctx_), "rh_ctx_fork"); }
 void DeviceContext::join() const { unwrap(rh_ctx_join(ctx_), "rh_ctx_join"); }
+void DeviceContext::begin_capture() const { unwrap(rh_ctx_begin_capture(ctx_), "rh_ctx_begin_capture"); }
+rh_graph* DeviceContext::end_capture() const {
+  rh_graph* g = nullptr;
+  unwrap(rh_ctx_end_capture(ctx_, &g), "rh_ctx_end_capture");
+  return g;
+}
+void DeviceContext::abort_capture() const { (void)rh_ctx_end_capture(ctx_, nullptr); }
+void DeviceContext::launch(rh_graph* g) const { unwrap(rh_graph_launch(g, ctx_), "rh_graph_launch"); }
 
 // ---- configs ----------------------------------------------------------------------------------------
 static size_t out_dim_floor(size_t in, size_t size, size_t stride, size_t pad) {
@@ -550,6 +558,13 @@ class Data3dOperator : public InputOperator {
     return true;
   }
   const char* kind() const override { return "Data3dOperator"; }
+  // random crops, flips and lighting noise draw new launch arguments for every training batch
+  bool graph_safe(OpPhase phase) const override {
+    if (!phase.training) return true;
+    for (const auto& p : config_.preprocs)
+      if (p.kind != Data3dPreproc::SubtractElemwiseMean) return false;
+    return true;
+  }
 
  private:
   struct PreprocState {
@@ -906,6 +921,7 @@ class DropoutOperator : public Operator {
     *seed = seed_; *stream_id = stream_id_; *first = last_first_;
   }
   const char* kind() const override { return "DropoutOperator"; }
+  bool graph_safe(OpPhase phase) const override { return !phase.training; }  // a new piece of the uniform stream per step
 
  private:
   size_t batch_cap_;
@@ -1288,6 +1304,7 @@ class BNormUnitsOperator : public Operator {
   Ctx context_;
   ExecOptions opts_;
   ParamsInit init_weights_ = ParamsInit::MakeDisabled();
+  BNormMovingAverage mov_avg_ = BNormMovingAverage::MakeCumulative();
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   std::unique_ptr<DeviceBuffer<float>> mid_act_, mid_delta_;
   std::unique_ptr<DeviceBuffer<uint8_t>> workspace_, workspace_aux_;
@@ -1295,6 +1312,11 @@ class BNormUnitsOperator : public Operator {
 
  public:
   void set_overlap_backward(bool on) override { overlap_on_ = on; }
+  // the weight of the newest batch in the moving statistics is a launch argument: constant only for the exponential
+  // average after its first step
+  bool graph_safe(OpPhase phase) const override {
+    return !phase.training || (mov_avg_.kind == BNormMovingAverage::Exponential && phase.t > 0);
+  }
 };
 
 // ---- BNormConv2dOperator (src/operator/conv.rs:106-912) ---------------------------------------------------
@@ -1305,6 +1327,7 @@ class BNormConv2dOperator : public BNormUnitsOperator {
       : BNormUnitsOperator(batch_size, 1, prev_op, context, opts, "BNormConv2dOperator"), config_(config) {
     RB_ASSERT(in_act_->len() >= config.in_dims.len() * batch_size);
     init_weights_ = config.init_weights;
+    mov_avg_ = config.bnorm_mov_avg;
     units_[0].alloc(batch_size, config.in_dims, config.conv_size, config.conv_stride, config.conv_pad, config.out_channels,
                     backward_enabled(capability), context);
     alloc_common(units_[0].out_dims, backward_enabled(capability));
@@ -1347,6 +1370,7 @@ class StackResConv2dOperator : public BNormUnitsOperator {
       : BNormUnitsOperator(batch_size, 2, prev_op, context, opts, "StackResConv2dOperator"), config_(config) {
     RB_ASSERT(in_act_->len() >= config.in_dims.len() * batch_size);
     init_weights_ = config.init_weights;
+    mov_avg_ = config.bnorm_mov_avg;
     const bool bwd = backward_enabled(capability);
     for (auto& u : units_) u.alloc(batch_size, config.in_dims, 3, 1, 1, config.in_dims.c, bwd, context);
     alloc_common(config.in_dims, bwd);
@@ -1397,6 +1421,7 @@ class ProjStackResConv2dOperator : public BNormUnitsOperator {
       : BNormUnitsOperator(batch_size, 3, prev_op, context, opts, "ProjStackResConv2dOperator"), config_(config) {
     RB_ASSERT(in_act_->len() >= config.in_dims.len() * batch_size);
     init_weights_ = config.init_weights;
+    mov_avg_ = config.bnorm_mov_avg;
     const Dims3 in = config.in_dims, out = config.out_dims;
     size_t stride;
     if (in.w == out.w && in.h == out.h) stride = 1;
@@ -1642,6 +1667,12 @@ void SequentialOperatorWorker::update_params2(float g, float u) { settle(); for 
 void SequentialOperatorWorker::save_params() { settle(); for (auto& op : hidden_ops_) op->save_params(); }
 void SequentialOperatorWorker::restore_params() { settle(); for (auto& op : hidden_ops_) op->restore_params(); }
 void SequentialOperatorWorker::reset() { settle(); for (auto& op : hidden_ops_) op->reset(); }
+bool SequentialOperatorWorker::graph_safe(OpPhase phase) const {
+  if (!input_op_->graph_safe(phase) || !loss_op_->graph_safe(phase)) return false;
+  for (const auto& op : hidden_ops_)
+    if (!op->graph_safe(phase)) return false;
+  return true;
+}
 void SequentialOperatorWorker::set_overlap_backward(bool on) {
   settle();
   context_->join();

@@ -47,6 +47,11 @@ class DeviceContext {
   rh_stream_t aux_stream() const;  // second stream for launches that may overlap the main one
   void fork() const;               // aux waits for main
   void join() const;               // main waits for aux
+  // Recording of the launches made on both streams into a replayable graph (rh_ctx_begin_capture / _end_capture).
+  void begin_capture() const;
+  rh_graph* end_capture() const;   // instantiated recording
+  void abort_capture() const;      // discards the recording (after a failure inside it)
+  void launch(rh_graph* g) const;
   rh_ctx* raw() const { return ctx_; }
   void sync() const;
 
@@ -245,6 +250,10 @@ struct OperatorConfig {
 // How kernels are scheduled inside the operators.  Both modes produce the same buffers at every
 // point where the reference's operators expose them.
 struct ExecOptions {
+  // A whole train step (forward, loss kernels, backward, update) recorded once per (batch size, step scalars) and
+  // replayed as one graph launch: for launch-bound networks.  Steps whose launch arguments change from one step to
+  // the next (random preprocessing, dropout streams, a cumulative batch-norm average) run launch by launch.
+  bool graph_steps = false;
   bool fuse_epilogue = true;  // conv bias + ReLU in the conv epilogue instead of K1 -> K2 -> K3
   bool bf16_forward = false;  // conv forward on bf16-rounded operands with fp32 accumulation (inference mode)
   // Conv backward: filter and bias gradients on the context's second stream beside the data gradient on the
@@ -284,6 +293,9 @@ class Operator {
   // next forward pass needs late: the affine layers) says so; the worker then joins the streams before that
   // operator's next forward and before anything else touches parameters.
   virtual bool updates_on_second_stream() const { return false; }
+  // Whether forward / backward in this phase make the same launches with the same arguments every step, so that a
+  // recording of one step can stand for the next.
+  virtual bool graph_safe(OpPhase /*phase*/) const { return true; }
   // Parameter / optimizer-state blobs: a sequence of serialised NdArrays (weights then bias; for the state the
   // momentum buffers).  decode_* return the number of bytes consumed (src/operator/mod.rs:1008-1073).
   virtual void encode_params(std::vector<uint8_t>& /*blob*/) {}
@@ -387,6 +399,7 @@ class SequentialOperatorWorker : public Operator {
   void reset() override;
   void fused_sgd_step(float l2, float scale, float momentum, float apply) override;
   void set_overlap_backward(bool on) override;
+  bool graph_safe(OpPhase phase) const override;
   // Joins the second stream if parameter updates are still in flight on it (called by every method but forward,
   // which joins lazily in front of the first operator concerned).
   void settle();

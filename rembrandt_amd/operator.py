@@ -48,6 +48,7 @@ PROTOTYPES = {
     "rho_config_new": (_int, [_P(_vp)]),
     "rho_config_free": (_int, [_vp]),
     "rho_config_data3d": (_int, [_vp, _i32, _i32, _i32, _int]),
+    "rho_worker_graph_launches": (_int, [_vp, _P(_i64)]),
     "rho_config_conv2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _int, _int, _f]),
     "rho_config_bnorm_conv2d": (_int, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _int, C.c_double, C.c_double, _int, _int, _f]),
     "rho_config_stack_res_conv2d": (_int, [_vp, _i32, _i32, _i32, _int, C.c_double, C.c_double, _int, _int, _f]),
@@ -281,11 +282,12 @@ class SequentialOperatorWorker:
     """src/operator/worker.rs:230-477 plus the Input/Loss operator calls the optimizer makes on it."""
 
     def __init__(self, config, batch_size, capability="Backward", shared_seed=(1, 2), device=0, fuse_epilogue=True,
-                 bf16_forward=False, overlap_backward=True):
+                 bf16_forward=False, overlap_backward=True, graph_steps=False):
+        """graph_steps: SgdOpt.train_batch records a whole step into a HIP graph and replays it (launch-bound networks)."""
         h = _vp()
+        flags = (1 if fuse_epilogue else 0) | (2 if bf16_forward else 0) | (4 if overlap_backward else 0) | (8 if graph_steps else 0)
         _chk(lib().rho_worker_new(config._h, batch_size, 0 if capability == "Forward" else 1, shared_seed[0],
-                                  shared_seed[1], device, (1 if fuse_epilogue else 0) | (2 if bf16_forward else 0) | (4 if overlap_backward else 0),
-                                  C.byref(h)))
+                                  shared_seed[1], device, flags, C.byref(h)))
         self._h = h
         self.batch_size = batch_size
         self.shared_seed = tuple(shared_seed)
@@ -296,6 +298,11 @@ class SequentialOperatorWorker:
             self._h = None
 
     __del__ = close
+
+    def graph_launches(self):
+        n = _i64()
+        _chk(lib().rho_worker_graph_launches(self._h, C.byref(n)))
+        return n.value
 
     def set_overlap_backward(self, on):
         _chk(lib().rho_worker_set_overlap_backward(self._h, int(on)))

@@ -27,6 +27,9 @@ pub struct rh_pool_geom {
 }
 
 #[repr(C)]
+pub struct rh_graph { _private: [u8; 0] }
+
+#[repr(C)]
 #[derive(Clone, Copy, Debug)]
 pub struct rh_lrn_geom {
   pub n: i32, pub c: i32, pub h: i32, pub w: i32,
@@ -115,6 +118,12 @@ extern "C" {
   pub fn rh_ctx_aux_stream(ctx: *mut rh_ctx) -> rh_stream_t;
   pub fn rh_ctx_fork(ctx: *mut rh_ctx) -> c_int;
   pub fn rh_ctx_join(ctx: *mut rh_ctx) -> c_int;
+
+  // Stream capture: launches between begin and end are recorded into a HIP graph; rh_graph_launch replays them.
+  pub fn rh_ctx_begin_capture(ctx: *mut rh_ctx) -> c_int;
+  pub fn rh_ctx_end_capture(ctx: *mut rh_ctx, out: *mut *mut rh_graph) -> c_int;
+  pub fn rh_graph_launch(g: *mut rh_graph, ctx: *mut rh_ctx) -> c_int;
+  pub fn rh_graph_destroy(g: *mut rh_graph) -> c_int;
 
   // Max-pool backward that also applies the ReLU backward mask of the operator below (one pass instead of two).
   pub fn rh_pool2d_bwd_relu_supported(g: *const rh_pool_geom) -> c_int;

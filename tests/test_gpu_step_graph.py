@@ -1,0 +1,106 @@
+"""Train steps recorded into a HIP graph and replayed (RHO_EXEC_GRAPH_STEPS) against the same steps launched kernel by
+kernel: losses, correct counts and every parameter and momentum buffer bit-identical after every step, over several
+replays with fresh inputs, with ordinary (non-recorded) work and synchronisation between the replays."""
+import numpy as np
+import pytest
+
+from rembrandt_amd import configs, synth
+from rembrandt_amd.operator import SequentialOperatorWorker, SgdOpt
+from conftest import say
+
+pytestmark = pytest.mark.gpu
+
+
+def param_buffers(net):
+    names = []
+    for i, l in enumerate(net[1]):
+        if l[0] in ("conv2d", "affine"):
+            names += [(i, b) for b in ("weights", "bias", "acc_grad_weights", "acc_grad_bias", "grad_weights")]
+        elif l[0] in ("bnorm_conv2d", "stack_res_conv2d", "proj_stack_res_conv2d"):
+            units = {"bnorm_conv2d": 1, "stack_res_conv2d": 2, "proj_stack_res_conv2d": 3}[l[0]]
+            for u in range(units):
+                names += [(i, "u%d.%s" % (u, b)) for b in ("weights", "bn_scale", "bn_bias", "bn_running_mean", "bn_running_ivar",
+                                                            "acc_grad_weights", "acc_bn_scale_grad")]
+    return names
+
+
+def run(net, batch, steps, graph, seed, sgd_kwargs, fused=True, toggle_at=None):
+    dims, layers, ncat = net
+    w = SequentialOperatorWorker(configs.build_config(net), batch, "Backward", shared_seed=(seed, seed + 1), graph_steps=graph)
+    w.init_params()
+    sgd = SgdOpt(batch, **sgd_kwargs)
+    sgd.begin(w)
+    names = param_buffers(net)
+    out = []
+    for step in range(steps):
+        if toggle_at is not None and step == toggle_at:
+            w.set_overlap_backward(False)
+        x = synth.normal(seed, 100 + step, (batch, dims[2], dims[1], dims[0]))
+        labels = synth.integers(seed, 200 + step, (batch,), ncat)
+        w.load_frames_f32(x)
+        w.stage_batch(labels, 1.0 / batch)
+        loss, correct = sgd.train_batch(w, batch, fused=fused)
+        # work outside the recording between two replays: blocking read-backs of every parameter buffer
+        out.append((loss, correct, [w.read(i, b).copy() for (i, b) in names]))
+    launches = w.graph_launches()
+    assert sgd.iter_counter() == steps
+    w.close()
+    return out, launches
+
+
+def same(a, b, tag):
+    assert len(a) == len(b)
+    for step, ((la, ca, pa), (lb, cb, pb)) in enumerate(zip(a, b)):
+        assert la == lb and ca == cb, "%s step %d: loss %r vs %r, correct %d vs %d" % (tag, step, la, lb, ca, cb)
+        for k, (u, v) in enumerate(zip(pa, pb)):
+            assert np.array_equal(u, v), "%s step %d: parameter buffer %d differs" % (tag, step, k)
+
+
+@pytest.mark.parametrize("name,batch,steps", [("lenet", 64, 8), ("cifar10", 128, 6)])
+def test_recorded_steps_equal_launched_steps(dev, name, batch, steps):
+    say("step graph", name)
+    net = configs.NETWORKS[name]()
+    kw = dict(step_size=0.01, momentum=("Update", 0.9), l2_reg_coef=5e-4)
+    eager, n0 = run(net, batch, steps, False, 0x6A01, kw)
+    graph, n1 = run(net, batch, steps, True, 0x6A01, kw)
+    assert n0 == 0
+    assert n1 == steps - 2, "iteration 0 and 1 are launched (first sight of their keys), iteration 2 records, the rest replay"
+    same(eager, graph, name)
+    assert not np.array_equal(graph[-1][2][0], graph[0][2][0]), "the replays did train"
+
+
+def test_recorded_steps_with_schedule_nesterov_and_placement_switch(dev):
+    """A step-size schedule (new scalars at its boundary: launched once, then recorded anew), the unfused Nesterov
+    update sequence, and a switch of the backward placement half-way (drops the recordings)."""
+    net = configs.lenet()
+    kw = dict(momentum=("UpdateNesterov", 0.9), l2_reg_coef=1e-4,
+              schedule={"kind": "Anneal1", "steps": [0.02, 0.005], "iters": [0, 5]})
+    eager, _ = run(net, 32, 12, False, 0x6A02, kw, fused=False, toggle_at=9)
+    graph, n = run(net, 32, 12, True, 0x6A02, kw, fused=False, toggle_at=9)
+    same(eager, graph, "lenet nesterov")
+    # keys: t=0 | t=1..4 (launch, record, replay x2) | t=5..8 (launch, record, replay x2) | after the switch t=9..11 (launch, record, replay)
+    assert n == 3 + 3 + 2
+
+
+def test_steps_that_cannot_be_recorded_are_launched(dev):
+    """Dropout draws a new piece of its random stream per step and a cumulative batch-norm average changes its weight
+    per step: such networks run launch by launch even with the flag, with the same results."""
+    dims = (12, 12, 3)
+    drop = (dims, *configs._chain(dims, [("conv", 3, 1, 1, 8, "Rect"), ("pool", 2, 2, 0, "Max"), ("dropout", 0.4), ("fc", 5, "Identity")]))
+    kw = dict(step_size=0.05, momentum=("Update", 0.9), l2_reg_coef=0.0)
+    eager, _ = run(drop, 16, 5, False, 0x6A03, kw)
+    graph, n = run(drop, 16, 5, True, 0x6A03, kw)
+    assert n == 0
+    same(eager, graph, "dropout net")
+
+
+def test_recorded_steps_of_a_batch_normalised_network(dev):
+    """Exponential moving average: constant launch arguments from iteration 1 on."""
+    dims = (16, 16, 3)
+    net = (dims, *configs._chain(dims, [("bnconv", 3, 1, 1, 8, "Rect"), ("pool", 2, 2, 0, "Max"), ("res", "Rect"),
+                                        ("projres", 16, 2, "Rect"), ("pool", 4, 1, 0, "Average"), ("fc", 5, "Identity")]))
+    kw = dict(step_size=0.05, momentum=("Update", 0.9), l2_reg_coef=1e-3)
+    eager, _ = run(net, 8, 7, False, 0x6A04, kw)
+    graph, n = run(net, 8, 7, True, 0x6A04, kw)
+    assert n == 7 - 2   # t=0 is not safe (first batch weighs 1), t=1 launched, t=2 records, the rest replay
+    same(eager, graph, "bnorm net")
