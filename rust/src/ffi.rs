@@ -8,6 +8,7 @@ use libc::{c_char, c_float, c_int, c_void, size_t};
 
 pub type rh_stream_t = *mut c_void; // hipStream_t
 pub enum rh_ctx {}
+pub enum rh_graph {}
 
 #[repr(C)]
 #[derive(Clone, Copy, Debug)]
@@ -25,9 +26,6 @@ pub struct rh_pool_geom {
   pub mode: i32,  // 0 max, 1 average (count includes padding)
   pub round: i32, // 0 floor (operator), 1 ceil (gen-1 layer)
 }
-
-#[repr(C)]
-pub struct rh_graph { _private: [u8; 0] }
 
 #[repr(C)]
 #[derive(Clone, Copy, Debug)]
