@@ -80,10 +80,47 @@ __global__ void split_reduce_kernel(const float* __restrict__ part, int splits, 
   }
 }
 
+// The same over a dense result (ld == cols) in 16-byte groups: the sums of each element are formed in the same order.
+__global__ __launch_bounds__(256) void split_reduce_vec_kernel(const float4* __restrict__ part, int splits, long long stride4,
+                                                               float4* __restrict__ out, unsigned total4, float alpha,
+                                                               float beta) {
+  const unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total4) return;
+  const float4 z = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  float4 a0 = z, a1 = z, a2 = z, a3 = z;
+  auto add = [](float4& a, const float4 v) { a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w; };
+  const float4* p = part + idx;
+  int s = 0;
+  for (; s + 3 < splits; s += 4) {
+    add(a0, p[(long long)s * stride4]);
+    add(a1, p[(long long)(s + 1) * stride4]);
+    add(a2, p[(long long)(s + 2) * stride4]);
+    add(a3, p[(long long)(s + 3) * stride4]);
+  }
+  for (; s < splits; ++s) add(a0, p[(long long)s * stride4]);
+  float4 v;
+  v.x = alpha * ((a0.x + a1.x) + (a2.x + a3.x));
+  v.y = alpha * ((a0.y + a1.y) + (a2.y + a3.y));
+  v.z = alpha * ((a0.z + a1.z) + (a2.z + a3.z));
+  v.w = alpha * ((a0.w + a1.w) + (a2.w + a3.w));
+  if (beta != 0.0f) {
+    const float4 o = out[idx];
+    v.x += beta * o.x; v.y += beta * o.y; v.z += beta * o.z; v.w += beta * o.w;
+  }
+  out[idx] = v;
+}
+
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
                          int ld, float alpha, float beta, hipStream_t stream) {
   const size_t total = (size_t)rows * cols;
   ProfScope prof("split_reduce", 4.0 * (double)total * (splits + 1), stream);
+  if (ld == cols && total % 4 == 0 && split_stride % 4 == 0 &&
+      ((reinterpret_cast<uintptr_t>(part) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+    hipLaunchKernelGGL(split_reduce_vec_kernel, dim3(stream_grid(total / 4, 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const float4*>(part), splits, split_stride / 4, reinterpret_cast<float4*>(out),
+                       (unsigned)(total / 4), alpha, beta);
+    return;
+  }
   hipLaunchKernelGGL(split_reduce_kernel, dim3(stream_grid(total, 256)), dim3(256), 0, stream, part, splits,
                      split_stride, out, rows, cols, ld, alpha, beta);
 }
@@ -294,6 +331,27 @@ __global__ __launch_bounds__(256) void bwd_bias_colsum_kernel(const float* __res
   part[(size_t)g * KP + j] = a0 + a1;
 }
 
+// The same with four columns per thread through 16-byte loads (K*plane and the pointers multiples of four floats);
+// each column's sum is formed in the same order.
+__global__ __launch_bounds__(256) void bwd_bias_colsum_vec_kernel(const float4* __restrict__ dy, int N, int KP4,
+                                                                  float4* __restrict__ part) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  const int g = blockIdx.y, G = gridDim.y;
+  if (j >= KP4) return;
+  float4 a0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), a1 = a0;
+  int n = g;
+  for (; n + G < N; n += 2 * G) {
+    const float4 u = dy[(size_t)n * KP4 + j], v = dy[(size_t)(n + G) * KP4 + j];
+    a0.x += u.x; a0.y += u.y; a0.z += u.z; a0.w += u.w;
+    a1.x += v.x; a1.y += v.y; a1.z += v.z; a1.w += v.w;
+  }
+  if (n < N) {
+    const float4 u = dy[(size_t)n * KP4 + j];
+    a0.x += u.x; a0.y += u.y; a0.z += u.z; a0.w += u.w;
+  }
+  part[(size_t)g * KP4 + j] = make_float4(a0.x + a1.x, a0.y + a1.y, a0.z + a1.z, a0.w + a1.w);
+}
+
 __global__ __launch_bounds__(256) void bwd_bias_planes_finish_kernel(const float* __restrict__ part, int G, int KP, int plane,
                                                                      float alpha, float beta, float* __restrict__ db) {
   const int k = blockIdx.x;
@@ -489,7 +547,11 @@ extern "C" int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float 
   ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
   if (plane < kBiasSmallPlane && (long long)K * plane < (1ll << 31)) {
     const int KP = K * plane, G = bwd_bias_col_groups(N, KP);
-    hipLaunchKernelGGL(bwd_bias_colsum_kernel, dim3(cdiv(KP, 256), G), dim3(256), 0, stream, dy, N, KP, rowsum);
+    if (KP % 4 == 0 && ((reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(rowsum)) & 15) == 0)
+      hipLaunchKernelGGL(bwd_bias_colsum_vec_kernel, dim3(cdiv(KP / 4, 256), G), dim3(256), 0, stream,
+                         reinterpret_cast<const float4*>(dy), N, KP / 4, reinterpret_cast<float4*>(rowsum));
+    else
+      hipLaunchKernelGGL(bwd_bias_colsum_kernel, dim3(cdiv(KP, 256), G), dim3(256), 0, stream, dy, N, KP, rowsum);
     if (int e = launch_status()) return e;
     hipLaunchKernelGGL(bwd_bias_planes_finish_kernel, dim3(K), dim3(256), 0, stream, rowsum, G, KP, plane, alpha, beta, db);
     return launch_status();
