@@ -416,7 +416,10 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
     case RH_CONV_FWD: {
       const size_t legacy = align256(sizeof(int4) * (size_t)round_up(CRS, kTabPad));
       const SoffPlan sp = plan_soff_fwd(d);
-      return sp.ok && sp.total() > legacy ? sp.total() : legacy;
+      size_t need = sp.ok && sp.total() > legacy ? sp.total() : legacy;
+      const Bf16FwdPlan bp = plan_bf16_fwd(d);  // the bf16 flag is not known here: room for either form
+      if (bp.ok && bp.total() > need) need = bp.total();
+      return need;
     }
     case RH_CONV_BWD_DATA: {
       const size_t legacy = align256(sizeof(int4) * (size_t)round_up(KRS, kTabPad)) +

@@ -97,7 +97,13 @@ inline int launch_mfma_gemm_bf16(const typename AL::Params& ap, const typename B
   if (splits_used) *splits_used = used;
   dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)used);
   constexpr size_t lds_bytes = 16 * 2 * (T::BK / 8) * (T::BM + T::BN);
-  static_assert(lds_bytes <= 48 * 1024, "bf16 tile is expected to fit the default dynamic LDS limit");
+  static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&mfma_gemm_bf16_kernel<T, AL, BL, NCHW, PASS>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (attr != hipSuccess) return (int)attr;
+  }
   ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)(k_algorithmic > 0 ? k_algorithmic : K), stream);
   hipLaunchKernelGGL((mfma_gemm_bf16_kernel<T, AL, BL, NCHW, PASS>), grid, dim3(T::NT), lds_bytes, stream, ap, bp, ep,
                      tiles_m, k_chunks, cps);
@@ -218,6 +224,31 @@ inline SoffPlan plan_soff_fwd(const ConvDims& d) {
   p.tail = plan_tail_split(d.K, (long long)d.N * d.P * d.Q, p.n_k);
   const int slabs_f = p.splits > 1 ? p.splits : p.tail.splits;
   p.part_bytes = slabs_f > 1 ? align256(sizeof(float) * (size_t)slabs_f * (size_t)d.y_elems) : 0;
+  return p;
+}
+
+// Forward with packed bf16 operands (RH_MATH_BF16_MFMA_FP32ACC, input channels a multiple of 8): the contraction runs
+// over k = (r, s, c) with c fastest, the image is copied once to bf16 as [n][hp][c/8][wp][8] with its zero border,
+// the filter to bf16 as [k/8][ko][8] (zero past C*R*S), so that eight consecutive k of one row are 16 contiguous
+// bytes of either operand and neighbouring rows are neighbouring 16-byte pieces.
+// Scratch: table of byte offsets per group of eight k | filter copy | image copy.
+struct Bf16FwdPlan {
+  int n_k, Hp, Wp;
+  size_t tab_bytes, wt_bytes, img_bytes;
+  bool ok;
+  size_t total() const { return tab_bytes + wt_bytes + img_bytes; }
+};
+
+inline Bf16FwdPlan plan_bf16_fwd(const ConvDims& d) {
+  Bf16FwdPlan p;
+  p.n_k = round_up(d.C * d.R * d.S, kTabPad);
+  p.Hp = d.H + 2 * d.pad;
+  p.Wp = d.W + 2 * d.pad;
+  p.tab_bytes = align256(sizeof(int) * (size_t)(p.n_k / 8));
+  p.wt_bytes = align256(2 * (size_t)p.n_k * d.K);
+  const size_t img = 2 * (size_t)d.N * d.C * p.Hp * p.Wp;
+  p.img_bytes = align256(img);
+  p.ok = d.C % 8 == 0 && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0 && (long long)p.Hp * p.Wp < (1ll << 31) / 64;
   return p;
 }
 

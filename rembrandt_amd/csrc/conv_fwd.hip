@@ -231,6 +231,104 @@ static int run_fwd_soff_bf16(const RowSParams& ap, const RowSParams& bp, const E
                                                              k_true);
 }
 
+// ------------------------------------------------------------------------------------------
+// Packed bf16 operands.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint4 pack8_bf16(const float (&v)[8]) {
+  uint4 q;
+  q.x = pack_bf16(v[0], v[1]);
+  q.y = pack_bf16(v[2], v[3]);
+  q.z = pack_bf16(v[4], v[5]);
+  q.w = pack_bf16(v[6], v[7]);
+  return q;
+}
+
+// Both operand copies keep the eight k of a group together and put the GEMM row next: consecutive lanes (rows) of a
+// 16-byte load then read consecutive 16-byte pieces, i.e. whole cache lines per instruction.  (With the rows strided by
+// a pixel's or a filter's full channel vector every lane touches a cache line of its own: the GEMM then ran at 0.55
+// instead of 0.86 PFLOP/s on 256 x 96 x 27 x 27 -> 256, 5x5.)
+//
+// wb[g][ko][8] (bf16) = w[ko][c][r][s] for k' = 8g + e = (r*S + s)*C + c, zero for k' >= C*R*S; one thread per (g, ko).
+// The threads of ko == 0 also write the table: soff8[g] = byte offset of (r, s, c/8) in the image copy (0 past the end:
+// the filter is zero there).
+__global__ __launch_bounds__(256) void prep_bf16_filter_kernel(const float* __restrict__ w, uint4* __restrict__ wb,
+                                                               int* __restrict__ soff8, int n_k, int CRS, int K, int C,
+                                                               int RS, int S, int Wp) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long long)(n_k / 8) * K) return;
+  const int g = (int)(i / K), ko = (int)(i - (long long)g * K);
+  const int k0 = g * 8;
+  float v[8];
+  const int rs = k0 / C, c0 = k0 - rs * C;  // C % 8 == 0: the eight k' share (r, s)
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = k0 < CRS ? w[(size_t)ko * CRS + (size_t)(c0 + e) * RS + rs] : 0.0f;
+  wb[i] = pack8_bf16(v);
+  if (ko == 0) {
+    const int r = rs / S, s2 = rs - r * S;
+    soff8[g] = k0 < CRS ? ((r * (C / 8) + c0 / 8) * Wp + s2) * 16 : 0;
+  }
+}
+
+// xb[n][hp][c/8][wp][8] (bf16) = x[n][c][hp - halo][wp - halo], zero outside; one thread per 16-byte group: eight
+// reads (one per channel, consecutive lanes along w) and one store.
+__global__ __launch_bounds__(256) void nchw_to_bf16_groups_kernel(const float* __restrict__ x, uint4* __restrict__ xb,
+                                                                 unsigned total, int H, int W, FastDiv dWp, FastDiv dCg,
+                                                                 FastDiv dHp, int halo) {
+  const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  uint32_t t, wp, cg, hp, n;
+  dWp.divmod(i, t, wp);
+  dCg.divmod(t, t, cg);
+  dHp.divmod(t, n, hp);
+  const int h = (int)hp - halo, wc = (int)wp - halo;
+  float v[8];
+  if ((unsigned)h < (unsigned)H && (unsigned)wc < (unsigned)W) {
+    const size_t plane = (size_t)H * W;
+    const float* src = x + ((size_t)n * dCg.div * 8 + cg * 8) * plane + (size_t)h * W + wc;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = src[e * plane];
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+  }
+  xb[i] = pack8_bf16(v);
+}
+
+template <class T>
+static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const float* x, const float* w, void* ws,
+                               const EpiParams& ep, hipStream_t stream, const char* tag) {
+  char* base = static_cast<char*>(ws);
+  int* soff8 = reinterpret_cast<int*>(base);
+  uint4* wb = reinterpret_cast<uint4*>(base + bpn.tab_bytes);
+  uint4* xb = reinterpret_cast<uint4*>(base + bpn.tab_bytes + bpn.wt_bytes);
+  const int CRS = d.C * d.R * d.S, HpWp = bpn.Hp * bpn.Wp, Cg = d.C / 8;
+  {
+    ProfScope prof("bf16_filter", 4.0 * (double)d.w_elems + 2.0 * (double)bpn.n_k * d.K, stream);
+    hipLaunchKernelGGL(prep_bf16_filter_kernel, dim3(cdiv((long long)(bpn.n_k / 8) * d.K, 256ll)), dim3(256), 0, stream, w, wb,
+                       soff8, bpn.n_k, CRS, d.K, d.C, d.R * d.S, d.S, bpn.Wp);
+  }
+  if (int e = launch_status()) return e;
+  {
+    const size_t groups = (size_t)d.N * Cg * HpWp;  // below 2^28: the copy is at most 2 GiB
+    ProfScope prof("nchw_to_bf16_groups", 4.0 * (double)d.x_elems + 16.0 * (double)groups, stream);
+    hipLaunchKernelGGL(nchw_to_bf16_groups_kernel, dim3(stream_grid(groups, 256)), dim3(256), 0, stream, x, xb, (unsigned)groups,
+                       d.H, d.W, FastDiv((uint32_t)bpn.Wp), FastDiv((uint32_t)Cg), FastDiv((uint32_t)bpn.Hp), d.pad);
+  }
+  if (int e = launch_status()) return e;
+  RowV8Params ap;  // filter: row ko of group g at (g*K + ko)*16
+  ap.ptr = wb; ap.bytes = (uint32_t)(2 * (size_t)bpn.n_k * d.K);
+  ap.M = d.K; ap.inner = 1; ap.innerW = 1; ap.img_stride = 16; ap.a_stride = 0; ap.b_stride = 0; ap.soff = nullptr;
+  ap.group_stride = d.K * 16;
+  RowV8Params bp;  // image copy, rows = output pixels (n, p, q)
+  bp.ptr = xb; bp.bytes = (uint32_t)(2 * (size_t)d.N * d.C * HpWp);
+  bp.M = d.N * d.P * d.Q; bp.inner = d.P * d.Q; bp.innerW = d.Q;
+  bp.img_stride = HpWp * d.C * 2; bp.a_stride = d.st * Cg * bpn.Wp * 16; bp.b_stride = d.st * 16; bp.soff = soff8;
+  bp.group_stride = 0;
+  typedef LoadRowV8<T::BM, T::BK, T::NT, true> AL;
+  typedef LoadRowV8<T::BN, T::BK, T::NT, false> BL;
+  return launch_mfma_gemm_bf16<T, AL, BL, true, PassConvFwd>(ap, bp, ep, bpn.n_k, 1, nullptr, stream, tag, CRS);
+}
+
 template <class T>
 static int run_fwd(const ConvDims& d, const DenseParams& ap, const GatherParams& bp,
                    const EpiParams& ep, hipStream_t stream, const char* tag) {
@@ -261,6 +359,16 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
   hipStream_t stream = to_stream(stream_);
 
   const int CRS = d.C * d.R * d.S;
+  if ((flags & RH_MATH_BF16_MFMA_FP32ACC) && !(flags & RH_ALGO_GATHER)) {
+    const Bf16FwdPlan bpn = plan_bf16_fwd(d);
+    if (bpn.ok) {
+      EpiParams ep;
+      ep.out = y; ep.bias = (flags & RH_FUSE_BIAS) ? bias : nullptr; ep.alpha = alpha; ep.beta = beta;
+      ep.rows = d.K; ep.cols = d.N * d.P * d.Q; ep.inner = d.P * d.Q; ep.ld = 0; ep.relu = (flags & RH_FUSE_RELU) ? 1 : 0;
+      ep.split_stride = 0;
+      return run_fwd_bf16_packed<T128x128bf>(d, bpn, x, w, ws, ep, stream, "conv_fwd_bf16p_128x128");
+    }
+  }
   const SoffPlan sp = plan_soff_fwd(d);
   if ((flags & RH_MATH_BF16_MFMA_FP32ACC) && (!sp.ok || (flags & RH_ALGO_GATHER))) return RH_E_UNSUPPORTED;
   if (sp.ok && !(flags & RH_ALGO_GATHER)) {

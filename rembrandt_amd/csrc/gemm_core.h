@@ -258,6 +258,7 @@ struct LoadRowS {
   static constexpr int LD = ROWS + lds_pad_kfast<BK>();
   static_assert(NT % ROWS == 0 && (ROWS * BK) % NT == 0 && ROWS % kWave == 0, "loader shape");
   typedef RowSParams Params;
+  typedef float Reg;  // what load_one returns and store_bf16 takes
   __amdgpu_buffer_rsrc_t rsrc;
   const int* tab;
   uint32_t vbase;
@@ -307,6 +308,63 @@ struct LoadRowS {
       q.w = pack_bf16(v[8 * g + 6], v[8 * g + 7]);
       s[(kk0c / 8 + g) * ROWS + row] = q;
     }
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// Packed bf16 operand for the bf16 kernel: the operand already sits in memory as bf16 in groups of eight consecutive
+// k of one row (16 bytes), so a lane's load is one buffer_load_dwordx4 of exactly what one v_mfma_f32_32x32x16_bf16
+// operand register holds, and the LDS slab [k/8][row] receives it unchanged: no conversion, an eighth of the load
+// instructions and half of the bytes of the fp32 loaders.
+//   lane = row m -> (n, a, b) as in LoadRowS, byte offset vbase = n*img_stride + a*a_stride + b*b_stride;
+//   group g of the contraction (k = 8g .. 8g+7): wave-uniform byte offset g*group_stride (LINEAR) or soff[g].
+// ------------------------------------------------------------------------------------------
+struct RowV8Params {
+  const void* ptr; uint32_t bytes;
+  int M, inner, innerW;
+  int img_stride, a_stride, b_stride;  // bytes
+  const int* soff;                     // per group of 8 k, bytes (not LINEAR)
+  int group_stride;                    // bytes between consecutive groups (LINEAR)
+};
+
+template <int ROWS, int BK, int NT, bool LINEAR>
+struct LoadRowV8 {
+  static constexpr int KG = BK / 8;
+  static constexpr int CNT = ROWS * KG / NT;  // 16-byte groups per thread and K step
+  static_assert(BK % 8 == 0 && NT % ROWS == 0 && (ROWS * KG) % NT == 0 && ROWS % kWave == 0, "loader shape");
+  typedef RowV8Params Params;
+  typedef uint4 Reg;
+  __amdgpu_buffer_rsrc_t rsrc;
+  const int* tab;
+  uint32_t vbase;
+  int g0, row, gstride;
+  int so[CNT];
+
+  __device__ __forceinline__ void init(const Params& p, int row0, int tid) {
+    rsrc = make_rsrc(p.ptr, p.bytes);
+    row = tid % ROWS;
+    g0 = __builtin_amdgcn_readfirstlane(tid / ROWS) * CNT;
+    tab = p.soff;
+    gstride = p.group_stride;
+    const int m = row0 + row;
+    const bool valid = m < p.M;
+    const int mm = valid ? m : 0;
+    const int n = mm / p.inner;
+    const int rem = mm - n * p.inner;
+    const int a = rem / p.innerW;
+    const int b = rem - a * p.innerW;
+    vbase = valid ? (uint32_t)(n * p.img_stride + a * p.a_stride + b * p.b_stride) : 0x80000000u;
+  }
+  __device__ __forceinline__ void prep(int k0) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) so[i] = LINEAR ? ((k0 >> 3) + g0 + i) * gstride : tab[(k0 >> 3) + g0 + i];
+  }
+  __device__ __forceinline__ uint4 load_one(int i) const {
+    return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)vbase, so[i], 0));
+  }
+  __device__ __forceinline__ void store_bf16(uint4* s, const uint4 (&v)[CNT]) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) s[(g0 + i) * ROWS + row] = v[i];
   }
 };
 
@@ -660,10 +718,11 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
 }
 
 // ------------------------------------------------------------------------------------------
-// bf16-operand form of the same tile engine (RH_MATH_BF16_MFMA_FP32ACC): operands are read as fp32 by the
-// same loaders, rounded to bf16 when they are written to LDS, multiplied with v_mfma_f32_32x32x16_bf16
-// (8 k per lane per operand) and accumulated in fp32.  LDS slabs are [k/8][row] of 16-byte groups, double
-// buffered: a loader writes one ds_write_b128 per 8 values and an MFMA operand is one ds_read_b128.
+// bf16-operand form of the same tile engine (RH_MATH_BF16_MFMA_FP32ACC): operands reach LDS as bf16 (rounded by the
+// fp32 loaders as they write, or already packed in memory: LoadRowV8), are multiplied with
+// v_mfma_f32_32x32x16_bf16 (8 k per lane per operand) and accumulated in fp32.  LDS slabs are [k/8][row] of
+// 16-byte groups, double buffered: a loader writes one ds_write_b128 per 8 values and an MFMA operand is one
+// ds_read_b128.
 // ------------------------------------------------------------------------------------------
 template <class T, class AL, class BL, bool NCHW, class PASS>
 __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_kernel(typename AL::Params ap,
@@ -707,7 +766,8 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_kernel(typename 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  float ra[AL::CNT], rb[BL::CNT];
+  typename AL::Reg ra[AL::CNT];
+  typename BL::Reg rb[BL::CNT];
   if (nk > 0) {
     la.prep(c_begin * BK);
     lb.prep(c_begin * BK);

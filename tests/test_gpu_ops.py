@@ -90,7 +90,19 @@ def test_conv2d_all_passes(dev, case, algo):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("case", CONV_CASES, ids=[str(c) for c in CONV_CASES])
+# input channels a multiple of 8 take the packed-operand form (bf16 copies of image and filter in 16-byte groups of
+# eight channels): channel groups that do not fill a 64-wide tile, rectangular images, stride with padding, no padding,
+# more filters than one row tile, a contraction shorter than one K step
+BF16_PACKED_CASES = [
+    (3, 72, 11, 9, 40, 3, 2, 1),
+    (2, 8, 17, 17, 200, 5, 1, 2),
+    (5, 16, 9, 12, 24, 3, 1, 0),
+    (2, 8, 6, 6, 3, 1, 1, 0),
+    (130, 8, 5, 5, 16, 3, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES + BF16_PACKED_CASES, ids=[str(c) for c in CONV_CASES + BF16_PACKED_CASES])
 def test_conv2d_fwd_bf16_operands(dev, case):
     """RH_MATH_BF16_MFMA_FP32ACC: operands rounded to bf16 (nearest even), products accumulated in fp32.
     Reference = the fp64-accumulating oracle on operands rounded the same way."""
