@@ -209,9 +209,70 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const float* __restri
   }
 }
 
+// The same for C % 4 == 0 in 16-byte accesses (4-byte accesses top out near 3.8 TB/s on this GPU): a block moves
+// 64 pixels x 64 channels; a thread reads four consecutive pixels of one channel (one 16-byte load where they lie in
+// one source row, which need not be 16-byte aligned; element by element across row ends and the halo) and writes four
+// consecutive channels of one pixel.  LDS tile [pixel][channel], the 16-byte channel groups of a row permuted by the
+// pixel's quad index so that the scattered writes of a wave spread over the banks.
+typedef float float4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+__global__ __launch_bounds__(256) void nchw_to_nhwc_vec_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                               int C, int H, int W, int Hp, int Wp, int halo) {
+  __shared__ __attribute__((aligned(16))) float tile[64 * 64];
+  const int pix0 = blockIdx.x * 64, c0 = blockIdx.y * 64, n = blockIdx.z;
+  const int HpWp = Hp * Wp;
+  {
+    const int pq = threadIdx.x & 15, cl0 = threadIdx.x >> 4;
+    const int pix = pix0 + 4 * pq;
+    const int hp = pix / Wp, wp = pix - hp * Wp;
+    const int h = hp - halo, w = wp - halo;
+    const bool whole = pix + 3 < HpWp && (unsigned)h < (unsigned)H && w >= 0 && w + 3 < W;
+    int off[4];  // element offsets within a plane, -1 = zero
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int pe = pix + e, hpe = pe / Wp, he = hpe - halo, we = pe - hpe * Wp - halo;
+      off[e] = (pe < HpWp && (unsigned)he < (unsigned)H && (unsigned)we < (unsigned)W) ? he * W + we : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int cl = cl0 + 16 * i, c = c0 + cl;
+      float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (c < C) {
+        const float* plane = src + ((size_t)n * C + c) * ((size_t)H * W);
+        if (whole) {
+          const float4_a4 q = *reinterpret_cast<const float4_a4*>(plane + off[0]);
+          v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (off[e] >= 0) v[e] = plane[off[e]];
+        }
+      }
+      const int col = 4 * ((cl >> 2) ^ pq) + (cl & 3);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) tile[(4 * pq + e) * 64 + col] = v[e];
+    }
+  }
+  __syncthreads();
+  const int cq = threadIdx.x & 15, c = c0 + 4 * cq;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int pl = (threadIdx.x >> 4) + 16 * j, pix = pix0 + pl;
+    if (pix < HpWp && c < C) {
+      const float4 q = *reinterpret_cast<const float4*>(&tile[pl * 64 + 4 * (cq ^ ((pl >> 2) & 15))]);
+      *reinterpret_cast<float4*>(dst + ((size_t)n * HpWp + pix) * C + c) = q;
+    }
+  }
+}
+
 static void launch_nchw_to_nhwc(const float* src, float* dst, int N, int C, int H, int W, int Hp, int Wp, int halo,
                                 hipStream_t stream) {
   ProfScope prof("nchw_to_nhwc", 4.0 * ((double)N * C * H * W + (double)N * C * Hp * Wp), stream);
+  if (C % 4 == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+    dim3 grid((unsigned)cdiv(Hp * Wp, 64), (unsigned)cdiv(C, 64), (unsigned)N);
+    hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel, grid, dim3(256), 0, stream, src, dst, C, H, W, Hp, Wp, halo);
+    return;
+  }
   dim3 grid((unsigned)cdiv(Hp * Wp, 32), (unsigned)cdiv(C, 32), (unsigned)N);
   hipLaunchKernelGGL(nchw_to_nhwc_kernel, grid, dim3(256), 0, stream, src, dst, C, H, W, Hp, Wp, halo);
 }
