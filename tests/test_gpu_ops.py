@@ -340,7 +340,7 @@ def test_lrn(dev, case):
 
 
 @pytest.mark.parametrize("shape", [(4, 3, 5, 6), (6, 5, 1, 1), (3, 2, 7, 7), (1, 4, 3, 3), (8, 64, 56, 56), (16, 512, 7, 7),
-                                   (2, 3, 112, 112), (5, 7, 13, 9)])
+                                   (2, 3, 112, 112), (5, 7, 13, 9), (3, 8, 2, 2), (2, 4, 14, 14)])
 def test_bnorm(dev, shape):
     """Spatial batch normalisation: training forward (batch statistics, moving averages, blend, fused ReLU),
     inference forward and backward against the fp64 restatement; one channel carries a mean 25x its deviation.
