@@ -148,7 +148,10 @@ static int run_bwd_data_soff(const RowSParams& ap, const RowSParams& bp, EpiPara
                              stream, tail->col0);
     return launch_status();
   }
-  if (splits <= 1) return launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
+  // one pass over the whole contraction: K steps that hold nothing but the table's zero padding are left out
+  if (splits <= 1)
+    return launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, min(n_k, round_up(k_true, T::BK)), 1, nullptr, stream,
+                                                             tag, k_true);
   // slices of the contraction write unblended partial results; one reduction applies the alpha / beta blend
   const EpiParams fin = ep;
   const long long total = (long long)ep.rows * ep.cols;

@@ -211,7 +211,10 @@ static int run_fwd_soff(const RowSParams& ap, const RowSParams& bp, EpiParams ep
                              fin.relu, stream, tail->col0);
     return launch_status();
   }
-  if (splits <= 1) return launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true);
+  // one pass over the whole contraction: K steps that hold nothing but the table's zero padding are left out
+  if (splits <= 1)
+    return launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, min(n_k, round_up(k_true, T::BK)), 1, nullptr, stream, tag,
+                                                         k_true);
   const EpiParams fin = ep;
   ep.out = part; ep.split_stride = total;
   int used = 1;
