@@ -294,15 +294,22 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
   // about 16 KB of input planes per block (measured best: more LDS per block leaves too few blocks per CU to
   // overlap one block's loads with another's window scans); a single larger plane still goes through LDS
   constexpr int kLdsFloats = 4096;
-  if (d.H * d.W <= 12288 && d.P * d.Q > 0) {
+  if (d.H * d.W <= 16000 && d.P * d.Q > 0) {  // up to 112 x 112 and a little more: 62.5 KB of LDS, two blocks per CU
     int PB = kLdsFloats / (d.H * d.W);
     if (PB < 1) PB = 1;
     if (PB > 64) PB = 64;
     const long long planes = (long long)d.N * d.C;
     const long long blocks = cdiv<long long>(planes, PB);
-    if (blocks < (1ll << 31) && (long long)PB * d.P * d.Q < (1ll << 31)) {
-      hipLaunchKernelGGL(pool_fwd_lds_kernel, dim3((unsigned)blocks), dim3(256), ((size_t)PB * d.H * d.W + 4) * sizeof(float),
-                         to_stream(stream), d, FastDiv((uint32_t)(d.P * d.Q)), PB, planes, x, y, opt_argmax);
+    const size_t lds_bytes = ((size_t)PB * d.H * d.W + 4) * sizeof(float);
+    bool lds_ok = true;
+    if (lds_bytes > 48 * 1024) {
+      static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_fwd_lds_kernel),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+      lds_ok = attr == hipSuccess;
+    }
+    if (lds_ok && blocks < (1ll << 31) && (long long)PB * d.P * d.Q < (1ll << 31)) {
+      hipLaunchKernelGGL(pool_fwd_lds_kernel, dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d,
+                         FastDiv((uint32_t)(d.P * d.Q)), PB, planes, x, y, opt_argmax);
       return launch_status();
     }
   }
