@@ -287,6 +287,15 @@ int rh_bnorm_fwd_infer(int N, int C, int plane, float alpha, const float* x, flo
 int rh_bnorm_bwd(int N, int C, int plane, float alpha_data, float beta_data, const float* x, const float* dy, float* dx,
                  float alpha_param, float beta_param, double epsilon, const float* scale, float* dscale, float* dbias,
                  const float* cached_mean, const float* cached_ivar, void* ws, size_t ws_bytes, rh_stream_t stream);
+/* rh_bnorm_bwd preceded by the backward of the ReLU that rh_bnorm_fwd_train fused (flags RH_FUSE_RELU, alpha 1, beta 0):
+ * dy counts only where the forward output was positive.  Replaces the pair the reference issues, its in-place ReLU
+ * backward kernel on the delta followed by the batch-norm backward (src/operator/conv.rs:577-607), without the pass
+ * over the delta: the sign of the forward output is recomputed from x, the cached statistics, `scale` and `bias`
+ * by the forward pass's own expression, so `scale` and `bias` must still hold the forward pass's values. */
+int rh_bnorm_bwd_relu(int N, int C, int plane, float alpha_data, float beta_data, const float* x, const float* dy, float* dx,
+                      float alpha_param, float beta_param, double epsilon, const float* scale, const float* bias,
+                      float* dscale, float* dbias, const float* cached_mean, const float* cached_ivar, void* ws,
+                      size_t ws_bytes, rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Host-side seeded generator for synthetic inputs and parameter initialisation (stands in for

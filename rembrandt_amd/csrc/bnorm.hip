@@ -42,13 +42,20 @@ __device__ __forceinline__ float wave_sum(float v) {
 // MODE 0: (sum d, sum d*d) with d = x - x[first value of the channel].
 // MODE 1: (sum dy, sum dy*(x - mean[c])).
 // VEC (plane % 4 == 0, 16-byte aligned tensors): a lane reads 16 bytes at a time, two such loads in flight per operand.
-template <int MODE, bool VEC>
+// MASK (MODE 1): dy counts only where the forward pass's ReLU let the value through, i.e. where
+// bn_affine(x, mean, scale*ivar, bias) > 0, recomputed here exactly as the forward pass computed it.
+__device__ __forceinline__ float bn_affine(float x, float mean, float si, float bias) { return fmaf(x - mean, si, bias); }
+
+struct BnMask { const float* scale; const float* ivar; const float* bias; };
+
+template <int MODE, bool VEC, bool MASK = false>
 __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                         const float* __restrict__ mean, int C, int plane, int chunks,
-                                                        long long units, float2* __restrict__ part) {
+                                                        long long units, float2* __restrict__ part, BnMask mk) {
   const int c = blockIdx.x, g = blockIdx.y, G = gridDim.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float shift = MODE == 0 ? x[(size_t)c * plane] : mean[c];
+  const float m_si = MASK ? mk.scale[c] * mk.ivar[c] : 0.0f, m_bias = MASK ? mk.bias[c] : 0.0f;
   float s0a = 0.0f, s0b = 0.0f, s1a = 0.0f, s1b = 0.0f;
   for (long long u = (long long)g * 4 + wave; u < units; u += (long long)G * 4) {
     const int n = (int)(u / chunks), ch = (int)(u - (long long)n * chunks);
@@ -57,7 +64,12 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
     if (VEC) {
       auto add4 = [&](const float4 xv, const float4 gv, float& t0, float& t1) {
         const float d[4] = {xv.x - shift, xv.y - shift, xv.z - shift, xv.w - shift};
-        const float gg[4] = {gv.x, gv.y, gv.z, gv.w};
+        float gg[4] = {gv.x, gv.y, gv.z, gv.w};
+        if (MASK) {
+          const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) gg[e] = bn_affine(xs[e], shift, m_si, m_bias) > 0.0f ? gg[e] : 0.0f;
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           if (MODE == 0) { t0 += d[e]; t1 = fmaf(d[e], d[e], t1); }
@@ -87,7 +99,11 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
         s0a += d0; s0b += d1;
         s1a = fmaf(d0, d0, s1a); s1b = fmaf(d1, d1, s1b);
       } else {
-        const float g0 = dy[base + i], g1 = dy[base + i + 64];
+        float g0 = dy[base + i], g1 = dy[base + i + 64];
+        if (MASK) {
+          g0 = bn_affine(x[base + i], shift, m_si, m_bias) > 0.0f ? g0 : 0.0f;
+          g1 = bn_affine(x[base + i + 64], shift, m_si, m_bias) > 0.0f ? g1 : 0.0f;
+        }
         s0a += g0; s0b += g1;
         s1a = fmaf(g0, d0, s1a); s1b = fmaf(g1, d1, s1b);
       }
@@ -98,7 +114,8 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
         s0a += d0;
         s1a = fmaf(d0, d0, s1a);
       } else {
-        const float g0 = dy[base + i];
+        float g0 = dy[base + i];
+        if (MASK) g0 = bn_affine(x[base + i], shift, m_si, m_bias) > 0.0f ? g0 : 0.0f;
         s0a += g0;
         s1a = fmaf(g0, d0, s1a);
       }
@@ -168,20 +185,23 @@ __global__ void bn_bwd_finish_kernel(const float2* __restrict__ part, int G, int
 // Forward:  out = alpha * f((x - mean)*a + b) + beta*out, f = identity or max(., 0) applied after the blend when RELU.
 // Backward: out = alpha * a*(dy - c2 - (x - mean)*c3) + beta*out.
 // VEC: 4 values per thread (plane % 4 == 0 and 16-byte aligned pointers, so a group never crosses a plane).
-template <bool BWD, bool RELU, bool VEC>
+// MASK (backward only): dy is taken as 0 where the forward ReLU clamped, see bn_reduce_kernel; mask_bias = the layer's bias.
+template <bool BWD, bool RELU, bool VEC, bool MASK = false>
 __global__ __launch_bounds__(256) void bn_apply_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                        float* __restrict__ out, const float4* __restrict__ coef,
                                                        long long groups, int C, FastDiv plane_groups, FastDiv chans,
-                                                       float alpha, float beta) {
+                                                       float alpha, float beta, const float* __restrict__ mask_bias) {
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < groups; i += stride) {
     const uint32_t row = plane_groups.quot((uint32_t)i);  // n*C + c
     const uint32_t c = row - chans.quot(row) * (uint32_t)C;
     const float4 k = coef[c];
+    const float mb = MASK ? mask_bias[c] : 0.0f;
     auto one = [&](float xv, float gv, float ov) {
       float v;
+      if (MASK) gv = bn_affine(xv, k.x, k.y, mb) > 0.0f ? gv : 0.0f;
       if (BWD) v = k.y * (gv - k.z - (xv - k.x) * k.w);
-      else v = fmaf(xv - k.x, k.y, k.z);
+      else v = bn_affine(xv, k.x, k.y, k.z);
       v *= alpha;
       if (beta != 0.0f) v = fmaf(beta, ov, v);
       if (RELU) v = v > 0.0f ? v : 0.0f;
@@ -201,19 +221,19 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const float* __restrict__
   }
 }
 
-template <bool BWD, bool RELU>
+template <bool BWD, bool RELU, bool MASK = false>
 void launch_bn_apply(const float* x, const float* dy, float* out, const float4* coef, int N, int C, int plane, float alpha,
-                     float beta, hipStream_t st) {
+                     float beta, hipStream_t st, const float* mask_bias = nullptr) {
   const long long total = (long long)N * C * plane;
   const bool vec = plane % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out) |
                                         reinterpret_cast<uintptr_t>(dy)) & 15) == 0;
   if (vec) {
     const long long groups = total / 4;
-    hipLaunchKernelGGL((bn_apply_kernel<BWD, RELU, true>), dim3(stream_grid((size_t)groups, 256)), dim3(256), 0, st, x, dy, out,
-                       coef, groups, C, FastDiv((uint32_t)(plane / 4)), FastDiv((uint32_t)C), alpha, beta);
+    hipLaunchKernelGGL((bn_apply_kernel<BWD, RELU, true, MASK>), dim3(stream_grid((size_t)groups, 256)), dim3(256), 0, st, x, dy,
+                       out, coef, groups, C, FastDiv((uint32_t)(plane / 4)), FastDiv((uint32_t)C), alpha, beta, mask_bias);
   } else {
-    hipLaunchKernelGGL((bn_apply_kernel<BWD, RELU, false>), dim3(stream_grid((size_t)total, 256)), dim3(256), 0, st, x, dy, out,
-                       coef, total, C, FastDiv((uint32_t)plane), FastDiv((uint32_t)C), alpha, beta);
+    hipLaunchKernelGGL((bn_apply_kernel<BWD, RELU, false, MASK>), dim3(stream_grid((size_t)total, 256)), dim3(256), 0, st, x, dy,
+                       out, coef, total, C, FastDiv((uint32_t)plane), FastDiv((uint32_t)C), alpha, beta, mask_bias);
   }
 }
 
@@ -254,10 +274,10 @@ extern "C" int rh_bnorm_fwd_train(int N, int C, int plane, float alpha, const fl
     ProfScope prof("bnorm_fwd_reduce", 4.0 * (double)total, st);
     if (plane % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
       hipLaunchKernelGGL((bn_reduce_kernel<0, true>), dim3(C, p.G), dim3(256), 0, st, x, (const float*)nullptr,
-                         (const float*)nullptr, C, plane, p.chunks, p.units, part);
+                         (const float*)nullptr, C, plane, p.chunks, p.units, part, BnMask());
     else
       hipLaunchKernelGGL((bn_reduce_kernel<0, false>), dim3(C, p.G), dim3(256), 0, st, x, (const float*)nullptr,
-                         (const float*)nullptr, C, plane, p.chunks, p.units, part);
+                         (const float*)nullptr, C, plane, p.chunks, p.units, part, BnMask());
     hipLaunchKernelGGL(bn_fwd_finish_kernel, dim3(cdiv(C, 64)), dim3(64), 0, st, x, part, p.G, C, plane,
                        (double)N * (double)plane, ema_factor, epsilon, scale, bias, running_mean, running_ivar, cached_mean,
                        cached_ivar, coef);
@@ -288,11 +308,10 @@ extern "C" int rh_bnorm_fwd_infer(int N, int C, int plane, float alpha, const fl
   return launch_status();
 }
 
-extern "C" int rh_bnorm_bwd(int N, int C, int plane, float alpha_data, float beta_data, const float* x, const float* dy,
-                            float* dx, float alpha_param, float beta_param, double epsilon, const float* scale, float* dscale,
-                            float* dbias, const float* cached_mean, const float* cached_ivar, void* ws, size_t ws_bytes,
-                            rh_stream_t stream) {
-  (void)epsilon;  // the cached inverse standard deviation of the forward pass is used
+static int bnorm_bwd(int N, int C, int plane, float alpha_data, float beta_data, const float* x, const float* dy, float* dx,
+                     float alpha_param, float beta_param, const float* scale, float* dscale, float* dbias,
+                     const float* cached_mean, const float* cached_ivar, void* ws, size_t ws_bytes, const float* relu_bias,
+                     rh_stream_t stream) {
   long long total;
   if (int e = bn_check(N, C, plane, &total)) return e;
   if (total == 0) return 0;
@@ -302,18 +321,50 @@ extern "C" int rh_bnorm_bwd(int N, int C, int plane, float alpha_data, float bet
   const BnPlan p = bn_plan(N, C, plane);
   float2* part = static_cast<float2*>(ws);
   float4* coef = reinterpret_cast<float4*>(static_cast<char*>(ws) + bn_part_bytes(p, C));
+  const bool vec = plane % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0;
   {
     ProfScope prof("bnorm_bwd_reduce", 8.0 * (double)total, st);
-    if (plane % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0)
-      hipLaunchKernelGGL((bn_reduce_kernel<1, true>), dim3(C, p.G), dim3(256), 0, st, x, dy, cached_mean, C, plane, p.chunks,
-                         p.units, part);
-    else
-      hipLaunchKernelGGL((bn_reduce_kernel<1, false>), dim3(C, p.G), dim3(256), 0, st, x, dy, cached_mean, C, plane, p.chunks,
-                         p.units, part);
+    const dim3 grid(C, p.G);
+    if (relu_bias) {
+      const BnMask mk = {scale, cached_ivar, relu_bias};
+      if (vec)
+        hipLaunchKernelGGL((bn_reduce_kernel<1, true, true>), grid, dim3(256), 0, st, x, dy, cached_mean, C, plane, p.chunks,
+                           p.units, part, mk);
+      else
+        hipLaunchKernelGGL((bn_reduce_kernel<1, false, true>), grid, dim3(256), 0, st, x, dy, cached_mean, C, plane, p.chunks,
+                           p.units, part, mk);
+    } else {
+      if (vec)
+        hipLaunchKernelGGL((bn_reduce_kernel<1, true>), grid, dim3(256), 0, st, x, dy, cached_mean, C, plane, p.chunks, p.units,
+                           part, BnMask());
+      else
+        hipLaunchKernelGGL((bn_reduce_kernel<1, false>), grid, dim3(256), 0, st, x, dy, cached_mean, C, plane, p.chunks, p.units,
+                           part, BnMask());
+    }
     hipLaunchKernelGGL(bn_bwd_finish_kernel, dim3(cdiv(C, 64)), dim3(64), 0, st, part, p.G, C, (double)N * (double)plane,
                        alpha_param, beta_param, scale, dscale, dbias, cached_mean, cached_ivar, coef);
   }
   ProfScope prof("bnorm_bwd_apply", (beta_data != 0.0f ? 16.0 : 12.0) * (double)total, st);
-  launch_bn_apply<true, false>(x, dy, dx, coef, N, C, plane, alpha_data, beta_data, st);
+  if (relu_bias) launch_bn_apply<true, false, true>(x, dy, dx, coef, N, C, plane, alpha_data, beta_data, st, relu_bias);
+  else launch_bn_apply<true, false>(x, dy, dx, coef, N, C, plane, alpha_data, beta_data, st);
   return launch_status();
+}
+
+extern "C" int rh_bnorm_bwd(int N, int C, int plane, float alpha_data, float beta_data, const float* x, const float* dy,
+                            float* dx, float alpha_param, float beta_param, double epsilon, const float* scale, float* dscale,
+                            float* dbias, const float* cached_mean, const float* cached_ivar, void* ws, size_t ws_bytes,
+                            rh_stream_t stream) {
+  (void)epsilon;  // the cached inverse standard deviation of the forward pass is used
+  return bnorm_bwd(N, C, plane, alpha_data, beta_data, x, dy, dx, alpha_param, beta_param, scale, dscale, dbias, cached_mean,
+                   cached_ivar, ws, ws_bytes, nullptr, stream);
+}
+
+extern "C" int rh_bnorm_bwd_relu(int N, int C, int plane, float alpha_data, float beta_data, const float* x, const float* dy,
+                                 float* dx, float alpha_param, float beta_param, double epsilon, const float* scale,
+                                 const float* bias, float* dscale, float* dbias, const float* cached_mean,
+                                 const float* cached_ivar, void* ws, size_t ws_bytes, rh_stream_t stream) {
+  (void)epsilon;
+  if (!bias) return RH_E_INVALID;
+  return bnorm_bwd(N, C, plane, alpha_data, beta_data, x, dy, dx, alpha_param, beta_param, scale, dscale, dbias, cached_mean,
+                   cached_ivar, ws, ws_bytes, bias, stream);
 }

@@ -1079,13 +1079,21 @@ struct BNormConvUnit {
   // pre_delta = dBN(out_delta) with the scale / bias gradients accumulated, then grad_weights += dconv(in, pre_delta).
   // With `ws_aux` the filter gradient goes to the context's second stream (scratch of its own) and overlaps whatever
   // the main stream does next with pre_delta (the data gradient); the worker joins at the end of backward.
+  // `relu_masked`: out_delta has not been through the backward of the ReLU that followed this unit's batch norm
+  // (forward with beta_out 0); the batch-norm backward applies that mask itself, from pre_act.
   void backward_params(size_t batch, const float* in, const float* out_delta, double epsilon, DeviceBuffer<uint8_t>& ws,
-                       DeviceBuffer<uint8_t>* ws_aux) {
+                       DeviceBuffer<uint8_t>* ws_aux, bool relu_masked = false) {
     RB_ASSERT(backward);
     const rh_conv_geom g = geom(batch);
-    unwrap(rh_bnorm_bwd(g.N, g.K, plane(), 1.0f, 0.0f, pre_act->as_ptr(), out_delta, pre_delta->as_mut_ptr(), 1.0f, 1.0f,
-                        epsilon, scale->as_ptr(), scale_grad->as_mut_ptr(), bias_grad->as_mut_ptr(), cached_mean->as_ptr(),
-                        cached_ivar->as_ptr(), ws.as_mut_ptr(), ws.len(), s()), "batch norm backward");
+    if (relu_masked)
+      unwrap(rh_bnorm_bwd_relu(g.N, g.K, plane(), 1.0f, 0.0f, pre_act->as_ptr(), out_delta, pre_delta->as_mut_ptr(), 1.0f, 1.0f,
+                               epsilon, scale->as_ptr(), bias->as_ptr(), scale_grad->as_mut_ptr(), bias_grad->as_mut_ptr(),
+                               cached_mean->as_ptr(), cached_ivar->as_ptr(), ws.as_mut_ptr(), ws.len(), s()),
+             "batch norm backward with ReLU mask");
+    else
+      unwrap(rh_bnorm_bwd(g.N, g.K, plane(), 1.0f, 0.0f, pre_act->as_ptr(), out_delta, pre_delta->as_mut_ptr(), 1.0f, 1.0f,
+                          epsilon, scale->as_ptr(), scale_grad->as_mut_ptr(), bias_grad->as_mut_ptr(), cached_mean->as_ptr(),
+                          cached_ivar->as_ptr(), ws.as_mut_ptr(), ws.len(), s()), "batch norm backward");
     rh_stream_t sg = s();
     DeviceBuffer<uint8_t>* wg = &ws;
     if (ws_aux) {
@@ -1397,8 +1405,12 @@ class StackResConv2dOperator : public BNormUnitsOperator {
     apply_rect_backprop(config_.act_func, out_act_->as_ptr(), len, batch_size, out_delta_->as_mut_ptr(), s);
     units_[1].backward_params(batch_size, mid_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
     units_[1].backward_data(batch_size, mid_delta_->as_mut_ptr(), 0.0f, *workspace_);
-    apply_rect_backprop(config_.act_func, mid_act_->as_ptr(), len, batch_size, mid_delta_->as_mut_ptr(), s);
-    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
+    // with fused epilogues the ReLU mask of mid is applied inside unit 0's batch-norm backward (mid_delta keeps the
+    // unmasked values); otherwise in place, as the reference does
+    const bool fold_mid = opts_.fuse_epilogue && config_.act_func == ActivationFunction::Rect;
+    if (!fold_mid) apply_rect_backprop(config_.act_func, mid_act_->as_ptr(), len, batch_size, mid_delta_->as_mut_ptr(), s);
+    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws(),
+                              fold_mid);
     if (in_delta_) {
       unwrap(rh_copy_d2d(in_delta_->as_mut_ptr(), out_delta_->as_ptr(), len * batch_size * 4, s), "send");
       units_[0].backward_data(batch_size, in_delta_->as_mut_ptr(), 1.0f, *workspace_);
@@ -1457,8 +1469,12 @@ class ProjStackResConv2dOperator : public BNormUnitsOperator {
     apply_rect_backprop(config_.act_func, out_act_->as_ptr(), len, batch_size, out_delta_->as_mut_ptr(), s);
     units_[1].backward_params(batch_size, mid_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
     units_[1].backward_data(batch_size, mid_delta_->as_mut_ptr(), 0.0f, *workspace_);
-    apply_rect_backprop(config_.act_func, mid_act_->as_ptr(), len, batch_size, mid_delta_->as_mut_ptr(), s);
-    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
+    // with fused epilogues the ReLU mask of mid is applied inside unit 0's batch-norm backward (mid_delta keeps the
+    // unmasked values); otherwise in place, as the reference does
+    const bool fold_mid = opts_.fuse_epilogue && config_.act_func == ActivationFunction::Rect;
+    if (!fold_mid) apply_rect_backprop(config_.act_func, mid_act_->as_ptr(), len, batch_size, mid_delta_->as_mut_ptr(), s);
+    units_[0].backward_params(batch_size, in_act_->as_ptr(), mid_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws(),
+                              fold_mid);
     units_[2].backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
     if (in_delta_) {
       units_[0].backward_data(batch_size, in_delta_->as_mut_ptr(), 0.0f, *workspace_);

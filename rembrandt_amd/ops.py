@@ -329,8 +329,9 @@ def bnorm_fwd_infer(x, scale, bias, running_mean, running_ivar, epsilon, alpha=1
 
 
 def bnorm_bwd(x, dy, scale, cached_mean, cached_ivar, epsilon, dscale=None, dbias=None, alpha_data=1.0, beta_data=0.0,
-              dx=None, alpha_param=1.0, beta_param=0.0):
-    """Returns (dx, dscale, dbias); with beta_param = 1 the parameter gradients accumulate as in the reference."""
+              dx=None, alpha_param=1.0, beta_param=0.0, relu_bias=None):
+    """Returns (dx, dscale, dbias); with beta_param = 1 the parameter gradients accumulate as in the reference.
+    `relu_bias` (the layer's bias): dy is first masked by the ReLU that the forward pass fused (rh_bnorm_bwd_relu)."""
     N, Cc, H, W = x.shape
     if dx is None:
         assert beta_data == 0.0
@@ -339,6 +340,11 @@ def bnorm_bwd(x, dy, scale, cached_mean, cached_ivar, epsilon, dscale=None, dbia
         assert beta_param == 0.0
         dscale, dbias = torch.empty_like(scale), torch.empty_like(scale)
     ws, nbytes = _bnorm_ws(x)
+    if relu_bias is not None:
+        check(lib().rh_bnorm_bwd_relu(N, Cc, H * W, alpha_data, beta_data, _p(x), _p(dy), _p(dx), alpha_param, beta_param,
+                                      epsilon, _p(scale), _p(relu_bias), _p(dscale), _p(dbias), _p(cached_mean),
+                                      _p(cached_ivar), _p(ws), nbytes, _stream()), "rh_bnorm_bwd_relu")
+        return dx, dscale, dbias
     check(lib().rh_bnorm_bwd(N, Cc, H * W, alpha_data, beta_data, _p(x), _p(dy), _p(dx), alpha_param, beta_param, epsilon,
                              _p(scale), _p(dscale), _p(dbias), _p(cached_mean), _p(cached_ivar), _p(ws), nbytes, _stream()),
           "rh_bnorm_bwd")

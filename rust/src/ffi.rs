@@ -161,6 +161,11 @@ extern "C" {
                       dy: *const f32, dx: *mut f32, alpha_param: c_float, beta_param: c_float, epsilon: f64,
                       scale: *const f32, dscale: *mut f32, dbias: *mut f32, cached_mean: *const f32,
                       cached_ivar: *const f32, ws: *mut c_void, ws_bytes: size_t, stream: rh_stream_t) -> c_int;
+  pub fn rh_bnorm_bwd_relu(n: c_int, c: c_int, plane: c_int, alpha_data: c_float, beta_data: c_float, x: *const f32,
+                           dy: *const f32, dx: *mut f32, alpha_param: c_float, beta_param: c_float, epsilon: f64,
+                           scale: *const f32, bias: *const f32, dscale: *mut f32, dbias: *mut f32,
+                           cached_mean: *const f32, cached_ivar: *const f32, ws: *mut c_void, ws_bytes: size_t,
+                           stream: rh_stream_t) -> c_int;
 }
 
 /// The reference `unwrap()`s / `panic!`s on every native error (src/operator/mod.rs:1685-1696).

@@ -130,7 +130,12 @@ def check_step(w, ref, sgd, rsgd, x, labels, fused_sgd, tag, teacher=False):
         delta = op.backward(want_in_delta=i > 0)
         if hasattr(op, "units"):
             if hasattr(op, "mid_delta"):
-                assert_close(w.read(i, "mid_delta"), op.mid_delta.ravel(), what + " mid_delta")
+                # with fused epilogues the device keeps mid_delta as it was before the ReLU mask (the mask is applied
+                # inside the first unit's batch-norm backward); the reference masks it in place
+                got_mid = w.read(i, "mid_delta").reshape(op.mid_act.shape).copy()
+                if getattr(op, "act", None) == "Rect":
+                    O.rect_backprop_inplace(op.mid_act, got_mid)
+                assert_close(got_mid.ravel(), op.mid_delta.ravel(), what + " mid_delta")
             for k, u in enumerate(op.units):
                 assert_close(w.read(i, "u%d.pre_delta" % k), u.pre_delta.ravel(), "%s unit %d pre_delta" % (what, k))
                 for gname, rname in UNIT_GRADS:

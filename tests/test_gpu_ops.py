@@ -388,6 +388,17 @@ def test_bnorm(dev, shape):
     dx2 = T(y0, dev)
     ops.bnorm_bwd(xd, T(dy, dev), sd, cm, ci, eps, alpha_data=1.0, beta_data=1.0, dx=dx2)
     assert_close(N(dx2), dx_ref.astype(np.float64) + y0, "bnorm bwd dx blended", atol=2e-5)
+    # backward through the ReLU the forward pass fused: the mask is the device's own forward output, and must be that
+    # exactly (an element the two passes disagree on would be off by a whole dy)
+    yr, _, _ = ops.bnorm_fwd_train(xd, sd, bd, T(rm, dev), T(ri, dev), ema, eps, relu=True)
+    dym = np.where(N(yr) > 0, dy, np.float32(0.0)).astype(np.float32)
+    dxm_ref, dsm_ref, dbm_ref = O.bnorm_bwd(x, dym, scale, N(cm), N(ci))
+    dxm, dsm, dbm = ops.bnorm_bwd(xd, T(dy, dev), sd, cm, ci, eps, relu_bias=bd)
+    assert_close(N(dxm), dxm_ref, "bnorm bwd through fused relu: dx", atol=2e-5)
+    assert_close(N(dsm), dsm_ref, "bnorm bwd through fused relu: dscale", atol=2e-5)
+    assert_close(N(dbm), dbm_ref, "bnorm bwd through fused relu: dbias", atol=2e-5)
+    same = ops.bnorm_bwd(xd, T(dym, dev), sd, cm, ci, eps)
+    assert np.array_equal(N(dxm), N(same[0])) and np.array_equal(N(dsm), N(same[1])), "identical to masking dy beforehand"
     torch.cuda.synchronize()
 
 
