@@ -107,7 +107,8 @@ typedef struct {
 enum { RH_CONV_FWD = 0, RH_CONV_BWD_FILTER = 1, RH_CONV_BWD_DATA = 2 };
 
 int32_t rh_conv2d_out_dim(int32_t in, int32_t size, int32_t stride, int32_t pad);
-/* Bytes of scratch the given pass needs (0 is possible). The scratch must be 256-byte aligned. */
+/* Bytes of scratch the given pass needs whatever flags it is called with (0 is possible).  The scratch must be
+ * 256-byte aligned. */
 size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass);
 /* y = alpha * corr(x, w) + beta * y.  With RH_FUSE_BIAS, `bias` (length K) is added after the
  * alpha/beta blend; with RH_FUSE_RELU the result is clamped at 0.  bias may be NULL otherwise. */
