@@ -17,6 +17,8 @@ inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 // Contraction tables are padded to a multiple of this many entries (>= every BK in use).
 constexpr int kTabPad = 64;
+// Readable bytes kept after an operand that LoadRow4 reads: its last group of four rows may begin at the last valid row.
+constexpr size_t kRow4Slack = 16;
 
 struct ConvDims {
   int N, C, H, W, K, R, S, st, pad, P, Q;
@@ -216,7 +218,7 @@ inline SoffPlan plan_soff_fwd(const ConvDims& d) {
   p.Hp = d.H + 2 * d.pad;
   p.Wp = d.W + 2 * d.pad;
   p.tab_bytes = align256(sizeof(int) * (size_t)p.n_k);
-  p.wt_bytes = align256(sizeof(float) * (size_t)p.n_k * d.K);
+  p.wt_bytes = align256(sizeof(float) * (size_t)p.n_k * d.K + kRow4Slack);
   const size_t img = sizeof(float) * (size_t)d.N * d.C * p.Hp * p.Wp;
   p.img_bytes = d.pad > 0 ? align256(img) : 0;
   p.ok = img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;

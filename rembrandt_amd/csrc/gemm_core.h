@@ -65,6 +65,7 @@ struct LoadDenseK {
   static constexpr int LD = ROWS + lds_pad_kfast<BK>();
   static_assert(NT % BK == 0 && (ROWS * BK) % NT == 0, "loader shape");
   typedef DenseParams Params;
+  typedef float Reg;
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t rowoff[CNT];
   const int* ktab;
@@ -109,6 +110,7 @@ struct LoadDenseR {
   static constexpr int LD = ROWS + lds_pad_kfast<BK>();
   static_assert(NT % ROWS == 0 && (ROWS * BK) % NT == 0, "loader shape");
   typedef DenseParams Params;
+  typedef float Reg;
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t rowoff;
   int kk0, K, ld, sbase;
@@ -171,6 +173,7 @@ struct LoadGatherR {
   static constexpr int LD = ROWS + lds_pad_kfast<BK>();
   static_assert(NT % ROWS == 0 && (ROWS * BK) % NT == 0 && ROWS % kWave == 0, "loader shape");
   typedef GatherParams Params;
+  typedef float Reg;
   __amdgpu_buffer_rsrc_t rsrc;
   const int4* ktab;
   int base, h0, w0, phase, Hlim, Wlim, sbase;
@@ -312,6 +315,50 @@ struct LoadRowS {
 };
 
 // ------------------------------------------------------------------------------------------
+// LINEAR scalar-offset operand whose rows are contiguous in memory (row m+1 sits 4 bytes after row m: the
+// transposed filter [k][row]): a lane loads four rows of one k with one buffer_load_dwordx4 and writes them with one
+// ds_write_b128, a quarter of the loader instructions of LoadRowS.  A wave's load covers 64/(ROWS/4) values of k,
+// so the lane's share of the k offset is part of its vector offset.  Same Params as LoadRowS (b_stride == 1, no
+// n / a decomposition).  The 12 bytes after the last valid row of the buffer must be readable: rows past M
+// inside a group read whatever follows, and only feed result rows that are never stored.
+// ------------------------------------------------------------------------------------------
+template <int ROWS, int BK, int NT>
+struct LoadRow4 {
+  static constexpr int LPK = ROWS / 4;           // lanes per k
+  static constexpr int KPI = NT / LPK;           // k values one instruction of the block covers
+  static constexpr int CNT = BK / KPI;           // loads per thread and K step
+  static constexpr int LD = ROWS + 4;            // rows of 16-byte aligned groups
+  static_assert(ROWS % 4 == 0 && NT % LPK == 0 && BK % KPI == 0 && CNT >= 1, "loader shape");
+  typedef RowSParams Params;
+  typedef float4 Reg;
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t vbase;
+  int ldk4, sbase;
+  int so[CNT];
+
+  __device__ __forceinline__ void init(const Params& p, int row0, int tid) {
+    rsrc = make_rsrc(p.ptr, p.bytes);
+    const int row = (tid % LPK) * 4;
+    const int kl = tid / LPK;  // this thread's k within an instruction
+    ldk4 = p.ldk4;
+    sbase = kl * LD + row;
+    const int m = row0 + row;
+    vbase = m < p.M ? ((uint32_t)m << 2) + (uint32_t)(kl * ldk4) : 0x80000000u;
+  }
+  __device__ __forceinline__ void prep(int k0) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) so[i] = (k0 + i * KPI) * ldk4;
+  }
+  __device__ __forceinline__ float4 load_one(int i) const {
+    return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)vbase, so[i], 0));
+  }
+  __device__ __forceinline__ void store(float* s, const float4 (&v)[CNT]) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) *reinterpret_cast<float4*>(s + sbase + i * KPI * LD) = v[i];
+  }
+};
+
+// ------------------------------------------------------------------------------------------
 // Packed bf16 operand for the bf16 kernel: the operand already sits in memory as bf16 in groups of eight consecutive
 // k of one row (16 bytes), so a lane's load is one buffer_load_dwordx4 of exactly what one v_mfma_f32_32x32x16_bf16
 // operand register holds, and the LDS slab [k/8][row] receives it unchanged: no conversion, an eighth of the load
@@ -389,6 +436,7 @@ struct LoadPixDy {
   static constexpr int LD = ROWS + lds_pad_kfast<BK>();
   static_assert(NT % BK == 0 && (ROWS * BK) % NT == 0, "loader shape");
   typedef PixDyParams Params;
+  typedef float Reg;
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t rowoff[CNT];
   int kk, M, PQ, img, sbase;
@@ -438,6 +486,7 @@ struct LoadPixX {
   static constexpr int LD = ROWS + lds_pad_kfast<BK>();
   static_assert(NT % BK == 0 && (ROWS * BK) % NT == 0, "loader shape");
   typedef PixXParams Params;
+  typedef float Reg;
   __amdgpu_buffer_rsrc_t rsrc;
   int roff[CNT], rr[CNT], rs[CNT];
   int kk, M, PQ, Q, img, H, W, st, pad, sbase;
@@ -631,7 +680,8 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  float ra[AL::CNT], rb[BL::CNT];
+  typename AL::Reg ra[AL::CNT];
+  typename BL::Reg rb[BL::CNT];
   if (nk > 0) {
     la.prep(c_begin * BK);
     lb.prep(c_begin * BK);
