@@ -134,6 +134,9 @@ def main():
     ap.add_argument("--no-kernel-events", action="store_true",
                     help="do not bracket each kernel with HIP events in the timed region (no per-kernel breakdown)")
     ap.add_argument("--no-calibration", action="store_true", help="skip the MFMA-loop / copy ceiling probes")
+    ap.add_argument("--host-frames", action="store_true",
+                    help="every timed step first copies its batch of u8 frames from the worker's host frame buffer "
+                         "(the PCIe-inclusive rate; the default keeps the inputs resident in HBM)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="first launch the library's plain copy kernel 4 times over MIB MiB (a known-size "
                          "reference for hardware byte counters collected around this command)")
@@ -162,7 +165,10 @@ def main():
     worker.init_params()
     x = synth.normal(seed, 100, (batch, dims[2], dims[1], dims[0]))
     labels = synth.integers(seed, 200, (batch,), ncat)
-    worker.load_frames_f32(x)             # inputs resident in HBM before the timed region
+    if args.host_frames:
+        worker.load_frames_u8(synth.integers(seed, 101, (batch, dims[2], dims[1], dims[0]), 256).astype("uint8"))
+    else:
+        worker.load_frames_f32(x)         # inputs resident in HBM before the timed region
     worker.stage_batch(labels, 1.0 / batch)
     sgd = SgdOpt(batch, 0.01, ("Update", 0.9), 0.0)
     sgd.begin(worker)
@@ -214,6 +220,8 @@ def main():
     t0 = time.perf_counter()
     loss = 0.0
     for _ in range(args.steps):
+        if args.host_frames:
+            worker.reload_frames(batch)   # the staged u8 frames again: host -> device, synchronous as in the reference
         loss, _ = sgd.train_batch(worker, batch, fused=not args.unfused)
     worker.sync()
     torch.cuda.synchronize()
@@ -245,6 +253,7 @@ def main():
                                "weights N(0,0.01), %s%s" % (args.workload, batch, dims[2], dims[1], dims[0],
                                                             "unfused reference sequence" if args.unfused else "fused epilogues",
                                                             ("" if args.no_overlap else ", two-stream backward") +
+                                                            (", u8 frames copied from host memory every step" if args.host_frames else "") +
                                                             (", steps replayed as a HIP graph" if args.graph else "")),
                    "global_batch": batch, "params": cfg.params_len(), "gemm_gflop_per_step": gemm_flops / 1e9},
         "roofline": None if dom is None else

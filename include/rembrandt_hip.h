@@ -85,6 +85,10 @@ int rh_graph_launch(rh_graph* g, rh_ctx* ctx);
 int rh_graph_destroy(rh_graph* g);
 int rh_malloc(rh_ctx* ctx, size_t bytes, void** dptr); /* zero-filled, like DeviceBuffer::zeros */
 int rh_free(rh_ctx* ctx, void* dptr);
+/* Page-locked, zero-filled host memory for what is copied to the device every batch: the u8 frame buffer that
+ * Data3dOperator stages its input in (in_buf_h, src/operator/mod.rs:640-700; a plain Vec<u8> there). */
+int rh_host_malloc(rh_ctx* ctx, size_t bytes, void** hptr);
+int rh_host_free(rh_ctx* ctx, void* hptr);
 int rh_memset_f32(float* d, float value, size_t n, rh_stream_t stream);
 int rh_copy_d2d(void* dst, const void* src, size_t bytes, rh_stream_t stream);
 int rh_load_sync(rh_ctx* ctx, void* dst_d, const void* src_h, size_t bytes);

@@ -205,6 +205,26 @@ extern "C" int rh_free(rh_ctx* ctx, void* dptr) {
   return (int)hipFree(dptr);
 }
 
+// Page-locked host memory for buffers that are copied to the device every batch (the input frames): copies from it
+// run at the link's rate and need no staging copy inside the driver.  Zero-filled.
+extern "C" int rh_host_malloc(rh_ctx* ctx, size_t bytes, void** hptr) {
+  if (!ctx || !hptr) return RH_E_INVALID;
+  *hptr = nullptr;
+  if (bytes == 0) return 0;
+  hipError_t e = hipHostMalloc(hptr, bytes, hipHostMallocDefault);
+  if (e != hipSuccess) return (int)e;
+  memset(*hptr, 0, bytes);
+  return 0;
+}
+
+extern "C" int rh_host_free(rh_ctx* ctx, void* hptr) {
+  if (!ctx) return RH_E_INVALID;
+  if (!hptr) return 0;
+  hipError_t e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) return (int)e;
+  return (int)hipHostFree(hptr);
+}
+
 extern "C" int rh_copy_d2d(void* dst, const void* src, size_t bytes, rh_stream_t stream) {
   if (bytes == 0) return 0;
   if (!dst || !src) return RH_E_INVALID;

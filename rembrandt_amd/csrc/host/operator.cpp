@@ -26,6 +26,13 @@ static void unwrap_last(const char* what) { unwrap(rh_last_error(), what); }
 DeviceContext::DeviceContext(int device_idx) : ctx_(nullptr) { unwrap(rh_ctx_create(device_idx, &ctx_), "rh_ctx_create"); }
 DeviceContext::~DeviceContext() { rh_ctx_destroy(ctx_); }
 void DeviceContext::sync() const { unwrap(rh_ctx_sync(ctx_), "rh_ctx_sync"); }
+PinnedBytes::PinnedBytes(size_t len, std::shared_ptr<DeviceContext> ctx) : len_(len), ctx_(std::move(ctx)) {
+  void* p = nullptr;
+  unwrap(rh_host_malloc(ctx_->raw(), len, &p), "rh_host_malloc");
+  ptr_ = static_cast<uint8_t*>(p);
+}
+PinnedBytes::~PinnedBytes() { rh_host_free(ctx_->raw(), ptr_); }
+
 rh_stream_t DeviceContext::aux_stream() const {
   rh_stream_t s = rh_ctx_aux_stream(ctx_);
   if (!s) panic("rh_ctx_aux_stream failed");
@@ -411,7 +418,7 @@ class Data3dOperator : public InputOperator {
  public:
   Data3dOperator(size_t batch_size, const Data3dOperatorConfig& config, Ctx context, const uint64_t seed[2])
       : batch_cap_(batch_size), config_(config), context_(context),
-        in_buf_h_(batch_size * config.in_dims.len(), 0),
+        in_buf_h_(batch_size * config.in_dims.len(), context),
         in_buf_(new DeviceBuffer<uint8_t>(batch_size * config.in_dims.len(), context)),
         out_buf_(new DeviceBuffer<float>(batch_size * config.in_dims.len(), context)),
         rng_(seed), noise_seed_(seed[0] ^ 0x5043414Eull) {
@@ -573,7 +580,7 @@ class Data3dOperator : public InputOperator {
   size_t batch_cap_;
   Data3dOperatorConfig config_;
   Ctx context_;
-  std::vector<uint8_t> in_buf_h_;
+  PinnedBytes in_buf_h_;  // page-locked: it is copied to the device every batch
   std::unique_ptr<DeviceBuffer<uint8_t>> in_buf_;
   std::unique_ptr<DeviceBuffer<float>> tmp_buf_, f32_frames_;
   SharedDeviceBuf out_buf_;

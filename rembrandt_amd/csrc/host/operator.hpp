@@ -59,6 +59,23 @@ class DeviceContext {
   rh_ctx* ctx_;
 };
 
+// Page-locked host bytes (zero-filled): staging for per-batch copies to the device.
+class PinnedBytes {
+ public:
+  PinnedBytes(size_t len, std::shared_ptr<DeviceContext> ctx);
+  ~PinnedBytes();
+  PinnedBytes(const PinnedBytes&) = delete;
+  PinnedBytes& operator=(const PinnedBytes&) = delete;
+  uint8_t* data() { return ptr_; }
+  const uint8_t* data() const { return ptr_; }
+  size_t size() const { return len_; }
+
+ private:
+  uint8_t* ptr_ = nullptr;
+  size_t len_;
+  std::shared_ptr<DeviceContext> ctx_;
+};
+
 template <class T>
 class DeviceBuffer {
  public:

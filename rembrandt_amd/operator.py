@@ -339,6 +339,10 @@ class SequentialOperatorWorker:
             C.memmove(p, frames[b].ctypes.data, flen)
         _chk(lib().rho_worker_load_frames(self._h, n))
 
+    def reload_frames(self, batch_size):
+        """Copies the frames already staged in the host frame buffer to the device again (load_frames)."""
+        _chk(lib().rho_worker_load_frames(self._h, batch_size))
+
     def load_frames_f32(self, frames):
         frames = np.ascontiguousarray(frames, np.float32)
         _chk(lib().rho_worker_load_frames_f32(self._h, frames.ctypes.data, frames.shape[0]))
