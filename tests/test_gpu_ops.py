@@ -424,3 +424,32 @@ def test_pool2d_bwd_with_folded_relu_mask(dev, case, rounding):
     ops.rect_backprop_inplace(xd, two)
     assert np.array_equal(got, N(two))
     torch.cuda.synchronize()
+
+
+def test_context_memory_calls(dev):
+    """rh_malloc (zero-filled), rh_host_malloc (page-locked, zero-filled), rh_load_sync / rh_store_sync round trip."""
+    import ctypes as C
+    lib = _lib.lib()
+    ctx = C.c_void_p()
+    _lib.check(lib.rh_ctx_create(0, C.byref(ctx)), "rh_ctx_create")
+    n = 3 * 1000 + 1   # not a multiple of four bytes
+    d, h, back = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    _lib.check(lib.rh_malloc(ctx, n, C.byref(d)), "rh_malloc")
+    _lib.check(lib.rh_host_malloc(ctx, n, C.byref(h)), "rh_host_malloc")
+    _lib.check(lib.rh_host_malloc(ctx, n, C.byref(back)), "rh_host_malloc")
+    host = (C.c_uint8 * n).from_address(h.value)
+    out = (C.c_uint8 * n).from_address(back.value)
+    assert not any(host) and not any(out), "page-locked memory starts zeroed"
+    _lib.check(lib.rh_store_sync(ctx, back, d, n), "rh_store_sync")
+    assert not any(out), "device memory starts zeroed, odd tail included"
+    pattern = synth.integers(21, 1, (n,), 256).astype(np.uint8)
+    C.memmove(h, pattern.ctypes.data, n)
+    _lib.check(lib.rh_load_sync(ctx, d, h, n), "rh_load_sync")
+    _lib.check(lib.rh_store_sync(ctx, back, d, n), "rh_store_sync")
+    assert np.array_equal(np.frombuffer(out, np.uint8), pattern)
+    assert lib.rh_host_malloc(ctx, 16, None) == _lib.RH_E_INVALID and lib.rh_host_free(None, h) == _lib.RH_E_INVALID
+    for p_ in (h, back):
+        _lib.check(lib.rh_host_free(ctx, p_), "rh_host_free")
+    _lib.check(lib.rh_free(ctx, d), "rh_free")
+    _lib.check(lib.rh_ctx_destroy(ctx), "rh_ctx_destroy")
+
