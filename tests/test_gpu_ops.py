@@ -453,3 +453,45 @@ def test_context_memory_calls(dev):
     _lib.check(lib.rh_free(ctx, d), "rh_free")
     _lib.check(lib.rh_ctx_destroy(ctx), "rh_ctx_destroy")
 
+
+def test_conv2d_random_geometries(dev):
+    """A seeded sweep over convolution geometries (filter 1-7, stride 1-4, any padding below the filter size, channel
+    counts on both sides of every tile and group size): all three passes, the forced scalar-offset backward-filter and
+    the bf16-operand forward against the oracle.  The hand-picked cases above name the paths; this guards the seams."""
+    import random
+    rnd = random.Random(20160417)
+    done = 0
+    while done < 60:
+        R = rnd.choice([1, 1, 2, 3, 3, 3, 4, 5, 7])
+        st = rnd.choice([1, 1, 1, 2, 2, 3, 4])
+        pad = rnd.randint(0, max(0, R - 1))
+        C = rnd.choice([1, 2, 3, 4, 7, 8, 12, 16, 24, 33, 40, 64, 72, 96])
+        K = rnd.choice([1, 3, 5, 8, 16, 20, 32, 50, 64, 96, 100, 128, 130, 200, 256])
+        H, W = rnd.randint(max(R - 2 * pad, 1), 24), rnd.randint(max(R - 2 * pad, 1), 24)
+        Nn = rnd.choice([1, 2, 3, 5, 9, 17, 40])
+        if Nn * C * H * W * K * R * R > 6e8:
+            Nn = 2
+        if (H + 2 * pad - R) // st + 1 < 1 or (W + 2 * pad - R) // st + 1 < 1:
+            continue
+        case = (Nn, C, H, W, K, R, st, pad)
+        say("random conv case", done, case)
+        x = synth.normal(31, done * 4 + 1, (Nn, C, H, W))
+        w = synth.normal(31, done * 4 + 2, (K, C, R, R))
+        b = synth.normal(31, done * 4 + 3, (K,))
+        y_ref = O.conv2d_fwd(x, w, st, pad)
+        dy = synth.normal(31, done * 4 + 4, y_ref.shape)
+        xd, wd, bd, dyd = T(x, dev), T(w, dev), T(b, dev), T(dy, dev)
+        tag = " %s" % (case,)
+        y = ops.conv2d_fwd(xd, wd, st, pad, bias=bd, relu=True)
+        assert_close(N(y), O.rect_inplace(O.add_bias_nchw(b, y_ref.copy())), "fwd" + tag)
+        y16 = ops.conv2d_fwd(xd, wd, st, pad, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)
+        assert_close(N(y16), O.conv2d_fwd(O.round_bf16(x), O.round_bf16(w), st, pad), "fwd bf16" + tag)
+        dw_ref = O.conv2d_bwd_filter(x, dy, w.shape, st, pad)
+        assert_close(N(ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad)), dw_ref, "bwd_filter" + tag)
+        assert_close(N(ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, algo=_lib.RH_ALGO_SCALAR_OFFSET)), dw_ref,
+                     "bwd_filter scalar-offset" + tag)
+        assert_close(N(ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad)), O.conv2d_bwd_data(w, dy, x.shape, st, pad),
+                     "bwd_data" + tag)
+        done += 1
+    torch.cuda.synchronize()
+
