@@ -495,3 +495,55 @@ def test_conv2d_random_geometries(dev):
         done += 1
     torch.cuda.synchronize()
 
+
+def test_sgemm_and_pool_random_shapes(dev):
+    """Seeded sweeps: SGEMM over transposes, odd extents, padded leading dimensions, alpha / beta pairs, with and
+    without scratch; pooling over window, stride, padding, both modes and both roundings on rectangular planes."""
+    import random
+    rnd = random.Random(20160418)
+    for it in range(40):
+        tA, tB = rnd.randint(0, 1), rnd.randint(0, 1)
+        m = rnd.choice([1, 2, 7, 10, 31, 64, 100, 128, 129, 300, 500, 1000, 4096])
+        n = rnd.choice([1, 3, 16, 32, 64, 100, 128, 200, 256])
+        k = rnd.choice([1, 2, 15, 16, 17, 64, 100, 256, 1000, 2450, 4096])
+        if m * n * k > 3e8:
+            k = 64
+        use_ws = rnd.random() < 0.7
+        a_shape = (m, k) if tA else (k, m)
+        b_shape = (k, n) if tB else (n, k)
+        lda, ldb, ldc = a_shape[1] + rnd.randint(0, 3), b_shape[1] + rnd.randint(0, 2), m + rnd.randint(0, 2)
+        alpha, beta = rnd.choice([(1.0, 0.0), (0.5, 1.0), (1.0, 1.0), (-2.0, 0.25)])
+        say("random sgemm", it, (tA, tB, m, n, k, lda, ldb, ldc, alpha, beta, use_ws))
+        A = synth.normal(41, it * 3 + 1, (a_shape[0], lda))
+        B = synth.normal(41, it * 3 + 2, (b_shape[0], ldb))
+        C0 = synth.normal(41, it * 3 + 3, (n, ldc))
+        ref = O.sgemm(tA, tB, m, n, k, alpha, A, lda, B, ldb, beta, C0.copy(), ldc)
+        Cd = T(C0, dev)
+        ops.sgemm(tA, tB, m, n, k, alpha, T(A, dev), lda, T(B, dev), ldb, beta, Cd, ldc, use_workspace=use_ws)
+        assert_close(N(Cd), ref, "sgemm %d" % it)
+    for it in range(40):
+        k = rnd.choice([2, 2, 3, 3, 4, 5])
+        st = rnd.choice([1, 2, 2, 3])
+        pad = rnd.randint(0, k // 2)
+        H, W = rnd.randint(k, 40), rnd.randint(k, 40)
+        Nn, C = rnd.choice([1, 2, 5]), rnd.choice([1, 3, 8, 17])
+        mode = rnd.choice([_lib.RH_POOL_MAX, _lib.RH_POOL_AVG_INCL_PAD])
+        rounding = rnd.choice([_lib.RH_ROUND_FLOOR, _lib.RH_ROUND_CEIL])
+        say("random pool", it, (Nn, C, H, W, k, st, pad, mode, rounding))
+        x = np.round(synth.normal(42, it * 2 + 1, (Nn, C, H, W)) * 2) / 2
+        y_ref, am_ref = O.pool2d_fwd(x, k, st, pad, mode, rounding, want_argmax=True)
+        if y_ref.size == 0:
+            continue
+        xd = T(x, dev)
+        y, am = ops.pool2d_fwd(xd, k, st, pad, mode, rounding, want_argmax=True)
+        assert_close(N(y), y_ref, "pool fwd %d" % it)
+        if mode == _lib.RH_POOL_MAX:
+            assert np.array_equal(N(am), am_ref), "arg-max mask %d" % it
+        dy = synth.normal(42, it * 2 + 2, y_ref.shape)
+        dx_ref = O.pool2d_bwd(x, y_ref, dy, k, st, pad, mode, rounding)
+        assert_close(N(ops.pool2d_bwd(xd, y, T(dy, dev), k, st, pad, mode, rounding)), dx_ref, "pool bwd %d" % it)
+        if mode == _lib.RH_POOL_MAX:
+            assert_close(N(ops.pool2d_bwd(xd, y, T(dy, dev), k, st, pad, mode, rounding, argmax=am)), dx_ref,
+                         "pool bwd from the mask %d" % it)
+    torch.cuda.synchronize()
+
