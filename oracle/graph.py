@@ -86,7 +86,7 @@ class Conv2dOperator:
         self.out_delta = np.zeros_like(self.out_act)
 
     def forward(self, in_act):
-        self.in_act = in_act
+        self.in_act = in_act = np.ascontiguousarray(in_act.reshape(self.x_shape))   # buffers are flat: any operator may precede
         if self.bf16_forward:
             O.conv2d_fwd(O.round_bf16(in_act), O.round_bf16(self.p.weights), self.stride, self.pad, y=self.out_act)
         elif self.fast:

@@ -224,6 +224,56 @@ def test_nin_forward_bf16(dev):
     w.close()
 
 
+def test_random_networks_train_steps(dev):
+    """Seeded sweep over operator chains: 1-3 convolutions (filter 1-5, stride 1-2, any legal padding, Rect or
+    Identity) with local response normalisation, max / average pooling and dropout between them, an optional hidden
+    affine layer, fused or reference-order epilogues and SGD, every momentum flavour; two checked steps each."""
+    import random
+    rnd = random.Random(20160419)
+    for it in range(14):
+        wdt, hgt, c = rnd.choice([8, 11, 14, 16, 20]), rnd.choice([8, 11, 14, 16, 20]), rnd.choice([1, 3, 4, 8])
+        dims, spec = (wdt, hgt, c), []
+        w_, h_ = wdt, hgt
+        for _ in range(rnd.randint(1, 3)):
+            k, st = rnd.choice([1, 3, 3, 5]), rnd.choice([1, 1, 2])
+            pad = rnd.randint(0, k // 2)
+            out = rnd.choice([4, 8, 12, 16, 20, 32])
+            if (w_ + 2 * pad - k) // st + 1 < 2 or (h_ + 2 * pad - k) // st + 1 < 2:
+                k, st, pad = 1, 1, 0
+            spec.append(("conv", k, st, pad, out, rnd.choice(["Rect", "Rect", "Identity"])))
+            w_, h_ = (w_ + 2 * pad - k) // st + 1, (h_ + 2 * pad - k) // st + 1
+            if rnd.random() < 0.25:
+                spec.append(("lrn", rnd.choice([3, 5]), 1e-2, 0.75, 2.0))
+            if rnd.random() < 0.6 and w_ >= 3 and h_ >= 3:
+                pk, ps = rnd.choice([2, 3]), rnd.choice([1, 2])
+                pp = rnd.choice([0, 0, 1]) if pk == 3 else 0
+                spec.append(("pool", pk, ps, pp, rnd.choice(["Max", "Max", "Average"])))
+                w_, h_ = (w_ + 2 * pp - pk) // ps + 1, (h_ + 2 * pp - pk) // ps + 1
+            if rnd.random() < 0.2:
+                spec.append(("dropout", 0.3))
+        if rnd.random() < 0.6:
+            spec.append(("fc", rnd.choice([16, 33, 64]), rnd.choice(["Rect", "Identity"])))
+            if rnd.random() < 0.3:
+                spec.append(("dropout", 0.5))
+        ncat = rnd.choice([3, 5, 10])
+        spec.append(("fc", ncat, "Identity"))
+        batch = rnd.choice([4, 8, 16, 33])
+        fuse, fused_sgd = rnd.random() < 0.7, rnd.random() < 0.6
+        flavour = rnd.choice([("Update", 0.9), ("UpdateNesterov", 0.9), ("Gradient", 0.8), "Zero", ("GradientNesterov", 0.9)])
+        say("random net", it, dims, spec, "batch", batch, fuse, fused_sgd, flavour)
+        net = (dims, *configs._chain(dims, spec))
+        w, ref = make_pair(net, batch, 1000 + it, fuse)
+        sgd = SgdOpt(batch, 0.05, flavour, 1e-4)
+        rsgd = OG.SgdOpt(0.05, flavour, 1e-4)
+        sgd.begin(w)
+        rsgd.begin(ref)
+        for step in range(2):
+            x = synth.normal(1000 + it, 100 + step, (batch, dims[2], dims[1], dims[0]))
+            labels = synth.integers(1000 + it, 200 + step, (batch,), ncat)
+            check_step(w, ref, sgd, rsgd, x, labels, batch, fused_sgd, "random net %d step %d" % (it, step))
+        w.close()
+
+
 @pytest.mark.parametrize("flavour", ["Zero", "Update", "UpdateNesterov", "Gradient", "GradientNesterov"])
 def test_momentum_flavours(dev, flavour):
     """All five Momentum flavours on a small conv net (3 steps each, unfused BLAS-1 sequence and, where it
