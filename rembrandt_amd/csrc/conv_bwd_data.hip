@@ -141,11 +141,12 @@ static int run_bwd_data_soff(const RowSParams& ap, const RowSParams& bp, EpiPara
     // whole tiles blend into dx as usual; the sliced tail goes through `part` and one reduction over its columns
     const EpiParams fin = ep;
     const long long total = (long long)ep.rows * ep.cols;
-    ep.part = part; ep.split_stride = total;
+    const long long first = tail_first_elem(*tail, ep.inner, ep.rows);
+    ep.part = part; ep.part_first = first; ep.split_stride = total - first;
     ep.full_tiles = tail->full_tiles; ep.tail_tiles = tail->tail_tiles; ep.tail_splits = tail->splits;
     if (int e = launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true)) return e;
-    launch_split_reduce_nchw(part, tail->splits, total, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta, nullptr, 0,
-                             stream, tail->col0);
+    launch_split_reduce_nchw(part, tail->splits, total - first, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta,
+                             nullptr, 0, stream, tail->col0);
     return launch_status();
   }
   // one pass over the whole contraction: K steps that hold nothing but the table's zero padding are left out

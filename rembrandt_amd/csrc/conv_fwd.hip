@@ -123,7 +123,7 @@ __global__ __launch_bounds__(256) void split_reduce_nchw_kernel(const float* __r
 #pragma unroll
   for (int e = 0; e < E; ++e) acc[e] = a1[e] = 0.0f;
   auto add = [&](float (&dst)[E], int s) {
-    const float* p = part + (long long)s * stride + i0;
+    const float* p = part + (long long)s * stride + (i0 - first);  // a slab starts at the result's element `first`
     if (VEC) {
       const float4 v = *reinterpret_cast<const float4*>(p);
       dst[0] += v.x; dst[E > 1 ? 1 : 0] += v.y; dst[E > 2 ? 2 : 0] += v.z; dst[E > 3 ? 3 : 0] += v.w;
@@ -208,11 +208,12 @@ static int run_fwd_soff(const RowSParams& ap, const RowSParams& bp, EpiParams ep
   if (splits <= 1 && tail && tail->splits > 1) {
     // whole tiles blend into y as usual; the sliced tail goes through `part` and one reduction over its columns
     const EpiParams fin = ep;
-    ep.part = part; ep.split_stride = total;
+    const long long first = tail_first_elem(*tail, ep.inner, ep.rows);
+    ep.part = part; ep.part_first = first; ep.split_stride = total - first;
     ep.full_tiles = tail->full_tiles; ep.tail_tiles = tail->tail_tiles; ep.tail_splits = tail->splits;
     if (int e = launch_mfma_gemm<T, AL, BL, true, PassConvFwd>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true)) return e;
-    launch_split_reduce_nchw(part, tail->splits, total, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta, fin.bias,
-                             fin.relu, stream, tail->col0);
+    launch_split_reduce_nchw(part, tail->splits, total - first, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta,
+                             fin.bias, fin.relu, stream, tail->col0);
     return launch_status();
   }
   // one pass over the whole contraction: K steps that hold nothing but the table's zero padding are left out

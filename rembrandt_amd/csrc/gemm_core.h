@@ -541,9 +541,10 @@ struct LoadPixX {
 //
 // Tail form (tail_tiles > 0, 1-D grid): the first full_tiles tiles of the logical order are computed whole and
 // blended into `out`; each of the last tail_tiles tiles is computed by tail_splits blocks over slices of the
-// contraction, which write unblended partial sums to part + slice * split_stride.  It evens out a grid whose tile
-// count is a little over a multiple of the CU count (676 tiles on 256 CUs: a quarter of the CUs would carry three
-// tiles, the rest two) without paying partial-sum traffic for the whole result.
+// contraction, which write unblended partial sums to part + slice * split_stride - part_first: a slab holds the
+// result's elements from index part_first on (the first image any tail column belongs to), not the whole result.
+// It evens out a grid whose tile count is a little over a multiple of the CU count (676 tiles on 256 CUs: a quarter
+// of the CUs would carry three tiles, the rest two) without paying partial-sum traffic for the whole result.
 // ------------------------------------------------------------------------------------------
 struct EpiParams {
   float* out;
@@ -553,6 +554,7 @@ struct EpiParams {
   int relu;
   long long split_stride;
   float* part = nullptr;
+  long long part_first = 0;
   int full_tiles = 0, tail_tiles = 0, tail_splits = 0;
 };
 
@@ -574,7 +576,9 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], co
                                            int wm, int wn, int lane, int split_idx) {
   constexpr int TM = T::TM, TN = T::TN;
   const bool split = split_idx >= 0;  // < 0: blend into the result
-  float* out = split ? (ep.tail_tiles > 0 ? ep.part : ep.out) + (long long)split_idx * ep.split_stride : ep.out;
+  float* out = !split ? ep.out
+               : ep.tail_tiles > 0 ? ep.part + ((long long)split_idx * ep.split_stride - ep.part_first)
+                                   : ep.out + (long long)split_idx * ep.split_stride;
   const float alpha = split ? 1.0f : ep.alpha;
   const float beta = split ? 0.0f : ep.beta;
   const int row_stride = NCHW ? ep.inner : ep.ld;

@@ -39,6 +39,9 @@ CONV_CASES = [
     (2, 4, 21, 21, 6, 5, 4, 2),
     (2, 8, 14, 14, 256, 3, 2, 1),
     (1, 3, 16, 16, 4, 5, 5, 0),
+    # 832 / 885 column tiles of 32 x 256 on 768 block slots: the tiles past the last multiple of the CU count are cut
+    # into slices of the contraction although the grid takes more than one round (forward and backward-data)
+    (52, 32, 66, 66, 32, 3, 1, 0),
 ]
 
 
