@@ -42,6 +42,9 @@ CONV_CASES = [
     # 832 / 885 column tiles of 32 x 256 on 768 block slots: the tiles past the last multiple of the CU count are cut
     # into slices of the contraction although the grid takes more than one round (forward and backward-data)
     (52, 32, 66, 66, 32, 3, 1, 0),
+    # stride 1 with output rows a multiple of four pixels long on a 128-row tile, padded and unpadded image
+    (3, 8, 12, 16, 128, 3, 1, 1),
+    (2, 16, 10, 12, 130, 1, 1, 0),
 ]
 
 
