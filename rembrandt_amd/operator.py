@@ -190,7 +190,10 @@ class SequentialOperatorConfig:
 
     def __del__(self):
         if getattr(self, "_h", None):
-            lib().rho_config_free(self._h)
+            try:
+                lib().rho_config_free(self._h)
+            except TypeError:   # interpreter shutdown: module globals are already gone, the process frees the rest
+                pass
             self._h = None
 
     def data3d(self, in_dims, normalize=False):
@@ -509,7 +512,10 @@ class DataSource:
 
     def __del__(self):
         if getattr(self, "_h", None):
-            lib().rho_dataset_free(self._h)
+            try:
+                lib().rho_dataset_free(self._h)
+            except TypeError:   # interpreter shutdown: module globals are already gone, the process frees the rest
+                pass
             self._h = None
 
     def num_samples(self):
@@ -552,7 +558,10 @@ class SgdOpt:
 
     def __del__(self):
         if getattr(self, "_h", None):
-            lib().rho_sgd_free(self._h)
+            try:
+                lib().rho_sgd_free(self._h)
+            except TypeError:   # interpreter shutdown: module globals are already gone, the process frees the rest
+                pass
             self._h = None
 
     def begin(self, worker):
