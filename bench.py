@@ -221,7 +221,15 @@ def main():
     loss = 0.0
     for _ in range(args.steps):
         if args.host_frames:
-            worker.reload_frames(batch)   # the staged u8 frames again: host -> device, synchronous as in the reference
+            # The step is launched piece by piece so that the next batch's frames can be handed over while it is still
+            # queued (load_frames returns when the host buffer is free again, as in the reference, but copies beside
+            # the kernels of the step before); the loss read-back then synchronises, as train_batch does.
+            worker.forward(batch, training=True, t=sgd.iter_counter())
+            worker.backward(batch)
+            sgd.step(worker, fused=not args.unfused)
+            worker.reload_frames(batch)
+            loss = worker.store_loss(batch)
+            continue
         loss, _ = sgd.train_batch(worker, batch, fused=not args.unfused)
     worker.sync()
     torch.cuda.synchronize()

@@ -93,6 +93,13 @@ int rh_memset_f32(float* d, float value, size_t n, rh_stream_t stream);
 int rh_copy_d2d(void* dst, const void* src, size_t bytes, rh_stream_t stream);
 int rh_load_sync(rh_ctx* ctx, void* dst_d, const void* src_h, size_t bytes);
 int rh_store_sync(rh_ctx* ctx, void* dst_h, const void* src_d, size_t bytes);
+/* sync_load of the per-batch input (Data3dOperator::load_frames, src/operator/mod.rs:690-700) without the wait for
+ * the kernels still queued on the context's stream: the copy runs on a stream of its own, after the last reader of
+ * dst_d that rh_mark_consumed recorded, and later work on the context's stream waits for it.  Returns when src_h may
+ * be reused.  Falls back to waiting for the context's stream when no reader was marked (first load, or the readers
+ * ran inside a recorded graph); RH_E_UNSUPPORTED between rh_ctx_begin_capture and rh_ctx_end_capture. */
+int rh_load_overlapped(rh_ctx* ctx, void* dst_d, const void* src_h, size_t bytes);
+int rh_mark_consumed(rh_ctx* ctx);
 int rh_cast_u8_f32(const uint8_t* x, float* y, size_t n, float scale, rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------

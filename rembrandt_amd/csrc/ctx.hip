@@ -20,6 +20,10 @@ struct rh_ctx {
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   bool aux_dirty = false;   // the second stream was given work (fork) that the main stream has not waited for yet
   bool capturing = false;   // between rh_ctx_begin_capture and rh_ctx_end_capture
+  // copy stream for host -> device loads that run beside the main stream's kernels (created on first use)
+  hipStream_t copy = nullptr;
+  hipEvent_t ev_copied = nullptr, ev_consumed = nullptr;
+  bool consumed_valid = false;  // ev_consumed was recorded after the last reader of the buffer loaded that way
 };
 
 // A captured and instantiated sequence of launches of one context (both streams).
@@ -65,6 +69,12 @@ extern "C" int rh_ctx_destroy(rh_ctx* ctx) {
     (void)hipStreamDestroy(ctx->aux);
     (void)hipEventDestroy(ctx->ev_fork);
     (void)hipEventDestroy(ctx->ev_join);
+  }
+  if (ctx->copy) {
+    (void)hipStreamSynchronize(ctx->copy);
+    (void)hipStreamDestroy(ctx->copy);
+    (void)hipEventDestroy(ctx->ev_copied);
+    (void)hipEventDestroy(ctx->ev_consumed);
   }
   hipError_t e = hipStreamSynchronize(ctx->stream);
   hipError_t e2 = hipStreamDestroy(ctx->stream);
@@ -168,6 +178,7 @@ extern "C" int rh_ctx_end_capture(rh_ctx* ctx, rh_graph** out) {
 
 extern "C" int rh_graph_launch(rh_graph* g, rh_ctx* ctx) {
   if (!g || !ctx || ctx->capturing) return RH_E_INVALID;
+  ctx->consumed_valid = false;  // the recorded launches may read a buffer that rh_load_overlapped fills
   return (int)hipGraphLaunch(g->exec, ctx->stream);
 }
 
@@ -238,6 +249,52 @@ extern "C" int rh_load_sync(rh_ctx* ctx, void* dst_d, const void* src_h, size_t 
   hipError_t e = hipMemcpyAsync(dst_d, src_h, bytes, hipMemcpyHostToDevice, ctx->stream);
   if (e != hipSuccess) return (int)e;
   return (int)hipStreamSynchronize(ctx->stream);
+}
+
+// Host -> device load that does not wait for the main stream's queued kernels: the copy runs on a stream of its own,
+// after the last reader of dst_d that rh_mark_consumed recorded, and the main stream's later work waits for it.
+// Returns when the copy is complete (src_h may be reused), like rh_load_sync.  Without a valid consumed mark (none
+// recorded yet, or the readers were launched inside a recording or a graph replay) it first waits for the main stream.
+extern "C" int rh_load_overlapped(rh_ctx* ctx, void* dst_d, const void* src_h, size_t bytes) {
+  if (!ctx) return RH_E_INVALID;
+  if (bytes == 0) return 0;
+  if (!dst_d || !src_h) return RH_E_INVALID;
+  if (ctx->capturing) return RH_E_UNSUPPORTED;
+  hipError_t e;
+  if (!ctx->copy) {
+    if ((e = hipSetDevice(ctx->device)) != hipSuccess) return (int)e;
+    hipStream_t s = nullptr;
+    hipEvent_t a = nullptr, b = nullptr;
+    if ((e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) != hipSuccess) return (int)e;  // default priority
+    if ((e = hipEventCreateWithFlags(&a, hipEventDisableTiming)) != hipSuccess ||
+        (e = hipEventCreateWithFlags(&b, hipEventDisableTiming)) != hipSuccess) {
+      (void)hipStreamDestroy(s);
+      if (a) (void)hipEventDestroy(a);
+      return (int)e;
+    }
+    ctx->copy = s; ctx->ev_copied = a; ctx->ev_consumed = b;
+  }
+  if (ctx->consumed_valid) {
+    if ((e = hipStreamWaitEvent(ctx->copy, ctx->ev_consumed, 0)) != hipSuccess) return (int)e;
+  } else if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) {
+    return (int)e;
+  }
+  ctx->consumed_valid = false;  // the next readers have to be marked again
+  if ((e = hipMemcpyAsync(dst_d, src_h, bytes, hipMemcpyHostToDevice, ctx->copy)) != hipSuccess) return (int)e;
+  if ((e = hipEventRecord(ctx->ev_copied, ctx->copy)) != hipSuccess) return (int)e;
+  if ((e = hipStreamWaitEvent(ctx->stream, ctx->ev_copied, 0)) != hipSuccess) return (int)e;
+  return (int)hipStreamSynchronize(ctx->copy);
+}
+
+// Marks the point of the main stream after which the buffer last filled by rh_load_overlapped is no longer read.
+// Inside a recording nothing is marked (the recorded readers run at replay time, unknown to the host).
+extern "C" int rh_mark_consumed(rh_ctx* ctx) {
+  if (!ctx) return RH_E_INVALID;
+  if (ctx->capturing || !ctx->copy) { ctx->consumed_valid = false; return 0; }
+  hipError_t e = hipEventRecord(ctx->ev_consumed, ctx->stream);
+  if (e != hipSuccess) return (int)e;
+  ctx->consumed_valid = true;
+  return 0;
 }
 
 extern "C" int rh_store_sync(rh_ctx* ctx, void* dst_h, const void* src_d, size_t bytes) {

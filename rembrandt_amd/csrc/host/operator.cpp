@@ -460,9 +460,11 @@ class Data3dOperator : public InputOperator {
     RB_ASSERT(batch_idx < batch_cap_);
     return in_buf_h_.data() + batch_idx * config_.in_dims.len();
   }
+  // The copy runs on the context's copy stream, beside whatever the main stream still holds of the previous batch
+  // (its backward pass and update), and only after that batch's cast has read in_buf; forward() marks that point.
   void load_frames(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
-    in_buf_->sync_load(in_buf_h_.data(), in_buf_h_.size());
+    unwrap(rh_load_overlapped(context_->raw(), in_buf_->as_mut_ptr(), in_buf_h_.data(), in_buf_h_.size()), "sync_load");
     f32_loaded_ = false;
   }
   void load_frames_f32(const float* host, size_t batch_size) override {
@@ -488,6 +490,7 @@ class Data3dOperator : public InputOperator {
       if (num_preprocs) unwrap(rh_copy_d2d(cur, f32_frames_->as_ptr(), in_len * sizeof(float), s), "send");
     } else {
       unwrap(rh_cast_u8_f32(in_buf_->as_ptr(), cur, in_len, config_.normalize ? 1.0f / 255.0f : 1.0f, s), "cast_bytes");
+      unwrap(rh_mark_consumed(context_->raw()), "mark_consumed");  // in_buf may be refilled from here on
     }
     Dims3 dims = config_.in_dims;
     last_alphas_.clear();

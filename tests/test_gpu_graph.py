@@ -348,6 +348,56 @@ def test_u8_frames_and_save_restore(dev):
     w.close()
 
 
+@pytest.mark.parametrize("graph", [False, True])
+def test_u8_frames_loaded_beside_queued_work(dev, graph):
+    """load_frames copies on a stream of its own, after the previous batch's cast has read the staging buffer and
+    beside whatever the main stream still holds: batches alternated without any synchronisation between a load and
+    the queued steps before it give the results of the same batches run one at a time (with recorded steps, where
+    the readers run at replay time, the load waits for the stream instead)."""
+    from rembrandt_amd.operator import SequentialOperatorConfig
+    dims = (24, 24, 3)
+    def make():
+        cfg = SequentialOperatorConfig().data3d(dims, normalize=True).conv2d(dims, 3, 1, 1, 16, "Rect") \
+            .pool2d((24, 24, 16), 2, 2, 0, "Max").affine(12 * 12 * 16, 5, "Identity").softmax_kl_loss(5)
+        w = SequentialOperatorWorker(cfg, 32, "Backward", shared_seed=(9, 10), graph_steps=graph)
+        w.init_params()
+        return w
+    batches = [synth.integers(6, 10 + i, (32, 3, 24, 24), 256).astype(np.uint8) for i in range(3)]
+    labels = synth.integers(6, 20, (32,), 5)
+    # one at a time, with a full synchronisation (the read-back) after every step
+    w = make()
+    sgd = SgdOpt(32, 0.05, ("Update", 0.9), 0.0)
+    sgd.begin(w)
+    w.stage_batch(labels, 1.0 / 32)
+    want = []
+    for step in range(9):
+        w.load_frames_u8(batches[step % 3])
+        loss, _ = sgd.train_batch(w, 32)
+        want.append((loss, w.read(0, "weights").copy(), w.read(-1, "out_act").copy()))
+    w.close()
+    # the same steps, each load issued while the step before it is still queued
+    w = make()
+    sgd = SgdOpt(32, 0.05, ("Update", 0.9), 0.0)
+    sgd.begin(w)
+    w.stage_batch(labels, 1.0 / 32)
+    w.load_frames_u8(batches[0])
+    for step in range(9):
+        w.forward(32, training=True, t=sgd.iter_counter())
+        w.backward(32)
+        sgd.step(w, fused=True)
+        inputs = None
+        if step % 4 == 3:
+            inputs = w.read(-1, "out_act").copy()   # now and then look at what the step consumed
+        if step + 1 < 9:
+            w.load_frames_u8(batches[(step + 1) % 3])   # no synchronisation before this
+        loss = w.store_loss(32)
+        assert loss == want[step][0], "step %d: loss %r vs %r" % (step, loss, want[step][0])
+        if inputs is not None:
+            assert np.array_equal(inputs, want[step][2])
+    assert np.array_equal(w.read(0, "weights"), want[-1][1])
+    w.close()
+
+
 def test_panics(dev):
     from rembrandt_amd.operator import Panic, SequentialOperatorConfig
     cfg = SequentialOperatorConfig().data3d((8, 8, 1)).affine(64, 3, "Identity").softmax_kl_loss(3)
