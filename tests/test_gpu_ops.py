@@ -460,6 +460,28 @@ def test_context_memory_calls(dev):
     _lib.check(lib.rh_ctx_destroy(ctx), "rh_ctx_destroy")
 
 
+def _check_conv_case_all_passes(dev, case, seed, idx):
+    """All three passes, the forced scalar-offset backward-filter and the bf16-operand forward of one geometry."""
+    Nn, C, H, W, K, R, st, pad = case
+    x = synth.normal(seed, idx * 4 + 1, (Nn, C, H, W))
+    w = synth.normal(seed, idx * 4 + 2, (K, C, R, R))
+    b = synth.normal(seed, idx * 4 + 3, (K,))
+    y_ref = O.conv2d_fwd(x, w, st, pad)
+    dy = synth.normal(seed, idx * 4 + 4, y_ref.shape)
+    xd, wd, bd, dyd = T(x, dev), T(w, dev), T(b, dev), T(dy, dev)
+    tag = " %s" % (case,)
+    y = ops.conv2d_fwd(xd, wd, st, pad, bias=bd, relu=True)
+    assert_close(N(y), O.rect_inplace(O.add_bias_nchw(b, y_ref.copy())), "fwd" + tag)
+    y16 = ops.conv2d_fwd(xd, wd, st, pad, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)
+    assert_close(N(y16), O.conv2d_fwd(O.round_bf16(x), O.round_bf16(w), st, pad), "fwd bf16" + tag)
+    dw_ref = O.conv2d_bwd_filter(x, dy, w.shape, st, pad)
+    assert_close(N(ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad)), dw_ref, "bwd_filter" + tag)
+    assert_close(N(ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, algo=_lib.RH_ALGO_SCALAR_OFFSET)), dw_ref,
+                 "bwd_filter scalar-offset" + tag)
+    assert_close(N(ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad)), O.conv2d_bwd_data(w, dy, x.shape, st, pad),
+                 "bwd_data" + tag)
+
+
 def test_conv2d_random_geometries(dev):
     """A seeded sweep over convolution geometries (filter 1-7, stride 1-4, any padding below the filter size, channel
     counts on both sides of every tile and group size): all three passes, the forced scalar-offset backward-filter and
@@ -481,23 +503,36 @@ def test_conv2d_random_geometries(dev):
             continue
         case = (Nn, C, H, W, K, R, st, pad)
         say("random conv case", done, case)
-        x = synth.normal(31, done * 4 + 1, (Nn, C, H, W))
-        w = synth.normal(31, done * 4 + 2, (K, C, R, R))
-        b = synth.normal(31, done * 4 + 3, (K,))
-        y_ref = O.conv2d_fwd(x, w, st, pad)
-        dy = synth.normal(31, done * 4 + 4, y_ref.shape)
-        xd, wd, bd, dyd = T(x, dev), T(w, dev), T(b, dev), T(dy, dev)
-        tag = " %s" % (case,)
-        y = ops.conv2d_fwd(xd, wd, st, pad, bias=bd, relu=True)
-        assert_close(N(y), O.rect_inplace(O.add_bias_nchw(b, y_ref.copy())), "fwd" + tag)
-        y16 = ops.conv2d_fwd(xd, wd, st, pad, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)
-        assert_close(N(y16), O.conv2d_fwd(O.round_bf16(x), O.round_bf16(w), st, pad), "fwd bf16" + tag)
-        dw_ref = O.conv2d_bwd_filter(x, dy, w.shape, st, pad)
-        assert_close(N(ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad)), dw_ref, "bwd_filter" + tag)
-        assert_close(N(ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, algo=_lib.RH_ALGO_SCALAR_OFFSET)), dw_ref,
-                     "bwd_filter scalar-offset" + tag)
-        assert_close(N(ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad)), O.conv2d_bwd_data(w, dy, x.shape, st, pad),
-                     "bwd_data" + tag)
+        _check_conv_case_all_passes(dev, case, 31, done)
+        done += 1
+    torch.cuda.synchronize()
+
+
+def test_conv2d_random_midsize_geometries(dev):
+    """A seeded sweep over layer-sized geometries (16-256 input and 32-512 output channels, planes of 7-56, batches up
+    to 128, capped at 30 GFLOP a pass): grids of tens to over a thousand tiles, so contraction splits, sliced tails in
+    one and in several rounds of tiles, the per-layer loader choice of backward-filter and the stride-2 class
+    decomposition of backward-data are all met at sizes the hand-picked cases do not name."""
+    import random
+    rnd = random.Random(20160418)
+    done = 0
+    while done < 24:
+        R = rnd.choice([1, 3, 3, 3, 5])
+        st = rnd.choice([1, 1, 1, 2])
+        pad = rnd.choice([0, R // 2, R // 2])
+        C = rnd.choice([16, 24, 32, 48, 64, 96, 128, 160, 256])
+        K = rnd.choice([32, 64, 96, 128, 192, 256, 384, 512])
+        H = rnd.randint(7, 56)
+        W = rnd.choice([H, H, rnd.randint(7, 56)])
+        Nn = rnd.choice([8, 16, 24, 32, 52, 64, 100, 128])
+        P, Q = (H + 2 * pad - R) // st + 1, (W + 2 * pad - R) // st + 1
+        if P < 1 or Q < 1:
+            continue
+        while 2.0 * Nn * C * K * R * R * P * Q > 3e10 and Nn > 1:
+            Nn //= 2
+        case = (Nn, C, H, W, K, R, st, pad)
+        say("random mid-size conv case", done, case, "forward tiles", -(-K // 128) * -(-(Nn * P * Q) // 128))
+        _check_conv_case_all_passes(dev, case, 51, done)
         done += 1
     torch.cuda.synchronize()
 
