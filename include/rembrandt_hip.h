@@ -100,6 +100,14 @@ int rh_store_sync(rh_ctx* ctx, void* dst_h, const void* src_d, size_t bytes);
  * ran inside a recorded graph); RH_E_UNSUPPORTED between rh_ctx_begin_capture and rh_ctx_end_capture. */
 int rh_load_overlapped(rh_ctx* ctx, void* dst_d, const void* src_h, size_t bytes);
 int rh_mark_consumed(rh_ctx* ctx);
+/* sync_store of the per-batch results (the predicted categories and the loss, src/operator/loss.rs:170-186, 212-213)
+ * in two halves, so that the host's wait does not have to come before the backward pass is enqueued: rh_store_begin
+ * copies src_d to dst_h on the copy stream as soon as what the context's stream holds now is complete, without
+ * delaying launches made after the call; rh_store_wait blocks until every copy begun so far has landed.  dst_h is
+ * page-locked memory from rh_host_malloc; launches enqueued between the two calls must not write src_d.
+ * RH_E_UNSUPPORTED between rh_ctx_begin_capture and rh_ctx_end_capture. */
+int rh_store_begin(rh_ctx* ctx, void* dst_h, const void* src_d, size_t bytes);
+int rh_store_wait(rh_ctx* ctx);
 int rh_cast_u8_f32(const uint8_t* x, float* y, size_t n, float scale, rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------

@@ -72,6 +72,8 @@ PROTOTYPES = {
                             _vp]),
     "rh_load_overlapped": (_int, [_vp, _vp, _vp, _sz]),
     "rh_mark_consumed": (_int, [_vp]),
+    "rh_store_begin": (_int, [_vp, _vp, _vp, _sz]),
+    "rh_store_wait": (_int, [_vp]),
     "rh_host_malloc": (_int, [_vp, _sz, C.POINTER(_vp)]),
     "rh_host_free": (_int, [_vp, _vp]),
     "rh_bnorm_bwd_relu": (_int, [_int, _int, _int, _f, _f, _vp, _vp, _vp, _f, _f, C.c_double, _vp, _vp, _vp, _vp, _vp, _vp, _vp,

@@ -24,7 +24,28 @@ struct rh_ctx {
   hipStream_t copy = nullptr;
   hipEvent_t ev_copied = nullptr, ev_consumed = nullptr;
   bool consumed_valid = false;  // ev_consumed was recorded after the last reader of the buffer loaded that way
+  // device -> host stores on the copy stream (rh_store_begin / rh_store_wait)
+  hipEvent_t ev_store_ready = nullptr, ev_stored = nullptr;
+  bool store_pending = false;
 };
+
+// The copy stream and its events, created on first use.
+static hipError_t ensure_copy_stream(rh_ctx* ctx) {
+  if (ctx->copy) return hipSuccess;
+  hipError_t e;
+  if ((e = hipSetDevice(ctx->device)) != hipSuccess) return e;
+  hipStream_t s = nullptr;
+  hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
+  if ((e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) != hipSuccess) return e;  // default priority
+  for (int i = 0; i < 4; ++i)
+    if ((e = hipEventCreateWithFlags(&ev[i], hipEventDisableTiming)) != hipSuccess) {
+      for (int j = 0; j < i; ++j) (void)hipEventDestroy(ev[j]);
+      (void)hipStreamDestroy(s);
+      return e;
+    }
+  ctx->copy = s; ctx->ev_copied = ev[0]; ctx->ev_consumed = ev[1]; ctx->ev_store_ready = ev[2]; ctx->ev_stored = ev[3];
+  return hipSuccess;
+}
 
 // A captured and instantiated sequence of launches of one context (both streams).
 struct rh_graph {
@@ -75,6 +96,8 @@ extern "C" int rh_ctx_destroy(rh_ctx* ctx) {
     (void)hipStreamDestroy(ctx->copy);
     (void)hipEventDestroy(ctx->ev_copied);
     (void)hipEventDestroy(ctx->ev_consumed);
+    (void)hipEventDestroy(ctx->ev_store_ready);
+    (void)hipEventDestroy(ctx->ev_stored);
   }
   hipError_t e = hipStreamSynchronize(ctx->stream);
   hipError_t e2 = hipStreamDestroy(ctx->stream);
@@ -261,19 +284,7 @@ extern "C" int rh_load_overlapped(rh_ctx* ctx, void* dst_d, const void* src_h, s
   if (!dst_d || !src_h) return RH_E_INVALID;
   if (ctx->capturing) return RH_E_UNSUPPORTED;
   hipError_t e;
-  if (!ctx->copy) {
-    if ((e = hipSetDevice(ctx->device)) != hipSuccess) return (int)e;
-    hipStream_t s = nullptr;
-    hipEvent_t a = nullptr, b = nullptr;
-    if ((e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) != hipSuccess) return (int)e;  // default priority
-    if ((e = hipEventCreateWithFlags(&a, hipEventDisableTiming)) != hipSuccess ||
-        (e = hipEventCreateWithFlags(&b, hipEventDisableTiming)) != hipSuccess) {
-      (void)hipStreamDestroy(s);
-      if (a) (void)hipEventDestroy(a);
-      return (int)e;
-    }
-    ctx->copy = s; ctx->ev_copied = a; ctx->ev_consumed = b;
-  }
+  if ((e = ensure_copy_stream(ctx)) != hipSuccess) return (int)e;
   if (ctx->consumed_valid) {
     if ((e = hipStreamWaitEvent(ctx->copy, ctx->ev_consumed, 0)) != hipSuccess) return (int)e;
   } else if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) {
@@ -304,6 +315,33 @@ extern "C" int rh_store_sync(rh_ctx* ctx, void* dst_h, const void* src_d, size_t
   hipError_t e = hipMemcpyAsync(dst_h, src_d, bytes, hipMemcpyDeviceToHost, ctx->stream);
   if (e != hipSuccess) return (int)e;
   return (int)hipStreamSynchronize(ctx->stream);
+}
+
+// sync_store in two halves.  rh_store_begin: the copy runs on the copy stream once everything the main stream holds
+// now is complete; the main stream itself does not wait for it, so launches made after this call run on while the
+// copy is under way.  rh_store_wait: blocks the host until every copy begun so far has landed.  The caller keeps
+// src_d unchanged between the two (launches enqueued in between must not write it) and passes page-locked host
+// memory (rh_host_malloc): with pageable memory the runtime may block inside rh_store_begin.
+extern "C" int rh_store_begin(rh_ctx* ctx, void* dst_h, const void* src_d, size_t bytes) {
+  if (!ctx) return RH_E_INVALID;
+  if (bytes == 0) return 0;
+  if (!dst_h || !src_d) return RH_E_INVALID;
+  if (ctx->capturing) return RH_E_UNSUPPORTED;
+  hipError_t e;
+  if ((e = ensure_copy_stream(ctx)) != hipSuccess) return (int)e;
+  if ((e = hipEventRecord(ctx->ev_store_ready, ctx->stream)) != hipSuccess) return (int)e;
+  if ((e = hipStreamWaitEvent(ctx->copy, ctx->ev_store_ready, 0)) != hipSuccess) return (int)e;
+  if ((e = hipMemcpyAsync(dst_h, src_d, bytes, hipMemcpyDeviceToHost, ctx->copy)) != hipSuccess) return (int)e;
+  if ((e = hipEventRecord(ctx->ev_stored, ctx->copy)) != hipSuccess) return (int)e;
+  ctx->store_pending = true;
+  return 0;
+}
+
+extern "C" int rh_store_wait(rh_ctx* ctx) {
+  if (!ctx) return RH_E_INVALID;
+  if (!ctx->store_pending) return 0;
+  ctx->store_pending = false;
+  return (int)hipEventSynchronize(ctx->ev_stored);
 }
 
 // ---- per-launch timing -------------------------------------------------------------------

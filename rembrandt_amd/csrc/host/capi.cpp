@@ -532,9 +532,21 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
         w->seen_steps.insert(key);
       }
     }
-    if (!done) enqueue_step();
-    op->loss_operator(0)->fetch_output_categories(b);
-    const float loss = op->loss_operator(0)->fetch_loss();
+    float loss;
+    if (!done) {
+      // launch by launch: the read-backs are started right behind the loss kernels and waited for after the backward
+      // pass and the update are enqueued, so the host returns (and enqueues the next batch) while those still run
+      op->forward(b, phase);
+      op->loss_operator(0)->enqueue_output_categories(b);
+      op->loss_operator(0)->enqueue_loss(b);
+      op->loss_operator(0)->begin_fetch(b);
+      op->backward(b);
+      s->opt->step(op, fused != 0);
+      loss = op->loss_operator(0)->finish_fetch(b);
+    } else {
+      op->loss_operator(0)->fetch_output_categories(b);
+      loss = op->loss_operator(0)->fetch_loss();
+    }
     const size_t correct = op->loss_operator(0)->accuracy_count(b);
     if (loss_out) *loss_out = loss;
     if (correct_out) *correct_out = (int32_t)correct;

@@ -754,7 +754,9 @@ class Conv2dOperator : public Operator {
       apply_rect_backprop(config_.act_func, out_act_->as_ptr(), out_dims_.len(), batch_size, out_delta_->as_mut_ptr(), s);
     rh_stream_t sg = s;                        // stream and scratch of the two gradient kernels
     DeviceBuffer<uint8_t>* wg = workspace_.get();
-    if (workspace_aux_ && overlap_on_) {
+    // (only where a data gradient follows on the main stream: the first layer's gradient kernels would only queue
+    // behind the second stream's earlier work)
+    if (workspace_aux_ && overlap_on_ && in_delta_) {
       context_->fork();                        // the second stream sees the masked out_delta
       sg = context_->aux_stream();
       wg = workspace_aux_.get();
@@ -1362,7 +1364,8 @@ class BNormConv2dOperator : public BNormUnitsOperator {
     BNormConvUnit& u = units_[0];
     if (!act_bwd_folded_)
       apply_rect_backprop(config_.act_func, out_act_->as_ptr(), u.out_dims.len(), batch_size, out_delta_->as_mut_ptr(), context_->stream());
-    u.backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_, aux_ws());
+    u.backward_params(batch_size, in_act_->as_ptr(), out_delta_->as_ptr(), config_.bnorm_epsilon, *workspace_,
+                      in_delta_ ? aux_ws() : nullptr);  // nothing to overlap with when no data gradient follows
     if (in_delta_) u.backward_data(batch_size, in_delta_->as_mut_ptr(), 0.0f, *workspace_);
   }
   const char* kind() const override { return "BNormConv2dOperator"; }
@@ -1505,7 +1508,7 @@ class SoftmaxKLLossOperator : public LossOperator {
         label_cats_(batch_size, context), label_cats_h_(batch_size, 0), weights_(batch_size, context),
         weights_h_(batch_size, 0.0f), out_values_(loss_config.num_categories * batch_size, context),
         max_value_(batch_size, context), out_cats_(batch_size, context), out_cats_h_(batch_size, 0),
-        out_loss1_(batch_size, context), out_loss_(1, context) {
+        out_loss1_(batch_size, context), out_loss_(1, context), readback_((batch_size + 1) * 4, context) {
     RB_ASSERT(prev_op != nullptr);
     in_act_ = prev_op->get_output_vars();
     if (!in_act_) panic("SoftmaxKLLossOperator missing required prev operator output vars");
@@ -1575,6 +1578,19 @@ class SoftmaxKLLossOperator : public LossOperator {
     RB_ASSERT(batch_size <= batch_cap_);
     out_cats_.sync_store(out_cats_h_.data(), batch_cap_);
   }
+  void begin_fetch(size_t batch_size) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    unwrap(rh_store_begin(context_->raw(), readback_.data(), out_cats_.as_ptr(), batch_cap_ * 4), "store (categories)");
+    unwrap(rh_store_begin(context_->raw(), readback_.data() + batch_cap_ * 4, out_loss_.as_ptr(), 4), "store (loss)");
+  }
+  float finish_fetch(size_t batch_size) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    unwrap(rh_store_wait(context_->raw()), "store wait");
+    std::memcpy(out_cats_h_.data(), readback_.data(), batch_cap_ * 4);
+    float h;
+    std::memcpy(&h, readback_.data() + batch_cap_ * 4, 4);
+    return h;
+  }
   const int32_t* get_output_categories(size_t) const override { return out_cats_h_.data(); }
   size_t accuracy_count(size_t batch_size) const override {
     RB_ASSERT(batch_size <= batch_cap_);
@@ -1603,6 +1619,7 @@ class SoftmaxKLLossOperator : public LossOperator {
   DeviceBuffer<int32_t> out_cats_;
   std::vector<int32_t> out_cats_h_;
   DeviceBuffer<float> out_loss1_, out_loss_;
+  PinnedBytes readback_;  // categories, then the loss: what begin_fetch copies
 };
 
 }  // namespace

@@ -361,6 +361,12 @@ class LossOperator : public Operator {
   virtual float fetch_loss() = 0;
   virtual void enqueue_output_categories(size_t batch_size) = 0;
   virtual void fetch_output_categories(size_t batch_size) = 0;
+  // A third way to read both back: begin_fetch (after the two enqueue_* calls) starts their copies to page-locked
+  // host memory on the context's copy stream, behind the kernels enqueued so far and beside whatever is enqueued
+  // next; finish_fetch waits for the copies only, leaves the categories where get_output_categories finds them and
+  // returns the loss.  The host then runs ahead of the GPU by the work enqueued in between.
+  virtual void begin_fetch(size_t batch_size) = 0;
+  virtual float finish_fetch(size_t batch_size) = 0;
   virtual const int32_t* get_output_categories(size_t batch_size) const = 0;
   virtual size_t accuracy_count(size_t batch_size) const = 0;
 };

@@ -86,6 +86,9 @@ __global__ void pool_fwd_kernel(PoolDims d, const float* __restrict__ x, float* 
 // Forward with the input planes of a block staged in LDS: PB consecutive (n, c) planes are read with coalesced
 // loads, windows are scanned in LDS (overlapping windows re-read LDS, not L1), and y / arg-max are written
 // coalesced.  Same arithmetic and tie rule as pool_fwd_kernel.
+// K, ST > 0 fix the window size and stride at compile time: windows that lie inside the plane (all of them without
+// padding and with an exact cover) are scanned by unrolled code from one base address, in the same order.
+template <int K, int ST>
 __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv dPQ, int PB, long long planes,
                                                            const float* __restrict__ x, float* __restrict__ y,
                                                            int* __restrict__ argmax) {
@@ -118,6 +121,35 @@ __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv d
     dPQ.divmod((uint32_t)o, pl, pq);
     d.dQ.divmod(pq, p, q);
     const float* xp = sx + pl * HW;
+    if constexpr (K > 0) {
+      const int hs = (int)p * ST - d.pad, ws = (int)q * ST - d.pad;
+      if (hs >= 0 && ws >= 0 && hs + K <= d.H && ws + K <= d.W) {
+        const int first = hs * d.W + ws;
+        const float* b = xp + first;
+        if (d.mode == RH_POOL_MAX) {
+          float best = b[0];
+          int bi = 0;
+#pragma unroll
+          for (int r = 0; r < K; ++r)
+#pragma unroll
+            for (int s2 = 0; s2 < K; ++s2) {
+              if (r == 0 && s2 == 0) continue;
+              const float v = b[r * d.W + s2];
+              if (v > best) { best = v; bi = r * d.W + s2; }
+            }
+          gy[o] = best;
+          if (gm) gm[o] = first + bi;
+        } else {
+          float acc = 0.0f;
+#pragma unroll
+          for (int r = 0; r < K; ++r)
+#pragma unroll
+            for (int s2 = 0; s2 < K; ++s2) acc += b[r * d.W + s2];
+          gy[o] = acc * inv;
+        }
+        continue;
+      }
+    }
     if (d.mode == RH_POOL_MAX) {
       float best;
       const int bi = window_argmax(xp, d.H, d.W, (int)p, (int)q, d.k, d.st, d.pad, &best);
@@ -253,6 +285,101 @@ __global__ __launch_bounds__(256) void pool_bwd_mask_lds_kernel(PoolDims d, Fast
   for (int e = head + (n4 << 2) + threadIdx.x; e < n_in; e += 256) gdx[e] = value(e);
 }
 
+// Max-pool backward from the arg-max mask with the windows dealt out by colour.  Windows p and p' of one axis share
+// input rows only if |p - p'| * stride < size, so the windows whose (p mod nA, q mod nA) agree, nA = ceil(size/stride),
+// touch disjoint elements: the block zeroes the dx of its PB planes in LDS, adds every window's dy to the element its
+// mask names, one colour after the other with a barrier between (plain LDS read-add-write, no atomics, fixed sum order:
+// colours in the order (0,0), (0,1), (1,0), (1,1)), and writes the planes out as 16-byte groups.  One pass over dy, the
+// mask and dx and some twenty instructions per window, where the gather form spends sixty per input element.
+// All of a thread's windows (at most J per colour) are loaded before the first barrier.  nA is 1 or 2.
+struct PoolColors {
+  int nA;             // colours per axis
+  int cnt[4];         // windows of one plane in colour (a, b) = cnt[a * 2 + b]
+  int Qb[2];          // windows per row in column colour b
+  FastDiv dCnt[4], dQb[2];
+};
+
+template <int J>
+__global__ __launch_bounds__(256) void pool_bwd_mask_color_kernel(PoolDims d, PoolColors pc, int PB, long long planes,
+                                                                  const float* __restrict__ dy, const int* __restrict__ argmax,
+                                                                  const float* __restrict__ y, float* __restrict__ dx) {
+  extern __shared__ float lds_pool[];
+  const int PQ = d.P * d.Q, HW = d.H * d.W;
+  const long long plane0 = (long long)blockIdx.x * PB;
+  const int np = (int)(planes - plane0 < PB ? planes - plane0 : PB);
+  const int n_in = np * HW;
+  const float* gdy = dy + plane0 * PQ;
+  const int* gm = argmax + plane0 * PQ;
+  const float* gy = y ? y + plane0 * PQ : nullptr;
+  float* gdx = dx + plane0 * HW;
+  // the LDS copy keeps the global address's position inside a 16-byte group
+  const int phase = (int)((reinterpret_cast<uintptr_t>(gdx) >> 2) & 3);
+  float* const sdx = lds_pool + phase;
+
+  int tgt[4][J];    // LDS index of the element a window routes to, -1: none
+  float val[4][J];
+  const int ncol = pc.nA * pc.nA;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+#pragma unroll
+    for (int j = 0; j < J; ++j) { tgt[c][j] = -1; val[c][j] = 0.0f; }
+    if (c < ncol) {
+      const int a = pc.nA == 2 ? c >> 1 : 0, b = pc.nA == 2 ? c & 1 : 0;
+      const int n_c = np * pc.cnt[c];
+#pragma unroll
+      for (int j = 0; j < J; ++j) {
+        const int t = (int)threadIdx.x + 256 * j;
+        if (t < n_c) {
+          uint32_t pl, rem, i, jj;
+          pc.dCnt[c].divmod((uint32_t)t, pl, rem);
+          pc.dQb[b].divmod(rem, i, jj);
+          const int o = (int)pl * PQ + ((int)i * pc.nA + a) * d.Q + (int)jj * pc.nA + b;
+          int m = gm[o];
+          val[c][j] = gdy[o];
+          if (gy && !(gy[o] > 0.0f)) m = -1;  // a window whose maximum is not positive routes nothing
+          tgt[c][j] = (unsigned)m < (unsigned)HW ? (int)pl * HW + m : -1;
+        }
+      }
+    }
+  }
+  {
+    float4* z4 = reinterpret_cast<float4*>(lds_pool);
+    const int nz = (n_in + 4 + 3) >> 2;
+    for (int i = threadIdx.x; i < nz; i += 256) z4[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    if (c < ncol) {
+#pragma unroll
+      for (int j = 0; j < J; ++j)
+        if (tgt[c][j] >= 0) sdx[tgt[c][j]] += val[c][j];
+      __syncthreads();
+    }
+  }
+  const int head = ((4 - phase) & 3) < n_in ? ((4 - phase) & 3) : n_in;
+  if ((int)threadIdx.x < head) gdx[threadIdx.x] = sdx[threadIdx.x];
+  const int n4 = (n_in - head) >> 2;
+  float4* g4 = reinterpret_cast<float4*>(gdx + head);
+  const float4* s4 = reinterpret_cast<const float4*>(sdx + head);
+  for (int g = threadIdx.x; g < n4; g += 256) g4[g] = s4[g];
+  for (int e = head + (n4 << 2) + threadIdx.x; e < n_in; e += 256) gdx[e] = sdx[e];
+}
+
+// Launches one instantiation of the LDS forward; RH_E_UNSUPPORTED when the block's LDS cannot be had.
+template <int K, int ST>
+static int launch_pool_fwd_lds(const PoolDims& d, FastDiv dPQ, int PB, long long planes, long long blocks, size_t lds_bytes,
+                               const float* x, float* y, int32_t* argmax, rh_stream_t stream) {
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_fwd_lds_kernel<K, ST>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    if (attr != hipSuccess) return RH_E_UNSUPPORTED;
+  }
+  hipLaunchKernelGGL((pool_fwd_lds_kernel<K, ST>), dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d, dPQ, PB,
+                     planes, x, y, argmax);
+  return launch_status();
+}
+
 static int pool_dims(const rh_pool_geom* g, PoolDims* d) {
   if (!g) return RH_E_INVALID;
   if (g->N <= 0 || g->C <= 0 || g->H <= 0 || g->W <= 0 || g->size <= 0 || g->stride <= 0 || g->pad < 0)
@@ -301,16 +428,14 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
     const long long planes = (long long)d.N * d.C;
     const long long blocks = cdiv<long long>(planes, PB);
     const size_t lds_bytes = ((size_t)PB * d.H * d.W + 4) * sizeof(float);
-    bool lds_ok = true;
-    if (lds_bytes > 48 * 1024) {
-      static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_fwd_lds_kernel),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-      lds_ok = attr == hipSuccess;
-    }
-    if (lds_ok && blocks < (1ll << 31) && (long long)PB * d.P * d.Q < (1ll << 31)) {
-      hipLaunchKernelGGL(pool_fwd_lds_kernel, dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d,
-                         FastDiv((uint32_t)(d.P * d.Q)), PB, planes, x, y, opt_argmax);
-      return launch_status();
+    if (blocks < (1ll << 31) && (long long)PB * d.P * d.Q < (1ll << 31)) {
+      const FastDiv dPQ((uint32_t)(d.P * d.Q));
+      int e;
+      if (d.k == 3 && d.st == 2)      e = launch_pool_fwd_lds<3, 2>(d, dPQ, PB, planes, blocks, lds_bytes, x, y, opt_argmax, stream);
+      else if (d.k == 2 && d.st == 2) e = launch_pool_fwd_lds<2, 2>(d, dPQ, PB, planes, blocks, lds_bytes, x, y, opt_argmax, stream);
+      else if (d.k == 3 && d.st == 1) e = launch_pool_fwd_lds<3, 1>(d, dPQ, PB, planes, blocks, lds_bytes, x, y, opt_argmax, stream);
+      else                            e = launch_pool_fwd_lds<0, 0>(d, dPQ, PB, planes, blocks, lds_bytes, x, y, opt_argmax, stream);
+      if (e != RH_E_UNSUPPORTED) return e;
     }
   }
   const dim3 grid((unsigned)cdiv<long long>(total, 256) > (1u << 20) ? (1u << 20) : (unsigned)cdiv<long long>(total, 256));
@@ -324,8 +449,69 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
 // The dy and mask of at least one whole plane must fit the block's LDS (8 bytes per pooled element, 32 KB at most).
 static bool lds_bwd_ok(const PoolDims& d) { return d.P * d.Q <= 4096 && d.H * d.W <= (1 << 20); }
 
+// The colour form: one or two colours per axis, a plane's dx within 60 KB of LDS, at most 8 windows per thread and
+// colour.  Returns RH_E_UNSUPPORTED when the geometry is outside that.
+template <int J>
+static int launch_pool_bwd_color_j(const PoolDims& d, const PoolColors& pc, int PB, long long planes, long long blocks,
+                                   size_t lds_bytes, const float* dy, const int32_t* argmax, const float* relu_y, float* dx,
+                                   rh_stream_t stream) {
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_bwd_mask_color_kernel<J>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    if (attr != hipSuccess) return RH_E_UNSUPPORTED;
+  }
+  hipLaunchKernelGGL((pool_bwd_mask_color_kernel<J>), dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d, pc, PB,
+                     planes, dy, argmax, relu_y, dx);
+  return launch_status();
+}
+
+static int launch_pool_bwd_color(const PoolDims& d, const float* dy, const int32_t* argmax, const float* relu_y, float* dx,
+                                 rh_stream_t stream) {
+  const int nA = cdiv(d.k, d.st);
+  const int HW = d.H * d.W;
+  if (nA > 2 || HW > 15000 || d.P * d.Q <= 0) return RH_E_UNSUPPORTED;
+  PoolColors pc;
+  pc.nA = nA;
+  int most = 0;
+  for (int a = 0; a < 2; ++a)
+    for (int b = 0; b < 2; ++b) {
+      const int Pa = a < nA && a < d.P ? (d.P - a + nA - 1) / nA : 0;
+      const int Qb = b < nA && b < d.Q ? (d.Q - b + nA - 1) / nA : 0;
+      const int c = nA == 2 ? a * 2 + b : 0;
+      if (nA == 1 && (a || b)) continue;
+      pc.cnt[c] = Pa * Qb;
+      pc.dCnt[c] = FastDiv((uint32_t)(pc.cnt[c] > 0 ? pc.cnt[c] : 1));
+      pc.Qb[b] = Qb;
+      pc.dQb[b] = FastDiv((uint32_t)(Qb > 0 ? Qb : 1));
+      if (pc.cnt[c] > most) most = pc.cnt[c];
+    }
+  if (nA == 1) {
+    for (int c = 1; c < 4; ++c) { pc.cnt[c] = 0; pc.dCnt[c] = FastDiv(1u); }
+    pc.Qb[1] = 0; pc.dQb[1] = FastDiv(1u);
+  }
+  if (most <= 0 || most > 256 * 8) return RH_E_UNSUPPORTED;
+  // planes per block: about 256 windows of the largest colour and 16 KB of dx
+  int PB = 256 / most;
+  if (PB > 4096 / HW) PB = 4096 / HW;
+  if (PB < 1) PB = 1;
+  if (PB > 64) PB = 64;
+  const int per_thread = cdiv(PB * most, 256);
+  const long long planes = (long long)d.N * d.C;
+  const long long blocks = cdiv<long long>(planes, PB);
+  if (blocks >= (1ll << 31)) return RH_E_LIMIT;
+  const size_t lds_bytes = ((size_t)PB * HW + 8) * sizeof(float);
+  if (per_thread <= 1) return launch_pool_bwd_color_j<1>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
+  if (per_thread <= 2) return launch_pool_bwd_color_j<2>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
+  if (per_thread <= 4) return launch_pool_bwd_color_j<4>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
+  return launch_pool_bwd_color_j<8>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
+}
+
 static int launch_pool_bwd_lds(const PoolDims& d, const float* dy, const int32_t* argmax, const float* relu_y, float* dx,
                                rh_stream_t stream) {
+  {
+    const int e = launch_pool_bwd_color(d, dy, argmax, relu_y, dx, stream);
+    if (e != RH_E_UNSUPPORTED) return e;
+  }
   const int PQ = d.P * d.Q;
   int PB = 2048 / PQ;
   if (PB > 64) PB = 64;

@@ -57,6 +57,8 @@ extern "C" {
   pub fn rh_free(ctx: *mut rh_ctx, dptr: *mut c_void) -> c_int;
   pub fn rh_load_overlapped(ctx: *mut rh_ctx, dst_d: *mut c_void, src_h: *const c_void, bytes: size_t) -> c_int;
   pub fn rh_mark_consumed(ctx: *mut rh_ctx) -> c_int;
+  pub fn rh_store_begin(ctx: *mut rh_ctx, dst_h: *mut c_void, src_d: *const c_void, bytes: size_t) -> c_int;
+  pub fn rh_store_wait(ctx: *mut rh_ctx) -> c_int;
   pub fn rh_host_malloc(ctx: *mut rh_ctx, bytes: size_t, hptr: *mut *mut c_void) -> c_int;
   pub fn rh_host_free(ctx: *mut rh_ctx, hptr: *mut c_void) -> c_int;
   pub fn rh_memset_f32(d: *mut f32, value: c_float, n: size_t, stream: rh_stream_t) -> c_int;
