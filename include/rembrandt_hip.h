@@ -65,7 +65,7 @@ typedef struct rh_ctx rh_ctx;
 int rh_ctx_create(int device, rh_ctx** out);
 int rh_ctx_destroy(rh_ctx* ctx);
 rh_stream_t rh_ctx_stream(rh_ctx* ctx);
-int rh_ctx_sync(rh_ctx* ctx);                       /* both streams */
+int rh_ctx_sync(rh_ctx* ctx);                       /* every stream of the context */
 /* A second stream of the context (default priority, created on first use) for launches that may overlap the main
  * stream's, e.g. a layer's filter gradient beside its data gradient.  rh_ctx_fork: the second stream waits for what
  * the main stream holds now; rh_ctx_join: the main stream waits for what the second holds now.  No host blocking. */

@@ -113,7 +113,13 @@ extern "C" int rh_ctx_sync(rh_ctx* ctx) {
     hipError_t e = hipStreamSynchronize(ctx->aux);
     if (e != hipSuccess) return (int)e;
   }
-  return (int)hipStreamSynchronize(ctx->stream);
+  hipError_t e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) return (int)e;
+  if (ctx->copy) {  // after the main stream: a store begun with rh_store_begin waits for a point of it
+    if ((e = hipStreamSynchronize(ctx->copy)) != hipSuccess) return (int)e;
+    ctx->store_pending = false;
+  }
+  return 0;
 }
 
 extern "C" rh_stream_t rh_ctx_aux_stream(rh_ctx* ctx) {
