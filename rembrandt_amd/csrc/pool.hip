@@ -21,8 +21,9 @@ inline int pool_out_dim(int in, int size, int stride, int pad, int round) {
   return t / stride;
 }
 
+// `xp[i - base]` holds plane element i (base > 0: only the rows from base / W on are staged).
 __device__ __forceinline__ int window_argmax(const float* __restrict__ xp, int H, int W, int p, int q, int k, int st,
-                                             int pad, float* best_out) {
+                                             int pad, float* best_out, int base = 0) {
   float best = 0.0f;
   int bi = -1;
   const int hs = p * st - pad, ws = q * st - pad;
@@ -32,7 +33,7 @@ __device__ __forceinline__ int window_argmax(const float* __restrict__ xp, int H
     for (int s = 0; s < k; ++s) {
       const int w = ws + s;
       if ((unsigned)w >= (unsigned)W) continue;
-      const float v = xp[h * W + w];
+      const float v = xp[h * W + w - base];
       if (bi < 0 || v > best) { best = v; bi = h * W + w; }
     }
   }
@@ -88,16 +89,32 @@ __global__ void pool_fwd_kernel(PoolDims d, const float* __restrict__ x, float* 
 // coalesced.  Same arithmetic and tie rule as pool_fwd_kernel.
 // K, ST > 0 fix the window size and stride at compile time: windows that lie inside the plane (all of them without
 // padding and with an exact cover) are scanned by unrolled code from one base address, in the same order.
+// Planes above the block's LDS share are cut into bands of `rb` output rows (bands > 1, PB = 1): a block stages the
+// input rows its band's windows reach, a contiguous piece of the plane.
 template <int K, int ST>
-__global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv dPQ, int PB, long long planes,
-                                                           const float* __restrict__ x, float* __restrict__ y,
-                                                           int* __restrict__ argmax) {
+__global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv dPQ, int PB, long long planes, int bands, int rb,
+                                                           FastDiv dBands, const float* __restrict__ x,
+                                                           float* __restrict__ y, int* __restrict__ argmax) {
   extern __shared__ float lds_pool[];
   const int HW = d.H * d.W, PQ = d.P * d.Q;
-  const long long plane0 = (long long)blockIdx.x * PB;
-  const int np = (int)(planes - plane0 < PB ? planes - plane0 : PB);
-  const float* gx = x + plane0 * HW;
-  const int n_in = np * HW, n_out = np * PQ;
+  long long plane0 = (long long)blockIdx.x * PB;
+  int np = (int)(planes - plane0 < PB ? planes - plane0 : PB);
+  int p0 = 0, h_lo = 0, n_in = np * HW, n_out = np * PQ;
+  if (bands > 1) {
+    uint32_t pl, bd;
+    dBands.divmod(blockIdx.x, pl, bd);
+    plane0 = pl;
+    np = 1;
+    p0 = (int)bd * rb;
+    const int p1 = p0 + rb < d.P ? p0 + rb : d.P;
+    h_lo = p0 * d.st - d.pad > 0 ? p0 * d.st - d.pad : 0;
+    int h_hi = (p1 - 1) * d.st - d.pad + d.k < d.H ? (p1 - 1) * d.st - d.pad + d.k : d.H;
+    if (h_hi < h_lo) h_hi = h_lo;
+    n_in = (h_hi - h_lo) * d.W;
+    n_out = (p1 - p0) * d.Q;
+  }
+  const int base = h_lo * d.W;
+  const float* gx = x + plane0 * HW + base;
   // The staged copy keeps the global address's position inside a 16-byte group, so that the body of the copy
   // is float4 on both sides whatever the plane size (55*55 floats is not a multiple of four).
   const int phase = (int)((reinterpret_cast<uintptr_t>(gx) >> 2) & 3);
@@ -113,19 +130,19 @@ __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv d
     for (int i = h + (n4 << 2) + threadIdx.x; i < n_in; i += 256) sx[i] = gx[i];
   }
   __syncthreads();
-  float* gy = y + plane0 * PQ;
-  int* gm = argmax ? argmax + plane0 * PQ : nullptr;
+  float* gy = y + plane0 * PQ + p0 * d.Q;
+  int* gm = argmax ? argmax + plane0 * PQ + p0 * d.Q : nullptr;
   const float inv = 1.0f / (float)(d.k * d.k);
   for (int o = threadIdx.x; o < n_out; o += 256) {
-    uint32_t pl, pq, p, q;
-    dPQ.divmod((uint32_t)o, pl, pq);
+    uint32_t pl = 0, pq = (uint32_t)(o + p0 * d.Q), p, q;
+    if (bands <= 1) dPQ.divmod((uint32_t)o, pl, pq);
     d.dQ.divmod(pq, p, q);
     const float* xp = sx + pl * HW;
     if constexpr (K > 0) {
       const int hs = (int)p * ST - d.pad, ws = (int)q * ST - d.pad;
       if (hs >= 0 && ws >= 0 && hs + K <= d.H && ws + K <= d.W) {
         const int first = hs * d.W + ws;
-        const float* b = xp + first;
+        const float* b = xp + (first - base);
         if (d.mode == RH_POOL_MAX) {
           float best = b[0];
           int bi = 0;
@@ -152,7 +169,7 @@ __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv d
     }
     if (d.mode == RH_POOL_MAX) {
       float best;
-      const int bi = window_argmax(xp, d.H, d.W, (int)p, (int)q, d.k, d.st, d.pad, &best);
+      const int bi = window_argmax(xp, d.H, d.W, (int)p, (int)q, d.k, d.st, d.pad, &best, base);
       gy[o] = bi < 0 ? 0.0f : best;
       if (gm) gm[o] = bi;
     } else {
@@ -163,7 +180,7 @@ __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv d
         if ((unsigned)h >= (unsigned)d.H) continue;
         for (int s2 = 0; s2 < d.k; ++s2) {
           const int w = ws + s2;
-          if ((unsigned)w < (unsigned)d.W) acc += xp[h * d.W + w];
+          if ((unsigned)w < (unsigned)d.W) acc += xp[h * d.W + w - base];
         }
       }
       gy[o] = acc * inv;
@@ -369,14 +386,14 @@ __global__ __launch_bounds__(256) void pool_bwd_mask_color_kernel(PoolDims d, Po
 // Launches one instantiation of the LDS forward; RH_E_UNSUPPORTED when the block's LDS cannot be had.
 template <int K, int ST>
 static int launch_pool_fwd_lds(const PoolDims& d, FastDiv dPQ, int PB, long long planes, long long blocks, size_t lds_bytes,
-                               const float* x, float* y, int32_t* argmax, rh_stream_t stream) {
+                               int bands, int rb, const float* x, float* y, int32_t* argmax, rh_stream_t stream) {
   if (lds_bytes > 48 * 1024) {
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_fwd_lds_kernel<K, ST>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
     if (attr != hipSuccess) return RH_E_UNSUPPORTED;
   }
   hipLaunchKernelGGL((pool_fwd_lds_kernel<K, ST>), dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d, dPQ, PB,
-                     planes, x, y, argmax);
+                     planes, bands, rb, FastDiv((uint32_t)bands), x, y, argmax);
   return launch_status();
 }
 
@@ -418,23 +435,33 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
   ProfScope prof(d.mode == RH_POOL_MAX ? "pool_max_fwd" : "pool_avg_fwd",
                  4.0 * ((double)d.N * d.C * d.H * d.W + (double)total * (opt_argmax ? 2 : 1)), to_stream(stream));
   const long long in_total = (long long)d.N * d.C * d.H * d.W;
-  // about 16 KB of input planes per block (measured best: more LDS per block leaves too few blocks per CU to
-  // overlap one block's loads with another's window scans); a single larger plane still goes through LDS
+  // about 16 KB of input per block (measured best: more LDS per block leaves too few blocks per CU to overlap one
+  // block's loads with another's window scans): several small planes, one plane, or a band of a larger plane's
+  // output rows with the input rows its windows reach
   constexpr int kLdsFloats = 4096;
-  if (d.H * d.W <= 16000 && d.P * d.Q > 0) {  // up to 112 x 112 and a little more: 62.5 KB of LDS, two blocks per CU
-    int PB = kLdsFloats / (d.H * d.W);
-    if (PB < 1) PB = 1;
-    if (PB > 64) PB = 64;
+  if (d.P * d.Q > 0 && (long long)d.W * d.k <= 15000) {
+    const int HW = d.H * d.W;
     const long long planes = (long long)d.N * d.C;
-    const long long blocks = cdiv<long long>(planes, PB);
-    const size_t lds_bytes = ((size_t)PB * d.H * d.W + 4) * sizeof(float);
+    int PB = 1, bands = 1, rb = d.P, rows_in = d.H;
+    if (HW <= kLdsFloats) {
+      PB = kLdsFloats / HW;
+      if (PB > 64) PB = 64;
+    } else {
+      const int rows_fit = kLdsFloats / d.W;  // input rows in the block's share (at least one window's)
+      rb = rows_fit > d.k ? (rows_fit - d.k) / d.st + 1 : 1;
+      if (rb > d.P) rb = d.P;
+      bands = cdiv(d.P, rb);
+      rows_in = (rb - 1) * d.st + d.k < d.H ? (rb - 1) * d.st + d.k : d.H;
+    }
+    const long long blocks = bands > 1 ? planes * bands : cdiv<long long>(planes, PB);
+    const size_t lds_bytes = ((size_t)(bands > 1 ? rows_in * d.W : PB * HW) + 4) * sizeof(float);
     if (blocks < (1ll << 31) && (long long)PB * d.P * d.Q < (1ll << 31)) {
       const FastDiv dPQ((uint32_t)(d.P * d.Q));
       int e;
-      if (d.k == 3 && d.st == 2)      e = launch_pool_fwd_lds<3, 2>(d, dPQ, PB, planes, blocks, lds_bytes, x, y, opt_argmax, stream);
-      else if (d.k == 2 && d.st == 2) e = launch_pool_fwd_lds<2, 2>(d, dPQ, PB, planes, blocks, lds_bytes, x, y, opt_argmax, stream);
-      else if (d.k == 3 && d.st == 1) e = launch_pool_fwd_lds<3, 1>(d, dPQ, PB, planes, blocks, lds_bytes, x, y, opt_argmax, stream);
-      else                            e = launch_pool_fwd_lds<0, 0>(d, dPQ, PB, planes, blocks, lds_bytes, x, y, opt_argmax, stream);
+      if (d.k == 3 && d.st == 2)      e = launch_pool_fwd_lds<3, 2>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, opt_argmax, stream);
+      else if (d.k == 2 && d.st == 2) e = launch_pool_fwd_lds<2, 2>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, opt_argmax, stream);
+      else if (d.k == 3 && d.st == 1) e = launch_pool_fwd_lds<3, 1>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, opt_argmax, stream);
+      else                            e = launch_pool_fwd_lds<0, 0>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, opt_argmax, stream);
       if (e != RH_E_UNSUPPORTED) return e;
     }
   }

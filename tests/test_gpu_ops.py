@@ -185,8 +185,9 @@ POOL_CASES = [
     # N, C, H, size, stride, pad
     (2, 3, 9, 3, 2, 0), (2, 3, 9, 3, 2, 1), (3, 4, 8, 2, 2, 0), (2, 2, 10, 3, 2, 0), (2, 5, 27, 3, 2, 0),
     (1, 2, 6, 6, 1, 0), (2, 3, 7, 3, 1, 1), (2, 2, 13, 3, 3, 1),
-    (1, 3, 112, 3, 2, 1),   # a plane above 48 KB, still staged in LDS
-    (1, 2, 130, 3, 2, 0),   # a plane too large for LDS
+    (1, 3, 112, 3, 2, 1),   # planes above a block's LDS share: forward in bands of output rows, backward with
+    (1, 2, 130, 3, 2, 0),   # several windows per thread and colour / (130: above 60 KB) by the gather kernel
+    (1, 1, 20, 7, 3, 2),    # three colours per axis: gather backward
 ]
 
 
