@@ -752,20 +752,22 @@ class Conv2dOperator : public Operator {
     rh_stream_t s = context_->stream();
     if (!act_bwd_folded_)
       apply_rect_backprop(config_.act_func, out_act_->as_ptr(), out_dims_.len(), batch_size, out_delta_->as_mut_ptr(), s);
-    rh_stream_t sg = s;                        // stream and scratch of the two gradient kernels
-    DeviceBuffer<uint8_t>* wg = workspace_.get();
-    // (only where a data gradient follows on the main stream: the first layer's gradient kernels would only queue
-    // behind the second stream's earlier work)
-    if (workspace_aux_ && overlap_on_ && in_delta_) {
+    // Streams and scratch of the two gradient kernels.  With a data gradient to follow on the main stream both go
+    // to the second stream; the first layer has none, so its filter gradient stays on the main stream (on the second
+    // it would only queue behind that stream's earlier work) and the bias gradient runs beside it.
+    rh_stream_t s_filter = s, s_bias = s;
+    DeviceBuffer<uint8_t>*w_filter = workspace_.get(), *w_bias = workspace_.get();
+    if (workspace_aux_ && overlap_on_) {
       context_->fork();                        // the second stream sees the masked out_delta
-      sg = context_->aux_stream();
-      wg = workspace_aux_.get();
+      s_bias = context_->aux_stream();
+      w_bias = workspace_aux_.get();
+      if (in_delta_) { s_filter = s_bias; w_filter = w_bias; }
     }
     unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in_act_->as_ptr(), out_delta_->as_ptr(), 1.0f, params_.grad_weights->as_mut_ptr(),
-                                wg->as_mut_ptr(), wg->len(), 0, sg), "conv2d backward filter");
+                                w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter");
     unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), 1.0f,
-                                 out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), wg->as_mut_ptr(),
-                                 wg->len(), sg), "conv2d backward bias");
+                                 out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
+                                 w_bias->len(), s_bias), "conv2d backward bias");
     if (in_delta_) {
       unwrap(rh_conv2d_bwd_data(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
                                 workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward data");
