@@ -784,7 +784,12 @@ class Conv2dOperator : public Operator {
   size_t decode_params(const uint8_t* blob, size_t len) override { return params_.decode_params(blob, len, kind()); }
   void encode_state(std::vector<uint8_t>& blob) override { params_.encode_state(blob); }
   size_t decode_state(const uint8_t* blob, size_t len) override { return params_.decode_state(blob, len, kind()); }
-  void fused_sgd_step(float l2, float scale, float mu, float apply) override { params_.fused_sgd_step(l2, scale, mu, apply); }
+  // Like the affine layers' updates, on the second stream, except for the first layer: the next forward pass joins
+  // in front of the first operator that was updated there, and the first layer's forward is what the others hide behind.
+  void fused_sgd_step(float l2, float scale, float mu, float apply) override {
+    params_.fused_sgd_step(l2, scale, mu, apply, updates_on_second_stream() ? context_->aux_stream() : nullptr);
+  }
+  bool updates_on_second_stream() const override { return workspace_aux_ && overlap_on_ && in_delta_; }
   bool buffer(int which, float** ptr, size_t* len) override {
     if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
     if (which == 1) { *ptr = out_delta_->as_mut_ptr(); *len = out_delta_->len(); return true; }
