@@ -618,6 +618,10 @@ class AffineOperator : public Operator {
       ws = std::max(ws, rh_sgemm_workspace_bytes(i, b, o));
     }
     if (ws) workspace_.reset(new DeviceBuffer<uint8_t>(ws, context));
+    if (overlap_built_) {
+      const size_t wa = rh_sgemm_workspace_bytes((int)config_.in_channels, (int)config_.out_channels, (int)batch_size);
+      if (wa) workspace_aux_.reset(new DeviceBuffer<uint8_t>(wa, context));
+    }
   }
   size_t batch_size() const override { return batch_cap_; }
   SharedDeviceBuf get_output_vars() const override { return out_act_; }
@@ -641,11 +645,22 @@ class AffineOperator : public Operator {
     const int i = (int)config_.in_channels, o = (int)config_.out_channels, b = (int)batch_size;
     rh_stream_t s = context_->stream();
     apply_rect_backprop(config_.act_func, out_act_->as_ptr(), config_.out_channels, batch_size, out_delta_->as_mut_ptr(), s);
+    // The two parameter gradients go to the second stream when a data gradient follows on the main stream (scratch
+    // of their own there); the worker joins at the end of backward.
+    rh_stream_t sg = s;
+    void* wg = ws_ptr();
+    size_t wg_len = ws_len();
+    if (overlap_on_ && in_delta_) {
+      context_->fork();
+      sg = context_->aux_stream();
+      wg = workspace_aux_ ? workspace_aux_->as_mut_ptr() : nullptr;
+      wg_len = workspace_aux_ ? workspace_aux_->len() : 0;
+    }
     // grad_weights(in, out) += in_act(in, B) * out_delta(out, B)^T
     unwrap(rh_sgemm(0, 1, i, o, b, 1.0f, in_act_->as_ptr(), i, out_delta_->as_ptr(), o, 1.0f,
-                    params_.grad_weights->as_mut_ptr(), i, ws_ptr(), ws_len(), 0, s), "matrix_prod");
+                    params_.grad_weights->as_mut_ptr(), i, wg, wg_len, 0, sg), "matrix_prod");
     // grad_bias(1, out) += 1(1, B) * out_delta^T: the column sums of out_delta, without the ones vector
-    unwrap(rh_conv2d_bwd_bias(b, o, 1, 1.0f, out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), s), "matrix_prod");
+    unwrap(rh_conv2d_bwd_bias(b, o, 1, 1.0f, out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), sg), "matrix_prod");
     if (in_delta_) {
       // in_delta(in, B) = weights(in, out) * out_delta(out, B)
       unwrap(rh_sgemm(0, 0, i, b, o, 1.0f, params_.weights->as_ptr(), i, out_delta_->as_ptr(), o, 0.0f,
@@ -683,8 +698,8 @@ class AffineOperator : public Operator {
   Ctx context_;
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   ParamTensors params_;
-  std::unique_ptr<DeviceBuffer<uint8_t>> workspace_;
-  bool overlap_built_, overlap_on_;  // fused SGD step of this (large) parameter block on the second stream
+  std::unique_ptr<DeviceBuffer<uint8_t>> workspace_, workspace_aux_;
+  bool overlap_built_, overlap_on_;  // parameter gradients and the fused SGD step of this block on the second stream
 };
 
 // ---- Conv2dOperator -------------------------------------------------------------------------------------
