@@ -1190,14 +1190,15 @@ struct BNormConvUnit {
     if (!backward) return;
     scal(0.0f, *grad_weights); scal(0.0f, *scale_grad); scal(0.0f, *bias_grad);
   }
-  void fused_sgd_step(float l2, float sc, float momentum, float apply) {
+  void fused_sgd_step(float l2, float sc, float momentum, float apply, rh_stream_t st = nullptr) {
     RB_ASSERT(backward);
+    if (!st) st = s();
     unwrap(rh_sgd_momentum_step((int64_t)wlen, weights->as_mut_ptr(), grad_weights->as_mut_ptr(), acc_grad_weights->as_mut_ptr(),
-                                l2, sc, momentum, apply, 1, s()), "rh_sgd_momentum_step");
+                                l2, sc, momentum, apply, 1, st), "rh_sgd_momentum_step");
     unwrap(rh_sgd_momentum_step((int64_t)chans, scale->as_mut_ptr(), scale_grad->as_mut_ptr(), acc_scale_grad->as_mut_ptr(),
-                                0.0f, sc, momentum, apply, 1, s()), "rh_sgd_momentum_step");
+                                0.0f, sc, momentum, apply, 1, st), "rh_sgd_momentum_step");
     unwrap(rh_sgd_momentum_step((int64_t)chans, bias->as_mut_ptr(), bias_grad->as_mut_ptr(), acc_bias_grad->as_mut_ptr(),
-                                0.0f, sc, momentum, apply, 1, s()), "rh_sgd_momentum_step");
+                                0.0f, sc, momentum, apply, 1, st), "rh_sgd_momentum_step");
   }
   // Blobs: filter as (size*size*in channels, out channels), then four (1, out channels) rows
   // (src/operator/conv.rs:361-406 params: scale, bias, moving mean, moving inverse deviation;
@@ -1292,7 +1293,12 @@ class BNormUnitsOperator : public Operator {
   void save_params() override { for (auto& u : units_) u.save_params(); }
   void restore_params() override { for (auto& u : units_) u.restore_params(); }
   void reset() override { for (auto& u : units_) u.reset(); }
-  void fused_sgd_step(float l2, float scale, float mu, float apply) override { for (auto& u : units_) u.fused_sgd_step(l2, scale, mu, apply); }
+  // On the second stream, like the plain convolution layers' updates, except for the network's first layer.
+  void fused_sgd_step(float l2, float scale, float mu, float apply) override {
+    rh_stream_t st = updates_on_second_stream() ? context_->aux_stream() : nullptr;
+    for (auto& u : units_) u.fused_sgd_step(l2, scale, mu, apply, st);
+  }
+  bool updates_on_second_stream() const override { return workspace_aux_ && overlap_on_ && in_delta_; }
   void encode_params(std::vector<uint8_t>& blob) override { for (auto& u : units_) u.encode_params(blob); }
   size_t decode_params(const uint8_t* blob, size_t len) override {
     size_t off = 0;
