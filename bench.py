@@ -24,9 +24,9 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # the same run (FETCH_SIZE reads 0.5 KiB per KiB copied -> x2.0, WRITE_SIZE 1.0 -> x1.0).  A counter run
 # cannot be nested inside this process, so the figures are carried here and named in `traffic_source`.
 MEASURED_TRAFFIC_BYTES = {
-    "alexnet": {"conv_bwd_filter_128x128": 1024 * (2.0 * 191940 + 62256),
-                "conv_fwd_128x128": 1024 * (2.0 * 68640 + 139477),
-                "conv_bwd_data_128x128": 1024 * (2.0 * 63334 + 84376)},
+    "alexnet": {"conv_bwd_filter_128x128": 1024 * (2.0 * 192077 + 62256),
+                "conv_fwd_128x128": 1024 * (2.0 * 68551 + 139719),
+                "conv_bwd_data_128x128": 1024 * (2.0 * 63353 + 84292)},
 }
 
 BATCH = {"alexnet": 256, "lenet": 64, "cifar10": 128, "nin": 128, "resnet18": 256}
