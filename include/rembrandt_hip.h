@@ -129,6 +129,11 @@ int32_t rh_conv2d_out_dim(int32_t in, int32_t size, int32_t stride, int32_t pad)
 /* Bytes of scratch the given pass needs whatever flags it is called with (0 is possible).  The scratch must be
  * 256-byte aligned. */
 size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass);
+/* The same for a scratch buffer that is allocated once and then used with every batch 1..g->N, the way the
+ * reference's operators size theirs for batch_cap (src/operator/mod.rs:1493-1507): the largest need of any such
+ * batch.  The need is not monotone in N (a pass with few result tiles cuts its contraction into slices and keeps
+ * their partial sums in the scratch), so this can exceed rh_conv2d_workspace_bytes of g itself. */
+size_t rh_conv2d_workspace_bytes_upto(const rh_conv_geom* g, int pass);
 /* y = alpha * corr(x, w) + beta * y.  With RH_FUSE_BIAS, `bias` (length K) is added after the
  * alpha/beta blend; with RH_FUSE_RELU the result is clamped at 0.  bias may be NULL otherwise. */
 int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x, const float* w, float beta,
@@ -144,6 +149,7 @@ int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alpha, const f
 /* Same result through a two-stage reduction that fills the GPU when K is small (scratch from the caller;
  * without scratch it falls back to the one-stage form). */
 size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane);
+size_t rh_conv2d_bwd_bias_workspace_bytes_upto(int32_t N, int32_t K, int32_t plane); /* largest need of N' = 1..N */
 int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
                           float* db, void* ws, size_t ws_bytes, rh_stream_t stream);
 /* dx = alpha * corr^T(dy, w) + beta * dx. */
@@ -174,6 +180,9 @@ void rembrandt_kernel_batch_map_rect_backprop_inplace(const float* y, int32_t fr
  * GPU split the contraction across blocks and reduce in a fixed order; without it (ws == NULL)
  * the same result is computed unsplit. */
 size_t rh_sgemm_workspace_bytes(int32_t m, int32_t n, int32_t k);
+/* Largest need when one extent varies from 1 up to the value given (which: 0 = m, 1 = n, 2 = k): the affine
+ * operators call with the batch as n (forward, data gradient) or k (weight gradient) and any batch <= batch_cap. */
+size_t rh_sgemm_workspace_bytes_upto(int32_t m, int32_t n, int32_t k, int which);
 int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k, float alpha, const float* A,
              int32_t lda, const float* B, int32_t ldb, float beta, float* C, int32_t ldc, void* ws,
              size_t ws_bytes, int flags, rh_stream_t stream);
@@ -298,6 +307,7 @@ int rh_lrn_bwd(const rh_lrn_geom* g, const float* x, const float* y, const float
  * RH_FUSE_RELU (forward only) clamps the blended result at 0: the in-place ReLU that follows the call in the
  * reference (src/operator/conv.rs:538-551).  `ws` needs rh_bnorm_workspace_bytes(N, C, plane) bytes. */
 size_t rh_bnorm_workspace_bytes(int N, int C, int plane);
+size_t rh_bnorm_workspace_bytes_upto(int N, int C, int plane); /* largest need of N' = 1..N */
 int rh_bnorm_fwd_train(int N, int C, int plane, float alpha, const float* x, float beta, float* y, double ema_factor,
                        double epsilon, const float* scale, const float* bias, float* running_mean, float* running_ivar,
                        float* cached_mean, float* cached_ivar, void* ws, size_t ws_bytes, int flags, rh_stream_t stream);

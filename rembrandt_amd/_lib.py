@@ -80,6 +80,10 @@ PROTOTYPES = {
                                  _sz, _vp]),
     "rh_conv2d_out_dim": (_i32, [_i32, _i32, _i32, _i32]),
     "rh_conv2d_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _int]),
+    "rh_conv2d_workspace_bytes_upto": (_sz, [C.POINTER(ConvGeom), _int]),
+    "rh_conv2d_bwd_bias_workspace_bytes_upto": (_sz, [_i32, _i32, _i32]),
+    "rh_sgemm_workspace_bytes_upto": (_sz, [_i32, _i32, _i32, _int]),
+    "rh_bnorm_workspace_bytes_upto": (_sz, [_int, _int, _int]),
     "rh_conv2d_fwd": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _vp, _sz, _int, _vp]),
     "rh_conv2d_bwd_filter": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _sz, _int, _vp]),
     "rh_conv2d_bwd_bias": (_int, [_i32, _i32, _i32, _f, _vp, _f, _vp, _vp]),

@@ -256,6 +256,15 @@ extern "C" size_t rh_bnorm_workspace_bytes(int N, int C, int plane) {
   return bn_part_bytes(p, C) + (((size_t)C * sizeof(float4) + 255) & ~(size_t)255);
 }
 
+extern "C" size_t rh_bnorm_workspace_bytes_upto(int N, int C, int plane) {
+  size_t need = 256;
+  for (int n = N; n >= 1; --n) {
+    const size_t b = rh_bnorm_workspace_bytes(n, C, plane);
+    if (b > need) need = b;
+  }
+  return need;
+}
+
 extern "C" int rh_bnorm_fwd_train(int N, int C, int plane, float alpha, const float* x, float beta, float* y,
                                   double ema_factor, double epsilon, const float* scale, const float* bias,
                                   float* running_mean, float* running_ivar, float* cached_mean, float* cached_ivar,

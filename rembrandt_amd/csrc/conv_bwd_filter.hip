@@ -501,6 +501,18 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
   }
 }
 
+extern "C" size_t rh_conv2d_workspace_bytes_upto(const rh_conv_geom* g, int pass) {
+  if (!g) return 0;
+  rh_conv_geom h = *g;
+  size_t need = 0;
+  for (int n = g->N; n >= 1; --n) {
+    h.N = n;
+    const size_t b = rh_conv2d_workspace_bytes(&h, pass);
+    if (b > need) need = b;
+  }
+  return need;
+}
+
 extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const float* x, const float* dy,
                                     float beta, float* dw, void* ws, size_t ws_bytes, int flags,
                                     rh_stream_t stream_) {
@@ -600,15 +612,20 @@ extern "C" size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32
   return align256(sizeof(float) * (size_t)N * K);
 }
 
-extern "C" int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
-                                     float* db, void* ws, size_t ws_bytes, void* stream_) {
-  if (N <= 0 || K <= 0 || plane <= 0 || !dy || !db) return RH_E_INVALID;
-  const size_t need = rh_conv2d_bwd_bias_workspace_bytes(N, K, plane);
-  if (plane == 1 || need == 0 || !ws || ws_bytes < need) return rh_conv2d_bwd_bias(N, K, plane, alpha, dy, beta, db, stream_);
-  hipStream_t stream = to_stream(stream_);
-  float* rowsum = static_cast<float*>(ws);
+extern "C" size_t rh_conv2d_bwd_bias_workspace_bytes_upto(int32_t N, int32_t K, int32_t plane) {
+  size_t need = 0;
+  for (int n = N; n >= 1; --n) {
+    const size_t b = rh_conv2d_bwd_bias_workspace_bytes(n, K, plane);
+    if (b > need) need = b;
+  }
+  return need;
+}
+
+// Both stages of the bias gradient with scratch `rowsum` of rh_conv2d_bwd_bias_workspace_bytes(N, K, plane) bytes.
+// Every scratch element that the second stage reads is written by the first: nothing has to start at zero.
+static int bwd_bias_two_stage(int N, int K, int plane, float alpha, const float* dy, float beta, float* db, float* rowsum,
+                              hipStream_t stream) {
   const long long rows = (long long)N * K;
-  ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
   if (plane < kBiasSmallPlane && (long long)K * plane < (1ll << 31)) {
     const int KP = K * plane, G = bwd_bias_col_groups(N, KP);
     if (KP % 4 == 0 && ((reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(rowsum)) & 15) == 0)
@@ -628,11 +645,8 @@ extern "C" int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float 
   return launch_status();
 }
 
-extern "C" int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy,
-                                  float beta, float* db, rh_stream_t stream_) {
-  if (N <= 0 || K <= 0 || plane <= 0 || !dy || !db) return RH_E_INVALID;
-  hipStream_t stream = to_stream(stream_);
-  ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
+static int bwd_bias_one_stage(int N, int K, int plane, float alpha, const float* dy, float beta, float* db,
+                              hipStream_t stream) {
   if (plane == 1) {
     hipLaunchKernelGGL(bwd_bias_rows_kernel, dim3(cdiv(K, 64)), dim3(256), 0, stream, dy, N, K, alpha, beta,
                        db);
@@ -640,4 +654,22 @@ extern "C" int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alp
     hipLaunchKernelGGL(bwd_bias_kernel, dim3(K), dim3(1024), 0, stream, dy, N, K, plane, alpha, beta, db);
   }
   return launch_status();
+}
+
+extern "C" int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
+                                     float* db, void* ws, size_t ws_bytes, void* stream_) {
+  if (N <= 0 || K <= 0 || plane <= 0 || !dy || !db) return RH_E_INVALID;
+  const size_t need = rh_conv2d_bwd_bias_workspace_bytes(N, K, plane);
+  if (plane == 1 || need == 0 || !ws || ws_bytes < need) return rh_conv2d_bwd_bias(N, K, plane, alpha, dy, beta, db, stream_);
+  hipStream_t stream = to_stream(stream_);
+  ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
+  return bwd_bias_two_stage(N, K, plane, alpha, dy, beta, db, static_cast<float*>(ws), stream);
+}
+
+extern "C" int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy,
+                                  float beta, float* db, rh_stream_t stream_) {
+  if (N <= 0 || K <= 0 || plane <= 0 || !dy || !db) return RH_E_INVALID;
+  hipStream_t stream = to_stream(stream_);
+  ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
+  return bwd_bias_one_stage(N, K, plane, alpha, dy, beta, db, stream);
 }

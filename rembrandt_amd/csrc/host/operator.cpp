@@ -211,6 +211,17 @@ namespace {
 
 typedef std::shared_ptr<DeviceContext> Ctx;
 
+// Scratch is allocated once for batch_cap, but a pass may be called with any batch <= batch_cap and the library's
+// plans are not monotone in the batch (fewer result tiles make it cut the contraction into more slices, whose partial
+// sums can need more room than the full batch does): every scratch buffer is sized with the *_upto functions.
+size_t conv_ws_upto(const rh_conv_geom& g, int pass) { return rh_conv2d_workspace_bytes_upto(&g, pass); }
+size_t bias_ws_upto(int batch, int K, int plane) { return rh_conv2d_bwd_bias_workspace_bytes_upto(batch, K, plane); }
+size_t bnorm_ws_upto(int batch, int C, int plane) { return rh_bnorm_workspace_bytes_upto(batch, C, plane); }
+// The affine GEMMs of a layer (out, B, in), (in, out, B), (in, B, out): B is the batch.
+size_t sgemm_ws_upto(int m, int n, int k, int batch_dim /* 1 = n is the batch, 2 = k is */, int /*batch*/) {
+  return rh_sgemm_workspace_bytes_upto(m, n, k, batch_dim);
+}
+
 struct ParamTensors {
   std::unique_ptr<DeviceBuffer<float>> weights, bias;
   // backward-capable operators only
@@ -612,14 +623,14 @@ class AffineOperator : public Operator {
     out_delta_.reset(new DeviceBuffer<float>(config.out_channels * batch_size, context));
     params_.alloc(config.in_channels * config.out_channels, config.out_channels, backward_enabled(capability), context);
     const int i = (int)config.in_channels, o = (int)config.out_channels, b = (int)batch_size;
-    size_t ws = rh_sgemm_workspace_bytes(o, b, i);
+    size_t ws = sgemm_ws_upto(o, b, i, 1, b);
     if (backward_enabled(capability)) {
-      ws = std::max(ws, rh_sgemm_workspace_bytes(i, o, b));
-      ws = std::max(ws, rh_sgemm_workspace_bytes(i, b, o));
+      ws = std::max(ws, sgemm_ws_upto(i, o, b, 2, b));
+      ws = std::max(ws, sgemm_ws_upto(i, b, o, 1, b));
     }
     if (ws) workspace_.reset(new DeviceBuffer<uint8_t>(ws, context));
     if (overlap_built_) {
-      const size_t wa = rh_sgemm_workspace_bytes((int)config_.in_channels, (int)config_.out_channels, (int)batch_size);
+      const size_t wa = sgemm_ws_upto(i, o, b, 2, b);
       if (wa) workspace_aux_.reset(new DeviceBuffer<uint8_t>(wa, context));
     }
   }
@@ -720,17 +731,17 @@ class Conv2dOperator : public Operator {
                   backward_enabled(capability), context);
     // one scratch buffer sized for the largest of the three passes (src/operator/mod.rs:1493-1507)
     const rh_conv_geom g = geom(batch_size);
-    size_t ws = rh_conv2d_workspace_bytes(&g, RH_CONV_FWD);
+    size_t ws = conv_ws_upto(g, RH_CONV_FWD);
     if (backward_enabled(capability)) {
-      ws = std::max(ws, rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_FILTER));
-      ws = std::max(ws, rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_DATA));
-      ws = std::max(ws, rh_conv2d_bwd_bias_workspace_bytes(g.N, g.K, (int)(out_dims_.w * out_dims_.h)));
+      ws = std::max(ws, conv_ws_upto(g, RH_CONV_BWD_FILTER));
+      ws = std::max(ws, conv_ws_upto(g, RH_CONV_BWD_DATA));
+      ws = std::max(ws, bias_ws_upto(g.N, g.K, (int)(out_dims_.w * out_dims_.h)));
     }
     workspace_.reset(new DeviceBuffer<uint8_t>(std::max<size_t>(ws, 256), context));
     if (backward_enabled(capability) && opts.overlap_backward) {
       // the filter / bias gradients run on the second stream with scratch of their own
-      size_t wa = rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_FILTER);
-      wa = std::max(wa, rh_conv2d_bwd_bias_workspace_bytes(g.N, g.K, (int)(out_dims_.w * out_dims_.h)));
+      size_t wa = conv_ws_upto(g, RH_CONV_BWD_FILTER);
+      wa = std::max(wa, bias_ws_upto(g.N, g.K, (int)(out_dims_.w * out_dims_.h)));
       workspace_aux_.reset(new DeviceBuffer<uint8_t>(std::max<size_t>(wa, 256), context));
     }
   }
@@ -1058,10 +1069,10 @@ struct BNormConvUnit {
   int plane() const { return (int)(out_dims.w * out_dims.h); }
   size_t workspace_bytes() const {
     const rh_conv_geom g = geom(batch_cap);
-    size_t ws = std::max(rh_conv2d_workspace_bytes(&g, RH_CONV_FWD), rh_bnorm_workspace_bytes(g.N, g.K, plane()));
+    size_t ws = std::max(conv_ws_upto(g, RH_CONV_FWD), bnorm_ws_upto(g.N, g.K, plane()));
     if (backward) {
-      ws = std::max(ws, rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_FILTER));
-      ws = std::max(ws, rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_DATA));
+      ws = std::max(ws, conv_ws_upto(g, RH_CONV_BWD_FILTER));
+      ws = std::max(ws, conv_ws_upto(g, RH_CONV_BWD_DATA));
     }
     return ws;
   }
@@ -1140,7 +1151,7 @@ struct BNormConvUnit {
   }
   size_t aux_workspace_bytes() const {
     const rh_conv_geom g = geom(batch_cap);
-    return rh_conv2d_workspace_bytes(&g, RH_CONV_BWD_FILTER);
+    return conv_ws_upto(g, RH_CONV_BWD_FILTER);
   }
   // in_delta = beta*in_delta + dconv^T(weights, pre_delta)
   void backward_data(size_t batch, float* in_delta, float beta, DeviceBuffer<uint8_t>& ws) {

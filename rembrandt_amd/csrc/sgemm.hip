@@ -140,6 +140,16 @@ extern "C" size_t rh_sgemm_workspace_bytes(int32_t m, int32_t n, int32_t k) {
   return align256(sizeof(float) * (size_t)p.splits * m * n);
 }
 
+extern "C" size_t rh_sgemm_workspace_bytes_upto(int32_t m, int32_t n, int32_t k, int which) {
+  size_t need = 0;
+  const int top = which == 0 ? m : which == 1 ? n : which == 2 ? k : 0;
+  for (int v = top; v >= 1; --v) {
+    const size_t b = rh_sgemm_workspace_bytes(which == 0 ? v : m, which == 1 ? v : n, which == 2 ? v : k);
+    if (b > need) need = b;
+  }
+  return need;
+}
+
 extern "C" int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k, float alpha, const float* A,
                         int32_t lda, const float* B, int32_t ldb, float beta, float* C, int32_t ldc,
                         void* ws, size_t ws_bytes, int flags, rh_stream_t stream_) {

@@ -37,7 +37,13 @@ FULL_CONV = {
     "sweep_b_alexnet_conv3": (256, 256, 13, 13, 384, 3, 1, 1),
     "sweep_c_1x1": (128, 96, 55, 55, 96, 1, 1, 0),
     "alexnet_conv1": (256, 3, 227, 227, 96, 11, 4, 0),
+    "alexnet_conv4": (256, 384, 13, 13, 384, 3, 1, 1),
     "alexnet_conv5": (256, 384, 13, 13, 256, 3, 1, 1),
+    # NIN at batch 128: the 3x3 layer into 1024 channels on 6x6, its 1x1 successors (1024 -> 1024 -> 1000), a mid-network 1x1
+    "nin_conv4_1024": (128, 384, 6, 6, 1024, 3, 1, 1),
+    "nin_cccp7": (128, 1024, 6, 6, 1024, 1, 1, 0),
+    "nin_cccp8": (128, 1024, 6, 6, 1000, 1, 1, 0),
+    "nin_cccp3": (128, 256, 27, 27, 256, 1, 1, 0),
     # ResNet-18 template at batch 64: 64-row tiles with the halved K step (784 tiles), contraction cut into slices
     # (7x7 and 14x14 extents), a strided 3x3 layer and a strided 1x1 projection
     "resnet_56_64": (64, 64, 56, 56, 64, 3, 1, 1),
@@ -157,8 +163,9 @@ def test_pool2d_full_size(dev, shape, mode):
 
 
 @pytest.mark.parametrize("case", [(1, 0, 4096, 256, 9216), (0, 1, 9216, 4096, 256), (0, 0, 9216, 256, 4096),
-                                  (1, 0, 1000, 256, 4096)],
-                         ids=["fc6_fwd", "fc6_bwd_w", "fc6_bwd_x", "fc8_fwd"])
+                                  (1, 0, 1000, 256, 4096), (1, 0, 4096, 256, 4096), (0, 1, 4096, 4096, 256),
+                                  (0, 0, 4096, 256, 4096)],
+                         ids=["fc6_fwd", "fc6_bwd_w", "fc6_bwd_x", "fc8_fwd", "fc7_fwd", "fc7_bwd_w", "fc7_bwd_x"])
 def test_sgemm_full_size(dev, case):
     """The AlexNet affine GEMMs (column-major, as the operator issues them) against numpy fp64."""
     ta, tb, m, n, k = case

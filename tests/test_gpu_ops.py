@@ -83,6 +83,11 @@ def test_conv2d_all_passes(dev, case, algo):
     dw0 = synth.normal(11, 6, w.shape)
     dwa = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, alpha=1.0, beta=1.0, dw=T(dw0, dev), algo=algo)
     assert_close(N(dwa), O.conv2d_bwd_filter(x, dy, w.shape, st, pad, 1.0, 1.0, dw0.copy()), "conv bwd filter beta=1")
+    # the scaled accumulation of the gen-2 layers: backward(batch, scale) passes `scale` as alpha (src/layer_new.rs:1093-1101)
+    dws = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, alpha=0.25, beta=1.0, dw=T(dw0, dev), algo=algo)
+    assert_close(N(dws), O.conv2d_bwd_filter(x, dy, w.shape, st, pad, 0.25, 1.0, dw0.copy()), "conv bwd filter alpha=0.25 beta=1")
+    dws = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, alpha=-3.0, beta=0.5, dw=T(dw0, dev), algo=algo)
+    assert_close(N(dws), O.conv2d_bwd_filter(x, dy, w.shape, st, pad, -3.0, 0.5, dw0.copy()), "conv bwd filter alpha=-3 beta=0.5")
 
     db = ops.conv2d_bwd_bias(dyd)
     assert_close(N(db), O.conv2d_bwd_bias(dy), "conv bwd bias")

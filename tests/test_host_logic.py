@@ -65,6 +65,43 @@ def test_workspace_and_shape_helpers():
     assert fwd >= 2400 * 16 and bwd >= 6400 * 20 and bwf > fwd
 
 
+def test_scratch_sized_once_covers_every_smaller_batch():
+    """Operators allocate scratch once for batch_cap and then run any batch <= batch_cap (partial last batches,
+    src/operator/mod.rs:1664,1722).  The need of a pass is not monotone in the batch, so the operators size with the
+    *_upto functions: for every layer of the four networks and every batch up to the capacity the per-call need must
+    fit, and the non-monotone case that made this necessary must still exist (else the *_upto functions are moot)."""
+    lib = _lib.lib()
+    non_monotone = 0
+    for name, cap in (("lenet", 128), ("cifar10", 128), ("alexnet", 256), ("nin", 256)):
+        for l in configs.NETWORKS[name]()[1]:
+            if l[0] == "conv2d":
+                (w, h, c), k, st, pad, out = l[1], l[2], l[3], l[4], l[5]
+                g = _lib.ConvGeom(cap, c, h, w, out, k, k, st, pad)
+                for ps in (_lib.RH_CONV_FWD, _lib.RH_CONV_BWD_FILTER, _lib.RH_CONV_BWD_DATA):
+                    room = lib.rh_conv2d_workspace_bytes_upto(C.byref(g), ps)
+                    at_cap = lib.rh_conv2d_workspace_bytes(C.byref(g), ps)
+                    assert room >= at_cap and room % 256 == 0
+                    for n in range(1, cap + 1):
+                        gn = _lib.ConvGeom(n, c, h, w, out, k, k, st, pad)
+                        need = lib.rh_conv2d_workspace_bytes(C.byref(gn), ps)
+                        assert need <= room, (name, l, ps, n)
+                        non_monotone += need > at_cap
+                P = lib.rh_conv2d_out_dim(h, k, st, pad) * lib.rh_conv2d_out_dim(w, k, st, pad)
+                room = lib.rh_conv2d_bwd_bias_workspace_bytes_upto(cap, out, P)
+                assert all(lib.rh_conv2d_bwd_bias_workspace_bytes(n, out, P) <= room for n in range(1, cap + 1))
+            elif l[0] == "affine":
+                i, o = l[1], l[2]
+                for (m, n, k, which) in ((o, cap, i, 1), (i, o, cap, 2), (i, cap, o, 1)):
+                    room = lib.rh_sgemm_workspace_bytes_upto(m, n, k, which)
+                    for b in range(1, cap + 1):
+                        need = lib.rh_sgemm_workspace_bytes(m, b, k) if which == 1 else lib.rh_sgemm_workspace_bytes(m, n, b)
+                        assert need <= room, (name, l, which, b)
+    assert non_monotone > 0
+    for (C_, plane) in ((64, 56 * 56), (512, 49)):
+        room = lib.rh_bnorm_workspace_bytes_upto(256, C_, plane)
+        assert all(lib.rh_bnorm_workspace_bytes(n, C_, plane) <= room for n in range(1, 257))
+
+
 def test_rng_is_a_pure_function_of_seed_stream_index():
     a = synth.normal(5, 7, (1000,))
     assert np.array_equal(a, synth.normal(5, 7, (1000,)))
