@@ -152,6 +152,17 @@ size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane);
 size_t rh_conv2d_bwd_bias_workspace_bytes_upto(int32_t N, int32_t K, int32_t plane); /* largest need of N' = 1..N */
 int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
                           float* db, void* ws, size_t ws_bytes, rh_stream_t stream);
+/* rh_conv2d_bwd_bias_ws without the scratch argument and without any allocation.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory or hand over a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The scratch of the two-stage reduction lives in an
+ * 8 MiB device array inside the library (rh_noalloc_scratch_bytes(); every GPU the library is used on holds its own
+ * copy until the process ends), whose address is looked up once per device by rh_ctx_create, or by the first call on
+ * a device with that device current.  Geometries whose scratch need (rh_conv2d_bwd_bias_workspace_bytes) exceeds the
+ * array return RH_E_LIMIT.  All calls on one GPU share the array: calls that overlap in time on one GPU (different
+ * streams, different threads) race; order them.  Nothing in the array has to be cleared between calls. */
+size_t rh_noalloc_scratch_bytes(void);
+int rh_conv2d_bwd_bias_noalloc(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
+                               float* db, rh_stream_t stream);
 /* dx = alpha * corr^T(dy, w) + beta * dx. */
 int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const float* w, const float* dy,
                        float beta, float* dx, void* ws, size_t ws_bytes, int flags,

@@ -73,4 +73,8 @@ struct ProfScope {
 };
 extern bool g_profile_enabled;
 
+// Per-device address of the library's static scratch array (see rh_conv2d_bwd_bias_noalloc); looks it up on the
+// current device the first time.  `out` may be null.
+int static_scratch_lookup(void** out);
+
 }  // namespace rh

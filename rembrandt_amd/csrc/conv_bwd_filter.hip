@@ -4,6 +4,8 @@
 // pixel range is cut into `splits` contiguous slices computed by different blocks; each slice
 // writes its partial filter gradient to scratch and a second kernel adds the slices in a fixed
 // order (results do not depend on scheduling).
+#include <mutex>
+
 #include "conv_common.h"
 
 namespace rh {
@@ -664,6 +666,52 @@ extern "C" int rh_conv2d_bwd_bias_ws(int32_t N, int32_t K, int32_t plane, float 
   hipStream_t stream = to_stream(stream_);
   ProfScope prof("bwd_bias", 4.0 * (double)N * K * plane, stream);
   return bwd_bias_two_stage(N, K, plane, alpha, dy, beta, db, static_cast<float*>(ws), stream);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------------------------
+// The scratch of the two-stage bias gradient in a device array that is part of the library's code object: each GPU
+// the library runs on holds its own 8 MiB copy from the first use of the library on it until the process ends.
+// `scratch` names the array for the device compiler only; host code uses the per-device address that
+// hipGetSymbolAddress returns.
+constexpr size_t kStaticScratchBytes = size_t(8) << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr[kMaxDevices];   // per device, set once under g_scratch_mutex
+static std::mutex g_scratch_mutex;
+
+namespace rh {
+// Address of `scratch` on the current device; looked up once per device (from rh_ctx_create, or on the first call of
+// rh_conv2d_bwd_bias_noalloc on a device whose context was made elsewhere).
+int static_scratch_lookup(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return RH_E_LIMIT;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p || (reinterpret_cast<uintptr_t>(p) & 255)) return RH_E_INVALID;
+    g_scratch_ptr[dev] = p;
+  }
+  if (out) *out = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace rh
+
+extern "C" size_t rh_noalloc_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int rh_conv2d_bwd_bias_noalloc(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy, float beta,
+                                          float* db, rh_stream_t stream_) {
+  if (N <= 0 || K <= 0 || plane <= 0 || !dy || !db) return RH_E_INVALID;
+  hipStream_t stream = to_stream(stream_);
+  const size_t need = rh_conv2d_bwd_bias_workspace_bytes(N, K, plane);
+  if (plane == 1 || need == 0) return bwd_bias_one_stage(N, K, plane, alpha, dy, beta, db, stream);  // needs no scratch
+  if (need > kStaticScratchBytes) return RH_E_LIMIT;
+  void* ptr = nullptr;
+  if (int e = static_scratch_lookup(&ptr)) return e;
+  return bwd_bias_two_stage(N, K, plane, alpha, dy, beta, db, static_cast<float*>(ptr), stream);
 }
 
 extern "C" int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy,

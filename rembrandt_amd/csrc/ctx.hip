@@ -75,6 +75,8 @@ extern "C" int rh_ctx_create(int device, rh_ctx** out) {
   if (e != hipSuccess) return (int)e;
   if (device < 0 || device >= count) return RH_E_INVALID;
   if ((e = hipSetDevice(device)) != hipSuccess) return (int)e;
+  // set-up of the entry point that must not allocate: the address of the static scratch array on this device
+  if (int se = rh::static_scratch_lookup(nullptr)) return se;
   rh_ctx* c = new rh_ctx;
   c->device = device;
   // default priority, non-blocking with respect to the legacy default stream
