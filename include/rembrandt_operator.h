@@ -164,6 +164,23 @@ int rho_worker_update_params2(rho_worker* w, float grad_scale, float update_scal
 int rho_worker_save_params(rho_worker* w);
 int rho_worker_restore_params(rho_worker* w);
 int rho_worker_reset(rho_worker* w);
+/* The second-generation layer / arch API over the same chain (src/layer_new.rs:43-60, src/arch_new.rs:527-552), where
+ * the gradient buffers double as the momentum buffers:
+ *   rho_worker_backward_scaled  PipelineArchWorker::backward(batch, scale): `scale` multiplies the filter and bias
+ *                               gradients a convolution accumulates (layer_new.rs:1093-1108); affine layers accumulate
+ *                               with factor 1 whatever it is (layer_new.rs:583-584); the loss layer ignores it (:1933)
+ *   rho_worker_descend          g += l2*W (weights and bias, if l2 > 0); W -= scale*g   (layer_new.rs:596-617,1133-1154)
+ *                               fused != 0: one pass per tensor instead of the BLAS-1 pair
+ *   rho_worker_reset_gradients  g *= momentum                                            (layer_new.rs:589-594)
+ *   rho_worker_reset_loss / _accumulate_loss / _store_accumulated_loss
+ *                               the loss summed over batches on the device (layer_new.rs:2103-2134)
+ * Batch-normalised operators have no second-generation counterpart and panic in descend / reset_gradients. */
+int rho_worker_backward_scaled(rho_worker* w, int32_t batch_size, float scale);
+int rho_worker_descend(rho_worker* w, float scale, float l2_reg_coef, int fused);
+int rho_worker_reset_gradients(rho_worker* w, float momentum);
+int rho_worker_reset_loss(rho_worker* w, int32_t batch_size);
+int rho_worker_accumulate_loss(rho_worker* w, int32_t batch_size);
+int rho_worker_store_accumulated_loss(rho_worker* w, float* out);
 /* Device view of one buffer of hidden operator `hidden_idx` (-1: input operator's out_act,
  * hidden_count: the loss operator's probabilities).  Returns RHO_E_PANIC if there is no such buffer. */
 int rho_worker_buffer(rho_worker* w, int32_t hidden_idx, int which, float** dptr, int64_t* len);
@@ -183,6 +200,19 @@ int rho_sgd_step_size_at(rho_sgd* s, int64_t t, float* out);                 /* 
 /* One whole training step on a staged batch, in the order of SgdOpt::train (new.rs:325-343 + the
  * update block): forward, store_output_categories, store_loss, backward, accuracy_count, step. */
 int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused, float* loss_out, int32_t* correct_out);
+
+/* ---- SgdOptimization::train, the second-generation minibatch block (src/opt_new.rs:279-325) ----
+ * rho_sgd2_begin: reset_gradients(0), reset_loss.  rho_sgd2_batch: forward(Training) -> backward(batch, 1.0) ->
+ * accumulate_loss on a staged batch (per-sample weights 1.0, staged by the caller).  rho_sgd2_end_minibatch:
+ * descend(step_size.at_iter(t) / minibatch_size, l2) -> reset_gradients(momentum) -> t += 1. */
+typedef struct rho_sgd2 rho_sgd2;
+int rho_sgd2_new(int32_t minibatch_size, int step_kind, const float* steps, const int64_t* step_iters, float momentum,
+                 float l2_reg_coef, rho_sgd2** out);
+int rho_sgd2_free(rho_sgd2* s);
+int rho_sgd2_begin(rho_sgd2* s, rho_worker* w);
+int rho_sgd2_batch(rho_sgd2* s, rho_worker* w, int32_t batch_size);
+int rho_sgd2_end_minibatch(rho_sgd2* s, rho_worker* w, int fused);
+int rho_sgd2_iter_counter(rho_sgd2* s, int64_t* out);
 
 /* ---- data sources (src/data_new.rs:282-357, 648-883) ----
  * source: "mnist" (idx3-ubyte frames + idx1-ubyte labels) or "cifar10" (3073-byte records: label, 3 planes of 32x32).

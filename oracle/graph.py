@@ -11,6 +11,10 @@ operator, same method names and the same order of operations as the Rust sources
                                             src/operator/mod.rs:1178-1236, 1355-1363
   SequentialOperatorWorker fan-out ........ src/operator/worker.rs:356-477
   SgdOpt update block ..................... src/opt/sgd/new.rs:345-495, 623-633
+  second-generation layer methods backward(batch, scale), descend, reset_gradients
+                                            src/layer_new.rs:537-617, 1044-1154
+  PipelineArchWorker fan-out .............. src/arch_new.rs:527-552
+  SgdOptimization minibatch block ......... src/opt_new.rs:279-325
   BNormConv2d / StackResConv2d / ProjStackResConv2d operators
                                             src/operator/conv.rs:461-912, 1497-2182, 2935-3560
 
@@ -69,6 +73,21 @@ class _Params:
         O.sscal(0.0, self.grad_weights)
         O.sscal(0.0, self.grad_bias)
 
+    # second generation: the gradient buffers double as the momentum buffers
+    def descend(self, scale, l2):
+        """g += l2*W (weights and bias); W -= scale*g: layer_new.rs:596-617 (affine), 1133-1154 (conv)."""
+        assert l2 >= 0.0
+        if l2 > 0.0:
+            O.saxpy(l2, self.weights, self.grad_weights)
+            O.saxpy(l2, self.bias, self.grad_bias)
+        O.saxpy(-scale, self.grad_weights, self.weights)
+        O.saxpy(-scale, self.grad_bias, self.bias)
+
+    def reset_gradients(self, scale):
+        """g *= scale: layer_new.rs:589-594, 1126-1131."""
+        O.sscal(scale, self.grad_weights)
+        O.sscal(scale, self.grad_bias)
+
 
 class Conv2dOperator:
     kind = "Conv2dOperator"
@@ -98,15 +117,18 @@ class Conv2dOperator:
             O.rect_inplace(self.out_act)
         return self.out_act
 
-    def backward(self, want_in_delta):
+    def backward(self, want_in_delta, scale=1.0):
+        """`scale`: the alpha of backward_filter / backward_bias; 1 in the operator generation (mod.rs:1765-1781), the
+        caller's `scale` in Conv2dLayer::backward (layer_new.rs:1093-1108)."""
         if self.act == "Rect":
             O.rect_backprop_inplace(self.out_act, self.out_delta)
         if self.fast:
+            assert scale == 1.0
             O.fast_conv2d_bwd_filter(self.in_act, self.out_delta, self.p.grad_weights, self.stride, self.pad)
         else:
-            O.conv2d_bwd_filter(self.in_act, self.out_delta, self.p.weights.shape, self.stride, self.pad, 1.0, 1.0,
+            O.conv2d_bwd_filter(self.in_act, self.out_delta, self.p.weights.shape, self.stride, self.pad, scale, 1.0,
                                 self.p.grad_weights)
-        O.conv2d_bwd_bias(self.out_delta, 1.0, 1.0, self.p.grad_bias)
+        O.conv2d_bwd_bias(self.out_delta, scale, 1.0, self.p.grad_bias)
         if not want_in_delta:
             return None
         if self.fast:
@@ -136,7 +158,8 @@ class AffineOperator:
             O.rect_inplace(self.out_act)
         return self.out_act
 
-    def backward(self, want_in_delta):
+    def backward(self, want_in_delta, scale=1.0):
+        """AffineLayer::backward takes `scale` and accumulates both gradients with factor 1.0 (layer_new.rs:583-584)."""
         if self.act == "Rect":
             O.rect_backprop_inplace(self.out_act, self.out_delta)
         if self.fast:
@@ -527,6 +550,29 @@ class SequentialOperatorWorker:
             op.out_delta = np.ascontiguousarray(delta.reshape(op.out_act.shape))
             delta = op.backward(want_in_delta=i > 0)  # the input operator exposes no deltas (mod.rs:632-634)
 
+    def backward_scaled(self, scale):
+        """PipelineArchWorker::backward(batch, scale), arch_new.rs:534-539: the loss layer ignores the scale
+        (layer_new.rs:1933); operators with parameters receive it, the others have nothing to scale."""
+        delta = O.softmax_kl_backward(self.out_values, self.labels, self.weights)
+        for i in range(len(self.hidden) - 1, -1, -1):
+            op = self.hidden[i]
+            op.out_delta = np.ascontiguousarray(delta.reshape(op.out_act.shape))
+            if op.kind in ("Conv2dOperator", "AffineOperator"):
+                delta = op.backward(want_in_delta=i > 0, scale=scale)
+            else:
+                delta = op.backward(want_in_delta=i > 0)
+
+    def descend(self, scale, l2): self._each("descend", scale, l2)              # arch_new.rs:541-545
+    def reset_gradients(self, momentum): self._each("reset_gradients", momentum)  # arch_new.rs:547-551
+
+    # second-generation loss bookkeeping, layer_new.rs:2103-2134: out_loss sums the batches until reset_loss
+    def reset_loss(self):
+        self.acc_loss = np.zeros((1,), np.float32)
+
+    def accumulate_loss(self):
+        loss1 = O.softmax_kl_loss1(self.out_values, self.labels, self.weights)
+        O.blockreduce_sum(loss1.reshape(1, -1), 1.0, self.acc_loss)
+
     def _each(self, fn, *a):
         for op in self.hidden:
             if op.p is not None:
@@ -592,3 +638,29 @@ class SgdOpt:
         op.reset()
         if self.kind == "UpdateNesterov":
             op.update_params(mu)
+
+
+class SgdOptimization:
+    """The minibatch block of the second-generation optimizer, src/opt_new.rs:279-325: per batch (per-sample weights
+    1.0) forward -> backward(batch, 1.0) -> accumulate_loss; when a minibatch is complete
+    descend(step_size.at_iter(t) / minibatch_size, l2) -> reset_gradients(momentum) -> t += 1."""
+
+    def __init__(self, minibatch_size, step_size=0.01, momentum=0.9, l2_reg_coef=0.0):
+        self.minibatch_size = minibatch_size
+        self.step_size, self.momentum, self.l2 = np.float32(step_size), np.float32(momentum), np.float32(l2_reg_coef)
+        self.t = 0
+
+    def begin(self, arch):
+        arch.reset_gradients(0.0)
+        arch.reset_loss()
+
+    def batch(self, arch, frames):
+        arch.forward(frames)
+        arch.backward_scaled(1.0)
+        arch.accumulate_loss()
+
+    def end_minibatch(self, arch):
+        descent_scale = float(self.step_size / np.float32(self.minibatch_size))
+        arch.descend(descent_scale, float(self.l2))
+        arch.reset_gradients(float(self.momentum))
+        self.t += 1

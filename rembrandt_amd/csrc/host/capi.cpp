@@ -415,6 +415,52 @@ int rho_worker_save_params(rho_worker* w) { RHO_TRY({ RHO_REQ(w); w->worker->sav
 int rho_worker_restore_params(rho_worker* w) { RHO_TRY({ RHO_REQ(w); w->worker->restore_params(); }) }
 int rho_worker_reset(rho_worker* w) { RHO_TRY({ RHO_REQ(w); w->worker->reset(); }) }
 
+int rho_worker_backward_scaled(rho_worker* w, int32_t batch_size, float scale) {
+  RHO_TRY({ RHO_REQ(w && batch_size >= 0); w->worker->backward_scaled((size_t)batch_size, scale); })
+}
+int rho_worker_descend(rho_worker* w, float scale, float l2, int fused) { RHO_TRY({ RHO_REQ(w); w->worker->descend(scale, l2, fused != 0); }) }
+int rho_worker_reset_gradients(rho_worker* w, float momentum) { RHO_TRY({ RHO_REQ(w); w->worker->reset_gradients(momentum); }) }
+int rho_worker_reset_loss(rho_worker* w, int32_t batch_size) {
+  RHO_TRY({ RHO_REQ(w && batch_size >= 0); w->worker->loss_operator(0)->reset_loss((size_t)batch_size); })
+}
+int rho_worker_accumulate_loss(rho_worker* w, int32_t batch_size) {
+  RHO_TRY({ RHO_REQ(w && batch_size >= 0); w->worker->loss_operator(0)->accumulate_loss((size_t)batch_size); })
+}
+int rho_worker_store_accumulated_loss(rho_worker* w, float* out) {
+  RHO_TRY({ RHO_REQ(w && out); *out = w->worker->loss_operator(0)->store_accumulated_loss(); })
+}
+
+struct rho_sgd2 {
+  std::unique_ptr<SgdOptimization> opt;
+};
+int rho_sgd2_new(int32_t minibatch_size, int step_kind, const float* steps, const int64_t* step_iters, float momentum,
+                 float l2_reg_coef, rho_sgd2** out) {
+  RHO_TRY({
+    RHO_REQ(out && steps && minibatch_size > 0 && step_kind >= 0 && step_kind <= RHO_STEP_INVERSE);
+    SgdOpt2Config c = SgdOpt2Config();
+    c.minibatch_size = (size_t)minibatch_size;
+    c.step_size.kind = (StepSizeSchedule::Kind)step_kind;
+    for (int i = 0; i < 5; ++i) {
+      c.step_size.step[i] = steps[i];
+      c.step_size.iters[i] = step_iters ? (size_t)step_iters[i] : 0;
+    }
+    c.momentum = momentum;
+    c.l2_reg_coef = l2_reg_coef;
+    std::unique_ptr<rho_sgd2> s(new rho_sgd2());
+    s->opt.reset(new SgdOptimization(c));
+    *out = s.release();
+  })
+}
+int rho_sgd2_free(rho_sgd2* s) { RHO_TRY({ delete s; }) }
+int rho_sgd2_begin(rho_sgd2* s, rho_worker* w) { RHO_TRY({ RHO_REQ(s && w); s->opt->begin(w->worker.get()); }) }
+int rho_sgd2_batch(rho_sgd2* s, rho_worker* w, int32_t batch_size) {
+  RHO_TRY({ RHO_REQ(s && w && batch_size > 0); s->opt->batch(w->worker.get(), (size_t)batch_size); })
+}
+int rho_sgd2_end_minibatch(rho_sgd2* s, rho_worker* w, int fused) {
+  RHO_TRY({ RHO_REQ(s && w); s->opt->end_minibatch(w->worker.get(), fused != 0); })
+}
+int rho_sgd2_iter_counter(rho_sgd2* s, int64_t* out) { RHO_TRY({ RHO_REQ(s && out); *out = (int64_t)s->opt->iter_counter(); }) }
+
 int rho_worker_buffer(rho_worker* w, int32_t hidden_idx, int which, float** dptr, int64_t* len) {
   RHO_TRY({
     RHO_REQ(dptr && len);

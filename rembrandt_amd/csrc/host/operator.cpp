@@ -298,6 +298,28 @@ struct ParamTensors {
     unwrap(rh_sscal((int64_t)wlen, 0.0f, grad_weights->as_mut_ptr(), s()), "matrix_scale");
     unwrap(rh_sscal((int64_t)blen, 0.0f, grad_bias->as_mut_ptr(), s()), "row_vector_scale");
   }
+  // g += l2*W for weights and bias; W -= scale*g (src/layer_new.rs:596-617, 1133-1154)
+  void descend(float scale, float l2, bool fused) {
+    RB_ASSERT(has_backward());
+    RB_ASSERT(l2 >= 0.0f);
+    if (fused) {
+      unwrap(rh_descend((int64_t)wlen, weights->as_mut_ptr(), grad_weights->as_mut_ptr(), scale, l2, s()), "rh_descend");
+      unwrap(rh_descend((int64_t)blen, bias->as_mut_ptr(), grad_bias->as_mut_ptr(), scale, l2, s()), "rh_descend");
+      return;
+    }
+    if (l2 > 0.0f) {
+      unwrap(rh_saxpy((int64_t)wlen, l2, weights->as_ptr(), grad_weights->as_mut_ptr(), s()), "matrix_sum");
+      unwrap(rh_saxpy((int64_t)blen, l2, bias->as_ptr(), grad_bias->as_mut_ptr(), s()), "row_vector_sum");
+    }
+    unwrap(rh_saxpy((int64_t)wlen, -scale, grad_weights->as_ptr(), weights->as_mut_ptr(), s()), "matrix_sum");
+    unwrap(rh_saxpy((int64_t)blen, -scale, grad_bias->as_ptr(), bias->as_mut_ptr(), s()), "row_vector_sum");
+  }
+  // g *= scale (src/layer_new.rs:589-594, 1126-1131)
+  void reset_gradients(float scale) {
+    RB_ASSERT(has_backward());
+    unwrap(rh_sscal((int64_t)wlen, scale, grad_weights->as_mut_ptr(), s()), "matrix_scale");
+    unwrap(rh_sscal((int64_t)blen, scale, grad_bias->as_mut_ptr(), s()), "row_vector_scale");
+  }
   void fused_sgd_step(float l2, float scale, float momentum, float apply, rh_stream_t st = nullptr) {
     RB_ASSERT(has_backward());
     if (!st) st = s();
@@ -685,6 +707,10 @@ class AffineOperator : public Operator {
   void save_params() override { params_.save_params(); }
   void restore_params() override { params_.restore_params(); }
   void reset() override { params_.reset(); }
+  // backward_scaled: the inherited form; AffineLayer::backward accumulates both gradients with factor 1.0 whatever
+  // `scale` is (src/layer_new.rs:583-584)
+  void descend(float scale, float l2, bool fused) override { params_.descend(scale, l2, fused); }
+  void reset_gradients(float scale) override { params_.reset_gradients(scale); }
   void encode_params(std::vector<uint8_t>& blob) override { params_.encode_params(blob); }
   size_t decode_params(const uint8_t* blob, size_t len) override { return params_.decode_params(blob, len, kind()); }
   void encode_state(std::vector<uint8_t>& blob) override { params_.encode_state(blob); }
@@ -771,7 +797,10 @@ class Conv2dOperator : public Operator {
       apply_rect(config_.act_func, out_act_->as_mut_ptr(), out_dims_.len(), batch_size, s);
     }
   }
-  void backward(size_t batch_size) override {
+  void backward(size_t batch_size) override { backward_scaled(batch_size, 1.0f); }
+  // `scale` is the factor of the filter and bias gradients (the alpha of backward_filter / backward_bias,
+  // src/layer_new.rs:1093-1108); the operator generation always passes 1 (src/operator/mod.rs:1765-1781).
+  void backward_scaled(size_t batch_size, float scale) override {
     RB_ASSERT(params_.has_backward());
     RB_ASSERT(batch_size <= batch_cap_);
     const rh_conv_geom g = geom(batch_size);
@@ -789,9 +818,9 @@ class Conv2dOperator : public Operator {
       w_bias = workspace_aux_.get();
       if (in_delta_) { s_filter = s_bias; w_filter = w_bias; }
     }
-    unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in_act_->as_ptr(), out_delta_->as_ptr(), 1.0f, params_.grad_weights->as_mut_ptr(),
+    unwrap(rh_conv2d_bwd_filter(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), 1.0f, params_.grad_weights->as_mut_ptr(),
                                 w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter");
-    unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), 1.0f,
+    unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), scale,
                                  out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
                                  w_bias->len(), s_bias), "conv2d backward bias");
     if (in_delta_) {
@@ -806,6 +835,8 @@ class Conv2dOperator : public Operator {
   void save_params() override { params_.save_params(); }
   void restore_params() override { params_.restore_params(); }
   void reset() override { params_.reset(); }
+  void descend(float scale, float l2, bool fused) override { params_.descend(scale, l2, fused); }
+  void reset_gradients(float scale) override { params_.reset_gradients(scale); }
   void encode_params(std::vector<uint8_t>& blob) override { params_.encode_params(blob); }
   size_t decode_params(const uint8_t* blob, size_t len) override { return params_.decode_params(blob, len, kind()); }
   void encode_state(std::vector<uint8_t>& blob) override { params_.encode_state(blob); }
@@ -1304,6 +1335,13 @@ class BNormUnitsOperator : public Operator {
   void save_params() override { for (auto& u : units_) u.save_params(); }
   void restore_params() override { for (auto& u : units_) u.restore_params(); }
   void reset() override { for (auto& u : units_) u.reset(); }
+  // The second-generation layer set has no batch-normalised layers (src/layer_new.rs): its update rule is not defined here.
+  void backward_scaled(size_t batch_size, float scale) override {
+    if (scale != 1.0f) panic(std::string(kind()) + ": backward(batch, scale) is unimplemented for scale != 1");
+    backward(batch_size);
+  }
+  void descend(float, float, bool) override { panic(std::string(kind()) + ": descend is unimplemented"); }
+  void reset_gradients(float) override { panic(std::string(kind()) + ": reset_gradients is unimplemented"); }
   // On the second stream, like the plain convolution layers' updates, except for the network's first layer.
   void fused_sgd_step(float l2, float scale, float mu, float apply) override {
     rh_stream_t st = updates_on_second_stream() ? context_->aux_stream() : nullptr;
@@ -1547,7 +1585,8 @@ class SoftmaxKLLossOperator : public LossOperator {
         label_cats_(batch_size, context), label_cats_h_(batch_size, 0), weights_(batch_size, context),
         weights_h_(batch_size, 0.0f), out_values_(loss_config.num_categories * batch_size, context),
         max_value_(batch_size, context), out_cats_(batch_size, context), out_cats_h_(batch_size, 0),
-        out_loss1_(batch_size, context), out_loss_(1, context), readback_((batch_size + 1) * 4, context) {
+        out_loss1_(batch_size, context), out_loss_(1, context), acc_loss_(1, context),
+        readback_((batch_size + 1) * 4, context) {
     RB_ASSERT(prev_op != nullptr);
     in_act_ = prev_op->get_output_vars();
     if (!in_act_) panic("SoftmaxKLLossOperator missing required prev operator output vars");
@@ -1601,6 +1640,30 @@ class SoftmaxKLLossOperator : public LossOperator {
   float fetch_loss() override {
     float h = 0.0f;
     out_loss_.sync_store(&h, 1);
+    return h;
+  }
+  // Second generation (src/layer_new.rs:2103-2134): out_loss sums the batches' losses until reset_loss.  The
+  // reference's per-sample kernel there (`..._softmax_cross_entropy_loss`, trailing argument 1.0) lives outside its
+  // tree; taken here: loss1[n] = -w_n log p[n, y_n] overwritten per batch (the kl_loss1 kernel with factor 0), then
+  // the block sum added to out_loss with factor 1.
+  void reset_loss(size_t batch_size) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    rh_stream_t s = context_->stream();
+    unwrap(rh_memset_f32(out_loss1_.as_mut_ptr(), 0.0f, batch_cap_, s), "set_constant");
+    unwrap(rh_memset_f32(acc_loss_.as_mut_ptr(), 0.0f, 1, s), "set_constant");
+  }
+  void accumulate_loss(size_t batch_size) override {
+    RB_ASSERT(batch_size <= batch_cap_);
+    rh_stream_t s = context_->stream();
+    rembrandt_kernel_batch_map_softmax_kl_loss1(out_values_.as_ptr(), (int)loss_config_.num_categories, (int)batch_size,
+                                                label_cats_.as_ptr(), weights_.as_ptr(), 0.0f, out_loss1_.as_mut_ptr(), s);
+    unwrap_last("rembrandt_kernel_batch_map_softmax_kl_loss1");
+    rembrandt_kernel_batch_blockreduce_sum(out_loss1_.as_ptr(), (int)batch_size, 1, acc_loss_.as_mut_ptr(), 1.0f, s);
+    unwrap_last("rembrandt_kernel_batch_blockreduce_sum");
+  }
+  float store_accumulated_loss() override {
+    float h = 0.0f;
+    acc_loss_.sync_store(&h, 1);
     return h;
   }
   void store_output_categories(size_t batch_size) override {
@@ -1657,7 +1720,7 @@ class SoftmaxKLLossOperator : public LossOperator {
   DeviceBuffer<float> out_values_, max_value_;
   DeviceBuffer<int32_t> out_cats_;
   std::vector<int32_t> out_cats_h_;
-  DeviceBuffer<float> out_loss1_, out_loss_;
+  DeviceBuffer<float> out_loss1_, out_loss_, acc_loss_;
   PinnedBytes readback_;  // categories, then the loss: what begin_fetch copies
 };
 
@@ -1749,6 +1812,20 @@ void SequentialOperatorWorker::update_params2(float g, float u) { settle(); for 
 void SequentialOperatorWorker::save_params() { settle(); for (auto& op : hidden_ops_) op->save_params(); }
 void SequentialOperatorWorker::restore_params() { settle(); for (auto& op : hidden_ops_) op->restore_params(); }
 void SequentialOperatorWorker::reset() { settle(); for (auto& op : hidden_ops_) op->reset(); }
+void SequentialOperatorWorker::backward_scaled(size_t batch_size, float scale) {
+  settle();
+  loss_op_->backward(batch_size);  // the loss layer ignores the scale (src/layer_new.rs:1933)
+  for (auto it = hidden_ops_.rbegin(); it != hidden_ops_.rend(); ++it) (*it)->backward_scaled(batch_size, scale);
+  context_->join();
+}
+void SequentialOperatorWorker::descend(float scale, float l2_reg_coef, bool fused) {
+  settle();
+  for (auto& op : hidden_ops_) op->descend(scale, l2_reg_coef, fused);
+}
+void SequentialOperatorWorker::reset_gradients(float momentum) {
+  settle();
+  for (auto& op : hidden_ops_) op->reset_gradients(momentum);
+}
 bool SequentialOperatorWorker::graph_safe(OpPhase phase) const {
   if (!input_op_->graph_safe(phase) || !loss_op_->graph_safe(phase)) return false;
   for (const auto& op : hidden_ops_)
@@ -1944,6 +2021,23 @@ void SgdOpt::step(Operator* op, bool fused, bool defer_reapply) {
   }
   op->reset();
   if (k == Momentum::UpdateNesterov && !defer_reapply) op->update_params(mu);
+}
+
+void SgdOptimization::begin(SequentialOperatorWorker* w) {
+  w->reset_gradients(0.0f);
+  w->loss_operator(0)->reset_loss(w->batch_size());
+  t_ = 0;
+}
+void SgdOptimization::batch(SequentialOperatorWorker* w, size_t batch_size) {
+  w->forward(batch_size, OpPhase::Training(t_));
+  w->backward_scaled(batch_size, 1.0f);
+  w->loss_operator(0)->accumulate_loss(batch_size);
+}
+void SgdOptimization::end_minibatch(SequentialOperatorWorker* w, bool fused) {
+  const float descent_scale = config_.step_size.at_iter(t_) / (float)config_.minibatch_size;
+  w->descend(descent_scale, config_.l2_reg_coef, fused);
+  w->reset_gradients(config_.momentum);
+  t_ += 1;
 }
 
 void SgdOpt::reapply(Operator* op) {

@@ -14,6 +14,9 @@
 //   Pool2dOperator ......................... src/operator/mod.rs:2005-2132
 //   LossOperator, SoftmaxKLLossOperator .... src/operator/loss.rs:20-262
 //   SequentialOperatorConfig / Worker ...... src/operator/worker.rs:133-477
+//   gen-2 layer methods backward(batch, scale),
+//   descend, reset_gradients; arch fan-out . src/layer_new.rs:537-617, 1044-1154; src/arch_new.rs:527-552
+//   gen-2 minibatch update ................. src/opt_new.rs:304-325
 //   SgdOptConfig, StepSizeSchedule,
 //   Momentum, the update block ............. src/opt/sgd/mod.rs:20-147, src/opt/sgd/new.rs:345-495
 //
@@ -296,6 +299,15 @@ class Operator {
   virtual void save_params() {}
   virtual void restore_params() {}
   virtual void reset() {}
+  // The second-generation layer API (src/layer_new.rs:43-60), in which the gradient buffer doubles as the momentum
+  // buffer.  backward_scaled: `scale` is the factor of the filter and bias gradients of a convolution
+  // (layer_new.rs:1093-1108); an affine layer takes the argument and accumulates with factor 1, as the reference's
+  // does (layer_new.rs:583-584); operators without parameters have nothing to scale.
+  virtual void backward_scaled(size_t batch_size, float /*scale*/) { backward(batch_size); }
+  // g += l2*W (if l2 > 0); W -= scale*g  (layer_new.rs:596-617, 1133-1154).  `fused`: one pass instead of two.
+  virtual void descend(float /*scale*/, float /*l2_reg_coef*/, bool /*fused*/) {}
+  // g *= scale: with scale = momentum the buffer carries the velocity into the next minibatch (layer_new.rs:589-594).
+  virtual void reset_gradients(float /*scale*/) {}
   // Fused regularize -> accumulate_grads(scale, momentum) -> update_params(apply) -> reset in
   // one pass per tensor (same arithmetic, 24 instead of 52 bytes per parameter).
   virtual void fused_sgd_step(float /*l2*/, float /*scale*/, float /*momentum*/, float /*apply*/) {}
@@ -353,6 +365,11 @@ class LossOperator : public Operator {
   virtual void stage_weight(size_t batch_idx, float weight) = 0;
   virtual void load_weights(size_t batch_size) = 0;
   virtual float store_loss(size_t batch_size) = 0;
+  // Second-generation loss bookkeeping (src/layer_new.rs:2103-2134): the loss is summed over batches on the device
+  // until reset_loss; accumulate_loss adds this batch's sum_n -w_n log p[n, y_n]; store_accumulated_loss reads it.
+  virtual void reset_loss(size_t batch_size) = 0;
+  virtual void accumulate_loss(size_t batch_size) = 0;
+  virtual float store_accumulated_loss() = 0;
   virtual void store_output_categories(size_t batch_size) = 0;
   // The two halves of store_loss / store_output_categories: enqueue_* launches the kernels that leave the result in
   // device buffers nothing else writes, fetch_* copies it to the host (blocking).  A caller may enqueue more work
@@ -420,6 +437,10 @@ class SequentialOperatorWorker : public Operator {
   void save_params() override;
   void restore_params() override;
   void reset() override;
+  // PipelineArchWorker::{backward, descend, reset_gradients} (src/arch_new.rs:534-551)
+  void backward_scaled(size_t batch_size, float scale) override;
+  void descend(float scale, float l2_reg_coef, bool fused) override;
+  void reset_gradients(float momentum) override;
   void fused_sgd_step(float l2, float scale, float momentum, float apply) override;
   void set_overlap_backward(bool on) override;
   bool graph_safe(OpPhase phase) const override;
@@ -493,6 +514,29 @@ class SgdOpt {
  private:
   SgdOptConfig config_;
   size_t iter_counter_ = 0;
+};
+
+// The per-minibatch block of the second-generation optimizer, SgdOptimization::train (src/opt_new.rs:304-325), for
+// one worker: per batch forward -> backward(batch, 1.0) -> accumulate_loss with per-sample weights 1.0; at the end of
+// a minibatch descend(step_size.at_iter(t) / minibatch_size, l2) -> reset_gradients(momentum) -> t += 1.
+struct SgdOpt2Config {
+  size_t minibatch_size;
+  StepSizeSchedule step_size;
+  float momentum;
+  float l2_reg_coef;
+};
+class SgdOptimization {
+ public:
+  explicit SgdOptimization(const SgdOpt2Config& config) : config_(config) {}
+  void begin(SequentialOperatorWorker* w);                       // reset_gradients(0), reset_loss (opt_new.rs:279-280)
+  void batch(SequentialOperatorWorker* w, size_t batch_size);    // forward, backward(1.0), accumulate_loss
+  void end_minibatch(SequentialOperatorWorker* w, bool fused);   // descend, reset_gradients, t += 1
+  size_t iter_counter() const { return t_; }
+  const SgdOpt2Config& config() const { return config_; }
+
+ private:
+  SgdOpt2Config config_;
+  size_t t_ = 0;
 };
 
 // ---- NdArray (de)serialisation (header of tools/dump-array3d-header.rs:8-15) ------------------------------

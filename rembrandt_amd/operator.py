@@ -106,6 +106,18 @@ PROTOTYPES = {
     "rho_worker_save_params": (_int, [_vp]),
     "rho_worker_restore_params": (_int, [_vp]),
     "rho_worker_reset": (_int, [_vp]),
+    "rho_worker_backward_scaled": (_int, [_vp, _i32, _f]),
+    "rho_worker_descend": (_int, [_vp, _f, _f, _int]),
+    "rho_worker_reset_gradients": (_int, [_vp, _f]),
+    "rho_worker_reset_loss": (_int, [_vp, _i32]),
+    "rho_worker_accumulate_loss": (_int, [_vp, _i32]),
+    "rho_worker_store_accumulated_loss": (_int, [_vp, _P(_f)]),
+    "rho_sgd2_new": (_int, [_i32, _int, _P(_f), _P(_i64), _f, _f, _P(_vp)]),
+    "rho_sgd2_free": (_int, [_vp]),
+    "rho_sgd2_begin": (_int, [_vp, _vp]),
+    "rho_sgd2_batch": (_int, [_vp, _vp, _i32]),
+    "rho_sgd2_end_minibatch": (_int, [_vp, _vp, _int]),
+    "rho_sgd2_iter_counter": (_int, [_vp, _P(_i64)]),
     "rho_worker_buffer": (_int, [_vp, _i32, _int, _P(_vp), _P(_i64)]),
     "rho_worker_read_buffer": (_int, [_vp, _i32, _int, _vp, _i64]),
     "rho_worker_write_buffer": (_int, [_vp, _i32, _int, _vp, _i64]),
@@ -473,6 +485,28 @@ class SequentialOperatorWorker:
     def restore_params(self):
         _chk(lib().rho_worker_restore_params(self._h))
 
+    # PipelineArchWorker::{backward, descend, reset_gradients} (src/arch_new.rs:534-551) and the second-generation loss
+    # bookkeeping (src/layer_new.rs:2103-2134)
+    def backward_scaled(self, batch_size, scale):
+        _chk(lib().rho_worker_backward_scaled(self._h, batch_size, scale))
+
+    def descend(self, scale, l2_reg_coef, fused=True):
+        _chk(lib().rho_worker_descend(self._h, scale, l2_reg_coef, int(fused)))
+
+    def reset_gradients(self, momentum):
+        _chk(lib().rho_worker_reset_gradients(self._h, momentum))
+
+    def reset_loss(self, batch_size):
+        _chk(lib().rho_worker_reset_loss(self._h, batch_size))
+
+    def accumulate_loss(self, batch_size):
+        _chk(lib().rho_worker_accumulate_loss(self._h, batch_size))
+
+    def store_accumulated_loss(self):
+        out = _f()
+        _chk(lib().rho_worker_store_accumulated_loss(self._h, C.byref(out)))
+        return out.value
+
     def reset(self):
         _chk(lib().rho_worker_reset(self._h))
 
@@ -534,6 +568,41 @@ class DataSource:
         cat = _i32()
         _chk(lib().rho_dataset_get_sample(self._h, idx, frame.ctypes.data, C.byref(cat)))
         return frame, cat.value
+
+
+class SgdOptimization:
+    """The per-minibatch block of the second-generation optimizer, src/opt_new.rs:279-325 (one worker): batches run
+    forward -> backward(batch, 1.0) -> accumulate_loss with per-sample weights 1.0 (staged by the caller); a minibatch
+    ends with descend(step_size.at_iter(t) / minibatch_size, l2) -> reset_gradients(momentum) -> t += 1."""
+
+    def __init__(self, minibatch_size, step_size=0.01, momentum=0.9, l2_reg_coef=0.0):
+        steps, iters = (_f * 5)(), (_i64 * 5)()
+        steps[0] = step_size
+        h = _vp()
+        _chk(lib().rho_sgd2_new(minibatch_size, STEP["Constant"], steps, iters, momentum, l2_reg_coef, C.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            try:
+                lib().rho_sgd2_free(self._h)
+            except TypeError:
+                pass
+            self._h = None
+
+    def begin(self, worker):
+        _chk(lib().rho_sgd2_begin(self._h, worker._h))
+
+    def batch(self, worker, batch_size):
+        _chk(lib().rho_sgd2_batch(self._h, worker._h, batch_size))
+
+    def end_minibatch(self, worker, fused=True):
+        _chk(lib().rho_sgd2_end_minibatch(self._h, worker._h, int(fused)))
+
+    def iter_counter(self):
+        out = _i64()
+        _chk(lib().rho_sgd2_iter_counter(self._h, C.byref(out)))
+        return out.value
 
 
 class SgdOpt:

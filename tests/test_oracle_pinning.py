@@ -516,3 +516,84 @@ def test_preproc_and_dropout_restatements():
     lhs = float((y.astype(np.float64) * dy).sum())
     rhs = float((x.astype(np.float64) * O.dropout_backprop(dy, 1.0, mask)).sum())
     assert abs(lhs - rhs) < 1e-9 * max(1.0, abs(lhs))
+
+
+def test_second_generation_update_is_torch_sgd_with_the_velocity_in_the_gradient_buffer():
+    """The gen-2 rule (backward accumulates unnormalised sums with per-sample weights 1; descend: g += l2*W,
+    W -= (eta/m)*g; reset_gradients: g *= mu) keeps buf_t = mu*buf_{t-1} + grad_t + l2*W_{t-1}, i.e. with b = buf/m it
+    is torch.optim.SGD(lr=eta, momentum=mu, weight_decay=l2/m, dampening=0) on the mean loss.  Checked on a whole
+    conv -> pool -> affine -> affine chain over 4 minibatches of 2 micro-batches each (weights, biases and the
+    accumulated device-side loss), against torch autograd in fp64.  A dropped l2 term, a wrong sign, the factor m in
+    the wrong place or momentum applied to the wrong buffer all fail it."""
+    from oracle import graph as OG
+    from rembrandt_amd import configs
+    dims = (8, 8, 2)
+    layers, ncat = configs._chain(dims, [("conv", 3, 1, 1, 4, "Rect"), ("pool", 2, 2, 0, "Max"), ("fc", 12, "Rect"),
+                                         ("fc", 5, "Identity")])
+    batch, micro, m = 6, 2, 12
+    eta, mu, l2 = 0.3, 0.8, 0.02
+    arch = OG.SequentialOperatorWorker(layers, ncat, batch)
+    params = []
+    for op in arch.hidden:
+        if op.p is not None:
+            op.p.weights[...] = rnd(*op.p.weights.shape) * 0.3
+            op.p.bias[...] = rnd(*op.p.bias.shape) * 0.1
+            params += [torch.tensor(op.p.weights.astype(np.float64), requires_grad=True),
+                       torch.tensor(op.p.bias.astype(np.float64), requires_grad=True)]
+    cw, cb, w1, b1, w2, b2 = params
+    topt = torch.optim.SGD(params, lr=eta, momentum=mu, weight_decay=l2 / m)
+    sgd = OG.SgdOptimization(m, eta, mu, l2)
+    sgd.begin(arch)
+    for t in range(4):
+        topt.zero_grad()
+        total = 0.0
+        for k in range(micro):
+            x, labels = rnd(batch, 2, 8, 8), np.random.default_rng(100 * t + k).integers(0, ncat, batch).astype(np.int32)
+            arch.stage_batch(labels, 1.0)
+            sgd.batch(arch, x)
+            h = F.max_pool2d(torch.relu(F.conv2d(torch.tensor(x.astype(np.float64)), cw, cb, padding=1)), 2)
+            h = torch.relu(h.reshape(batch, -1) @ w1.T + b1) @ w2.T + b2
+            loss = F.cross_entropy(h, torch.tensor(labels.astype(np.int64)), reduction="sum")
+            (loss / m).backward()
+            total += float(loss.detach())
+        np.testing.assert_allclose(arch.acc_loss[0], total, rtol=1e-5)
+        arch.reset_loss()
+        sgd.end_minibatch(arch)
+        topt.step()
+        got = [a for op in arch.hidden if op.p is not None for a in (op.p.weights, op.p.bias)]
+        for a, b in zip(got, params):
+            np.testing.assert_allclose(a, b.detach().numpy(), rtol=2e-4, atol=2e-6)
+    assert sgd.t == 4
+    # the velocity lives in the gradient buffers: after reset_gradients they hold mu * m * (torch's momentum buffer)
+    for a, b in zip([a for op in arch.hidden if op.p is not None for a in (op.p.grad_weights, op.p.grad_bias)], params):
+        np.testing.assert_allclose(a, mu * m * topt.state[b]["momentum_buffer"].numpy(), rtol=2e-4, atol=2e-5)
+
+
+def test_second_generation_backward_scale_reaches_convolutions_only():
+    """backward(batch, scale): a convolution accumulates scale * (filter, bias) gradients (layer_new.rs:1093-1108), an
+    affine layer accumulates with factor 1 whatever the scale (layer_new.rs:583-584), deltas are not scaled."""
+    from oracle import graph as OG
+    from rembrandt_amd import configs
+    dims = (6, 6, 3)
+    layers, ncat = configs._chain(dims, [("conv", 3, 1, 0, 4, "Rect"), ("fc", 5, "Identity")])
+    batch = 4
+    x, labels = rnd(batch, 3, 6, 6), np.array([0, 3, 1, 4], np.int32)
+    grads = {}
+    for scale in (1.0, 0.25):
+        arch = OG.SequentialOperatorWorker(layers, ncat, batch)
+        for i, op in enumerate(arch.hidden):
+            op.p.weights[...] = np.random.default_rng(i).standard_normal(op.p.weights.shape).astype(np.float32) * 0.3
+            op.p.grad_weights[...] = 1.0    # beta = 1: what is there stays
+        arch.stage_batch(labels, 1.0)
+        arch.forward(x)
+        arch.backward_scaled(scale)
+        grads[scale] = [(op.p.grad_weights.copy(), op.p.grad_bias.copy(), op.out_delta.copy()) for op in arch.hidden]
+    (cw1, cb1, cd1), (aw1, ab1, ad1) = grads[1.0]
+    (cw2, cb2, cd2), (aw2, ab2, ad2) = grads[0.25]
+    np.testing.assert_allclose(cw2 - 1.0, 0.25 * (cw1 - 1.0), rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(cb2, 0.25 * cb1, rtol=1e-5, atol=1e-7)
+    np.testing.assert_array_equal(aw2, aw1)
+    np.testing.assert_array_equal(ab2, ab1)
+    np.testing.assert_array_equal(cd2, cd1)
+    np.testing.assert_array_equal(ad2, ad1)
+    assert np.abs(cw1 - 1.0).max() > 1e-3
