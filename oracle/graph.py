@@ -11,6 +11,7 @@ operator, same method names and the same order of operations as the Rust sources
                                             src/operator/mod.rs:1178-1236, 1355-1363
   SequentialOperatorWorker fan-out ........ src/operator/worker.rs:356-477
   SgdOpt update block ..................... src/opt/sgd/new.rs:345-495, 623-633
+  SgdOpt::train / validate loops .......... src/opt/sgd/new.rs:209-344, 495-766
   second-generation layer methods backward(batch, scale), descend, reset_gradients
                                             src/layer_new.rs:537-617, 1044-1154
   PipelineArchWorker fan-out .............. src/arch_new.rs:527-552
@@ -617,7 +618,9 @@ class SgdOpt:
             op.update_params(self.mu)
         op.reset()
 
-    def step(self, op):
+    def step(self, op, defer_reapply=False):
+        """`defer_reapply`: leave out the Nesterov look-ahead that the reference applies at the very end of an iteration,
+        after the checkpoint block (new.rs:623-633); the caller then runs reapply()."""
         step, mu = float(self.step_size), float(self.mu)
         op.regularize(float(self.l2))
         if self.kind == "UpdateNesterov" and self.iter_counter > 0:
@@ -636,8 +639,12 @@ class SgdOpt:
         else:
             op.update_params2(-step, float(np.float32(-step) * self.mu))
         op.reset()
-        if self.kind == "UpdateNesterov":
+        if self.kind == "UpdateNesterov" and not defer_reapply:
             op.update_params(mu)
+
+    def reapply(self, op):
+        if self.kind == "UpdateNesterov":
+            op.update_params(float(self.mu))
 
 
 class SgdOptimization:
@@ -664,3 +671,74 @@ class SgdOptimization:
         arch.descend(descent_scale, float(self.l2))
         arch.reset_gradients(float(self.momentum))
         self.t += 1
+
+
+def sgd_validate(operator, frames, labels):
+    """SgdOpt::validate for one worker, new.rs:641-766: the samples in order, full batches then the remainder, Inference
+    phase, per-sample weight 1/num_total_samples; returns (sum of the batches' losses, accuracy).  `frames`: float32
+    [num][c][h][w] as the input operator hands them on (after its cast)."""
+    num = len(labels)
+    correct, loss, b0 = 0, np.float32(0.0), 0
+    full = operator.batch
+    while b0 < num:
+        b = min(full, num - b0)
+        x = np.zeros((full,) + frames.shape[1:], np.float32)     # operators are built for the batch capacity
+        x[:b] = frames[b0:b0 + b]
+        lab = np.zeros((full,), np.int32)
+        lab[:b] = labels[b0:b0 + b]
+        operator.stage_batch(lab, 0.0)
+        operator.weights[:b] = np.float32(1.0) / np.float32(num)  # samples past b carry weight 0: they add nothing
+        operator.forward(x, training=False, t=0)
+        cats = operator.store_output_categories()
+        correct += int((cats[:b] == lab[:b]).sum())
+        loss = np.float32(loss + np.float32(operator.store_loss()))
+        b0 += b
+    return float(loss), correct / num
+
+
+def sgd_train(opt, operator, frames, labels, minibatch_size, max_iters, checkpoint_iters=0, checkpoint_discard=False,
+              valid=None, valid_iters=0):
+    """SgdOpt::train for one worker from freshly initialised parameters, new.rs:209-640, without its files: returns the
+    rows the reference writes to its trace ((iter, "step"|"valid", loss, error)).  Order restated: begin (Nesterov
+    look-ahead, reset) -> per sample stage (weight 1/minibatch), per full batch forward(Training{t}) -> categories ->
+    loss -> backward -> accuracy count; per minibatch the update block with iter += 1 inside it -> trace row ->
+    every checkpoint_iters: [save_params if Discard] -> validation every valid_iters -> [restore_params] -> Nesterov
+    look-ahead re-applied last.  Epochs restart at sample 0; a batch never straddles two epochs here
+    (len(frames) % batch == 0)."""
+    batch = operator.batch
+    assert minibatch_size % batch == 0 and len(frames) % batch == 0
+    weight = np.float32(1.0) / np.float32(minibatch_size)
+    opt.begin(operator)
+    rows = []
+    local_counter, elapsed_checkpoint_iters = 0, 0
+    mb_loss, mb_correct, mb_total = np.float32(0.0), 0, 0
+    while opt.iter_counter < max_iters:
+        for b0 in range(0, len(frames), batch):
+            if opt.iter_counter >= max_iters:
+                break
+            lab = labels[b0:b0 + batch].astype(np.int32)
+            operator.stage_batch(lab, weight)
+            local_counter += batch
+            operator.forward(frames[b0:b0 + batch], training=True, t=opt.iter_counter)
+            cats = operator.store_output_categories()
+            mb_loss = np.float32(mb_loss + np.float32(operator.store_loss()))
+            operator.backward()
+            mb_correct += int((cats == lab).sum())
+            mb_total += batch
+            if local_counter % minibatch_size != 0:
+                continue
+            opt.step(operator, defer_reapply=True)
+            it = opt.iter_counter
+            rows.append((it, "step", float(mb_loss), 1.0 - mb_correct / mb_total))
+            mb_loss, mb_correct, mb_total = np.float32(0.0), 0, 0
+            if checkpoint_iters and it % checkpoint_iters == 0:
+                elapsed_checkpoint_iters += checkpoint_iters
+                if checkpoint_discard:
+                    operator.save_params()
+                if valid is not None and valid_iters and elapsed_checkpoint_iters % valid_iters == 0:
+                    vloss, vacc = sgd_validate(operator, valid[0], valid[1])
+                    rows.append((it, "valid", vloss, 1.0 - vacc))
+                if checkpoint_discard:
+                    operator.restore_params()
+            opt.reapply(operator)
+    return rows

@@ -23,11 +23,14 @@ struct StepKey {
   int fused, momentum_kind;
   uint32_t step_size_bits, l2_bits, mu_bits;
   bool first_iter;  // the Nesterov un-apply is skipped at iteration 0
+  int input_mode;   // which loader filled the input frames: the input operator's forward launches differ
   bool operator<(const StepKey& o) const {
-    return std::tie(batch, fused, momentum_kind, step_size_bits, l2_bits, mu_bits, first_iter) <
-           std::tie(o.batch, o.fused, o.momentum_kind, o.step_size_bits, o.l2_bits, o.mu_bits, o.first_iter);
+    return std::tie(batch, fused, momentum_kind, step_size_bits, l2_bits, mu_bits, first_iter, input_mode) <
+           std::tie(o.batch, o.fused, o.momentum_kind, o.step_size_bits, o.l2_bits, o.mu_bits, o.first_iter, o.input_mode);
   }
 };
+// A schedule whose step size changes every iteration (Inverse) never repeats a key: neither set may grow with it.
+constexpr size_t kMaxSeenSteps = 64, kMaxStepGraphs = 16;
 
 struct rho_worker {
   std::shared_ptr<DeviceContext> ctx;
@@ -549,14 +552,15 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
     if (w->graph_steps && !rh_profile_enabled() && op->graph_safe(phase)) {
       const SgdOptConfig& c = s->opt->config();
       const StepKey key = {b, fused != 0 ? 1 : 0, (int)c.momentum.kind, float_bits(c.step_size.at_iter(t)),
-                           float_bits(c.l2_reg_coef), float_bits(c.momentum.mu), t == 0};
+                           float_bits(c.l2_reg_coef), float_bits(c.momentum.mu), t == 0,
+                           op->input_operator()->input_mode()};
       auto it = w->step_graphs.find(key);
       if (it != w->step_graphs.end()) {
         w->ctx->launch(it->second);
         s->opt->set_iter_counter(t + 1);  // what step() does on the host
         w->graph_launches += 1;
         done = true;
-      } else if (w->seen_steps.count(key)) {
+      } else if (w->seen_steps.count(key) && w->step_graphs.size() < kMaxStepGraphs) {
         // second time: record.  (The first time ran launch by launch, which also created everything that is made on
         // first use: the second stream, kernel attributes.)
         op->settle();
@@ -566,6 +570,7 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
           op->settle();  // updates issued on the second stream rejoin the recording
         } catch (...) {
           w->ctx->abort_capture();
+          op->forget_pending();
           s->opt->set_iter_counter(t);
           throw;
         }
@@ -575,6 +580,7 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
         w->graph_launches += 1;
         done = true;
       } else {
+        if (w->seen_steps.size() >= kMaxSeenSteps) w->seen_steps.clear();
         w->seen_steps.insert(key);
       }
     }

@@ -594,6 +594,7 @@ class Data3dOperator : public InputOperator {
     if (flipped) *flipped = last_flip_;
     if (alphas) *alphas = last_alphas_;
   }
+  int input_mode() const override { return f32_loaded_ ? 1 : 0; }
   bool buffer(int which, float** ptr, size_t* len) override {
     if (which != 0) return false;
     *ptr = out_buf_->as_mut_ptr();

@@ -352,6 +352,9 @@ class InputOperator : public Operator {
   // Synthetic fp32 frames (N(0,1) inputs of the benchmark configs): bypasses the u8 cast.
   virtual void load_frames_f32(const float* host, size_t batch_size) = 0;
   virtual size_t in_frame_len() const = 0;  // bytes per staged frame
+  // Which of the two loaders filled the frames that the next forward() reads (0: load_frames, u8 cast on the device;
+  // 1: load_frames_f32): forward() makes different launches for the two, so a recorded step is valid for one only.
+  virtual int input_mode() const = 0;
   // What the last forward() drew for its random preprocessing steps: crop offsets (of the last Crop), whether
   // the batch was flipped, and the 3*batch PCA lighting coefficients (empty if that step is absent or idle).
   virtual void last_preproc_draws(size_t* crop_off_w, size_t* crop_off_h, bool* flipped, std::vector<float>* alphas) const = 0;
@@ -447,6 +450,8 @@ class SequentialOperatorWorker : public Operator {
   // Joins the second stream if parameter updates are still in flight on it (called by every method but forward,
   // which joins lazily in front of the first operator concerned).
   void settle();
+  // After a recording of a step was abandoned half-way: the launches that would have needed the join never ran.
+  void forget_pending() { aux_pending_ = false; }
   const char* kind() const override { return "SequentialOperatorWorker"; }
   void encode_params(std::vector<uint8_t>& blob) override;
   size_t decode_params(const uint8_t* blob, size_t len) override;

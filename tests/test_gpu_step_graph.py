@@ -104,3 +104,47 @@ def test_recorded_steps_of_a_batch_normalised_network(dev):
     graph, n = run(net, 8, 7, True, 0x6A04, kw)
     assert n == 7 - 2   # t=0 is not safe (first batch weighs 1), t=1 launched, t=2 records, the rest replay
     same(eager, graph, "bnorm net")
+
+
+def test_recording_is_keyed_by_the_input_loader(dev):
+    """The input operator casts u8 frames or copies fp32 frames depending on which loader ran last; a step recorded
+    with one must not be replayed for the other.  Alternating loaders with graphs on == the same with graphs off."""
+    net = configs.lenet()
+    dims, layers, ncat = net
+    batch = 16
+
+    def go(graph):
+        w = SequentialOperatorWorker(configs.build_config(net), batch, "Backward", shared_seed=(0x6A05, 0x6A06), graph_steps=graph)
+        w.init_params()
+        sgd = SgdOpt(batch, 0.02, ("Update", 0.9), 0.0)
+        sgd.begin(w)
+        out = []
+        for step in range(10):
+            labels = synth.integers(0x6A05, 200 + step, (batch,), ncat)
+            if step in (4, 5, 6, 9):   # u8 frames (values 0..255, unnormalised) after fp32 steps were recorded, and back
+                w.load_frames_u8(synth.integers(0x6A05, 300 + step, (batch, dims[2], dims[1], dims[0]), 4).astype(np.uint8))
+            else:
+                w.load_frames_f32(synth.uniform(0x6A05, 100 + step, (batch, dims[2], dims[1], dims[0])))
+            w.stage_batch(labels, 1.0 / batch)
+            loss, correct = sgd.train_batch(w, batch)
+            out.append((loss, correct, [w.read(0, "weights").copy(), w.read(-1, "out_act").copy()]))
+        n = w.graph_launches()
+        w.close()
+        return out, n
+
+    eager, _ = go(False)
+    graph, n = go(True)
+    same(eager, graph, "alternating loaders")
+    assert n > 0, "some steps did replay"
+
+
+def test_schedule_that_never_repeats_a_step_size_is_launched(dev):
+    """Inverse schedule: a new step size every iteration, so no key is ever seen twice; every step is launched and the
+    bookkeeping of seen keys stays bounded (100 iterations > its cap)."""
+    dims = (8, 8, 1)
+    net = (dims, *configs._chain(dims, [("conv", 3, 1, 1, 4, "Rect"), ("fc", 3, "Identity")]))
+    kw = dict(momentum=("Update", 0.9), l2_reg_coef=0.0, schedule={"kind": "Inverse", "steps": [0.05, 0.1], "iters": []})
+    eager, _ = run(net, 4, 100, False, 0x6A07, kw)
+    graph, n = run(net, 4, 100, True, 0x6A07, kw)
+    assert n == 0
+    same(eager, graph, "inverse schedule")

@@ -6,8 +6,10 @@ import struct
 import numpy as np
 import pytest
 
+from oracle import graph as OG
+from rembrandt_amd import configs
 from rembrandt_amd.operator import DataSource, SequentialOperatorConfig, SequentialOperatorWorker, SgdOpt
-from conftest import say
+from conftest import assert_close, say
 
 pytestmark = pytest.mark.gpu
 
@@ -142,3 +144,54 @@ def test_train_driver(dev, tmp_path, momentum):
         sgd3.train(w3, train, max_iters=20, checkpoint_dir=ckpt, resume_from=16)   # beyond the latest checkpoint
     for x in (w, w2, w3, w4):
         x.close()
+
+
+@pytest.mark.parametrize("momentum", [("Update", 0.9), ("UpdateNesterov", 0.9)], ids=["update", "nesterov"])
+def test_train_driver_against_oracle_loop(dev, tmp_path, momentum):
+    """The driver against oracle.graph.sgd_train, an independent restatement of SgdOpt::train / ::validate (pinned on
+    the CPU against a torch training loop): same idx files, 10 iterations of two batches each across an epoch boundary,
+    Discard checkpoints every 2 iterations, validation (with a partial last batch) every 4.  Checked: the order and
+    values of the trace rows, and every parameter and momentum buffer at the end.  The chain pools by averaging so that
+    ten steps of rounding differences stay rounding differences."""
+    say("train driver vs oracle loop", momentum)
+    imgs, labels = make_digits(tmp_path / "train", 192, 3)
+    vimgs, vlabels = make_digits(tmp_path / "valid", 52, 4)
+    train = DataSource("mnist", tmp_path / "train-images.idx", tmp_path / "train-labels.idx")
+    valid = DataSource("mnist", tmp_path / "valid-images.idx", tmp_path / "valid-labels.idx")
+    batch, minibatch, iters = 16, 32, 10
+    dims = (28, 28, 1)
+    layers, ncat = configs._chain(dims, [("conv", 5, 1, 2, 8, "Rect"), ("pool", 2, 2, 0, "Average"),
+                                         ("conv", 3, 2, 1, 12, "Rect"), ("fc", 32, "Rect"), ("fc", 10, "Identity")])
+    cfg = SequentialOperatorConfig().data3d(dims, normalize=True)
+    for l in layers:
+        if l[0] == "conv2d":
+            cfg.conv2d(l[1], l[2], l[3], l[4], l[5], l[6], ("Normal", 0.08))
+        elif l[0] == "pool2d":
+            cfg.pool2d(l[1], l[2], l[3], l[4], l[5], l[6])
+        else:
+            cfg.affine(l[1], l[2], l[3], ("Normal", 0.08))
+    cfg.softmax_kl_loss(ncat)
+    w = SequentialOperatorWorker(cfg, batch, "Backward", shared_seed=(41, 42))
+    # the driver initialises from the worker's shared seed: the same call here gives the oracle its starting point
+    w.init_params()
+    ref = OG.SequentialOperatorWorker(layers, ncat, batch)
+    for i, op in enumerate(ref.hidden):
+        if op.p is not None:
+            op.p.weights[...] = w.read(i, "weights").reshape(op.p.weights.shape)
+    sgd = SgdOpt(minibatch, 0.05, momentum, 1e-3)
+    st = sgd.train(w, train, max_iters=iters, valid_data=valid, checkpoint_dir=tmp_path / "ckpt", display_iters=1,
+                   checkpoint_iters=2, save_iters=0, valid_iters=4, checkpoint_discard=True)
+    rows = [l.split(",") for l in open(st["log_path"]).read().splitlines()][1:]
+    f32 = lambda a: a.astype(np.float32)[:, None] / np.float32(255.0)
+    want = OG.sgd_train(OG.SgdOpt(0.05, momentum, 1e-3), ref, f32(imgs), labels, minibatch, iters, checkpoint_iters=2,
+                        checkpoint_discard=True, valid=(f32(vimgs), vlabels), valid_iters=4)
+    assert [(int(r[0]), r[1]) for r in rows] == [(r[0], r[1]) for r in want]
+    for got, exp in zip(rows, want):
+        assert abs(float(got[2]) - exp[2]) <= 2e-4 * max(1.0, abs(exp[2])), (got, exp)
+        assert abs(float(got[3]) - exp[3]) <= 1.0 / minibatch + 1e-4, (got, exp)   # one near-tie may flip
+    for i, op in enumerate(ref.hidden):
+        if op.p is None:
+            continue
+        for k in ("weights", "bias", "acc_grad_weights", "acc_grad_bias"):
+            assert_close(w.read(i, k), getattr(op.p, k).ravel(), "driver vs oracle loop: %s[%d]" % (k, i), rtol=1e-3, atol=1e-5)
+    w.close()

@@ -597,3 +597,68 @@ def test_second_generation_backward_scale_reaches_convolutions_only():
     np.testing.assert_array_equal(cd2, cd1)
     np.testing.assert_array_equal(ad2, ad1)
     assert np.abs(cw1 - 1.0).max() > 1e-3
+
+
+@pytest.mark.parametrize("flavour", ["Update", "UpdateNesterov"])
+def test_train_loop_restatement_against_a_torch_training_loop(flavour):
+    """oracle.graph.sgd_train / sgd_validate (SgdOpt::train, ::validate) against an independent torch loop: minibatches
+    of two batches with per-sample weight 1/minibatch (= the mean loss), epochs that restart at sample 0, the trace's
+    step rows (loss at the parameters before the update, error rate), validation rows every second checkpoint on the
+    *plain* parameters (for UpdateNesterov the stored ones carry the look-ahead mu*v, un-applied around the checkpoint
+    block), a last partial validation batch, Discard checkpoints that must leave the trajectory alone, and the final
+    parameters.  Update{mu} at constant step is torch SGD(momentum); UpdateNesterov's stored parameters follow torch
+    SGD(nesterov=True), its plain parameters are those plus eta*mu*b."""
+    from oracle import graph as OG
+    from rembrandt_amd import configs
+    dims = (6, 6, 1)
+    layers, ncat = configs._chain(dims, [("conv", 3, 1, 1, 4, "Rect"), ("pool", 2, 2, 0, "Average"), ("fc", 5, "Identity")])
+    batch, minibatch, iters = 4, 8, 7
+    eta, mu, l2 = 0.2, 0.7, 1e-2
+    rng = np.random.default_rng(3)
+    frames = (rng.integers(0, 256, (24, 1, 6, 6)).astype(np.float32) / np.float32(255.0))
+    labels = rng.integers(0, ncat, 24).astype(np.int32)
+    vframes = (rng.integers(0, 256, (10, 1, 6, 6)).astype(np.float32) / np.float32(255.0))
+    vlabels = rng.integers(0, ncat, 10).astype(np.int32)
+    arch = OG.SequentialOperatorWorker(layers, ncat, batch)
+    params = []
+    for op in arch.hidden:
+        if op.p is not None:
+            op.p.weights[...] = rnd(*op.p.weights.shape) * 0.4
+            params += [torch.tensor(op.p.weights.astype(np.float64), requires_grad=True),
+                       torch.tensor(op.p.bias.astype(np.float64), requires_grad=True)]
+    cw, cb, w1, b1 = params
+
+    def net(x, ps):
+        cw_, cb_, w1_, b1_ = ps
+        h = F.avg_pool2d(torch.relu(F.conv2d(torch.tensor(x.astype(np.float64)), cw_, cb_, padding=1)), 2)
+        return h.reshape(len(x), -1) @ w1_.T + b1_
+
+    rows = OG.sgd_train(OG.SgdOpt(eta, (flavour, mu), l2), arch, frames, labels, minibatch, iters, checkpoint_iters=2,
+                        checkpoint_discard=True, valid=(vframes, vlabels), valid_iters=4)
+    topt = torch.optim.SGD(params, lr=eta, momentum=mu, weight_decay=l2, nesterov=flavour == "UpdateNesterov")
+    want, pos = [], 0
+    for it in range(1, iters + 1):
+        idx = [(pos + i) % 24 for i in range(minibatch)]
+        pos = (pos + minibatch) % 24
+        topt.zero_grad()
+        logits = net(frames[idx], params)
+        loss = F.cross_entropy(logits, torch.tensor(labels[idx].astype(np.int64)))
+        loss.backward()
+        err = 1.0 - float((logits.argmax(1).numpy() == labels[idx]).mean())
+        want.append((it, "step", float(loss.detach()), err))
+        topt.step()
+        if it % 4 == 0:
+            plain = params
+            if flavour == "UpdateNesterov":
+                plain = [p.detach() + eta * mu * topt.state[p]["momentum_buffer"] for p in params]
+            with torch.no_grad():
+                vl = net(vframes, plain)
+                want.append((it, "valid", float(F.cross_entropy(vl, torch.tensor(vlabels.astype(np.int64)))),
+                             1.0 - float((vl.argmax(1).numpy() == vlabels).mean())))
+    assert [(r[0], r[1]) for r in rows] == [(r[0], r[1]) for r in want]
+    for got, ref in zip(rows, want):
+        np.testing.assert_allclose(got[2], ref[2], rtol=2e-5, err_msg=str(ref[:2]))
+        assert abs(got[3] - ref[3]) < 1e-9, (got, ref)
+    got = [a for op in arch.hidden if op.p is not None for a in (op.p.weights, op.p.bias)]
+    for a, b in zip(got, params):
+        np.testing.assert_allclose(a, b.detach().numpy(), rtol=2e-4, atol=2e-6)
