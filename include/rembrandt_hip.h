@@ -259,6 +259,19 @@ void rembrandt_kernel_batch_blockreduce_argmax(const float* src, int32_t len, in
  * ------------------------------------------------------------------------------------------- */
 int rh_sgd_momentum_step(int64_t n, float* W, float* g, float* v, float l2, float scale, float mu,
                          float apply, int zero_grad, rh_stream_t stream);
+/* rh_sgd_momentum_step over several tensors in one launch (`tensors` is a host array; each entry carries its own l2,
+ * as the batch-normalised operators decay their filters only, src/operator/conv.rs:647): what one `update` fan-out
+ * over a chain of operators (src/operator/worker.rs:420-445) issues, without a launch per parameter block.  Same
+ * arithmetic per element as rh_sgd_momentum_step. */
+typedef struct rh_sgd_tensor {
+  float* W;
+  float* g;
+  float* v;
+  int64_t n;
+  float l2;
+} rh_sgd_tensor;
+int rh_sgd_momentum_step_multi(int32_t count, const rh_sgd_tensor* tensors, float scale, float mu, float apply,
+                               int zero_grad, rh_stream_t stream);
 int rh_descend(int64_t n, float* W, float* g, float s, float l2, rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------

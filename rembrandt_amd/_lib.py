@@ -26,6 +26,10 @@ class LrnGeom(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "size")] + [(n, C.c_float) for n in ("scale", "power", "min_div")]
 
 
+class SgdTensor(C.Structure):
+    _fields_ = [("W", C.c_void_p), ("g", C.c_void_p), ("v", C.c_void_p), ("n", C.c_int64), ("l2", C.c_float)]
+
+
 class PoolGeom(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "size", "stride", "pad", "mode", "round")]
 
@@ -110,6 +114,7 @@ PROTOTYPES = {
     "rembrandt_kernel_batch_blockreduce_sum": (None, [_vp, _i32, _i32, _vp, _f, _vp]),
     "rembrandt_kernel_batch_blockreduce_argmax": (None, [_vp, _i32, _i32, _vp, _vp, _vp]),
     "rh_sgd_momentum_step": (_int, [_i64, _vp, _vp, _vp, _f, _f, _f, _f, _int, _vp]),
+    "rh_sgd_momentum_step_multi": (_int, [_i32, C.POINTER(SgdTensor), _f, _f, _f, _int, _vp]),
     "rh_descend": (_int, [_i64, _vp, _vp, _f, _f, _vp]),
     "rh_profile_enable": (_int, [_int]),
     "rh_profile_filter": (_int, [C.c_char_p]),

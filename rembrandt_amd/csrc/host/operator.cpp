@@ -328,6 +328,11 @@ struct ParamTensors {
     unwrap(rh_sgd_momentum_step((int64_t)blen, bias->as_mut_ptr(), grad_bias->as_mut_ptr(),
                                 acc_grad_bias->as_mut_ptr(), l2, scale, momentum, apply, 1, st), "rh_sgd_momentum_step");
   }
+  void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) {
+    RB_ASSERT(has_backward());
+    out.push_back({weights->as_mut_ptr(), grad_weights->as_mut_ptr(), acc_grad_weights->as_mut_ptr(), (int64_t)wlen, l2});
+    out.push_back({bias->as_mut_ptr(), grad_bias->as_mut_ptr(), acc_grad_bias->as_mut_ptr(), (int64_t)blen, l2});
+  }
   // Host-side sampling in memory order, then a blocking H2D copy (src/operator/mod.rs:964-1006, 1554-1592).
   void init(const ParamsInit& init, const uint64_t seed[2], size_t fan_in, size_t fan_out, bool xavier_ok, const char* who) {
     std::vector<float> w(wlen);
@@ -719,6 +724,7 @@ class AffineOperator : public Operator {
   void fused_sgd_step(float l2, float scale, float mu, float apply) override {
     params_.fused_sgd_step(l2, scale, mu, apply, overlap_on_ ? context_->aux_stream() : nullptr);
   }
+  void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) override { params_.sgd_tensors(l2, out); }
   bool updates_on_second_stream() const override { return overlap_on_; }
   void set_overlap_backward(bool on) override { overlap_on_ = on && overlap_built_; }
   bool buffer(int which, float** ptr, size_t* len) override {
@@ -847,6 +853,7 @@ class Conv2dOperator : public Operator {
   void fused_sgd_step(float l2, float scale, float mu, float apply) override {
     params_.fused_sgd_step(l2, scale, mu, apply, updates_on_second_stream() ? context_->aux_stream() : nullptr);
   }
+  void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) override { params_.sgd_tensors(l2, out); }
   bool updates_on_second_stream() const override { return workspace_aux_ && overlap_on_ && in_delta_; }
   bool buffer(int which, float** ptr, size_t* len) override {
     if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
@@ -1243,6 +1250,12 @@ struct BNormConvUnit {
     unwrap(rh_sgd_momentum_step((int64_t)chans, bias->as_mut_ptr(), bias_grad->as_mut_ptr(), acc_bias_grad->as_mut_ptr(),
                                 0.0f, sc, momentum, apply, 1, st), "rh_sgd_momentum_step");
   }
+  void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) {   // weight decay on the filter only
+    RB_ASSERT(backward);
+    out.push_back({weights->as_mut_ptr(), grad_weights->as_mut_ptr(), acc_grad_weights->as_mut_ptr(), (int64_t)wlen, l2});
+    out.push_back({scale->as_mut_ptr(), scale_grad->as_mut_ptr(), acc_scale_grad->as_mut_ptr(), (int64_t)chans, 0.0f});
+    out.push_back({bias->as_mut_ptr(), bias_grad->as_mut_ptr(), acc_bias_grad->as_mut_ptr(), (int64_t)chans, 0.0f});
+  }
   // Blobs: filter as (size*size*in channels, out channels), then four (1, out channels) rows
   // (src/operator/conv.rs:361-406 params: scale, bias, moving mean, moving inverse deviation;
   //  :408-459 state: momentum of filter, scale, bias, then the cached batch mean and inverse deviation).
@@ -1348,6 +1361,7 @@ class BNormUnitsOperator : public Operator {
     rh_stream_t st = updates_on_second_stream() ? context_->aux_stream() : nullptr;
     for (auto& u : units_) u.fused_sgd_step(l2, scale, mu, apply, st);
   }
+  void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) override { for (auto& u : units_) u.sgd_tensors(l2, out); }
   bool updates_on_second_stream() const override { return workspace_aux_ && overlap_on_ && in_delta_; }
   void encode_params(std::vector<uint8_t>& blob) override { for (auto& u : units_) u.encode_params(blob); }
   size_t decode_params(const uint8_t* blob, size_t len) override {
@@ -1842,13 +1856,21 @@ void SequentialOperatorWorker::fused_sgd_step(float l2, float scale, float mu, f
   settle();
   // Operators that say so take their step on the second stream (forked here: it sees the finished gradients); the
   // next forward pass joins in front of the first of them, so these updates hide behind the layers before it.
-  for (auto& op : hidden_ops_) {
-    if (op->updates_on_second_stream() && !aux_pending_) {
+  // All parameter blocks of a stream go in one launch: most of them are far too small to fill a launch of their own.
+  std::vector<rh_sgd_tensor> on_main, on_aux;
+  for (auto& op : hidden_ops_) op->sgd_tensors(l2, op->updates_on_second_stream() ? on_aux : on_main);
+  RB_ASSERT(l2 >= 0.0f);
+  if (!on_aux.empty()) {
+    if (!aux_pending_) {
       context_->fork();
       aux_pending_ = true;
     }
-    op->fused_sgd_step(l2, scale, mu, apply);
+    unwrap(rh_sgd_momentum_step_multi((int32_t)on_aux.size(), on_aux.data(), scale, mu, apply, 1, context_->aux_stream()),
+           "rh_sgd_momentum_step_multi");
   }
+  if (!on_main.empty())
+    unwrap(rh_sgd_momentum_step_multi((int32_t)on_main.size(), on_main.data(), scale, mu, apply, 1, context_->stream()),
+           "rh_sgd_momentum_step_multi");
 }
 
 void SequentialOperatorWorker::encode_params(std::vector<uint8_t>& blob) { settle(); for (auto& op : hidden_ops_) op->encode_params(blob); }

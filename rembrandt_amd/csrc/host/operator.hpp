@@ -311,6 +311,9 @@ class Operator {
   // Fused regularize -> accumulate_grads(scale, momentum) -> update_params(apply) -> reset in
   // one pass per tensor (same arithmetic, 24 instead of 52 bytes per parameter).
   virtual void fused_sgd_step(float /*l2*/, float /*scale*/, float /*momentum*/, float /*apply*/) {}
+  // The {W, g, v} blocks that fused_sgd_step(l2, ...) would update, each with the l2 factor that applies to it, so that
+  // a chain of operators can take the step in one launch per stream (rh_sgd_momentum_step_multi).
+  virtual void sgd_tensors(float /*l2*/, std::vector<rh_sgd_tensor>& /*out*/) {}
   // A consumer that can apply this operator's activation backward mask itself (max-pool backward folds the ReLU
   // mask) asks for it at construction; an operator that agrees skips its own mask pass in backward().  The
   // out_delta buffer holds the same values after the chain's backward either way.

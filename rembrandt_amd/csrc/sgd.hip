@@ -43,6 +43,52 @@ __global__ void sgd_momentum_kernel(long long n, float* __restrict__ W, float* _
   }
 }
 
+// The same update over several tensors in one launch: a network's parameter blocks are mostly small (biases,
+// first-layer filters), and a launch per block costs more than its bytes.  Block b serves 1024 consecutive
+// elements of the tensor whose block range [first[s], first[s+1]) holds b; the table travels as a kernel argument.
+constexpr int kSgdSegs = 48;
+struct SgdSegs {
+  float* W[kSgdSegs];
+  float* G[kSgdSegs];
+  float* V[kSgdSegs];
+  long long n[kSgdSegs];
+  float l2[kSgdSegs];
+  int first[kSgdSegs + 1];
+  int count;
+};
+
+__global__ __launch_bounds__(256) void sgd_momentum_multi_kernel(SgdSegs segs, float scale, float mu, float apply,
+                                                                 int zero_grad) {
+  const int b = blockIdx.x;
+  int lo = 0, hi = segs.count - 1;          // last segment whose first block is <= b (uniform over the block)
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (segs.first[mid] <= b) lo = mid; else hi = mid - 1;
+  }
+  float* __restrict__ W = segs.W[lo];
+  float* __restrict__ G = segs.G[lo];
+  float* __restrict__ V = segs.V[lo];
+  const long long n = segs.n[lo];
+  const float l2 = segs.l2[lo];
+  const bool use_l2 = l2 > 0.0f, zg = zero_grad != 0;
+  const long long base = (long long)(b - segs.first[lo]) * 1024;
+  const bool vec = ((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(G) | reinterpret_cast<uintptr_t>(V)) & 15) == 0;
+  const long long i = base + 4 * (long long)threadIdx.x;
+  if (vec && i + 3 < n) {
+    float4 w = *reinterpret_cast<float4*>(W + i), g = *reinterpret_cast<float4*>(G + i), v = *reinterpret_cast<float4*>(V + i);
+    sgd_one(w.x, g.x, v.x, l2, scale, mu, apply, use_l2, zg);
+    sgd_one(w.y, g.y, v.y, l2, scale, mu, apply, use_l2, zg);
+    sgd_one(w.z, g.z, v.z, l2, scale, mu, apply, use_l2, zg);
+    sgd_one(w.w, g.w, v.w, l2, scale, mu, apply, use_l2, zg);
+    *reinterpret_cast<float4*>(W + i) = w;
+    *reinterpret_cast<float4*>(G + i) = g;
+    *reinterpret_cast<float4*>(V + i) = v;
+  } else {
+    for (int j = 0; j < 4; ++j)
+      if (i + j < n) sgd_one(W[i + j], G[i + j], V[i + j], l2, scale, mu, apply, use_l2, zg);
+  }
+}
+
 // g = fma(l2, W, g) (if l2 > 0); W = fma(-s, g, W)
 __global__ void descend_kernel(long long n, float* __restrict__ W, float* __restrict__ G, float s, float l2) {
   const long long stride = (long long)gridDim.x * blockDim.x;
@@ -68,6 +114,45 @@ extern "C" int rh_sgd_momentum_step(int64_t n, float* W, float* g, float* v, flo
   hipLaunchKernelGGL(sgd_momentum_kernel, dim3(stream_grid((size_t)(n + 3) / 4, 256)), dim3(256), 0,
                      to_stream(stream), (long long)n, W, g, v, l2, scale, mu, apply, zero_grad);
   return launch_status();
+}
+
+extern "C" int rh_sgd_momentum_step_multi(int32_t count, const rh_sgd_tensor* tensors, float scale, float mu, float apply,
+                                          int zero_grad, rh_stream_t stream) {
+  if (count < 0 || (count > 0 && !tensors)) return RH_E_INVALID;
+  double bytes = 0.0;
+  for (int i = 0; i < count; ++i) {
+    const rh_sgd_tensor& t = tensors[i];
+    if (t.n < 0 || (t.n > 0 && (!t.W || !t.g || !t.v)) || !(t.l2 >= 0.0f)) return RH_E_INVALID;
+    if (t.n > (int64_t)1023 * (int64_t)0x7fffffff / 2) return RH_E_LIMIT;
+    bytes += 24.0 * (double)t.n;
+  }
+  if (bytes == 0.0) return 0;
+  ProfScope prof("sgd_fused", bytes, to_stream(stream));
+  int i = 0;
+  while (i < count) {
+    SgdSegs segs;
+    segs.count = 0;
+    long long blocks = 0;
+    for (; i < count && segs.count < kSgdSegs; ++i) {
+      const rh_sgd_tensor& t = tensors[i];
+      if (t.n == 0) continue;
+      const long long nb = (t.n + 1023) / 1024;
+      if (blocks + nb > 0x7fffffffll) break;       // the rest goes to another launch
+      const int s = segs.count++;
+      segs.W[s] = t.W; segs.G[s] = t.g; segs.V[s] = t.v; segs.n[s] = t.n; segs.l2[s] = t.l2;
+      segs.first[s] = (int)blocks;
+      blocks += nb;
+    }
+    if (segs.count == 0) {
+      if (i < count && tensors[i].n > 0) return RH_E_LIMIT;   // a single tensor beyond one launch's block range
+      continue;
+    }
+    segs.first[segs.count] = (int)blocks;
+    hipLaunchKernelGGL(sgd_momentum_multi_kernel, dim3((unsigned)blocks), dim3(256), 0, to_stream(stream), segs, scale, mu,
+                       apply, zero_grad);
+    if (int e = launch_status()) return e;
+  }
+  return 0;
 }
 
 extern "C" int rh_descend(int64_t n, float* W, float* g, float s, float l2, rh_stream_t stream) {

@@ -223,6 +223,15 @@ def sgd_momentum_step(W, g, v, l2, scale, mu, apply, zero_grad=True):
                                      _stream()), "rh_sgd_momentum_step")
 
 
+def sgd_momentum_step_multi(tensors, scale, mu, apply, zero_grad=True):
+    """tensors: sequence of (W, g, v, l2) device tensors; one launch for all of them."""
+    arr = (_lib.SgdTensor * len(tensors))()
+    for i, (W, g, v, l2) in enumerate(tensors):
+        arr[i] = _lib.SgdTensor(W.data_ptr(), g.data_ptr(), v.data_ptr(), W.numel(), l2)
+    check(lib().rh_sgd_momentum_step_multi(len(tensors), arr, scale, mu, apply, int(zero_grad), _stream()),
+          "rh_sgd_momentum_step_multi")
+
+
 def descend(W, g, s, l2):
     check(lib().rh_descend(W.numel(), _p(W), _p(g), s, l2, _stream()), "rh_descend")
 

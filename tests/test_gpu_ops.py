@@ -297,6 +297,36 @@ def test_blas1_sgd(dev, n):
     assert_close(N(gd), gr, "descend g", atol=1e-7)
 
 
+def test_sgd_multi_tensor_step(dev):
+    """One launch over many parameter blocks == one rh_sgd_momentum_step per block, bit for bit, and the oracle:
+    lengths around the 1024-element block and the 4-element vector boundaries, an empty block, unaligned views,
+    per-block l2 (zero for some), more blocks than one launch's table holds (48), both zero_grad settings."""
+    lens = [1, 3, 4, 5, 96, 1023, 1024, 1025, 4096, 0, 2049, 34848, 1 << 18 | 1] + [7 * i + 1 for i in range(60)]
+    say("multi-tensor sgd over", len(lens), "blocks")
+    for zg in (True, False):
+        host, multi, single = [], [], []
+        for k, n in enumerate(lens):
+            off = k % 3 if n > 16 else 0        # some blocks start 4 or 8 bytes off a 16-byte boundary
+            W, g, v = (synth.normal(17, 10 * k + j, (n + off,)) for j in range(3))
+            l2 = 0.0 if k % 4 == 0 else 1e-3 * (1 + k % 5)
+            host.append((W[off:].copy(), g[off:].copy(), v[off:].copy(), l2))
+            multi.append(tuple(T(a, dev)[off:] for a in (W, g, v)) + (l2,))
+            single.append(tuple(T(a, dev)[off:] for a in (W, g, v)) + (l2,))
+        ops.sgd_momentum_step_multi(multi, -0.01, 0.9, 1.0, zg)
+        for (W, g, v, l2) in single:
+            if W.numel():
+                ops.sgd_momentum_step(W, g, v, l2, -0.01, 0.9, 1.0, zg)
+        for k, ((Wm, gm, vm, _), (Ws, gs, vs, _), (Wh, gh, vh, l2)) in enumerate(zip(multi, single, host)):
+            assert torch.equal(Wm, Ws) and torch.equal(gm, gs) and torch.equal(vm, vs), "block %d" % k
+            if Wh.size:
+                O.sgd_momentum_step(Wh, gh, vh, l2, -0.01, 0.9, 1.0, zg)
+                assert_close(N(Wm), Wh, "multi sgd W[%d]" % k, atol=1e-7)
+                assert_close(N(vm), vh, "multi sgd v[%d]" % k, atol=1e-7)
+                assert_close(N(gm), gh, "multi sgd g[%d]" % k, atol=1e-7)
+    assert _lib.lib().rh_sgd_momentum_step_multi(1, None, 1.0, 0.9, 1.0, 1, None) == _lib.RH_E_INVALID
+    torch.cuda.synchronize()
+
+
 def test_cast_and_fill(dev):
     x = (synth.integers(17, 1, (1000003,), 256)).astype(np.uint8)
     y = ops.cast_u8_f32(T(x, dev), 1.0 / 255.0)
