@@ -1,0 +1,268 @@
+// 1x1 convolution, stride 1, no padding, few channels on both sides (<= 128): forward and backward-data.
+//
+//   y[n][row][pix] = alpha * sum_k A(row, k) * src[n][k][pix] + beta * y (+ bias[row], ReLU)
+//   forward:        A(ko, c) = w[ko][c],  src = x,  rows = K, contraction = C
+//   backward-data:  A(c, ko) = w[ko][c],  src = dy, rows = C, contraction = K
+//
+// Such a layer (NIN's "cccp" layers after the first convolution: 96 -> 96 on 54 x 54) sits on the ridge between the
+// matrix pipe and HBM: 2*96 FLOPs per 8 bytes moved.  The block-tiled engine spends most of a tile's life in its
+// prologue and epilogue there (six K steps per tile) and reloads the 36 KB filter for each of its thousands of tiles.
+// Here a block copies the filter into LDS once, already in the operand layout of v_mfma_f32_32x32x2_f32
+// (a = A[lane % 32][lane / 32]: one conflict-free ds_read_b32 per MFMA), and then every wave streams 32-pixel column
+// tiles on its own: the other operand of that instruction, b = B[lane / 32][lane % 32], is for a pixel-contiguous
+// source exactly one coalesced dword load per (k pair): lanes 0-31 read 32 consecutive pixels of channel 2s, lanes
+// 32-63 those of channel 2s + 1, straight into the operand register.  One barrier in the life of a block; a wave
+// keeps the loads of its next tile in flight while the matrix pipe works on the current one, and the waves of the
+// grid sweep the tensor in address order.
+#include "conv_common.h"
+
+namespace rh {
+
+struct Conv1x1Params {
+  const float* A;       // filter
+  int a_row_stride, a_k_stride;
+  const float* src;     // [N][Cin][PQ]
+  uint32_t src_bytes;
+  int rows, kdim;       // result rows (channels), contraction length (= Cin)
+  int PQ;
+  long long cols;       // N * PQ
+  int tiles;            // ceil(cols / 32)
+};
+
+template <int TM_>
+struct StreamTile {
+  static constexpr int TM = TM_, TN = 1;
+};
+
+// FAST: alpha == 1, beta == 0, rows == 32 * TM and the contraction == 2 * KH, so the loads need no channel guard
+// and a column tile that lies inside one image is stored without per-element checks.
+template <int TM, int KH, bool FAST, class PASS>
+__global__ __launch_bounds__(256, 2) void conv1x1_stream_kernel(Conv1x1Params p, EpiParams ep, FastDiv dPQ) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
+  const int nwaves = (int)gridDim.x * 4;
+  const int half = lane >> 5, l32 = lane & 31;
+
+  // the filter, once per block: sa[(s * TM + i) * 64 + lane] = A(32 i + lane % 32, 2 s + lane / 32), zero outside
+  extern __shared__ float sa[];
+  for (int e = threadIdx.x; e < KH * TM * 64; e += 256) {
+    const int l = e & 63, si = e >> 6, i = si % TM, s = si / TM;
+    const int row = 32 * i + (l & 31), k = 2 * s + (l >> 5);
+    sa[e] = (row < p.rows && k < p.kdim) ? p.A[(size_t)row * p.a_row_stride + (size_t)k * p.a_k_stride] : 0.0f;
+  }
+  __syncthreads();
+  const float* const sal = sa + lane;
+
+  const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.src, p.src_bytes);
+  const __amdgpu_buffer_rsrc_t rdst = make_rsrc(ep.out, (uint32_t)(sizeof(float) * (size_t)p.cols * p.rows));
+  const int PQ4 = p.PQ * 4;
+  const uint32_t img_bytes = (uint32_t)p.kdim * (uint32_t)PQ4;
+  const uint32_t out_img_bytes = (uint32_t)p.rows * (uint32_t)PQ4;
+
+  // Loads of one column tile: b[s] = src[img][2 s + half][pix]; lanes past the last column (and, unless FAST, channel
+  // pairs past the contraction) read zero: offset 0x80000000 is out of range of the buffer.  The address advances in
+  // a register from one channel pair to the next.
+  auto load_tile = [&](float (&b)[KH], int tile) __attribute__((always_inline)) {
+    const long long col64 = (long long)tile * 32 + l32;   // tile may be up to nwaves past the last one
+    const uint32_t col = (uint32_t)col64;
+    uint32_t v = 0x80000000u;
+    if (col64 < p.cols) {
+      uint32_t img, pix;
+      dPQ.divmod(col, img, pix);
+      v = img * img_bytes + pix * 4u + (uint32_t)(half * PQ4);
+    }
+    const uint32_t step = col64 < p.cols ? (uint32_t)(2 * PQ4) : 0u;
+#pragma unroll
+    for (int s = 0; s < KH; ++s) {
+      const uint32_t vv = (FAST || 2 * s + half < p.kdim) ? v : 0x80000000u;
+      b[s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)vv, 0, 0));
+      v += step;
+    }
+  };
+  auto compute_tile = [&](const float (&b)[KH], int tile) __attribute__((always_inline)) {
+    f32x16 acc[TM][1];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][0][v] = 0.0f;
+    // (opaque pointer: the filter reads must stay in the loop, one per MFMA, not be hoisted into KH * TM registers)
+    // An LDS-space pointer: through a generic one these become flat loads, whose waits also cover the global loads.
+    typedef const __attribute__((address_space(3))) float* lds_ptr;
+    lds_ptr sl = (lds_ptr)sal;
+    asm volatile("" : "+v"(sl));
+    // pinned order per channel pair: [filter reads of the next pair] [MFMAs of this pair]; left alone the scheduler
+    // issues every read of the tile first and spills
+    float av[2][TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) av[0][i] = sl[i * 64];
+#pragma unroll
+    for (int s = 0; s < KH; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 1 < KH) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) av[(s + 1) & 1][i] = sl[((s + 1) * TM + i) * 64];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s & 1][i], b[s], acc[i][0], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (FAST) {
+      if (ep.bias) {
+        // added after the sum, as the separate bias pass of the reference does (same rounding).  Rows
+        // 32 i + 8 (v / 4) + 4 half + v % 4: four consecutive rows per 16-byte load; the pointer is made opaque so
+        // that these (cached) loads stay here instead of occupying 16 * TM registers for the life of the wave.
+        typedef const __attribute__((address_space(1))) float* global_ptr;   // (a generic pointer would mean flat loads)
+        global_ptr bias = (global_ptr)ep.bias;
+        asm volatile("" : "+s"(bias));
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            global_ptr bq = bias + 32 * i + 8 * q + 4 * half;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][0][4 * q + e] += bq[e];
+          }
+      }
+      const uint32_t col0 = (uint32_t)tile * 32u;
+      uint32_t img0, pix0;
+      dPQ.divmod(col0, img0, pix0);
+      const bool inside = (long long)col0 + 31 < p.cols && pix0 + 31u < (uint32_t)p.PQ;   // uniform over the wave
+      if (inside) {
+        if (ep.relu) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][0][v] = acc[i][0][v] > 0.0f ? acc[i][0][v] : 0.0f;
+        }
+        uint32_t o = img0 * out_img_bytes + (pix0 + (uint32_t)l32) * 4u + (uint32_t)(4 * half * PQ4);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float val = acc[i][0][4 * q + e];   // (bit-casting the vector element directly stored element 4q)
+              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), rdst, (int)o, 0, 0);
+              o += (uint32_t)PQ4;
+            }
+            o += (uint32_t)(4 * PQ4);
+          }
+        return;
+      }
+      // A tile that straddles two images or ends ragged (one in PQ / 32): element by element.  The bias is already
+      // added.  Everything here derives from an opaque copy of PQ so that none of it is computed (and kept
+      // in registers) outside this branch.
+      int inner = p.PQ;
+      asm volatile("" : "+s"(inner));
+      const long long col = (long long)col0 + l32;
+      if (col < p.cols) {
+        const int img = (int)(col / inner), pix = (int)(col - (long long)img * inner);
+        float* dst = ep.out + ((size_t)img * p.rows + 4 * half) * inner + pix;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            float val = acc[i][0][v];
+            if (ep.relu) val = val > 0.0f ? val : 0.0f;
+            dst[(size_t)(32 * i + 8 * (v >> 2) + (v & 3)) * inner] = val;
+          }
+      }
+      return;
+    }
+    store_tile<StreamTile<TM>, true>(acc, ep, 0, tile * 32, 0, 0, lane, -1);
+  };
+
+  // The prefetch is unconditional (a tile past the end reads nothing: every lane's offset is out of range), so that
+  // the code between two uses of a buffer is straight-line and the compiler's wait counts let the prefetched loads
+  // stay in flight during the MFMAs; behind a condition it has to wait for them first.
+  float b0[KH], b1[KH];
+  int t = wave;
+  if (t >= p.tiles) return;
+  load_tile(b0, t);
+  while (true) {
+    load_tile(b1, t + nwaves);
+    compute_tile(b0, t);
+    t += nwaves;
+    if (t >= p.tiles) break;
+    load_tile(b0, t + nwaves);
+    compute_tile(b1, t);
+    t += nwaves;
+    if (t >= p.tiles) break;
+  }
+}
+
+template <int TM, int KH, class PASS>
+static int launch_stream(const Conv1x1Params& p, const EpiParams& ep, hipStream_t stream) {
+  const int blocks = p.tiles >= 4 * 512 ? 512 : cdiv(p.tiles, 4);   // two blocks per CU
+  const FastDiv dPQ((uint32_t)p.PQ);
+  constexpr size_t lds = sizeof(float) * KH * TM * 64;
+  if (lds > 48 * 1024) {
+    static const hipError_t a1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv1x1_stream_kernel<TM, KH, true, PASS>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    static const hipError_t a2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv1x1_stream_kernel<TM, KH, false, PASS>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (a1 != hipSuccess) return (int)a1;
+    if (a2 != hipSuccess) return (int)a2;
+  }
+  const bool fast = ep.alpha == 1.0f && ep.beta == 0.0f && p.rows == 32 * TM && p.kdim == 2 * KH &&
+                    (!ep.bias || (reinterpret_cast<uintptr_t>(ep.bias) & 15) == 0);
+  if (fast)
+    hipLaunchKernelGGL((conv1x1_stream_kernel<TM, KH, true, PASS>), dim3((unsigned)blocks), dim3(256), lds, stream, p, ep, dPQ);
+  else
+    hipLaunchKernelGGL((conv1x1_stream_kernel<TM, KH, false, PASS>), dim3((unsigned)blocks), dim3(256), lds, stream, p, ep, dPQ);
+  return launch_status();
+}
+
+template <int TM, class PASS>
+static int pick_kh(const Conv1x1Params& p, const EpiParams& ep, hipStream_t stream) {
+  const int kh = cdiv(p.kdim, 2);
+  if (kh <= 16) return launch_stream<TM, 16, PASS>(p, ep, stream);
+  if (kh <= 32) return launch_stream<TM, 32, PASS>(p, ep, stream);
+  if (kh <= 48) return launch_stream<TM, 48, PASS>(p, ep, stream);
+  return launch_stream<TM, 64, PASS>(p, ep, stream);
+}
+
+bool conv1x1_stream_applies(const ConvDims& d) {
+  return d.R == 1 && d.S == 1 && d.st == 1 && d.pad == 0 && d.C <= kConv1x1MaxChannels && d.K <= kConv1x1MaxChannels &&
+         (long long)d.N * d.P * d.Q < (1ll << 31) - 64;
+}
+
+// pass: RH_CONV_FWD (src = x, out = y) or RH_CONV_BWD_DATA (src = dy, out = dx).
+int launch_conv1x1_stream(const ConvDims& d, int pass, const float* w, const float* src, float* out, float alpha, float beta,
+                          const float* bias, int relu, hipStream_t stream) {
+  const bool fwd = pass == RH_CONV_FWD;
+  Conv1x1Params p;
+  p.A = w;
+  p.a_row_stride = fwd ? d.C : 1;
+  p.a_k_stride = fwd ? 1 : d.C;
+  p.src = src;
+  p.rows = fwd ? d.K : d.C;
+  p.kdim = fwd ? d.C : d.K;
+  p.PQ = d.P * d.Q;
+  p.cols = (long long)d.N * p.PQ;
+  p.src_bytes = (uint32_t)(sizeof(float) * (size_t)p.cols * p.kdim);
+  p.tiles = (int)cdiv<long long>(p.cols, 32);
+  EpiParams ep;
+  ep.out = out; ep.bias = bias; ep.alpha = alpha; ep.beta = beta;
+  ep.rows = p.rows; ep.cols = (int)p.cols; ep.inner = p.PQ; ep.ld = 0; ep.relu = relu; ep.split_stride = 0;
+  ProfScope prof(fwd ? "conv_fwd_1x1_stream" : "conv_bwd_data_1x1_stream", 2.0 * (double)p.rows * (double)p.cols * (double)p.kdim,
+                 stream);
+  const int tm = cdiv(p.rows, 32);
+  if (fwd) {
+    switch (tm) {
+      case 1: return pick_kh<1, PassConvFwd>(p, ep, stream);
+      case 2: return pick_kh<2, PassConvFwd>(p, ep, stream);
+      case 3: return pick_kh<3, PassConvFwd>(p, ep, stream);
+      default: return pick_kh<4, PassConvFwd>(p, ep, stream);
+    }
+  }
+  switch (tm) {
+    case 1: return pick_kh<1, PassConvBwdData>(p, ep, stream);
+    case 2: return pick_kh<2, PassConvBwdData>(p, ep, stream);
+    case 3: return pick_kh<3, PassConvBwdData>(p, ep, stream);
+    default: return pick_kh<4, PassConvBwdData>(p, ep, stream);
+  }
+}
+
+}  // namespace rh

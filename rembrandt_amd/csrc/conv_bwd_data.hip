@@ -186,6 +186,10 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
   if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return RH_E_WORKSPACE;
   hipStream_t stream = to_stream(stream_);
 
+  if (!(flags & (RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET)) && conv1x1_stream_applies(d)) {
+    if (d.x_elems == 0) return 0;
+    return launch_conv1x1_stream(d, RH_CONV_BWD_DATA, w, dy, dx, alpha, beta, nullptr, 0, stream);
+  }
   const int KRS = d.K * d.R * d.S;
   const PhasePlan pp = plan_phase_bwd_data(d);
   if (pp.ok && !(flags & RH_ALGO_GATHER)) {

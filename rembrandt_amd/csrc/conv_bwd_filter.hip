@@ -328,6 +328,16 @@ static int run_bwd_filter(const PixDyParams& ap, const PixXParams& bp, const Epi
   return launch_mfma_gemm<T, AL, BL, false, PassConvBwdFilter>(ap, bp, ep, M, splits, used, stream, tag);
 }
 
+// 1x1 filter, stride 1, no padding: x is read exactly like dy (row c of pixel (n, pq) at (n*C + c)*PQ + pq), so both
+// operands take the pixel loader without tap table or bounds checks.
+template <class T>
+static int run_bwd_filter_1x1(const PixDyParams& ap, const PixDyParams& bp, const EpiParams& ep, int M,
+                              int splits, int* used, hipStream_t stream, const char* tag) {
+  typedef LoadPixDy<T::BM, T::BK, T::NT> AL;
+  typedef LoadPixDy<T::BN, T::BK, T::NT> BL;
+  return launch_mfma_gemm<T, AL, BL, false, PassConvBwdFilter>(ap, bp, ep, M, splits, used, stream, tag);
+}
+
 // db[k] = alpha * sum_{n, i<plane} dy[(n*K + k)*plane + i] + beta * db[k].  grid = (K, 1): the 16 waves of
 // a block each walk whole planes (one image at a time), lanes along the plane, no index divisions.
 __global__ __launch_bounds__(1024) void bwd_bias_kernel(const float* __restrict__ dy, int N, int K,
@@ -576,11 +586,32 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
   const int M = d.N * d.P * d.Q;
   int4* tab = static_cast<int4*>(ws);
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + plan.tab_bytes);
+  PixDyParams ap;
+  ap.ptr = dy; ap.bytes = (uint32_t)(d.y_elems * 4); ap.rows = d.K; ap.M = M; ap.PQ = d.P * d.Q;
+  if (d.R == 1 && d.S == 1 && d.st == 1 && d.pad == 0 && M > 0) {
+    PixDyParams xp;
+    xp.ptr = x; xp.bytes = (uint32_t)(d.x_elems * 4); xp.rows = d.C; xp.M = M; xp.PQ = d.P * d.Q;
+    EpiParams ep;
+    ep.out = part; ep.bias = nullptr; ep.alpha = 1.0f; ep.beta = 0.0f;
+    ep.rows = d.K; ep.cols = CRS; ep.inner = 0; ep.ld = CRS; ep.relu = 0;
+    ep.split_stride = (long long)d.K * CRS;
+    int used = 1, e = 0;
+    switch (plan.bm) {
+      case 128: e = run_bwd_filter_1x1<T128x128>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_128x128"); break;
+      case 96:
+        e = plan.bn == 128 ? run_bwd_filter_1x1<T96x128>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x128")
+                           : run_bwd_filter_1x1<T96x256>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x256");
+        break;
+      case 64:  e = run_bwd_filter_1x1<T64x256>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_64x256"); break;
+      default:  e = run_bwd_filter_1x1<T32x256>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x256"); break;
+    }
+    if (e) return e;
+    launch_split_reduce(part, used, (long long)d.K * CRS, dw, d.K, CRS, CRS, alpha, beta, stream);
+    return launch_status();
+  }
   launch_build_fwd_tab(tab, round_up(CRS, kTabPad), CRS, d.R, d.S, d.H * d.W, d.W, stream);
   if (int e = launch_status()) return e;
 
-  PixDyParams ap;
-  ap.ptr = dy; ap.bytes = (uint32_t)(d.y_elems * 4); ap.rows = d.K; ap.M = M; ap.PQ = d.P * d.Q;
   PixXParams bp;
   bp.ptr = x; bp.bytes = (uint32_t)(d.x_elems * 4); bp.rows = CRS; bp.M = M; bp.PQ = d.P * d.Q; bp.Q = d.Q;
   bp.img_stride = d.C * d.H * d.W; bp.H = d.H; bp.W = d.W; bp.st = d.st; bp.pad = d.pad; bp.rtab = tab;

@@ -357,6 +357,13 @@ inline PhasePlan plan_phase_bwd_data(const ConvDims& d) {
   return p;
 }
 
+// 1x1 / stride 1 / no padding layers with at most this many channels on both sides run on the register-resident
+// streaming kernel (conv1x1.hip) in forward and backward-data.
+constexpr int kConv1x1MaxChannels = 128;
+bool conv1x1_stream_applies(const ConvDims& d);
+int launch_conv1x1_stream(const ConvDims& d, int pass, const float* w, const float* src, float* out, float alpha, float beta,
+                          const float* bias, int relu, hipStream_t stream);
+
 // dst[n][c][halo + dil*h][halo + dil*w] = src[n][c][h][w], zeros elsewhere; dst is planes x Hp x Wp.
 void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
                       hipStream_t stream, int dil = 1);

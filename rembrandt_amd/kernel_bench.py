@@ -23,6 +23,16 @@ CONV_LAYERS = {
     "alexnet_conv1": (256, 3, 227, 227, 96, 11, 4, 0),
     "alexnet_conv4": (256, 384, 13, 13, 384, 3, 1, 1),
     "alexnet_conv5": (256, 384, 13, 13, 256, 3, 1, 1),
+    # the distinct convolutions of the NIN-shaped network at batch 128 (1x1 "cccp" layers after each spatial one)
+    "nin_conv1": (128, 3, 224, 224, 96, 11, 4, 0),
+    "nin_cccp1": (128, 96, 54, 54, 96, 1, 1, 0),
+    "nin_conv2": (128, 96, 27, 27, 256, 5, 1, 2),
+    "nin_cccp3": (128, 256, 27, 27, 256, 1, 1, 0),
+    "nin_conv3": (128, 256, 13, 13, 384, 3, 1, 1),
+    "nin_cccp5": (128, 384, 13, 13, 384, 1, 1, 0),
+    "nin_conv4": (128, 384, 6, 6, 1024, 3, 1, 1),
+    "nin_cccp7": (128, 1024, 6, 6, 1024, 1, 1, 0),
+    "nin_cccp8": (128, 1024, 6, 6, 1000, 1, 1, 0),
     "stride2_3x3": (64, 64, 56, 56, 128, 3, 2, 1),   # a strided layer in mid-network (its backward-data is needed)
     # the distinct convolutions of the ResNet-18 template at batch 64
     "resnet_conv1": (64, 3, 224, 224, 64, 7, 2, 3),

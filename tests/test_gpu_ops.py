@@ -45,6 +45,14 @@ CONV_CASES = [
     # stride 1 with output rows a multiple of four pixels long on a 128-row tile, padded and unpadded image
     (3, 8, 12, 16, 128, 3, 1, 1),
     (2, 16, 10, 12, 130, 1, 1, 0),
+    # 1x1, stride 1, no padding, at most 128 channels on both sides: the register-resident streaming kernel (forward
+    # and backward-data) and the pixel loaders for both operands of backward-filter.  Odd channel counts (a last
+    # channel pair with one live half), column tiles that straddle images and end ragged, all four row-tile counts.
+    (3, 5, 7, 9, 33, 1, 1, 0),
+    (2, 96, 9, 11, 96, 1, 1, 0),
+    (1, 128, 6, 5, 128, 1, 1, 0),
+    (5, 17, 8, 8, 100, 1, 1, 0),
+    (2, 64, 13, 13, 20, 1, 1, 0),
 ]
 
 
