@@ -12,8 +12,13 @@
 // tiles on its own: the other operand of that instruction, b = B[lane / 32][lane % 32], is for a pixel-contiguous
 // source exactly one coalesced dword load per (k pair): lanes 0-31 read 32 consecutive pixels of channel 2s, lanes
 // 32-63 those of channel 2s + 1, straight into the operand register.  One barrier in the life of a block; a wave
-// keeps the loads of its next tile in flight while the matrix pipe works on the current one, and the waves of the
-// grid sweep the tensor in address order.
+// refills its operand registers for the next tile as the current tile's MFMAs free them, and the waves of an XCD
+// sweep that XCD's eighth of the tensor in address order.
+//
+// Measured on the 96 -> 96, 54 x 54, batch 128 layer (286 MB, 6.9 GFLOP; 46 us at the 6.2 TB/s a copy reaches, 44 us
+// at the matrix peak): 96 us.  With parts removed: MFMAs and filter reads alone 65 us (the matrix pipe at the
+// clock it gets, three or four tiles per wave, prologue), loads and stores alone 77 us (dword accesses: what a
+// one-float-per-thread copy reaches), loads alone 40, stores alone 38.
 #include "conv_common.h"
 
 namespace rh {
@@ -36,19 +41,63 @@ struct StreamTile {
 
 // FAST: alpha == 1, beta == 0, rows == 32 * TM and the contraction == 2 * KH, so the loads need no channel guard
 // and a column tile that lies inside one image is stored without per-element checks.
+// Registers: 16 TM accumulators + KH operands + about seventy (the general epilogue of the non-FAST form needs more
+// and runs two blocks per CU): as many blocks per CU (four waves each, one per SIMD) as fit 512 registers per lane,
+// two to four; the filter's LDS copy (256 TM KH bytes) fits as often.
+template <int TM, int KH, bool FAST>
+constexpr int stream_blocks_per_cu() {
+  const int regs = 16 * TM + KH + 72 + (TM == 4 ? 8 : 0);
+  return !FAST || 512 / regs < 2 ? 2 : (512 / regs > 4 ? 4 : 512 / regs);
+}
+
 template <int TM, int KH, bool FAST, class PASS>
-__global__ __launch_bounds__(256, 2) void conv1x1_stream_kernel(Conv1x1Params p, EpiParams ep, FastDiv dPQ) {
+__global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST>())) void conv1x1_stream_kernel(Conv1x1Params p, EpiParams ep, FastDiv dPQ) {
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
-  const int nwaves = (int)gridDim.x * 4;
+  // Blocks go to the eight XCDs in turn (block b to XCD b % 8), each with an L2 of its own.  An XCD takes a
+  // contiguous eighth of the column tiles and its waves sweep that eighth in address order, so the two halves of a
+  // cache line that neighbouring tiles share (planes are not line-aligned) meet in one L2: read from memory once,
+  // and written back as a whole line.  Grids that are no multiple of eight blocks sweep the whole range together.
+  const bool by_xcd = (gridDim.x & 7) == 0;
+  const int nwaves = by_xcd ? (int)(gridDim.x >> 3) * 4 : (int)gridDim.x * 4;
+  const int wave = __builtin_amdgcn_readfirstlane(
+      (int)((by_xcd ? blockIdx.x >> 3 : blockIdx.x) * 4 + (threadIdx.x >> 6)));
+  const int span = by_xcd ? (p.tiles + 7) >> 3 : p.tiles;            // column tiles per XCD
+  const int first = by_xcd ? (int)(blockIdx.x & 7) * span : 0;
+  const int last = min(first + span, p.tiles);                      // (one past) this XCD's range
   const int half = lane >> 5, l32 = lane & 31;
 
-  // the filter, once per block: sa[(s * TM + i) * 64 + lane] = A(32 i + lane % 32, 2 s + lane / 32), zero outside
+  // The filter, once per block: sa[(s * TM + i) * 64 + lane] = A(32 i + lane % 32, 2 s + lane / 32), zero outside.
+  // Every thread first issues all its loads (KH TM / 4 of them, out-of-range ones read zero) and then writes LDS, so
+  // a block waits for memory once.  Which element a thread takes follows the filter's layout in memory: with the
+  // contraction index contiguous (forward) a wave reads eight rows by eight consecutive k (32-byte pieces; its LDS
+  // writes meet eight to a bank), with the row index contiguous (backward-data) a wave reads LDS order directly.
   extern __shared__ float sa[];
-  for (int e = threadIdx.x; e < KH * TM * 64; e += 256) {
-    const int l = e & 63, si = e >> 6, i = si % TM, s = si / TM;
-    const int row = 32 * i + (l & 31), k = 2 * s + (l >> 5);
-    sa[e] = (row < p.rows && k < p.kdim) ? p.A[(size_t)row * p.a_row_stride + (size_t)k * p.a_k_stride] : 0.0f;
+  {
+    constexpr int PER = KH * TM / 4;
+    const __amdgpu_buffer_rsrc_t rflt = make_rsrc(p.A, (uint32_t)(sizeof(float) * (size_t)p.rows * p.kdim));
+    const bool k_major = p.a_k_stride == 1;
+    float tmp[PER];
+    int pos[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = (int)threadIdx.x + 256 * j;
+      int row, k;
+      if (k_major) {
+        const int rest = e >> 6, k_hi = rest % (KH / 4), r_hi = rest / (KH / 4);
+        k = 8 * k_hi + (e & 7);
+        row = 8 * r_hi + ((e >> 3) & 7);
+        pos[j] = ((k >> 1) * TM + (row >> 5)) * 64 + (k & 1) * 32 + (row & 31);
+      } else {
+        const int l = e & 63, si = e >> 6;
+        row = 32 * (si % TM) + (l & 31);
+        k = 2 * (si / TM) + (l >> 5);
+        pos[j] = e;
+      }
+      const uint32_t off = (row < p.rows && k < p.kdim) ? 4u * (uint32_t)(row * p.a_row_stride + k * p.a_k_stride) : 0x80000000u;
+      tmp[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rflt, (int)off, 0, 0));
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) sa[pos[j]] = tmp[j];
   }
   __syncthreads();
   const float* const sal = sa + lane;
@@ -61,25 +110,35 @@ __global__ __launch_bounds__(256, 2) void conv1x1_stream_kernel(Conv1x1Params p,
 
   // Loads of one column tile: b[s] = src[img][2 s + half][pix]; lanes past the last column (and, unless FAST, channel
   // pairs past the contraction) read zero: offset 0x80000000 is out of range of the buffer.  The address advances in
-  // a register from one channel pair to the next.
-  auto load_tile = [&](float (&b)[KH], int tile) __attribute__((always_inline)) {
-    const long long col64 = (long long)tile * 32 + l32;   // tile may be up to nwaves past the last one
-    const uint32_t col = (uint32_t)col64;
-    uint32_t v = 0x80000000u;
-    if (col64 < p.cols) {
+  // a register from one channel pair to the next.  tile_addr gives a lane's first address and the step between
+  // channel pairs (both "nowhere" for a tile past the range), load_part issues the loads of pairs [s0, s1).
+  auto tile_addr = [&](int tile, uint32_t& v, uint32_t& step) __attribute__((always_inline)) {
+    const long long col64 = (long long)tile * 32 + l32;   // tile may be up to nwaves past the range's last one
+    v = 0x80000000u;
+    step = 0u;
+    if (tile < last && col64 < p.cols) {
       uint32_t img, pix;
-      dPQ.divmod(col, img, pix);
+      dPQ.divmod((uint32_t)col64, img, pix);
       v = img * img_bytes + pix * 4u + (uint32_t)(half * PQ4);
+      step = (uint32_t)(2 * PQ4);
     }
-    const uint32_t step = col64 < p.cols ? (uint32_t)(2 * PQ4) : 0u;
+  };
+  auto load_part = [&](float (&b)[KH], uint32_t& v, uint32_t step, int s0, int s1) __attribute__((always_inline)) {
 #pragma unroll
-    for (int s = 0; s < KH; ++s) {
+    for (int s = s0; s < s1; ++s) {
       const uint32_t vv = (FAST || 2 * s + half < p.kdim) ? v : 0x80000000u;
       b[s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)vv, 0, 0));
       v += step;
     }
   };
-  auto compute_tile = [&](const float (&b)[KH], int tile) __attribute__((always_inline)) {
+  // One column tile: the MFMAs over the operand registers b, which are refilled for the tile `next` as they fall
+  // free (first half of the channel pairs in the middle of the contraction, second half at its end), then the
+  // epilogue and the stores.  A wave therefore holds one tile's operands, not two, four blocks fit a CU, and the waits
+  // of one wave (for its loads, and for the write acknowledgements that the shared memory counter makes it sit out
+  // too) are covered by the matrix work of the three others on its SIMD.
+  auto compute_tile = [&](float (&b)[KH], int tile, int next) __attribute__((always_inline)) {
+    uint32_t nv, nstep;
+    tile_addr(next, nv, nstep);
     f32x16 acc[TM][1];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -105,7 +164,13 @@ __global__ __launch_bounds__(256, 2) void conv1x1_stream_kernel(Conv1x1Params p,
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i) acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s & 1][i], b[s], acc[i][0], 0, 0, 0);
+      if (s == KH / 2 - 1) {
+        __builtin_amdgcn_sched_barrier(0);
+        load_part(b, nv, nstep, 0, KH / 2);
+      }
     }
+    __builtin_amdgcn_sched_barrier(0);
+    load_part(b, nv, nstep, KH / 2, KH);
     __builtin_amdgcn_sched_barrier(0);
     if (FAST) {
       if (ep.bias) {
@@ -173,28 +238,21 @@ __global__ __launch_bounds__(256, 2) void conv1x1_stream_kernel(Conv1x1Params p,
     store_tile<StreamTile<TM>, true>(acc, ep, 0, tile * 32, 0, 0, lane, -1);
   };
 
-  // The prefetch is unconditional (a tile past the end reads nothing: every lane's offset is out of range), so that
-  // the code between two uses of a buffer is straight-line and the compiler's wait counts let the prefetched loads
-  // stay in flight during the MFMAs; behind a condition it has to wait for them first.
-  float b0[KH], b1[KH];
-  int t = wave;
-  if (t >= p.tiles) return;
-  load_tile(b0, t);
-  while (true) {
-    load_tile(b1, t + nwaves);
-    compute_tile(b0, t);
-    t += nwaves;
-    if (t >= p.tiles) break;
-    load_tile(b0, t + nwaves);
-    compute_tile(b1, t);
-    t += nwaves;
-    if (t >= p.tiles) break;
+  // The refill is unconditional (a tile past the end reads nothing: every lane's offset is out of range), so the
+  // loop body is straight-line code.
+  float b0[KH];
+  int t = first + wave;
+  if (t >= last) return;
+  {
+    uint32_t v, step;
+    tile_addr(t, v, step);
+    load_part(b0, v, step, 0, KH);
   }
+  for (; t < last; t += nwaves) compute_tile(b0, t, t + nwaves);
 }
 
 template <int TM, int KH, class PASS>
 static int launch_stream(const Conv1x1Params& p, const EpiParams& ep, hipStream_t stream) {
-  const int blocks = p.tiles >= 4 * 512 ? 512 : cdiv(p.tiles, 4);   // two blocks per CU
   const FastDiv dPQ((uint32_t)p.PQ);
   constexpr size_t lds = sizeof(float) * KH * TM * 64;
   if (lds > 48 * 1024) {
@@ -207,6 +265,9 @@ static int launch_stream(const Conv1x1Params& p, const EpiParams& ep, hipStream_
   }
   const bool fast = ep.alpha == 1.0f && ep.beta == 0.0f && p.rows == 32 * TM && p.kdim == 2 * KH &&
                     (!ep.bias || (reinterpret_cast<uintptr_t>(ep.bias) & 15) == 0);
+  // every block slot of the GPU; smaller problems: a wave per tile, in whole blocks per XCD when there are enough tiles
+  const int full = 256 * (fast ? stream_blocks_per_cu<TM, KH, true>() : stream_blocks_per_cu<TM, KH, false>());
+  const int blocks = p.tiles >= 4 * full ? full : (p.tiles >= 256 ? 8 * cdiv(cdiv(p.tiles, 8), 4) : cdiv(p.tiles, 4));
   if (fast)
     hipLaunchKernelGGL((conv1x1_stream_kernel<TM, KH, true, PASS>), dim3((unsigned)blocks), dim3(256), lds, stream, p, ep, dPQ);
   else

@@ -112,12 +112,56 @@ __global__ __launch_bounds__(256) void split_reduce_vec_kernel(const float4* __r
   out[idx] = v;
 }
 
+// The same for a small dense result under many slices (a 1x1 layer's 96 x 96 gradient from a thousand slices): one
+// thread per element would be a few dozen waves that each walk every slice.  Here 32 threads share a 16-byte group:
+// thread j of them adds slices j, j + 32, ... in increasing order, and the 32 sums meet in LDS in a fixed pairwise tree.
+// A block holds eight consecutive groups (128 bytes of every slice it reads).
+constexpr int kReduceLanes = 32, kReduceGroups = 8;
+__global__ __launch_bounds__(256) void split_reduce_vec_par_kernel(const float4* __restrict__ part, int splits, long long stride4,
+                                                                   float4* __restrict__ out, unsigned total4, float alpha,
+                                                                   float beta) {
+  __shared__ float4 red[kReduceLanes][kReduceGroups];
+  const int g = (int)threadIdx.x % kReduceGroups, j = (int)threadIdx.x / kReduceGroups;
+  const unsigned idx = blockIdx.x * kReduceGroups + g;
+  float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  if (idx < total4) {
+    const float4* p = part + idx;
+    for (int s = j; s < splits; s += kReduceLanes) {
+      const float4 v = p[(long long)s * stride4];
+      a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+    }
+  }
+  red[j][g] = a;
+  for (int w = kReduceLanes / 2; w >= 1; w >>= 1) {
+    __syncthreads();
+    if (j < w) {
+      const float4 u = red[j][g], v = red[j + w][g];
+      red[j][g] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+    }
+  }
+  if (j == 0 && idx < total4) {
+    const float4 t = red[0][g];
+    float4 v = make_float4(alpha * t.x, alpha * t.y, alpha * t.z, alpha * t.w);
+    if (beta != 0.0f) {
+      const float4 o = out[idx];
+      v.x += beta * o.x; v.y += beta * o.y; v.z += beta * o.z; v.w += beta * o.w;
+    }
+    out[idx] = v;
+  }
+}
+
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
                          int ld, float alpha, float beta, hipStream_t stream) {
   const size_t total = (size_t)rows * cols;
   ProfScope prof("split_reduce", 4.0 * (double)total * (splits + 1), stream);
   if (ld == cols && total % 4 == 0 && split_stride % 4 == 0 &&
       ((reinterpret_cast<uintptr_t>(part) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+    if (total / 4 < 64 * 1024 && splits >= 2 * kReduceLanes) {   // under 1024 waves with a thread per group
+      hipLaunchKernelGGL(split_reduce_vec_par_kernel, dim3((unsigned)cdiv<size_t>(total / 4, kReduceGroups)), dim3(256), 0,
+                         stream, reinterpret_cast<const float4*>(part), splits, split_stride / 4,
+                         reinterpret_cast<float4*>(out), (unsigned)(total / 4), alpha, beta);
+      return;
+    }
     hipLaunchKernelGGL(split_reduce_vec_kernel, dim3(stream_grid(total / 4, 256)), dim3(256), 0, stream,
                        reinterpret_cast<const float4*>(part), splits, split_stride / 4, reinterpret_cast<float4*>(out),
                        (unsigned)(total / 4), alpha, beta);

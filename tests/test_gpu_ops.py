@@ -53,6 +53,9 @@ CONV_CASES = [
     (1, 128, 6, 5, 128, 1, 1, 0),
     (5, 17, 8, 8, 100, 1, 1, 0),
     (2, 64, 13, 13, 20, 1, 1, 0),
+    # enough column tiles (313 / 1250) for the per-XCD ranges, with a ragged last range and tiles that straddle images
+    (4, 64, 50, 50, 64, 1, 1, 0),
+    (5, 32, 89, 90, 96, 1, 1, 0),
 ]
 
 
