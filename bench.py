@@ -18,16 +18,50 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
-# HBM-side bytes per launch (average over the launches of one step) of the MFMA kernels of the AlexNet
-# workload, from two hardware-counter runs of this script under `rocprofv3 --pmc FETCH_SIZE` and
-# `--pmc WRITE_SIZE`; each counter scaled by what it reads for the library's plain 256 MiB copy kernel in
-# the same run (FETCH_SIZE reads 0.5 KiB per KiB copied -> x2.0, WRITE_SIZE 1.0 -> x1.0).  A counter run
-# cannot be nested inside this process, so the figures are carried here and named in `traffic_source`.
-MEASURED_TRAFFIC_BYTES = {
-    "alexnet": {"conv_bwd_filter_128x128": 1024 * (2.0 * 192077 + 62256),
-                "conv_fwd_128x128": 1024 * (2.0 * 68551 + 139719),
-                "conv_bwd_data_128x128": 1024 * (2.0 * 63353 + 84292)},
-}
+# HBM-side bytes per launch (average over the launches of one step) of the MFMA kernels come from two
+# hardware-counter runs of this script under `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`, each counter
+# scaled by what it reads for the library's plain 256 MiB copy kernel in the same run.  A counter run cannot be
+# nested inside this process, so the summary of those runs (a tracked text file) is read here; a kernel it has no
+# row for reports `traffic: null`.
+TRAFFIC_SUMMARY = {"alexnet": "profiles/alexnet_b256_train_step_hbm_traffic.md"}
+PARITY_SUMMARY = "profiles/%s_b%d_train_step_parity.md"
+TOLERANCE = "|got-ref| <= 1e-5*max(1, rms(ref)) + 1e-4*|ref| and relative L2 <= 1e-4 against the fp64-accumulating CPU oracle; " \
+            "labels, arg-max, masks, counts exact"
+
+
+def measured_traffic(workload, kernel):
+    """Bytes per launch of `kernel` from the counter summary's table: row "| `tag` | .. | fetch KiB | write KiB |",
+    scale factors from its "multiply FETCH_SIZE by F" / "multiply WRITE_SIZE by W" line."""
+    import re
+    rel = TRAFFIC_SUMMARY.get(workload)
+    path = os.path.join(ROOT, rel) if rel else None
+    if not path or not os.path.exists(path):
+        return None, None
+    text = open(path).read()
+    f = re.search(r"multiply FETCH_SIZE by ([\d.]+)", text)
+    w = re.search(r"multiply WRITE_SIZE by ([\d.]+)", text)
+    row = re.search(r"^\| `%s` \|[^|]*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|" % re.escape(kernel), text, re.M)
+    if not (f and w and row):
+        return None, rel
+    return 1024.0 * (float(f.group(1)) * float(row.group(1)) + float(w.group(1)) * float(row.group(2))), rel
+
+
+def recorded_parity(workload, batch):
+    """Worst error per tensor class of the benchmark-size parity test (tests/test_gpu_bench_size.py runs this very
+    step and checks it against the CPU oracle; this script only reports what that test recorded)."""
+    rel = PARITY_SUMMARY % (workload, batch)
+    path = os.path.join(ROOT, rel)
+    if not os.path.exists(path):
+        return {"tolerance": TOLERANCE, "recorded": None}
+    text = open(path).read()
+    a = text.find("```json")
+    if a < 0:
+        return {"tolerance": TOLERANCE, "recorded": None, "source": rel}
+    rec = json.loads(text[a + 7:text.index("```", a + 7)])
+    rec["source"] = rel
+    rec["tolerance"] = TOLERANCE
+    return rec
+
 
 BATCH = {"alexnet": 256, "lenet": 64, "cifar10": 128, "nin": 128, "resnet18": 256}
 NUM_CLASSES_SEED = 0x5EED0000
@@ -241,6 +275,7 @@ def main():
     lib.rh_profile_reset()
     lib.rh_profile_filter(None)
 
+    traffic, traffic_source = measured_traffic(args.workload, dom["kernel"]) if dom is not None else (None, None)
     gemm_ms = sum(k["ms_per_step"] for k in mfma)
     gemm_flops = configs.train_flops(net, batch)
     result = {
@@ -267,16 +302,19 @@ def main():
         "roofline": None if dom is None else
                     {"bound": dom["bound"], "kernel": dom["kernel"], "achieved": dom["achieved"], "peak": dom["peak"],
                      "unit": dom["unit"], "frac": dom["frac"], "avg_launch_ms": dom["avg_launch_ms"],
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom["kernel"]),
+                     "traffic": traffic,
                      "traffic_unit": "bytes per launch (L2<->fabric, FETCH_SIZE + WRITE_SIZE counters)",
-                     "traffic_source": "rocprofv3 --pmc runs of this script; summary under profiles/"},
+                     "traffic_source": traffic_source},
         "all_mfma": {"ms_per_step": gemm_ms, "achieved": gemm_flops / gemm_ms / 1e9 if gemm_ms else None,
                      "unit": "TFLOP/s", "frac": gemm_flops / gemm_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS if gemm_ms else None},
         "calibration": calibration,
         "kernels_note": "per-kernel table from an untimed pass of %d steps with HIP events on every launch and the "
                         "backward kernels on one stream; roofline.* is from events on the dominant forward kernel inside "
-                        "the timed region (where filter/bias gradients overlap the data gradients on a second stream)"
+                        "the timed region (where filter/bias gradients overlap the data gradients on a second stream); "
+                        "the backward-filter kernel of the same tile takes as much of a step as that forward kernel "
+                        "(see `kernels`), it is not chosen because its live durations are stretched by the other stream"
                         % breakdown_steps,
+        "parity": recorded_parity(args.workload, batch),
         "kernels": kernels,
         "final_loss": loss,
     }
