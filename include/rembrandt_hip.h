@@ -197,6 +197,13 @@ size_t rh_sgemm_workspace_bytes_upto(int32_t m, int32_t n, int32_t k, int which)
 int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k, float alpha, const float* A,
              int32_t lda, const float* B, int32_t ldb, float beta, float* C, int32_t ldc, void* ws,
              size_t ws_bytes, int flags, rh_stream_t stream);
+/* rh_sgemm followed, in the same pass over C, by what AffineOperator::forward does next (mod.rs:1168-1176: matrix_prod,
+ * then the bias row added to every column of the (out, batch) result, then the activation): with RH_FUSE_BIAS in `flags`,
+ * bias[i], i < m, is added to C(i, j) after the alpha/beta blend; with RH_FUSE_RELU the result is then clamped at 0.
+ * Each element goes through the same roundings as in the three separate calls. */
+int rh_sgemm_bias_act(int transA, int transB, int32_t m, int32_t n, int32_t k, float alpha, const float* A,
+                      int32_t lda, const float* B, int32_t ldb, float beta, float* C, int32_t ldc, const float* bias,
+                      void* ws, size_t ws_bytes, int flags, rh_stream_t stream);
 int rh_saxpy(int64_t n, float alpha, const float* x, float* y, rh_stream_t stream);
 int rh_sscal(int64_t n, float alpha, float* x, rh_stream_t stream);
 

@@ -101,6 +101,7 @@ PROTOTYPES = {
     "rembrandt_kernel_batch_map_rect_backprop_inplace": (None, [_vp, _i32, _i32, _vp, _vp]),
     "rh_sgemm_workspace_bytes": (_sz, [_i32, _i32, _i32]),
     "rh_sgemm": (_int, [_int, _int, _i32, _i32, _i32, _f, _vp, _i32, _vp, _i32, _f, _vp, _i32, _vp, _sz, _int, _vp]),
+    "rh_sgemm_bias_act": (_int, [_int, _int, _i32, _i32, _i32, _f, _vp, _i32, _vp, _i32, _f, _vp, _i32, _vp, _vp, _sz, _int, _vp]),
     "rh_saxpy": (_int, [_i64, _f, _vp, _vp, _vp]),
     "rh_sscal": (_int, [_i64, _f, _vp, _vp]),
     "rh_pool2d_out_dim": (_i32, [_i32, _i32, _i32, _i32, _i32]),

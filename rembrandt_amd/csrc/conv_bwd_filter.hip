@@ -68,9 +68,10 @@ __device__ __forceinline__ float sum_splits(const float* __restrict__ part, int 
 }
 
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
+// (+ bias_col[j], then ReLU, where given: the epilogue of an affine layer's forward product)
 __global__ void split_reduce_kernel(const float* __restrict__ part, int splits, long long split_stride,
                                     float* __restrict__ out, int rows, int cols, int ld, float alpha,
-                                    float beta) {
+                                    float beta, const float* __restrict__ bias_col, int relu) {
   const unsigned total = (unsigned)rows * (unsigned)cols;  // a filter gradient / GEMM result: far below 2^31
   for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     const float acc = sum_splits(part, splits, split_stride, idx);
@@ -78,14 +79,28 @@ __global__ void split_reduce_kernel(const float* __restrict__ part, int splits, 
     float* dst = out + (size_t)i * ld + j;
     float val = alpha * acc;
     if (beta != 0.0f) val += beta * *dst;
+    if (bias_col) val += bias_col[j];
+    if (relu) val = val > 0.0f ? val : 0.0f;
     *dst = val;
   }
 }
 
 // The same over a dense result (ld == cols) in 16-byte groups: the sums of each element are formed in the same order.
+__device__ __forceinline__ void bias_relu4(float4& v, unsigned idx, const float* __restrict__ bias_col, unsigned cols4, int relu) {
+  if (bias_col) {
+    const float4 b = reinterpret_cast<const float4*>(bias_col)[idx % cols4];
+    v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+  }
+  if (relu) {
+    v.x = v.x > 0.0f ? v.x : 0.0f; v.y = v.y > 0.0f ? v.y : 0.0f;
+    v.z = v.z > 0.0f ? v.z : 0.0f; v.w = v.w > 0.0f ? v.w : 0.0f;
+  }
+}
+
 __global__ __launch_bounds__(256) void split_reduce_vec_kernel(const float4* __restrict__ part, int splits, long long stride4,
                                                                float4* __restrict__ out, unsigned total4, float alpha,
-                                                               float beta) {
+                                                               float beta, const float* __restrict__ bias_col,
+                                                               unsigned cols4, int relu) {
   const unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total4) return;
   const float4 z = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -109,6 +124,7 @@ __global__ __launch_bounds__(256) void split_reduce_vec_kernel(const float4* __r
     const float4 o = out[idx];
     v.x += beta * o.x; v.y += beta * o.y; v.z += beta * o.z; v.w += beta * o.w;
   }
+  bias_relu4(v, idx, bias_col, cols4, relu);
   out[idx] = v;
 }
 
@@ -119,7 +135,8 @@ __global__ __launch_bounds__(256) void split_reduce_vec_kernel(const float4* __r
 constexpr int kReduceLanes = 32, kReduceGroups = 8;
 __global__ __launch_bounds__(256) void split_reduce_vec_par_kernel(const float4* __restrict__ part, int splits, long long stride4,
                                                                    float4* __restrict__ out, unsigned total4, float alpha,
-                                                                   float beta) {
+                                                                   float beta, const float* __restrict__ bias_col,
+                                                                   unsigned cols4, int relu) {
   __shared__ float4 red[kReduceLanes][kReduceGroups];
   const int g = (int)threadIdx.x % kReduceGroups, j = (int)threadIdx.x / kReduceGroups;
   const unsigned idx = blockIdx.x * kReduceGroups + g;
@@ -146,29 +163,30 @@ __global__ __launch_bounds__(256) void split_reduce_vec_par_kernel(const float4*
       const float4 o = out[idx];
       v.x += beta * o.x; v.y += beta * o.y; v.z += beta * o.z; v.w += beta * o.w;
     }
+    bias_relu4(v, idx, bias_col, cols4, relu);
     out[idx] = v;
   }
 }
 
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
-                         int ld, float alpha, float beta, hipStream_t stream) {
+                         int ld, float alpha, float beta, hipStream_t stream, const float* bias_col, int relu) {
   const size_t total = (size_t)rows * cols;
   ProfScope prof("split_reduce", 4.0 * (double)total * (splits + 1), stream);
-  if (ld == cols && total % 4 == 0 && split_stride % 4 == 0 &&
-      ((reinterpret_cast<uintptr_t>(part) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+  if (ld == cols && cols % 4 == 0 && split_stride % 4 == 0 &&
+      ((reinterpret_cast<uintptr_t>(part) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(bias_col)) & 15) == 0) {
     if (total / 4 < 64 * 1024 && splits >= 2 * kReduceLanes) {   // under 1024 waves with a thread per group
       hipLaunchKernelGGL(split_reduce_vec_par_kernel, dim3((unsigned)cdiv<size_t>(total / 4, kReduceGroups)), dim3(256), 0,
                          stream, reinterpret_cast<const float4*>(part), splits, split_stride / 4,
-                         reinterpret_cast<float4*>(out), (unsigned)(total / 4), alpha, beta);
+                         reinterpret_cast<float4*>(out), (unsigned)(total / 4), alpha, beta, bias_col, (unsigned)(cols / 4), relu);
       return;
     }
     hipLaunchKernelGGL(split_reduce_vec_kernel, dim3(stream_grid(total / 4, 256)), dim3(256), 0, stream,
                        reinterpret_cast<const float4*>(part), splits, split_stride / 4, reinterpret_cast<float4*>(out),
-                       (unsigned)(total / 4), alpha, beta);
+                       (unsigned)(total / 4), alpha, beta, bias_col, (unsigned)(cols / 4), relu);
     return;
   }
   hipLaunchKernelGGL(split_reduce_kernel, dim3(stream_grid(total, 256)), dim3(256), 0, stream, part, splits,
-                     split_stride, out, rows, cols, ld, alpha, beta);
+                     split_stride, out, rows, cols, ld, alpha, beta, bias_col, relu);
 }
 
 // ---- scalar-offset path ------------------------------------------------------------------------

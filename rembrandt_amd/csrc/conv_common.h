@@ -139,7 +139,7 @@ inline bool prefer_k8_64(long long cols) {
 
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
-                         int ld, float alpha, float beta, hipStream_t stream);
+                         int ld, float alpha, float beta, hipStream_t stream, const float* bias_col = nullptr, int relu = 0);
 
 // Tail form of a forward / backward-data launch (see EpiParams): when the tile count is not close to a multiple of
 // the 256 CUs, the column tiles beyond the last multiple are cut into `splits` slices so that every CU ends up with

@@ -553,6 +553,7 @@ struct EpiParams {
   int rows, cols, inner, ld;
   int relu;
   long long split_stride;
+  const float* bias_col = nullptr;   // one value per result column (the dense, non-NCHW form: an affine layer's bias)
   float* part = nullptr;
   long long part_first = 0;
   int full_tiles = 0, tail_tiles = 0, tail_splits = 0;
@@ -587,11 +588,13 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], co
     const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
     if (col >= ep.cols) continue;
     int coloff;
+    float cbias = 0.0f;
     if (NCHW) {
       const int img = col / ep.inner;
       coloff = img * ep.rows * ep.inner + (col - img * ep.inner);
     } else {
       coloff = col;
+      if (!split && ep.bias_col) cbias = ep.bias_col[col];
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -604,6 +607,7 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], co
           float val = alpha * acc[i][j][v];
           if (beta != 0.0f) val += beta * *dst;
           if (!split && ep.bias) val += ep.bias[row];
+          if (!NCHW && !split && ep.bias_col) val += cbias;
           if (!split && ep.relu) val = val > 0.0f ? val : 0.0f;
           *dst = val;
         }

@@ -640,7 +640,7 @@ class AffineOperator : public Operator {
  public:
   AffineOperator(size_t batch_size, OpCapability capability, const AffineOperatorConfig& config, const Operator* prev_op,
                  Ctx context, const ExecOptions& opts)
-      : batch_cap_(batch_size), config_(config), context_(context),
+      : batch_cap_(batch_size), config_(config), context_(context), fuse_epilogue_(opts.fuse_epilogue),
         overlap_built_(opts.overlap_backward && backward_enabled(capability)), overlap_on_(overlap_built_) {
     RB_ASSERT(prev_op != nullptr);
     in_act_ = prev_op->get_output_vars();
@@ -673,6 +673,14 @@ class AffineOperator : public Operator {
     const int i = (int)config_.in_channels, o = (int)config_.out_channels, b = (int)batch_size;
     rh_stream_t s = context_->stream();
     // out_act(out, B) = weights(in, out)^T * in_act(in, B)
+    const bool rect = config_.act_func == ActivationFunction::Rect;
+    if (fuse_epilogue_ && (rect || config_.act_func == ActivationFunction::Identity)) {
+      // bias and activation in the product's epilogue: one kernel for the reference's three
+      unwrap(rh_sgemm_bias_act(1, 0, o, b, i, 1.0f, params_.weights->as_ptr(), i, in_act_->as_ptr(), i, 0.0f,
+                               out_act_->as_mut_ptr(), o, params_.bias->as_ptr(), ws_ptr(), ws_len(),
+                               RH_FUSE_BIAS | (rect ? RH_FUSE_RELU : 0), s), "matrix_prod");
+      return;
+    }
     unwrap(rh_sgemm(1, 0, o, b, i, 1.0f, params_.weights->as_ptr(), i, in_act_->as_ptr(), i, 0.0f,
                     out_act_->as_mut_ptr(), o, ws_ptr(), ws_len(), 0, s), "matrix_prod");
     unwrap(rh_add_bias_nchw(params_.bias->as_ptr(), out_act_->as_mut_ptr(), 1, o, b, 1.0f, 1.0f, s), "add_bias");
@@ -740,6 +748,7 @@ class AffineOperator : public Operator {
   size_t batch_cap_;
   AffineOperatorConfig config_;
   Ctx context_;
+  bool fuse_epilogue_;               // bias and activation inside the forward product
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   ParamTensors params_;
   std::unique_ptr<DeviceBuffer<uint8_t>> workspace_, workspace_aux_;

@@ -153,6 +153,16 @@ extern "C" size_t rh_sgemm_workspace_bytes_upto(int32_t m, int32_t n, int32_t k,
 extern "C" int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k, float alpha, const float* A,
                         int32_t lda, const float* B, int32_t ldb, float beta, float* C, int32_t ldc,
                         void* ws, size_t ws_bytes, int flags, rh_stream_t stream_) {
+  return rh_sgemm_bias_act(transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, nullptr, ws, ws_bytes, flags,
+                           stream_);
+}
+
+extern "C" int rh_sgemm_bias_act(int transA, int transB, int32_t m, int32_t n, int32_t k, float alpha, const float* A,
+                                 int32_t lda, const float* B, int32_t ldb, float beta, float* C, int32_t ldc,
+                                 const float* bias, void* ws, size_t ws_bytes, int flags, rh_stream_t stream_) {
+  if ((flags & RH_FUSE_BIAS) && !bias) return RH_E_INVALID;
+  const float* bias_col = (flags & RH_FUSE_BIAS) ? bias : nullptr;
+  const int relu = (flags & RH_FUSE_RELU) ? 1 : 0;
   if (m < 0 || n < 0 || k < 0 || !C) return RH_E_INVALID;
   if (m == 0 || n == 0) return 0;
   if (k > 0 && (!A || !B)) return RH_E_INVALID;
@@ -176,7 +186,8 @@ extern "C" int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k,
   if (plan.splits > 1 && (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255))) plan.splits = 1;
 
   EpiParams ep;
-  ep.bias = nullptr; ep.alpha = alpha; ep.beta = beta; ep.rows = n; ep.cols = m; ep.inner = 0; ep.relu = 0;
+  ep.bias = nullptr; ep.alpha = alpha; ep.beta = beta; ep.rows = n; ep.cols = m; ep.inner = 0;
+  ep.relu = relu; ep.bias_col = bias_col;   // (ignored by blocks that write partial sums)
   if (plan.splits > 1) {
     ep.out = static_cast<float*>(ws); ep.ld = m; ep.split_stride = (long long)m * n;
   } else {
@@ -190,7 +201,8 @@ extern "C" int rh_sgemm(int transA, int transB, int32_t m, int32_t n, int32_t k,
   else                         e = dispatch_tile<true, true>(plan.bm, ap, bp, ep, k, plan.splits, &used, stream);
   if (e) return e;
   if (plan.splits > 1) {
-    launch_split_reduce(static_cast<const float*>(ws), used, (long long)m * n, C, n, m, ldc, alpha, beta, stream);
+    launch_split_reduce(static_cast<const float*>(ws), used, (long long)m * n, C, n, m, ldc, alpha, beta, stream, bias_col,
+                        relu);
     return launch_status();
   }
   return 0;

@@ -120,15 +120,21 @@ def rect_backprop_inplace(y, dy):
     return dy
 
 
-def sgemm(transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, use_workspace=True):
+def sgemm(transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, use_workspace=True, bias=None, relu=False):
+    """C = alpha op(A) op(B) + beta C; with `bias` (length m) and / or `relu` through rh_sgemm_bias_act."""
     ws, nbytes = None, 0
     if use_workspace:
         nbytes = lib().rh_sgemm_workspace_bytes(m, n, k)
         if nbytes:
             ws = workspace(nbytes, Cm.device)
             nbytes = ws.numel()
-    check(lib().rh_sgemm(int(transA), int(transB), m, n, k, alpha, _p(A), lda, _p(B), ldb, beta, _p(Cm), ldc,
-                         _p(ws), nbytes, 0, _stream()), "rh_sgemm")
+    if bias is None and not relu:
+        check(lib().rh_sgemm(int(transA), int(transB), m, n, k, alpha, _p(A), lda, _p(B), ldb, beta, _p(Cm), ldc,
+                             _p(ws), nbytes, 0, _stream()), "rh_sgemm")
+        return Cm
+    flags = (_lib.RH_FUSE_BIAS if bias is not None else 0) | (_lib.RH_FUSE_RELU if relu else 0)
+    check(lib().rh_sgemm_bias_act(int(transA), int(transB), m, n, k, alpha, _p(A), lda, _p(B), ldb, beta, _p(Cm), ldc,
+                                  _p(bias), _p(ws), nbytes, flags, _stream()), "rh_sgemm_bias_act")
     return Cm
 
 

@@ -178,6 +178,40 @@ def test_sgemm(dev, case, use_ws):
         assert np.array_equal(got[:, m:], C0[:, m:]), "sgemm wrote outside ldc padding"
 
 
+@pytest.mark.parametrize("case", [
+    # (m = out channels, n = batch, k = in channels): one block, several tiles, a split contraction with the dense
+    # 16-byte reduction, one with the many-slice reduction, odd extents with a padded result (scalar reduction)
+    (10, 4, 50), (500, 64, 800), (4096, 32, 1024), (96, 16, 9216), (1001, 33, 2450), (1000, 256, 4096),
+])
+def test_sgemm_bias_act(dev, case):
+    """rh_sgemm_bias_act = matrix product, bias row, activation of the affine forward pass in one call: bit-identical
+    to the library's own three calls, and within tolerance of the oracle's."""
+    m, n, k = case
+    W = synth.normal(14, 1, (m, k))
+    X = synth.normal(14, 2, (n, k))
+    b = synth.normal(14, 3, (m,))
+    for ldc, use_ws, relu, beta in ((m, True, True, 0.0), (m + (4 if m % 4 == 0 else 3), True, True, 0.0),
+                                    (m, False, False, 0.0), (m, True, True, 0.5)):
+        say("sgemm_bias_act", case, "ldc", ldc, "ws", use_ws, "relu", relu, "beta", beta)
+        C0 = synth.normal(14, 4, (n, ldc))
+        ref = O.sgemm(1, 0, m, n, k, 1.0, W, k, X, k, beta, C0.copy(), ldc)
+        ref[:, :m] += b[None, :]
+        if relu:
+            ref[:, :m] = np.maximum(ref[:, :m], 0)
+        Cd = T(C0, dev)
+        ops.sgemm(1, 0, m, n, k, 1.0, T(W, dev), k, T(X, dev), k, beta, Cd, ldc, use_workspace=use_ws, bias=T(b, dev), relu=relu)
+        got = N(Cd)
+        assert_close(got[:, :m], ref[:, :m], "sgemm_bias_act")
+        assert np.array_equal(got[:, m:], C0[:, m:]), "wrote into the ldc padding"
+        if ldc == m:
+            Cs = T(C0, dev)
+            ops.sgemm(1, 0, m, n, k, 1.0, T(W, dev), k, T(X, dev), k, beta, Cs, ldc, use_workspace=use_ws)
+            ops.add_bias_nchw(T(b, dev), Cs.view(n, m, 1, 1))
+            if relu:
+                ops.rect_inplace(Cs)
+            assert np.array_equal(N(Cs), got), "fused and separate calls differ"
+
+
 def test_bias_relu(dev):
     for shape in [(3, 7, 5, 9), (2, 96, 27, 27), (64, 500), (5, 3, 16, 20)]:
         say("bias/relu", shape)
