@@ -41,7 +41,7 @@ static BwdFilterPlan plan_bwd_filter(const ConvDims& d) {
   // steps so the prologue and the partial-sum traffic stay small next to the contraction.
   const int slots = resident_slots(p.bm, p.bn);
   int want = slots / p.tiles;
-  const int max_by_depth = k_chunks / 32 > 0 ? k_chunks / 32 : 1;
+  const int max_by_depth = (int)slices_by_depth(k_chunks, p.tiles, slots, 32, 8);
   if (want > max_by_depth) want = max_by_depth;
   if (want > 512) want = 512;
   if (want < 1) want = 1;
@@ -231,7 +231,7 @@ static BwdFilterSoffPlan plan_bwd_filter_soff(const ConvDims& d) {
   const int k_chunks = p.n_k / 16;
   const int slots = resident_slots(p.bm, p.bn);
   int want = slots / p.tiles;
-  const int max_by_depth = k_chunks / 32 > 0 ? k_chunks / 32 : 1;
+  const int max_by_depth = (int)slices_by_depth(k_chunks, p.tiles, slots, 32, 8);
   if (want > max_by_depth) want = max_by_depth;
   if (want > 256) want = 256;
   if (want < 1) want = 1;

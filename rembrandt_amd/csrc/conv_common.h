@@ -199,15 +199,26 @@ struct SoffPlan {
 // (small images late in a network, small batches) cuts the contraction into slices so that the slots fill; every
 // slice keeps at least 16 K steps.  Partial results go to scratch slabs shaped like the output and are added in a
 // fixed order by split_reduce_nchw.  Returns the slice count (1: no split).
+// How many slices the depth of a contraction allows: every slice keeps `normal_min` K steps, so that prologue and
+// partial-sum traffic stay small next to it.  Where even that many slices leave three quarters of the block slots
+// empty (the layers of a small network at a small batch) a block's chain of K steps, each a memory round trip, is
+// what the kernel takes, and the slices go down to `small_min` steps.
+inline long long slices_by_depth(long long k_steps, long long tiles, long long slots, int normal_min, int small_min) {
+  long long by = k_steps / normal_min;
+  if (by < 1) by = 1;
+  if (tiles * by * 4 <= slots) by = k_steps / small_min;
+  return by < 1 ? 1 : by;
+}
+
 inline int plan_k_split(int rows, long long cols, int n_k) {
   const int bm = pick_bm(rows), bn = bm >= 96 ? 128 : 256;
   const long long slots = 256 * (bm >= 96 ? 4 : 3);
   const long long tiles = (long long)cdiv(rows, bm) * cdiv<long long>(cols, bn);
   if (tiles * 2 > slots) return 1;
   long long want = slots / tiles;
-  const long long by_depth = (n_k / 16) / 16;
+  const long long by_depth = slices_by_depth(n_k / 16, tiles, slots, 16, 4);
   if (want > by_depth) want = by_depth;
-  if (want > 16) want = 16;
+  if (want > 16) want = tiles * 64 <= slots ? (want > 32 ? 32 : want) : 16;
   return want < 3 ? 1 : (int)want;   // two slices only trade one round of blocks for the partial-sum traffic
 }
 

@@ -23,7 +23,7 @@ static SgemmPlan plan_sgemm(int m, int n, int k) {
   const int slots = 256 * (p.bm == 128 ? RH_OCC_128 : 3);  // blocks of this tile the GPU holds at a time
   if (tiles <= slots / 2) {
     want = slots / tiles;
-    const int max_by_depth = k_chunks / 16 > 0 ? k_chunks / 16 : 1;
+    const int max_by_depth = (int)slices_by_depth(k_chunks, tiles, slots, 16, 4);
     if (want > max_by_depth) want = max_by_depth;
     if (want > 64) want = 64;
   }
