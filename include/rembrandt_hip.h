@@ -256,6 +256,14 @@ void rembrandt_kernel_batch_blockreduce_sum(const float* src, int32_t len, int32
 void rembrandt_kernel_batch_blockreduce_argmax(const float* src, int32_t len, int32_t batch,
                                                float* max_out, int32_t* idx_out,
                                                rh_stream_t stream);
+/* The five calls above as one launch, for a train step (SgdOpt::train, src/opt/sgd/new.rs:383-420: forward,
+ * store_output_categories, store_loss, then backward starts with the loss operator): p = softmax(x) (N rows of C),
+ * max_out / idx_out = row maximum and lowest arg-max of p, loss1[n] = -weights[n] log p[n, labels[n]],
+ * loss_sum[0] = sum_n loss1[n], dx[n, c] = weights[n] (p[n, c] - [c == labels[n]]).  Bit-identical to the separate
+ * calls.  `counter` is one device word that is zero before the first call; every call leaves it zero. */
+int rh_softmax_kl_step(const float* x, int32_t C, int32_t N, const int32_t* labels, const float* weights, float* p,
+                       float* max_out, int32_t* idx_out, float* loss1, float* loss_sum, float* dx, uint32_t* counter,
+                       rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * SGD.  rh_sgd_momentum_step is the fused form of the BLAS-1 sequence regularize ->

@@ -168,6 +168,33 @@ __global__ __launch_bounds__(256) void split_reduce_vec_par_kernel(const float4*
   }
 }
 
+// The many-slice form for results that are not dense 16-byte groups (odd extents, a padded leading dimension).
+__global__ __launch_bounds__(256) void split_reduce_par_kernel(const float* __restrict__ part, int splits, long long split_stride,
+                                                               float* __restrict__ out, int rows, int cols, int ld, float alpha,
+                                                               float beta, const float* __restrict__ bias_col, int relu) {
+  __shared__ float red[kReduceLanes][kReduceGroups];
+  const int g = (int)threadIdx.x % kReduceGroups, j = (int)threadIdx.x / kReduceGroups;
+  const unsigned total = (unsigned)rows * (unsigned)cols;
+  const unsigned idx = blockIdx.x * kReduceGroups + g;
+  float a = 0.0f;
+  if (idx < total)
+    for (int s = j; s < splits; s += kReduceLanes) a += part[(long long)s * split_stride + idx];
+  red[j][g] = a;
+  for (int w = kReduceLanes / 2; w >= 1; w >>= 1) {
+    __syncthreads();
+    if (j < w) red[j][g] += red[j + w][g];
+  }
+  if (j == 0 && idx < total) {
+    const int i = (int)(idx / (unsigned)cols), c = (int)(idx - (unsigned)i * (unsigned)cols);
+    float* dst = out + (size_t)i * ld + c;
+    float val = alpha * red[0][g];
+    if (beta != 0.0f) val += beta * *dst;
+    if (bias_col) val += bias_col[c];
+    if (relu) val = val > 0.0f ? val : 0.0f;
+    *dst = val;
+  }
+}
+
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
                          int ld, float alpha, float beta, hipStream_t stream, const float* bias_col, int relu) {
   const size_t total = (size_t)rows * cols;
@@ -183,6 +210,11 @@ void launch_split_reduce(const float* part, int splits, long long split_stride, 
     hipLaunchKernelGGL(split_reduce_vec_kernel, dim3(stream_grid(total / 4, 256)), dim3(256), 0, stream,
                        reinterpret_cast<const float4*>(part), splits, split_stride / 4, reinterpret_cast<float4*>(out),
                        (unsigned)(total / 4), alpha, beta, bias_col, (unsigned)(cols / 4), relu);
+    return;
+  }
+  if (total < 256 * 1024 && splits >= 2 * kReduceLanes) {
+    hipLaunchKernelGGL(split_reduce_par_kernel, dim3((unsigned)cdiv<size_t>(total, kReduceGroups)), dim3(256), 0, stream, part,
+                       splits, split_stride, out, rows, cols, ld, alpha, beta, bias_col, relu);
     return;
   }
   hipLaunchKernelGGL(split_reduce_kernel, dim3(stream_grid(total, 256)), dim3(256), 0, stream, part, splits,
@@ -701,8 +733,13 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
   return launch_status();
 }
 
+// Up to this many elements of dy one launch (a block per channel) is as fast as the first of the two stages, and the
+// small layers it covers are bound by the number of dependent launches.
+constexpr long long kBiasOneStageElems = 1ll << 20;
+
 extern "C" size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane) {
   if (N <= 0 || K <= 0 || plane <= 1) return 0;
+  if ((long long)N * K * plane <= kBiasOneStageElems) return 0;
   if (plane < kBiasSmallPlane) return align256(sizeof(float) * (size_t)bwd_bias_col_groups(N, (long long)K * plane) * K * plane);
   return align256(sizeof(float) * (size_t)N * K);
 }

@@ -36,6 +36,7 @@ struct rho_worker {
   std::shared_ptr<DeviceContext> ctx;
   std::unique_ptr<SequentialOperatorWorker> worker;
   bool graph_steps = false;
+  bool fuse_epilogue = false;                // also: the loss operator's one-launch form inside rho_sgd_train_batch
   int64_t graph_launches = 0;                // steps that ran as a graph launch
   std::map<StepKey, rh_graph*> step_graphs;  // recorded steps
   std::set<StepKey> seen_steps;              // combinations that ran once launch by launch
@@ -269,6 +270,7 @@ int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, ui
     opts.overlap_backward = (exec_flags & RHO_EXEC_OVERLAP_BACKWARD) != 0;
     opts.graph_steps = (exec_flags & RHO_EXEC_GRAPH_STEPS) != 0;
     w->graph_steps = opts.graph_steps;
+    w->fuse_epilogue = opts.fuse_epilogue;
     w->worker.reset(new SequentialOperatorWorker(cfg->cfg, (size_t)batch_size,
                                                  capability == RHO_CAP_FORWARD ? OpCapability::Forward : OpCapability::Backward,
                                                  seed, w->ctx, opts));
@@ -538,6 +540,13 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
     const size_t b = (size_t)batch_size;
     const size_t t = s->opt->iter_counter();
     const OpPhase phase = OpPhase::Training(t);
+    // With fused epilogues the loss operator produces probabilities, categories, loss and delta in one launch of its
+    // forward(); the three calls below that ask for them then launch nothing.
+    struct Armed {
+      LossOperator* l;
+      Armed(LossOperator* l_, bool on) : l(on && l_->arm_train_step(true) ? l_ : nullptr) {}
+      ~Armed() { if (l) l->arm_train_step(false); }
+    } armed(op->loss_operator(0), w->fuse_epilogue);
     // forward -> arg-max and loss kernels -> backward -> update are all enqueued before the two read-backs, so
     // the GPU works through the step without waiting for the host (same results as the reference's order:
     // store_output_categories, store_loss, backward; nothing in between writes what they read)

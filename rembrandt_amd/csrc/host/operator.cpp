@@ -1609,9 +1609,10 @@ class SoftmaxKLLossOperator : public LossOperator {
         label_cats_(batch_size, context), label_cats_h_(batch_size, 0), weights_(batch_size, context),
         weights_h_(batch_size, 0.0f), out_values_(loss_config.num_categories * batch_size, context),
         max_value_(batch_size, context), out_cats_(batch_size, context), out_cats_h_(batch_size, 0),
-        out_loss1_(batch_size, context), out_loss_(1, context), acc_loss_(1, context),
+        out_loss1_(batch_size, context), out_loss_(1, context), acc_loss_(1, context), step_counter_(1, context),
         readback_((batch_size + 1) * 4, context) {
     RB_ASSERT(prev_op != nullptr);
+    unwrap(rh_memset_f32(step_counter_.as_mut_ptr(), 0.0f, 1, context_->stream()), "set_constant");
     in_act_ = prev_op->get_output_vars();
     if (!in_act_) panic("SoftmaxKLLossOperator missing required prev operator output vars");
     in_delta_ = prev_op->get_output_deltas();
@@ -1619,13 +1620,29 @@ class SoftmaxKLLossOperator : public LossOperator {
     RB_ASSERT(in_act_->len() >= loss_config.num_categories * batch_size);
   }
   size_t batch_size() const override { return batch_cap_; }
-  void forward(size_t batch_size, OpPhase) override {
+  void forward(size_t batch_size, OpPhase phase) override {
     RB_ASSERT(batch_size <= batch_cap_);
+    step_valid_ = 0;
+    if (armed_ && phase.training) {
+      unwrap(rh_softmax_kl_step(in_act_->as_ptr(), (int)loss_config_.num_categories, (int)batch_size, label_cats_.as_ptr(),
+                                weights_.as_ptr(), out_values_.as_mut_ptr(), max_value_.as_mut_ptr(), out_cats_.as_mut_ptr(),
+                                out_loss1_.as_mut_ptr(), out_loss_.as_mut_ptr(),
+                                in_delta_->as_mut_ptr(), reinterpret_cast<uint32_t*>(step_counter_.as_mut_ptr()),
+                                context_->stream()), "softmax / loss step");
+      step_valid_ = batch_size;
+      return;
+    }
     unwrap(rh_softmax_fwd(in_act_->as_ptr(), out_values_.as_mut_ptr(), (int)loss_config_.num_categories, (int)batch_size,
                           context_->stream()), "softmax forward");
   }
+  bool arm_train_step(bool on) override {
+    armed_ = on;
+    if (!on) step_valid_ = 0;
+    return true;
+  }
   void backward(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
+    if (step_valid_ == batch_size && batch_size > 0) return;   // forward() already left the delta in in_delta_
     rembrandt_kernel_batch_map_softmax_kl_backward(out_values_.as_ptr(), (int)loss_config_.num_categories, (int)batch_size,
                                                    label_cats_.as_ptr(), weights_.as_ptr(), in_delta_->as_mut_ptr(),
                                                    context_->stream());
@@ -1638,6 +1655,7 @@ class SoftmaxKLLossOperator : public LossOperator {
   }
   void load_labels(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
+    step_valid_ = 0;
     label_cats_.sync_load(label_cats_h_.data(), batch_cap_);
   }
   void stage_weight(size_t batch_idx, float weight) override {
@@ -1646,6 +1664,7 @@ class SoftmaxKLLossOperator : public LossOperator {
   }
   void load_weights(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
+    step_valid_ = 0;
     weights_.sync_load(weights_h_.data(), batch_cap_);
   }
   float store_loss(size_t batch_size) override {
@@ -1654,6 +1673,7 @@ class SoftmaxKLLossOperator : public LossOperator {
   }
   void enqueue_loss(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
+    if (step_valid_ == batch_size && batch_size > 0) return;
     rh_stream_t s = context_->stream();
     rembrandt_kernel_batch_map_softmax_kl_loss1(out_values_.as_ptr(), (int)loss_config_.num_categories, (int)batch_size,
                                                 label_cats_.as_ptr(), weights_.as_ptr(), 0.0f, out_loss1_.as_mut_ptr(), s);
@@ -1696,6 +1716,7 @@ class SoftmaxKLLossOperator : public LossOperator {
   }
   void enqueue_output_categories(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
+    if (step_valid_ == batch_size && batch_size > 0) return;
     rembrandt_kernel_batch_blockreduce_argmax(out_values_.as_ptr(), (int)loss_config_.num_categories, (int)batch_size,
                                               max_value_.as_mut_ptr(), out_cats_.as_mut_ptr(), context_->stream());
     unwrap_last("rembrandt_kernel_batch_blockreduce_argmax");
@@ -1743,8 +1764,11 @@ class SoftmaxKLLossOperator : public LossOperator {
   std::vector<float> weights_h_;
   DeviceBuffer<float> out_values_, max_value_;
   DeviceBuffer<int32_t> out_cats_;
+  bool armed_ = false;       // arm_train_step
+  size_t step_valid_ = 0;    // batch size whose categories, loss and delta the last forward() produced; 0: none
   std::vector<int32_t> out_cats_h_;
   DeviceBuffer<float> out_loss1_, out_loss_, acc_loss_;
+  DeviceBuffer<float> step_counter_;   // the one word rh_softmax_kl_step counts its blocks in (zero between calls)
   PinnedBytes readback_;  // categories, then the loss: what begin_fetch copies
 };
 

@@ -392,6 +392,11 @@ class LossOperator : public Operator {
   virtual float finish_fetch(size_t batch_size) = 0;
   virtual const int32_t* get_output_categories(size_t batch_size) const = 0;
   virtual size_t accuracy_count(size_t batch_size) const = 0;
+  // A train step asks the loss operator for its probabilities, predicted categories, loss and delta in a fixed
+  // order with nothing in between that changes their inputs (labels and weights are loaded before the step).  While
+  // armed, a training-phase forward() produces all four in one launch, and the enqueue_output_categories,
+  // enqueue_loss and backward calls that follow it launch nothing.  Returns false where there is no such form.
+  virtual bool arm_train_step(bool on) { (void)on; return false; }
 };
 
 // ---- graph ----------------------------------------------------------------------------------------

@@ -109,6 +109,76 @@ __global__ __launch_bounds__(256) void blockreduce_argmax_kernel(const float* __
   }
 }
 
+// Everything a train step takes from the loss operator, in one launch of one block per sample row: softmax_fwd, the
+// row arg-max of the probabilities, loss1 (factor 0), the KL backward into dx, and, by the block that finishes last
+// (a device-wide counter that this block leaves at zero again), blockreduce_sum of loss1 into loss_sum.  Each value is
+// formed by the same operations in the same order as in the separate kernels above: the results are bit-identical.
+__global__ __launch_bounds__(256) void softmax_kl_step_kernel(const float* __restrict__ x, int C, int N,
+                                                              const int* __restrict__ labels,
+                                                              const float* __restrict__ weights, float* __restrict__ p,
+                                                              float* __restrict__ max_out, int* __restrict__ idx_out,
+                                                              float* __restrict__ loss1, float* __restrict__ loss_sum,
+                                                              float* __restrict__ dx, unsigned* __restrict__ counter) {
+  __shared__ float sm[4];
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  __shared__ bool last;
+  const int n = blockIdx.x;
+  const float* xr = x + (size_t)n * C;
+  float* pr = p + (size_t)n * C;
+  float* dr = dx + (size_t)n * C;
+  float mx = -INFINITY;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) mx = fmaxf(mx, xr[c]);
+  mx = block_reduce_max(mx, sm);
+  float z = 0.0f;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) z += expf(xr[c] - mx);
+  z = block_reduce_sum(z, sm);
+  const float inv = 1.0f / z;
+  const int label = labels[n];
+  const float wgt = weights[n];
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float v = expf(xr[c] - mx) * inv;
+    asm volatile("" : "+v"(v));   // the rounded product, as the separate kernels read it back: no fused multiply-subtract below
+    pr[c] = v;
+    if (v > best || bi == 0x7fffffff) { best = v; bi = c; }
+    dr[c] = wgt * (v - (c == label ? 1.0f : 0.0f));
+    if (c == label) loss1[n] = -wgt * logf(v);
+  }
+  if (threadIdx.x == 0 && (unsigned)label >= (unsigned)C) loss1[n] = NAN;
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_down(best, o, 64);
+    const int oi = __shfl_down(bi, o, 64);
+    if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { sv[wave] = best; si[wave] = bi; }
+  __threadfence();   // this row's loss1 is visible device-wide before the block is counted
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) {
+      const float ov = sv[w];
+      const int oi = si[w];
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
+    }
+    max_out[n] = best;
+    idx_out[n] = bi == 0x7fffffff ? 0 : bi;
+    last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)N - 1u;
+  }
+  __syncthreads();
+  if (!last) return;
+  __threadfence();
+  float acc = 0.0f;
+  for (int i = threadIdx.x; i < N; i += blockDim.x)
+    acc += __hip_atomic_load(loss1 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  acc = block_reduce_sum(acc, sm);
+  if (threadIdx.x == 0) {
+    loss_sum[0] = acc;
+    *counter = 0u;
+  }
+}
+
 }  // namespace rh
 
 using namespace rh;
@@ -159,4 +229,16 @@ extern "C" void rembrandt_kernel_batch_blockreduce_argmax(const float* src, int3
   hipLaunchKernelGGL(blockreduce_argmax_kernel, dim3(batch), dim3(256), 0, to_stream(stream), src, len, max_out,
                      idx_out);
   g_last_error = launch_status();
+}
+
+extern "C" int rh_softmax_kl_step(const float* x, int32_t C, int32_t N, const int32_t* labels, const float* weights,
+                                  float* p, float* max_out, int32_t* idx_out, float* loss1, float* loss_sum, float* dx,
+                                  uint32_t* counter, rh_stream_t stream) {
+  if (!x || !labels || !weights || !p || !max_out || !idx_out || !loss1 || !loss_sum || !dx || !counter || C <= 0 || N < 0)
+    return RH_E_INVALID;
+  if (N == 0) return 0;
+  ProfScope prof("softmax_kl_step", 16.0 * (double)C * N, to_stream(stream));
+  hipLaunchKernelGGL(softmax_kl_step_kernel, dim3(N), dim3(256), 0, to_stream(stream), x, C, N, labels, weights, p, max_out,
+                     idx_out, loss1, loss_sum, dx, counter);
+  return launch_status();
 }

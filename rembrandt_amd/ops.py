@@ -224,6 +224,22 @@ def blockreduce_argmax(src):
     return mx, idx
 
 
+def softmax_kl_step(x, labels, weights, counter=None):
+    """softmax, row arg-max, per-sample loss, its sum and the KL backward in one launch (rh_softmax_kl_step).
+    Returns (p, row max, arg-max, loss1, loss sum, dx, counter)."""
+    N, Cc = x.shape
+    p, dx = torch.empty_like(x), torch.empty_like(x)
+    mx = torch.empty((N,), dtype=torch.float32, device=x.device)
+    idx = torch.empty((N,), dtype=torch.int32, device=x.device)
+    loss1 = torch.empty((N,), dtype=torch.float32, device=x.device)
+    total = torch.empty((1,), dtype=torch.float32, device=x.device)
+    if counter is None:
+        counter = torch.zeros((1,), dtype=torch.int32, device=x.device)
+    check(lib().rh_softmax_kl_step(_p(x), Cc, N, _p(labels), _p(weights), _p(p), _p(mx), _p(idx), _p(loss1), _p(total),
+                                   _p(dx), _p(counter), _stream()), "rh_softmax_kl_step")
+    return p, mx, idx, loss1, total, dx, counter
+
+
 def sgd_momentum_step(W, g, v, l2, scale, mu, apply, zero_grad=True):
     check(lib().rh_sgd_momentum_step(W.numel(), _p(W), _p(g), _p(v), l2, scale, mu, apply, int(zero_grad),
                                      _stream()), "rh_sgd_momentum_step")

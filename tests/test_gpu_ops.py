@@ -298,6 +298,34 @@ def test_softmax_loss_argmax(dev, shape):
     assert np.array_equal(N(mx), mx_ref)
 
 
+@pytest.mark.parametrize("shape", [(1, 1), (3, 10), (64, 10), (128, 1000), (256, 1000), (700, 37), (5, 3000)])
+def test_softmax_kl_step_equals_separate_calls(dev, shape):
+    """The one-launch form of the loss operator's train step is bit-identical to the five separate kernels, three
+    calls in a row on one counter word (the kernel leaves it at zero)."""
+    Nn, C = shape
+    counter = None
+    for rep in range(3):
+        say("softmax_kl_step", shape, "call", rep)
+        x = synth.normal(17, rep + 1, shape, 0.0, 3.0)
+        if rep == 2 and C > 2:
+            x[:, 1] = x[:, 0] = x.max(axis=1) + 1.0      # ties for the maximum: the lowest index wins
+        labels = synth.integers(17, 10 + rep, (Nn,), C)
+        weights = synth.uniform(17, 20 + rep, (Nn,), 0.1, 1.0)
+        xd, ld, wd = T(x, dev), T(labels, dev), T(weights, dev)
+        p, mx, idx, l1, tot, dx, counter = ops.softmax_kl_step(xd, ld, wd, counter)
+        p_s = ops.softmax_fwd(xd)
+        mx_s, idx_s = ops.blockreduce_argmax(p_s)
+        l1_s = ops.softmax_kl_loss1(p_s, ld, wd)
+        tot_s = ops.blockreduce_sum(l1_s.reshape(1, Nn))
+        dx_s = ops.softmax_kl_backward(p_s, ld, wd)
+        for name, a, b in (("p", p, p_s), ("max", mx, mx_s), ("argmax", idx, idx_s), ("loss1", l1, l1_s), ("loss", tot, tot_s),
+                           ("dx", dx, dx_s)):
+            assert np.array_equal(N(a), N(b)), name
+        assert int(N(counter)[0]) == 0
+        assert_close(N(p), O.softmax_fwd(x), "softmax", atol=1e-7)
+        assert np.array_equal(N(idx), O.blockreduce_argmax(N(p))[1])
+
+
 def test_argmax_ties(dev):
     x = np.zeros((4, 700), np.float32)
     x[0, [5, 300, 699]] = 2.0
