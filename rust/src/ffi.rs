@@ -67,7 +67,10 @@ extern "C" {
   pub fn rh_store_sync(ctx: *mut rh_ctx, dst_h: *mut c_void, src_d: *const c_void, bytes: size_t) -> c_int;
   pub fn rh_cast_u8_f32(x: *const u8, y: *mut f32, n: size_t, scale: c_float, stream: rh_stream_t) -> c_int;
 
+  pub fn rh_conv2d_out_dim(input: i32, size: i32, stride: i32, pad: i32) -> i32;
+  pub fn rh_pool2d_out_dim(input: i32, size: i32, stride: i32, pad: i32, round: i32) -> i32;
   pub fn rh_conv2d_workspace_bytes(g: *const rh_conv_geom, pass: c_int) -> size_t;
+  pub fn rh_conv2d_workspace_bytes_upto(g: *const rh_conv_geom, pass: c_int) -> size_t;
   pub fn rh_conv2d_fwd(g: *const rh_conv_geom, alpha: c_float, x: *const f32, w: *const f32, beta: c_float,
                        y: *mut f32, bias: *const f32, ws: *mut c_void, ws_bytes: size_t, flags: c_int,
                        stream: rh_stream_t) -> c_int;
@@ -94,6 +97,10 @@ extern "C" {
   pub fn rh_sgemm(trans_a: c_int, trans_b: c_int, m: i32, n: i32, k: i32, alpha: c_float, a: *const f32,
                   lda: i32, b: *const f32, ldb: i32, beta: c_float, c: *mut f32, ldc: i32, ws: *mut c_void,
                   ws_bytes: size_t, flags: c_int, stream: rh_stream_t) -> c_int;
+  pub fn rh_sgemm_workspace_bytes_upto(m: i32, n: i32, k: i32, which: c_int) -> size_t;
+  pub fn rh_sgemm_bias_act(trans_a: c_int, trans_b: c_int, m: i32, n: i32, k: i32, alpha: c_float, a: *const f32,
+                           lda: i32, b: *const f32, ldb: i32, beta: c_float, c: *mut f32, ldc: i32, bias: *const f32,
+                           ws: *mut c_void, ws_bytes: size_t, flags: c_int, stream: rh_stream_t) -> c_int;
   pub fn rh_saxpy(n: i64, alpha: c_float, x: *const f32, y: *mut f32, stream: rh_stream_t) -> c_int;
   pub fn rh_sscal(n: i64, alpha: c_float, x: *mut f32, stream: rh_stream_t) -> c_int;
 
@@ -113,6 +120,14 @@ extern "C" {
                                                 beta: c_float, stream: rh_stream_t);
   pub fn rembrandt_kernel_batch_blockreduce_argmax(src: *const f32, len: i32, batch: i32, max_out: *mut f32,
                                                    idx_out: *mut i32, stream: rh_stream_t);
+
+  // The five loss-operator calls of a train step as one launch (bit-identical to them).
+  pub fn rh_softmax_kl_step(x: *const f32, c: i32, n: i32, labels: *const i32, weights: *const f32, p: *mut f32,
+                            max_out: *mut f32, idx_out: *mut i32, loss1: *mut f32, loss_sum: *mut f32, dx: *mut f32,
+                            counter: *mut u32, stream: rh_stream_t) -> c_int;
+  // Host generator behind init_params (the reference's random stream lives in crates outside its tree).
+  pub fn rh_rng_fill_uniform(seed: u64, stream_id: u64, host: *mut f32, n: size_t, lo: c_float, hi: c_float) -> c_int;
+  pub fn rh_rng_fill_normal(seed: u64, stream_id: u64, host: *mut f32, n: size_t, mean: c_float, std: c_float) -> c_int;
 
   pub fn rh_sgd_momentum_step(n: i64, w: *mut f32, g: *mut f32, v: *mut f32, l2: c_float, scale: c_float,
                               mu: c_float, apply: c_float, zero_grad: c_int, stream: rh_stream_t) -> c_int;
