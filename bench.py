@@ -16,6 +16,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
 # HBM-side bytes per launch (average over the launches of one step) of the MFMA kernels come from two
@@ -87,7 +88,8 @@ def collect_profile(lib, steps):
         if ms <= 0.0:
             continue
         if mfma:
-            achieved, peak, unit = work / ms / 1e9, PEAK_FP32_MFMA_TFLOPS, "TFLOP/s"
+            achieved, unit = work / ms / 1e9, "TFLOP/s"
+            peak = PEAK_BF16_MFMA_TFLOPS if name.startswith("conv_fwd_bf16") else PEAK_FP32_MFMA_TFLOPS
         else:
             achieved, peak, unit = work / ms / 1e6, PEAK_HBM_GBS, "GB/s"
         out.append({"kernel": name, "bound": "mfma" if mfma else "hbm", "launches_per_step": count / steps,
@@ -153,6 +155,68 @@ def cpu_baseline(net, sample_images):
             "sample": "one fwd+bwd+SGD step of the same operator graph on %d images (%.1f s)" % (sample_images, dt)}
 
 
+def bench_bf16_forward(args, lib, net, cfg, batch, seed):
+    """Forward pass only, inference phase, convolution operands rounded to bf16 (fp32 accumulation): the reduced-
+    precision forward option.  One JSON line of the same shape as the train-step line."""
+    import torch
+    from rembrandt_amd import configs, synth
+    from rembrandt_amd.operator import SequentialOperatorWorker
+    dims, layers, ncat = net
+    worker = SequentialOperatorWorker(cfg, batch, "Forward", shared_seed=(seed, seed + 1), device=0, bf16_forward=True)
+    worker.init_params()
+    worker.load_frames_f32(synth.normal(seed, 100, (batch, dims[2], dims[1], dims[0])))
+    for _ in range(args.warmup):
+        worker.forward(batch, training=False, t=0)
+    worker.sync()
+    kernels = []
+    if not args.no_kernel_events:
+        lib.rh_profile_reset()
+        lib.rh_profile_filter(None)
+        lib.rh_profile_enable(1)
+        n = max(1, min(args.steps, 10))
+        for _ in range(n):
+            worker.forward(batch, training=False, t=0)
+        worker.sync()
+        lib.rh_profile_enable(0)
+        kernels = collect_profile(lib, n)
+        lib.rh_profile_reset()
+    bf = [k for k in kernels if k["kernel"].startswith("conv_fwd_bf16")]
+    dom = bf[0] if bf else None
+    if dom is not None:
+        lib.rh_profile_filter(dom["kernel"].encode())
+        lib.rh_profile_enable(1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        worker.forward(batch, training=False, t=0)
+    worker.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lib.rh_profile_enable(0)
+    if dom is not None:
+        live = [k for k in collect_profile(lib, args.steps) if k["kernel"] == dom["kernel"]]
+        dom = live[0] if live else dom
+    lib.rh_profile_reset()
+    lib.rh_profile_filter(None)
+    print(json.dumps({
+        "metric": "inference images/sec (forward only) %s b%d, bf16 conv operands, fp32 accumulation" % (args.workload, batch),
+        "value": batch * args.steps / dt, "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 operands, f32 accumulate (affine layers f32)", "data": "synthetic",
+        "config": {"workload": "%s-shaped forward pass, inference phase, batch %d, input %dx%dx%d N(0,1), convolutions on "
+                               "bf16-rounded operands" % (args.workload, batch, dims[2], dims[1], dims[0]),
+                   "global_batch": batch, "params": cfg.params_len(),
+                   "gemm_gflop_per_step": configs.train_flops(net, batch, forward_only=True) / 1e9},
+        "roofline": None if dom is None else
+                    {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["achieved"], "peak": PEAK_BF16_MFMA_TFLOPS,
+                     "unit": "TFLOP/s", "frac": dom["achieved"] / PEAK_BF16_MFMA_TFLOPS, "avg_launch_ms": dom["avg_launch_ms"],
+                     "traffic": None},
+        "kernels": kernels,
+        "parity": {"tolerance": TOLERANCE + "; the oracle is evaluated on the bf16-rounded operands (round to nearest even), "
+                                "so only the accumulation order differs"},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -171,6 +235,9 @@ def main():
     ap.add_argument("--host-frames", action="store_true",
                     help="every timed step first copies its batch of u8 frames from the worker's host frame buffer "
                          "(the PCIe-inclusive rate; the default keeps the inputs resident in HBM)")
+    ap.add_argument("--bf16-forward", action="store_true",
+                    help="forward pass only (inference phase) with bf16 convolution operands and fp32 accumulation; "
+                         "reports inference images/sec and the bf16 kernel against the bf16 matrix peak")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="first launch the library's plain copy kernel 4 times over MIB MiB (a known-size "
                          "reference for hardware byte counters collected around this command)")
@@ -193,6 +260,8 @@ def main():
     batch = BATCH[args.workload]
     seed = NUM_CLASSES_SEED + 4
     cfg = configs.build_config(net)
+    if args.bf16_forward:
+        return bench_bf16_forward(args, lib, net, cfg, batch, seed)
     worker = SequentialOperatorWorker(cfg, batch, "Backward", shared_seed=(seed, seed + 1), device=0,
                                       fuse_epilogue=not args.unfused, overlap_backward=not args.no_overlap,
                                       graph_steps=args.graph)

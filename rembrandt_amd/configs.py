@@ -147,28 +147,29 @@ def build_config(net, init_std=0.01, bnorm_mov_avg=("Exponential", 0.1), bnorm_e
     return cfg.softmax_kl_loss(num_categories)
 
 
-def train_flops(net, batch):
+def train_flops(net, batch, forward_only=False):
     """GEMM-equivalent FLOPs of one train step: 2*N*K*C*R*S*P*Q per conv pass (no backward-data
-    for the first layer), 2*B*in*out per affine GEMM."""
+    for the first layer), 2*B*in*out per affine GEMM; of the forward pass alone with forward_only."""
     _, layers, _ = net
     total = 0
     first = True
+    passes = (lambda first: 1) if forward_only else (lambda first: 2 if first else 3)
     for l in layers:
         if l[0] in ("conv2d", "bnorm_conv2d"):
             (w, h, c), k, st, pad, out = l[1], l[2], l[3], l[4], l[5]
             P = max(0, h + 2 * pad - k + st) // st
             Q = max(0, w + 2 * pad - k + st) // st
             f = 2 * batch * out * c * k * k * P * Q
-            total += f * (2 if first else 3)
+            total += f * passes(first)
         elif l[0] == "stack_res_conv2d":
             (w, h, c) = l[1]
-            total += 2 * 3 * (2 * batch * c * c * 9 * w * h)
+            total += 2 * passes(False) * (2 * batch * c * c * 9 * w * h)
         elif l[0] == "proj_stack_res_conv2d":
             (w, h, c), (ow, oh, oc) = l[1], l[2]
-            total += 3 * (2 * batch * ow * oh * oc * (9 * c + 9 * oc + c))
+            total += passes(False) * (2 * batch * ow * oh * oc * (9 * c + 9 * oc + c))
         elif l[0] == "affine":
             f = 2 * batch * l[1] * l[2]
-            total += f * (2 if first else 3)
+            total += f * passes(first)
         else:
             continue
         first = False
