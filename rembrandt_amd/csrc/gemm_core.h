@@ -101,6 +101,58 @@ struct LoadDenseK {
 };
 
 // ------------------------------------------------------------------------------------------
+// The same operand read four k at a time: a lane loads 16 bytes (k = 4q .. 4q+3 of one row) with one
+// buffer_load_dwordx4, a quarter of the load instructions and address additions of LoadDenseK, and writes the four
+// values to four k rows of the same [k][row] slab.  A wave's instruction covers 16 rows of 64 contiguous bytes.
+// Needs ld % 4 == 0 and a 16-byte aligned base (aligned loads) and K % 4 == 0 (a group never straddles the end of
+// its row: it is read whole or not at all).
+// ------------------------------------------------------------------------------------------
+template <int ROWS, int BK, int NT>
+struct LoadDenseK4 {
+  static constexpr int QPR = BK / 4;                      // lanes per row
+  static constexpr int RPI = NT / QPR;                    // rows one instruction of the block covers
+  static constexpr int CNT = (ROWS + RPI - 1) / RPI;
+  static constexpr int LD = ROWS + lds_pad_kfast<BK>();
+  static_assert(BK % 4 == 0 && NT % QPR == 0, "loader shape");
+  typedef DenseParams Params;
+  typedef float4 Reg;
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t rowoff[CNT];
+  int kq, r, K, sbase;
+
+  __device__ __forceinline__ void init(const Params& p, int row0, int tid) {
+    rsrc = make_rsrc(p.ptr, p.bytes);
+    kq = (tid % QPR) * 4;
+    r = tid / QPR;
+    K = p.K;
+    sbase = kq * LD + r;
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      const int slot = r + i * RPI, row = row0 + slot;
+      rowoff[i] = (slot < ROWS && row < p.rows) ? (uint32_t)row * (uint32_t)p.ld : kInvalidOff;
+    }
+  }
+  uint32_t koff;
+  __device__ __forceinline__ void prep(int k0) {
+    const int k = k0 + kq;
+    koff = k < K ? (uint32_t)k : kInvalidOff;
+  }
+  __device__ __forceinline__ float4 load_one(int i) const {
+    const uint32_t e = rowoff[i] + koff;
+    const uint32_t o = e < kInvalidOff ? e : kInvalidOff;
+    return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(o << 2), 0, 0));
+  }
+  __device__ __forceinline__ void store(float* s, const float4 (&v)[CNT]) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      if (ROWS % RPI != 0 && r + i * RPI >= ROWS) continue;   // a thread past the slab's rows (tiles narrower than RPI)
+      float* d = s + sbase + i * RPI;
+      d[0] = v[i].x; d[LD] = v[i].y; d[2 * LD] = v[i].z; d[3 * LD] = v[i].w;
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------------------
 // Dense operand, rows contiguous in memory: element (row, k) at ptr[k*ld + row].
 // Lanes run along rows.
 // ------------------------------------------------------------------------------------------

@@ -6,6 +6,8 @@
 //   engine B operand (row im): opA.  transA == 0: A[im + l*lda] (rows contiguous); else A[l + im*lda].
 // When the result has too few tiles to fill the GPU (batch-sized GEMMs of the affine layers) and
 // scratch is given, the contraction is split across blocks and reduced in a fixed order.
+#include <type_traits>
+
 #include "conv_common.h"
 
 namespace rh {
@@ -43,12 +45,13 @@ static RowSParams rows_params(const DenseParams& d) {
   return r;
 }
 
-template <class T, bool B_TRANS, bool A_TRANS, bool RS>
+// K4: the k-contiguous operands are read 16 bytes at a time (see k4_ok).
+template <class T, bool B_TRANS, bool A_TRANS, bool RS, bool K4>
 static int run_sgemm(const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k, int splits,
                      int* used, hipStream_t stream, const char* tag) {
   // engine A operand = opB: k contiguous unless transB; engine B operand = opA: rows contiguous unless transA
-  typedef LoadDenseK<T::BM, T::BK, T::NT, false> AK;
-  typedef LoadDenseK<T::BN, T::BK, T::NT, false> BK_;
+  typedef typename std::conditional<K4, LoadDenseK4<T::BM, T::BK, T::NT>, LoadDenseK<T::BM, T::BK, T::NT, false>>::type AK;
+  typedef typename std::conditional<K4, LoadDenseK4<T::BN, T::BK, T::NT>, LoadDenseK<T::BN, T::BK, T::NT, false>>::type BK_;
   if constexpr (RS) {
     typedef LoadRowS<T::BM, T::BK, T::NT, true> AR;
     typedef LoadRowS<T::BN, T::BK, T::NT, true> BR;
@@ -74,18 +77,35 @@ static int run_sgemm(const DenseParams& ap, const DenseParams& bp, const EpiPara
   }
 }
 
+// A k-contiguous operand can be read in aligned 16-byte groups that stay inside a row.
+static bool k4_ok(const DenseParams& d, int k) {
+  return k % 4 == 0 && d.ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d.ptr) & 15) == 0;
+}
+
+template <class T, bool B_TRANS, bool A_TRANS, bool RS>
+static int run_sgemm_k4(bool k4, const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k, int splits,
+                        int* used, hipStream_t stream, const char* tag) {
+  if constexpr (B_TRANS && !A_TRANS) {   // no k-contiguous operand
+    return run_sgemm<T, B_TRANS, A_TRANS, RS, false>(ap, bp, ep, k, splits, used, stream, tag);
+  } else {
+    return k4 ? run_sgemm<T, B_TRANS, A_TRANS, RS, true>(ap, bp, ep, k, splits, used, stream, tag)
+              : run_sgemm<T, B_TRANS, A_TRANS, RS, false>(ap, bp, ep, k, splits, used, stream, tag);
+  }
+}
+
 template <bool B_TRANS, bool A_TRANS>
 static int dispatch_tile(int bm, const DenseParams& ap, const DenseParams& bp, const EpiParams& ep, int k,
                          int splits, int* used, hipStream_t stream) {
   const bool rs = k % 16 == 0 && (B_TRANS || !A_TRANS);
+  const bool k4 = (B_TRANS || k4_ok(ap, k)) && (!A_TRANS || k4_ok(bp, k));   // every k-contiguous operand qualifies
   switch (bm) {
     case 128:
-      return rs ? run_sgemm<T128x128, B_TRANS, A_TRANS, true>(ap, bp, ep, k, splits, used, stream, "sgemm_128x128")
-                : run_sgemm<T128x128, B_TRANS, A_TRANS, false>(ap, bp, ep, k, splits, used, stream, "sgemm_128x128");
+      return rs ? run_sgemm_k4<T128x128, B_TRANS, A_TRANS, true>(k4, ap, bp, ep, k, splits, used, stream, "sgemm_128x128")
+                : run_sgemm_k4<T128x128, B_TRANS, A_TRANS, false>(k4, ap, bp, ep, k, splits, used, stream, "sgemm_128x128");
     case 64:
-      return rs ? run_sgemm<T64x256, B_TRANS, A_TRANS, true>(ap, bp, ep, k, splits, used, stream, "sgemm_64x256")
-                : run_sgemm<T64x256, B_TRANS, A_TRANS, false>(ap, bp, ep, k, splits, used, stream, "sgemm_64x256");
-    default:  return run_sgemm<T32x256, B_TRANS, A_TRANS, false>(ap, bp, ep, k, splits, used, stream, "sgemm_32x256");
+      return rs ? run_sgemm_k4<T64x256, B_TRANS, A_TRANS, true>(k4, ap, bp, ep, k, splits, used, stream, "sgemm_64x256")
+                : run_sgemm_k4<T64x256, B_TRANS, A_TRANS, false>(k4, ap, bp, ep, k, splits, used, stream, "sgemm_64x256");
+    default:  return run_sgemm_k4<T32x256, B_TRANS, A_TRANS, false>(k4, ap, bp, ep, k, splits, used, stream, "sgemm_32x256");
   }
 }
 
