@@ -284,6 +284,7 @@ typedef struct rh_sgd_tensor {
   float* v;
   int64_t n;
   float l2;
+  int32_t keep_grad;   /* nonzero: leave g as it is even with zero_grad (the caller overwrites it, beta = 0, next time) */
 } rh_sgd_tensor;
 int rh_sgd_momentum_step_multi(int32_t count, const rh_sgd_tensor* tensors, float scale, float mu, float apply,
                                int zero_grad, rh_stream_t stream);

@@ -27,7 +27,8 @@ class LrnGeom(C.Structure):
 
 
 class SgdTensor(C.Structure):
-    _fields_ = [("W", C.c_void_p), ("g", C.c_void_p), ("v", C.c_void_p), ("n", C.c_int64), ("l2", C.c_float)]
+    _fields_ = [("W", C.c_void_p), ("g", C.c_void_p), ("v", C.c_void_p), ("n", C.c_int64), ("l2", C.c_float),
+                ("keep_grad", C.c_int32)]
 
 
 class PoolGeom(C.Structure):

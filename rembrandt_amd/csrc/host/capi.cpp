@@ -24,9 +24,11 @@ struct StepKey {
   uint32_t step_size_bits, l2_bits, mu_bits;
   bool first_iter;  // the Nesterov un-apply is skipped at iteration 0
   int input_mode;   // which loader filled the input frames: the input operator's forward launches differ
+  std::vector<char> grad_state;  // which operators' gradient buffers stand for zeros: their backward passes overwrite (beta = 0)
   bool operator<(const StepKey& o) const {
-    return std::tie(batch, fused, momentum_kind, step_size_bits, l2_bits, mu_bits, first_iter, input_mode) <
-           std::tie(o.batch, o.fused, o.momentum_kind, o.step_size_bits, o.l2_bits, o.mu_bits, o.first_iter, o.input_mode);
+    return std::tie(batch, fused, momentum_kind, step_size_bits, l2_bits, mu_bits, first_iter, input_mode, grad_state) <
+           std::tie(o.batch, o.fused, o.momentum_kind, o.step_size_bits, o.l2_bits, o.mu_bits, o.first_iter, o.input_mode,
+                    o.grad_state);
   }
 };
 // A schedule whose step size changes every iteration (Inverse) never repeats a key: neither set may grow with it.
@@ -38,10 +40,14 @@ struct rho_worker {
   bool graph_steps = false;
   bool fuse_epilogue = false;                // also: the loss operator's one-launch form inside rho_sgd_train_batch
   int64_t graph_launches = 0;                // steps that ran as a graph launch
-  std::map<StepKey, rh_graph*> step_graphs;  // recorded steps
+  struct RecordedStep {
+    rh_graph* graph;
+    std::vector<char> grad_state_after;      // host-side state the recorded calls left behind (restored after a replay)
+  };
+  std::map<StepKey, RecordedStep> step_graphs;  // recorded steps
   std::set<StepKey> seen_steps;              // combinations that ran once launch by launch
   void drop_graphs() {
-    for (auto& kv : step_graphs) (void)rh_graph_destroy(kv.second);
+    for (auto& kv : step_graphs) (void)rh_graph_destroy(kv.second.graph);
     step_graphs.clear();
     seen_steps.clear();
   }
@@ -562,11 +568,12 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
       const SgdOptConfig& c = s->opt->config();
       const StepKey key = {b, fused != 0 ? 1 : 0, (int)c.momentum.kind, float_bits(c.step_size.at_iter(t)),
                            float_bits(c.l2_reg_coef), float_bits(c.momentum.mu), t == 0,
-                           op->input_operator()->input_mode()};
+                           op->input_operator()->input_mode(), op->grad_state()};
       auto it = w->step_graphs.find(key);
       if (it != w->step_graphs.end()) {
-        w->ctx->launch(it->second);
+        w->ctx->launch(it->second.graph);
         s->opt->set_iter_counter(t + 1);  // what step() does on the host
+        op->set_grad_state(it->second.grad_state_after);
         w->graph_launches += 1;
         done = true;
       } else if (w->seen_steps.count(key) && w->step_graphs.size() < kMaxStepGraphs) {
@@ -581,10 +588,11 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
           w->ctx->abort_capture();
           op->forget_pending();
           s->opt->set_iter_counter(t);
+          op->set_grad_state(key.grad_state);
           throw;
         }
         rh_graph* g = w->ctx->end_capture();
-        w->step_graphs[key] = g;
+        w->step_graphs[key] = {g, op->grad_state()};
         w->ctx->launch(g);  // nothing ran while recording; step() already advanced the iteration counter
         w->graph_launches += 1;
         done = true;

@@ -229,6 +229,23 @@ struct ParamTensors {
   size_t wlen = 0, blen = 0;
   size_t wrows = 0, wcols = 0;  // bound of the weights as the reference's Array2d: (in or R*S*C, out), first index fastest
   Ctx ctx;
+  // The fused SGD step would write 4 bytes of zero per parameter into the gradient, and the next backward pass would
+  // read them back to add to (beta = 1).  Instead the step leaves the gradient buffers as they are and marks them
+  // stale: they stand for zeros.  The next backward pass then overwrites (beta = 0); anything else that looks at the
+  // gradients first makes the zeros real (touch_grads).
+  bool grads_stale = false;
+  void touch_grads() {
+    if (!grads_stale) return;
+    grads_stale = false;
+    unwrap(rh_memset_f32(grad_weights->as_mut_ptr(), 0.0f, wlen, s()), "set_constant");
+    unwrap(rh_memset_f32(grad_bias->as_mut_ptr(), 0.0f, blen, s()), "set_constant");
+  }
+  // beta of the gradient accumulation of one backward pass (weights and bias alike); the buffers are real afterwards
+  float take_backward_beta() {
+    const float b = grads_stale ? 0.0f : 1.0f;
+    grads_stale = false;
+    return b;
+  }
 
   void alloc(size_t wl, size_t bl, bool backward, Ctx c) {
     wlen = wl; blen = bl; ctx = c;
@@ -251,6 +268,7 @@ struct ParamTensors {
   void regularize(Regularization reg) {
     RB_ASSERT(has_backward());
     RB_ASSERT(reg.l2_reg_coef >= 0.0f);
+    touch_grads();
     if (reg.l2_reg_coef > 0.0f) {
       unwrap(rh_saxpy((int64_t)wlen, reg.l2_reg_coef, weights->as_ptr(), grad_weights->as_mut_ptr(), s()), "matrix_sum");
       unwrap(rh_saxpy((int64_t)blen, reg.l2_reg_coef, bias->as_ptr(), grad_bias->as_mut_ptr(), s()), "row_vector_sum");
@@ -259,6 +277,7 @@ struct ParamTensors {
   // v = momentum*v; v += scale*g (src/operator/mod.rs:1195-1207)
   void accumulate_grads(float scale, float momentum) {
     RB_ASSERT(has_backward());
+    touch_grads();
     unwrap(rh_sscal((int64_t)wlen, momentum, acc_grad_weights->as_mut_ptr(), s()), "matrix_scale");
     unwrap(rh_sscal((int64_t)blen, momentum, acc_grad_bias->as_mut_ptr(), s()), "row_vector_scale");
     unwrap(rh_saxpy((int64_t)wlen, scale, grad_weights->as_ptr(), acc_grad_weights->as_mut_ptr(), s()), "matrix_sum");
@@ -273,6 +292,7 @@ struct ParamTensors {
   // W += grad_scale*g + update_scale*v (src/operator/mod.rs:1220-1236)
   void update_params2(float grad_scale, float update_scale) {
     RB_ASSERT(has_backward());
+    touch_grads();
     if (grad_scale != 0.0f) {
       unwrap(rh_saxpy((int64_t)wlen, grad_scale, grad_weights->as_ptr(), weights->as_mut_ptr(), s()), "matrix_sum");
       unwrap(rh_saxpy((int64_t)blen, grad_scale, grad_bias->as_ptr(), bias->as_mut_ptr(), s()), "row_vector_sum");
@@ -295,6 +315,7 @@ struct ParamTensors {
   // g *= 0 (src/operator/mod.rs:1355-1363)
   void reset() {
     if (!has_backward()) return;
+    if (grads_stale) return;   // they already stand for zeros
     unwrap(rh_sscal((int64_t)wlen, 0.0f, grad_weights->as_mut_ptr(), s()), "matrix_scale");
     unwrap(rh_sscal((int64_t)blen, 0.0f, grad_bias->as_mut_ptr(), s()), "row_vector_scale");
   }
@@ -302,6 +323,7 @@ struct ParamTensors {
   void descend(float scale, float l2, bool fused) {
     RB_ASSERT(has_backward());
     RB_ASSERT(l2 >= 0.0f);
+    touch_grads();
     if (fused) {
       unwrap(rh_descend((int64_t)wlen, weights->as_mut_ptr(), grad_weights->as_mut_ptr(), scale, l2, s()), "rh_descend");
       unwrap(rh_descend((int64_t)blen, bias->as_mut_ptr(), grad_bias->as_mut_ptr(), scale, l2, s()), "rh_descend");
@@ -317,6 +339,7 @@ struct ParamTensors {
   // g *= scale (src/layer_new.rs:589-594, 1126-1131)
   void reset_gradients(float scale) {
     RB_ASSERT(has_backward());
+    touch_grads();
     unwrap(rh_sscal((int64_t)wlen, scale, grad_weights->as_mut_ptr(), s()), "matrix_scale");
     unwrap(rh_sscal((int64_t)blen, scale, grad_bias->as_mut_ptr(), s()), "row_vector_scale");
   }
@@ -328,10 +351,13 @@ struct ParamTensors {
     unwrap(rh_sgd_momentum_step((int64_t)blen, bias->as_mut_ptr(), grad_bias->as_mut_ptr(),
                                 acc_grad_bias->as_mut_ptr(), l2, scale, momentum, apply, 1, st), "rh_sgd_momentum_step");
   }
+  // Rows of one multi-tensor step: the gradients are read, not zeroed, and stand for zeros from then on.
   void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) {
     RB_ASSERT(has_backward());
-    out.push_back({weights->as_mut_ptr(), grad_weights->as_mut_ptr(), acc_grad_weights->as_mut_ptr(), (int64_t)wlen, l2});
-    out.push_back({bias->as_mut_ptr(), grad_bias->as_mut_ptr(), acc_grad_bias->as_mut_ptr(), (int64_t)blen, l2});
+    touch_grads();   // (a step without a backward pass since the last one: the update must see zeros)
+    out.push_back({weights->as_mut_ptr(), grad_weights->as_mut_ptr(), acc_grad_weights->as_mut_ptr(), (int64_t)wlen, l2, 1});
+    out.push_back({bias->as_mut_ptr(), grad_bias->as_mut_ptr(), acc_grad_bias->as_mut_ptr(), (int64_t)blen, l2, 1});
+    grads_stale = true;
   }
   // Host-side sampling in memory order, then a blocking H2D copy (src/operator/mod.rs:964-1006, 1554-1592).
   void init(const ParamsInit& init, const uint64_t seed[2], size_t fan_in, size_t fan_out, bool xavier_ok, const char* who) {
@@ -392,6 +418,7 @@ struct ParamTensors {
   }
   bool buffer(int which, float** ptr, size_t* len) {
     DeviceBuffer<float>* b = nullptr;
+    if ((which == 4 || which == 5) && has_backward()) touch_grads();
     switch (which) {
       case 2: b = weights.get(); break;
       case 3: b = bias.get(); break;
@@ -703,11 +730,12 @@ class AffineOperator : public Operator {
       wg = workspace_aux_ ? workspace_aux_->as_mut_ptr() : nullptr;
       wg_len = workspace_aux_ ? workspace_aux_->len() : 0;
     }
+    const float beta = params_.take_backward_beta();   // 1: accumulate (the reference's call); 0: the buffers stand for zeros
     // grad_weights(in, out) += in_act(in, B) * out_delta(out, B)^T
-    unwrap(rh_sgemm(0, 1, i, o, b, 1.0f, in_act_->as_ptr(), i, out_delta_->as_ptr(), o, 1.0f,
+    unwrap(rh_sgemm(0, 1, i, o, b, 1.0f, in_act_->as_ptr(), i, out_delta_->as_ptr(), o, beta,
                     params_.grad_weights->as_mut_ptr(), i, wg, wg_len, 0, sg), "matrix_prod");
     // grad_bias(1, out) += 1(1, B) * out_delta^T: the column sums of out_delta, without the ones vector
-    unwrap(rh_conv2d_bwd_bias(b, o, 1, 1.0f, out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), sg), "matrix_prod");
+    unwrap(rh_conv2d_bwd_bias(b, o, 1, 1.0f, out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), sg), "matrix_prod");
     if (in_delta_) {
       // in_delta(in, B) = weights(in, out) * out_delta(out, B)
       unwrap(rh_sgemm(0, 0, i, b, o, 1.0f, params_.weights->as_ptr(), i, out_delta_->as_ptr(), o, 0.0f,
@@ -733,6 +761,8 @@ class AffineOperator : public Operator {
     params_.fused_sgd_step(l2, scale, mu, apply, overlap_on_ ? context_->aux_stream() : nullptr);
   }
   void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) override { params_.sgd_tensors(l2, out); }
+  bool grads_stale() const override { return params_.grads_stale; }
+  void set_grads_stale(bool stale) override { params_.grads_stale = stale && params_.has_backward(); }
   bool updates_on_second_stream() const override { return overlap_on_; }
   void set_overlap_backward(bool on) override { overlap_on_ = on && overlap_built_; }
   bool buffer(int which, float** ptr, size_t* len) override {
@@ -834,10 +864,11 @@ class Conv2dOperator : public Operator {
       w_bias = workspace_aux_.get();
       if (in_delta_) { s_filter = s_bias; w_filter = w_bias; }
     }
-    unwrap(rh_conv2d_bwd_filter(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), 1.0f, params_.grad_weights->as_mut_ptr(),
+    const float beta = params_.take_backward_beta();   // 1: accumulate (the reference's call); 0: the buffers stand for zeros
+    unwrap(rh_conv2d_bwd_filter(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta, params_.grad_weights->as_mut_ptr(),
                                 w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter");
     unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), scale,
-                                 out_delta_->as_ptr(), 1.0f, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
+                                 out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
                                  w_bias->len(), s_bias), "conv2d backward bias");
     if (in_delta_) {
       unwrap(rh_conv2d_bwd_data(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
@@ -863,6 +894,8 @@ class Conv2dOperator : public Operator {
     params_.fused_sgd_step(l2, scale, mu, apply, updates_on_second_stream() ? context_->aux_stream() : nullptr);
   }
   void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) override { params_.sgd_tensors(l2, out); }
+  bool grads_stale() const override { return params_.grads_stale; }
+  void set_grads_stale(bool stale) override { params_.grads_stale = stale && params_.has_backward(); }
   bool updates_on_second_stream() const override { return workspace_aux_ && overlap_on_ && in_delta_; }
   bool buffer(int which, float** ptr, size_t* len) override {
     if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
@@ -1884,6 +1917,15 @@ void SequentialOperatorWorker::set_overlap_backward(bool on) {
   settle();
   context_->join();
   for (auto& op : hidden_ops_) op->set_overlap_backward(on);
+}
+std::vector<char> SequentialOperatorWorker::grad_state() const {
+  std::vector<char> state(hidden_ops_.size());
+  for (size_t i = 0; i < hidden_ops_.size(); ++i) state[i] = hidden_ops_[i]->grads_stale() ? 1 : 0;
+  return state;
+}
+void SequentialOperatorWorker::set_grad_state(const std::vector<char>& state) {
+  RB_ASSERT(state.size() == hidden_ops_.size());
+  for (size_t i = 0; i < hidden_ops_.size(); ++i) hidden_ops_[i]->set_grads_stale(state[i] != 0);
 }
 void SequentialOperatorWorker::fused_sgd_step(float l2, float scale, float mu, float apply) {
   settle();

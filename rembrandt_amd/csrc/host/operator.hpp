@@ -314,6 +314,13 @@ class Operator {
   // The {W, g, v} blocks that fused_sgd_step(l2, ...) would update, each with the l2 factor that applies to it, so that
   // a chain of operators can take the step in one launch per stream (rh_sgd_momentum_step_multi).
   virtual void sgd_tensors(float /*l2*/, std::vector<rh_sgd_tensor>& /*out*/) {}
+  // True while the operator's gradient buffers stand for zeros without holding them (after a multi-tensor step that
+  // did not zero them): its next backward pass overwrites instead of accumulating.  Part of what decides which
+  // launches a step makes, hence of the key a recorded step is filed under.
+  virtual bool grads_stale() const { return false; }
+  // A recorded step was replayed: the host did not run the calls that flip this state, so it is set to what the
+  // recording left behind.
+  virtual void set_grads_stale(bool /*stale*/) {}
   // A consumer that can apply this operator's activation backward mask itself (max-pool backward folds the ReLU
   // mask) asks for it at construction; an operator that agrees skips its own mask pass in backward().  The
   // out_delta buffer holds the same values after the chain's backward either way.
@@ -455,6 +462,9 @@ class SequentialOperatorWorker : public Operator {
   void fused_sgd_step(float l2, float scale, float momentum, float apply) override;
   void set_overlap_backward(bool on) override;
   bool graph_safe(OpPhase phase) const override;
+  // Operator::grads_stale of every hidden operator, and the way back.
+  std::vector<char> grad_state() const;
+  void set_grad_state(const std::vector<char>& state);
   // Joins the second stream if parameter updates are still in flight on it (called by every method but forward,
   // which joins lazily in front of the first operator concerned).
   void settle();

@@ -55,6 +55,7 @@ struct SgdSegs {
   float l2[kSgdSegs];
   int first[kSgdSegs + 1];
   int count;
+  unsigned long long keep;   // bit s: segment s keeps its gradient
 };
 
 __global__ __launch_bounds__(256) void sgd_momentum_multi_kernel(SgdSegs segs, float scale, float mu, float apply,
@@ -70,6 +71,7 @@ __global__ __launch_bounds__(256) void sgd_momentum_multi_kernel(SgdSegs segs, f
   float* __restrict__ V = segs.V[lo];
   const long long n = segs.n[lo];
   const float l2 = segs.l2[lo];
+  const bool keep = (segs.keep >> lo) & 1ull;   // this tensor's gradient is neither zeroed nor written back
   const bool use_l2 = l2 > 0.0f, zg = zero_grad != 0;
   const long long base = (long long)(b - segs.first[lo]) * 1024;
   const bool vec = ((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(G) | reinterpret_cast<uintptr_t>(V)) & 15) == 0;
@@ -81,11 +83,15 @@ __global__ __launch_bounds__(256) void sgd_momentum_multi_kernel(SgdSegs segs, f
     sgd_one(w.z, g.z, v.z, l2, scale, mu, apply, use_l2, zg);
     sgd_one(w.w, g.w, v.w, l2, scale, mu, apply, use_l2, zg);
     *reinterpret_cast<float4*>(W + i) = w;
-    *reinterpret_cast<float4*>(G + i) = g;
+    if (!keep) *reinterpret_cast<float4*>(G + i) = g;
     *reinterpret_cast<float4*>(V + i) = v;
   } else {
     for (int j = 0; j < 4; ++j)
-      if (i + j < n) sgd_one(W[i + j], G[i + j], V[i + j], l2, scale, mu, apply, use_l2, zg);
+      if (i + j < n) {
+        float g = G[i + j];
+        sgd_one(W[i + j], g, V[i + j], l2, scale, mu, apply, use_l2, zg);
+        if (!keep) G[i + j] = g;
+      }
   }
 }
 
@@ -124,7 +130,7 @@ extern "C" int rh_sgd_momentum_step_multi(int32_t count, const rh_sgd_tensor* te
     const rh_sgd_tensor& t = tensors[i];
     if (t.n < 0 || (t.n > 0 && (!t.W || !t.g || !t.v)) || !(t.l2 >= 0.0f)) return RH_E_INVALID;
     if (t.n > (int64_t)1023 * (int64_t)0x7fffffff / 2) return RH_E_LIMIT;
-    bytes += 24.0 * (double)t.n;
+    bytes += (t.keep_grad ? 20.0 : 24.0) * (double)t.n;
   }
   if (bytes == 0.0) return 0;
   ProfScope prof("sgd_fused", bytes, to_stream(stream));
@@ -132,6 +138,7 @@ extern "C" int rh_sgd_momentum_step_multi(int32_t count, const rh_sgd_tensor* te
   while (i < count) {
     SgdSegs segs;
     segs.count = 0;
+    segs.keep = 0;
     long long blocks = 0;
     for (; i < count && segs.count < kSgdSegs; ++i) {
       const rh_sgd_tensor& t = tensors[i];
@@ -140,6 +147,7 @@ extern "C" int rh_sgd_momentum_step_multi(int32_t count, const rh_sgd_tensor* te
       if (blocks + nb > 0x7fffffffll) break;       // the rest goes to another launch
       const int s = segs.count++;
       segs.W[s] = t.W; segs.G[s] = t.g; segs.V[s] = t.v; segs.n[s] = t.n; segs.l2[s] = t.l2;
+      if (t.keep_grad) segs.keep |= 1ull << s;
       segs.first[s] = (int)blocks;
       blocks += nb;
     }

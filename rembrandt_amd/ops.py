@@ -245,11 +245,12 @@ def sgd_momentum_step(W, g, v, l2, scale, mu, apply, zero_grad=True):
                                      _stream()), "rh_sgd_momentum_step")
 
 
-def sgd_momentum_step_multi(tensors, scale, mu, apply, zero_grad=True):
-    """tensors: sequence of (W, g, v, l2) device tensors; one launch for all of them."""
+def sgd_momentum_step_multi(tensors, scale, mu, apply, zero_grad=True, keep_grad=()):
+    """tensors: sequence of (W, g, v, l2) device tensors; one launch for all of them.  keep_grad: indices of the
+    tensors whose gradient the step must leave as it is."""
     arr = (_lib.SgdTensor * len(tensors))()
     for i, (W, g, v, l2) in enumerate(tensors):
-        arr[i] = _lib.SgdTensor(W.data_ptr(), g.data_ptr(), v.data_ptr(), W.numel(), l2)
+        arr[i] = _lib.SgdTensor(W.data_ptr(), g.data_ptr(), v.data_ptr(), W.numel(), l2, 1 if i in keep_grad else 0)
     check(lib().rh_sgd_momentum_step_multi(len(tensors), arr, scale, mu, apply, int(zero_grad), _stream()),
           "rh_sgd_momentum_step_multi")
 

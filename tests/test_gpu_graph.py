@@ -296,7 +296,9 @@ def test_momentum_flavours(dev, flavour):
 
 
 def test_gradient_accumulation_over_microbatches(dev):
-    """batch_size = minibatch_size / 4: four forward/backward passes accumulate (beta = 1) before one update."""
+    """batch_size = minibatch_size / 4: four forward/backward passes accumulate (beta = 1) before one update.  Two
+    minibatches: at the start of the second the fused step has left the gradient buffers standing for zeros, so its
+    first backward pass overwrites and the other three accumulate."""
     net = ((10, 10, 3), *configs._chain((10, 10, 3), [("conv", 3, 1, 1, 8, "Rect"), ("pool", 3, 2, 0, "Average"),
                                                          ("fc", 7, "Identity")]))
     batch, minibatch = 4, 16
@@ -304,26 +306,72 @@ def test_gradient_accumulation_over_microbatches(dev):
     sgd, rsgd = SgdOpt(minibatch, 0.1, ("Update", 0.5), 0.0), OG.SgdOpt(0.1, ("Update", 0.5), 0.0)
     sgd.begin(w)
     rsgd.begin(ref)
-    for micro in range(4):
-        x = synth.normal(99, 10 + micro, (batch, 3, 10, 10))
-        labels = synth.integers(99, 20 + micro, (batch,), 7)
-        w.load_frames_f32(x)
-        w.stage_batch(labels, 1.0 / minibatch)
-        ref.stage_batch(labels, 1.0 / minibatch)
-        w.forward(batch)
-        ref.forward(x)
-        w.backward(batch)
-        ref.backward()
-    for i, op in enumerate(ref.hidden):
-        if op.p is not None:
-            assert_close(w.read(i, "grad_weights"), op.p.grad_weights.ravel(), "accumulated grad_weights[%d]" % i)
-            assert_close(w.read(i, "grad_bias"), op.p.grad_bias.ravel(), "accumulated grad_bias[%d]" % i)
-    sgd.step(w, fused=True)
-    rsgd.step(ref)
-    for i, op in enumerate(ref.hidden):
-        if op.p is not None:
-            assert_close(w.read(i, "weights"), op.p.weights.ravel(), "weights[%d]" % i)
+    for mini in range(2):
+        for micro in range(4):
+            x = synth.normal(99, 10 + micro + 100 * mini, (batch, 3, 10, 10))
+            labels = synth.integers(99, 20 + micro + 100 * mini, (batch,), 7)
+            w.load_frames_f32(x)
+            w.stage_batch(labels, 1.0 / minibatch)
+            ref.stage_batch(labels, 1.0 / minibatch)
+            w.forward(batch)
+            ref.forward(x)
+            w.backward(batch)
+            ref.backward()
+        for i, op in enumerate(ref.hidden):
+            if op.p is not None:
+                assert_close(w.read(i, "grad_weights"), op.p.grad_weights.ravel(), "accumulated grad_weights[%d]" % i)
+                assert_close(w.read(i, "grad_bias"), op.p.grad_bias.ravel(), "accumulated grad_bias[%d]" % i)
+        sgd.step(w, fused=True)
+        rsgd.step(ref)
+        for i, op in enumerate(ref.hidden):
+            if op.p is not None:
+                assert_close(w.read(i, "weights"), op.p.weights.ravel(), "weights[%d] after minibatch %d" % (i, mini))
     w.close()
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_gradients_standing_for_zeros(dev, overlap):
+    """After a fused step the gradient buffers are not zeroed but stand for zeros until the next backward pass
+    overwrites them.  Reading them makes the zeros real; a worker whose gradients are read after every step (its
+    backward passes then accumulate onto real zeros) must stay bit-identical to one that is left alone, also through
+    two steps in a row without a backward pass in between and a step of the unfused sequence."""
+    net = configs.lenet()
+    dims, layers, ncat = net
+    batch = 8
+    ws = []
+    for _ in range(2):
+        w = SequentialOperatorWorker(configs.build_config(net), batch, "Backward", shared_seed=(5, 6), overlap_backward=overlap)
+        w.init_params()
+        ws.append(w)
+    sgds = [SgdOpt(batch, 0.05, ("Update", 0.9), 1e-3) for _ in ws]
+    for sgd, w in zip(sgds, ws):
+        sgd.begin(w)
+    param_layers = [i for i, l in enumerate(layers) if l[0] in ("conv2d", "affine")]
+    for step in range(5):
+        x = synth.normal(5, 10 + step, (batch, dims[2], dims[1], dims[0]))
+        labels = synth.integers(5, 50 + step, (batch,), ncat)
+        losses = []
+        for k, (sgd, w) in enumerate(zip(sgds, ws)):
+            w.load_frames_f32(x)
+            w.stage_batch(labels, 1.0 / batch)
+            if step == 3:                       # the reference's own call sequence on both
+                w.forward(batch, training=True, t=sgd.iter_counter())
+                w.backward(batch)
+                sgd.step(w, fused=False)
+                losses.append(w.store_loss(batch))
+            else:
+                losses.append(sgd.train_batch(w, batch, fused=True)[0])
+            if step == 1:
+                sgd.step(w, fused=True)         # a second step on gradients that stand for zeros (momentum only)
+            if k == 1:
+                for i in param_layers:
+                    assert not w.read(i, "grad_weights").any() and not w.read(i, "grad_bias").any(), "gradients after a step"
+        assert losses[0] == losses[1], "step %d" % step
+        for i in param_layers:
+            for name in ("weights", "bias", "acc_grad_weights", "acc_grad_bias"):
+                assert np.array_equal(ws[0].read(i, name), ws[1].read(i, name)), (step, i, name)
+    for w in ws:
+        w.close()
 
 
 def test_u8_frames_and_save_restore(dev):

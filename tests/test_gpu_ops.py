@@ -397,6 +397,21 @@ def test_sgd_multi_tensor_step(dev):
                 assert_close(N(vm), vh, "multi sgd v[%d]" % k, atol=1e-7)
                 assert_close(N(gm), gh, "multi sgd g[%d]" % k, atol=1e-7)
     assert _lib.lib().rh_sgd_momentum_step_multi(1, None, 1.0, 0.9, 1.0, 1, None) == _lib.RH_E_INVALID
+    # keep_grad: those tensors' gradients are read for the update and left untouched (not zeroed, not regularised in
+    # place); W and v as in the plain step, the other tensors as without the flag
+    lens = (5, 4099, 1 << 16)
+    host = [(synth.normal(19, 3 * k + 1, (n,)), synth.normal(19, 3 * k + 2, (n,)), synth.normal(19, 3 * k + 3, (n,))) for k, n in enumerate(lens)]
+    for zg in (True, False):
+        a = [tuple(T(x, dev) for x in h) + (0.01,) for h in host]
+        b = [tuple(T(x, dev) for x in h) + (0.01,) for h in host]
+        ops.sgd_momentum_step_multi(a, -0.01, 0.9, 1.0, zg, keep_grad=(0, 2))
+        ops.sgd_momentum_step_multi(b, -0.01, 0.9, 1.0, zg)
+        for k in range(3):
+            assert torch.equal(a[k][0], b[k][0]) and torch.equal(a[k][2], b[k][2]), "keep_grad changed W or v of block %d" % k
+            if k in (0, 2):
+                assert np.array_equal(N(a[k][1]), host[k][1]), "a kept gradient was written"
+            else:
+                assert torch.equal(a[k][1], b[k][1])
     torch.cuda.synchronize()
 
 
