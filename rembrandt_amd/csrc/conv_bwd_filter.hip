@@ -322,7 +322,8 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_vec_kernel(const float* __re
     const int pix = pix0 + 4 * pq;
     const int hp = pix / Wp, wp = pix - hp * Wp;
     const int h = hp - halo, w = wp - halo;
-    const bool whole = pix + 3 < HpWp && (unsigned)h < (unsigned)H && w >= 0 && w + 3 < W;
+    // (without a halo the plane is one contiguous run: four pixels may cross a row end)
+    const bool whole = pix + 3 < HpWp && (halo == 0 || ((unsigned)h < (unsigned)H && w >= 0 && w + 3 < W));
     int off[4];  // element offsets within a plane, -1 = zero
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -402,6 +403,40 @@ __global__ void split_reduce_rsc_kernel(const float* __restrict__ part, int spli
     float val = alpha * acc;
     if (beta != 0.0f) val += beta * *dst;
     *dst = val;
+  }
+}
+
+// The same for C % 4 == 0: a thread takes four consecutive channels of one (ko, r, s), read as 16-byte groups from
+// every slab (4-byte reads top out well below what 16-byte reads reach); sums in the order of sum_splits.
+__global__ __launch_bounds__(256) void split_reduce_rsc_vec_kernel(const float4* __restrict__ part, int splits, long long stride4,
+                                                                   float* __restrict__ dw, int K, int C, int R, int S,
+                                                                   float alpha, float beta) {
+  const int CRS4 = (C * R * S) >> 2;
+  const unsigned total4 = (unsigned)K * (unsigned)CRS4;
+  const unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total4) return;
+  const float4 z = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  float4 a0 = z, a1 = z, a2 = z, a3 = z;
+  auto add = [](float4& a, const float4 v) { a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w; };
+  const float4* p = part + idx;
+  int sp = 0;
+  for (; sp + 3 < splits; sp += 4) {
+    add(a0, p[(long long)sp * stride4]);
+    add(a1, p[(long long)(sp + 1) * stride4]);
+    add(a2, p[(long long)(sp + 2) * stride4]);
+    add(a3, p[(long long)(sp + 3) * stride4]);
+  }
+  for (; sp < splits; ++sp) add(a0, p[(long long)sp * stride4]);
+  const float v[4] = {(a0.x + a1.x) + (a2.x + a3.x), (a0.y + a1.y) + (a2.y + a3.y), (a0.z + a1.z) + (a2.z + a3.z),
+                      (a0.w + a1.w) + (a2.w + a3.w)};
+  const int ko = (int)(idx / (unsigned)CRS4), j = 4 * (int)(idx - (unsigned)ko * (unsigned)CRS4);
+  const int r = j / (S * C), rem = j - r * (S * C), s2 = rem / C, c = rem - s2 * C;
+  float* dst = dw + (((size_t)ko * C + c) * R + r) * S + s2;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float val = alpha * v[e];
+    if (beta != 0.0f) val += beta * dst[(size_t)e * R * S];
+    dst[(size_t)e * R * S] = val;
   }
 }
 
@@ -671,8 +706,13 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
     if (e) return e;
     const long long total = (long long)d.K * CRSs;
     ProfScope prof("split_reduce", 4.0 * (double)total * (used + 1), stream);
-    hipLaunchKernelGGL(split_reduce_rsc_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, parts, used,
-                       (long long)d.K * CRSs, dw, d.K, d.C, d.R, d.S, alpha, beta);
+    if (d.C % 4 == 0 && (reinterpret_cast<uintptr_t>(parts) & 15) == 0)
+      hipLaunchKernelGGL(split_reduce_rsc_vec_kernel, dim3(stream_grid((size_t)total / 4, 256)), dim3(256), 0, stream,
+                         reinterpret_cast<const float4*>(parts), used, (long long)d.K * CRSs / 4, dw, d.K, d.C, d.R, d.S, alpha,
+                         beta);
+    else
+      hipLaunchKernelGGL(split_reduce_rsc_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, parts, used,
+                         (long long)d.K * CRSs, dw, d.K, d.C, d.R, d.S, alpha, beta);
     return launch_status();
   }
 
