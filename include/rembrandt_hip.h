@@ -143,6 +143,12 @@ int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x, const floa
 int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const float* x, const float* dy,
                          float beta, float* dw, void* ws, size_t ws_bytes, int flags,
                          rh_stream_t stream);
+/* rh_conv2d_bwd_filter followed by rh_conv2d_bwd_bias (mod.rs:1765-1781) with the same alpha and beta, as one call:
+ * db = alpha * sum_{n,p,q} dy + beta * db as well.  Where the filter gradient makes a pass of its own over dy (the
+ * channel-last copy of the large layers) that pass also leaves the plane sums, so dy is not read a second time.
+ * Scratch as for rh_conv2d_bwd_filter (rh_conv2d_workspace_bytes covers both). */
+int rh_conv2d_bwd_filter_bias(const rh_conv_geom* g, float alpha, const float* x, const float* dy, float beta,
+                              float* dw, float* db, void* ws, size_t ws_bytes, int flags, rh_stream_t stream);
 /* db[k] = alpha * sum_{n,p,q} dy[n,k,p,q] + beta * db[k];  plane = P*Q. */
 int rh_conv2d_bwd_bias(int32_t N, int32_t K, int32_t plane, float alpha, const float* dy,
                        float beta, float* db, rh_stream_t stream);

@@ -91,6 +91,7 @@ PROTOTYPES = {
     "rh_bnorm_workspace_bytes_upto": (_sz, [_int, _int, _int]),
     "rh_conv2d_fwd": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _vp, _sz, _int, _vp]),
     "rh_conv2d_bwd_filter": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _sz, _int, _vp]),
+    "rh_conv2d_bwd_filter_bias": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _vp, _sz, _int, _vp]),
     "rh_conv2d_bwd_bias": (_int, [_i32, _i32, _i32, _f, _vp, _f, _vp, _vp]),
     "rh_conv2d_bwd_bias_workspace_bytes": (_sz, [_i32, _i32, _i32]),
     "rh_conv2d_bwd_bias_ws": (_int, [_i32, _i32, _i32, _f, _vp, _f, _vp, _vp, _sz, _vp]),

@@ -310,13 +310,21 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const float* __restri
 // one source row, which need not be 16-byte aligned; element by element across row ends and the halo) and writes four
 // consecutive channels of one pixel.  LDS tile [pixel][channel], the 16-byte channel groups of a row permuted by the
 // pixel's quad index so that the scattered writes of a wave spread over the banks.
+// BIAS: the pass over dy that backward-filter makes anyway also yields the bias gradient's first stage.  A block then
+// walks all 64-pixel pieces of its (image, 64 channels) itself (grid x = 1), each thread adding its sixteen pixels of
+// one channel piece after piece, and leaves bias_part[n][c] = sum over the plane of src[n][c][.]; the sums over n are
+// bwd_bias_rows_kernel's.  Fixed order: the same call gives the same bits.
 typedef float float4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
+template <bool BIAS>
 __global__ __launch_bounds__(256) void nchw_to_nhwc_vec_kernel(const float* __restrict__ src, float* __restrict__ dst,
-                                                               int C, int H, int W, int Hp, int Wp, int halo) {
+                                                               int C, int H, int W, int Hp, int Wp, int halo,
+                                                               float* __restrict__ bias_part) {
   __shared__ __attribute__((aligned(16))) float tile[64 * 64];
-  const int pix0 = blockIdx.x * 64, c0 = blockIdx.y * 64, n = blockIdx.z;
+  const int c0 = blockIdx.y * 64, n = blockIdx.z;
   const int HpWp = Hp * Wp;
+  float bsum = 0.0f;
+  for (int pix0 = blockIdx.x * 64; pix0 < HpWp; pix0 += gridDim.x * 64) {
   {
     const int pq = threadIdx.x & 15, cl0 = threadIdx.x >> 4;
     const int pix = pix0 + 4 * pq;
@@ -360,14 +368,41 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_vec_kernel(const float* __re
       *reinterpret_cast<float4*>(dst + ((size_t)n * HpWp + pix) * C + c) = q;
     }
   }
+  if (BIAS) {
+    // channel cl of pixels 16 q .. 16 q + 15 of this piece (pixels past the plane and channels past C were staged as 0)
+    const int cl = threadIdx.x & 63, q = threadIdx.x >> 6;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int pl = 16 * q + e;
+      bsum += tile[pl * 64 + 4 * ((cl >> 2) ^ ((pl >> 2) & 15)) + (cl & 3)];
+    }
+  }
+  __syncthreads();   // the next piece overwrites the tile
+  }
+  if (BIAS) {
+    const int cl = threadIdx.x & 63, q = threadIdx.x >> 6;
+    tile[q * 64 + cl] = bsum;
+    __syncthreads();
+    if (q == 0 && c0 + cl < C)
+      bias_part[(size_t)n * C + c0 + cl] = (tile[cl] + tile[64 + cl]) + (tile[128 + cl] + tile[192 + cl]);
+  }
 }
 
+// The 16-byte form can carry the per-image plane sums along (bias_part, N x C floats; no halo).
+static bool nhwc_vec_ok(int C, const float* dst) { return C % 4 == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0; }
+
 static void launch_nchw_to_nhwc(const float* src, float* dst, int N, int C, int H, int W, int Hp, int Wp, int halo,
-                                hipStream_t stream) {
+                                hipStream_t stream, float* bias_part = nullptr) {
   ProfScope prof("nchw_to_nhwc", 4.0 * ((double)N * C * H * W + (double)N * C * Hp * Wp), stream);
-  if (C % 4 == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+  if (nhwc_vec_ok(C, dst)) {
+    if (bias_part) {
+      dim3 grid(1, (unsigned)cdiv(C, 64), (unsigned)N);
+      hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<true>, grid, dim3(256), 0, stream, src, dst, C, H, W, Hp, Wp, halo, bias_part);
+      return;
+    }
     dim3 grid((unsigned)cdiv(Hp * Wp, 64), (unsigned)cdiv(C, 64), (unsigned)N);
-    hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel, grid, dim3(256), 0, stream, src, dst, C, H, W, Hp, Wp, halo);
+    hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<false>, grid, dim3(256), 0, stream, src, dst, C, H, W, Hp, Wp, halo,
+                       (float*)nullptr);
     return;
   }
   dim3 grid((unsigned)cdiv(Hp * Wp, 32), (unsigned)cdiv(C, 32), (unsigned)N);
@@ -587,17 +622,21 @@ __global__ __launch_bounds__(256) void bwd_bias_rows_kernel(const float* __restr
                                                             float beta, float* __restrict__ db) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int k = blockIdx.x * 64 + lane;
-  float a0 = 0.0f, a1 = 0.0f;
+  // eight independent partial sums per thread (rows wave, wave + 4, ... in turn): the loop is a chain of memory round
+  // trips, so its length is what the kernel takes
+  float a[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
   if (k < K) {
     int n = wave;
-    for (; n + 4 < N; n += 8) {
-      a0 += dy[(size_t)n * K + k];
-      a1 += dy[(size_t)(n + 4) * K + k];
+    for (; n + 28 < N; n += 32) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a[j] += dy[(size_t)(n + 4 * j) * K + k];
     }
-    for (; n < N; n += 4) a0 += dy[(size_t)n * K + k];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (n + 4 * j < N) a[j] += dy[(size_t)(n + 4 * j) * K + k];
   }
   __shared__ float sm[4][64];
-  sm[wave][lane] = a0 + a1;
+  sm[wave][lane] = ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
   __syncthreads();
   if (wave == 0 && k < K) {
     float v = alpha * ((sm[0][lane] + sm[1][lane]) + (sm[2][lane] + sm[3][lane]));
@@ -609,6 +648,25 @@ __global__ __launch_bounds__(256) void bwd_bias_rows_kernel(const float* __restr
 }  // namespace rh
 
 using namespace rh;
+
+// Scratch of the filter gradient proper, and behind it what rh_conv2d_bwd_filter_bias needs for the bias gradient: the
+// per-image plane sums that the pass over dy leaves (N x K floats), or the scratch of the two-stage bias gradient.
+static size_t bwd_filter_plan_bytes(const ConvDims& d) {
+  const BwdFilterPlan p = plan_bwd_filter(d);
+  const BwdFilterSoffPlan sp = plan_bwd_filter_soff(d);
+  const size_t legacy = p.tab_bytes + p.part_bytes;
+  return sp.ok && sp.total() > legacy ? sp.total() : legacy;
+}
+extern "C" size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane);
+static size_t bwd_filter_bias_bytes(const ConvDims& d) {
+  const size_t part = align256(sizeof(float) * (size_t)d.N * d.K);
+  const size_t two = rh_conv2d_bwd_bias_workspace_bytes(d.N, d.K, d.P * d.Q);
+  return part > two ? part : two;
+}
+static int bwd_bias_two_stage(int N, int K, int plane, float alpha, const float* dy, float beta, float* db, float* rowsum,
+                              hipStream_t stream);
+static int bwd_bias_one_stage(int N, int K, int plane, float alpha, const float* dy, float beta, float* db,
+                              hipStream_t stream);
 
 extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
   ConvDims d;
@@ -631,12 +689,8 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
       const SoffPlan sp = plan_soff_bwd_data(d);
       return sp.ok && sp.total() > legacy ? sp.total() : legacy;
     }
-    case RH_CONV_BWD_FILTER: {
-      const BwdFilterPlan p = plan_bwd_filter(d);
-      const BwdFilterSoffPlan sp = plan_bwd_filter_soff(d);
-      const size_t legacy = p.tab_bytes + p.part_bytes;
-      return sp.ok && sp.total() > legacy ? sp.total() : legacy;
-    }
+    case RH_CONV_BWD_FILTER:
+      return bwd_filter_plan_bytes(d) + bwd_filter_bias_bytes(d);
     default:
       return 0;
   }
@@ -654,9 +708,10 @@ extern "C" size_t rh_conv2d_workspace_bytes_upto(const rh_conv_geom* g, int pass
   return need;
 }
 
-extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const float* x, const float* dy,
-                                    float beta, float* dw, void* ws, size_t ws_bytes, int flags,
-                                    rh_stream_t stream_) {
+// bias_part: where the pass over dy may leave the per-image plane sums (N x K floats) if it makes one in a form that
+// can; *folded says whether it did.
+static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, const float* dy, float beta, float* dw,
+                           void* ws, size_t ws_bytes, int flags, rh_stream_t stream_, float* bias_part, bool* folded) {
   ConvDims d;
   if (int e = conv_dims(g, &d)) return e;
   if (!x || !dy || !dw) return RH_E_INVALID;
@@ -677,8 +732,10 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
     hipLaunchKernelGGL(prep_bwd_filter_soff_kernel, dim3(cdiv(sp.n_k, 256)), dim3(256), 0, stream, soff, dyT, sp.n_k, Ms,
                        d.P * d.Q, d.Q, d.st, sp.Hp, sp.Wp, d.C, d.K);
     if (int e = launch_status()) return e;
-    launch_nchw_to_nhwc(dy, dyT, d.N, d.K, d.P, d.Q, d.P, d.Q, 0, stream);
+    float* const bpart = (bias_part && nhwc_vec_ok(d.K, dyT)) ? bias_part : nullptr;
+    launch_nchw_to_nhwc(dy, dyT, d.N, d.K, d.P, d.Q, d.P, d.Q, 0, stream, bpart);
     if (int e = launch_status()) return e;
+    if (bpart) *folded = true;
     launch_nchw_to_nhwc(x, xT, d.N, d.C, d.H, d.W, sp.Hp, sp.Wp, d.pad, stream);
     if (int e = launch_status()) return e;
     RowSParams ap;  // dyT [pix][ko]
@@ -771,6 +828,38 @@ extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const fl
   }
   launch_split_reduce(part, used, (long long)d.K * CRS, dw, d.K, CRS, CRS, alpha, beta, stream);
   return launch_status();
+}
+
+extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const float* x, const float* dy,
+                                    float beta, float* dw, void* ws, size_t ws_bytes, int flags,
+                                    rh_stream_t stream_) {
+  bool folded = false;
+  return bwd_filter_impl(g, alpha, x, dy, beta, dw, ws, ws_bytes, flags, stream_, nullptr, &folded);
+}
+
+extern "C" int rh_conv2d_bwd_filter_bias(const rh_conv_geom* g, float alpha, const float* x, const float* dy,
+                                         float beta, float* dw, float* db, void* ws, size_t ws_bytes, int flags,
+                                         rh_stream_t stream_) {
+  ConvDims d;
+  if (int e = conv_dims(g, &d)) return e;
+  if (!db) return RH_E_INVALID;
+  if (!ws || ws_bytes < rh_conv2d_workspace_bytes(g, RH_CONV_BWD_FILTER) || (reinterpret_cast<uintptr_t>(ws) & 255))
+    return RH_E_WORKSPACE;
+  float* const bias_ws = reinterpret_cast<float*>(static_cast<char*>(ws) + bwd_filter_plan_bytes(d));
+  bool folded = false;
+  if (int e = bwd_filter_impl(g, alpha, x, dy, beta, dw, ws, ws_bytes, flags, stream_, bias_ws, &folded)) return e;
+  if (d.y_elems == 0) return 0;
+  hipStream_t stream = to_stream(stream_);
+  const int plane = d.P * d.Q;
+  if (folded) {   // the sums over the images of what the pass over dy left
+    ProfScope prof("bwd_bias_finish", 4.0 * (double)d.N * d.K, stream);
+    hipLaunchKernelGGL(bwd_bias_rows_kernel, dim3(cdiv(d.K, 64)), dim3(256), 0, stream, bias_ws, d.N, d.K, alpha, beta, db);
+    return launch_status();
+  }
+  ProfScope prof("bwd_bias", 4.0 * (double)d.y_elems, stream);
+  if (plane == 1 || rh_conv2d_bwd_bias_workspace_bytes(d.N, d.K, plane) == 0)
+    return bwd_bias_one_stage(d.N, d.K, plane, alpha, dy, beta, db, stream);
+  return bwd_bias_two_stage(d.N, d.K, plane, alpha, dy, beta, db, bias_ws, stream);
 }
 
 // Up to this many elements of dy one launch (a block per channel) is as fast as the first of the two stages, and the

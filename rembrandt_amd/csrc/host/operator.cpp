@@ -865,11 +865,18 @@ class Conv2dOperator : public Operator {
       if (in_delta_) { s_filter = s_bias; w_filter = w_bias; }
     }
     const float beta = params_.take_backward_beta();   // 1: accumulate (the reference's call); 0: the buffers stand for zeros
-    unwrap(rh_conv2d_bwd_filter(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta, params_.grad_weights->as_mut_ptr(),
-                                w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter");
-    unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), scale,
-                                 out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
-                                 w_bias->len(), s_bias), "conv2d backward bias");
+    if (s_filter == s_bias && w_filter == w_bias) {
+      // one stream for both: one call, which reads out_delta once where the filter gradient makes a pass over it anyway
+      unwrap(rh_conv2d_bwd_filter_bias(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta,
+                                       params_.grad_weights->as_mut_ptr(), params_.grad_bias->as_mut_ptr(),
+                                       w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter / bias");
+    } else {
+      unwrap(rh_conv2d_bwd_filter(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta, params_.grad_weights->as_mut_ptr(),
+                                  w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter");
+      unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), scale,
+                                   out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
+                                   w_bias->len(), s_bias), "conv2d backward bias");
+    }
     if (in_delta_) {
       unwrap(rh_conv2d_bwd_data(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
                                 workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward data");

@@ -71,6 +71,20 @@ def conv2d_bwd_filter(x, dy, w_shape, stride, pad, alpha=1.0, beta=0.0, dw=None,
     return dw
 
 
+def conv2d_bwd_filter_bias(x, dy, w_shape, stride, pad, alpha=1.0, beta=0.0, dw=None, db=None, algo=0):
+    """Filter and bias gradient in one call (rh_conv2d_bwd_filter_bias)."""
+    g = conv_geom(x.shape, w_shape, stride, pad)
+    if dw is None:
+        dw = torch.zeros(tuple(w_shape), dtype=torch.float32, device=x.device)
+    if db is None:
+        db = torch.zeros((w_shape[0],), dtype=torch.float32, device=x.device)
+    need = lib().rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_BWD_FILTER)
+    ws = workspace(need, x.device)
+    check(lib().rh_conv2d_bwd_filter_bias(C.byref(g), alpha, _p(x), _p(dy), beta, _p(dw), _p(db), _p(ws), ws.numel(), algo,
+                                          _stream()), "rh_conv2d_bwd_filter_bias")
+    return dw, db
+
+
 def conv2d_bwd_bias(dy, alpha=1.0, beta=0.0, db=None, two_stage=False):
     N, K = dy.shape[0], dy.shape[1]
     plane = dy.numel() // (N * K)

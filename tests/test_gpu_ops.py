@@ -106,6 +106,18 @@ def test_conv2d_all_passes(dev, case, algo):
     db2 = ops.conv2d_bwd_bias(dyd, alpha=0.5, beta=1.0, db=T(db0, dev), two_stage=True)
     assert_close(N(db2), O.conv2d_bwd_bias(dy, 0.5, 1.0, db0.copy()), "conv bwd bias (two-stage)")
 
+    # both gradients in one call: the filter gradient bit-identical to the call of its own, the bias gradient within
+    # tolerance of the oracle (where the pass over dy carries the plane sums it is added up in another order)
+    for alpha, beta in ((1.0, 0.0), (0.25, 1.0)):
+        dwc, dbc = ops.conv2d_bwd_filter_bias(xd, dyd, w.shape, st, pad, alpha=alpha, beta=beta, dw=T(dw0, dev), db=T(db0, dev),
+                                              algo=algo)
+        dws = ops.conv2d_bwd_filter(xd, dyd, w.shape, st, pad, alpha=alpha, beta=beta, dw=T(dw0, dev), algo=algo)
+        assert torch.equal(dwc, dws), "filter gradient of the combined call"
+        assert_close(N(dbc), O.conv2d_bwd_bias(dy, alpha, beta, db0.copy()), "bias gradient of the combined call")
+        dbc2 = ops.conv2d_bwd_filter_bias(xd, dyd, w.shape, st, pad, alpha=alpha, beta=beta, dw=T(dw0, dev), db=T(db0, dev),
+                                          algo=algo)[1]
+        assert torch.equal(dbc, dbc2), "the combined call is not deterministic"
+
     dx_ref = O.conv2d_bwd_data(w, dy, x.shape, st, pad)
     dx = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad, algo=algo)
     assert_close(N(dx), dx_ref, "conv bwd data")
