@@ -509,11 +509,20 @@ __global__ __launch_bounds__(1024) void bwd_bias_kernel(const float* __restrict_
                                                         float* __restrict__ db) {
   const int k = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-  float acc = 0.0f;
+  // four independent partial sums per lane: the loads of a plane are in flight together instead of one by one
+  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
   for (int n = wave; n < N; n += nwaves) {
     const float* p = dy + ((size_t)n * K + k) * plane;
-    for (int i = lane; i < plane; i += 64) acc += p[i];
+    int i = lane;
+    for (; i + 192 < plane; i += 256) {
+      a0 += p[i];
+      a1 += p[i + 64];
+      a2 += p[i + 128];
+      a3 += p[i + 192];
+    }
+    for (; i < plane; i += 64) a0 += p[i];
   }
+  float acc = (a0 + a1) + (a2 + a3);
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
   __shared__ float part[16];
   if (lane == 0) part[wave] = acc;
