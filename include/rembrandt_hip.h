@@ -173,6 +173,14 @@ int rh_conv2d_bwd_bias_noalloc(int32_t N, int32_t K, int32_t plane, float alpha,
 int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const float* w, const float* dy,
                        float beta, float* dx, void* ws, size_t ws_bytes, int flags,
                        rh_stream_t stream);
+/* rh_conv2d_bwd_data followed by the in-place ReLU backward of the operator below (the
+ * rembrandt_kernel_batch_map_rect_backprop_inplace(x_act, ., ., dx) that opens that operator's backward, mod.rs:1730-1737),
+ * as one call: dx[i] = x_act[i] > 0 ? alpha * corr^T(dy, w)[i] + beta * dx[i] : 0, where x_act is this convolution's
+ * input, i.e. that ReLU's output.  Same values as the two calls, without the extra pass over dx.
+ * rh_conv2d_bwd_data_relu_supported: nonzero for the geometries that have this form (all with stride 1). */
+int rh_conv2d_bwd_data_relu_supported(const rh_conv_geom* g);
+int rh_conv2d_bwd_data_relu(const rh_conv_geom* g, float alpha, const float* w, const float* dy, float beta,
+                            float* dx, const float* x_act, void* ws, size_t ws_bytes, int flags, rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Bias add and ReLU.  rh_add_bias_nchw replaces CudnnAddOp::forward (mod.rs:1097-1103,

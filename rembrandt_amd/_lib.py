@@ -98,6 +98,8 @@ PROTOTYPES = {
     "rh_noalloc_scratch_bytes": (_sz, []),
     "rh_conv2d_bwd_bias_noalloc": (_int, [_i32, _i32, _i32, _f, _vp, _f, _vp, _vp]),
     "rh_conv2d_bwd_data": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _sz, _int, _vp]),
+    "rh_conv2d_bwd_data_relu_supported": (_int, [C.POINTER(ConvGeom)]),
+    "rh_conv2d_bwd_data_relu": (_int, [C.POINTER(ConvGeom), _f, _vp, _vp, _f, _vp, _vp, _vp, _sz, _int, _vp]),
     "rh_add_bias_nchw": (_int, [_vp, _vp, _i32, _i32, _i32, _f, _f, _vp]),
     "rembrandt_kernel_batch_map_rect_inplace": (None, [_vp, _i32, _i32, _vp]),
     "rembrandt_kernel_batch_map_rect_backprop_inplace": (None, [_vp, _i32, _i32, _vp, _vp]),

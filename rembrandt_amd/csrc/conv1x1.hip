@@ -19,6 +19,8 @@
 // at the matrix peak): 96 us.  With parts removed: MFMAs and filter reads alone 65 us (the matrix pipe at the
 // clock it gets, three or four tiles per wave, prologue), loads and stores alone 77 us (dword accesses: what a
 // one-float-per-thread copy reaches), loads alone 40, stores alone 38.
+#include <type_traits>
+
 #include "conv_common.h"
 
 namespace rh {
@@ -50,8 +52,10 @@ constexpr int stream_blocks_per_cu() {
   return !FAST || 512 / regs < 2 ? 2 : (512 / regs > 4 ? 4 : 512 / regs);
 }
 
-template <int TM, int KH, bool FAST, class PASS>
-__global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST>())) void conv1x1_stream_kernel(Conv1x1Params p, EpiParams ep, FastDiv dPQ) {
+// MASK: ep.mask (a tensor shaped like the result) zeroes the result where it is not > 0 (backward-data that applies
+// the backward of the ReLU before this layer as it writes; sixteen more loads per row tile and column tile).
+template <int TM, int KH, bool FAST, class PASS, bool MASK = false>
+__global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST && !MASK>())) void conv1x1_stream_kernel(Conv1x1Params p, EpiParams ep, FastDiv dPQ) {
   const int lane = threadIdx.x & 63;
   // Blocks go to the eight XCDs in turn (block b to XCD b % 8), each with an L2 of its own.  An XCD takes a
   // contiguous eighth of the column tiles and its waves sweep that eighth in address order, so the two halves of a
@@ -104,6 +108,7 @@ __global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST>())) void c
 
   const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.src, p.src_bytes);
   const __amdgpu_buffer_rsrc_t rdst = make_rsrc(ep.out, (uint32_t)(sizeof(float) * (size_t)p.cols * p.rows));
+  const __amdgpu_buffer_rsrc_t rmask = make_rsrc(MASK ? ep.mask : ep.out, (uint32_t)(sizeof(float) * (size_t)p.cols * p.rows));
   const int PQ4 = p.PQ * 4;
   const uint32_t img_bytes = (uint32_t)p.kdim * (uint32_t)PQ4;
   const uint32_t out_img_bytes = (uint32_t)p.rows * (uint32_t)PQ4;
@@ -144,6 +149,15 @@ __global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST>())) void c
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][0][v] = 0.0f;
+    // where this tile goes, if it lies inside one image (then it is stored without per-element checks)
+    const uint32_t col0 = (uint32_t)tile * 32u;
+    uint32_t img0, pix0;
+    dPQ.divmod(col0, img0, pix0);
+    const bool inside = (long long)col0 + 31 < p.cols && pix0 + 31u < (uint32_t)p.PQ;   // uniform over the wave
+    const uint32_t out_o = img0 * out_img_bytes + (pix0 + (uint32_t)l32) * 4u + (uint32_t)(4 * half * PQ4);
+    float mreg[MASK ? TM : 1][16];
+    const uint32_t mask_o = inside ? out_o : 0x80000000u, mask_step = inside ? (uint32_t)PQ4 : 0u;
+    (void)mreg; (void)mask_o; (void)mask_step;
     // (opaque pointer: the filter reads must stay in the loop, one per MFMA, not be hoisted into KH * TM registers)
     // An LDS-space pointer: through a generic one these become flat loads, whose waits also cover the global loads.
     typedef const __attribute__((address_space(3))) float* lds_ptr;
@@ -167,6 +181,22 @@ __global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST>())) void c
       if (s == KH / 2 - 1) {
         __builtin_amdgcn_sched_barrier(0);
         load_part(b, nv, nstep, 0, KH / 2);
+        if (FAST && MASK) {
+          // this tile's mask values, in flight during the second half of the contraction (nothing for a tile that is
+          // stored element by element: every offset out of range)
+          uint32_t om = mask_o;
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                mreg[i][4 * q + e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rmask, (int)om, 0, 0));
+                om += mask_step;
+              }
+              om += 4u * mask_step;
+            }
+        }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -189,10 +219,6 @@ __global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST>())) void c
             for (int e = 0; e < 4; ++e) acc[i][0][4 * q + e] += bq[e];
           }
       }
-      const uint32_t col0 = (uint32_t)tile * 32u;
-      uint32_t img0, pix0;
-      dPQ.divmod(col0, img0, pix0);
-      const bool inside = (long long)col0 + 31 < p.cols && pix0 + 31u < (uint32_t)p.PQ;   // uniform over the wave
       if (inside) {
         if (ep.relu) {
 #pragma unroll
@@ -200,7 +226,13 @@ __global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST>())) void c
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][0][v] = acc[i][0][v] > 0.0f ? acc[i][0][v] : 0.0f;
         }
-        uint32_t o = img0 * out_img_bytes + (pix0 + (uint32_t)l32) * 4u + (uint32_t)(4 * half * PQ4);
+        uint32_t o = out_o;
+        if (MASK) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][0][v] = mreg[i][v] > 0.0f ? acc[i][0][v] : 0.0f;
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -230,7 +262,9 @@ __global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST>())) void c
           for (int v = 0; v < 16; ++v) {
             float val = acc[i][0][v];
             if (ep.relu) val = val > 0.0f ? val : 0.0f;
-            dst[(size_t)(32 * i + 8 * (v >> 2) + (v & 3)) * inner] = val;
+            const size_t at = (size_t)(32 * i + 8 * (v >> 2) + (v & 3)) * inner;
+            if (MASK && !(ep.mask[(dst - ep.out) + at] > 0.0f)) val = 0.0f;
+            dst[at] = val;
           }
       }
       return;
@@ -266,8 +300,25 @@ static int launch_stream(const Conv1x1Params& p, const EpiParams& ep, hipStream_
   const bool fast = ep.alpha == 1.0f && ep.beta == 0.0f && p.rows == 32 * TM && p.kdim == 2 * KH &&
                     (!ep.bias || (reinterpret_cast<uintptr_t>(ep.bias) & 15) == 0);
   // every block slot of the GPU; smaller problems: a wave per tile, in whole blocks per XCD when there are enough tiles
-  const int full = 256 * (fast ? stream_blocks_per_cu<TM, KH, true>() : stream_blocks_per_cu<TM, KH, false>());
+  const int full = 256 * (fast && !ep.mask ? stream_blocks_per_cu<TM, KH, true>() : stream_blocks_per_cu<TM, KH, false>());
   const int blocks = p.tiles >= 4 * full ? full : (p.tiles >= 256 ? 8 * cdiv(cdiv(p.tiles, 8), 4) : cdiv(p.tiles, 4));
+  if constexpr (std::is_same<PASS, PassConvBwdData>::value) {
+    if (ep.mask) {   // (the forward pass has no masked form)
+      if (lds > 48 * 1024) {
+        static const hipError_t a3 = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv1x1_stream_kernel<TM, KH, true, PASS, true>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        static const hipError_t a4 = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv1x1_stream_kernel<TM, KH, false, PASS, true>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (a3 != hipSuccess) return (int)a3;
+        if (a4 != hipSuccess) return (int)a4;
+      }
+      if (fast)
+        hipLaunchKernelGGL((conv1x1_stream_kernel<TM, KH, true, PASS, true>), dim3((unsigned)blocks), dim3(256), lds, stream, p, ep, dPQ);
+      else
+        hipLaunchKernelGGL((conv1x1_stream_kernel<TM, KH, false, PASS, true>), dim3((unsigned)blocks), dim3(256), lds, stream, p, ep, dPQ);
+      return launch_status();
+    }
+  }
   if (fast)
     hipLaunchKernelGGL((conv1x1_stream_kernel<TM, KH, true, PASS>), dim3((unsigned)blocks), dim3(256), lds, stream, p, ep, dPQ);
   else
@@ -291,7 +342,7 @@ bool conv1x1_stream_applies(const ConvDims& d) {
 
 // pass: RH_CONV_FWD (src = x, out = y) or RH_CONV_BWD_DATA (src = dy, out = dx).
 int launch_conv1x1_stream(const ConvDims& d, int pass, const float* w, const float* src, float* out, float alpha, float beta,
-                          const float* bias, int relu, hipStream_t stream) {
+                          const float* bias, int relu, hipStream_t stream, const float* mask) {
   const bool fwd = pass == RH_CONV_FWD;
   Conv1x1Params p;
   p.A = w;
@@ -307,6 +358,7 @@ int launch_conv1x1_stream(const ConvDims& d, int pass, const float* w, const flo
   EpiParams ep;
   ep.out = out; ep.bias = bias; ep.alpha = alpha; ep.beta = beta;
   ep.rows = p.rows; ep.cols = (int)p.cols; ep.inner = p.PQ; ep.ld = 0; ep.relu = relu; ep.split_stride = 0;
+  ep.mask = fwd ? nullptr : mask;
   ProfScope prof(fwd ? "conv_fwd_1x1_stream" : "conv_bwd_data_1x1_stream", 2.0 * (double)p.rows * (double)p.cols * (double)p.kdim,
                  stream);
   const int tm = cdiv(p.rows, 32);

@@ -146,7 +146,7 @@ static int run_bwd_data_soff(const RowSParams& ap, const RowSParams& bp, EpiPara
     ep.full_tiles = tail->full_tiles; ep.tail_tiles = tail->tail_tiles; ep.tail_splits = tail->splits;
     if (int e = launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, n_k, 1, nullptr, stream, tag, k_true)) return e;
     launch_split_reduce_nchw(part, tail->splits, total - first, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta,
-                             nullptr, 0, stream, tail->col0);
+                             nullptr, 0, stream, tail->col0, fin.mask);
     return launch_status();
   }
   // one pass over the whole contraction: K steps that hold nothing but the table's zero padding are left out
@@ -159,7 +159,8 @@ static int run_bwd_data_soff(const RowSParams& ap, const RowSParams& bp, EpiPara
   ep.out = part; ep.split_stride = total;
   int used = 1;
   if (int e = launch_mfma_gemm<T, AL, BL, true, PassConvBwdData>(ap, bp, ep, n_k, splits, &used, stream, tag, k_true)) return e;
-  launch_split_reduce_nchw(part, used, total, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta, nullptr, 0, stream);
+  launch_split_reduce_nchw(part, used, total, fin.out, total, fin.inner, fin.rows, fin.alpha, fin.beta, nullptr, 0, stream, 0,
+                           fin.mask);
   return launch_status();
 }
 
@@ -175,9 +176,10 @@ static int run_bwd_data(int KRS, const DenseParams& ap, const GatherParams& bp, 
 
 using namespace rh;
 
-extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const float* w, const float* dy,
-                                  float beta, float* dx, void* ws, size_t ws_bytes, int flags,
-                                  rh_stream_t stream_) {
+// mask: nullptr, or the output of the ReLU whose backward is applied to dx as it is written (never with the
+// residue-class form: see rh_conv2d_bwd_data_relu_supported).
+static int bwd_data_impl(const rh_conv_geom* g, float alpha, const float* w, const float* dy, float beta, float* dx,
+                         void* ws, size_t ws_bytes, int flags, rh_stream_t stream_, const float* mask) {
   ConvDims d;
   if (int e = conv_dims(g, &d)) return e;
   if (!w || !dy || !dx) return RH_E_INVALID;
@@ -188,11 +190,12 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
 
   if (!(flags & (RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET)) && conv1x1_stream_applies(d)) {
     if (d.x_elems == 0) return 0;
-    return launch_conv1x1_stream(d, RH_CONV_BWD_DATA, w, dy, dx, alpha, beta, nullptr, 0, stream);
+    return launch_conv1x1_stream(d, RH_CONV_BWD_DATA, w, dy, dx, alpha, beta, nullptr, 0, stream, mask);
   }
   const int KRS = d.K * d.R * d.S;
   const PhasePlan pp = plan_phase_bwd_data(d);
   if (pp.ok && !(flags & RH_ALGO_GATHER)) {
+    if (mask) return RH_E_UNSUPPORTED;
     if (d.x_elems == 0) return 0;
     char* base = static_cast<char*>(ws);
     int* soff = reinterpret_cast<int*>(base);
@@ -274,6 +277,7 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
     EpiParams ep;
     ep.out = dx; ep.bias = nullptr; ep.alpha = alpha; ep.beta = beta;
     ep.rows = d.C; ep.cols = bp.M; ep.inner = d.H * d.W; ep.ld = 0; ep.relu = 0; ep.split_stride = 0;
+    ep.mask = mask;
     float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes + sp.img_bytes);
     switch (pick_bm(d.C)) {
       case 128: return run_bwd_data_soff<T128x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_128x128", sp.splits, part, &sp.tail);
@@ -302,6 +306,7 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
   EpiParams ep;
   ep.out = dx; ep.bias = nullptr; ep.alpha = alpha; ep.beta = beta;
   ep.rows = d.C; ep.cols = bp.M; ep.inner = d.H * d.W; ep.ld = 0; ep.relu = 0; ep.split_stride = 0;
+  ep.mask = mask;
 
   switch (pick_bm(d.C)) {
     case 128: return run_bwd_data<T128x128>(KRS, ap, bp, ep, stream, "conv_bwd_data_128x128");
@@ -309,4 +314,25 @@ extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const floa
     case 64:  return run_bwd_data<T64x256>(KRS, ap, bp, ep, stream, "conv_bwd_data_64x256");
     default:  return run_bwd_data<T32x256>(KRS, ap, bp, ep, stream, "conv_bwd_data_32x256");
   }
+}
+
+extern "C" int rh_conv2d_bwd_data(const rh_conv_geom* g, float alpha, const float* w, const float* dy,
+                                  float beta, float* dx, void* ws, size_t ws_bytes, int flags,
+                                  rh_stream_t stream_) {
+  return bwd_data_impl(g, alpha, w, dy, beta, dx, ws, ws_bytes, flags, stream_, nullptr);
+}
+
+extern "C" int rh_conv2d_bwd_data_relu_supported(const rh_conv_geom* g) {
+  ConvDims d;
+  if (conv_dims(g, &d)) return 0;
+  if (conv1x1_stream_applies(d)) return 1;
+  return plan_phase_bwd_data(d).ok ? 0 : 1;   // strides above one take the residue-class form, which has no masked epilogue
+}
+
+extern "C" int rh_conv2d_bwd_data_relu(const rh_conv_geom* g, float alpha, const float* w, const float* dy,
+                                       float beta, float* dx, const float* x_act, void* ws, size_t ws_bytes,
+                                       int flags, rh_stream_t stream_) {
+  if (!x_act) return RH_E_INVALID;
+  if (!rh_conv2d_bwd_data_relu_supported(g)) return RH_E_UNSUPPORTED;
+  return bwd_data_impl(g, alpha, w, dy, beta, dx, ws, ws_bytes, flags, stream_, x_act);
 }

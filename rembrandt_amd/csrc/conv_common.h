@@ -226,7 +226,7 @@ inline int plan_k_split(int rows, long long cols, int n_k) {
 // elements, channel = (i / inner) % rows; only elements whose column (image * inner + pixel) is >= col0.
 void launch_split_reduce_nchw(const float* part, int splits, long long stride, float* out, long long total, int inner,
                               int rows, float alpha, float beta, const float* bias, int relu, hipStream_t stream,
-                              long long col0 = 0);
+                              long long col0 = 0, const float* mask = nullptr);
 
 
 inline SoffPlan plan_soff_fwd(const ConvDims& d) {
@@ -373,7 +373,7 @@ inline PhasePlan plan_phase_bwd_data(const ConvDims& d) {
 constexpr int kConv1x1MaxChannels = 128;
 bool conv1x1_stream_applies(const ConvDims& d);
 int launch_conv1x1_stream(const ConvDims& d, int pass, const float* w, const float* src, float* out, float alpha, float beta,
-                          const float* bias, int relu, hipStream_t stream);
+                          const float* bias, int relu, hipStream_t stream, const float* mask = nullptr);
 
 // dst[n][c][halo + dil*h][halo + dil*w] = src[n][c][h][w], zeros elsewhere; dst is planes x Hp x Wp.
 void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,

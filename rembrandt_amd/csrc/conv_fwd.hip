@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256) void split_reduce_nchw_kernel(const float* __r
                                                                 float* __restrict__ out, unsigned first, unsigned total,
                                                                 FastDiv inner, FastDiv rows, float alpha, float beta,
                                                                 const float* __restrict__ bias, int relu,
-                                                                unsigned col0) {
+                                                                unsigned col0, const float* __restrict__ mask) {
   constexpr int E = VEC ? 4 : 1;
   const unsigned i0 = first + (blockIdx.x * blockDim.x + threadIdx.x) * (unsigned)E;
   if (i0 >= total) return;
@@ -160,6 +160,7 @@ __global__ __launch_bounds__(256) void split_reduce_nchw_kernel(const float* __r
     if (beta != 0.0f) v = fmaf(beta, old[e], v);
     if (bias) v += bias[plane - img * rows.div];
     if (relu) v = v > 0.0f ? v : 0.0f;
+    if (mask && !(mask[i < total ? i : i0] > 0.0f)) v = 0.0f;
     res[e] = v;
   }
   if (VEC) {
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(256) void split_reduce_nchw_kernel(const float* __r
 
 void launch_split_reduce_nchw(const float* part, int splits, long long stride, float* out, long long total, int inner,
                               int rows, float alpha, float beta, const float* bias, int relu, hipStream_t stream,
-                              long long col0) {
+                              long long col0, const float* mask) {
   // elements before the image that holds column col0 are not part of the reduction
   const long long first = col0 > 0 ? (col0 / inner) * (long long)rows * inner : 0;
   ProfScope prof("split_reduce", 4.0 * (double)(total - first) * (splits + 1), stream);
@@ -184,11 +185,11 @@ void launch_split_reduce_nchw(const float* part, int splits, long long stride, f
   if (vec)
     hipLaunchKernelGGL((split_reduce_nchw_kernel<true>), dim3(stream_grid((size_t)(total - first) / 4, 256)), dim3(256), 0, stream,
                        part, splits, stride, out, (unsigned)first, (unsigned)total, FastDiv((uint32_t)inner),
-                       FastDiv((uint32_t)rows), alpha, beta, bias, relu, (unsigned)col0);
+                       FastDiv((uint32_t)rows), alpha, beta, bias, relu, (unsigned)col0, mask);
   else
     hipLaunchKernelGGL((split_reduce_nchw_kernel<false>), dim3(stream_grid((size_t)(total - first), 256)), dim3(256), 0, stream,
                        part, splits, stride, out, (unsigned)first, (unsigned)total, FastDiv((uint32_t)inner),
-                       FastDiv((uint32_t)rows), alpha, beta, bias, relu, (unsigned)col0);
+                       FastDiv((uint32_t)rows), alpha, beta, bias, relu, (unsigned)col0, mask);
 }
 
 // `splits` > 1: slices of the contraction write unblended partial results to `part`, then one reduction applies the

@@ -606,6 +606,9 @@ struct EpiParams {
   int relu;
   long long split_stride;
   const float* bias_col = nullptr;   // one value per result column (the dense, non-NCHW form: an affine layer's bias)
+  // NCHW form: a tensor of the result's shape; result elements whose mask value is not > 0 are stored as 0 (backward-data
+  // that also applies the backward of the ReLU that produced its input: the mask is that ReLU's output).
+  const float* mask = nullptr;
   float* part = nullptr;
   long long part_first = 0;
   int full_tiles = 0, tail_tiles = 0, tail_splits = 0;
@@ -661,6 +664,7 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], co
           if (!split && ep.bias) val += ep.bias[row];
           if (!NCHW && !split && ep.bias_col) val += cbias;
           if (!split && ep.relu) val = val > 0.0f ? val : 0.0f;
+          if (NCHW && !split && ep.mask && !(ep.mask[(size_t)coloff + (size_t)row * row_stride] > 0.0f)) val = 0.0f;
           *dst = val;
         }
       }

@@ -788,7 +788,7 @@ class AffineOperator : public Operator {
 // ---- Conv2dOperator -------------------------------------------------------------------------------------
 class Conv2dOperator : public Operator {
  public:
-  Conv2dOperator(size_t batch_size, OpCapability capability, const Conv2dOperatorConfig& config, const Operator* prev_op,
+  Conv2dOperator(size_t batch_size, OpCapability capability, const Conv2dOperatorConfig& config, Operator* prev_op,
                  Ctx context, ExecOptions opts)
       : batch_cap_(batch_size), config_(config), context_(context), opts_(opts) {
     RB_ASSERT(prev_op != nullptr);
@@ -816,6 +816,9 @@ class Conv2dOperator : public Operator {
       wa = std::max(wa, bias_ws_upto(g.N, g.K, (int)(out_dims_.w * out_dims_.h)));
       workspace_aux_.reset(new DeviceBuffer<uint8_t>(std::max<size_t>(wa, 256), context));
     }
+    // the data gradient can zero what the ReLU below would have masked in a pass of its own
+    if (backward_enabled(capability) && in_delta_ && opts.fuse_epilogue && rh_conv2d_bwd_data_relu_supported(&g))
+      fold_prev_relu_ = prev_op->fold_activation_backward();
   }
   size_t batch_size() const override { return batch_cap_; }
   SharedDeviceBuf get_output_vars() const override { return out_act_; }
@@ -877,7 +880,12 @@ class Conv2dOperator : public Operator {
                                    out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
                                    w_bias->len(), s_bias), "conv2d backward bias");
     }
-    if (in_delta_) {
+    if (in_delta_ && fold_prev_relu_) {
+      // the operator below left its ReLU backward mask to this call: in_act_ is that ReLU's output
+      unwrap(rh_conv2d_bwd_data_relu(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
+                                     in_act_->as_ptr(), workspace_->as_mut_ptr(), workspace_->len(), 0, s),
+             "conv2d backward data");
+    } else if (in_delta_) {
       unwrap(rh_conv2d_bwd_data(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
                                 workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward data");
     }
@@ -918,7 +926,8 @@ class Conv2dOperator : public Operator {
   void set_overlap_backward(bool on) override { overlap_on_ = on; }
 
  private:
-  bool act_bwd_folded_ = false;
+  bool act_bwd_folded_ = false;   // the operator above applies this operator's ReLU backward mask
+  bool fold_prev_relu_ = false;   // this operator's data gradient applies the ReLU backward mask of the operator below
   rh_conv_geom geom(size_t batch) const {
     rh_conv_geom g;
     g.N = (int)batch; g.C = (int)config_.in_dims.c; g.H = (int)config_.in_dims.h; g.W = (int)config_.in_dims.w;

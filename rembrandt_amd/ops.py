@@ -99,15 +99,26 @@ def conv2d_bwd_bias(dy, alpha=1.0, beta=0.0, db=None, two_stage=False):
     return db
 
 
-def conv2d_bwd_data(w, dy, x_shape, stride, pad, alpha=1.0, beta=0.0, dx=None, algo=0):
+def conv2d_bwd_data(w, dy, x_shape, stride, pad, alpha=1.0, beta=0.0, dx=None, algo=0, relu_of=None):
+    """relu_of: this convolution's input (a ReLU's output); its backward mask is applied to dx as it is written
+    (rh_conv2d_bwd_data_relu)."""
     g = conv_geom(x_shape, w.shape, stride, pad)
     if dx is None:
         dx = torch.zeros(tuple(x_shape), dtype=torch.float32, device=w.device)
     need = lib().rh_conv2d_workspace_bytes(C.byref(g), _lib.RH_CONV_BWD_DATA)
     ws = workspace(need, w.device)
+    if relu_of is not None:
+        check(lib().rh_conv2d_bwd_data_relu(C.byref(g), alpha, _p(w), _p(dy), beta, _p(dx), _p(relu_of), _p(ws), ws.numel(),
+                                            algo, _stream()), "rh_conv2d_bwd_data_relu")
+        return dx
     check(lib().rh_conv2d_bwd_data(C.byref(g), alpha, _p(w), _p(dy), beta, _p(dx), _p(ws), ws.numel(), algo,
                                    _stream()), "rh_conv2d_bwd_data")
     return dx
+
+
+def conv2d_bwd_data_relu_supported(x_shape, w_shape, stride, pad):
+    g = conv_geom(x_shape, w_shape, stride, pad)
+    return bool(lib().rh_conv2d_bwd_data_relu_supported(C.byref(g)))
 
 
 def add_bias_nchw(bias, y, alpha=1.0, beta=1.0):

@@ -121,6 +121,17 @@ def test_conv2d_all_passes(dev, case, algo):
     dx_ref = O.conv2d_bwd_data(w, dy, x.shape, st, pad)
     dx = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad, algo=algo)
     assert_close(N(dx), dx_ref, "conv bwd data")
+    # with the backward of the ReLU that produced x applied as dx is written: bit-identical to the data gradient
+    # followed by the in-place mask (x here stands for that ReLU's output: its sign pattern is all that matters)
+    if ops.conv2d_bwd_data_relu_supported(x.shape, w.shape, st, pad):
+        dx0 = synth.normal(11, 8, x.shape)
+        for alpha, beta in ((1.0, 0.0), (0.5, 2.0)):
+            two = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad, alpha=alpha, beta=beta, dx=T(dx0, dev), algo=algo)
+            ops.rect_backprop_inplace(xd, two)
+            one = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad, alpha=alpha, beta=beta, dx=T(dx0, dev), algo=algo, relu_of=xd)
+            assert torch.equal(one, two), "masked data gradient alpha=%g beta=%g" % (alpha, beta)
+    else:
+        assert st > 1
     torch.cuda.synchronize()
 
 
