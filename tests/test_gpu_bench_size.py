@@ -11,7 +11,7 @@ Gradients are zeroed by the fused update, so they are checked through what the u
 v_t = mu*v_{t-1} - eta*g_t on sampled elements, W_t = W_{t-1} + v_t on all of them, bit for bit.
 A second worker runs the same steps back to back without any read-back in between (reading a buffer joins the
 streams), and must end with bit-identical parameters: the cross-step overlap changes nothing.
-The worst absolute / relative error per checked tensor is printed and written to gpurun_out/parity_<net>.json.
+The worst absolute / relative error per checked tensor is printed and written to parity_<net>_b<batch>.json in the output folder of the run.
 """
 import json
 import os

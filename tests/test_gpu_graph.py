@@ -103,7 +103,7 @@ def check_step(w, ref, sgd, rsgd, x, labels, minibatch, fused_sgd, tag):
 
 @pytest.mark.parametrize("fuse,fused_sgd", [(True, True), (False, False)])
 def test_lenet_train_steps(dev, fuse, fused_sgd):
-    """BASELINE config 1: LeNet, batch 64, U[0,1) inputs, lr 0.01, momentum 0.9, weight decay 5e-4; 3 steps."""
+    """Benchmark configuration 1: LeNet, batch 64, U[0,1) inputs, lr 0.01, momentum 0.9, weight decay 5e-4; 3 steps."""
     net, batch = configs.lenet(), 64
     say("lenet fuse", fuse, fused_sgd)
     w, ref = make_pair(net, batch, 0x5EED0001, fuse)
@@ -119,7 +119,7 @@ def test_lenet_train_steps(dev, fuse, fused_sgd):
 
 
 def test_cifar_train_steps(dev):
-    """BASELINE config 3: CIFAR-10-shaped net, batch 128, N(0,1) inputs, momentum 0.9; 2 steps."""
+    """Benchmark configuration 3: CIFAR-10-shaped net, batch 128, N(0,1) inputs, momentum 0.9; 2 steps."""
     net, batch = configs.cifar10(), 128
     w, ref = make_pair(net, batch, 0x5EED0003, True)
     sgd = SgdOpt(batch, 0.01, ("Update", 0.9), 0.0)
@@ -135,7 +135,7 @@ def test_cifar_train_steps(dev):
 
 
 def test_alexnet_train_step(dev):
-    """BASELINE config 4 geometry (AlexNet-shaped: 11x11 stride-4 conv on 227x227, three 3x3/2 max-pools,
+    """Benchmark configuration 4 geometry (AlexNet-shaped: 11x11 stride-4 conv on 227x227, three 3x3/2 max-pools,
     4096-wide affine layers, 1000 classes) at batch 4: one whole step, checkpoint by checkpoint."""
     net, batch = configs.alexnet(), 4
     w, ref = make_pair(net, batch, 0x5EED0004, True)
@@ -179,7 +179,7 @@ def test_dropout_lrn_train_steps(dev):
 
 
 def test_nin_train_step(dev):
-    """BASELINE config 5 geometry (NIN-shaped: 1x1 "cccp" convolutions, ceil-mode max-pools, 6x6 average pool
+    """Benchmark configuration 5 geometry (NIN-shaped: 1x1 "cccp" convolutions, ceil-mode max-pools, 6x6 average pool
     into 1000 classes) at batch 2, fp32: one whole step, checkpoint by checkpoint."""
     net, batch = configs.nin(), 2
     w, ref = make_pair(net, batch, 0x5EED0005, True)
@@ -195,7 +195,7 @@ def test_nin_train_step(dev):
 
 
 def test_nin_forward_bf16(dev):
-    """BASELINE config 5, forward only with bf16 operands and fp32 accumulation.  Each operator is compared
+    """Benchmark configuration 5, forward only with bf16 operands and fp32 accumulation.  Each operator is compared
     from the GPU's own input to it (a last-bit difference upstream may round to a different bf16 value)."""
     net, batch = configs.nin(), 2
     dims, layers, ncat = net
