@@ -112,6 +112,26 @@ inline int launch_mfma_gemm_bf16(const typename AL::Params& ap, const typename B
   return launch_status();
 }
 
+// The direct-to-LDS form for packed operands (ring of four LDS buffers, one pass over the whole contraction).
+template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS>
+inline int launch_mfma_gemm_bf16_dma(const RowV8Params& ap, const RowV8Params& bp, const EpiParams& ep, int K,
+                                     hipStream_t stream, const char* tag, int k_algorithmic = 0) {
+  const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
+  if (K <= 0 || K % T::BK != 0) return RH_E_INVALID;
+  constexpr size_t lds_bytes = 16 * 4 * (T::BK / 8) * (T::BM + T::BN);
+  static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (attr != hipSuccess) return (int)attr;
+  }
+  ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)(k_algorithmic > 0 ? k_algorithmic : K), stream);
+  hipLaunchKernelGGL((mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS>), dim3((unsigned)(tiles_m * tiles_n)),
+                     dim3(T::NT), lds_bytes, stream, ap, bp, ep, tiles_m, K / T::BK);
+  return launch_status();
+}
+
 #ifndef RH_OCC_128
 #define RH_OCC_128 4
 #endif
@@ -127,6 +147,8 @@ typedef Tile<96, 128, 16, 1, 4, 4> T96x128;
 #endif
 // bf16-operand kernel: a deeper K step keeps more operand loads in flight per wave (its MFMAs are 16x shorter)
 typedef Tile<128, 128, RH_BF16_BK, 2, 2, RH_BF16_OCC> T128x128bf;
+// Tile of the direct-to-LDS bf16 kernel: eight waves of 128x64 each, one block per CU, four 32-k LDS buffers.
+typedef Tile<256, 256, 32, 2, 4, 1> T256x256bf;
 typedef Tile<64, 256, 16, 1, 4, 3> T64x256;
 typedef Tile<32, 256, 16, 1, 4, 3> T32x256;
 // Half the K step: 20 KB of LDS, so a CU holds 4 blocks instead of 3.  For grids that need a second round of

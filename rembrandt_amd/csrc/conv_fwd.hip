@@ -303,7 +303,7 @@ __global__ __launch_bounds__(256) void nchw_to_bf16_groups_kernel(const float* _
   xb[i] = pack8_bf16(v);
 }
 
-template <class T>
+template <class T, bool DMA = false>
 static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const float* x, const float* w, void* ws,
                                const EpiParams& ep, hipStream_t stream, const char* tag) {
   char* base = static_cast<char*>(ws);
@@ -335,6 +335,7 @@ static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const 
   bp.group_stride = 0;
   typedef LoadRowV8<T::BM, T::BK, T::NT, true> AL;
   typedef LoadRowV8<T::BN, T::BK, T::NT, false> BL;
+  if (DMA) return launch_mfma_gemm_bf16_dma<T, true, false, true, PassConvFwd>(ap, bp, ep, bpn.n_k, stream, tag, CRS);
   return launch_mfma_gemm_bf16<T, AL, BL, true, PassConvFwd>(ap, bp, ep, bpn.n_k, 1, nullptr, stream, tag, CRS);
 }
 
@@ -378,6 +379,12 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
       ep.out = y; ep.bias = (flags & RH_FUSE_BIAS) ? bias : nullptr; ep.alpha = alpha; ep.beta = beta;
       ep.rows = d.K; ep.cols = d.N * d.P * d.Q; ep.inner = d.P * d.Q; ep.ld = 0; ep.relu = (flags & RH_FUSE_RELU) ? 1 : 0;
       ep.split_stride = 0;
+      // Long contractions on grids that fill all 256 CUs with 256-row tiles (and waste no more filter rows than
+      // 128-row tiles would) take the direct-to-LDS kernel: 14 % faster on 256 x 96 x 27 x 27 -> 256, 5x5.  Short
+      // contractions lose there (one block per CU: nothing hides a tile's first loads and its stores).
+      if (bpn.n_k >= 512 && cdiv(d.K, 256) * 256 == cdiv(d.K, 128) * 128 &&
+          (long long)cdiv(d.K, 256) * cdiv(ep.cols, 256) >= 256)
+        return run_fwd_bf16_packed<T256x256bf, true>(d, bpn, x, w, ws, ep, stream, "conv_fwd_bf16p_256x256");
       return run_fwd_bf16_packed<T128x128bf>(d, bpn, x, w, ws, ep, stream, "conv_fwd_bf16p_128x128");
     }
   }

@@ -941,4 +941,223 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_kernel(typename 
   store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, ep.split_stride != 0 ? split_idx : -1);
 }
 
+// ------------------------------------------------------------------------------------------
+// The bf16 kernel for operands that are already packed in memory (RowV8Params on both sides), with the operand slabs
+// brought into a ring of four LDS buffers by direct global -> LDS loads (buffer_load_dwordx4 ... lds: lane l's 16
+// bytes land at M0 + 16 l, which is exactly 64 neighbouring rows of one 8-k group of a [k/8][row] slab).
+//
+// Why: through registers (global load, then ds_write_b128) the LDS accepts about 70 bytes per clock and CU, and a
+// wave that issues its writes stalls while the queue is full, so the writes of a step stand in front of its MFMAs
+// instead of under them; and a 128x128 tile needs 64 bytes per clock of such fill at full MFMA rate, which is all
+// the path has.  A 256x256 tile halves the fill per MFMA, the direct loads need no registers, no ds_write and no
+// issue slots beyond the load itself, and they complete in the background.
+//
+// Step `it` of a wave: multiplies out of buffer it; issues the loads of step it+3 into buffer it+3 (= it-1, read
+// for the last time before the barrier that ended step it-1); reads, during its last group of MFMAs, the first
+// operands of step it+1 (buffer it+1); then waits until only the loads it has just issued are still in flight
+// (so those of step it+2 have landed) and meets the other waves at the step's one barrier.  A load therefore has
+// two steps to land, and nothing the matrix pipe has to wait for follows a barrier.
+// The compiler does not see these loads (inline asm): their completion is counted by hand (vmcnt is in order),
+// and no other vector memory instruction is issued between the prologue and the epilogue.
+// One block per CU (128 KB of LDS): the first loads and the stores of a tile are not hidden behind another block,
+// which is why this form pays only for long contractions.
+// ------------------------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void dma_load16(u32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// RowV8Params operand loaded straight into an LDS slab.  Thread -> (row, groups) as in LoadRowV8; a wave covers 64
+// neighbouring rows of each of its groups.  Two sets of group offsets: the loads of a step use `so` while `so_next`
+// is being fetched for the step after.
+template <int ROWS, int BK, int NT, bool LINEAR>
+struct DmaRowV8 {
+  static constexpr int KG = BK / 8;
+  static constexpr int CNT = ROWS * KG / NT;
+  static_assert(BK % 8 == 0 && NT % ROWS == 0 && (ROWS * KG) % NT == 0 && ROWS % kWave == 0, "loader shape");
+  typedef RowV8Params Params;
+  typedef const __attribute__((address_space(4))) int* ctab_t;
+  u32x4 rsrc;
+  const int* tab;
+  uint32_t vbase;
+  int g0, wrow, gstride;
+  int so[CNT], so_next[CNT];
+
+  __device__ __forceinline__ void init(const Params& p, int row0, int tid) {
+    const uint64_t a = reinterpret_cast<uint64_t>(p.ptr);
+    rsrc.x = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    rsrc.y = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+    rsrc.z = __builtin_amdgcn_readfirstlane(p.bytes);
+    rsrc.w = 0x00020000u;
+    const int row = tid % ROWS;
+    wrow = __builtin_amdgcn_readfirstlane((tid & ~(kWave - 1)) % ROWS);
+    g0 = __builtin_amdgcn_readfirstlane(tid / ROWS) * CNT;
+    tab = p.soff;
+    gstride = p.group_stride;
+    const int m = row0 + row;
+    const bool valid = m < p.M;
+    const int mm = valid ? m : 0;
+    const int n = mm / p.inner;
+    const int rem = mm - n * p.inner;
+    const int a2 = rem / p.innerW;
+    const int b2 = rem - a2 * p.innerW;
+    vbase = valid ? (uint32_t)(n * p.img_stride + a2 * p.a_stride + b2 * p.b_stride) : 0x80000000u;
+  }
+  // The table is read through the constant address space: scalar loads, which the hand-counted vmcnt of the
+  // direct loads does not see.  (As a global load it becomes a vector load, since the asm statements may write
+  // memory for all the compiler knows, and the wait for it would also wait for every direct load in flight.)
+  __device__ __forceinline__ int group_off(int k0, int i) const {
+    return LINEAR ? ((k0 >> 3) + g0 + i) * gstride : ((ctab_t)(uintptr_t)tab)[(k0 >> 3) + g0 + i];
+  }
+  __device__ __forceinline__ void prep(int k0) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) so[i] = group_off(k0, i);
+  }
+  __device__ __forceinline__ void prep_next(int k0) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) so_next[i] = group_off(k0, i);
+  }
+  __device__ __forceinline__ void rotate() {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) so[i] = so_next[i];
+  }
+  // slab_addr: LDS byte address of the [KG][ROWS] slab of 16-byte groups
+  __device__ __forceinline__ void issue(uint32_t slab_addr) const {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i)
+      dma_load16(rsrc, slab_addr + (uint32_t)((g0 + i) * ROWS + wrow) * 16u, vbase, (uint32_t)so[i]);
+  }
+};
+
+template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS>
+__global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8Params ap, RowV8Params bp, EpiParams ep,
+                                                                           int tiles_m, int k_chunks) {
+  constexpr int BM = T::BM, BN = T::BN, BK = T::BK, TM = T::TM, TN = T::TN;
+  static_assert(BK % 32 == 0, "an even number of 16-k groups per step keeps the operand register sets in phase");
+  typedef DmaRowV8<BM, BK, T::NT, A_LINEAR> AL;
+  typedef DmaRowV8<BN, BK, T::NT, B_LINEAR> BL;
+  constexpr int KG = BK / 8, STEPS = BK / 16, R = 4;
+  constexpr int SA = KG * BM, SB = KG * BN;  // 16-byte groups per buffer
+  extern __shared__ float lds_dyn[];
+  uint4* const sA_base = reinterpret_cast<uint4*>(lds_dyn);  // [R][KG][BM]
+  uint4* const sB_base = sA_base + R * SA;                   // [R][KG][BN]
+  const uint32_t ldsA = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)sA_base;
+  const uint32_t ldsB = ldsA + R * SA * 16;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % T::WM, wn = wave / T::WM;
+
+  const int logical = __builtin_amdgcn_readfirstlane(xcd_remap(blockIdx.x, gridDim.x));
+  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int nk = k_chunks;
+
+  AL la;
+  BL lb;
+  la.init(ap, m0, tid);
+  lb.init(bp, n0, tid);
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  auto prep_step = [&](int s) {
+    la.prep(s * BK);
+    lb.prep(s * BK);
+  };
+  auto issue_step = [&](int buf) {
+    la.issue(ldsA + (uint32_t)(buf * SA) * 16u);
+    lb.issue(ldsB + (uint32_t)(buf * SB) * 16u);
+  };
+  // steps 0..2 on their way, the offsets of step 3 fetched
+  prep_step(0);
+  issue_step(0);
+  if (nk > 1) { prep_step(1); issue_step(1); }
+  if (nk > 2) { prep_step(2); issue_step(2); }
+  if (nk > 3) prep_step(3);
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  const int a_rd = (lane >> 5) * BM + wm * (TM * 32) + (lane & 31);
+  const int b_rd = (lane >> 5) * BN + wn * (TN * 32) + (lane & 31);
+  uint4 a[2][TM], b[2][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) a[0][i] = sA_base[a_rd + i * 32];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) b[0][j] = sB_base[b_rd + j * 32];
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the loop is entered with nothing in flight, so its waits can be exact
+
+  auto step = [&](int it, auto more_tag) {
+    constexpr bool MORE = decltype(more_tag)::value;  // this step issues the loads of step it+3
+    const int rd = it & (R - 1), nx = (it + 1) & (R - 1);
+    const uint4* pa = sA_base + rd * SA + a_rd;
+    const uint4* pb = sB_base + rd * SB + b_rd;
+    const uint4* pna = sA_base + nx * SA + a_rd;
+    const uint4* pnb = sB_base + nx * SB + b_rd;
+#pragma unroll
+    for (int g = 0; g < STEPS; ++g) {
+      const int c = g & 1, n = c ^ 1;
+      __builtin_amdgcn_sched_barrier(0);
+      // Everything this wave has asked of the LDS and of the scalar cache was issued at least a group of MFMAs
+      // ago: an explicit wait here costs nothing, and it lets the wait in front of this group's MFMAs disappear
+      // (otherwise that one, being a wait for "everything" because scalar loads return out of order, would also
+      // cover the operand reads issued just before it).
+      if (g > 0) __builtin_amdgcn_s_waitcnt(0xc07f);
+      if (MORE && g == 0) {
+        // the offsets of step it+4 (used by the loads the next step issues), fetched first for the same reason
+        const int s4 = it + 4 < nk ? it + 4 : nk - 1;
+        la.prep_next(s4 * BK);
+        lb.prep_next(s4 * BK);
+      }
+      if (g + 1 < STEPS) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[n][i] = pa[(2 * g + 2) * BM + i * 32];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[n][j] = pb[(2 * g + 2) * BN + j * 32];
+      } else {  // (after the last step this reads a buffer nobody uses: harmless)
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[n][i] = pna[i * 32];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[n][j] = pnb[j * 32];
+      }
+      if (MORE && g == 0) issue_step((it + 3) & (R - 1));
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[c][i]),
+                                                              __builtin_bit_cast(bf16x8_t, b[c][j]), acc[i][j], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (MORE) {
+      la.rotate();
+      lb.rotate();
+      wait_vmcnt<AL::CNT + BL::CNT>();
+    } else {
+      wait_vmcnt<0>();
+    }
+    __syncthreads();
+  };
+  int it = 0;
+  for (; it + 3 < nk; ++it) step(it, std::true_type());
+  for (; it < nk; ++it) step(it, std::false_type());
+
+  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, -1);
+}
+
 }  // namespace rh

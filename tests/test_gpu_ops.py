@@ -144,6 +144,15 @@ BF16_PACKED_CASES = [
     (5, 16, 9, 12, 24, 3, 1, 0),
     (2, 8, 6, 6, 3, 1, 1, 0),
     (130, 8, 5, 5, 16, 3, 1, 1),
+    # long contractions on grids of 256 and more 256-row tiles take the direct-to-LDS kernel: ragged rows and columns,
+    # two row tiles, a strided layer, a 1x1 layer whose contraction is exactly four ring buffers long plus twelve steps;
+    # the last two are grids as large on short contractions (the 128x128 kernel)
+    (80, 24, 30, 30, 130, 5, 1, 2),
+    (40, 64, 31, 29, 500, 3, 1, 1),
+    (120, 64, 47, 45, 200, 3, 2, 1),
+    (70, 512, 34, 33, 256, 1, 1, 0),
+    (70, 8, 34, 33, 384, 1, 1, 0),
+    (80, 8, 30, 30, 130, 5, 1, 2),
 ]
 
 
