@@ -277,21 +277,36 @@ inline SoffPlan plan_soff_fwd(const ConvDims& d) {
 // Scratch: table of byte offsets per group of eight k | filter copy | image copy.
 struct Bf16FwdPlan {
   int n_k, Hp, Wp;
+  int s_groups;  // 0: groups of eight channels; > 0: groups of eight filter columns, this many per filter row
   size_t tab_bytes, wt_bytes, img_bytes;
   bool ok;
   size_t total() const { return tab_bytes + wt_bytes + img_bytes; }
 };
 
+// Channel counts that are not a multiple of 8 (first layers: 3 channels) with an even stride group the contraction
+// by filter columns instead: k = (c, r, s) with s padded to a multiple of 8, the image copied to bf16 in its own
+// NCHW order with its zero border (rows widened by the padding of s, to an even width), so that the eight s of a
+// group are 16 contiguous bytes starting at an even element (4-byte aligned, as a vector load needs) and
+// neighbouring pixels are `stride` elements apart.  An 11x11 filter pads to 16 columns (1.45x the contraction; with
+// channels padded 3 -> 8 it would be 2.7x), a 7x7 to 8.
 inline Bf16FwdPlan plan_bf16_fwd(const ConvDims& d) {
   Bf16FwdPlan p;
-  p.n_k = round_up(d.C * d.R * d.S, kTabPad);
   p.Hp = d.H + 2 * d.pad;
-  p.Wp = d.W + 2 * d.pad;
+  if (d.C % 8 == 0) {
+    p.s_groups = 0;
+    p.n_k = round_up(d.C * d.R * d.S, kTabPad);
+    p.Wp = d.W + 2 * d.pad;
+  } else {
+    p.s_groups = cdiv(d.S, 8);
+    p.n_k = round_up(d.C * d.R * p.s_groups * 8, kTabPad);
+    p.Wp = round_up(d.W + 2 * d.pad + p.s_groups * 8 - d.S, 2);
+  }
   p.tab_bytes = align256(sizeof(int) * (size_t)(p.n_k / 8));
   p.wt_bytes = align256(2 * (size_t)p.n_k * d.K);
   const size_t img = 2 * (size_t)d.N * d.C * p.Hp * p.Wp;
   p.img_bytes = align256(img);
-  p.ok = d.C % 8 == 0 && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0 && (long long)p.Hp * p.Wp < (1ll << 31) / 64;
+  p.ok = (d.C % 8 == 0 || d.st % 2 == 0) && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0 &&
+         (long long)p.Hp * p.Wp < (1ll << 31) / 64;
   return p;
 }
 

@@ -303,6 +303,48 @@ __global__ __launch_bounds__(256) void nchw_to_bf16_groups_kernel(const float* _
   xb[i] = pack8_bf16(v);
 }
 
+// The same two copies for groups of eight filter columns (Bf16FwdPlan::s_groups > 0).
+// wb[g][ko][8] = w[ko][c][r][8 sg + e] (zero for columns past S and groups past the end), g = (c*R + r)*Sg + sg;
+// soff8[g] = byte offset of (c, r, 8 sg) in one image of the copy.
+__global__ __launch_bounds__(256) void prep_bf16_filter_cols_kernel(const float* __restrict__ w, uint4* __restrict__ wb,
+                                                                    int* __restrict__ soff8, int n_k, int groups, int K,
+                                                                    int CRS, int R, int S, int Sg, int Hp, int Wp) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long long)(n_k / 8) * K) return;
+  const int g = (int)(i / K), ko = (int)(i - (long long)g * K);
+  const int cr = g / Sg, sg = g - cr * Sg;
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int s2 = 8 * sg + e;
+    v[e] = (g < groups && s2 < S) ? w[(size_t)ko * CRS + (size_t)cr * S + s2] : 0.0f;
+  }
+  wb[i] = pack8_bf16(v);
+  if (ko == 0) {
+    const int c = cr / R, r = cr - c * R;
+    soff8[g] = g < groups ? ((c * Hp + r) * Wp + 8 * sg) * 2 : 0;
+  }
+}
+
+// xb[n][c][hp][wp] (bf16) = x[n][c][hp - halo][wp - halo], zero outside; one thread per two elements (Wp is even).
+__global__ __launch_bounds__(256) void nchw_to_bf16_planes_kernel(const float* __restrict__ x, uint32_t* __restrict__ xb,
+                                                                 unsigned total, int H, int W, FastDiv dWp2, FastDiv dHp,
+                                                                 int halo) {
+  const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  uint32_t t, w2, plane, hp;
+  dWp2.divmod(i, t, w2);
+  dHp.divmod(t, plane, hp);
+  const int h = (int)hp - halo, w0 = 2 * (int)w2 - halo;
+  float lo = 0.0f, hi = 0.0f;
+  if ((unsigned)h < (unsigned)H) {
+    const float* row = x + ((size_t)plane * H + h) * W;
+    if ((unsigned)w0 < (unsigned)W) lo = row[w0];
+    if ((unsigned)(w0 + 1) < (unsigned)W) hi = row[w0 + 1];
+  }
+  xb[i] = pack_bf16(lo, hi);
+}
+
 template <class T, bool DMA = false>
 static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const float* x, const float* w, void* ws,
                                const EpiParams& ep, hipStream_t stream, const char* tag) {
@@ -311,13 +353,25 @@ static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const 
   uint4* wb = reinterpret_cast<uint4*>(base + bpn.tab_bytes);
   uint4* xb = reinterpret_cast<uint4*>(base + bpn.tab_bytes + bpn.wt_bytes);
   const int CRS = d.C * d.R * d.S, HpWp = bpn.Hp * bpn.Wp, Cg = d.C / 8;
+  const bool cols = bpn.s_groups > 0;
   {
     ProfScope prof("bf16_filter", 4.0 * (double)d.w_elems + 2.0 * (double)bpn.n_k * d.K, stream);
-    hipLaunchKernelGGL(prep_bf16_filter_kernel, dim3(cdiv((long long)(bpn.n_k / 8) * d.K, 256ll)), dim3(256), 0, stream, w, wb,
-                       soff8, bpn.n_k, CRS, d.K, d.C, d.R * d.S, d.S, bpn.Wp);
+    const dim3 grid((unsigned)cdiv((long long)(bpn.n_k / 8) * d.K, 256ll));
+    if (cols)
+      hipLaunchKernelGGL(prep_bf16_filter_cols_kernel, grid, dim3(256), 0, stream, w, wb, soff8, bpn.n_k,
+                         d.C * d.R * bpn.s_groups, d.K, CRS, d.R, d.S, bpn.s_groups, bpn.Hp, bpn.Wp);
+    else
+      hipLaunchKernelGGL(prep_bf16_filter_kernel, grid, dim3(256), 0, stream, w, wb, soff8, bpn.n_k, CRS, d.K, d.C,
+                         d.R * d.S, d.S, bpn.Wp);
   }
   if (int e = launch_status()) return e;
-  {
+  if (cols) {
+    const size_t pairs = (size_t)d.N * d.C * HpWp / 2;  // below 2^30: the copy is at most 2 GiB
+    ProfScope prof("nchw_to_bf16_planes", 4.0 * (double)d.x_elems + 4.0 * (double)pairs, stream);
+    hipLaunchKernelGGL(nchw_to_bf16_planes_kernel, dim3(stream_grid(pairs, 256)), dim3(256), 0, stream, x,
+                       reinterpret_cast<uint32_t*>(xb), (unsigned)pairs, d.H, d.W, FastDiv((uint32_t)(bpn.Wp / 2)),
+                       FastDiv((uint32_t)bpn.Hp), d.pad);
+  } else {
     const size_t groups = (size_t)d.N * Cg * HpWp;  // below 2^28: the copy is at most 2 GiB
     ProfScope prof("nchw_to_bf16_groups", 4.0 * (double)d.x_elems + 16.0 * (double)groups, stream);
     hipLaunchKernelGGL(nchw_to_bf16_groups_kernel, dim3(stream_grid(groups, 256)), dim3(256), 0, stream, x, xb, (unsigned)groups,
@@ -331,7 +385,13 @@ static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const 
   RowV8Params bp;  // image copy, rows = output pixels (n, p, q)
   bp.ptr = xb; bp.bytes = (uint32_t)(2 * (size_t)d.N * d.C * HpWp);
   bp.M = d.N * d.P * d.Q; bp.inner = d.P * d.Q; bp.innerW = d.Q;
-  bp.img_stride = HpWp * d.C * 2; bp.a_stride = d.st * Cg * bpn.Wp * 16; bp.b_stride = d.st * 16; bp.soff = soff8;
+  bp.img_stride = HpWp * d.C * 2;
+  if (cols) {
+    bp.a_stride = d.st * bpn.Wp * 2; bp.b_stride = d.st * 2;
+  } else {
+    bp.a_stride = d.st * Cg * bpn.Wp * 16; bp.b_stride = d.st * 16;
+  }
+  bp.soff = soff8;
   bp.group_stride = 0;
   typedef LoadRowV8<T::BM, T::BK, T::NT, true> AL;
   typedef LoadRowV8<T::BN, T::BK, T::NT, false> BL;
