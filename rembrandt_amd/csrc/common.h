@@ -41,7 +41,7 @@ inline int stream_grid(size_t work_items, int block) {
 // more instructions than everything else in the kernel.
 struct FastDiv {
   uint32_t mul, shift, div;
-  FastDiv() : mul(1), shift(0), div(1) {}
+  __host__ __device__ FastDiv() : mul(1), shift(0), div(1) {}
   explicit FastDiv(uint32_t d) : div(d) {
     uint32_t l = 0;
     while ((1ull << l) < d) ++l;

@@ -488,7 +488,11 @@ template <class T>
 static int run_bwd_filter(const PixDyParams& ap, const PixXParams& bp, const EpiParams& ep, int M,
                           int splits, int* used, hipStream_t stream, const char* tag) {
   typedef LoadPixDy<T::BM, T::BK, T::NT> AL;
-  typedef LoadPixX<T::BN, T::BK, T::NT> BL;
+  if (bp.pad == 0) {
+    typedef LoadPixX<T::BN, T::BK, T::NT, true> BL;
+    return launch_mfma_gemm<T, AL, BL, false, PassConvBwdFilter>(ap, bp, ep, M, splits, used, stream, tag);
+  }
+  typedef LoadPixX<T::BN, T::BK, T::NT, false> BL;
   return launch_mfma_gemm<T, AL, BL, false, PassConvBwdFilter>(ap, bp, ep, M, splits, used, stream, tag);
 }
 
@@ -787,10 +791,10 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
   int4* tab = static_cast<int4*>(ws);
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + plan.tab_bytes);
   PixDyParams ap;
-  ap.ptr = dy; ap.bytes = (uint32_t)(d.y_elems * 4); ap.rows = d.K; ap.M = M; ap.PQ = d.P * d.Q;
+  ap.ptr = dy; ap.bytes = (uint32_t)(d.y_elems * 4); ap.rows = d.K; ap.M = M; ap.set_pq(d.P * d.Q);
   if (d.R == 1 && d.S == 1 && d.st == 1 && d.pad == 0 && M > 0) {
     PixDyParams xp;
-    xp.ptr = x; xp.bytes = (uint32_t)(d.x_elems * 4); xp.rows = d.C; xp.M = M; xp.PQ = d.P * d.Q;
+    xp.ptr = x; xp.bytes = (uint32_t)(d.x_elems * 4); xp.rows = d.C; xp.M = M; xp.set_pq(d.P * d.Q);
     EpiParams ep;
     ep.out = part; ep.bias = nullptr; ep.alpha = 1.0f; ep.beta = 0.0f;
     ep.rows = d.K; ep.cols = CRS; ep.inner = 0; ep.ld = CRS; ep.relu = 0;
@@ -813,7 +817,7 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
   if (int e = launch_status()) return e;
 
   PixXParams bp;
-  bp.ptr = x; bp.bytes = (uint32_t)(d.x_elems * 4); bp.rows = CRS; bp.M = M; bp.PQ = d.P * d.Q; bp.Q = d.Q;
+  bp.ptr = x; bp.bytes = (uint32_t)(d.x_elems * 4); bp.rows = CRS; bp.M = M; bp.set_pq(d.P * d.Q, d.Q);
   bp.img_stride = d.C * d.H * d.W; bp.H = d.H; bp.W = d.W; bp.st = d.st; bp.pad = d.pad; bp.rtab = tab;
   EpiParams ep;
   ep.out = part; ep.bias = nullptr; ep.alpha = 1.0f; ep.beta = 0.0f;

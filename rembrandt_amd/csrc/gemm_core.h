@@ -25,6 +25,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // Element offset whose byte offset (x4) is 0x80000000: beyond every accepted tensor, so a
 // buffer load from it returns 0.  Sums of offsets are clamped to it before the shift.
 constexpr uint32_t kInvalidOff = 0x20000000u;
+constexpr uint32_t kInvalidByteOff = 0x80000000u;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
@@ -480,6 +481,8 @@ struct PixDyParams {
   int rows;  // Kout
   int M;     // N*P*Q
   int PQ;
+  FastDiv dPQ;  // division by PQ (set_pq): the loaders split a pixel index every K step
+  void set_pq(int pq) { PQ = pq; dPQ = FastDiv((uint32_t)(pq > 0 ? pq : 1)); }
 };
 
 template <int ROWS, int BK, int NT>
@@ -491,32 +494,39 @@ struct LoadPixDy {
   typedef float Reg;
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t rowoff[CNT];
-  int kk, M, PQ, img, sbase;
+  int kk, M, img, sbase;
+  FastDiv dPQ;
 
   __device__ __forceinline__ void init(const Params& p, int row0, int tid) {
     rsrc = make_rsrc(p.ptr, p.bytes);
     kk = tid % BK;
     const int r = tid / BK;
     M = p.M;
-    PQ = p.PQ;
+    dPQ = p.dPQ;
     img = p.rows * p.PQ;
     sbase = kk * LD + r;
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
       const int row = row0 + r + i * RSTEP;
-      rowoff[i] = row < p.rows ? (uint32_t)row * (uint32_t)p.PQ : kInvalidOff;
+      rowoff[i] = row < p.rows ? ((uint32_t)row * (uint32_t)p.PQ) << 2 : kInvalidByteOff;
     }
   }
+  // Byte offsets; an absent row or pixel carries 0x80000000, so the sum of a present and an absent part lies past
+  // every accepted tensor (the load returns 0) without a clamp.  (Both absent: the sum wraps to a small offset and
+  // the load returns some element, into a product of an absent row and an absent pixel, which is never stored.)
   uint32_t kbase;
   __device__ __forceinline__ void prep(int k0) {
     const int pix = k0 + kk;
-    kbase = kInvalidOff;
+    kbase = kInvalidByteOff;
     if (pix < M) {
-      const int n = pix / PQ;
-      kbase = (uint32_t)(n * img + (pix - n * PQ));
+      uint32_t n, pq;
+      dPQ.divmod((uint32_t)pix, n, pq);
+      kbase = (n * (uint32_t)img + pq) << 2;
     }
   }
-  __device__ __forceinline__ float load_one(int i) const { return buf_load_f32(rsrc, rowoff[i] + kbase); }
+  __device__ __forceinline__ float load_one(int i) const {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(rowoff[i] + kbase), 0, 0));
+  }
   __device__ __forceinline__ void store(float* s, const float (&v)[CNT]) {
 #pragma unroll
     for (int i = 0; i < CNT; ++i) s[sbase + i * RSTEP] = v[i];
@@ -530,9 +540,18 @@ struct PixXParams {
   int img_stride;  // C*H*W
   int H, W, st, pad;
   const int4* rtab;  // per (c,r,s): {c*H*W + r*W + s, r, s, 0}
+  FastDiv dPQ, dQ;   // divisions by PQ and Q (set_pq)
+  void set_pq(int pq, int q) {
+    PQ = pq; Q = q;
+    dPQ = FastDiv((uint32_t)(pq > 0 ? pq : 1));
+    dQ = FastDiv((uint32_t)(q > 0 ? q : 1));
+  }
 };
 
-template <int ROWS, int BK, int NT>
+// NOPAD: no padding, so every tap of every output pixel lies inside the image and the bounds checks fall away
+// (three vector instructions per element instead of nine; the loader's arithmetic shares the issue port with the
+// MFMAs: AlexNet conv1's filter gradient ran nine vector instructions per MFMA with the checks and runtime divisions).
+template <int ROWS, int BK, int NT, bool NOPAD = false>
 struct LoadPixX {
   static constexpr int CNT = ROWS * BK / NT, RSTEP = NT / BK;
   static constexpr int LD = ROWS + lds_pad_kfast<BK>();
@@ -541,13 +560,14 @@ struct LoadPixX {
   typedef float Reg;
   __amdgpu_buffer_rsrc_t rsrc;
   int roff[CNT], rr[CNT], rs[CNT];
-  int kk, M, PQ, Q, img, H, W, st, pad, sbase;
+  int kk, M, img, H, W, st, pad, sbase;
+  FastDiv dPQ, dQ;
 
   __device__ __forceinline__ void init(const Params& p, int row0, int tid) {
     rsrc = make_rsrc(p.ptr, p.bytes);
     kk = tid % BK;
     const int r = tid / BK;
-    M = p.M; PQ = p.PQ; Q = p.Q; img = p.img_stride; H = p.H; W = p.W; st = p.st; pad = p.pad;
+    M = p.M; dPQ = p.dPQ; dQ = p.dQ; img = p.img_stride; H = p.H; W = p.W; st = p.st; pad = p.pad;
     sbase = kk * LD + r;
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
@@ -556,25 +576,28 @@ struct LoadPixX {
         const int4 e = p.rtab[row];
         roff[i] = e.x; rr[i] = e.y; rs[i] = e.z;
       } else {
-        roff[i] = 0; rr[i] = -(1 << 28); rs[i] = 0;
+        roff[i] = NOPAD ? (int)kInvalidByteOff : 0; rr[i] = -(1 << 28); rs[i] = 0;
       }
+      if (NOPAD && row < p.rows) roff[i] <<= 2;  // byte offsets, as in LoadPixDy
     }
   }
   int h0, w0, base;
   __device__ __forceinline__ void prep(int k0) {
     const int pix = k0 + kk;
-    h0 = -(1 << 28); w0 = 0; base = 0;
+    h0 = -(1 << 28); w0 = 0; base = NOPAD ? (int)kInvalidByteOff : 0;
     if (pix < M) {
-      const int n = pix / PQ;
-      const int pq = pix - n * PQ;
-      const int p = pq / Q;
-      const int q = pq - p * Q;
-      h0 = p * st - pad;
-      w0 = q * st - pad;
-      base = n * img + h0 * W + w0;
+      uint32_t n, pq, p, q;
+      dPQ.divmod((uint32_t)pix, n, pq);
+      dQ.divmod(pq, p, q);
+      h0 = (int)p * st - pad;
+      w0 = (int)q * st - pad;
+      base = (int)n * img + h0 * W + w0;
+      if (NOPAD) base <<= 2;
     }
   }
   __device__ __forceinline__ float load_one(int i) const {
+    if (NOPAD)
+      return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)((uint32_t)base + (uint32_t)roff[i]), 0, 0));
     const int ok = (int)((unsigned)(h0 + rr[i]) < (unsigned)H) & (int)((unsigned)(w0 + rs[i]) < (unsigned)W);
     return buf_load_f32(rsrc, ok ? (uint32_t)(base + roff[i]) : kInvalidOff);
   }
