@@ -34,14 +34,24 @@ __global__ __launch_bounds__(256) void pad_image_kernel(const float* __restrict_
   dWp.divmod(i0, t, wp);
   dHp.divmod(t, plane, hp);
   float v[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
+  {
     const int h = (int)hp - halo, w = (int)wp - halo;
-    v[e] = ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W && i0 + e < total)
-               ? src[((size_t)plane * H + h) * W + w] : 0.0f;
-    if (++wp == dWp.div) {
-      wp = 0;
-      if (++hp == dHp.div) { hp = 0; ++plane; }
+    if ((unsigned)h < (unsigned)H && w >= 0 && w + 3 < W) {
+      // all four inside one source row: one 16-byte load (4-byte aligned: source rows start anywhere)
+      typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+      const f4u q = *reinterpret_cast<const f4u*>(src + ((size_t)plane * H + h) * W + w);
+      v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int he = (int)hp - halo, we = (int)wp - halo;
+        v[e] = ((unsigned)he < (unsigned)H && (unsigned)we < (unsigned)W && i0 + e < total)
+                   ? src[((size_t)plane * H + he) * W + we] : 0.0f;
+        if (++wp == dWp.div) {
+          wp = 0;
+          if (++hp == dHp.div) { hp = 0; ++plane; }
+        }
+      }
     }
   }
   if (vec && i0 + 3 < total) {
