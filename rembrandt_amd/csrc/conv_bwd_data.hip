@@ -21,26 +21,6 @@ __global__ void build_bwd_data_tab_kernel(int4* tab, int* atab, int n_entries, i
   }
 }
 
-// Scalar-offset path (stride 1): wT[k][c] = w[ko][c][r][s] for k = (ko,r,s) (zero rows past the end) and
-// the k -> byte offset table into the padded dy, soff[k] = 4*(ko*Pp*Qp + (R-1-r)*Qp + (S-1-s)).
-__global__ void prep_bwd_data_soff_kernel(const float* __restrict__ w, float* __restrict__ wT, int* __restrict__ soff,
-                                          int n_k, int KRS, int C, int R, int S, int PpQp, int Qp) {
-  const long long total = (long long)n_k * C;
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int k = (int)(i / C), c = (int)(i - (long long)k * C);
-    float v = 0.0f;
-    int off = 0;
-    if (k < KRS) {
-      const int ko = k / (R * S), rs = k - ko * (R * S), r = rs / S, s2 = rs - r * S;
-      v = w[((size_t)ko * C + c) * (R * S) + rs];
-      off = (ko * PpQp + (R - 1 - r) * Qp + (S - 1 - s2)) * 4;
-    }
-    wT[i] = v;
-    if (c == 0) soff[k] = off;
-  }
-}
-
 // One residue class of the strided form: wT[k][c] = w[ko][c][a + st*i][b + st*j] for k = (ko, i, j) (zero rows past
 // the end) and soff[k] = 4*(ko*Hp*Wp + (Ra-1-i)*Wp + (Sb-1-j)) into the padded dy.
 __global__ void prep_bwd_data_phase_kernel(const float* __restrict__ w, float* __restrict__ wT, int* __restrict__ soff,
@@ -256,14 +236,20 @@ static int bwd_data_impl(const rh_conv_geom* g, float alpha, const float* w, con
     int* soff = static_cast<int*>(ws);
     float* wT = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes);
     const float* img = dy;
-    if (sp.img_bytes) {
+    if (sp.img_bytes && d.st == 1) {
       float* dyp = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes);
-      launch_pad_image(dy, dyp, (long long)d.N * d.K, d.P, d.Q, sp.Hp, sp.Wp, sp.halo, stream, d.st);
-      if (int e = launch_status()) return e;
+      launch_pad_image_prep_soff(dy, dyp, (long long)d.N * d.K, d.P, d.Q, sp.Hp, sp.Wp, sp.halo, w, wT, soff, sp.n_k, KRS, d.C,
+                                 d.R, d.S, 1, stream);
       img = dyp;
+    } else {
+      if (sp.img_bytes) {
+        float* dyp = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes);
+        launch_pad_image(dy, dyp, (long long)d.N * d.K, d.P, d.Q, sp.Hp, sp.Wp, sp.halo, stream, d.st);
+        if (int e = launch_status()) return e;
+        img = dyp;
+      }
+      launch_prep_soff(w, wT, soff, sp.n_k, KRS, d.C, d.R, d.S, sp.Hp * sp.Wp, sp.Wp, 1, stream);
     }
-    hipLaunchKernelGGL(prep_bwd_data_soff_kernel, dim3(stream_grid((size_t)sp.n_k * d.C, 256)), dim3(256), 0, stream, w,
-                       wT, soff, sp.n_k, KRS, d.C, d.R, d.S, sp.Hp * sp.Wp, sp.Wp);
     if (int e = launch_status()) return e;
     RowSParams ap;  // transposed filter [k][c]
     ap.ptr = wT; ap.bytes = (uint32_t)(sizeof(float) * (size_t)sp.n_k * d.C);

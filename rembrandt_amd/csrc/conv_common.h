@@ -416,6 +416,15 @@ int launch_conv1x1_stream(const ConvDims& d, int pass, const float* w, const flo
 void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
                       hipStream_t stream, int dil = 1);
 
+// Filter-side scratch of the scalar-offset paths: wT[k][row] and the byte-offset table soff[k] into the padded copy
+// (bwd = 0: forward, k = (c,r,s), rows = output channels; bwd = 1: stride-1 backward-data, k = (ko,r,s) with the
+// filter flipped, rows = input channels), alone or in one launch with the padded copy of the image (no dilation).
+void launch_prep_soff(const float* w, float* wT, int* soff, int n_k, int k_true, int rows, int R, int S, int HpWp, int Wp,
+                      int bwd, hipStream_t stream);
+void launch_pad_image_prep_soff(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
+                                const float* w, float* wT, int* soff, int n_k, int k_true, int rows, int R, int S, int bwd,
+                                hipStream_t stream);
+
 void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int HW, int W,
                           hipStream_t stream);
 

@@ -25,9 +25,9 @@ void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int H
 // dst (planes x Hp x Wp) = src (planes x H x W) surrounded by `halo` zeros.  A thread produces four consecutive
 // elements of dst (they may straddle a row or a plane) and writes them as one 16-byte store when dst is aligned:
 // stores of 16 bytes per lane over one sweep of consecutive blocks are what this GPU's memory system wants.
-__global__ __launch_bounds__(256) void pad_image_kernel(const float* __restrict__ src, float* __restrict__ dst, unsigned total,
-                                                        int H, int W, FastDiv dHp, FastDiv dWp, int halo, int vec) {
-  const unsigned g = blockIdx.x * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void pad_image_body(unsigned block, const float* __restrict__ src, float* __restrict__ dst,
+                                               unsigned total, int H, int W, FastDiv dHp, FastDiv dWp, int halo, int vec) {
+  const unsigned g = block * blockDim.x + threadIdx.x;
   const unsigned i0 = g * 4u;
   if (i0 >= total) return;
   uint32_t t, wp, plane, hp;
@@ -60,6 +60,60 @@ __global__ __launch_bounds__(256) void pad_image_kernel(const float* __restrict_
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       if (i0 + e < total) dst[i0 + e] = v[e];
+  }
+}
+
+__global__ __launch_bounds__(256) void pad_image_kernel(const float* __restrict__ src, float* __restrict__ dst, unsigned total,
+                                                        int H, int W, FastDiv dHp, FastDiv dWp, int halo, int vec) {
+  pad_image_body(blockIdx.x, src, dst, total, H, W, dHp, dWp, halo, vec);
+}
+
+// The filter-side scratch of the scalar-offset forward and stride-1 backward-data paths, as a function of a virtual
+// grid (first element, stride) so that it can share a launch with the image copy:
+//   forward:       wT[k][ko] = w[ko][k] for k = (c,r,s)  (zero rows for k >= CRS), soff[k] = 4*(c*HpWp + r*Wp + s);
+//   backward-data: wT[k][c] = w[ko][c][r][s] for k = (ko,r,s), soff[k] = 4*(ko*HpWp + (R-1-r)*Wp + (S-1-s));
+// soff is 0 past the end of the contraction.
+struct PrepSoffArgs {
+  const float* w; float* wT; int* soff;
+  int n_k, k_true, rows, R, S, HpWp, Wp, bwd;
+};
+
+__device__ __forceinline__ void prep_soff_body(const PrepSoffArgs& a, long long first, long long stride) {
+  const long long total = (long long)a.n_k * a.rows;
+  const int RS = a.R * a.S;
+  for (long long i = first; i < total; i += stride) {
+    const int k = (int)(i / a.rows), row = (int)(i - (long long)k * a.rows);
+    float v = 0.0f;
+    int off = 0;
+    if (k < a.k_true) {
+      const int c = k / RS, rs = k - c * RS, r = rs / a.S, s2 = rs - r * a.S;
+      if (a.bwd) {
+        v = a.w[((size_t)c * a.rows + row) * RS + rs];
+        off = (c * a.HpWp + (a.R - 1 - r) * a.Wp + (a.S - 1 - s2)) * 4;
+      } else {
+        v = a.w[(size_t)row * a.k_true + k];
+        off = (c * a.HpWp + r * a.Wp + s2) * 4;
+      }
+    }
+    a.wT[i] = v;
+    if (row == 0) a.soff[k] = off;
+  }
+}
+
+__global__ __launch_bounds__(256) void prep_soff_kernel(PrepSoffArgs a) {
+  prep_soff_body(a, (long long)blockIdx.x * blockDim.x + threadIdx.x, (long long)gridDim.x * blockDim.x);
+}
+
+// Both in one launch: the first pad_blocks blocks copy the image, the others prepare the filter side.  The two are
+// independent, and a launch less in front of a contraction is a launch gap less on the chain of a small layer.
+__global__ __launch_bounds__(256) void pad_image_prep_soff_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                                  unsigned total, int H, int W, FastDiv dHp, FastDiv dWp,
+                                                                  int halo, int vec, unsigned pad_blocks, PrepSoffArgs a) {
+  if (blockIdx.x < pad_blocks) {
+    pad_image_body(blockIdx.x, src, dst, total, H, W, dHp, dWp, halo, vec);
+  } else {
+    const unsigned b = blockIdx.x - pad_blocks, nb = gridDim.x - pad_blocks;
+    prep_soff_body(a, (long long)b * blockDim.x + threadIdx.x, (long long)nb * blockDim.x);
   }
 }
 
@@ -98,24 +152,31 @@ void launch_pad_image(const float* src, float* dst, long long planes, int H, int
                      (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, vec);
 }
 
-// Forward scratch preparation: wT[k][ko] = w[ko][k] (zero rows for k >= CRS) and the k -> byte offset
-// table into the padded image, soff[k] = 4*(c*Hp*Wp + r*Wp + s) (0 past the end).
-__global__ void prep_fwd_soff_kernel(const float* __restrict__ w, float* __restrict__ wT, int* __restrict__ soff,
-                                     int n_k, int CRS, int K, int R, int S, int HpWp, int Wp) {
-  const long long total = (long long)n_k * K;
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int k = (int)(i / K), ko = (int)(i - (long long)k * K);
-    wT[i] = k < CRS ? w[(size_t)ko * CRS + k] : 0.0f;
-    if (ko == 0) {
-      int off = 0;
-      if (k < CRS) {
-        const int c = k / (R * S), rs = k - c * (R * S), r = rs / S, s2 = rs - r * S;
-        off = (c * HpWp + r * Wp + s2) * 4;
-      }
-      soff[k] = off;
-    }
-  }
+static PrepSoffArgs prep_args(const float* w, float* wT, int* soff, int n_k, int k_true, int rows, int R, int S, int HpWp,
+                              int Wp, int bwd) {
+  PrepSoffArgs a;
+  a.w = w; a.wT = wT; a.soff = soff; a.n_k = n_k; a.k_true = k_true; a.rows = rows; a.R = R; a.S = S; a.HpWp = HpWp; a.Wp = Wp;
+  a.bwd = bwd;
+  return a;
+}
+
+void launch_prep_soff(const float* w, float* wT, int* soff, int n_k, int k_true, int rows, int R, int S, int HpWp, int Wp,
+                      int bwd, hipStream_t stream) {
+  const PrepSoffArgs a = prep_args(w, wT, soff, n_k, k_true, rows, R, S, HpWp, Wp, bwd);
+  hipLaunchKernelGGL(prep_soff_kernel, dim3(stream_grid((size_t)n_k * rows, 256)), dim3(256), 0, stream, a);
+}
+
+void launch_pad_image_prep_soff(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
+                                const float* w, float* wT, int* soff, int n_k, int k_true, int rows, int R, int S, int bwd,
+                                hipStream_t stream) {
+  const long long total = planes * Hp * Wp;
+  const PrepSoffArgs a = prep_args(w, wT, soff, n_k, k_true, rows, R, S, Hp * Wp, Wp, bwd);
+  ProfScope prof("pad_image", 4.0 * ((double)planes * H * W + (double)total) + 4.0 * 2.0 * (double)n_k * rows, stream);
+  const int vec = (reinterpret_cast<uintptr_t>(dst) & 15) == 0 ? 1 : 0;
+  const unsigned pad_blocks = (unsigned)stream_grid((size_t)(total + 3) / 4, 256);
+  const unsigned prep_blocks = (unsigned)stream_grid((size_t)n_k * rows, 256);
+  hipLaunchKernelGGL(pad_image_prep_soff_kernel, dim3(pad_blocks + prep_blocks), dim3(256), 0, stream, src, dst, (unsigned)total,
+                     H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, vec, pad_blocks, a);
 }
 
 // VEC: four consecutive elements per thread through 16-byte loads and stores (slab stride, first element and all
@@ -466,12 +527,12 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
     const float* img = x;
     if (sp.img_bytes) {
       float* xp = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes);
-      launch_pad_image(x, xp, (long long)d.N * d.C, d.H, d.W, sp.Hp, sp.Wp, sp.halo, stream);
-      if (int e = launch_status()) return e;
+      launch_pad_image_prep_soff(x, xp, (long long)d.N * d.C, d.H, d.W, sp.Hp, sp.Wp, sp.halo, w, wT, soff, sp.n_k, CRS, d.K,
+                                 d.R, d.S, 0, stream);
       img = xp;
+    } else {
+      launch_prep_soff(w, wT, soff, sp.n_k, CRS, d.K, d.R, d.S, sp.Hp * sp.Wp, sp.Wp, 0, stream);
     }
-    hipLaunchKernelGGL(prep_fwd_soff_kernel, dim3(stream_grid((size_t)sp.n_k * d.K, 256)), dim3(256), 0, stream, w, wT,
-                       soff, sp.n_k, CRS, d.K, d.R, d.S, sp.Hp * sp.Wp, sp.Wp);
     if (int e = launch_status()) return e;
     RowSParams ap;  // transposed filter [k][ko]
     ap.ptr = wT; ap.bytes = (uint32_t)(sizeof(float) * (size_t)sp.n_k * d.K + kRow4Slack);
