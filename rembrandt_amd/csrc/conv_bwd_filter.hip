@@ -316,15 +316,17 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const float* __restri
 // bwd_bias_rows_kernel's.  Fixed order: the same call gives the same bits.
 typedef float float4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
+// (bx, by, bz) of a grid (gx, ., .): the block's place, given by the caller so that the body can also run as one
+// range of blocks of a larger launch; `tile` is the block's 16 KB of LDS.
 template <bool BIAS>
-__global__ __launch_bounds__(256) void nchw_to_nhwc_vec_kernel(const float* __restrict__ src, float* __restrict__ dst,
-                                                               int C, int H, int W, int Hp, int Wp, int halo,
-                                                               float* __restrict__ bias_part) {
-  __shared__ __attribute__((aligned(16))) float tile[64 * 64];
-  const int c0 = blockIdx.y * 64, n = blockIdx.z;
+__device__ __forceinline__ void nchw_to_nhwc_vec_body(float* __restrict__ tile, int bx, int by, int bz, int gx,
+                                                      const float* __restrict__ src, float* __restrict__ dst,
+                                                      int C, int H, int W, int Hp, int Wp, int halo,
+                                                      float* __restrict__ bias_part) {
+  const int c0 = by * 64, n = bz;
   const int HpWp = Hp * Wp;
   float bsum = 0.0f;
-  for (int pix0 = blockIdx.x * 64; pix0 < HpWp; pix0 += gridDim.x * 64) {
+  for (int pix0 = bx * 64; pix0 < HpWp; pix0 += gx * 64) {
   {
     const int pq = threadIdx.x & 15, cl0 = threadIdx.x >> 4;
     const int pix = pix0 + 4 * pq;
@@ -388,6 +390,14 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_vec_kernel(const float* __re
   }
 }
 
+template <bool BIAS>
+__global__ __launch_bounds__(256) void nchw_to_nhwc_vec_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                               int C, int H, int W, int Hp, int Wp, int halo,
+                                                               float* __restrict__ bias_part) {
+  __shared__ __attribute__((aligned(16))) float tile[64 * 64];
+  nchw_to_nhwc_vec_body<BIAS>(tile, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.x, src, dst, C, H, W, Hp, Wp, halo, bias_part);
+}
+
 // The 16-byte form can carry the per-image plane sums along (bias_part, N x C floats; no halo).
 static bool nhwc_vec_ok(int C, const float* dst) { return C % 4 == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0; }
 
@@ -410,10 +420,19 @@ static void launch_nchw_to_nhwc(const float* src, float* dst, int N, int C, int 
 }
 
 // soff[pix] = 4*C*((n*Hp + p*st)*Wp + q*st) for pix = (n,p,q) < M, else 0; also zeroes the rows M..n_k of dyT.
+__device__ __forceinline__ void prep_bwd_filter_soff_body(int first, int stride, int* __restrict__ soff,
+                                                          float* __restrict__ dyT, int n_k, int M, int PQ, int Q, int st,
+                                                          int Hp, int Wp, int C, int Kout);
 __global__ void prep_bwd_filter_soff_kernel(int* __restrict__ soff, float* __restrict__ dyT, int n_k, int M, int PQ,
                                             int Q, int st, int Hp, int Wp, int C, int Kout) {
-  const int stride = gridDim.x * blockDim.x;
-  for (int pix = blockIdx.x * blockDim.x + threadIdx.x; pix < n_k; pix += stride) {
+  prep_bwd_filter_soff_body(blockIdx.x * blockDim.x + threadIdx.x, gridDim.x * blockDim.x, soff, dyT, n_k, M, PQ, Q, st, Hp, Wp,
+                            C, Kout);
+}
+
+__device__ __forceinline__ void prep_bwd_filter_soff_body(int first, int stride, int* __restrict__ soff,
+                                                          float* __restrict__ dyT, int n_k, int M, int PQ, int Q, int st,
+                                                          int Hp, int Wp, int C, int Kout) {
+  for (int pix = first; pix < n_k; pix += stride) {
     int off = 0;
     if (pix < M) {
       const int n = pix / PQ, pq = pix - n * PQ, p = pq / Q, q = pq - p * Q;
@@ -423,6 +442,39 @@ __global__ void prep_bwd_filter_soff_kernel(int* __restrict__ soff, float* __res
     }
     soff[pix] = off;
   }
+}
+
+// The three operand preparations of the scalar-offset backward-filter in one launch (they are independent of one
+// another): blocks [0, nb_dy) copy dy channel-last (BIAS: with the plane sums), the next nb_x blocks copy x channel-last
+// with its zero border, the rest write the offset table and zero dyT's tail rows.
+struct NhwcCopyArgs {
+  const float* src; float* dst;
+  int C, H, W, Hp, Wp, halo;
+  int gx, gy;   // grid of 64-pixel x 64-channel pieces: (gx, gy, images)
+};
+
+template <bool BIAS>
+__global__ __launch_bounds__(256) void bwd_filter_prep_kernel(NhwcCopyArgs dy, float* __restrict__ bias_part, int nb_dy,
+                                                              NhwcCopyArgs x, int nb_x, int* __restrict__ soff, int n_k, int M,
+                                                              int PQ, int Q, int st, int Kout) {
+  __shared__ __attribute__((aligned(16))) float tile[64 * 64];
+  int b = blockIdx.x;
+  if (b < nb_dy) {
+    const int bx = b % dy.gx, t = b / dy.gx;
+    nchw_to_nhwc_vec_body<BIAS>(tile, bx, t % dy.gy, t / dy.gy, dy.gx, dy.src, dy.dst, dy.C, dy.H, dy.W, dy.Hp, dy.Wp, dy.halo,
+                                bias_part);
+    return;
+  }
+  b -= nb_dy;
+  if (b < nb_x) {
+    const int bx = b % x.gx, t = b / x.gx;
+    nchw_to_nhwc_vec_body<false>(tile, bx, t % x.gy, t / x.gy, x.gx, x.src, x.dst, x.C, x.H, x.W, x.Hp, x.Wp, x.halo, nullptr);
+    return;
+  }
+  b -= nb_x;
+  const int nb = (int)gridDim.x - nb_dy - nb_x;
+  prep_bwd_filter_soff_body(b * (int)blockDim.x + (int)threadIdx.x, nb * (int)blockDim.x, soff, dy.dst, n_k, M, PQ, Q, st, x.Hp,
+                            x.Wp, x.C, Kout);
 }
 
 // dw[ko][c][r][s] = alpha * sum_s part[s][ko][(r,s,c)] + beta * dw
@@ -742,15 +794,36 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     float* dyT = reinterpret_cast<float*>(base + sp.tab_bytes);
     float* xT = reinterpret_cast<float*>(base + sp.tab_bytes + sp.dyt_bytes);
     float* parts = reinterpret_cast<float*>(base + sp.tab_bytes + sp.dyt_bytes + sp.xt_bytes);
-    hipLaunchKernelGGL(prep_bwd_filter_soff_kernel, dim3(cdiv(sp.n_k, 256)), dim3(256), 0, stream, soff, dyT, sp.n_k, Ms,
-                       d.P * d.Q, d.Q, d.st, sp.Hp, sp.Wp, d.C, d.K);
-    if (int e = launch_status()) return e;
     float* const bpart = (bias_part && nhwc_vec_ok(d.K, dyT)) ? bias_part : nullptr;
-    launch_nchw_to_nhwc(dy, dyT, d.N, d.K, d.P, d.Q, d.P, d.Q, 0, stream, bpart);
-    if (int e = launch_status()) return e;
+    if (nhwc_vec_ok(d.K, dyT) && nhwc_vec_ok(d.C, xT)) {
+      // both copies take the 16-byte form: they and the table share one launch
+      NhwcCopyArgs a, b;
+      a.src = dy; a.dst = dyT; a.C = d.K; a.H = d.P; a.W = d.Q; a.Hp = d.P; a.Wp = d.Q; a.halo = 0;
+      a.gx = bpart ? 1 : cdiv(d.P * d.Q, 64); a.gy = cdiv(d.K, 64);
+      b.src = x; b.dst = xT; b.C = d.C; b.H = d.H; b.W = d.W; b.Hp = sp.Hp; b.Wp = sp.Wp; b.halo = d.pad;
+      b.gx = cdiv(sp.Hp * sp.Wp, 64); b.gy = cdiv(d.C, 64);
+      const long long nb_dy = (long long)a.gx * a.gy * d.N, nb_x = (long long)b.gx * b.gy * d.N;
+      const long long nb_tab = cdiv(sp.n_k, 256);
+      if (nb_dy + nb_x + nb_tab >= (1ll << 31)) return RH_E_LIMIT;
+      ProfScope prof("nchw_to_nhwc", 8.0 * ((double)d.N * d.K * d.P * d.Q) +
+                                         4.0 * ((double)d.N * d.C * d.H * d.W + (double)d.N * d.C * sp.Hp * sp.Wp), stream);
+      if (bpart)
+        hipLaunchKernelGGL(bwd_filter_prep_kernel<true>, dim3((unsigned)(nb_dy + nb_x + nb_tab)), dim3(256), 0, stream, a, bpart,
+                           (int)nb_dy, b, (int)nb_x, soff, sp.n_k, Ms, d.P * d.Q, d.Q, d.st, d.K);
+      else
+        hipLaunchKernelGGL(bwd_filter_prep_kernel<false>, dim3((unsigned)(nb_dy + nb_x + nb_tab)), dim3(256), 0, stream, a,
+                           (float*)nullptr, (int)nb_dy, b, (int)nb_x, soff, sp.n_k, Ms, d.P * d.Q, d.Q, d.st, d.K);
+      if (int e = launch_status()) return e;
+    } else {
+      hipLaunchKernelGGL(prep_bwd_filter_soff_kernel, dim3(cdiv(sp.n_k, 256)), dim3(256), 0, stream, soff, dyT, sp.n_k, Ms,
+                         d.P * d.Q, d.Q, d.st, sp.Hp, sp.Wp, d.C, d.K);
+      if (int e = launch_status()) return e;
+      launch_nchw_to_nhwc(dy, dyT, d.N, d.K, d.P, d.Q, d.P, d.Q, 0, stream, bpart);
+      if (int e = launch_status()) return e;
+      launch_nchw_to_nhwc(x, xT, d.N, d.C, d.H, d.W, sp.Hp, sp.Wp, d.pad, stream);
+      if (int e = launch_status()) return e;
+    }
     if (bpart) *folded = true;
-    launch_nchw_to_nhwc(x, xT, d.N, d.C, d.H, d.W, sp.Hp, sp.Wp, d.pad, stream);
-    if (int e = launch_status()) return e;
     RowSParams ap;  // dyT [pix][ko]
     ap.ptr = dyT; ap.bytes = (uint32_t)(sizeof(float) * (size_t)sp.n_k * d.K);
     ap.M = d.K; ap.inner = d.K; ap.innerW = d.K; ap.img_stride = 0; ap.a_stride = 0; ap.b_stride = 1;
