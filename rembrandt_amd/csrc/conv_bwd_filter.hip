@@ -279,11 +279,12 @@ static BwdFilterSoffPlan plan_bwd_filter_soff(const ConvDims& d) {
 
 // dst[n][pix][c] (pix over Hp x Wp, zero halo) = src[n][c][h][w]: 32 x 32 tiles through LDS so that both
 // the reads (along w) and the writes (along c) are contiguous.
-__global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst,
-                                                           int C, int H, int W, int Hp, int Wp, int halo) {
-  __shared__ float tile[32][33];
+__device__ __forceinline__ void nchw_to_nhwc_body(float* __restrict__ lds, int bx, int by, int bz,
+                                                  const float* __restrict__ src, float* __restrict__ dst,
+                                                  int C, int H, int W, int Hp, int Wp, int halo) {
+  float (*tile)[33] = reinterpret_cast<float (*)[33]>(lds);
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-  const int pix0 = blockIdx.x * 32, c0 = blockIdx.y * 32, n = blockIdx.z;
+  const int pix0 = bx * 32, c0 = by * 32, n = bz;
   const int HpWp = Hp * Wp;
   {
     const int pix = pix0 + tx;
@@ -303,6 +304,12 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const float* __restri
     const int pix = pix0 + ty + j;
     if (pix < HpWp && c < C) dst[((size_t)n * HpWp + pix) * C + c] = tile[tx][ty + j];
   }
+}
+
+__global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                           int C, int H, int W, int Hp, int Wp, int halo) {
+  __shared__ float tile[32 * 33];
+  nchw_to_nhwc_body(tile, blockIdx.x, blockIdx.y, blockIdx.z, src, dst, C, H, W, Hp, Wp, halo);
 }
 
 // The same for C % 4 == 0 in 16-byte accesses (4-byte accesses top out near 3.8 TB/s on this GPU): a block moves
@@ -450,7 +457,8 @@ __device__ __forceinline__ void prep_bwd_filter_soff_body(int first, int stride,
 struct NhwcCopyArgs {
   const float* src; float* dst;
   int C, H, W, Hp, Wp, halo;
-  int gx, gy;   // grid of 64-pixel x 64-channel pieces: (gx, gy, images)
+  int vec;      // 16-byte form (64 x 64 pieces) or the element form (32 x 32 pieces)
+  int gx, gy;   // grid of pieces: (gx, gy, images)
 };
 
 template <bool BIAS>
@@ -461,14 +469,20 @@ __global__ __launch_bounds__(256) void bwd_filter_prep_kernel(NhwcCopyArgs dy, f
   int b = blockIdx.x;
   if (b < nb_dy) {
     const int bx = b % dy.gx, t = b / dy.gx;
-    nchw_to_nhwc_vec_body<BIAS>(tile, bx, t % dy.gy, t / dy.gy, dy.gx, dy.src, dy.dst, dy.C, dy.H, dy.W, dy.Hp, dy.Wp, dy.halo,
-                                bias_part);
+    if (BIAS || dy.vec)
+      nchw_to_nhwc_vec_body<BIAS>(tile, bx, t % dy.gy, t / dy.gy, dy.gx, dy.src, dy.dst, dy.C, dy.H, dy.W, dy.Hp, dy.Wp, dy.halo,
+                                  bias_part);
+    else
+      nchw_to_nhwc_body(tile, bx, t % dy.gy, t / dy.gy, dy.src, dy.dst, dy.C, dy.H, dy.W, dy.Hp, dy.Wp, dy.halo);
     return;
   }
   b -= nb_dy;
   if (b < nb_x) {
     const int bx = b % x.gx, t = b / x.gx;
-    nchw_to_nhwc_vec_body<false>(tile, bx, t % x.gy, t / x.gy, x.gx, x.src, x.dst, x.C, x.H, x.W, x.Hp, x.Wp, x.halo, nullptr);
+    if (x.vec)
+      nchw_to_nhwc_vec_body<false>(tile, bx, t % x.gy, t / x.gy, x.gx, x.src, x.dst, x.C, x.H, x.W, x.Hp, x.Wp, x.halo, nullptr);
+    else
+      nchw_to_nhwc_body(tile, bx, t % x.gy, t / x.gy, x.src, x.dst, x.C, x.H, x.W, x.Hp, x.Wp, x.halo);
     return;
   }
   b -= nb_x;
@@ -795,13 +809,15 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     float* xT = reinterpret_cast<float*>(base + sp.tab_bytes + sp.dyt_bytes);
     float* parts = reinterpret_cast<float*>(base + sp.tab_bytes + sp.dyt_bytes + sp.xt_bytes);
     float* const bpart = (bias_part && nhwc_vec_ok(d.K, dyT)) ? bias_part : nullptr;
-    if (nhwc_vec_ok(d.K, dyT) && nhwc_vec_ok(d.C, xT)) {
-      // both copies take the 16-byte form: they and the table share one launch
+    {
+      // the two channel-last copies and the table share one launch
       NhwcCopyArgs a, b;
       a.src = dy; a.dst = dyT; a.C = d.K; a.H = d.P; a.W = d.Q; a.Hp = d.P; a.Wp = d.Q; a.halo = 0;
-      a.gx = bpart ? 1 : cdiv(d.P * d.Q, 64); a.gy = cdiv(d.K, 64);
+      a.vec = nhwc_vec_ok(d.K, dyT) ? 1 : 0;
+      a.gx = bpart ? 1 : cdiv(d.P * d.Q, a.vec ? 64 : 32); a.gy = cdiv(d.K, a.vec ? 64 : 32);
       b.src = x; b.dst = xT; b.C = d.C; b.H = d.H; b.W = d.W; b.Hp = sp.Hp; b.Wp = sp.Wp; b.halo = d.pad;
-      b.gx = cdiv(sp.Hp * sp.Wp, 64); b.gy = cdiv(d.C, 64);
+      b.vec = nhwc_vec_ok(d.C, xT) ? 1 : 0;
+      b.gx = cdiv(sp.Hp * sp.Wp, b.vec ? 64 : 32); b.gy = cdiv(d.C, b.vec ? 64 : 32);
       const long long nb_dy = (long long)a.gx * a.gy * d.N, nb_x = (long long)b.gx * b.gy * d.N;
       const long long nb_tab = cdiv(sp.n_k, 256);
       if (nb_dy + nb_x + nb_tab >= (1ll << 31)) return RH_E_LIMIT;
@@ -813,14 +829,6 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
       else
         hipLaunchKernelGGL(bwd_filter_prep_kernel<false>, dim3((unsigned)(nb_dy + nb_x + nb_tab)), dim3(256), 0, stream, a,
                            (float*)nullptr, (int)nb_dy, b, (int)nb_x, soff, sp.n_k, Ms, d.P * d.Q, d.Q, d.st, d.K);
-      if (int e = launch_status()) return e;
-    } else {
-      hipLaunchKernelGGL(prep_bwd_filter_soff_kernel, dim3(cdiv(sp.n_k, 256)), dim3(256), 0, stream, soff, dyT, sp.n_k, Ms,
-                         d.P * d.Q, d.Q, d.st, sp.Hp, sp.Wp, d.C, d.K);
-      if (int e = launch_status()) return e;
-      launch_nchw_to_nhwc(dy, dyT, d.N, d.K, d.P, d.Q, d.P, d.Q, 0, stream, bpart);
-      if (int e = launch_status()) return e;
-      launch_nchw_to_nhwc(x, xT, d.N, d.C, d.H, d.W, sp.Hp, sp.Wp, d.pad, stream);
       if (int e = launch_status()) return e;
     }
     if (bpart) *folded = true;
@@ -861,7 +869,6 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
 
   const int CRS = d.C * d.R * d.S;
   const int M = d.N * d.P * d.Q;
-  int4* tab = static_cast<int4*>(ws);
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + plan.tab_bytes);
   PixDyParams ap;
   ap.ptr = dy; ap.bytes = (uint32_t)(d.y_elems * 4); ap.rows = d.K; ap.M = M; ap.set_pq(d.P * d.Q);
@@ -886,12 +893,10 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     launch_split_reduce(part, used, (long long)d.K * CRS, dw, d.K, CRS, CRS, alpha, beta, stream);
     return launch_status();
   }
-  launch_build_fwd_tab(tab, round_up(CRS, kTabPad), CRS, d.R, d.S, d.H * d.W, d.W, stream);
-  if (int e = launch_status()) return e;
 
   PixXParams bp;
   bp.ptr = x; bp.bytes = (uint32_t)(d.x_elems * 4); bp.rows = CRS; bp.M = M; bp.set_pq(d.P * d.Q, d.Q);
-  bp.img_stride = d.C * d.H * d.W; bp.H = d.H; bp.W = d.W; bp.st = d.st; bp.pad = d.pad; bp.rtab = tab;
+  bp.img_stride = d.C * d.H * d.W; bp.H = d.H; bp.W = d.W; bp.st = d.st; bp.pad = d.pad; bp.set_filter(d.R, d.S);
   EpiParams ep;
   ep.out = part; ep.bias = nullptr; ep.alpha = 1.0f; ep.beta = 0.0f;
   ep.rows = d.K; ep.cols = CRS; ep.inner = 0; ep.ld = CRS; ep.relu = 0;

@@ -539,12 +539,16 @@ struct PixXParams {
   int M, PQ, Q;
   int img_stride;  // C*H*W
   int H, W, st, pad;
-  const int4* rtab;  // per (c,r,s): {c*H*W + r*W + s, r, s, 0}
   FastDiv dPQ, dQ;   // divisions by PQ and Q (set_pq)
+  FastDiv dRS, dS;   // a row (c,r,s) is decoded where the loader starts: tap (r, s) at c*H*W + r*W + s (set_filter)
   void set_pq(int pq, int q) {
     PQ = pq; Q = q;
     dPQ = FastDiv((uint32_t)(pq > 0 ? pq : 1));
     dQ = FastDiv((uint32_t)(q > 0 ? q : 1));
+  }
+  void set_filter(int R, int S) {
+    dRS = FastDiv((uint32_t)(R * S > 0 ? R * S : 1));
+    dS = FastDiv((uint32_t)(S > 0 ? S : 1));
   }
 };
 
@@ -573,8 +577,10 @@ struct LoadPixX {
     for (int i = 0; i < CNT; ++i) {
       const int row = row0 + r + i * RSTEP;
       if (row < p.rows) {
-        const int4 e = p.rtab[row];
-        roff[i] = e.x; rr[i] = e.y; rs[i] = e.z;
+        uint32_t c, t, r2, s2;
+        p.dRS.divmod((uint32_t)row, c, t);
+        p.dS.divmod(t, r2, s2);
+        roff[i] = (int)c * p.H * p.W + (int)r2 * p.W + (int)s2; rr[i] = (int)r2; rs[i] = (int)s2;
       } else {
         roff[i] = NOPAD ? (int)kInvalidByteOff : 0; rr[i] = -(1 << 28); rs[i] = 0;
       }
