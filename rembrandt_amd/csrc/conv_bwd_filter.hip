@@ -809,18 +809,19 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     float* xT = reinterpret_cast<float*>(base + sp.tab_bytes + sp.dyt_bytes);
     float* parts = reinterpret_cast<float*>(base + sp.tab_bytes + sp.dyt_bytes + sp.xt_bytes);
     float* const bpart = (bias_part && nhwc_vec_ok(d.K, dyT)) ? bias_part : nullptr;
-    {
-      // the two channel-last copies and the table share one launch
-      NhwcCopyArgs a, b;
-      a.src = dy; a.dst = dyT; a.C = d.K; a.H = d.P; a.W = d.Q; a.Hp = d.P; a.Wp = d.Q; a.halo = 0;
-      a.vec = nhwc_vec_ok(d.K, dyT) ? 1 : 0;
-      a.gx = bpart ? 1 : cdiv(d.P * d.Q, a.vec ? 64 : 32); a.gy = cdiv(d.K, a.vec ? 64 : 32);
-      b.src = x; b.dst = xT; b.C = d.C; b.H = d.H; b.W = d.W; b.Hp = sp.Hp; b.Wp = sp.Wp; b.halo = d.pad;
-      b.vec = nhwc_vec_ok(d.C, xT) ? 1 : 0;
-      b.gx = cdiv(sp.Hp * sp.Wp, b.vec ? 64 : 32); b.gy = cdiv(d.C, b.vec ? 64 : 32);
-      const long long nb_dy = (long long)a.gx * a.gy * d.N, nb_x = (long long)b.gx * b.gy * d.N;
-      const long long nb_tab = cdiv(sp.n_k, 256);
-      if (nb_dy + nb_x + nb_tab >= (1ll << 31)) return RH_E_LIMIT;
+    NhwcCopyArgs a, b;
+    a.src = dy; a.dst = dyT; a.C = d.K; a.H = d.P; a.W = d.Q; a.Hp = d.P; a.Wp = d.Q; a.halo = 0;
+    a.vec = nhwc_vec_ok(d.K, dyT) ? 1 : 0;
+    a.gx = bpart ? 1 : cdiv(d.P * d.Q, a.vec ? 64 : 32); a.gy = cdiv(d.K, a.vec ? 64 : 32);
+    b.src = x; b.dst = xT; b.C = d.C; b.H = d.H; b.W = d.W; b.Hp = sp.Hp; b.Wp = sp.Wp; b.halo = d.pad;
+    b.vec = nhwc_vec_ok(d.C, xT) ? 1 : 0;
+    b.gx = cdiv(sp.Hp * sp.Wp, b.vec ? 64 : 32); b.gy = cdiv(d.C, b.vec ? 64 : 32);
+    const long long nb_dy = (long long)a.gx * a.gy * d.N, nb_x = (long long)b.gx * b.gy * d.N;
+    const long long nb_tab = cdiv(sp.n_k, 256);
+    // Small layers: the two channel-last copies and the table share one launch (a launch gap less twice over on a
+    // chain of kernels of a few microseconds).  Large layers keep three launches: as one, the copies of a ResNet-18
+    // step's filter gradients, which run beside the data gradients of the other stream, made the step 3 % slower.
+    if (nb_dy + nb_x <= 4096) {
       ProfScope prof("nchw_to_nhwc", 8.0 * ((double)d.N * d.K * d.P * d.Q) +
                                          4.0 * ((double)d.N * d.C * d.H * d.W + (double)d.N * d.C * sp.Hp * sp.Wp), stream);
       if (bpart)
@@ -829,6 +830,14 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
       else
         hipLaunchKernelGGL(bwd_filter_prep_kernel<false>, dim3((unsigned)(nb_dy + nb_x + nb_tab)), dim3(256), 0, stream, a,
                            (float*)nullptr, (int)nb_dy, b, (int)nb_x, soff, sp.n_k, Ms, d.P * d.Q, d.Q, d.st, d.K);
+      if (int e = launch_status()) return e;
+    } else {
+      hipLaunchKernelGGL(prep_bwd_filter_soff_kernel, dim3(cdiv(sp.n_k, 256)), dim3(256), 0, stream, soff, dyT, sp.n_k, Ms,
+                         d.P * d.Q, d.Q, d.st, sp.Hp, sp.Wp, d.C, d.K);
+      if (int e = launch_status()) return e;
+      launch_nchw_to_nhwc(dy, dyT, d.N, d.K, d.P, d.Q, d.P, d.Q, 0, stream, bpart);
+      if (int e = launch_status()) return e;
+      launch_nchw_to_nhwc(x, xT, d.N, d.C, d.H, d.W, sp.Hp, sp.Wp, d.pad, stream);
       if (int e = launch_status()) return e;
     }
     if (bpart) *folded = true;
