@@ -857,18 +857,26 @@ class Conv2dOperator : public Operator {
     if (!act_bwd_folded_)
       apply_rect_backprop(config_.act_func, out_act_->as_ptr(), out_dims_.len(), batch_size, out_delta_->as_mut_ptr(), s);
     // Streams and scratch of the two gradient kernels.  With a data gradient to follow on the main stream both go
-    // to the second stream; the first layer has none, so its filter gradient stays on the main stream (on the second
-    // it would only queue behind that stream's earlier work) and the bias gradient runs beside it.
+    // to the second stream; the first layer has none, so its gradients stay on the main stream (on the second
+    // they would only queue behind that stream's earlier work).
     rh_stream_t s_filter = s, s_bias = s;
     DeviceBuffer<uint8_t>*w_filter = workspace_.get(), *w_bias = workspace_.get();
-    if (workspace_aux_ && overlap_on_) {
+    if (workspace_aux_ && overlap_on_ && in_delta_) {
       context_->fork();                        // the second stream sees the masked out_delta
-      s_bias = context_->aux_stream();
-      w_bias = workspace_aux_.get();
-      if (in_delta_) { s_filter = s_bias; w_filter = w_bias; }
+      s_filter = s_bias = context_->aux_stream();
+      w_filter = w_bias = workspace_aux_.get();
     }
     const float beta = params_.take_backward_beta();   // 1: accumulate (the reference's call); 0: the buffers stand for zeros
-    if (s_filter == s_bias && w_filter == w_bias) {
+    if (!in_delta_ && workspace_aux_ && overlap_on_) {
+      // First layer, backward on two streams: its gradients are the last kernels of the pass.  The bias gradient goes
+      // first (a memory-bound pass beside the second stream's last contraction), so that only the filter gradient's
+      // reduction follows the last contraction of the step.
+      unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), scale,
+                                   out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
+                                   w_bias->len(), s_bias), "conv2d backward bias");
+      unwrap(rh_conv2d_bwd_filter(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta, params_.grad_weights->as_mut_ptr(),
+                                  w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter");
+    } else if (s_filter == s_bias && w_filter == w_bias) {
       // one stream for both: one call, which reads out_delta once where the filter gradient makes a pass over it anyway
       unwrap(rh_conv2d_bwd_filter_bias(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta,
                                        params_.grad_weights->as_mut_ptr(), params_.grad_bias->as_mut_ptr(),
