@@ -329,7 +329,7 @@ template <bool BIAS>
 __device__ __forceinline__ void nchw_to_nhwc_vec_body(float* __restrict__ tile, int bx, int by, int bz, int gx,
                                                       const float* __restrict__ src, float* __restrict__ dst,
                                                       int C, int H, int W, int Hp, int Wp, int halo,
-                                                      float* __restrict__ bias_part) {
+                                                      float* __restrict__ bias_part, long long src_elems) {
   const int c0 = by * 64, n = bz;
   const int HpWp = Hp * Wp;
   float bsum = 0.0f;
@@ -337,26 +337,36 @@ __device__ __forceinline__ void nchw_to_nhwc_vec_body(float* __restrict__ tile, 
   {
     const int pq = threadIdx.x & 15, cl0 = threadIdx.x >> 4;
     const int pix = pix0 + 4 * pq;
-    const int hp = pix / Wp, wp = pix - hp * Wp;
-    const int h = hp - halo, w = wp - halo;
-    // (without a halo the plane is one contiguous run: four pixels may cross a row end)
-    const bool whole = pix + 3 < HpWp && (halo == 0 || ((unsigned)h < (unsigned)H && w >= 0 && w + 3 < W));
-    int off[4];  // element offsets within a plane, -1 = zero
+    // Element offsets within a plane, -1 = zero.  A plane is dense and the map from padded pixels to source elements
+    // keeps their order, so the source elements of four consecutive pixels are one run of consecutive addresses
+    // however the four lie across row ends and the halo: one 16-byte load from the run's start (4-byte aligned)
+    // brings them all, and each pixel picks its element by its distance from that start.
+    int off[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int pe = pix + e, hpe = pe / Wp, he = hpe - halo, we = pe - hpe * Wp - halo;
       off[e] = (pe < HpWp && (unsigned)he < (unsigned)H && (unsigned)we < (unsigned)W) ? he * W + we : -1;
     }
+    int first = off[3];
+    if (off[2] >= 0) first = off[2];
+    if (off[1] >= 0) first = off[1];
+    if (off[0] >= 0) first = off[0];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int cl = cl0 + 16 * i, c = c0 + cl;
       float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (c < C) {
-        const float* plane = src + ((size_t)n * C + c) * ((size_t)H * W);
-        if (whole) {
-          const float4_a4 q = *reinterpret_cast<const float4_a4*>(plane + off[0]);
-          v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
-        } else {
+      if (c < C && first >= 0) {
+        const long long base = ((long long)n * C + c) * ((long long)H * W);
+        const float* plane = src + base;
+        if (base + first + 3 < src_elems) {
+          const float4_a4 q = *reinterpret_cast<const float4_a4*>(plane + first);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int d = off[e] - first;
+            const float t = d == 0 ? q.x : d == 1 ? q.y : d == 2 ? q.z : q.w;
+            v[e] = off[e] >= 0 ? t : 0.0f;
+          }
+        } else {   // the tensor's last three elements
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (off[e] >= 0) v[e] = plane[off[e]];
@@ -402,7 +412,8 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_vec_kernel(const float* __re
                                                                int C, int H, int W, int Hp, int Wp, int halo,
                                                                float* __restrict__ bias_part) {
   __shared__ __attribute__((aligned(16))) float tile[64 * 64];
-  nchw_to_nhwc_vec_body<BIAS>(tile, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.x, src, dst, C, H, W, Hp, Wp, halo, bias_part);
+  nchw_to_nhwc_vec_body<BIAS>(tile, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.x, src, dst, C, H, W, Hp, Wp, halo, bias_part,
+                              (long long)gridDim.z * C * H * W);
 }
 
 // The 16-byte form can carry the per-image plane sums along (bias_part, N x C floats; no halo).
@@ -457,6 +468,7 @@ __device__ __forceinline__ void prep_bwd_filter_soff_body(int first, int stride,
 struct NhwcCopyArgs {
   const float* src; float* dst;
   int C, H, W, Hp, Wp, halo;
+  long long elems;  // elements of src
   int vec;      // 16-byte form (64 x 64 pieces) or the element form (32 x 32 pieces)
   int gx, gy;   // grid of pieces: (gx, gy, images)
 };
@@ -471,7 +483,7 @@ __global__ __launch_bounds__(256) void bwd_filter_prep_kernel(NhwcCopyArgs dy, f
     const int bx = b % dy.gx, t = b / dy.gx;
     if (BIAS || dy.vec)
       nchw_to_nhwc_vec_body<BIAS>(tile, bx, t % dy.gy, t / dy.gy, dy.gx, dy.src, dy.dst, dy.C, dy.H, dy.W, dy.Hp, dy.Wp, dy.halo,
-                                  bias_part);
+                                  bias_part, dy.elems);
     else
       nchw_to_nhwc_body(tile, bx, t % dy.gy, t / dy.gy, dy.src, dy.dst, dy.C, dy.H, dy.W, dy.Hp, dy.Wp, dy.halo);
     return;
@@ -480,7 +492,8 @@ __global__ __launch_bounds__(256) void bwd_filter_prep_kernel(NhwcCopyArgs dy, f
   if (b < nb_x) {
     const int bx = b % x.gx, t = b / x.gx;
     if (x.vec)
-      nchw_to_nhwc_vec_body<false>(tile, bx, t % x.gy, t / x.gy, x.gx, x.src, x.dst, x.C, x.H, x.W, x.Hp, x.Wp, x.halo, nullptr);
+      nchw_to_nhwc_vec_body<false>(tile, bx, t % x.gy, t / x.gy, x.gx, x.src, x.dst, x.C, x.H, x.W, x.Hp, x.Wp, x.halo, nullptr,
+                                   x.elems);
     else
       nchw_to_nhwc_body(tile, bx, t % x.gy, t / x.gy, x.src, x.dst, x.C, x.H, x.W, x.Hp, x.Wp, x.halo);
     return;
@@ -811,6 +824,7 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     float* const bpart = (bias_part && nhwc_vec_ok(d.K, dyT)) ? bias_part : nullptr;
     NhwcCopyArgs a, b;
     a.src = dy; a.dst = dyT; a.C = d.K; a.H = d.P; a.W = d.Q; a.Hp = d.P; a.Wp = d.Q; a.halo = 0;
+    a.elems = d.y_elems; b.elems = d.x_elems;
     a.vec = nhwc_vec_ok(d.K, dyT) ? 1 : 0;
     a.gx = bpart ? 1 : cdiv(d.P * d.Q, a.vec ? 64 : 32); a.gy = cdiv(d.K, a.vec ? 64 : 32);
     b.src = x; b.dst = xT; b.C = d.C; b.H = d.H; b.W = d.W; b.Hp = sp.Hp; b.Wp = sp.Wp; b.halo = d.pad;

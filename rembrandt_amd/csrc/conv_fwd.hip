@@ -26,32 +26,48 @@ void launch_build_fwd_tab(int4* tab, int n_entries, int CRS, int R, int S, int H
 // elements of dst (they may straddle a row or a plane) and writes them as one 16-byte store when dst is aligned:
 // stores of 16 bytes per lane over one sweep of consecutive blocks are what this GPU's memory system wants.
 __device__ __forceinline__ void pad_image_body(unsigned block, const float* __restrict__ src, float* __restrict__ dst,
-                                               unsigned total, int H, int W, FastDiv dHp, FastDiv dWp, int halo, int vec) {
+                                               unsigned total, int H, int W, FastDiv dHp, FastDiv dWp, int halo, int vec,
+                                               unsigned src_total) {
   const unsigned g = block * blockDim.x + threadIdx.x;
   const unsigned i0 = g * 4u;
   if (i0 >= total) return;
   uint32_t t, wp, plane, hp;
   dWp.divmod(i0, t, wp);
   dHp.divmod(t, plane, hp);
-  float v[4];
-  {
-    const int h = (int)hp - halo, w = (int)wp - halo;
-    if ((unsigned)h < (unsigned)H && w >= 0 && w + 3 < W) {
-      // all four inside one source row: one 16-byte load (4-byte aligned: source rows start anywhere)
+  // Source offsets of the four, -1 = zero.  src is dense and the map from dst to src keeps the order of the elements,
+  // so the source elements of four consecutive dst elements are one run of consecutive addresses, however the four
+  // lie across row ends, plane ends and the halo: one 16-byte load from the run's start (4-byte aligned: it starts
+  // anywhere) brings them all, and each element picks its value by its distance from that start.
+  int o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int he = (int)hp - halo, we = (int)wp - halo;
+    o[e] = ((unsigned)he < (unsigned)H && (unsigned)we < (unsigned)W && i0 + e < total)
+               ? (int)((plane * (unsigned)H + (unsigned)he) * (unsigned)W + (unsigned)we) : -1;
+    if (++wp == dWp.div) {
+      wp = 0;
+      if (++hp == dHp.div) { hp = 0; ++plane; }
+    }
+  }
+  int first = o[3];
+  if (o[2] >= 0) first = o[2];
+  if (o[1] >= 0) first = o[1];
+  if (o[0] >= 0) first = o[0];
+  float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (first >= 0) {
+    if ((unsigned)first + 3u < src_total) {
       typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
-      const f4u q = *reinterpret_cast<const f4u*>(src + ((size_t)plane * H + h) * W + w);
-      v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
-    } else {
+      const f4u q = *reinterpret_cast<const f4u*>(src + first);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int he = (int)hp - halo, we = (int)wp - halo;
-        v[e] = ((unsigned)he < (unsigned)H && (unsigned)we < (unsigned)W && i0 + e < total)
-                   ? src[((size_t)plane * H + he) * W + we] : 0.0f;
-        if (++wp == dWp.div) {
-          wp = 0;
-          if (++hp == dHp.div) { hp = 0; ++plane; }
-        }
+        const int d = o[e] - first;
+        const float t = d == 0 ? q.x : d == 1 ? q.y : d == 2 ? q.z : q.w;
+        v[e] = o[e] >= 0 ? t : 0.0f;
       }
+    } else {   // the tensor's last three elements
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (o[e] >= 0) v[e] = src[o[e]];
     }
   }
   if (vec && i0 + 3 < total) {
@@ -64,8 +80,9 @@ __device__ __forceinline__ void pad_image_body(unsigned block, const float* __re
 }
 
 __global__ __launch_bounds__(256) void pad_image_kernel(const float* __restrict__ src, float* __restrict__ dst, unsigned total,
-                                                        int H, int W, FastDiv dHp, FastDiv dWp, int halo, int vec) {
-  pad_image_body(blockIdx.x, src, dst, total, H, W, dHp, dWp, halo, vec);
+                                                        int H, int W, FastDiv dHp, FastDiv dWp, int halo, int vec,
+                                                        unsigned src_total) {
+  pad_image_body(blockIdx.x, src, dst, total, H, W, dHp, dWp, halo, vec, src_total);
 }
 
 // The filter-side scratch of the scalar-offset forward and stride-1 backward-data paths, as a function of a virtual
@@ -108,9 +125,10 @@ __global__ __launch_bounds__(256) void prep_soff_kernel(PrepSoffArgs a) {
 // independent, and a launch less in front of a contraction is a launch gap less on the chain of a small layer.
 __global__ __launch_bounds__(256) void pad_image_prep_soff_kernel(const float* __restrict__ src, float* __restrict__ dst,
                                                                   unsigned total, int H, int W, FastDiv dHp, FastDiv dWp,
-                                                                  int halo, int vec, unsigned pad_blocks, PrepSoffArgs a) {
+                                                                  int halo, int vec, unsigned pad_blocks, PrepSoffArgs a,
+                                                                  unsigned src_total) {
   if (blockIdx.x < pad_blocks) {
-    pad_image_body(blockIdx.x, src, dst, total, H, W, dHp, dWp, halo, vec);
+    pad_image_body(blockIdx.x, src, dst, total, H, W, dHp, dWp, halo, vec, src_total);
   } else {
     const unsigned b = blockIdx.x - pad_blocks, nb = gridDim.x - pad_blocks;
     prep_soff_body(a, (long long)b * blockDim.x + threadIdx.x, (long long)nb * blockDim.x);
@@ -149,7 +167,7 @@ void launch_pad_image(const float* src, float* dst, long long planes, int H, int
   }
   const int vec = (reinterpret_cast<uintptr_t>(dst) & 15) == 0 ? 1 : 0;
   hipLaunchKernelGGL(pad_image_kernel, dim3(stream_grid((size_t)(total + 3) / 4, 256)), dim3(256), 0, stream, src, dst,
-                     (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, vec);
+                     (unsigned)total, H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, vec, (unsigned)(planes * H * W));
 }
 
 static PrepSoffArgs prep_args(const float* w, float* wT, int* soff, int n_k, int k_true, int rows, int R, int S, int HpWp,
@@ -176,7 +194,7 @@ void launch_pad_image_prep_soff(const float* src, float* dst, long long planes, 
   const unsigned pad_blocks = (unsigned)stream_grid((size_t)(total + 3) / 4, 256);
   const unsigned prep_blocks = (unsigned)stream_grid((size_t)n_k * rows, 256);
   hipLaunchKernelGGL(pad_image_prep_soff_kernel, dim3(pad_blocks + prep_blocks), dim3(256), 0, stream, src, dst, (unsigned)total,
-                     H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, vec, pad_blocks, a);
+                     H, W, FastDiv((uint32_t)Hp), FastDiv((uint32_t)Wp), halo, vec, pad_blocks, a, (unsigned)(planes * H * W));
 }
 
 // VEC: four consecutive elements per thread through 16-byte loads and stores (slab stride, first element and all
