@@ -52,6 +52,40 @@ constexpr int stream_blocks_per_cu() {
   return !FAST || 512 / regs < 2 ? 2 : (512 / regs > 4 ? 4 : 512 / regs);
 }
 
+// The filter, once per block: sa[(s * TM + i) * 64 + lane] = A(32 i + lane % 32, 2 s + lane / 32), zero outside.
+// Every thread first issues all its loads (KH TM / 4 of them, out-of-range ones read zero) and then writes LDS, so
+// a block waits for memory once.  Which element a thread takes follows the filter's layout in memory: with the
+// contraction index contiguous (forward) a wave reads eight rows by eight consecutive k (32-byte pieces; its LDS
+// writes meet eight to a bank), with the row index contiguous (backward-data) a wave reads LDS order directly.
+template <int TM, int KH>
+__device__ __forceinline__ void stage_filter(const Conv1x1Params& p, float* __restrict__ sa) {
+  constexpr int PER = KH * TM / 4;
+  const __amdgpu_buffer_rsrc_t rflt = make_rsrc(p.A, (uint32_t)(sizeof(float) * (size_t)p.rows * p.kdim));
+  const bool k_major = p.a_k_stride == 1;
+  float tmp[PER];
+  int pos[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int e = (int)threadIdx.x + 256 * j;
+    int row, k;
+    if (k_major) {
+      const int rest = e >> 6, k_hi = rest % (KH / 4), r_hi = rest / (KH / 4);
+      k = 8 * k_hi + (e & 7);
+      row = 8 * r_hi + ((e >> 3) & 7);
+      pos[j] = ((k >> 1) * TM + (row >> 5)) * 64 + (k & 1) * 32 + (row & 31);
+    } else {
+      const int l = e & 63, si = e >> 6;
+      row = 32 * (si % TM) + (l & 31);
+      k = 2 * (si / TM) + (l >> 5);
+      pos[j] = e;
+    }
+    const uint32_t off = (row < p.rows && k < p.kdim) ? 4u * (uint32_t)(row * p.a_row_stride + k * p.a_k_stride) : 0x80000000u;
+    tmp[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rflt, (int)off, 0, 0));
+  }
+#pragma unroll
+  for (int j = 0; j < PER; ++j) sa[pos[j]] = tmp[j];
+}
+
 // MASK: ep.mask (a tensor shaped like the result) zeroes the result where it is not > 0 (backward-data that applies
 // the backward of the ReLU before this layer as it writes; sixteen more loads per row tile and column tile).
 template <int TM, int KH, bool FAST, class PASS, bool MASK = false>
@@ -70,39 +104,8 @@ __global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST && !MASK>()
   const int last = min(first + span, p.tiles);                      // (one past) this XCD's range
   const int half = lane >> 5, l32 = lane & 31;
 
-  // The filter, once per block: sa[(s * TM + i) * 64 + lane] = A(32 i + lane % 32, 2 s + lane / 32), zero outside.
-  // Every thread first issues all its loads (KH TM / 4 of them, out-of-range ones read zero) and then writes LDS, so
-  // a block waits for memory once.  Which element a thread takes follows the filter's layout in memory: with the
-  // contraction index contiguous (forward) a wave reads eight rows by eight consecutive k (32-byte pieces; its LDS
-  // writes meet eight to a bank), with the row index contiguous (backward-data) a wave reads LDS order directly.
   extern __shared__ float sa[];
-  {
-    constexpr int PER = KH * TM / 4;
-    const __amdgpu_buffer_rsrc_t rflt = make_rsrc(p.A, (uint32_t)(sizeof(float) * (size_t)p.rows * p.kdim));
-    const bool k_major = p.a_k_stride == 1;
-    float tmp[PER];
-    int pos[PER];
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int e = (int)threadIdx.x + 256 * j;
-      int row, k;
-      if (k_major) {
-        const int rest = e >> 6, k_hi = rest % (KH / 4), r_hi = rest / (KH / 4);
-        k = 8 * k_hi + (e & 7);
-        row = 8 * r_hi + ((e >> 3) & 7);
-        pos[j] = ((k >> 1) * TM + (row >> 5)) * 64 + (k & 1) * 32 + (row & 31);
-      } else {
-        const int l = e & 63, si = e >> 6;
-        row = 32 * (si % TM) + (l & 31);
-        k = 2 * (si / TM) + (l >> 5);
-        pos[j] = e;
-      }
-      const uint32_t off = (row < p.rows && k < p.kdim) ? 4u * (uint32_t)(row * p.a_row_stride + k * p.a_k_stride) : 0x80000000u;
-      tmp[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rflt, (int)off, 0, 0));
-    }
-#pragma unroll
-    for (int j = 0; j < PER; ++j) sa[pos[j]] = tmp[j];
-  }
+  stage_filter<TM, KH>(p, sa);
   __syncthreads();
   const float* const sal = sa + lane;
 
@@ -285,6 +288,237 @@ __global__ __launch_bounds__(256, (stream_blocks_per_cu<TM, KH, FAST && !MASK>()
   for (; t < last; t += nwaves) compute_tile(b0, t, t + nwaves);
 }
 
+
+// The same kernel for column counts per image that are a multiple of W (2 or 4), alpha == 1, beta == 0, full row tiles
+// and a contraction of exactly 2 KH: a wave takes 32 W columns at a time and lane l holds the W consecutive pixels
+// W l .. W l + W - 1 of each, so that every access to the source and to the result is W dwords wide (dword accesses top
+// out near 3.8 TB/s on this GPU, 16-byte ones reach 6).  The W pixels of a lane are the same column of W different
+// MFMA tiles (tile j = pixels W l + j over the 32 lanes: which 32 pixels make up a tile is free), and since both the
+// count of columns and of pixels per image are multiples of W, a lane's pixels lie in one image and are either all
+// inside the tensor or all outside: every lane computes its own image and pixel once per 32 W columns, no case
+// distinction for a group of columns that straddles two images.  One filter read from LDS serves W MFMAs.
+// The second half of the next group's operands is requested after the stores of this one, so that their registers are
+// free for the mask values of the epilogue in between.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int W>
+__device__ __forceinline__ void load_w(float (&d)[W], __amdgpu_buffer_rsrc_t r, uint32_t off) {
+  if constexpr (W == 4) {
+    const u32x4 q = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) d[j] = __uint_as_float(q[j]);
+  } else {
+    const u32x2 q = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0);
+    d[0] = __uint_as_float(q[0]); d[1] = __uint_as_float(q[1]);
+  }
+}
+template <int W>
+__device__ __forceinline__ void store_w(const float (&d)[W], __amdgpu_buffer_rsrc_t r, uint32_t off) {
+  if constexpr (W == 4) {
+    u32x4 q;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) q[j] = __float_as_uint(d[j]);
+    __builtin_amdgcn_raw_buffer_store_b128(q, r, (int)off, 0, 0);
+  } else {
+    u32x2 q;
+    q[0] = __float_as_uint(d[0]); q[1] = __float_as_uint(d[1]);
+    __builtin_amdgcn_raw_buffer_store_b64(q, r, (int)off, 0, 0);
+  }
+}
+
+template <int TM, int KH, int W>
+constexpr int wide_blocks_per_cu() {
+  return (16 * TM * W + KH * W + 64) <= 256 ? 2 : 1;
+}
+
+template <int TM, int KH, int W, class PASS, bool MASK>
+__global__ __launch_bounds__(256, (wide_blocks_per_cu<TM, KH, W>())) void conv1x1_stream_wide_kernel(Conv1x1Params p, EpiParams ep, FastDiv dPQ) {
+  const int lane = threadIdx.x & 63;
+  const bool by_xcd = (gridDim.x & 7) == 0;   // (see conv1x1_stream_kernel: an XCD sweeps its eighth in address order)
+  const int nwaves = by_xcd ? (int)(gridDim.x >> 3) * 4 : (int)gridDim.x * 4;
+  const int wave = __builtin_amdgcn_readfirstlane(
+      (int)((by_xcd ? blockIdx.x >> 3 : blockIdx.x) * 4 + (threadIdx.x >> 6)));
+  const int span = by_xcd ? (p.tiles + 7) >> 3 : p.tiles;            // groups of 32 W columns per XCD
+  const int first = by_xcd ? (int)(blockIdx.x & 7) * span : 0;
+  const int last = min(first + span, p.tiles);
+  const int half = lane >> 5, l32 = lane & 31;
+
+  extern __shared__ float sa[];
+  stage_filter<TM, KH>(p, sa);
+  __syncthreads();
+  const float* const sal = sa + lane;
+
+  const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.src, p.src_bytes);
+  const __amdgpu_buffer_rsrc_t rdst = make_rsrc(ep.out, (uint32_t)(sizeof(float) * (size_t)p.cols * p.rows));
+  const __amdgpu_buffer_rsrc_t rmask = make_rsrc(MASK ? ep.mask : ep.out, (uint32_t)(sizeof(float) * (size_t)p.cols * p.rows));
+  const int PQ4 = p.PQ * 4;
+  const uint32_t img_bytes = (uint32_t)p.kdim * (uint32_t)PQ4;
+  const uint32_t out_img_bytes = (uint32_t)p.rows * (uint32_t)PQ4;
+
+  // A lane's place in group g: image and pixel of its first column (W l32 columns into the group); "nowhere" (offset
+  // 0x80000000: loads return 0, stores are dropped) past this XCD's range or the tensor's last column.
+  auto place = [&](int g, uint32_t& img, uint32_t& pix) __attribute__((always_inline)) -> bool {
+    const long long col64 = (long long)g * (32 * W) + W * l32;
+    if (g >= last || col64 >= p.cols) return false;
+    dPQ.divmod((uint32_t)col64, img, pix);
+    return true;
+  };
+  auto src_addr = [&](int g, uint32_t& v, uint32_t& step) __attribute__((always_inline)) {
+    uint32_t img, pix;
+    v = 0x80000000u;
+    step = 0u;
+    if (place(g, img, pix)) {
+      v = img * img_bytes + pix * 4u + (uint32_t)(half * PQ4);
+      step = (uint32_t)(2 * PQ4);
+    }
+  };
+  auto load_part = [&](float (&b)[KH][W], uint32_t& v, uint32_t step, int s0, int s1) __attribute__((always_inline)) {
+#pragma unroll
+    for (int s = s0; s < s1; ++s) {
+      load_w<W>(b[s], rsrc, v);
+      v += step;
+    }
+  };
+
+  auto compute_group = [&](float (&b)[KH][W], int g, int next, uint32_t& nv, uint32_t& nstep) __attribute__((always_inline)) {
+    // (nv, nstep): where the second half of this group's successor starts, left by the first-half request below
+    f32x16 acc[TM][W];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < W; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    uint32_t out_o = 0x80000000u;
+    {
+      uint32_t img, pix;
+      if (place(g, img, pix)) out_o = img * out_img_bytes + pix * 4u + (uint32_t)(4 * half * PQ4);
+    }
+    typedef const __attribute__((address_space(3))) float* lds_ptr;
+    lds_ptr sl = (lds_ptr)sal;
+    asm volatile("" : "+v"(sl));   // (the filter reads stay in the loop, one per row tile and channel pair)
+    float av[2][TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) av[0][i] = sl[i * 64];
+#pragma unroll
+    for (int s = 0; s < KH; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 1 < KH) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) av[(s + 1) & 1][i] = sl[((s + 1) * TM + i) * 64];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < W; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s & 1][i], b[s][j], acc[i][j], 0, 0, 0);
+      if (s == KH / 2 - 1) {
+        __builtin_amdgcn_sched_barrier(0);
+        src_addr(next, nv, nstep);
+        load_part(b, nv, nstep, 0, KH / 2);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (ep.bias) {
+      // rows 32 i + 8 q + 4 half + e: added after the sum, as the separate bias pass of the reference does
+      typedef const __attribute__((address_space(1))) float* global_ptr;
+      global_ptr bias = (global_ptr)ep.bias;
+      asm volatile("" : "+s"(bias));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          global_ptr bq = bias + 32 * i + 8 * q + 4 * half;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float bv = bq[e];
+#pragma unroll
+            for (int j = 0; j < W; ++j) acc[i][j][4 * q + e] += bv;
+          }
+        }
+    }
+    if (ep.relu) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < W; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[i][j][v] = acc[i][j][v] > 0.0f ? acc[i][j][v] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      float m[MASK ? 16 : 1][W];
+      (void)m;
+      if (MASK) {   // one row tile's mask values at a time: sixteen loads in flight, then its stores
+        uint32_t om = out_o + (uint32_t)(32 * i) * (uint32_t)PQ4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            load_w<W>(m[4 * q + e], rmask, om);
+            om += (uint32_t)PQ4;
+          }
+          om += (uint32_t)(4 * PQ4);
+        }
+      }
+      uint32_t o = out_o + (uint32_t)(32 * i) * (uint32_t)PQ4;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float val[W];
+#pragma unroll
+          for (int j = 0; j < W; ++j) {
+            val[j] = acc[i][j][4 * q + e];
+            if (MASK) val[j] = m[4 * q + e][j] > 0.0f ? val[j] : 0.0f;
+          }
+          store_w<W>(val, rdst, o);
+          o += (uint32_t)PQ4;
+        }
+        o += (uint32_t)(4 * PQ4);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    load_part(b, nv, nstep, KH / 2, KH);
+  };
+
+  float b0[KH][W];
+  int g = first + wave;
+  if (g >= last) return;
+  {
+    uint32_t v, step;
+    src_addr(g, v, step);
+    load_part(b0, v, step, 0, KH);
+  }
+  uint32_t nv = 0x80000000u, nstep = 0u;
+  for (; g < last; g += nwaves) compute_group(b0, g, g + nwaves, nv, nstep);
+}
+
+template <int TM, int KH, int W>
+constexpr bool wide_fits() { return TM * W <= 12 && 16 * TM * W + KH * W + 80 <= 512; }
+
+template <int TM, int KH, int W, class PASS, bool MASK>
+static int launch_stream_wide_one(Conv1x1Params p, const EpiParams& ep, const FastDiv& dPQ, size_t lds, hipStream_t stream) {
+  if (lds > 48 * 1024) {
+    static const hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv1x1_stream_wide_kernel<TM, KH, W, PASS, MASK>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (a != hipSuccess) return (int)a;
+  }
+  p.tiles = (int)cdiv<long long>(p.cols, 32 * W);   // groups of 32 W columns
+  const int full = 256 * wide_blocks_per_cu<TM, KH, W>();
+  const int blocks = p.tiles >= 4 * full ? full : (p.tiles >= 256 ? 8 * cdiv(cdiv(p.tiles, 8), 4) : cdiv(p.tiles, 4));
+  hipLaunchKernelGGL((conv1x1_stream_wide_kernel<TM, KH, W, PASS, MASK>), dim3((unsigned)blocks), dim3(256), lds, stream, p, ep, dPQ);
+  return launch_status();
+}
+
+template <int TM, int KH, int W, class PASS>
+static int launch_stream_wide(const Conv1x1Params& p, const EpiParams& ep, const FastDiv& dPQ, size_t lds, hipStream_t stream) {
+  if constexpr (std::is_same<PASS, PassConvBwdData>::value && W == 2) {   // (the masked form exists for two pixels per lane)
+    if (ep.mask) return launch_stream_wide_one<TM, KH, W, PASS, true>(p, ep, dPQ, lds, stream);
+  }
+  return launch_stream_wide_one<TM, KH, W, PASS, false>(p, ep, dPQ, lds, stream);
+}
+
 template <int TM, int KH, class PASS>
 static int launch_stream(const Conv1x1Params& p, const EpiParams& ep, hipStream_t stream) {
   const FastDiv dPQ((uint32_t)p.PQ);
@@ -299,6 +533,20 @@ static int launch_stream(const Conv1x1Params& p, const EpiParams& ep, hipStream_
   }
   const bool fast = ep.alpha == 1.0f && ep.beta == 0.0f && p.rows == 32 * TM && p.kdim == 2 * KH &&
                     (!ep.bias || (reinterpret_cast<uintptr_t>(ep.bias) & 15) == 0);
+  // Long contractions (96 channels and more) with a pixel count per image that allows it take the form that moves
+  // two or four pixels per lane (measured on 96 -> 96, 54 x 54, batch 128: forward 97 -> 92 us with two, backward-data
+  // 97 -> 88 with four, backward-data with the mask 132 -> 117 with two; on 128 -> 128, 28 x 28 the masked form
+  // 86 -> 31).  Short ones lose there (32 -> 64 on 56 x 56: 27 -> 29-32 us: less matrix work per group of columns to
+  // cover the epilogue of a wave that has its SIMD to itself or shares it with one other).
+  if constexpr (KH >= 48) {
+    if (fast && p.PQ % 2 == 0) {
+      constexpr bool bwd = std::is_same<PASS, PassConvBwdData>::value;
+      if constexpr (bwd && wide_fits<TM, KH, 4>()) {
+        if (!ep.mask && p.PQ % 4 == 0) return launch_stream_wide<TM, KH, 4, PASS>(p, ep, dPQ, lds, stream);
+      }
+      return launch_stream_wide<TM, KH, 2, PASS>(p, ep, dPQ, lds, stream);
+    }
+  }
   // every block slot of the GPU; smaller problems: a wave per tile, in whole blocks per XCD when there are enough tiles
   const int full = 256 * (fast && !ep.mask ? stream_blocks_per_cu<TM, KH, true>() : stream_blocks_per_cu<TM, KH, false>());
   const int blocks = p.tiles >= 4 * full ? full : (p.tiles >= 256 ? 8 * cdiv(cdiv(p.tiles, 8), 4) : cdiv(p.tiles, 4));

@@ -56,6 +56,15 @@ CONV_CASES = [
     # enough column tiles (313 / 1250) for the per-XCD ranges, with a ragged last range and tiles that straddle images
     (4, 64, 50, 50, 64, 1, 1, 0),
     (5, 32, 89, 90, 96, 1, 1, 0),
+    # contractions of 96 and more with full row tiles and channel pairs and an even pixel count per image: the form
+    # of the streaming kernel that moves two pixels per lane (forward, masked backward-data) or four (backward-data,
+    # pixel count a multiple of four, up to three row tiles); groups of columns that straddle images and end ragged,
+    # enough groups for the per-XCD ranges; a short contraction beside them (the one-pixel form)
+    (3, 96, 12, 12, 96, 1, 1, 0),
+    (2, 128, 10, 10, 64, 1, 1, 0),
+    (6, 32, 20, 22, 32, 1, 1, 0),
+    (3, 64, 9, 10, 96, 1, 1, 0),
+    (4, 96, 64, 66, 96, 1, 1, 0),
 ]
 
 
