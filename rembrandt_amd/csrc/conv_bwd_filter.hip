@@ -906,8 +906,9 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     switch (plan.bm) {
       case 128: e = run_bwd_filter_1x1<T128x128>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_128x128"); break;
       case 96:
-        e = plan.bn == 128 ? run_bwd_filter_1x1<T96x128>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x128")
-                           : run_bwd_filter_1x1<T96x256>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x256");
+        e = CRS <= 96 ? run_bwd_filter_1x1<T96x96>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x96")
+            : plan.bn == 128 ? run_bwd_filter_1x1<T96x128>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x128")
+                             : run_bwd_filter_1x1<T96x256>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x256");
         break;
       case 64:  e = run_bwd_filter_1x1<T64x256>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_64x256"); break;
       default:  e = run_bwd_filter_1x1<T32x256>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x256"); break;

@@ -139,6 +139,7 @@ inline int launch_mfma_gemm_bf16_dma(const RowV8Params& ap, const RowV8Params& b
 typedef Tile<128, 128, 16, 2, 2, RH_OCC_128> T128x128;
 typedef Tile<96, 256, 16, 1, 4> T96x256;
 typedef Tile<96, 128, 16, 1, 4, 4> T96x128;
+typedef Tile<96, 96, 16, 1, 3, 4> T96x96;   // three waves: a 96 x 96 result (1x1 layer, 96 -> 96 channels) without a quarter of dead columns
 #ifndef RH_BF16_BK
 #define RH_BF16_BK 32
 #endif
