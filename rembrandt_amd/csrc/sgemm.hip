@@ -109,6 +109,75 @@ static int dispatch_tile(int bm, const DenseParams& ap, const DenseParams& bp, c
   }
 }
 
+
+// Products with a side of at most a few dozen (the classifier layer of a small network: 500 -> 10 at batch 64) are
+// microseconds of arithmetic; on the tile engine they cost a contraction kernel of 10-20 us (one tile, a chain of K
+// steps or slices plus their reduction).  Two plain forms with a fixed order of additions:
+//   a wave per result element, lanes along the contraction (k >= 128: both operands of the forward product are
+//   k-contiguous), lane sums added by a butterfly;
+//   a thread per result element, consecutive threads along C's rows (k < 128: data gradient, weight gradient).
+// A(im, l) = A[im sa_m + l sa_k], B(l, jn) = B[l sb_k + jn sb_n]; epilogue as the tile engine's.
+struct SkinnyArgs {
+  const float* A; const float* B; float* C; const float* bias_col;
+  int m, n, k, sa_m, sa_k, sb_k, sb_n, ldc, relu;
+  float alpha, beta;
+};
+
+__device__ __forceinline__ void skinny_store(const SkinnyArgs& a, int im, int jn, float sum) {
+  float* c = a.C + (size_t)jn * a.ldc + im;
+  float val = a.alpha * sum;
+  if (a.beta != 0.0f) val += a.beta * *c;
+  if (a.bias_col) val += a.bias_col[im];
+  if (a.relu) val = val > 0.0f ? val : 0.0f;
+  *c = val;
+}
+
+__global__ __launch_bounds__(256) void sgemm_skinny_wave_kernel(SkinnyArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);   // result element: im fastest
+  if (e >= a.m * a.n) return;
+  const int jn = e / a.m, im = e - jn * a.m;
+  const float* pa = a.A + (size_t)im * a.sa_m;
+  const float* pb = a.B + (size_t)jn * a.sb_n;
+  float s0 = 0.0f, s1 = 0.0f;
+  int l = lane;
+  for (; l + 64 < a.k; l += 128) {
+    s0 = fmaf(pa[(size_t)l * a.sa_k], pb[(size_t)l * a.sb_k], s0);
+    s1 = fmaf(pa[(size_t)(l + 64) * a.sa_k], pb[(size_t)(l + 64) * a.sb_k], s1);
+  }
+  if (l < a.k) s0 = fmaf(pa[(size_t)l * a.sa_k], pb[(size_t)l * a.sb_k], s0);
+  float sum = s0 + s1;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  if (lane == 0) skinny_store(a, im, jn, sum);
+}
+
+__global__ __launch_bounds__(256) void sgemm_skinny_thread_kernel(SkinnyArgs a) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= a.m * a.n) return;
+  const int jn = e / a.m, im = e - jn * a.m;
+  const float* pa = a.A + (size_t)im * a.sa_m;
+  const float* pb = a.B + (size_t)jn * a.sb_n;
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  int l = 0;
+  for (; l + 3 < a.k; l += 4) {
+    s0 = fmaf(pa[(size_t)l * a.sa_k], pb[(size_t)l * a.sb_k], s0);
+    s1 = fmaf(pa[(size_t)(l + 1) * a.sa_k], pb[(size_t)(l + 1) * a.sb_k], s1);
+    s2 = fmaf(pa[(size_t)(l + 2) * a.sa_k], pb[(size_t)(l + 2) * a.sb_k], s2);
+    s3 = fmaf(pa[(size_t)(l + 3) * a.sa_k], pb[(size_t)(l + 3) * a.sb_k], s3);
+  }
+  for (; l < a.k; ++l) s0 = fmaf(pa[(size_t)l * a.sa_k], pb[(size_t)l * a.sb_k], s0);
+  skinny_store(a, im, jn, (s0 + s1) + (s2 + s3));
+}
+
+// 0: the tile engine; 1: a wave per element; 2: a thread per element
+static int skinny_mode(int m, int n, int k) {
+  const long long mn = (long long)m * n;
+  if (k >= 128) return mn <= 4096 && (m <= 16 || n <= 16) ? 1 : 0;
+  if (k >= 1 && mn * k <= (1ll << 22) && (m <= 16 || n <= 16 || k <= 16)) return 2;
+  return 0;
+}
+
 // y[i] += alpha * x[i]
 __global__ void saxpy_kernel(long long n, float alpha, const float* __restrict__ x, float* __restrict__ y) {
   const long long stride = (long long)gridDim.x * blockDim.x;
@@ -196,6 +265,21 @@ extern "C" int rh_sgemm_bias_act(int transA, int transB, int32_t m, int32_t n, i
       ((size_t)ldc * (n - 1) + m) * 4 > kMaxBufferBytes)
     return RH_E_LIMIT;
 
+  if (!(flags & RH_ALGO_GATHER)) {
+    if (const int mode = skinny_mode(m, n, k)) {
+      SkinnyArgs a;
+      a.A = A; a.B = B; a.C = C; a.bias_col = bias_col;
+      a.m = m; a.n = n; a.k = k; a.ldc = ldc; a.relu = relu; a.alpha = alpha; a.beta = beta;
+      a.sa_m = transA ? lda : 1; a.sa_k = transA ? 1 : lda;
+      a.sb_k = transB ? ldb : 1; a.sb_n = transB ? 1 : ldb;
+      ProfScope prof("sgemm_skinny", 2.0 * (double)m * n * k, stream);
+      if (mode == 1)
+        hipLaunchKernelGGL(sgemm_skinny_wave_kernel, dim3((unsigned)cdiv(m * n, 4)), dim3(256), 0, stream, a);
+      else
+        hipLaunchKernelGGL(sgemm_skinny_thread_kernel, dim3((unsigned)cdiv(m * n, 256)), dim3(256), 0, stream, a);
+      return launch_status();
+    }
+  }
   DenseParams ap;  // engine A operand = opB, rows = n
   ap.ptr = B; ap.bytes = (uint32_t)(b_elems * 4); ap.rows = n; ap.K = k; ap.ld = ldb; ap.ktab = nullptr;
   DenseParams bp;  // engine B operand = opA, rows = m

@@ -196,6 +196,15 @@ SGEMM_CASES = [
     (0, 0, 1, 10, 64),
     (0, 1, 1, 130, 70),      # the bias-gradient GEMV shape
     (1, 0, 4096, 32, 1024),  # few tiles, deep contraction -> split path
+    # a side of at most sixteen: the plain kernels (a wave per element for long contractions, a thread per element
+    # otherwise): a ten-class classifier's forward, data-gradient and weight-gradient products, every transposition
+    (1, 0, 10, 64, 500),
+    (0, 0, 500, 64, 10),
+    (0, 1, 500, 10, 64),
+    (0, 1, 64, 10, 128),
+    (1, 1, 10, 33, 200),
+    (1, 0, 16, 256, 129),
+    (0, 0, 3, 5, 1),
 ]
 
 
@@ -222,7 +231,7 @@ def test_sgemm(dev, case, use_ws):
 @pytest.mark.parametrize("case", [
     # (m = out channels, n = batch, k = in channels): one block, several tiles, a split contraction with the dense
     # 16-byte reduction, one with the many-slice reduction, odd extents with a padded result (scalar reduction)
-    (10, 4, 50), (500, 64, 800), (4096, 32, 1024), (96, 16, 9216), (1001, 33, 2450), (1000, 256, 4096),
+    (10, 4, 50), (10, 64, 500), (500, 64, 800), (4096, 32, 1024), (96, 16, 9216), (1001, 33, 2450), (1000, 256, 4096),
 ])
 def test_sgemm_bias_act(dev, case):
     """rh_sgemm_bias_act = matrix product, bias row, activation of the affine forward pass in one call: bit-identical
