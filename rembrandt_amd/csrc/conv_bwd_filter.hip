@@ -12,14 +12,15 @@ namespace rh {
 
 // Column tile (filter taps) for a row tile: 128-row tiles pair with 128 columns; narrower row tiles take 256
 // columns unless 128 pads the tap count less (AlexNet conv1: 363 taps = 3 x 128 - 21 instead of 2 x 256 - 149).
-static int pick_bn(int bm, int cols) {
+static int pick_bn(int bm, int cols, bool narrow = false) {
   if (bm == 128) return 128;
+  if (narrow && bm == 32 && cols <= 128) return cols <= 64 ? 64 : 128;
   if (bm == 96 && round_up(cols, 128) < round_up(cols, 256)) return 128;
   return 256;
 }
 // Blocks of a tile shape that one CU holds at a time (registers and LDS), times 256 CUs.
 static int resident_slots(int bm, int bn) {
-  return 256 * (bm == 128 ? RH_OCC_128 : bm == 96 ? (bn == 128 ? 4 : 2) : 3);
+  return 256 * (bm == 128 ? RH_OCC_128 : bm == 96 ? (bn == 128 ? 4 : 2) : (bm == 32 && bn <= 128) ? 4 : 3);
 }
 
 struct BwdFilterPlan {
@@ -31,7 +32,7 @@ static BwdFilterPlan plan_bwd_filter(const ConvDims& d) {
   BwdFilterPlan p;
   const int CRS = d.C * d.R * d.S;
   p.bm = pick_bm(d.K);
-  p.bn = pick_bn(p.bm, CRS);
+  p.bn = pick_bn(p.bm, CRS, !(d.R == 1 && d.S == 1 && d.st == 1 && d.pad == 0));
   p.tiles = cdiv(d.K, p.bm) * cdiv(CRS, p.bn);
   const long long M = (long long)d.N * d.P * d.Q;
   const int k_chunks = (int)cdiv<long long>(M, 16);
@@ -937,7 +938,11 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
                            : run_bwd_filter<T96x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_96x256");
         break;
       case 64:  e = run_bwd_filter<T64x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_64x256"); break;
-      default:  e = run_bwd_filter<T32x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x256"); break;
+      default:
+        e = plan.bn == 64    ? run_bwd_filter<T32x64>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x64")
+            : plan.bn == 128 ? run_bwd_filter<T32x128>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x128")
+                             : run_bwd_filter<T32x256>(ap, bp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x256");
+        break;
     }
     if (e) return e;
   }

@@ -152,6 +152,9 @@ typedef Tile<128, 128, RH_BF16_BK, 2, 2, RH_BF16_OCC> T128x128bf;
 typedef Tile<256, 256, 32, 2, 4, 1> T256x256bf;
 typedef Tile<64, 256, 16, 1, 4, 3> T64x256;
 typedef Tile<32, 256, 16, 1, 4, 3> T32x256;
+// few result columns as well (a first layer's filter gradient: 20 x 25, 32 x 75): narrower tiles, fewer dead columns
+typedef Tile<32, 128, 16, 1, 4, 4> T32x128;
+typedef Tile<32, 64, 16, 1, 2, 4> T32x64;
 // Half the K step: 20 KB of LDS, so a CU holds 4 blocks instead of 3.  For grids that need a second round of
 // blocks at 3 per CU but fit in one at 4 (e.g. 64 output channels over 64 x 56 x 56 pixels: 784 tiles).
 typedef Tile<64, 256, 8, 1, 4, 4> T64x256k8;
