@@ -113,9 +113,9 @@ static int dispatch_tile(int bm, const DenseParams& ap, const DenseParams& bp, c
 // Products with a side of at most a few dozen (the classifier layer of a small network: 500 -> 10 at batch 64) are
 // microseconds of arithmetic; on the tile engine they cost a contraction kernel of 10-20 us (one tile, a chain of K
 // steps or slices plus their reduction).  Two plain forms with a fixed order of additions:
-//   a wave per result element, lanes along the contraction (k >= 128: both operands of the forward product are
-//   k-contiguous), lane sums added by a butterfly;
-//   a thread per result element, consecutive threads along C's rows (k < 128: data gradient, weight gradient).
+//   a wave per result element, lanes along the contraction (k >= 64 and at most 4096 elements: both operands of the
+//   forward product are k-contiguous), lane sums added by a butterfly;
+//   a thread per result element, consecutive threads along C's rows (k < 128 otherwise: data gradient, weight gradient).
 // A(im, l) = A[im sa_m + l sa_k], B(l, jn) = B[l sb_k + jn sb_n]; epilogue as the tile engine's.
 struct SkinnyArgs {
   const float* A; const float* B; float* C; const float* bias_col;
@@ -158,8 +158,24 @@ __global__ __launch_bounds__(256) void sgemm_skinny_thread_kernel(SkinnyArgs a) 
   const int jn = e / a.m, im = e - jn * a.m;
   const float* pa = a.A + (size_t)im * a.sa_m;
   const float* pb = a.B + (size_t)jn * a.sb_n;
+  // four running sums; sixteen steps (thirty-two loads) per trip, so that a thread waits for memory once per trip
   float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
   int l = 0;
+  for (; l + 15 < a.k; l += 16) {
+    float va[16], vb[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      va[u] = pa[(size_t)(l + u) * a.sa_k];
+      vb[u] = pb[(size_t)(l + u) * a.sb_k];
+    }
+#pragma unroll
+    for (int u = 0; u < 16; u += 4) {
+      s0 = fmaf(va[u], vb[u], s0);
+      s1 = fmaf(va[u + 1], vb[u + 1], s1);
+      s2 = fmaf(va[u + 2], vb[u + 2], s2);
+      s3 = fmaf(va[u + 3], vb[u + 3], s3);
+    }
+  }
   for (; l + 3 < a.k; l += 4) {
     s0 = fmaf(pa[(size_t)l * a.sa_k], pb[(size_t)l * a.sb_k], s0);
     s1 = fmaf(pa[(size_t)(l + 1) * a.sa_k], pb[(size_t)(l + 1) * a.sb_k], s1);
@@ -173,7 +189,8 @@ __global__ __launch_bounds__(256) void sgemm_skinny_thread_kernel(SkinnyArgs a) 
 // 0: the tile engine; 1: a wave per element; 2: a thread per element
 static int skinny_mode(int m, int n, int k) {
   const long long mn = (long long)m * n;
-  if (k >= 128) return mn <= 4096 && (m <= 16 || n <= 16) ? 1 : 0;
+  if (k >= 64 && mn <= 4096 && (m <= 16 || n <= 16)) return 1;
+  if (k >= 128) return 0;
   if (k >= 1 && mn * k <= (1ll << 22) && (m <= 16 || n <= 16 || k <= 16)) return 2;
   return 0;
 }
