@@ -170,9 +170,24 @@ __global__ __launch_bounds__(256) void softmax_kl_step_kernel(const float* __res
   if (!last) return;
   __threadfence();
   float acc = 0.0f;
-  for (int i = threadIdx.x; i < N; i += blockDim.x)
-    acc += __hip_atomic_load(loss1 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  acc = block_reduce_sum(acc, sm);
+  if (blockDim.x == 64) {
+    // one wave adds in the order 256 threads would: lane l stands for threads l, 64 + l, 128 + l, 192 + l, each of the
+    // four groups goes through the wave's tree, and the four results are added in wave order
+    float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      for (int i = 64 * w + (int)threadIdx.x; i < N; i += 256)
+        part[w] += __hip_atomic_load(loss1 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int o = 32; o > 0; o >>= 1) part[w] += __shfl_down(part[w], o, 64);
+    }
+    acc = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) acc += part[w];
+  } else {
+    for (int i = threadIdx.x; i < N; i += blockDim.x)
+      acc += __hip_atomic_load(loss1 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    acc = block_reduce_sum(acc, sm);
+  }
   if (threadIdx.x == 0) {
     loss_sum[0] = acc;
     *counter = 0u;
@@ -238,7 +253,9 @@ extern "C" int rh_softmax_kl_step(const float* x, int32_t C, int32_t N, const in
     return RH_E_INVALID;
   if (N == 0) return 0;
   ProfScope prof("softmax_kl_step", 16.0 * (double)C * N, to_stream(stream));
-  hipLaunchKernelGGL(softmax_kl_step_kernel, dim3(N), dim3(256), 0, to_stream(stream), x, C, N, labels, weights, p, max_out,
-                     idx_out, loss1, loss_sum, dx, counter);
+  // Up to 64 categories one wave holds a whole row: the other three would only add identities to the block's reductions
+  // (same bits) and take part in its barriers and its fence.
+  hipLaunchKernelGGL(softmax_kl_step_kernel, dim3(N), dim3(C <= 64 ? 64 : 256), 0, to_stream(stream), x, C, N, labels, weights,
+                     p, max_out, idx_out, loss1, loss_sum, dx, counter);
   return launch_status();
 }
