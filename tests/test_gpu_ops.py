@@ -65,6 +65,11 @@ CONV_CASES = [
     (6, 32, 20, 22, 32, 1, 1, 0),
     (3, 64, 9, 10, 96, 1, 1, 0),
     (4, 96, 64, 66, 96, 1, 1, 0),
+    # filter gradients of at most 32 x 64 and 32 x 128 (first layers): the narrow tiles of the gather path
+    (4, 1, 12, 12, 20, 5, 1, 2),
+    (3, 3, 10, 11, 32, 5, 1, 2),
+    (2, 2, 9, 9, 8, 3, 2, 1),
+    (2, 4, 8, 8, 30, 5, 1, 0),
 ]
 
 
