@@ -271,8 +271,12 @@ static int bwd_data_impl(const rh_conv_geom* g, float alpha, const float* w, con
       case 64:
         if (cdiv(d.C, 64) == 1 && prefer_k8_64(ep.cols))
           return run_bwd_data_soff<T64x256k8>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_64x256k8", sp.splits, part, &sp.tail);
+        // (sliced contractions on the half-width tile, as in the forward pass)
+        if (sp.splits > 1) return run_bwd_data_soff<T64x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_64x128", sp.splits, part, &sp.tail);
         return run_bwd_data_soff<T64x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_64x256", sp.splits, part, &sp.tail);
-      default:  return run_bwd_data_soff<T32x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_32x256", sp.splits, part, &sp.tail);
+      default:
+        if (sp.splits > 1) return run_bwd_data_soff<T32x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_32x128", sp.splits, part, &sp.tail);
+        return run_bwd_data_soff<T32x256>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_32x256", sp.splits, part, &sp.tail);
     }
   }
   const int n_tab = round_up(KRS, kTabPad);

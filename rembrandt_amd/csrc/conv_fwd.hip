@@ -573,8 +573,13 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
       case 64:
         if (cdiv(d.K, 64) == 1 && prefer_k8_64(ep.cols))
           return run_fwd_soff<T64x256k8>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x256k8", sp.splits, part, &sp.tail);
+        // a sliced contraction (a small layer) on the half-width tile: twice the blocks over the same slices, so that a
+        // CU has others to run while one waits for its next K step's loads
+        if (sp.splits > 1) return run_fwd_soff<T64x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x128", sp.splits, part, &sp.tail);
         return run_fwd_soff<T64x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_64x256", sp.splits, part, &sp.tail);
-      default:  return run_fwd_soff<T32x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_32x256", sp.splits, part, &sp.tail);
+      default:
+        if (sp.splits > 1) return run_fwd_soff<T32x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_32x128", sp.splits, part, &sp.tail);
+        return run_fwd_soff<T32x256>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_32x256", sp.splits, part, &sp.tail);
     }
   }
   const int n_tab = round_up(CRS, kTabPad);
