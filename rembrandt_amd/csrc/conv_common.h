@@ -155,6 +155,7 @@ typedef Tile<32, 256, 16, 1, 4, 3> T32x256;
 // few result columns as well (a first layer's filter gradient: 20 x 25, 32 x 75): narrower tiles, fewer dead columns
 typedef Tile<32, 128, 16, 1, 4, 4> T32x128;
 typedef Tile<32, 64, 16, 1, 2, 4> T32x64;
+typedef Tile<128, 64, 16, 2, 2, 4> T128x64;   // sliced forward contractions (small images late in a network)
 typedef Tile<64, 128, 16, 1, 4, 4> T64x128;   // sliced forward / backward-data contractions of small layers
 // Half the K step: 20 KB of LDS, so a CU holds 4 blocks instead of 3.  For grids that need a second round of
 // blocks at 3 per CU but fit in one at 4 (e.g. 64 output channels over 64 x 56 x 56 pixels: 784 tiles).
