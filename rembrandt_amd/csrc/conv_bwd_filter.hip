@@ -615,14 +615,24 @@ __global__ __launch_bounds__(1024) void bwd_bias_kernel(const float* __restrict_
   float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
   for (int n = wave; n < N; n += nwaves) {
     const float* p = dy + ((size_t)n * K + k) * plane;
-    int i = lane;
-    for (; i + 192 < plane; i += 256) {
-      a0 += p[i];
-      a1 += p[i + 64];
-      a2 += p[i + 128];
-      a3 += p[i + 192];
+    // sixteen loads of a plane in flight per lane, added in the order of the plain loop (groups of four strides to
+    // a0..a3 while four are left, the rest to a0)
+    for (int i0 = lane; i0 < plane; i0 += 1024) {
+      float v[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) v[j] = i0 + 64 * j < plane ? p[i0 + 64 * j] : 0.0f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int i = i0 + 256 * g;
+        if (i + 192 < plane) {
+          a0 += v[4 * g]; a1 += v[4 * g + 1]; a2 += v[4 * g + 2]; a3 += v[4 * g + 3];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (i + 64 * e < plane) a0 += v[4 * g + e];
+        }
+      }
     }
-    for (; i < plane; i += 64) a0 += p[i];
   }
   float acc = (a0 + a1) + (a2 + a3);
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
