@@ -176,9 +176,9 @@ struct TailSplit {
   int full_tiles, tail_tiles, splits;
   long long col0;  // first column of the tail
 };
-inline TailSplit plan_tail_split(int rows, long long cols, int n_k) {
+inline TailSplit plan_tail_split(int rows, long long cols, int n_k, int bn_force = 0) {
   TailSplit t = {0, 0, 1, 0};
-  const int bm = pick_bm(rows), bn = bm >= 96 ? 128 : 256;
+  const int bm = pick_bm(rows), bn = bn_force ? bn_force : bm >= 96 ? 128 : 256;
   const int tiles_m = cdiv(rows, bm);
   const long long tiles_n = cdiv<long long>(cols, bn), T = tiles_m * tiles_n;
   const bool k8 = bm == 64 && tiles_m == 1 && prefer_k8_64(cols);  // the 64x256 tile with the halved K step: 4 per CU
@@ -218,6 +218,7 @@ struct SoffPlan {
   size_t tab_bytes, wt_bytes, img_bytes;  // img_bytes == 0: the image is used in place
   int splits;      // > 1: the contraction is cut into this many slices, partial results in part_bytes of scratch
   TailSplit tail;  // tail.splits > 1: only the last tiles are cut (splits == 1 then)
+  bool narrow128 = false;  // forward, 128-row tiles: the 128 x 64 tile, planned as such
   size_t part_bytes;
   bool ok;         // false: fall back to the per-element gather path
   size_t total() const { return tab_bytes + wt_bytes + img_bytes + part_bytes; }
@@ -238,8 +239,8 @@ inline long long slices_by_depth(long long k_steps, long long tiles, long long s
   return by < 1 ? 1 : by;
 }
 
-inline int plan_k_split(int rows, long long cols, int n_k) {
-  const int bm = pick_bm(rows), bn = bm >= 96 ? 128 : 256;
+inline int plan_k_split(int rows, long long cols, int n_k, int bn_force = 0) {
+  const int bm = pick_bm(rows), bn = bn_force ? bn_force : bm >= 96 ? 128 : 256;
   const long long slots = 256 * (bm >= 96 ? 4 : 3);
   const long long tiles = (long long)cdiv(rows, bm) * cdiv<long long>(cols, bn);
   if (tiles * 2 > slots) return 1;
@@ -270,6 +271,14 @@ inline SoffPlan plan_soff_fwd(const ConvDims& d) {
   p.ok = img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
   p.splits = plan_k_split(d.K, (long long)d.N * d.P * d.Q, p.n_k);
   p.tail = plan_tail_split(d.K, (long long)d.N * d.P * d.Q, p.n_k);
+  if (pick_bm(d.K) == 128 && p.splits > 1) {
+    // Few 128 x 128 tiles (small images late in a network): the half-width tile, planned as such.  Twice the tiles often
+    // need no slices any more, only a cut of the tiles past the last multiple of 256 (NIN's 1024-channel layers on
+    // 6 x 6: 576 tiles = 512 + 64 in eight slices, instead of 288 x 3 with a reduction over the whole result).
+    p.narrow128 = true;
+    p.splits = plan_k_split(d.K, (long long)d.N * d.P * d.Q, p.n_k, 64);
+    p.tail = plan_tail_split(d.K, (long long)d.N * d.P * d.Q, p.n_k, 64);
+  }
   const size_t tail_elems_f = (size_t)(d.y_elems - tail_first_elem(p.tail, (long long)d.P * d.Q, d.K));
   p.part_bytes = p.splits > 1 ? align256(sizeof(float) * (size_t)p.splits * (size_t)d.y_elems)
                : p.tail.splits > 1 ? align256(sizeof(float) * (size_t)p.tail.splits * tail_elems_f) : 0;

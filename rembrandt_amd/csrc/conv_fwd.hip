@@ -570,7 +570,7 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
     switch (pick_bm(d.K)) {
       case 128:
         // (sliced contractions on the half-width tile, as below: NIN's 6 x 6 layers 4-7 % faster)
-        if (sp.splits > 1) return run_fwd_soff<T128x64>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_128x64", sp.splits, part, &sp.tail);
+        if (sp.narrow128) return run_fwd_soff<T128x64>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_128x64", sp.splits, part, &sp.tail);
         return run_fwd_soff<T128x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_128x128", sp.splits, part, &sp.tail);
       case 96:  return run_fwd_soff<T96x128>(ap, bp, ep, sp.n_k, CRS, stream, "conv_fwd_96x128", sp.splits, part, &sp.tail);
       case 64:
