@@ -266,7 +266,9 @@ static int bwd_data_impl(const rh_conv_geom* g, float alpha, const float* w, con
     ep.mask = mask;
     float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes + sp.wt_bytes + sp.img_bytes);
     switch (pick_bm(d.C)) {
-      case 128: return run_bwd_data_soff<T128x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_128x128", sp.splits, part, &sp.tail);
+      case 128:
+        if (sp.narrow128) return run_bwd_data_soff<T128x64>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_128x64", sp.splits, part, &sp.tail);
+        return run_bwd_data_soff<T128x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_128x128", sp.splits, part, &sp.tail);
       case 96:  return run_bwd_data_soff<T96x128>(ap, bp, ep, sp.n_k, KRS, stream, "conv_bwd_data_96x128", sp.splits, part, &sp.tail);
       case 64:
         if (cdiv(d.C, 64) == 1 && prefer_k8_64(ep.cols))

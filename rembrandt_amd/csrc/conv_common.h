@@ -343,6 +343,13 @@ inline SoffPlan plan_soff_bwd_data(const ConvDims& d) {
   p.ok = p.halo >= 0 && d.R == d.S && img <= kMaxBufferBytes && d.P > 0 && d.Q > 0;
   p.splits = plan_k_split(d.C, (long long)d.N * d.H * d.W, p.n_k);
   p.tail = plan_tail_split(d.C, (long long)d.N * d.H * d.W, p.n_k);
+  if (pick_bm(d.C) == 128 && p.splits > 1 && plan_k_split(d.C, (long long)d.N * d.H * d.W, p.n_k, 64) == 1) {
+    // As in the forward pass, where 128 x 64 tiles need no slices (NIN's 1024-channel 1x1 layers: 0.120 -> 0.098 ms).
+    // Where they would still be sliced the 128 x 128 tile stays (a 384-channel 3x3 layer on 6 x 6 lost 9 %).
+    p.narrow128 = true;
+    p.splits = 1;
+    p.tail = plan_tail_split(d.C, (long long)d.N * d.H * d.W, p.n_k, 64);
+  }
   if (d.st > 1) p.tail.splits = 1;  // the zero-dilated form is a fallback only
   const size_t tail_elems_b = (size_t)(d.x_elems - tail_first_elem(p.tail, (long long)d.H * d.W, d.C));
   p.part_bytes = p.splits > 1 ? align256(sizeof(float) * (size_t)p.splits * (size_t)d.x_elems)
