@@ -217,6 +217,178 @@ def bench_bf16_forward(args, lib, net, cfg, batch, seed):
     }))
 
 
+def _dominant(kernels, prefix=None):
+    """The contraction kernel tag that takes the most time of a step (optionally among tags with a prefix)."""
+    c = [k for k in kernels if k["bound"] == "mfma" and (prefix is None or k["kernel"].startswith(prefix))]
+    return c[0] if c else (kernels[0] if kernels else None)
+
+
+def _roof(k):
+    return None if k is None else {"bound": k["bound"], "kernel": k["kernel"], "achieved": k["achieved"], "peak": k["peak"],
+                                   "unit": k["unit"], "frac": k["frac"], "avg_launch_ms": k["avg_launch_ms"],
+                                   "launches_per_step": k["launches_per_step"]}
+
+
+def short_train_leg(lib, name, steps, warmup):
+    """One of the other benchmark networks through the same train step as the headline: images/s over `steps` timed
+    steps, launches per step and the dominant contraction kernel's roofline position (HIP events, untimed pass)."""
+    import torch
+    from rembrandt_amd import configs, synth
+    from rembrandt_amd.operator import SequentialOperatorWorker, SgdOpt
+    net = configs.NETWORKS[name]()
+    dims, layers, ncat = net
+    batch = BATCH[name]
+    seed = NUM_CLASSES_SEED + 4
+    cfg = configs.build_config(net)
+    worker = SequentialOperatorWorker(cfg, batch, "Backward", shared_seed=(seed, seed + 1), device=0)
+    worker.init_params()
+    x = synth.uniform(seed, 100, (batch, dims[2], dims[1], dims[0])) if name == "lenet" else \
+        synth.normal(seed, 100, (batch, dims[2], dims[1], dims[0]))
+    worker.load_frames_f32(x)
+    worker.stage_batch(synth.integers(seed, 200, (batch,), ncat), 1.0 / batch)
+    sgd = SgdOpt(batch, 0.01, ("Update", 0.9), 5e-4 if name == "lenet" else 0.0)
+    sgd.begin(worker)
+    for _ in range(warmup):
+        sgd.train_batch(worker, batch, fused=True)
+    worker.sync()
+    n = max(1, min(steps, 10))
+    worker.set_overlap_backward(False)
+    lib.rh_profile_reset()
+    lib.rh_profile_filter(None)
+    lib.rh_profile_enable(1)
+    for _ in range(n):
+        sgd.train_batch(worker, batch, fused=True)
+    worker.sync()
+    lib.rh_profile_enable(0)
+    kernels = collect_profile(lib, n)
+    lib.rh_profile_reset()
+    worker.set_overlap_backward(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sgd.train_batch(worker, batch, fused=True)
+    worker.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    worker.close()
+    flops = configs.train_flops(net, batch)
+    mfma_ms = sum(k["ms_per_step"] for k in kernels if k["bound"] == "mfma")
+    return {"metric": "train images/sec (fwd+bwd+SGD) %s b%d fp32" % (name, batch), "value": batch * steps / dt,
+            "unit": "images/sec", "ms_per_step": dt / steps * 1e3, "steps": steps, "dtype": "f32",
+            "launches_per_step": sum(k["launches_per_step"] for k in kernels),
+            "gemm_gflop_per_step": flops / 1e9,
+            "step_frac_of_mfma_peak": flops / (dt / steps) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+            "all_mfma": {"ms_per_step": mfma_ms, "frac": flops / mfma_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS if mfma_ms else None},
+            "roofline": _roof(_dominant(kernels))}
+
+
+def short_bf16_forward_leg(lib, name, steps, warmup):
+    """Forward pass alone, inference phase, bf16 convolution operands with fp32 accumulation."""
+    import torch
+    from rembrandt_amd import configs, synth
+    from rembrandt_amd.operator import SequentialOperatorWorker
+    net = configs.NETWORKS[name]()
+    dims, layers, ncat = net
+    batch = BATCH[name]
+    seed = NUM_CLASSES_SEED + 4
+    worker = SequentialOperatorWorker(configs.build_config(net), batch, "Forward", shared_seed=(seed, seed + 1), device=0,
+                                      bf16_forward=True)
+    worker.init_params()
+    worker.load_frames_f32(synth.normal(seed, 100, (batch, dims[2], dims[1], dims[0])))
+    for _ in range(warmup):
+        worker.forward(batch, training=False, t=0)
+    worker.sync()
+    n = max(1, min(steps, 10))
+    lib.rh_profile_reset()
+    lib.rh_profile_filter(None)
+    lib.rh_profile_enable(1)
+    for _ in range(n):
+        worker.forward(batch, training=False, t=0)
+    worker.sync()
+    lib.rh_profile_enable(0)
+    kernels = collect_profile(lib, n)
+    lib.rh_profile_reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        worker.forward(batch, training=False, t=0)
+    worker.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    worker.close()
+    flops = configs.train_flops(net, batch, forward_only=True)
+    conversions = [k for k in kernels if k["kernel"].startswith("nchw_to_bf16") or k["kernel"].startswith("bf16_filter")]
+    return {"metric": "inference images/sec (forward only) %s b%d, bf16 conv operands, fp32 accumulation" % (name, batch),
+            "value": batch * steps / dt, "unit": "images/sec", "ms_per_step": dt / steps * 1e3, "steps": steps,
+            "dtype": "bf16 operands, f32 accumulate", "launches_per_step": sum(k["launches_per_step"] for k in kernels),
+            "gemm_gflop_per_step": flops / 1e9,
+            "step_frac_of_bf16_mfma_peak": flops / (dt / steps) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+            "operand_conversion_ms_per_step": sum(k["ms_per_step"] for k in conversions),
+            "operand_conversion_launches_per_step": sum(k["launches_per_step"] for k in conversions),
+            "roofline": _roof(_dominant(kernels, "conv_fwd_bf16"))}
+
+
+SWEEP = {  # the single-operator sweep: N, C, H, W, K, R, stride, pad
+    "a_5x5_96to256_27x27_b256": (256, 96, 27, 27, 256, 5, 1, 2),
+    "b_3x3_256to384_13x13_b256": (256, 256, 13, 13, 384, 3, 1, 1),
+    "c_1x1_96to96_55x55_b128": (128, 96, 55, 55, 96, 1, 1, 0),
+}
+
+
+def conv_sweep_leg(iters, warmup):
+    """Forward, backward-data and backward-filter of the three sweep shapes, each call timed alone (HIP events on the
+    stream the kernels run on; a call includes the operand copies it makes): ms, TFLOP/s against the fp32 matrix peak and
+    algorithmic bytes (x, w, y once) per second against the HBM peak: the 1x1 shape sits on the ridge of both roofs."""
+    import torch
+    from rembrandt_amd import ops
+    dev = torch.device("cuda:0")
+    out = {}
+    for name, (N, C, H, W, K, R, st, pad) in SWEEP.items():
+        g = torch.Generator(device=dev)
+        g.manual_seed(1234)
+        x = torch.randn(N, C, H, W, device=dev, generator=g)
+        w = torch.randn(K, C, R, R, device=dev, generator=g)
+        y = ops.conv2d_fwd(x, w, st, pad)
+        dy = torch.randn(y.shape, device=dev, generator=g)
+        dw, dx = torch.zeros_like(w), torch.zeros_like(x)
+        flops = 2.0 * y.numel() * C * R * R
+        byts = 4.0 * (x.numel() + w.numel() + y.numel())
+        calls = {"fwd": lambda: ops.conv2d_fwd(x, w, st, pad, y=y),
+                 "bwd_data": lambda: ops.conv2d_bwd_data(w, dy, x.shape, st, pad, dx=dx),
+                 "bwd_filter": lambda: ops.conv2d_bwd_filter(x, dy, w.shape, st, pad, dw=dw)}
+        row = {"gflop": flops / 1e9, "algorithmic_mb": byts / 1e6}
+        for pname, fn in calls.items():
+            for _ in range(warmup):
+                fn()
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for _ in range(iters):
+                fn()
+            e.record()
+            torch.cuda.synchronize()
+            ms = s.elapsed_time(e) / iters
+            row[pname] = {"ms": ms, "tflops": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS,
+                          "gbs": byts / ms / 1e6, "frac_hbm": byts / ms / 1e6 / PEAK_HBM_GBS}
+        out[name] = row
+        del x, w, y, dy, dw, dx
+    return out
+
+
+def other_configs(lib):
+    """The benchmark configurations other than the headline one, run after the timed region (a few seconds together)."""
+    out = {}
+    for key, fn in (("lenet_b64_train", lambda: short_train_leg(lib, "lenet", 200, 20)),
+                    ("cifar10_b128_train", lambda: short_train_leg(lib, "cifar10", 200, 20)),
+                    ("nin_b128_train", lambda: short_train_leg(lib, "nin", 20, 3)),
+                    ("nin_b128_bf16_forward", lambda: short_bf16_forward_leg(lib, "nin", 50, 5)),
+                    ("conv_sweep", lambda: conv_sweep_leg(20, 3))):
+        t0 = time.perf_counter()
+        out[key] = fn()
+        out[key]["leg_seconds"] = time.perf_counter() - t0
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -238,6 +410,9 @@ def main():
     ap.add_argument("--bf16-forward", action="store_true",
                     help="forward pass only (inference phase) with bf16 convolution operands and fp32 accumulation; "
                          "reports inference images/sec and the bf16 kernel against the bf16 matrix peak")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short legs over the other benchmark configurations (LeNet, CIFAR-10, NIN fp32 / bf16 "
+                         "forward, the convolution sweep) that the default alexnet run appends as `other_configs`")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="first launch the library's plain copy kernel 4 times over MIB MiB (a known-size "
                          "reference for hardware byte counters collected around this command)")
@@ -387,6 +562,9 @@ def main():
         "kernels": kernels,
         "final_loss": loss,
     }
+    if args.workload == "alexnet" and not args.no_other_configs and not args.unfused and not args.graph:
+        worker.close()
+        result["other_configs"] = other_configs(lib)
     if args.cpu_sample > 0:
         result["cpu_baseline"] = cpu_baseline(net, args.cpu_sample)
     print(json.dumps(result))

@@ -416,13 +416,6 @@ int rh_probe_mfma_loop(int blocks, int nacc, int iters, float* sink, rh_stream_t
 /* The same loop on operands that differ per lane and per instruction (realistic data toggling and power draw). */
 int rh_probe_mfma_loop_varied(int blocks, int iters, float* sink, rh_stream_t stream);
 int rh_probe_copy(const float* src, float* dst, size_t n, rh_stream_t stream);
-/* What the bf16 kernels are designed against (no counterpart in the reference): a register-only loop of
- * v_mfma_f32_32x32x16_bf16 (blocks x 4 waves, iters * 16 MFMAs of 32768 FLOP each), and the rates of the ways into and
- * out of the LDS: mode 0 ds_read_b128, 1 ds_write_b128, 2 direct global -> LDS loads from `src` (at least 16 MiB,
- * 16-byte aligned); blocks x threads (256 or 512), 64 bytes per thread and round.  Figures through rh_profile_*. */
-int rh_probe_bf16_mfma_loop(int blocks, int iters, float* sink, rh_stream_t stream);
-int rh_probe_lds_path(int mode, int blocks, int threads, int iters, const float* src, float* sink, rh_stream_t stream);
-
 #ifdef __cplusplus
 }
 #endif

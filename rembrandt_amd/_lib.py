@@ -130,8 +130,6 @@ PROTOTYPES = {
     "rh_probe_mfma_loop": (_int, [_int, _int, _int, _vp, _vp]),
     "rh_probe_mfma_loop_varied": (_int, [_int, _int, _vp, _vp]),
     "rh_probe_copy": (_int, [_vp, _vp, _sz, _vp]),
-    "rh_probe_bf16_mfma_loop": (_int, [_int, _int, _vp, _vp]),
-    "rh_probe_lds_path": (_int, [_int, _int, _int, _int, _vp, _vp, _vp]),
     "rh_rng_fill_uniform": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_normal": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_int": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _i32]),

@@ -4,7 +4,6 @@ bandwidth-bound kernels at AlexNet sizes.
 
     python -m rembrandt_amd.kernel_bench                 # everything, one JSON line per kernel
     python -m rembrandt_amd.kernel_bench conv --layer sweep_b --passes fwd,bwd_filter --iters 3
-    python -m rembrandt_amd.kernel_bench probes          # register-only MFMA loops and the LDS paths (what kernels are designed against)
 
 Times are HIP-event averages over --iters launches after --warmup launches; `frac` is measured against the
 datasheet peaks (fp32 MFMA 157.3 TFLOP/s, bf16 MFMA 2500 TFLOP/s, HBM 8000 GB/s).  A conv "call" includes the
@@ -53,7 +52,7 @@ FC_LAYERS = {"alexnet_fc6": (256, 9216, 4096), "alexnet_fc7": (256, 4096, 4096),
 
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("what", nargs="*", default=["conv", "fc", "mem"], help="conv | fc | mem | probes")
+    ap.add_argument("what", nargs="*", default=["conv", "fc", "mem"], help="conv | fc | mem")
     ap.add_argument("--layer", default=None, help="a prefix of: %s" % ", ".join(list(CONV_LAYERS) + list(FC_LAYERS)))
     ap.add_argument("--passes", default="fwd,bwd_filter,bwd_data,fwd_bf16")
     ap.add_argument("--iters", type=int, default=5)
@@ -87,25 +86,6 @@ def main(argv=None):
         print(json.dumps({"kernel": kernel, "layer": layer, "ms": round(ms, 4), "achieved": round(achieved, 1), "unit": unit,
                           "peak": PEAK[bound], "frac": round(achieved / PEAK[bound], 4)}), flush=True)
 
-    if "probes" in args.what:
-        import ctypes as C_
-        lib = _lib.lib()
-        sink = torch.zeros(16, device=dev)
-        src = torch.randn(4 << 20, device=dev)   # 16 MiB
-        st_ = C_.c_void_p(torch.cuda.current_stream().cuda_stream)
-        sp, cp = C_.c_void_p(sink.data_ptr()), C_.c_void_p(src.data_ptr())
-        report("probe_mfma_fp32_loop", "256 blocks x 4 waves", timeit(lambda: lib.rh_probe_mfma_loop_varied(256, 4000, sp, st_)),
-               256 * 4.0 * 4000 * 16 * 4096.0, "fp32")
-        for blocks in (256, 512):   # one / two waves per SIMD
-            report("probe_mfma_bf16_loop", "%d blocks x 4 waves" % blocks,
-                   timeit(lambda: lib.rh_probe_bf16_mfma_loop(blocks, 8000, sp, st_)), blocks * 4.0 * 8000 * 16 * 32768.0, "bf16")
-        for mode, tag in ((0, "probe_lds_read_b128"), (1, "probe_lds_write_b128"), (2, "probe_lds_direct_load_b128")):
-            for threads in (256, 512):   # one / two waves per SIMD
-                ms = timeit(lambda: lib.rh_probe_lds_path(mode, 256, threads, 4000, cp, sp, st_))
-                byts = 256.0 * threads * 4000 * 64.0
-                print(json.dumps({"kernel": tag, "layer": "256 blocks x %d threads" % threads, "ms": round(ms, 4),
-                                  "achieved": round(byts / ms / 1e9, 1), "unit": "TB/s over 256 CUs",
-                                  "bytes_per_clk_per_cu_at_2.4GHz": round(byts / (ms * 1e-3) / 256 / 2.4e9, 1)}), flush=True)
     if "conv" in args.what:
         for name, (N, C, H, W, K, R, st, pad) in CONV_LAYERS.items():
             if args.layer and not name.startswith(args.layer):

@@ -35,6 +35,18 @@ pub struct rh_lrn_geom {
   pub scale: c_float, pub power: c_float, pub min_div: c_float,
 }
 
+/// One parameter block of rh_sgd_momentum_step_multi (weights, gradient, momentum buffer).
+#[repr(C)]
+#[derive(Clone, Copy, Debug)]
+pub struct rh_sgd_tensor {
+  pub w: *mut f32,
+  pub g: *mut f32,
+  pub v: *mut f32,
+  pub n: i64,
+  pub l2: c_float,
+  pub keep_grad: i32,  // nonzero: g is left as it is (the caller overwrites it, beta = 0, in its next backward pass)
+}
+
 pub const RH_CONV_FWD: c_int = 0;
 pub const RH_CONV_BWD_FILTER: c_int = 1;
 pub const RH_CONV_BWD_DATA: c_int = 2;
@@ -46,6 +58,7 @@ pub const RH_ALGO_SCALAR_OFFSET: c_int = 0x200;
 
 #[link(name = "rembrandt_hip")]
 extern "C" {
+  pub fn rh_version() -> *const c_char;
   pub fn rh_error_string(code: c_int) -> *const c_char;
   pub fn rh_last_error() -> c_int;
 
@@ -85,6 +98,20 @@ extern "C" {
   pub fn rh_conv2d_bwd_data(g: *const rh_conv_geom, alpha: c_float, w: *const f32, dy: *const f32,
                             beta: c_float, dx: *mut f32, ws: *mut c_void, ws_bytes: size_t, flags: c_int,
                             stream: rh_stream_t) -> c_int;
+  // Filter and bias gradient in one call: dy is read once where the filter gradient copies it anyway.
+  pub fn rh_conv2d_bwd_filter_bias(g: *const rh_conv_geom, alpha: c_float, x: *const f32, dy: *const f32,
+                                   beta: c_float, dw: *mut f32, db: *mut f32, ws: *mut c_void, ws_bytes: size_t,
+                                   flags: c_int, stream: rh_stream_t) -> c_int;
+  pub fn rh_conv2d_bwd_bias_workspace_bytes_upto(n: i32, k: i32, plane: i32) -> size_t;
+  // The two-stage bias gradient on the library's own static scratch (callers that cannot allocate).
+  pub fn rh_noalloc_scratch_bytes() -> size_t;
+  pub fn rh_conv2d_bwd_bias_noalloc(n: i32, k: i32, plane: i32, alpha: c_float, dy: *const f32, beta: c_float,
+                                    db: *mut f32, stream: rh_stream_t) -> c_int;
+  // Data gradient that also applies the backward mask of the ReLU that produced this layer's input (x_act).
+  pub fn rh_conv2d_bwd_data_relu_supported(g: *const rh_conv_geom) -> c_int;
+  pub fn rh_conv2d_bwd_data_relu(g: *const rh_conv_geom, alpha: c_float, w: *const f32, dy: *const f32,
+                                 beta: c_float, dx: *mut f32, x_act: *const f32, ws: *mut c_void, ws_bytes: size_t,
+                                 flags: c_int, stream: rh_stream_t) -> c_int;
 
   pub fn rh_add_bias_nchw(bias: *const f32, y: *mut f32, plane: i32, k: i32, n: i32, alpha: c_float,
                           beta: c_float, stream: rh_stream_t) -> c_int;
@@ -128,9 +155,13 @@ extern "C" {
   // Host generator behind init_params (the reference's random stream lives in crates outside its tree).
   pub fn rh_rng_fill_uniform(seed: u64, stream_id: u64, host: *mut f32, n: size_t, lo: c_float, hi: c_float) -> c_int;
   pub fn rh_rng_fill_normal(seed: u64, stream_id: u64, host: *mut f32, n: size_t, mean: c_float, std: c_float) -> c_int;
+  pub fn rh_rng_fill_int(seed: u64, stream_id: u64, host: *mut i32, n: size_t, modulus: i32) -> c_int;
 
   pub fn rh_sgd_momentum_step(n: i64, w: *mut f32, g: *mut f32, v: *mut f32, l2: c_float, scale: c_float,
                               mu: c_float, apply: c_float, zero_grad: c_int, stream: rh_stream_t) -> c_int;
+  // One launch over a table of parameter blocks: what one `update` fan-out over a chain of operators issues.
+  pub fn rh_sgd_momentum_step_multi(count: i32, tensors: *const rh_sgd_tensor, scale: c_float, mu: c_float,
+                                    apply: c_float, zero_grad: c_int, stream: rh_stream_t) -> c_int;
   pub fn rh_descend(n: i64, w: *mut f32, g: *mut f32, s: c_float, l2: c_float, stream: rh_stream_t) -> c_int;
 
   // Second stream of the context (no counterpart in the reference, which issues everything on ctx.stream).
@@ -169,6 +200,7 @@ extern "C" {
 
   // CudnnBatchNormOp in Spatial mode (src/operator/conv.rs:493-535, 594-607): same alpha/beta pairs and buffer order.
   pub fn rh_bnorm_workspace_bytes(n: c_int, c: c_int, plane: c_int) -> size_t;
+  pub fn rh_bnorm_workspace_bytes_upto(n: c_int, c: c_int, plane: c_int) -> size_t;
   pub fn rh_bnorm_fwd_train(n: c_int, c: c_int, plane: c_int, alpha: c_float, x: *const f32, beta: c_float,
                             y: *mut f32, ema_factor: f64, epsilon: f64, scale: *const f32, bias: *const f32,
                             running_mean: *mut f32, running_ivar: *mut f32, cached_mean: *mut f32,
@@ -187,6 +219,17 @@ extern "C" {
                            scale: *const f32, bias: *const f32, dscale: *mut f32, dbias: *mut f32,
                            cached_mean: *const f32, cached_ivar: *const f32, ws: *mut c_void, ws_bytes: size_t,
                            stream: rh_stream_t) -> c_int;
+
+  // Per-launch timing and the calibration launches of the roofline report (no counterpart in the reference).
+  pub fn rh_profile_enable(on: c_int) -> c_int;
+  pub fn rh_profile_enabled() -> c_int;
+  pub fn rh_profile_filter(prefix: *const c_char) -> c_int;
+  pub fn rh_profile_count() -> c_int;
+  pub fn rh_profile_get(i: c_int, tag: *mut *const c_char, work: *mut f64, ms: *mut c_float) -> c_int;
+  pub fn rh_profile_reset() -> c_int;
+  pub fn rh_probe_mfma_loop(blocks: c_int, nacc: c_int, iters: c_int, sink: *mut f32, stream: rh_stream_t) -> c_int;
+  pub fn rh_probe_mfma_loop_varied(blocks: c_int, iters: c_int, sink: *mut f32, stream: rh_stream_t) -> c_int;
+  pub fn rh_probe_copy(src: *const f32, dst: *mut f32, n: size_t, stream: rh_stream_t) -> c_int;
 }
 
 /// The reference `unwrap()`s / `panic!`s on every native error (src/operator/mod.rs:1685-1696).
