@@ -4,10 +4,16 @@
 //! operator are `weights` then `bias`, gradients accumulate (beta = 1) until `reset`, and the SGD calls are the
 //! BLAS-1 sequences of src/operator/mod.rs:1178-1236.  The second-generation calls (`backward_scaled`, `descend`,
 //! `reset_gradients`: src/layer_new.rs:596-617, 1093-1154, src/arch_new.rs:527-552) are methods of the same trait.
+//! Beyond the reference's call list the operators use the library's folded forms where they give the same values:
+//! filter and bias gradient in one call, the ReLU backward mask inside the consumer's backward kernel, and the whole
+//! SGD update as one multi-tensor launch (`SequentialOperatorWorker::fused_sgd_step`).
 use ffi::*;
 use super::{DeviceBuffer, DeviceContext, SharedDeviceBuf, shared};
 
 use libc::{c_void};
+use std::fs::{self, File};
+use std::io::{Read, Write};
+use std::path::{Path, PathBuf};
 use std::rc::Rc;
 
 #[derive(Clone, Copy, Debug, PartialEq)]
@@ -33,6 +39,12 @@ pub trait Operator {
   fn get_output_vars(&self) -> Option<SharedDeviceBuf<f32>> { None }
   fn get_output_deltas(&self) -> Option<SharedDeviceBuf<f32>> { None }
   fn init_params(&mut self, _shared_seed: [u64; 2]) {}
+  /// Parameter / optimizer-state blobs (src/operator/mod.rs:65-68): NdArray records, weights then bias
+  /// (momentum buffers for the state); `decode_*` returns the number of bytes it consumed.
+  fn decode_params(&mut self, _blob: &[u8]) -> usize { 0 }
+  fn encode_params(&mut self, _blob: &mut Vec<u8>) {}
+  fn decode_state(&mut self, _blob: &[u8]) -> usize { 0 }
+  fn encode_state(&mut self, _blob: &mut Vec<u8>) {}
   fn forward(&mut self, batch_size: usize, phase: OpPhase);
   fn backward(&mut self, batch_size: usize);
   fn regularize(&mut self, _reg: Regularization) {}
@@ -46,6 +58,21 @@ pub trait Operator {
   fn backward_scaled(&mut self, batch_size: usize, _scale: f32) { self.backward(batch_size); }
   fn descend(&mut self, _scale: f32, _l2_reg_coef: f32) {}
   fn reset_gradients(&mut self, _momentum: f32) {}
+  /// Rows of one multi-tensor SGD launch (rh_sgd_momentum_step_multi): every parameter block of this operator.
+  fn sgd_tensors(&mut self, _l2_reg_coef: f32, _out: &mut Vec<rh_sgd_tensor>) {}
+  /// The operator above applies this operator's ReLU backward mask inside its own backward kernel
+  /// (rh_conv2d_bwd_data_relu, rh_pool2d_bwd_relu); returns whether this operator agrees to skip its own pass.
+  fn fold_activation_backward(&mut self) -> bool { false }
+}
+
+/// src/operator/mod.rs:101-109.
+pub trait InputOperator: Operator {
+  fn downcast(&self) -> &Operator;
+  fn expose_host_frame_buf(&mut self, batch_idx: usize) -> &mut [u8];
+  fn load_frames(&mut self, batch_size: usize);
+  fn stage_shape(&mut self, batch_idx: usize, shape: (usize, usize, usize));
+  fn preload_frame(&mut self, _batch_idx: usize) { unimplemented!(); }
+  fn wait_preload_frames(&mut self, _batch_size: usize) { unimplemented!(); }
 }
 
 pub trait LossOperator: Operator {
@@ -63,8 +90,52 @@ pub trait OperatorWorker: Operator {
   fn num_workers(&self) -> usize;
   fn worker_rank(&self) -> usize;
   fn shared_seed(&self) -> [u64; 2];
+  fn input_operator(&mut self) -> &mut InputOperator;
   fn loss_count(&self) -> usize;
   fn loss_operator(&mut self, rank: usize) -> &mut LossOperator;
+  // src/operator/worker.rs:62-72: what SgdOpt::train calls around its loop
+  fn next(&mut self) {}
+  fn checkpoint_params(&mut self, _t: usize, _prefix: &Path) { unimplemented!(); }
+  fn checkpoint_state(&mut self, _prefix: &Path) { unimplemented!(); }
+  fn can_rollback(&mut self, _prefix: &Path) -> Option<usize> { unimplemented!(); }
+  fn rollback_params(&mut self, _t: Option<usize>, _prefix: &Path) { unimplemented!(); }
+  fn rollback_state(&mut self, _prefix: &Path) { unimplemented!(); }
+}
+
+/// NdArray record: 'N','D',0,1; u32 rank; u64 dims (first index fastest); f32 data, all little-endian.
+pub fn ndarray_serialize(out: &mut Vec<u8>, data: &[f32], dims: &[usize]) {
+  out.extend_from_slice(&[b'N', b'D', 0, 1]);
+  let nd = dims.len() as u32;
+  for b in 0 .. 4 { out.push((nd >> (8 * b)) as u8); }
+  for &d in dims.iter() { for b in 0 .. 8 { out.push(((d as u64) >> (8 * b)) as u8); } }
+  assert_eq!(dims.iter().fold(1usize, |a, &d| a * d), data.len());
+  for &v in data.iter() {
+    let bits: u32 = unsafe { ::std::mem::transmute(v) };
+    for b in 0 .. 4 { out.push((bits >> (8 * b)) as u8); }
+  }
+}
+
+/// Returns (bytes consumed, dims, data); panics on a foreign or truncated record, as the reference's decoder does.
+pub fn ndarray_deserialize(blob: &[u8]) -> (usize, Vec<usize>, Vec<f32>) {
+  assert!(blob.len() >= 8 && blob[0] == b'N' && blob[1] == b'D' && blob[2] == 0 && blob[3] == 1, "NdArray: bad magic");
+  let nd = (0 .. 4).fold(0u32, |a, b| a | (blob[4 + b] as u32) << (8 * b)) as usize;
+  assert!(nd > 0 && nd <= 8 && blob.len() >= 8 + 8 * nd, "NdArray: bad rank or truncated header");
+  let mut dims = Vec::with_capacity(nd);
+  let mut off = 8;
+  let mut count = 1usize;
+  for _ in 0 .. nd {
+    let d = (0 .. 8).fold(0u64, |a, b| a | (blob[off + b] as u64) << (8 * b)) as usize;
+    dims.push(d);
+    count *= d;
+    off += 8;
+  }
+  assert!(blob.len() - off >= 4 * count, "NdArray: truncated data");
+  let mut data = Vec::with_capacity(count);
+  for i in 0 .. count {
+    let bits = (0 .. 4).fold(0u32, |a, b| a | (blob[off + 4 * i + b] as u32) << (8 * b));
+    data.push(unsafe { ::std::mem::transmute::<u32, f32>(bits) });
+  }
+  (off + 4 * count, dims, data)
 }
 
 /// weights / bias with their gradient, accumulated-gradient (momentum) and saved copies, and the update arithmetic
@@ -79,6 +150,26 @@ pub struct ParamTensors {
   pub save_weights:     DeviceBuffer<f32>,
   pub save_bias:        DeviceBuffer<f32>,
   context: Rc<DeviceContext>,
+}
+
+fn encode_pair(blob: &mut Vec<u8>, w: &DeviceBuffer<f32>, b: &DeviceBuffer<f32>) {
+  // the reference's Array2d bound of the weights: (in or R*S*C, out), first index fastest; the bias is (1, out)
+  let (mut hw, mut hb) = (vec![0.0f32; w.len()], vec![0.0f32; b.len()]);
+  w.context().sync();
+  w.sync_store(&mut hw);
+  b.sync_store(&mut hb);
+  ndarray_serialize(blob, &hw, &[w.len() / b.len(), b.len()]);
+  ndarray_serialize(blob, &hb, &[1, b.len()]);
+}
+
+fn decode_pair(blob: &[u8], w: &mut DeviceBuffer<f32>, b: &mut DeviceBuffer<f32>) -> usize {
+  let (n0, d0, hw) = ndarray_deserialize(blob);
+  assert!(d0.len() == 2 && d0[0] == w.len() / b.len() && d0[1] == b.len(), "weights blob has the wrong bound");
+  w.sync_load(&hw);
+  let (n1, d1, hb) = ndarray_deserialize(&blob[n0 ..]);
+  assert!(d1.len() == 2 && d1[0] == 1 && d1[1] == b.len(), "bias blob has the wrong bound");
+  b.sync_load(&hb);
+  n0 + n1
 }
 
 fn axpy(alpha: f32, x: &DeviceBuffer<f32>, y: &mut DeviceBuffer<f32>, s: rh_stream_t) {
@@ -130,12 +221,30 @@ impl ParamTensors {
     self.bias.sync_load(&b);
   }
 
-  /// grad += l2 * params
+  /// grad += l2 * params; nothing is launched for l2 == 0 (src/operator/mod.rs:1185), so a non-finite weight does
+  /// not leak 0 * inf into the gradient.
   pub fn regularize(&mut self, reg: Regularization) {
     let s = self.context.stream();
     let Regularization::L2{l2_reg_coef} = reg;
-    axpy(l2_reg_coef, &self.weights, &mut self.grad_weights, s);
-    axpy(l2_reg_coef, &self.bias, &mut self.grad_bias, s);
+    assert!(l2_reg_coef >= 0.0);
+    if l2_reg_coef > 0.0 {
+      axpy(l2_reg_coef, &self.weights, &mut self.grad_weights, s);
+      axpy(l2_reg_coef, &self.bias, &mut self.grad_bias, s);
+    }
+  }
+  pub fn encode_params(&self, blob: &mut Vec<u8>) { encode_pair(blob, &self.weights, &self.bias); }
+  pub fn decode_params(&mut self, blob: &[u8]) -> usize { decode_pair(blob, &mut self.weights, &mut self.bias) }
+  pub fn encode_state(&self, blob: &mut Vec<u8>) { encode_pair(blob, &self.acc_grad_weights, &self.acc_grad_bias); }
+  pub fn decode_state(&mut self, blob: &[u8]) -> usize {
+    decode_pair(blob, &mut self.acc_grad_weights, &mut self.acc_grad_bias)
+  }
+  /// This block's two rows of a multi-tensor SGD launch.  keep_grad = 0: the launch zeroes the gradients, which is
+  /// the reference's `reset`, so a raw gradient pointer read afterwards shows zeros.
+  pub fn sgd_tensors(&mut self, l2: f32, out: &mut Vec<rh_sgd_tensor>) {
+    out.push(rh_sgd_tensor{w: self.weights.as_mut_ptr(), g: self.grad_weights.as_mut_ptr(),
+                           v: self.acc_grad_weights.as_mut_ptr(), n: self.weights.len() as i64, l2: l2, keep_grad: 0});
+    out.push(rh_sgd_tensor{w: self.bias.as_mut_ptr(), g: self.grad_bias.as_mut_ptr(),
+                           v: self.acc_grad_bias.as_mut_ptr(), n: self.bias.len() as i64, l2: l2, keep_grad: 0});
   }
   /// acc = momentum * acc + scale * grad
   pub fn accumulate_grads(&mut self, scale: f32, momentum: f32) {
@@ -218,6 +327,22 @@ fn rect_backprop(act: ActivationFunction, out_act: &SharedDeviceBuf<f32>, out_de
 
 // ---- Conv2dOperator (src/operator/mod.rs:1366-1870) ------------------------------------------------------------
 
+/// The reference's algorithm selectors (src/operator/mod.rs:1366-1377).  They name cuDNN algorithms; this library
+/// chooses its kernel per geometry, so both fields are accepted and ignored (the reference itself never reads
+/// `bwd_backend`).  Every choice here is deterministic, which is what `CudnnDeterministic` asks for.
+#[derive(Clone, Copy, Debug)]
+pub enum Conv2dFwdBackend {
+  CudnnFastest,
+  CudnnImplicitPrecompGemm,
+  CudnnFftTiling,
+}
+
+#[derive(Clone, Copy, Debug)]
+pub enum Conv2dBwdBackend {
+  CudnnFastest,
+  CudnnDeterministic,
+}
+
 #[derive(Clone, Copy, Debug)]
 pub struct Conv2dOperatorConfig {
   pub in_dims:      (usize, usize, usize),   // (width, height, channels)
@@ -227,6 +352,8 @@ pub struct Conv2dOperatorConfig {
   pub out_channels: usize,
   pub act_func:     ActivationFunction,
   pub init_weights: ParamsInit,
+  pub fwd_backend:  Conv2dFwdBackend,
+  pub bwd_backend:  Conv2dBwdBackend,
 }
 
 impl Conv2dOperatorConfig {
@@ -253,10 +380,12 @@ pub struct Conv2dOperator {
   params:     ParamTensors,
   backward:   bool,
   workspace:  DeviceBuffer<u8>,
+  act_bwd_folded: bool,   // the operator above applies this operator's ReLU backward mask
+  fold_prev_relu: bool,   // this operator's data gradient applies the ReLU backward mask of the operator below
 }
 
 impl Conv2dOperator {
-  pub fn new(batch_size: usize, capability: OpCapability, config: Conv2dOperatorConfig, prev_op: &Operator,
+  pub fn new(batch_size: usize, capability: OpCapability, config: Conv2dOperatorConfig, prev_op: &mut Operator,
              context: Rc<DeviceContext>) -> Conv2dOperator {
     let (ow, oh, oc) = config.get_out_dims();
     let out_len = ow * oh * oc * batch_size;
@@ -269,12 +398,17 @@ impl Conv2dOperator {
       params: ParamTensors::new(config.params_len() - config.out_channels, config.out_channels, context.clone()),
       backward: capability == OpCapability::Backward,
       workspace: DeviceBuffer::zeros(0, context.clone()),
+      act_bwd_folded: false, fold_prev_relu: false,
     };
     let g = op.geom(batch_size);
     let mut ws = unsafe { rh_conv2d_workspace_bytes_upto(&g, RH_CONV_FWD) };
     if op.backward {
       ws = ::std::cmp::max(ws, unsafe { rh_conv2d_workspace_bytes_upto(&g, RH_CONV_BWD_FILTER) });
       ws = ::std::cmp::max(ws, unsafe { rh_conv2d_workspace_bytes_upto(&g, RH_CONV_BWD_DATA) });
+      ws = ::std::cmp::max(ws, unsafe { rh_conv2d_bwd_bias_workspace_bytes_upto(g.n, g.k, (ow * oh) as i32) });
+      if op.in_delta.is_some() && unsafe { rh_conv2d_bwd_data_relu_supported(&g) } != 0 {
+        op.fold_prev_relu = prev_op.fold_activation_backward();
+      }
     }
     op.workspace = DeviceBuffer::zeros(ws, context);
     op
@@ -293,19 +427,26 @@ impl Conv2dOperator {
     let g = self.geom(batch_size);
     let stream = self.context.stream();
     let frame_len = self.out_act.borrow().len() / self.batch_cap;
-    let plane = (frame_len / self.config.out_channels) as i32;
-    rect_backprop(self.config.act_func, &self.out_act, &self.out_delta, frame_len, batch_size, stream);
+    if !self.act_bwd_folded {
+      rect_backprop(self.config.act_func, &self.out_act, &self.out_delta, frame_len, batch_size, stream);
+    }
     let ws_len = self.workspace.len();
     let ws = self.workspace.as_mut_ptr() as *mut c_void;
     unsafe {
-      unwrap(rh_conv2d_bwd_filter(&g, scale, self.in_act.borrow().as_ptr(), self.out_delta.borrow().as_ptr(), 1.0,
-                                  self.params.grad_weights.as_mut_ptr(), ws, ws_len, 0, stream), "conv2d backward filter");
-      unwrap(rh_conv2d_bwd_bias(batch_size as i32, self.config.out_channels as i32, plane, scale,
-                                self.out_delta.borrow().as_ptr(), 1.0, self.params.grad_bias.as_mut_ptr(), stream),
-             "conv2d backward bias");
+      // filter and bias gradient in one call (out_delta is read once where the filter gradient copies it anyway)
+      unwrap(rh_conv2d_bwd_filter_bias(&g, scale, self.in_act.borrow().as_ptr(), self.out_delta.borrow().as_ptr(), 1.0,
+                                       self.params.grad_weights.as_mut_ptr(), self.params.grad_bias.as_mut_ptr(),
+                                       ws, ws_len, 0, stream), "conv2d backward filter / bias");
       if let Some(ref in_delta) = self.in_delta {
-        unwrap(rh_conv2d_bwd_data(&g, 1.0, self.params.weights.as_ptr(), self.out_delta.borrow().as_ptr(), 0.0,
-                                  in_delta.borrow_mut().as_mut_ptr(), ws, ws_len, 0, stream), "conv2d backward data");
+        if self.fold_prev_relu {
+          // in_act is the output of the ReLU below: its backward mask is applied as the data gradient is written
+          unwrap(rh_conv2d_bwd_data_relu(&g, 1.0, self.params.weights.as_ptr(), self.out_delta.borrow().as_ptr(), 0.0,
+                                         in_delta.borrow_mut().as_mut_ptr(), self.in_act.borrow().as_ptr(), ws, ws_len,
+                                         0, stream), "conv2d backward data");
+        } else {
+          unwrap(rh_conv2d_bwd_data(&g, 1.0, self.params.weights.as_ptr(), self.out_delta.borrow().as_ptr(), 0.0,
+                                    in_delta.borrow_mut().as_mut_ptr(), ws, ws_len, 0, stream), "conv2d backward data");
+        }
       }
     }
   }
@@ -344,6 +485,17 @@ impl Operator for Conv2dOperator {
   fn reset(&mut self) { self.params.reset(); }
   fn descend(&mut self, scale: f32, l2: f32) { self.params.descend(scale, l2); }
   fn reset_gradients(&mut self, momentum: f32) { self.params.reset_gradients(momentum); }
+  fn decode_params(&mut self, blob: &[u8]) -> usize { self.params.decode_params(blob) }
+  fn encode_params(&mut self, blob: &mut Vec<u8>) { self.params.encode_params(blob); }
+  fn decode_state(&mut self, blob: &[u8]) -> usize { self.params.decode_state(blob) }
+  fn encode_state(&mut self, blob: &mut Vec<u8>) { self.params.encode_state(blob); }
+  fn sgd_tensors(&mut self, l2: f32, out: &mut Vec<rh_sgd_tensor>) { self.params.sgd_tensors(l2, out); }
+  fn fold_activation_backward(&mut self) -> bool {
+    match self.config.act_func {
+      ActivationFunction::Rect => { self.act_bwd_folded = true; true }
+      _ => false,
+    }
+  }
 }
 
 // ---- AffineOperator (src/operator/mod.rs:1029-1236) ------------------------------------------------------------
@@ -444,6 +596,11 @@ impl Operator for AffineOperator {
   // the inherited backward_scaled.
   fn descend(&mut self, scale: f32, l2: f32) { self.params.descend(scale, l2); }
   fn reset_gradients(&mut self, momentum: f32) { self.params.reset_gradients(momentum); }
+  fn decode_params(&mut self, blob: &[u8]) -> usize { self.params.decode_params(blob) }
+  fn encode_params(&mut self, blob: &mut Vec<u8>) { self.params.encode_params(blob); }
+  fn decode_state(&mut self, blob: &[u8]) -> usize { self.params.decode_state(blob) }
+  fn encode_state(&mut self, blob: &mut Vec<u8>) { self.params.encode_state(blob); }
+  fn sgd_tensors(&mut self, l2: f32, out: &mut Vec<rh_sgd_tensor>) { self.params.sgd_tensors(l2, out); }
 }
 
 // ---- Pool2dOperator (src/operator/mod.rs:1990-2125) ------------------------------------------------------------
@@ -476,20 +633,29 @@ pub struct Pool2dOperator {
   out_act:    SharedDeviceBuf<f32>,
   out_delta:  SharedDeviceBuf<f32>,
   argmax:     DeviceBuffer<i32>,   // which input element each max window took: makes the backward pass a scatter
+  fold_relu:  bool,                // backward also applies the ReLU backward mask of the operator below
 }
 
 impl Pool2dOperator {
-  pub fn new(batch_size: usize, config: Pool2dOperatorConfig, prev_op: &Operator, context: Rc<DeviceContext>) -> Pool2dOperator {
+  pub fn new(batch_size: usize, config: Pool2dOperatorConfig, prev_op: &mut Operator, context: Rc<DeviceContext>) -> Pool2dOperator {
     let (ow, oh, oc) = config.get_out_dims();
     let out_len = ow * oh * oc * batch_size;
-    Pool2dOperator{
+    let mut op = Pool2dOperator{
       batch_cap: batch_size, config: config, context: context.clone(),
       in_act: prev_op.get_output_vars().expect("Pool2dOperator missing required prev operator output vars"),
       in_delta: prev_op.get_output_deltas(),
       out_act: shared(out_len, context.clone()),
       out_delta: shared(out_len, context.clone()),
       argmax: DeviceBuffer::zeros(out_len, context),
+      fold_relu: false,
+    };
+    let g = op.geom(batch_size);
+    if let PoolOperation::Max = config.pool_op {
+      if op.in_delta.is_some() && unsafe { rh_pool2d_bwd_relu_supported(&g) } != 0 {
+        op.fold_relu = prev_op.fold_activation_backward();
+      }
     }
+    op
   }
   fn geom(&self, batch_size: usize) -> rh_pool_geom {
     let (w, h, c) = self.config.in_dims;
@@ -513,9 +679,16 @@ impl Operator for Pool2dOperator {
     assert!(batch_size <= self.batch_cap);
     let g = self.geom(batch_size);
     if let Some(ref in_delta) = self.in_delta {
-      unwrap(unsafe { rh_pool2d_bwd(&g, self.in_act.borrow().as_ptr(), self.out_act.borrow().as_ptr(),
-                                    self.out_delta.borrow().as_ptr(), in_delta.borrow_mut().as_mut_ptr(),
-                                    self.argmax.as_ptr(), self.context.stream()) }, "pool2d backward");
+      if self.fold_relu {
+        // an arg-max element carries x = y, so windows with y <= 0 route nothing: the ReLU mask without a pass of its own
+        unwrap(unsafe { rh_pool2d_bwd_relu(&g, self.out_act.borrow().as_ptr(), self.out_delta.borrow().as_ptr(),
+                                           in_delta.borrow_mut().as_mut_ptr(), self.argmax.as_ptr(),
+                                           self.context.stream()) }, "pool2d backward");
+      } else {
+        unwrap(unsafe { rh_pool2d_bwd(&g, self.in_act.borrow().as_ptr(), self.out_act.borrow().as_ptr(),
+                                      self.out_delta.borrow().as_ptr(), in_delta.borrow_mut().as_mut_ptr(),
+                                      self.argmax.as_ptr(), self.context.stream()) }, "pool2d backward");
+      }
     }
   }
 }
@@ -633,15 +806,24 @@ impl LossOperator for SoftmaxKLLossOperator {
 
 // ---- input + SequentialOperatorWorker (src/operator/worker.rs:100-480) -----------------------------------------
 
-/// The head of a chain: frames already cast to f32 in device memory (`Data3dOperator` without preprocessing).
+/// The head of a chain (`Data3dOperator` without preprocessing, src/operator/mod.rs:507-640): u8 frames are staged in
+/// host memory, copied to the device and cast to f32 (`normalize`: divided by 255), or loaded as f32 directly.
 pub struct FrameInputOperator {
   batch_cap: usize,
+  frame_len: usize,
+  normalize: bool,
+  context:   Rc<DeviceContext>,
+  in_buf_h:  Vec<u8>,
+  in_buf:    DeviceBuffer<u8>,
   out_act:   SharedDeviceBuf<f32>,
 }
 
 impl FrameInputOperator {
-  pub fn new(batch_size: usize, frame_len: usize, context: Rc<DeviceContext>) -> FrameInputOperator {
-    FrameInputOperator{batch_cap: batch_size, out_act: shared(frame_len * batch_size, context)}
+  pub fn new(batch_size: usize, frame_len: usize, normalize: bool, context: Rc<DeviceContext>) -> FrameInputOperator {
+    FrameInputOperator{batch_cap: batch_size, frame_len: frame_len, normalize: normalize, context: context.clone(),
+                       in_buf_h: vec![0u8; frame_len * batch_size],
+                       in_buf: DeviceBuffer::zeros(frame_len * batch_size, context.clone()),
+                       out_act: shared(frame_len * batch_size, context)}
   }
   pub fn load_frames_f32(&mut self, frames: &[f32]) { self.out_act.borrow_mut().sync_load(frames); }
 }
@@ -653,6 +835,24 @@ impl Operator for FrameInputOperator {
   fn backward(&mut self, _batch_size: usize) {}
 }
 
+impl InputOperator for FrameInputOperator {
+  fn downcast(&self) -> &Operator { self }
+  fn expose_host_frame_buf(&mut self, batch_idx: usize) -> &mut [u8] {
+    assert!(batch_idx < self.batch_cap);
+    &mut self.in_buf_h[batch_idx * self.frame_len .. (batch_idx + 1) * self.frame_len]
+  }
+  /// `sync_load` of the staged frames, then the cast kernel (src/operator/mod.rs:640-664).
+  fn load_frames(&mut self, batch_size: usize) {
+    assert!(batch_size <= self.batch_cap);
+    let n = batch_size * self.frame_len;
+    self.in_buf.sync_load(&self.in_buf_h[ .. n]);
+    let scale = if self.normalize { 1.0 / 255.0 } else { 1.0 };
+    unwrap(unsafe { rh_cast_u8_f32(self.in_buf.as_ptr(), self.out_act.borrow_mut().as_mut_ptr(), n, scale,
+                                   self.context.stream()) }, "rh_cast_u8_f32");
+  }
+  fn stage_shape(&mut self, _batch_idx: usize, _shape: (usize, usize, usize)) {}
+}
+
 pub enum OperatorConfig {
   Affine(AffineOperatorConfig),
   Conv2d(Conv2dOperatorConfig),
@@ -662,6 +862,7 @@ pub enum OperatorConfig {
 pub struct SequentialOperatorWorker {
   batch_cap:   usize,
   shared_seed: [u64; 2],
+  context:     Rc<DeviceContext>,
   input_op:    FrameInputOperator,
   hidden_ops:  Vec<Box<Operator>>,
   loss_op:     SoftmaxKLLossOperator,
@@ -670,11 +871,11 @@ pub struct SequentialOperatorWorker {
 impl SequentialOperatorWorker {
   pub fn new(batch_size: usize, capability: OpCapability, shared_seed: [u64; 2], in_frame_len: usize,
              hidden: &[OperatorConfig], loss: CategoricalLossConfig, context: Rc<DeviceContext>) -> SequentialOperatorWorker {
-    let input_op = FrameInputOperator::new(batch_size, in_frame_len, context.clone());
+    let mut input_op = FrameInputOperator::new(batch_size, in_frame_len, false, context.clone());
     let mut hidden_ops: Vec<Box<Operator>> = Vec::with_capacity(hidden.len());
     for cfg in hidden.iter() {
       let op: Box<Operator> = {
-        let prev: &Operator = match hidden_ops.last() { Some(p) => &**p, None => &input_op };
+        let prev: &mut Operator = match hidden_ops.last_mut() { Some(p) => &mut **p, None => &mut input_op };
         match *cfg {
           OperatorConfig::Affine(c) => Box::new(AffineOperator::new(batch_size, capability, c, prev, context.clone())),
           OperatorConfig::Conv2d(c) => Box::new(Conv2dOperator::new(batch_size, capability, c, prev, context.clone())),
@@ -685,10 +886,32 @@ impl SequentialOperatorWorker {
     }
     let loss_op = SoftmaxKLLossOperator::new(batch_size, loss, &**hidden_ops.last().expect("a chain needs a hidden operator"),
                                              context);
-    SequentialOperatorWorker{batch_cap: batch_size, shared_seed: shared_seed, input_op: input_op, hidden_ops: hidden_ops,
-                             loss_op: loss_op}
+    SequentialOperatorWorker{batch_cap: batch_size, shared_seed: shared_seed, context: context, input_op: input_op,
+                             hidden_ops: hidden_ops, loss_op: loss_op}
   }
-  pub fn input_operator(&mut self) -> &mut FrameInputOperator { &mut self.input_op }
+  pub fn frame_input_operator(&mut self) -> &mut FrameInputOperator { &mut self.input_op }
+
+  /// `regularize -> accumulate_grads -> update_params -> reset` of every operator as ONE launch over the table of all
+  /// parameter blocks (rh_sgd_momentum_step_multi): v = mu v + scale (g + l2 W); W += apply v; g = 0.  Same arithmetic
+  /// per element as the four fan-outs of src/opt/sgd/new.rs:423-452.
+  pub fn fused_sgd_step(&mut self, l2_reg_coef: f32, scale: f32, momentum: f32, apply: f32) {
+    let mut rows: Vec<rh_sgd_tensor> = Vec::new();
+    for op in self.hidden_ops.iter_mut() { op.sgd_tensors(l2_reg_coef, &mut rows); }
+    if rows.is_empty() { return; }
+    unwrap(unsafe { rh_sgd_momentum_step_multi(rows.len() as i32, rows.as_ptr(), scale, momentum, apply, 1,
+                                               self.context.stream()) }, "rh_sgd_momentum_step_multi");
+  }
+}
+
+fn write_file(path: &Path, blob: &[u8]) {
+  let mut f = File::create(path).ok().expect("failed to create blob file");
+  f.write_all(blob).ok().expect("failed to write blob file");
+}
+
+fn read_file(path: &Path) -> Vec<u8> {
+  let mut blob = Vec::new();
+  File::open(path).ok().expect("failed to open blob file").read_to_end(&mut blob).ok().expect("failed to read blob file");
+  blob
 }
 
 impl Operator for SequentialOperatorWorker {
@@ -736,15 +959,73 @@ impl Operator for SequentialOperatorWorker {
   fn reset(&mut self) { for op in self.hidden_ops.iter_mut() { op.reset(); } }
   fn descend(&mut self, scale: f32, l2: f32) { for op in self.hidden_ops.iter_mut() { op.descend(scale, l2); } }
   fn reset_gradients(&mut self, momentum: f32) { for op in self.hidden_ops.iter_mut() { op.reset_gradients(momentum); } }
+  fn encode_params(&mut self, blob: &mut Vec<u8>) { for op in self.hidden_ops.iter_mut() { op.encode_params(blob); } }
+  fn decode_params(&mut self, blob: &[u8]) -> usize {
+    let mut off = 0;
+    for op in self.hidden_ops.iter_mut() { off += op.decode_params(&blob[off ..]); }
+    off
+  }
+  fn encode_state(&mut self, blob: &mut Vec<u8>) { for op in self.hidden_ops.iter_mut() { op.encode_state(blob); } }
+  fn decode_state(&mut self, blob: &[u8]) -> usize {
+    let mut off = 0;
+    for op in self.hidden_ops.iter_mut() { off += op.decode_state(&blob[off ..]); }
+    off
+  }
 }
 
 impl OperatorWorker for SequentialOperatorWorker {
   fn num_workers(&self) -> usize { 1 }
   fn worker_rank(&self) -> usize { 0 }
   fn shared_seed(&self) -> [u64; 2] { self.shared_seed }
+  fn input_operator(&mut self) -> &mut InputOperator { &mut self.input_op }
   fn loss_count(&self) -> usize { 1 }
   fn loss_operator(&mut self, rank: usize) -> &mut LossOperator {
     assert_eq!(rank, 0);
     &mut self.loss_op
+  }
+  /// `params.t_<t>.blob`, the `params.latest.blob` symlink, `checkpoint` (the iteration as a decimal line) with the
+  /// previous one kept as `checkpoint.0` (src/operator/worker.rs:447-480).
+  fn checkpoint_params(&mut self, t: usize, prefix: &Path) {
+    fs::create_dir_all(prefix).ok();
+    let mut blob = Vec::new();
+    self.encode_params(&mut blob);
+    let name = format!("params.t_{}.blob", t);
+    write_file(&prefix.join(&name), &blob);
+    let latest = prefix.join("params.latest.blob");
+    fs::remove_file(&latest).ok();
+    ::std::os::unix::fs::symlink(&PathBuf::from(&name), &latest).ok().expect("failed to symlink latest blob");
+    let ck = prefix.join("checkpoint");
+    if ck.exists() { fs::copy(&ck, &prefix.join("checkpoint.0")).ok(); }
+    write_file(&ck, format!("{}\n", t).as_bytes());
+  }
+  fn checkpoint_state(&mut self, prefix: &Path) {
+    fs::create_dir_all(prefix).ok();
+    let mut blob = Vec::new();
+    self.encode_state(&mut blob);
+    write_file(&prefix.join(format!("state.latest.blob.{}", self.worker_rank())), &blob);
+  }
+  fn can_rollback(&mut self, prefix: &Path) -> Option<usize> {
+    let mut text = String::new();
+    match File::open(&prefix.join("checkpoint")) {
+      Ok(mut f) => { f.read_to_string(&mut text).ok(); }
+      Err(_) => return None,
+    }
+    text.lines().next().and_then(|l| l.trim().parse().ok())
+  }
+  fn rollback_params(&mut self, t: Option<usize>, prefix: &Path) {
+    let path = match t {
+      Some(t) => {
+        let latest = self.can_rollback(prefix).expect("checkpoint file is missing or empty");
+        assert!(t <= latest);
+        prefix.join(format!("params.t_{}.blob", t))
+      }
+      None => prefix.join("params.latest.blob"),
+    };
+    let blob = read_file(&path);
+    self.decode_params(&blob);
+  }
+  fn rollback_state(&mut self, prefix: &Path) {
+    let blob = read_file(&prefix.join(format!("state.latest.blob.{}", self.worker_rank())));
+    self.decode_state(&blob);
   }
 }

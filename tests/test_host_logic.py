@@ -31,6 +31,59 @@ def test_library_exports_every_declared_symbol():
     assert b"gfx950" in _lib.lib().rh_version()
 
 
+def _c_prototypes(header):
+    """name -> argument count of every function include/<header> declares."""
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for name, args in re.findall(r"\b((?:rh|rembrandt_kernel)_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text):
+        args = args.strip()
+        out[name] = 0 if args in ("", "void") else len(args.split(","))
+    return out
+
+
+def _rust_prototypes(path):
+    text = re.sub(r"//.*", "", open(path).read())
+    block = text[text.index('extern "C" {'):]
+    block = block[:block.index("\n}")]
+    out = {}
+    for name, args in re.findall(r"pub fn (\w+)\s*\(([^)]*)\)", block):
+        out[name] = len([a for a in args.split(",") if a.strip()])
+    return out
+
+
+def test_rust_facade_binds_the_whole_kernel_abi():
+    """rust/src/ffi.rs (source for the reference's toolchain; no rustc in this image) declares every function of
+    include/rembrandt_hip.h with the same number of arguments and nothing else, every rh_* / rembrandt_kernel_*
+    function the facade's sources call is declared there, and the configuration types carry the reference's fields."""
+    header = _c_prototypes("rembrandt_hip.h")
+    rust = _rust_prototypes(os.path.join(ROOT, "rust", "src", "ffi.rs"))
+    assert len(header) > 80
+    assert sorted(set(header) - set(rust)) == []
+    assert sorted(set(rust) - set(header)) == []
+    assert [(n, header[n], rust[n]) for n in header if header[n] != rust[n]] == []
+    types = set(re.findall(r"pub (?:struct|enum|type) (\w+)", open(os.path.join(ROOT, "rust", "src", "ffi.rs")).read()))
+    for src in ("operator.rs", "lib.rs"):
+        text = re.sub(r"//.*", "", open(os.path.join(ROOT, "rust", "src", src)).read())
+        used = set(re.findall(r"\b((?:rh|rembrandt_kernel)_[a-z0-9_]+)\b", text))
+        assert sorted(used - set(rust) - types) == [], src
+    op = open(os.path.join(ROOT, "rust", "src", "operator.rs")).read()
+    # src/operator/mod.rs:1366-1389, 61-109; src/operator/worker.rs:52-76
+    for needle in ("pub enum Conv2dFwdBackend", "pub enum Conv2dBwdBackend", "pub fwd_backend:", "pub bwd_backend:",
+                   "fn decode_params(&mut self, _blob: &[u8]) -> usize", "fn encode_params(&mut self, _blob: &mut Vec<u8>)",
+                   "fn decode_state(&mut self, _blob: &[u8]) -> usize", "fn encode_state(&mut self, _blob: &mut Vec<u8>)",
+                   "pub trait InputOperator: Operator", "fn expose_host_frame_buf(&mut self, batch_idx: usize) -> &mut [u8]",
+                   "fn load_frames(&mut self, batch_size: usize)", "fn input_operator(&mut self) -> &mut InputOperator",
+                   "fn checkpoint_params(&mut self, _t: usize, _prefix: &Path)", "fn checkpoint_state(&mut self, _prefix: &Path)",
+                   "fn can_rollback(&mut self, _prefix: &Path) -> Option<usize>",
+                   "fn rollback_params(&mut self, _t: Option<usize>, _prefix: &Path)", "fn rollback_state(&mut self, _prefix: &Path)"):
+        assert needle in op, needle
+    # the folded paths the benchmark uses are reachable from the facade, and regularize launches nothing for l2 == 0
+    for call in ("rh_conv2d_bwd_filter_bias(", "rh_conv2d_bwd_data_relu(", "rh_sgd_momentum_step_multi(", "rh_pool2d_bwd_relu("):
+        assert call in op, call
+    assert re.search(r"if l2_reg_coef > 0\.0 \{\s*axpy\(l2_reg_coef, &self\.weights", op)
+
+
 def test_error_codes_without_gpu():
     lib = _lib.lib()
     g = _lib.ConvGeom(0, 3, 8, 8, 4, 3, 3, 1, 1)
