@@ -396,6 +396,43 @@ int rh_rng_fill_uniform01_device(uint64_t seed, uint64_t stream_id, uint64_t fir
                                  rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Packed bf16 activations for forward-only chains (RH_MATH_BF16_MFMA_FP32ACC without its per-call conversions; no
+ * counterpart in the reference, whose inference pass, OpPhase::Inference in src/operator/mod.rs:1663-1718, is the fp32
+ * forward).  A packed activation tensor holds bf16 values as [n][H + 2*halo][C/8][W + 2*halo][8] (C a multiple of 8;
+ * rh_bf16_act_bytes), with a zero border of `halo` elements that the producer never writes: zero the buffer once.  It is
+ * what the bf16 convolution's loaders read when halo equals that convolution's padding, so a producer that writes it
+ * (the convolution below, or a max-pool between them) removes the consumer's fp32 -> bf16 pass and halves the
+ * producer's store.  Values are the fp32 results rounded to nearest even, i.e. exactly what the consumer of an fp32
+ * activation would have rounded them to (ReLU and max commute with the rounding), so a chain run this way is
+ * bit-identical to the same chain through rh_conv2d_fwd(..., RH_MATH_BF16_MFMA_FP32ACC) on fp32 activations.
+ *   rh_bf16_pack_nchw / rh_bf16_unpack_nchw   fp32 NCHW <-> packed (unpack gives the bf16 values as fp32).
+ *   rh_conv2d_fwd_bf16_filter_bytes           size of a convolution's converted filter (0: the geometry has no packed
+ *                                             form); rh_conv2d_fwd_bf16_prep_filter fills it (256-byte aligned).  It
+ *                                             stays valid until the weights change.
+ *   rh_conv2d_fwd_bf16_takes_packed           nonzero if the geometry reads a packed input (input channels a multiple
+ *                                             of 8); otherwise pass the fp32 image `x`.
+ *   rh_conv2d_fwd_bf16_packed                 y = conv(x, w) (+ bias) (ReLU) from exactly one of `xp` (packed, halo =
+ *                                             g->pad) and `x` (fp32 NCHW, converted into `ws` of
+ *                                             rh_conv2d_fwd_bf16_workspace_bytes), to exactly one of `y` (fp32 NCHW) and
+ *                                             `yp` (packed with halo yp_halo; K a multiple of 8).  flags: RH_FUSE_*.
+ *   rh_pool2d_fwd_bf16_packed                 max pooling from a packed input (halo 0) to a packed output.
+ * ------------------------------------------------------------------------------------------- */
+size_t rh_bf16_act_bytes(int32_t N, int32_t C, int32_t H, int32_t W, int32_t halo);
+int rh_bf16_pack_nchw(int32_t N, int32_t C, int32_t H, int32_t W, int32_t halo, const float* x, void* xp,
+                      rh_stream_t stream);
+int rh_bf16_unpack_nchw(int32_t N, int32_t C, int32_t H, int32_t W, int32_t halo, const void* xp, float* x,
+                        rh_stream_t stream);
+size_t rh_conv2d_fwd_bf16_filter_bytes(const rh_conv_geom* g);
+int rh_conv2d_fwd_bf16_takes_packed(const rh_conv_geom* g);
+size_t rh_conv2d_fwd_bf16_workspace_bytes(const rh_conv_geom* g);
+int rh_conv2d_fwd_bf16_prep_filter(const rh_conv_geom* g, const float* w, void* wprep, size_t wprep_bytes,
+                                   rh_stream_t stream);
+int rh_conv2d_fwd_bf16_packed(const rh_conv_geom* g, const void* xp, const float* x, const void* wprep,
+                              const float* bias, float* y, void* yp, int32_t yp_halo, void* ws, size_t ws_bytes,
+                              int flags, rh_stream_t stream);
+int rh_pool2d_fwd_bf16_packed(const rh_pool_geom* g, const void* xp, void* yp, int32_t yp_halo, rh_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Per-launch timing (no counterpart in the reference, which only takes wall-clock laps around
  * minibatches, src/opt/sgd/new.rs:273-274).  While enabled, every kernel launch of this library is
  * bracketed by HIP events on its stream.  Record i = {kernel tag, algorithmic work (FLOPs for the

@@ -130,6 +130,15 @@ PROTOTYPES = {
     "rh_probe_mfma_loop": (_int, [_int, _int, _int, _vp, _vp]),
     "rh_probe_mfma_loop_varied": (_int, [_int, _int, _vp, _vp]),
     "rh_probe_copy": (_int, [_vp, _vp, _sz, _vp]),
+    "rh_bf16_act_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32]),
+    "rh_bf16_pack_nchw": (_int, [_i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "rh_bf16_unpack_nchw": (_int, [_i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "rh_conv2d_fwd_bf16_filter_bytes": (_sz, [C.POINTER(ConvGeom)]),
+    "rh_conv2d_fwd_bf16_takes_packed": (_int, [C.POINTER(ConvGeom)]),
+    "rh_conv2d_fwd_bf16_workspace_bytes": (_sz, [C.POINTER(ConvGeom)]),
+    "rh_conv2d_fwd_bf16_prep_filter": (_int, [C.POINTER(ConvGeom), _vp, _vp, _sz, _vp]),
+    "rh_conv2d_fwd_bf16_packed": (_int, [C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _sz, _int, _vp]),
+    "rh_pool2d_fwd_bf16_packed": (_int, [C.POINTER(PoolGeom), _vp, _vp, _i32, _vp]),
     "rh_rng_fill_uniform": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_normal": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _f, _f]),
     "rh_rng_fill_int": (_int, [C.c_uint64, C.c_uint64, _vp, _sz, _i32]),

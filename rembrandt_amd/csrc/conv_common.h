@@ -87,10 +87,11 @@ inline int launch_mfma_gemm(const typename AL::Params& ap, const typename BL::Pa
 }
 
 // Same grid and split logic for the bf16-operand kernel.  FLOPs are counted as for fp32.
-template <class T, class AL, class BL, bool NCHW, class PASS>
+template <class T, class AL, class BL, bool NCHW, class PASS, bool PK = false>
 inline int launch_mfma_gemm_bf16(const typename AL::Params& ap, const typename BL::Params& bp,
                                  const EpiParams& ep, int K, int splits, int* splits_used,
-                                 hipStream_t stream, const char* tag, int k_algorithmic = 0) {
+                                 hipStream_t stream, const char* tag, int k_algorithmic = 0,
+                                 const PackedOut& pk = PackedOut()) {
   const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
   const int k_chunks = cdiv(K, T::BK);
   if (splits < 1) splits = 1;
@@ -102,33 +103,36 @@ inline int launch_mfma_gemm_bf16(const typename AL::Params& ap, const typename B
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
   if (lds_bytes > 48 * 1024) {
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&mfma_gemm_bf16_kernel<T, AL, BL, NCHW, PASS>),
+        reinterpret_cast<const void*>(&mfma_gemm_bf16_kernel<T, AL, BL, NCHW, PASS, PK>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr != hipSuccess) return (int)attr;
   }
   ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)(k_algorithmic > 0 ? k_algorithmic : K), stream);
-  hipLaunchKernelGGL((mfma_gemm_bf16_kernel<T, AL, BL, NCHW, PASS>), grid, dim3(T::NT), lds_bytes, stream, ap, bp, ep,
-                     tiles_m, k_chunks, cps);
+  if (PK && (splits != 1 || !pk.ptr)) return RH_E_INVALID;
+  hipLaunchKernelGGL((mfma_gemm_bf16_kernel<T, AL, BL, NCHW, PASS, PK>), grid, dim3(T::NT), lds_bytes, stream, ap, bp, ep,
+                     tiles_m, k_chunks, cps, pk);
   return launch_status();
 }
 
 // The direct-to-LDS form for packed operands (ring of four LDS buffers, one pass over the whole contraction).
-template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS>
+template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS, bool PK = false>
 inline int launch_mfma_gemm_bf16_dma(const RowV8Params& ap, const RowV8Params& bp, const EpiParams& ep, int K,
-                                     hipStream_t stream, const char* tag, int k_algorithmic = 0) {
+                                     hipStream_t stream, const char* tag, int k_algorithmic = 0,
+                                     const PackedOut& pk = PackedOut()) {
   const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
   if (K <= 0 || K % T::BK != 0) return RH_E_INVALID;
   constexpr size_t lds_bytes = 16 * 4 * (T::BK / 8) * (T::BM + T::BN);
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
   if (lds_bytes > 48 * 1024) {
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS>),
+        reinterpret_cast<const void*>(&mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS, PK>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr != hipSuccess) return (int)attr;
   }
   ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)(k_algorithmic > 0 ? k_algorithmic : K), stream);
-  hipLaunchKernelGGL((mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS>), dim3((unsigned)(tiles_m * tiles_n)),
-                     dim3(T::NT), lds_bytes, stream, ap, bp, ep, tiles_m, K / T::BK);
+  if (PK && !pk.ptr) return RH_E_INVALID;
+  hipLaunchKernelGGL((mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS, PK>), dim3((unsigned)(tiles_m * tiles_n)),
+                     dim3(T::NT), lds_bytes, stream, ap, bp, ep, tiles_m, K / T::BK, pk);
   return launch_status();
 }
 

@@ -392,6 +392,28 @@ __global__ __launch_bounds__(256) void nchw_to_bf16_groups_kernel(const float* _
   xb[i] = pack8_bf16(v);
 }
 
+// The inverse: x[n][c][h][w] (fp32) = xb[n][h + halo][c/8][w + halo][c%8]; one thread per 16-byte group of the interior.
+__global__ __launch_bounds__(256) void bf16_groups_to_nchw_kernel(const uint4* __restrict__ xb, float* __restrict__ x,
+                                                                 unsigned total, int H, int W, FastDiv dW, FastDiv dCg,
+                                                                 FastDiv dH, int halo) {
+  const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  uint32_t t, wc, cg, h, n;
+  dW.divmod(i, t, wc);
+  dCg.divmod(t, t, cg);
+  dH.divmod(t, n, h);
+  const int Hp = H + 2 * halo, Wp = W + 2 * halo;
+  const uint4 q = xb[(((size_t)n * Hp + h + halo) * dCg.div + cg) * Wp + wc + halo];
+  const uint32_t d[4] = {q.x, q.y, q.z, q.w};
+  const size_t plane = (size_t)H * W;
+  float* dst = x + ((size_t)n * dCg.div * 8 + cg * 8) * plane + (size_t)h * W + wc;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    dst[(2 * e) * plane] = __builtin_bit_cast(float, d[e] << 16);
+    dst[(2 * e + 1) * plane] = __builtin_bit_cast(float, d[e] & 0xffff0000u);
+  }
+}
+
 // The same two copies for groups of eight filter columns (Bf16FwdPlan::s_groups > 0).
 // wb[g][ko][8] = w[ko][c][r][8 sg + e] (zero for columns past S and groups past the end), g = (c*R + r)*Sg + sg;
 // soff8[g] = byte offset of (c, r, 8 sg) in one image of the copy.
@@ -434,27 +456,28 @@ __global__ __launch_bounds__(256) void nchw_to_bf16_planes_kernel(const float* _
   xb[i] = pack_bf16(lo, hi);
 }
 
-template <class T, bool DMA = false>
-static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const float* x, const float* w, void* ws,
-                               const EpiParams& ep, hipStream_t stream, const char* tag) {
-  char* base = static_cast<char*>(ws);
+// The three stages of a packed bf16 forward.  The filter stage's result (table + filter copy, tab_bytes + wt_bytes at
+// `wprep`) depends on the weights and the geometry only, so a caller whose weights do not change between calls keeps it.
+static int bf16_prep_filter(const ConvDims& d, const Bf16FwdPlan& bpn, const float* w, void* wprep, hipStream_t stream) {
+  char* base = static_cast<char*>(wprep);
   int* soff8 = reinterpret_cast<int*>(base);
   uint4* wb = reinterpret_cast<uint4*>(base + bpn.tab_bytes);
-  uint4* xb = reinterpret_cast<uint4*>(base + bpn.tab_bytes + bpn.wt_bytes);
-  const int CRS = d.C * d.R * d.S, HpWp = bpn.Hp * bpn.Wp, Cg = d.C / 8;
-  const bool cols = bpn.s_groups > 0;
-  {
-    ProfScope prof("bf16_filter", 4.0 * (double)d.w_elems + 2.0 * (double)bpn.n_k * d.K, stream);
-    const dim3 grid((unsigned)cdiv((long long)(bpn.n_k / 8) * d.K, 256ll));
-    if (cols)
-      hipLaunchKernelGGL(prep_bf16_filter_cols_kernel, grid, dim3(256), 0, stream, w, wb, soff8, bpn.n_k,
-                         d.C * d.R * bpn.s_groups, d.K, CRS, d.R, d.S, bpn.s_groups, bpn.Hp, bpn.Wp);
-    else
-      hipLaunchKernelGGL(prep_bf16_filter_kernel, grid, dim3(256), 0, stream, w, wb, soff8, bpn.n_k, CRS, d.K, d.C,
-                         d.R * d.S, d.S, bpn.Wp);
-  }
-  if (int e = launch_status()) return e;
-  if (cols) {
+  const int CRS = d.C * d.R * d.S;
+  ProfScope prof("bf16_filter", 4.0 * (double)d.w_elems + 2.0 * (double)bpn.n_k * d.K, stream);
+  const dim3 grid((unsigned)cdiv((long long)(bpn.n_k / 8) * d.K, 256ll));
+  if (bpn.s_groups > 0)
+    hipLaunchKernelGGL(prep_bf16_filter_cols_kernel, grid, dim3(256), 0, stream, w, wb, soff8, bpn.n_k,
+                       d.C * d.R * bpn.s_groups, d.K, CRS, d.R, d.S, bpn.s_groups, bpn.Hp, bpn.Wp);
+  else
+    hipLaunchKernelGGL(prep_bf16_filter_kernel, grid, dim3(256), 0, stream, w, wb, soff8, bpn.n_k, CRS, d.K, d.C,
+                       d.R * d.S, d.S, bpn.Wp);
+  return launch_status();
+}
+
+// fp32 NCHW image -> the bf16 copy the plan's loaders read (img_bytes at `xb`), zero border included.
+static int bf16_pack_input(const ConvDims& d, const Bf16FwdPlan& bpn, const float* x, void* xb, hipStream_t stream) {
+  const int HpWp = bpn.Hp * bpn.Wp, Cg = d.C / 8;
+  if (bpn.s_groups > 0) {
     const size_t pairs = (size_t)d.N * d.C * HpWp / 2;  // below 2^30: the copy is at most 2 GiB
     ProfScope prof("nchw_to_bf16_planes", 4.0 * (double)d.x_elems + 4.0 * (double)pairs, stream);
     hipLaunchKernelGGL(nchw_to_bf16_planes_kernel, dim3(stream_grid(pairs, 256)), dim3(256), 0, stream, x,
@@ -463,10 +486,24 @@ static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const 
   } else {
     const size_t groups = (size_t)d.N * Cg * HpWp;  // below 2^28: the copy is at most 2 GiB
     ProfScope prof("nchw_to_bf16_groups", 4.0 * (double)d.x_elems + 16.0 * (double)groups, stream);
-    hipLaunchKernelGGL(nchw_to_bf16_groups_kernel, dim3(stream_grid(groups, 256)), dim3(256), 0, stream, x, xb, (unsigned)groups,
-                       d.H, d.W, FastDiv((uint32_t)bpn.Wp), FastDiv((uint32_t)Cg), FastDiv((uint32_t)bpn.Hp), d.pad);
+    hipLaunchKernelGGL(nchw_to_bf16_groups_kernel, dim3(stream_grid(groups, 256)), dim3(256), 0, stream, x,
+                       reinterpret_cast<uint4*>(xb), (unsigned)groups, d.H, d.W, FastDiv((uint32_t)bpn.Wp),
+                       FastDiv((uint32_t)Cg), FastDiv((uint32_t)bpn.Hp), d.pad);
   }
-  if (int e = launch_status()) return e;
+  return launch_status();
+}
+
+// The contraction on prepared operands: `xb` the image copy, `wprep` the filter stage's result.  The result goes to
+// ep.out as fp32 NCHW, or, with pk.ptr set, as packed bf16 for the next convolution (ep.out unused).  Which kernel
+// runs depends on the geometry only, so both forms of the result come from the same accumulators.
+template <class T, bool DMA, bool PK>
+static int bf16_gemm_on(const ConvDims& d, const Bf16FwdPlan& bpn, const void* xb, const void* wprep, const EpiParams& ep,
+                        const PackedOut& pk, hipStream_t stream, const char* tag) {
+  const char* base = static_cast<const char*>(wprep);
+  const int* soff8 = reinterpret_cast<const int*>(base);
+  const void* wb = base + bpn.tab_bytes;
+  const int CRS = d.C * d.R * d.S, HpWp = bpn.Hp * bpn.Wp, Cg = d.C / 8;
+  const bool cols = bpn.s_groups > 0;
   RowV8Params ap;  // filter: row ko of group g at (g*K + ko)*16
   ap.ptr = wb; ap.bytes = (uint32_t)(2 * (size_t)bpn.n_k * d.K);
   ap.M = d.K; ap.inner = 1; ap.innerW = 1; ap.img_stride = 16; ap.a_stride = 0; ap.b_stride = 0; ap.soff = nullptr;
@@ -484,8 +521,25 @@ static int run_fwd_bf16_packed(const ConvDims& d, const Bf16FwdPlan& bpn, const 
   bp.group_stride = 0;
   typedef LoadRowV8<T::BM, T::BK, T::NT, true> AL;
   typedef LoadRowV8<T::BN, T::BK, T::NT, false> BL;
-  if (DMA) return launch_mfma_gemm_bf16_dma<T, true, false, true, PassConvFwd>(ap, bp, ep, bpn.n_k, stream, tag, CRS);
-  return launch_mfma_gemm_bf16<T, AL, BL, true, PassConvFwd>(ap, bp, ep, bpn.n_k, 1, nullptr, stream, tag, CRS);
+  if constexpr (DMA)
+    return launch_mfma_gemm_bf16_dma<T, true, false, true, PassConvFwd, PK>(ap, bp, ep, bpn.n_k, stream, tag, CRS, pk);
+  else
+    return launch_mfma_gemm_bf16<T, AL, BL, true, PassConvFwd, PK>(ap, bp, ep, bpn.n_k, 1, nullptr, stream, tag, CRS, pk);
+}
+
+static int bf16_gemm(const ConvDims& d, const Bf16FwdPlan& bpn, const void* xb, const void* wprep, const EpiParams& ep,
+                     const PackedOut& pk, hipStream_t stream) {
+  // Long contractions on grids that fill all 256 CUs with 256-row tiles (and waste no more filter rows than
+  // 128-row tiles would) take the direct-to-LDS kernel: 14 % faster on 256 x 96 x 27 x 27 -> 256, 5x5.  Short
+  // contractions lose there (one block per CU: nothing hides a tile's first loads and its stores).
+  const bool dma = bpn.n_k >= 512 && cdiv(d.K, 256) * 256 == cdiv(d.K, 128) * 128 &&
+                   (long long)cdiv(d.K, 256) * cdiv(ep.cols, 256) >= 256;
+  if (pk.ptr) {
+    if (dma) return bf16_gemm_on<T256x256bf, true, true>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
+    return bf16_gemm_on<T128x128bf, false, true>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x128");
+  }
+  if (dma) return bf16_gemm_on<T256x256bf, true, false>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
+  return bf16_gemm_on<T128x128bf, false, false>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x128");
 }
 
 template <class T>
@@ -528,13 +582,11 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
       ep.out = y; ep.bias = (flags & RH_FUSE_BIAS) ? bias : nullptr; ep.alpha = alpha; ep.beta = beta;
       ep.rows = d.K; ep.cols = d.N * d.P * d.Q; ep.inner = d.P * d.Q; ep.ld = 0; ep.relu = (flags & RH_FUSE_RELU) ? 1 : 0;
       ep.split_stride = 0;
-      // Long contractions on grids that fill all 256 CUs with 256-row tiles (and waste no more filter rows than
-      // 128-row tiles would) take the direct-to-LDS kernel: 14 % faster on 256 x 96 x 27 x 27 -> 256, 5x5.  Short
-      // contractions lose there (one block per CU: nothing hides a tile's first loads and its stores).
-      if (bpn.n_k >= 512 && cdiv(d.K, 256) * 256 == cdiv(d.K, 128) * 128 &&
-          (long long)cdiv(d.K, 256) * cdiv(ep.cols, 256) >= 256)
-        return run_fwd_bf16_packed<T256x256bf, true>(d, bpn, x, w, ws, ep, stream, "conv_fwd_bf16p_256x256");
-      return run_fwd_bf16_packed<T128x128bf>(d, bpn, x, w, ws, ep, stream, "conv_fwd_bf16p_128x128");
+      // scratch: [table | filter copy | image copy]
+      char* xb = static_cast<char*>(ws) + bpn.tab_bytes + bpn.wt_bytes;
+      if (int e = bf16_prep_filter(d, bpn, w, ws, stream)) return e;
+      if (int e = bf16_pack_input(d, bpn, x, xb, stream)) return e;
+      return bf16_gemm(d, bpn, xb, ws, ep, PackedOut(), stream);
     }
   }
   const SoffPlan sp = plan_soff_fwd(d);
@@ -608,4 +660,114 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
     case 64:  return run_fwd<T64x256>(d, ap, bp, ep, stream, "conv_fwd_64x256");
     default:  return run_fwd<T32x256>(d, ap, bp, ep, stream, "conv_fwd_32x256");
   }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Packed bf16 activations between layers: a forward-only chain keeps its activations as bf16 in the layout the next
+// convolution's loaders read, written by the producing kernel's epilogue, and its converted filters for as long as
+// the weights stay the same.
+// ---------------------------------------------------------------------------------------------------------------
+static bool packed_act_dims_ok(int32_t N, int32_t C, int32_t H, int32_t W, int32_t halo) {
+  return N > 0 && C > 0 && C % 8 == 0 && H > 0 && W > 0 && halo >= 0 &&
+         2 * (size_t)N * C * (size_t)(H + 2 * halo) * (size_t)(W + 2 * halo) <= kMaxBufferBytes;
+}
+
+extern "C" size_t rh_bf16_act_bytes(int32_t N, int32_t C, int32_t H, int32_t W, int32_t halo) {
+  if (!packed_act_dims_ok(N, C, H, W, halo)) return 0;
+  return align256(2 * (size_t)N * C * (size_t)(H + 2 * halo) * (size_t)(W + 2 * halo));
+}
+
+extern "C" int rh_bf16_pack_nchw(int32_t N, int32_t C, int32_t H, int32_t W, int32_t halo, const float* x, void* xp,
+                                 rh_stream_t stream_) {
+  if (!packed_act_dims_ok(N, C, H, W, halo) || !x || !xp || (reinterpret_cast<uintptr_t>(xp) & 15)) return RH_E_INVALID;
+  const int Hp = H + 2 * halo, Wp = W + 2 * halo, Cg = C / 8;
+  const size_t groups = (size_t)N * Cg * Hp * Wp;
+  hipStream_t stream = to_stream(stream_);
+  ProfScope prof("nchw_to_bf16_groups", 4.0 * (double)N * C * H * W + 16.0 * (double)groups, stream);
+  hipLaunchKernelGGL(nchw_to_bf16_groups_kernel, dim3(stream_grid(groups, 256)), dim3(256), 0, stream, x,
+                     static_cast<uint4*>(xp), (unsigned)groups, H, W, FastDiv((uint32_t)Wp), FastDiv((uint32_t)Cg),
+                     FastDiv((uint32_t)Hp), halo);
+  return launch_status();
+}
+
+extern "C" int rh_bf16_unpack_nchw(int32_t N, int32_t C, int32_t H, int32_t W, int32_t halo, const void* xp, float* x,
+                                   rh_stream_t stream_) {
+  if (!packed_act_dims_ok(N, C, H, W, halo) || !x || !xp || (reinterpret_cast<uintptr_t>(xp) & 15)) return RH_E_INVALID;
+  const int Cg = C / 8;
+  const size_t groups = (size_t)N * Cg * H * W;
+  hipStream_t stream = to_stream(stream_);
+  ProfScope prof("bf16_groups_to_nchw", 4.0 * (double)N * C * H * W + 16.0 * (double)groups, stream);
+  hipLaunchKernelGGL(bf16_groups_to_nchw_kernel, dim3(stream_grid(groups, 256)), dim3(256), 0, stream,
+                     static_cast<const uint4*>(xp), x, (unsigned)groups, H, W, FastDiv((uint32_t)W), FastDiv((uint32_t)Cg),
+                     FastDiv((uint32_t)H), halo);
+  return launch_status();
+}
+
+extern "C" size_t rh_conv2d_fwd_bf16_filter_bytes(const rh_conv_geom* g) {
+  ConvDims d;
+  if (conv_dims(g, &d)) return 0;
+  const Bf16FwdPlan bpn = plan_bf16_fwd(d);
+  return bpn.ok ? bpn.tab_bytes + bpn.wt_bytes : 0;
+}
+
+extern "C" int rh_conv2d_fwd_bf16_takes_packed(const rh_conv_geom* g) {
+  ConvDims d;
+  if (conv_dims(g, &d)) return 0;
+  const Bf16FwdPlan bpn = plan_bf16_fwd(d);
+  return bpn.ok && bpn.s_groups == 0 ? 1 : 0;
+}
+
+extern "C" size_t rh_conv2d_fwd_bf16_workspace_bytes(const rh_conv_geom* g) {
+  ConvDims d;
+  if (conv_dims(g, &d)) return 0;
+  const Bf16FwdPlan bpn = plan_bf16_fwd(d);
+  return bpn.ok ? bpn.img_bytes : 0;
+}
+
+extern "C" int rh_conv2d_fwd_bf16_prep_filter(const rh_conv_geom* g, const float* w, void* wprep, size_t wprep_bytes,
+                                              rh_stream_t stream) {
+  ConvDims d;
+  if (int e = conv_dims(g, &d)) return e;
+  if (!w || !wprep || (reinterpret_cast<uintptr_t>(wprep) & 255)) return RH_E_INVALID;
+  const Bf16FwdPlan bpn = plan_bf16_fwd(d);
+  if (!bpn.ok) return RH_E_UNSUPPORTED;
+  if (wprep_bytes < bpn.tab_bytes + bpn.wt_bytes) return RH_E_WORKSPACE;
+  return bf16_prep_filter(d, bpn, w, wprep, to_stream(stream));
+}
+
+extern "C" int rh_conv2d_fwd_bf16_packed(const rh_conv_geom* g, const void* xp, const float* x, const void* wprep,
+                                         const float* bias, float* y, void* yp, int32_t yp_halo, void* ws, size_t ws_bytes,
+                                         int flags, rh_stream_t stream_) {
+  ConvDims d;
+  if (int e = conv_dims(g, &d)) return e;
+  if ((!xp) == (!x) || !wprep || (!y) == (!yp)) return RH_E_INVALID;  // one input form, one output form
+  if ((flags & RH_FUSE_BIAS) && !bias) return RH_E_INVALID;
+  if (flags & ~(RH_FUSE_BIAS | RH_FUSE_RELU)) return RH_E_INVALID;
+  const Bf16FwdPlan bpn = plan_bf16_fwd(d);
+  if (!bpn.ok) return RH_E_UNSUPPORTED;
+  if (xp && bpn.s_groups > 0) return RH_E_UNSUPPORTED;  // grouped by filter columns: the copy is made from the fp32 image
+  if (d.y_elems == 0) return 0;
+  hipStream_t stream = to_stream(stream_);
+  const void* xb = xp;
+  if (x) {
+    if (!ws || ws_bytes < bpn.img_bytes || (reinterpret_cast<uintptr_t>(ws) & 255)) return RH_E_WORKSPACE;
+    if (int e = bf16_pack_input(d, bpn, x, ws, stream)) return e;
+    xb = ws;
+  } else if (reinterpret_cast<uintptr_t>(xp) & 15) {
+    return RH_E_INVALID;
+  }
+  EpiParams ep;
+  ep.out = y; ep.bias = (flags & RH_FUSE_BIAS) ? bias : nullptr; ep.alpha = 1.0f; ep.beta = 0.0f;
+  ep.rows = d.K; ep.cols = d.N * d.P * d.Q; ep.inner = d.P * d.Q; ep.ld = 0; ep.relu = (flags & RH_FUSE_RELU) ? 1 : 0;
+  ep.split_stride = 0;
+  PackedOut pk;
+  if (yp) {
+    if (d.K % 8 != 0 || yp_halo < 0 || !packed_act_dims_ok(d.N, d.K, d.P, d.Q, yp_halo) ||
+        (reinterpret_cast<uintptr_t>(yp) & 15))
+      return RH_E_INVALID;
+    pk.ptr = yp; pk.halo = yp_halo; pk.Cg = d.K / 8; pk.Wp = d.Q + 2 * yp_halo;
+    pk.img_groups = (d.P + 2 * yp_halo) * pk.Cg * pk.Wp;
+    pk.dQ = FastDiv((uint32_t)d.Q);
+  }
+  return bf16_gemm(d, bpn, xb, wprep, ep, pk, stream);
 }

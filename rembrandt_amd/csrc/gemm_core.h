@@ -701,6 +701,57 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], co
   }
 }
 
+// Packed bf16 result: the NCHW result (img, row, p, q) written as bf16 in the operand layout the packed loaders read,
+//   [img][Hp][Cg][Wp][8]:  16-byte group ((img*Hp + p + halo)*Cg + row/8)*Wp + q + halo, element row % 8,
+// Hp = P + 2*halo, Wp = Q + 2*halo, Cg = rows / 8 (rows a multiple of 8); the border is left alone (the owner of the
+// buffer zeroed it once).  A consumer convolution with padding `halo` then reads it as it is: no conversion pass and
+// half the bytes of an fp32 store.  value = acc (+ bias[row]) (clamped at 0 if relu), rounded to nearest even.
+struct PackedOut {
+  void* ptr = nullptr;
+  int halo = 0, Cg = 0, Wp = 0;
+  int img_groups = 0;  // 16-byte groups per image: Hp * Cg * Wp
+  FastDiv dQ;          // division of a pixel index by Q
+};
+
+template <class T>
+__device__ __forceinline__ void store_tile_packed(const f32x16 (&acc)[T::TM][T::TN], const EpiParams& ep, const PackedOut& pk,
+                                                  int m0, int n0, int wm, int wn, int lane) {
+  constexpr int TM = T::TM, TN = T::TN;
+  char* const base = static_cast<char*>(pk.ptr);
+  const int sub = (lane >> 5) * 4;  // this lane's four rows inside a group of eight
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+    if (col >= ep.cols) continue;
+    const int img = col / ep.inner;
+    uint32_t p, q;
+    pk.dQ.divmod((uint32_t)(col - img * ep.inner), p, q);
+    const size_t g0 = (size_t)img * pk.img_groups + (size_t)((int)p + pk.halo) * pk.Cg * pk.Wp + (size_t)((int)q + pk.halo);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int rbase = m0 + wm * (TM * 32) + i * 32 + sub;
+#pragma unroll
+      for (int vg = 0; vg < 4; ++vg) {
+        const int row0 = rbase + vg * 8;
+        if (row0 < ep.rows) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float val = acc[i][j][vg * 4 + e];
+            if (ep.bias) val += ep.bias[row0 + e];
+            if (ep.relu) val = val > 0.0f ? val : 0.0f;
+            v[e] = val;
+          }
+          uint2 w;
+          w.x = pack_bf16(v[0], v[1]);
+          w.y = pack_bf16(v[2], v[3]);
+          *reinterpret_cast<uint2*>(base + (g0 + (size_t)(row0 >> 3) * pk.Wp) * 16 + sub * 2) = w;
+        }
+      }
+    }
+  }
+}
+
 // Pass tags: they only make the instantiations of one pass distinct kernels (and kernel names) from
 // those of another pass that uses the same tile and loaders.
 struct PassConvFwd {};
@@ -867,11 +918,11 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_kernel(typename AL::P
 // 16-byte groups, double buffered: a loader writes one ds_write_b128 per 8 values and an MFMA operand is one
 // ds_read_b128.
 // ------------------------------------------------------------------------------------------
-template <class T, class AL, class BL, bool NCHW, class PASS>
+template <class T, class AL, class BL, bool NCHW, class PASS, bool PK = false>
 __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_kernel(typename AL::Params ap,
                                                                        typename BL::Params bp, EpiParams ep,
                                                                        int tiles_m, int k_chunks,
-                                                                       int chunks_per_split) {
+                                                                       int chunks_per_split, PackedOut pk) {
   constexpr int BM = T::BM, BN = T::BN, BK = T::BK, TM = T::TM, TN = T::TN;
   static_assert(BK % 16 == 0, "one bf16 MFMA contracts 16 k");
   constexpr int KG = BK / 8;  // 16-byte groups per row and K step
@@ -967,7 +1018,8 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_kernel(typename 
   for (int it = 0; it + 1 < nk; ++it) k_step(it, std::true_type());
   if (nk > 0) k_step(nk - 1, std::false_type());
 
-  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, ep.split_stride != 0 ? split_idx : -1);
+  if constexpr (PK) store_tile_packed<T>(acc, ep, pk, m0, n0, wm, wn, lane);
+  else store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, ep.split_stride != 0 ? split_idx : -1);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1071,9 +1123,9 @@ struct DmaRowV8 {
   }
 };
 
-template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS>
+template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS, bool PK = false>
 __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8Params ap, RowV8Params bp, EpiParams ep,
-                                                                           int tiles_m, int k_chunks) {
+                                                                           int tiles_m, int k_chunks, PackedOut pk) {
   constexpr int BM = T::BM, BN = T::BN, BK = T::BK, TM = T::TM, TN = T::TN;
   static_assert(BK % 32 == 0, "an even number of 16-k groups per step keeps the operand register sets in phase");
   typedef DmaRowV8<BM, BK, T::NT, A_LINEAR> AL;
@@ -1191,7 +1243,8 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8
   for (; it + 3 < nk; ++it) step(it, std::true_type());
   for (; it < nk; ++it) step(it, std::false_type());
 
-  store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, -1);
+  if constexpr (PK) store_tile_packed<T>(acc, ep, pk, m0, n0, wm, wn, lane);
+  else store_tile<T, NCHW>(acc, ep, m0, n0, wm, wn, lane, -1);
 }
 
 }  // namespace rh

@@ -819,6 +819,17 @@ class Conv2dOperator : public Operator {
     // the data gradient can zero what the ReLU below would have masked in a pass of its own
     if (backward_enabled(capability) && in_delta_ && opts.fuse_epilogue && rh_conv2d_bwd_data_relu_supported(&g))
       fold_prev_relu_ = prev_op->fold_activation_backward();
+    if (opts.bf16_forward) {
+      // the converted filter is kept from one forward pass to the next for as long as the weights stay the same
+      const size_t fb = rh_conv2d_fwd_bf16_filter_bytes(&g);
+      if (fb) {
+        wprep_.reset(new DeviceBuffer<uint8_t>(fb, context));
+        const size_t wb = rh_conv2d_fwd_bf16_workspace_bytes(&g);
+        if (wb > workspace_->len()) workspace_.reset(new DeviceBuffer<uint8_t>(wb, context));
+        if (opts.bf16_packed_chain && rh_conv2d_fwd_bf16_takes_packed(&g) && prev_op->can_emit_packed())
+          in_packed_ = prev_op->emit_packed(g.pad);
+      }
+    }
   }
   size_t batch_size() const override { return batch_cap_; }
   SharedDeviceBuf get_output_vars() const override { return out_act_; }
@@ -826,6 +837,7 @@ class Conv2dOperator : public Operator {
   void init_params(const uint64_t seed[2]) override {
     const size_t fan_in = config_.conv_size * config_.conv_size * config_.in_dims.c;
     params_.init(config_.init_weights, seed, fan_in, config_.out_channels, false, "Conv2dOperator");
+    wprep_valid_ = false;
   }
   void forward(size_t batch_size, OpPhase) override {
     RB_ASSERT(batch_size <= batch_cap_);
@@ -833,6 +845,24 @@ class Conv2dOperator : public Operator {
     rh_stream_t s = context_->stream();
     const bool rect = config_.act_func == ActivationFunction::Rect;
     if (config_.act_func != ActivationFunction::Identity && !rect) panic("unimplemented activation function");
+    if (wprep_) {
+      if (!wprep_valid_) {
+        unwrap(rh_conv2d_fwd_bf16_prep_filter(&g, params_.weights->as_ptr(), wprep_->as_mut_ptr(), wprep_->len(), s),
+               "conv2d forward (filter conversion)");
+        wprep_valid_ = true;
+      }
+      const int flags = opts_.fuse_epilogue ? RH_FUSE_BIAS | (rect ? RH_FUSE_RELU : 0) : 0;
+      unwrap(rh_conv2d_fwd_bf16_packed(&g, in_packed_ ? in_packed_->as_ptr() : nullptr, in_packed_ ? nullptr : in_act_->as_ptr(),
+                                       wprep_->as_ptr(), params_.bias->as_ptr(), out_packed_ ? nullptr : out_act_->as_mut_ptr(),
+                                       out_packed_ ? out_packed_->as_mut_ptr() : nullptr, out_halo_, workspace_->as_mut_ptr(),
+                                       workspace_->len(), flags, s), "conv2d forward");
+      if (!opts_.fuse_epilogue) {   // (never with a packed output: can_emit_packed asks for the fused epilogue)
+        unwrap(rh_add_bias_nchw(params_.bias->as_ptr(), out_act_->as_mut_ptr(), (int)(out_dims_.w * out_dims_.h),
+                                (int)out_dims_.c, (int)batch_size, 1.0f, 1.0f, s), "add_bias");
+        apply_rect(config_.act_func, out_act_->as_mut_ptr(), out_dims_.len(), batch_size, s);
+      }
+      return;
+    }
     const int math = opts_.bf16_forward ? RH_MATH_BF16_MFMA_FP32ACC : 0;
     if (opts_.fuse_epilogue) {
       const int flags = RH_FUSE_BIAS | (rect ? RH_FUSE_RELU : 0) | math;
@@ -900,30 +930,52 @@ class Conv2dOperator : public Operator {
   }
   void regularize(Regularization reg) override { params_.regularize(reg); }
   void accumulate_grads(float scale, float momentum) override { params_.accumulate_grads(scale, momentum); }
-  void update_params(float scale) override { params_.update_params(scale); }
-  void update_params2(float g, float u) override { params_.update_params2(g, u); }
+  // (every method that can change the weights drops the converted filter of the bf16 forward)
+  void update_params(float scale) override { wprep_valid_ = false; params_.update_params(scale); }
+  void update_params2(float g, float u) override { wprep_valid_ = false; params_.update_params2(g, u); }
   void save_params() override { params_.save_params(); }
-  void restore_params() override { params_.restore_params(); }
+  void restore_params() override { wprep_valid_ = false; params_.restore_params(); }
   void reset() override { params_.reset(); }
-  void descend(float scale, float l2, bool fused) override { params_.descend(scale, l2, fused); }
+  void descend(float scale, float l2, bool fused) override { wprep_valid_ = false; params_.descend(scale, l2, fused); }
   void reset_gradients(float scale) override { params_.reset_gradients(scale); }
   void encode_params(std::vector<uint8_t>& blob) override { params_.encode_params(blob); }
-  size_t decode_params(const uint8_t* blob, size_t len) override { return params_.decode_params(blob, len, kind()); }
+  size_t decode_params(const uint8_t* blob, size_t len) override {
+    wprep_valid_ = false;
+    return params_.decode_params(blob, len, kind());
+  }
   void encode_state(std::vector<uint8_t>& blob) override { params_.encode_state(blob); }
   size_t decode_state(const uint8_t* blob, size_t len) override { return params_.decode_state(blob, len, kind()); }
   // Like the affine layers' updates, on the second stream, except for the first layer: the next forward pass joins
   // in front of the first operator that was updated there, and the first layer's forward is what the others hide behind.
   void fused_sgd_step(float l2, float scale, float mu, float apply) override {
+    wprep_valid_ = false;
     params_.fused_sgd_step(l2, scale, mu, apply, updates_on_second_stream() ? context_->aux_stream() : nullptr);
   }
-  void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) override { params_.sgd_tensors(l2, out); }
+  void sgd_tensors(float l2, std::vector<rh_sgd_tensor>& out) override { wprep_valid_ = false; params_.sgd_tensors(l2, out); }
   bool grads_stale() const override { return params_.grads_stale; }
   void set_grads_stale(bool stale) override { params_.grads_stale = stale && params_.has_backward(); }
   bool updates_on_second_stream() const override { return workspace_aux_ && overlap_on_ && in_delta_; }
   bool buffer(int which, float** ptr, size_t* len) override {
-    if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
+    if (which == 0) {
+      if (out_packed_)   // the activations live in the packed buffer: their values as fp32, on demand
+        unwrap(rh_bf16_unpack_nchw((int)batch_cap_, (int)out_dims_.c, (int)out_dims_.h, (int)out_dims_.w, out_halo_,
+                                   out_packed_->as_ptr(), out_act_->as_mut_ptr(), context_->stream()), "bf16 unpack");
+      *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true;
+    }
     if (which == 1) { *ptr = out_delta_->as_mut_ptr(); *len = out_delta_->len(); return true; }
+    if (which == 2 || which == 3) wprep_valid_ = false;   // the caller may write through the pointer
     return params_.buffer(which, ptr, len);
+  }
+  bool can_emit_packed() const override {
+    return opts_.bf16_packed_chain && opts_.fuse_epilogue && wprep_ && !out_packed_ && out_dims_.c % 8 == 0 &&
+           rh_bf16_act_bytes((int)batch_cap_, (int)out_dims_.c, (int)out_dims_.h, (int)out_dims_.w, 0) > 0;
+  }
+  std::shared_ptr<DeviceBuffer<uint8_t>> emit_packed(int halo) override {
+    const size_t bytes = rh_bf16_act_bytes((int)batch_cap_, (int)out_dims_.c, (int)out_dims_.h, (int)out_dims_.w, halo);
+    if (!can_emit_packed() || !bytes) panic("Conv2dOperator: no packed output for this configuration");
+    out_packed_.reset(new DeviceBuffer<uint8_t>(bytes, context_));   // zero-filled: the border stays zero
+    out_halo_ = halo;
+    return out_packed_;
   }
   const char* kind() const override { return "Conv2dOperator"; }
   bool fold_activation_backward() override {
@@ -952,13 +1004,19 @@ class Conv2dOperator : public Operator {
   ParamTensors params_;
   std::unique_ptr<DeviceBuffer<uint8_t>> workspace_, workspace_aux_;
   bool overlap_on_ = true;
+  // bf16 forward: the converted filter (valid until the weights change) and the packed activations on either side
+  std::unique_ptr<DeviceBuffer<uint8_t>> wprep_;
+  bool wprep_valid_ = false;
+  std::shared_ptr<DeviceBuffer<uint8_t>> in_packed_, out_packed_;
+  int out_halo_ = 0;
 };
 
 // ---- Pool2dOperator -------------------------------------------------------------------------------------
 class Pool2dOperator : public Operator {
  public:
   Pool2dOperator(size_t batch_size, const Pool2dOperatorConfig& config, Operator* prev_op, Ctx context, const ExecOptions& opts)
-      : batch_cap_(batch_size), config_(config), context_(context) {
+      : batch_cap_(batch_size), config_(config), context_(context), prev_op_(prev_op),
+        packed_chain_(opts.bf16_packed_chain) {
     RB_ASSERT(prev_op != nullptr);
     in_act_ = prev_op->get_output_vars();
     if (!in_act_) panic("Pool2dOperator missing required prev operator output vars");
@@ -980,8 +1038,27 @@ class Pool2dOperator : public Operator {
   void forward(size_t batch_size, OpPhase) override {
     RB_ASSERT(batch_size <= batch_cap_);
     const rh_pool_geom g = geom(batch_size);
+    if (out_packed_) {
+      unwrap(rh_pool2d_fwd_bf16_packed(&g, in_packed_->as_ptr(), out_packed_->as_mut_ptr(), out_halo_, context_->stream()),
+             "pooling forward");
+      return;
+    }
     unwrap(rh_pool2d_fwd(&g, in_act_->as_ptr(), out_act_->as_mut_ptr(), argmax_ ? argmax_->as_mut_ptr() : nullptr,
                          context_->stream()), "pooling forward");
+  }
+  // A max-pool between two convolutions of a packed bf16 chain pools the packed activations.
+  bool can_emit_packed() const override {
+    return packed_chain_ && !out_packed_ && config_.pool_op == PoolOperation::Max && config_.in_dims.c % 8 == 0 &&
+           prev_op_->can_emit_packed() &&
+           rh_bf16_act_bytes((int)batch_cap_, (int)out_dims_.c, (int)out_dims_.h, (int)out_dims_.w, 0) > 0;
+  }
+  std::shared_ptr<DeviceBuffer<uint8_t>> emit_packed(int halo) override {
+    const size_t bytes = rh_bf16_act_bytes((int)batch_cap_, (int)out_dims_.c, (int)out_dims_.h, (int)out_dims_.w, halo);
+    if (!can_emit_packed() || !bytes) panic("Pool2dOperator: no packed output for this configuration");
+    in_packed_ = prev_op_->emit_packed(0);
+    out_packed_.reset(new DeviceBuffer<uint8_t>(bytes, context_));   // zero-filled: the border stays zero
+    out_halo_ = halo;
+    return out_packed_;
   }
   void backward(size_t batch_size) override {
     if (!in_delta_) return;
@@ -996,7 +1073,12 @@ class Pool2dOperator : public Operator {
                          argmax_ ? argmax_->as_ptr() : nullptr, context_->stream()), "pooling backward");
   }
   bool buffer(int which, float** ptr, size_t* len) override {
-    if (which == 0) { *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true; }
+    if (which == 0) {
+      if (out_packed_)
+        unwrap(rh_bf16_unpack_nchw((int)batch_cap_, (int)out_dims_.c, (int)out_dims_.h, (int)out_dims_.w, out_halo_,
+                                   out_packed_->as_ptr(), out_act_->as_mut_ptr(), context_->stream()), "bf16 unpack");
+      *ptr = out_act_->as_mut_ptr(); *len = out_act_->len(); return true;
+    }
     if (which == 1) { *ptr = out_delta_->as_mut_ptr(); *len = out_delta_->len(); return true; }
     return false;
   }
@@ -1018,6 +1100,10 @@ class Pool2dOperator : public Operator {
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
   std::unique_ptr<DeviceBuffer<int32_t>> argmax_;
   bool fold_relu_ = false;  // backward also applies the producer's ReLU mask
+  Operator* prev_op_;       // (owned by the worker, which outlives this operator's use of it: construction only)
+  bool packed_chain_;
+  std::shared_ptr<DeviceBuffer<uint8_t>> in_packed_, out_packed_;
+  int out_halo_ = 0;
 };
 
 // ---- DropoutOperator (src/operator/mod.rs:2134-2255) -------------------------------------------------------
@@ -1843,6 +1929,7 @@ SequentialOperatorWorker::SequentialOperatorWorker(const SequentialOperatorConfi
   if (!config.has_loss) panic("SequentialOperatorWorker: missing loss operator");
   const uint64_t input_seed[2] = {shared_seed[0] ^ 0x44617461336421ull, shared_seed[1] + 0x9E3779B97F4A7C15ull};
   input_op_.reset(new Data3dOperator(batch_size, config.input_op.data3d, context, input_seed));
+  opts.bf16_packed_chain = opts.bf16_forward && !backward_enabled(capability);
   Operator* prev = input_op_.get();
   size_t params_off = 0;
   for (const auto& c : config.hidden_ops) {

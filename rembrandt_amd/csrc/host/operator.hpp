@@ -276,6 +276,9 @@ struct ExecOptions {
   bool graph_steps = false;
   bool fuse_epilogue = true;  // conv bias + ReLU in the conv epilogue instead of K1 -> K2 -> K3
   bool bf16_forward = false;  // conv forward on bf16-rounded operands with fp32 accumulation (inference mode)
+  // Set by the worker for forward-only chains with bf16_forward: neighbouring convolutions (and max-pools between
+  // them) hand each other packed bf16 activations instead of fp32 ones (same values as rounding the fp32 ones).
+  bool bf16_packed_chain = false;
   // Conv backward: filter and bias gradients on the context's second stream beside the data gradient on the
   // main one (the bandwidth-bound operand copies of one hide behind the other's contraction); joined at the end
   // of SequentialOperatorWorker::backward.
@@ -325,6 +328,13 @@ class Operator {
   // mask) asks for it at construction; an operator that agrees skips its own mask pass in backward().  The
   // out_delta buffer holds the same values after the chain's backward either way.
   virtual bool fold_activation_backward() { return false; }
+  // Packed bf16 activations (ExecOptions::bf16_packed_chain).  A convolution that reads a packed input asks the
+  // operator below, at construction, whether it can write its output in that form (can_emit_packed) and, if so, for
+  // the buffer (emit_packed, with the zero border the consumer's padding needs).  From then on the producer's forward
+  // writes the packed buffer instead of its fp32 out_act; buffer(0) still answers with fp32 values (the bf16 values,
+  // unpacked on demand).
+  virtual bool can_emit_packed() const { return false; }
+  virtual std::shared_ptr<DeviceBuffer<uint8_t>> emit_packed(int /*halo*/) { return nullptr; }
   // Switches the second-stream placement of gradient kernels on or off at run time (no effect on results, nor on
   // operators built without it).
   virtual void set_overlap_backward(bool /*on*/) {}

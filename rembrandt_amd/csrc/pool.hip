@@ -84,6 +84,51 @@ __global__ void pool_fwd_kernel(PoolDims d, const float* __restrict__ x, float* 
   }
 }
 
+// Max pooling on packed bf16 activations ([n][H][C/8][W][8] in, [n][P + 2*halo][C/8][Q + 2*halo][8] out, the border left
+// alone): one thread per output group of eight channels, same scan order and tie rule as above on each channel.
+// Rounding to bf16 is monotone, so the maximum of the rounded values is the rounded maximum: a chain that keeps its
+// activations packed gets the values a consumer would have rounded from the fp32 result.
+__global__ __launch_bounds__(256) void pool_max_fwd_bf16_kernel(PoolDims d, FastDiv dCg, const uint4* __restrict__ x,
+                                                               uint4* __restrict__ y, unsigned total, int halo) {
+  const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  uint32_t t, q, cg, n, p;
+  d.dQ.divmod(i, t, q);
+  dCg.divmod(t, t, cg);
+  d.dP.divmod(t, n, p);
+  const int Cg = (int)dCg.div;
+  const int hs = (int)p * d.st - d.pad, ws = (int)q * d.st - d.pad;
+  float best[8];
+  bool any = false;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) best[e] = 0.0f;
+  for (int r = 0; r < d.k; ++r) {
+    const int h = hs + r;
+    if ((unsigned)h >= (unsigned)d.H) continue;
+    const uint4* row = x + ((size_t)((int)n * d.H + h) * Cg + cg) * d.W;
+    for (int s = 0; s < d.k; ++s) {
+      const int w = ws + s;
+      if ((unsigned)w >= (unsigned)d.W) continue;
+      const uint4 v = row[w];
+      const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __builtin_bit_cast(float, u[e] << 16), hi = __builtin_bit_cast(float, u[e] & 0xffff0000u);
+        if (!any || lo > best[2 * e]) best[2 * e] = lo;
+        if (!any || hi > best[2 * e + 1]) best[2 * e + 1] = hi;
+      }
+      any = true;
+    }
+  }
+  uint4 o;
+  uint32_t* po = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+  for (int e = 0; e < 4; ++e)   // the values are bf16 already: their upper halves are the encoding
+    po[e] = (__builtin_bit_cast(uint32_t, best[2 * e]) >> 16) | (__builtin_bit_cast(uint32_t, best[2 * e + 1]) & 0xffff0000u);
+  const int Pp = d.P + 2 * halo, Qp = d.Q + 2 * halo;
+  y[((size_t)((int)n * Pp + (int)p + halo) * Cg + cg) * Qp + q + halo] = o;
+}
+
 // Forward with the input planes of a block staged in LDS: PB consecutive (n, c) planes are read with coalesced
 // loads, windows are scanned in LDS (overlapping windows re-read LDS, not L1), and y / arg-max are written
 // coalesced.  Same arithmetic and tie rule as pool_fwd_kernel.
@@ -470,6 +515,24 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
     hipLaunchKernelGGL(pool_fwd_kernel<unsigned>, grid, dim3(256), 0, to_stream(stream), d, x, y, opt_argmax);
   else
     hipLaunchKernelGGL(pool_fwd_kernel<long long>, grid, dim3(256), 0, to_stream(stream), d, x, y, opt_argmax);
+  return launch_status();
+}
+
+extern "C" int rh_pool2d_fwd_bf16_packed(const rh_pool_geom* g, const void* xp, void* yp, int32_t yp_halo,
+                                         rh_stream_t stream) {
+  PoolDims d;
+  if (int e = pool_dims(g, &d)) return e;
+  if (!xp || !yp || yp_halo < 0 || ((reinterpret_cast<uintptr_t>(xp) | reinterpret_cast<uintptr_t>(yp)) & 15)) return RH_E_INVALID;
+  if (d.mode != RH_POOL_MAX || d.C % 8 != 0) return RH_E_UNSUPPORTED;
+  const long long groups = (long long)d.N * (d.C / 8) * d.P * d.Q;
+  const long long in_bytes = 2ll * d.N * d.C * d.H * d.W;
+  const long long out_bytes = 2ll * d.N * d.C * (d.P + 2 * yp_halo) * (d.Q + 2 * yp_halo);
+  if (groups >= (1ll << 31) || in_bytes > (long long)kMaxBufferBytes || out_bytes > (long long)kMaxBufferBytes) return RH_E_LIMIT;
+  if (groups == 0) return 0;
+  ProfScope prof("pool_max_fwd_bf16", (double)in_bytes + 16.0 * (double)groups, to_stream(stream));
+  hipLaunchKernelGGL(pool_max_fwd_bf16_kernel, dim3(stream_grid((size_t)groups, 256)), dim3(256), 0, to_stream(stream), d,
+                     FastDiv((uint32_t)(d.C / 8)), static_cast<const uint4*>(xp), static_cast<uint4*>(yp), (unsigned)groups,
+                     yp_halo);
   return launch_status();
 }
 

@@ -191,6 +191,59 @@ def pool2d_fwd(x, size, stride, pad, mode, rounding=_lib.RH_ROUND_FLOOR, want_ar
     return (y, am) if want_argmax else y
 
 
+def bf16_pack(x, halo):
+    """fp32 NCHW -> packed bf16 activation tensor [n][H + 2 halo][C/8][W + 2 halo][8] (a uint8 tensor; zero border)."""
+    Nn, Cc, H, W = x.shape
+    nbytes = lib().rh_bf16_act_bytes(Nn, Cc, H, W, halo)
+    assert nbytes > 0, "no packed form for this shape"
+    xp = torch.zeros(nbytes, dtype=torch.uint8, device=x.device)
+    check(lib().rh_bf16_pack_nchw(Nn, Cc, H, W, halo, _p(x), _p(xp), _stream()), "rh_bf16_pack_nchw")
+    return xp
+
+
+def bf16_unpack(xp, shape, halo):
+    Nn, Cc, H, W = shape
+    x = torch.empty(tuple(shape), dtype=torch.float32, device=xp.device)
+    check(lib().rh_bf16_unpack_nchw(Nn, Cc, H, W, halo, _p(xp), _p(x), _stream()), "rh_bf16_unpack_nchw")
+    return x
+
+
+def conv2d_fwd_bf16_packed(x, w, stride, pad, bias=None, relu=False, x_packed=None, out_halo=None):
+    """The bf16 forward on a converted filter.  Input: `x_packed` (from bf16_pack(x, pad) or a producer) or the fp32 `x`
+    (x.shape is used for the geometry either way).  out_halo None: fp32 NCHW result; an int: packed bf16 result with
+    that border.  Returns the result tensor."""
+    g = conv_geom(x.shape, w.shape, stride, pad)
+    fb = lib().rh_conv2d_fwd_bf16_filter_bytes(C.byref(g))
+    assert fb > 0, "no packed form for this geometry"
+    wprep = torch.empty(fb, dtype=torch.uint8, device=w.device)
+    check(lib().rh_conv2d_fwd_bf16_prep_filter(C.byref(g), _p(w), _p(wprep), fb, _stream()), "rh_conv2d_fwd_bf16_prep_filter")
+    ws = workspace(lib().rh_conv2d_fwd_bf16_workspace_bytes(C.byref(g)), w.device)
+    shape = conv_out_shape(g)
+    y = yp = None
+    if out_halo is None:
+        y = torch.empty(shape, dtype=torch.float32, device=w.device)
+    else:
+        nbytes = lib().rh_bf16_act_bytes(shape[0], shape[1], shape[2], shape[3], out_halo)
+        assert nbytes > 0
+        yp = torch.zeros(nbytes, dtype=torch.uint8, device=w.device)
+    flags = (_lib.RH_FUSE_BIAS if bias is not None else 0) | (_lib.RH_FUSE_RELU if relu else 0)
+    check(lib().rh_conv2d_fwd_bf16_packed(C.byref(g), _p(x_packed), _p(None if x_packed is not None else x), _p(wprep), _p(bias),
+                                          _p(y), _p(yp), 0 if out_halo is None else out_halo, _p(ws), ws.numel(), flags,
+                                          _stream()), "rh_conv2d_fwd_bf16_packed")
+    return y if out_halo is None else yp
+
+
+def pool2d_fwd_bf16_packed(xp, x_shape, size, stride, pad, rounding=_lib.RH_ROUND_FLOOR, out_halo=0):
+    """Max pooling of a packed bf16 activation tensor (border 0) into a packed one with border out_halo."""
+    g = pool_geom(x_shape, size, stride, pad, _lib.RH_POOL_MAX, rounding)
+    shape = pool_out_shape(g)
+    nbytes = lib().rh_bf16_act_bytes(shape[0], shape[1], shape[2], shape[3], out_halo)
+    assert nbytes > 0
+    yp = torch.zeros(nbytes, dtype=torch.uint8, device=xp.device)
+    check(lib().rh_pool2d_fwd_bf16_packed(C.byref(g), _p(xp), _p(yp), out_halo, _stream()), "rh_pool2d_fwd_bf16_packed")
+    return yp, shape
+
+
 def pool2d_bwd(x, y, dy, size, stride, pad, mode, rounding=_lib.RH_ROUND_FLOOR, argmax=None):
     g = pool_geom(x.shape, size, stride, pad, mode, rounding)
     dx = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)

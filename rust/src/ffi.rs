@@ -220,6 +220,23 @@ extern "C" {
                            cached_mean: *const f32, cached_ivar: *const f32, ws: *mut c_void, ws_bytes: size_t,
                            stream: rh_stream_t) -> c_int;
 
+  // Packed bf16 activations for forward-only chains: producers write the consumer's operand, filters are converted once.
+  pub fn rh_bf16_act_bytes(n: i32, c: i32, h: i32, w: i32, halo: i32) -> size_t;
+  pub fn rh_bf16_pack_nchw(n: i32, c: i32, h: i32, w: i32, halo: i32, x: *const f32, xp: *mut c_void,
+                           stream: rh_stream_t) -> c_int;
+  pub fn rh_bf16_unpack_nchw(n: i32, c: i32, h: i32, w: i32, halo: i32, xp: *const c_void, x: *mut f32,
+                             stream: rh_stream_t) -> c_int;
+  pub fn rh_conv2d_fwd_bf16_filter_bytes(g: *const rh_conv_geom) -> size_t;
+  pub fn rh_conv2d_fwd_bf16_takes_packed(g: *const rh_conv_geom) -> c_int;
+  pub fn rh_conv2d_fwd_bf16_workspace_bytes(g: *const rh_conv_geom) -> size_t;
+  pub fn rh_conv2d_fwd_bf16_prep_filter(g: *const rh_conv_geom, w: *const f32, wprep: *mut c_void, wprep_bytes: size_t,
+                                        stream: rh_stream_t) -> c_int;
+  pub fn rh_conv2d_fwd_bf16_packed(g: *const rh_conv_geom, xp: *const c_void, x: *const f32, wprep: *const c_void,
+                                   bias: *const f32, y: *mut f32, yp: *mut c_void, yp_halo: i32, ws: *mut c_void,
+                                   ws_bytes: size_t, flags: c_int, stream: rh_stream_t) -> c_int;
+  pub fn rh_pool2d_fwd_bf16_packed(g: *const rh_pool_geom, xp: *const c_void, yp: *mut c_void, yp_halo: i32,
+                                   stream: rh_stream_t) -> c_int;
+
   // Per-launch timing and the calibration launches of the roofline report (no counterpart in the reference).
   pub fn rh_profile_enable(on: c_int) -> c_int;
   pub fn rh_profile_enabled() -> c_int;

@@ -194,9 +194,17 @@ def test_nin_train_step(dev):
     w.close()
 
 
+def _is_bf16_valued(a):
+    return not (np.ascontiguousarray(a, dtype=np.float32).view(np.uint32) & 0xFFFF).any()
+
+
 def test_nin_forward_bf16(dev):
     """Benchmark configuration 5, forward only with bf16 operands and fp32 accumulation.  Each operator is compared
-    from the GPU's own input to it (a last-bit difference upstream may round to a different bf16 value)."""
+    from the GPU's own input to it (a last-bit difference upstream may round to a different bf16 value).  A forward-only
+    worker keeps the activations between convolutions as packed bf16: such a layer's out_act reads back as the fp32
+    result rounded to nearest even, which is compared with the oracle's result rounded the same way (stated looser
+    bound: equal except where the last-bit difference of the accumulation moves a value across a rounding boundary,
+    then one bf16 step, 2^-7 relative, on at most 0.2 % of the elements; next to zero, the fp32 absolute bound)."""
     net, batch = configs.nin(), 2
     dims, layers, ncat = net
     cfg = configs.build_config(net, init_std=0.05)
@@ -212,16 +220,75 @@ def test_nin_forward_bf16(dev):
     w.load_frames_f32(x)
     w.forward(batch, training=False, t=0)
     prev = x
+    packed_layers = 0
     for i, op in enumerate(ref.hidden):
         want = op.forward(np.ascontiguousarray(prev.reshape(op.x_shape if hasattr(op, "x_shape") else prev.shape)))
         got = w.read(i, "out_act")
         assert np.abs(got).max() > 0, "layer %d is not all zero" % i
-        assert_close(got, want.ravel(), "nin bf16 out_act[%d] %s" % (i, op.kind))
+        if _is_bf16_valued(got) and not _is_bf16_valued(want):
+            packed_layers += 1
+            want_r = O.round_bf16(want).ravel()
+            diff = got != want_r
+            assert diff.mean() <= 2e-3, "nin bf16 out_act[%d] %s: %.3g of the elements round differently" % (i, op.kind, diff.mean())
+            # one bf16 step, or the fp32 tolerance itself where a value lies next to zero (a ReLU's cut)
+            slack = 2e-5 * max(1.0, float(np.sqrt(np.mean(want_r.astype(np.float64) ** 2))))
+            assert (np.abs(got - want_r) <= 2.0 ** -7 * np.abs(want_r) + slack).all(), "nin bf16 out_act[%d]: more than one bf16 step" % i
+        else:
+            assert_close(got, want.ravel(), "nin bf16 out_act[%d] %s" % (i, op.kind))
         prev = got.reshape(want.shape).copy()
+    assert packed_layers >= 11, packed_layers   # every convolution but the last, which feeds the average pool
     n = len(ref.hidden)
     assert_close(w.read(n, "out_act"), O.softmax_fwd(np.ascontiguousarray(prev.reshape(batch, ncat))).ravel(),
                  "nin bf16 softmax", atol=1e-7)
     w.close()
+
+
+@pytest.mark.parametrize("name", ["nin", "alexnet", "cifar10"])
+def test_bf16_packed_chain_is_bit_identical(dev, name):
+    """A forward-only bf16 worker (packed bf16 activations between convolutions, written by the producers' epilogues,
+    filters converted once) against a worker that keeps fp32 activations and converts every convolution's input
+    (Backward capability): every layer's activations are the other's rounded to bf16, bit for bit, and the final
+    probabilities are identical.  Then the converted filters: a second pass repeats the first, and a weight written
+    through the worker's buffer is seen by the next pass."""
+    net, batch = configs.NETWORKS[name](), 3
+    dims, layers, ncat = net
+    cfg = configs.build_config(net, init_std=0.05)
+    a = SequentialOperatorWorker(cfg, batch, "Forward", shared_seed=(0x5EED0015, 0x5EED0016), bf16_forward=True)
+    b = SequentialOperatorWorker(cfg, batch, "Backward", shared_seed=(0x5EED0015, 0x5EED0016), bf16_forward=True)
+    a.init_params()
+    b.init_params()
+    x = synth.normal(0x5EED0015, 101, (batch, dims[2], dims[1], dims[0]))
+    n = len(layers)
+
+    def run_and_compare(tag):
+        for w in (a, b):
+            w.load_frames_f32(x)
+            w.forward(batch, training=False, t=0)
+        packed = 0
+        for i in range(n):
+            ga, gb = a.read(i, "out_act"), b.read(i, "out_act")
+            assert np.abs(gb).max() > 0
+            if not np.array_equal(ga, gb):
+                packed += 1
+                assert np.array_equal(ga, O.round_bf16(gb)), "%s %s layer %d" % (tag, name, i)
+        pa, pb = a.read(n, "out_act"), b.read(n, "out_act")
+        assert np.array_equal(pa, pb), "%s %s probabilities" % (tag, name)
+        return packed, pa.copy()
+
+    say("bf16 packed chain", name)
+    packed, p1 = run_and_compare("first pass")
+    assert packed >= {"nin": 11, "alexnet": 3, "cifar10": 0}[name], packed   # (cifar10: stride-1 3-channel first layer, average pools)
+    _, p2 = run_and_compare("second pass")
+    assert np.array_equal(p1, p2)
+    conv_idx = [i for i, l in enumerate(layers) if l[0] == "conv2d"][1]
+    wts = a.read(conv_idx, "weights")
+    wts[::7] *= np.float32(-1.5)
+    a.write(conv_idx, "weights", wts)
+    b.write(conv_idx, "weights", wts)
+    _, p3 = run_and_compare("after a weight write")
+    assert not np.array_equal(p1, p3)
+    a.close()
+    b.close()
 
 
 def test_random_networks_train_steps(dev):

@@ -192,6 +192,76 @@ def test_conv2d_fwd_bf16_operands(dev, case):
     torch.cuda.synchronize()
 
 
+BF16_CHAIN_CASES = [
+    # N, C, H, W, K, R, stride, pad, halo of the packed result
+    (3, 72, 11, 9, 40, 3, 2, 1, 0),
+    (2, 8, 17, 17, 200, 5, 1, 2, 2),
+    (5, 16, 9, 12, 24, 3, 1, 0, 1),
+    (130, 8, 5, 5, 16, 3, 1, 1, 0),
+    (80, 24, 30, 30, 136, 5, 1, 2, 1),     # the direct-to-LDS kernel
+    (70, 512, 34, 33, 256, 1, 1, 0, 0),
+    (4, 3, 35, 35, 16, 7, 2, 0, 0),        # grouped by filter columns: fp32 image in, packed result out
+]
+
+
+@pytest.mark.parametrize("case", BF16_CHAIN_CASES, ids=[str(c) for c in BF16_CHAIN_CASES])
+def test_conv2d_fwd_bf16_packed_chain_forms(dev, case):
+    """The forms of the bf16 forward that a forward-only chain uses are bit-identical to rh_conv2d_fwd with
+    RH_MATH_BF16_MFMA_FP32ACC: a converted filter kept between calls, a packed bf16 input, and a packed bf16 result,
+    which holds the fp32 result rounded to nearest even inside a border that stays zero."""
+    Nn, C, H, W, K, R, st, pad, halo = case
+    say("bf16 chain case", case)
+    x = synth.normal(14, 1, (Nn, C, H, W))
+    w = synth.normal(14, 2, (K, C, R, R))
+    b = synth.normal(14, 3, (K,))
+    xd, wd, bd = T(x, dev), T(w, dev), T(b, dev)
+    for relu in (False, True):
+        legacy = ops.conv2d_fwd(xd, wd, st, pad, bias=bd, relu=relu, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)
+        y = ops.conv2d_fwd_bf16_packed(xd, wd, st, pad, bias=bd, relu=relu)
+        assert torch.equal(y, legacy), "fp32 image in, fp32 result"
+        yp = ops.conv2d_fwd_bf16_packed(xd, wd, st, pad, bias=bd, relu=relu, out_halo=halo)
+        want = O.round_bf16(N(legacy))
+        assert np.array_equal(N(ops.bf16_unpack(yp, legacy.shape, halo)), want), "packed result == rounded fp32 result"
+        # the border of the packed result is untouched (zero): re-packing the unpacked interior reproduces every byte
+        assert torch.equal(ops.bf16_pack(T(want, dev), halo), yp), "border"
+        if C % 8 == 0:
+            xp = ops.bf16_pack(xd, pad)
+            assert np.array_equal(N(ops.bf16_unpack(xp, x.shape, pad)), O.round_bf16(x)), "pack / unpack"
+            y2 = ops.conv2d_fwd_bf16_packed(xd, wd, st, pad, bias=bd, relu=relu, x_packed=xp)
+            assert torch.equal(y2, legacy), "packed image in, fp32 result"
+            yp2 = ops.conv2d_fwd_bf16_packed(xd, wd, st, pad, bias=bd, relu=relu, x_packed=xp, out_halo=halo)
+            assert torch.equal(yp2, yp), "packed image in, packed result"
+    torch.cuda.synchronize()
+
+
+BF16_POOL_CASES = [
+    # N, C, H, W, size, stride, pad, rounding, halo of the result
+    (3, 16, 13, 13, 3, 2, 0, 0, 1),
+    (2, 96, 54, 54, 3, 2, 0, 1, 2),     # ceil extent: clipped windows at the bottom / right edge
+    (4, 8, 9, 7, 2, 2, 0, 0, 0),
+    (2, 24, 10, 11, 3, 2, 1, 0, 1),     # padded windows: padding never wins
+    (1, 8, 5, 5, 3, 1, 1, 1, 0),
+]
+
+
+@pytest.mark.parametrize("case", BF16_POOL_CASES, ids=[str(c) for c in BF16_POOL_CASES])
+def test_pool2d_fwd_bf16_packed(dev, case):
+    """Max pooling of packed bf16 activations == the fp32 pooling's result rounded to bf16 (rounding is monotone),
+    bit for bit, on inputs with ties, negative values and all-negative windows."""
+    Nn, C, H, W, k, st, pad, rnd, halo = case
+    say("bf16 pool case", case)
+    x = synth.normal(15, 1, (Nn, C, H, W))
+    x[:, :, ::3, ::2] = np.float32(-0.75)     # ties
+    xd = T(x, dev)
+    want = O.round_bf16(N(ops.pool2d_fwd(xd, k, st, pad, _lib.RH_POOL_MAX, rnd)))
+    want_oracle = O.round_bf16(O.pool2d_fwd(x, k, st, pad, O.POOL_MAX, rnd))
+    assert np.array_equal(want, want_oracle)
+    yp, shape = ops.pool2d_fwd_bf16_packed(ops.bf16_pack(xd, 0), x.shape, k, st, pad, rnd, out_halo=halo)
+    assert np.array_equal(N(ops.bf16_unpack(yp, shape, halo)), want)
+    assert torch.equal(ops.bf16_pack(T(want, dev), halo), yp), "border"
+    torch.cuda.synchronize()
+
+
 SGEMM_CASES = [
     # transA, transB, m, n, k
     (1, 0, 500, 64, 2450),   # affine forward  Y = W^T X
