@@ -26,8 +26,12 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # row for reports `traffic: null`.
 TRAFFIC_SUMMARY = {"alexnet": "profiles/alexnet_b256_train_step_hbm_traffic.md"}
 PARITY_SUMMARY = "profiles/%s_b%d_train_step_parity.md"
-TOLERANCE = "|got-ref| <= 1e-5*max(1, rms(ref)) + 1e-4*|ref| and relative L2 <= 1e-4 against the fp64-accumulating CPU oracle; " \
-            "labels, arg-max, masks, counts exact"
+TOLERANCE = "asked: rel 1e-4 / abs 1e-5 (|got-ref| <= 1e-5 + 1e-4*|ref|), indices exact.  Tested: |got-ref| <= " \
+            "1e-5*max(1, rms(ref)) + 1e-4*|ref| (the absolute term grows with tensors whose values reach the tens: 1e-5 is " \
+            "below the fp32 resolution of their partial sums) and relative L2 <= 1e-4 against the fp64-accumulating CPU " \
+            "oracle; for tensors below unit scale (every backward tensor: values 1e-7 and smaller, where an absolute 1e-5 says " \
+            "nothing) the element-wise error is held to 2 * (1e-5*rms(ref) + 1e-4*|ref|) as well, reported per tensor class " \
+            "as `max_err_over_scaled_bound`; labels, arg-max, masks, counts exact"
 
 
 def measured_traffic(workload, kernel):
@@ -44,6 +48,10 @@ def measured_traffic(workload, kernel):
     row = re.search(r"^\| `%s` \|[^|]*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|" % re.escape(kernel), text, re.M)
     if not (f and w and row):
         return None, rel
+    lib_line = re.search(r"^Library: (.*)$", text, re.M)
+    from rembrandt_amd import _lib
+    if not lib_line or lib_line.group(1).strip() != _lib.lib().rh_version().decode():
+        rel += " (recorded with another build of the library: stale)"
     return 1024.0 * (float(f.group(1)) * float(row.group(1)) + float(w.group(1)) * float(row.group(2))), rel
 
 
@@ -61,6 +69,10 @@ def recorded_parity(workload, batch):
     rec = json.loads(text[a + 7:text.index("```", a + 7)])
     rec["source"] = rel
     rec["tolerance"] = TOLERANCE
+    # the summary names the library build it was recorded with: a different one at hand means the figures are of an
+    # older build (the test still ran, and passed, against this tolerance when this build's GPU tests ran)
+    from rembrandt_amd import _lib
+    rec["stale"] = rec.get("library") != _lib.lib().rh_version().decode()
     return rec
 
 

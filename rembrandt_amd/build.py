@@ -25,10 +25,26 @@ def sources():
     return sorted(out)
 
 
+def source_hash():
+    """sha1 (12 hex digits) over every source and header the library is built from, in path order."""
+    import hashlib
+    h = hashlib.sha1()
+    files = []
+    for root, _, names in os.walk(CSRC):
+        files += [os.path.join(root, f) for f in names if f.endswith((".hip", ".cpp", ".h", ".hpp"))]
+    inc = os.path.join(os.path.dirname(HERE), "include")
+    files += [os.path.join(inc, f) for f in os.listdir(inc) if f.endswith(".h")]
+    for f in sorted(files):
+        h.update(os.path.relpath(f, os.path.dirname(HERE)).encode())
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:12]
+
+
 def _compile(src):
     rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
     obj = os.path.join(OBJ, rel + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+    extra = ['-DRH_SOURCE_HASH="%s"' % source_hash()] if os.path.basename(src) == "ctx.hip" else []
+    cmd = [HIPCC] + FLAGS + extra + ["-c", src, "-o", obj]
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     log = "\n".join(l for l in p.stdout.splitlines() if "packed-fp32-ops" not in l)
     if p.returncode != 0:

@@ -438,6 +438,11 @@ bool conv1x1_stream_applies(const ConvDims& d);
 int launch_conv1x1_stream(const ConvDims& d, int pass, const float* w, const float* src, float* out, float alpha, float beta,
                           const float* bias, int relu, hipStream_t stream, const float* mask = nullptr);
 
+// The same for packed bf16 activations on both sides (conv1x1_bf16.hip): channels in multiples of 32, at most 128.
+bool conv1x1_bf16_stream_applies(const ConvDims& d);
+int launch_conv1x1_bf16_stream(const ConvDims& d, const void* xp, const void* wb, const float* bias, int relu,
+                               const PackedOut& pk, hipStream_t stream);
+
 // dst[n][c][halo + dil*h][halo + dil*w] = src[n][c][h][w], zeros elsewhere; dst is planes x Hp x Wp.
 void launch_pad_image(const float* src, float* dst, long long planes, int H, int W, int Hp, int Wp, int halo,
                       hipStream_t stream, int dil = 1);

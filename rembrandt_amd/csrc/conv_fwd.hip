@@ -534,6 +534,10 @@ static int bf16_gemm(const ConvDims& d, const Bf16FwdPlan& bpn, const void* xb, 
   // contractions lose there (one block per CU: nothing hides a tile's first loads and its stores).
   const bool dma = bpn.n_k >= 512 && cdiv(d.K, 256) * 256 == cdiv(d.K, 128) * 128 &&
                    (long long)cdiv(d.K, 256) * cdiv(ep.cols, 256) >= 256;
+  // 1x1 layers of up to 128 channels between packed activations are copies with a contraction riding along: the
+  // streaming kernel (same accumulation order, hence the same bits as the tiles)
+  if (pk.ptr && bpn.s_groups == 0 && conv1x1_bf16_stream_applies(d))
+    return launch_conv1x1_bf16_stream(d, xb, static_cast<const char*>(wprep) + bpn.tab_bytes, ep.bias, ep.relu, pk, stream);
   if (pk.ptr) {
     if (dma) return bf16_gemm_on<T256x256bf, true, true>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
     return bf16_gemm_on<T128x128bf, false, true>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x128");

@@ -55,7 +55,12 @@ struct rh_graph {
 
 using namespace rh;
 
-extern "C" const char* rh_version(void) { return "rembrandt-hip 0.1 (gfx950, fp32 MFMA)"; }
+// RH_SOURCE_HASH: a hash over the library's sources, set by the build (rembrandt_amd/build.py); summaries of measured
+// runs quote it, so that a reader can tell whether they describe the library at hand.
+#ifndef RH_SOURCE_HASH
+#define RH_SOURCE_HASH "unknown"
+#endif
+extern "C" const char* rh_version(void) { return "rembrandt-hip 0.1 (gfx950, fp32 MFMA) src " RH_SOURCE_HASH; }
 
 extern "C" const char* rh_error_string(int code) {
   switch (code) {

@@ -13,12 +13,36 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+# The element-wise error is also measured against a bound that shrinks with the tensor, 1e-5*rms(ref) + 1e-4*|ref|
+# (for a gradient tensor of values ~1e-8 an absolute 1e-5 says nothing), and asserted at this multiple of it.  The
+# worst element of the whole suite sits at 0.6 of that bound (an element near zero of a deep filter-gradient
+# contraction); the multiple leaves room for other summation orders, not for other arithmetic.
+TIGHT_MULTIPLE = 2.0
+LAST = {"tight_ratio": 0.0}   # max |got-ref| / (1e-5*rms + 1e-4*|ref|) of the most recent assert_close
+WORST = {"tight_ratio": 0.0, "what": ""}   # and of the whole session (written to gpurun_out/ at its end)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    if WORST["what"]:
+        try:
+            import json
+            os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+            with open(os.path.join(ROOT, "gpurun_out", "scaled_bound_worst.json"), "w") as f:
+                json.dump({"bound": "1e-5*rms(ref) + 1e-4*|ref|", "asserted_multiple": TIGHT_MULTIPLE,
+                           "worst_multiple_seen": WORST["tight_ratio"], "tensor": WORST["what"]}, f)
+        except OSError:
+            pass
+
+
 def assert_close(got, ref, what, rtol=1e-4, atol=1e-5, scale_atol=True):
     """fp32 parity bound |got - ref| <= atol' + rtol*|ref| against the fp64-accumulated oracle.
 
     atol' = atol * max(1, rms(ref)): an absolute 1e-5 is below the fp32 resolution of the partial
     sums once a tensor's values reach the tens (N(0,1) x N(0,1) contractions of depth ~2400), so
     the absolute term follows the tensor's scale; for unit-scale tensors it is exactly 1e-5.
+    Tensors below unit scale are held to the relative L2 bound and to TIGHT_MULTIPLE times the bound
+    atol*rms(ref) + rtol*|ref|, element by element, so a local error in a small-valued tensor cannot
+    hide inside the norm.
     """
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
@@ -34,6 +58,17 @@ def assert_close(got, ref, what, rtol=1e-4, atol=1e-5, scale_atol=True):
     if ref_norm > 0.0:
         rel_l2 = float(np.sqrt(np.sum(err * err))) / ref_norm
         assert rel_l2 <= 1e-4, "%s: relative L2 error %.3g > 1e-4" % (what, rel_l2)
+    LAST["tight_ratio"] = 0.0
+    if scale_atol and ref.size and ref_norm > 0.0:
+        tight = atol * float(np.sqrt(np.mean(ref * ref))) + rtol * np.abs(ref)
+        ratio = err / tight
+        j = int(np.argmax(ratio))
+        LAST["tight_ratio"] = float(ratio.ravel()[j])
+        if LAST["tight_ratio"] > WORST["tight_ratio"]:
+            WORST["tight_ratio"], WORST["what"] = LAST["tight_ratio"], what
+        assert LAST["tight_ratio"] <= TIGHT_MULTIPLE, \
+            "%s: element %d is %.3g times the bound 1e-5*rms + 1e-4*|ref| (got %r ref %r, rms %.3g; allowed %g)" % (
+                what, j, LAST["tight_ratio"], got.ravel()[j], ref.ravel()[j], float(np.sqrt(np.mean(ref * ref))), TIGHT_MULTIPLE)
     bound = a + rtol * np.abs(ref)
     bad = err > bound
     if bad.any():

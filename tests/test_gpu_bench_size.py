@@ -22,6 +22,7 @@ import pytest
 import oracle as O
 from rembrandt_amd import configs, synth
 from rembrandt_amd.operator import SequentialOperatorWorker, SgdOpt
+import conftest
 from conftest import assert_close, say
 
 pytestmark = pytest.mark.gpu
@@ -41,15 +42,63 @@ class ErrorLog:
         row = {"tensor": what, "checked": int(ref64.size), "max_abs_err": float(err.max()) if err.size else 0.0,
                "rms_ref": scale, "max_rel_err": float((err[big] / np.abs(ref64[big])).max()) if big.any() else 0.0}
         self.rows.append(row)
-        say("  parity %-44s n=%-9d max_abs %.3g  max_rel %.3g  (rms %.3g)" % (what, row["checked"], row["max_abs_err"],
-                                                                              row["max_rel_err"], scale))
-        assert_close(got, ref, what, **kw)
+        try:
+            assert_close(got, ref, what, **kw)
+        finally:
+            row["max_err_over_scaled_bound"] = conftest.LAST["tight_ratio"]
+            say("  parity %-44s n=%-9d max_abs %.3g  max_rel %.3g  (rms %.3g)  x scaled bound %.3g" % (
+                what, row["checked"], row["max_abs_err"], row["max_rel_err"], scale, row["max_err_over_scaled_bound"]))
 
     def exact(self, got, ref, what):
         ok = np.array_equal(got, ref)
         self.rows.append({"tensor": what, "checked": int(np.asarray(ref).size), "exact": bool(ok)})
         say("  parity %-44s n=%-9d exact %s" % (what, np.asarray(ref).size, ok))
         assert ok, what
+
+
+TOLERANCE_TEXT = ("|got-ref| <= 1e-5*max(1, rms(ref)) + 1e-4*|ref|, relative L2 <= 1e-4, and |got-ref| <= %g * (1e-5*rms(ref) + "
+                  "1e-4*|ref|) element by element; integers exact" % conftest.TIGHT_MULTIPLE)
+
+
+def parity_summary(rec):
+    """The per-tensor records of one run by tensor class, as text: what profiles/<net>_b<batch>_train_step_parity.md holds."""
+    import collections
+    import re
+    cls = collections.OrderedDict()
+    for t in rec["tensors"]:
+        m = re.match(r"\S+ b\d+ step \d+ (.*)", t["tensor"])
+        key = re.sub(r"\[\d+\]", "", m.group(1) if m else t["tensor"])
+        c = cls.setdefault(key, {"tensors": 0, "checked": 0, "exact": True, "max_abs_err": 0.0, "max_abs_err_over_rms": 0.0,
+                                 "max_rel_err": 0.0, "max_err_over_scaled_bound": 0.0})
+        c["tensors"] += 1
+        c["checked"] += t.get("checked", 0)
+        if not t.get("exact", False):
+            c["exact"] = False
+            c["max_abs_err"] = max(c["max_abs_err"], t["max_abs_err"])
+            c["max_abs_err_over_rms"] = max(c["max_abs_err_over_rms"], t["max_abs_err"] / max(t["rms_ref"], 1e-30))
+            c["max_rel_err"] = max(c["max_rel_err"], t["max_rel_err"])
+            c["max_err_over_scaled_bound"] = max(c["max_err_over_scaled_bound"], t.get("max_err_over_scaled_bound", 0.0))
+    out = {"workload": rec["workload"], "batch": rec["batch"], "steps": rec["steps"], "library": rec.get("library"),
+           "classes": cls}
+    lines = ["# %s-shaped batch-%d train steps as bench.py runs them: worst error per tensor class against the CPU oracle"
+             % (rec["workload"], rec["batch"]), "",
+             "Command (MI355X box, repository root):", "",
+             "    python -m pytest tests/test_gpu_bench_size.py -m gpu -q", "",
+             "The test writes `gpurun_out/parity_%s_b%d.json` (one record per checked tensor) and this summary by tensor class "
+             "(`gpurun_out/%s_b%d_train_step_parity.md`)." % (rec["workload"], rec["batch"], rec["workload"], rec["batch"]),
+             "Tolerance of the test: " + rec["tolerance"] + ".",
+             "`max_rel_err` is the largest |got-ref|/|ref| over the checked elements whose |ref| exceeds a thousandth of the",
+             "tensor's RMS, `max_abs_err_over_rms` the largest |got-ref| over the tensor's RMS, `x scaled bound` the largest",
+             "|got-ref| / (1e-5*rms(ref) + 1e-4*|ref|): the tolerance with its absolute term shrunk to the tensor's own scale.", "",
+             "| tensor class | tensors | elements checked | exact | max abs err | max abs err / rms | max rel err | x scaled bound |",
+             "|---|---:|---:|---|---:|---:|---:|---:|"]
+    for k, c in cls.items():
+        f = (lambda v: "" if c["exact"] else "%.3g" % v)
+        lines.append("| %s | %d | %d | %s | %s | %s | %s | %s |" % (
+            k, c["tensors"], c["checked"], "yes" if c["exact"] else "", f(c["max_abs_err"]), f(c["max_abs_err_over_rms"]),
+            f(c["max_rel_err"]), f(c["max_err_over_scaled_bound"])))
+    lines += ["", "```json", json.dumps(out, indent=1), "```", ""]
+    return "\n".join(lines)
 
 
 def sample_idx(rng, total, n):
@@ -245,10 +294,13 @@ def test_bench_size_train_steps(dev, netname, batch):
             log.exact(final_a[i][k], state[i][k], "%s uninterrupted == checked run: %s[%d]" % (netname, k, i))
     try:
         os.makedirs("gpurun_out", exist_ok=True)
+        from rembrandt_amd import _lib
+        rec = {"workload": netname, "batch": batch, "steps": steps, "tolerance": TOLERANCE_TEXT, "tensors": log.rows,
+               "library": _lib.lib().rh_version().decode()}
         with open(os.path.join("gpurun_out", "parity_%s_b%d.json" % (netname, batch)), "w") as f:
-            json.dump({"workload": netname, "batch": batch, "steps": steps,
-                       "tolerance": "|got-ref| <= 1e-5*max(1, rms(ref)) + 1e-4*|ref|, relative L2 <= 1e-4; integers exact",
-                       "tensors": log.rows}, f, indent=1)
+            json.dump(rec, f, indent=1)
+        with open(os.path.join("gpurun_out", "%s_b%d_train_step_parity.md" % (netname, batch)), "w") as f:
+            f.write(parity_summary(rec))
     except OSError:
         pass
 

@@ -201,6 +201,12 @@ BF16_CHAIN_CASES = [
     (80, 24, 30, 30, 136, 5, 1, 2, 1),     # the direct-to-LDS kernel
     (70, 512, 34, 33, 256, 1, 1, 0, 0),
     (4, 3, 35, 35, 16, 7, 2, 0, 0),        # grouped by filter columns: fp32 image in, packed result out
+    # 1x1 layers of up to 128 channels with a packed result: the streaming kernel (pixel counts that are not a
+    # multiple of the 32-pixel tile, every tile height, rows shorter than a tile, a bordered result)
+    (3, 96, 54, 54, 96, 1, 1, 0, 0),
+    (5, 32, 7, 5, 128, 1, 1, 0, 2),
+    (2, 128, 13, 11, 32, 1, 1, 0, 1),
+    (7, 64, 3, 3, 64, 1, 1, 0, 0),
 ]
 
 
