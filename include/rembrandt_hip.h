@@ -251,6 +251,16 @@ int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float* y, const f
 int rh_pool2d_bwd_relu_supported(const rh_pool_geom* g);
 int rh_pool2d_bwd_relu(const rh_pool_geom* g, const float* y, const float* dy, float* dx, const int32_t* argmax,
                        rh_stream_t stream);
+/* The same pooling with a one-byte mask: slot[n,c,p,q] = r*size + s of the winning element inside its window (first
+ * maximum, as above), 255 for a window without elements.  For an operator's private mask (a quarter of the int32
+ * form's bytes on both passes; the gen-1 API's int32 plane index, src/layer.rs:1797-1813, stays rh_pool2d_fwd's).
+ * rh_pool2d_slot_supported: nonzero for the geometries that have this form (max pooling, size <= 15, planes that fit the
+ * LDS kernels).  rh_pool2d_bwd_slot: dx from dy and the slots; with relu_y (the pooled outputs) it also applies the
+ * backward mask of the ReLU that produced x, as rh_pool2d_bwd_relu does. */
+int rh_pool2d_slot_supported(const rh_pool_geom* g);
+int rh_pool2d_fwd_slot(const rh_pool_geom* g, const float* x, float* y, uint8_t* slot, rh_stream_t stream);
+int rh_pool2d_bwd_slot(const rh_pool_geom* g, const float* relu_y, const float* dy, float* dx, const uint8_t* slot,
+                       rh_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Softmax / KL loss / reductions.  rh_softmax_fwd replaces CudnnSoftmaxOp::forward
@@ -414,7 +424,9 @@ int rh_rng_fill_uniform01_device(uint64_t seed, uint64_t stream_id, uint64_t fir
  *   rh_conv2d_fwd_bf16_packed                 y = conv(x, w) (+ bias) (ReLU) from exactly one of `xp` (packed, halo =
  *                                             g->pad) and `x` (fp32 NCHW, converted into `ws` of
  *                                             rh_conv2d_fwd_bf16_workspace_bytes), to exactly one of `y` (fp32 NCHW) and
- *                                             `yp` (packed with halo yp_halo; K a multiple of 8).  flags: RH_FUSE_*.
+ *                                             `yp` (packed with halo yp_halo; K a multiple of 8).  flags: RH_FUSE_*;
+ *                                             RH_ALGO_SCALAR_OFFSET takes the streaming 1x1 kernel wherever it can run
+ *                                             (tests: the same bits as the kernel chosen by default).
  *   rh_pool2d_fwd_bf16_packed                 max pooling from a packed input (halo 0) to a packed output.
  * ------------------------------------------------------------------------------------------- */
 size_t rh_bf16_act_bytes(int32_t N, int32_t C, int32_t H, int32_t W, int32_t halo);

@@ -113,6 +113,9 @@ PROTOTYPES = {
     "rh_pool2d_bwd": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp, _vp, _vp]),
     "rh_pool2d_bwd_relu_supported": (_int, [C.POINTER(PoolGeom)]),
     "rh_pool2d_bwd_relu": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp, _vp]),
+    "rh_pool2d_slot_supported": (_int, [C.POINTER(PoolGeom)]),
+    "rh_pool2d_fwd_slot": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp]),
+    "rh_pool2d_bwd_slot": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp, _vp]),
     "rh_softmax_fwd": (_int, [_vp, _vp, _i32, _i32, _vp]),
     "rembrandt_kernel_batch_map_softmax_kl_backward": (None, [_vp, _i32, _i32, _vp, _vp, _vp, _vp]),
     "rembrandt_kernel_batch_map_softmax_kl_loss1": (None, [_vp, _i32, _i32, _vp, _vp, _f, _vp, _vp]),

@@ -439,7 +439,8 @@ int launch_conv1x1_stream(const ConvDims& d, int pass, const float* w, const flo
                           const float* bias, int relu, hipStream_t stream, const float* mask = nullptr);
 
 // The same for packed bf16 activations on both sides (conv1x1_bf16.hip): channels in multiples of 32, at most 128.
-bool conv1x1_bf16_stream_applies(const ConvDims& d);
+bool conv1x1_bf16_stream_applies(const ConvDims& d);   // the layers it is chosen for
+bool conv1x1_bf16_stream_runs(const ConvDims& d);      // the layers it can run (RH_ALGO_SCALAR_OFFSET forces it on those)
 int launch_conv1x1_bf16_stream(const ConvDims& d, const void* xp, const void* wb, const float* bias, int relu,
                                const PackedOut& pk, hipStream_t stream);
 

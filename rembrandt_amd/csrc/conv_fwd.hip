@@ -528,7 +528,7 @@ static int bf16_gemm_on(const ConvDims& d, const Bf16FwdPlan& bpn, const void* x
 }
 
 static int bf16_gemm(const ConvDims& d, const Bf16FwdPlan& bpn, const void* xb, const void* wprep, const EpiParams& ep,
-                     const PackedOut& pk, hipStream_t stream) {
+                     const PackedOut& pk, hipStream_t stream, bool force_stream = false) {
   // Long contractions on grids that fill all 256 CUs with 256-row tiles (and waste no more filter rows than
   // 128-row tiles would) take the direct-to-LDS kernel: 14 % faster on 256 x 96 x 27 x 27 -> 256, 5x5.  Short
   // contractions lose there (one block per CU: nothing hides a tile's first loads and its stores).
@@ -536,7 +536,7 @@ static int bf16_gemm(const ConvDims& d, const Bf16FwdPlan& bpn, const void* xb, 
                    (long long)cdiv(d.K, 256) * cdiv(ep.cols, 256) >= 256;
   // 1x1 layers of up to 128 channels between packed activations are copies with a contraction riding along: the
   // streaming kernel (same accumulation order, hence the same bits as the tiles)
-  if (pk.ptr && bpn.s_groups == 0 && conv1x1_bf16_stream_applies(d))
+  if (pk.ptr && bpn.s_groups == 0 && (conv1x1_bf16_stream_applies(d) || (force_stream && conv1x1_bf16_stream_runs(d))))
     return launch_conv1x1_bf16_stream(d, xb, static_cast<const char*>(wprep) + bpn.tab_bytes, ep.bias, ep.relu, pk, stream);
   if (pk.ptr) {
     if (dma) return bf16_gemm_on<T256x256bf, true, true>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
@@ -746,7 +746,7 @@ extern "C" int rh_conv2d_fwd_bf16_packed(const rh_conv_geom* g, const void* xp, 
   if (int e = conv_dims(g, &d)) return e;
   if ((!xp) == (!x) || !wprep || (!y) == (!yp)) return RH_E_INVALID;  // one input form, one output form
   if ((flags & RH_FUSE_BIAS) && !bias) return RH_E_INVALID;
-  if (flags & ~(RH_FUSE_BIAS | RH_FUSE_RELU)) return RH_E_INVALID;
+  if (flags & ~(RH_FUSE_BIAS | RH_FUSE_RELU | RH_ALGO_SCALAR_OFFSET)) return RH_E_INVALID;
   const Bf16FwdPlan bpn = plan_bf16_fwd(d);
   if (!bpn.ok) return RH_E_UNSUPPORTED;
   if (xp && bpn.s_groups > 0) return RH_E_UNSUPPORTED;  // grouped by filter columns: the copy is made from the fp32 image
@@ -773,5 +773,6 @@ extern "C" int rh_conv2d_fwd_bf16_packed(const rh_conv_geom* g, const void* xp, 
     pk.img_groups = (d.P + 2 * yp_halo) * pk.Cg * pk.Wp;
     pk.dQ = FastDiv((uint32_t)d.Q);
   }
-  return bf16_gemm(d, bpn, xb, wprep, ep, pk, stream);
+  // (RH_ALGO_SCALAR_OFFSET: the streaming 1x1 kernel wherever it can run, not only where it is the faster one)
+  return bf16_gemm(d, bpn, xb, wprep, ep, pk, stream, (flags & RH_ALGO_SCALAR_OFFSET) != 0);
 }

@@ -1027,8 +1027,10 @@ class Pool2dOperator : public Operator {
     out_delta_.reset(new DeviceBuffer<float>(out_dims_.len() * batch_size, context));
     // private arg-max mask: lets backward route deltas without re-scanning the windows
     if (config.pool_op == PoolOperation::Max && in_delta_) {
-      argmax_.reset(new DeviceBuffer<int32_t>(out_dims_.len() * batch_size, context));
       const rh_pool_geom g = geom(batch_size);
+      // one byte per window (the winner's slot) where the library has that form, else the int32 plane index
+      if (rh_pool2d_slot_supported(&g)) slot_.reset(new DeviceBuffer<uint8_t>(out_dims_.len() * batch_size, context));
+      else argmax_.reset(new DeviceBuffer<int32_t>(out_dims_.len() * batch_size, context));
       if (opts.fuse_epilogue && rh_pool2d_bwd_relu_supported(&g)) fold_relu_ = prev_op->fold_activation_backward();
     }
   }
@@ -1040,6 +1042,11 @@ class Pool2dOperator : public Operator {
     const rh_pool_geom g = geom(batch_size);
     if (out_packed_) {
       unwrap(rh_pool2d_fwd_bf16_packed(&g, in_packed_->as_ptr(), out_packed_->as_mut_ptr(), out_halo_, context_->stream()),
+             "pooling forward");
+      return;
+    }
+    if (slot_) {
+      unwrap(rh_pool2d_fwd_slot(&g, in_act_->as_ptr(), out_act_->as_mut_ptr(), slot_->as_mut_ptr(), context_->stream()),
              "pooling forward");
       return;
     }
@@ -1064,6 +1071,11 @@ class Pool2dOperator : public Operator {
     if (!in_delta_) return;
     RB_ASSERT(batch_size <= batch_cap_);
     const rh_pool_geom g = geom(batch_size);
+    if (slot_) {
+      unwrap(rh_pool2d_bwd_slot(&g, fold_relu_ ? out_act_->as_ptr() : nullptr, out_delta_->as_ptr(), in_delta_->as_mut_ptr(),
+                                slot_->as_ptr(), context_->stream()), "pooling backward");
+      return;
+    }
     if (fold_relu_) {
       unwrap(rh_pool2d_bwd_relu(&g, out_act_->as_ptr(), out_delta_->as_ptr(), in_delta_->as_mut_ptr(), argmax_->as_ptr(),
                                 context_->stream()), "pooling backward");
@@ -1098,7 +1110,8 @@ class Pool2dOperator : public Operator {
   Ctx context_;
   Dims3 out_dims_;
   SharedDeviceBuf in_act_, in_delta_, out_act_, out_delta_;
-  std::unique_ptr<DeviceBuffer<int32_t>> argmax_;
+  std::unique_ptr<DeviceBuffer<int32_t>> argmax_;   // private arg-max mask, one of the two forms
+  std::unique_ptr<DeviceBuffer<uint8_t>> slot_;
   bool fold_relu_ = false;  // backward also applies the producer's ReLU mask
   Operator* prev_op_;       // (owned by the worker, which outlives this operator's use of it: construction only)
   bool packed_chain_;

@@ -7,7 +7,29 @@
 
 namespace rh {
 
-struct PoolDims { int N, C, H, W, k, st, pad, P, Q, mode; FastDiv dP, dQ, dH, dW, dSt; };
+struct PoolDims { int N, C, H, W, k, st, pad, P, Q, mode; FastDiv dP, dQ, dH, dW, dSt, dK; };
+
+// The arg-max mask of a max-pool comes in two encodings.  int32: the index h*W + w of the winning element inside its
+// plane, -1 for a window without elements (the form of rh_pool2d_fwd / rh_pool2d_bwd).  uint8: the winner's slot
+// r*size + s inside its window, 255 for none (size <= 15): a quarter of the bytes, for an operator's private mask.
+template <class MT> struct MaskCode;
+template <> struct MaskCode<int> {
+  // plane: index inside the plane (or -1); hs, ws: the window's first row / column
+  static __device__ __forceinline__ int from_plane(int plane, int, int, int, int) { return plane; }
+  static __device__ __forceinline__ int to_plane(int m, int, int, const PoolDims&) { return m; }
+};
+template <> struct MaskCode<uint8_t> {
+  static __device__ __forceinline__ uint8_t from_plane(int plane, int hs, int ws, int W, int k) {
+    if (plane < 0) return 255;
+    const int h = plane / W, w = plane - h * W;
+    return (uint8_t)((h - hs) * k + (w - ws));
+  }
+  static __device__ __forceinline__ int to_plane(uint8_t m, int hs, int ws, const PoolDims& d) {
+    if (m == 255) return -1;
+    const uint32_t r = d.dK.quot(m), s2 = m - r * (uint32_t)d.k;
+    return (hs + (int)r) * d.W + ws + (int)s2;
+  }
+};
 
 inline int pool_out_dim(int in, int size, int stride, int pad, int round) {
   if (round == RH_ROUND_CEIL) {
@@ -136,10 +158,10 @@ __global__ __launch_bounds__(256) void pool_max_fwd_bf16_kernel(PoolDims d, Fast
 // padding and with an exact cover) are scanned by unrolled code from one base address, in the same order.
 // Planes above the block's LDS share are cut into bands of `rb` output rows (bands > 1, PB = 1): a block stages the
 // input rows its band's windows reach, a contiguous piece of the plane.
-template <int K, int ST>
+template <int K, int ST, class MT>
 __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv dPQ, int PB, long long planes, int bands, int rb,
                                                            FastDiv dBands, const float* __restrict__ x,
-                                                           float* __restrict__ y, int* __restrict__ argmax) {
+                                                           float* __restrict__ y, MT* __restrict__ argmax) {
   extern __shared__ float lds_pool[];
   const int HW = d.H * d.W, PQ = d.P * d.Q;
   long long plane0 = (long long)blockIdx.x * PB;
@@ -176,7 +198,7 @@ __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv d
   }
   __syncthreads();
   float* gy = y + plane0 * PQ + p0 * d.Q;
-  int* gm = argmax ? argmax + plane0 * PQ + p0 * d.Q : nullptr;
+  MT* gm = argmax ? argmax + plane0 * PQ + p0 * d.Q : nullptr;
   const float inv = 1.0f / (float)(d.k * d.k);
   for (int o = threadIdx.x; o < n_out; o += 256) {
     uint32_t pl = 0, pq = (uint32_t)(o + p0 * d.Q), p, q;
@@ -190,17 +212,17 @@ __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv d
         const float* b = xp + (first - base);
         if (d.mode == RH_POOL_MAX) {
           float best = b[0];
-          int bi = 0;
+          int bi = 0;   // the winner's offset from the window's first element, or its slot
 #pragma unroll
           for (int r = 0; r < K; ++r)
 #pragma unroll
             for (int s2 = 0; s2 < K; ++s2) {
               if (r == 0 && s2 == 0) continue;
               const float v = b[r * d.W + s2];
-              if (v > best) { best = v; bi = r * d.W + s2; }
+              if (v > best) { best = v; bi = sizeof(MT) == 1 ? r * K + s2 : r * d.W + s2; }
             }
           gy[o] = best;
-          if (gm) gm[o] = first + bi;
+          if (gm) gm[o] = sizeof(MT) == 1 ? (MT)bi : (MT)(first + bi);
         } else {
           float acc = 0.0f;
 #pragma unroll
@@ -216,7 +238,7 @@ __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv d
       float best;
       const int bi = window_argmax(xp, d.H, d.W, (int)p, (int)q, d.k, d.st, d.pad, &best, base);
       gy[o] = bi < 0 ? 0.0f : best;
-      if (gm) gm[o] = bi;
+      if (gm) gm[o] = MaskCode<MT>::from_plane(bi, (int)p * d.st - d.pad, (int)q * d.st - d.pad, d.W, d.k);
     } else {
       float acc = 0.0f;
       const int hs = (int)p * d.st - d.pad, ws = (int)q * d.st - d.pad;
@@ -361,9 +383,9 @@ struct PoolColors {
   FastDiv dCnt[4], dQb[2];
 };
 
-template <int J>
+template <int J, class MT>
 __global__ __launch_bounds__(256) void pool_bwd_mask_color_kernel(PoolDims d, PoolColors pc, int PB, long long planes,
-                                                                  const float* __restrict__ dy, const int* __restrict__ argmax,
+                                                                  const float* __restrict__ dy, const MT* __restrict__ argmax,
                                                                   const float* __restrict__ y, float* __restrict__ dx) {
   extern __shared__ float lds_pool[];
   const int PQ = d.P * d.Q, HW = d.H * d.W;
@@ -371,7 +393,7 @@ __global__ __launch_bounds__(256) void pool_bwd_mask_color_kernel(PoolDims d, Po
   const int np = (int)(planes - plane0 < PB ? planes - plane0 : PB);
   const int n_in = np * HW;
   const float* gdy = dy + plane0 * PQ;
-  const int* gm = argmax + plane0 * PQ;
+  const MT* gm = argmax + plane0 * PQ;
   const float* gy = y ? y + plane0 * PQ : nullptr;
   float* gdx = dx + plane0 * HW;
   // the LDS copy keeps the global address's position inside a 16-byte group
@@ -395,8 +417,9 @@ __global__ __launch_bounds__(256) void pool_bwd_mask_color_kernel(PoolDims d, Po
           uint32_t pl, rem, i, jj;
           pc.dCnt[c].divmod((uint32_t)t, pl, rem);
           pc.dQb[b].divmod(rem, i, jj);
-          const int o = (int)pl * PQ + ((int)i * pc.nA + a) * d.Q + (int)jj * pc.nA + b;
-          int m = gm[o];
+          const int wp = (int)i * pc.nA + a, wq = (int)jj * pc.nA + b;
+          const int o = (int)pl * PQ + wp * d.Q + wq;
+          int m = MaskCode<MT>::to_plane(gm[o], wp * d.st - d.pad, wq * d.st - d.pad, d);
           val[c][j] = gdy[o];
           if (gy && !(gy[o] > 0.0f)) m = -1;  // a window whose maximum is not positive routes nothing
           tgt[c][j] = (unsigned)m < (unsigned)HW ? (int)pl * HW + m : -1;
@@ -429,15 +452,15 @@ __global__ __launch_bounds__(256) void pool_bwd_mask_color_kernel(PoolDims d, Po
 }
 
 // Launches one instantiation of the LDS forward; RH_E_UNSUPPORTED when the block's LDS cannot be had.
-template <int K, int ST>
+template <int K, int ST, class MT>
 static int launch_pool_fwd_lds(const PoolDims& d, FastDiv dPQ, int PB, long long planes, long long blocks, size_t lds_bytes,
-                               int bands, int rb, const float* x, float* y, int32_t* argmax, rh_stream_t stream) {
+                               int bands, int rb, const float* x, float* y, MT* argmax, rh_stream_t stream) {
   if (lds_bytes > 48 * 1024) {
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_fwd_lds_kernel<K, ST>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_fwd_lds_kernel<K, ST, MT>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
     if (attr != hipSuccess) return RH_E_UNSUPPORTED;
   }
-  hipLaunchKernelGGL((pool_fwd_lds_kernel<K, ST>), dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d, dPQ, PB,
+  hipLaunchKernelGGL((pool_fwd_lds_kernel<K, ST, MT>), dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d, dPQ, PB,
                      planes, bands, rb, FastDiv((uint32_t)bands), x, y, argmax);
   return launch_status();
 }
@@ -458,6 +481,7 @@ static int pool_dims(const rh_pool_geom* g, PoolDims* d) {
   d->dH = FastDiv((uint32_t)d->H);
   d->dW = FastDiv((uint32_t)d->W);
   d->dSt = FastDiv((uint32_t)d->st);
+  d->dK = FastDiv((uint32_t)d->k);
   return 0;
 }
 
@@ -470,6 +494,37 @@ extern "C" int32_t rh_pool2d_out_dim(int32_t in, int32_t size, int32_t stride, i
   return pool_out_dim(in, size, stride, pad, round);
 }
 
+// The LDS forward: about 16 KB of input per block (measured best: more LDS per block leaves too few blocks per CU to
+// overlap one block's loads with another's window scans): several small planes, one plane, or a band of a larger
+// plane's output rows with the input rows its windows reach.  RH_E_UNSUPPORTED: the geometry is outside this form.
+template <class MT>
+static int pool_fwd_lds(const PoolDims& d, const float* x, float* y, MT* mask, rh_stream_t stream, bool dry_run = false) {
+  constexpr int kLdsFloats = 4096;
+  if (!(d.P * d.Q > 0 && (long long)d.W * d.k <= 15000)) return RH_E_UNSUPPORTED;
+  const int HW = d.H * d.W;
+  const long long planes = (long long)d.N * d.C;
+  int PB = 1, bands = 1, rb = d.P, rows_in = d.H;
+  if (HW <= kLdsFloats) {
+    PB = kLdsFloats / HW;
+    if (PB > 64) PB = 64;
+  } else {
+    const int rows_fit = kLdsFloats / d.W;  // input rows in the block's share (at least one window's)
+    rb = rows_fit > d.k ? (rows_fit - d.k) / d.st + 1 : 1;
+    if (rb > d.P) rb = d.P;
+    bands = cdiv(d.P, rb);
+    rows_in = (rb - 1) * d.st + d.k < d.H ? (rb - 1) * d.st + d.k : d.H;
+  }
+  const long long blocks = bands > 1 ? planes * bands : cdiv<long long>(planes, PB);
+  const size_t lds_bytes = ((size_t)(bands > 1 ? rows_in * d.W : PB * HW) + 4) * sizeof(float);
+  if (!(blocks < (1ll << 31) && (long long)PB * d.P * d.Q < (1ll << 31)) || lds_bytes > 64 * 1024) return RH_E_UNSUPPORTED;
+  if (dry_run) return 0;
+  const FastDiv dPQ((uint32_t)(d.P * d.Q));
+  if (d.k == 3 && d.st == 2) return launch_pool_fwd_lds<3, 2, MT>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, mask, stream);
+  if (d.k == 2 && d.st == 2) return launch_pool_fwd_lds<2, 2, MT>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, mask, stream);
+  if (d.k == 3 && d.st == 1) return launch_pool_fwd_lds<3, 1, MT>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, mask, stream);
+  return launch_pool_fwd_lds<0, 0, MT>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, mask, stream);
+}
+
 extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, int32_t* opt_argmax,
                              rh_stream_t stream) {
   PoolDims d;
@@ -477,38 +532,13 @@ extern "C" int rh_pool2d_fwd(const rh_pool_geom* g, const float* x, float* y, in
   if (!x || !y) return RH_E_INVALID;
   const long long total = (long long)d.N * d.C * d.P * d.Q;
   if (total == 0) return 0;
+  // algorithmic bytes: x read, y written (and the arg-max mask where the caller asks for one)
   ProfScope prof(d.mode == RH_POOL_MAX ? "pool_max_fwd" : "pool_avg_fwd",
                  4.0 * ((double)d.N * d.C * d.H * d.W + (double)total * (opt_argmax ? 2 : 1)), to_stream(stream));
   const long long in_total = (long long)d.N * d.C * d.H * d.W;
-  // about 16 KB of input per block (measured best: more LDS per block leaves too few blocks per CU to overlap one
-  // block's loads with another's window scans): several small planes, one plane, or a band of a larger plane's
-  // output rows with the input rows its windows reach
-  constexpr int kLdsFloats = 4096;
-  if (d.P * d.Q > 0 && (long long)d.W * d.k <= 15000) {
-    const int HW = d.H * d.W;
-    const long long planes = (long long)d.N * d.C;
-    int PB = 1, bands = 1, rb = d.P, rows_in = d.H;
-    if (HW <= kLdsFloats) {
-      PB = kLdsFloats / HW;
-      if (PB > 64) PB = 64;
-    } else {
-      const int rows_fit = kLdsFloats / d.W;  // input rows in the block's share (at least one window's)
-      rb = rows_fit > d.k ? (rows_fit - d.k) / d.st + 1 : 1;
-      if (rb > d.P) rb = d.P;
-      bands = cdiv(d.P, rb);
-      rows_in = (rb - 1) * d.st + d.k < d.H ? (rb - 1) * d.st + d.k : d.H;
-    }
-    const long long blocks = bands > 1 ? planes * bands : cdiv<long long>(planes, PB);
-    const size_t lds_bytes = ((size_t)(bands > 1 ? rows_in * d.W : PB * HW) + 4) * sizeof(float);
-    if (blocks < (1ll << 31) && (long long)PB * d.P * d.Q < (1ll << 31)) {
-      const FastDiv dPQ((uint32_t)(d.P * d.Q));
-      int e;
-      if (d.k == 3 && d.st == 2)      e = launch_pool_fwd_lds<3, 2>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, opt_argmax, stream);
-      else if (d.k == 2 && d.st == 2) e = launch_pool_fwd_lds<2, 2>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, opt_argmax, stream);
-      else if (d.k == 3 && d.st == 1) e = launch_pool_fwd_lds<3, 1>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, opt_argmax, stream);
-      else                            e = launch_pool_fwd_lds<0, 0>(d, dPQ, PB, planes, blocks, lds_bytes, bands, rb, x, y, opt_argmax, stream);
-      if (e != RH_E_UNSUPPORTED) return e;
-    }
+  {
+    const int e = pool_fwd_lds<int>(d, x, y, opt_argmax, stream);
+    if (e != RH_E_UNSUPPORTED) return e;
   }
   const dim3 grid((unsigned)cdiv<long long>(total, 256) > (1u << 20) ? (1u << 20) : (unsigned)cdiv<long long>(total, 256));
   if (total < (1ll << 31) && in_total < (1ll << 31))
@@ -541,22 +571,23 @@ static bool lds_bwd_ok(const PoolDims& d) { return d.P * d.Q <= 4096 && d.H * d.
 
 // The colour form: one or two colours per axis, a plane's dx within 60 KB of LDS, at most 8 windows per thread and
 // colour.  Returns RH_E_UNSUPPORTED when the geometry is outside that.
-template <int J>
+template <int J, class MT>
 static int launch_pool_bwd_color_j(const PoolDims& d, const PoolColors& pc, int PB, long long planes, long long blocks,
-                                   size_t lds_bytes, const float* dy, const int32_t* argmax, const float* relu_y, float* dx,
+                                   size_t lds_bytes, const float* dy, const MT* argmax, const float* relu_y, float* dx,
                                    rh_stream_t stream) {
   if (lds_bytes > 48 * 1024) {
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_bwd_mask_color_kernel<J>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&pool_bwd_mask_color_kernel<J, MT>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
     if (attr != hipSuccess) return RH_E_UNSUPPORTED;
   }
-  hipLaunchKernelGGL((pool_bwd_mask_color_kernel<J>), dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d, pc, PB,
+  hipLaunchKernelGGL((pool_bwd_mask_color_kernel<J, MT>), dim3((unsigned)blocks), dim3(256), lds_bytes, to_stream(stream), d, pc, PB,
                      planes, dy, argmax, relu_y, dx);
   return launch_status();
 }
 
-static int launch_pool_bwd_color(const PoolDims& d, const float* dy, const int32_t* argmax, const float* relu_y, float* dx,
-                                 rh_stream_t stream) {
+template <class MT>
+static int launch_pool_bwd_color(const PoolDims& d, const float* dy, const MT* argmax, const float* relu_y, float* dx,
+                                 rh_stream_t stream, bool dry_run = false) {
   const int nA = cdiv(d.k, d.st);
   const int HW = d.H * d.W;
   if (nA > 2 || HW > 15000 || d.P * d.Q <= 0) return RH_E_UNSUPPORTED;
@@ -590,16 +621,17 @@ static int launch_pool_bwd_color(const PoolDims& d, const float* dy, const int32
   const long long blocks = cdiv<long long>(planes, PB);
   if (blocks >= (1ll << 31)) return RH_E_LIMIT;
   const size_t lds_bytes = ((size_t)PB * HW + 8) * sizeof(float);
-  if (per_thread <= 1) return launch_pool_bwd_color_j<1>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
-  if (per_thread <= 2) return launch_pool_bwd_color_j<2>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
-  if (per_thread <= 4) return launch_pool_bwd_color_j<4>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
-  return launch_pool_bwd_color_j<8>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
+  if (dry_run) return 0;
+  if (per_thread <= 1) return launch_pool_bwd_color_j<1, MT>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
+  if (per_thread <= 2) return launch_pool_bwd_color_j<2, MT>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
+  if (per_thread <= 4) return launch_pool_bwd_color_j<4, MT>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
+  return launch_pool_bwd_color_j<8, MT>(d, pc, PB, planes, blocks, lds_bytes, dy, argmax, relu_y, dx, stream);
 }
 
 static int launch_pool_bwd_lds(const PoolDims& d, const float* dy, const int32_t* argmax, const float* relu_y, float* dx,
                                rh_stream_t stream) {
   {
-    const int e = launch_pool_bwd_color(d, dy, argmax, relu_y, dx, stream);
+    const int e = launch_pool_bwd_color<int>(d, dy, argmax, relu_y, dx, stream);
     if (e != RH_E_UNSUPPORTED) return e;
   }
   const int PQ = d.P * d.Q;
@@ -630,6 +662,41 @@ extern "C" int rh_pool2d_bwd_relu(const rh_pool_geom* g, const float* y, const f
   if (in_elems == 0) return 0;
   ProfScope prof("pool_max_bwd_relu", 4.0 * (in_elems + 3.0 * out_elems), to_stream(stream));
   return launch_pool_bwd_lds(d, dy, argmax, y, dx, stream);
+}
+
+// The one-byte mask: max pooling with size <= 15 on the geometries that both the LDS forward and the colour backward take.
+extern "C" int rh_pool2d_slot_supported(const rh_pool_geom* g) {
+  PoolDims d;
+  if (pool_dims(g, &d)) return 0;
+  if (d.mode != RH_POOL_MAX || d.k > 15 || !lds_bwd_ok(d) || (long long)d.N * d.C >= (1ll << 31)) return 0;
+  return pool_fwd_lds<uint8_t>(d, nullptr, nullptr, nullptr, nullptr, true) == 0 &&
+         launch_pool_bwd_color<uint8_t>(d, nullptr, nullptr, nullptr, nullptr, nullptr, true) == 0 ? 1 : 0;
+}
+
+extern "C" int rh_pool2d_fwd_slot(const rh_pool_geom* g, const float* x, float* y, uint8_t* slot, rh_stream_t stream) {
+  PoolDims d;
+  if (int e = pool_dims(g, &d)) return e;
+  if (!x || !y || !slot) return RH_E_INVALID;
+  if (!rh_pool2d_slot_supported(g)) return RH_E_UNSUPPORTED;
+  const double in_elems = (double)d.N * d.C * d.H * d.W, out_elems = (double)d.N * d.C * d.P * d.Q;
+  if (out_elems == 0) return 0;
+  // algorithmic bytes: x read, y written; the mask's byte per output is the operator's own bookkeeping and not counted
+  ProfScope prof("pool_max_fwd", 4.0 * (in_elems + out_elems), to_stream(stream));
+  return pool_fwd_lds<uint8_t>(d, x, y, slot, stream);
+}
+
+extern "C" int rh_pool2d_bwd_slot(const rh_pool_geom* g, const float* relu_y, const float* dy, float* dx, const uint8_t* slot,
+                                  rh_stream_t stream) {
+  PoolDims d;
+  if (int e = pool_dims(g, &d)) return e;
+  if (!dy || !dx || !slot) return RH_E_INVALID;
+  if (!rh_pool2d_slot_supported(g)) return RH_E_UNSUPPORTED;
+  const double in_elems = (double)d.N * d.C * d.H * d.W, out_elems = (double)d.N * d.C * d.P * d.Q;
+  if (in_elems == 0) return 0;
+  // algorithmic bytes: dy read, dx written, and y read where the ReLU mask of the operator below is folded in
+  ProfScope prof(relu_y ? "pool_max_bwd_relu" : "pool_max_bwd", 4.0 * (in_elems + (relu_y ? 2.0 : 1.0) * out_elems),
+                 to_stream(stream));
+  return launch_pool_bwd_color<uint8_t>(d, dy, slot, relu_y, dx, stream);
 }
 
 extern "C" int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float* y, const float* dy, float* dx,

@@ -191,6 +191,27 @@ def pool2d_fwd(x, size, stride, pad, mode, rounding=_lib.RH_ROUND_FLOOR, want_ar
     return (y, am) if want_argmax else y
 
 
+def pool2d_slot_supported(x_shape, size, stride, pad, rounding=_lib.RH_ROUND_FLOOR):
+    g = pool_geom(x_shape, size, stride, pad, _lib.RH_POOL_MAX, rounding)
+    return bool(lib().rh_pool2d_slot_supported(C.byref(g)))
+
+
+def pool2d_fwd_slot(x, size, stride, pad, rounding=_lib.RH_ROUND_FLOOR):
+    """Max pooling with the one-byte mask: returns (y, slot) with slot = r*size + s of each window's winner (255: none)."""
+    g = pool_geom(x.shape, size, stride, pad, _lib.RH_POOL_MAX, rounding)
+    y = torch.empty(pool_out_shape(g), dtype=torch.float32, device=x.device)
+    slot = torch.empty(y.shape, dtype=torch.uint8, device=x.device)
+    check(lib().rh_pool2d_fwd_slot(C.byref(g), _p(x), _p(y), _p(slot), _stream()), "rh_pool2d_fwd_slot")
+    return y, slot
+
+
+def pool2d_bwd_slot(x_shape, dy, slot, size, stride, pad, rounding=_lib.RH_ROUND_FLOOR, relu_y=None):
+    g = pool_geom(x_shape, size, stride, pad, _lib.RH_POOL_MAX, rounding)
+    dx = torch.empty(tuple(x_shape), dtype=torch.float32, device=dy.device)
+    check(lib().rh_pool2d_bwd_slot(C.byref(g), _p(relu_y), _p(dy), _p(dx), _p(slot), _stream()), "rh_pool2d_bwd_slot")
+    return dx
+
+
 def bf16_pack(x, halo):
     """fp32 NCHW -> packed bf16 activation tensor [n][H + 2 halo][C/8][W + 2 halo][8] (a uint8 tensor; zero border)."""
     Nn, Cc, H, W = x.shape
@@ -208,7 +229,7 @@ def bf16_unpack(xp, shape, halo):
     return x
 
 
-def conv2d_fwd_bf16_packed(x, w, stride, pad, bias=None, relu=False, x_packed=None, out_halo=None):
+def conv2d_fwd_bf16_packed(x, w, stride, pad, bias=None, relu=False, x_packed=None, out_halo=None, algo=0):
     """The bf16 forward on a converted filter.  Input: `x_packed` (from bf16_pack(x, pad) or a producer) or the fp32 `x`
     (x.shape is used for the geometry either way).  out_halo None: fp32 NCHW result; an int: packed bf16 result with
     that border.  Returns the result tensor."""
@@ -226,7 +247,7 @@ def conv2d_fwd_bf16_packed(x, w, stride, pad, bias=None, relu=False, x_packed=No
         nbytes = lib().rh_bf16_act_bytes(shape[0], shape[1], shape[2], shape[3], out_halo)
         assert nbytes > 0
         yp = torch.zeros(nbytes, dtype=torch.uint8, device=w.device)
-    flags = (_lib.RH_FUSE_BIAS if bias is not None else 0) | (_lib.RH_FUSE_RELU if relu else 0)
+    flags = (_lib.RH_FUSE_BIAS if bias is not None else 0) | (_lib.RH_FUSE_RELU if relu else 0) | algo
     check(lib().rh_conv2d_fwd_bf16_packed(C.byref(g), _p(x_packed), _p(None if x_packed is not None else x), _p(wprep), _p(bias),
                                           _p(y), _p(yp), 0 if out_halo is None else out_halo, _p(ws), ws.numel(), flags,
                                           _stream()), "rh_conv2d_fwd_bf16_packed")

@@ -136,6 +136,12 @@ extern "C" {
   pub fn rh_pool2d_bwd(g: *const rh_pool_geom, x: *const f32, y: *const f32, dy: *const f32, dx: *mut f32,
                        opt_argmax: *const i32, stream: rh_stream_t) -> c_int;
 
+  // Max pooling with a one-byte mask (the winner's slot inside its window) for an operator's private use.
+  pub fn rh_pool2d_slot_supported(g: *const rh_pool_geom) -> c_int;
+  pub fn rh_pool2d_fwd_slot(g: *const rh_pool_geom, x: *const f32, y: *mut f32, slot: *mut u8, stream: rh_stream_t) -> c_int;
+  pub fn rh_pool2d_bwd_slot(g: *const rh_pool_geom, relu_y: *const f32, dy: *const f32, dx: *mut f32, slot: *const u8,
+                            stream: rh_stream_t) -> c_int;
+
   pub fn rh_softmax_fwd(x: *const f32, p: *mut f32, c: i32, n: i32, stream: rh_stream_t) -> c_int;
   // Same names and argument lists as rembrandt_kernels::ffi (src/operator/loss.rs:132-140, 191-210, 229-239).
   pub fn rembrandt_kernel_batch_map_softmax_kl_backward(p: *const f32, c: i32, n: i32, labels: *const i32,

@@ -1,4 +1,6 @@
 """GPU parity: every C-ABI kernel against the CPU oracle on the same seeded inputs (small shapes)."""
+import ctypes as C_
+
 import numpy as np
 import pytest
 import torch
@@ -207,6 +209,8 @@ BF16_CHAIN_CASES = [
     (5, 32, 7, 5, 128, 1, 1, 0, 2),
     (2, 128, 13, 11, 32, 1, 1, 0, 1),
     (7, 64, 3, 3, 64, 1, 1, 0, 0),
+    (3, 256, 9, 10, 256, 1, 1, 0, 1),     # two chunks of 128 output channels, the deep contraction
+    (2, 256, 5, 5, 192, 1, 1, 0, 0),      # two chunks of 96
 ]
 
 
@@ -237,6 +241,10 @@ def test_conv2d_fwd_bf16_packed_chain_forms(dev, case):
             assert torch.equal(y2, legacy), "packed image in, fp32 result"
             yp2 = ops.conv2d_fwd_bf16_packed(xd, wd, st, pad, bias=bd, relu=relu, x_packed=xp, out_halo=halo)
             assert torch.equal(yp2, yp), "packed image in, packed result"
+            # (the streaming 1x1 kernel wherever it can run, also where the tiled kernel is the one chosen)
+            yp3 = ops.conv2d_fwd_bf16_packed(xd, wd, st, pad, bias=bd, relu=relu, x_packed=xp, out_halo=halo,
+                                             algo=_lib.RH_ALGO_SCALAR_OFFSET)
+            assert torch.equal(yp3, yp), "packed image in, packed result, streaming kernel where it runs"
     torch.cuda.synchronize()
 
 
@@ -401,6 +409,40 @@ def test_pool2d(dev, case, mode, rounding):
         assert np.allclose(N(dx2), N(dx), rtol=1e-6, atol=2e-6), "mask-driven backward equals recomputed"
         again = ops.pool2d_bwd(xd, y, T(dy, dev), k, st, pad, mode, rounding, argmax=am)
         assert np.array_equal(N(dx2), N(again)), "the mask-driven backward is deterministic"
+
+
+@pytest.mark.parametrize("case", POOL_CASES + [(2, 3, 55, 3, 2, 0), (3, 2, 31, 5, 4, 2)], ids=str)
+@pytest.mark.parametrize("rounding", [_lib.RH_ROUND_FLOOR, _lib.RH_ROUND_CEIL])
+def test_pool2d_one_byte_mask(dev, case, rounding):
+    """The one-byte mask (the winner's slot r*size + s inside its window, 255 for none) names the same elements as the
+    int32 plane index, bit for bit; the pooled values are identical; the backward pass from it, without and with the ReLU
+    mask of the operator below folded in, is bit-identical to the one from the int32 mask."""
+    Nn, C, H, k, st, pad = case
+    shape = (Nn, C, H, H + 1)
+    say("pool one-byte mask case", case, rounding)
+    if not ops.pool2d_slot_supported(shape, k, st, pad, rounding):
+        g = ops.pool_geom(shape, k, st, pad, _lib.RH_POOL_MAX, rounding)
+        dummy = torch.zeros(16, device=dev)
+        assert _lib.lib().rh_pool2d_fwd_slot(C_.byref(g), dummy.data_ptr(), dummy.data_ptr(), dummy.data_ptr(), None) == _lib.RH_E_UNSUPPORTED
+        pytest.skip("no one-byte form for this geometry (three colours per axis or planes beyond the LDS kernels)")
+    x = np.round(synth.normal(17, 1, shape) * 2) / 2 - np.float32(0.5)     # ties, and windows that are all negative
+    xd = T(x, dev)
+    y, am = ops.pool2d_fwd(xd, k, st, pad, _lib.RH_POOL_MAX, rounding, want_argmax=True)
+    y2, slot = ops.pool2d_fwd_slot(xd, k, st, pad, rounding)
+    assert torch.equal(y, y2)
+    am_h, slot_h = N(am), N(slot).astype(np.int64)
+    P, Q = am_h.shape[2], am_h.shape[3]
+    hs = (np.arange(P) * st - pad)[:, None]
+    ws = (np.arange(Q) * st - pad)[None, :]
+    plane = (hs + slot_h // k) * shape[3] + ws + slot_h % k
+    assert np.array_equal(np.where(slot_h == 255, -1, plane), am_h), "slot names the element the plane index names"
+    assert (slot_h[slot_h != 255] < k * k).all()
+    dy = T(synth.normal(17, 2, tuple(y.shape)), dev)
+    assert torch.equal(ops.pool2d_bwd_slot(shape, dy, slot, k, st, pad, rounding),
+                       ops.pool2d_bwd(xd, y, dy, k, st, pad, _lib.RH_POOL_MAX, rounding, argmax=am))
+    assert torch.equal(ops.pool2d_bwd_slot(shape, dy, slot, k, st, pad, rounding, relu_y=y),
+                       ops.pool2d_bwd_relu(shape, y, dy, k, st, pad, am, rounding))
+    torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("shape", [(64, 10), (256, 1000), (7, 1), (3, 5000)])
