@@ -494,6 +494,271 @@ __global__ __launch_bounds__(256, (wide_blocks_per_cu<TM, KH, W>())) void conv1x
   for (; g < last; g += nwaves) compute_group(b0, g, g + nwaves, nv, nstep);
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// The same layer with every global access 16 bytes wide, no wave ever waiting for a store, the epilogue of one tile
+// issued in the shadow of the next tile's MFMAs, and two tiles of loads in flight per wave: the image's way through
+// LDS, the filter in registers.  (Dword accesses top out near 3.8 TB/s on this GPU whatever is done around them; a wave
+// that waits for loads behind its own fresh stores sits out their acknowledgements, since the memory counter retires
+// in order; an epilogue that a wave runs between two tiles costs it 1.8 us per tile, a fifth of the tile's matrix
+// time; and with one tile of loads in flight per wave, 48 KB per CU, the memory system delivers 3.5 TB/s.)
+// One block of four waves per CU, one per SIMD, each wave on column tiles of its own with private LDS: three source
+// buffers of 32 pixels by the contraction and a 4 KB result buffer (160 KB per CU for a contraction of 96).
+//   * The filter is staged through LDS once (before the buffers are in use) into registers: a lane holds its
+//     A(32 i + lane % 32, 2 s + lane / 32) for every row tile i and channel pair s, TM * KH values.
+//   * A tile of the source arrives by direct global -> LDS loads (buffer_load_dwordx4 ... lds: eight channel rows of
+//     32 pixels per instruction, no registers), requested two tiles ahead: loads(j+2) go out at the top of tile j,
+//     into the buffer tile j-1 was multiplied from.
+//   * The MFMAs read the image operand from LDS, one conflict-free ds_read_b32 per channel pair.
+//   * Two sets of accumulators: while tile j is multiplied into one, the other (tile j-1) is drained, one element per
+//     K step (bias, ReLU, into the result buffer as Y[row][32 pixels]); after each row tile of 32 rows the buffer is read
+//     back as eight rows of 128 bytes per instruction and stored with 16 bytes per lane.
+// Memory instructions of a wave in program order: loads(j+2), then the stores of tile j-1 spread over tile j; the wait
+// for loads(j) at the top of tile j allows the two younger tiles' loads and the two younger tiles' stores to be in flight.
+// Column tiles are cut per image (the last one of an image is ragged), so a tile never straddles two images.  No
+// block-wide barrier once the filter is in registers.
+// ------------------------------------------------------------------------------------------------------------------
+template <int TM, int KH>
+constexpr size_t lds_kernel_bytes() {
+  const size_t bufs = sizeof(float) * 4 * (3 * 32 * (size_t)(2 * KH) + 1024);
+  const size_t stage = sizeof(float) * ((size_t)TM * KH * 64 + 32 * TM);
+  return bufs > stage ? bufs : stage;
+}
+template <int TM, int KH>
+constexpr bool lds_kernel_fits() {
+  return KH % 4 == 0 && KH >= 16 * TM && TM * KH <= 160 && lds_kernel_bytes<TM, KH>() <= 160 * 1024;
+}
+
+template <int TM, int KH, bool RELU, class PASS>
+__global__ __launch_bounds__(256, 1) void conv1x1_lds_kernel(Conv1x1Params p, EpiParams ep, FastDiv dTpi) {
+  constexpr int KD = 2 * KH, ROWS = 32 * TM;
+  constexpr int XBUF = 32 * KD;               // floats per source buffer
+  constexpr int LD = KD / 8, ST = ROWS / 8;   // load / store instructions per tile
+  static_assert(KH >= 16 * TM, "one K step per drained accumulator element");
+  static_assert(2 * LD + 2 * ST <= 63, "the memory counter counts to 63");
+  const int lane = threadIdx.x & 63;
+  const int wib = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const bool by_xcd = (gridDim.x & 7) == 0;   // (see conv1x1_stream_kernel: an XCD sweeps its eighth in address order)
+  const int nwaves = by_xcd ? (int)(gridDim.x >> 3) * 4 : (int)gridDim.x * 4;
+  const int wave = __builtin_amdgcn_readfirstlane((int)((by_xcd ? blockIdx.x >> 3 : blockIdx.x) * 4) + wib);
+  const int span = by_xcd ? (p.tiles + 7) >> 3 : p.tiles;
+  const int first = by_xcd ? (int)(blockIdx.x & 7) * span : 0;
+  const int last = min(first + span, p.tiles);
+  const int half = lane >> 5, l32 = lane & 31;
+
+  extern __shared__ float sa[];
+  // filter and bias: through LDS into registers, in accumulator / operand order, for the life of the wave
+  float areg[KH][TM], breg[16 * TM];
+  {
+    float* const sbias = sa + TM * KH * 64;
+    stage_filter<TM, KH>(p, sa);
+    if (threadIdx.x < ROWS) sbias[threadIdx.x] = ep.bias ? ep.bias[threadIdx.x] : 0.0f;
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < KH; ++s)
+#pragma unroll
+      for (int i = 0; i < TM; ++i) areg[s][i] = sa[(s * TM + i) * 64 + lane];
+#pragma unroll
+    for (int u = 0; u < 16 * TM; ++u) breg[u] = sbias[32 * (u >> 4) + 8 * ((u & 15) >> 2) + 4 * half + (u & 3)];
+    __syncthreads();   // the staging area becomes the waves' buffers
+  }
+  float* const xbuf = sa + wib * (3 * XBUF + 1024);   // this wave's three source buffers ...
+  float* const ybuf = xbuf + 3 * XBUF;                // ... and its result buffer (32 rows x 32 pixels)
+
+  const int PQ4 = p.PQ * 4;
+  const uint32_t img_bytes = (uint32_t)p.kdim * (uint32_t)PQ4;
+  const uint32_t out_img_bytes = (uint32_t)p.rows * (uint32_t)PQ4;
+  u32x4 rsrc;
+  {
+    const uint64_t a = reinterpret_cast<uint64_t>(p.src);
+    rsrc.x = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    rsrc.y = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+    rsrc.z = __builtin_amdgcn_readfirstlane(p.src_bytes);
+    rsrc.w = 0x00020000u;
+  }
+  const __amdgpu_buffer_rsrc_t rdst = make_rsrc(ep.out, (uint32_t)(sizeof(float) * (size_t)p.cols * p.rows));
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)xbuf;
+  const int row8 = lane >> 3, px4 = (lane & 7) * 4;   // this lane's place in a 16-byte access: row within eight, first pixel
+
+  // tile -> image and first pixel (wave-uniform)
+  auto where = [&](int t, uint32_t& img, uint32_t& pix0) __attribute__((always_inline)) {
+    uint32_t ti;
+    dTpi.divmod((uint32_t)t, img, ti);
+    pix0 = ti * 32u;
+  };
+  auto issue_loads = [&](int t, int buf) __attribute__((always_inline)) {
+    uint32_t img, pix0;
+    where(t, img, pix0);
+    const uint32_t px = pix0 + (uint32_t)px4;
+    const uint32_t voff = px < (uint32_t)p.PQ ? img * img_bytes + (uint32_t)(row8 * PQ4) + px * 4u : 0x80000000u;
+    const uint32_t dst = lds0 + (uint32_t)(buf * XBUF * 4);
+#pragma unroll
+    for (int g = 0; g < LD; ++g) dma_load16(rsrc, dst + (uint32_t)(g * 1024), voff, (uint32_t)(g * 8 * PQ4));
+  };
+  // the memory counter may stand at `loads` tiles of loads plus `stores` tiles of stores (each 0, 1 or 2)
+  auto wait_for_tile = [&](int loads, int stores) __attribute__((always_inline)) {
+    switch (loads * 3 + stores) {
+      case 0: wait_vmcnt<0>(); break;
+      case 1: wait_vmcnt<ST>(); break;
+      case 2: wait_vmcnt<2 * ST>(); break;
+      case 3: wait_vmcnt<LD>(); break;
+      case 4: wait_vmcnt<LD + ST>(); break;
+      case 5: wait_vmcnt<LD + 2 * ST>(); break;
+      case 6: wait_vmcnt<2 * LD>(); break;
+      case 7: wait_vmcnt<2 * LD + ST>(); break;
+      default: wait_vmcnt<2 * LD + 2 * ST>(); break;
+    }
+  };
+  typedef const __attribute__((address_space(3))) float* lds_ptr;
+
+  // Where a drained tile's rows go (per lane: the 16-byte access of row 8 r + row8) and the stores of one row tile.
+  struct Dest { uint32_t o0, ow; int nvalid; };
+  auto dest_of = [&](int t) __attribute__((always_inline)) -> Dest {
+    uint32_t img, pix0;
+    where(t, img, pix0);
+    const uint32_t px = pix0 + (uint32_t)px4;
+    Dest d;
+    d.o0 = img * out_img_bytes + (uint32_t)(row8 * PQ4) + px * 4u;
+    d.ow = px + 3u < (uint32_t)p.PQ ? d.o0 : 0x80000000u;   // lanes whose four pixels lie inside the image
+    d.nvalid = px < (uint32_t)p.PQ && px + 3u >= (uint32_t)p.PQ ? p.PQ - (int)px : 0;   // the image's ragged end
+    return d;
+  };
+  // Row tile i of a drained tile is complete in the result buffer (32 rows x 128 bytes): read_rows fetches it, four
+  // instructions of eight rows, and store_rows, a K step later, stores it the same way.
+  auto read_rows = [&](float4 (&yv)[4]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) yv[r] = *reinterpret_cast<const float4*>(ybuf + (8 * r + row8) * 32 + px4);
+  };
+  auto store_rows = [&](const Dest& d, const float4 (&yv)[4], int i) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      u32x4 q;
+      q[0] = __float_as_uint(yv[r].x); q[1] = __float_as_uint(yv[r].y); q[2] = __float_as_uint(yv[r].z); q[3] = __float_as_uint(yv[r].w);
+      __builtin_amdgcn_raw_buffer_store_b128(q, rdst, (int)d.ow, (4 * i + r) * 8 * PQ4, 0);
+    }
+    if (d.nvalid) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float vals[4] = {yv[r].x, yv[r].y, yv[r].z, yv[r].w};
+#pragma unroll
+        for (int e = 0; e < 3; ++e)
+          if (e < d.nvalid)
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(vals[e]), rdst, (int)(d.o0 + 4u * e), (4 * i + r) * 8 * PQ4, 0);
+      }
+    }
+  };
+  // element u (0 .. 16 TM - 1) of a drained accumulator set: row 32 i + 8 q + 4 half + e of this lane's pixel
+  auto drain_one = [&](const f32x16 (&acc)[TM], int u) __attribute__((always_inline)) {
+    const int i = u >> 4, v = u & 15;
+    float val = acc[i][v] + breg[u];   // added after the sum, as the reference's bias pass
+    if (RELU) val = val > 0.0f ? val : 0.0f;
+    ybuf[(8 * (v >> 2) + 4 * half + (v & 3)) * 32 + l32] = val;
+  };
+  auto drain_all = [&](const f32x16 (&acc)[TM], const Dest& d) __attribute__((always_inline)) {
+    float4 yv[4];
+#pragma unroll
+    for (int u = 0; u < 16 * TM; ++u) {
+      drain_one(acc, u);
+      if ((u & 15) == 15) { read_rows(yv); store_rows(d, yv, u >> 4); }
+    }
+  };
+
+  // One tile: the contraction from source buffer `cur` into `acc`; with DRAIN, the tile before (accumulators `old`,
+  // destination `od`) leaves through the result buffer meanwhile, one element per K step.
+  auto tile = [&](f32x16 (&acc)[TM], const f32x16 (&old)[TM], const Dest& od, int cur, auto drain_tag, int next_t, int next_buf) __attribute__((always_inline)) {
+    constexpr bool DRAIN = decltype(drain_tag)::value;
+    // the loads of the tile after next, one instruction per K step (next_t < 0: none)
+    uint32_t nvoff = 0x80000000u, ndst = 0;
+    if (next_t >= 0) {
+      uint32_t img, pix0;
+      where(next_t, img, pix0);
+      const uint32_t px = pix0 + (uint32_t)px4;
+      nvoff = px < (uint32_t)p.PQ ? img * img_bytes + (uint32_t)(row8 * PQ4) + px * 4u : 0x80000000u;
+      ndst = lds0 + (uint32_t)(next_buf * XBUF * 4);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
+    lds_ptr bl = (lds_ptr)(xbuf + cur * XBUF + half * 32 + l32);
+    asm volatile("" : "+v"(bl));
+    float bv[2];
+    float4 yv[4];
+    bv[0] = bl[0];
+#pragma unroll
+    for (int s = 0; s < KH; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (DRAIN) {
+        // the row tile read back in the step before leaves (its reads were issued ahead of that step's operand read,
+        // which this step's MFMAs waited for)
+        if (s > 0 && (s & 15) == 0 && s <= 16 * TM) store_rows(od, yv, (s >> 4) - 1);
+      }
+      if (s + 1 < KH) bv[(s + 1) & 1] = bl[(s + 1) * 64];
+      if (s < LD && next_t >= 0) dma_load16(rsrc, ndst + (uint32_t)(s * 1024), nvoff, (uint32_t)(s * 8 * PQ4));
+      if (DRAIN) {
+        if (s < 16 * TM) drain_one(old, s);
+        if (s < 16 * TM && (s & 15) == 15) read_rows(yv);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s][i], bv[s & 1], acc[i], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (DRAIN && KH == 16 * TM) store_rows(od, yv, TM - 1);
+  };
+
+  int t = first + wave;
+  if (t >= last) return;
+  // tile j of this wave: t + j * nwaves, in source buffer j % 3; loads two tiles ahead
+  const int n = (last - t + nwaves - 1) / nwaves;
+  f32x16 accA[TM], accB[TM];
+  Dest dA, dB = {0x80000000u, 0x80000000u, 0};
+  issue_loads(t, 0);
+  if (n > 1) issue_loads(t + nwaves, 1);
+  int cur = 0;
+  for (int j = 0; j < n; j += 2) {
+    // even tile into A while B (tile j-1) drains
+    {
+      wait_for_tile((j + 1 < n), j >= 3 ? 2 : j >= 2 ? 1 : 0);
+      dA = dest_of(t + j * nwaves);
+      const int nt = j + 2 < n ? t + (j + 2) * nwaves : -1, nb = cur == 0 ? 2 : cur - 1;
+      if (j == 0) tile(accA, accB, dB, cur, std::false_type(), nt, nb);
+      else        tile(accA, accB, dB, cur, std::true_type(), nt, nb);
+      cur = cur == 2 ? 0 : cur + 1;
+    }
+    if (j + 1 >= n) {   // the even tile was the last one
+      drain_all(accA, dA);
+      return;
+    }
+    // odd tile into B while A drains
+    {
+      const int k = j + 1;
+      wait_for_tile((k + 1 < n), k >= 3 ? 2 : k >= 2 ? 1 : 0);
+      dB = dest_of(t + k * nwaves);
+      tile(accB, accA, dA, cur, std::true_type(), k + 2 < n ? t + (k + 2) * nwaves : -1, cur == 0 ? 2 : cur - 1);
+      cur = cur == 2 ? 0 : cur + 1;
+    }
+  }
+  drain_all(accB, dB);
+}
+
+template <int TM, int KH, class PASS>
+static int launch_lds_kernel(Conv1x1Params p, const EpiParams& ep, hipStream_t stream) {
+  constexpr size_t lds = lds_kernel_bytes<TM, KH>();
+  static const hipError_t a1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv1x1_lds_kernel<TM, KH, true, PASS>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  static const hipError_t a2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv1x1_lds_kernel<TM, KH, false, PASS>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (a1 != hipSuccess) return (int)a1;
+  if (a2 != hipSuccess) return (int)a2;
+  const int tpi = cdiv(p.PQ, 32);
+  p.tiles = (int)(p.cols / p.PQ) * tpi;   // per-image tiles
+  if (ep.relu)
+    hipLaunchKernelGGL((conv1x1_lds_kernel<TM, KH, true, PASS>), dim3(256u), dim3(256), lds, stream, p, ep, FastDiv((uint32_t)tpi));
+  else
+    hipLaunchKernelGGL((conv1x1_lds_kernel<TM, KH, false, PASS>), dim3(256u), dim3(256), lds, stream, p, ep, FastDiv((uint32_t)tpi));
+  return launch_status();
+}
+
 template <int TM, int KH, int W>
 constexpr bool wide_fits() { return TM * W <= 12 && 16 * TM * W + KH * W + 80 <= 512; }
 
@@ -538,6 +803,16 @@ static int launch_stream(const Conv1x1Params& p, const EpiParams& ep, hipStream_
   // 97 -> 88 with four, backward-data with the mask 132 -> 117 with two; on 128 -> 128, 28 x 28 the masked form
   // 86 -> 31).  Short ones lose there (32 -> 64 on 56 x 56: 27 -> 29-32 us: less matrix work per group of columns to
   // cover the epilogue of a wave that has its SIMD to itself or shares it with one other).
+  // Large layers without a mask: the image through LDS with 16-byte accesses on both sides (conv1x1_lds_kernel).
+  // Measured with the library's events on 96 -> 96 at batch 128: forward with bias and ReLU 101 -> 94 us on 54 x 54,
+  // 115 -> 104 us on 55 x 55 (no even pixel count: the register form falls back to dword accesses there); backward-data
+  // 97 -> 94 and 107 -> 103; 64 -> 64 on 56 x 56 at batch 256 forward 101 -> 91, backward-data 87 -> 90, which therefore
+  // stays with four pixels per lane where the pixel count is a multiple of four.
+  if constexpr (lds_kernel_fits<TM, KH>()) {
+    constexpr bool bwd = std::is_same<PASS, PassConvBwdData>::value;
+    if (fast && !ep.mask && p.cols / p.PQ * (long long)cdiv(p.PQ, 32) >= 4096 && !(bwd && KH < 48 && p.PQ % 4 == 0))
+      return launch_lds_kernel<TM, KH, PASS>(p, ep, stream);
+  }
   if constexpr (KH >= 48) {
     if (fast && p.PQ % 2 == 0) {
       constexpr bool bwd = std::is_same<PASS, PassConvBwdData>::value;

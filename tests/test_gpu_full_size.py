@@ -53,6 +53,11 @@ FULL_CONV = {
     "resnet_proj_128": (64, 64, 56, 56, 128, 1, 2, 0),
     # 784 tiles on 256 CUs: the last 16 tiles are cut into slices (as are the last 164 of alexnet_conv5's 676)
     "resnet_14_256_b256": (256, 256, 14, 14, 256, 3, 1, 1),
+    # large 1x1 layers of up to 128 channels: the image through LDS (two row tiles with a pixel count that is a multiple
+    # of four; one row tile with ragged image ends; different channel counts on the two sides)
+    "lds1x1_64_56x56": (48, 64, 56, 56, 64, 1, 1, 0),
+    "lds1x1_32_ragged": (80, 32, 40, 41, 32, 1, 1, 0),
+    "lds1x1_64_to_32": (96, 64, 37, 43, 32, 1, 1, 0),
 }
 
 
