@@ -182,7 +182,16 @@ int rho_worker_reset_loss(rho_worker* w, int32_t batch_size);
 int rho_worker_accumulate_loss(rho_worker* w, int32_t batch_size);
 int rho_worker_store_accumulated_loss(rho_worker* w, float* out);
 /* Device view of one buffer of hidden operator `hidden_idx` (-1: input operator's out_act,
- * hidden_count: the loss operator's probabilities).  Returns RHO_E_PANIC if there is no such buffer. */
+ * hidden_count: the loss operator's probabilities).  Returns RHO_E_PANIC if there is no such buffer.
+ * How long a pointer stays meaningful: the fused train step (rho_sgd_train_batch / rho_sgd_step with fused != 0) does
+ * not write the zeros that the reference's `reset` leaves in grad_weights / grad_bias (which = 4, 5); it remembers that
+ * they stand for zeros and its next backward pass overwrites them.  This call (and every other operator method that
+ * looks at the gradients) makes the zeros real first, so what it shows is the reference's state; a gradient pointer kept
+ * across a later fused step shows that step's gradients instead of zeros.  Ask again after each step, or use
+ * rho_worker_read_buffer.  Likewise a weights / bias pointer (which = 2, 3) may be written through until the next
+ * forward pass; a forward-only bf16 worker converts its filters when this call hands the pointer out, so write before
+ * the next forward pass, not during it.  In a forward-only bf16 worker out_act (which = 0) of the operators between
+ * convolutions holds the bf16 activations' values, unpacked when this call is made. */
 int rho_worker_buffer(rho_worker* w, int32_t hidden_idx, int which, float** dptr, int64_t* len);
 /* Blocking copies between host memory and such a buffer (sync_store / sync_load). */
 int rho_worker_read_buffer(rho_worker* w, int32_t hidden_idx, int which, float* host, int64_t len);

@@ -858,7 +858,12 @@ static int pick_kh(const Conv1x1Params& p, const EpiParams& ep, hipStream_t stre
   return launch_stream<TM, 64, PASS>(p, ep, stream);
 }
 
+// The kernels above address both tensors with 32-bit byte offsets in which 0x80000000 means "nowhere": every byte
+// of a tensor must lie below that.
+static_assert(kMaxBufferBytes <= (size_t(1) << 31), "conv1x1 offsets: 0x80000000 must stay out of range");
+
 bool conv1x1_stream_applies(const ConvDims& d) {
+  if (4 * (size_t)d.N * d.P * d.Q * (size_t)(d.C > d.K ? d.C : d.K) > (size_t(1) << 31)) return false;
   return d.R == 1 && d.S == 1 && d.st == 1 && d.pad == 0 && d.C <= kConv1x1MaxChannels && d.K <= kConv1x1MaxChannels &&
          (long long)d.N * d.P * d.Q < (1ll << 31) - 64;
 }

@@ -1844,8 +1844,11 @@ class SoftmaxKLLossOperator : public LossOperator {
   }
   // Second generation (src/layer_new.rs:2103-2134): out_loss sums the batches' losses until reset_loss.  The
   // reference's per-sample kernel there (`..._softmax_cross_entropy_loss`, trailing argument 1.0) lives outside its
-  // tree; taken here: loss1[n] = -w_n log p[n, y_n] overwritten per batch (the kl_loss1 kernel with factor 0), then
-  // the block sum added to out_loss with factor 1.
+  // tree, so what that 1.0 means is this build's reading: loss1[n] = -w_n log p[n, y_n] is overwritten per batch
+  // (kGen2Loss1Accumulate = 0: the kl_loss1 kernel with factor 0), then the block sum is added to out_loss with factor
+  // 1.  The other reading (loss1 itself accumulates over the batches, which reset_loss zeroing out_loss1 hints at)
+  // is kGen2Loss1Accumulate = 1; it would count every earlier batch's sample losses again in each later block sum.
+  static constexpr float kGen2Loss1Accumulate = 0.0f;
   void reset_loss(size_t batch_size) override {
     RB_ASSERT(batch_size <= batch_cap_);
     rh_stream_t s = context_->stream();
@@ -1856,7 +1859,8 @@ class SoftmaxKLLossOperator : public LossOperator {
     RB_ASSERT(batch_size <= batch_cap_);
     rh_stream_t s = context_->stream();
     rembrandt_kernel_batch_map_softmax_kl_loss1(out_values_.as_ptr(), (int)loss_config_.num_categories, (int)batch_size,
-                                                label_cats_.as_ptr(), weights_.as_ptr(), 0.0f, out_loss1_.as_mut_ptr(), s);
+                                                label_cats_.as_ptr(), weights_.as_ptr(), kGen2Loss1Accumulate,
+                                                out_loss1_.as_mut_ptr(), s);
     unwrap_last("rembrandt_kernel_batch_map_softmax_kl_loss1");
     rembrandt_kernel_batch_blockreduce_sum(out_loss1_.as_ptr(), (int)batch_size, 1, acc_loss_.as_mut_ptr(), 1.0f, s);
     unwrap_last("rembrandt_kernel_batch_blockreduce_sum");

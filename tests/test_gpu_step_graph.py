@@ -11,11 +11,11 @@ from conftest import say
 pytestmark = pytest.mark.gpu
 
 
-def param_buffers(net):
+def param_buffers(net, read_grads=True):
     names = []
     for i, l in enumerate(net[1]):
         if l[0] in ("conv2d", "affine"):
-            names += [(i, b) for b in ("weights", "bias", "acc_grad_weights", "acc_grad_bias", "grad_weights")]
+            names += [(i, b) for b in ("weights", "bias", "acc_grad_weights", "acc_grad_bias") + (("grad_weights",) if read_grads else ())]
         elif l[0] in ("bnorm_conv2d", "stack_res_conv2d", "proj_stack_res_conv2d"):
             units = {"bnorm_conv2d": 1, "stack_res_conv2d": 2, "proj_stack_res_conv2d": 3}[l[0]]
             for u in range(units):
@@ -24,13 +24,13 @@ def param_buffers(net):
     return names
 
 
-def run(net, batch, steps, graph, seed, sgd_kwargs, fused=True, toggle_at=None):
+def run(net, batch, steps, graph, seed, sgd_kwargs, fused=True, toggle_at=None, read_grads=True):
     dims, layers, ncat = net
     w = SequentialOperatorWorker(configs.build_config(net), batch, "Backward", shared_seed=(seed, seed + 1), graph_steps=graph)
     w.init_params()
     sgd = SgdOpt(batch, **sgd_kwargs)
     sgd.begin(w)
-    names = param_buffers(net)
+    names = param_buffers(net, read_grads)
     out = []
     for step in range(steps):
         if toggle_at is not None and step == toggle_at:
@@ -67,6 +67,37 @@ def test_recorded_steps_equal_launched_steps(dev, name, batch, steps):
     assert n1 == steps - 2, "iteration 0 and 1 are launched (first sight of their keys), iteration 2 records, the rest replay"
     same(eager, graph, name)
     assert not np.array_equal(graph[-1][2][0], graph[0][2][0]), "the replays did train"
+
+
+BN_NET_DIMS = (16, 16, 3)
+
+
+def bn_net():
+    return (BN_NET_DIMS, *configs._chain(BN_NET_DIMS, [("bnconv", 3, 1, 1, 8, "Rect"), ("pool", 2, 2, 0, "Max"), ("res", "Rect"),
+                                                       ("conv", 3, 1, 1, 8, "Rect"), ("projres", 16, 2, "Rect"),
+                                                       ("pool", 4, 1, 0, "Average"), ("fc", 5, "Identity")]))
+
+
+@pytest.mark.parametrize("name,batch,steps", [("lenet", 64, 7), ("cifar10", 128, 6), ("bn", 16, 7)])
+def test_recorded_steps_with_gradients_left_standing_for_zeros(dev, name, batch, steps):
+    """The same comparison without ever reading a gradient buffer between steps: the fused step then leaves the gradients
+    of the plain convolution and affine operators as they are (they stand for zeros, the next backward pass overwrites
+    them), and the recordings are filed under, and replayed in, that state."""
+    say("step graph, gradients never read", name)
+    net = bn_net() if name == "bn" else configs.NETWORKS[name]()
+    kw = dict(step_size=0.01, momentum=("Update", 0.9), l2_reg_coef=5e-4)
+    eager, n0 = run(net, batch, steps, False, 0x6A11, kw, read_grads=False)
+    graph, n1 = run(net, batch, steps, True, 0x6A11, kw, read_grads=False)
+    assert n0 == 0 and n1 > 0
+    same(eager, graph, name)
+    # and it is the state the gradient-reading run reaches as well
+    checked, _ = run(net, batch, steps, False, 0x6A11, kw, read_grads=True)
+    for (la, ca, pa), (lb, cb, pb) in zip(eager, checked):
+        assert la == lb and ca == cb
+    names_g = param_buffers(net, True)
+    names_n = param_buffers(net, False)
+    for k, nb in enumerate(names_n):
+        assert np.array_equal(eager[-1][2][k], checked[-1][2][names_g.index(nb)]), nb
 
 
 def test_recorded_steps_with_schedule_nesterov_and_placement_switch(dev):

@@ -27,10 +27,15 @@ def noalloc_bias(dy, alpha=1.0, beta=0.0, db=None):
     return db
 
 
-# (N, K, P, Q): column form (planes under 1024 elements), row form (larger planes), an affine layer (plane 1, no scratch)
-PAIRS = [((256, 256, 27, 27), (37, 96, 13, 13)),
-         ((64, 96, 55, 55), (5, 20, 40, 40)),
-         ((256, 384, 13, 13), (64, 64, 56, 56)),
+# (N, K, P, Q): column form (planes under 1024 elements), row form (larger planes), an affine layer (plane 1, no scratch).
+# Inputs of more than 2^20 elements with planes of more than one element take the two-stage reduction over the scratch
+# array; the second call of the first four pairs does too, over what the first one left there, in the same form and in
+# the other one.
+PAIRS = [((256, 256, 27, 27), (40, 256, 27, 27)),     # column form after column form
+         ((64, 96, 55, 55), (40, 256, 27, 27)),       # column form after row form
+         ((256, 384, 13, 13), (64, 64, 56, 56)),      # row form after column form
+         ((64, 96, 55, 55), (24, 20, 57, 57)),        # row form after row form
+         ((256, 256, 27, 27), (37, 96, 13, 13)),      # a one-stage call (no scratch) after a two-stage one
          ((128, 1000, 1, 1), (3, 7, 1, 1))]
 
 
@@ -38,10 +43,14 @@ PAIRS = [((256, 256, 27, 27), (37, 96, 13, 13)),
 def test_noalloc_bias_gradient_matches_workspace_form(dev, first, second):
     lib = _lib.lib()
     assert lib.rh_noalloc_scratch_bytes() == 8 << 20
+    other = torch.randn(1 << 20, device=dev)
+    if PAIRS.index((first, second)) < 4:   # both calls run the two-stage reduction over the static array
+        assert all(lib.rh_conv2d_bwd_bias_workspace_bytes(s[0], s[1], s[2] * s[3]) > 0 for s in (first, second))
     for shape in (first, second):
         say("no-alloc bias gradient", shape)
         N, K, P, Q = shape
         assert lib.rh_conv2d_bwd_bias_workspace_bytes(N, K, P * Q) <= lib.rh_noalloc_scratch_bytes()
+        ops.rect_inplace(other)    # unrelated work of the library between the calls
         dy = synth.normal(41, N + K, shape)
         db0 = synth.normal(41, 7, (K,))
         dyd = torch.from_numpy(dy).to(dev)
