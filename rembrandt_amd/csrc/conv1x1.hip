@@ -38,7 +38,7 @@ struct Conv1x1Params {
 
 template <int TM_>
 struct StreamTile {
-  static constexpr int TM = TM_, TN = 1;
+  static constexpr int TM = TM_, TN = 1, BM = 32 * TM_, BN = 32;
 };
 
 // FAST: alpha == 1, beta == 0, rows == 32 * TM and the contraction == 2 * KH, so the loads need no channel guard

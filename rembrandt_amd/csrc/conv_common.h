@@ -115,23 +115,23 @@ inline int launch_mfma_gemm_bf16(const typename AL::Params& ap, const typename B
 }
 
 // The direct-to-LDS form for packed operands (ring of four LDS buffers, one pass over the whole contraction).
-template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS, bool PK = false>
+template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS, bool PK = false, int R = 4>
 inline int launch_mfma_gemm_bf16_dma(const RowV8Params& ap, const RowV8Params& bp, const EpiParams& ep, int K,
                                      hipStream_t stream, const char* tag, int k_algorithmic = 0,
                                      const PackedOut& pk = PackedOut()) {
   const int tiles_m = cdiv(ep.rows, T::BM), tiles_n = cdiv(ep.cols, T::BN);
   if (K <= 0 || K % T::BK != 0) return RH_E_INVALID;
-  constexpr size_t lds_bytes = 16 * 4 * (T::BK / 8) * (T::BM + T::BN);
-  static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
+  constexpr size_t lds_bytes = 16 * R * (T::BK / 8) * (T::BM + T::BN);
+  static_assert(lds_bytes * T::OCC <= 160 * 1024, "the blocks meant to share a CU do not fit its 160 KB of LDS");
   if (lds_bytes > 48 * 1024) {
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS, PK>),
+        reinterpret_cast<const void*>(&mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS, PK, R>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr != hipSuccess) return (int)attr;
   }
   ProfScope prof(tag, 2.0 * (double)ep.rows * (double)ep.cols * (double)(k_algorithmic > 0 ? k_algorithmic : K), stream);
   if (PK && !pk.ptr) return RH_E_INVALID;
-  hipLaunchKernelGGL((mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS, PK>), dim3((unsigned)(tiles_m * tiles_n)),
+  hipLaunchKernelGGL((mfma_gemm_bf16_dma_kernel<T, A_LINEAR, B_LINEAR, NCHW, PASS, PK, R>), dim3((unsigned)(tiles_m * tiles_n)),
                      dim3(T::NT), lds_bytes, stream, ap, bp, ep, tiles_m, K / T::BK, pk);
   return launch_status();
 }
@@ -154,6 +154,7 @@ typedef Tile<96, 96, 16, 1, 3, 4> T96x96;   // three waves: a 96 x 96 result (1x
 typedef Tile<128, 128, RH_BF16_BK, 2, 2, RH_BF16_OCC> T128x128bf;
 // Tile of the direct-to-LDS bf16 kernel: eight waves of 128x64 each, one block per CU, four 32-k LDS buffers.
 typedef Tile<256, 256, 32, 2, 4, 1> T256x256bf;
+typedef Tile<256, 128, 32, 2, 2, 2> T256x128bf;   // direct-to-LDS form with a ring of three: two blocks of four waves share a CU
 typedef Tile<64, 256, 16, 1, 4, 3> T64x256;
 typedef Tile<32, 256, 16, 1, 4, 3> T32x256;
 // few result columns as well (a first layer's filter gradient: 20 x 25, 32 x 75): narrower tiles, fewer dead columns

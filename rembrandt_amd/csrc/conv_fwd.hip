@@ -496,7 +496,7 @@ static int bf16_pack_input(const ConvDims& d, const Bf16FwdPlan& bpn, const floa
 // The contraction on prepared operands: `xb` the image copy, `wprep` the filter stage's result.  The result goes to
 // ep.out as fp32 NCHW, or, with pk.ptr set, as packed bf16 for the next convolution (ep.out unused).  Which kernel
 // runs depends on the geometry only, so both forms of the result come from the same accumulators.
-template <class T, bool DMA, bool PK>
+template <class T, bool DMA, bool PK, int R = 4>
 static int bf16_gemm_on(const ConvDims& d, const Bf16FwdPlan& bpn, const void* xb, const void* wprep, const EpiParams& ep,
                         const PackedOut& pk, hipStream_t stream, const char* tag) {
   const char* base = static_cast<const char*>(wprep);
@@ -522,27 +522,36 @@ static int bf16_gemm_on(const ConvDims& d, const Bf16FwdPlan& bpn, const void* x
   typedef LoadRowV8<T::BM, T::BK, T::NT, true> AL;
   typedef LoadRowV8<T::BN, T::BK, T::NT, false> BL;
   if constexpr (DMA)
-    return launch_mfma_gemm_bf16_dma<T, true, false, true, PassConvFwd, PK>(ap, bp, ep, bpn.n_k, stream, tag, CRS, pk);
+    return launch_mfma_gemm_bf16_dma<T, true, false, true, PassConvFwd, PK, R>(ap, bp, ep, bpn.n_k, stream, tag, CRS, pk);
   else
     return launch_mfma_gemm_bf16<T, AL, BL, true, PassConvFwd, PK>(ap, bp, ep, bpn.n_k, 1, nullptr, stream, tag, CRS, pk);
 }
 
 static int bf16_gemm(const ConvDims& d, const Bf16FwdPlan& bpn, const void* xb, const void* wprep, const EpiParams& ep,
                      const PackedOut& pk, hipStream_t stream, bool force_stream = false) {
-  // Long contractions on grids that fill all 256 CUs with 256-row tiles (and waste no more filter rows than
-  // 128-row tiles would) take the direct-to-LDS kernel: 14 % faster on 256 x 96 x 27 x 27 -> 256, 5x5.  Short
-  // contractions lose there (one block per CU: nothing hides a tile's first loads and its stores).
-  const bool dma = bpn.n_k >= 512 && cdiv(d.K, 256) * 256 == cdiv(d.K, 128) * 128 &&
-                   (long long)cdiv(d.K, 256) * cdiv(ep.cols, 256) >= 256;
   // 1x1 layers of up to 128 channels between packed activations are copies with a contraction riding along: the
   // streaming kernel (same accumulation order, hence the same bits as the tiles)
   if (pk.ptr && bpn.s_groups == 0 && (conv1x1_bf16_stream_applies(d) || (force_stream && conv1x1_bf16_stream_runs(d))))
     return launch_conv1x1_bf16_stream(d, xb, static_cast<const char*>(wprep) + bpn.tab_bytes, ep.bias, ep.relu, pk, stream);
+  // Filter counts that waste no more rows in 256-row tiles than in 128-row ones take a direct-to-LDS kernel:
+  //  - 256 x 256 (one block of eight waves per CU, ring of four) for long contractions on grids of two rounds of
+  //    the 256 CUs and more: 1.19 PFLOP/s on 256 x 96 x 27 x 27 -> 256, 5x5 (729 tiles);
+  //  - 256 x 128 (two blocks of four waves per CU, ring of three) otherwise, from contractions of 256 and grids
+  //    of one round on: a block's first loads and its stores hide behind the other block, and a grid of 365
+  //    256 x 256 tiles (the same layer at batch 128) is no longer two rounds with the second 43 % full.
+  // Short contractions and small grids stay with the 128 x 128 tile (three blocks per CU, through registers).
+  const bool rows_ok = cdiv(d.K, 256) * 256 == cdiv(d.K, 128) * 128;
+  const long long t256 = (long long)cdiv(d.K, 256) * cdiv(ep.cols, 256);
+  const long long t128 = (long long)cdiv(d.K, 256) * cdiv(ep.cols, 128);
+  const bool big = rows_ok && bpn.n_k >= 512 && t256 >= 512;
+  const bool mid = rows_ok && !big && bpn.n_k >= 256 && t128 >= 256;
   if (pk.ptr) {
-    if (dma) return bf16_gemm_on<T256x256bf, true, true>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
+    if (big) return bf16_gemm_on<T256x256bf, true, true, 4>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
+    if (mid) return bf16_gemm_on<T256x128bf, true, true, 3>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x128");
     return bf16_gemm_on<T128x128bf, false, true>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x128");
   }
-  if (dma) return bf16_gemm_on<T256x256bf, true, false>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
+  if (big) return bf16_gemm_on<T256x256bf, true, false, 4>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
+  if (mid) return bf16_gemm_on<T256x128bf, true, false, 3>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x128");
   return bf16_gemm_on<T128x128bf, false, false>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x128");
 }
 

@@ -656,6 +656,15 @@ __device__ __forceinline__ int xcd_remap(int b, int nb) {
 // Epilogue shared by the fp32 and bf16 kernels: D (in the 32x32 MFMA accumulator layout: lane%32 = column,
 // rows 8*(v/4) + 4*(lane/32) + v%4) -> out, with the alpha/beta blend, optional bias and ReLU, or unblended
 // into this split's slab of the partial-sum buffer.
+//
+// Loads and stores of a wave complete in order and share one counter, and the compiler cannot know that bias and
+// mask do not alias the result: written element by element (load bias, load mask, store) every load waits for
+// the store before it, a round trip to memory per element.  So the loads stand ahead of the stores here: the
+// result goes out one 32 x 32 block at a time, and the bias of the next row of blocks (or the mask values of the
+// next block) is fetched before the current block's stores are issued, never between two stores.
+// Addresses: buffer instructions over the result (and the mask, which has its shape), a per-lane byte offset for
+// each column block plus a wave-uniform offset for the row, so that a store costs no vector arithmetic and no
+// address registers.  (Results, like operands, are at most kMaxBufferBytes long: the callers check.)
 template <class T, bool NCHW>
 __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], const EpiParams& ep, int m0, int n0,
                                            int wm, int wn, int lane, int split_idx) {
@@ -666,39 +675,152 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], co
                                    : ep.out + (long long)split_idx * ep.split_stride;
   const float alpha = split ? 1.0f : ep.alpha;
   const float beta = split ? 0.0f : ep.beta;
-  const int row_stride = NCHW ? ep.inner : ep.ld;
+  const uint32_t rs4 = 4u * (uint32_t)(NCHW ? ep.inner : ep.ld);  // bytes from a row to the next
+  const int rlane = m0 + wm * (TM * 32) + (lane >> 5) * 4;
+  const int clane = n0 + wn * (TN * 32) + (lane & 31);
+  const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, 0x80000000u);
+  // byte offset of (row rlane, this lane's column of block j)
+  uint32_t voff[TN];
+  bool col_ok[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
-    if (col >= ep.cols) continue;
-    int coloff;
-    float cbias = 0.0f;
+    const int col = clane + j * 32;
+    col_ok[j] = col < ep.cols;
+    uint32_t e = (uint32_t)col;
     if (NCHW) {
       const int img = col / ep.inner;
-      coloff = img * ep.rows * ep.inner + (col - img * ep.inner);
-    } else {
-      coloff = col;
-      if (!split && ep.bias_col) cbias = ep.bias_col[col];
+      e = (uint32_t)img * (uint32_t)ep.rows * (uint32_t)ep.inner + (uint32_t)(col - img * ep.inner);
     }
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int rbase = m0 + wm * (TM * 32) + i * 32 + (lane >> 5) * 4;
+    voff[j] = e * 4u + (uint32_t)rlane * rs4;
+  }
+  auto krow = [](int i, int v) { return i * 32 + (v >> 2) * 8 + (v & 3); };  // row of element v of block row i, from rlane
+  const bool has_bias = !split && ep.bias != nullptr;
+  const bool has_cbias = !NCHW && !split && ep.bias_col != nullptr;
+  const bool relu = !split && ep.relu;
+  const float* mask = NCHW && !split ? ep.mask : nullptr;
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(has_bias ? ep.bias : out, has_bias ? 4u * (uint32_t)ep.rows : 0u);
+  const __amdgpu_buffer_rsrc_t rm = make_rsrc(mask ? mask : out, mask ? 0x80000000u : 0u);
+
+  // One 32 x 32 block at a time, so that only its 16 values are live next to the accumulators (which die block
+  // by block) and whatever has been fetched ahead.
+  auto run = [&](auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;  // no element of this block's tile lies outside the result
+    auto ok = [&](int i, int j, int v) { return FULL || (col_ok[j] && rlane + krow(i, v) < ep.rows); };
+    auto load16 = [&](__amdgpu_buffer_rsrc_t rs, int i, int j, float (&x)[16]) {  // the block's elements of a tensor shaped like the result
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int row = rbase + (v >> 2) * 8 + (v & 3);
-        if (row < ep.rows) {
-          float* dst = out + (size_t)coloff + (size_t)row * row_stride;
+        x[v] = 0.0f;
+        if (ok(i, j, v))
+          x[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (int)voff[j], (int)((uint32_t)krow(i, v) * rs4), 0));
+      }
+    };
+    auto load_bias = [&](int i, float (&x)[16]) {  // rows past the last read as 0
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        x[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb, rlane * 4, krow(i, v) * 4, 0));
+    };
+    auto store16 = [&](int i, int j, const float (&x)[16]) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        if (ok(i, j, v))
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(x[v]), rout, (int)voff[j], (int)((uint32_t)krow(i, v) * rs4), 0);
+    };
+    float cb[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) cb[j] = 0.0f;
+    if (has_cbias) {
+      const __amdgpu_buffer_rsrc_t rc = make_rsrc(ep.bias_col, 4u * (uint32_t)ep.cols);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        cb[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rc, (clane + j * 32) * 4, 0, 0));
+    }
+    // value = alpha * acc (+ beta * old) (+ bias[row]) (+ bias_col[col]) (clamped at 0) (0 where the mask is not > 0)
+    if (beta != 0.0f || (mask && (has_bias || has_cbias))) {
+      // accumulating calls (and combinations nothing in the library asks for): what a block needs is read
+      // ahead of its own stores, behind those of the block before, one kind of operand at a time (registers)
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          float x[16], t[16];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) x[v] = alpha * acc[i][j][v];
+          if (beta != 0.0f) {
+            load16(rout, i, j, t);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] += beta * t[v];
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (has_bias) {
+            load_bias(i, t);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] += t[v];
+          }
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            if (has_cbias) x[v] += cb[j];
+            if (relu) x[v] = x[v] > 0.0f ? x[v] : 0.0f;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (mask) {
+            load16(rm, i, j, t);
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+              if (!(t[v] > 0.0f)) x[v] = 0.0f;
+          }
+          store16(i, j, x);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else if (mask) {
+      // backward-data with the ReLU backward folded in: a block's mask values are fetched after the block before
+      // it has taken its own (one set of registers) and before that block's stores are issued
+      float mk[16];
+      load16(rm, 0, 0, mk);
+#pragma unroll
+      for (int b = 0; b < TM * TN; ++b) {
+        const int i = b % TM, j = b / TM;
+        float x[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
           float val = alpha * acc[i][j][v];
-          if (beta != 0.0f) val += beta * *dst;
-          if (!split && ep.bias) val += ep.bias[row];
-          if (!NCHW && !split && ep.bias_col) val += cbias;
-          if (!split && ep.relu) val = val > 0.0f ? val : 0.0f;
-          if (NCHW && !split && ep.mask && !(ep.mask[(size_t)coloff + (size_t)row * row_stride] > 0.0f)) val = 0.0f;
-          *dst = val;
+          if (relu) val = val > 0.0f ? val : 0.0f;
+          if (!(mk[v] > 0.0f)) val = 0.0f;
+          x[v] = val;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (b + 1 < TM * TN) load16(rm, (b + 1) % TM, (b + 1) / TM, mk);
+        store16(i, j, x);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      // forward passes and partial sums: the bias of the next row of blocks is fetched once the last block of
+      // this row has taken its own, before that block's stores are issued
+      float bv[16];
+      if (has_bias) load_bias(0, bv);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          float x[16];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            float val = alpha * acc[i][j][v];
+            if (has_bias) val += bv[v];
+            if (has_cbias) val += cb[j];
+            if (relu) val = val > 0.0f ? val : 0.0f;
+            x[v] = val;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (has_bias && j == TN - 1 && i + 1 < TM) load_bias(i + 1, bv);
+          store16(i, j, x);
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
-  }
+  };
+  if (m0 + T::BM <= ep.rows && n0 + T::BN <= ep.cols) run(std::true_type());
+  else run(std::false_type());
 }
 
 // Packed bf16 result: the NCHW result (img, row, p, q) written as bf16 in the operand layout the packed loaders read,
@@ -713,12 +835,51 @@ struct PackedOut {
   FastDiv dQ;          // division of a pixel index by Q
 };
 
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
 template <class T>
 __device__ __forceinline__ void store_tile_packed(const f32x16 (&acc)[T::TM][T::TN], const EpiParams& ep, const PackedOut& pk,
                                                   int m0, int n0, int wm, int wn, int lane) {
   constexpr int TM = T::TM, TN = T::TN;
-  char* const base = static_cast<char*>(pk.ptr);
   const int sub = (lane >> 5) * 4;  // this lane's four rows inside a group of eight
+  const int rwave = m0 + wm * (TM * 32);  // first row of the wave's part: a multiple of 32
+  float r[TM][TN][16];  // separate scalars (see store_tile)
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) r[i][j][v] = acc[i][j][v];
+  // bias first, for all of the lane's rows, so that no load stands between the stores (see store_tile);
+  // rows past the last read as 0
+  if (ep.bias) {
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(ep.bias, 4u * (uint32_t)ep.rows);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      float bv[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        bv[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb, (rwave + sub) * 4,
+                                                                               (i * 32 + (v >> 2) * 8 + (v & 3)) * 4, 0));
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) r[i][j][v] += bv[v];
+    }
+  }
+  if (ep.relu) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) r[i][j][v] = r[i][j][v] > 0.0f ? r[i][j][v] : 0.0f;
+  }
+  // Buffer stores: a per-lane byte offset for each column block (the pixel's group of row group 0, plus this
+  // lane's half of the group) and a wave-uniform one for the row group.  (The packed tensor is at most
+  // kMaxBufferBytes long: the callers check.)
+  const __amdgpu_buffer_rsrc_t rout = make_rsrc(pk.ptr, 0x80000000u);
+  const uint32_t wp16 = 16u * (uint32_t)pk.Wp;
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
@@ -726,26 +887,18 @@ __device__ __forceinline__ void store_tile_packed(const f32x16 (&acc)[T::TM][T::
     const int img = col / ep.inner;
     uint32_t p, q;
     pk.dQ.divmod((uint32_t)(col - img * ep.inner), p, q);
-    const size_t g0 = (size_t)img * pk.img_groups + (size_t)((int)p + pk.halo) * pk.Cg * pk.Wp + (size_t)((int)q + pk.halo);
+    const uint32_t voff = 16u * ((uint32_t)img * (uint32_t)pk.img_groups + (uint32_t)((int)p + pk.halo) * (uint32_t)(pk.Cg * pk.Wp) +
+                                 (uint32_t)((int)q + pk.halo)) + (uint32_t)sub * 2u;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int rbase = m0 + wm * (TM * 32) + i * 32 + sub;
 #pragma unroll
       for (int vg = 0; vg < 4; ++vg) {
-        const int row0 = rbase + vg * 8;
-        if (row0 < ep.rows) {
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float val = acc[i][j][vg * 4 + e];
-            if (ep.bias) val += ep.bias[row0 + e];
-            if (ep.relu) val = val > 0.0f ? val : 0.0f;
-            v[e] = val;
-          }
-          uint2 w;
-          w.x = pack_bf16(v[0], v[1]);
-          w.y = pack_bf16(v[2], v[3]);
-          *reinterpret_cast<uint2*>(base + (g0 + (size_t)(row0 >> 3) * pk.Wp) * 16 + sub * 2) = w;
+        const int rg = (rwave >> 3) + i * 4 + vg;  // row group of eight (wave-uniform)
+        if (rg * 8 < ep.rows) {
+          u32x2 w;
+          w.x = pack_bf16(r[i][j][vg * 4 + 0], r[i][j][vg * 4 + 1]);
+          w.y = pack_bf16(r[i][j][vg * 4 + 2], r[i][j][vg * 4 + 3]);
+          __builtin_amdgcn_raw_buffer_store_b64(w, rout, (int)voff, (int)((uint32_t)rg * wp16), 0);
         }
       }
     }
@@ -1033,15 +1186,18 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_kernel(typename 
 // the path has.  A 256x256 tile halves the fill per MFMA, the direct loads need no registers, no ds_write and no
 // issue slots beyond the load itself, and they complete in the background.
 //
-// Step `it` of a wave: multiplies out of buffer it; issues the loads of step it+3 into buffer it+3 (= it-1, read
-// for the last time before the barrier that ended step it-1); reads, during its last group of MFMAs, the first
-// operands of step it+1 (buffer it+1); then waits until only the loads it has just issued are still in flight
-// (so those of step it+2 have landed) and meets the other waves at the step's one barrier.  A load therefore has
-// two steps to land, and nothing the matrix pipe has to wait for follows a barrier.
+// Ring of R buffers, loads issued D = R - 1 steps ahead.  Step `it` of a wave: multiplies out of buffer it; issues
+// the loads of step it+D into buffer it+D (= it-1 mod R, read for the last time before the barrier of step it-1);
+// in front of its last group of MFMAs waits until only the loads of steps it+2 .. it+D are still in flight,
+// meets the other waves at the step's one barrier, and reads the first operands of step it+1 (whose buffer is now
+// complete for every wave) under that last group.  A load therefore has D - 1/2 steps to land (2.5 with a ring of
+// four), and nothing the matrix pipe has to wait for follows a barrier: with the barrier at the end of the step and
+// two steps to land the same loop was 14 % slower on 256 x 2400 x 186624.
 // The compiler does not see these loads (inline asm): their completion is counted by hand (vmcnt is in order),
 // and no other vector memory instruction is issued between the prologue and the epilogue.
-// One block per CU (128 KB of LDS): the first loads and the stores of a tile are not hidden behind another block,
-// which is why this form pays only for long contractions.
+// Shapes: 256 x 256 with eight waves and a ring of four (128 KB: one block per CU, so the first loads and the
+// stores of a tile are not hidden behind another block: long contractions on large grids), or 256 x 128 with four
+// waves and a ring of three (72 KB: two blocks per CU).
 // ------------------------------------------------------------------------------------------
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -1123,14 +1279,15 @@ struct DmaRowV8 {
   }
 };
 
-template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS, bool PK = false>
+template <class T, bool A_LINEAR, bool B_LINEAR, bool NCHW, class PASS, bool PK = false, int R = 4>
 __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8Params ap, RowV8Params bp, EpiParams ep,
                                                                            int tiles_m, int k_chunks, PackedOut pk) {
   constexpr int BM = T::BM, BN = T::BN, BK = T::BK, TM = T::TM, TN = T::TN;
   static_assert(BK % 32 == 0, "an even number of 16-k groups per step keeps the operand register sets in phase");
   typedef DmaRowV8<BM, BK, T::NT, A_LINEAR> AL;
   typedef DmaRowV8<BN, BK, T::NT, B_LINEAR> BL;
-  constexpr int KG = BK / 8, STEPS = BK / 16, R = 4;
+  constexpr int KG = BK / 8, STEPS = BK / 16, D = R - 1;  // D: how many steps ahead the loads are issued
+  static_assert(R >= 3, "the ring holds the step being read, one landed or landing, and one in flight at least");
   constexpr int SA = KG * BM, SB = KG * BN;  // 16-byte groups per buffer
   extern __shared__ float lds_dyn[];
   uint4* const sA_base = reinterpret_cast<uint4*>(lds_dyn);  // [R][KG][BM]
@@ -1169,12 +1326,11 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8
     la.issue(ldsA + (uint32_t)(buf * SA) * 16u);
     lb.issue(ldsB + (uint32_t)(buf * SB) * 16u);
   };
-  // steps 0..2 on their way, the offsets of step 3 fetched
-  prep_step(0);
-  issue_step(0);
-  if (nk > 1) { prep_step(1); issue_step(1); }
-  if (nk > 2) { prep_step(2); issue_step(2); }
-  if (nk > 3) prep_step(3);
+  // steps 0..D-1 on their way, the offsets of step D fetched
+#pragma unroll
+  for (int s = 0; s < D; ++s)
+    if (s < nk) { prep_step(s); issue_step(s); }
+  if (nk > D) prep_step(D);
   wait_vmcnt<0>();
   __syncthreads();
 
@@ -1188,8 +1344,8 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8
   __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the loop is entered with nothing in flight, so its waits can be exact
 
   auto step = [&](int it, auto more_tag) {
-    constexpr bool MORE = decltype(more_tag)::value;  // this step issues the loads of step it+3
-    const int rd = it & (R - 1), nx = (it + 1) & (R - 1);
+    constexpr bool MORE = decltype(more_tag)::value;  // this step issues the loads of step it+D
+    const int rd = it % R, nx = (it + 1) % R;
     const uint4* pa = sA_base + rd * SA + a_rd;
     const uint4* pb = sB_base + rd * SB + b_rd;
     const uint4* pna = sA_base + nx * SA + a_rd;
@@ -1202,10 +1358,10 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8
       // ago: an explicit wait here costs nothing, and it lets the wait in front of this group's MFMAs disappear
       // (otherwise that one, being a wait for "everything" because scalar loads return out of order, would also
       // cover the operand reads issued just before it).
-      if (g > 0) __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_s_waitcnt(0xc07f);
       if (MORE && g == 0) {
-        // the offsets of step it+4 (used by the loads the next step issues), fetched first for the same reason
-        const int s4 = it + 4 < nk ? it + 4 : nk - 1;
+        // the offsets of step it+D+1 (used by the loads the next step issues), fetched first for the same reason
+        const int s4 = it + D + 1 < nk ? it + D + 1 : nk - 1;
         la.prep_next(s4 * BK);
         lb.prep_next(s4 * BK);
       }
@@ -1214,13 +1370,21 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8
         for (int i = 0; i < TM; ++i) a[n][i] = pa[(2 * g + 2) * BM + i * 32];
 #pragma unroll
         for (int j = 0; j < TN; ++j) b[n][j] = pb[(2 * g + 2) * BN + j * 32];
-      } else {  // (after the last step this reads a buffer nobody uses: harmless)
+      } else {
+        // The step's one barrier stands here, in front of its last group of MFMAs.  Every wave has read all it
+        // needs of buffer `it` (the wait above), so the loads the next step issues may overwrite it; and with
+        // only the loads of steps it+2 .. it+D allowed in flight, buffer it+1 is complete once all waves are
+        // past: its first operands are read under this group's MFMAs.  A load has D - 1/STEPS steps to land.
+        // (After the last step this reads a buffer nobody uses: harmless.)
+        if (MORE) wait_vmcnt<(R - 2) * (AL::CNT + BL::CNT)>();
+        else wait_vmcnt<0>();
+        __syncthreads();
 #pragma unroll
         for (int i = 0; i < TM; ++i) a[n][i] = pna[i * 32];
 #pragma unroll
         for (int j = 0; j < TN; ++j) b[n][j] = pnb[j * 32];
       }
-      if (MORE && g == 0) issue_step((it + 3) & (R - 1));
+      if (MORE && g == 0) issue_step((it + D) % R);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -1233,14 +1397,10 @@ __global__ __launch_bounds__(T::NT, T::OCC) void mfma_gemm_bf16_dma_kernel(RowV8
     if (MORE) {
       la.rotate();
       lb.rotate();
-      wait_vmcnt<AL::CNT + BL::CNT>();
-    } else {
-      wait_vmcnt<0>();
     }
-    __syncthreads();
   };
   int it = 0;
-  for (; it + 3 < nk; ++it) step(it, std::true_type());
+  for (; it + D < nk; ++it) step(it, std::true_type());
   for (; it < nk; ++it) step(it, std::false_type());
 
   if constexpr (PK) store_tile_packed<T>(acc, ep, pk, m0, n0, wm, wn, lane);
