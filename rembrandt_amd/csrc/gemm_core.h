@@ -706,12 +706,24 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[T::TM][T::TN], co
   auto run = [&](auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;  // no element of this block's tile lies outside the result
     auto ok = [&](int i, int j, int v) { return FULL || (col_ok[j] && rlane + krow(i, v) < ep.rows); };
-    auto load16 = [&](__amdgpu_buffer_rsrc_t rs, int i, int j, float (&x)[16]) {  // the block's elements of a tensor shaped like the result
+    // the block's elements of a tensor shaped like the result; elements outside it read 0.  Without branches where
+    // the wave-uniform part of the offset cannot reach 2^31 (an offset with the top bit set is out of the buffer's
+    // range): a load under a branch is waited for before the next one is issued.
+    const bool select_form = rs4 <= 0x7fffffffu / (32u * TM);
+    auto load16 = [&](__amdgpu_buffer_rsrc_t rs, int i, int j, float (&x)[16]) {
+      if (FULL || select_form) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        x[v] = 0.0f;
-        if (ok(i, j, v))
-          x[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (int)voff[j], (int)((uint32_t)krow(i, v) * rs4), 0));
+        for (int v = 0; v < 16; ++v) {
+          const uint32_t vo = ok(i, j, v) ? voff[j] : 0x80000000u;
+          x[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (int)vo, (int)((uint32_t)krow(i, v) * rs4), 0));
+        }
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          x[v] = 0.0f;
+          if (ok(i, j, v))
+            x[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (int)voff[j], (int)((uint32_t)krow(i, v) * rs4), 0));
+        }
       }
     };
     auto load_bias = [&](int i, float (&x)[16]) {  // rows past the last read as 0
