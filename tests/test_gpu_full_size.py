@@ -106,6 +106,46 @@ def test_conv2d_full_size(dev, name):
     torch.cuda.synchronize()
 
 
+
+def test_conv2d_epilogue_on_a_16m_pixel_plane(dev):
+    """One image of 4099 x 4099 pixels, eight channels either side: rows of the result are 67 MB apart, so the
+    wave-uniform row offsets of the tile epilogue's edge tiles could pass 2^31 and its operand loads (old values for
+    beta, the ReLU mask of the data gradient) take their guarded form.  Sampled oracle, whole-tensor identities."""
+    Nn, C, H, W, K, R, st, pad = 1, 8, 4099, 4099, 8, 3, 1, 1
+    say("conv epilogue, 16 M pixel plane")
+    rng = np.random.default_rng(9)
+    x = synth.normal(31, 1, (Nn, C, H, W))
+    w = synth.normal(31, 2, (K, C, R, R))
+    b = synth.normal(31, 3, (K,))
+    y0 = synth.normal(31, 4, (Nn, K, H, W))
+    xd, wd = T(x, dev), T(w, dev)
+    y = ops.conv2d_fwd(xd, wd, st, pad)
+    i_y = sample_idx(rng, y.numel(), 4096)
+    ref = O.conv2d_fwd_at(x, w, st, pad, i_y)
+    assert_close(y.flatten()[T(i_y, dev)].cpu().numpy(), ref, "large plane fwd (sampled)")
+    yb = ops.conv2d_fwd(xd, wd, st, pad, bias=T(b, dev), relu=True, alpha=0.5, beta=2.0, y=T(y0, dev))
+    kk = (i_y // (H * W)) % K
+    want = np.maximum(0.5 * ref.astype(np.float64) + 2.0 * y0.ravel()[i_y] + b[kk], 0.0)
+    assert_close(yb.flatten()[T(i_y, dev)].cpu().numpy(), want, "large plane fwd alpha/beta/bias/relu (sampled)")
+    del yb
+    dy = synth.normal(31, 5, (Nn, K, H, W))
+    dyd = T(dy, dev)
+    dx0 = synth.normal(31, 6, (Nn, C, H, W))
+    dx = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad)
+    i_x = sample_idx(rng, dx.numel(), 4096)
+    refx = O.conv2d_bwd_data_at(w, dy, x.shape, st, pad, i_x)
+    assert_close(dx.flatten()[T(i_x, dev)].cpu().numpy(), refx, "large plane bwd data (sampled)")
+    for alpha, beta in ((1.0, 0.0), (0.5, 2.0)):
+        two = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad, alpha=alpha, beta=beta, dx=T(dx0, dev))
+        two = torch.where(xd > 0, two, torch.zeros_like(two))
+        one = ops.conv2d_bwd_data(wd, dyd, x.shape, st, pad, alpha=alpha, beta=beta, dx=T(dx0, dev), relu_of=xd)
+        assert torch.equal(one, two), "large plane masked data gradient alpha=%g beta=%g" % (alpha, beta)
+        del one, two
+    a = dot64(y, dyd)
+    scale = float(y.double().norm().item() * dyd.double().norm().item()) / np.sqrt(y.numel())
+    assert abs(a - dot64(xd, dx)) <= 1e-4 * scale, ("large plane bwd data adjoint", a, dot64(xd, dx), scale)
+    torch.cuda.synchronize()
+
 @pytest.mark.parametrize("name", sorted(FULL_CONV))
 def test_conv2d_fwd_bf16_full_size(dev, name):
     Nn, C, H, W, K, R, st, pad = FULL_CONV[name]
