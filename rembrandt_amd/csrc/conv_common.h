@@ -155,6 +155,7 @@ typedef Tile<128, 128, RH_BF16_BK, 2, 2, RH_BF16_OCC> T128x128bf;
 // Tile of the direct-to-LDS bf16 kernel: eight waves of 128x64 each, one block per CU, four 32-k LDS buffers.
 typedef Tile<256, 256, 32, 2, 4, 1> T256x256bf;
 typedef Tile<256, 128, 32, 2, 2, 2> T256x128bf;   // direct-to-LDS form with a ring of three: two blocks of four waves share a CU
+typedef Tile<128, 256, 32, 2, 2, 2> T128x256bf;   // the same for filter counts that would waste rows of a 256-row tile
 typedef Tile<64, 256, 16, 1, 4, 3> T64x256;
 typedef Tile<32, 256, 16, 1, 4, 3> T32x256;
 // few result columns as well (a first layer's filter gradient: 20 x 25, 32 x 75): narrower tiles, fewer dead columns

@@ -544,14 +544,18 @@ static int bf16_gemm(const ConvDims& d, const Bf16FwdPlan& bpn, const void* xb, 
   const long long t256 = (long long)cdiv(d.K, 256) * cdiv(ep.cols, 256);
   const long long t128 = (long long)cdiv(d.K, 256) * cdiv(ep.cols, 128);
   const bool big = rows_ok && bpn.n_k >= 512 && t256 >= 512;
-  const bool mid = rows_ok && !big && bpn.n_k >= 256 && t128 >= 256;
+  const bool mid = rows_ok && !big && bpn.n_k >= 256 && t128 >= 96;
+  // other filter counts (384: one and a half 256-row tiles) take the same loop on 128 rows x 256 pixels
+  const bool mid128 = !rows_ok && bpn.n_k >= 256 && (long long)cdiv(d.K, 128) * cdiv(ep.cols, 256) >= 96;
   if (pk.ptr) {
     if (big) return bf16_gemm_on<T256x256bf, true, true, 4>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
     if (mid) return bf16_gemm_on<T256x128bf, true, true, 3>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x128");
+    if (mid128) return bf16_gemm_on<T128x256bf, true, true, 3>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x256");
     return bf16_gemm_on<T128x128bf, false, true>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x128");
   }
   if (big) return bf16_gemm_on<T256x256bf, true, false, 4>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x256");
   if (mid) return bf16_gemm_on<T256x128bf, true, false, 3>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_256x128");
+  if (mid128) return bf16_gemm_on<T128x256bf, true, false, 3>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x256");
   return bf16_gemm_on<T128x128bf, false, false>(d, bpn, xb, wprep, ep, pk, stream, "conv_fwd_bf16p_128x128");
 }
 
