@@ -31,6 +31,19 @@ def sample_idx(rng, total, n):
     return idx
 
 
+def edge_idx(rng, shape, n):
+    """Flat indices of elements of an NCHW tensor that sit on the seams of the kernels' tiles: channel (GEMM row)
+    and column (image * plane + pixel) positions one either side of multiples of 32 (the MFMA block; 64-, 96-, 128-
+    and 256-wide tiles and wave parts start on these), where an indexing mistake would touch only a few elements."""
+    Nn, K, P, Q = shape
+    inner, cols = P * Q, Nn * P * Q
+    c = 32 * rng.integers(0, (cols + 31) // 32 + 1, n) + rng.integers(-1, 2, n)
+    r = 32 * rng.integers(0, (K + 31) // 32 + 1, n) + rng.integers(-1, 1, n)
+    c = np.clip(c, 0, cols - 1).astype(np.int64)
+    r = np.clip(r, 0, K - 1).astype(np.int64)
+    return (c // inner) * (K * inner) + r * inner + c % inner
+
+
 FULL_CONV = {
     # name: N, C, H, W, K, R, stride, pad
     "sweep_a_alexnet_conv2": (256, 96, 27, 27, 256, 5, 1, 2),
@@ -84,6 +97,12 @@ def test_conv2d_full_size(dev, name):
     i_x = sample_idx(rng, dx.numel(), 4096)
     assert_close(dx.flatten()[T(i_x, dev)].cpu().numpy(), O.conv2d_bwd_data_at(w, dy, x.shape, st, pad, i_x),
                  name + " bwd data (sampled)")
+    # and on the seams of the tiles
+    e_y = edge_idx(rng, tuple(y.shape), 2048)
+    assert_close(y.flatten()[T(e_y, dev)].cpu().numpy(), O.conv2d_fwd_at(x, w, st, pad, e_y), name + " fwd (tile seams)")
+    e_x = edge_idx(rng, x.shape, 2048)
+    assert_close(dx.flatten()[T(e_x, dev)].cpu().numpy(), O.conv2d_bwd_data_at(w, dy, x.shape, st, pad, e_x),
+                 name + " bwd data (tile seams)")
 
     # adjoint identities over the whole tensors (fp64 sums); scale = size of such a sum for unrelated vectors
     a = dot64(y, dyd)
@@ -146,6 +165,7 @@ def test_conv2d_epilogue_on_a_16m_pixel_plane(dev):
     assert abs(a - dot64(xd, dx)) <= 1e-4 * scale, ("large plane bwd data adjoint", a, dot64(xd, dx), scale)
     torch.cuda.synchronize()
 
+
 @pytest.mark.parametrize("name", sorted(FULL_CONV))
 def test_conv2d_fwd_bf16_full_size(dev, name):
     Nn, C, H, W, K, R, st, pad = FULL_CONV[name]
@@ -157,6 +177,9 @@ def test_conv2d_fwd_bf16_full_size(dev, name):
     i_y = sample_idx(rng, y.numel(), 4096)
     ref = O.conv2d_fwd_at(O.round_bf16(x), O.round_bf16(w), st, pad, i_y)
     assert_close(y.flatten()[T(i_y, dev)].cpu().numpy(), ref, name + " bf16 fwd (sampled)")
+    e_y = edge_idx(rng, tuple(y.shape), 2048)
+    assert_close(y.flatten()[T(e_y, dev)].cpu().numpy(), O.conv2d_fwd_at(O.round_bf16(x), O.round_bf16(w), st, pad, e_y),
+                 name + " bf16 fwd (tile seams)")
     # exact linearity and agreement with the fp32 kernel on operands that are already bf16 values
     xr, wr = T(O.round_bf16(x), dev), T(O.round_bf16(w), dev)
     assert torch.equal(ops.conv2d_fwd(xr, wr * 2.0, st, pad, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC), y * 2.0)
