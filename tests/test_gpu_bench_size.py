@@ -4,7 +4,8 @@ bias gradients on the second stream, fused SGD steps on the second stream joined
 
 The CPU oracle cannot recompute these tensors whole in seconds, so every operator is checked *teacher-forced* from the
 GPU's own inputs to it (the buffers of the neighbouring operators, read back after the step) on
-  * a random sample of elements through the oracle's `*_at` functions (convolution forward, data and filter gradients),
+  * a random sample of elements, plus elements on the seams of the kernels' tiles, through the oracle's `*_at` functions
+    (convolution forward, data and filter gradients),
   * whole sampled planes for the pooling operators, whole tensors for the affine operators (numpy fp64),
   * loss, predicted categories (exact) and accuracy count (exact) from the GPU's own probabilities.
 Gradients are zeroed by the fused update, so they are checked through what the update leaves:
@@ -107,6 +108,18 @@ def sample_idx(rng, total, n):
     return idx
 
 
+def edge_idx(rng, shape, n):
+    """Elements of an NCHW tensor on the seams of the kernels' tiles: channel and column (image * plane + pixel)
+    positions either side of multiples of 32, where an indexing mistake would touch only a few elements."""
+    Nn, K, P, Q = shape
+    inner, cols = P * Q, Nn * P * Q
+    c = 32 * rng.integers(0, (cols + 31) // 32 + 1, n) + rng.integers(-1, 2, n)
+    r = 32 * rng.integers(0, (K + 31) // 32 + 1, n) + rng.integers(-1, 1, n)
+    c = np.clip(c, 0, cols - 1).astype(np.int64)
+    r = np.clip(r, 0, K - 1).astype(np.int64)
+    return (c // inner) * (K * inner) + r * inner + c % inner
+
+
 def read_params(w, layers):
     out = {}
     for i, l in enumerate(layers):
@@ -154,7 +167,7 @@ def check_forward(w, layers, shapes, x, batch, before, log, rng, tag):
         if l[0] == "conv2d":
             K, R = l[5], l[2]
             W_ = before[i]["weights"].reshape(K, shapes[i][0][1], R, R)
-            idx = sample_idx(rng, y.size, 4096)
+            idx = np.concatenate([sample_idx(rng, y.size, 4096), edge_idx(rng, y.shape, 2048)])
             ref = O.conv2d_fwd_at(xin, W_, l[3], l[4], idx).astype(np.float64)
             ref += before[i]["bias"].astype(np.float64)[(idx // (y.shape[2] * y.shape[3])) % K]
             if act_of(l) == "Rect":
@@ -205,7 +218,7 @@ def check_step(w, layers, shapes, x, labels, batch, before, after, log, rng, tag
             K, R, C_ = l[5], l[2], shapes[i][0][1]
             W_ = before[i]["weights"].reshape(K, C_, R, R)
             if i > 0:
-                idx = sample_idx(rng, xin.size, 4096)
+                idx = np.concatenate([sample_idx(rng, xin.size, 4096), edge_idx(rng, tuple(shapes[i][0]), 2048)])
                 ref = O.conv2d_bwd_data_at(W_, dy, shapes[i][0], l[3], l[4], idx)
                 if mask_prev:
                     ref = ref * (acts[i].ravel()[idx] > 0)
