@@ -396,7 +396,10 @@ def other_configs(lib):
                     ("nin_b128_bf16_forward", lambda: short_bf16_forward_leg(lib, "nin", 50, 5)),
                     ("conv_sweep", lambda: conv_sweep_leg(20, 3))):
         t0 = time.perf_counter()
-        out[key] = fn()
+        try:
+            out[key] = fn()
+        except Exception as e:   # a side leg must not cost the headline line
+            out[key] = {"error": "%s: %s" % (type(e).__name__, e)}
         out[key]["leg_seconds"] = time.perf_counter() - t0
     return out
 
@@ -578,7 +581,11 @@ def main():
         worker.close()
         result["other_configs"] = other_configs(lib)
     if args.cpu_sample > 0:
-        result["cpu_baseline"] = cpu_baseline(net, args.cpu_sample)
+        try:
+            result["cpu_baseline"] = cpu_baseline(net, args.cpu_sample)
+        except Exception as e:   # (the oracle library missing or a host without OpenMP: the measured line still prints)
+            result["cpu_baseline"] = {"value": None, "unit": "images/sec", "cores": 0, "kind": "port",
+                                      "sample": "not run: %s: %s" % (type(e).__name__, e)}
     print(json.dumps(result))
 
 
