@@ -289,6 +289,32 @@ int rh_softmax_kl_step(const float* x, int32_t C, int32_t N, const int32_t* labe
                        float* max_out, int32_t* idx_out, float* loss1, float* loss_sum, float* dx, uint32_t* counter,
                        rh_stream_t stream);
 
+/* The classifier tail of a train step in two launches: AffineOperator::forward of two layers (mod.rs:1168-1176; the
+ * first with ReLU or identity, the second with identity), the loss operator's step above (loss.rs:118-240), and the
+ * backward passes of the two layers (mod.rs:1186-1217).  Weights are the reference's column-major (in, out) = [out][in],
+ * activations [sample][channel].
+ *   rh_affine2_softmax_kl_step   h = act(W1 x + b1) (B x H), logits = W2 h + b2 (B x C), then p, max_out, idx_out, loss1,
+ *                                loss_sum, dlogits exactly as rh_softmax_kl_step's p .. dx, and the data gradients
+ *                                dh = [h > 0] * W2^T dlogits (the first layer's delta after its activation's backward)
+ *                                and, where dx is not NULL, dx = W1^T dh.  One block per sample.  `counter` as above.
+ *   rh_affine2_bwd_params        dW1 = dh^T x, db1 = sum_n dh, dW2 = dlogits^T h, db2 = sum_n dlogits, each
+ *                                out = sum + beta * out (beta 0: out is not read).
+ *   rh_affine2_softmax_kl_step_supported   1 where the sizes have this form (a sample's chain in one block's LDS:
+ *                                I <= 4096, H <= 2048, C <= 64, I * H <= 2^17, B * I * H <= 2^26: every block reads the
+ *                                first layer's weights), else both return
+ *                                RH_E_UNSUPPORTED.
+ * Sums are taken in a fixed order that differs from the tiled products': results agree with the separate calls to
+ * rounding, not bit for bit. */
+int rh_affine2_softmax_kl_step_supported(int32_t B, int32_t I, int32_t H, int32_t C);
+int rh_affine2_softmax_kl_step(int32_t B, int32_t I, int32_t H, int32_t C, int32_t relu1, const float* x, const float* w1,
+                               const float* b1, const float* w2, const float* b2, const int32_t* labels,
+                               const float* weights, float* h, float* logits, float* p, float* max_out, int32_t* idx_out,
+                               float* loss1, float* loss_sum, float* dlogits, float* dh, float* dx, uint32_t* counter,
+                               rh_stream_t stream);
+int rh_affine2_bwd_params(int32_t B, int32_t I, int32_t H, int32_t C, const float* x, const float* h, const float* dh,
+                          const float* dlogits, float beta1, float* dw1, float* db1, float beta2, float* dw2, float* db2,
+                          rh_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * SGD.  rh_sgd_momentum_step is the fused form of the BLAS-1 sequence regularize ->
  * accumulate_grads -> update_params -> reset (mod.rs:1178-1218, 1355-1363; driven by

@@ -108,6 +108,13 @@ int rho_config_from_model_file(const char* path, rho_config** out);
  *                           batch-norm average, a step-size schedule at a boundary) run launch by launch as usual;
  *                           results are bit-identical either way. */
 #define RHO_EXEC_GRAPH_STEPS 0x8
+/*   RHO_EXEC_SEPARATE_TAIL  with RHO_EXEC_FUSE_EPILOGUE, rho_sgd_train_batch runs a classifier tail (affine -> affine ->
+ *                           softmax loss, of at most 4096 x 2048 x 64 units and 2^17 first-layer weights) as two launches:
+ *                           both layers' forward, the loss step and the data gradients per sample in one, the four
+ *                           parameter gradients in another (rh_affine2_softmax_kl_step, rh_affine2_bwd_params), ten
+ *                           launches otherwise.  Same buffers with the same meaning; sums in another order, so results
+ *                           agree with the separate operators to rounding.  This flag keeps the separate operators. */
+#define RHO_EXEC_SEPARATE_TAIL 0x10
 int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1,
                    int device, int exec_flags, rho_worker** out);
 int rho_worker_free(rho_worker* w);

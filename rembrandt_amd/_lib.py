@@ -122,6 +122,9 @@ PROTOTYPES = {
     "rembrandt_kernel_batch_blockreduce_sum": (None, [_vp, _i32, _i32, _vp, _f, _vp]),
     "rembrandt_kernel_batch_blockreduce_argmax": (None, [_vp, _i32, _i32, _vp, _vp, _vp]),
     "rh_softmax_kl_step": (_int, [_vp, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "rh_affine2_softmax_kl_step_supported": (_int, [_i32, _i32, _i32, _i32]),
+    "rh_affine2_softmax_kl_step": (_int, [_i32, _i32, _i32, _i32, _i32] + [_vp] * 19),
+    "rh_affine2_bwd_params": (_int, [_i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _f, _vp, _vp, _f, _vp, _vp, _vp]),
     "rh_sgd_momentum_step": (_int, [_i64, _vp, _vp, _vp, _f, _f, _f, _f, _int, _vp]),
     "rh_sgd_momentum_step_multi": (_int, [_i32, C.POINTER(SgdTensor), _f, _f, _f, _int, _vp]),
     "rh_descend": (_int, [_i64, _vp, _vp, _f, _f, _vp]),

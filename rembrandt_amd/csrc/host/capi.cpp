@@ -275,6 +275,7 @@ int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, ui
     opts.bf16_forward = (exec_flags & RHO_EXEC_BF16_FORWARD) != 0;
     opts.overlap_backward = (exec_flags & RHO_EXEC_OVERLAP_BACKWARD) != 0;
     opts.graph_steps = (exec_flags & RHO_EXEC_GRAPH_STEPS) != 0;
+    opts.fuse_tail = (exec_flags & RHO_EXEC_SEPARATE_TAIL) == 0;
     w->graph_steps = opts.graph_steps;
     w->fuse_epilogue = opts.fuse_epilogue;
     w->worker.reset(new SequentialOperatorWorker(cfg->cfg, (size_t)batch_size,
@@ -548,11 +549,12 @@ int rho_sgd_train_batch(rho_sgd* s, rho_worker* w, int32_t batch_size, int fused
     const OpPhase phase = OpPhase::Training(t);
     // With fused epilogues the loss operator produces probabilities, categories, loss and delta in one launch of its
     // forward(); the three calls below that ask for them then launch nothing.
+    // (so does the classifier tail, where the chain ends in one: two launches for its ten)
     struct Armed {
-      LossOperator* l;
-      Armed(LossOperator* l_, bool on) : l(on && l_->arm_train_step(true) ? l_ : nullptr) {}
-      ~Armed() { if (l) l->arm_train_step(false); }
-    } armed(op->loss_operator(0), w->fuse_epilogue);
+      SequentialOperatorWorker* o;
+      Armed(SequentialOperatorWorker* o_, bool on) : o(on && o_->arm_train_step(true) ? o_ : nullptr) {}
+      ~Armed() { if (o) o->arm_train_step(false); }
+    } armed(op, w->fuse_epilogue);
     // forward -> arg-max and loss kernels -> backward -> update are all enqueued before the two read-backs, so
     // the GPU works through the step without waiting for the host (same results as the reference's order:
     // store_output_categories, store_loss, backward; nothing in between writes what they read)

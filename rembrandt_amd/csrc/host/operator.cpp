@@ -773,6 +773,7 @@ class AffineOperator : public Operator {
   const char* kind() const override { return "AffineOperator"; }
 
  private:
+  friend struct ::rembrandt::ClassifierTail;
   void* ws_ptr() { return workspace_ ? workspace_->as_mut_ptr() : nullptr; }
   size_t ws_len() { return workspace_ ? workspace_->len() : 0; }
   size_t batch_cap_;
@@ -1914,6 +1915,7 @@ class SoftmaxKLLossOperator : public LossOperator {
   const char* kind() const override { return "SoftmaxKLLossOperator"; }
 
  private:
+  friend struct ::rembrandt::ClassifierTail;
   size_t batch_cap_;
   CategoricalLossConfig loss_config_;
   Ctx context_;
@@ -1933,6 +1935,69 @@ class SoftmaxKLLossOperator : public LossOperator {
 };
 
 }  // namespace
+
+// ---- the classifier tail of a train step as two launches ---------------------------------------------------
+// AffineOperator (ReLU or identity) -> AffineOperator (identity) -> SoftmaxKLLossOperator, of a size where one block
+// holds a sample's whole chain (rh_affine2_softmax_kl_step_supported).  forward_train stands for the three
+// operators' forward(), the loss operator's enqueue_* and backward(), and the data-gradient halves of the two
+// affine backward() calls; backward_train for their parameter-gradient halves.  Every buffer the operators expose
+// holds what the separate calls leave there (the first layer's delta after its activation's backward).
+struct ClassifierTail {
+  AffineOperator* fc1;
+  AffineOperator* fc2;
+  SoftmaxKLLossOperator* loss;
+  Ctx context;
+
+  static std::shared_ptr<ClassifierTail> detect(std::vector<std::unique_ptr<Operator>>& hidden, LossOperator* loss_op,
+                                                size_t batch_cap, const ExecOptions& opts, Ctx context) {
+    if (!opts.fuse_tail || !opts.fuse_epilogue || hidden.size() < 2) return nullptr;
+    auto* a1 = dynamic_cast<AffineOperator*>(hidden[hidden.size() - 2].get());
+    auto* a2 = dynamic_cast<AffineOperator*>(hidden[hidden.size() - 1].get());
+    auto* l = dynamic_cast<SoftmaxKLLossOperator*>(loss_op);
+    if (!a1 || !a2 || !l || !a1->params_.has_backward() || !a2->params_.has_backward()) return nullptr;
+    if (a2->config_.act_func != ActivationFunction::Identity) return nullptr;
+    if (a1->config_.act_func != ActivationFunction::Identity && a1->config_.act_func != ActivationFunction::Rect) return nullptr;
+    if (a1->config_.out_channels != a2->config_.in_channels || a2->config_.out_channels != l->loss_config_.num_categories)
+      return nullptr;
+    if (!rh_affine2_softmax_kl_step_supported((int)batch_cap, (int)a1->config_.in_channels, (int)a1->config_.out_channels,
+                                              (int)a2->config_.out_channels))
+      return nullptr;
+    std::shared_ptr<ClassifierTail> t(new ClassifierTail());
+    t->fc1 = a1; t->fc2 = a2; t->loss = l; t->context = context;
+    return t;
+  }
+  bool updates_on_second_stream() const { return fc1->updates_on_second_stream() || fc2->updates_on_second_stream(); }
+  void forward_train(size_t batch_size) {
+    RB_ASSERT(batch_size <= fc1->batch_cap_);
+    const int I = (int)fc1->config_.in_channels, H = (int)fc1->config_.out_channels, C = (int)fc2->config_.out_channels;
+    unwrap(rh_affine2_softmax_kl_step(
+               (int)batch_size, I, H, C, fc1->config_.act_func == ActivationFunction::Rect ? 1 : 0, fc1->in_act_->as_ptr(),
+               fc1->params_.weights->as_ptr(), fc1->params_.bias->as_ptr(), fc2->params_.weights->as_ptr(),
+               fc2->params_.bias->as_ptr(), loss->label_cats_.as_ptr(), loss->weights_.as_ptr(), fc1->out_act_->as_mut_ptr(),
+               fc2->out_act_->as_mut_ptr(), loss->out_values_.as_mut_ptr(), loss->max_value_.as_mut_ptr(),
+               loss->out_cats_.as_mut_ptr(), loss->out_loss1_.as_mut_ptr(), loss->out_loss_.as_mut_ptr(),
+               fc2->out_delta_->as_mut_ptr(), fc1->out_delta_->as_mut_ptr(),
+               fc1->in_delta_ ? fc1->in_delta_->as_mut_ptr() : nullptr,
+               reinterpret_cast<uint32_t*>(loss->step_counter_.as_mut_ptr()), context->stream()),
+           "classifier tail (forward, loss, data gradients)");
+    loss->step_valid_ = batch_size;   // categories, loss and delta are there: the loss operator's calls launch nothing
+  }
+  void backward_train(size_t batch_size) {
+    const int I = (int)fc1->config_.in_channels, H = (int)fc1->config_.out_channels, C = (int)fc2->config_.out_channels;
+    rh_stream_t sg = context->stream();
+    if (fc1->overlap_on_ && fc1->in_delta_) {   // as AffineOperator::backward places its parameter gradients
+      context->fork();
+      sg = context->aux_stream();
+    }
+    const float beta2 = fc2->params_.take_backward_beta();
+    const float beta1 = fc1->params_.take_backward_beta();
+    unwrap(rh_affine2_bwd_params((int)batch_size, I, H, C, fc1->in_act_->as_ptr(), fc1->out_act_->as_ptr(),
+                                 fc1->out_delta_->as_ptr(), fc2->out_delta_->as_ptr(), beta1,
+                                 fc1->params_.grad_weights->as_mut_ptr(), fc1->params_.grad_bias->as_mut_ptr(), beta2,
+                                 fc2->params_.grad_weights->as_mut_ptr(), fc2->params_.grad_bias->as_mut_ptr(), sg),
+           "classifier tail (parameter gradients)");
+  }
+};
 
 // ---- SequentialOperatorWorker ---------------------------------------------------------------------------
 SequentialOperatorWorker::SequentialOperatorWorker(const SequentialOperatorConfig& config, size_t batch_size,
@@ -1977,7 +2042,15 @@ SequentialOperatorWorker::SequentialOperatorWorker(const SequentialOperatorConfi
   }
   RB_ASSERT(params_off == config.params_len());  // src/operator/worker.rs:289
   loss_op_.reset(new SoftmaxKLLossOperator(batch_size, config.loss_op.loss, prev, context));
+  if (backward_enabled(capability)) tail_ = ClassifierTail::detect(hidden_ops_, loss_op_.get(), batch_size, opts, context);
   context_->sync();
+}
+
+bool SequentialOperatorWorker::arm_train_step(bool on) {
+  const bool armed = loss_op_->arm_train_step(on);
+  tail_armed_ = on && armed && tail_ != nullptr;
+  if (!on) tail_done_ = 0;
+  return armed;
 }
 
 LossOperator* SequentialOperatorWorker::loss_operator(size_t rank) {
@@ -2002,16 +2075,33 @@ void SequentialOperatorWorker::init_params(const uint64_t shared_seed[2]) {
 }
 void SequentialOperatorWorker::forward(size_t batch_size, OpPhase phase) {
   input_op_->forward(batch_size, phase);
-  for (auto& op : hidden_ops_) {
+  const bool tail = tail_armed_ && phase.training && batch_size > 0;
+  const size_t n = hidden_ops_.size() - (tail ? 2 : 0);
+  for (size_t i = 0; i < n; ++i) {
+    Operator* op = hidden_ops_[i].get();
     if (aux_pending_ && op->updates_on_second_stream()) settle();  // its parameters were updated on the second stream
     op->forward(batch_size, phase);
+  }
+  tail_done_ = 0;
+  if (tail) {
+    if (aux_pending_ && tail_->updates_on_second_stream()) settle();
+    tail_->forward_train(batch_size);
+    tail_done_ = batch_size;
+    return;
   }
   loss_op_->forward(batch_size, phase);
 }
 void SequentialOperatorWorker::backward(size_t batch_size) {
   settle();
-  loss_op_->backward(batch_size);
-  for (auto it = hidden_ops_.rbegin(); it != hidden_ops_.rend(); ++it) (*it)->backward(batch_size);
+  size_t n = hidden_ops_.size();
+  if (tail_armed_ && tail_done_ == batch_size && batch_size > 0) {
+    tail_->backward_train(batch_size);   // the deltas are there since forward(): only the parameter gradients are left
+    n -= 2;
+  } else {
+    loss_op_->backward(batch_size);
+  }
+  tail_done_ = 0;
+  for (size_t i = n; i-- > 0;) hidden_ops_[i]->backward(batch_size);
   context_->join();  // gradients computed on the second stream are complete for whatever the main stream does next
 }
 void SequentialOperatorWorker::regularize(Regularization reg) { settle(); for (auto& op : hidden_ops_) op->regularize(reg); }

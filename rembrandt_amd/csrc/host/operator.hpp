@@ -283,6 +283,11 @@ struct ExecOptions {
   // main one (the bandwidth-bound operand copies of one hide behind the other's contraction); joined at the end
   // of SequentialOperatorWorker::backward.
   bool overlap_backward = true;
+  // A train step's classifier tail (two affine layers in front of the softmax loss, small enough for a sample's chain
+  // to fit one block) as one launch for forward + loss + data gradients and one for the parameter gradients, instead
+  // of ten launches of a few microseconds of work each; only inside armed train steps with fused epilogues.  Same
+  // buffers with the same meaning at every point the operators expose; sums in a different (fixed) order.
+  bool fuse_tail = true;
 };
 
 // ---- Operator trait -------------------------------------------------------------------------------
@@ -438,6 +443,8 @@ class SequentialOperatorConfig {
   SequentialOperatorConfig& softmax_kl_loss(const CategoricalLossConfig& cfg);
 };
 
+struct ClassifierTail;   // (operator.cpp)
+
 class SequentialOperatorWorker : public Operator {
  public:
   SequentialOperatorWorker(const SequentialOperatorConfig& config, size_t batch_size, OpCapability capability,
@@ -480,6 +487,11 @@ class SequentialOperatorWorker : public Operator {
   void settle();
   // After a recording of a step was abandoned half-way: the launches that would have needed the join never ran.
   void forget_pending() { aux_pending_ = false; }
+  // Arms (or disarms) the one-launch forms of a train step: the loss operator's, and the classifier tail's where the
+  // chain ends in one (ExecOptions::fuse_tail).  While armed, forward() in the training phase also leaves the tail's
+  // deltas behind and the following backward() of the same batch size only adds its parameter gradients.
+  bool arm_train_step(bool on);
+  bool has_fused_tail() const { return tail_ != nullptr; }
   const char* kind() const override { return "SequentialOperatorWorker"; }
   void encode_params(std::vector<uint8_t>& blob) override;
   size_t decode_params(const uint8_t* blob, size_t len) override;
@@ -504,6 +516,9 @@ class SequentialOperatorWorker : public Operator {
   std::vector<std::unique_ptr<Operator>> hidden_ops_;
   std::unique_ptr<LossOperator> loss_op_;
   bool aux_pending_ = false;
+  std::shared_ptr<ClassifierTail> tail_;   // set when the chain ends in affine, affine, softmax loss of a fitting size
+  bool tail_armed_ = false;
+  size_t tail_done_ = 0;                   // batch size whose tail the last forward() ran in one launch; 0: none
 };
 
 // ---- SGD policy (src/opt/sgd/mod.rs:20-147) ---------------------------------------------------------

@@ -194,6 +194,257 @@ __global__ __launch_bounds__(256) void softmax_kl_step_kernel(const float* __res
   }
 }
 
+
+// ---- the classifier tail of a train step: two affine layers and the loss in one launch ---------------------------
+// x (B x I) -> h = act(W1 x + b1) (B x H) -> logits = W2 h + b2 (B x C) -> softmax, arg-max, per-sample loss, its sum,
+// the KL delta, and the data gradients back through both layers: dlogits, dh = [h > 0] * W2^T dlogits, dx = W1^T dh.
+// One block per sample: nothing of a sample's chain depends on another sample, so the whole chain is one kernel
+// (the separate operators are eight to ten launches of a few microseconds of work each, on a path that is a chain of
+// dependent launches).  Every block reads all of W1 twice, so this form is for first layers of a few hundred KB.
+// Plain FMA arithmetic, fixed summation orders.  Each phase asks for its weights in batches of 32-64 loads per lane
+// before it uses any (indices past the end are clamped and their products zeroed: no load under a branch), so a phase
+// costs a few memory round trips.  Weights are [out][in] (the reference's column-major (in, out)), activations
+// [sample][channel].  LDS: x row (I), h (H), dh (H), logits / delta (64).
+template <int NT>
+__global__ __launch_bounds__(NT) void affine2_softmax_kl_step_kernel(
+    int B, int I, int H, int C, int relu1, const float* __restrict__ x, const float* __restrict__ w1,
+    const float* __restrict__ b1, const float* __restrict__ w2, const float* __restrict__ b2,
+    const int* __restrict__ labels, const float* __restrict__ weights, float* __restrict__ h_out,
+    float* __restrict__ logits_out, float* __restrict__ p_out, float* __restrict__ max_out, int* __restrict__ idx_out,
+    float* __restrict__ loss1, float* __restrict__ loss_sum, float* __restrict__ dlogits_out, float* __restrict__ dh_out,
+    float* __restrict__ dx_out, unsigned* __restrict__ counter) {
+  extern __shared__ float lds_tail[];
+  float* const xs = lds_tail;          // [I]
+  float* const hs = xs + I;            // [H]
+  float* const dhs = hs + H;           // [H]
+  float* const ls = dhs + H;           // [64] logits, then the delta
+  __shared__ float sm[NT / 64];
+  __shared__ bool last;
+  constexpr int NW = NT / 64;
+  const int n = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < I; i += NT) xs[i] = x[(size_t)n * I + i];
+  __syncthreads();
+  // h: a wave per group of four outputs, lanes along the input, 16 x 4 weights per lane in flight
+  for (int j0 = wave * 4; j0 < H; j0 += NW * 4) {
+    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const float* r[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) r[k] = w1 + (size_t)(j0 + k < H ? j0 + k : H - 1) * I;
+    for (int i0 = 0; i0 < I; i0 += 1024) {
+      float wv[4][16], xv[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int i = i0 + u * 64 + lane, ii = i < I ? i : I - 1;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) wv[k][u] = r[k][ii];
+        xv[u] = i < I ? xs[ii] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) a[k] = fmaf(wv[k][u], xv[u], a[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      for (int o = 32; o > 0; o >>= 1) a[k] += __shfl_xor(a[k], o, 64);
+    if (lane < 4 && j0 + lane < H) {
+      float v = (lane == 0 ? a[0] : lane == 1 ? a[1] : lane == 2 ? a[2] : a[3]) + b1[j0 + lane];
+      if (relu1) v = v > 0.0f ? v : 0.0f;
+      hs[j0 + lane] = v;
+      h_out[(size_t)n * H + j0 + lane] = v;
+    }
+  }
+  __syncthreads();
+  // logits: a wave per class, lanes along h, 16 weights per lane in flight
+  for (int c = wave; c < C; c += NW) {
+    float a = 0.0f;
+    const float* r = w2 + (size_t)c * H;
+    for (int j0 = 0; j0 < H; j0 += 1024) {
+      float wv[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int j = j0 + u * 64 + lane;
+        wv[u] = r[j < H ? j : H - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int j = j0 + u * 64 + lane;
+        a = fmaf(wv[u], j < H ? hs[j] : 0.0f, a);
+      }
+    }
+    for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o, 64);
+    if (lane == 0) {
+      a += b2[c];
+      ls[c] = a;
+      logits_out[(size_t)n * C + c] = a;
+    }
+  }
+  __syncthreads();
+  // softmax, arg-max (first maximum), loss and delta: the first wave, a lane per class (C <= 64)
+  if (wave == 0) {
+    const float v = lane < C ? ls[lane] : -INFINITY;
+    float mx = v;
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    const float e = lane < C ? expf(v - mx) : 0.0f;
+    float z = e;
+    for (int o = 32; o > 0; o >>= 1) z += __shfl_xor(z, o, 64);
+    float pv = e * (1.0f / z);
+    asm volatile("" : "+v"(pv));   // the rounded product is what is stored and what the delta is formed from
+    const int label = labels[n];
+    const float wgt = weights[n];
+    float best = lane < C ? pv : -INFINITY;
+    int bi = lane < C ? lane : 0x7fffffff;
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
+    }
+    const float d = wgt * (pv - (lane == label ? 1.0f : 0.0f));
+    if (lane < C) {
+      p_out[(size_t)n * C + lane] = pv;
+      dlogits_out[(size_t)n * C + lane] = d;
+      if (lane == label) loss1[n] = -wgt * logf(pv);
+      ls[lane] = d;
+    }
+    if (lane == 0) {
+      if ((unsigned)label >= (unsigned)C) loss1[n] = NAN;
+      max_out[n] = best;
+      idx_out[n] = bi == 0x7fffffff ? 0 : bi;
+    }
+  }
+  __syncthreads();
+  // dh = [h > 0] * W2^T delta: a thread per hidden unit, 16 classes' weights in flight
+  for (int j = tid; j < H; j += NT) {
+    float a = 0.0f;
+    for (int c0 = 0; c0 < C; c0 += 16) {
+      float wv[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) wv[u] = w2[(size_t)(c0 + u < C ? c0 + u : C - 1) * H + j];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) a = fmaf(wv[u], c0 + u < C ? ls[c0 + u] : 0.0f, a);
+    }
+    if (relu1 && !(hs[j] > 0.0f)) a = 0.0f;
+    dhs[j] = a;
+    dh_out[(size_t)n * H + j] = a;
+  }
+  __syncthreads();
+  // dx = W1^T dh: a thread per input element (rows of W1 read along the lanes), 32 rows' weights in flight
+  if (dx_out) {
+    for (int i = tid; i < I; i += NT) {
+      float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+      for (int j0 = 0; j0 < H; j0 += 32) {
+        float wv[32];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) wv[u] = w1[(size_t)(j0 + u < H ? j0 + u : H - 1) * I + i];
+#pragma unroll
+        for (int u = 0; u < 32; u += 4) {
+          a0 = fmaf(wv[u], j0 + u < H ? dhs[j0 + u] : 0.0f, a0);
+          a1 = fmaf(wv[u + 1], j0 + u + 1 < H ? dhs[j0 + u + 1] : 0.0f, a1);
+          a2 = fmaf(wv[u + 2], j0 + u + 2 < H ? dhs[j0 + u + 2] : 0.0f, a2);
+          a3 = fmaf(wv[u + 3], j0 + u + 3 < H ? dhs[j0 + u + 3] : 0.0f, a3);
+        }
+      }
+      dx_out[(size_t)n * I + i] = (a0 + a1) + (a2 + a3);
+    }
+  }
+  // The sum of the per-sample losses, by the block that finishes last (it leaves the counter at zero again).  What
+  // that block reads of the others is loss1, written by the thread that counts its block below (its own wave wrote
+  // it): the release is part of its atomic, once per block.  (A device-scope fence in every wave of every block
+  // writes back and invalidates an XCD's whole L2 sixteen times per block: 40 us of a 50 us kernel.)
+  __syncthreads();
+  if (tid == 0) last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)B - 1u;
+  __syncthreads();
+  if (!last) return;
+  if (wave == 0) __threadfence();
+  __syncthreads();
+  float acc = 0.0f;
+  for (int i = tid; i < B; i += NT) acc += __hip_atomic_load(loss1 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  acc = block_reduce_sum(acc, sm);
+  if (tid == 0) {
+    loss_sum[0] = acc;
+    *counter = 0u;
+  }
+}
+
+// The parameter gradients of the same two layers in one launch: dW1[j][i] = sum_n dh[n][j] x[n][i], db1[j] = sum_n dh[n][j],
+// dW2[c][j] = sum_n dlogits[n][c] h[n][j], db2[c] = sum_n dlogits[n][c]; out = sum + beta * old (beta 0: old is not read).
+// A block of 256 threads takes 32 result items (four consecutive i of dW1 where I is a multiple of four, else one
+// element) and cuts the batch into eight slices, one per group of 32 threads: every thread adds its slice's samples
+// (16 of them in flight at a time), the slices' sums meet in LDS and are added in slice order.
+__global__ __launch_bounds__(256) void affine2_bwd_params_kernel(int B, int I, int H, int C, int vec, const float* __restrict__ x,
+                                                                 const float* __restrict__ h, const float* __restrict__ dh,
+                                                                 const float* __restrict__ dl, float beta1, float* __restrict__ dw1,
+                                                                 float* __restrict__ db1, float beta2, float* __restrict__ dw2,
+                                                                 float* __restrict__ db2, unsigned n1, unsigned n2, unsigned n3) {
+  __shared__ float4 part[8][32];
+  const int t = threadIdx.x & 31, s = threadIdx.x >> 5;
+  const unsigned idx = blockIdx.x * 32u + (unsigned)t, total = n1 + n2 + n3;
+  const int per = (B + 7) / 8, nb = s * per, ne = nb + per < B ? nb + per : B;
+  // what this item multiplies: a[n * sa + oa] * b[n * sb + ob .. +3] (a scalar of the delta, a run of the activation)
+  const float* pa = dh;
+  const float* pb = x;
+  size_t sa = 0, sb = 0, oa = 0, ob = 0;
+  int kind = -1;   // 0: dW1 (four wide), 1: dW1 (one), 2: dW2, 3: db1, 4: db2
+  if (idx < n1) {
+    if (vec) {
+      const unsigned I4 = (unsigned)I >> 2, j = idx / I4, i4 = idx - j * I4;
+      kind = 0; sa = H; oa = j; sb = I; ob = 4 * (size_t)i4;
+    } else {
+      const unsigned j = idx / (unsigned)I, i = idx - j * (unsigned)I;
+      kind = 1; sa = H; oa = j; sb = I; ob = i;
+    }
+  } else if (idx < n1 + n2) {
+    const unsigned k = idx - n1, c = k / (unsigned)H, j = k - c * (unsigned)H;
+    kind = 2; pa = dl; sa = C; oa = c; pb = h; sb = H; ob = j;
+  } else if (idx < total) {
+    const unsigned k = idx - n1 - n2;
+    if (k < (unsigned)H) { kind = 3; sa = H; oa = k; }
+    else { kind = 4; pa = dl; sa = C; oa = k - (unsigned)H; }
+  }
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  if (kind >= 0) {
+    for (int n0 = nb; n0 < ne; n0 += 16) {
+      float av[16];
+      float4 bv[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int n = n0 + u < ne ? n0 + u : ne - 1;
+        av[u] = pa[(size_t)n * sa + oa];
+        if (kind == 0) bv[u] = *reinterpret_cast<const float4*>(pb + (size_t)n * sb + ob);
+        else if (kind <= 2) bv[u] = make_float4(pb[(size_t)n * sb + ob], 0.0f, 0.0f, 0.0f);
+        else bv[u] = make_float4(1.0f, 0.0f, 0.0f, 0.0f);
+        if (n0 + u >= ne) av[u] = 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        acc.x = fmaf(av[u], bv[u].x, acc.x); acc.y = fmaf(av[u], bv[u].y, acc.y);
+        acc.z = fmaf(av[u], bv[u].z, acc.z); acc.w = fmaf(av[u], bv[u].w, acc.w);
+      }
+    }
+  }
+  part[s][t] = acc;
+  __syncthreads();
+  if (s != 0 || kind < 0) return;
+  float4 r = part[0][t];
+#pragma unroll
+  for (int k = 1; k < 8; ++k) {
+    const float4 v = part[k][t];
+    r.x += v.x; r.y += v.y; r.z += v.z; r.w += v.w;
+  }
+  if (kind == 0) {
+    float4* o = reinterpret_cast<float4*>(dw1 + oa * (size_t)I + ob);
+    if (beta1 != 0.0f) {
+      const float4 old = *o;
+      r.x = fmaf(beta1, old.x, r.x); r.y = fmaf(beta1, old.y, r.y); r.z = fmaf(beta1, old.z, r.z); r.w = fmaf(beta1, old.w, r.w);
+    }
+    *o = r;
+    return;
+  }
+  float* o = kind == 1 ? dw1 + oa * (size_t)I + ob : kind == 2 ? dw2 + oa * (size_t)H + ob : kind == 3 ? db1 + oa : db2 + oa;
+  const float beta = kind == 1 || kind == 3 ? beta1 : beta2;
+  *o = beta != 0.0f ? fmaf(beta, *o, r.x) : r.x;
+}
+
 }  // namespace rh
 
 using namespace rh;
@@ -259,3 +510,49 @@ extern "C" int rh_softmax_kl_step(const float* x, int32_t C, int32_t N, const in
                      p, max_out, idx_out, loss1, loss_sum, dx, counter);
   return launch_status();
 }
+
+// The classifier tail is taken as one kernel per direction where a sample's chain fits a block's LDS and every block can
+// afford to read the whole first layer (twice): up to 4096 inputs, 2048 hidden units, 64 classes, 2^17 weights (512 KB)
+// in the first layer and 2^26 multiply-adds in its products over the batch.  Beyond that the tiled products, which read
+// the weights once, are the faster form.
+extern "C" int rh_affine2_softmax_kl_step_supported(int32_t B, int32_t I, int32_t H, int32_t C) {
+  return B > 0 && I > 0 && H > 0 && C > 0 && I <= 4096 && H <= 2048 && C <= 64 && (long long)I * H <= (1ll << 17) &&
+                 (long long)B * I * H <= (1ll << 26)
+             ? 1 : 0;
+}
+
+extern "C" int rh_affine2_softmax_kl_step(int32_t B, int32_t I, int32_t H, int32_t C, int32_t relu1, const float* x,
+                                          const float* w1, const float* b1, const float* w2, const float* b2,
+                                          const int32_t* labels, const float* weights, float* h, float* logits, float* p,
+                                          float* max_out, int32_t* idx_out, float* loss1, float* loss_sum, float* dlogits,
+                                          float* dh, float* dx, uint32_t* counter, rh_stream_t stream) {
+  if (B < 0 || I <= 0 || H <= 0 || C <= 0) return RH_E_INVALID;
+  if (B == 0) return 0;
+  if (!rh_affine2_softmax_kl_step_supported(B, I, H, C)) return RH_E_UNSUPPORTED;
+  if (!x || !w1 || !b1 || !w2 || !b2 || !labels || !weights || !h || !logits || !p || !max_out || !idx_out || !loss1 ||
+      !loss_sum || !dlogits || !dh || !counter)
+    return RH_E_INVALID;
+  constexpr int NT = 1024;
+  const size_t lds = sizeof(float) * ((size_t)I + 2 * (size_t)H + 64);
+  ProfScope prof("affine2_softmax_kl_step",
+                 4.0 * ((double)B * (2.0 * I + 3.0 * H + 4.0 * C) + 2.0 * ((double)I * H + (double)H * C)), to_stream(stream));
+  hipLaunchKernelGGL((affine2_softmax_kl_step_kernel<NT>), dim3(B), dim3(NT), lds, to_stream(stream), B, I, H, C, relu1 ? 1 : 0,
+                     x, w1, b1, w2, b2, labels, weights, h, logits, p, max_out, idx_out, loss1, loss_sum, dlogits, dh, dx, counter);
+  return launch_status();
+}
+
+extern "C" int rh_affine2_bwd_params(int32_t B, int32_t I, int32_t H, int32_t C, const float* x, const float* h, const float* dh,
+                                     const float* dlogits, float beta1, float* dw1, float* db1, float beta2, float* dw2,
+                                     float* db2, rh_stream_t stream) {
+  if (B < 0 || I <= 0 || H <= 0 || C <= 0) return RH_E_INVALID;
+  if (!rh_affine2_softmax_kl_step_supported(B > 0 ? B : 1, I, H, C)) return RH_E_UNSUPPORTED;
+  if (!x || !h || !dh || !dlogits || !dw1 || !db1 || !dw2 || !db2) return RH_E_INVALID;
+  const int vec = I % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dw1)) & 15) == 0 ? 1 : 0;
+  const unsigned n1 = (unsigned)((size_t)H * I / (vec ? 4 : 1)), n2 = (unsigned)((size_t)C * H), n3 = (unsigned)(H + C);
+  const size_t total = (size_t)n1 + n2 + n3;
+  ProfScope prof("affine2_bwd_params", 4.0 * ((double)B * (I + 2.0 * H + C) + (double)I * H + (double)H * C), to_stream(stream));
+  hipLaunchKernelGGL(affine2_bwd_params_kernel, dim3((unsigned)cdiv<size_t>(total, 32)), dim3(256), 0, to_stream(stream), B, I, H,
+                     C, vec, x, h, dh, dlogits, beta1, dw1, db1, beta2, dw2, db2, n1, n2, n3);
+  return launch_status();
+}
+

@@ -339,6 +339,37 @@ def softmax_kl_step(x, labels, weights, counter=None):
     return p, mx, idx, loss1, total, dx, counter
 
 
+def affine2_softmax_kl_step_supported(B, I, H, Cc):
+    return bool(lib().rh_affine2_softmax_kl_step_supported(B, I, H, Cc))
+
+
+def affine2_softmax_kl_step(x, w1, b1, w2, b2, labels, weights, relu1=True, want_dx=True, counter=None):
+    """Two affine layers, the loss step and their data gradients in one launch (rh_affine2_softmax_kl_step).
+    x: (B, I); w1: (H, I); w2: (C, H).  Returns a dict of every tensor the launch writes."""
+    B, I = x.shape
+    H, Cc = w1.shape[0], w2.shape[0]
+    f = lambda *shape: torch.empty(shape, dtype=torch.float32, device=x.device)
+    out = {"h": f(B, H), "logits": f(B, Cc), "p": f(B, Cc), "max": f(B), "idx": torch.empty((B,), dtype=torch.int32, device=x.device),
+           "loss1": f(B), "loss": f(1), "dlogits": f(B, Cc), "dh": f(B, H), "dx": f(B, I) if want_dx else None}
+    if counter is None:
+        counter = torch.zeros((1,), dtype=torch.int32, device=x.device)
+    out["counter"] = counter
+    check(lib().rh_affine2_softmax_kl_step(B, I, H, Cc, int(relu1), _p(x), _p(w1), _p(b1), _p(w2), _p(b2), _p(labels),
+                                           _p(weights), _p(out["h"]), _p(out["logits"]), _p(out["p"]), _p(out["max"]),
+                                           _p(out["idx"]), _p(out["loss1"]), _p(out["loss"]), _p(out["dlogits"]), _p(out["dh"]),
+                                           _p(out["dx"]) if want_dx else None, _p(counter), _stream()),
+          "rh_affine2_softmax_kl_step")
+    return out
+
+
+def affine2_bwd_params(x, h, dh, dlogits, dw1, db1, dw2, db2, beta1=0.0, beta2=0.0):
+    """dW1, db1, dW2, db2 of the two layers in one launch (rh_affine2_bwd_params); out = sum + beta * out."""
+    B, I = x.shape
+    H, Cc = h.shape[1], dlogits.shape[1]
+    check(lib().rh_affine2_bwd_params(B, I, H, Cc, _p(x), _p(h), _p(dh), _p(dlogits), beta1, _p(dw1), _p(db1), beta2, _p(dw2),
+                                      _p(db2), _stream()), "rh_affine2_bwd_params")
+
+
 def sgd_momentum_step(W, g, v, l2, scale, mu, apply, zero_grad=True):
     check(lib().rh_sgd_momentum_step(W.numel(), _p(W), _p(g), _p(v), l2, scale, mu, apply, int(zero_grad),
                                      _stream()), "rh_sgd_momentum_step")

@@ -158,6 +158,17 @@ extern "C" {
   pub fn rh_softmax_kl_step(x: *const f32, c: i32, n: i32, labels: *const i32, weights: *const f32, p: *mut f32,
                             max_out: *mut f32, idx_out: *mut i32, loss1: *mut f32, loss_sum: *mut f32, dx: *mut f32,
                             counter: *mut u32, stream: rh_stream_t) -> c_int;
+  // The classifier tail of a train step (two affine layers, the loss step, their data gradients) and its parameter
+  // gradients, one launch each.
+  pub fn rh_affine2_softmax_kl_step_supported(b: i32, i: i32, h: i32, c: i32) -> c_int;
+  pub fn rh_affine2_softmax_kl_step(b: i32, i: i32, h: i32, c: i32, relu1: i32, x: *const f32, w1: *const f32, b1: *const f32,
+                                    w2: *const f32, b2: *const f32, labels: *const i32, weights: *const f32, h_out: *mut f32,
+                                    logits: *mut f32, p: *mut f32, max_out: *mut f32, idx_out: *mut i32, loss1: *mut f32,
+                                    loss_sum: *mut f32, dlogits: *mut f32, dh: *mut f32, dx: *mut f32, counter: *mut u32,
+                                    stream: rh_stream_t) -> c_int;
+  pub fn rh_affine2_bwd_params(b: i32, i: i32, h: i32, c: i32, x: *const f32, h_act: *const f32, dh: *const f32,
+                               dlogits: *const f32, beta1: c_float, dw1: *mut f32, db1: *mut f32, beta2: c_float,
+                               dw2: *mut f32, db2: *mut f32, stream: rh_stream_t) -> c_int;
   // Host generator behind init_params (the reference's random stream lives in crates outside its tree).
   pub fn rh_rng_fill_uniform(seed: u64, stream_id: u64, host: *mut f32, n: size_t, lo: c_float, hi: c_float) -> c_int;
   pub fn rh_rng_fill_normal(seed: u64, stream_id: u64, host: *mut f32, n: size_t, mean: c_float, std: c_float) -> c_int;

@@ -499,6 +499,94 @@ def test_softmax_kl_step_equals_separate_calls(dev, shape):
         assert np.array_equal(N(idx), O.blockreduce_argmax(N(p))[1])
 
 
+AFFINE2_CASES = [
+    # B, I, H, C, relu
+    (64, 800, 160, 10, True),     # a LeNet-like classifier of 2^17 weights
+    (128, 1024, 64, 10, True),    # the CIFAR-10 network's
+    (1, 7, 5, 3, False),
+    (5, 33, 130, 64, True),       # ragged wave groups, the widest class count
+    (37, 1022, 1, 2, False),      # odd input count: the element-wise weight-gradient form
+    (256, 4096, 32, 17, True),    # the widest input the form takes
+]
+
+
+@pytest.mark.parametrize("case", AFFINE2_CASES)
+def test_affine2_softmax_kl_step(dev, case):
+    """The classifier tail in two launches against the oracle's separate operators: two affine layers, softmax,
+    arg-max, loss, KL delta, the data gradients of both layers, then all four parameter gradients (beta 0 and 1);
+    two calls in a row on one counter word."""
+    B, I, H, Cc, relu = case
+    assert ops.affine2_softmax_kl_step_supported(B, I, H, Cc)
+    counter = None
+    for rep in range(2):
+        say("affine2_softmax_kl_step", case, "call", rep)
+        x = synth.normal(41, 10 * rep + 1, (B, I))
+        w1 = synth.normal(41, 10 * rep + 2, (H, I), 0.0, 1.0 / np.sqrt(I))
+        b1 = synth.normal(41, 10 * rep + 3, (H,), 0.0, 0.5)
+        w2 = synth.normal(41, 10 * rep + 4, (Cc, H), 0.0, 1.0 / np.sqrt(H))
+        b2 = synth.normal(41, 10 * rep + 5, (Cc,), 0.0, 0.5)
+        labels = synth.integers(41, 10 * rep + 6, (B,), Cc)
+        weights = synth.uniform(41, 10 * rep + 7, (B,), 0.1, 1.0)
+        # the oracle's operators, one after the other (column-major products as AffineOperator issues them)
+        h = O.sgemm(1, 0, H, B, I, 1.0, w1, I, x, I, 0.0, np.zeros((B, H), np.float32), H) + b1
+        if relu:
+            h = np.maximum(h, 0.0).astype(np.float32)
+        logits = O.sgemm(1, 0, Cc, B, H, 1.0, w2, H, h, H, 0.0, np.zeros((B, Cc), np.float32), Cc) + b2
+        p = O.softmax_fwd(logits)
+        dl = O.softmax_kl_backward(p, labels, weights)
+        l1 = O.softmax_kl_loss1(p, labels, weights)
+        dh = O.sgemm(0, 0, H, B, Cc, 1.0, w2, H, dl, Cc, 0.0, np.zeros((B, H), np.float32), H)
+        if relu:
+            dh = dh * (h > 0)
+        dx = O.sgemm(0, 0, I, B, H, 1.0, w1, I, dh, H, 0.0, np.zeros((B, I), np.float32), I)
+        out = ops.affine2_softmax_kl_step(T(x, dev), T(w1, dev), T(b1, dev), T(w2, dev), T(b2, dev), T(labels, dev), T(weights, dev),
+                                          relu1=relu, want_dx=(rep == 0), counter=counter)
+        counter = out["counter"]
+        assert int(N(counter)[0]) == 0
+        assert_close(N(out["h"]), h, "affine2 h")
+        assert_close(N(out["logits"]), logits, "affine2 logits")
+        assert_close(N(out["p"]), p, "affine2 softmax", atol=1e-6)
+        assert np.array_equal(N(out["idx"]), O.blockreduce_argmax(N(out["p"]))[1]), "affine2 arg-max of its own probabilities"
+        assert np.array_equal(N(out["max"]), N(out["p"]).max(axis=1))
+        assert_close(N(out["loss1"]), l1, "affine2 loss1")
+        assert_close(N(out["loss"]), np.array([l1.astype(np.float64).sum()], np.float32), "affine2 loss sum")
+        assert_close(N(out["dlogits"]), dl, "affine2 dlogits")
+        # the hidden delta is masked by the GPU's own h (an h within rounding of 0 may differ in sign from the oracle's)
+        dh_gpu_mask = O.sgemm(0, 0, H, B, Cc, 1.0, w2, H, N(out["dlogits"]), Cc, 0.0, np.zeros((B, H), np.float32), H)
+        if relu:
+            dh_gpu_mask = dh_gpu_mask * (N(out["h"]) > 0)
+        assert_close(N(out["dh"]), dh_gpu_mask, "affine2 dh")
+        if rep == 0:
+            dx_ref = O.sgemm(0, 0, I, B, H, 1.0, w1, I, N(out["dh"]), H, 0.0, np.zeros((B, I), np.float32), I)
+            assert_close(N(out["dx"]), dx_ref, "affine2 dx")
+            if not relu:
+                assert_close(N(out["dx"]), dx, "affine2 dx (oracle chain)")
+        # parameter gradients from the GPU's own activations and deltas
+        hh, dhh, dll = N(out["h"]), N(out["dh"]), N(out["dlogits"])
+        for beta1, beta2 in ((0.0, 0.0), (1.0, 1.0), (0.5, 0.0)):
+            dw1_0, db1_0 = synth.normal(41, 10 * rep + 8, (H, I)), synth.normal(41, 10 * rep + 9, (H,))
+            dw2_0, db2_0 = synth.normal(41, 10 * rep + 10, (Cc, H)), synth.normal(41, 10 * rep + 11, (Cc,))
+            dw1, db1, dw2, db2 = T(dw1_0, dev), T(db1_0, dev), T(dw2_0, dev), T(db2_0, dev)
+            ops.affine2_bwd_params(T(x, dev), out["h"], out["dh"], out["dlogits"], dw1, db1, dw2, db2, beta1, beta2)
+            r1 = O.sgemm(0, 1, I, H, B, 1.0, x, I, dhh, H, beta1, dw1_0.copy(), I)
+            r2 = O.sgemm(0, 1, H, Cc, B, 1.0, hh, H, dll, Cc, beta2, dw2_0.copy(), H)
+            assert_close(N(dw1), r1, "affine2 dW1 beta %g" % beta1)
+            assert_close(N(dw2), r2, "affine2 dW2 beta %g" % beta2)
+            assert_close(N(db1), (dhh.astype(np.float64).sum(axis=0) + beta1 * db1_0).astype(np.float32), "affine2 db1 beta %g" % beta1)
+            assert_close(N(db2), (dll.astype(np.float64).sum(axis=0) + beta2 * db2_0).astype(np.float32), "affine2 db2 beta %g" % beta2)
+
+
+def test_affine2_softmax_kl_step_limits(dev):
+    assert not ops.affine2_softmax_kl_step_supported(64, 4097, 10, 10)
+    assert not ops.affine2_softmax_kl_step_supported(64, 2450, 500, 10)     # more than 2^17 weights in the first layer
+    assert not ops.affine2_softmax_kl_step_supported(1024, 4096, 32, 10)    # more than 2^26 multiply-adds over the batch
+    assert not ops.affine2_softmax_kl_step_supported(64, 100, 100, 65)
+    x = torch.zeros((2, 8), device=dev)
+    z = lambda *s: torch.zeros(s, device=dev)
+    rc = _lib.lib().rh_affine2_softmax_kl_step(2, 8, 4, 65, 1, *([x.data_ptr()] * 19), None)
+    assert rc == _lib.RH_E_UNSUPPORTED
+
+
 def test_argmax_ties(dev):
     x = np.zeros((4, 700), np.float32)
     x[0, [5, 300, 699]] = 2.0

@@ -24,9 +24,10 @@ def param_buffers(net, read_grads=True):
     return names
 
 
-def run(net, batch, steps, graph, seed, sgd_kwargs, fused=True, toggle_at=None, read_grads=True):
+def run(net, batch, steps, graph, seed, sgd_kwargs, fused=True, toggle_at=None, read_grads=True, fuse_tail=True, extra=()):
     dims, layers, ncat = net
-    w = SequentialOperatorWorker(configs.build_config(net), batch, "Backward", shared_seed=(seed, seed + 1), graph_steps=graph)
+    w = SequentialOperatorWorker(configs.build_config(net), batch, "Backward", shared_seed=(seed, seed + 1), graph_steps=graph,
+                                 fuse_tail=fuse_tail)
     w.init_params()
     sgd = SgdOpt(batch, **sgd_kwargs)
     sgd.begin(w)
@@ -41,7 +42,7 @@ def run(net, batch, steps, graph, seed, sgd_kwargs, fused=True, toggle_at=None, 
         w.stage_batch(labels, 1.0 / batch)
         loss, correct = sgd.train_batch(w, batch, fused=fused)
         # work outside the recording between two replays: blocking read-backs of every parameter buffer
-        out.append((loss, correct, [w.read(i, b).copy() for (i, b) in names]))
+        out.append((loss, correct, [w.read(i, b).copy() for (i, b) in names] + [w.read(i, b).copy() for (i, b) in extra]))
     launches = w.graph_launches()
     assert sgd.iter_counter() == steps
     w.close()
@@ -179,3 +180,49 @@ def test_schedule_that_never_repeats_a_step_size_is_launched(dev):
     graph, n = run(net, 4, 100, True, 0x6A07, kw)
     assert n == 0
     same(eager, graph, "inverse schedule")
+
+
+TAIL_DIMS = (12, 12, 3)
+
+
+def tail_net(fc1_act):
+    return (TAIL_DIMS, *configs._chain(TAIL_DIMS, [("conv", 3, 1, 1, 8, "Rect"), ("pool", 2, 2, 0, "Max"), ("fc", 70, fc1_act),
+                                                   ("fc", 5, "Identity")]))
+
+
+@pytest.mark.parametrize("name,batch,steps", [("cifar10", 128, 4), ("tail_rect", 7, 3), ("tail_identity", 33, 3)])
+def test_classifier_tail_in_two_launches(dev, name, batch, steps):
+    """Train steps whose classifier tail (affine, affine, softmax loss) runs as two launches against the same steps
+    through the separate operators: same losses, correct counts, parameters, momentum, and the same activations and
+    deltas in the buffers the tail's operators expose, to rounding (the two forms add in different orders); and the
+    two-launch form did run."""
+    import ctypes as C
+    from rembrandt_amd import _lib
+    from conftest import assert_close
+    say("classifier tail", name, batch)
+    net = configs.NETWORKS[name]() if name in configs.NETWORKS else tail_net("Rect" if name == "tail_rect" else "Identity")
+    layers = net[1]
+    fc = [i for i, l in enumerate(layers) if l[0] == "affine"]
+    assert len(fc) >= 2 and fc[-1] == len(layers) - 1 and fc[-2] == len(layers) - 2
+    extra = [(fc[-2], "out_act"), (fc[-2], "out_delta"), (fc[-1], "out_act"), (fc[-1], "out_delta"), (fc[-2] - 1, "out_delta")]
+    kw = dict(step_size=0.01, momentum=("Update", 0.9), l2_reg_coef=5e-4)
+    lib = _lib.lib()
+    lib.rh_profile_reset(); lib.rh_profile_filter(None); lib.rh_profile_enable(1)
+    try:
+        fusedrun, _ = run(net, batch, steps, False, 0x7A11, kw, fuse_tail=True, extra=extra)
+        n = lib.rh_profile_count()
+        tag, work, ms = C.c_char_p(), C.c_double(), C.c_float()
+        tags = []
+        for i in range(n):
+            lib.rh_profile_get(i, C.byref(tag), C.byref(work), C.byref(ms))
+            tags.append(tag.value.decode())
+    finally:
+        lib.rh_profile_enable(0)
+    assert tags.count("affine2_softmax_kl_step") == steps and tags.count("affine2_bwd_params") == steps, "the two-launch tail ran"
+    assert "softmax_kl_step" not in tags and "sgemm_skinny" not in tags
+    plain, _ = run(net, batch, steps, False, 0x7A11, kw, fuse_tail=False, extra=extra)
+    for step, ((la, ca, pa), (lb, cb, pb)) in enumerate(zip(fusedrun, plain)):
+        assert abs(la - lb) <= 1e-5 * max(1.0, abs(lb)), (step, la, lb)
+        assert ca == cb, (step, ca, cb)
+        for k, (u, v) in enumerate(zip(pa, pb)):
+            assert_close(u, v, "%s step %d buffer %d" % (name, step, k))
