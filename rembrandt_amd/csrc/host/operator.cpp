@@ -718,7 +718,9 @@ class AffineOperator : public Operator {
     RB_ASSERT(batch_size <= batch_cap_);
     const int i = (int)config_.in_channels, o = (int)config_.out_channels, b = (int)batch_size;
     rh_stream_t s = context_->stream();
-    apply_rect_backprop(config_.act_func, out_act_->as_ptr(), config_.out_channels, batch_size, out_delta_->as_mut_ptr(), s);
+    if (!delta_masked_once_)
+      apply_rect_backprop(config_.act_func, out_act_->as_ptr(), config_.out_channels, batch_size, out_delta_->as_mut_ptr(), s);
+    delta_masked_once_ = false;
     // The two parameter gradients go to the second stream when a data gradient follows on the main stream (scratch
     // of their own there); the worker joins at the end of backward.
     rh_stream_t sg = s;
@@ -784,6 +786,7 @@ class AffineOperator : public Operator {
   ParamTensors params_;
   std::unique_ptr<DeviceBuffer<uint8_t>> workspace_, workspace_aux_;
   bool overlap_built_, overlap_on_;  // parameter gradients and the fused SGD step of this block on the second stream
+  bool delta_masked_once_ = false;   // out_delta_ already went through the activation's backward (the classifier tail)
 };
 
 // ---- Conv2dOperator -------------------------------------------------------------------------------------
@@ -1942,11 +1945,15 @@ class SoftmaxKLLossOperator : public LossOperator {
 // operators' forward(), the loss operator's enqueue_* and backward(), and the data-gradient halves of the two
 // affine backward() calls; backward_train for their parameter-gradient halves.  Every buffer the operators expose
 // holds what the separate calls leave there (the first layer's delta after its activation's backward).
+// A first layer too large for that (LeNet's 2450 x 500) keeps its three tiled products: from_h, where the fused
+// kernels start from its output and stand for the second layer and the loss only.
 struct ClassifierTail {
   AffineOperator* fc1;
   AffineOperator* fc2;
   SoftmaxKLLossOperator* loss;
   Ctx context;
+  bool from_h = false;
+  size_t replaced() const { return from_h ? 1 : 2; }   // hidden operators, counted from the end, whose calls it stands for
 
   static std::shared_ptr<ClassifierTail> detect(std::vector<std::unique_ptr<Operator>>& hidden, LossOperator* loss_op,
                                                 size_t batch_cap, const ExecOptions& opts, Ctx context) {
@@ -1959,39 +1966,43 @@ struct ClassifierTail {
     if (a1->config_.act_func != ActivationFunction::Identity && a1->config_.act_func != ActivationFunction::Rect) return nullptr;
     if (a1->config_.out_channels != a2->config_.in_channels || a2->config_.out_channels != l->loss_config_.num_categories)
       return nullptr;
-    if (!rh_affine2_softmax_kl_step_supported((int)batch_cap, (int)a1->config_.in_channels, (int)a1->config_.out_channels,
-                                              (int)a2->config_.out_channels))
-      return nullptr;
+    const int H = (int)a1->config_.out_channels, C = (int)a2->config_.out_channels;
+    const bool whole = rh_affine2_softmax_kl_step_supported((int)batch_cap, (int)a1->config_.in_channels, H, C) != 0;
+    if (!whole && !rh_affine2_softmax_kl_step_supported((int)batch_cap, 0, H, C)) return nullptr;
     std::shared_ptr<ClassifierTail> t(new ClassifierTail());
-    t->fc1 = a1; t->fc2 = a2; t->loss = l; t->context = context;
+    t->fc1 = a1; t->fc2 = a2; t->loss = l; t->context = context; t->from_h = !whole;
     return t;
   }
-  bool updates_on_second_stream() const { return fc1->updates_on_second_stream() || fc2->updates_on_second_stream(); }
+  bool updates_on_second_stream() const {
+    return (!from_h && fc1->updates_on_second_stream()) || fc2->updates_on_second_stream();
+  }
   void forward_train(size_t batch_size) {
     RB_ASSERT(batch_size <= fc1->batch_cap_);
-    const int I = (int)fc1->config_.in_channels, H = (int)fc1->config_.out_channels, C = (int)fc2->config_.out_channels;
+    const int I = from_h ? 0 : (int)fc1->config_.in_channels, H = (int)fc1->config_.out_channels, C = (int)fc2->config_.out_channels;
     unwrap(rh_affine2_softmax_kl_step(
-               (int)batch_size, I, H, C, fc1->config_.act_func == ActivationFunction::Rect ? 1 : 0, fc1->in_act_->as_ptr(),
+               (int)batch_size, I, H, C, fc1->config_.act_func == ActivationFunction::Rect ? 1 : 0,
+               from_h ? nullptr : fc1->in_act_->as_ptr(),
                fc1->params_.weights->as_ptr(), fc1->params_.bias->as_ptr(), fc2->params_.weights->as_ptr(),
                fc2->params_.bias->as_ptr(), loss->label_cats_.as_ptr(), loss->weights_.as_ptr(), fc1->out_act_->as_mut_ptr(),
                fc2->out_act_->as_mut_ptr(), loss->out_values_.as_mut_ptr(), loss->max_value_.as_mut_ptr(),
                loss->out_cats_.as_mut_ptr(), loss->out_loss1_.as_mut_ptr(), loss->out_loss_.as_mut_ptr(),
                fc2->out_delta_->as_mut_ptr(), fc1->out_delta_->as_mut_ptr(),
-               fc1->in_delta_ ? fc1->in_delta_->as_mut_ptr() : nullptr,
+               !from_h && fc1->in_delta_ ? fc1->in_delta_->as_mut_ptr() : nullptr,
                reinterpret_cast<uint32_t*>(loss->step_counter_.as_mut_ptr()), context->stream()),
            "classifier tail (forward, loss, data gradients)");
     loss->step_valid_ = batch_size;   // categories, loss and delta are there: the loss operator's calls launch nothing
   }
   void backward_train(size_t batch_size) {
-    const int I = (int)fc1->config_.in_channels, H = (int)fc1->config_.out_channels, C = (int)fc2->config_.out_channels;
+    const int I = from_h ? 0 : (int)fc1->config_.in_channels, H = (int)fc1->config_.out_channels, C = (int)fc2->config_.out_channels;
     rh_stream_t sg = context->stream();
-    if (fc1->overlap_on_ && fc1->in_delta_) {   // as AffineOperator::backward places its parameter gradients
+    if (from_h ? fc2->overlap_on_ : fc1->overlap_on_ && fc1->in_delta_) {   // as AffineOperator::backward places its parameter gradients
       context->fork();
       sg = context->aux_stream();
     }
     const float beta2 = fc2->params_.take_backward_beta();
-    const float beta1 = fc1->params_.take_backward_beta();
-    unwrap(rh_affine2_bwd_params((int)batch_size, I, H, C, fc1->in_act_->as_ptr(), fc1->out_act_->as_ptr(),
+    const float beta1 = from_h ? 0.0f : fc1->params_.take_backward_beta();
+    if (from_h) fc1->delta_masked_once_ = true;   // its backward() follows: the delta it finds is the masked one
+    unwrap(rh_affine2_bwd_params((int)batch_size, I, H, C, from_h ? nullptr : fc1->in_act_->as_ptr(), fc1->out_act_->as_ptr(),
                                  fc1->out_delta_->as_ptr(), fc2->out_delta_->as_ptr(), beta1,
                                  fc1->params_.grad_weights->as_mut_ptr(), fc1->params_.grad_bias->as_mut_ptr(), beta2,
                                  fc2->params_.grad_weights->as_mut_ptr(), fc2->params_.grad_bias->as_mut_ptr(), sg),
@@ -2076,7 +2087,7 @@ void SequentialOperatorWorker::init_params(const uint64_t shared_seed[2]) {
 void SequentialOperatorWorker::forward(size_t batch_size, OpPhase phase) {
   input_op_->forward(batch_size, phase);
   const bool tail = tail_armed_ && phase.training && batch_size > 0;
-  const size_t n = hidden_ops_.size() - (tail ? 2 : 0);
+  const size_t n = hidden_ops_.size() - (tail ? tail_->replaced() : 0);
   for (size_t i = 0; i < n; ++i) {
     Operator* op = hidden_ops_[i].get();
     if (aux_pending_ && op->updates_on_second_stream()) settle();  // its parameters were updated on the second stream
@@ -2096,7 +2107,7 @@ void SequentialOperatorWorker::backward(size_t batch_size) {
   size_t n = hidden_ops_.size();
   if (tail_armed_ && tail_done_ == batch_size && batch_size > 0) {
     tail_->backward_train(batch_size);   // the deltas are there since forward(): only the parameter gradients are left
-    n -= 2;
+    n -= tail_->replaced();
   } else {
     loss_op_->backward(batch_size);
   }

@@ -222,10 +222,15 @@ __global__ __launch_bounds__(NT) void affine2_softmax_kl_step_kernel(
   __shared__ bool last;
   constexpr int NW = NT / 64;
   const int n = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int i = tid; i < I; i += NT) xs[i] = x[(size_t)n * I + i];
+  const bool have_h = x == nullptr;   // the first layer's forward already ran (a layer too large for this form): I = 0
+  if (have_h) {
+    for (int j = tid; j < H; j += NT) hs[j] = h_out[(size_t)n * H + j];
+  } else {
+    for (int i = tid; i < I; i += NT) xs[i] = x[(size_t)n * I + i];
+  }
   __syncthreads();
   // h: a wave per group of four outputs, lanes along the input, 16 x 4 weights per lane in flight
-  for (int j0 = wave * 4; j0 < H; j0 += NW * 4) {
+  for (int j0 = wave * 4; j0 < H && !have_h; j0 += NW * 4) {
     float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const float* r[4];
 #pragma unroll
@@ -329,7 +334,7 @@ __global__ __launch_bounds__(NT) void affine2_softmax_kl_step_kernel(
   }
   __syncthreads();
   // dx = W1^T dh: a thread per input element (rows of W1 read along the lanes), 32 rows' weights in flight
-  if (dx_out) {
+  if (dx_out && !have_h) {
     for (int i = tid; i < I; i += NT) {
       float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
       for (int j0 = 0; j0 < H; j0 += 32) {
@@ -397,9 +402,9 @@ __global__ __launch_bounds__(256) void affine2_bwd_params_kernel(int B, int I, i
     const unsigned k = idx - n1, c = k / (unsigned)H, j = k - c * (unsigned)H;
     kind = 2; pa = dl; sa = C; oa = c; pb = h; sb = H; ob = j;
   } else if (idx < total) {
-    const unsigned k = idx - n1 - n2;
-    if (k < (unsigned)H) { kind = 3; sa = H; oa = k; }
-    else { kind = 4; pa = dl; sa = C; oa = k - (unsigned)H; }
+    const unsigned k = idx - n1 - n2, hb = n3 - (unsigned)C;   // hb = H, or 0 when the first layer's gradients are not asked for
+    if (k < hb) { kind = 3; sa = H; oa = k; }
+    else { kind = 4; pa = dl; sa = C; oa = k - hb; }
   }
   float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
   if (kind >= 0) {
@@ -515,9 +520,10 @@ extern "C" int rh_softmax_kl_step(const float* x, int32_t C, int32_t N, const in
 // afford to read the whole first layer (twice): up to 4096 inputs, 2048 hidden units, 64 classes, 2^17 weights (512 KB)
 // in the first layer and 2^26 multiply-adds in its products over the batch.  Beyond that the tiled products, which read
 // the weights once, are the faster form.
+// I = 0 asks for the form that starts from h (the first layer's products stay with the tiled kernels).
 extern "C" int rh_affine2_softmax_kl_step_supported(int32_t B, int32_t I, int32_t H, int32_t C) {
-  return B > 0 && I > 0 && H > 0 && C > 0 && I <= 4096 && H <= 2048 && C <= 64 && (long long)I * H <= (1ll << 17) &&
-                 (long long)B * I * H <= (1ll << 26)
+  return B > 0 && I >= 0 && H > 0 && C > 0 && I <= 4096 && H <= 2048 && C <= 64 && (long long)I * H <= (1ll << 17) &&
+                 (long long)B * I * H <= (1ll << 26) && (long long)B * H < (1ll << 31)
              ? 1 : 0;
 }
 
@@ -526,10 +532,10 @@ extern "C" int rh_affine2_softmax_kl_step(int32_t B, int32_t I, int32_t H, int32
                                           const int32_t* labels, const float* weights, float* h, float* logits, float* p,
                                           float* max_out, int32_t* idx_out, float* loss1, float* loss_sum, float* dlogits,
                                           float* dh, float* dx, uint32_t* counter, rh_stream_t stream) {
-  if (B < 0 || I <= 0 || H <= 0 || C <= 0) return RH_E_INVALID;
+  if (B < 0 || I < 0 || H <= 0 || C <= 0 || (I == 0) != (x == nullptr)) return RH_E_INVALID;
   if (B == 0) return 0;
   if (!rh_affine2_softmax_kl_step_supported(B, I, H, C)) return RH_E_UNSUPPORTED;
-  if (!x || !w1 || !b1 || !w2 || !b2 || !labels || !weights || !h || !logits || !p || !max_out || !idx_out || !loss1 ||
+  if ((x && (!w1 || !b1)) || !w2 || !b2 || !labels || !weights || !h || !logits || !p || !max_out || !idx_out || !loss1 ||
       !loss_sum || !dlogits || !dh || !counter)
     return RH_E_INVALID;
   constexpr int NT = 1024;
@@ -544,11 +550,13 @@ extern "C" int rh_affine2_softmax_kl_step(int32_t B, int32_t I, int32_t H, int32
 extern "C" int rh_affine2_bwd_params(int32_t B, int32_t I, int32_t H, int32_t C, const float* x, const float* h, const float* dh,
                                      const float* dlogits, float beta1, float* dw1, float* db1, float beta2, float* dw2,
                                      float* db2, rh_stream_t stream) {
-  if (B < 0 || I <= 0 || H <= 0 || C <= 0) return RH_E_INVALID;
+  if (B < 0 || I < 0 || H <= 0 || C <= 0 || (I == 0) != (x == nullptr)) return RH_E_INVALID;
   if (!rh_affine2_softmax_kl_step_supported(B > 0 ? B : 1, I, H, C)) return RH_E_UNSUPPORTED;
-  if (!x || !h || !dh || !dlogits || !dw1 || !db1 || !dw2 || !db2) return RH_E_INVALID;
-  const int vec = I % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dw1)) & 15) == 0 ? 1 : 0;
-  const unsigned n1 = (unsigned)((size_t)H * I / (vec ? 4 : 1)), n2 = (unsigned)((size_t)C * H), n3 = (unsigned)(H + C);
+  if (!h || !dlogits || !dw2 || !db2 || (x && (!dh || !dw1 || !db1))) return RH_E_INVALID;
+  const int vec = x && I % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dw1)) & 15) == 0 ? 1 : 0;
+  // (without x only the second layer's gradients are formed: no dW1 items and no db1 among the bias items)
+  const unsigned n1 = x ? (unsigned)((size_t)H * I / (vec ? 4 : 1)) : 0u, n2 = (unsigned)((size_t)C * H),
+                 n3 = (unsigned)((x ? H : 0) + C);
   const size_t total = (size_t)n1 + n2 + n3;
   ProfScope prof("affine2_bwd_params", 4.0 * ((double)B * (I + 2.0 * H + C) + (double)I * H + (double)H * C), to_stream(stream));
   hipLaunchKernelGGL(affine2_bwd_params_kernel, dim3((unsigned)cdiv<size_t>(total, 32)), dim3(256), 0, to_stream(stream), B, I, H,

@@ -362,6 +362,31 @@ def affine2_softmax_kl_step(x, w1, b1, w2, b2, labels, weights, relu1=True, want
     return out
 
 
+def affine_softmax_kl_step_from_h(h, w2, b2, labels, weights, relu1=True, counter=None):
+    """The same launch started from the first layer's output h (B, H) (I = 0, x = NULL): logits .. dh."""
+    B, H = h.shape
+    Cc = w2.shape[0]
+    f = lambda *shape: torch.empty(shape, dtype=torch.float32, device=h.device)
+    out = {"h": h, "logits": f(B, Cc), "p": f(B, Cc), "max": f(B), "idx": torch.empty((B,), dtype=torch.int32, device=h.device),
+           "loss1": f(B), "loss": f(1), "dlogits": f(B, Cc), "dh": f(B, H)}
+    if counter is None:
+        counter = torch.zeros((1,), dtype=torch.int32, device=h.device)
+    out["counter"] = counter
+    check(lib().rh_affine2_softmax_kl_step(B, 0, H, Cc, int(relu1), None, None, None, _p(w2), _p(b2), _p(labels),
+                                           _p(weights), _p(h), _p(out["logits"]), _p(out["p"]), _p(out["max"]),
+                                           _p(out["idx"]), _p(out["loss1"]), _p(out["loss"]), _p(out["dlogits"]), _p(out["dh"]),
+                                           None, _p(counter), _stream()),
+          "rh_affine2_softmax_kl_step")
+    return out
+
+
+def affine_bwd_params_from_h(h, dlogits, dw2, db2, beta2=0.0):
+    """dW2 and db2 only (rh_affine2_bwd_params with I = 0, x = NULL)."""
+    B, H = h.shape
+    check(lib().rh_affine2_bwd_params(B, 0, H, dlogits.shape[1], None, _p(h), None, _p(dlogits), 0.0, None, None, beta2,
+                                      _p(dw2), _p(db2), _stream()), "rh_affine2_bwd_params")
+
+
 def affine2_bwd_params(x, h, dh, dlogits, dw1, db1, dw2, db2, beta1=0.0, beta2=0.0):
     """dW1, db1, dW2, db2 of the two layers in one launch (rh_affine2_bwd_params); out = sum + beta * out."""
     B, I = x.shape

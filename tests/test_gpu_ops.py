@@ -576,7 +576,60 @@ def test_affine2_softmax_kl_step(dev, case):
             assert_close(N(db2), (dll.astype(np.float64).sum(axis=0) + beta2 * db2_0).astype(np.float32), "affine2 db2 beta %g" % beta2)
 
 
+@pytest.mark.parametrize("case", [(64, 500, 10, True), (3, 2048, 64, False), (130, 1, 2, True), (256, 384, 17, True)])
+def test_affine_softmax_kl_step_from_h(dev, case):
+    """The form that starts from the first layer's output (I = 0, x = NULL): second layer, loss step and the hidden
+    delta in one launch, dW2 and db2 in another; h and the first layer's gradients are left untouched."""
+    B, H, Cc, relu = case
+    assert ops.affine2_softmax_kl_step_supported(B, 0, H, Cc)
+    counter = None
+    for rep in range(2):
+        say("affine_softmax_kl_step_from_h", case, "call", rep)
+        h = synth.normal(43, 10 * rep + 1, (B, H))
+        if relu:
+            h = np.maximum(h, 0.0).astype(np.float32)
+        w2 = synth.normal(43, 10 * rep + 4, (Cc, H), 0.0, 1.0 / np.sqrt(H))
+        b2 = synth.normal(43, 10 * rep + 5, (Cc,), 0.0, 0.5)
+        labels = synth.integers(43, 10 * rep + 6, (B,), Cc)
+        weights = synth.uniform(43, 10 * rep + 7, (B,), 0.1, 1.0)
+        logits = O.sgemm(1, 0, Cc, B, H, 1.0, w2, H, h, H, 0.0, np.zeros((B, Cc), np.float32), Cc) + b2
+        p = O.softmax_fwd(logits)
+        dl = O.softmax_kl_backward(p, labels, weights)
+        l1 = O.softmax_kl_loss1(p, labels, weights)
+        h_dev = T(h, dev)
+        out = ops.affine_softmax_kl_step_from_h(h_dev, T(w2, dev), T(b2, dev), T(labels, dev), T(weights, dev), relu1=relu,
+                                                counter=counter)
+        counter = out["counter"]
+        assert int(N(counter)[0]) == 0
+        assert np.array_equal(N(h_dev), h), "h is an input here"
+        assert_close(N(out["logits"]), logits, "from_h logits")
+        assert_close(N(out["p"]), p, "from_h softmax", atol=1e-6)
+        assert np.array_equal(N(out["idx"]), O.blockreduce_argmax(N(out["p"]))[1])
+        assert np.array_equal(N(out["max"]), N(out["p"]).max(axis=1))
+        assert_close(N(out["loss1"]), l1, "from_h loss1")
+        assert_close(N(out["loss"]), np.array([l1.astype(np.float64).sum()], np.float32), "from_h loss sum")
+        assert_close(N(out["dlogits"]), dl, "from_h dlogits")
+        dh = O.sgemm(0, 0, H, B, Cc, 1.0, w2, H, N(out["dlogits"]), Cc, 0.0, np.zeros((B, H), np.float32), H)
+        if relu:
+            dh = dh * (h > 0)
+        assert_close(N(out["dh"]), dh, "from_h dh")
+        dll = N(out["dlogits"])
+        for beta2 in (0.0, 1.0):
+            dw2_0, db2_0 = synth.normal(43, 10 * rep + 10, (Cc, H)), synth.normal(43, 10 * rep + 11, (Cc,))
+            dw2, db2 = T(dw2_0, dev), T(db2_0, dev)
+            ops.affine_bwd_params_from_h(h_dev, out["dlogits"], dw2, db2, beta2)
+            r2 = O.sgemm(0, 1, H, Cc, B, 1.0, h, H, dll, Cc, beta2, dw2_0.copy(), H)
+            assert_close(N(dw2), r2, "from_h dW2 beta %g" % beta2)
+            assert_close(N(db2), (dll.astype(np.float64).sum(axis=0) + beta2 * db2_0).astype(np.float32), "from_h db2 beta %g" % beta2)
+
+
 def test_affine2_softmax_kl_step_limits(dev):
+    x8 = torch.zeros((2, 8), device=dev)
+    # I = 0 goes with x = NULL and the other way round
+    assert _lib.lib().rh_affine2_softmax_kl_step(2, 0, 4, 2, 1, *([x8.data_ptr()] * 19), None) == _lib.RH_E_INVALID
+    assert _lib.lib().rh_affine2_softmax_kl_step(2, 8, 4, 2, 1, None, *([x8.data_ptr()] * 18), None) == _lib.RH_E_INVALID
+    assert ops.affine2_softmax_kl_step_supported(64, 0, 500, 10)
+    assert not ops.affine2_softmax_kl_step_supported(64, 0, 2049, 10)
     assert not ops.affine2_softmax_kl_step_supported(64, 4097, 10, 10)
     assert not ops.affine2_softmax_kl_step_supported(64, 2450, 500, 10)     # more than 2^17 weights in the first layer
     assert not ops.affine2_softmax_kl_step_supported(1024, 4096, 32, 10)    # more than 2^26 multiply-adds over the batch

@@ -185,12 +185,15 @@ def test_schedule_that_never_repeats_a_step_size_is_launched(dev):
 TAIL_DIMS = (12, 12, 3)
 
 
-def tail_net(fc1_act):
-    return (TAIL_DIMS, *configs._chain(TAIL_DIMS, [("conv", 3, 1, 1, 8, "Rect"), ("pool", 2, 2, 0, "Max"), ("fc", 70, fc1_act),
+def tail_net(fc1_act, hidden=70):
+    return (TAIL_DIMS, *configs._chain(TAIL_DIMS, [("conv", 3, 1, 1, 8, "Rect"), ("pool", 2, 2, 0, "Max"), ("fc", hidden, fc1_act),
                                                    ("fc", 5, "Identity")]))
 
 
-@pytest.mark.parametrize("name,batch,steps", [("cifar10", 128, 4), ("tail_rect", 7, 3), ("tail_identity", 33, 3)])
+# lenet and tail_wide have a first classifier layer of more than 2^17 weights: it keeps its tiled products and the two
+# launches stand for the second layer and the loss
+@pytest.mark.parametrize("name,batch,steps", [("cifar10", 128, 4), ("tail_rect", 7, 3), ("tail_identity", 33, 3),
+                                              ("lenet", 64, 4), ("tail_wide", 19, 3)])
 def test_classifier_tail_in_two_launches(dev, name, batch, steps):
     """Train steps whose classifier tail (affine, affine, softmax loss) runs as two launches against the same steps
     through the separate operators: same losses, correct counts, parameters, momentum, and the same activations and
@@ -200,7 +203,9 @@ def test_classifier_tail_in_two_launches(dev, name, batch, steps):
     from rembrandt_amd import _lib
     from conftest import assert_close
     say("classifier tail", name, batch)
-    net = configs.NETWORKS[name]() if name in configs.NETWORKS else tail_net("Rect" if name == "tail_rect" else "Identity")
+    net = (configs.NETWORKS[name]() if name in configs.NETWORKS else tail_net("Rect", 500) if name == "tail_wide"
+           else tail_net("Rect" if name == "tail_rect" else "Identity"))
+    from_h = name in ("lenet", "tail_wide")
     layers = net[1]
     fc = [i for i, l in enumerate(layers) if l[0] == "affine"]
     assert len(fc) >= 2 and fc[-1] == len(layers) - 1 and fc[-2] == len(layers) - 2
@@ -219,7 +224,7 @@ def test_classifier_tail_in_two_launches(dev, name, batch, steps):
     finally:
         lib.rh_profile_enable(0)
     assert tags.count("affine2_softmax_kl_step") == steps and tags.count("affine2_bwd_params") == steps, "the two-launch tail ran"
-    assert "softmax_kl_step" not in tags and "sgemm_skinny" not in tags
+    assert "softmax_kl_step" not in tags and (from_h or "sgemm_skinny" not in tags)
     plain, _ = run(net, batch, steps, False, 0x7A11, kw, fuse_tail=False, extra=extra)
     for step, ((la, ca, pa), (lb, cb, pb)) in enumerate(zip(fusedrun, plain)):
         assert abs(la - lb) <= 1e-5 * max(1.0, abs(lb)), (step, la, lb)
