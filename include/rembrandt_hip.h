@@ -48,6 +48,11 @@ typedef void* rh_stream_t; /* hipStream_t */
 #define RH_ALGO_GATHER             0x100 /* k -> {offset, dr, ds} table gather straight from the NCHW tensors      */
 #define RH_ALGO_SCALAR_OFFSET      0x200 /* scalar-offset loads on padded / transposed copies in the workspace,
                                             wherever the geometry allows it (else the gather family)             */
+#define RH_ALGO_WINOGRAD           0x400 /* conv fwd / bwd-data of a 3x3 stride-1 layer by Winograd F(2x2, 3x3): 2.25x
+                                            fewer multiply-adds, sums in another order (RH_E_UNSUPPORTED for other
+                                            geometries).  Without an RH_ALGO_* bit the library takes it for such layers
+                                            of 64 channels and more on both sides; either bit above keeps the direct form */
+#define RH_ALGO_DIRECT             0x800 /* never the Winograd form; the direct forms chosen as without any RH_ALGO_* bit */
 
 const char* rh_version(void);
 /* Status of the most recent launch made by a void `rembrandt_kernel_*` entry point on this thread. */

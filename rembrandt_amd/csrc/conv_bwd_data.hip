@@ -168,9 +168,18 @@ static int bwd_data_impl(const rh_conv_geom* g, float alpha, const float* w, con
   if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return RH_E_WORKSPACE;
   hipStream_t stream = to_stream(stream_);
 
+  if ((flags & RH_ALGO_WINOGRAD) && (!wino_shape(d) || (flags & (RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT)))) return RH_E_UNSUPPORTED;
   if (!(flags & (RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET)) && conv1x1_stream_applies(d)) {
     if (d.x_elems == 0) return 0;
     return launch_conv1x1_stream(d, RH_CONV_BWD_DATA, w, dy, dx, alpha, beta, nullptr, 0, stream, mask);
+  }
+  if (wino_shape(d) && !(flags & (RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))) {
+    const WinoGeom wg = wino_geom_bwd_data(d);
+    if (flags & RH_ALGO_WINOGRAD ? wg.ok : wino_pays(wg)) {
+      if (d.x_elems == 0) return 0;
+      return launch_conv_wino(wg, true, dy, w, dx, alpha, beta, nullptr, 0, mask, ws, stream, "conv_bwd_data_wino");
+    }
+    if (flags & RH_ALGO_WINOGRAD) return RH_E_UNSUPPORTED;
   }
   const int KRS = d.K * d.R * d.S;
   const PhasePlan pp = plan_phase_bwd_data(d);

@@ -800,6 +800,10 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
       size_t need = sp.ok && sp.total() > legacy ? sp.total() : legacy;
       const Bf16FwdPlan bp = plan_bf16_fwd(d);  // the bf16 flag is not known here: room for either form
       if (bp.ok && bp.total() > need) need = bp.total();
+      if (wino_shape(d)) {   // the flags are not known here: room for the Winograd form wherever the geometry has one
+        const WinoGeom wg = wino_geom_fwd(d);
+        if (wg.ok && wg.total() > need) need = wg.total();
+      }
       return need;
     }
     case RH_CONV_BWD_DATA: {
@@ -808,7 +812,12 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
       const PhasePlan pp = plan_phase_bwd_data(d);
       if (pp.ok) return pp.total() > legacy ? pp.total() : legacy;
       const SoffPlan sp = plan_soff_bwd_data(d);
-      return sp.ok && sp.total() > legacy ? sp.total() : legacy;
+      size_t need = sp.ok && sp.total() > legacy ? sp.total() : legacy;
+      if (wino_shape(d)) {
+        const WinoGeom wg = wino_geom_bwd_data(d);
+        if (wg.ok && wg.total() > need) need = wg.total();
+      }
+      return need;
     }
     case RH_CONV_BWD_FILTER:
       return bwd_filter_plan_bytes(d) + bwd_filter_bias_bytes(d);

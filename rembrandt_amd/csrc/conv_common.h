@@ -291,6 +291,31 @@ inline SoffPlan plan_soff_fwd(const ConvDims& d) {
   return p;
 }
 
+// Winograd F(2x2, 3x3) form of a 3x3 stride-1 layer (conv_wino.hip), written as a forward convolution: an input of
+// (N, Ci, Hi, Wi) with `halo` zeros around it, Ko filters, a result of (N, Ko, P, Q).  Backward-data is the same over dy
+// with halo 2 - pad.  Scratch: [U: transformed filter][V: transformed image patches].
+constexpr int kWinoBM = 128, kWinoBN = 32, kWinoR = 3;
+struct WinoGeom {
+  int N, Ci, Hi, Wi, Ko, halo, P, Q, TP, TQ;
+  int Cg;                     // groups of four input channels
+  int rows_p;                 // Ko rounded up to whole row tiles
+  long long tiles, tiles_p;   // 2x2 output tiles; rounded up to whole column tiles
+  size_t u_bytes, v_bytes;
+  bool ok;
+  size_t total() const { return u_bytes + v_bytes; }
+};
+WinoGeom wino_geom(int N, int Ci, int Hi, int Wi, int Ko, int halo);
+inline bool wino_shape(const ConvDims& d) { return d.R == 3 && d.S == 3 && d.st == 1 && d.pad <= 2; }
+inline WinoGeom wino_geom_fwd(const ConvDims& d) { return wino_geom(d.N, d.C, d.H, d.W, d.K, d.pad); }
+inline WinoGeom wino_geom_bwd_data(const ConvDims& d) { return wino_geom(d.N, d.K, d.P, d.Q, d.C, 2 - d.pad); }
+// Where the library takes it by itself: enough channels on both sides for the 16 products to be worth their
+// transforms, and a grid that fills the GPU.
+inline bool wino_pays(const WinoGeom& g) {
+  return g.ok && g.Ci >= 64 && g.Ko >= 64 && (long long)(g.rows_p / kWinoBM) * (g.tiles_p / kWinoBN) >= 192;
+}
+int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* w, float* out, float alpha, float beta,
+                     const float* bias, int relu, const float* mask, void* ws, hipStream_t stream, const char* tag);
+
 // Forward with packed bf16 operands (RH_MATH_BF16_MFMA_FP32ACC, input channels a multiple of 8): the contraction runs
 // over k = (r, s, c) with c fastest, the image is copied once to bf16 as [n][hp][c/8][wp][8] with its zero border,
 // the filter to bf16 as [k/8][ko][8] (zero past C*R*S), so that eight consecutive k of one row are 16 contiguous

@@ -276,6 +276,7 @@ int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, ui
     opts.overlap_backward = (exec_flags & RHO_EXEC_OVERLAP_BACKWARD) != 0;
     opts.graph_steps = (exec_flags & RHO_EXEC_GRAPH_STEPS) != 0;
     opts.fuse_tail = (exec_flags & RHO_EXEC_SEPARATE_TAIL) == 0;
+    opts.winograd = (exec_flags & RHO_EXEC_DIRECT_CONV) == 0;
     w->graph_steps = opts.graph_steps;
     w->fuse_epilogue = opts.fuse_epilogue;
     w->worker.reset(new SequentialOperatorWorker(cfg->cfg, (size_t)batch_size,

@@ -867,7 +867,7 @@ class Conv2dOperator : public Operator {
       }
       return;
     }
-    const int math = opts_.bf16_forward ? RH_MATH_BF16_MFMA_FP32ACC : 0;
+    const int math = (opts_.bf16_forward ? RH_MATH_BF16_MFMA_FP32ACC : 0) | (opts_.winograd ? 0 : RH_ALGO_DIRECT);
     if (opts_.fuse_epilogue) {
       const int flags = RH_FUSE_BIAS | (rect ? RH_FUSE_RELU : 0) | math;
       unwrap(rh_conv2d_fwd(&g, 1.0f, in_act_->as_ptr(), params_.weights->as_ptr(), 0.0f, out_act_->as_mut_ptr(),
@@ -925,11 +925,13 @@ class Conv2dOperator : public Operator {
     if (in_delta_ && fold_prev_relu_) {
       // the operator below left its ReLU backward mask to this call: in_act_ is that ReLU's output
       unwrap(rh_conv2d_bwd_data_relu(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
-                                     in_act_->as_ptr(), workspace_->as_mut_ptr(), workspace_->len(), 0, s),
+                                     in_act_->as_ptr(), workspace_->as_mut_ptr(), workspace_->len(),
+                                     opts_.winograd ? 0 : RH_ALGO_DIRECT, s),
              "conv2d backward data");
     } else if (in_delta_) {
       unwrap(rh_conv2d_bwd_data(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
-                                workspace_->as_mut_ptr(), workspace_->len(), 0, s), "conv2d backward data");
+                                workspace_->as_mut_ptr(), workspace_->len(), opts_.winograd ? 0 : RH_ALGO_DIRECT, s),
+             "conv2d backward data");
     }
   }
   void regularize(Regularization reg) override { params_.regularize(reg); }
@@ -1250,6 +1252,7 @@ struct BNormConvUnit {
   Buf running_mean, running_ivar, save_running_mean, save_running_ivar, cached_mean, cached_ivar;
   Buf pre_act, pre_delta;  // the conv output the batch norm reads, and the gradient w.r.t. it
   bool backward = false;
+  int conv_algo = 0;       // RH_ALGO_* bits of the unit's convolution calls
 
   void alloc(size_t batch, Dims3 in, size_t size, size_t stride, size_t pad, size_t out_channels, bool bwd, Ctx c) {
     in_dims = in; conv_size = size; conv_stride = stride; conv_pad = pad; chans = out_channels; ctx = c; backward = bwd;
@@ -1315,7 +1318,7 @@ struct BNormConvUnit {
                double epsilon, bool relu, DeviceBuffer<uint8_t>& ws, bool bf16) {
     const rh_conv_geom g = geom(batch);
     unwrap(rh_conv2d_fwd(&g, 1.0f, in, weights->as_ptr(), 0.0f, pre_act->as_mut_ptr(), nullptr, ws.as_mut_ptr(), ws.len(),
-                         bf16 ? RH_MATH_BF16_MFMA_FP32ACC : 0, s()), "conv2d forward");
+                         (bf16 ? RH_MATH_BF16_MFMA_FP32ACC : 0) | conv_algo, s()), "conv2d forward");
     const int flags = relu ? RH_FUSE_RELU : 0;
     if (phase.training) {
       if (!backward) panic("batch norm training missing backward operator");
@@ -1364,8 +1367,8 @@ struct BNormConvUnit {
   // in_delta = beta*in_delta + dconv^T(weights, pre_delta)
   void backward_data(size_t batch, float* in_delta, float beta, DeviceBuffer<uint8_t>& ws) {
     const rh_conv_geom g = geom(batch);
-    unwrap(rh_conv2d_bwd_data(&g, 1.0f, weights->as_ptr(), pre_delta->as_ptr(), beta, in_delta, ws.as_mut_ptr(), ws.len(), 0,
-                              s()), "conv2d backward data");
+    unwrap(rh_conv2d_bwd_data(&g, 1.0f, weights->as_ptr(), pre_delta->as_ptr(), beta, in_delta, ws.as_mut_ptr(), ws.len(),
+                              conv_algo, s()), "conv2d backward data");
   }
 
   void axpy(float a, const DeviceBuffer<float>& x, DeviceBuffer<float>& y) {
@@ -1507,6 +1510,7 @@ class BNormUnitsOperator : public Operator {
     in_act_ = prev_op->get_output_vars();
     if (!in_act_) panic(std::string(who) + " missing required prev operator output vars");
     in_delta_ = prev_op->get_output_deltas();
+    for (auto& u : units_) u.conv_algo = opts.winograd ? 0 : RH_ALGO_DIRECT;
   }
   size_t batch_size() const override { return batch_cap_; }
   SharedDeviceBuf get_output_vars() const override { return out_act_; }

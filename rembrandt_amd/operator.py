@@ -297,11 +297,11 @@ class SequentialOperatorWorker:
     """src/operator/worker.rs:230-477 plus the Input/Loss operator calls the optimizer makes on it."""
 
     def __init__(self, config, batch_size, capability="Backward", shared_seed=(1, 2), device=0, fuse_epilogue=True,
-                 bf16_forward=False, overlap_backward=True, graph_steps=False, fuse_tail=True):
+                 bf16_forward=False, overlap_backward=True, graph_steps=False, fuse_tail=True, winograd=True):
         """graph_steps: SgdOpt.train_batch records a whole step into a HIP graph and replays it (launch-bound networks)."""
         h = _vp()
         flags = ((1 if fuse_epilogue else 0) | (2 if bf16_forward else 0) | (4 if overlap_backward else 0) | (8 if graph_steps else 0) |
-                 (0 if fuse_tail else 16))
+                 (0 if fuse_tail else 16) | (0 if winograd else 32))
         _chk(lib().rho_worker_new(config._h, batch_size, 0 if capability == "Forward" else 1, shared_seed[0],
                                   shared_seed[1], device, flags, C.byref(h)))
         self._h = h

@@ -55,6 +55,8 @@ pub const RH_FUSE_RELU: c_int = 0x20;
 pub const RH_MATH_BF16_MFMA_FP32ACC: c_int = 0x1;
 pub const RH_ALGO_GATHER: c_int = 0x100;
 pub const RH_ALGO_SCALAR_OFFSET: c_int = 0x200;
+pub const RH_ALGO_WINOGRAD: c_int = 0x400;
+pub const RH_ALGO_DIRECT: c_int = 0x800;
 
 #[link(name = "rembrandt_hip")]
 extern "C" {

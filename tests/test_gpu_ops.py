@@ -151,6 +151,91 @@ def test_conv2d_all_passes(dev, case, algo):
     torch.cuda.synchronize()
 
 
+# 3x3 stride-1 layers in the Winograd F(2x2, 3x3) form: odd and even extents (tiles that hang over the edge), every
+# padding it takes, channel counts that do not fill a group of four, filter counts around the 128-row tile, tile counts
+# that are no multiple of the 32-tile block, more blocks than CUs, and the sizes the library takes the form for by itself
+WINO_CASES = [
+    # N, C, H, W, K, pad
+    (2, 8, 6, 6, 8, 1),
+    (3, 5, 7, 9, 130, 1),
+    (1, 12, 8, 8, 16, 0),
+    (2, 16, 5, 6, 20, 2),
+    (1, 1, 3, 3, 1, 0),           # one output pixel
+    (1, 2, 2, 2, 3, 1),
+    (4, 70, 13, 13, 140, 1),
+    (2, 64, 13, 13, 96, 1),
+    (33, 64, 14, 15, 128, 1),
+    (70, 66, 13, 13, 384, 1),     # 3 x 108 blocks
+    (16, 128, 28, 28, 64, 1),
+]
+
+
+@pytest.mark.parametrize("case", WINO_CASES, ids=str)
+def test_conv2d_winograd(dev, case):
+    """RH_ALGO_WINOGRAD against the oracle's direct convolution, forward and backward-data, with every epilogue the
+    direct kernels have; the masked data gradient bit-identical to gradient + in-place mask; RH_ALGO_DIRECT and the
+    loader bits keep the direct form; other geometries are refused."""
+    Nn, C, H, W, K, pad = case
+    say("winograd case", case)
+    WG = _lib.RH_ALGO_WINOGRAD
+    x = synth.normal(15, 1, (Nn, C, H, W))
+    w = synth.normal(15, 2, (K, C, 3, 3))
+    b = synth.normal(15, 3, (K,))
+    y_ref = O.conv2d_fwd(x, w, 1, pad)
+    dy = synth.normal(15, 4, y_ref.shape)
+    xd, wd, bd, dyd = T(x, dev), T(w, dev), T(b, dev), T(dy, dev)
+    y = ops.conv2d_fwd(xd, wd, 1, pad, algo=WG)
+    assert_close(N(y), y_ref, "winograd fwd")
+    yf = ops.conv2d_fwd(xd, wd, 1, pad, bias=bd, relu=True, algo=WG)
+    assert_close(N(yf), O.rect_inplace(O.add_bias_nchw(b, y_ref.copy())), "winograd fwd fused bias+relu")
+    # the fused epilogue is the separate passes' arithmetic
+    two = ops.conv2d_fwd(xd, wd, 1, pad, algo=WG)
+    assert torch.equal(torch.clamp_min(two + bd.view(1, -1, 1, 1), 0.0), yf), "winograd fused epilogue == conv, add_bias, rect"
+    y0 = synth.normal(15, 5, y_ref.shape)
+    yb = ops.conv2d_fwd(xd, wd, 1, pad, alpha=0.5, beta=2.0, y=T(y0, dev), algo=WG)
+    assert_close(N(yb), O.conv2d_fwd(x, w, 1, pad, alpha=0.5, beta=2.0, y=y0.copy()), "winograd fwd alpha/beta")
+    dx_ref = O.conv2d_bwd_data(w, dy, x.shape, 1, pad)
+    dx = ops.conv2d_bwd_data(wd, dyd, x.shape, 1, pad, algo=WG)
+    assert_close(N(dx), dx_ref, "winograd bwd data")
+    dx0 = synth.normal(15, 8, x.shape)
+    dxb = ops.conv2d_bwd_data(wd, dyd, x.shape, 1, pad, alpha=0.5, beta=2.0, dx=T(dx0, dev), algo=WG)
+    assert_close(N(dxb), O.conv2d_bwd_data(w, dy, x.shape, 1, pad, 0.5, 2.0, dx0.copy()), "winograd bwd data alpha/beta")
+    for alpha, beta in ((1.0, 0.0), (0.5, 2.0)):
+        two = ops.conv2d_bwd_data(wd, dyd, x.shape, 1, pad, alpha=alpha, beta=beta, dx=T(dx0, dev), algo=WG)
+        ops.rect_backprop_inplace(xd, two)
+        one = ops.conv2d_bwd_data(wd, dyd, x.shape, 1, pad, alpha=alpha, beta=beta, dx=T(dx0, dev), algo=WG, relu_of=xd)
+        assert torch.equal(one, two), "winograd masked data gradient alpha=%g beta=%g" % (alpha, beta)
+    # run to run the same bits
+    assert torch.equal(ops.conv2d_fwd(xd, wd, 1, pad, algo=WG), y)
+    # what the library picks by itself: this form from 64 channels on both sides and 192 blocks on, else a direct one
+    auto = ops.conv2d_fwd(xd, wd, 1, pad)
+    direct = ops.conv2d_fwd(xd, wd, 1, pad, algo=_lib.RH_ALGO_DIRECT)
+    assert_close(N(direct), y_ref, "RH_ALGO_DIRECT fwd")
+    blocks = -(-K // 128) * -(-(Nn * -(-y_ref.shape[2] // 2) * -(-y_ref.shape[3] // 2)) // 32)
+    takes = C >= 64 and K >= 64 and blocks >= 192
+    assert torch.equal(auto, y if takes else direct), "library's choice"
+    torch.cuda.synchronize()
+
+
+def test_conv2d_winograd_refused_geometries(dev):
+    import ctypes as C
+    x = torch.zeros((2, 4, 8, 8), device=dev)
+    ws = torch.zeros((1 << 22,), dtype=torch.uint8, device=dev)
+    for R, st, pad, extra in ((5, 1, 2, 0), (3, 2, 1, 0), (1, 1, 0, 0), (3, 1, 3, 0), (3, 1, 1, _lib.RH_ALGO_GATHER),
+                              (3, 1, 1, _lib.RH_ALGO_DIRECT), (3, 1, 1, _lib.RH_MATH_BF16_MFMA_FP32ACC)):
+        g = _lib.ConvGeom(2, 4, 8, 8, 4, R, R, st, pad)
+        w = torch.zeros((4, 4, R, R), device=dev)
+        P = (8 + 2 * pad - R) // st + 1
+        y = torch.zeros((2, 4, P, P), device=dev)
+        rc = _lib.lib().rh_conv2d_fwd(C.byref(g), 1.0, x.data_ptr(), w.data_ptr(), 0.0, y.data_ptr(), None, ws.data_ptr(), ws.numel(),
+                                      _lib.RH_ALGO_WINOGRAD | extra, None)
+        assert rc == _lib.RH_E_UNSUPPORTED, (R, st, pad, extra, rc)
+        if not (extra & _lib.RH_MATH_BF16_MFMA_FP32ACC):
+            rc = _lib.lib().rh_conv2d_bwd_data(C.byref(g), 1.0, w.data_ptr(), y.data_ptr(), 0.0, x.data_ptr(), ws.data_ptr(), ws.numel(),
+                                               _lib.RH_ALGO_WINOGRAD | extra, None)
+            assert rc == _lib.RH_E_UNSUPPORTED, ("bwd", R, st, pad, extra, rc)
+
+
 # input channels a multiple of 8 take the packed-operand form (bf16 copies of image and filter in 16-byte groups of
 # eight channels): channel groups that do not fill a 64-wide tile, rectangular images, stride with padding, no padding,
 # more filters than one row tile, a contraction shorter than one K step

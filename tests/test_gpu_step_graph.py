@@ -24,10 +24,11 @@ def param_buffers(net, read_grads=True):
     return names
 
 
-def run(net, batch, steps, graph, seed, sgd_kwargs, fused=True, toggle_at=None, read_grads=True, fuse_tail=True, extra=()):
+def run(net, batch, steps, graph, seed, sgd_kwargs, fused=True, toggle_at=None, read_grads=True, fuse_tail=True, extra=(),
+        winograd=True):
     dims, layers, ncat = net
     w = SequentialOperatorWorker(configs.build_config(net), batch, "Backward", shared_seed=(seed, seed + 1), graph_steps=graph,
-                                 fuse_tail=fuse_tail)
+                                 fuse_tail=fuse_tail, winograd=winograd)
     w.init_params()
     sgd = SgdOpt(batch, **sgd_kwargs)
     sgd.begin(w)
@@ -231,3 +232,62 @@ def test_classifier_tail_in_two_launches(dev, name, batch, steps):
         assert ca == cb, (step, ca, cb)
         for k, (u, v) in enumerate(zip(pa, pb)):
             assert_close(u, v, "%s step %d buffer %d" % (name, step, k))
+
+
+def profile_tags(fn):
+    """Runs fn() with the library's per-launch records on; returns (fn's result, list of the tags launched)."""
+    import ctypes as C
+    from rembrandt_amd import _lib
+    lib = _lib.lib()
+    lib.rh_profile_reset(); lib.rh_profile_filter(None); lib.rh_profile_enable(1)
+    try:
+        res = fn()
+        tag, work, ms = C.c_char_p(), C.c_double(), C.c_float()
+        tags = []
+        for i in range(lib.rh_profile_count()):
+            lib.rh_profile_get(i, C.byref(tag), C.byref(work), C.byref(ms))
+            tags.append(tag.value.decode())
+    finally:
+        lib.rh_profile_enable(0)
+        lib.rh_profile_reset()
+    return res, tags
+
+
+WINO_DIMS = (16, 16, 8)
+
+
+def wino_net(kind):
+    if kind == "plain":      # conv -> conv (ReLU backward folded into the second layer's data gradient) -> pool -> fc
+        spec = [("conv", 3, 1, 1, 64, "Rect"), ("conv", 3, 1, 1, 64, "Rect"), ("conv", 3, 1, 1, 128, "Identity"),
+                ("pool", 2, 2, 0, "Max"), ("fc", 10, "Identity")]
+    else:                    # batch-normalised residual units: their 3x3 convolutions take the same form
+        spec = [("conv", 3, 1, 1, 64, "Rect"), ("res", "Rect"), ("projres", 128, 2, "Rect"), ("pool", 2, 2, 0, "Average"),
+                ("fc", 10, "Identity")]
+    return (WINO_DIMS, *configs._chain(WINO_DIMS, spec))
+
+
+@pytest.mark.parametrize("kind", ["plain", "bnorm"])
+def test_winograd_steps_match_direct_steps(dev, kind):
+    """Train steps whose 3x3 layers of 64 channels and more run in the Winograd form (forward and backward-data, what
+    the library picks by itself at this size) against the same steps with RHO_EXEC_DIRECT_CONV: same losses, counts,
+    parameters and momentum to rounding; the Winograd kernels did run in the first and not in the second.
+    Two fp32 paths that add in different orders are compared here, through ReLU masks (an activation within rounding
+    of zero changes side) and bias gradients (sums of 32768 deltas that largely cancel): relative L2 distance 2e-3 after the first step, 1e-2 after
+    the later ones, which start from parameters that already differ.
+    Parity of the form itself against the fp64-accumulating oracle is test_conv2d_winograd and, at the benchmark's
+    size through whole train steps, tests/test_gpu_bench_size.py."""
+    net = wino_net(kind)
+    batch, steps = 128, 3
+    kw = dict(step_size=0.01, momentum=("Update", 0.9), l2_reg_coef=5e-4)
+    say("winograd steps", kind)
+    (a, _), tags_a = profile_tags(lambda: run(net, batch, steps, False, 0x3141, kw, read_grads=False))
+    (b, _), tags_b = profile_tags(lambda: run(net, batch, steps, False, 0x3141, kw, read_grads=False, winograd=False))
+    assert "conv_fwd_wino" in tags_a and "conv_bwd_data_wino" in tags_a and "wino_transform" in tags_a
+    assert not any("wino" in t for t in tags_b)
+    for step, ((la, ca, pa), (lb, cb, pb)) in enumerate(zip(a, b)):
+        assert abs(la - lb) <= 1e-4 * max(1.0, abs(lb)), (step, la, lb)
+        assert abs(ca - cb) <= 1, (step, ca, cb)
+        for k, (u, v) in enumerate(zip(pa, pb)):
+            u, v = u.astype(np.float64), v.astype(np.float64)
+            dist = np.sqrt(((u - v) ** 2).sum()) / max(np.sqrt((v ** 2).sum()), 1e-30)
+            assert dist <= (2e-3 if step == 0 else 1e-2), "%s step %d buffer %d: relative L2 distance %.3g" % (kind, step, k, dist)
