@@ -166,6 +166,113 @@ struct WinoEpi {
   FastDiv dTQ, dTP;
 };
 
+// A^T M A per (row, tile) with A^T = [1 1 1 0; 0 1 -1 -1], then the blend, bias, ReLU / mask, and the 2x2 pixels out.
+// acc[f] holds M_f of rows m0 + 32 wave .. + 31 x tiles n0 .. n0 + 31 in the MFMA's accumulator layout.
+__device__ __forceinline__ void wino_epilogue(const f32x16 (&acc)[16], const WinoEpi& ep, int m0, unsigned n0, int wave, int lane) {
+  const int h = lane >> 5, r = lane & 31;
+  const unsigned t = n0 + (unsigned)r;
+  uint32_t q1, tx, n, ty;
+  ep.dTQ.divmod(t, q1, tx);
+  ep.dTP.divmod(q1, n, ty);
+  const int PQ = ep.P * ep.Q;
+  const int row_lane = m0 + wave * 32 + 4 * h;     // + 8 (e / 4) + e % 4
+  const int rows_left = ep.Ko - row_lane;
+  uint32_t voff[2][2];
+#pragma unroll
+  for (int ai = 0; ai < 2; ++ai)
+#pragma unroll
+    for (int bi = 0; bi < 2; ++bi) {
+      const bool ok = t < ep.tiles && 2 * (int)ty + ai < ep.P && 2 * (int)tx + bi < ep.Q;
+      voff[ai][bi] = ok ? ((n * (unsigned)ep.Ko + 4u * (unsigned)h) * (unsigned)PQ + (2u * ty + ai) * (unsigned)ep.Q + 2u * tx + bi) * 4u
+                        : kInvalidByteOff;
+    }
+  const __amdgpu_buffer_rsrc_t rout = make_rsrc(ep.out, ep.out_bytes);
+  const __amdgpu_buffer_rsrc_t rmask = make_rsrc(ep.mask ? ep.mask : ep.out, ep.out_bytes);
+  const __amdgpu_buffer_rsrc_t rbias = make_rsrc(ep.bias ? ep.bias : ep.out, ep.bias ? 4u * (unsigned)ep.Ko : 0u);
+  float bv[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int re = 8 * (e >> 2) + (e & 3);
+    bv[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rbias, (row_lane + re) * 4, 0, 0));
+  }
+  const int srow = (m0 + wave * 32) * PQ * 4;   // wave-uniform byte offset of the wave's first row
+  const bool blend = ep.beta != 0.0f, masked = ep.mask != nullptr;
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) {
+    __builtin_amdgcn_sched_barrier(0);   // (a block's 64 accumulator values are read when its turn comes, not all 256 up front)
+    float y[4][2][2];
+    uint32_t vo[4][2][2];
+    float aux[4][2][2];   // mask values, or the old result
+#pragma unroll
+    for (int e4 = 0; e4 < 4; ++e4) {
+      const int e = 4 * eb + e4, re = 8 * eb + e4;
+      float s0[4], s1[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s0[j] = acc[j][e] + acc[4 + j][e] + acc[8 + j][e];
+        s1[j] = acc[4 + j][e] - acc[8 + j][e] - acc[12 + j][e];
+      }
+      y[e4][0][0] = s0[0] + s0[1] + s0[2];
+      y[e4][0][1] = s0[1] - s0[2] - s0[3];
+      y[e4][1][0] = s1[0] + s1[1] + s1[2];
+      y[e4][1][1] = s1[1] - s1[2] - s1[3];
+      const bool row_ok = re < rows_left;
+#pragma unroll
+      for (int ai = 0; ai < 2; ++ai)
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+          vo[e4][ai][bi] = row_ok ? voff[ai][bi] : kInvalidByteOff;
+          y[e4][ai][bi] *= ep.alpha;
+        }
+    }
+    if (masked || blend) {
+      // (both at once: the mask first, then the old values, block by block; neither occurs in a train step's forward pass)
+#pragma unroll
+      for (int e4 = 0; e4 < 4; ++e4)
+#pragma unroll
+        for (int ai = 0; ai < 2; ++ai)
+#pragma unroll
+          for (int bi = 0; bi < 2; ++bi)
+            aux[e4][ai][bi] = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(blend ? rout : rmask, (int)vo[e4][ai][bi], srow + (8 * eb + e4) * PQ * 4, 0));
+    }
+#pragma unroll
+    for (int e4 = 0; e4 < 4; ++e4)
+#pragma unroll
+      for (int ai = 0; ai < 2; ++ai)
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+          float x = y[e4][ai][bi];
+          if (blend) x = fmaf(ep.beta, aux[e4][ai][bi], x);
+          x += bv[4 * eb + e4];
+          if (ep.relu) x = fmaxf(x, 0.0f);
+          if (masked && !blend) x = aux[e4][ai][bi] > 0.0f ? x : 0.0f;
+          y[e4][ai][bi] = x;
+        }
+    if (masked && blend) {
+#pragma unroll
+      for (int e4 = 0; e4 < 4; ++e4)
+#pragma unroll
+        for (int ai = 0; ai < 2; ++ai)
+#pragma unroll
+          for (int bi = 0; bi < 2; ++bi) {
+            const float mk = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rmask, (int)vo[e4][ai][bi], srow + (8 * eb + e4) * PQ * 4, 0));
+            y[e4][ai][bi] = mk > 0.0f ? y[e4][ai][bi] : 0.0f;
+          }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e4 = 0; e4 < 4; ++e4)
+#pragma unroll
+      for (int ai = 0; ai < 2; ++ai)
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi)
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, y[e4][ai][bi]), rout, (int)vo[e4][ai][bi],
+                                                srow + (8 * eb + e4) * PQ * 4, 0);
+  }
+}
+
 constexpr int kWinoSA = 16 * 2 * kWinoBM * 8, kWinoSB = 16 * 2 * kWinoBN * 8, kWinoStage = kWinoSA + kWinoSB;
 constexpr int kWinoCnt = 10;   // direct loads per thread and stage: 8 of U, 2 of V
 
@@ -304,107 +411,239 @@ __global__ __launch_bounds__(256, 1) void wino_gemm_kernel(const float* __restri
   for (; it + 2 < nk; ++it) step(it, std::true_type());
   for (; it < nk; ++it) step(it, std::false_type());
 
-  // ---- epilogue: A^T M A per (row, tile), A^T = [1 1 1 0; 0 1 -1 -1] -------------------------------------------------
-  const unsigned t = n0 + (unsigned)r;
-  uint32_t q1, tx, n, ty;
-  ep.dTQ.divmod(t, q1, tx);
-  ep.dTP.divmod(q1, n, ty);
-  const int PQ = ep.P * ep.Q;
-  const int row_lane = m0 + wave * 32 + 4 * h;     // + 8 (e / 4) + e % 4
-  const int rows_left = ep.Ko - row_lane;
-  uint32_t voff[2][2];
-#pragma unroll
-  for (int ai = 0; ai < 2; ++ai)
-#pragma unroll
-    for (int bi = 0; bi < 2; ++bi) {
-      const bool ok = t < ep.tiles && 2 * (int)ty + ai < ep.P && 2 * (int)tx + bi < ep.Q;
-      voff[ai][bi] = ok ? ((n * (unsigned)ep.Ko + 4u * (unsigned)h) * (unsigned)PQ + (2u * ty + ai) * (unsigned)ep.Q + 2u * tx + bi) * 4u
-                        : kInvalidByteOff;
-    }
-  const __amdgpu_buffer_rsrc_t rout = make_rsrc(ep.out, ep.out_bytes);
-  const __amdgpu_buffer_rsrc_t rmask = make_rsrc(ep.mask ? ep.mask : ep.out, ep.out_bytes);
-  const __amdgpu_buffer_rsrc_t rbias = make_rsrc(ep.bias ? ep.bias : ep.out, ep.bias ? 4u * (unsigned)ep.Ko : 0u);
-  float bv[16];
-#pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int re = 8 * (e >> 2) + (e & 3);
-    bv[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rbias, (row_lane + re) * 4, 0, 0));
+  wino_epilogue(acc, ep, m0, n0, wave, lane);
+}
+
+// ---- the same product with B^T d B made inside the kernel ------------------------------------------------------------
+// No V in memory: a stage's image operand (4 channels x 32 tiles x 16 f) is computed by the block from the image's
+// patches.  Wave w owns channel 4 cg + w of the stage, lane = (tile, half): a thread brings three rows of its tile's
+// 4x4 patch (rows half .. half + 2, what two rows of B^T d need) as twelve 4-byte direct loads into a per-thread LDS
+// slot, three stages ahead of their use; one stage ahead it reads them back, forms its two rows of B^T d B (8 values)
+// and writes them where the MFMA operand reads expect them.  Out-of-image taps (padding, tiles hanging over the edge)
+// are out-of-range buffer offsets: they arrive as zeros.  All vector memory traffic of the loop is direct-to-LDS
+// loads counted by hand; everything else is LDS and register work the compiler sees.
+struct WinoImage {
+  const float* x; unsigned x_bytes; int Ci, Hi, Wi, halo;
+};
+
+constexpr int kWinoRaw = 12 * 256 * 4;             // bytes of one stage's raw patch rows
+constexpr int kWinoFusedCnt = 20;                  // direct loads per thread and stage: 12 patch dwords, 8 of U
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma_load4(u32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+__global__ __launch_bounds__(256, 1) void wino_gemm_fused_kernel(const float* __restrict__ U, WinoImage im, int Cg, int rows_p,
+                                                                int tiles_m, unsigned u_bytes, WinoEpi ep) {
+  constexpr int R = kWinoR;
+  extern __shared__ float lds_dyn[];   // [R stages: U | V][2 raw patch slots]
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_dyn;
+  const uint32_t raw0 = lds0 + (uint32_t)R * kWinoStage;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, r = lane & 31;
+  const int logical = __builtin_amdgcn_readfirstlane(xcd_remap(blockIdx.x, gridDim.x));
+  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  const int m0 = tile_m * kWinoBM;
+  const unsigned n0 = (unsigned)tile_n * kWinoBN;
+
+  u32x4 rsU, rsX;
+  {
+    const uint64_t pu = reinterpret_cast<uint64_t>(U), px = reinterpret_cast<uint64_t>(im.x);
+    rsU.x = __builtin_amdgcn_readfirstlane((uint32_t)pu);
+    rsU.y = __builtin_amdgcn_readfirstlane((uint32_t)(pu >> 32) & 0xffffu);
+    rsU.z = u_bytes; rsU.w = 0x00020000u;
+    rsX.x = __builtin_amdgcn_readfirstlane((uint32_t)px);
+    rsX.y = __builtin_amdgcn_readfirstlane((uint32_t)(px >> 32) & 0xffffu);
+    rsX.z = im.x_bytes; rsX.w = 0x00020000u;
   }
-  const int srow = (m0 + wave * 32) * PQ * 4;   // wave-uniform byte offset of the wave's first row
-  const bool blend = ep.beta != 0.0f, masked = ep.mask != nullptr;
+  const uint32_t voffA = (uint32_t)m0 * 8u + (uint32_t)lane * 16u;
+  const uint32_t strideA = 2u * (uint32_t)rows_p * 8u;
+  uint32_t soA[8];
 #pragma unroll
-  for (int eb = 0; eb < 4; ++eb) {
-    float y[4][2][2];
-    uint32_t vo[4][2][2];
-    float aux[4][2][2];   // mask values, or the old result
+  for (int i = 0; i < 8; ++i) {
+    const int idx = wave * 8 + i;
+    soA[i] = ((uint32_t)(idx >> 1) * (uint32_t)Cg * 2u + (uint32_t)(idx & 1)) * (uint32_t)rows_p * 8u;
+  }
+  // this thread's twelve patch taps: rows h .. h + 2 of the 4x4 patch of tile n0 + r, as byte offsets in channel 0 of its image
+  const int HW = im.Hi * im.Wi;
+  uint32_t poff[3][4];
+  {
+    const unsigned t = n0 + (unsigned)r;
+    uint32_t q1, tx, n, ty;
+    ep.dTQ.divmod(t, q1, tx);
+    ep.dTP.divmod(q1, n, ty);
 #pragma unroll
-    for (int e4 = 0; e4 < 4; ++e4) {
-      const int e = 4 * eb + e4, re = 8 * eb + e4;
-      float s0[4], s1[4];
+    for (int a = 0; a < 3; ++a)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        s0[j] = acc[j][e] + acc[4 + j][e] + acc[8 + j][e];
-        s1[j] = acc[4 + j][e] - acc[8 + j][e] - acc[12 + j][e];
+      for (int k = 0; k < 4; ++k) {
+        const int hh = 2 * (int)ty - im.halo + h + a, ww = 2 * (int)tx - im.halo + k;
+        const bool in = t < ep.tiles && (unsigned)hh < (unsigned)im.Hi && (unsigned)ww < (unsigned)im.Wi;
+        poff[a][k] = in ? ((n * (unsigned)im.Ci) * (unsigned)HW + (unsigned)(hh * im.Wi + ww)) * 4u : kInvalidByteOff;
       }
-      y[e4][0][0] = s0[0] + s0[1] + s0[2];
-      y[e4][0][1] = s0[1] - s0[2] - s0[3];
-      y[e4][1][0] = s1[0] + s1[1] + s1[2];
-      y[e4][1][1] = s1[1] - s1[2] - s1[3];
-      const bool row_ok = re < rows_left;
-#pragma unroll
-      for (int ai = 0; ai < 2; ++ai)
-#pragma unroll
-        for (int bi = 0; bi < 2; ++bi) {
-          vo[e4][ai][bi] = row_ok ? voff[ai][bi] : kInvalidByteOff;
-          y[e4][ai][bi] *= ep.alpha;
-        }
-    }
-    if (masked || blend) {
-      // (both at once: the mask first, then the old values, block by block; neither occurs in a train step's forward pass)
-#pragma unroll
-      for (int e4 = 0; e4 < 4; ++e4)
-#pragma unroll
-        for (int ai = 0; ai < 2; ++ai)
-#pragma unroll
-          for (int bi = 0; bi < 2; ++bi)
-            aux[e4][ai][bi] = __builtin_bit_cast(
-                float, __builtin_amdgcn_raw_buffer_load_b32(blend ? rout : rmask, (int)vo[e4][ai][bi], srow + (8 * eb + e4) * PQ * 4, 0));
-    }
-#pragma unroll
-    for (int e4 = 0; e4 < 4; ++e4)
-#pragma unroll
-      for (int ai = 0; ai < 2; ++ai)
-#pragma unroll
-        for (int bi = 0; bi < 2; ++bi) {
-          float x = y[e4][ai][bi];
-          if (blend) x = fmaf(ep.beta, aux[e4][ai][bi], x);
-          x += bv[4 * eb + e4];
-          if (ep.relu) x = fmaxf(x, 0.0f);
-          if (masked && !blend) x = aux[e4][ai][bi] > 0.0f ? x : 0.0f;
-          y[e4][ai][bi] = x;
-        }
-    if (masked && blend) {
-#pragma unroll
-      for (int e4 = 0; e4 < 4; ++e4)
-#pragma unroll
-        for (int ai = 0; ai < 2; ++ai)
-#pragma unroll
-          for (int bi = 0; bi < 2; ++bi) {
-            const float mk = __builtin_bit_cast(
-                float, __builtin_amdgcn_raw_buffer_load_b32(rmask, (int)vo[e4][ai][bi], srow + (8 * eb + e4) * PQ * 4, 0));
-            y[e4][ai][bi] = mk > 0.0f ? y[e4][ai][bi] : 0.0f;
-          }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int e4 = 0; e4 < 4; ++e4)
-#pragma unroll
-      for (int ai = 0; ai < 2; ++ai)
-#pragma unroll
-        for (int bi = 0; bi < 2; ++bi)
-          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, y[e4][ai][bi]), rout, (int)vo[e4][ai][bi],
-                                                srow + (8 * eb + e4) * PQ * 4, 0);
   }
+  const uint32_t chan_stride = (uint32_t)HW * 4u;
+  // direct load i (0..11: patch taps into raw slot `par`; 12..19: U into ring buffer `buf`) of stage cg
+  auto issue_one = [&](int i, int cg, int buf, int par) {
+    if (i < 12)
+      dma_load4(rsX, raw0 + (uint32_t)par * kWinoRaw + (uint32_t)i * 1024u + (uint32_t)wave * 256u, poff[i >> 2][i & 3],
+                (uint32_t)(4 * cg + wave) * chan_stride);
+    else
+      dma_load16(rsU, lds0 + (uint32_t)buf * kWinoStage + (uint32_t)(wave * 8 + (i - 12)) * 1024u, voffA,
+                 soA[i - 12] + (uint32_t)cg * strideA);
+  };
+  // the thread's part of stage s's image operand: raw slot s & 1 -> two rows of B^T d B -> V area of ring buffer buf
+  const float* rawp = lds_dyn + R * (kWinoStage / 4) + tid;
+  const int fe = h ? 12 : 0, fo = h ? 8 : 4;   // first f of the row made from d(a0) - d(a2), and of the other one
+  float* const vdst = lds_dyn + kWinoSA / 4 + (wave >> 1) * (kWinoBN * 2) + r * 2 + (wave & 1);
+  float da[3][4];
+  auto raw_read = [&](int par, int a) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) da[a][k] = rawp[par * (kWinoRaw / 4) + (a * 4 + k) * 256];
+  };
+  float te[4], to[4];
+  auto transform_cols = [&]() {   // the column pass: this thread's two rows of B^T d
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      te[k] = da[0][k] - da[2][k];
+      to[k] = h ? da[1][k] - da[0][k] : da[1][k] + da[2][k];
+    }
+  };
+  auto transform_row = [&](int which, int buf) {   // the row pass of one of them, into the V area of ring buffer buf
+    float* d = vdst + buf * (kWinoStage / 4) + (which ? fo : fe) * 128;   // an f is 2 x 32 x 2 floats
+    const float* t = which ? to : te;
+    d[0 * 128] = t[0] - t[2];
+    d[1 * 128] = t[1] + t[2];
+    d[2 * 128] = t[2] - t[1];
+    d[3 * 128] = t[1] - t[3];
+  };
+
+  f32x16 acc[16];
+#pragma unroll
+  for (int f = 0; f < 16; ++f)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[f][v] = 0.0f;
+
+  const int nk = Cg;
+  // Stages 0 and 1 on their way, their image operands made, the taps of stage 2 on their way (into the slot stage
+  // 0's were read from): the taps run three stages ahead of the MFMAs, U two.
+#pragma unroll
+  for (int i = 0; i < kWinoFusedCnt; ++i) issue_one(i, 0, 0, 0);
+  if (nk > 1) {
+#pragma unroll
+    for (int i = 0; i < kWinoFusedCnt; ++i) issue_one(i, 1, 1, 1);
+  }
+  wait_vmcnt<0>();
+  __builtin_amdgcn_sched_barrier(0);
+  raw_read(0, 0); raw_read(0, 1); raw_read(0, 2);
+  transform_cols();
+  transform_row(0, 0);
+  transform_row(1, 0);
+  if (nk > 1) {
+    raw_read(1, 0); raw_read(1, 1); raw_read(1, 2);
+    transform_cols();
+    transform_row(0, 1);
+    transform_row(1, 1);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  if (nk > 2) {
+#pragma unroll
+    for (int i = 0; i < 12; ++i) issue_one(i, 2, 2, 0);
+  }
+  __syncthreads();
+
+  const int a_rd = h * (kWinoBM * 2) + (wave * 32 + r) * 2;
+  const int b_rd = h * (kWinoBN * 2) + r * 2;
+  auto stage_a = [&](int buf) { return reinterpret_cast<const float2*>(lds_dyn + buf * (kWinoStage / 4) + a_rd); };
+  auto stage_b = [&](int buf) { return reinterpret_cast<const float2*>(lds_dyn + buf * (kWinoStage / 4) + kWinoSA / 4 + b_rd); };
+  float2 a[2][4], b[2][4];
+  {
+    const float2* pa = stage_a(0);
+    const float2* pb = stage_b(0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      a[0][q] = pa[q * kWinoBM * 2];
+      b[0][q] = pb[q * kWinoBN * 2];
+    }
+  }
+
+  // Stage `it`: MFMAs on ring buffer rd.  Behind them, one instruction or two per MFMA, in issue order:
+  //   groups 0, 1 (first half):  the patch taps of stage it + 3 (12 loads) into raw slot (it + 1) & 1;
+  //   groups 1 (second half), 2 (first half):  U of stage it + 2 (8 loads) into ring buffer wr;
+  //   group 2:  stage it + 2's taps (issued a stage and a half ago) read back from raw slot it & 1;
+  //   group 3, first half:  B^T d B of those, written into ring buffer wr: nobody reads it before the barrier of
+  //   stage it + 1, so none of this stands between a stage's last operand reads and the next stage's first;
+  //   then the stage's one barrier, which also waits for U of stage it + 1; second half: the first operands of stage it + 1.
+  int rd = 0, nx = 1, wr = 2, par = 0;   // ring buffers of stages it, it + 1, it + 2; raw slot of stage it + 2 (= it & 1)
+  auto step = [&](int it, auto ip_tag, auto iu_tag) {
+    constexpr bool IP = decltype(ip_tag)::value;       // there is a stage it + 3: its taps are issued here
+    constexpr bool IU = decltype(iu_tag)::value;       // there is a stage it + 2: its U is issued and its image operand made here
+    const float2* pa = stage_a(rd);
+    const float2* pb = stage_b(rd);
+    const float2* pna = stage_a(nx);
+    const float2* pnb = stage_b(nx);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int c = g & 1, n = c ^ 1;
+      __builtin_amdgcn_sched_barrier(0);
+      if (g == 2 && IU) {
+        // Stage it + 2's taps are there once all but the loads issued after them are: the taps of stage it + 3 (12)
+        // and the first four loads of U of stage it + 2.  (U of stage it + 1 lies between them except in stage 0, and
+        // need not be waited for yet; it was issued a stage ago and the barrier below needs it anyway.)
+        wait_vmcnt<(IP ? 12 : 0) + 4>();
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[4 * g + q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c][q].x, b[c][q].x, acc[4 * g + q], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g < 3) {
+          a[n][q] = pa[(4 * (g + 1) + q) * kWinoBM * 2];
+          b[n][q] = pb[(4 * (g + 1) + q) * kWinoBN * 2];
+        }
+        if (IP && g < 2) issue_one(8 * g + q, it + 3, 0, par ^ 1);          // taps 0-3, 8-11
+        if (IU && g == 2) issue_one(16 + q, it + 2, wr, 0);                 // U 4-7
+        if (IU && g == 2 && q < 3) raw_read(par, q);
+        if (IU && g == 3) {
+          if (q == 0) transform_cols();
+          if (q == 1) transform_row(0, wr);
+          if (q == 2) transform_row(1, wr);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (g == 3) {
+        // every wave has read all of stage `it` once it is here; U of stage it + 1 is complete when only the loads
+        // issued after it are in flight
+        wait_vmcnt<(IP ? 12 : 0) + (IU ? 8 : 0)>();
+        __syncthreads();
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[4 * g + q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c][q].y, b[c][q].y, acc[4 * g + q], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g == 3) {
+          a[n][q] = pna[q * kWinoBM * 2];
+          b[n][q] = pnb[q * kWinoBN * 2];
+        }
+        if (IP && g == 0) issue_one(4 + q, it + 3, 0, par ^ 1);             // taps 4-7
+        if (IU && g == 1) issue_one(12 + q, it + 2, wr, 0);                 // U 0-3
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    const int t = rd; rd = nx; nx = wr; wr = t;
+    par ^= 1;
+  };
+  int it = 0;
+  for (; it + 3 < nk; ++it) step(it, std::true_type(), std::true_type());
+  if (it + 2 < nk) { step(it, std::false_type(), std::true_type()); ++it; }
+  for (; it < nk; ++it) step(it, std::false_type(), std::false_type());
+
+  wino_epilogue(acc, ep, m0, n0, wave, lane);
 }
 
 }  // namespace
@@ -426,12 +665,14 @@ int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* 
   a.dTQ = FastDiv((uint32_t)g.TQ); a.dTP = FastDiv((uint32_t)g.TP);
   const unsigned long long fi = (unsigned long long)g.Cg * 2 * g.rows_p, ii = (unsigned long long)g.Cg * 2 * (g.tiles_p / 2);
   if (fi >= (1ull << 31) || ii >= (1ull << 31)) return RH_E_LIMIT;
-  a.filt_items = (unsigned)fi; a.in_items = (unsigned)ii;
-  a.in_blocks = (unsigned)cdiv<unsigned long long>(ii, 256);
+  // channel counts that fill groups of four take the kernel that makes V itself: only the filter is prepared here
+  const bool fused = g.Ci % 4 == 0;
+  a.filt_items = (unsigned)fi; a.in_items = fused ? 0u : (unsigned)ii;
+  a.in_blocks = (unsigned)cdiv<unsigned long long>(a.in_items, 256);
   const unsigned filt_blocks = (unsigned)cdiv<unsigned long long>(fi, 256);
   {
-    ProfScope prof("wino_transform", 4.0 * ((double)g.N * g.Ci * g.Hi * g.Wi + 9.0 * g.Ko * g.Ci) +
-                                         128.0 * ((double)g.Cg * g.rows_p + (double)g.Cg * g.tiles_p), stream);
+    ProfScope prof("wino_transform", 4.0 * ((fused ? 0.0 : (double)g.N * g.Ci * g.Hi * g.Wi) + 9.0 * g.Ko * g.Ci) +
+                                         128.0 * ((double)g.Cg * g.rows_p + (fused ? 0.0 : (double)g.Cg * g.tiles_p)), stream);
     hipLaunchKernelGGL(wino_prep_kernel, dim3(a.in_blocks + filt_blocks), dim3(256), 0, stream, a);
     if (int e = launch_status()) return e;
   }
@@ -440,6 +681,21 @@ int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* 
   ep.Ko = g.Ko; ep.P = g.P; ep.Q = g.Q; ep.tiles = (unsigned)g.tiles;
   ep.out_bytes = (unsigned)(4ull * (unsigned long long)g.N * g.Ko * g.P * g.Q);
   ep.dTQ = a.dTQ; ep.dTP = a.dTP;
+  const int tiles_m_ = g.rows_p / kWinoBM;
+  const long long tiles_n_ = g.tiles_p / kWinoBN;
+  if (fused) {
+    constexpr size_t lds_f = (size_t)kWinoR * kWinoStage + 2 * (size_t)kWinoRaw;
+    static_assert(lds_f <= 160 * 1024, "ring and patch slots do not fit the 160 KB LDS of a CU");
+    static const hipError_t attr_f = hipFuncSetAttribute(reinterpret_cast<const void*>(&wino_gemm_fused_kernel),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_f);
+    if (attr_f != hipSuccess) return (int)attr_f;
+    WinoImage im;
+    im.x = in; im.x_bytes = a.x_bytes; im.Ci = g.Ci; im.Hi = g.Hi; im.Wi = g.Wi; im.halo = g.halo;
+    ProfScope prof(tag, 2.0 * 16.0 * (double)g.Ko * g.Ci * (double)g.tiles, stream);
+    hipLaunchKernelGGL(wino_gemm_fused_kernel, dim3((unsigned)(tiles_m_ * tiles_n_)), dim3(256), lds_f, stream, U, im, g.Cg,
+                       g.rows_p, tiles_m_, (unsigned)(16ull * g.Cg * 2 * g.rows_p * 8), ep);
+    return launch_status();
+  }
   constexpr size_t lds_bytes = (size_t)kWinoR * kWinoStage;
   static_assert(lds_bytes <= 160 * 1024, "the ring does not fit the 160 KB LDS of a CU");
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&wino_gemm_kernel),
