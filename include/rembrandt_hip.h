@@ -139,6 +139,13 @@ size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass);
  * batch.  The need is not monotone in N (a pass with few result tiles cuts its contraction into slices and keeps
  * their partial sums in the scratch), so this can exceed rh_conv2d_workspace_bytes of g itself. */
 size_t rh_conv2d_workspace_bytes_upto(const rh_conv_geom* g, int pass);
+/* FLOPs (2 per multiply-add) that pass RH_CONV_FWD or RH_CONV_BWD_DATA executes on this geometry when the library takes
+ * the Winograd F(2x2, 3x3) form for it under `flags` (16 multiply-adds per 2x2 output tile, filter and channel; tiles
+ * that hang over an odd extent count whole), 0 when it takes a direct form.  The direct form's count is
+ * 2 * N*K*P*Q * C*R*S.  No counterpart in the reference (cuDNN picks its algorithm through cudnnGet*Algorithm,
+ * src/operator/mod.rs:1629-1661, and never says what it costs). */
+double rh_conv2d_winograd_flops(const rh_conv_geom* g, int pass, int flags);
+
 /* y = alpha * corr(x, w) + beta * y.  With RH_FUSE_BIAS, `bias` (length K) is added after the
  * alpha/beta blend; with RH_FUSE_RELU the result is clamped at 0.  bias may be NULL otherwise. */
 int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x, const float* w, float beta,

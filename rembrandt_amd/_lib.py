@@ -84,6 +84,7 @@ PROTOTYPES = {
     "rh_bnorm_bwd_relu": (_int, [_int, _int, _int, _f, _f, _vp, _vp, _vp, _f, _f, C.c_double, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _sz, _vp]),
     "rh_conv2d_out_dim": (_i32, [_i32, _i32, _i32, _i32]),
+    "rh_conv2d_winograd_flops": (C.c_double, [C.POINTER(ConvGeom), _int, _int]),
     "rh_conv2d_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _int]),
     "rh_conv2d_workspace_bytes_upto": (_sz, [C.POINTER(ConvGeom), _int]),
     "rh_conv2d_bwd_bias_workspace_bytes_upto": (_sz, [_i32, _i32, _i32]),

@@ -713,3 +713,15 @@ int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* 
 }
 
 }  // namespace rh
+
+using namespace rh;
+
+extern "C" double rh_conv2d_winograd_flops(const rh_conv_geom* g, int pass, int flags) {
+  ConvDims d;
+  if (conv_dims(g, &d) || !wino_shape(d) || (pass != RH_CONV_FWD && pass != RH_CONV_BWD_DATA)) return 0.0;
+  if (flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT)) return 0.0;
+  const WinoGeom wg = pass == RH_CONV_FWD ? wino_geom_fwd(d) : wino_geom_bwd_data(d);
+  if (!(flags & RH_ALGO_WINOGRAD ? wg.ok : wino_pays(wg))) return 0.0;
+  return 2.0 * 16.0 * (double)wg.Ko * wg.Ci * (double)wg.tiles;
+}
+

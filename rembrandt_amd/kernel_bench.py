@@ -80,11 +80,16 @@ def main(argv=None):
         torch.cuda.synchronize()
         return s.elapsed_time(e) / args.iters
 
-    def report(kernel, layer, ms, work, bound):
+    def report(kernel, layer, ms, work, bound, executed=0.0):
+        """executed: the FLOPs the call executes where that is not `work` (the Winograd form of a 3x3 layer: `achieved`
+        stays the direct form's multiply-adds per second, `frac` is what the kernel executes against the peak)."""
         unit = "GB/s" if bound == "hbm" else "TFLOP/s"
         achieved = work / ms / (1e6 if bound == "hbm" else 1e9)
-        print(json.dumps({"kernel": kernel, "layer": layer, "ms": round(ms, 4), "achieved": round(achieved, 1), "unit": unit,
-                          "peak": PEAK[bound], "frac": round(achieved / PEAK[bound], 4)}), flush=True)
+        rec = {"kernel": kernel, "layer": layer, "ms": round(ms, 4), "achieved": round(achieved, 1), "unit": unit,
+               "peak": PEAK[bound], "frac": round((executed or work) / ms / (1e6 if bound == "hbm" else 1e9) / PEAK[bound], 4)}
+        if executed:
+            rec.update({"form": "winograd F(2x2,3x3)", "executed": round(executed / ms / 1e9, 1)})
+        print(json.dumps(rec), flush=True)
 
     if "conv" in args.what:
         for name, (N, C, H, W, K, R, st, pad) in CONV_LAYERS.items():
@@ -98,13 +103,15 @@ def main(argv=None):
             dy = torch.randn_like(y)
             flops = 2.0 * y.numel() * C * R * R
             if "fwd" in passes:
-                report("conv_fwd", name, timeit(lambda: ops.conv2d_fwd(x, w, st, pad, y=y)), flops, "fp32")
+                report("conv_fwd", name, timeit(lambda: ops.conv2d_fwd(x, w, st, pad, y=y)), flops, "fp32",
+                       ops.conv2d_winograd_flops(x.shape, w.shape, st, pad, "fwd"))
             if "bwd_filter" in passes:
                 dw = torch.zeros_like(w)
                 report("conv_bwd_filter", name, timeit(lambda: ops.conv2d_bwd_filter(x, dy, w.shape, st, pad, dw=dw)), flops, "fp32")
             if "bwd_data" in passes:
                 dx = torch.zeros_like(x)
-                report("conv_bwd_data", name, timeit(lambda: ops.conv2d_bwd_data(w, dy, x.shape, st, pad, dx=dx)), flops, "fp32")
+                report("conv_bwd_data", name, timeit(lambda: ops.conv2d_bwd_data(w, dy, x.shape, st, pad, dx=dx)), flops, "fp32",
+                       ops.conv2d_winograd_flops(x.shape, w.shape, st, pad, "bwd_data"))
             if "fwd_bf16" in passes:
                 report("conv_fwd_bf16", name,
                        timeit(lambda: ops.conv2d_fwd(x, w, st, pad, y=y, algo=_lib.RH_MATH_BF16_MFMA_FP32ACC)), flops, "bf16")

@@ -84,6 +84,7 @@ extern "C" {
 
   pub fn rh_conv2d_out_dim(input: i32, size: i32, stride: i32, pad: i32) -> i32;
   pub fn rh_pool2d_out_dim(input: i32, size: i32, stride: i32, pad: i32, round: i32) -> i32;
+  pub fn rh_conv2d_winograd_flops(g: *const rh_conv_geom, pass: c_int, flags: c_int) -> f64;
   pub fn rh_conv2d_workspace_bytes(g: *const rh_conv_geom, pass: c_int) -> size_t;
   pub fn rh_conv2d_workspace_bytes_upto(g: *const rh_conv_geom, pass: c_int) -> size_t;
   pub fn rh_conv2d_fwd(g: *const rh_conv_geom, alpha: c_float, x: *const f32, w: *const f32, beta: c_float,
