@@ -48,7 +48,7 @@ typedef void* rh_stream_t; /* hipStream_t */
 #define RH_ALGO_GATHER             0x100 /* k -> {offset, dr, ds} table gather straight from the NCHW tensors      */
 #define RH_ALGO_SCALAR_OFFSET      0x200 /* scalar-offset loads on padded / transposed copies in the workspace,
                                             wherever the geometry allows it (else the gather family)             */
-#define RH_ALGO_WINOGRAD           0x400 /* conv fwd / bwd-data of a 3x3 stride-1 layer by Winograd F(2x2, 3x3): 2.25x
+#define RH_ALGO_WINOGRAD           0x400 /* every pass of a 3x3 stride-1 layer by Winograd F(2x2, 3x3): 2.25x
                                             fewer multiply-adds, sums in another order (RH_E_UNSUPPORTED for other
                                             geometries).  Without an RH_ALGO_* bit the library takes it for such layers
                                             of 64 channels and more on both sides; either bit above keeps the direct form */
@@ -139,7 +139,7 @@ size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass);
  * batch.  The need is not monotone in N (a pass with few result tiles cuts its contraction into slices and keeps
  * their partial sums in the scratch), so this can exceed rh_conv2d_workspace_bytes of g itself. */
 size_t rh_conv2d_workspace_bytes_upto(const rh_conv_geom* g, int pass);
-/* FLOPs (2 per multiply-add) that pass RH_CONV_FWD or RH_CONV_BWD_DATA executes on this geometry when the library takes
+/* FLOPs (2 per multiply-add) that a pass (RH_CONV_FWD, RH_CONV_BWD_DATA, RH_CONV_BWD_FILTER) executes on this geometry when the library takes
  * the Winograd F(2x2, 3x3) form for it under `flags` (16 multiply-adds per 2x2 output tile, filter and channel; tiles
  * that hang over an odd extent count whole), 0 when it takes a direct form.  The direct form's count is
  * 2 * N*K*P*Q * C*R*S.  No counterpart in the reference (cuDNN picks its algorithm through cudnnGet*Algorithm,

@@ -819,8 +819,14 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
       }
       return need;
     }
-    case RH_CONV_BWD_FILTER:
-      return bwd_filter_plan_bytes(d) + bwd_filter_bias_bytes(d);
+    case RH_CONV_BWD_FILTER: {
+      size_t need = bwd_filter_plan_bytes(d);
+      if (wino_shape(d)) {
+        const WinoFilterPlan wp = plan_wino_bwd_filter(d);
+        if (wp.ok && wp.total() > need) need = wp.total();
+      }
+      return need + bwd_filter_bias_bytes(d);
+    }
     default:
       return 0;
   }
@@ -851,6 +857,16 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     return RH_E_WORKSPACE;
   hipStream_t stream = to_stream(stream_);
 
+  if ((flags & RH_ALGO_WINOGRAD) && (!wino_shape(d) || (flags & (RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))))
+    return RH_E_UNSUPPORTED;
+  if (wino_shape(d) && !(flags & (RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))) {
+    const WinoFilterPlan wp = plan_wino_bwd_filter(d);
+    if (flags & RH_ALGO_WINOGRAD ? wp.ok : wino_filter_pays(d, wp)) {
+      if (d.w_elems == 0) return 0;
+      return launch_conv_wino_bwd_filter(d, wp, x, dy, dw, alpha, beta, ws, stream);
+    }
+    if (flags & RH_ALGO_WINOGRAD) return RH_E_UNSUPPORTED;
+  }
   const BwdFilterSoffPlan sp = plan_bwd_filter_soff(d);
   if (sp.ok && !(flags & RH_ALGO_GATHER) && ((flags & RH_ALGO_SCALAR_OFFSET) || use_soff_bwd_filter(d))) {
     const int CRSs = d.C * d.R * d.S, Ms = d.N * d.P * d.Q;

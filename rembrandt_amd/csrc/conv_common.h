@@ -313,6 +313,21 @@ inline WinoGeom wino_geom_bwd_data(const ConvDims& d) { return wino_geom(d.N, d.
 inline bool wino_pays(const WinoGeom& g) {
   return g.ok && g.Ci >= 64 && g.Ko >= 64 && (long long)(g.rows_p / kWinoBM) * (g.tiles_p / kWinoBN) >= 192;
 }
+// Filter gradient in the same form: zero-bordered copies of x and dy, S slices of the tiles, their partial sums.
+struct WinoFilterPlan {
+  bool ok;
+  int TP, TQ, Kp, Cp, S, stages;   // S slices of `stages` tile groups (of four tiles) each
+  long long tiles, TGs;            // tiles; tile groups over all slices
+  size_t vt_bytes, dyt_bytes, part_bytes;
+  size_t total() const { return vt_bytes + dyt_bytes + part_bytes; }
+};
+WinoFilterPlan plan_wino_bwd_filter(const ConvDims& d);
+// Where the library takes it by itself: as for the other two passes, and few enough slices for their traffic not to matter.
+inline bool wino_filter_pays(const ConvDims& d, const WinoFilterPlan& p) {
+  return p.ok && d.C >= 64 && d.K >= 64 && p.tiles >= 4096;
+}
+int launch_conv_wino_bwd_filter(const ConvDims& d, const WinoFilterPlan& p, const float* x, const float* dy, float* dw, float alpha,
+                                float beta, void* ws, hipStream_t stream);
 int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* w, float* out, float alpha, float beta,
                      const float* bias, int relu, const float* mask, void* ws, hipStream_t stream, const char* tag);
 

@@ -168,7 +168,25 @@ struct WinoEpi {
 
 // A^T M A per (row, tile) with A^T = [1 1 1 0; 0 1 -1 -1], then the blend, bias, ReLU / mask, and the 2x2 pixels out.
 // acc[f] holds M_f of rows m0 + 32 wave .. + 31 x tiles n0 .. n0 + 31 in the MFMA's accumulator layout.
-__device__ __forceinline__ void wino_epilogue(const f32x16 (&acc)[16], const WinoEpi& ep, int m0, unsigned n0, int wave, int lane) {
+// (Accumulators live in the accumulation registers, which ordinary arithmetic cannot read; left alone the compiler
+// copies all 256 to ordinary registers behind the loop and the kernel's allocation becomes all 512 registers of a SIMD
+// lane: nothing else can run on a CU beside it.  wino_pin_acc says "these are still in accumulation registers here"
+// in front of every block of the epilogue, so that a block's 64 values are fetched when its turn comes and the
+// allocation stays near 360: a bandwidth-bound kernel of another stream finds room on the same CUs.)
+__device__ __forceinline__ void wino_pin_acc(f32x16 (&acc)[16]) {
+#pragma unroll
+  for (int f = 0; f < 16; ++f) asm volatile("" : "+a"(acc[f]));
+}
+
+// One accumulator element, fetched where it is used (written as the instruction itself: as an ordinary element access
+// the compiler moves whole 16-register tuples out of the accumulation registers ahead of time).
+__device__ __forceinline__ float wino_acc_elem(const f32x16& v, int e) {
+  float r;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(v[e]));
+  return r;
+}
+
+__device__ __forceinline__ void wino_epilogue(f32x16 (&acc)[16], const WinoEpi& ep, int m0, unsigned n0, int wave, int lane) {
   const int h = lane >> 5, r = lane & 31;
   const unsigned t = n0 + (unsigned)r;
   uint32_t q1, tx, n, ty;
@@ -197,20 +215,24 @@ __device__ __forceinline__ void wino_epilogue(const f32x16 (&acc)[16], const Win
   }
   const int srow = (m0 + wave * 32) * PQ * 4;   // wave-uniform byte offset of the wave's first row
   const bool blend = ep.beta != 0.0f, masked = ep.mask != nullptr;
+  constexpr int EB = 4;   // accumulator elements per block (loads of a block stand ahead of its stores)
 #pragma unroll
-  for (int eb = 0; eb < 4; ++eb) {
-    __builtin_amdgcn_sched_barrier(0);   // (a block's 64 accumulator values are read when its turn comes, not all 256 up front)
-    float y[4][2][2];
-    uint32_t vo[4][2][2];
-    float aux[4][2][2];   // mask values, or the old result
+  for (int eb = 0; eb < 16 / EB; ++eb) {
+    __builtin_amdgcn_sched_barrier(0);
+    wino_pin_acc(acc);
+    float y[EB][2][2];
+    uint32_t vo[EB][2][2];
+    float aux[EB][2][2];   // mask values, or the old result
 #pragma unroll
-    for (int e4 = 0; e4 < 4; ++e4) {
-      const int e = 4 * eb + e4, re = 8 * eb + e4;
+    for (int e4 = 0; e4 < EB; ++e4) {
+      const int e = EB * eb + e4, re = 8 * (e >> 2) + (e & 3);
       float s0[4], s1[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        s0[j] = acc[j][e] + acc[4 + j][e] + acc[8 + j][e];
-        s1[j] = acc[4 + j][e] - acc[8 + j][e] - acc[12 + j][e];
+        const float m0j = wino_acc_elem(acc[j], e), m1j = wino_acc_elem(acc[4 + j], e), m2j = wino_acc_elem(acc[8 + j], e),
+                    m3j = wino_acc_elem(acc[12 + j], e);
+        s0[j] = m0j + m1j + m2j;
+        s1[j] = m1j - m2j - m3j;
       }
       y[e4][0][0] = s0[0] + s0[1] + s0[2];
       y[e4][0][1] = s0[1] - s0[2] - s0[3];
@@ -228,48 +250,48 @@ __device__ __forceinline__ void wino_epilogue(const f32x16 (&acc)[16], const Win
     if (masked || blend) {
       // (both at once: the mask first, then the old values, block by block; neither occurs in a train step's forward pass)
 #pragma unroll
-      for (int e4 = 0; e4 < 4; ++e4)
+      for (int e4 = 0; e4 < EB; ++e4)
 #pragma unroll
         for (int ai = 0; ai < 2; ++ai)
 #pragma unroll
           for (int bi = 0; bi < 2; ++bi)
             aux[e4][ai][bi] = __builtin_bit_cast(
-                float, __builtin_amdgcn_raw_buffer_load_b32(blend ? rout : rmask, (int)vo[e4][ai][bi], srow + (8 * eb + e4) * PQ * 4, 0));
+                float, __builtin_amdgcn_raw_buffer_load_b32(blend ? rout : rmask, (int)vo[e4][ai][bi], srow + (8 * ((EB * eb + e4) >> 2) + ((EB * eb + e4) & 3)) * PQ * 4, 0));
     }
 #pragma unroll
-    for (int e4 = 0; e4 < 4; ++e4)
+    for (int e4 = 0; e4 < EB; ++e4)
 #pragma unroll
       for (int ai = 0; ai < 2; ++ai)
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi) {
           float x = y[e4][ai][bi];
           if (blend) x = fmaf(ep.beta, aux[e4][ai][bi], x);
-          x += bv[4 * eb + e4];
+          x += bv[EB * eb + e4];
           if (ep.relu) x = fmaxf(x, 0.0f);
           if (masked && !blend) x = aux[e4][ai][bi] > 0.0f ? x : 0.0f;
           y[e4][ai][bi] = x;
         }
     if (masked && blend) {
 #pragma unroll
-      for (int e4 = 0; e4 < 4; ++e4)
+      for (int e4 = 0; e4 < EB; ++e4)
 #pragma unroll
         for (int ai = 0; ai < 2; ++ai)
 #pragma unroll
           for (int bi = 0; bi < 2; ++bi) {
             const float mk = __builtin_bit_cast(
-                float, __builtin_amdgcn_raw_buffer_load_b32(rmask, (int)vo[e4][ai][bi], srow + (8 * eb + e4) * PQ * 4, 0));
+                float, __builtin_amdgcn_raw_buffer_load_b32(rmask, (int)vo[e4][ai][bi], srow + (8 * ((EB * eb + e4) >> 2) + ((EB * eb + e4) & 3)) * PQ * 4, 0));
             y[e4][ai][bi] = mk > 0.0f ? y[e4][ai][bi] : 0.0f;
           }
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int e4 = 0; e4 < 4; ++e4)
+    for (int e4 = 0; e4 < EB; ++e4)
 #pragma unroll
       for (int ai = 0; ai < 2; ++ai)
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi)
           __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, y[e4][ai][bi]), rout, (int)vo[e4][ai][bi],
-                                                srow + (8 * eb + e4) * PQ * 4, 0);
+                                                srow + (8 * ((EB * eb + e4) >> 2) + ((EB * eb + e4) & 3)) * PQ * 4, 0);
   }
 }
 
@@ -646,6 +668,351 @@ __global__ __launch_bounds__(256, 1) void wino_gemm_fused_kernel(const float* __
   wino_epilogue(acc, ep, m0, n0, wave, lane);
 }
 
+// ---- filter gradient --------------------------------------------------------------------------------------------------
+//   dg = G^T [ sum over tiles (A dY A^T) o (B^T d B) ] G      A dY A^T: the 2x2 tile of dy -> 4x4,  A = [1 0; 1 1; 1 -1; 0 -1]
+// The same 16 products with the roles turned: rows = filters, columns = input channels, the contraction runs over
+// the tiles, four to a stage.  A tile's patch and its dy taps are a few floats in each of hundreds of planes: loaded
+// where they lie they are one cache line per lane and 4 bytes used of each (measured: 2 us per stage instead of 1).
+// So a prep launch (wino_filter_prep_kernel) writes both operands tile-major:
+//   Vt[f][tile / 4][h][channel][2] = B^T d B in the product's operand order (tile = 4 (tile / 4) + 2 h + j), which goes
+//      straight to LDS like U in the forward kernel;
+//   dyt[tile][filter][4] = the tile's four dy taps, 16 bytes a filter: a lane (= a filter) brings two tiles' taps as two
+//      16-byte direct loads into its LDS slot two stages ahead, reads them back a stage ahead, forms A dY A^T of both
+//      (12 VALU instructions a tile) and writes the 16 pairs into the next stage's ring buffer.
+// Zeros for the tiles the count is rounded up with, for taps past an odd extent, for filters and channels up to
+// whole blocks.  The last row of A is taken as (0, 1) instead of (0, -1): no negations in the loop; the reduction flips
+// the sign of the f that have exactly one index 3.  Few (filters x channels) tiles exist (36 for 384 x 384), so the
+// image's tiles are cut into S slices, one block each; the slices' partial dU go to scratch and
+// wino_filter_reduce_kernel adds them in slice order, applies G^T . G and the alpha / beta blend.
+struct WinoFilterArgs {
+  const float* Vt; const float* dyt; float* part;
+  unsigned vt_bytes, dyt_bytes, part_bytes;
+  int Kp, Cp, TGs;                // padded filter / channel counts, tile groups (stages) over all slices
+  int tiles_m, tiles_c, stages;   // stages (of four tiles) per slice
+};
+
+constexpr int kWinoFRaw = 2 * 256 * 16;   // bytes of one stage's dy taps: two tiles x 16 bytes per thread
+constexpr int kWinoFCnt = 4;              // direct loads per thread and stage: 2 of dy taps, 2 of Vt
+
+__global__ __launch_bounds__(256, 1) void wino_bwd_filter_kernel(WinoFilterArgs p) {
+  constexpr int R = kWinoR;
+  extern __shared__ float lds_dyn[];   // [R stages: A | B][2 raw slots]
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_dyn;
+  const uint32_t raw0 = lds0 + (uint32_t)R * kWinoStage;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, r = lane & 31;
+  const int logical = __builtin_amdgcn_readfirstlane(xcd_remap(blockIdx.x, gridDim.x));
+  const int tile_m = logical % p.tiles_m, rest = logical / p.tiles_m;
+  const int tile_c = rest % p.tiles_c, split = rest / p.tiles_c;
+  const int m0 = tile_m * kWinoBM, c0 = tile_c * kWinoBN;
+  const uint32_t tg0 = (uint32_t)split * (uint32_t)p.stages;   // this slice's first tile group
+
+  u32x4 rsV, rsY;
+  {
+    const uint64_t pv = reinterpret_cast<uint64_t>(p.Vt), py = reinterpret_cast<uint64_t>(p.dyt);
+    rsV.x = __builtin_amdgcn_readfirstlane((uint32_t)pv);
+    rsV.y = __builtin_amdgcn_readfirstlane((uint32_t)(pv >> 32) & 0xffffu);
+    rsV.z = p.vt_bytes; rsV.w = 0x00020000u;
+    rsY.x = __builtin_amdgcn_readfirstlane((uint32_t)py);
+    rsY.y = __builtin_amdgcn_readfirstlane((uint32_t)(py >> 32) & 0xffffu);
+    rsY.z = p.dyt_bytes; rsY.w = 0x00020000u;
+  }
+  // dy taps: filter m0 + 64 (wave & 1) + lane of tiles 4 tg + 2 (wave / 2) + {0, 1}
+  const uint32_t voffY = (uint32_t)(m0 + 64 * (wave & 1) + lane) * 16u;
+  const uint32_t tileY = (uint32_t)p.Kp * 16u;   // bytes per tile of dyt
+  // Vt: wave-load idx = 2 wave + i covers f = 2 idx, 2 idx + 1 and both h: four runs of 32 channels x 8 bytes
+  const int seg = lane >> 4;
+  const uint32_t strideB = 2u * (uint32_t)p.Cp * 8u;   // bytes per tile group within one f
+  const uint32_t voffB = ((uint32_t)(seg >> 1) * (uint32_t)p.TGs * 2u + (uint32_t)(seg & 1)) * (uint32_t)p.Cp * 8u +
+                         (uint32_t)c0 * 8u + (uint32_t)(lane & 15) * 16u;
+  // direct load i of stage st (tile group tg0 + st): 0, 1 the dy taps of the wave's two tiles into raw slot par;
+  // 2, 3 Vt into ring buffer buf
+  auto issue_one = [&](int i, int st, int buf, int par) {
+    const uint32_t tg = tg0 + (uint32_t)st;
+    if (i < 2)
+      dma_load16(rsY, raw0 + (uint32_t)par * kWinoFRaw + (uint32_t)i * 4096u + (uint32_t)wave * 1024u, voffY,
+                 (4u * tg + 2u * (uint32_t)(wave >> 1) + (uint32_t)i) * tileY);
+    else
+      dma_load16(rsV, lds0 + (uint32_t)buf * kWinoStage + kWinoSA + (uint32_t)(wave * 2 + (i - 2)) * 1024u, voffB,
+                 ((uint32_t)(2 * (wave * 2 + (i - 2))) * (uint32_t)p.TGs + tg) * strideB);
+  };
+  const float4* rawp = reinterpret_cast<const float4*>(lds_dyn + R * (kWinoStage / 4)) + tid;
+  float4 yv[2];
+  auto raw_read = [&](int par) {
+    yv[0] = rawp[par * (kWinoFRaw / 16)];
+    yv[1] = rawp[par * (kWinoFRaw / 16) + 256];
+  };
+  // A operand: [f][h'][128 filters][2 tiles], this thread's filter 64 (wave & 1) + lane, tile pair h' = wave / 2
+  float2* const adst = reinterpret_cast<float2*>(lds_dyn + (wave >> 1) * (kWinoBM * 2) + (64 * (wave & 1) + lane) * 2);
+  auto transform_y_rows = [&](int i0, int buf) {   // rows i0, i0 + 1 of A' dY A'^T of both tiles (taps: x y / z w)
+    float2* d = adst + buf * (kWinoStage / 8);
+#pragma unroll
+    for (int i = i0; i < i0 + 2; ++i) {
+      float ra[2], rb[2];   // row i of A' dY: (first column, second column), per tile
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        ra[j] = i == 0 ? yv[j].x : i == 1 ? yv[j].x + yv[j].z : i == 2 ? yv[j].x - yv[j].z : yv[j].z;
+        rb[j] = i == 0 ? yv[j].y : i == 1 ? yv[j].y + yv[j].w : i == 2 ? yv[j].y - yv[j].w : yv[j].w;
+      }
+      // an f is 2 x 128 x 2 floats = 256 float2
+      d[(4 * i + 0) * 256] = make_float2(ra[0], ra[1]);
+      d[(4 * i + 1) * 256] = make_float2(ra[0] + rb[0], ra[1] + rb[1]);
+      d[(4 * i + 2) * 256] = make_float2(ra[0] - rb[0], ra[1] - rb[1]);
+      d[(4 * i + 3) * 256] = make_float2(rb[0], rb[1]);
+    }
+  };
+
+  f32x16 acc[16];
+#pragma unroll
+  for (int f = 0; f < 16; ++f)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[f][v] = 0.0f;
+
+  const int nk = p.stages;
+  // stages 0 and 1 on their way (taps ahead of Vt, as in the loop), stage 0's A operand made
+#pragma unroll
+  for (int i = 0; i < kWinoFCnt; ++i) issue_one(i, 0, 0, 0);
+  if (nk > 1) {
+#pragma unroll
+    for (int i = 0; i < kWinoFCnt; ++i) issue_one(i, 1, 1, 1);
+  }
+  wait_vmcnt<0>();
+  __builtin_amdgcn_sched_barrier(0);
+  raw_read(0);
+  transform_y_rows(0, 0);
+  transform_y_rows(2, 0);
+  __syncthreads();
+
+  const int a_rd = h * (kWinoBM * 2) + (wave * 32 + r) * 2;
+  const int b_rd = h * (kWinoBN * 2) + r * 2;
+  auto stage_a = [&](int buf) { return reinterpret_cast<const float2*>(lds_dyn + buf * (kWinoStage / 4) + a_rd); };
+  auto stage_b = [&](int buf) { return reinterpret_cast<const float2*>(lds_dyn + buf * (kWinoStage / 4) + kWinoSA / 4 + b_rd); };
+  float2 a[2][4], b[2][4];
+  {
+    const float2* pa = stage_a(0);
+    const float2* pb = stage_b(0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      a[0][q] = pa[q * kWinoBM * 2];
+      b[0][q] = pb[q * kWinoBN * 2];
+    }
+  }
+
+  // Stage `it`: MFMAs on ring buffer rd.  Behind them: group 0, the four loads of stage it + 2 (taps into raw slot
+  // it & 1, Vt into ring buffer wr); group 2, stage it + 1's taps read back from the other slot; group 3 (first half), A
+  // dY A^T of those written into ring buffer nx; the stage's barrier, which also waits for Vt of stage it + 1; then the
+  // first operands of stage it + 1.
+  int rd = 0, nx = 1, wr = 2, par = 0;
+  auto step = [&](int it, auto i2_tag, auto t1_tag) {
+    constexpr bool I2 = decltype(i2_tag)::value;   // there is a stage it + 2: its loads are issued here
+    constexpr bool T1 = decltype(t1_tag)::value;   // there is a stage it + 1: its A operand is made here
+    const float2* pa = stage_a(rd);
+    const float2* pb = stage_b(rd);
+    const float2* pna = stage_a(nx);
+    const float2* pnb = stage_b(nx);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int c = g & 1, n = c ^ 1;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[4 * g + q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c][q].x, b[c][q].x, acc[4 * g + q], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g < 3) {
+          a[n][q] = pa[(4 * (g + 1) + q) * kWinoBM * 2];
+          b[n][q] = pb[(4 * (g + 1) + q) * kWinoBN * 2];
+        }
+        if (I2 && g == 0) issue_one(q, it + 2, wr, par);
+        if (T1 && g == 3 && q < 2) transform_y_rows(2 * q, nx);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (g == 1 && T1) {
+        // stage it + 1's taps (the first two loads issued during stage it - 1) are there once only the two Vt loads
+        // behind them and this stage's four are in flight
+        if (I2) wait_vmcnt<6>();
+        else wait_vmcnt<2>();
+      }
+      if (g == 3) {
+        // every wave has read all of stage `it` and written its part of stage it + 1's A; Vt of stage it + 1 is complete
+        // when only this stage's loads are in flight
+        if (I2) wait_vmcnt<kWinoFCnt>();
+        else wait_vmcnt<0>();
+        __syncthreads();
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[4 * g + q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c][q].y, b[c][q].y, acc[4 * g + q], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g == 3) {
+          a[n][q] = pna[q * kWinoBM * 2];
+          b[n][q] = pnb[q * kWinoBN * 2];
+        }
+        if (T1 && g == 1 && q == 0) raw_read(par ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    const int t = rd; rd = nx; nx = wr; wr = t;
+    par ^= 1;
+  };
+  int it = 0;
+  for (; it + 2 < nk; ++it) step(it, std::true_type(), std::true_type());
+  if (it + 1 < nk) { step(it, std::false_type(), std::true_type()); ++it; }
+  if (it < nk) step(it, std::false_type(), std::false_type());
+
+  // this slice's partial dU: part[slice][f][filter][channel]
+  const __amdgpu_buffer_rsrc_t rpart = make_rsrc(p.part, p.part_bytes);
+  const uint32_t voff = ((uint32_t)(m0 + 32 * wave + 4 * h) * (uint32_t)p.Cp + (uint32_t)(c0 + r)) * 4u;
+  const uint32_t plane = (uint32_t)p.Kp * (uint32_t)p.Cp * 4u;
+#pragma unroll
+  for (int f = 0; f < 16; ++f) {
+    __builtin_amdgcn_sched_barrier(0);
+    wino_pin_acc(acc);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const float v = acc[f][e];   // (a copy: __builtin_bit_cast straight from the vector element takes element 0 every time)
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rpart, (int)voff,
+                                            (int)(((uint32_t)split * 16u + (uint32_t)f) * plane +
+                                                  (uint32_t)(8 * (e >> 2) + (e & 3)) * (uint32_t)p.Cp * 4u), 0);
+    }
+  }
+}
+
+// dw[k][c][r][s] = alpha * (G^T dU G)[r][s] + beta * dw, dU = the slices' partial sums added in slice order
+__global__ __launch_bounds__(256) void wino_filter_reduce_kernel(const float* __restrict__ part, int S, int K, int C, int Kp, int Cp,
+                                                               float alpha, float beta, float* __restrict__ dw) {
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  if (idx >= (unsigned)K * (unsigned)C) return;
+  const unsigned k = idx / (unsigned)C, c = idx - k * (unsigned)C;
+  const size_t plane = (size_t)Kp * Cp;
+  float u[16];
+#pragma unroll
+  for (int f = 0; f < 16; ++f) u[f] = 0.0f;
+  for (int sl = 0; sl < S; ++sl) {   // a slice's 16 values in flight together, the slices added in order
+    float v[16];
+#pragma unroll
+    for (int f = 0; f < 16; ++f) v[f] = part[((size_t)sl * 16 + f) * plane + (size_t)k * Cp + c];
+#pragma unroll
+    for (int f = 0; f < 16; ++f) u[f] += v[f];
+  }
+#pragma unroll
+  for (int f = 0; f < 16; ++f)
+    if (((f >> 2) == 3) != ((f & 3) == 3)) u[f] = -u[f];   // the sign the loop's (0, 1) for A's last row left out
+  float t[3][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    t[0][j] = u[j] + 0.5f * (u[4 + j] + u[8 + j]);
+    t[1][j] = 0.5f * (u[4 + j] - u[8 + j]);
+    t[2][j] = 0.5f * (u[4 + j] + u[8 + j]) + u[12 + j];
+  }
+  float* o = dw + (size_t)idx * 9;
+#pragma unroll
+  for (int rr = 0; rr < 3; ++rr) {
+    const float g0 = t[rr][0] + 0.5f * (t[rr][1] + t[rr][2]);
+    const float g1 = 0.5f * (t[rr][1] - t[rr][2]);
+    const float g2 = 0.5f * (t[rr][1] + t[rr][2]) + t[rr][3];
+    const float g[3] = {g0, g1, g2};
+#pragma unroll
+    for (int ss = 0; ss < 3; ++ss) o[rr * 3 + ss] = beta != 0.0f ? fmaf(beta, o[rr * 3 + ss], alpha * g[ss]) : alpha * g[ss];
+  }
+}
+
+// The filter gradient's operands, both in one launch (two kinds of blocks).
+struct WinoFilterPrepArgs {
+  const float* x; const float* dy; float* Vt; float* dyt;
+  unsigned x_bytes, dy_bytes;
+  int N, C, H, W, K, P, Q, halo, Kp, Cp, TGs;
+  unsigned tiles;
+  FastDiv dTQ, dTP, dPairs, dKp;
+  unsigned v_items, y_items, v_blocks;
+};
+
+// Vt of channels (2 ch, 2 ch + 1) x tiles (2 up, 2 up + 1): one 16-byte store per f, [channel][tile of the pair]
+__device__ __forceinline__ void wino_filter_v_item(const WinoFilterPrepArgs& a, unsigned idx) {
+  // eight neighbouring lanes take eight channel pairs of one tile pair (their stores are 128 consecutive bytes), the
+  // next eight the next tile pair (their loads are neighbours in eight planes)
+  uint32_t ch_hi, up;
+  a.dPairs.divmod(idx >> 3, ch_hi, up);   // up: tile pair = 2 (tile group) + h
+  const uint32_t ch = ch_hi * 8u + (idx & 7u);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, a.x_bytes);
+  float v[16][4];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    const unsigned t = 2 * up + tt;
+    uint32_t q1, tx, n, ty;
+    a.dTQ.divmod(t, q1, tx);
+    a.dTP.divmod(q1, n, ty);
+    const int h0 = 2 * (int)ty - a.halo, w0 = 2 * (int)tx - a.halo;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = (int)ch * 2 + j;
+      const bool live = t < a.tiles && c < a.C;
+      const unsigned base = (n * (unsigned)a.C + (unsigned)c) * (unsigned)(a.H * a.W);
+      float d[4][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int hh = h0 + i, ww = w0 + k;
+          const bool in = live && (unsigned)hh < (unsigned)a.H && (unsigned)ww < (unsigned)a.W;
+          const unsigned off = in ? (base + (unsigned)(hh * a.W + ww)) * 4u : kInvalidByteOff;
+          d[i][k] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)off, 0, 0));
+        }
+      float s[4][4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        s[0][k] = d[0][k] - d[2][k];
+        s[1][k] = d[1][k] + d[2][k];
+        s[2][k] = d[2][k] - d[1][k];
+        s[3][k] = d[1][k] - d[3][k];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[4 * i + 0][2 * j + tt] = s[i][0] - s[i][2];
+        v[4 * i + 1][2 * j + tt] = s[i][1] + s[i][2];
+        v[4 * i + 2][2 * j + tt] = s[i][2] - s[i][1];
+        v[4 * i + 3][2 * j + tt] = s[i][1] - s[i][3];
+      }
+    }
+  }
+  float4* V4 = reinterpret_cast<float4*>(a.Vt);
+  const size_t half_cp = (size_t)a.Cp / 2, plane = (size_t)a.TGs * 2 * half_cp;   // float4s per f
+#pragma unroll
+  for (int f = 0; f < 16; ++f) V4[f * plane + (size_t)up * half_cp + ch] = make_float4(v[f][0], v[f][1], v[f][2], v[f][3]);
+}
+
+// dyt[tile][filter] = the tile's four dy taps
+__device__ __forceinline__ void wino_filter_y_item(const WinoFilterPrepArgs& a, unsigned idx) {
+  uint32_t k_hi, t;   // (eight filters of one tile, then the next tile: as above)
+  a.dKp.divmod(idx >> 3, k_hi, t);
+  const uint32_t k = k_hi * 8u + (idx & 7u);
+  uint32_t q1, tx, n, ty;
+  a.dTQ.divmod(t, q1, tx);
+  a.dTP.divmod(q1, n, ty);
+  const __amdgpu_buffer_rsrc_t ry = make_rsrc(a.dy, a.dy_bytes);
+  const bool live = t < a.tiles && (int)k < a.K;
+  const unsigned base = (n * (unsigned)a.K + k) * (unsigned)(a.P * a.Q);
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int pp = 2 * (int)ty + (e >> 1), qq = 2 * (int)tx + (e & 1);
+    const bool in = live && pp < a.P && qq < a.Q;
+    const unsigned off = in ? (base + (unsigned)(pp * a.Q + qq)) * 4u : kInvalidByteOff;
+    v[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ry, (int)off, 0, 0));
+  }
+  reinterpret_cast<float4*>(a.dyt)[(size_t)t * a.Kp + k] = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+__global__ __launch_bounds__(256) void wino_filter_prep_kernel(WinoFilterPrepArgs a) {
+  if (blockIdx.x < a.v_blocks) {
+    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx < a.v_items) wino_filter_v_item(a, idx);
+  } else {
+    const unsigned idx = (blockIdx.x - a.v_blocks) * 256u + threadIdx.x;
+    if (idx < a.y_items) wino_filter_y_item(a, idx);
+  }
+}
+
 }  // namespace
 
 // in: (N, Ci, Hi, Wi) with g.halo zeros around; w: the layer's filter (K, C, 3, 3): forward reads it as (Ko, Ci), the
@@ -712,14 +1079,93 @@ int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* 
   return launch_status();
 }
 
+WinoFilterPlan plan_wino_bwd_filter(const ConvDims& d) {
+  WinoFilterPlan p;
+  p.ok = false;
+  if (!wino_shape(d) || d.P <= 0 || d.Q <= 0) return p;
+  p.TP = cdiv(d.P, 2); p.TQ = cdiv(d.Q, 2);
+  p.tiles = (long long)d.N * p.TP * p.TQ;
+  p.Kp = round_up(d.K, kWinoBM); p.Cp = round_up(d.C, kWinoBN);
+  const long long tiles_mc = (long long)(p.Kp / kWinoBM) * (p.Cp / kWinoBN);
+  const long long stages_all = (p.tiles + 3) / 4;
+  // slices: the count (16 at most, 32 stages a slice at least) that fills the 256 CUs best in whole rounds, the smaller
+  // one on a tie
+  int best = 1;
+  double best_fill = 0.0;
+  for (int S = 1; S <= 16 && (S == 1 || stages_all / S >= 32); ++S) {
+    const long long blocks = tiles_mc * S;
+    const double fill = (double)blocks / (double)(cdiv<long long>(blocks, 256) * 256);
+    if (fill > best_fill + 1e-9) { best_fill = fill; best = S; }
+  }
+  p.S = best;
+  p.stages = (int)cdiv<long long>(stages_all, p.S);
+  p.TGs = (long long)p.S * p.stages;
+  const unsigned long long vb = 16ull * p.TGs * 2 * p.Cp * 8, yb = 16ull * p.TGs * 4 * p.Kp;
+  const unsigned long long pb = 4ull * p.S * 16 * p.Kp * p.Cp;
+  p.vt_bytes = align256((size_t)vb); p.dyt_bytes = align256((size_t)yb); p.part_bytes = align256((size_t)pb);
+  p.ok = vb < (1ull << 31) && yb < (1ull << 31) && pb < (1ull << 31) && p.TGs * 4 < (1ll << 30);
+  return p;
+}
+
+int launch_conv_wino_bwd_filter(const ConvDims& d, const WinoFilterPlan& p, const float* x, const float* dy, float* dw, float alpha,
+                                float beta, void* ws, hipStream_t stream) {
+  if (!p.ok) return RH_E_UNSUPPORTED;
+  char* base = static_cast<char*>(ws);
+  float* Vt = reinterpret_cast<float*>(base);
+  float* dyt = reinterpret_cast<float*>(base + p.vt_bytes);
+  float* part = reinterpret_cast<float*>(base + p.vt_bytes + p.dyt_bytes);
+  {
+    WinoFilterPrepArgs a;
+    a.x = x; a.dy = dy; a.Vt = Vt; a.dyt = dyt;
+    a.x_bytes = (unsigned)(4ull * d.x_elems); a.dy_bytes = (unsigned)(4ull * d.y_elems);
+    a.N = d.N; a.C = d.C; a.H = d.H; a.W = d.W; a.K = d.K; a.P = d.P; a.Q = d.Q; a.halo = d.pad;
+    a.Kp = p.Kp; a.Cp = p.Cp; a.TGs = (int)p.TGs; a.tiles = (unsigned)p.tiles;
+    a.dTQ = FastDiv((uint32_t)p.TQ); a.dTP = FastDiv((uint32_t)p.TP);
+    a.dPairs = FastDiv((uint32_t)(p.TGs * 2)); a.dKp = FastDiv((uint32_t)(p.TGs * 4));   // (dKp: tiles, the divisor of the dy items)
+    const unsigned long long vi = (unsigned long long)(p.Cp / 2) * (p.TGs * 2), yi = (unsigned long long)p.TGs * 4 * p.Kp;
+    if (vi >= (1ull << 31) || yi >= (1ull << 31)) return RH_E_LIMIT;
+    a.v_items = (unsigned)vi; a.y_items = (unsigned)yi;
+    a.v_blocks = (unsigned)cdiv<unsigned long long>(vi, 256);
+    ProfScope prof("wino_filter_prep", 4.0 * ((double)d.x_elems + (double)d.y_elems) + 128.0 * (double)p.TGs * p.Cp + 16.0 * (double)yi, stream);
+    hipLaunchKernelGGL(wino_filter_prep_kernel, dim3(a.v_blocks + (unsigned)cdiv<unsigned long long>(yi, 256)), dim3(256), 0, stream, a);
+    if (int e = launch_status()) return e;
+  }
+  WinoFilterArgs a;
+  a.Vt = Vt; a.dyt = dyt; a.part = part;
+  a.vt_bytes = (unsigned)(16ull * p.TGs * 2 * p.Cp * 8); a.dyt_bytes = (unsigned)(16ull * p.TGs * 4 * p.Kp);
+  a.part_bytes = (unsigned)(4ull * p.S * 16 * p.Kp * p.Cp);
+  a.Kp = p.Kp; a.Cp = p.Cp; a.TGs = (int)p.TGs;
+  a.tiles_m = p.Kp / kWinoBM; a.tiles_c = p.Cp / kWinoBN; a.stages = p.stages;
+  constexpr size_t lds_b = (size_t)kWinoR * kWinoStage + 2 * (size_t)kWinoFRaw;
+  static_assert(lds_b <= 160 * 1024, "ring and tap slots do not fit the 160 KB LDS of a CU");
+  static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&wino_bwd_filter_kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_b);
+  if (attr != hipSuccess) return (int)attr;
+  {
+    ProfScope prof("conv_bwd_filter_wino", 2.0 * 16.0 * (double)d.K * d.C * (double)p.tiles, stream);
+    hipLaunchKernelGGL(wino_bwd_filter_kernel, dim3((unsigned)(a.tiles_m * a.tiles_c * p.S)), dim3(256), lds_b, stream, a);
+    if (int e = launch_status()) return e;
+  }
+  ProfScope prof("wino_filter_reduce", 4.0 * (16.0 * p.S + 9.0) * (double)d.K * d.C, stream);
+  hipLaunchKernelGGL(wino_filter_reduce_kernel, dim3(cdiv((unsigned)(d.K * d.C), 256u)), dim3(256), 0, stream, part, p.S, d.K, d.C,
+                     p.Kp, p.Cp, alpha, beta, dw);
+  return launch_status();
+}
+
 }  // namespace rh
 
 using namespace rh;
 
 extern "C" double rh_conv2d_winograd_flops(const rh_conv_geom* g, int pass, int flags) {
   ConvDims d;
-  if (conv_dims(g, &d) || !wino_shape(d) || (pass != RH_CONV_FWD && pass != RH_CONV_BWD_DATA)) return 0.0;
+  if (conv_dims(g, &d) || !wino_shape(d)) return 0.0;
   if (flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT)) return 0.0;
+  if (pass == RH_CONV_BWD_FILTER) {
+    const WinoFilterPlan wp = plan_wino_bwd_filter(d);
+    if (!(flags & RH_ALGO_WINOGRAD ? wp.ok : wino_filter_pays(d, wp))) return 0.0;
+    return 2.0 * 16.0 * (double)d.K * d.C * (double)wp.tiles;
+  }
+  if (pass != RH_CONV_FWD && pass != RH_CONV_BWD_DATA) return 0.0;
   const WinoGeom wg = pass == RH_CONV_FWD ? wino_geom_fwd(d) : wino_geom_bwd_data(d);
   if (!(flags & RH_ALGO_WINOGRAD ? wg.ok : wino_pays(wg))) return 0.0;
   return 2.0 * 16.0 * (double)wg.Ko * wg.Ci * (double)wg.tiles;

@@ -901,6 +901,7 @@ class Conv2dOperator : public Operator {
       w_filter = w_bias = workspace_aux_.get();
     }
     const float beta = params_.take_backward_beta();   // 1: accumulate (the reference's call); 0: the buffers stand for zeros
+    const int algo = opts_.winograd ? 0 : RH_ALGO_DIRECT;
     if (!in_delta_ && workspace_aux_ && overlap_on_) {
       // First layer, backward on two streams: its gradients are the last kernels of the pass.  The bias gradient goes
       // first (a memory-bound pass beside the second stream's last contraction), so that only the filter gradient's
@@ -909,15 +910,15 @@ class Conv2dOperator : public Operator {
                                    out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
                                    w_bias->len(), s_bias), "conv2d backward bias");
       unwrap(rh_conv2d_bwd_filter(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta, params_.grad_weights->as_mut_ptr(),
-                                  w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter");
+                                  w_filter->as_mut_ptr(), w_filter->len(), algo, s_filter), "conv2d backward filter");
     } else if (s_filter == s_bias && w_filter == w_bias) {
       // one stream for both: one call, which reads out_delta once where the filter gradient makes a pass over it anyway
       unwrap(rh_conv2d_bwd_filter_bias(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta,
                                        params_.grad_weights->as_mut_ptr(), params_.grad_bias->as_mut_ptr(),
-                                       w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter / bias");
+                                       w_filter->as_mut_ptr(), w_filter->len(), algo, s_filter), "conv2d backward filter / bias");
     } else {
       unwrap(rh_conv2d_bwd_filter(&g, scale, in_act_->as_ptr(), out_delta_->as_ptr(), beta, params_.grad_weights->as_mut_ptr(),
-                                  w_filter->as_mut_ptr(), w_filter->len(), 0, s_filter), "conv2d backward filter");
+                                  w_filter->as_mut_ptr(), w_filter->len(), algo, s_filter), "conv2d backward filter");
       unwrap(rh_conv2d_bwd_bias_ws((int)batch_size, (int)out_dims_.c, (int)(out_dims_.w * out_dims_.h), scale,
                                    out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
                                    w_bias->len(), s_bias), "conv2d backward bias");
@@ -1358,7 +1359,7 @@ struct BNormConvUnit {
       wg = ws_aux;
     }
     unwrap(rh_conv2d_bwd_filter(&g, 1.0f, in, pre_delta->as_ptr(), 1.0f, grad_weights->as_mut_ptr(), wg->as_mut_ptr(),
-                                wg->len(), 0, sg), "conv2d backward filter");
+                                wg->len(), conv_algo, sg), "conv2d backward filter");
   }
   size_t aux_workspace_bytes() const {
     const rh_conv_geom g = geom(batch_cap);

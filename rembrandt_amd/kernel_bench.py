@@ -107,7 +107,8 @@ def main(argv=None):
                        ops.conv2d_winograd_flops(x.shape, w.shape, st, pad, "fwd"))
             if "bwd_filter" in passes:
                 dw = torch.zeros_like(w)
-                report("conv_bwd_filter", name, timeit(lambda: ops.conv2d_bwd_filter(x, dy, w.shape, st, pad, dw=dw)), flops, "fp32")
+                report("conv_bwd_filter", name, timeit(lambda: ops.conv2d_bwd_filter(x, dy, w.shape, st, pad, dw=dw)), flops, "fp32",
+                       ops.conv2d_winograd_flops(x.shape, w.shape, st, pad, "bwd_filter"))
             if "bwd_data" in passes:
                 dx = torch.zeros_like(x)
                 report("conv_bwd_data", name, timeit(lambda: ops.conv2d_bwd_data(w, dy, x.shape, st, pad, dx=dx)), flops, "fp32",

@@ -120,7 +120,7 @@ def conv2d_winograd_flops(x_shape, w_shape, stride, pad, which="fwd", algo=0):
     """FLOPs the pass executes when the library takes the Winograd form for this geometry, 0 for a direct form."""
     N, Cc, H, W = x_shape
     g = _lib.ConvGeom(N, Cc, H, W, w_shape[0], w_shape[2], w_shape[3], stride, pad)
-    return float(lib().rh_conv2d_winograd_flops(C.byref(g), {"fwd": 0, "bwd_data": 2}.get(which, 1), algo))
+    return float(lib().rh_conv2d_winograd_flops(C.byref(g), {"fwd": 0, "bwd_filter": 1, "bwd_data": 2}[which], algo))
 
 
 def conv2d_bwd_data_relu_supported(x_shape, w_shape, stride, pad):

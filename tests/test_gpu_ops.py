@@ -167,6 +167,7 @@ WINO_CASES = [
     (33, 64, 14, 15, 128, 1),
     (70, 66, 13, 13, 384, 1),     # 3 x 108 blocks
     (16, 128, 28, 28, 64, 1),
+    (90, 64, 13, 13, 128, 1),     # 4410 tiles: the filter gradient in the form too, its tiles in several slices
 ]
 
 
@@ -205,8 +206,22 @@ def test_conv2d_winograd(dev, case):
         ops.rect_backprop_inplace(xd, two)
         one = ops.conv2d_bwd_data(wd, dyd, x.shape, 1, pad, alpha=alpha, beta=beta, dx=T(dx0, dev), algo=WG, relu_of=xd)
         assert torch.equal(one, two), "winograd masked data gradient alpha=%g beta=%g" % (alpha, beta)
+    # the filter gradient in the same form (its sums run over the tiles, cut into slices added in a fixed order)
+    dw_ref = O.conv2d_bwd_filter(x, dy, w.shape, 1, pad)
+    dw = ops.conv2d_bwd_filter(xd, dyd, w.shape, 1, pad, algo=WG)
+    assert_close(N(dw), dw_ref, "winograd bwd filter")
+    dw0 = synth.normal(15, 6, w.shape)
+    for alpha, beta in ((1.0, 1.0), (0.25, 1.0), (-3.0, 0.5)):
+        dwa = ops.conv2d_bwd_filter(xd, dyd, w.shape, 1, pad, alpha=alpha, beta=beta, dw=T(dw0, dev), algo=WG)
+        assert_close(N(dwa), O.conv2d_bwd_filter(x, dy, w.shape, 1, pad, alpha, beta, dw0.copy()),
+                     "winograd bwd filter alpha=%g beta=%g" % (alpha, beta))
+    db0 = synth.normal(15, 7, (K,))
+    dwc, dbc = ops.conv2d_bwd_filter_bias(xd, dyd, w.shape, 1, pad, alpha=0.25, beta=1.0, dw=T(dw0, dev), db=T(db0, dev), algo=WG)
+    assert torch.equal(dwc, ops.conv2d_bwd_filter(xd, dyd, w.shape, 1, pad, alpha=0.25, beta=1.0, dw=T(dw0, dev), algo=WG))
+    assert_close(N(dbc), O.conv2d_bwd_bias(dy, 0.25, 1.0, db0.copy()), "bias gradient of the combined call (winograd)")
     # run to run the same bits
     assert torch.equal(ops.conv2d_fwd(xd, wd, 1, pad, algo=WG), y)
+    assert torch.equal(ops.conv2d_bwd_filter(xd, dyd, w.shape, 1, pad, algo=WG), dw)
     # what the library picks by itself: this form from 64 channels on both sides and 192 blocks on, else a direct one
     auto = ops.conv2d_fwd(xd, wd, 1, pad)
     direct = ops.conv2d_fwd(xd, wd, 1, pad, algo=_lib.RH_ALGO_DIRECT)
@@ -234,6 +249,9 @@ def test_conv2d_winograd_refused_geometries(dev):
             rc = _lib.lib().rh_conv2d_bwd_data(C.byref(g), 1.0, w.data_ptr(), y.data_ptr(), 0.0, x.data_ptr(), ws.data_ptr(), ws.numel(),
                                                _lib.RH_ALGO_WINOGRAD | extra, None)
             assert rc == _lib.RH_E_UNSUPPORTED, ("bwd", R, st, pad, extra, rc)
+            rc = _lib.lib().rh_conv2d_bwd_filter(C.byref(g), 1.0, x.data_ptr(), y.data_ptr(), 0.0, w.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                 _lib.RH_ALGO_WINOGRAD | extra, None)
+            assert rc == _lib.RH_E_UNSUPPORTED, ("bwd filter", R, st, pad, extra, rc)
 
 
 # input channels a multiple of 8 take the packed-operand form (bf16 copies of image and filter in 16-byte groups of

@@ -283,6 +283,7 @@ def test_winograd_steps_match_direct_steps(dev, kind):
     (a, _), tags_a = profile_tags(lambda: run(net, batch, steps, False, 0x3141, kw, read_grads=False))
     (b, _), tags_b = profile_tags(lambda: run(net, batch, steps, False, 0x3141, kw, read_grads=False, winograd=False))
     assert "conv_fwd_wino" in tags_a and "conv_bwd_data_wino" in tags_a and "wino_transform" in tags_a
+    assert "conv_bwd_filter_wino" in tags_a
     assert not any("wino" in t for t in tags_b)
     for step, ((la, ca, pa), (lb, cb, pb)) in enumerate(zip(a, b)):
         assert abs(la - lb) <= 1e-4 * max(1.0, abs(lb)), (step, la, lb)
