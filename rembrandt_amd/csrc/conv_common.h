@@ -311,7 +311,9 @@ inline WinoGeom wino_geom_bwd_data(const ConvDims& d) { return wino_geom(d.N, d.
 // Where the library takes it by itself: enough channels on both sides for the 16 products to be worth their
 // transforms, and a grid that fills the GPU.
 inline bool wino_pays(const WinoGeom& g) {
-  return g.ok && g.Ci >= 64 && g.Ko >= 64 && (long long)(g.rows_p / kWinoBM) * (g.tiles_p / kWinoBN) >= 192;
+  // (rows: 128-row tiles at least three quarters full: 64 filters in one would execute as much as the direct form)
+  return g.ok && g.Ci >= 64 && g.Ko >= 64 && 4 * g.Ko >= 3 * g.rows_p &&
+         (long long)(g.rows_p / kWinoBM) * (g.tiles_p / kWinoBN) >= 192;
 }
 // Filter gradient in the same form: zero-bordered copies of x and dy, S slices of the tiles, their partial sums.
 struct WinoFilterPlan {
@@ -324,7 +326,8 @@ struct WinoFilterPlan {
 WinoFilterPlan plan_wino_bwd_filter(const ConvDims& d);
 // Where the library takes it by itself: as for the other two passes, and few enough slices for their traffic not to matter.
 inline bool wino_filter_pays(const ConvDims& d, const WinoFilterPlan& p) {
-  return p.ok && d.C >= 64 && d.K >= 64 && p.tiles >= 4096;
+  return p.ok && d.C >= 64 && d.K >= 64 && 4 * d.K >= 3 * p.Kp && 4 * d.C >= 3 * p.Cp && p.tiles >= 4096 &&
+         (long long)(p.Kp / kWinoBM) * (p.Cp / kWinoBN) * p.S >= 192;
 }
 int launch_conv_wino_bwd_filter(const ConvDims& d, const WinoFilterPlan& p, const float* x, const float* dy, float* dw, float alpha,
                                 float beta, void* ws, hipStream_t stream);

@@ -1,5 +1,6 @@
-// 3x3 stride-1 convolutions by Winograd's minimal filtering F(2x2, 3x3): forward, and backward-data as the forward form
-// of the flipped, transposed filter over dy (CudnnConvFwdOp / CudnnConvBwdDataOp of a 3x3 layer, src/operator/mod.rs).
+// 3x3 stride-1 convolutions by Winograd's minimal filtering F(2x2, 3x3): forward, backward-data (the forward form of the
+// flipped, transposed filter over dy) and the filter gradient (CudnnConvFwdOp / CudnnConvBwdDataOp / CudnnConvBwdFilterOp
+// of a 3x3 layer, src/operator/mod.rs:1684-1696, 1765-1793).
 //
 //   Y = A^T [ (G g G^T) o (B^T d B) ] A      per 2x2 output tile, 4x4 input patch d, 3x3 filter g
 //
@@ -7,21 +8,26 @@
 // independent products  M_f (rows x tiles) = U_f (rows x channels) * V_f (channels x tiles),  f = 4i + j the position
 // in the 4x4 transformed patch, 2.25 times fewer multiply-adds than the direct form.
 //
-// Three kernels:
-//  * wino_prep_kernel (one launch, two kinds of blocks): U = G g G^T for every (row, channel) and V = B^T d B for every
-//    (channel, tile), both in the operand order of the product kernel, zeros where the patch leaves the image, for
-//    rows, channels and tiles that pad the operands to whole blocks;
-//  * wino_gemm_kernel: a block of four waves owns 128 rows x 32 tiles for all 16 f; wave w holds rows 32w .. 32w+31 as
-//    16 accumulator tiles of v_mfma_f32_32x32x2_f32 (256 accumulator registers, one wave per SIMD).  Both operands go
-//    straight from memory to LDS (buffer_load_dwordx4 ... lds) into a ring of three stages of four channels each,
-//    two stages ahead of the MFMAs; the one barrier of a stage stands in front of its last quarter of MFMAs;
-//  * its epilogue: a lane's element e of the 16 accumulators is the whole 4x4 M of one (row, tile): A^T M A is 24
+// Forward / backward-data:
+//  * wino_prep_kernel: U = G g G^T for every (row, channel) in the operand order of the product kernel, zero rows and
+//    channels up to whole blocks (and V = B^T d B for channel counts that are no multiple of four, see below);
+//  * wino_gemm_fused_kernel: a block of four waves owns 128 rows x 32 tiles for all 16 f; wave w holds rows 32w .. 32w+31
+//    as 16 accumulator tiles of v_mfma_f32_32x32x2_f32 (256 accumulation registers, one wave per SIMD).  U goes straight
+//    from memory to LDS (buffer_load_dwordx4 ... lds) into a ring of three stages of four channels each, two stages
+//    ahead of the MFMAs; V is made in the kernel from the image's patches; the one barrier of a stage stands in front
+//    of its last quarter of MFMAs.  (wino_gemm_kernel: the same with V read from memory, for other channel counts.)
+//  * the epilogue: a lane's element e of the 16 accumulators is the whole 4x4 M of one (row, tile): A^T M A is 24
 //    additions in registers, then alpha / beta, bias, ReLU or the mask of a folded ReLU backward, and the 2x2 pixels
 //    go to the NCHW result (odd extents: the tile's pixels past the edge are dropped).
+// Filter gradient: wino_filter_prep_kernel, wino_bwd_filter_kernel, wino_filter_reduce_kernel, described further down.
 //
 // Operand layout (floats):  U[f][cg][h][rows_p][2],  V[f][cg][h][tiles_p][2]  with channel = 4 cg + 2 h + j.  The MFMA
 // takes A[row][k], B[k][col] with k = lane / 32: the half-wave h reads channel 4 cg + 2 h + j for the stage's MFMA j,
 // one 8-byte LDS read per operand and stage and f, each half-wave reading 256 consecutive bytes.
+//
+// A wave's own VALU instructions are not hidden behind its MFMAs (each one between two MFMAs adds its 4-7 cycles;
+// LDS, scalar and memory instructions there cost nothing), and these kernels run one wave per SIMD: the loops keep
+// vector arithmetic to the transforms themselves.
 #include "conv_common.h"
 
 namespace rh {
@@ -1088,11 +1094,12 @@ WinoFilterPlan plan_wino_bwd_filter(const ConvDims& d) {
   p.Kp = round_up(d.K, kWinoBM); p.Cp = round_up(d.C, kWinoBN);
   const long long tiles_mc = (long long)(p.Kp / kWinoBM) * (p.Cp / kWinoBN);
   const long long stages_all = (p.tiles + 3) / 4;
-  // slices: the count (16 at most, 32 stages a slice at least) that fills the 256 CUs best in whole rounds, the smaller
-  // one on a tie
+  // slices: the count (64 at most, 32 stages a slice at least, 128 MB of partial sums at most) that fills the 256 CUs
+  // best in whole rounds, the smaller one on a tie
   int best = 1;
   double best_fill = 0.0;
-  for (int S = 1; S <= 16 && (S == 1 || stages_all / S >= 32); ++S) {
+  const long long slice_bytes = 4ll * 16 * p.Kp * p.Cp;
+  for (int S = 1; S <= 64 && (S == 1 || (stages_all / S >= 32 && slice_bytes * S <= (128ll << 20))); ++S) {
     const long long blocks = tiles_mc * S;
     const double fill = (double)blocks / (double)(cdiv<long long>(blocks, 256) * 256);
     if (fill > best_fill + 1e-9) { best_fill = fill; best = S; }

@@ -288,8 +288,8 @@ struct ExecOptions {
   // of ten launches of a few microseconds of work each; only inside armed train steps with fused epilogues.  Same
   // buffers with the same meaning at every point the operators expose; sums in a different (fixed) order.
   bool fuse_tail = true;
-  // 3x3 stride-1 convolutions of 64 channels and more (forward and backward-data) by Winograd F(2x2, 3x3), where the
-  // library takes that form by itself; false keeps the direct form everywhere (RH_ALGO_DIRECT).
+  // 3x3 stride-1 convolutions of 64 channels and more (all three passes) by Winograd F(2x2, 3x3), where the library
+  // takes that form by itself; false keeps the direct form everywhere (RH_ALGO_DIRECT).
   bool winograd = true;
 };
 

@@ -222,12 +222,13 @@ def test_conv2d_winograd(dev, case):
     # run to run the same bits
     assert torch.equal(ops.conv2d_fwd(xd, wd, 1, pad, algo=WG), y)
     assert torch.equal(ops.conv2d_bwd_filter(xd, dyd, w.shape, 1, pad, algo=WG), dw)
-    # what the library picks by itself: this form from 64 channels on both sides and 192 blocks on, else a direct one
+    # what the library picks by itself: this form from 64 channels on both sides, 128-row tiles three quarters full and
+    # 192 blocks on, else a direct one
     auto = ops.conv2d_fwd(xd, wd, 1, pad)
     direct = ops.conv2d_fwd(xd, wd, 1, pad, algo=_lib.RH_ALGO_DIRECT)
     assert_close(N(direct), y_ref, "RH_ALGO_DIRECT fwd")
     blocks = -(-K // 128) * -(-(Nn * -(-y_ref.shape[2] // 2) * -(-y_ref.shape[3] // 2)) // 32)
-    takes = C >= 64 and K >= 64 and blocks >= 192
+    takes = C >= 64 and K >= 64 and 4 * K >= 3 * (-(-K // 128) * 128) and blocks >= 192
     assert torch.equal(auto, y if takes else direct), "library's choice"
     torch.cuda.synchronize()
 

@@ -258,22 +258,23 @@ WINO_DIMS = (16, 16, 8)
 
 def wino_net(kind):
     if kind == "plain":      # conv -> conv (ReLU backward folded into the second layer's data gradient) -> pool -> fc
-        spec = [("conv", 3, 1, 1, 64, "Rect"), ("conv", 3, 1, 1, 64, "Rect"), ("conv", 3, 1, 1, 128, "Identity"),
+        spec = [("conv", 3, 1, 1, 128, "Rect"), ("conv", 3, 1, 1, 128, "Rect"), ("conv", 3, 1, 1, 128, "Identity"),
                 ("pool", 2, 2, 0, "Max"), ("fc", 10, "Identity")]
     else:                    # batch-normalised residual units: their 3x3 convolutions take the same form
-        spec = [("conv", 3, 1, 1, 64, "Rect"), ("res", "Rect"), ("projres", 128, 2, "Rect"), ("pool", 2, 2, 0, "Average"),
+        spec = [("conv", 3, 1, 1, 128, "Rect"), ("res", "Rect"), ("projres", 256, 2, "Rect"), ("pool", 2, 2, 0, "Average"),
                 ("fc", 10, "Identity")]
     return (WINO_DIMS, *configs._chain(WINO_DIMS, spec))
 
 
 @pytest.mark.parametrize("kind", ["plain", "bnorm"])
 def test_winograd_steps_match_direct_steps(dev, kind):
-    """Train steps whose 3x3 layers of 64 channels and more run in the Winograd form (forward and backward-data, what
-    the library picks by itself at this size) against the same steps with RHO_EXEC_DIRECT_CONV: same losses, counts,
+    """Train steps whose 3x3 layers of 128 channels run in the Winograd form (all three passes, what the library picks
+    by itself at this size) against the same steps with RHO_EXEC_DIRECT_CONV: same losses, counts,
     parameters and momentum to rounding; the Winograd kernels did run in the first and not in the second.
     Two fp32 paths that add in different orders are compared here, through ReLU masks (an activation within rounding
     of zero changes side) and bias gradients (sums of 32768 deltas that largely cancel): relative L2 distance 2e-3 after the first step, 1e-2 after
-    the later ones, which start from parameters that already differ.
+    the later ones, which start from parameters that already differ (5e-2 behind batch normalisation, whose backward
+    pass subtracts means of nearly equal size: the first step, from identical parameters, is the kernels' comparison).
     Parity of the form itself against the fp64-accumulating oracle is test_conv2d_winograd and, at the benchmark's
     size through whole train steps, tests/test_gpu_bench_size.py."""
     net = wino_net(kind)
@@ -291,4 +292,5 @@ def test_winograd_steps_match_direct_steps(dev, kind):
         for k, (u, v) in enumerate(zip(pa, pb)):
             u, v = u.astype(np.float64), v.astype(np.float64)
             dist = np.sqrt(((u - v) ** 2).sum()) / max(np.sqrt((v ** 2).sum()), 1e-30)
-            assert dist <= (2e-3 if step == 0 else 1e-2), "%s step %d buffer %d: relative L2 distance %.3g" % (kind, step, k, dist)
+            bound = 2e-3 if step == 0 else 1e-2 if kind == "plain" else 5e-2
+            assert dist <= bound, "%s step %d buffer %d: relative L2 distance %.3g" % (kind, step, k, dist)
