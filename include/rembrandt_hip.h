@@ -53,6 +53,11 @@ typedef void* rh_stream_t; /* hipStream_t */
                                             geometries).  Without an RH_ALGO_* bit the library takes it for such layers
                                             of 64 channels and more on both sides; either bit above keeps the direct form */
 #define RH_ALGO_DIRECT             0x800 /* never the Winograd form; the direct forms chosen as without any RH_ALGO_* bit */
+#define RH_ALGO_SHARED_GPU         0x1000 /* a hint, with any of the above: kernels of another stream run beside this call.
+                                             Forms that spend compute-unit time to shorten the call's own last round of
+                                             blocks (the Winograd kernels' sliced tail blocks) are not taken: beside
+                                             other work the idle units of that round are not idle (measured: the
+                                             ResNet-18 template step 26.5 -> 26.1 ms).  Same result up to summation order. */
 
 const char* rh_version(void);
 /* Status of the most recent launch made by a void `rembrandt_kernel_*` entry point on this thread. */

@@ -14,6 +14,7 @@ RH_POOL_MAX, RH_POOL_AVG_INCL_PAD = 0, 1
 RH_ROUND_FLOOR, RH_ROUND_CEIL = 0, 1
 RH_FUSE_BIAS, RH_FUSE_RELU = 0x10, 0x20
 RH_ALGO_GATHER, RH_ALGO_SCALAR_OFFSET, RH_ALGO_WINOGRAD, RH_ALGO_DIRECT = 0x100, 0x200, 0x400, 0x800
+RH_ALGO_SHARED_GPU = 0x1000
 RH_MATH_BF16_MFMA_FP32ACC = 0x1
 RH_E_INVALID, RH_E_WORKSPACE, RH_E_UNSUPPORTED, RH_E_LIMIT = -1, -2, -3, -4
 

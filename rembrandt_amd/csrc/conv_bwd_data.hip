@@ -174,9 +174,10 @@ static int bwd_data_impl(const rh_conv_geom* g, float alpha, const float* w, con
     return launch_conv1x1_stream(d, RH_CONV_BWD_DATA, w, dy, dx, alpha, beta, nullptr, 0, stream, mask);
   }
   if (wino_shape(d) && !(flags & (RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))) {
-    const WinoGeom wg = wino_geom_bwd_data(d);
+    WinoGeom wg = wino_geom_bwd_data(d);
     if (flags & RH_ALGO_WINOGRAD ? wg.ok : wino_pays(wg)) {
       if (d.x_elems == 0) return 0;
+      if (flags & RH_ALGO_SHARED_GPU) wg.tail_S = 1;
       return launch_conv_wino(wg, true, dy, w, dx, alpha, beta, nullptr, 0, mask, ws, stream, "conv_bwd_data_wino");
     }
     if (flags & RH_ALGO_WINOGRAD) return RH_E_UNSUPPORTED;

@@ -302,7 +302,13 @@ struct WinoGeom {
   long long tiles, tiles_p;   // 2x2 output tiles; rounded up to whole column tiles
   size_t u_bytes, v_bytes;
   bool ok;
-  size_t total() const { return u_bytes + v_bytes; }
+  // Tail form (V made in the kernel only): the blocks past the last multiple of 256 are cut into tail_S slices of the
+  // channel loop, tail_L stages each, whose untransformed-blend partial results go to slabs of scratch that hold the
+  // result from element part_first on (the first image a tail block touches); tail_S == 1: not worth it.
+  int full_tiles, tail_S, tail_L;
+  long long part_first, slab_elems;
+  size_t part_bytes;
+  size_t total() const { return u_bytes + v_bytes + part_bytes; }
 };
 WinoGeom wino_geom(int N, int Ci, int Hi, int Wi, int Ko, int halo);
 inline bool wino_shape(const ConvDims& d) { return d.R == 3 && d.S == 3 && d.st == 1 && d.pad <= 2; }

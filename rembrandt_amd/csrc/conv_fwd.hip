@@ -594,7 +594,8 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
     return launch_conv1x1_stream(d, RH_CONV_FWD, w, x, y, alpha, beta, (flags & RH_FUSE_BIAS) ? bias : nullptr,
                                  (flags & RH_FUSE_RELU) ? 1 : 0, stream);
   if (wino_shape(d) && !(flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))) {
-    const WinoGeom wg = wino_geom_fwd(d);
+    WinoGeom wg = wino_geom_fwd(d);
+    if (flags & RH_ALGO_SHARED_GPU) wg.tail_S = 1;
     if (flags & RH_ALGO_WINOGRAD ? wg.ok : wino_pays(wg))
       return launch_conv_wino(wg, false, x, w, y, alpha, beta, (flags & RH_FUSE_BIAS) ? bias : nullptr,
                               (flags & RH_FUSE_RELU) ? 1 : 0, nullptr, ws, stream, "conv_fwd_wino");

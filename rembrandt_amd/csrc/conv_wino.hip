@@ -44,9 +44,35 @@ WinoGeom wino_geom(int N, int Ci, int Hi, int Wi, int Ko, int halo) {
   const unsigned long long ub = 16ull * g.Cg * 2 * (unsigned long long)g.rows_p * 8;
   const unsigned long long vb = 16ull * g.Cg * 2 * (unsigned long long)g.tiles_p * 8;
   g.u_bytes = align256((size_t)ub);
-  g.v_bytes = align256((size_t)vb);
+  g.v_bytes = Ci % 4 == 0 ? 0 : align256((size_t)vb);   // (channel counts in whole groups of four: V is made in the kernel)
   // 32-bit byte offsets into U and V, 31-bit tile indices
-  g.ok = g.P > 0 && g.Q > 0 && halo >= 0 && halo <= 2 && ub < (1ull << 31) && vb < (1ull << 31) && g.tiles_p < (1ll << 30);
+  g.ok = g.P > 0 && g.Q > 0 && halo >= 0 && halo <= 2 && ub < (1ull << 31) && (Ci % 4 == 0 || vb < (1ull << 31)) &&
+         g.tiles_p < (1ll << 30) && (long long)N * Ko * g.P * g.Q < (1ll << 30) && (long long)N * Ci * Hi * Wi < (1ll << 30);
+  // One block per CU at a time: 784 blocks are four rounds of the 256 CUs with the last one 6 % full.  The blocks past
+  // the last whole round are cut into slices of the channel loop (every slice a whole number of stages, four at
+  // least), so that the last round is as short as its share of the work; their partial results are added by
+  // wino_tail_reduce_kernel.  A block costs about eight stages' time before and after its loop (measured: 1176 blocks
+  // of 64 stages gain nothing from five slices of 13), and the slabs and that kernel 3 % of a round.
+  g.full_tiles = 0; g.tail_S = 1; g.tail_L = g.Cg; g.part_first = 0; g.slab_elems = 0; g.part_bytes = 0;
+  const long long tiles_m = g.rows_p / kWinoBM, T = tiles_m * (g.tiles_p / kWinoBN);
+  const long long full = T / 256 * 256, tail = T - full;
+  if (g.ok && Ci % 4 == 0 && full > 0 && tail > 0) {
+    double best = (double)cdiv<long long>(T, 256) * 0.97;
+    for (int S = 2; S <= 16; ++S) {
+      const int L = cdiv(g.Cg, S);
+      if (L < 4 || cdiv(g.Cg, L) != S) continue;
+      const double cost = (double)(full / 256) + (double)cdiv<long long>(tail * S, 256) * (L + 8.0) / (g.Cg + 8.0) + 0.03;
+      if (cost < best) { best = cost; g.tail_S = S; g.tail_L = L; }
+    }
+    if (g.tail_S > 1) {
+      g.full_tiles = (int)full;
+      const long long first_tile = (full / tiles_m) * kWinoBN;   // first image tile of the first column tile with a tail block
+      const long long n0 = first_tile / ((long long)g.TP * g.TQ);
+      g.part_first = n0 * g.Ko * g.P * g.Q;
+      g.slab_elems = (long long)N * g.Ko * g.P * g.Q - g.part_first;
+      g.part_bytes = align256(sizeof(float) * (size_t)g.slab_elems * g.tail_S);
+    }
+  }
   return g;
 }
 
@@ -467,8 +493,13 @@ __device__ __forceinline__ void dma_load4(u32x4 rsrc, uint32_t lds_addr, uint32_
 }
 #pragma clang diagnostic pop
 
+struct WinoTail {
+  int full, S, L;                     // blocks that take a whole tile; slices of a tail tile; stages per slice
+  float* part; long long slab_elems, part_first;
+};
+
 __global__ __launch_bounds__(256, 1) void wino_gemm_fused_kernel(const float* __restrict__ U, WinoImage im, int Cg, int rows_p,
-                                                                int tiles_m, unsigned u_bytes, WinoEpi ep) {
+                                                                int tiles_m, unsigned u_bytes, WinoEpi ep, WinoTail tl) {
   constexpr int R = kWinoR;
   extern __shared__ float lds_dyn[];   // [R stages: U | V][2 raw patch slots]
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_dyn;
@@ -476,8 +507,24 @@ __global__ __launch_bounds__(256, 1) void wino_gemm_fused_kernel(const float* __
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, r = lane & 31;
-  const int logical = __builtin_amdgcn_readfirstlane(xcd_remap(blockIdx.x, gridDim.x));
-  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  // a block past the whole rounds takes one slice of a tail tile's channel loop: stages cg0 .. cg0 + nk - 1, and
+  // writes its part of the result unblended into the slice's slab.  The whole-tile blocks and the tail blocks are
+  // each dealt evenly to the XCDs (tl.full is a multiple of 256).
+  int tile, cg0 = 0, nk = Cg;
+  if (tl.S <= 1) {
+    tile = __builtin_amdgcn_readfirstlane(xcd_remap(blockIdx.x, gridDim.x));
+  } else if ((int)blockIdx.x < tl.full) {
+    tile = __builtin_amdgcn_readfirstlane(xcd_remap(blockIdx.x, tl.full));
+  } else {
+    const int ti = __builtin_amdgcn_readfirstlane(xcd_remap((int)blockIdx.x - tl.full, (int)gridDim.x - tl.full));
+    const int slice = ti % tl.S;
+    tile = tl.full + ti / tl.S;
+    cg0 = slice * tl.L;
+    nk = Cg - cg0 < tl.L ? Cg - cg0 : tl.L;
+    ep.out = tl.part + (long long)slice * tl.slab_elems - tl.part_first;
+    ep.bias = nullptr; ep.mask = nullptr; ep.alpha = 1.0f; ep.beta = 0.0f; ep.relu = 0;
+  }
+  const int tile_m = tile % tiles_m, tile_n = tile / tiles_m;
   const int m0 = tile_m * kWinoBM;
   const unsigned n0 = (unsigned)tile_n * kWinoBN;
 
@@ -521,10 +568,10 @@ __global__ __launch_bounds__(256, 1) void wino_gemm_fused_kernel(const float* __
   auto issue_one = [&](int i, int cg, int buf, int par) {
     if (i < 12)
       dma_load4(rsX, raw0 + (uint32_t)par * kWinoRaw + (uint32_t)i * 1024u + (uint32_t)wave * 256u, poff[i >> 2][i & 3],
-                (uint32_t)(4 * cg + wave) * chan_stride);
+                (uint32_t)(4 * (cg0 + cg) + wave) * chan_stride);
     else
       dma_load16(rsU, lds0 + (uint32_t)buf * kWinoStage + (uint32_t)(wave * 8 + (i - 12)) * 1024u, voffA,
-                 soA[i - 12] + (uint32_t)cg * strideA);
+                 soA[i - 12] + (uint32_t)(cg0 + cg) * strideA);
   };
   // the thread's part of stage s's image operand: raw slot s & 1 -> two rows of B^T d B -> V area of ring buffer buf
   const float* rawp = lds_dyn + R * (kWinoStage / 4) + tid;
@@ -558,7 +605,6 @@ __global__ __launch_bounds__(256, 1) void wino_gemm_fused_kernel(const float* __
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[f][v] = 0.0f;
 
-  const int nk = Cg;
   // Stages 0 and 1 on their way, their image operands made, the taps of stage 2 on their way (into the slot stage
   // 0's were read from): the taps run three stages ahead of the MFMAs, U two.
 #pragma unroll
@@ -936,7 +982,8 @@ struct WinoFilterPrepArgs {
 // Vt of channels (2 ch, 2 ch + 1) x tiles (2 up, 2 up + 1): one 16-byte store per f, [channel][tile of the pair]
 __device__ __forceinline__ void wino_filter_v_item(const WinoFilterPrepArgs& a, unsigned idx) {
   // eight neighbouring lanes take eight channel pairs of one tile pair (their stores are 128 consecutive bytes), the
-  // next eight the next tile pair (their loads are neighbours in eight planes)
+  // next eight the next tile pair (their loads are neighbours in eight planes): 0.133 ms for 385 MB; runs of 4 and of 16
+  // channel pairs measured 0.174 and 0.149
   uint32_t ch_hi, up;
   a.dPairs.divmod(idx >> 3, ch_hi, up);   // up: tile pair = 2 (tile group) + h
   const uint32_t ch = ch_hi * 8u + (idx & 7u);
@@ -1019,6 +1066,37 @@ __global__ __launch_bounds__(256) void wino_filter_prep_kernel(WinoFilterPrepArg
   }
 }
 
+// The tail form's second pass: out = alpha * (sum of the slices' slabs) + beta * out (+ bias, ReLU or mask) on the
+// elements that a tail block produced; elements of the same images that a whole-tile block wrote are left alone.
+struct WinoTailReduce {
+  const float* part; float* out; const float* bias; const float* mask;
+  float alpha, beta;
+  int relu, S, Ko, P, Q, TP, TQ, tiles_m, full;
+  unsigned first, total;       // elements [first, total) of the result
+  long long slab_elems;
+  FastDiv dPQ, dQ, dKo;
+};
+__global__ __launch_bounds__(256) void wino_tail_reduce_kernel(WinoTailReduce a) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= a.total - a.first) return;
+  const unsigned g = a.first + i;
+  uint32_t plane, pix, n, k, pp, qq;
+  a.dPQ.divmod(g, plane, pix);
+  a.dKo.divmod(plane, n, k);
+  a.dQ.divmod(pix, pp, qq);
+  const unsigned t = (n * (unsigned)a.TP + (pp >> 1)) * (unsigned)a.TQ + (qq >> 1);
+  const unsigned logical = (t / kWinoBN) * (unsigned)a.tiles_m + k / kWinoBM;
+  if (logical < (unsigned)a.full) return;
+  float v = 0.0f;
+  for (int sl = 0; sl < a.S; ++sl) v += a.part[(long long)sl * a.slab_elems + i];
+  v *= a.alpha;
+  if (a.beta != 0.0f) v = fmaf(a.beta, a.out[g], v);
+  if (a.bias) v += a.bias[k];
+  if (a.relu) v = fmaxf(v, 0.0f);
+  if (a.mask) v = a.mask[g] > 0.0f ? v : 0.0f;
+  a.out[g] = v;
+}
+
 }  // namespace
 
 // in: (N, Ci, Hi, Wi) with g.halo zeros around; w: the layer's filter (K, C, 3, 3): forward reads it as (Ko, Ci), the
@@ -1065,8 +1143,24 @@ int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* 
     WinoImage im;
     im.x = in; im.x_bytes = a.x_bytes; im.Ci = g.Ci; im.Hi = g.Hi; im.Wi = g.Wi; im.halo = g.halo;
     ProfScope prof(tag, 2.0 * 16.0 * (double)g.Ko * g.Ci * (double)g.tiles, stream);
-    hipLaunchKernelGGL(wino_gemm_fused_kernel, dim3((unsigned)(tiles_m_ * tiles_n_)), dim3(256), lds_f, stream, U, im, g.Cg,
-                       g.rows_p, tiles_m_, (unsigned)(16ull * g.Cg * 2 * g.rows_p * 8), ep);
+    WinoTail tl;
+    tl.full = g.full_tiles; tl.S = g.tail_S; tl.L = g.tail_L;
+    tl.part = reinterpret_cast<float*>(static_cast<char*>(ws) + g.u_bytes + g.v_bytes);
+    tl.slab_elems = g.slab_elems; tl.part_first = g.part_first;
+    const long long T = (long long)tiles_m_ * tiles_n_;
+    const long long blocks = g.tail_S > 1 ? g.full_tiles + (T - g.full_tiles) * g.tail_S : T;
+    hipLaunchKernelGGL(wino_gemm_fused_kernel, dim3((unsigned)blocks), dim3(256), lds_f, stream, U, im, g.Cg, g.rows_p, tiles_m_,
+                       (unsigned)(16ull * g.Cg * 2 * g.rows_p * 8), ep, tl);
+    if (g.tail_S > 1) {
+      if (int e = launch_status()) return e;
+      WinoTailReduce r;
+      r.part = tl.part; r.out = out; r.bias = bias; r.mask = mask; r.alpha = alpha; r.beta = beta; r.relu = relu;
+      r.S = g.tail_S; r.Ko = g.Ko; r.P = g.P; r.Q = g.Q; r.TP = g.TP; r.TQ = g.TQ; r.tiles_m = tiles_m_; r.full = g.full_tiles;
+      r.first = (unsigned)g.part_first; r.total = (unsigned)((long long)g.N * g.Ko * g.P * g.Q);
+      r.slab_elems = g.slab_elems;
+      r.dPQ = FastDiv((uint32_t)(g.P * g.Q)); r.dQ = FastDiv((uint32_t)g.Q); r.dKo = FastDiv((uint32_t)g.Ko);
+      hipLaunchKernelGGL(wino_tail_reduce_kernel, dim3(cdiv((unsigned)g.slab_elems, 256u)), dim3(256), 0, stream, r);
+    }
     return launch_status();
   }
   constexpr size_t lds_bytes = (size_t)kWinoR * kWinoStage;

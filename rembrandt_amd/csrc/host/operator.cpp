@@ -923,15 +923,15 @@ class Conv2dOperator : public Operator {
                                    out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), w_bias->as_mut_ptr(),
                                    w_bias->len(), s_bias), "conv2d backward bias");
     }
+    const int beside = s_filter != s ? RH_ALGO_SHARED_GPU : 0;   // the filter gradient runs beside the data gradient
     if (in_delta_ && fold_prev_relu_) {
       // the operator below left its ReLU backward mask to this call: in_act_ is that ReLU's output
       unwrap(rh_conv2d_bwd_data_relu(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
-                                     in_act_->as_ptr(), workspace_->as_mut_ptr(), workspace_->len(),
-                                     opts_.winograd ? 0 : RH_ALGO_DIRECT, s),
+                                     in_act_->as_ptr(), workspace_->as_mut_ptr(), workspace_->len(), algo | beside, s),
              "conv2d backward data");
     } else if (in_delta_) {
       unwrap(rh_conv2d_bwd_data(&g, 1.0f, params_.weights->as_ptr(), out_delta_->as_ptr(), 0.0f, in_delta_->as_mut_ptr(),
-                                workspace_->as_mut_ptr(), workspace_->len(), opts_.winograd ? 0 : RH_ALGO_DIRECT, s),
+                                workspace_->as_mut_ptr(), workspace_->len(), algo | beside, s),
              "conv2d backward data");
     }
   }
@@ -1254,6 +1254,7 @@ struct BNormConvUnit {
   Buf pre_act, pre_delta;  // the conv output the batch norm reads, and the gradient w.r.t. it
   bool backward = false;
   int conv_algo = 0;       // RH_ALGO_* bits of the unit's convolution calls
+  bool beside = false;     // the last backward_params put the filter gradient on the second stream: the data gradient runs beside it
 
   void alloc(size_t batch, Dims3 in, size_t size, size_t stride, size_t pad, size_t out_channels, bool bwd, Ctx c) {
     in_dims = in; conv_size = size; conv_stride = stride; conv_pad = pad; chans = out_channels; ctx = c; backward = bwd;
@@ -1353,6 +1354,7 @@ struct BNormConvUnit {
                           cached_ivar->as_ptr(), ws.as_mut_ptr(), ws.len(), s()), "batch norm backward");
     rh_stream_t sg = s();
     DeviceBuffer<uint8_t>* wg = &ws;
+    beside = ws_aux != nullptr;
     if (ws_aux) {
       ctx->fork();
       sg = ctx->aux_stream();
@@ -1369,7 +1371,7 @@ struct BNormConvUnit {
   void backward_data(size_t batch, float* in_delta, float beta, DeviceBuffer<uint8_t>& ws) {
     const rh_conv_geom g = geom(batch);
     unwrap(rh_conv2d_bwd_data(&g, 1.0f, weights->as_ptr(), pre_delta->as_ptr(), beta, in_delta, ws.as_mut_ptr(), ws.len(),
-                              conv_algo, s()), "conv2d backward data");
+                              conv_algo | (beside ? RH_ALGO_SHARED_GPU : 0), s()), "conv2d backward data");
   }
 
   void axpy(float a, const DeviceBuffer<float>& x, DeviceBuffer<float>& y) {

@@ -57,6 +57,7 @@ pub const RH_ALGO_GATHER: c_int = 0x100;
 pub const RH_ALGO_SCALAR_OFFSET: c_int = 0x200;
 pub const RH_ALGO_WINOGRAD: c_int = 0x400;
 pub const RH_ALGO_DIRECT: c_int = 0x800;
+pub const RH_ALGO_SHARED_GPU: c_int = 0x1000;
 
 #[link(name = "rembrandt_hip")]
 extern "C" {

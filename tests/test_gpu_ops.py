@@ -166,6 +166,8 @@ WINO_CASES = [
     (2, 64, 13, 13, 96, 1),
     (33, 64, 14, 15, 128, 1),
     (70, 66, 13, 13, 384, 1),     # 3 x 108 blocks
+    (70, 64, 13, 13, 384, 1),     # forward: 324 blocks, the 68 past 256 in three slices of the channel loop (6, 6, 4 stages)
+    (70, 384, 13, 13, 64, 1),     # the same in the data gradient
     (16, 128, 28, 28, 64, 1),
     (90, 64, 13, 13, 128, 1),     # 4410 tiles: the filter gradient in the form too, its tiles in several slices
 ]
@@ -222,6 +224,17 @@ def test_conv2d_winograd(dev, case):
     # run to run the same bits
     assert torch.equal(ops.conv2d_fwd(xd, wd, 1, pad, algo=WG), y)
     assert torch.equal(ops.conv2d_bwd_filter(xd, dyd, w.shape, 1, pad, algo=WG), dw)
+    # RH_ALGO_SHARED_GPU (other kernels run beside the call): whole blocks only, no sliced tail; the same result up to
+    # summation order where a tail was sliced, the same bits where none was
+    SH = _lib.RH_ALGO_SHARED_GPU
+    ys = ops.conv2d_fwd(xd, wd, 1, pad, algo=WG | SH)
+    dxs = ops.conv2d_bwd_data(wd, dyd, x.shape, 1, pad, algo=WG | SH)
+    assert_close(N(ys), y_ref, "winograd fwd, shared-GPU hint")
+    assert_close(N(dxs), dx_ref, "winograd bwd data, shared-GPU hint")
+    blocks_b = -(-C // 128) * -(-(Nn * -(-H // 2) * -(-W // 2)) // 32)
+    blocks_f = -(-K // 128) * -(-(Nn * -(-y_ref.shape[2] // 2) * -(-y_ref.shape[3] // 2)) // 32)
+    if blocks_f <= 256 or C % 4: assert torch.equal(ys, y)
+    if blocks_b <= 256 or K % 4: assert torch.equal(dxs, dx)
     # what the library picks by itself: this form from 64 channels on both sides, 128-row tiles three quarters full and
     # 192 blocks on, else a direct one
     auto = ops.conv2d_fwd(xd, wd, 1, pad)
