@@ -322,7 +322,7 @@ int rh_softmax_kl_step(const float* x, int32_t C, int32_t N, const int32_t* labe
  *                                RH_E_UNSUPPORTED.
  * With I = 0 and x = NULL both start from an h that is already there (a first layer too large for this form, whose
  * products stay with rh_sgemm): rh_affine2_softmax_kl_step then reads h, writes logits .. dh and leaves dx alone (w1, b1
- * unused); rh_affine2_bwd_params forms dW2 and db2 only (dh, dw1, db1 unused).
+ * unused); rh_affine2_bwd_params forms dW2 and db2 (dw1 unused) and, where db1 is not NULL, db1 = sum_n dh + beta1 * db1.
  * Sums are taken in a fixed order that differs from the tiled products': results agree with the separate calls to
  * rounding, not bit for bit. */
 int rh_affine2_softmax_kl_step_supported(int32_t B, int32_t I, int32_t H, int32_t C);

@@ -86,13 +86,84 @@ __device__ __forceinline__ float sum_splits(const float* __restrict__ part, int 
   return (a0 + a1) + (a2 + a3);
 }
 
+// Column sums of an [N][K] matrix (dy of an affine layer, or per-image plane sums) for the 64 columns from 64 b on by
+// one block of 256 threads: its 4 waves take every fourth row and are combined through LDS in a fixed order.
+__device__ __forceinline__ void bwd_bias_rows_block(const float* __restrict__ dy, int N, int K, float alpha, float beta,
+                                                    float* __restrict__ db, unsigned b) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int k = (int)b * 64 + lane;
+  // eight independent partial sums per thread (rows wave, wave + 4, ... in turn): the loop is a chain of memory round
+  // trips, so its length is what the kernel takes
+  float a[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  if (k < K) {
+    int n = wave;
+    for (; n + 28 < N; n += 32) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a[j] += dy[(size_t)(n + 4 * j) * K + k];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (n + 4 * j < N) a[j] += dy[(size_t)(n + 4 * j) * K + k];
+  }
+  __shared__ float sm[4][64];
+  sm[wave][lane] = ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+  __syncthreads();
+  if (wave == 0 && k < K) {
+    float v = alpha * ((sm[0][lane] + sm[1][lane]) + (sm[2][lane] + sm[3][lane]));
+    if (beta != 0.0f) v += beta * db[k];
+    db[k] = v;
+  }
+}
+
+// The same sum for one channel by a block of 256 threads, for the small layers whose bias gradient rides in another
+// launch: wave w takes the images w, w + 4, ..., eight of them at a time with four strides of the plane each (32 loads
+// in flight per lane; a block is alone with its channel, so the chain of memory round trips is what it takes).  A fixed
+// order, not the one of bwd_bias_kernel.
+__device__ __forceinline__ void bwd_bias_planes_job(const float* __restrict__ dy, int N, int K, int plane, float alpha,
+                                                    float beta, float* __restrict__ db, int k) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float a[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  for (int n0 = wave; n0 < N; n0 += 32) {
+    for (int i0 = lane; i0 < plane; i0 += 256) {
+      float v[8][4];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int n = n0 + 4 * u;
+        const float* p = dy + ((size_t)(n < N ? n : 0) * K + k) * plane;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[u][j] = n < N && i0 + 64 * j < plane ? p[i0 + 64 * j] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) a[u] += (v[u][0] + v[u][1]) + (v[u][2] + v[u][3]);
+    }
+  }
+  float acc = ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
+  __shared__ float part[4];
+  if (lane == 0) part[wave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float v = alpha * ((part[0] + part[1]) + (part[2] + part[3]));
+    if (beta != 0.0f) v += beta * db[k];
+    db[k] = v;
+  }
+}
+
+// A bias gradient that rides in a reduction launch (BiasJob): block b of the job, 256 threads.
+__device__ __forceinline__ void bias_job_block(const BiasJob& j, unsigned b) {
+  if (j.plane == 1) bwd_bias_rows_block(j.src, j.N, j.K, j.alpha, j.beta, j.db, b);
+  else bwd_bias_planes_job(j.src, j.N, j.K, j.plane, j.alpha, j.beta, j.db, (int)b);
+}
+
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
 // (+ bias_col[j], then ReLU, where given: the epilogue of an affine layer's forward product)
 __global__ void split_reduce_kernel(const float* __restrict__ part, int splits, long long split_stride,
                                     float* __restrict__ out, int rows, int cols, int ld, float alpha,
-                                    float beta, const float* __restrict__ bias_col, int relu) {
+                                    float beta, const float* __restrict__ bias_col, int relu, BiasJob bj) {
+  if (bj.db && blockIdx.x >= bj.first) { bias_job_block(bj, blockIdx.x - bj.first); return; }
+  const unsigned nb = bj.db ? bj.first : gridDim.x;
   const unsigned total = (unsigned)rows * (unsigned)cols;  // a filter gradient / GEMM result: far below 2^31
-  for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+  for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += nb * blockDim.x) {
     const float acc = sum_splits(part, splits, split_stride, idx);
     const int i = (int)(idx / (unsigned)cols), j = (int)(idx - (unsigned)i * (unsigned)cols);
     float* dst = out + (size_t)i * ld + j;
@@ -119,7 +190,8 @@ __device__ __forceinline__ void bias_relu4(float4& v, unsigned idx, const float*
 __global__ __launch_bounds__(256) void split_reduce_vec_kernel(const float4* __restrict__ part, int splits, long long stride4,
                                                                float4* __restrict__ out, unsigned total4, float alpha,
                                                                float beta, const float* __restrict__ bias_col,
-                                                               unsigned cols4, int relu) {
+                                                               unsigned cols4, int relu, BiasJob bj) {
+  if (bj.db && blockIdx.x >= bj.first) { bias_job_block(bj, blockIdx.x - bj.first); return; }
   const unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total4) return;
   const float4 z = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -155,7 +227,8 @@ constexpr int kReduceLanes = 32, kReduceGroups = 8;
 __global__ __launch_bounds__(256) void split_reduce_vec_par_kernel(const float4* __restrict__ part, int splits, long long stride4,
                                                                    float4* __restrict__ out, unsigned total4, float alpha,
                                                                    float beta, const float* __restrict__ bias_col,
-                                                                   unsigned cols4, int relu) {
+                                                                   unsigned cols4, int relu, BiasJob bj) {
+  if (bj.db && blockIdx.x >= bj.first) { bias_job_block(bj, blockIdx.x - bj.first); return; }
   __shared__ float4 red[kReduceLanes][kReduceGroups];
   const int g = (int)threadIdx.x % kReduceGroups, j = (int)threadIdx.x / kReduceGroups;
   const unsigned idx = blockIdx.x * kReduceGroups + g;
@@ -190,7 +263,8 @@ __global__ __launch_bounds__(256) void split_reduce_vec_par_kernel(const float4*
 // The many-slice form for results that are not dense 16-byte groups (odd extents, a padded leading dimension).
 __global__ __launch_bounds__(256) void split_reduce_par_kernel(const float* __restrict__ part, int splits, long long split_stride,
                                                                float* __restrict__ out, int rows, int cols, int ld, float alpha,
-                                                               float beta, const float* __restrict__ bias_col, int relu) {
+                                                               float beta, const float* __restrict__ bias_col, int relu, BiasJob bj) {
+  if (bj.db && blockIdx.x >= bj.first) { bias_job_block(bj, blockIdx.x - bj.first); return; }
   __shared__ float red[kReduceLanes][kReduceGroups];
   const int g = (int)threadIdx.x % kReduceGroups, j = (int)threadIdx.x / kReduceGroups;
   const unsigned total = (unsigned)rows * (unsigned)cols;
@@ -215,29 +289,37 @@ __global__ __launch_bounds__(256) void split_reduce_par_kernel(const float* __re
 }
 
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
-                         int ld, float alpha, float beta, hipStream_t stream, const float* bias_col, int relu) {
+                         int ld, float alpha, float beta, hipStream_t stream, const float* bias_col, int relu,
+                         const BiasJob* bias_job) {
   const size_t total = (size_t)rows * cols;
-  ProfScope prof("split_reduce", 4.0 * (double)total * (splits + 1), stream);
+  BiasJob bj;
+  if (bias_job) bj = *bias_job;
+  const unsigned jb = bj.blocks();
+  ProfScope prof("split_reduce", 4.0 * (double)total * (splits + 1) + (jb ? 4.0 * (double)bj.N * bj.K * bj.plane : 0.0), stream);
   if (ld == cols && cols % 4 == 0 && split_stride % 4 == 0 &&
       ((reinterpret_cast<uintptr_t>(part) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(bias_col)) & 15) == 0) {
     if (total / 4 < 64 * 1024 && splits >= 2 * kReduceLanes) {   // under 1024 waves with a thread per group
-      hipLaunchKernelGGL(split_reduce_vec_par_kernel, dim3((unsigned)cdiv<size_t>(total / 4, kReduceGroups)), dim3(256), 0,
+      bj.first = (unsigned)cdiv<size_t>(total / 4, kReduceGroups);
+      hipLaunchKernelGGL(split_reduce_vec_par_kernel, dim3(bj.first + jb), dim3(256), 0,
                          stream, reinterpret_cast<const float4*>(part), splits, split_stride / 4,
-                         reinterpret_cast<float4*>(out), (unsigned)(total / 4), alpha, beta, bias_col, (unsigned)(cols / 4), relu);
+                         reinterpret_cast<float4*>(out), (unsigned)(total / 4), alpha, beta, bias_col, (unsigned)(cols / 4), relu, bj);
       return;
     }
-    hipLaunchKernelGGL(split_reduce_vec_kernel, dim3(stream_grid(total / 4, 256)), dim3(256), 0, stream,
+    bj.first = stream_grid(total / 4, 256);
+    hipLaunchKernelGGL(split_reduce_vec_kernel, dim3(bj.first + jb), dim3(256), 0, stream,
                        reinterpret_cast<const float4*>(part), splits, split_stride / 4, reinterpret_cast<float4*>(out),
-                       (unsigned)(total / 4), alpha, beta, bias_col, (unsigned)(cols / 4), relu);
+                       (unsigned)(total / 4), alpha, beta, bias_col, (unsigned)(cols / 4), relu, bj);
     return;
   }
   if (total < 256 * 1024 && splits >= 2 * kReduceLanes) {
-    hipLaunchKernelGGL(split_reduce_par_kernel, dim3((unsigned)cdiv<size_t>(total, kReduceGroups)), dim3(256), 0, stream, part,
-                       splits, split_stride, out, rows, cols, ld, alpha, beta, bias_col, relu);
+    bj.first = (unsigned)cdiv<size_t>(total, kReduceGroups);
+    hipLaunchKernelGGL(split_reduce_par_kernel, dim3(bj.first + jb), dim3(256), 0, stream, part,
+                       splits, split_stride, out, rows, cols, ld, alpha, beta, bias_col, relu, bj);
     return;
   }
-  hipLaunchKernelGGL(split_reduce_kernel, dim3(stream_grid(total, 256)), dim3(256), 0, stream, part, splits,
-                     split_stride, out, rows, cols, ld, alpha, beta, bias_col, relu);
+  bj.first = stream_grid(total, 256);
+  hipLaunchKernelGGL(split_reduce_kernel, dim3(bj.first + jb), dim3(256), 0, stream, part, splits,
+                     split_stride, out, rows, cols, ld, alpha, beta, bias_col, relu, bj);
 }
 
 // ---- scalar-offset path ------------------------------------------------------------------------
@@ -525,10 +607,12 @@ __global__ __launch_bounds__(256) void bwd_filter_prep_kernel(NhwcCopyArgs dy, f
 
 // dw[ko][c][r][s] = alpha * sum_s part[s][ko][(r,s,c)] + beta * dw
 __global__ void split_reduce_rsc_kernel(const float* __restrict__ part, int splits, long long split_stride,
-                                        float* __restrict__ dw, int K, int C, int R, int S, float alpha, float beta) {
+                                        float* __restrict__ dw, int K, int C, int R, int S, float alpha, float beta, BiasJob bj) {
+  if (bj.db && blockIdx.x >= bj.first) { bias_job_block(bj, blockIdx.x - bj.first); return; }
+  const unsigned nb = bj.db ? bj.first : gridDim.x;
   const int CRS = C * R * S;
   const unsigned total = (unsigned)K * (unsigned)CRS;
-  for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+  for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += nb * blockDim.x) {
     const float acc = sum_splits(part, splits, split_stride, idx);
     const int ko = (int)(idx / (unsigned)CRS), j = (int)(idx - (unsigned)ko * (unsigned)CRS);
     const int r = j / (S * C), rem = j - r * (S * C), s2 = rem / C, c = rem - s2 * C;
@@ -543,7 +627,8 @@ __global__ void split_reduce_rsc_kernel(const float* __restrict__ part, int spli
 // every slab (4-byte reads top out well below what 16-byte reads reach); sums in the order of sum_splits.
 __global__ __launch_bounds__(256) void split_reduce_rsc_vec_kernel(const float4* __restrict__ part, int splits, long long stride4,
                                                                    float* __restrict__ dw, int K, int C, int R, int S,
-                                                                   float alpha, float beta) {
+                                                                   float alpha, float beta, BiasJob bj) {
+  if (bj.db && blockIdx.x >= bj.first) { bias_job_block(bj, blockIdx.x - bj.first); return; }
   const int CRS4 = (C * R * S) >> 2;
   const unsigned total4 = (unsigned)K * (unsigned)CRS4;
   const unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
@@ -737,33 +822,10 @@ static int bwd_bias_col_groups(int N, long long KP) {
 }
 constexpr int kBiasSmallPlane = 1024;  // below: column form; from here on: one wave per (n, k) row
 
-// Column sums of an [N][K] matrix (dy of an affine layer, or the row sums above): a block covers 64
-// columns; its 4 waves take every fourth row and are combined through LDS in a fixed order.
+// Column sums of an [N][K] matrix (dy of an affine layer, or the row sums above): a block covers 64 columns.
 __global__ __launch_bounds__(256) void bwd_bias_rows_kernel(const float* __restrict__ dy, int N, int K, float alpha,
                                                             float beta, float* __restrict__ db) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int k = blockIdx.x * 64 + lane;
-  // eight independent partial sums per thread (rows wave, wave + 4, ... in turn): the loop is a chain of memory round
-  // trips, so its length is what the kernel takes
-  float a[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-  if (k < K) {
-    int n = wave;
-    for (; n + 28 < N; n += 32) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) a[j] += dy[(size_t)(n + 4 * j) * K + k];
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if (n + 4 * j < N) a[j] += dy[(size_t)(n + 4 * j) * K + k];
-  }
-  __shared__ float sm[4][64];
-  sm[wave][lane] = ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
-  __syncthreads();
-  if (wave == 0 && k < K) {
-    float v = alpha * ((sm[0][lane] + sm[1][lane]) + (sm[2][lane] + sm[3][lane]));
-    if (beta != 0.0f) v += beta * db[k];
-    db[k] = v;
-  }
+  bwd_bias_rows_block(dy, N, K, alpha, beta, db, blockIdx.x);
 }
 
 }  // namespace rh
@@ -844,12 +906,34 @@ extern "C" size_t rh_conv2d_workspace_bytes_upto(const rh_conv_geom* g, int pass
   return need;
 }
 
-// bias_part: where the pass over dy may leave the per-image plane sums (N x K floats) if it makes one in a form that
-// can; *folded says whether it did.
+// The bias gradient beside the filter gradient (rh_conv2d_bwd_filter_bias).  part: where the pass over dy may leave the
+// per-image plane sums (N x K floats) if it makes one in a form that can; folded says whether it did; done: the bias
+// gradient was formed in the launch of the filter gradient's reduction, from those sums or, for a small layer, from dy.
+struct BiasFold {
+  float* db = nullptr;
+  float* part = nullptr;
+  bool folded = false, done = false;
+};
+// Up to this many elements of dy one launch (a block per channel) is as fast as the first of the two stages, and the
+// small layers it covers are bound by the number of dependent launches.
+constexpr long long kBiasOneStageElems = 1ll << 20;
+
 static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, const float* dy, float beta, float* dw,
-                           void* ws, size_t ws_bytes, int flags, rh_stream_t stream_, float* bias_part, bool* folded) {
+                           void* ws, size_t ws_bytes, int flags, rh_stream_t stream_, BiasFold* bf) {
   ConvDims d;
   if (int e = conv_dims(g, &d)) return e;
+  float* const bias_part = bf ? bf->part : nullptr;
+  // the job a reduction launch takes along: the sums over the images of what the pass over dy left, or the whole bias
+  // gradient of a small layer
+  auto bias_job = [&](BiasJob* job) -> const BiasJob* {
+    if (!bf || !bf->db || d.y_elems == 0) return nullptr;
+    job->db = bf->db; job->N = d.N; job->K = d.K; job->alpha = alpha; job->beta = beta;
+    if (bf->folded) { job->src = bf->part; job->plane = 1; }
+    else if (d.y_elems <= kBiasOneStageElems) { job->src = dy; job->plane = d.P * d.Q; }
+    else return nullptr;
+    bf->done = true;
+    return job;
+  };
   if (!x || !dy || !dw) return RH_E_INVALID;
   if (flags & RH_MATH_BF16_MFMA_FP32ACC) return RH_E_UNSUPPORTED;
   const BwdFilterPlan plan = plan_bwd_filter(d);
@@ -908,7 +992,7 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
       launch_nchw_to_nhwc(x, xT, d.N, d.C, d.H, d.W, sp.Hp, sp.Wp, d.pad, stream);
       if (int e = launch_status()) return e;
     }
-    if (bpart) *folded = true;
+    if (bpart) bf->folded = true;
     RowSParams ap;  // dyT [pix][ko]
     ap.ptr = dyT; ap.bytes = (uint32_t)(sizeof(float) * (size_t)sp.n_k * d.K);
     ap.M = d.K; ap.inner = d.K; ap.innerW = d.K; ap.img_stride = 0; ap.a_stride = 0; ap.b_stride = 1;
@@ -933,14 +1017,20 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     }
     if (e) return e;
     const long long total = (long long)d.K * CRSs;
-    ProfScope prof("split_reduce", 4.0 * (double)total * (used + 1), stream);
-    if (d.C % 4 == 0 && (reinterpret_cast<uintptr_t>(parts) & 15) == 0)
-      hipLaunchKernelGGL(split_reduce_rsc_vec_kernel, dim3(stream_grid((size_t)total / 4, 256)), dim3(256), 0, stream,
+    BiasJob bj;
+    bias_job(&bj);
+    const unsigned jb = bj.blocks();
+    ProfScope prof("split_reduce", 4.0 * (double)total * (used + 1) + (jb ? 4.0 * (double)bj.N * bj.K * bj.plane : 0.0), stream);
+    if (d.C % 4 == 0 && (reinterpret_cast<uintptr_t>(parts) & 15) == 0) {
+      bj.first = stream_grid((size_t)total / 4, 256);
+      hipLaunchKernelGGL(split_reduce_rsc_vec_kernel, dim3(bj.first + jb), dim3(256), 0, stream,
                          reinterpret_cast<const float4*>(parts), used, (long long)d.K * CRSs / 4, dw, d.K, d.C, d.R, d.S, alpha,
-                         beta);
-    else
-      hipLaunchKernelGGL(split_reduce_rsc_kernel, dim3(stream_grid((size_t)total, 256)), dim3(256), 0, stream, parts, used,
-                         (long long)d.K * CRSs, dw, d.K, d.C, d.R, d.S, alpha, beta);
+                         beta, bj);
+    } else {
+      bj.first = stream_grid((size_t)total, 256);
+      hipLaunchKernelGGL(split_reduce_rsc_kernel, dim3(bj.first + jb), dim3(256), 0, stream, parts, used,
+                         (long long)d.K * CRSs, dw, d.K, d.C, d.R, d.S, alpha, beta, bj);
+    }
     return launch_status();
   }
 
@@ -968,7 +1058,8 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
       default:  e = run_bwd_filter_1x1<T32x256>(ap, xp, ep, M, plan.splits, &used, stream, "conv_bwd_filter_32x256"); break;
     }
     if (e) return e;
-    launch_split_reduce(part, used, (long long)d.K * CRS, dw, d.K, CRS, CRS, alpha, beta, stream);
+    BiasJob bj;
+    launch_split_reduce(part, used, (long long)d.K * CRS, dw, d.K, CRS, CRS, alpha, beta, stream, nullptr, 0, bias_job(&bj));
     return launch_status();
   }
 
@@ -999,15 +1090,15 @@ static int bwd_filter_impl(const rh_conv_geom* g, float alpha, const float* x, c
     }
     if (e) return e;
   }
-  launch_split_reduce(part, used, (long long)d.K * CRS, dw, d.K, CRS, CRS, alpha, beta, stream);
+  BiasJob bj;
+  launch_split_reduce(part, used, (long long)d.K * CRS, dw, d.K, CRS, CRS, alpha, beta, stream, nullptr, 0, bias_job(&bj));
   return launch_status();
 }
 
 extern "C" int rh_conv2d_bwd_filter(const rh_conv_geom* g, float alpha, const float* x, const float* dy,
                                     float beta, float* dw, void* ws, size_t ws_bytes, int flags,
                                     rh_stream_t stream_) {
-  bool folded = false;
-  return bwd_filter_impl(g, alpha, x, dy, beta, dw, ws, ws_bytes, flags, stream_, nullptr, &folded);
+  return bwd_filter_impl(g, alpha, x, dy, beta, dw, ws, ws_bytes, flags, stream_, nullptr);
 }
 
 extern "C" int rh_conv2d_bwd_filter_bias(const rh_conv_geom* g, float alpha, const float* x, const float* dy,
@@ -1019,12 +1110,13 @@ extern "C" int rh_conv2d_bwd_filter_bias(const rh_conv_geom* g, float alpha, con
   if (!ws || ws_bytes < rh_conv2d_workspace_bytes(g, RH_CONV_BWD_FILTER) || (reinterpret_cast<uintptr_t>(ws) & 255))
     return RH_E_WORKSPACE;
   float* const bias_ws = reinterpret_cast<float*>(static_cast<char*>(ws) + bwd_filter_plan_bytes(d));
-  bool folded = false;
-  if (int e = bwd_filter_impl(g, alpha, x, dy, beta, dw, ws, ws_bytes, flags, stream_, bias_ws, &folded)) return e;
-  if (d.y_elems == 0) return 0;
+  BiasFold bf;
+  bf.db = db; bf.part = bias_ws;
+  if (int e = bwd_filter_impl(g, alpha, x, dy, beta, dw, ws, ws_bytes, flags, stream_, &bf)) return e;
+  if (d.y_elems == 0 || bf.done) return 0;
   hipStream_t stream = to_stream(stream_);
   const int plane = d.P * d.Q;
-  if (folded) {   // the sums over the images of what the pass over dy left
+  if (bf.folded) {   // the sums over the images of what the pass over dy left
     ProfScope prof("bwd_bias_finish", 4.0 * (double)d.N * d.K, stream);
     hipLaunchKernelGGL(bwd_bias_rows_kernel, dim3(cdiv(d.K, 64)), dim3(256), 0, stream, bias_ws, d.N, d.K, alpha, beta, db);
     return launch_status();
@@ -1034,10 +1126,6 @@ extern "C" int rh_conv2d_bwd_filter_bias(const rh_conv_geom* g, float alpha, con
     return bwd_bias_one_stage(d.N, d.K, plane, alpha, dy, beta, db, stream);
   return bwd_bias_two_stage(d.N, d.K, plane, alpha, dy, beta, db, bias_ws, stream);
 }
-
-// Up to this many elements of dy one launch (a block per channel) is as fast as the first of the two stages, and the
-// small layers it covers are bound by the number of dependent launches.
-constexpr long long kBiasOneStageElems = 1ll << 20;
 
 extern "C" size_t rh_conv2d_bwd_bias_workspace_bytes(int32_t N, int32_t K, int32_t plane) {
   if (N <= 0 || K <= 0 || plane <= 1) return 0;

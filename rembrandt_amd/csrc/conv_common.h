@@ -172,8 +172,20 @@ inline bool prefer_k8_64(long long cols) {
 }
 
 // Second pass of a split contraction: out[i*ld + j] = alpha * sum_s part[s][i*cols + j] + beta*out.
+// A bias gradient that rides in a reduction's launch, in blocks of its own behind the reduction's (small layers are
+// bound by the number of dependent launches): db[k] = alpha * sum over n and the plane of src[(n K + k) plane + i] +
+// beta * db[k]; plane == 1: src is an [N][K] matrix (an affine layer's delta, or per-image plane sums).
+struct BiasJob {
+  const float* src = nullptr;
+  float* db = nullptr;           // nullptr: no job
+  int N = 0, K = 0, plane = 0;
+  float alpha = 1.0f, beta = 0.0f;
+  unsigned first = 0;            // the job's first block (filled in by the launcher)
+  unsigned blocks() const { return !db ? 0u : plane == 1 ? (unsigned)((K + 63) / 64) : (unsigned)K; }
+};
 void launch_split_reduce(const float* part, int splits, long long split_stride, float* out, int rows, int cols,
-                         int ld, float alpha, float beta, hipStream_t stream, const float* bias_col = nullptr, int relu = 0);
+                         int ld, float alpha, float beta, hipStream_t stream, const float* bias_col = nullptr, int relu = 0,
+                         const BiasJob* bias_job = nullptr);
 
 // Tail form of a forward / backward-data launch (see EpiParams): when the tile count is not close to a multiple of
 // the 256 CUs, the column tiles beyond the last multiple are cut into `splits` slices so that every CU ends up with

@@ -618,7 +618,9 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
   }
   const SoffPlan sp = plan_soff_fwd(d);
   if ((flags & RH_MATH_BF16_MFMA_FP32ACC) && (!sp.ok || (flags & RH_ALGO_GATHER))) return RH_E_UNSUPPORTED;
-  if (sp.ok && !(flags & RH_ALGO_GATHER)) {
+  // (fp32, a contraction of up to 32, a 5x5 layer on one channel: the gather form is as fast and needs no launch in front of it)
+  const bool tiny_k = CRS <= 32 && !(flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_SCALAR_OFFSET));
+  if (sp.ok && !(flags & RH_ALGO_GATHER) && !tiny_k) {
     int* soff = static_cast<int*>(ws);
     float* wT = reinterpret_cast<float*>(static_cast<char*>(ws) + sp.tab_bytes);
     const float* img = x;

@@ -737,7 +737,9 @@ class AffineOperator : public Operator {
     unwrap(rh_sgemm(0, 1, i, o, b, 1.0f, in_act_->as_ptr(), i, out_delta_->as_ptr(), o, beta,
                     params_.grad_weights->as_mut_ptr(), i, wg, wg_len, 0, sg), "matrix_prod");
     // grad_bias(1, out) += 1(1, B) * out_delta^T: the column sums of out_delta, without the ones vector
-    unwrap(rh_conv2d_bwd_bias(b, o, 1, 1.0f, out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), sg), "matrix_prod");
+    if (!bias_grad_done_)
+      unwrap(rh_conv2d_bwd_bias(b, o, 1, 1.0f, out_delta_->as_ptr(), beta, params_.grad_bias->as_mut_ptr(), sg), "matrix_prod");
+    bias_grad_done_ = false;
     if (in_delta_) {
       // in_delta(in, B) = weights(in, out) * out_delta(out, B)
       unwrap(rh_sgemm(0, 0, i, b, o, 1.0f, params_.weights->as_ptr(), i, out_delta_->as_ptr(), o, 0.0f,
@@ -787,6 +789,7 @@ class AffineOperator : public Operator {
   std::unique_ptr<DeviceBuffer<uint8_t>> workspace_, workspace_aux_;
   bool overlap_built_, overlap_on_;  // parameter gradients and the fused SGD step of this block on the second stream
   bool delta_masked_once_ = false;   // out_delta_ already went through the activation's backward (the classifier tail)
+  bool bias_grad_done_ = false;      // this pass's bias gradient is already in grad_bias (the classifier tail's launch formed it)
 };
 
 // ---- Conv2dOperator -------------------------------------------------------------------------------------
@@ -902,7 +905,9 @@ class Conv2dOperator : public Operator {
     }
     const float beta = params_.take_backward_beta();   // 1: accumulate (the reference's call); 0: the buffers stand for zeros
     const int algo = opts_.winograd ? 0 : RH_ALGO_DIRECT;
-    if (!in_delta_ && workspace_aux_ && overlap_on_) {
+    // (a small layer's bias gradient rides in the launch of the filter gradient's reduction: the combined call below)
+    const bool small = batch_size * out_dims_.len() <= (size_t(1) << 20);
+    if (!in_delta_ && workspace_aux_ && overlap_on_ && !small) {
       // First layer, backward on two streams: its gradients are the last kernels of the pass.  The bias gradient goes
       // first (a memory-bound pass beside the second stream's last contraction), so that only the filter gradient's
       // reduction follows the last contraction of the step.
@@ -2007,8 +2012,10 @@ struct ClassifierTail {
       sg = context->aux_stream();
     }
     const float beta2 = fc2->params_.take_backward_beta();
-    const float beta1 = from_h ? 0.0f : fc1->params_.take_backward_beta();
-    if (from_h) fc1->delta_masked_once_ = true;   // its backward() follows: the delta it finds is the masked one
+    // (from h: the first layer's backward() follows and takes its beta itself; its bias gradient, the column sums of the
+    // delta this launch reads anyway, is formed here with the same beta)
+    const float beta1 = from_h ? (fc1->params_.grads_stale ? 0.0f : 1.0f) : fc1->params_.take_backward_beta();
+    if (from_h) fc1->delta_masked_once_ = fc1->bias_grad_done_ = true;   // the delta it finds is the masked one
     unwrap(rh_affine2_bwd_params((int)batch_size, I, H, C, from_h ? nullptr : fc1->in_act_->as_ptr(), fc1->out_act_->as_ptr(),
                                  fc1->out_delta_->as_ptr(), fc2->out_delta_->as_ptr(), beta1,
                                  fc1->params_.grad_weights->as_mut_ptr(), fc1->params_.grad_bias->as_mut_ptr(), beta2,

@@ -552,11 +552,11 @@ extern "C" int rh_affine2_bwd_params(int32_t B, int32_t I, int32_t H, int32_t C,
                                      float* db2, rh_stream_t stream) {
   if (B < 0 || I < 0 || H <= 0 || C <= 0 || (I == 0) != (x == nullptr)) return RH_E_INVALID;
   if (!rh_affine2_softmax_kl_step_supported(B > 0 ? B : 1, I, H, C)) return RH_E_UNSUPPORTED;
-  if (!h || !dlogits || !dw2 || !db2 || (x && (!dh || !dw1 || !db1))) return RH_E_INVALID;
+  if (!h || !dlogits || !dw2 || !db2 || (x && (!dh || !dw1 || !db1)) || (!x && db1 && !dh)) return RH_E_INVALID;
   const int vec = x && I % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dw1)) & 15) == 0 ? 1 : 0;
-  // (without x only the second layer's gradients are formed: no dW1 items and no db1 among the bias items)
+  // (without x no dW1 items, and db1 among the bias items only where it is asked for)
   const unsigned n1 = x ? (unsigned)((size_t)H * I / (vec ? 4 : 1)) : 0u, n2 = (unsigned)((size_t)C * H),
-                 n3 = (unsigned)((x ? H : 0) + C);
+                 n3 = (unsigned)((x || db1 ? H : 0) + C);
   const size_t total = (size_t)n1 + n2 + n3;
   ProfScope prof("affine2_bwd_params", 4.0 * ((double)B * (I + 2.0 * H + C) + (double)I * H + (double)H * C), to_stream(stream));
   hipLaunchKernelGGL(affine2_bwd_params_kernel, dim3((unsigned)cdiv<size_t>(total, 32)), dim3(256), 0, to_stream(stream), B, I, H,

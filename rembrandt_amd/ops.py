@@ -387,11 +387,12 @@ def affine_softmax_kl_step_from_h(h, w2, b2, labels, weights, relu1=True, counte
     return out
 
 
-def affine_bwd_params_from_h(h, dlogits, dw2, db2, beta2=0.0):
-    """dW2 and db2 only (rh_affine2_bwd_params with I = 0, x = NULL)."""
+def affine_bwd_params_from_h(h, dlogits, dw2, db2, beta2=0.0, dh=None, db1=None, beta1=0.0):
+    """dW2 and db2 (rh_affine2_bwd_params with I = 0, x = NULL) and, with dh and db1, db1 = sum_n dh + beta1 * db1."""
     B, H = h.shape
-    check(lib().rh_affine2_bwd_params(B, 0, H, dlogits.shape[1], None, _p(h), None, _p(dlogits), 0.0, None, None, beta2,
-                                      _p(dw2), _p(db2), _stream()), "rh_affine2_bwd_params")
+    check(lib().rh_affine2_bwd_params(B, 0, H, dlogits.shape[1], None, _p(h), _p(dh) if dh is not None else None, _p(dlogits),
+                                      beta1, None, _p(db1) if db1 is not None else None, beta2, _p(dw2), _p(db2), _stream()),
+          "rh_affine2_bwd_params")
 
 
 def affine2_bwd_params(x, h, dh, dlogits, dw1, db1, dw2, db2, beta1=0.0, beta2=0.0):

@@ -738,6 +738,16 @@ def test_affine_softmax_kl_step_from_h(dev, case):
             r2 = O.sgemm(0, 1, H, Cc, B, 1.0, h, H, dll, Cc, beta2, dw2_0.copy(), H)
             assert_close(N(dw2), r2, "from_h dW2 beta %g" % beta2)
             assert_close(N(db2), (dll.astype(np.float64).sum(axis=0) + beta2 * db2_0).astype(np.float32), "from_h db2 beta %g" % beta2)
+            # with dh and db1: the first layer's bias gradient too, the second layer's unchanged bit for bit
+            db1_0 = synth.normal(43, 10 * rep + 12, (H,))
+            dw2b, db2b, db1 = T(dw2_0, dev), T(db2_0, dev), T(db1_0, dev)
+            ops.affine_bwd_params_from_h(h_dev, out["dlogits"], dw2b, db2b, beta2, dh=out["dh"], db1=db1, beta1=beta2)
+            assert torch.equal(dw2b, dw2) and torch.equal(db2b, db2)
+            assert_close(N(db1), (N(out["dh"]).astype(np.float64).sum(axis=0) + beta2 * db1_0).astype(np.float32),
+                         "from_h db1 beta %g" % beta2)
+        # db1 without dh is refused
+        assert _lib.lib().rh_affine2_bwd_params(B, 0, H, Cc, None, h_dev.data_ptr(), None, out["dlogits"].data_ptr(), 0.0, None,
+                                                db1.data_ptr(), 0.0, dw2.data_ptr(), db2.data_ptr(), None) == _lib.RH_E_INVALID
 
 
 def test_affine2_softmax_kl_step_limits(dev):
