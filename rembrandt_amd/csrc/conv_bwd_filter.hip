@@ -862,8 +862,8 @@ extern "C" size_t rh_conv2d_workspace_bytes(const rh_conv_geom* g, int pass) {
       size_t need = sp.ok && sp.total() > legacy ? sp.total() : legacy;
       const Bf16FwdPlan bp = plan_bf16_fwd(d);  // the bf16 flag is not known here: room for either form
       if (bp.ok && bp.total() > need) need = bp.total();
-      if (wino_shape(d)) {   // the flags are not known here: room for the Winograd form wherever the geometry has one
-        const WinoGeom wg = wino_geom_fwd(d);
+      if (wino_shape(d) || wino_shape5(d)) {   // the flags are not known here: room for the Winograd form wherever the geometry has one
+        const WinoGeom wg = wino_shape5(d) ? wino_geom_fwd5(d) : wino_geom_fwd(d);
         if (wg.ok && wg.total() > need) need = wg.total();
       }
       return need;

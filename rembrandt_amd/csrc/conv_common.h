@@ -320,10 +320,19 @@ struct WinoGeom {
   int full_tiles, tail_S, tail_L;
   long long part_first, slab_elems;
   size_t part_bytes;
-  size_t total() const { return u_bytes + v_bytes + part_bytes; }
+  // 5x5 forward (wino_geom_fwd5): the filter, extended with zeros to 6x6, is four 3x3 filters at offsets (3 bi, 3 bj);
+  // the layer is the sum of their four 3x3 layers over shifted inputs, added in the transform domain: the same 16
+  // products over 4 C "channels" (channel 4 c + 2 bi + bj = input channel c read 3 bi rows and 3 bj columns further
+  // on): 64 multiply-adds per 2x2 outputs, filter and channel instead of 100.  Ci = 4 C here; the input is read from a
+  // zero-bordered copy of Hp x Wp a plane (pad zeros in front, the rest behind), made in img_bytes of scratch.
+  int blk5 = 0, C5 = 0, H5 = 0, W5 = 0, pad5 = 0;
+  size_t img_bytes = 0;
+  size_t total() const { return u_bytes + v_bytes + img_bytes + part_bytes; }
 };
-WinoGeom wino_geom(int N, int Ci, int Hi, int Wi, int Ko, int halo);
+WinoGeom wino_geom(int N, int Ci, int Hi, int Wi, int Ko, int halo, int blk5 = 0);
 inline bool wino_shape(const ConvDims& d) { return d.R == 3 && d.S == 3 && d.st == 1 && d.pad <= 2; }
+inline bool wino_shape5(const ConvDims& d) { return d.R == 5 && d.S == 5 && d.st == 1 && d.pad <= 4 && d.P > 0 && d.Q > 0; }
+inline WinoGeom wino_geom_fwd5(const ConvDims& d) { return wino_geom(d.N, d.C, d.H, d.W, d.K, d.pad, 1); }
 inline WinoGeom wino_geom_fwd(const ConvDims& d) { return wino_geom(d.N, d.C, d.H, d.W, d.K, d.pad); }
 inline WinoGeom wino_geom_bwd_data(const ConvDims& d) { return wino_geom(d.N, d.K, d.P, d.Q, d.C, 2 - d.pad); }
 // Where the library takes it by itself: enough channels on both sides for the 16 products to be worth their
@@ -332,6 +341,13 @@ inline bool wino_pays(const WinoGeom& g) {
   // (rows: 128-row tiles at least three quarters full: 64 filters in one would execute as much as the direct form)
   return g.ok && g.Ci >= 64 && g.Ko >= 64 && 4 * g.Ko >= 3 * g.rows_p &&
          (long long)(g.rows_p / kWinoBM) * (g.tiles_p / kWinoBN) >= 192;
+}
+// The 5x5 forward form executes 64 % of the direct form's multiply-adds (a little more where the 2x2 tiles overhang
+// the result) at a lower rate than the direct kernels reach, 18 % less time on 96 -> 256 channels, 27 x 27, batch 256:
+// taken for full row tiles, a channel loop long next to a block's prologue and epilogue, and several rounds of blocks.
+inline bool wino_pays5(const WinoGeom& g) {
+  return g.ok && g.blk5 && g.C5 >= 64 && g.Ko >= 64 && 8 * g.Ko >= 7 * g.rows_p &&
+         (long long)(g.rows_p / kWinoBM) * (g.tiles_p / kWinoBN) >= 512;
 }
 // Filter gradient in the same form: zero-bordered copies of x and dy, S slices of the tiles, their partial sums.
 struct WinoFilterPlan {

@@ -588,15 +588,17 @@ extern "C" int rh_conv2d_fwd(const rh_conv_geom* g, float alpha, const float* x,
   if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return RH_E_WORKSPACE;
   hipStream_t stream = to_stream(stream_);
 
-  if ((flags & RH_ALGO_WINOGRAD) && (!wino_shape(d) || (flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))))
+  if ((flags & RH_ALGO_WINOGRAD) && (!(wino_shape(d) || wino_shape5(d)) ||
+                                     (flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))))
     return RH_E_UNSUPPORTED;
   if (!(flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET)) && conv1x1_stream_applies(d))
     return launch_conv1x1_stream(d, RH_CONV_FWD, w, x, y, alpha, beta, (flags & RH_FUSE_BIAS) ? bias : nullptr,
                                  (flags & RH_FUSE_RELU) ? 1 : 0, stream);
-  if (wino_shape(d) && !(flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))) {
-    WinoGeom wg = wino_geom_fwd(d);
+  if ((wino_shape(d) || wino_shape5(d)) && !(flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT))) {
+    const bool five = wino_shape5(d);   // a 5x5 layer as four 3x3 layers, added in the transform domain
+    WinoGeom wg = five ? wino_geom_fwd5(d) : wino_geom_fwd(d);
     if (flags & RH_ALGO_SHARED_GPU) wg.tail_S = 1;
-    if (flags & RH_ALGO_WINOGRAD ? wg.ok : wino_pays(wg))
+    if (flags & RH_ALGO_WINOGRAD ? wg.ok : five ? wino_pays5(wg) : wino_pays(wg))
       return launch_conv_wino(wg, false, x, w, y, alpha, beta, (flags & RH_FUSE_BIAS) ? bias : nullptr,
                               (flags & RH_FUSE_RELU) ? 1 : 0, nullptr, ws, stream, "conv_fwd_wino");
     if (flags & RH_ALGO_WINOGRAD) return RH_E_UNSUPPORTED;

@@ -32,10 +32,20 @@
 
 namespace rh {
 
-WinoGeom wino_geom(int N, int Ci, int Hi, int Wi, int Ko, int halo) {
+WinoGeom wino_geom(int N, int Ci, int Hi, int Wi, int Ko, int halo, int blk5) {
   WinoGeom g;
   g.N = N; g.Ci = Ci; g.Hi = Hi; g.Wi = Wi; g.Ko = Ko; g.halo = halo;
   g.P = Hi + 2 * halo - 2; g.Q = Wi + 2 * halo - 2;
+  if (blk5) {
+    // the 5x5 layer as four 3x3 layers over a zero-bordered copy: the kernel sees an image of Hp x Wp without halo and
+    // 4 C channels; patch rows 2 ty + 3 bi .. + 3 of the copy reach row 2 TP + 4
+    g.blk5 = 1; g.C5 = Ci; g.H5 = Hi; g.W5 = Wi; g.pad5 = halo;
+    g.P = Hi + 2 * halo - 4; g.Q = Wi + 2 * halo - 4;
+    g.Hi = 2 * cdiv(g.P > 0 ? g.P : 1, 2) + 5; g.Wi = 2 * cdiv(g.Q > 0 ? g.Q : 1, 2) + 5;
+    g.halo = 0; g.Ci = 4 * Ci;
+    Ci = g.Ci; Hi = g.Hi; Wi = g.Wi; halo = 0;
+    g.img_bytes = align256(sizeof(float) * (size_t)N * g.C5 * g.Hi * g.Wi);
+  }
   g.TP = g.P > 0 ? cdiv(g.P, 2) : 0; g.TQ = g.Q > 0 ? cdiv(g.Q, 2) : 0;
   g.tiles = (long long)N * g.TP * g.TQ;
   g.tiles_p = (g.tiles + kWinoBN - 1) / kWinoBN * kWinoBN;
@@ -48,6 +58,7 @@ WinoGeom wino_geom(int N, int Ci, int Hi, int Wi, int Ko, int halo) {
   // 32-bit byte offsets into U and V, 31-bit tile indices
   g.ok = g.P > 0 && g.Q > 0 && halo >= 0 && halo <= 2 && ub < (1ull << 31) && (Ci % 4 == 0 || vb < (1ull << 31)) &&
          g.tiles_p < (1ll << 30) && (long long)N * Ko * g.P * g.Q < (1ll << 30) && (long long)N * Ci * Hi * Wi < (1ll << 30);
+  if (blk5) g.ok = g.ok && g.pad5 <= 4 && g.Hi >= g.H5 + g.pad5 && g.Wi >= g.W5 + g.pad5;
   // One block per CU at a time: 784 blocks are four rounds of the 256 CUs with the last one 6 % full.  The blocks past
   // the last whole round are cut into slices of the channel loop (every slice a whole number of stages, four at
   // least), so that the last round is as short as its share of the work; their partial results are added by
@@ -81,6 +92,7 @@ namespace {
 struct WinoPrepArgs {
   const float* w; const float* x; float* U; float* V;
   int Ko, Ci, Cg, rows_p, bwd;
+  int blk5, C5;       // the 5x5 form: "channel" v = 4 c + 2 bi + bj is the 3x3 block at (3 bi, 3 bj) of input channel c's filter
   int Hi, Wi, halo;
   unsigned tiles, tiles_p, x_bytes;
   FastDiv dRows, dPairs, dTQ, dTP;
@@ -103,6 +115,11 @@ __device__ __forceinline__ void wino_filter_item(const WinoPrepArgs& a, unsigned
       for (int s = 0; s < 3; ++s) {
         // forward: w[row][c][r][s]; backward-data: rows are the input channels of w, the contraction runs over its
         // filters, taps flipped: w[c][row][2-r][2-s]
+        if (a.blk5) {
+          const int rr = 3 * ((c >> 1) & 1) + r, ss = 3 * (c & 1) + s;   // the 5x5 filter with a sixth row and column of zeros
+          g[r][s] = live && rr < 5 && ss < 5 ? a.w[((size_t)row * a.C5 + (c >> 2)) * 25 + (size_t)(rr * 5 + ss)] : 0.0f;
+          continue;
+        }
         const size_t at = a.bwd ? ((size_t)c * a.Ko + row) * 9 + (size_t)((2 - r) * 3 + (2 - s))
                                 : ((size_t)row * a.Ci + c) * 9 + (size_t)(r * 3 + s);
         g[r][s] = live ? a.w[at] : 0.0f;
@@ -478,6 +495,7 @@ __global__ __launch_bounds__(256, 1) void wino_gemm_kernel(const float* __restri
 // loads counted by hand; everything else is LDS and register work the compiler sees.
 struct WinoImage {
   const float* x; unsigned x_bytes; int Ci, Hi, Wi, halo;
+  int blk5;   // the 5x5 form: Ci is the planes an image has; the four channels of a stage are one plane read at four offsets
 };
 
 constexpr int kWinoRaw = 12 * 256 * 4;             // bytes of one stage's raw patch rows
@@ -564,11 +582,15 @@ __global__ __launch_bounds__(256, 1) void wino_gemm_fused_kernel(const float* __
       }
   }
   const uint32_t chan_stride = (uint32_t)HW * 4u;
+  // this wave's channel of stage cg lies at cg * tap_mul + tap_add: plane 4 cg + wave, or in the 5x5 form plane cg read
+  // 3 (wave / 2) rows and 3 (wave % 2) columns further on
+  const uint32_t tap_mul = im.blk5 ? chan_stride : 4u * chan_stride;
+  const uint32_t tap_add = im.blk5 ? (uint32_t)(3 * (wave >> 1) * im.Wi + 3 * (wave & 1)) * 4u : (uint32_t)wave * chan_stride;
   // direct load i (0..11: patch taps into raw slot `par`; 12..19: U into ring buffer `buf`) of stage cg
   auto issue_one = [&](int i, int cg, int buf, int par) {
     if (i < 12)
       dma_load4(rsX, raw0 + (uint32_t)par * kWinoRaw + (uint32_t)i * 1024u + (uint32_t)wave * 256u, poff[i >> 2][i & 3],
-                (uint32_t)(4 * (cg0 + cg) + wave) * chan_stride);
+                (uint32_t)(cg0 + cg) * tap_mul + tap_add);
     else
       dma_load16(rsU, lds0 + (uint32_t)buf * kWinoStage + (uint32_t)(wave * 8 + (i - 12)) * 1024u, voffA,
                  soA[i - 12] + (uint32_t)(cg0 + cg) * strideA);
@@ -1106,12 +1128,21 @@ int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* 
   if (!g.ok) return RH_E_UNSUPPORTED;
   float* U = static_cast<float*>(ws);
   float* V = reinterpret_cast<float*>(static_cast<char*>(ws) + g.u_bytes);
+  if (g.blk5) {
+    // the zero-bordered copy the 5x5 form reads (behind U; V is made in the kernel)
+    if (bwd) return RH_E_UNSUPPORTED;
+    float* xp = reinterpret_cast<float*>(static_cast<char*>(ws) + g.u_bytes + g.v_bytes);
+    launch_pad_image(in, xp, (long long)g.N * g.C5, g.H5, g.W5, g.Hi, g.Wi, g.pad5, stream);
+    if (int e = launch_status()) return e;
+    in = xp;
+  }
   WinoPrepArgs a;
   a.w = w; a.x = in; a.U = U; a.V = V;
+  a.blk5 = g.blk5; a.C5 = g.C5;
   a.Ko = g.Ko; a.Ci = g.Ci; a.Cg = g.Cg; a.rows_p = g.rows_p; a.bwd = bwd ? 1 : 0;
   a.Hi = g.Hi; a.Wi = g.Wi; a.halo = g.halo;
   a.tiles = (unsigned)g.tiles; a.tiles_p = (unsigned)g.tiles_p;
-  a.x_bytes = (unsigned)(4ull * (unsigned long long)g.N * g.Ci * g.Hi * g.Wi);
+  a.x_bytes = (unsigned)(4ull * (unsigned long long)g.N * (g.blk5 ? g.C5 : g.Ci) * g.Hi * g.Wi);
   a.dRows = FastDiv((uint32_t)g.rows_p); a.dPairs = FastDiv((uint32_t)(g.tiles_p / 2));
   a.dTQ = FastDiv((uint32_t)g.TQ); a.dTP = FastDiv((uint32_t)g.TP);
   const unsigned long long fi = (unsigned long long)g.Cg * 2 * g.rows_p, ii = (unsigned long long)g.Cg * 2 * (g.tiles_p / 2);
@@ -1141,11 +1172,12 @@ int launch_conv_wino(const WinoGeom& g, bool bwd, const float* in, const float* 
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_f);
     if (attr_f != hipSuccess) return (int)attr_f;
     WinoImage im;
-    im.x = in; im.x_bytes = a.x_bytes; im.Ci = g.Ci; im.Hi = g.Hi; im.Wi = g.Wi; im.halo = g.halo;
+    im.x = in; im.x_bytes = a.x_bytes; im.Ci = g.blk5 ? g.C5 : g.Ci; im.Hi = g.Hi; im.Wi = g.Wi; im.halo = g.halo;
+    im.blk5 = g.blk5;
     ProfScope prof(tag, 2.0 * 16.0 * (double)g.Ko * g.Ci * (double)g.tiles, stream);
     WinoTail tl;
     tl.full = g.full_tiles; tl.S = g.tail_S; tl.L = g.tail_L;
-    tl.part = reinterpret_cast<float*>(static_cast<char*>(ws) + g.u_bytes + g.v_bytes);
+    tl.part = reinterpret_cast<float*>(static_cast<char*>(ws) + g.u_bytes + g.v_bytes + g.img_bytes);
     tl.slab_elems = g.slab_elems; tl.part_first = g.part_first;
     const long long T = (long long)tiles_m_ * tiles_n_;
     const long long blocks = g.tail_S > 1 ? g.full_tiles + (T - g.full_tiles) * g.tail_S : T;
@@ -1259,8 +1291,14 @@ using namespace rh;
 
 extern "C" double rh_conv2d_winograd_flops(const rh_conv_geom* g, int pass, int flags) {
   ConvDims d;
-  if (conv_dims(g, &d) || !wino_shape(d)) return 0.0;
+  if (conv_dims(g, &d)) return 0.0;
   if (flags & (RH_MATH_BF16_MFMA_FP32ACC | RH_ALGO_GATHER | RH_ALGO_SCALAR_OFFSET | RH_ALGO_DIRECT)) return 0.0;
+  if (wino_shape5(d) && pass == RH_CONV_FWD) {
+    const WinoGeom wg = wino_geom_fwd5(d);
+    if (!(flags & RH_ALGO_WINOGRAD ? wg.ok : wino_pays5(wg))) return 0.0;
+    return 2.0 * 16.0 * (double)wg.Ko * wg.Ci * (double)wg.tiles;
+  }
+  if (!wino_shape(d)) return 0.0;
   if (pass == RH_CONV_BWD_FILTER) {
     const WinoFilterPlan wp = plan_wino_bwd_filter(d);
     if (!(flags & RH_ALGO_WINOGRAD ? wp.ok : wino_filter_pays(d, wp))) return 0.0;

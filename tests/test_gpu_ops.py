@@ -246,11 +246,65 @@ def test_conv2d_winograd(dev, case):
     torch.cuda.synchronize()
 
 
+WINO5_CASES = [
+    # N, C, H, W, K, pad
+    (2, 3, 9, 9, 8, 2),
+    (1, 1, 5, 5, 1, 0),            # one output pixel
+    (3, 5, 8, 11, 130, 1),
+    (2, 8, 7, 6, 20, 4),
+    (2, 16, 12, 13, 64, 3),
+    (4, 32, 27, 27, 96, 2),
+    (40, 32, 27, 27, 256, 2),      # 504 blocks: whole rounds and sliced tail blocks
+    (70, 96, 13, 14, 128, 2),
+    (44, 64, 27, 27, 128, 2),      # 539 blocks: the library takes this form by itself
+]
+
+
+@pytest.mark.parametrize("case", WINO5_CASES, ids=str)
+def test_conv2d_winograd_5x5_forward(dev, case):
+    """RH_ALGO_WINOGRAD on a 5x5 stride-1 layer (forward only): the filter as four 3x3 blocks of its 6x6 zero extension,
+    F(2x2, 3x3) on each over the shifted input, added in the transform domain; against the oracle's direct convolution,
+    with every epilogue; the backward passes refuse the bit; the library's own choice and RH_ALGO_DIRECT."""
+    Nn, C, H, W, K, pad = case
+    say("winograd 5x5 case", case)
+    WG = _lib.RH_ALGO_WINOGRAD
+    x = synth.normal(17, 1, (Nn, C, H, W))
+    w = synth.normal(17, 2, (K, C, 5, 5))
+    b = synth.normal(17, 3, (K,))
+    y_ref = O.conv2d_fwd(x, w, 1, pad)
+    xd, wd, bd = T(x, dev), T(w, dev), T(b, dev)
+    y = ops.conv2d_fwd(xd, wd, 1, pad, algo=WG)
+    assert_close(N(y), y_ref, "winograd 5x5 fwd")
+    yf = ops.conv2d_fwd(xd, wd, 1, pad, bias=bd, relu=True, algo=WG)
+    assert_close(N(yf), O.rect_inplace(O.add_bias_nchw(b, y_ref.copy())), "winograd 5x5 fwd fused bias+relu")
+    assert torch.equal(torch.clamp_min(y + bd.view(1, -1, 1, 1), 0.0), yf), "fused epilogue == conv, add_bias, rect"
+    y0 = synth.normal(17, 5, y_ref.shape)
+    yb = ops.conv2d_fwd(xd, wd, 1, pad, alpha=0.5, beta=2.0, y=T(y0, dev), algo=WG)
+    assert_close(N(yb), O.conv2d_fwd(x, w, 1, pad, alpha=0.5, beta=2.0, y=y0.copy()), "winograd 5x5 fwd alpha/beta")
+    assert torch.equal(ops.conv2d_fwd(xd, wd, 1, pad, algo=WG), y), "run to run the same bits"
+    assert_close(N(ops.conv2d_fwd(xd, wd, 1, pad, algo=WG | _lib.RH_ALGO_SHARED_GPU)), y_ref, "winograd 5x5 fwd, shared-GPU hint")
+    assert ops.conv2d_winograd_flops(x.shape, w.shape, 1, pad, "fwd", algo=WG) == \
+        2.0 * 16 * K * 4 * C * Nn * (-(-y_ref.shape[2] // 2)) * (-(-y_ref.shape[3] // 2))
+    # forward only
+    dy = T(synth.normal(17, 4, y_ref.shape), dev)
+    for fn in (lambda: ops.conv2d_bwd_data(wd, dy, x.shape, 1, pad, algo=WG), lambda: ops.conv2d_bwd_filter(xd, dy, w.shape, 1, pad, algo=WG)):
+        with pytest.raises(_lib.RembrandtHipError):
+            fn()
+    # the library's choice: this form for full row tiles and several rounds of blocks, else the direct one
+    auto = ops.conv2d_fwd(xd, wd, 1, pad)
+    direct = ops.conv2d_fwd(xd, wd, 1, pad, algo=_lib.RH_ALGO_DIRECT)
+    assert_close(N(direct), y_ref, "RH_ALGO_DIRECT fwd (5x5)")
+    blocks = -(-K // 128) * -(-(Nn * -(-y_ref.shape[2] // 2) * -(-y_ref.shape[3] // 2)) // 32)
+    takes = C >= 64 and K >= 64 and 8 * K >= 7 * (-(-K // 128) * 128) and blocks >= 512
+    assert torch.equal(auto, y if takes else direct), "library's choice (5x5)"
+    torch.cuda.synchronize()
+
+
 def test_conv2d_winograd_refused_geometries(dev):
     import ctypes as C
     x = torch.zeros((2, 4, 8, 8), device=dev)
     ws = torch.zeros((1 << 22,), dtype=torch.uint8, device=dev)
-    for R, st, pad, extra in ((5, 1, 2, 0), (3, 2, 1, 0), (1, 1, 0, 0), (3, 1, 3, 0), (3, 1, 1, _lib.RH_ALGO_GATHER),
+    for R, st, pad, extra in ((5, 2, 2, 0), (7, 1, 3, 0), (3, 2, 1, 0), (1, 1, 0, 0), (3, 1, 3, 0), (3, 1, 1, _lib.RH_ALGO_GATHER),
                               (3, 1, 1, _lib.RH_ALGO_DIRECT), (3, 1, 1, _lib.RH_MATH_BF16_MFMA_FP32ACC)):
         g = _lib.ConvGeom(2, 4, 8, 8, 4, R, R, st, pad)
         w = torch.zeros((4, 4, R, R), device=dev)
