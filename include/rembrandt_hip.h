@@ -49,9 +49,11 @@ typedef void* rh_stream_t; /* hipStream_t */
 #define RH_ALGO_SCALAR_OFFSET      0x200 /* scalar-offset loads on padded / transposed copies in the workspace,
                                             wherever the geometry allows it (else the gather family)             */
 #define RH_ALGO_WINOGRAD           0x400 /* every pass of a 3x3 stride-1 layer by Winograd F(2x2, 3x3): 2.25x
-                                            fewer multiply-adds, sums in another order (RH_E_UNSUPPORTED for other
-                                            geometries).  Without an RH_ALGO_* bit the library takes it for such layers
-                                            of 64 channels and more on both sides; either bit above keeps the direct form */
+                                            fewer multiply-adds, sums in another order; the forward pass of a 5x5
+                                            stride-1 layer in the same form (its filter as four 3x3 blocks: 1.56x
+                                            fewer).  RH_E_UNSUPPORTED for other geometries and passes.  Without an
+                                            RH_ALGO_* bit the library takes it for such layers of 64 channels and more
+                                            on both sides; either bit above keeps the direct form */
 #define RH_ALGO_DIRECT             0x800 /* never the Winograd form; the direct forms chosen as without any RH_ALGO_* bit */
 #define RH_ALGO_SHARED_GPU         0x1000 /* a hint, with any of the above: kernels of another stream run beside this call.
                                              Forms that spend compute-unit time to shorten the call's own last round of

@@ -115,9 +115,10 @@ int rho_config_from_model_file(const char* path, rho_config** out);
  *                           launches otherwise.  Same buffers with the same meaning; sums in another order, so results
  *                           agree with the separate operators to rounding.  This flag keeps the separate operators. */
 #define RHO_EXEC_SEPARATE_TAIL 0x10
-/*   RHO_EXEC_DIRECT_CONV    3x3 stride-1 convolutions keep the direct form in all three passes (RH_ALGO_DIRECT).
- *                           Without it the library takes Winograd's F(2x2, 3x3) for such layers of 64 channels and more:
- *                           2.25x fewer multiply-adds, sums in another order (same tolerance against the oracle). */
+/*   RHO_EXEC_DIRECT_CONV    3x3 and 5x5 stride-1 convolutions keep the direct form in all three passes (RH_ALGO_DIRECT).
+ *                           Without it the library takes Winograd's F(2x2, 3x3) for 3x3 layers of 64 channels and more
+ *                           (2.25x fewer multiply-adds) and for the forward pass of such 5x5 layers (1.56x fewer):
+ *                           sums in another order, same tolerance against the oracle. */
 #define RHO_EXEC_DIRECT_CONV 0x20
 int rho_worker_new(const rho_config* cfg, int32_t batch_size, int capability, uint64_t seed0, uint64_t seed1,
                    int device, int exec_flags, rho_worker** out);

@@ -19,6 +19,12 @@
 //  * the epilogue: a lane's element e of the 16 accumulators is the whole 4x4 M of one (row, tile): A^T M A is 24
 //    additions in registers, then alpha / beta, bias, ReLU or the mask of a folded ReLU backward, and the 2x2 pixels
 //    go to the NCHW result (odd extents: the tile's pixels past the edge are dropped).
+//  * blocks past the last whole round of the 256 CUs take slices of the channel loop and wino_tail_reduce_kernel adds
+//    their partial results (wino_geom); not where the caller says that other kernels run beside the call.
+//  * the forward pass of a 5x5 stride-1 layer is the same kernel over four times the channels: the filter's zero
+//    extension to 6x6 is four 3x3 filters, the layer the sum of their four 3x3 layers over the input read 3 rows / 3
+//    columns further on, and that sum is taken in the transform domain like the one over the channels
+//    (wino_geom_fwd5, WinoImage::blk5): 64 multiply-adds per 2x2 outputs, filter and channel instead of 100.
 // Filter gradient: wino_filter_prep_kernel, wino_bwd_filter_kernel, wino_filter_reduce_kernel, described further down.
 //
 // Operand layout (floats):  U[f][cg][h][rows_p][2],  V[f][cg][h][tiles_p][2]  with channel = 4 cg + 2 h + j.  The MFMA
