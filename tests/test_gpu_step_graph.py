@@ -254,22 +254,26 @@ def profile_tags(fn):
 
 
 WINO_DIMS = (16, 16, 8)
+WINO5_DIMS = (24, 24, 8)
 
 
 def wino_net(kind):
     if kind == "plain":      # conv -> conv (ReLU backward folded into the second layer's data gradient) -> pool -> fc
         spec = [("conv", 3, 1, 1, 128, "Rect"), ("conv", 3, 1, 1, 128, "Rect"), ("conv", 3, 1, 1, 128, "Identity"),
                 ("pool", 2, 2, 0, "Max"), ("fc", 10, "Identity")]
+    elif kind == "five":     # a 5x5 layer of 64 -> 128 channels on 24 x 24: its forward pass in the same form (four 3x3 blocks), 576 blocks
+        spec = [("conv", 3, 1, 1, 64, "Rect"), ("conv", 5, 1, 2, 128, "Rect"), ("pool", 2, 2, 0, "Max"), ("fc", 10, "Identity")]
+        return (WINO5_DIMS, *configs._chain(WINO5_DIMS, spec))
     else:                    # batch-normalised residual units: their 3x3 convolutions take the same form
         spec = [("conv", 3, 1, 1, 128, "Rect"), ("res", "Rect"), ("projres", 256, 2, "Rect"), ("pool", 2, 2, 0, "Average"),
                 ("fc", 10, "Identity")]
     return (WINO_DIMS, *configs._chain(WINO_DIMS, spec))
 
 
-@pytest.mark.parametrize("kind", ["plain", "bnorm"])
+@pytest.mark.parametrize("kind", ["plain", "bnorm", "five"])
 def test_winograd_steps_match_direct_steps(dev, kind):
     """Train steps whose 3x3 layers of 128 channels run in the Winograd form (all three passes, what the library picks
-    by itself at this size) against the same steps with RHO_EXEC_DIRECT_CONV: same losses, counts,
+    by itself at this size; "five": the forward pass of a 5x5 layer) against the same steps with RHO_EXEC_DIRECT_CONV: same losses, counts,
     parameters and momentum to rounding; the Winograd kernels did run in the first and not in the second.
     Two fp32 paths that add in different orders are compared here, through ReLU masks (an activation within rounding
     of zero changes side) and bias gradients (sums of 32768 deltas that largely cancel): relative L2 distance 2e-3 after the first step, 1e-2 after
@@ -283,8 +287,11 @@ def test_winograd_steps_match_direct_steps(dev, kind):
     say("winograd steps", kind)
     (a, _), tags_a = profile_tags(lambda: run(net, batch, steps, False, 0x3141, kw, read_grads=False))
     (b, _), tags_b = profile_tags(lambda: run(net, batch, steps, False, 0x3141, kw, read_grads=False, winograd=False))
-    assert "conv_fwd_wino" in tags_a and "conv_bwd_data_wino" in tags_a and "wino_transform" in tags_a
-    assert "conv_bwd_filter_wino" in tags_a
+    assert "conv_fwd_wino" in tags_a and "wino_transform" in tags_a
+    if kind == "five":   # forward only: the backward passes of a 5x5 layer stay direct
+        assert "conv_bwd_data_wino" not in tags_a and "conv_bwd_filter_wino" not in tags_a
+    else:
+        assert "conv_bwd_data_wino" in tags_a and "conv_bwd_filter_wino" in tags_a
     assert not any("wino" in t for t in tags_b)
     for step, ((la, ca, pa), (lb, cb, pb)) in enumerate(zip(a, b)):
         assert abs(la - lb) <= 1e-4 * max(1.0, abs(lb)), (step, la, lb)
@@ -294,3 +301,16 @@ def test_winograd_steps_match_direct_steps(dev, kind):
             dist = np.sqrt(((u - v) ** 2).sum()) / max(np.sqrt((v ** 2).sum()), 1e-30)
             bound = 2e-3 if step == 0 else 1e-2 if kind == "plain" else 5e-2
             assert dist <= bound, "%s step %d buffer %d: relative L2 distance %.3g" % (kind, step, k, dist)
+
+
+@pytest.mark.parametrize("kind", ["plain", "five"])
+def test_recorded_steps_of_winograd_networks(dev, kind):
+    """Steps whose convolutions run in the Winograd form (transform launches, sliced last-round blocks with their reduction,
+    the zero-bordered copy of the 5x5 form), recorded and replayed: the same bits as launched."""
+    say("step graph, winograd", kind)
+    net = wino_net(kind)
+    kw = dict(step_size=0.01, momentum=("Update", 0.9), l2_reg_coef=5e-4)
+    eager, n0 = run(net, 128, 5, False, 0x6A11, kw)
+    graph, n1 = run(net, 128, 5, True, 0x6A11, kw)
+    assert n0 == 0 and n1 == 3
+    same(eager, graph, "winograd " + kind)
