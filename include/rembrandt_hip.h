@@ -270,6 +270,10 @@ int rh_pool2d_bwd(const rh_pool_geom* g, const float* x, const float* y, const f
 int rh_pool2d_bwd_relu_supported(const rh_pool_geom* g);
 int rh_pool2d_bwd_relu(const rh_pool_geom* g, const float* y, const float* dy, float* dx, const int32_t* argmax,
                        rh_stream_t stream);
+/* Average-pool backward with the same fold: dx = [x > 0] * pool_bwd(dy), x the pool's input (the ReLU's output);
+ * bit-identical to rh_pool2d_bwd followed by rembrandt_kernel_batch_map_rect_backprop_inplace on dx.
+ * RH_E_UNSUPPORTED for max pooling. */
+int rh_pool2d_bwd_avg_relu(const rh_pool_geom* g, const float* x, const float* dy, float* dx, rh_stream_t stream);
 /* The same pooling with a one-byte mask: slot[n,c,p,q] = r*size + s of the winning element inside its window (first
  * maximum, as above), 255 for a window without elements.  For an operator's private mask (a quarter of the int32
  * form's bytes on both passes; the gen-1 API's int32 plane index, src/layer.rs:1797-1813, stays rh_pool2d_fwd's).

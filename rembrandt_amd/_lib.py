@@ -115,6 +115,7 @@ PROTOTYPES = {
     "rh_pool2d_bwd": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp, _vp, _vp]),
     "rh_pool2d_bwd_relu_supported": (_int, [C.POINTER(PoolGeom)]),
     "rh_pool2d_bwd_relu": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp, _vp]),
+    "rh_pool2d_bwd_avg_relu": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp]),
     "rh_pool2d_slot_supported": (_int, [C.POINTER(PoolGeom)]),
     "rh_pool2d_fwd_slot": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp]),
     "rh_pool2d_bwd_slot": (_int, [C.POINTER(PoolGeom), _vp, _vp, _vp, _vp, _vp]),

@@ -1045,6 +1045,9 @@ class Pool2dOperator : public Operator {
       else argmax_.reset(new DeviceBuffer<int32_t>(out_dims_.len() * batch_size, context));
       if (opts.fuse_epilogue && rh_pool2d_bwd_relu_supported(&g)) fold_relu_ = prev_op->fold_activation_backward();
     }
+    // average pooling: the same fold, with the pool's input (the ReLU's output) as the mask
+    if (config.pool_op == PoolOperation::Average && in_delta_ && opts.fuse_epilogue)
+      fold_relu_ = prev_op->fold_activation_backward();
   }
   size_t batch_size() const override { return batch_cap_; }
   SharedDeviceBuf get_output_vars() const override { return out_act_; }
@@ -1086,6 +1089,11 @@ class Pool2dOperator : public Operator {
     if (slot_) {
       unwrap(rh_pool2d_bwd_slot(&g, fold_relu_ ? out_act_->as_ptr() : nullptr, out_delta_->as_ptr(), in_delta_->as_mut_ptr(),
                                 slot_->as_ptr(), context_->stream()), "pooling backward");
+      return;
+    }
+    if (fold_relu_ && config_.pool_op == PoolOperation::Average) {
+      unwrap(rh_pool2d_bwd_avg_relu(&g, in_act_->as_ptr(), out_delta_->as_ptr(), in_delta_->as_mut_ptr(), context_->stream()),
+             "pooling backward");
       return;
     }
     if (fold_relu_) {

@@ -255,9 +255,11 @@ __global__ __launch_bounds__(256) void pool_fwd_lds_kernel(PoolDims d, FastDiv d
   }
 }
 
+// relu_x (average pooling): the pool's input, the output of a ReLU; dx is 0 where it is not > 0 (that ReLU's backward).
 template <class I>
 __global__ void pool_bwd_kernel(PoolDims d, const float* __restrict__ x, const float* __restrict__ dy,
-                                float* __restrict__ dx, const int* __restrict__ argmax) {
+                                float* __restrict__ dx, const int* __restrict__ argmax,
+                                const float* __restrict__ relu_x = nullptr) {
   const I total = (I)d.N * d.C * d.H * d.W;
   const I stride = (I)gridDim.x * blockDim.x;
   const float inv = 1.0f / (float)(d.k * d.k);
@@ -302,6 +304,7 @@ __global__ void pool_bwd_kernel(PoolDims d, const float* __restrict__ x, const f
     } else {
       for (int p = p_lo; p <= p_hi; ++p)
         for (int q = q_lo; q <= q_hi; ++q) acc += dyp[p * d.Q + q] * inv;
+      if (relu_x && !(relu_x[idx] > 0.0f)) acc = 0.0f;
     }
     dx[idx] = acc;
   }
@@ -662,6 +665,24 @@ extern "C" int rh_pool2d_bwd_relu(const rh_pool_geom* g, const float* y, const f
   if (in_elems == 0) return 0;
   ProfScope prof("pool_max_bwd_relu", 4.0 * (in_elems + 3.0 * out_elems), to_stream(stream));
   return launch_pool_bwd_lds(d, dy, argmax, y, dx, stream);
+}
+
+extern "C" int rh_pool2d_bwd_avg_relu(const rh_pool_geom* g, const float* x, const float* dy, float* dx, rh_stream_t stream) {
+  PoolDims d;
+  if (int e = pool_dims(g, &d)) return e;
+  if (!x || !dy || !dx) return RH_E_INVALID;
+  if (d.mode != RH_POOL_AVG_INCL_PAD) return RH_E_UNSUPPORTED;
+  const long long total = (long long)d.N * d.C * d.H * d.W;
+  if (total == 0) return 0;
+  ProfScope prof("pool_avg_bwd_relu", 4.0 * (2.0 * (double)total + (double)d.N * d.C * d.P * d.Q), to_stream(stream));
+  const dim3 grid((unsigned)cdiv<long long>(total, 256) > (1u << 20) ? (1u << 20) : (unsigned)cdiv<long long>(total, 256));
+  if (total < (1ll << 31))
+    hipLaunchKernelGGL(pool_bwd_kernel<unsigned>, grid, dim3(256), 0, to_stream(stream), d, (const float*)nullptr, dy, dx,
+                       (const int*)nullptr, x);
+  else
+    hipLaunchKernelGGL(pool_bwd_kernel<long long>, grid, dim3(256), 0, to_stream(stream), d, (const float*)nullptr, dy, dx,
+                       (const int*)nullptr, x);
+  return launch_status();
 }
 
 // The one-byte mask: max pooling with size <= 15 on the geometries that both the LDS forward and the colour backward take.

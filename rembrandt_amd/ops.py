@@ -287,6 +287,14 @@ def pool2d_bwd_relu(x_shape, y, dy, size, stride, pad, argmax, rounding=_lib.RH_
     return dx
 
 
+def pool2d_bwd_avg_relu(x, dy, size, stride, pad, rounding=_lib.RH_ROUND_FLOOR):
+    """Average-pool backward with the backward of the ReLU that produced the pool's input x folded in."""
+    g = pool_geom(x.shape, size, stride, pad, _lib.RH_POOL_AVG_INCL_PAD, rounding)
+    dx = torch.empty(tuple(x.shape), dtype=torch.float32, device=dy.device)
+    check(lib().rh_pool2d_bwd_avg_relu(C.byref(g), _p(x), _p(dy), _p(dx), _stream()), "rh_pool2d_bwd_avg_relu")
+    return dx
+
+
 def softmax_fwd(x):
     N, Cc = x.shape
     p = torch.empty_like(x)

@@ -200,6 +200,7 @@ extern "C" {
   pub fn rh_pool2d_bwd_relu_supported(g: *const rh_pool_geom) -> c_int;
   pub fn rh_pool2d_bwd_relu(g: *const rh_pool_geom, y: *const f32, dy: *const f32, dx: *mut f32,
                             argmax: *const i32, stream: rh_stream_t) -> c_int;
+  pub fn rh_pool2d_bwd_avg_relu(g: *const rh_pool_geom, x: *const f32, dy: *const f32, dx: *mut f32, stream: rh_stream_t) -> c_int;
 
   // Data3dOperator preprocessing (src/operator/mod.rs:666-691, 716-725, 767-773) and dropout (mod.rs:2220-2246).
   pub fn rh_crop_nchw(src: *const f32, dst: *mut f32, planes: i64, in_w: i32, in_h: i32, crop_w: i32, crop_h: i32,

@@ -31,7 +31,7 @@ pub enum ActivationFunction { Identity, Rect, Logistic, Tanh }
 #[derive(Clone, Copy, Debug)]
 pub enum ParamsInit { Disabled, Uniform{half_range: f32}, Normal{std: f32}, Xavier, KaimingFwd }
 
-#[derive(Clone, Copy, Debug)]
+#[derive(Clone, Copy, Debug, PartialEq)]
 pub enum PoolOperation { Max, Average }
 
 pub trait Operator {
@@ -650,9 +650,15 @@ impl Pool2dOperator {
       fold_relu: false,
     };
     let g = op.geom(batch_size);
-    if let PoolOperation::Max = config.pool_op {
-      if op.in_delta.is_some() && unsafe { rh_pool2d_bwd_relu_supported(&g) } != 0 {
-        op.fold_relu = prev_op.fold_activation_backward();
+    match config.pool_op {
+      PoolOperation::Max => {
+        if op.in_delta.is_some() && unsafe { rh_pool2d_bwd_relu_supported(&g) } != 0 {
+          op.fold_relu = prev_op.fold_activation_backward();
+        }
+      }
+      // average pooling: the same fold with the pool's input (the ReLU's output) as the mask
+      PoolOperation::Average => {
+        if op.in_delta.is_some() { op.fold_relu = prev_op.fold_activation_backward(); }
       }
     }
     op
@@ -679,7 +685,10 @@ impl Operator for Pool2dOperator {
     assert!(batch_size <= self.batch_cap);
     let g = self.geom(batch_size);
     if let Some(ref in_delta) = self.in_delta {
-      if self.fold_relu {
+      if self.fold_relu && self.config.pool_op == PoolOperation::Average {
+        unwrap(unsafe { rh_pool2d_bwd_avg_relu(&g, self.in_act.borrow().as_ptr(), self.out_delta.borrow().as_ptr(),
+                                               in_delta.borrow_mut().as_mut_ptr(), self.context.stream()) }, "pool2d backward");
+      } else if self.fold_relu {
         // an arg-max element carries x = y, so windows with y <= 0 route nothing: the ReLU mask without a pass of its own
         unwrap(unsafe { rh_pool2d_bwd_relu(&g, self.out_act.borrow().as_ptr(), self.out_delta.borrow().as_ptr(),
                                            in_delta.borrow_mut().as_mut_ptr(), self.argmax.as_ptr(),

@@ -1056,6 +1056,30 @@ def test_pool2d_bwd_with_folded_relu_mask(dev, case, rounding):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("case", [(2, 3, 9, 3, 2, 0), (2, 3, 9, 3, 2, 1), (3, 4, 8, 2, 2, 0), (2, 5, 27, 3, 2, 0), (2, 2, 13, 3, 3, 1)])
+@pytest.mark.parametrize("rounding", [_lib.RH_ROUND_FLOOR, _lib.RH_ROUND_CEIL])
+def test_avg_pool2d_bwd_with_folded_relu_mask(dev, case, rounding):
+    """rh_pool2d_bwd_avg_relu == average-pool backward followed by the ReLU backward mask of the pool's input: against the
+    oracle's two passes, and bit-identical to the two GPU kernels it replaces; max pooling is refused."""
+    Nn, C, H, k, st, pad = case
+    say("avg pool bwd + relu case", case, rounding)
+    x = O.rect_inplace(synth.normal(18, 1, (Nn, C, H, H)) - np.float32(0.3))
+    xd = T(x, dev)
+    y = ops.pool2d_fwd(xd, k, st, pad, _lib.RH_POOL_AVG_INCL_PAD, rounding)
+    dy = synth.normal(18, 2, tuple(y.shape))
+    want = O.pool2d_bwd(x, N(y), dy, k, st, pad, O.POOL_AVG, rounding)
+    O.rect_backprop_inplace(x, want)
+    got = ops.pool2d_bwd_avg_relu(xd, T(dy, dev), k, st, pad, rounding)
+    assert_close(N(got), want, "avg pool bwd with folded relu mask")
+    two = ops.pool2d_bwd(xd, y, T(dy, dev), k, st, pad, _lib.RH_POOL_AVG_INCL_PAD, rounding)
+    ops.rect_backprop_inplace(xd, two)
+    assert torch.equal(got, two)
+    import ctypes as C
+    g = ops.pool_geom(x.shape, k, st, pad, _lib.RH_POOL_MAX, rounding)
+    assert _lib.lib().rh_pool2d_bwd_avg_relu(C.byref(g), xd.data_ptr(), T(dy, dev).data_ptr(), got.data_ptr(), None) == _lib.RH_E_UNSUPPORTED
+    torch.cuda.synchronize()
+
+
 def test_context_memory_calls(dev):
     """rh_malloc (zero-filled), rh_host_malloc (page-locked, zero-filled), rh_load_sync / rh_store_sync round trip,
     rh_store_begin / rh_store_wait."""
