@@ -348,6 +348,42 @@ SWEEP = {  # the single-operator sweep: N, C, H, W, K, R, stride, pad
 }
 
 
+def _wino_direct_form_flops(net, batch, tag):
+    """Direct-form FLOPs (2*N*K*C*R*S*P*Q) per step of the convolution passes that run under a Winograd tag
+    (conv_fwd_wino, conv_bwd_data_wino, conv_bwd_filter_wino), for plain convolution layers; None for other tags
+    and for networks with other kinds of convolution operators."""
+    which = {"conv_fwd_wino": "fwd", "conv_bwd_data_wino": "bwd_data", "conv_bwd_filter_wino": "bwd_filter"}.get(tag)
+    if which is None:
+        return None
+    from rembrandt_amd import ops
+    total, first = 0.0, True
+    for l in net[1]:
+        if l[0] in ("bnorm_conv2d", "stack_res_conv2d", "proj_stack_res_conv2d"):
+            return None
+        if l[0] == "affine":
+            first = False
+        if l[0] != "conv2d":
+            continue
+        (w, h, c), k, st, pad, out = l[1], l[2], l[3], l[4], l[5]
+        P, Q = max(0, h + 2 * pad - k + st) // st, max(0, w + 2 * pad - k + st) // st
+        if not (which == "bwd_data" and first) and ops.conv2d_winograd_flops((batch, c, h, w), (out, c, k, k), st, pad, which) > 0:
+            total += 2.0 * batch * out * c * k * k * P * Q
+        first = False
+    return total
+
+
+def _wino_note(net, batch, dom):
+    """For a Winograd tag: `achieved` / `frac` count the multiply-adds the kernels execute (16 per 2x2 tile, filter and
+    channel); the same launches priced in the direct form's FLOPs ride along."""
+    direct = _wino_direct_form_flops(net, batch, dom["kernel"])
+    if not direct or not dom.get("launches_per_step") or not dom.get("avg_launch_ms"):
+        return {}
+    per_launch = direct / dom["launches_per_step"]
+    return {"flops_counted": "executed by the Winograd F(2x2,3x3) form (16 multiply-adds per 2x2 tile, filter and channel)",
+            "direct_form_gflop_per_launch": per_launch / 1e9,
+            "direct_form_tflops": per_launch / dom["avg_launch_ms"] / 1e9}
+
+
 def _executed_flops(kernels):
     """FLOPs per step that the contraction kernels execute: what the kernels report as their work (the Winograd
     kernels 16 multiply-adds per 2x2 tile, filter and channel, where the direct form's count has 36)."""
@@ -576,7 +612,7 @@ def main():
                      "unit": dom["unit"], "frac": dom["frac"], "avg_launch_ms": dom["avg_launch_ms"],
                      "traffic": traffic,
                      "traffic_unit": "bytes per launch (L2<->fabric, FETCH_SIZE + WRITE_SIZE counters)",
-                     "traffic_source": traffic_source},
+                     "traffic_source": traffic_source, **_wino_note(net, batch, dom)},
         # all contraction kernels together: executed FLOPs (the Winograd kernels' own count) against the matrix peak;
         # `direct_form_tflops` prices the same time in the direct form's multiply-adds (config.gemm_gflop_per_step)
         "all_mfma": {"ms_per_step": gemm_ms, "executed_gflop_per_step": _executed_flops(mfma) / 1e9,
