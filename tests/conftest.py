@@ -19,7 +19,7 @@ def pytest_configure(config):
 # contraction); the multiple leaves room for other summation orders, not for other arithmetic.
 TIGHT_MULTIPLE = 2.0
 LAST = {"tight_ratio": 0.0}   # max |got-ref| / (1e-5*rms + 1e-4*|ref|) of the most recent assert_close
-WORST = {"tight_ratio": 0.0, "what": ""}   # and of the whole session (written to gpurun_out/ at its end)
+WORST = {"tight_ratio": 0.0, "what": ""}   # and of the whole session (written to the output folder at its end)
 
 
 def pytest_sessionfinish(session, exitstatus):
